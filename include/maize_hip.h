@@ -1,0 +1,184 @@
+/*
+ * maize_hip.h -- C ABI of libmaize_hip.so: the MI355X (gfx950) launch path for
+ * maize's pipelined tiled BF16 GEMM.
+ *
+ * The reference (averyparr/maize) stops at a PTX string: it has no launch
+ * path and no FFI (src/main.rs:80-89 prints the artefact and exits).  The
+ * entry points below are what a Rust host crate binds to carry the same
+ * builder -> compile -> artefact flow through to a launch on an AMD GPU, and
+ * each one names the reference item whose role it takes over.
+ *
+ * Conventions
+ *  - Every function returns int32_t: 0 = MAIZE_OK, negative = maize error
+ *    (enum below), positive = the hipError_t that HIP reported.
+ *  - maize_hip_last_error() returns a thread-local, NUL-terminated message
+ *    for the most recent failure on the calling thread.
+ *  - No exception or panic crosses the boundary.  Handles are opaque, owned by
+ *    the caller and released with the matching destroy/unload/free call.
+ *  - Device buffers are caller-owned.  A context may be used from one thread
+ *    at a time (the reference's builders are thread-local and !Send,
+ *    crates/maize_core/src/codegen/mod.rs:15-33); distinct contexts are
+ *    independent.
+ *  - Launches are asynchronous on the stream passed in (NULL = the null
+ *    stream).
+ *  - All matrices are row-major with leading dimension == ncols, as in the
+ *    reference (crates/maize_tile/src/gmem/row_panel.rs:55,
+ *    crates/maize_tile/src/gmem/col_panel.rs:108).  BF16 is a 2-byte,
+ *    2-aligned, u16-backed type (crates/maize_core/src/ty/sized.rs:62-68).
+ */
+#ifndef MAIZE_HIP_H
+#define MAIZE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    MAIZE_OK = 0,
+    MAIZE_ERR_NULL = -1,        /* a required pointer argument is NULL */
+    MAIZE_ERR_SHAPE = -2,       /* zero/mismatched dimensions or batch/stride inconsistency */
+    MAIZE_ERR_ALIGN = -3,       /* a device pointer is not 2-byte aligned */
+    MAIZE_ERR_LAYOUT = -4,      /* unknown maize_layout_t value */
+    MAIZE_ERR_KERNEL = -5,      /* unknown kernel name, or the kernel cannot run this descriptor */
+    MAIZE_ERR_NO_DEVICE = -6,   /* no usable HIP device / device is not gfx950 */
+    MAIZE_ERR_ARG = -7          /* any other invalid argument */
+};
+
+typedef struct maize_ctx maize_ctx_t;
+typedef struct maize_module maize_module_t;
+typedef struct maize_kernel maize_kernel_t;
+typedef struct maize_event maize_event_t;
+
+/* == GlobalMatrix<T>::Realized, the #[repr(C)] host twin that struct_reflect!
+ * generates for the reference's kernel-side descriptor (src/main.rs:20-27,
+ * crates/maize_core/src/ty/struct_ty.rs:113-121): a global pointer and two
+ * u32 extents, 16-byte aligned. */
+typedef struct {
+    void* ptr;
+    uint32_t nrows;
+    uint32_t ncols;
+} __attribute__((aligned(16))) maize_matrix_t;
+
+/* How B is stored.  NN is the reference's layout (A row panels x B column
+ * panels of a K x N row-major B, src/main.rs:56-57).  NT stores B
+ * transposed, N x K row-major, so both operands are K-contiguous. */
+typedef enum { MAIZE_LAYOUT_NN = 0, MAIZE_LAYOUT_NT = 1 } maize_layout_t;
+
+/* One (optionally strided-batched) GEMM C = A.B.
+ *   a: M x K.   b: K x N (NN) or N x K (NT).   c: M x N.
+ * batch >= 1; strides are in elements between consecutive batch members and
+ * are ignored when batch == 1. */
+typedef struct {
+    maize_matrix_t a, b, c;
+    uint32_t layout; /* maize_layout_t */
+    uint32_t batch;
+    uint64_t stride_a, stride_b, stride_c;
+} maize_gemm_desc_t;
+
+/* Kernel parameter block of every GEMM kernel in the embedded code object.
+ * It keeps the order and widths of the reference kernel's parameter list
+ * (example_ptx/gen.ptx:12-19: A ptr, arows u32, acols u32, B ptr, brows u32,
+ * bcols u32) and appends the C operand the reference never had, the batch
+ * strides, the batch count and the layout. */
+typedef struct {
+    const void* a; uint32_t arows, acols;
+    const void* b; uint32_t brows, bcols;
+    void* c;       uint32_t crows, ccols;
+    uint64_t stride_a, stride_b, stride_c;
+    uint32_t batch;
+    uint32_t layout;
+} maize_gemm_args_t;
+
+typedef struct {
+    char name[64];          /* hipDeviceProp_t::gcnArchName */
+    uint32_t compute_units;
+    uint32_t clock_khz;     /* max engine clock */
+    uint32_t lds_bytes_per_block;
+    uint32_t wavefront_size;
+    uint64_t hbm_bytes;
+} maize_device_info_t;
+
+const char* maize_hip_last_error(void);
+
+/* ---- context ------------------------------------------------------------
+ * Takes the role of the reference's thread-local codegen context
+ * (crates/maize_core/src/codegen/mod.rs:15-33): everything else hangs off it.
+ * Creating a context selects the device, checks that it is gfx950 and loads
+ * the embedded code object. */
+int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out);
+int32_t maize_hip_ctx_destroy(maize_ctx_t* ctx);
+int32_t maize_hip_device_info(maize_ctx_t* ctx, maize_device_info_t* out);
+
+/* ---- artefact -> module -> kernel -> launch ------------------------------
+ * Continues the reference's compile step, which ends in an in-memory
+ * artefact (PreJitFunction::compile*, crates/maize_core/src/codegen/
+ * typed_func.rs:749-874): load a gfx950 code object (hipModuleLoadData), look
+ * a kernel up by name (hipModuleGetFunction) and launch it with an explicit
+ * grid, block, dynamic LDS size and packed argument block
+ * (hipModuleLaunchKernel with HIP_LAUNCH_PARAM_BUFFER_POINTER).  block[] plays
+ * the role of with_launch_bounds_2d (crates/maize_core/src/codegen/
+ * calling_convention.rs:66-78). */
+int32_t maize_hip_module_load(maize_ctx_t* ctx, const void* hsaco, size_t nbytes, maize_module_t** out);
+int32_t maize_hip_module_unload(maize_module_t* mod);
+int32_t maize_hip_kernel_get(maize_module_t* mod, const char* name, maize_kernel_t** out);
+int32_t maize_hip_kernel_release(maize_kernel_t* k);
+int32_t maize_hip_launch(maize_kernel_t* k, const uint32_t grid[3], const uint32_t block[3],
+                         uint32_t lds_bytes, void* stream, const void* args, size_t args_bytes);
+/* The code object embedded in the library (what ctx_create loads). */
+int32_t maize_hip_embedded_code_object(const void** data, size_t* nbytes);
+
+/* ---- the GEMM path --------------------------------------------------------
+ * maize_hip_gemm_bf16 is the north-star entry: it validates the descriptor,
+ * picks a kernel and a grid for it and launches on `stream`.  It replaces
+ * the kernel that src/main.rs:31-90 builds from sm80_gemm_smem_multibuffer
+ * (crates/maize_tile/src/gemm/mod.rs:37-90), adds the C store and the
+ * edge-tile handling the reference leaves out (src/main.rs:56-57,71). */
+int32_t maize_hip_gemm_bf16(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream);
+/* Same, but with the kernel named by the caller (see maize_hip_kernel_name);
+ * fails with MAIZE_ERR_KERNEL if that kernel cannot run the descriptor. */
+int32_t maize_hip_gemm_bf16_with(maize_ctx_t* ctx, const maize_gemm_desc_t* desc,
+                                 const char* kernel, void* stream);
+/* Which kernel maize_hip_gemm_bf16 would pick; writes a NUL-terminated name. */
+int32_t maize_hip_gemm_select(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, char* name, size_t cap);
+/* Validation only (no device access): the checks gemm_bf16 performs first. */
+int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* desc);
+/* Enumerates the GEMM kernels of the embedded code object. */
+uint32_t maize_hip_kernel_count(void);
+const char* maize_hip_kernel_name(uint32_t index);
+/* Whether kernel `kernel` accepts `desc` (1), does not (0), or error (<0). */
+int32_t maize_hip_kernel_supports(const char* kernel, const maize_gemm_desc_t* desc);
+
+/* ---- thin pass-throughs ---------------------------------------------------
+ * Device memory, streams and events, so that a host crate needs no other HIP
+ * binding. */
+int32_t maize_hip_malloc(maize_ctx_t* ctx, size_t nbytes, void** out);
+int32_t maize_hip_free(maize_ctx_t* ctx, void* ptr);
+int32_t maize_hip_memcpy_h2d(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes);
+int32_t maize_hip_memcpy_d2h(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes);
+int32_t maize_hip_memset(maize_ctx_t* ctx, void* dst, int value, size_t nbytes);
+int32_t maize_hip_stream_create(maize_ctx_t* ctx, void** out);
+int32_t maize_hip_stream_destroy(maize_ctx_t* ctx, void* stream);
+int32_t maize_hip_sync(maize_ctx_t* ctx, void* stream); /* NULL: whole device */
+int32_t maize_hip_event_create(maize_ctx_t* ctx, maize_event_t** out);
+int32_t maize_hip_event_record(maize_event_t* ev, void* stream);
+int32_t maize_hip_event_synchronize(maize_event_t* ev);
+int32_t maize_hip_event_elapsed_ms(maize_event_t* start, maize_event_t* stop, float* ms);
+int32_t maize_hip_event_destroy(maize_event_t* ev);
+
+/* ---- host-side helpers ----------------------------------------------------
+ * Seeded, counter-based, libm-free input generators (bit-reproducible on any
+ * machine) and bf16 conversion.  Element i of a logical matrix is a pure
+ * function of (seed, i). */
+uint16_t maize_bf16_from_f32(float x); /* round-to-nearest-even */
+float maize_bf16_to_f32(uint16_t h);
+void maize_fill_uniform_bf16(uint16_t* dst, size_t n, uint64_t seed, size_t first_index);
+/* sigma is applied in fp64 before the single rounding to bf16. */
+void maize_fill_normal_bf16(uint16_t* dst, size_t n, uint64_t seed, double sigma, size_t first_index);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

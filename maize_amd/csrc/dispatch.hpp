@@ -1,0 +1,49 @@
+// Kernel registry and shape dispatch (host logic only; no HIP calls).
+//
+// Plays the part of the reference's panel iterators, which turn matrix
+// extents and a grid into per-block work (Matrix::collective_aligned_row_
+// panel_iter, crates/maize_tile/src/gmem/row_panel.rs:85-127, and its column
+// twin col_panel.rs:88-124): given a descriptor, decide which kernel covers
+// it and with what grid.
+#pragma once
+#include <stdint.h>
+
+#include "maize_hip.h"
+
+namespace maize {
+
+constexpr uint32_t kMaxKernels = 32;
+
+struct LaunchDims {
+    uint32_t grid[3];
+    uint32_t block[3];
+    uint32_t lds_bytes;
+};
+
+struct KernelInfo {
+    const char* name;
+    bool (*supports)(const maize_gemm_desc_t&);
+    // Fills the launch dimensions; false if the grid would exceed HIP limits.
+    bool (*plan)(const maize_gemm_desc_t&, uint32_t compute_units, LaunchDims*);
+};
+
+uint32_t kernel_count();
+const KernelInfo& kernel_at(uint32_t i);
+int kernel_index(const char* name);  // -1 if unknown
+// Index of the kernel the dispatcher picks for a validated descriptor.
+uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units);
+
+struct Dims {
+    uint32_t m, n, k;
+    bool nt;
+};
+inline Dims dims_of(const maize_gemm_desc_t& d) {
+    Dims r;
+    r.m = d.c.nrows;
+    r.n = d.c.ncols;
+    r.k = d.a.ncols;
+    r.nt = d.layout == MAIZE_LAYOUT_NT;
+    return r;
+}
+
+}  // namespace maize

@@ -1,0 +1,4 @@
+// Single translation unit of the gfx950 code object embedded in libmaize_hip.so.
+#include "common.hpp"
+#include "gemm_wave32.hpp"
+#include "probes.hpp"

@@ -1,0 +1,73 @@
+// maize_gemm_bf16_wave32: the any-shape kernel.
+//
+// One wavefront owns one 32x32 tile of C and walks K in steps of 16 with
+// v_mfma_f32_32x32x16_bf16, loading its operand fragments straight from
+// global memory with per-element bounds checks.  No alignment, divisibility
+// or minimum-size requirement: it is the kernel the dispatcher falls back to
+// when a shape or pointer does not meet the tiled kernels' 16-byte rules.
+// Mirrors the reference's per-warp fragment loop (sync_mma_from_smem,
+// crates/maize_tile/src/gemm/mod.rs:18-33) without the shared-memory ring.
+//
+// MFMA 32x32x16 operand maps (lane l, 0..63):
+//   A operand: row  = l % 32, k = 8*(l/32) + e, e = 0..7
+//   B operand: col  = l % 32, k = 8*(l/32) + e
+//   D result : col  = l % 32, row = 8*(v/4) + 4*(l/32) + v%4, v = 0..15
+// The kernel feeds B's fragment as the first operand and A's as the second,
+// so D holds C transposed: each lane then owns 4 consecutive columns of one
+// row of C per group of 4 accumulator registers.
+#pragma once
+#include "common.hpp"
+
+namespace maize {
+
+__device__ __forceinline__ __bf16 bf16_from_bits(uint16_t h) {
+    return __builtin_bit_cast(__bf16, h);
+}
+
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArgs p) {
+    const uint32_t M = p.crows, N = p.ccols, K = p.acols;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;  // 0..3, arranged 2 x 2
+    const uint32_t m0 = blockIdx.y * 64u + (wave >> 1) * 32u;
+    const uint32_t n0 = blockIdx.x * 64u + (wave & 1u) * 32u;
+    if (m0 >= M || n0 >= N) return;  // whole wave leaves together
+
+    const uint64_t bz = blockIdx.z;
+    const uint16_t* __restrict__ A = p.a + bz * p.stride_a;
+    const uint16_t* __restrict__ B = p.b + bz * p.stride_b;
+    uint16_t* __restrict__ C = p.c + bz * p.stride_c;
+
+    const uint32_t r = lane & 31u;   // row of A / column of B owned by this lane
+    const uint32_t kg = lane >> 5;   // which 8-wide k group
+    const uint32_t am = m0 + r;
+    const uint32_t bn = n0 + r;
+    const bool nt = p.layout != 0u;
+
+    floatx16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    for (uint32_t k0 = 0; k0 < K; k0 += 16u) {
+        bf16x8 fa, fb;
+#pragma unroll
+        for (uint32_t e = 0; e < 8u; ++e) {
+            const uint32_t k = k0 + kg * 8u + e;
+            uint16_t av = 0, bv = 0;
+            if (k < K) {
+                if (am < M) av = A[(uint64_t)am * K + k];
+                if (bn < N) bv = nt ? B[(uint64_t)bn * K + k] : B[(uint64_t)k * N + bn];
+            }
+            fa[e] = bf16_from_bits(av);
+            fb[e] = bf16_from_bits(bv);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb, fa, acc, 0, 0, 0);
+    }
+    // D[i][j] with i = column of C (n), j = row of C (m).
+    const uint32_t cm = m0 + r;
+    if (cm < M) {
+#pragma unroll
+        for (uint32_t v = 0; v < 16u; ++v) {
+            const uint32_t cn = n0 + 8u * (v >> 2) + 4u * kg + (v & 3u);
+            if (cn < N) C[(uint64_t)cm * N + cn] = f32_to_bf16_rne(acc[v]);
+        }
+    }
+}
+
+}  // namespace maize

@@ -1,0 +1,416 @@
+// libmaize_hip.so -- the C ABI declared in include/maize_hip.h.
+//
+// Host-only C++ over the HIP module API (hipModuleLoadData /
+// hipModuleGetFunction / hipModuleLaunchKernel) on a gfx950 code object that is
+// embedded in this library.  There is no CPU execution path: every compute
+// entry point needs a gfx950 device and fails with an error code otherwise.
+#include "maize_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "dispatch.hpp"
+
+extern "C" const unsigned char maize_embedded_hsaco[];
+extern "C" const unsigned char maize_embedded_hsaco_end[];
+
+static_assert(sizeof(maize_matrix_t) == 16 && alignof(maize_matrix_t) == 16, "GlobalMatrix twin");
+static_assert(sizeof(maize_gemm_args_t) == 80, "kernel parameter block");
+static_assert(offsetof(maize_gemm_args_t, arows) == 8 && offsetof(maize_gemm_args_t, acols) == 12 &&
+                  offsetof(maize_gemm_args_t, b) == 16 && offsetof(maize_gemm_args_t, brows) == 24 &&
+                  offsetof(maize_gemm_args_t, bcols) == 28 && offsetof(maize_gemm_args_t, c) == 32,
+              "reference (ptr,u32,u32) x 2 prefix");
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int32_t fail(int32_t code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int32_t hip_fail(hipError_t e, const char* what) {
+    snprintf(g_err, sizeof g_err, "%s: %s (hipError_t %d)", what, hipGetErrorString(e), (int)e);
+    return (int32_t)e;
+}
+
+#define HIP_TRY(expr)                                  \
+    do {                                               \
+        hipError_t e_ = (expr);                        \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+}  // namespace
+
+struct maize_ctx {
+    int device;
+    hipDeviceProp_t prop;
+    hipModule_t module;
+    hipFunction_t fn[maize::kMaxKernels];
+};
+struct maize_module {
+    maize_ctx* ctx;
+    hipModule_t module;
+};
+struct maize_kernel {
+    maize_ctx* ctx;
+    hipFunction_t fn;
+};
+struct maize_event {
+    hipEvent_t ev;
+};
+
+extern "C" {
+
+const char* maize_hip_last_error(void) { return g_err; }
+
+int32_t maize_hip_embedded_code_object(const void** data, size_t* nbytes) {
+    if (!data || !nbytes) return fail(MAIZE_ERR_NULL, "embedded_code_object: NULL output pointer");
+    *data = maize_embedded_hsaco;
+    *nbytes = (size_t)(maize_embedded_hsaco_end - maize_embedded_hsaco);
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
+    if (!out) return fail(MAIZE_ERR_NULL, "ctx_create: out is NULL");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(MAIZE_ERR_NO_DEVICE, "ctx_create: no HIP device (%s)", hipGetErrorString(e));
+    if (device < 0 || device >= count)
+        return fail(MAIZE_ERR_NO_DEVICE, "ctx_create: device %d out of range (%d devices)", device, count);
+    HIP_TRY(hipSetDevice(device));
+    maize_ctx* ctx = new (std::nothrow) maize_ctx();
+    if (!ctx) return fail(MAIZE_ERR_ARG, "ctx_create: out of host memory");
+    ctx->device = device;
+    e = hipGetDeviceProperties(&ctx->prop, device);
+    if (e != hipSuccess) {
+        delete ctx;
+        return hip_fail(e, "hipGetDeviceProperties");
+    }
+    if (strncmp(ctx->prop.gcnArchName, "gfx950", 6) != 0) {
+        int32_t rc = fail(MAIZE_ERR_NO_DEVICE, "ctx_create: device %d is %s, this library only carries gfx950 code",
+                          device, ctx->prop.gcnArchName);
+        delete ctx;
+        return rc;
+    }
+    e = hipModuleLoadData(&ctx->module, maize_embedded_hsaco);
+    if (e != hipSuccess) {
+        delete ctx;
+        return hip_fail(e, "hipModuleLoadData(embedded code object)");
+    }
+    for (uint32_t i = 0; i < maize::kernel_count(); ++i) {
+        e = hipModuleGetFunction(&ctx->fn[i], ctx->module, maize::kernel_at(i).name);
+        if (e != hipSuccess) {
+            int32_t rc = hip_fail(e, maize::kernel_at(i).name);
+            (void)hipModuleUnload(ctx->module);
+            delete ctx;
+            return rc;
+        }
+    }
+    *out = ctx;
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_ctx_destroy(maize_ctx_t* ctx) {
+    if (!ctx) return fail(MAIZE_ERR_NULL, "ctx_destroy: ctx is NULL");
+    (void)hipSetDevice(ctx->device);
+    hipError_t e = hipModuleUnload(ctx->module);
+    delete ctx;
+    if (e != hipSuccess) return hip_fail(e, "hipModuleUnload");
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_device_info(maize_ctx_t* ctx, maize_device_info_t* out) {
+    if (!ctx || !out) return fail(MAIZE_ERR_NULL, "device_info: NULL argument");
+    memset(out, 0, sizeof *out);
+    snprintf(out->name, sizeof out->name, "%.63s", ctx->prop.gcnArchName);
+    out->compute_units = (uint32_t)ctx->prop.multiProcessorCount;
+    out->clock_khz = (uint32_t)ctx->prop.clockRate;
+    out->lds_bytes_per_block = (uint32_t)ctx->prop.sharedMemPerBlock;
+    out->wavefront_size = (uint32_t)ctx->prop.warpSize;
+    out->hbm_bytes = (uint64_t)ctx->prop.totalGlobalMem;
+    return MAIZE_OK;
+}
+
+/* ---- artefact -> module -> kernel -> launch ------------------------------ */
+
+int32_t maize_hip_module_load(maize_ctx_t* ctx, const void* hsaco, size_t nbytes, maize_module_t** out) {
+    if (!ctx || !hsaco || !out) return fail(MAIZE_ERR_NULL, "module_load: NULL argument");
+    *out = nullptr;
+    if (nbytes < 64 || memcmp(hsaco, "\177ELF", 4) != 0)
+        return fail(MAIZE_ERR_ARG, "module_load: not an ELF code object (%zu bytes)", nbytes);
+    HIP_TRY(hipSetDevice(ctx->device));
+    maize_module* m = new (std::nothrow) maize_module();
+    if (!m) return fail(MAIZE_ERR_ARG, "module_load: out of host memory");
+    m->ctx = ctx;
+    hipError_t e = hipModuleLoadData(&m->module, hsaco);
+    if (e != hipSuccess) {
+        delete m;
+        return hip_fail(e, "hipModuleLoadData");
+    }
+    *out = m;
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_module_unload(maize_module_t* mod) {
+    if (!mod) return fail(MAIZE_ERR_NULL, "module_unload: module is NULL");
+    (void)hipSetDevice(mod->ctx->device);
+    hipError_t e = hipModuleUnload(mod->module);
+    delete mod;
+    if (e != hipSuccess) return hip_fail(e, "hipModuleUnload");
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_kernel_get(maize_module_t* mod, const char* name, maize_kernel_t** out) {
+    if (!mod || !name || !out) return fail(MAIZE_ERR_NULL, "kernel_get: NULL argument");
+    *out = nullptr;
+    HIP_TRY(hipSetDevice(mod->ctx->device));
+    hipFunction_t fn;
+    hipError_t e = hipModuleGetFunction(&fn, mod->module, name);
+    if (e != hipSuccess) return hip_fail(e, name);
+    maize_kernel* k = new (std::nothrow) maize_kernel();
+    if (!k) return fail(MAIZE_ERR_ARG, "kernel_get: out of host memory");
+    k->ctx = mod->ctx;
+    k->fn = fn;
+    *out = k;
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_kernel_release(maize_kernel_t* k) {
+    if (!k) return fail(MAIZE_ERR_NULL, "kernel_release: kernel is NULL");
+    delete k;
+    return MAIZE_OK;
+}
+
+static int32_t launch_raw(int device, uint32_t lds_limit, hipFunction_t fn, const uint32_t grid[3],
+                          const uint32_t block[3], uint32_t lds_bytes, void* stream, const void* args,
+                          size_t args_bytes) {
+    for (int i = 0; i < 3; ++i)
+        if (grid[i] == 0 || block[i] == 0) return fail(MAIZE_ERR_ARG, "launch: zero grid/block extent");
+    const uint64_t threads = (uint64_t)block[0] * block[1] * block[2];
+    if (threads > 1024) return fail(MAIZE_ERR_ARG, "launch: %llu threads per block exceeds 1024", (unsigned long long)threads);
+    if (grid[1] > 65535u || grid[2] > 65535u) return fail(MAIZE_ERR_ARG, "launch: grid.y/z exceeds 65535");
+    if (lds_bytes > lds_limit) return fail(MAIZE_ERR_ARG, "launch: %u bytes of LDS exceeds the device's %u", lds_bytes, lds_limit);
+    HIP_TRY(hipSetDevice(device));
+    size_t sz = args_bytes;
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(args), HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz,
+                     HIP_LAUNCH_PARAM_END};
+    HIP_TRY(hipModuleLaunchKernel(fn, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes,
+                                  (hipStream_t)stream, nullptr, extra));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_launch(maize_kernel_t* k, const uint32_t grid[3], const uint32_t block[3], uint32_t lds_bytes,
+                         void* stream, const void* args, size_t args_bytes) {
+    if (!k || !grid || !block) return fail(MAIZE_ERR_NULL, "launch: NULL argument");
+    if (!args && args_bytes) return fail(MAIZE_ERR_NULL, "launch: args is NULL but args_bytes is %zu", args_bytes);
+    return launch_raw(k->ctx->device, (uint32_t)k->ctx->prop.sharedMemPerBlock, k->fn, grid, block, lds_bytes, stream,
+                      args, args_bytes);
+}
+
+/* ---- the GEMM path --------------------------------------------------------- */
+
+int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* d) {
+    if (!d) return fail(MAIZE_ERR_NULL, "gemm: descriptor is NULL");
+    if (d->layout != MAIZE_LAYOUT_NN && d->layout != MAIZE_LAYOUT_NT)
+        return fail(MAIZE_ERR_LAYOUT, "gemm: unknown layout %u", d->layout);
+    if (d->batch == 0) return fail(MAIZE_ERR_SHAPE, "gemm: batch is 0");
+    if (d->batch > 65535u) return fail(MAIZE_ERR_SHAPE, "gemm: batch %u exceeds 65535", d->batch);
+    const uint32_t M = d->a.nrows, K = d->a.ncols;
+    const uint32_t Kb = d->layout == MAIZE_LAYOUT_NN ? d->b.nrows : d->b.ncols;
+    const uint32_t N = d->layout == MAIZE_LAYOUT_NN ? d->b.ncols : d->b.nrows;
+    if (M == 0 || N == 0 || K == 0)
+        return fail(MAIZE_ERR_SHAPE, "gemm: empty operand (M=%u N=%u K=%u)", M, N, K);
+    if (Kb != K) return fail(MAIZE_ERR_SHAPE, "gemm: inner dimensions differ (A has K=%u, B has K=%u)", K, Kb);
+    if (d->c.nrows != M || d->c.ncols != N)
+        return fail(MAIZE_ERR_SHAPE, "gemm: C is %ux%u, expected %ux%u", d->c.nrows, d->c.ncols, M, N);
+    if (!d->a.ptr || !d->b.ptr || !d->c.ptr) return fail(MAIZE_ERR_NULL, "gemm: NULL matrix pointer");
+    if (((uintptr_t)d->a.ptr | (uintptr_t)d->b.ptr | (uintptr_t)d->c.ptr) & 1u)
+        return fail(MAIZE_ERR_ALIGN, "gemm: matrix pointers must be 2-byte aligned");
+    if (d->batch > 1) {
+        if (d->stride_a < (uint64_t)M * K || d->stride_b < (uint64_t)K * N || d->stride_c < (uint64_t)M * N)
+            return fail(MAIZE_ERR_SHAPE, "gemm: batch stride smaller than one matrix");
+    }
+    return MAIZE_OK;
+}
+
+uint32_t maize_hip_kernel_count(void) { return maize::kernel_count(); }
+
+const char* maize_hip_kernel_name(uint32_t index) {
+    return index < maize::kernel_count() ? maize::kernel_at(index).name : nullptr;
+}
+
+int32_t maize_hip_kernel_supports(const char* kernel, const maize_gemm_desc_t* desc) {
+    if (!kernel) return fail(MAIZE_ERR_NULL, "kernel_supports: kernel name is NULL");
+    int32_t rc = maize_hip_gemm_validate(desc);
+    if (rc != MAIZE_OK) return rc;
+    const int idx = maize::kernel_index(kernel);
+    if (idx < 0) return fail(MAIZE_ERR_KERNEL, "kernel_supports: no kernel named %s", kernel);
+    return maize::kernel_at((uint32_t)idx).supports(*desc) ? 1 : 0;
+}
+
+int32_t maize_hip_gemm_select(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, char* name, size_t cap) {
+    if (!ctx || !name || cap == 0) return fail(MAIZE_ERR_NULL, "gemm_select: NULL argument");
+    int32_t rc = maize_hip_gemm_validate(desc);
+    if (rc != MAIZE_OK) return rc;
+    const uint32_t idx = maize::select_kernel(*desc, (uint32_t)ctx->prop.multiProcessorCount);
+    snprintf(name, cap, "%s", maize::kernel_at(idx).name);
+    return MAIZE_OK;
+}
+
+static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_desc_t* d, uint32_t idx, void* stream) {
+    const maize::KernelInfo& ki = maize::kernel_at(idx);
+    maize_gemm_args_t args;
+    memset(&args, 0, sizeof args);
+    args.a = d->a.ptr; args.arows = d->a.nrows; args.acols = d->a.ncols;
+    args.b = d->b.ptr; args.brows = d->b.nrows; args.bcols = d->b.ncols;
+    args.c = d->c.ptr; args.crows = d->c.nrows; args.ccols = d->c.ncols;
+    args.batch = d->batch;
+    args.layout = d->layout;
+    if (d->batch > 1) {
+        args.stride_a = d->stride_a; args.stride_b = d->stride_b; args.stride_c = d->stride_c;
+    }
+    maize::LaunchDims ld;
+    if (!ki.plan(*d, (uint32_t)ctx->prop.multiProcessorCount, &ld))
+        return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s cannot run M=%u N=%u K=%u batch=%u (grid limit)", ki.name,
+                    d->c.nrows, d->c.ncols, d->a.ncols, d->batch);
+    return launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->fn[idx], ld.grid, ld.block,
+                      ld.lds_bytes, stream, &args, sizeof args);
+}
+
+int32_t maize_hip_gemm_bf16(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream) {
+    if (!ctx) return fail(MAIZE_ERR_NULL, "gemm: ctx is NULL");
+    int32_t rc = maize_hip_gemm_validate(desc);
+    if (rc != MAIZE_OK) return rc;
+    return gemm_launch(ctx, desc, maize::select_kernel(*desc, (uint32_t)ctx->prop.multiProcessorCount), stream);
+}
+
+int32_t maize_hip_gemm_bf16_with(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, const char* kernel, void* stream) {
+    if (!ctx || !kernel) return fail(MAIZE_ERR_NULL, "gemm_with: NULL argument");
+    int32_t rc = maize_hip_gemm_validate(desc);
+    if (rc != MAIZE_OK) return rc;
+    const int idx = maize::kernel_index(kernel);
+    if (idx < 0) return fail(MAIZE_ERR_KERNEL, "gemm_with: no kernel named %s", kernel);
+    if (!maize::kernel_at((uint32_t)idx).supports(*desc))
+        return fail(MAIZE_ERR_KERNEL, "gemm_with: kernel %s does not support this descriptor", kernel);
+    return gemm_launch(ctx, desc, (uint32_t)idx, stream);
+}
+
+/* ---- thin pass-throughs ------------------------------------------------------ */
+
+int32_t maize_hip_malloc(maize_ctx_t* ctx, size_t nbytes, void** out) {
+    if (!ctx || !out) return fail(MAIZE_ERR_NULL, "malloc: NULL argument");
+    *out = nullptr;
+    if (nbytes == 0) return fail(MAIZE_ERR_ARG, "malloc: zero bytes");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMalloc(out, nbytes));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_free(maize_ctx_t* ctx, void* ptr) {
+    if (!ctx) return fail(MAIZE_ERR_NULL, "free: ctx is NULL");
+    if (!ptr) return MAIZE_OK;
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipFree(ptr));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_memcpy_h2d(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes) {
+    if (!ctx || !dst || !src) return fail(MAIZE_ERR_NULL, "memcpy_h2d: NULL argument");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMemcpy(dst, src, nbytes, hipMemcpyHostToDevice));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_memcpy_d2h(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes) {
+    if (!ctx || !dst || !src) return fail(MAIZE_ERR_NULL, "memcpy_d2h: NULL argument");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMemcpy(dst, src, nbytes, hipMemcpyDeviceToHost));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_memset(maize_ctx_t* ctx, void* dst, int value, size_t nbytes) {
+    if (!ctx || !dst) return fail(MAIZE_ERR_NULL, "memset: NULL argument");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMemset(dst, value, nbytes));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_stream_create(maize_ctx_t* ctx, void** out) {
+    if (!ctx || !out) return fail(MAIZE_ERR_NULL, "stream_create: NULL argument");
+    HIP_TRY(hipSetDevice(ctx->device));
+    hipStream_t s;
+    HIP_TRY(hipStreamCreate(&s));  // default priority
+    *out = (void*)s;
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_stream_destroy(maize_ctx_t* ctx, void* stream) {
+    if (!ctx || !stream) return fail(MAIZE_ERR_NULL, "stream_destroy: NULL argument");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipStreamDestroy((hipStream_t)stream));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_sync(maize_ctx_t* ctx, void* stream) {
+    if (!ctx) return fail(MAIZE_ERR_NULL, "sync: ctx is NULL");
+    HIP_TRY(hipSetDevice(ctx->device));
+    if (stream)
+        HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    else
+        HIP_TRY(hipDeviceSynchronize());
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_event_create(maize_ctx_t* ctx, maize_event_t** out) {
+    if (!ctx || !out) return fail(MAIZE_ERR_NULL, "event_create: NULL argument");
+    *out = nullptr;
+    HIP_TRY(hipSetDevice(ctx->device));
+    maize_event* ev = new (std::nothrow) maize_event();
+    if (!ev) return fail(MAIZE_ERR_ARG, "event_create: out of host memory");
+    hipError_t e = hipEventCreate(&ev->ev);
+    if (e != hipSuccess) {
+        delete ev;
+        return hip_fail(e, "hipEventCreate");
+    }
+    *out = ev;
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_event_record(maize_event_t* ev, void* stream) {
+    if (!ev) return fail(MAIZE_ERR_NULL, "event_record: event is NULL");
+    HIP_TRY(hipEventRecord(ev->ev, (hipStream_t)stream));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_event_synchronize(maize_event_t* ev) {
+    if (!ev) return fail(MAIZE_ERR_NULL, "event_synchronize: event is NULL");
+    HIP_TRY(hipEventSynchronize(ev->ev));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_event_elapsed_ms(maize_event_t* start, maize_event_t* stop, float* ms) {
+    if (!start || !stop || !ms) return fail(MAIZE_ERR_NULL, "event_elapsed_ms: NULL argument");
+    HIP_TRY(hipEventElapsedTime(ms, start->ev, stop->ev));
+    return MAIZE_OK;
+}
+
+int32_t maize_hip_event_destroy(maize_event_t* ev) {
+    if (!ev) return fail(MAIZE_ERR_NULL, "event_destroy: event is NULL");
+    hipError_t e = hipEventDestroy(ev->ev);
+    delete ev;
+    if (e != hipSuccess) return hip_fail(e, "hipEventDestroy");
+    return MAIZE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,201 @@
+/*
+ * maize_oracle.c -- CPU oracle for the tiled BF16 GEMM path (see the header:
+ * test infrastructure only, never linked into the product).
+ *
+ * Follows the mathematical intent of the reference mainloop
+ * (crates/maize_tile/src/gemm/mod.rs:37-90: zip A/B K-tiles, accumulate
+ * A-fragment x B-fragment products into one accumulator per output element)
+ * with the accumulator widened to fp64 and one final rounding to bf16.
+ */
+#include "maize_oracle.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+
+float mzo_bf16_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, sizeof f);
+    return f;
+}
+
+/* One RNE rounding from double: scale so that one bf16 quantum is 1.0, round
+ * to the nearest integer (ties to even, the default rounding mode), scale
+ * back.  The result is exactly representable as a float whose low 16 bits
+ * are zero (or overflows to infinity), so taking the high half is exact. */
+uint16_t mzo_bf16_from_f64(double x) {
+    if (isnan(x)) return (uint16_t)((signbit(x) ? 0x8000u : 0u) | 0x7FC0u);
+    if (isinf(x)) return (uint16_t)(signbit(x) ? 0xFF80u : 0x7F80u);
+    if (x == 0.0) return (uint16_t)(signbit(x) ? 0x8000u : 0u);
+    int e;
+    (void)frexp(x, &e);       /* |x| = f * 2^e, f in [0.5, 1)  ->  floor(log2|x|) = e-1 */
+    int ex = e - 1;
+    if (ex < -126) ex = -126; /* subnormal range shares the quantum of the smallest normal binade */
+    int q = ex - 7;           /* bf16 keeps 7 fraction bits */
+    double r = nearbyint(ldexp(x, -q));
+    float f = (float)ldexp(r, q); /* exact, or +-inf past the largest finite bf16 */
+    uint32_t u;
+    memcpy(&u, &f, sizeof u);
+    return (uint16_t)(u >> 16);
+}
+
+uint16_t mzo_bf16_from_f32(float x) { return mzo_bf16_from_f64((double)x); }
+
+int32_t mzo_bf16_ord(uint16_t h) {
+    int32_t mag = (int32_t)(h & 0x7FFFu);
+    return (h & 0x8000u) ? -mag : mag;
+}
+
+static int is_nan16(uint16_t h) { return (h & 0x7FFFu) > 0x7F80u; }
+
+uint32_t mzo_bf16_ulp_distance(uint16_t a, uint16_t b) {
+    int na = is_nan16(a), nb = is_nan16(b);
+    if (na || nb) return (na && nb) ? 0u : 0xFFFFFFFFu;
+    int32_t d = mzo_bf16_ord(a) - mzo_bf16_ord(b);
+    return (uint32_t)(d < 0 ? -d : d);
+}
+
+/* ---- GEMM ---------------------------------------------------------------- */
+
+typedef struct {
+    const uint16_t* a;   /* M x K, this batch */
+    const float* bf;     /* K x N, logical B of this batch widened to float (exact) */
+    uint32_t n, k;
+    const uint32_t* rows; /* NULL: identity */
+    uint32_t r0, r1;      /* range of output rows handled by this worker */
+    uint16_t* c;          /* row r of the output is at c + r * ldc */
+    uint64_t ldc;
+    double* c_f64;        /* dense, leading dimension n, or NULL */
+    double* c_abs;
+} job_t;
+
+static void* worker(void* p) {
+    job_t* j = (job_t*)p;
+    const uint32_t n = j->n, k = j->k;
+    double* acc = (double*)malloc(sizeof(double) * n * 2);
+    double* aab = acc + n;
+    for (uint32_t r = j->r0; r < j->r1; ++r) {
+        const uint32_t row = j->rows ? j->rows[r] : r;
+        const uint16_t* arow = j->a + (size_t)row * k;
+        for (uint32_t x = 0; x < n; ++x) acc[x] = 0.0;
+        if (j->c_abs) {
+            for (uint32_t x = 0; x < n; ++x) aab[x] = 0.0;
+            for (uint32_t kk = 0; kk < k; ++kk) {
+                const double av = (double)mzo_bf16_to_f32(arow[kk]);
+                const double aa = fabs(av);
+                const float* brow = j->bf + (size_t)kk * n;
+                for (uint32_t x = 0; x < n; ++x) {
+                    const double bv = (double)brow[x];
+                    acc[x] += av * bv;          /* bf16 x bf16 is exact in fp64 */
+                    aab[x] += aa * fabs(bv);
+                }
+            }
+        } else {
+            for (uint32_t kk = 0; kk < k; ++kk) {
+                const double av = (double)mzo_bf16_to_f32(arow[kk]);
+                const float* brow = j->bf + (size_t)kk * n;
+                for (uint32_t x = 0; x < n; ++x) acc[x] += av * (double)brow[x];
+            }
+        }
+        if (j->c) {
+            uint16_t* crow = j->c + (size_t)r * j->ldc;
+            for (uint32_t x = 0; x < n; ++x) crow[x] = mzo_bf16_from_f64(acc[x]);
+        }
+        if (j->c_f64) memcpy(j->c_f64 + (size_t)r * n, acc, sizeof(double) * n);
+        if (j->c_abs) memcpy(j->c_abs + (size_t)r * n, aab, sizeof(double) * n);
+    }
+    free(acc);
+    return NULL;
+}
+
+/* Logical B (K x N) of one batch as floats. */
+static float* widen_b(const uint16_t* b, uint32_t n, uint32_t k, int layout) {
+    float* bf = (float*)malloc(sizeof(float) * (size_t)n * k);
+    if (!bf) return NULL;
+    if (layout == MZO_LAYOUT_NN) {
+        for (size_t i = 0; i < (size_t)n * k; ++i) bf[i] = mzo_bf16_to_f32(b[i]);
+    } else {
+        for (uint32_t x = 0; x < n; ++x)
+            for (uint32_t kk = 0; kk < k; ++kk)
+                bf[(size_t)kk * n + x] = mzo_bf16_to_f32(b[(size_t)x * k + kk]);
+    }
+    return bf;
+}
+
+static void run_rows(job_t base, uint32_t nrows, uint32_t nthreads) {
+    if (nthreads < 1) nthreads = 1;
+    if (nthreads > nrows) nthreads = nrows ? nrows : 1;
+    if (nthreads > 256) nthreads = 256;
+    if (nthreads == 1) {
+        base.r0 = 0;
+        base.r1 = nrows;
+        worker(&base);
+        return;
+    }
+    pthread_t th[256];
+    job_t jobs[256];
+    for (uint32_t t = 0; t < nthreads; ++t) {
+        jobs[t] = base;
+        jobs[t].r0 = (uint32_t)((uint64_t)nrows * t / nthreads);
+        jobs[t].r1 = (uint32_t)((uint64_t)nrows * (t + 1) / nthreads);
+        pthread_create(&th[t], NULL, worker, &jobs[t]);
+    }
+    for (uint32_t t = 0; t < nthreads; ++t) pthread_join(th[t], NULL);
+}
+
+int mzo_ref_gemm_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c,
+                      uint32_t m, uint32_t n, uint32_t k, int layout,
+                      uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                      uint64_t stride_c, double* c_f64, double* c_abs,
+                      uint32_t nthreads) {
+    if (!a || !b || !c || batch == 0) return -1;
+    if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
+    if (m == 0 || n == 0) return 0;
+    for (uint32_t bi = 0; bi < batch; ++bi) {
+        float* bf = widen_b(b + bi * stride_b, n, k, layout);
+        if (!bf) return -1;
+        job_t j;
+        memset(&j, 0, sizeof j);
+        j.a = a + bi * stride_a;
+        j.bf = bf;
+        j.n = n;
+        j.k = k;
+        j.rows = NULL;
+        j.c = c + bi * stride_c;
+        j.ldc = n;
+        j.c_f64 = c_f64 ? c_f64 + (size_t)bi * m * n : NULL;
+        j.c_abs = c_abs ? c_abs + (size_t)bi * m * n : NULL;
+        run_rows(j, m, nthreads);
+        free(bf);
+    }
+    return 0;
+}
+
+int mzo_ref_gemm_rows(const uint16_t* a, const uint16_t* b, uint32_t m,
+                      uint32_t n, uint32_t k, int layout, const uint32_t* rows,
+                      uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
+                      uint32_t nthreads) {
+    if (!a || !b || !rows) return -1;
+    if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
+    for (uint32_t r = 0; r < nsel; ++r)
+        if (rows[r] >= m) return -1;
+    if (n == 0 || nsel == 0) return 0;
+    float* bf = widen_b(b, n, k, layout);
+    if (!bf) return -1;
+    job_t j;
+    memset(&j, 0, sizeof j);
+    j.a = a;
+    j.bf = bf;
+    j.n = n;
+    j.k = k;
+    j.rows = rows;
+    j.c = c;
+    j.ldc = n;
+    j.c_f64 = c_f64;
+    j.c_abs = c_abs;
+    run_rows(j, nsel, nthreads);
+    free(bf);
+    return 0;
+}

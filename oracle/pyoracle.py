@@ -1,0 +1,143 @@
+"""ctypes wrapper of the CPU oracle (oracle/libmaize_oracle.so) plus the comparator.
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
+the cpu_baseline leg of bench.py, as the checker.  The product (maize_amd,
+libmaize_hip.so) never imports or links it.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmaize_oracle.so")
+
+NN, NT = 0, 1
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: run `make -C oracle`")
+        L = C.CDLL(LIB_PATH)
+        vp, u32, u64 = C.c_void_p, C.c_uint32, C.c_uint64
+        L.mzo_bf16_from_f64.restype = C.c_uint16
+        L.mzo_bf16_from_f64.argtypes = [C.c_double]
+        L.mzo_bf16_from_f32.restype = C.c_uint16
+        L.mzo_bf16_from_f32.argtypes = [C.c_float]
+        L.mzo_bf16_to_f32.restype = C.c_float
+        L.mzo_bf16_to_f32.argtypes = [C.c_uint16]
+        L.mzo_bf16_ord.restype = C.c_int32
+        L.mzo_bf16_ord.argtypes = [C.c_uint16]
+        L.mzo_bf16_ulp_distance.restype = u32
+        L.mzo_bf16_ulp_distance.argtypes = [C.c_uint16, C.c_uint16]
+        L.mzo_ref_gemm_bf16.restype = C.c_int
+        L.mzo_ref_gemm_bf16.argtypes = [vp, vp, vp, u32, u32, u32, C.c_int, u32, u64, u64, u64, vp, vp, u32]
+        L.mzo_ref_gemm_rows.restype = C.c_int
+        L.mzo_ref_gemm_rows.argtypes = [vp, vp, u32, u32, u32, C.c_int, vp, u32, vp, vp, vp, u32]
+        _lib = L
+    return _lib
+
+
+def default_threads():
+    return max(1, min(os.cpu_count() or 1, 16))
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data
+
+
+def ref_gemm(a, b, m, n, k, layout=NN, batch=1, stride_a=None, stride_b=None, stride_c=None,
+             want_f64=False, want_abs=False, nthreads=None):
+    """C (uint16, batch*stride_c elements) and optionally the fp64 sums / |a||b| sums (batch x M x N)."""
+    a = np.ascontiguousarray(a, dtype=np.uint16).ravel()
+    b = np.ascontiguousarray(b, dtype=np.uint16).ravel()
+    sa = m * k if stride_a is None else stride_a
+    sb = k * n if stride_b is None else stride_b
+    sc = m * n if stride_c is None else stride_c
+    assert a.size >= (batch - 1) * sa + m * k and b.size >= (batch - 1) * sb + k * n
+    c = np.zeros((batch - 1) * sc + m * n, dtype=np.uint16)
+    f64 = np.empty((batch, m, n), dtype=np.float64) if want_f64 else None
+    ab = np.empty((batch, m, n), dtype=np.float64) if want_abs else None
+    rc = lib().mzo_ref_gemm_bf16(_p(a), _p(b), _p(c), m, n, k, layout, batch, sa, sb, sc, _p(f64), _p(ab),
+                                 nthreads or default_threads())
+    if rc != 0:
+        raise ValueError("mzo_ref_gemm_bf16 rejected its arguments")
+    return c, f64, ab
+
+
+def ref_gemm_rows(a, b, m, n, k, rows, layout=NN, want_abs=True, nthreads=None):
+    """Rows ``rows`` of C = A.B for one batch: (bits nsel x N, f64 nsel x N, abs nsel x N)."""
+    a = np.ascontiguousarray(a, dtype=np.uint16).ravel()
+    b = np.ascontiguousarray(b, dtype=np.uint16).ravel()
+    rows = np.ascontiguousarray(rows, dtype=np.uint32)
+    nsel = rows.size
+    c = np.zeros((nsel, n), dtype=np.uint16)
+    f64 = np.empty((nsel, n), dtype=np.float64)
+    ab = np.empty((nsel, n), dtype=np.float64) if want_abs else None
+    rc = lib().mzo_ref_gemm_rows(_p(a), _p(b), m, n, k, layout, _p(rows), nsel, _p(c), _p(f64), _p(ab),
+                                 nthreads or default_threads())
+    if rc != 0:
+        raise ValueError("mzo_ref_gemm_rows rejected its arguments")
+    return c, f64, ab
+
+
+# ---- comparator -----------------------------------------------------------------
+
+def _ordinal(bits):
+    b = np.asarray(bits, dtype=np.uint16).astype(np.int64)
+    mag = b & 0x7FFF
+    return np.where(b & 0x8000, -mag, mag)
+
+
+def _isnan(bits):
+    return (np.asarray(bits, dtype=np.uint16) & 0x7FFF) > 0x7F80
+
+
+def floor_coeff(k):
+    """Relative size (to sum_k |a||b|) of the absolute-error floor granted to an
+    fp32-accumulating kernel: one fp32 rounding (2^-24) per 16-deep MFMA step of
+    the K loop, i.e. the deterministic worst case of sequential fp32 accumulation
+    of K/16 partial dot products, plus two for the final conversions."""
+    return (k / 16.0 + 2.0) * 2.0 ** -24
+
+
+def compare(got_bits, ref_bits, ref_f64, ref_abs, k):
+    """Compare device output with the oracle.
+
+    An element passes if it is within 1 bf16 ULP (ordinal distance) of the
+    oracle's bits, or -- for results that nearly cancel, where one bf16 ULP of
+    the tiny result is finer than fp32 accumulation can resolve -- if its
+    absolute error against the fp64 sum is at most floor_coeff(K) * sum|a||b|
+    plus half a bf16 ULP of the returned value.  Both counts are reported.
+    """
+    got = np.asarray(got_bits, dtype=np.uint16).ravel()
+    ref = np.asarray(ref_bits, dtype=np.uint16).ravel()
+    f64 = np.asarray(ref_f64, dtype=np.float64).ravel()
+    ab = np.asarray(ref_abs, dtype=np.float64).ravel()
+    assert got.size == ref.size == f64.size == ab.size
+    ng, nr = _isnan(got), _isnan(ref)
+    ulp = np.abs(_ordinal(got) - _ordinal(ref))
+    ulp = np.where(ng & nr, 0, ulp)
+    ulp = np.where(ng ^ nr, 2 ** 31, ulp)
+    gotf = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    with np.errstate(invalid="ignore", over="ignore"):
+        err = np.abs(gotf - f64)
+        half_ulp = np.abs(gotf) * 2.0 ** -8
+        floor = floor_coeff(k) * ab + half_ulp
+        strict_bad = ulp > 1
+        bad = strict_bad & ~(err <= floor)
+        rel = np.where(ab > 0, err / np.where(ab > 0, ab, 1.0), 0.0)
+    worst = int(np.argmax(ulp)) if ulp.size else -1
+    return {
+        "n": int(got.size),
+        "max_ulp": int(ulp.max()) if ulp.size else 0,
+        "n_gt1ulp": int(strict_bad.sum()),
+        "n_fail": int(bad.sum()),
+        "max_err_over_abs": float(rel.max()) if rel.size else 0.0,
+        "floor_coeff": floor_coeff(k),
+        "worst_index": worst,
+        "first_fail": int(np.argmax(bad)) if bad.any() else -1,
+    }

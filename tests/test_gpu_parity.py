@@ -1,0 +1,254 @@
+"""Parity of the HIP GEMM path (through the C ABI) with the CPU oracle.
+
+Bar: every element within 1 bf16 ULP of the oracle (fp64 accumulate, one RNE), except
+results that nearly cancel, where the absolute error must stay under
+floor_coeff(K) * sum_k|a||b| + half a bf16 ULP (oracle/pyoracle.py: compare); exact
+(bit-for-bit) for the closed-form cases, whose products and sums fp32 holds exactly.
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import maize_amd as mz
+from tests.gpu_util import run_gemm, check_against_oracle, check_rows_against_oracle, sample_rows, f32_of
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gemm_exact.npz")
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def kernels_for(desc_kwargs):
+    """Every kernel of the library that accepts the shape, plus None = the dispatcher's choice."""
+    m, n, k = desc_kwargs["m"], desc_kwargs["n"], desc_kwargs["k"]
+    layout = desc_kwargs.get("layout", mz.LAYOUT_NN)
+    batch = desc_kwargs.get("batch", 1)
+    a = mz.GlobalMatrix(0x1000, m, k)
+    b = mz.GlobalMatrix(0x1000, k, n) if layout == mz.LAYOUT_NN else mz.GlobalMatrix(0x1000, n, k)
+    c = mz.GlobalMatrix(0x1000, m, n)
+    d = mz.gemm_desc(a, b, c, layout=layout, batch=batch, stride_a=m * k, stride_b=k * n, stride_c=m * n)
+    return [None] + [name for name in mz.kernel_names() if mz.kernel_supports(name, d)]
+
+
+def inputs(m, n, k, batch=1, dist="uniform"):
+    if dist == "uniform":
+        return (mz.gen.uniform_bf16(batch * m * k, mz.gen.SEED_A), mz.gen.uniform_bf16(batch * k * n, mz.gen.SEED_B))
+    return (mz.gen.normal_bf16(batch * m * k, mz.gen.SEED_A, 1.0), mz.gen.normal_bf16(batch * k * n, mz.gen.SEED_B, 0.02))
+
+
+SMALL_SHAPES = [  # (m, n, k)
+    (1, 1, 1), (1, 7, 3), (5, 1, 9), (16, 16, 16), (31, 33, 17), (32, 32, 16), (33, 17, 65), (64, 64, 64),
+    (65, 63, 40), (100, 200, 72), (128, 128, 128), (129, 255, 136), (256, 256, 64), (256, 256, 256),
+    (257, 264, 320), (300, 520, 264), (16, 512, 256), (8, 1024, 512), (16, 264, 1000), (512, 256, 1024),
+]
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape", SMALL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_small_shapes_all_kernels(ctx, oracle, shape, layout):
+    m, n, k = shape
+    a, b = inputs(m, n, k)
+    for kern in kernels_for(dict(m=m, n=n, k=k, layout=layout)):
+        _say(f"parity: {m}x{n}x{k} layout={layout} kernel={kern}")
+        got = run_gemm(ctx, a, b, m, n, k, layout=layout, kernel=kern)
+        check_against_oracle(oracle, got, a, b, m, n, k, layout=layout, label=f"{shape} {layout} {kern}")
+
+
+def test_golden_exact_rational_cases(ctx):
+    z = np.load(GOLDEN)
+    names = sorted({key.split("/")[0] for key in z.files if not key.startswith("rne/")})
+    for name in names:
+        batch, m, n, k, nt = (int(v) for v in z[name + "/shape"])
+        if "subnormal" in name:
+            continue  # MFMA flushes bf16 subnormal inputs; the path makes no claim there
+        for kern in kernels_for(dict(m=m, n=n, k=k, layout=nt, batch=batch)):
+            _say(f"golden: {name} kernel={kern}")
+            got = run_gemm(ctx, z[name + "/a"], z[name + "/b"], m, n, k, layout=nt, batch=batch, kernel=kern)
+            d = mz.bf16.ulp_distance(got, z[name + "/c"])
+            assert d.max() <= 1, (name, kern, int(d.max()))
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+def test_closed_forms_are_bit_exact(ctx, layout):
+    rng = np.random.default_rng(21)
+    for n in (37, 256, 300):
+        x = (rng.integers(0, 2, n * n).astype(np.uint16) << 15) | (rng.integers(100, 140, n * n).astype(np.uint16) << 7) \
+            | rng.integers(0, 128, n * n).astype(np.uint16)
+        x = x.astype(np.uint16)
+        eye = np.where(np.eye(n, dtype=bool), 0x3F80, 0).astype(np.uint16).ravel()
+        perm = rng.permutation(n)
+        pm = np.zeros((n, n), dtype=np.uint16)
+        pm[np.arange(n), perm] = 0x3F80
+        xs = x if layout == mz.LAYOUT_NN else x.reshape(n, n).T.ravel()      # storage of logical B = x
+        for kern in kernels_for(dict(m=n, n=n, k=n, layout=layout)):
+            _say(f"closed forms: n={n} layout={layout} kernel={kern}")
+            assert np.array_equal(run_gemm(ctx, eye, xs, n, n, n, layout=layout, kernel=kern), x)       # I.B = B
+            assert np.array_equal(run_gemm(ctx, x, eye, n, n, n, layout=layout, kernel=kern), x)        # A.I = A
+            got = run_gemm(ctx, pm.ravel(), xs, n, n, n, layout=layout, kernel=kern).reshape(n, n)
+            assert np.array_equal(got, x.reshape(n, n)[perm])                                           # row routing
+    for k, want in ((1, 1.0), (256, 256.0), (257, 256.0), (259, 260.0), (4096, 4096.0)):
+        ones_a = np.full(40 * k, 0x3F80, dtype=np.uint16)
+        ones_b = np.full(k * 72, 0x3F80, dtype=np.uint16)
+        for kern in kernels_for(dict(m=40, n=72, k=k, layout=layout)):
+            c = run_gemm(ctx, ones_a, ones_b, 40, 72, k, layout=layout, kernel=kern)
+            assert np.all(f32_of(c) == want), (k, kern)
+
+
+def test_one_hot_routing_every_position(ctx):
+    """A single 1 at A[i,k] and B[k,j] puts a single 1 at C[i,j]: catches any tile/lane index slip."""
+    m, n, k = 70, 90, 50
+    rng = np.random.default_rng(22)
+    for kern in kernels_for(dict(m=m, n=n, k=k)):
+        for _ in range(12):
+            i, j, kk = int(rng.integers(m)), int(rng.integers(n)), int(rng.integers(k))
+            a = np.zeros((m, k), dtype=np.uint16); a[i, kk] = 0x3F80
+            b = np.zeros((k, n), dtype=np.uint16); b[kk, j] = 0x4000
+            c = run_gemm(ctx, a, b, m, n, k, kernel=kern).reshape(m, n)
+            want = np.zeros((m, n), dtype=np.uint16); want[i, j] = 0x4000
+            assert np.array_equal(c, want), (kern, i, j, kk)
+
+
+def test_nt_equals_nn_bit_for_bit(ctx):
+    m, n, k = 200, 136, 328
+    a, b = inputs(m, n, k)
+    bt = b.reshape(k, n).T.ravel()
+    for kern in kernels_for(dict(m=m, n=n, k=k)):
+        c_nn = run_gemm(ctx, a, b, m, n, k, kernel=kern)
+        c_nt = run_gemm(ctx, a, bt, m, n, k, layout=mz.LAYOUT_NT, kernel=kern)
+        assert np.array_equal(c_nn, c_nt), kern
+
+
+def test_ragged_equals_block_of_zero_padded(ctx):
+    m, n, k = 200, 264, 136
+    M, N, K = 256, 512, 192
+    a, b = inputs(m, n, k)
+    ap = np.zeros((M, K), dtype=np.uint16); ap[:m, :k] = a.reshape(m, k)
+    bp = np.zeros((K, N), dtype=np.uint16); bp[:k, :n] = b.reshape(k, n)
+    small = run_gemm(ctx, a, b, m, n, k).reshape(m, n)
+    big = run_gemm(ctx, ap, bp, M, N, K).reshape(M, N)
+    assert np.array_equal(small, big[:m, :n])
+    assert not (big[m:, :] & 0x7FFF).any() and not (big[:, n:] & 0x7FFF).any()
+
+
+def test_batched_equals_loop_of_singles_and_respects_strides(ctx, oracle):
+    m, n, k, batch = 96, 136, 72, 5
+    a, b = inputs(m, n, k, batch=batch)
+    sa, sb, sc = m * k + 8, k * n + 24, m * n + 40
+    ap = np.zeros(batch * sa, dtype=np.uint16)
+    bp = np.zeros(batch * sb, dtype=np.uint16)
+    for i in range(batch):
+        ap[i * sa:i * sa + m * k] = a[i * m * k:(i + 1) * m * k]
+        bp[i * sb:i * sb + k * n] = b[i * k * n:(i + 1) * k * n]
+    for kern in kernels_for(dict(m=m, n=n, k=k, batch=batch)):
+        _say(f"batched: kernel={kern}")
+        dense = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel=kern)
+        check_against_oracle(oracle, dense, a, b, m, n, k, batch=batch, label=f"batched {kern}")
+        strided = run_gemm(ctx, ap, bp, m, n, k, batch=batch, stride_a=sa, stride_b=sb, stride_c=sc, kernel=kern)
+        for i in range(batch):
+            single = run_gemm(ctx, a[i * m * k:(i + 1) * m * k], b[i * k * n:(i + 1) * k * n], m, n, k, kernel=kern)
+            assert np.array_equal(single, dense[i * m * n:(i + 1) * m * n])
+            assert np.array_equal(single, strided[i * sc:i * sc + m * n])
+
+
+def test_misaligned_pointers_fall_back_and_stay_correct(ctx, oracle):
+    """2-byte-aligned (not 16-byte-aligned) operands must still give the right answer."""
+    m, n, k = 130, 264, 200
+    a, b = inputs(m, n, k)
+    da, db = ctx.upload(np.concatenate([[0], a]).astype(np.uint16)), ctx.upload(np.concatenate([[0, 0, 0], b]).astype(np.uint16))
+    dc = ctx.malloc((m * n + 16) * 2)
+    desc = mz.gemm_desc(mz.Matrix(da, m, k, offset_elems=1), mz.Matrix(db, k, n, offset_elems=3),
+                        mz.Matrix(dc, m, n, offset_elems=5))
+    ctx.gemm_bf16(desc)
+    ctx.sync()
+    got = dc.download(np.uint16)[5:5 + m * n]
+    check_against_oracle(oracle, got, a, b, m, n, k, label="misaligned")
+    for x in (da, db, dc):
+        x.free()
+
+
+def test_launch_on_a_user_stream(ctx, oracle):
+    m, n, k = 64, 128, 96
+    a, b = inputs(m, n, k)
+    s = ctx.stream()
+    got = run_gemm(ctx, a, b, m, n, k, stream=s)
+    ctx.stream_destroy(s)
+    check_against_oracle(oracle, got, a, b, m, n, k, label="stream")
+
+
+def test_builder_chain_launches_the_kernel(ctx, oracle):
+    """new_hip_kernel(..).with_launch_bounds_2d(..).finalize().compile(Gfx950) -> launch with a hand-packed
+    parameter block: the reference's builder flow carried through to a launch."""
+    from maize_amd import _ffi
+    m, n, k = 64, 64, 48
+    a, b = inputs(m, n, k)
+    da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(m * n * 2)
+    kern = mz.new_hip_kernel("maize_gemm_bf16_wave32").with_launch_bounds_2d((256, 1)).finalize().compile(mz.Gfx.Gfx950, ctx)
+    args = _ffi.GemmArgsT(da.ptr, m, k, db.ptr, k, n, dc.ptr, m, n, 0, 0, 0, 1, 0)
+    kern.launch((1, 1, 1), args)
+    ctx.sync()
+    got = dc.download(np.uint16)
+    kern.release()
+    check_against_oracle(oracle, got, a, b, m, n, k, label="builder chain")
+    for x in (da, db, dc):
+        x.free()
+
+
+# ---- the five benchmark configurations at full size (sampled rows + invariants) ---------
+
+def _full_size(ctx, oracle, m, n, k, layout, dist, label, sigma_b=None):
+    if dist == "uniform":
+        a, b = mz.gen.uniform_bf16(m * k, mz.gen.SEED_A), mz.gen.uniform_bf16(k * n, mz.gen.SEED_B)
+    elif dist == "normal_scaled":
+        s = mz.gen.SIGMA_INV_SQRT_8192
+        a, b = mz.gen.normal_bf16(m * k, mz.gen.SEED_A, s), mz.gen.normal_bf16(k * n, mz.gen.SEED_B, s)
+    else:
+        a, b = mz.gen.normal_bf16(m * k, mz.gen.SEED_A, 1.0), mz.gen.normal_bf16(k * n, mz.gen.SEED_B, 0.02)
+    bs = b if layout == mz.LAYOUT_NN else b.reshape(k, n).T.copy().ravel()    # logical B is the same in both layouts
+    _say(f"full size: {label} launching")
+    got = run_gemm(ctx, a, bs, m, n, k, layout=layout)
+    rows = sample_rows(m, count=24)
+    _say(f"full size: {label} checking {rows.size} rows on the CPU")
+    s = check_rows_against_oracle(oracle, got, a, bs, m, n, k, rows, layout=layout, label=label)
+    _say(f"full size: {label} {s}")
+    return got, a, b
+
+
+def test_config1_4096_cubed(ctx, oracle):
+    _full_size(ctx, oracle, 4096, 4096, 4096, mz.LAYOUT_NN, "uniform", "cfg1 4096^3 NN")
+
+
+def test_config2_ragged(ctx, oracle):
+    _full_size(ctx, oracle, 4000, 4104, 4032, mz.LAYOUT_NN, "uniform", "cfg2 4000x4104x4032 NN")
+
+
+def test_config3_8192_cubed_nt(ctx, oracle):
+    _full_size(ctx, oracle, 8192, 8192, 8192, mz.LAYOUT_NT, "normal_scaled", "cfg3 8192^3 NT")
+
+
+def test_config4_skinny(ctx, oracle):
+    m, n, k = 16, 14336, 4096
+    a, b = mz.gen.normal_bf16(m * k, mz.gen.SEED_A, 1.0), mz.gen.normal_bf16(k * n, mz.gen.SEED_B, 0.02)
+    got = run_gemm(ctx, a, b, m, n, k)
+    s = check_against_oracle(oracle, got, a, b, m, n, k, label="cfg4 skinny")
+    _say(f"full size: cfg4 {s}")
+
+
+def test_config5_batched(ctx, oracle):
+    m = n = k = 2048
+    batch = 32
+    a, b = mz.gen.uniform_bf16(batch * m * k, mz.gen.SEED_A), mz.gen.uniform_bf16(batch * k * n, mz.gen.SEED_B)
+    _say("full size: cfg5 launching")
+    got = run_gemm(ctx, a, b, m, n, k, batch=batch, stride_a=m * k, stride_b=k * n, stride_c=m * n)
+    rows = sample_rows(m, count=6)[:12]
+    for bi in (0, 13, 31):
+        s = check_rows_against_oracle(oracle, got[bi * m * n:(bi + 1) * m * n], a[bi * m * k:(bi + 1) * m * k],
+                                      b[bi * k * n:(bi + 1) * k * n], m, n, k, rows, label=f"cfg5 batch {bi}")
+        _say(f"full size: cfg5 batch {bi} {s}")
+    # one launch covers every batch member: a single launch equals the per-member launch bit for bit
+    single = run_gemm(ctx, a[7 * m * k:8 * m * k], b[7 * k * n:8 * k * n], m, n, k)
+    assert np.array_equal(single, got[7 * m * n:8 * m * n])

@@ -1,0 +1,227 @@
+"""Pins the CPU oracle (oracle/maize_oracle.c) without a GPU.
+
+The reference holds no golden vector, known-answer test or fixture for its GEMM
+path (its kernel stores no C), so the oracle is pinned by what the mathematics
+fixes: exact-rational golden cases (tests/golden/gemm_exact.npz), bf16 rounding
+known answers and exhaustive round trips, closed forms (identity, permutation,
+all-ones, powers of two), and numpy float64 matmul on the same bit patterns.
+"""
+import math
+import os
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gemm_exact.npz")
+
+
+def f32_of(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def rand_bits(rng, count, emin=118, emax=127):
+    sign = rng.integers(0, 2, count).astype(np.uint16) << 15
+    e = rng.integers(emin, emax + 1, count).astype(np.uint16) << 7
+    m = rng.integers(0, 128, count).astype(np.uint16)
+    return (sign | e | m).astype(np.uint16)
+
+
+# ---- bf16 rounding ---------------------------------------------------------------
+
+def test_rne_known_answers(oracle):
+    L = oracle.lib()
+    f = L.mzo_bf16_from_f64
+    assert f(1.0) == 0x3F80
+    assert f(1.0 + 2.0 ** -8) == 0x3F80            # tie -> even (down)
+    assert f(1.0 + 3 * 2.0 ** -8) == 0x3F82        # tie -> even (up)
+    assert f(1.0 + 2.0 ** -8 + 2.0 ** -20) == 0x3F81
+    assert f(1.0 + 2.0 ** -8 - 2.0 ** -40) == 0x3F80  # only visible without an intermediate fp32 rounding
+    assert f(-1.0) == 0xBF80
+    assert f(0.0) == 0x0000 and f(-0.0) == 0x8000
+    assert f(float("inf")) == 0x7F80 and f(float("-inf")) == 0xFF80
+    assert (f(float("nan")) & 0x7FFF) > 0x7F80
+    max_finite = float(f32_of([0x7F7F])[0])
+    assert f(max_finite) == 0x7F7F
+    assert f(max_finite + 2.0 ** 119) == 0x7F80   # half a quantum above the largest finite: tie -> inf
+    assert f(max_finite + 2.0 ** 118) == 0x7F7F
+    assert f(2.0 ** -133) == 0x0001                    # smallest subnormal
+    assert f(2.0 ** -134) == 0x0000                    # tie -> even (zero)
+    assert f(3 * 2.0 ** -135) == 0x0001
+    assert f(2.0 ** -126) == 0x0080                    # smallest normal
+    assert f((127.5) * 2.0 ** -133) == 0x0080          # subnormal tie rounds up into the normal range
+
+
+def test_rne_golden_exact_rationals(oracle):
+    z = np.load(GOLDEN)
+    for (num, den), bits in zip(z["rne/num_log2den"], z["rne/bits"]):
+        x = math.ldexp(num, -int(den))
+        assert oracle.lib().mzo_bf16_from_f64(x) == int(bits), (num, den)
+
+
+def test_rne_exhaustive_round_trip_and_midpoints(oracle):
+    L = oracle.lib()
+    enc = np.arange(0x0000, 0x7F80, dtype=np.uint16)  # all non-negative finite encodings
+    vals = f32_of(enc).astype(np.float64)
+    for h, v in zip(enc[::7], vals[::7]):             # every 7th: ~4.6k values, all binades
+        assert L.mzo_bf16_from_f64(float(v)) == int(h)
+        assert L.mzo_bf16_from_f64(float(-v)) == (int(h) | 0x8000)
+    # exact midpoints between neighbours go to the even encoding
+    for i in range(0, len(enc) - 1, 5):
+        mid = (vals[i] + vals[i + 1]) / 2.0           # exact in fp64
+        want = int(enc[i]) if enc[i] % 2 == 0 else int(enc[i + 1])
+        assert L.mzo_bf16_from_f64(float(mid)) == want
+        assert L.mzo_bf16_from_f64(float(np.nextafter(mid, np.inf))) == int(enc[i + 1])
+        assert L.mzo_bf16_from_f64(float(np.nextafter(mid, -np.inf))) == int(enc[i])
+
+
+def test_rne_matches_exact_fraction_rounding_on_random_doubles(oracle):
+    from tests.golden.make_golden import fraction_to_bf16_rne
+    rng = np.random.default_rng(1)
+    xs = rng.standard_normal(400) * np.exp2(rng.integers(-30, 30, 400))
+    for x in xs:
+        assert oracle.lib().mzo_bf16_from_f64(float(x)) == fraction_to_bf16_rne(Fraction(float(x)))
+
+
+def test_to_f32_exact(oracle):
+    for h in (0x0000, 0x8000, 0x3F80, 0xBF80, 0x0001, 0x7F7F, 0x4049):
+        assert oracle.lib().mzo_bf16_to_f32(h) == float(f32_of([h])[0])
+
+
+# ---- ULP distance ------------------------------------------------------------------
+
+def test_ulp_distance_properties(oracle):
+    d = oracle.lib().mzo_bf16_ulp_distance
+    assert d(0x3F80, 0x3F80) == 0
+    assert d(0x0000, 0x8000) == 0                      # +0 vs -0
+    assert d(0x3F80, 0x3F81) == 1 and d(0x3F81, 0x3F80) == 1
+    assert d(0x0001, 0x8001) == 2                      # across zero
+    assert d(0x3F7F, 0x3F80) == 1                      # across a binade
+    assert d(0x7FC0, 0x7FC1) == 0                      # both NaN
+    assert d(0x7FC0, 0x3F80) == 0xFFFFFFFF
+    rng = np.random.default_rng(2)
+    for a, b in rng.integers(0, 0x7F80, (200, 2)):
+        assert d(int(a), int(b)) == d(int(b), int(a)) == abs(int(a) - int(b))
+
+
+# ---- GEMM vs exact arithmetic ------------------------------------------------------
+
+def _golden_cases():
+    z = np.load(GOLDEN)
+    names = sorted({k.split("/")[0] for k in z.files if not k.startswith("rne/")})
+    return z, names
+
+
+def test_gemm_matches_exact_rational_golden(oracle):
+    z, names = _golden_cases()
+    assert len(names) == 10
+    for name in names:
+        batch, m, n, k, nt = (int(v) for v in z[name + "/shape"])
+        c, _, _ = oracle.ref_gemm(z[name + "/a"], z[name + "/b"], m, n, k, layout=nt, batch=batch, nthreads=1)
+        assert np.array_equal(c, z[name + "/c"]), name
+
+
+def test_gemm_vs_numpy_float64(oracle):
+    rng = np.random.default_rng(3)
+    m, n, k = 48, 40, 160
+    a, b = rand_bits(rng, m * k), rand_bits(rng, k * n)
+    c, f64, ab = oracle.ref_gemm(a, b, m, n, k, want_f64=True, want_abs=True)
+    A = f32_of(a).astype(np.float64).reshape(m, k)
+    B = f32_of(b).astype(np.float64).reshape(k, n)
+    np.testing.assert_allclose(f64[0], A @ B, rtol=0, atol=1e-12 * float(ab.max()))
+    np.testing.assert_allclose(ab[0], np.abs(A) @ np.abs(B), rtol=1e-13)
+    # the bits are one RNE of the fp64 sums (independent numpy rounding of the same sums)
+    import maize_amd.bf16 as hb
+    f32 = f64[0].astype(np.float32)
+    exact32 = f32.astype(np.float64) == f64[0]         # only where fp32 holds the sum exactly is this a single rounding
+    assert exact32.sum() >= 5
+    assert np.array_equal(hb.from_f32(f32)[exact32], c.reshape(m, n)[exact32])
+
+
+def test_gemm_closed_forms(oracle):
+    rng = np.random.default_rng(4)
+    n = 37
+    x = rand_bits(rng, n * n, 100, 140)
+    eye = np.where(np.eye(n, dtype=bool), 0x3F80, 0).astype(np.uint16).ravel()
+    assert np.array_equal(oracle.ref_gemm(eye, x, n, n, n)[0], x)          # I.B = B
+    assert np.array_equal(oracle.ref_gemm(x, eye, n, n, n)[0], x)          # A.I = A
+    perm = rng.permutation(n)
+    pm = np.zeros((n, n), dtype=np.uint16)
+    pm[np.arange(n), perm] = 0x3F80                                         # row i picks row perm[i] of B
+    assert np.array_equal(oracle.ref_gemm(pm.ravel(), x, n, n, n)[0].reshape(n, n), x.reshape(n, n)[perm])
+    # all-ones: C = K, rounded: 256 exact, 257 -> 256 (tie to even), 259 -> 260, 4096 exact
+    for k, want in ((1, 1.0), (256, 256.0), (257, 256.0), (259, 260.0), (4096, 4096.0)):
+        ones_a = np.full(3 * k, 0x3F80, dtype=np.uint16)
+        ones_b = np.full(k * 5, 0x3F80, dtype=np.uint16)
+        c = oracle.ref_gemm(ones_a, ones_b, 3, 5, k)[0]
+        assert np.all(f32_of(c) == want), k
+    # powers of two: every product and the sum are exact
+    a = np.array([0x4000, 0x3F00, 0xC080], dtype=np.uint16)                 # 2, 0.5, -4
+    b = np.array([0x4080, 0x4100, 0x3E80], dtype=np.uint16)                 # 4, 8, 0.25
+    assert f32_of(oracle.ref_gemm(a, b, 1, 1, 3)[0])[0] == 2 * 4 + 0.5 * 8 - 4 * 0.25
+
+
+def test_gemm_layout_batch_rows_identities(oracle):
+    rng = np.random.default_rng(5)
+    m, n, k, batch = 19, 23, 71, 3
+    a, b = rand_bits(rng, batch * m * k), rand_bits(rng, batch * k * n)
+    c_nn = oracle.ref_gemm(a, b, m, n, k, batch=batch)[0]
+    bt = np.concatenate([b[i * k * n:(i + 1) * k * n].reshape(k, n).T.ravel() for i in range(batch)])
+    c_nt = oracle.ref_gemm(a, bt, m, n, k, layout=oracle.NT, batch=batch)[0]
+    assert np.array_equal(c_nn, c_nt)                                       # NT(B^T stored) == NN(B)
+    for i in range(batch):                                                  # batched == loop of singles
+        single = oracle.ref_gemm(a[i * m * k:(i + 1) * m * k], b[i * k * n:(i + 1) * k * n], m, n, k)[0]
+        assert np.array_equal(single, c_nn[i * m * n:(i + 1) * m * n])
+    # padded batch strides
+    sa, sb, sc = m * k + 5, k * n + 3, m * n + 7
+    ap = np.zeros(batch * sa, dtype=np.uint16)
+    bp = np.zeros(batch * sb, dtype=np.uint16)
+    for i in range(batch):
+        ap[i * sa:i * sa + m * k] = a[i * m * k:(i + 1) * m * k]
+        bp[i * sb:i * sb + k * n] = b[i * k * n:(i + 1) * k * n]
+    cp = oracle.ref_gemm(ap, bp, m, n, k, batch=batch, stride_a=sa, stride_b=sb, stride_c=sc)[0]
+    for i in range(batch):
+        assert np.array_equal(cp[i * sc:i * sc + m * n], c_nn[i * m * n:(i + 1) * m * n])
+    # row subset == rows of the full result; threads do not change bits
+    rows = np.array([0, 7, 18, 7], dtype=np.uint32)
+    full, f64, ab = oracle.ref_gemm(a[:m * k], b[:k * n], m, n, k, want_f64=True, want_abs=True, nthreads=1)
+    cr, fr, ar = oracle.ref_gemm_rows(a[:m * k], b[:k * n], m, n, k, rows, nthreads=4)
+    assert np.array_equal(cr, full.reshape(m, n)[rows])
+    assert np.array_equal(fr, f64[0][rows]) and np.array_equal(ar, ab[0][rows])
+    cr_nt, _, _ = oracle.ref_gemm_rows(a[:m * k], bt[:k * n], m, n, k, rows, layout=oracle.NT)
+    assert np.array_equal(cr_nt, cr)
+
+
+def test_gemm_ragged_equals_block_of_zero_padded(oracle):
+    rng = np.random.default_rng(6)
+    m, n, k = 13, 11, 29
+    M, N, K = 16, 16, 32
+    a, b = rand_bits(rng, m * k).reshape(m, k), rand_bits(rng, k * n).reshape(k, n)
+    ap = np.zeros((M, K), dtype=np.uint16)
+    bp = np.zeros((K, N), dtype=np.uint16)
+    ap[:m, :k], bp[:k, :n] = a, b
+    small = oracle.ref_gemm(a.ravel(), b.ravel(), m, n, k)[0].reshape(m, n)
+    big = oracle.ref_gemm(ap.ravel(), bp.ravel(), M, N, K)[0].reshape(M, N)
+    assert np.array_equal(small, big[:m, :n])
+    assert not big[m:, :].any() and not big[:, n:].any()
+
+
+def test_gemm_rejects_bad_arguments(oracle):
+    a = np.zeros(4, dtype=np.uint16)
+    with pytest.raises(ValueError):
+        oracle.ref_gemm(a, a, 2, 2, 2, layout=7)
+    with pytest.raises(ValueError):
+        oracle.ref_gemm_rows(a, a, 2, 2, 2, np.array([2], dtype=np.uint32))
+
+
+def test_comparator_flags_and_floors(oracle):
+    k = 4096
+    ref_bits = np.array([0x3F80, 0x3F80, 0x3F80, 0x3000, 0x7FC0, 0x3F80], dtype=np.uint16)
+    ref64 = f32_of(ref_bits).astype(np.float64)
+    ref64[4] = np.nan
+    ab = np.array([10.0, 10.0, 10.0, 1000.0, 1.0, 1.0])
+    got = np.array([0x3F80, 0x3F81, 0x3F83, 0x3003, 0x7FC1, 0x7FC0], dtype=np.uint16)
+    s = oracle.compare(got, ref_bits, ref64, ab, k)
+    # 0x3F83 is 3 ULP off a large value -> fail; 0x3003 is 3 ULP off a tiny value under the floor -> counted, not failed
+    assert s["n_gt1ulp"] == 3 and s["n_fail"] == 2 and s["max_ulp"] == 2 ** 31
+    assert oracle.floor_coeff(k) == (k / 16 + 2) * 2.0 ** -24
