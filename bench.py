@@ -1,0 +1,177 @@
+#!/usr/bin/env python3
+"""Benchmark of the BF16 GEMM path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5] [--kernel NAME]
+
+A step is one launch of maize_hip_gemm_bf16 on synthetic, seeded inputs that are already
+resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s (wall clock around exactly K
+steps), the roofline object of the kernel (HIP events on the launch stream) and the CPU
+oracle timed on a bounded slab of the same problem on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+
+# name -> (M, N, K, layout, batch, A distribution, B distribution, bound)
+CONFIGS = {
+    "cfg1": dict(m=4096, n=4096, k=4096, nt=0, batch=1, da=("uniform",), db=("uniform",), bound="mfma",
+                 label="bf16 GEMM 4096x4096x4096 NN, uniform[-1,1)"),
+    "cfg2": dict(m=4000, n=4104, k=4032, nt=0, batch=1, da=("uniform",), db=("uniform",), bound="mfma",
+                 label="bf16 GEMM 4000x4104x4032 NN ragged, uniform[-1,1)"),
+    "cfg3": dict(m=8192, n=8192, k=8192, nt=1, batch=1, da=("normal", "inv_sqrt_k"), db=("normal", "inv_sqrt_k"),
+                 bound="mfma", label="bf16 GEMM 8192x8192x8192 NT, N(0,1)/sqrt(K)"),
+    "cfg4": dict(m=16, n=14336, k=4096, nt=0, batch=1, da=("normal", 1.0), db=("normal", 0.02), bound="hbm",
+                 label="bf16 GEMM 16x14336x4096 NN skinny, A~N(0,1), B~N(0,0.02)"),
+    "cfg5": dict(m=2048, n=2048, k=2048, nt=0, batch=32, da=("uniform",), db=("uniform",), bound="mfma",
+                 label="bf16 strided-batched GEMM 32 x 2048^3 NN, uniform[-1,1)"),
+}
+
+
+def make(mz, dist, count, seed):
+    if dist[0] == "uniform":
+        return mz.gen.uniform_bf16(count, seed)
+    sigma = mz.gen.SIGMA_INV_SQRT_8192 if dist[1] == "inv_sqrt_k" else dist[1]
+    return mz.gen.normal_bf16(count, seed, sigma)
+
+
+def cpu_baseline(cfg, a, b_storage, got, seconds_target=12.0):
+    """Times the CPU oracle (fp64 accumulate, one RNE) on the first R rows of batch 0 and
+    uses the same rows to check the device result.  The oracle is only the checker and
+    the reported baseline here; it is never on the measured GPU path."""
+    from oracle import pyoracle
+    m, n, k = cfg["m"], cfg["n"], cfg["k"]
+    threads = pyoracle.default_threads()
+    probe_rows = min(m, 4)
+    t0 = time.perf_counter()
+    pyoracle.ref_gemm_rows(a[:m * k], b_storage[:k * n], m, n, k, np.arange(probe_rows, dtype=np.uint32),
+                           layout=cfg["nt"], want_abs=False, nthreads=1)
+    per_row = max((time.perf_counter() - t0) / probe_rows, 1e-6)
+    rows = int(min(m, max(threads, seconds_target * threads / per_row)))
+    rows = max(1, (rows // threads) * threads) if rows >= threads else rows
+    sel = np.arange(rows, dtype=np.uint32)
+    t0 = time.perf_counter()
+    ref, f64, _ = pyoracle.ref_gemm_rows(a[:m * k], b_storage[:k * n], m, n, k, sel, layout=cfg["nt"], want_abs=False,
+                                         nthreads=threads)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * rows * n * k
+    out = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+           "sample": f"rows 0..{rows - 1} of batch 0 ({rows}x{n}x{k}, {flops / 1e9:.1f} GFLOP, {dt:.1f} s), "
+                     f"fp64 accumulate + one RNE to bf16, {threads} POSIX threads"}
+    parity = None
+    if got is not None:
+        _, _, ab = pyoracle.ref_gemm_rows(a[:m * k], b_storage[:k * n], m, n, k, sel[:min(rows, 64)], layout=cfg["nt"],
+                                          nthreads=threads)
+        r = min(rows, 64)
+        parity = pyoracle.compare(got[:r * n], ref[:r], f64[:r], ab, k)
+        parity = {key: parity[key] for key in ("n", "max_ulp", "n_gt1ulp", "n_fail", "max_err_over_abs")}
+    return out, parity
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="cfg1", choices=sorted(CONFIGS))
+    ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--rotate", type=int, default=0,
+                    help="number of distinct operand sets cycled through (0: enough to exceed the 256 MiB "
+                         "last-level cache for the HBM-bound config, 1 otherwise)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only (independent output tiles need no exchange step; "
+              "every box here has one GPU) -- run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import maize_amd as mz
+    cfg = CONFIGS[args.config]
+    m, n, k, batch, nt = cfg["m"], cfg["n"], cfg["k"], cfg["batch"], cfg["nt"]
+    flops = 2.0 * batch * m * n * k
+    alg_bytes = 2.0 * batch * (m * k + k * n + m * n)
+
+    a = make(mz, cfg["da"], batch * m * k, mz.gen.SEED_A)
+    b = make(mz, cfg["db"], batch * k * n, mz.gen.SEED_B)
+    if nt:  # same logical B, stored N x K
+        b = np.concatenate([b[i * k * n:(i + 1) * k * n].reshape(k, n).T.ravel() for i in range(batch)])
+
+    ctx = mz.Context(0)
+    info = ctx.info()
+    nsets = args.rotate or (max(2, int(np.ceil(3 * 256 * 2 ** 20 / alg_bytes))) if cfg["bound"] == "hbm" else 1)
+    sets = []
+    for _ in range(nsets):
+        da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(2 * batch * m * n)
+        A = mz.Matrix(da, m, k)
+        B = mz.Matrix(db, n, k) if nt else mz.Matrix(db, k, n)
+        desc = mz.gemm_desc(A, B, mz.Matrix(dc, m, n), layout=nt, batch=batch, stride_a=m * k, stride_b=k * n,
+                            stride_c=m * n)
+        sets.append((da, db, dc, desc))
+    kernel = args.kernel or ctx.gemm_select(sets[0][3])
+    stream = ctx.stream()
+    ev0, ev1 = ctx.event(), ctx.event()
+
+    for i in range(args.warmup):
+        ctx.gemm_bf16(sets[i % nsets][3], stream=stream, kernel=args.kernel)
+    ctx.sync()
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for i in range(args.steps):
+        ctx.gemm_bf16(sets[i % nsets][3], stream=stream, kernel=args.kernel)
+    ev1.record(stream)
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    ev_ms = ev0.elapsed_ms(ev1)
+
+    got = sets[(args.steps - 1) % nsets][2].download(np.uint16, count=m * n)
+    ms_per_step = wall * 1e3 / args.steps
+    kern_ms = ev_ms / args.steps
+    value = flops / (wall / args.steps) / 1e12
+    if cfg["bound"] == "mfma":
+        ach = flops / (kern_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None}
+    else:
+        ach = alg_bytes / (kern_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
+                "traffic": None}
+    roof["kernel"] = kernel
+    roof["kernel_avg_us"] = kern_ms * 1e3
+    roof["algorithmic_flop"] = flops
+    roof["algorithmic_bytes"] = alg_bytes
+
+    cpu, parity = (None, None)
+    if not args.no_cpu:
+        cpu, parity = cpu_baseline(cfg, a, b, got)
+
+    line = {
+        "metric": "bf16 GEMM TFLOP/s at 4096^3 on 1 MI355X" if args.config == "cfg1" else f"bf16 GEMM TFLOP/s, {args.config}",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (seeded counter-based generators, inputs resident in HBM)",
+        "config": {"workload": cfg["label"], "M": m, "N": n, "K": k, "batch": batch, "layout": "NT" if nt else "NN",
+                   "accumulate": "fp32", "output": "bf16", "operand_sets_cycled": nsets},
+        "pct_of_mfma_bf16_peak": 100.0 * flops / (wall / args.steps) / 1e12 / PEAK_BF16_TFLOPS,
+        "roofline": roof, "cpu_baseline": cpu, "parity_vs_oracle": parity,
+        "device": {"name": info["name"], "compute_units": info["compute_units"], "clock_khz": info["clock_khz"]},
+    }
+    print(json.dumps(line), flush=True)
+    for da, db, dc, _ in sets:
+        da.free(); db.free(); dc.free()
+    ev0.destroy(); ev1.destroy()
+    ctx.stream_destroy(stream)
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

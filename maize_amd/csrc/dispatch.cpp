@@ -1,5 +1,6 @@
 #include "dispatch.hpp"
 
+#include <cstdint>
 #include <cstring>
 
 namespace maize {
@@ -19,8 +20,41 @@ bool wave32_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
     return ld->grid[1] <= 65535u && ld->grid[2] <= 65535u;
 }
 
+// ---- maize_gemm_bf16_mt256_{nn,nt}: 256 x 256 x 64 macro-tile pipeline -------
+// 128-bit loads and stores: K % 8 == 0 (A rows, and B rows when NT), N % 8 == 0
+// (C rows, and B rows when NN), 16-byte aligned bases and batch strides.
+// 32-bit buffer offsets: every matrix of one batch member stays below 2 GiB.
+bool aligned16(const maize_gemm_desc_t& d) {
+    if (((uintptr_t)d.a.ptr | (uintptr_t)d.b.ptr | (uintptr_t)d.c.ptr) & 15u) return false;
+    if (d.batch > 1 && ((d.stride_a | d.stride_b | d.stride_c) & 7u)) return false;
+    return true;
+}
+bool mt256_common(const maize_gemm_desc_t& d) {
+    const Dims s = dims_of(d);
+    if ((s.k & 7u) || (s.n & 7u) || !aligned16(d)) return false;
+    const uint64_t lim = 1ull << 31;
+    if ((uint64_t)s.m * s.k * 2 >= lim || (uint64_t)s.n * s.k * 2 >= lim || (uint64_t)s.m * s.n * 2 >= lim) return false;
+    if (s.k >= (1u << 21) || s.n >= (1u << 21)) return false;
+    return true;
+}
+bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
+bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
+bool mt256_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256);
+    if (tiles > 0x7FFFFFFFull) return false;
+    ld->grid[0] = (uint32_t)tiles;
+    ld->grid[1] = 1;
+    ld->grid[2] = d.batch;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0;  // static LDS
+    return true;
+}
+
 const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_wave32", wave32_supports, wave32_plan},
+    {"maize_gemm_bf16_mt256_nn", mt256_nn_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nt", mt256_nt_supports, mt256_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -36,7 +70,13 @@ int kernel_index(const char* name) {
 }
 
 uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units) {
-    (void)d; (void)compute_units;
+    (void)compute_units;
+    const Dims s = dims_of(d);
+    const char* tiled = s.nt ? "maize_gemm_bf16_mt256_nt" : "maize_gemm_bf16_mt256_nn";
+    const int ti = kernel_index(tiled);
+    // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below
+    // half a tile in either direction the per-wave kernel wastes less.
+    if (ti >= 0 && kKernels[ti].supports(d) && s.m >= 128 && s.n >= 128) return (uint32_t)ti;
     return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
 }
 

@@ -1,4 +1,5 @@
 // Single translation unit of the gfx950 code object embedded in libmaize_hip.so.
 #include "common.hpp"
 #include "gemm_wave32.hpp"
+#include "gemm_mt256.hpp"
 #include "probes.hpp"

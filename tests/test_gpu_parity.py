@@ -114,13 +114,19 @@ def test_one_hot_routing_every_position(ctx):
 
 
 def test_nt_equals_nn_bit_for_bit(ctx):
+    """The same logical B stored K x N (NN) or N x K (NT) gives the same bits: both layouts feed the
+    MFMAs the same operands in the same K order."""
     m, n, k = 200, 136, 328
     a, b = inputs(m, n, k)
     bt = b.reshape(k, n).T.ravel()
-    for kern in kernels_for(dict(m=m, n=n, k=k)):
-        c_nn = run_gemm(ctx, a, b, m, n, k, kernel=kern)
-        c_nt = run_gemm(ctx, a, bt, m, n, k, layout=mz.LAYOUT_NT, kernel=kern)
-        assert np.array_equal(c_nn, c_nt), kern
+    nn = kernels_for(dict(m=m, n=n, k=k))
+    nt = kernels_for(dict(m=m, n=n, k=k, layout=mz.LAYOUT_NT))
+    assert len(nn) == len(nt)
+    for kn, kt in zip(nn, nt):                      # None/None, wave32/wave32, tiled_nn/tiled_nt, ...
+        _say(f"nn vs nt: {kn} / {kt}")
+        c_nn = run_gemm(ctx, a, b, m, n, k, kernel=kn)
+        c_nt = run_gemm(ctx, a, bt, m, n, k, layout=mz.LAYOUT_NT, kernel=kt)
+        assert np.array_equal(c_nn, c_nt), (kn, kt)
 
 
 def test_ragged_equals_block_of_zero_padded(ctx):
