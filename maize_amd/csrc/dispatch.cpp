@@ -37,8 +37,12 @@ bool mt256_common(const maize_gemm_desc_t& d) {
     if (s.k >= (1u << 21) || s.n >= (1u << 21)) return false;
     return true;
 }
-bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
-bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
+// The plain kernels advance K with a scalar offset and never mask a lane in K: K % 64 == 0.
+bool k64(const maize_gemm_desc_t& d) { return (d.a.ncols & 63u) == 0; }
+bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d) && k64(d); }
+bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k64(d); }
+bool mt256_nn_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
+bool mt256_nt_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
 bool mt256_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
     const Dims s = dims_of(d);
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256);
@@ -55,6 +59,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_wave32", wave32_supports, wave32_plan},
     {"maize_gemm_bf16_mt256_nn", mt256_nn_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt", mt256_nt_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_ktail", mt256_nn_ktail_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nt_ktail", mt256_nt_ktail_supports, mt256_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -72,7 +78,8 @@ int kernel_index(const char* name) {
 uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units) {
     (void)compute_units;
     const Dims s = dims_of(d);
-    const char* tiled = s.nt ? "maize_gemm_bf16_mt256_nt" : "maize_gemm_bf16_mt256_nn";
+    const char* tiled = (s.k & 63u) ? (s.nt ? "maize_gemm_bf16_mt256_nt_ktail" : "maize_gemm_bf16_mt256_nn_ktail")
+                                    : (s.nt ? "maize_gemm_bf16_mt256_nt" : "maize_gemm_bf16_mt256_nn");
     const int ti = kernel_index(tiled);
     // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below
     // half a tile in either direction the per-wave kernel wastes less.

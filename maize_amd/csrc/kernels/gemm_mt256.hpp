@@ -1,4 +1,4 @@
-// maize_gemm_bf16_mt256_{nn,nt}: the pipelined macro-tile kernel.
+// maize_gemm_bf16_mt256_{nn,nt}[_ktail]: the pipelined macro-tile kernel.
 //
 // The reference schedule (sm80_gemm_smem_multibuffer, crates/maize_tile/src/
 // gemm/mod.rs:37-90: prime a ring of shared-memory TilePairs, then
@@ -8,20 +8,20 @@
 //   * one workgroup of 4 wavefronts (2 x 2) owns a 256 x 256 tile of C; each
 //     wavefront owns a 128 x 128 sub-tile as 4 x 4 MFMA 32x32x16 accumulators
 //     (256 fp32 registers per lane, in AccVGPRs);
-//   * K advances in steps of 64 through a two-stage LDS ring.  Three tiles are
-//     in flight: tile t is consumed from LDS, tile t+1 is being written to the
-//     other LDS stage from registers, tile t+2 is being fetched into those
-//     registers with 128-bit buffer loads whose hardware range check zero-fills
-//     the M/N/K edges (the reference discards its ragged panels,
-//     src/main.rs:56-57);
+//   * K advances in steps of 64 through a two-stage LDS ring filled by 128-bit
+//     direct-to-LDS buffer loads (no register round trip; the hardware range
+//     check zero-fills the M/N/K edges, where the reference discards its
+//     ragged panels, src/main.rs:56-57);
 //   * one barrier per K step, placed before the last quarter of the step's
-//     MFMAs: the fragments of that quarter are already in registers, so the
-//     first fragments of the next tile are read behind the barrier while the
-//     matrix pipe is still busy;
+//     MFMAs: the fragments of that quarter are already in registers, so behind
+//     the barrier the first fragments of tile t+1 are read and the stage that
+//     held tile t is refilled with tile t+2 while the matrix pipe stays busy;
+//     the refill is spread over the last quarter of this step and the first
+//     quarter of the next one so the memory pipe sees a stream, not a burst;
 //   * LDS tiles are XOR-swizzled at 16-byte (K-contiguous tiles) or 64-byte
-//     (row-major K x N tile) granularity so that the 128-bit copies, the
-//     128-bit fragment reads and the transposing reads are all bank-conflict
-//     free without padding;
+//     (row-major K x N tile) granularity so that the direct-to-LDS deposits,
+//     the 128-bit fragment reads and the transposing reads are all
+//     bank-conflict free without padding;
 //   * A (and B when stored N x K) fragments are read with ds_read_b128; a
 //     row-major K x N B is read with ds_read_b64_tr_b16, which hands each lane
 //     the 4 K-consecutive values of its column;
@@ -31,7 +31,9 @@
 //     row-contiguous segments with M/N edge masks.
 //
 // Requirements (checked by the dispatcher): K % 8 == 0, N % 8 == 0, 16-byte
-// aligned operands, each matrix (per batch member) below 2 GiB.
+// aligned operands, each matrix (per batch member) below 2 GiB.  The plain
+// kernels need K % 64 == 0 (the K advance is then a scalar offset and no lane
+// ever needs a K mask); the _ktail kernels take any K % 8 == 0.
 #pragma once
 #include "common.hpp"
 
@@ -43,13 +45,13 @@ constexpr int THREADS = 256;
 constexpr int KROW = 128;               // bytes per LDS row of a K-contiguous tile (64 bf16)
 constexpr int NROW = 512;               // bytes per LDS row of a K x N tile (256 bf16)
 constexpr int TILE = 32768;             // bytes of one operand tile
-constexpr int STAGE = 2 * TILE;         // 65536
-constexpr int LDS_BYTES = 2 * STAGE;    // 131072
 constexpr uint32_t OOB = 0x80000000u;   // OR-ed into an offset: >= num_records, reads as zero
+constexpr int NQ3 = 8;                  // pieces of tile t+2 issued in the last quarter of step t (rest: first quarter of t+1)
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
 typedef __attribute__((address_space(3))) u32x4* lds_v4;
 typedef __attribute__((address_space(3))) u32x2* lds_v2;
+typedef __attribute__((address_space(3))) bf16x8* lds_f8;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
@@ -83,15 +85,22 @@ __device__ __forceinline__ void tile_of(uint32_t pid, uint32_t tm, uint32_t tn, 
 
 #define MAIZE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <bool NT>
+template <bool NT, bool KTAIL>
 __device__ __forceinline__ void body(const GemmArgs& p) {
-    __shared__ __attribute__((aligned(16))) char lds_raw[LDS_BYTES];
-    lds_ptr lds = (lds_ptr)lds_raw;
+    // Four separate arrays (operand x ring stage): the compiler can then tell that a
+    // direct-to-LDS load into one stage does not alias fragment reads of the other, and does
+    // not make every read wait for the loads that were just issued.
+    __shared__ __attribute__((aligned(1024))) char lds_a0[TILE];
+    __shared__ __attribute__((aligned(1024))) char lds_a1[TILE];
+    __shared__ __attribute__((aligned(1024))) char lds_b0[TILE];
+    __shared__ __attribute__((aligned(1024))) char lds_b1[TILE];
+    lds_ptr const A0 = (lds_ptr)lds_a0, A1 = (lds_ptr)lds_a1, B0 = (lds_ptr)lds_b0, B1 = (lds_ptr)lds_b1;
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
     const uint32_t wave = tid >> 6;
+    const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t wm = wave >> 1, wn = wave & 1u;
     const uint32_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     uint32_t tile_m, tile_n;
@@ -102,52 +111,52 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint16_t* Ag = p.a + bz * p.stride_a;
     const uint16_t* Bg = p.b + bz * p.stride_b;
     uint16_t* Cg = p.c + bz * p.stride_c;
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ag, M * K * 2u);
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bg, N * K * 2u);
+    const uint32_t a_bytes = M * K * 2u, b_bytes = N * K * 2u;
 
-    // ---- global -> register -> LDS copy maps --------------------------------
-    // K-contiguous tile (A, and B when NT): 8 lanes cover one 128-byte row;
-    // thread handles rows kr + 32 i.  LDS chunk index is XOR-ed with bits 1..3
-    // of the row.
-    const uint32_t kc = tid & 7u, kr = tid >> 3;
-    // K x N tile (B when NN): 32 lanes cover one 512-byte row; thread handles
-    // rows nr + 8 i.  The 64-byte granule index is XOR-ed with the row's low 2 bits.
-    const uint32_t nc = tid & 31u, nr = tid >> 5;
-
-    uint32_t a_goff = ((m0 + kr) * K + kc * 8u) * 2u;         // advanced by 128 B per K step
-    const uint32_t a_gstep = 32u * K * 2u;
-    const uint32_t a_loff = kr * KROW + ((kc ^ ((kr >> 1) & 7u)) * 16u);
-    uint32_t b_goff, b_gstep, b_gadv, b_loff, b_lstep;
-    if (NT) {
-        b_goff = ((n0 + kr) * K + kc * 8u) * 2u;
-        b_gstep = 32u * K * 2u;
-        b_gadv = BK * 2u;
-        b_loff = TILE + a_loff;
-        b_lstep = 32u * KROW;
-    } else {
-        b_goff = (nr * N + n0 + nc * 8u) * 2u;
-        b_gstep = 8u * N * 2u;
-        b_gadv = BK * N * 2u;
-        b_loff = TILE + nr * NROW + ((nc ^ ((nr & 3u) << 2)) * 16u);
-        b_lstep = 8u * NROW;
-    }
-    const uint32_t b_colmask = (NT || (n0 + nc * 8u) < N) ? 0u : OOB;
-    uint32_t kpos = kc * 8u;                                   // k index of this thread's chunk in the tile being fetched
-
-    u32x4 g[16];
-    auto fetch = [&](int i) {                                  // i: 0..7 = A chunks, 8..15 = B chunks
-        const uint32_t kmask = kpos < K ? 0u : OOB;
-        if (i < 8) {
-            g[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, (a_goff + (uint32_t)i * a_gstep) | kmask, 0, 0);
+    // ---- global -> LDS copy maps (direct-to-LDS buffer loads) -----------------------
+    // One wave-wide 128-bit load deposits 1 KiB contiguously in LDS (lane l at byte 16*l),
+    // so the swizzle is applied on the global side: lane l fetches the chunk whose swizzled
+    // home is position l.  Wave w issues pieces w*8 .. w*8+7 of each operand tile.
+    //   K-contiguous tile (A, and B when NT): piece = 8 rows of 128 B; position l -> row l/8,
+    //     stored chunk l%8 = logical chunk ^ ((row>>1)&7).
+    //   K x N tile (B when NN): piece = 2 rows of 512 B; position l -> row l/32, stored chunk
+    //     l%32 = logical chunk ^ ((row&3)<<2).
+    // vo = byte offset of the lane's chunk at k = 0 (with the N-edge mask folded in); the K
+    // advance is a scalar offset (plain kernels) or added per lane (K-tail kernels).
+    uint32_t a_vo[8], b_vo[8];
+    uint32_t a_k[2];                      // k index of the lane's chunk inside a tile, even/odd piece (K masks)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t row = (wave * 8u + i) * 8u + (lane >> 3);
+        const uint32_t c = (lane & 7u) ^ ((row >> 1) & 7u);
+        a_vo[i] = ((m0 + row) * K + c * 8u) * 2u;
+        if (i < 2) a_k[i] = c * 8u;
+        if (NT) {
+            b_vo[i] = ((n0 + row) * K + c * 8u) * 2u;
         } else {
-            const uint32_t off = b_goff + (uint32_t)(i - 8) * b_gstep;
-            g[i] = __builtin_amdgcn_raw_buffer_load_b128(rb, off | (NT ? kmask : b_colmask), 0, 0);
+            const uint32_t brow = (wave * 8u + i) * 2u + (lane >> 5);
+            const uint32_t bc = (lane & 31u) ^ ((brow & 3u) << 2);
+            b_vo[i] = ((brow * N + n0 + bc * 8u) * 2u) | ((n0 + bc * 8u) < N ? 0u : OOB);
         }
-    };
-    auto advance = [&]() { a_goff += BK * 2u; b_goff += b_gadv; kpos += BK; };
-    auto stash = [&](int i, uint32_t stage_off) {             // registers -> LDS stage
-        if (i < 8) *(lds_v4)(lds + stage_off + a_loff + i * 32 * KROW) = g[i];
-        else       *(lds_v4)(lds + stage_off + b_loff + (i - 8) * b_lstep) = g[i];
+    }
+    const uint32_t b_kscale = NT ? 2u : N * 2u;    // bytes per unit of k in B
+    // Issues piece pc (0..7 = A, 8..15 = B) of the tile that starts at k into stages (sa, sb).
+    auto dma = [&](int pc, lds_ptr sa, lds_ptr sb, uint32_t k) {
+        typedef __attribute__((address_space(3))) void* lvp;
+        const bool is_a = pc < 8;
+        const int i = is_a ? pc : pc - 8;
+        lds_ptr dst = (is_a ? sa : sb) + (wave_u * 8u + i) * 1024u;
+        // Tiles that start at or past K read through a zero-length descriptor: all zeros.
+        const uint32_t bytes = k < K ? (is_a ? a_bytes : b_bytes) : 0u;
+        const __amdgpu_buffer_rsrc_t rs = make_rsrc(is_a ? (const void*)Ag : (const void*)Bg, bytes);
+        if (!KTAIL) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i],
+                                                     k * (is_a ? 2u : b_kscale), 0, 0);
+        } else {
+            uint32_t off = (is_a ? a_vo[i] : b_vo[i]) + k * (is_a ? 2u : b_kscale);
+            if (is_a || NT) off |= (a_k[i & 1] + k) < K ? 0u : OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, off, 0, 0, 0);
+        }
     };
 
     // ---- fragment read maps ---------------------------------------------------
@@ -160,7 +169,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     for (int kk = 0; kk < 4; ++kk) a_rd[kk] = (wm * 128u + l32) * KROW + ((sw ^ (2u * kk)) * 16u);
     if (NT) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) b_rd[kk] = TILE + (wn * 128u + l32) * KROW + ((sw ^ (2u * kk)) * 16u);
+        for (int kk = 0; kk < 4; ++kk) b_rd[kk] = (wn * 128u + l32) * KROW + ((sw ^ (2u * kk)) * 16u);
     } else {
         // Transposing read: in each group of 16 lanes, lane q addresses 4 consecutive columns
         // (q%4) of row (q/4); lane q receives column q of the 4 x 16 block, rows 0..3.
@@ -169,29 +178,28 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const uint32_t row = lhi * 8u + s;                     // + kk*16 (+4 for the second read)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            b_rd[j] = TILE + row * NROW + (wn * 4u + ((uint32_t)j ^ s)) * 64u + half * 32u + (q & 3u) * 8u;
+            b_rd[j] = row * NROW + (wn * 4u + ((uint32_t)j ^ s)) * 64u + half * 32u + (q & 3u) * 8u;
     }
 
     bf16x8 fa[2][4];
     bf16x8 fb[2][4];
     short4v fbl[2][4], fbh[2][4];
     constexpr int NREADS = NT ? 8 : 12;
-    // Read r of the fragments of step kk of the tile in `stage_off` into buffer `buf`.
+    // Read r of the fragments of quarter kk of the tile in (sa, sb) into buffer `buf`.
     // Order: the operands of the first MFMA first.
-    auto read_frag = [&](int buf, int kk, int r, uint32_t stage_off) {
-        lds_ptr base = lds + stage_off;
+    auto read_frag = [&](int buf, int kk, int r, lds_ptr sa, lds_ptr sb) {
         if (NT) {
-            if (r == 0) fa[buf][0] = *(__attribute__((address_space(3))) bf16x8*)(base + a_rd[kk]);
-            else if (r <= 4) fb[buf][r - 1] = *(__attribute__((address_space(3))) bf16x8*)(base + b_rd[kk] + (r - 1) * 32 * KROW);
-            else fa[buf][r - 4] = *(__attribute__((address_space(3))) bf16x8*)(base + a_rd[kk] + (r - 4) * 32 * KROW);
+            if (r == 0) fa[buf][0] = *(lds_f8)(sa + a_rd[kk]);
+            else if (r <= 4) fb[buf][r - 1] = *(lds_f8)(sb + b_rd[kk] + (r - 1) * 32 * KROW);
+            else fa[buf][r - 4] = *(lds_f8)(sa + a_rd[kk] + (r - 4) * 32 * KROW);
         } else {
             typedef short4v __attribute__((address_space(3))) * v4p;
-            if (r == 0) fa[buf][0] = *(__attribute__((address_space(3))) bf16x8*)(base + a_rd[kk]);
+            if (r == 0) fa[buf][0] = *(lds_f8)(sa + a_rd[kk]);
             else if (r <= 8) {
                 const int j = (r - 1) >> 1, h = (r - 1) & 1;
-                short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(base + b_rd[j] + kk * 16 * NROW + h * 4 * NROW));
+                short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(sb + b_rd[j] + kk * 16 * NROW + h * 4 * NROW));
                 if (h == 0) fbl[buf][j] = v; else fbh[buf][j] = v;
-            } else fa[buf][r - 8] = *(__attribute__((address_space(3))) bf16x8*)(base + a_rd[kk] + (r - 8) * 32 * KROW);
+            } else fa[buf][r - 8] = *(lds_f8)(sa + a_rd[kk] + (r - 8) * 32 * KROW);
         }
     };
     auto b_operand = [&](int buf, int j) -> bf16x8 {
@@ -212,60 +220,63 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // ---- prime ---------------------------------------------------------------------
     const uint32_t nk = (K + BK - 1) / BK;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) fetch(i);
-    advance();
+    for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, 0);        // tile 0, whole
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < 16; ++i) stash(i, 0);
+    for (int r = 0; r < NREADS; ++r) read_frag(0, 0, r, A0, B0);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) fetch(i);                     // tile 1 (all zero past K)
-    advance();
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < NREADS; ++r) read_frag(0, 0, r, 0);
+    for (int pc = 0; pc < NQ3; ++pc) dma(pc, A1, B1, BK);      // tile 1, early pieces
+    uint32_t k_early = 2 * BK;   // tile whose early pieces are issued next (last quarter of a step)
+    uint32_t k_late = BK;        // tile whose late pieces are issued next (first quarter of a step)
 
     // ---- steady state ----------------------------------------------------------------
-    // Invariant at the top of step t: LDS stage t&1 holds tile t, fragment buffer 0 holds its
-    // kk = 0 fragments, g[] holds (or is receiving) tile t+1.  Steps past the end fetch zeros
-    // and write them to a stage nobody reads, which keeps the loop body branch-free.
-    for (uint32_t kt = 0; kt < nk; ++kt) {
-        const uint32_t cur = (kt & 1u) * STAGE, nxt = STAGE - cur;
+    // One K step.  On entry: (ca, cb) hold tile t, fragment buffer 0 holds its quarter-0
+    // fragments, the early pieces of tile t+1 are landing in (na, nb).
+    auto step = [&](lds_ptr ca, lds_ptr cb, lds_ptr na, lds_ptr nb) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             const int buf = kk & 1;
             if (kk == 3) {
-                // Everything this step reads from `cur` is in registers and every write to `nxt`
-                // has been issued: wait for the LDS queue, then meet the other waves.
+                // Every fragment this step still needs from (ca, cb) is in registers.  Wait until
+                // this wave's share of tile t+1 has landed, then meet the other waves: after the
+                // barrier (na, nb) is complete and (ca, cb) is free to be refilled with tile t+2.
                 MAIZE_FENCE();
-                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
                 MAIZE_FENCE();
             }
 #pragma unroll
             for (int s = 0; s < 16; ++s) {
                 acc[s >> 2][s & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_operand(buf, s & 3), fa[buf][s >> 2],
                                                                             acc[s >> 2][s & 3], 0, 0, 0);
-                // Side work of this slot: fragment reads for the next step ...
+                // Side work of this slot: fragment reads for the next quarter ...
                 if (s < NREADS) {
-                    if (kk < 3) read_frag(buf ^ 1, kk + 1, s, cur);
-                    else        read_frag(buf ^ 1, 0, s, nxt);
+                    if (kk < 3) read_frag(buf ^ 1, kk + 1, s, ca, cb);
+                    else        read_frag(buf ^ 1, 0, s, na, nb);
                 }
-                // ... and, in the first half of the step, LDS stage refill + the next global fetch.
-                if (kk < 2 && s >= 8) {
-                    const int i = kk * 8 + (s - 8);
-                    stash(i, nxt);
-                    fetch(i);
-                }
+                // ... the late pieces of tile t+1 (its stage was freed by the previous barrier) ...
+                if (kk == 0 && (s & 1) == 1 && NQ3 + (s >> 1) < 16) dma(NQ3 + (s >> 1), na, nb, k_late);
+                // ... and, behind this step's barrier, the early pieces of tile t+2.
+                if (kk == 3 && (s & 1) == 1 && (s >> 1) < NQ3) dma(s >> 1, ca, cb, k_early);
                 MAIZE_FENCE();
             }
-            if (kk == 1) advance();
         }
+        k_early += BK;
+        k_late += BK;
+    };
+    // Two steps per trip so that each step sees its stages as compile-time constants.  An odd
+    // step count runs one extra step on an all-zero tile (loads past K return zeros).
+    for (uint32_t kt = 0; kt < nk; kt += 2) {
+        step(A0, B0, A1, B1);
+        step(A1, B1, A0, B0);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no direct-to-LDS write may land during the epilogue
 
     // ---- epilogue: fp32 -> bf16 (RNE), stage through LDS, 128-bit row stores --------------
-    // Each wave stages its 128 x 128 sub-tile in a private 32 KiB region (row = 256 B).  The
+    // Each wave stages its 128 x 128 sub-tile in a private 32 KiB array (row = 256 B).  The
     // 16-byte chunk index is XOR-ed with row%16 and the 8-byte half with bit 4 of the row, so
     // the 8-byte writes of 32 rows and the 16-byte reads of 4 rows are conflict free.
     __syncthreads();                                           // all waves are done with the operand stages
-    lds_ptr cw = lds + wave * 32768;
+    lds_ptr cw = wave_u == 0 ? A0 : wave_u == 1 ? A1 : wave_u == 2 ? B0 : B1;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -296,7 +307,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
 }  // namespace mt256
 
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn(GemmArgs p) { mt256::body<false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt(GemmArgs p) { mt256::body<true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn(GemmArgs p) { mt256::body<false, false>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt(GemmArgs p) { mt256::body<true, false>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_ktail(GemmArgs p) { mt256::body<false, true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_ktail(GemmArgs p) { mt256::body<true, true>(p); }
 
 }  // namespace maize
