@@ -37,10 +37,10 @@ bool mt256_common(const maize_gemm_desc_t& d) {
     if (s.k >= (1u << 21) || s.n >= (1u << 21)) return false;
     return true;
 }
-// The plain kernels advance K with a scalar offset and never mask a lane in K: K % 64 == 0.
-bool k64(const maize_gemm_desc_t& d) { return (d.a.ncols & 63u) == 0; }
-bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d) && k64(d); }
-bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k64(d); }
+// The plain kernels advance K with a scalar offset and never mask a lane in K: K % 32 == 0.
+bool k32(const maize_gemm_desc_t& d) { return (d.a.ncols & 31u) == 0; }
+bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d) && k32(d); }
+bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k32(d); }
 bool mt256_nn_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
 bool mt256_nt_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
 bool mt256_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
@@ -55,12 +55,30 @@ bool mt256_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
     return true;
 }
 
+// ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
+bool skinny_nn_supports(const maize_gemm_desc_t& d) {
+    const Dims s = dims_of(d);
+    if (d.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
+    const uint64_t lim = 1ull << 31;
+    return (uint64_t)s.n * s.k * 2 < lim && (uint64_t)s.m * s.k * 2 < lim && s.n < (1u << 21);
+}
+bool skinny_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    ld->grid[0] = cdiv(s.n, 64);
+    ld->grid[1] = 1;
+    ld->grid[2] = d.batch;
+    ld->block[0] = 512; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0;
+    return true;
+}
+
 const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_wave32", wave32_supports, wave32_plan},
     {"maize_gemm_bf16_mt256_nn", mt256_nn_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt", mt256_nt_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_ktail", mt256_nn_ktail_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_ktail", mt256_nt_ktail_supports, mt256_plan},
+    {"maize_gemm_bf16_skinny_nn", skinny_nn_supports, skinny_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -78,7 +96,10 @@ int kernel_index(const char* name) {
 uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units) {
     (void)compute_units;
     const Dims s = dims_of(d);
-    const char* tiled = (s.k & 63u) ? (s.nt ? "maize_gemm_bf16_mt256_nt_ktail" : "maize_gemm_bf16_mt256_nn_ktail")
+    // Few rows against a wide row-major B: bound by streaming B once.
+    const int sk = kernel_index("maize_gemm_bf16_skinny_nn");
+    if (sk >= 0 && kKernels[sk].supports(d) && s.n >= 64) return (uint32_t)sk;
+    const char* tiled = (s.k & 31u) ? (s.nt ? "maize_gemm_bf16_mt256_nt_ktail" : "maize_gemm_bf16_mt256_nn_ktail")
                                     : (s.nt ? "maize_gemm_bf16_mt256_nt" : "maize_gemm_bf16_mt256_nn");
     const int ti = kernel_index(tiled);
     // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below

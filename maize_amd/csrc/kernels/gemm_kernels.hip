@@ -2,4 +2,5 @@
 #include "common.hpp"
 #include "gemm_wave32.hpp"
 #include "gemm_mt256.hpp"
+#include "gemm_skinny.hpp"
 #include "probes.hpp"

@@ -45,6 +45,7 @@ SMALL_SHAPES = [  # (m, n, k)
     (1, 1, 1), (1, 7, 3), (5, 1, 9), (16, 16, 16), (31, 33, 17), (32, 32, 16), (33, 17, 65), (64, 64, 64),
     (65, 63, 40), (100, 200, 72), (128, 128, 128), (129, 255, 136), (256, 256, 64), (256, 256, 256),
     (257, 264, 320), (300, 520, 264), (16, 512, 256), (8, 1024, 512), (16, 264, 1000), (512, 256, 1024),
+    (3, 64, 32), (16, 8, 32), (5, 72, 96), (16, 200, 64), (1, 4104, 288), (16, 1096, 2560), (13, 640, 8192 + 32),
 ]
 
 
