@@ -82,7 +82,8 @@ typedef struct {
  * It keeps the order and widths of the reference kernel's parameter list
  * (example_ptx/gen.ptx:12-19: A ptr, arows u32, acols u32, B ptr, brows u32,
  * bcols u32) and appends the C operand the reference never had, the batch
- * strides, the batch count and the layout. */
+ * strides, the batch count, the layout and -- for the split-K kernel only --
+ * a library-owned workspace and the number of K ranges (0 elsewhere). */
 typedef struct {
     const void* a; uint32_t arows, acols;
     const void* b; uint32_t brows, bcols;
@@ -90,6 +91,9 @@ typedef struct {
     uint64_t stride_a, stride_b, stride_c;
     uint32_t batch;
     uint32_t layout;
+    void* workspace;
+    uint32_t ksplit;
+    uint32_t reserved;
 } maize_gemm_args_t;
 
 typedef struct {

@@ -52,7 +52,8 @@ class GemmArgsT(C.Structure):
                 ("b", C.c_void_p), ("brows", C.c_uint32), ("bcols", C.c_uint32),
                 ("c", C.c_void_p), ("crows", C.c_uint32), ("ccols", C.c_uint32),
                 ("stride_a", C.c_uint64), ("stride_b", C.c_uint64), ("stride_c", C.c_uint64),
-                ("batch", C.c_uint32), ("layout", C.c_uint32)]
+                ("batch", C.c_uint32), ("layout", C.c_uint32),
+                ("workspace", C.c_void_p), ("ksplit", C.c_uint32), ("reserved", C.c_uint32)]
 
 
 class DeviceInfoT(C.Structure):
@@ -60,7 +61,7 @@ class DeviceInfoT(C.Structure):
                 ("lds_bytes_per_block", C.c_uint32), ("wavefront_size", C.c_uint32), ("hbm_bytes", C.c_uint64)]
 
 
-assert C.sizeof(MatrixT) == 16 and C.sizeof(GemmArgsT) == 80 and C.sizeof(GemmDescT) == 80
+assert C.sizeof(MatrixT) == 16 and C.sizeof(GemmArgsT) == 96 and C.sizeof(GemmDescT) == 80
 
 _lib = None
 

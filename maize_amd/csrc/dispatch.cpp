@@ -17,6 +17,7 @@ bool wave32_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
     ld->grid[2] = d.batch;
     ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
+    ld->ksplit = 0; ld->workspace_bytes = 0;
     return ld->grid[1] <= 65535u && ld->grid[2] <= 65535u;
 }
 
@@ -52,6 +53,7 @@ bool mt256_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
     ld->grid[2] = d.batch;
     ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;  // static LDS
+    ld->ksplit = 0; ld->workspace_bytes = 0;
     return true;
 }
 
@@ -60,16 +62,29 @@ bool skinny_nn_supports(const maize_gemm_desc_t& d) {
     const Dims s = dims_of(d);
     if (d.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
     const uint64_t lim = 1ull << 31;
-    return (uint64_t)s.n * s.k * 2 < lim && (uint64_t)s.m * s.k * 2 < lim && s.n < (1u << 21);
+    if ((uint64_t)s.n * s.k * 2 >= lim || (uint64_t)s.m * s.k * 2 >= lim || s.n >= (1u << 21)) return false;
+    return (uint64_t)cdiv(s.n, 256) * d.batch <= 16384u;   // one ticket counter per (batch member, slab)
 }
-bool skinny_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
+// K ranges: the smallest power of two that gives the grid at least ~7/8 of a workgroup per
+// compute unit, as long as every range keeps a whole number of 32-row blocks and at least 8 of them.
+uint32_t skinny_ksplit(const Dims& s, uint32_t batch, uint32_t compute_units) {
+    const uint64_t slabs = (uint64_t)cdiv(s.n, 256) * batch;
+    uint32_t ks = 1;
+    while (ks < 16u && slabs * ks * 8u < (uint64_t)compute_units * 7u && s.k % (64u * ks) == 0 && s.k / (2u * ks) >= 256u)
+        ks *= 2;
+    return ks;
+}
+bool skinny_plan(const maize_gemm_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
     const Dims s = dims_of(d);
-    ld->grid[0] = cdiv(s.n, 64);
-    ld->grid[1] = 1;
+    const uint32_t ks = skinny_ksplit(s, d.batch, compute_units ? compute_units : 256u);
+    ld->grid[0] = cdiv(s.n, 256);
+    ld->grid[1] = ks;
     ld->grid[2] = d.batch;
     ld->block[0] = 512; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
-    return true;
+    ld->ksplit = ks;
+    ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.batch * ks * 16u * 256u * 4u : 0;
+    return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
 }
 
 const KernelInfo kKernels[] = {

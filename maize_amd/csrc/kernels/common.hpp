@@ -15,8 +15,11 @@ struct GemmArgs {
     uint64_t stride_a, stride_b, stride_c;
     uint32_t batch;
     uint32_t layout;  // 0 = NN (B is K x N), 1 = NT (B is N x K)
+    void* workspace;  // split-K kernels: ticket counters + fp32 partial tiles (library owned)
+    uint32_t ksplit;  // split-K kernels: number of K ranges (grid.y)
+    uint32_t reserved;
 };
-static_assert(sizeof(GemmArgs) == 80, "kernel parameter block layout");
+static_assert(sizeof(GemmArgs) == 96, "kernel parameter block layout");
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));

@@ -2,42 +2,44 @@
 // against a row-major K x N weight matrix).
 //
 // Every byte of B is streamed from HBM exactly once and nothing else of size moves, so the
-// kernel is built around keeping as many 128-bit direct-to-LDS loads in flight as the chip
-// will take:
+// kernel is built around long contiguous requests and a deep queue of them:
 //
-//   * a workgroup of 8 wavefronts owns a slab of 64 columns of C for all of K; wave w owns
-//     the K blocks w, w+8, w+16, ... (a block is 32 rows of B x 64 columns = 4 KiB).  The
-//     waves never synchronise inside the K loop: each has a private four-slot LDS ring and
-//     paces itself with s_waitcnt vmcnt alone (up to 3 blocks = 12 KiB in flight per wave,
-//     96 KiB per compute unit);
-//   * the reference's per-warp pipeline (prime, wait / consume / refill, drain --
-//     CpAsyncPipeline, crates/maize_core/src/intrinsics/cuda/cp_async.rs:92-210) maps onto
-//     this ring one to one, with the hardware load counter in place of commit/wait groups;
+//   * a workgroup of 8 wavefronts owns a slab of 256 columns of C and one of `ksplit` equal
+//     ranges of K (the dispatcher picks ksplit so that the grid covers the chip).  It walks its
+//     K range in blocks of 32 rows x 256 columns (16 KiB); a block is fetched by 16 direct-to-LDS
+//     128-bit loads, each covering 2 full 512-byte row segments -- requests shorter than that
+//     lose a fifth of the achievable HBM rate on this part;
+//   * an 8-slot LDS ring holds the blocks: while block b is consumed, blocks b+1 .. b+6 are
+//     landing and block b+7 is being requested (up to 112 KiB in flight per compute unit).
+//     This is the reference's prime / wait-consume-refill / drain pipeline (CpAsyncPipeline,
+//     crates/maize_core/src/intrinsics/cuda/cp_async.rs:92-210) with the hardware load counter
+//     in place of commit/wait groups and one workgroup barrier per block;
 //   * B must reach the MFMA with K running along the lane's registers, but it is stored with
 //     N contiguous: the block is deposited in LDS as it is in memory and read back with
 //     ds_read_b64_tr_b16 (4 K-consecutive values of the lane's column per read).  A 32-byte
-//     granule XOR keeps those reads bank-conflict free;
-//   * A (16 x K, 128 KiB at K = 4096, L2 resident) is fetched straight into MFMA operand
-//     registers, one 16-byte load per lane per block, in the same in-order load stream as
-//     the block it multiplies, so one counter wait covers both;
-//   * v_mfma_f32_16x16x32_bf16 with B's fragment first: each lane ends up holding 4
-//     consecutive columns of one row of C;
-//   * the 8 partial sums are added in wave order through LDS (deterministic), rounded once
-//     to bf16 (RNE) and stored as 8-byte segments.
+//     granule XOR keeps those reads bank-conflict free.  Wave w multiplies columns 32w .. 32w+31;
+//   * A (16 x K, L2 resident) is fetched straight into MFMA operand registers, one 16-byte load
+//     per lane per block, in the same in-order load stream as the block it multiplies;
+//   * v_mfma_f32_16x16x32_bf16 with B's fragment first: each lane ends up holding 4 consecutive
+//     columns of one row of C;
+//   * split K: every workgroup writes its fp32 partial tile to a workspace and takes a ticket;
+//     the last one to arrive for a slab adds the partials in split order (deterministic),
+//     rounds once to bf16 (RNE), stores C and resets the ticket counter.
 //
-// Requirements (checked by the dispatcher): layout NN, M <= 16, K % 32 == 0, N % 8 == 0,
-// 16-byte aligned operands, every matrix (per batch member) below 2 GiB.
+// Requirements (checked by the dispatcher): layout NN, M <= 16, K % (32 * ksplit) == 0,
+// N % 8 == 0, 16-byte aligned operands, every matrix (per batch member) below 2 GiB.
 #pragma once
 #include "common.hpp"
 
 namespace maize {
 namespace skinny {
 
-constexpr int SN = 64;                 // columns per workgroup
+constexpr int SN = 256;                // columns per workgroup
 constexpr int WAVES = 8;
 constexpr int KB = 32;                 // K rows per block
-constexpr int BLOCK_BYTES = KB * SN * 2;   // 4096
-constexpr int RING = 4;
+constexpr int ROW = SN * 2;            // 512 bytes per LDS row
+constexpr int BLOCK_BYTES = KB * ROW;  // 16384
+constexpr int RING = 8;
 constexpr uint32_t OOB = 0x80000000u;
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
@@ -53,23 +55,31 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));  // v_cvt_pk_bf16_f32, RNE
 }
 
-// Granule swizzle of a block: the 16-byte chunk index c (0..7) of row r is stored at
-// c ^ (g(r) << 1), g(r) = bit1(r) | bit3(r) << 1.
-__device__ __forceinline__ uint32_t gsw(uint32_t r) { return (((r >> 1) & 1u) | (((r >> 3) & 1u) << 1)) << 1; }
+// Granule swizzle of a block: the 32-byte granule index (0..15) of row r is XOR-ed with
+// f(r) = r%4 + 4*bit3(r), so the 8 rows one transposing read touches land in 8 different
+// granules of the 256-byte bank period.
+__device__ __forceinline__ uint32_t gsw(uint32_t r) { return (r & 3u) | (((r >> 3) & 1u) << 2); }
 
 __device__ __forceinline__ void body(const GemmArgs& p) {
-    // One array per ring slot (each holds the 8 waves' private 4 KiB blocks): distinct objects
-    // let the compiler see that a load into one slot does not alias reads of another.
-    __shared__ __attribute__((aligned(1024))) char ring0[WAVES * BLOCK_BYTES];
-    __shared__ __attribute__((aligned(1024))) char ring1[WAVES * BLOCK_BYTES];
-    __shared__ __attribute__((aligned(1024))) char ring2[WAVES * BLOCK_BYTES];
-    __shared__ __attribute__((aligned(1024))) char ring3[WAVES * BLOCK_BYTES];
+    // One array per ring slot: distinct objects let the compiler see that a load into one slot
+    // does not alias reads of another.
+    __shared__ __attribute__((aligned(1024))) char ring0[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring1[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring2[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring3[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring4[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring5[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring6[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring7[BLOCK_BYTES];
+    __shared__ uint32_t ticket;
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
+    const uint32_t ks = p.ksplit ? p.ksplit : 1u;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t n0 = blockIdx.x * SN;
+    const uint32_t slab = blockIdx.x, z = blockIdx.y;
+    const uint32_t n0 = slab * SN;
     const uint64_t bz = blockIdx.z;
     const uint16_t* Ag = p.a + bz * p.stride_a;
     const uint16_t* Bg = p.b + bz * p.stride_b;
@@ -78,126 +88,157 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bg, K * N * 2u);
     const __amdgpu_buffer_rsrc_t rnull = make_rsrc(Bg, 0u);
 
-    lds_ptr const s0 = (lds_ptr)ring0 + wave * BLOCK_BYTES;
-    lds_ptr const s1 = (lds_ptr)ring1 + wave * BLOCK_BYTES;
-    lds_ptr const s2 = (lds_ptr)ring2 + wave * BLOCK_BYTES;
-    lds_ptr const s3 = (lds_ptr)ring3 + wave * BLOCK_BYTES;
+    lds_ptr const s0 = (lds_ptr)ring0, s1 = (lds_ptr)ring1, s2 = (lds_ptr)ring2, s3 = (lds_ptr)ring3;
+    lds_ptr const s4 = (lds_ptr)ring4, s5 = (lds_ptr)ring5, s6 = (lds_ptr)ring6, s7 = (lds_ptr)ring7;
 
-    // ---- copy map: piece pc (0..3) = rows 8pc .. 8pc+7 of the block; lane l lands at byte 16 l
-    // of the piece = row 8pc + l/8, stored chunk l%8, and therefore fetches logical chunk
-    // (l%8) ^ gsw(row).
-    uint32_t b_vo[4];
+    // ---- copy map: wave w issues pieces 2w and 2w+1 of a block; piece pc = rows 2pc, 2pc+1.
+    // Lane l lands at byte 16 l of the piece = row 2pc + l/32, stored chunk l%32, and therefore
+    // fetches logical chunk (l%32) ^ (gsw(row) << 1).
+    uint32_t b_vo[2];
 #pragma unroll
-    for (int pc = 0; pc < 4; ++pc) {
-        const uint32_t row = pc * 8u + (lane >> 3);
-        const uint32_t c = (lane & 7u) ^ gsw(row);
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t row = (wave * 2u + i) * 2u + (lane >> 5);
+        const uint32_t c = (lane & 31u) ^ (gsw(row) << 1);
         const uint32_t col = n0 + c * 8u;
-        b_vo[pc] = ((row * N + col) * 2u) | (col < N ? 0u : OOB);      // N % 8 == 0: a chunk is all in or all out
+        b_vo[i] = ((row * N + col) * 2u) | (col < N ? 0u : OOB);       // N % 8 == 0: a chunk is all in or all out
     }
     // A operand of MFMA 16x16x32: lane l holds row l%16, k = 8*(l/16) + 0..7 of the block.
     const uint32_t a_vo = ((lane & 15u) * K + (lane >> 4) * 8u) * 2u;  // rows >= M fall past the descriptor: zeros
 
     // ---- transposing-read map.  In each group of 16 lanes, lane q addresses 4 consecutive
     // columns (q%4) of row (q/4) of a 4 x 16 sub-block and receives column q, rows 0..3.  Lane
-    // group g = l/16 needs k = 8g .. 8g+7 (two reads) of columns 16cg .. 16cg+15.
+    // group g = l/16 needs k = 8g .. 8g+7 (two reads, h = 0,1) of column group cg (16 columns).
+    // Byte address = row*512 + ((cg ^ gsw(row)) * 32) + ((q%4)/2)*16 + (q%2)*8.
     const uint32_t q = lane & 15u, g = lane >> 4;
-    uint32_t rd[2];
+    uint32_t rd[2][2];                                   // [h][which of the wave's two column groups]
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         const uint32_t row = g * 8u + h * 4u + (q >> 2);
-        // chunk index of columns 16cg + 4(q%4): 2cg + (q%4)/2; XOR only touches bits 1..2, so it
-        // commutes with adding cg: address = row*128 + ((2cg) ^ gsw(row))*16 + ((q%4)/2)*16 + (q%2)*8
-        rd[h] = row * 128u + ((q & 3u) >> 1) * 16u + (q & 1u) * 8u;
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2)
+            rd[h][c2] = row * ROW + (((wave * 2u + c2) ^ gsw(row)) * 32u) + ((q & 3u) >> 1) * 16u + (q & 1u) * 8u;
     }
-    uint32_t rsw[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) rsw[h] = gsw(g * 8u + h * 4u + (q >> 2));
 
-    const uint32_t nblocks = K / KB;
-    // Wave w owns blocks w, w+8, ...: nb of them.
-    const uint32_t nb = nblocks > wave ? (nblocks - wave + WAVES - 1) / WAVES : 0u;
+    const uint32_t krange = K / ks, k0 = z * krange;
+    const uint32_t nb = krange / KB;                     // blocks of this workgroup
 
-    floatx4 acc[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+    floatx4 acc[2];
+    acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
+    acc[1] = floatx4{0.f, 0.f, 0.f, 0.f};
     bf16x8 af[RING];
 
-    // Requests block j of this wave (global block wave + 8j) into ring slot `slot`, and its A
-    // fragment into af[j % RING]: 5 loads in the in-order stream.
+    // Requests block j (rows k0 + 32j ..) into `slot`, and its A fragment into af[ai]: 3 loads
+    // per wave in the in-order stream.  Blocks past the end read a zero-length descriptor.
     auto request = [&](uint32_t j, lds_ptr slot, int ai) {
         typedef __attribute__((address_space(3))) void* lvp;
-        const uint32_t kb = (wave + j * WAVES) * KB;
+        const uint32_t kb = k0 + j * KB;
         const bool live = j < nb;
         const __amdgpu_buffer_rsrc_t rs_b = live ? rb : rnull;
         const __amdgpu_buffer_rsrc_t rs_a = live ? ra : rnull;
+        // The fences pin the issue order (A fragment, piece, piece): the counter waits below
+        // count loads in that order.
+        __builtin_amdgcn_sched_barrier(0);
         af[ai] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rs_a, a_vo, kb * 2u, 0));
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int pc = 0; pc < 4; ++pc)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lvp)(slot + pc * 1024), 16, b_vo[pc], kb * N * 2u, 0, 0);
+        for (int i = 0; i < 2; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lvp)(slot + (wave * 2u + i) * 1024u), 16, b_vo[i],
+                                                     kb * N * 2u, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
     };
     auto consume = [&](lds_ptr slot, int ai) {
         typedef short4v __attribute__((address_space(3))) * v4p;
 #pragma unroll
-        for (int cg = 0; cg < 4; ++cg) {
-            short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(slot + rd[0] + (((2u * cg) ^ rsw[0]) * 16u)));
-            short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(slot + rd[1] + (((2u * cg) ^ rsw[1]) * 16u)));
+        for (int c2 = 0; c2 < 2; ++c2) {
+            short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(slot + rd[0][c2]));
+            short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(slot + rd[1][c2]));
             short8v bb = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            acc[cg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bb), af[ai], acc[cg], 0, 0, 0);
+            acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bb), af[ai], acc[c2], 0, 0, 0);
         }
     };
+    // One block: wait until this wave's share of block b has landed (the 18 loads of blocks
+    // b+1 .. b+6 may stay in flight), meet the other waves -- which also tells us everyone is
+    // done reading block b-1 -- refill that block's slot with block b+7, then multiply block b.
+    auto turn = [&](uint32_t b, lds_ptr cur, int ai, lds_ptr prev, int pi) {
+        asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        request(b + 7, prev, pi);
+        consume(cur, ai);
+        __builtin_amdgcn_sched_barrier(0);
+    };
 
-    // ---- prime: blocks 0..2 in flight --------------------------------------------------
-    request(0, s0, 0);
-    request(1, s1, 1);
-    request(2, s2, 2);
-    // ---- steady state: request j+3, wait for j (15 newer loads may stay in flight), consume j
-    // The scheduling fences keep a slot's refill behind the MFMAs that consumed it: those MFMAs
-    // have waited for the slot's LDS reads, so the reads are complete before the refill is issued.
-    for (uint32_t j = 0; j < nb; j += RING) {
-        request(j + 3, s3, 3);
-        asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
-        consume(s0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        request(j + 4, s0, 0);
-        asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
-        consume(s1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        request(j + 5, s1, 1);
-        asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
-        consume(s2, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        request(j + 6, s2, 2);
-        asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
-        consume(s3, 3);
-        __builtin_amdgcn_sched_barrier(0);
+    // ---- prime: blocks 0 .. 6 -----------------------------------------------------------
+    request(0, s0, 0); request(1, s1, 1); request(2, s2, 2); request(3, s3, 3);
+    request(4, s4, 4); request(5, s5, 5); request(6, s6, 6);
+    // ---- steady state ---------------------------------------------------------------------
+    for (uint32_t b = 0; b < nb; b += RING) {
+        turn(b + 0, s0, 0, s7, 7);
+        turn(b + 1, s1, 1, s0, 0);
+        turn(b + 2, s2, 2, s1, 1);
+        turn(b + 3, s3, 3, s2, 2);
+        turn(b + 4, s4, 4, s3, 3);
+        turn(b + 5, s5, 5, s4, 4);
+        turn(b + 6, s6, 6, s5, 5);
+        turn(b + 7, s7, 7, s6, 6);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // nothing may land in LDS after this point
-    __syncthreads();
 
-    // ---- reduce the 8 partial tiles in wave order, round once, store ---------------------
-    // Lane holds C[m = l%16][n = 16cg + 4*(l/16) + 0..3].  Partial layout in LDS: [wave][m][n] fp32.
-    float* part = (float*)ring0;                          // 8 x 16 x 64 x 4 B = 32 KiB, generic pointer into LDS
-    {
-        const uint32_t m = lane & 15u;
+    // ---- combine the K splits in split order, round once, store ---------------------------
+    // Lane holds C[m = l%16][n = n0 + 16(2w + c2) + 4g + 0..3].
+    const uint32_t m = lane & 15u;
+    if (ks == 1u) {
+        // Single split: straight from registers, 8 bytes per lane.
 #pragma unroll
-        for (int cg = 0; cg < 4; ++cg)
-            *(floatx4*)(part + (wave * 16u + m) * 64u + cg * 16u + g * 4u) = acc[cg];
+        for (int c2 = 0; c2 < 2; ++c2) {
+            const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
+            if (m < M && col < N) {
+                u32x2 v = {cvt_pk_bf16(acc[c2][0], acc[c2][1]), cvt_pk_bf16(acc[c2][2], acc[c2][3])};
+                *(u32x2*)(Cg + (uint64_t)m * N + col) = v;
+            }
+        }
+        return;
     }
+    // Workspace: 16384 ticket counters (zero between launches), then one fp32 tile of 16 x 256
+    // per (batch member, slab, split).  The tiles are written and read with device-coherent
+    // accesses (they cross the per-XCD L2s), so no cache-wide write-back or invalidate is needed:
+    // each wave waits for its own stores, the barrier collects the waves, then one thread takes
+    // the ticket with a device-scope atomic.
+    constexpr int COHERENT = 17;                          // buffer cache policy: sc0 | sc1
+    constexpr uint32_t TILE_BYTES = 16u * SN * 4u;
+    uint32_t* counters = (uint32_t*)p.workspace;
+    const uint32_t slab_id = (uint32_t)bz * gridDim.x + slab;
+    const __amdgpu_buffer_rsrc_t rws =
+        make_rsrc((const char*)p.workspace + 65536, gridDim.z * gridDim.x * ks * TILE_BYTES);
+    const uint32_t tile0 = slab_id * ks * TILE_BYTES;     // byte offset of this slab's split-0 tile
+#pragma unroll
+    for (int c2 = 0; c2 < 2; ++c2)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[c2]), rws,
+                                               tile0 + z * TILE_BYTES + (m * SN + (wave * 2u + c2) * 16u + g * 4u) * 4u,
+                                               0, COHERENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wave's partial tile has reached memory
     __syncthreads();
-    if (tid < 256u) {
-        const uint32_t m = tid >> 4, nq = (tid & 15u) * 4u;
-        floatx4 s = *(floatx4*)(part + m * 64u + nq);
+    if (tid == 0) ticket = __hip_atomic_fetch_add(&counters[slab_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket != ks - 1u) return;                        // not the last split of this slab to finish
+    {
+        const uint32_t row = tid >> 5, cq = (tid & 31u) * 8u;     // 512 threads x 8 columns = 16 x 256
+        const uint32_t off = tile0 + (row * SN + cq) * 4u;
+        floatx4 s_lo = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off, 0, COHERENT));
+        floatx4 s_hi = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off + 16u, 0, COHERENT));
+        for (uint32_t zz = 1; zz < ks; ++zz) {
+            const floatx4 t_lo = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off + zz * TILE_BYTES, 0, COHERENT));
+            const floatx4 t_hi = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off + zz * TILE_BYTES + 16u, 0, COHERENT));
 #pragma unroll
-        for (int w = 1; w < WAVES; ++w) {
-            const floatx4 t = *(floatx4*)(part + (w * 16u + m) * 64u + nq);
-            s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
+            for (int e = 0; e < 4; ++e) { s_lo[e] += t_lo[e]; s_hi[e] += t_hi[e]; }
         }
-        const uint32_t col = n0 + nq;
-        if (m < M && col < N) {                            // N % 8 == 0, col % 4 == 0: 4 columns are all in or all out
-            u32x2 v = {cvt_pk_bf16(s[0], s[1]), cvt_pk_bf16(s[2], s[3])};
-            *(u32x2*)(Cg + (uint64_t)m * N + col) = v;
+        const uint32_t col = n0 + cq;
+        if (row < M && col < N) {                          // N % 8 == 0: 8 columns are all in or all out
+            u32x4 v = {cvt_pk_bf16(s_lo[0], s_lo[1]), cvt_pk_bf16(s_lo[2], s_lo[3]),
+                       cvt_pk_bf16(s_hi[0], s_hi[1]), cvt_pk_bf16(s_hi[2], s_hi[3])};
+            *(u32x4*)(Cg + (uint64_t)row * N + col) = v;
         }
     }
+    if (tid == 0) counters[slab_id] = 0u;                 // ready for the next launch
 }
 
 }  // namespace skinny

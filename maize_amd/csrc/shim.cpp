@@ -12,6 +12,7 @@
 #include <cstdio>
 #include <cstring>
 #include <new>
+#include <unordered_map>
 
 #include "dispatch.hpp"
 
@@ -19,7 +20,7 @@ extern "C" const unsigned char maize_embedded_hsaco[];
 extern "C" const unsigned char maize_embedded_hsaco_end[];
 
 static_assert(sizeof(maize_matrix_t) == 16 && alignof(maize_matrix_t) == 16, "GlobalMatrix twin");
-static_assert(sizeof(maize_gemm_args_t) == 80, "kernel parameter block");
+static_assert(sizeof(maize_gemm_args_t) == 96, "kernel parameter block");
 static_assert(offsetof(maize_gemm_args_t, arows) == 8 && offsetof(maize_gemm_args_t, acols) == 12 &&
                   offsetof(maize_gemm_args_t, b) == 16 && offsetof(maize_gemm_args_t, brows) == 24 &&
                   offsetof(maize_gemm_args_t, bcols) == 28 && offsetof(maize_gemm_args_t, c) == 32,
@@ -50,11 +51,17 @@ int32_t hip_fail(hipError_t e, const char* what) {
 
 }  // namespace
 
+struct maize_workspace {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
 struct maize_ctx {
     int device;
     hipDeviceProp_t prop;
     hipModule_t module;
     hipFunction_t fn[maize::kMaxKernels];
+    // Split-K scratch, one per stream so that launches on different streams never share it.
+    std::unordered_map<void*, maize_workspace> workspaces;
 };
 struct maize_module {
     maize_ctx* ctx;
@@ -124,6 +131,8 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
 int32_t maize_hip_ctx_destroy(maize_ctx_t* ctx) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "ctx_destroy: ctx is NULL");
     (void)hipSetDevice(ctx->device);
+    for (auto& kv : ctx->workspaces)
+        if (kv.second.ptr) (void)hipFree(kv.second.ptr);
     hipError_t e = hipModuleUnload(ctx->module);
     delete ctx;
     if (e != hipSuccess) return hip_fail(e, "hipModuleUnload");
@@ -268,6 +277,27 @@ int32_t maize_hip_gemm_select(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, c
     return MAIZE_OK;
 }
 
+// Returns the stream's workspace, grown to `bytes` if needed.  A new or grown workspace is
+// zero-filled (the ticket counters must start at zero; the kernels leave them at zero).
+static int32_t workspace_for(maize_ctx_t* ctx, void* stream, size_t bytes, void** out) {
+    maize_workspace& w = ctx->workspaces[stream];
+    if (w.bytes < bytes) {
+        HIP_TRY(hipSetDevice(ctx->device));
+        if (w.ptr) {
+            HIP_TRY(hipStreamSynchronize((hipStream_t)stream));  // earlier launches may still use the old one
+            HIP_TRY(hipFree(w.ptr));
+            w.ptr = nullptr;
+            w.bytes = 0;
+        }
+        const size_t want = bytes + bytes / 2;
+        HIP_TRY(hipMalloc(&w.ptr, want));
+        w.bytes = want;
+        HIP_TRY(hipMemsetAsync(w.ptr, 0, want, (hipStream_t)stream));
+    }
+    *out = w.ptr;
+    return MAIZE_OK;
+}
+
 static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_desc_t* d, uint32_t idx, void* stream) {
     const maize::KernelInfo& ki = maize::kernel_at(idx);
     maize_gemm_args_t args;
@@ -284,6 +314,11 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_desc_t* d, uint32_
     if (!ki.plan(*d, (uint32_t)ctx->prop.multiProcessorCount, &ld))
         return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s cannot run M=%u N=%u K=%u batch=%u (grid limit)", ki.name,
                     d->c.nrows, d->c.ncols, d->a.ncols, d->batch);
+    args.ksplit = ld.ksplit;
+    if (ld.workspace_bytes) {
+        int32_t rc = workspace_for(ctx, stream, ld.workspace_bytes, &args.workspace);
+        if (rc != MAIZE_OK) return rc;
+    }
     return launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->fn[idx], ld.grid, ld.block,
                       ld.lds_bytes, stream, &args, sizeof args);
 }

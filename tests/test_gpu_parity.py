@@ -259,3 +259,53 @@ def test_config5_batched(ctx, oracle):
     # one launch covers every batch member: a single launch equals the per-member launch bit for bit
     single = run_gemm(ctx, a[7 * m * k:8 * m * k], b[7 * k * n:8 * k * n], m, n, k)
     assert np.array_equal(single, got[7 * m * n:8 * m * n])
+
+
+# ---- the split-K path of the skinny kernel -------------------------------------------------
+
+def test_skinny_split_k_repeats_streams_and_batches(ctx, oracle):
+    """The M <= 16 kernel combines K ranges through a library-owned workspace whose ticket counters it
+    must leave at zero: repeated launches, launches on another stream and batched launches all have to
+    give the same bits."""
+    m, n, k = 16, 1096, 4096                      # 5 slabs -> the dispatcher splits K
+    a = mz.gen.normal_bf16(m * k, mz.gen.SEED_A, 1.0)
+    b = mz.gen.normal_bf16(k * n, mz.gen.SEED_B, 0.02)
+    first = run_gemm(ctx, a, b, m, n, k)
+    check_against_oracle(oracle, first, a, b, m, n, k, label="skinny split-K")
+    for _ in range(3):
+        assert np.array_equal(run_gemm(ctx, a, b, m, n, k), first)
+    s = ctx.stream()
+    assert np.array_equal(run_gemm(ctx, a, b, m, n, k, stream=s), first)
+    ctx.stream_destroy(s)
+    # a different shape in between (its workspace layout differs), then the first one again
+    a2 = mz.gen.normal_bf16(7 * 2048, 3, 1.0)
+    b2 = mz.gen.normal_bf16(2048 * 264, 4, 0.02)
+    got2 = run_gemm(ctx, a2, b2, 7, 264, 2048)
+    check_against_oracle(oracle, got2, a2, b2, 7, 264, 2048, label="skinny 7x264x2048")
+    assert np.array_equal(run_gemm(ctx, a, b, m, n, k), first)
+    # batched: every member equals its single launch
+    batch = 3
+    ab = mz.gen.normal_bf16(batch * m * k, 5, 1.0)
+    bb = mz.gen.normal_bf16(batch * k * n, 6, 0.02)
+    dense = run_gemm(ctx, ab, bb, m, n, k, batch=batch)
+    for i in range(batch):
+        single = run_gemm(ctx, ab[i * m * k:(i + 1) * m * k], bb[i * k * n:(i + 1) * k * n], m, n, k)
+        assert np.array_equal(single, dense[i * m * n:(i + 1) * m * n])
+
+
+def test_dispatcher_choices(ctx):
+    """The kernel the dispatcher picks for each benchmark configuration."""
+    def pick(m, n, k, layout=mz.LAYOUT_NN, batch=1):
+        a = mz.GlobalMatrix(0x10000, m, k)
+        b = mz.GlobalMatrix(0x10000, k, n) if layout == mz.LAYOUT_NN else mz.GlobalMatrix(0x10000, n, k)
+        c = mz.GlobalMatrix(0x10000, m, n)
+        return ctx.gemm_select(mz.gemm_desc(a, b, c, layout=layout, batch=batch, stride_a=m * k, stride_b=k * n,
+                                            stride_c=m * n))
+    assert pick(4096, 4096, 4096) == "maize_gemm_bf16_mt256_nn"
+    assert pick(4000, 4104, 4032) == "maize_gemm_bf16_mt256_nn"
+    assert pick(8192, 8192, 8192, mz.LAYOUT_NT) == "maize_gemm_bf16_mt256_nt"
+    assert pick(16, 14336, 4096) == "maize_gemm_bf16_skinny_nn"
+    assert pick(2048, 2048, 2048, batch=32) == "maize_gemm_bf16_mt256_nn"
+    assert pick(4096, 4096, 4072) == "maize_gemm_bf16_mt256_nn_ktail"
+    assert pick(4096, 4099, 4096) == "maize_gemm_bf16_wave32"
+    assert pick(33, 17, 65) == "maize_gemm_bf16_wave32"

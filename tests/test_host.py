@@ -39,7 +39,7 @@ def test_struct_layouts_match_the_reference_abi():
     A = _ffi.GemmArgsT
     assert (A.a.offset, A.arows.offset, A.acols.offset, A.b.offset, A.brows.offset, A.bcols.offset) == (0, 8, 12, 16, 24, 28)
     assert (A.c.offset, A.crows.offset, A.ccols.offset) == (32, 40, 44)
-    assert C.sizeof(A) == 80 and C.sizeof(_ffi.GemmDescT) == 80
+    assert C.sizeof(A) == 96 and C.sizeof(_ffi.GemmDescT) == 80
 
 
 def test_embedded_code_object_is_a_gfx950_elf_with_all_kernels():
