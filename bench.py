@@ -22,6 +22,10 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each
+# scaled by what the same counter reads for a 256 MiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x
+# 1.000): profiles/hbm_traffic_fetch_write_size.md.  Not measured for the other configurations.
+MEASURED_TRAFFIC_BYTES = {"cfg1": 235.1e6, "cfg4": 126.4e6}
 
 # name -> (M, N, K, layout, batch, A distribution, B distribution, bound)
 CONFIGS = {
@@ -78,12 +82,47 @@ def cpu_baseline(cfg, a, b_storage, got, seconds_target=12.0):
     return out, parity
 
 
+def copy_calibration(steps, warmup):
+    """Streams 256 MiB through maize_copy_u128 (one read + one write of every byte): the
+    known-size copy that the FETCH_SIZE / WRITE_SIZE hardware counters are scaled against."""
+    import ctypes as C
+    import maize_amd as mz
+
+    class CopyArgs(C.Structure):
+        _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("n_vec", C.c_uint64)]
+
+    nbytes = 256 * 2 ** 20
+    ctx = mz.Context(0)
+    src, dst = ctx.malloc(nbytes), ctx.malloc(nbytes)
+    src.fill(0x5A)
+    kern = mz.new_hip_kernel("maize_copy_u128").with_launch_bounds_1d(256).finalize().compile(mz.Gfx.Gfx950, ctx)
+    args = CopyArgs(src.ptr, dst.ptr, nbytes // 16)
+    grid = (ctx.info()["compute_units"] * 8, 1, 1)
+    ev0, ev1 = ctx.event(), ctx.event()
+    for _ in range(warmup):
+        kern.launch(grid, args)
+    ctx.sync()
+    ev0.record(None)
+    for _ in range(steps):
+        kern.launch(grid, args)
+    ev1.record(None)
+    ctx.sync()
+    us = ev0.elapsed_ms(ev1) / steps * 1e3
+    print(json.dumps({"metric": "copy calibration", "kernel": "maize_copy_u128", "bytes_read": nbytes,
+                      "bytes_written": nbytes, "kernel_avg_us": us, "value": 2 * nbytes / us / 1e3, "unit": "GB/s",
+                      "steps": steps, "warmup": warmup}), flush=True)
+    kern.release()
+    src.free(); dst.free()
+    ctx.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--config", default="cfg1", choices=sorted(CONFIGS))
+    ap.add_argument("--config", default="cfg1", choices=sorted(CONFIGS) + ["copy"],
+                    help="cfg1..cfg5: a benchmark configuration; copy: the 256 MiB copy used to scale HBM counters")
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--rotate", type=int, default=0,
@@ -95,6 +134,9 @@ def main():
               "every box here has one GPU) -- run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.config == "copy":
+        copy_calibration(args.steps, args.warmup)
+        return
     import maize_amd as mz
     cfg = CONFIGS[args.config]
     m, n, k, batch, nt = cfg["m"], cfg["n"], cfg["k"], cfg["batch"], cfg["nt"]
@@ -160,6 +202,7 @@ def main():
         ach = alg_bytes / (kern_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
                 "traffic": None}
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.config) if args.kernel is None else None
     roof["kernel"] = kernel
     roof["kernel_avg_us"] = kern_ms * 1e3
     roof["algorithmic_flop"] = flops

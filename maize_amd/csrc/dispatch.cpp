@@ -38,10 +38,10 @@ bool mt256_common(const maize_gemm_desc_t& d) {
     if (s.k >= (1u << 21) || s.n >= (1u << 21)) return false;
     return true;
 }
-// The plain kernels advance K with a scalar offset and never mask a lane in K: K % 32 == 0.
-bool k32(const maize_gemm_desc_t& d) { return (d.a.ncols & 31u) == 0; }
-bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d) && k32(d); }
-bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k32(d); }
+// The plain kernels advance K with a scalar offset and never mask a lane in K: K % 64 == 0.
+bool k64(const maize_gemm_desc_t& d) { return (d.a.ncols & 63u) == 0; }
+bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d) && k64(d); }
+bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k64(d); }
 bool mt256_nn_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
 bool mt256_nt_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
 bool mt256_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
@@ -114,7 +114,7 @@ uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units) {
     // Few rows against a wide row-major B: bound by streaming B once.
     const int sk = kernel_index("maize_gemm_bf16_skinny_nn");
     if (sk >= 0 && kKernels[sk].supports(d) && s.n >= 64) return (uint32_t)sk;
-    const char* tiled = (s.k & 31u) ? (s.nt ? "maize_gemm_bf16_mt256_nt_ktail" : "maize_gemm_bf16_mt256_nn_ktail")
+    const char* tiled = (s.k & 63u) ? (s.nt ? "maize_gemm_bf16_mt256_nt_ktail" : "maize_gemm_bf16_mt256_nn_ktail")
                                     : (s.nt ? "maize_gemm_bf16_mt256_nt" : "maize_gemm_bf16_mt256_nn");
     const int ti = kernel_index(tiled);
     // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below
