@@ -17,7 +17,7 @@ bool wave32_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
     ld->grid[2] = d.batch;
     ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
-    ld->ksplit = 0; ld->workspace_bytes = 0;
+    ld->ksplit = 0; ld->workspace_bytes = 0; ld->split_first = 0;
     return ld->grid[1] <= 65535u && ld->grid[2] <= 65535u;
 }
 
@@ -44,18 +44,54 @@ bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LA
 bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k64(d); }
 bool mt256_nn_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
 bool mt256_nt_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
-bool mt256_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
+// Edge splitting.  A ragged N leaves a last column of tiles that are almost empty but cost a
+// whole tile each (likewise a ragged M and the last row).  When that edge is at most 32 elements
+// wide and setting it aside saves a round of workgroups (one workgroup per compute unit per
+// round), the edge tiles are given `ks` workgroups each, one K range apiece, which finish in
+// ~1/ks of a tile time; their partial tiles are narrow, so combining them is cheap.  Single batch
+// member only, at least 4 K steps per range, at most 16 ranges.
+struct EdgeSplit { uint32_t mode, whole, nedge, ks; };   // mode 0 = none, 1 = last tile column, 2 = last tile row
+EdgeSplit mt256_edge(const Dims& s, uint32_t batch, uint32_t cus) {
+    const uint32_t tm = cdiv(s.m, 256), tn = cdiv(s.n, 256);
+    EdgeSplit e = {0, tm * tn, 0, 0};
+    if (batch != 1 || cus == 0) return e;
+    const uint32_t nk = cdiv(s.k, 64);
+    uint32_t kmax = nk / 4u < 16u ? nk / 4u : 16u;
+    if (kmax < 2u) return e;
+    const uint32_t w_n = s.n - (tn - 1u) * 256u, h_m = s.m - (tm - 1u) * 256u;
+    const uint32_t rounds = cdiv(tm * tn, cus);
+    uint32_t mode = 0;
+    if (tn >= 2u && w_n <= 32u && cdiv(tm * (tn - 1u), cus) < rounds) mode = 1;
+    else if (tm >= 2u && h_m <= 32u && cdiv((tm - 1u) * tn, cus) < rounds) mode = 2;
+    if (!mode) return e;
+    const uint32_t nedge = mode == 1 ? tm : tn;
+    uint32_t k = cus / nedge;                              // fill the chip once with edge workgroups
+    if (k > kmax) k = kmax;
+    if (k < 2u) return e;
+    k = cdiv(nk, cdiv(nk, k));                             // no empty range
+    if (k < 2u) return e;
+    e.mode = mode; e.nedge = nedge; e.ks = k;
+    e.whole = mode == 1 ? tm * (tn - 1u) : (tm - 1u) * tn;
+    return e;
+}
+bool mt256_plan_impl(const maize_gemm_desc_t& d, uint32_t compute_units, bool allow_edge, LaunchDims* ld) {
     const Dims s = dims_of(d);
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256);
-    if (tiles > 0x7FFFFFFFull) return false;
-    ld->grid[0] = (uint32_t)tiles;
+    if (tiles > 0x1FFFFFFFull) return false;
+    EdgeSplit e = mt256_edge(s, d.batch, compute_units);
+    if (!allow_edge) e = EdgeSplit{0, (uint32_t)tiles, 0, 0};
+    ld->grid[0] = e.mode ? e.whole + e.nedge * e.ks : (uint32_t)tiles;
     ld->grid[1] = 1;
     ld->grid[2] = d.batch;
     ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;  // static LDS
-    ld->ksplit = 0; ld->workspace_bytes = 0;
-    return true;
+    ld->ksplit = e.ks;
+    ld->split_first = e.mode ? ((e.mode << 30) | (e.whole + 1u)) : 0u;
+    ld->workspace_bytes = e.mode ? kTicketBytes + (size_t)e.nedge * e.ks * 256u * 256u * 4u : 0;
+    return ld->workspace_bytes < (1ull << 31) && e.nedge <= 16384u;
 }
+bool mt256_plan(const maize_gemm_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, false, ld); }
+bool mt256_edge_plan(const maize_gemm_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
 
 // ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
 bool skinny_nn_supports(const maize_gemm_desc_t& d) {
@@ -83,6 +119,7 @@ bool skinny_plan(const maize_gemm_desc_t& d, uint32_t compute_units, LaunchDims*
     ld->block[0] = 512; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
     ld->ksplit = ks;
+    ld->split_first = 0;
     ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.batch * ks * 16u * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
 }
@@ -93,6 +130,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt", mt256_nt_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_ktail", mt256_nn_ktail_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_ktail", mt256_nt_ktail_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_edge", mt256_nn_supports, mt256_edge_plan},
+    {"maize_gemm_bf16_mt256_nt_edge", mt256_nt_supports, mt256_edge_plan},
+    {"maize_gemm_bf16_mt256_nn_ktail_edge", mt256_nn_ktail_supports, mt256_edge_plan},
+    {"maize_gemm_bf16_mt256_nt_ktail_edge", mt256_nt_ktail_supports, mt256_edge_plan},
     {"maize_gemm_bf16_skinny_nn", skinny_nn_supports, skinny_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
@@ -109,14 +150,17 @@ int kernel_index(const char* name) {
 }
 
 uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units) {
-    (void)compute_units;
     const Dims s = dims_of(d);
     // Few rows against a wide row-major B: bound by streaming B once.
     const int sk = kernel_index("maize_gemm_bf16_skinny_nn");
     if (sk >= 0 && kKernels[sk].supports(d) && s.n >= 64) return (uint32_t)sk;
-    const char* tiled = (s.k & 63u) ? (s.nt ? "maize_gemm_bf16_mt256_nt_ktail" : "maize_gemm_bf16_mt256_nn_ktail")
-                                    : (s.nt ? "maize_gemm_bf16_mt256_nt" : "maize_gemm_bf16_mt256_nn");
-    const int ti = kernel_index(tiled);
+    static const char* const kTiled[2][2][2] = {   // [edge split][K tail][NT]
+        {{"maize_gemm_bf16_mt256_nn", "maize_gemm_bf16_mt256_nt"},
+         {"maize_gemm_bf16_mt256_nn_ktail", "maize_gemm_bf16_mt256_nt_ktail"}},
+        {{"maize_gemm_bf16_mt256_nn_edge", "maize_gemm_bf16_mt256_nt_edge"},
+         {"maize_gemm_bf16_mt256_nn_ktail_edge", "maize_gemm_bf16_mt256_nt_ktail_edge"}}};
+    const bool edge = mt256_edge(s, d.batch, compute_units).mode != 0;
+    const int ti = kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt]);
     // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below
     // half a tile in either direction the per-wave kernel wastes less.
     if (ti >= 0 && kKernels[ti].supports(d) && s.m >= 128 && s.n >= 128) return (uint32_t)ti;

@@ -19,6 +19,7 @@ struct LaunchDims {
     uint32_t block[3];
     uint32_t lds_bytes;
     uint32_t ksplit;          // split-K kernels: number of K ranges (0 = kernel takes no workspace)
+    uint32_t split_first;     // tiled kernels: edge mode << 30 | 1 + number of tiles computed whole (0 = every tile whole)
     size_t workspace_bytes;   // bytes of zero-initialised, library-owned workspace the launch needs
 };
 constexpr size_t kTicketBytes = 16384 * 4;  // ticket counters at the start of a workspace

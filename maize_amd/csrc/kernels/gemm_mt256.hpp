@@ -1,4 +1,4 @@
-// maize_gemm_bf16_mt256_{nn,nt}[_ktail]: the pipelined macro-tile kernel.
+// maize_gemm_bf16_mt256_{nn,nt}[_ktail][_edge]: the pipelined macro-tile kernel.
 //
 // The reference schedule (sm80_gemm_smem_multibuffer, crates/maize_tile/src/
 // gemm/mod.rs:37-90: prime a ring of shared-memory TilePairs, then
@@ -29,6 +29,13 @@
 //     consecutive columns of one row of C; the epilogue converts to bf16 (RNE)
 //     and stages the wave's sub-tile through LDS to store full 128-bit,
 //     row-contiguous segments with M/N edge masks.
+//
+//   * a ragged N (or M) leaves a last column (row) of tiles that are almost empty but cost a full
+//     tile each, and can push the tile count just past a multiple of the CU count.  The _edge
+//     kernels let the dispatcher hand those tiles to `ksplit` workgroups each, one K range apiece.  Such a workgroup
+//     writes the part of its fp32 partial tile that lies inside the matrix to a library-owned
+//     workspace (device-coherent stores), takes a ticket with a device-scope atomic, and the last
+//     arriver re-reads all partials in range order (deterministic), then runs the normal epilogue.
 //
 // Requirements (checked by the dispatcher): K % 8 == 0, N % 8 == 0, 16-byte
 // aligned operands, each matrix (per batch member) below 2 GiB.  The plain
@@ -76,12 +83,13 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
 // on one XCD (ids congruent mod 8) form a contiguous run of tiles and (b) a
 // run covers a compact block of the tile grid, so an XCD's L2 sees few
 // distinct A row panels and B column panels.
-__device__ __forceinline__ void tile_of(uint32_t pid, uint32_t tm, uint32_t tn, uint32_t* tile_m, uint32_t* tile_n) {
-    const uint32_t total = tm * tn;
+__device__ __forceinline__ uint32_t xcd_run(uint32_t pid, uint32_t total) {
     const uint32_t per = (total + 7u) / 8u;
     const uint32_t tall = (total % 8u) ? (total % 8u) : 8u;
     const uint32_t xcd = pid % 8u, local = pid / 8u;
-    uint32_t id = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1u) + local;
+    return xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1u) + local;
+}
+__device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, uint32_t* tile_m, uint32_t* tile_n) {
     constexpr uint32_t GM = 4;
     const uint32_t group = id / (GM * tn);
     const uint32_t first = group * GM;
@@ -93,7 +101,7 @@ __device__ __forceinline__ void tile_of(uint32_t pid, uint32_t tm, uint32_t tn, 
 
 #define MAIZE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <bool NT, bool KTAIL>
+template <bool NT, bool KTAIL, bool EDGE>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     // Four separate arrays (operand x ring stage): the compiler can then tell that a
     // direct-to-LDS load into one stage does not alias fragment reads of the other, and does
@@ -111,9 +119,31 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t wm = wave >> 1, wn = wave & 1u;
     const uint32_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    // Workgroups 0 .. whole-1 compute one tile each over all of K.  With edge splitting
+    // (p.reserved = mode << 30 | whole + 1; mode 1: last tile column, mode 2: last tile row) the
+    // whole tiles are the grid without that edge, and the rest of the workgroups share the edge
+    // tiles, `ksplit` workgroups (K ranges) per tile.
+    const uint32_t mode = EDGE ? p.reserved >> 30 : 0u;
+    const uint32_t whole = (EDGE && p.reserved) ? (p.reserved & 0x3FFFFFFFu) - 1u : tm * tn;
+    const bool split = EDGE && blockIdx.x >= whole;
+    const uint32_t ks = split ? p.ksplit : 1u;
+    const uint32_t edge = split ? (blockIdx.x - whole) / ks : 0u;     // which edge tile
+    const uint32_t z = split ? (blockIdx.x - whole) % ks : 0u;        // which K range
     uint32_t tile_m, tile_n;
-    tile_of(blockIdx.x, tm, tn, &tile_m, &tile_n);
+    if (!split) {
+        tile_of(xcd_run(blockIdx.x, whole), tm - (mode == 2u), tn - (mode == 1u), &tile_m, &tile_n);
+    } else {
+        tile_m = mode == 1u ? edge : tm - 1u;
+        tile_n = mode == 1u ? tn - 1u : edge;
+    }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    // K steps of this workgroup: [kt0, kt0 + nk) of the ceil(K / BK) steps.
+    const uint32_t nk_all = (K + BK - 1) / BK;
+    const uint32_t per_range = (nk_all + ks - 1u) / ks;
+    const uint32_t kt0 = z * per_range;
+    const uint32_t nk = kt0 < nk_all ? (nk_all - kt0 < per_range ? nk_all - kt0 : per_range) : 0u;
+    const uint32_t k_begin = kt0 * BK;
+    const uint32_t k_end = (kt0 + nk) * BK < K ? (kt0 + nk) * BK : K;   // loads at or past k_end return zeros
 
     const uint64_t bz = blockIdx.z;
     const uint16_t* Ag = p.a + bz * p.stride_a;
@@ -155,7 +185,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const int i = is_a ? pc : pc - 8;
         lds_ptr dst = (is_a ? sa : sb) + (wave_u * 8u + i) * 1024u;
         // Tiles that start at or past K read through a zero-length descriptor: all zeros.
-        const uint32_t bytes = k < K ? (is_a ? a_bytes : b_bytes) : 0u;
+        const uint32_t bytes = k < k_end ? (is_a ? a_bytes : b_bytes) : 0u;
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(is_a ? (const void*)Ag : (const void*)Bg, bytes);
         if (!KTAIL) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i],
@@ -226,16 +256,15 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     // ---- prime ---------------------------------------------------------------------
-    const uint32_t nk = (K + BK - 1) / BK;
 #pragma unroll
-    for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, 0);        // tile 0, whole
+    for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, k_begin);  // tile 0, whole
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
     for (int r = 0; r < NREADS; ++r) read_frag(0, 0, r, A0, B0);
 #pragma unroll
-    for (int pc = 0; pc < early_pieces(); ++pc) dma(pc, A1, B1, BK);   // tile 1, early pieces
-    uint32_t k_early = 2 * BK;   // tile whose early pieces are issued next (last quarter of a step)
-    uint32_t k_late = BK;        // tile whose late pieces are issued next (first quarter of a step)
+    for (int pc = 0; pc < early_pieces(); ++pc) dma(pc, A1, B1, k_begin + BK);   // tile 1, early pieces
+    uint32_t k_early = k_begin + 2 * BK;   // tile whose early pieces are issued next (last quarter of a step)
+    uint32_t k_late = k_begin + BK;        // tile whose late pieces are issued next (first quarter of a step)
 
     // ---- steady state ----------------------------------------------------------------
     // One K step.  On entry: (ca, cb) hold tile t, fragment buffer 0 holds its quarter-0
@@ -285,6 +314,62 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no direct-to-LDS write may land during the epilogue
 
+    // ---- K ranges: publish the partial tile, take a ticket, last arriver sums in range order ----
+    if (EDGE && split) {
+        constexpr int COHERENT = 17;                      // buffer cache policy sc0 | sc1: visible across the XCDs' L2s
+        constexpr uint32_t UNIT = BM * BN * 4u;           // one fp32 partial tile
+        constexpr uint32_t DROP = 0xFFFFFFF0u;            // out-of-range offset: store dropped, load returns zeros
+        __shared__ uint32_t ticket;
+        uint32_t* counters = (uint32_t*)p.workspace;      // 16384 counters (zero between launches), then the tiles
+        const uint32_t nedge = mode == 1u ? tm : tn;
+        const uint32_t slot = (uint32_t)bz * nedge + edge;
+        const __amdgpu_buffer_rsrc_t rws = make_rsrc((const char*)p.workspace + 65536, gridDim.z * nedge * ks * UNIT);
+        // A partial tile is stored in register order, not row-major: chunk c = (i, j, q) of wave w is
+        // 64 lanes x 16 bytes = 1 KiB contiguous, so every store and load instruction moves whole
+        // cache lines.  Lane's chunk = row wm*128 + i*32 + l%32, columns wn*128 + j*32 + 8q + 4(l/32)
+        // + 0..3.  Chunks wholly outside the matrix are skipped (a wave-uniform test); lanes outside
+        // it inside a chunk use an out-of-range offset.
+        const uint32_t l32e = lane & 31u, lhie = lane >> 5;
+        const uint32_t wmu = wave_u >> 1, wnu = wave_u & 1u;
+        const uint32_t lane_off = wave_u * 65536u + lane * 16u;
+        const uint32_t rows_ok = M - m0, cols_ok = N - n0;    // valid extent of this tile (may exceed 256)
+        auto chunk_live = [&](int c) { return wmu * 128u + (c >> 4) * 32u < rows_ok && wnu * 128u + ((c >> 2) & 3) * 32u + (c & 3) * 8u < cols_ok; };
+        auto lane_live = [&](int c) { return wm * 128u + (c >> 4) * 32u + l32e < rows_ok && wn * 128u + ((c >> 2) & 3) * 32u + (c & 3) * 8u + lhie * 4u < cols_ok; };
+#pragma unroll
+        for (int c = 0; c < 64; ++c) {
+            if (!chunk_live(c)) continue;
+            const int i = c >> 4, j = (c >> 2) & 3, q = c & 3;
+            const uint32_t off = lane_live(c) ? (slot * ks + z) * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
+            const floatx4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rws, off, 0, COHERENT);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of the tile has reached memory
+        __syncthreads();
+        if (tid == 0) ticket = __hip_atomic_fetch_add(&counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket != ks - 1u) return;                    // another workgroup will finish this tile
+        // Sum the ranges in order, chunk by chunk; the (up to 16) loads of one chunk are issued
+        // together, ranges past ksplit read zeros.
+#pragma unroll
+        for (int c = 0; c < 64; ++c) {
+            const int i = c >> 4, j = (c >> 2) & 3, q = c & 3;
+            floatx4 sum = {0.f, 0.f, 0.f, 0.f};
+            if (chunk_live(c)) {
+                const uint32_t base = lane_live(c) ? slot * ks * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
+                floatx4 t[16];
+#pragma unroll
+                for (int zz = 0; zz < 16; ++zz)
+                    t[zz] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                        rws, ((uint32_t)zz < ks && base != DROP) ? base + (uint32_t)zz * UNIT : DROP, 0, COHERENT));
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int zz = 0; zz < 16; ++zz) { sum[0] += t[zz][0]; sum[1] += t[zz][1]; sum[2] += t[zz][2]; sum[3] += t[zz][3]; }
+            }
+            acc[i][j][4 * q] = sum[0]; acc[i][j][4 * q + 1] = sum[1]; acc[i][j][4 * q + 2] = sum[2]; acc[i][j][4 * q + 3] = sum[3];
+        }
+        if (tid == 0) counters[slot] = 0u;                // ready for the next launch
+    }
+
     // ---- epilogue: fp32 -> bf16 (RNE), stage through LDS, 128-bit row stores --------------
     // Each wave stages its 128 x 128 sub-tile in a private 32 KiB array (row = 256 B).  The
     // 16-byte chunk index is XOR-ed with row%16 and the 8-byte half with bit 4 of the row, so
@@ -321,9 +406,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
 }  // namespace mt256
 
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn(GemmArgs p) { mt256::body<false, false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt(GemmArgs p) { mt256::body<true, false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_ktail(GemmArgs p) { mt256::body<false, true>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_ktail(GemmArgs p) { mt256::body<true, true>(p); }
+#define MAIZE_MT256_KERNEL(name, nt, ktail, edge) \
+    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, edge>(p); }
+MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn, false, false, false)
+MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt, true, false, false)
+MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail, false, true, false)
+MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_ktail, true, true, false)
+MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_edge, false, false, true)
+MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_edge, true, false, true)
+MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail_edge, false, true, true)
+MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_ktail_edge, true, true, true)
+#undef MAIZE_MT256_KERNEL
 
 }  // namespace maize

@@ -315,6 +315,7 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_desc_t* d, uint32_
         return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s cannot run M=%u N=%u K=%u batch=%u (grid limit)", ki.name,
                     d->c.nrows, d->c.ncols, d->a.ncols, d->batch);
     args.ksplit = ld.ksplit;
+    args.reserved = ld.split_first;
     if (ld.workspace_bytes) {
         int32_t rc = workspace_for(ctx, stream, ld.workspace_bytes, &args.workspace);
         if (rc != MAIZE_OK) return rc;

@@ -302,7 +302,7 @@ def test_dispatcher_choices(ctx):
         return ctx.gemm_select(mz.gemm_desc(a, b, c, layout=layout, batch=batch, stride_a=m * k, stride_b=k * n,
                                             stride_c=m * n))
     assert pick(4096, 4096, 4096) == "maize_gemm_bf16_mt256_nn"
-    assert pick(4000, 4104, 4032) == "maize_gemm_bf16_mt256_nn"
+    assert pick(4000, 4104, 4032) == "maize_gemm_bf16_mt256_nn_edge"     # 8-column last tile column, 272 tiles
     assert pick(8192, 8192, 8192, mz.LAYOUT_NT) == "maize_gemm_bf16_mt256_nt"
     assert pick(16, 14336, 4096) == "maize_gemm_bf16_skinny_nn"
     assert pick(2048, 2048, 2048, batch=32) == "maize_gemm_bf16_mt256_nn"
@@ -310,3 +310,24 @@ def test_dispatcher_choices(ctx):
     assert pick(4096, 4096, 4064) == "maize_gemm_bf16_mt256_nn_ktail"
     assert pick(4096, 4099, 4096) == "maize_gemm_bf16_wave32"
     assert pick(33, 17, 65) == "maize_gemm_bf16_wave32"
+
+
+# ---- tail splitting of the tiled kernels -----------------------------------------------------
+
+@pytest.mark.parametrize("shape,layout", [((4096, 4104, 512), mz.LAYOUT_NN), ((4100, 4096, 1024), mz.LAYOUT_NN),
+                                          ((4128, 4096, 576), mz.LAYOUT_NT), ((4090, 4120, 1000), mz.LAYOUT_NN),
+                                          ((520, 264, 2048), mz.LAYOUT_NN)],
+                         ids=["edge_col", "edge_row", "edge_row_nt", "edge_col_ktail", "forced_small"])
+def test_edge_tiles_split_over_k(ctx, oracle, shape, layout):
+    """A ragged last tile column (or row) that pushes the tile count past the CU count: the dispatcher
+    gives each edge tile several K ranges, combined through the workspace in range order.  Checked in
+    full against the oracle and twice (the ticket counters must be back at zero).  The last case is
+    too small for the dispatcher to split: it only runs the _edge kernels unsplit, through kernels_for."""
+    m, n, k = shape
+    a, b = inputs(m, n, k)
+    bs = b if layout == mz.LAYOUT_NN else b.reshape(k, n).T.copy().ravel()
+    for kern in [x for x in kernels_for(dict(m=m, n=n, k=k, layout=layout)) if x is None or x.endswith("_edge")]:
+        _say(f"edge split: {shape} layout={layout} kernel={kern}")
+        got = run_gemm(ctx, a, bs, m, n, k, layout=layout, kernel=kern)
+        check_against_oracle(oracle, got, a, bs, m, n, k, layout=layout, label=f"edge split {shape} {kern}")
+        assert np.array_equal(run_gemm(ctx, a, bs, m, n, k, layout=layout, kernel=kern), got)
