@@ -61,6 +61,10 @@ constexpr uint32_t OOB = 0x80000000u;   // OR-ed into an offset: >= num_records,
 #define MAIZE_MT256_SCHED {1, 3, 5, 7, 9, 11, 13, 15, 17, 19, 21, 23, 25, 27, 29, 31}
 #endif
 constexpr int kIssueSlot[16] = MAIZE_MT256_SCHED;
+// Cache policy bits of the direct-to-LDS loads (bit 0 sc0, bit 1 nt, bit 4 sc1).
+#ifndef MAIZE_MT256_DMA_AUX
+#define MAIZE_MT256_DMA_AUX 0
+#endif
 constexpr int early_pieces() { int n = 0; for (int i = 0; i < 16; ++i) n += kIssueSlot[i] < 16; return n; }
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
@@ -189,11 +193,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(is_a ? (const void*)Ag : (const void*)Bg, bytes);
         if (!KTAIL) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i],
-                                                     k * (is_a ? 2u : b_kscale), 0, 0);
+                                                     k * (is_a ? 2u : b_kscale), 0, MAIZE_MT256_DMA_AUX);
         } else {
             uint32_t off = (is_a ? a_vo[i] : b_vo[i]) + k * (is_a ? 2u : b_kscale);
             if (is_a || NT) off |= (a_k[i & 1] + k) < K ? 0u : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, off, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, off, 0, 0, MAIZE_MT256_DMA_AUX);
         }
     };
 
@@ -400,7 +404,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         u32x4 v = *(lds_v4)(cw + row * 256u + ((cc ^ (row & 15u)) * 16u));
         if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
         const uint32_t grow = m0 + wm * 128u + row;
-        if (col_ok && grow < M) *(u32x4*)(Cg + (uint64_t)grow * N + gcol) = v;
+        // C is written once and not read again by this kernel: non-temporal stores keep it from
+        // displacing the operand panels in L2.
+        if (col_ok && grow < M) __builtin_nontemporal_store(v, (u32x4*)(Cg + (uint64_t)grow * N + gcol));
     }
 }
 
