@@ -147,6 +147,23 @@ int32_t maize_hip_gemm_bf16_with(maize_ctx_t* ctx, const maize_gemm_desc_t* desc
                                  const char* kernel, void* stream);
 /* Which kernel maize_hip_gemm_bf16 would pick; writes a NUL-terminated name. */
 int32_t maize_hip_gemm_select(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, char* name, size_t cap);
+/* Launch geometry for `desc` on a device with `compute_units` compute units (no device access):
+ * which kernel (`kernel` == NULL: the dispatcher's choice), its grid and block, the number of K
+ * ranges of a split kernel and the bytes of library-owned workspace the launch uses.  This is
+ * the decision the reference's panel iterators make when they turn extents and a grid into
+ * per-block work (crates/maize_tile/src/gmem/row_panel.rs:85-127, col_panel.rs:88-124). */
+typedef struct {
+    char kernel[64];
+    uint32_t grid[3];
+    uint32_t block[3];
+    uint32_t lds_bytes;     /* dynamic LDS (the kernels here use static LDS: 0) */
+    uint32_t ksplit;        /* K ranges per split tile / slab; 0 or 1 = no split */
+    uint32_t split_first;   /* tiled kernels: edge mode << 30 | 1 + tiles computed whole; 0 = all whole */
+    uint32_t reserved;
+    uint64_t workspace_bytes;
+} maize_gemm_plan_t;
+int32_t maize_hip_gemm_plan(const maize_gemm_desc_t* desc, const char* kernel, uint32_t compute_units,
+                            maize_gemm_plan_t* out);
 /* Validation only (no device access): the checks gemm_bf16 performs first. */
 int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* desc);
 /* Enumerates the GEMM kernels of the embedded code object. */

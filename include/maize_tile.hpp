@@ -95,6 +95,13 @@ inline maize_gemm_desc_t gemm_desc(const Matrix& a, const Matrix& b, const Matri
 }
 
 // C = A.B through the dispatcher: the reference's mainloop entry, carried through to a launch.
+// Kernel choice and launch geometry for a descriptor; needs no device.
+inline maize_gemm_plan_t gemm_plan(const maize_gemm_desc_t& d, uint32_t compute_units = 256, const char* kernel = nullptr) {
+    maize_gemm_plan_t p;
+    check(maize_hip_gemm_plan(&d, kernel, compute_units, &p));
+    return p;
+}
+
 inline void gemm_smem_multibuffer(Ctx& ctx, const Matrix& a, const Matrix& b, const Matrix& c, Layout layout = Layout::NN,
                                   void* stream = nullptr) {
     const maize_gemm_desc_t d = gemm_desc(a, b, c, layout);

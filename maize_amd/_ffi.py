@@ -15,7 +15,7 @@ EXPORTS = (
     "maize_hip_last_error", "maize_hip_ctx_create", "maize_hip_ctx_destroy", "maize_hip_device_info",
     "maize_hip_module_load", "maize_hip_module_unload", "maize_hip_kernel_get", "maize_hip_kernel_release",
     "maize_hip_launch", "maize_hip_embedded_code_object", "maize_hip_gemm_bf16", "maize_hip_gemm_bf16_with",
-    "maize_hip_gemm_select", "maize_hip_gemm_validate", "maize_hip_kernel_count", "maize_hip_kernel_name",
+    "maize_hip_gemm_select", "maize_hip_gemm_plan", "maize_hip_gemm_validate", "maize_hip_kernel_count", "maize_hip_kernel_name",
     "maize_hip_kernel_supports", "maize_hip_malloc", "maize_hip_free", "maize_hip_memcpy_h2d",
     "maize_hip_memcpy_d2h", "maize_hip_memset", "maize_hip_stream_create", "maize_hip_stream_destroy",
     "maize_hip_sync", "maize_hip_event_create", "maize_hip_event_record", "maize_hip_event_synchronize",
@@ -61,6 +61,14 @@ class DeviceInfoT(C.Structure):
                 ("lds_bytes_per_block", C.c_uint32), ("wavefront_size", C.c_uint32), ("hbm_bytes", C.c_uint64)]
 
 
+class GemmPlanT(C.Structure):
+    """maize_gemm_plan_t: kernel choice and launch geometry for one descriptor."""
+    _fields_ = [("kernel", C.c_char * 64), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3),
+                ("lds_bytes", C.c_uint32), ("ksplit", C.c_uint32), ("split_first", C.c_uint32),
+                ("reserved", C.c_uint32), ("workspace_bytes", C.c_uint64)]
+
+
+assert C.sizeof(GemmPlanT) == 112
 assert C.sizeof(MatrixT) == 16 and C.sizeof(GemmArgsT) == 96 and C.sizeof(GemmDescT) == 80
 
 _lib = None
@@ -92,6 +100,7 @@ def lib():
         "maize_hip_gemm_bf16": (i32, [vp, P(GemmDescT), vp]),
         "maize_hip_gemm_bf16_with": (i32, [vp, P(GemmDescT), C.c_char_p, vp]),
         "maize_hip_gemm_select": (i32, [vp, P(GemmDescT), C.c_char_p, sz]),
+        "maize_hip_gemm_plan": (i32, [P(GemmDescT), C.c_char_p, u32, P(GemmPlanT)]),
         "maize_hip_gemm_validate": (i32, [P(GemmDescT)]),
         "maize_hip_kernel_count": (u32, []),
         "maize_hip_kernel_name": (C.c_char_p, [u32]),

@@ -193,6 +193,14 @@ def validate(desc):
     check(_ffi.lib().maize_hip_gemm_validate(C.byref(desc)))
 
 
+def gemm_plan(desc, kernel=None, compute_units=256):
+    """Kernel choice and launch geometry for ``desc`` (no device needed); a dict."""
+    out = _ffi.GemmPlanT()
+    check(_ffi.lib().maize_hip_gemm_plan(C.byref(desc), kernel.encode() if kernel else None, compute_units, C.byref(out)))
+    return {"kernel": out.kernel.decode(), "grid": tuple(out.grid), "block": tuple(out.block), "lds_bytes": out.lds_bytes,
+            "ksplit": out.ksplit, "split_first": out.split_first, "workspace_bytes": out.workspace_bytes}
+
+
 def kernel_names():
     L = _ffi.lib()
     return [L.maize_hip_kernel_name(i).decode() for i in range(L.maize_hip_kernel_count())]

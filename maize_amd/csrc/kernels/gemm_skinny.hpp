@@ -223,13 +223,26 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     {
         const uint32_t row = tid >> 5, cq = (tid & 31u) * 8u;     // 512 threads x 8 columns = 16 x 256
         const uint32_t off = tile0 + (row * SN + cq) * 4u;
-        floatx4 s_lo = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off, 0, COHERENT));
-        floatx4 s_hi = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off + 16u, 0, COHERENT));
-        for (uint32_t zz = 1; zz < ks; ++zz) {
-            const floatx4 t_lo = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off + zz * TILE_BYTES, 0, COHERENT));
-            const floatx4 t_hi = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off + zz * TILE_BYTES + 16u, 0, COHERENT));
+        // The partial tiles are requested four splits at a time, so a slab pays one memory round
+        // trip per group rather than one per split; the additions still run in split order.
+        constexpr uint32_t DROP = 0xFFFFFFE0u;                    // past the descriptor: reads as zeros
+        floatx4 s_lo = floatx4{0.f, 0.f, 0.f, 0.f}, s_hi = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (uint32_t z0 = 0; z0 < ks; z0 += 4u) {
+            floatx4 t_lo[4], t_hi[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { s_lo[e] += t_lo[e]; s_hi[e] += t_hi[e]; }
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t o = z0 + u < ks ? off + (z0 + u) * TILE_BYTES : DROP;
+                t_lo[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o, 0, COHERENT));
+                t_hi[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o + 16u, 0, COHERENT));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (z0 + u == 0u) { s_lo = t_lo[0]; s_hi = t_hi[0]; }
+                else if (z0 + u < ks) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { s_lo[e] += t_lo[u][e]; s_hi[e] += t_hi[u][e]; }
+                }
+            }
         }
         const uint32_t col = n0 + cq;
         if (row < M && col < N) {                          // N % 8 == 0: 8 columns are all in or all out

@@ -268,6 +268,34 @@ int32_t maize_hip_kernel_supports(const char* kernel, const maize_gemm_desc_t* d
     return maize::kernel_at((uint32_t)idx).supports(*desc) ? 1 : 0;
 }
 
+int32_t maize_hip_gemm_plan(const maize_gemm_desc_t* desc, const char* kernel, uint32_t compute_units,
+                            maize_gemm_plan_t* out) {
+    if (!out) return fail(MAIZE_ERR_NULL, "gemm_plan: NULL argument");
+    int32_t rc = maize_hip_gemm_validate(desc);
+    if (rc != MAIZE_OK) return rc;
+    if (compute_units == 0) return fail(MAIZE_ERR_ARG, "gemm_plan: compute_units must be positive");
+    int idx;
+    if (kernel) {
+        idx = maize::kernel_index(kernel);
+        if (idx < 0) return fail(MAIZE_ERR_KERNEL, "gemm_plan: unknown kernel '%s'", kernel);
+        if (!maize::kernel_at((uint32_t)idx).supports(*desc))
+            return fail(MAIZE_ERR_KERNEL, "gemm_plan: kernel '%s' cannot run this descriptor", kernel);
+    } else {
+        idx = (int)maize::select_kernel(*desc, compute_units);
+    }
+    const maize::KernelInfo& ki = maize::kernel_at((uint32_t)idx);
+    maize::LaunchDims ld;
+    if (!ki.plan(*desc, compute_units, &ld)) return fail(MAIZE_ERR_SHAPE, "gemm_plan: grid of '%s' exceeds the launch limits", ki.name);
+    memset(out, 0, sizeof(*out));
+    snprintf(out->kernel, sizeof(out->kernel), "%s", ki.name);
+    for (int i = 0; i < 3; ++i) { out->grid[i] = ld.grid[i]; out->block[i] = ld.block[i]; }
+    out->lds_bytes = ld.lds_bytes;
+    out->ksplit = ld.ksplit;
+    out->split_first = ld.split_first;
+    out->workspace_bytes = ld.workspace_bytes;
+    return MAIZE_OK;
+}
+
 int32_t maize_hip_gemm_select(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, char* name, size_t cap) {
     if (!ctx || !name || cap == 0) return fail(MAIZE_ERR_NULL, "gemm_select: NULL argument");
     int32_t rc = maize_hip_gemm_validate(desc);

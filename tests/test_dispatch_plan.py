@@ -1,0 +1,148 @@
+"""CPU-only checks of the dispatcher: for a sweep of descriptors, the kernel it picks accepts
+the descriptor, the grid covers every output tile exactly once, split-K geometry leaves no
+empty or over-long K range, and the workspace the library allocates is at least what the
+kernels address.  These are the memory-safety preconditions of the hand-written kernels; no
+device is touched (maize_hip_gemm_plan needs none)."""
+import itertools
+
+import pytest
+
+import maize_amd as mz
+from maize_amd import _ffi
+
+TICKET_BYTES = 16384 * 4
+CUS = 256
+
+
+def desc(m, n, k, layout=mz.LAYOUT_NN, batch=1, base=0x10000):
+    a = mz.GlobalMatrix(base, m, k)
+    b = mz.GlobalMatrix(base + (1 << 32), k, n) if layout == mz.LAYOUT_NN else mz.GlobalMatrix(base + (1 << 32), n, k)
+    c = mz.GlobalMatrix(base + (2 << 32), m, n)
+    return mz.gemm_desc(a, b, c, layout=layout, batch=batch, stride_a=m * k, stride_b=k * n, stride_c=m * n)
+
+
+def cdiv(a, b):
+    return (a + b - 1) // b
+
+
+SHAPES = [
+    (4096, 4096, 4096), (4000, 4104, 4032), (8192, 8192, 8192), (16, 14336, 4096), (2048, 2048, 2048),
+    (1, 1, 1), (33, 17, 65), (128, 128, 64), (256, 256, 64), (257, 264, 72), (4096, 4104, 256), (4128, 4096, 4096),
+    (4104, 4096, 512), (16, 64, 256), (16, 56, 256), (8, 512, 8192), (16, 14336, 4128), (16, 28672, 16384),
+    (300, 4000, 40), (4096, 8, 4096), (8, 8, 8), (1024, 1032, 1024), (8200, 4096, 2048), (4096, 8200, 2048),
+]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("batch", [1, 3])
+def test_selected_kernel_supports_the_descriptor_and_its_grid_covers_c(m, n, k, layout, batch):
+    d = desc(m, n, k, layout, batch)
+    p = mz.gemm_plan(d, compute_units=CUS)
+    assert p["kernel"] in mz.kernel_names()
+    assert mz.kernel_supports(p["kernel"], d)
+    check_plan(p, m, n, k, layout, batch)
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+def test_every_kernel_that_accepts_a_descriptor_plans_a_covering_grid(m, n, k, layout):
+    d = desc(m, n, k, layout)
+    for name in mz.kernel_names():
+        if not mz.kernel_supports(name, d):
+            with pytest.raises(mz.MaizeError):
+                mz.gemm_plan(d, kernel=name, compute_units=CUS)
+            continue
+        for cus in (1, 8, 80, 256, 304):
+            check_plan(mz.gemm_plan(d, kernel=name, compute_units=cus), m, n, k, layout, 1)
+
+
+def check_plan(p, m, n, k, layout, batch):
+    gx, gy, gz = p["grid"]
+    assert gx >= 1 and gy >= 1 and gz == batch
+    assert gy <= 65535 and gz <= 65535 and gx < (1 << 31)
+    name = p["kernel"]
+    if name == "maize_gemm_bf16_wave32":
+        assert p["block"] == (256, 1, 1)
+        assert gx == cdiv(n, 64) and gy == cdiv(m, 64)
+        assert p["workspace_bytes"] == 0 and p["ksplit"] == 0
+    elif name.startswith("maize_gemm_bf16_mt256"):
+        assert p["block"] == (256, 1, 1) and gy == 1
+        assert ("_nt" in name) == (layout == mz.LAYOUT_NT)
+        assert k % 8 == 0 and n % 8 == 0
+        if "ktail" not in name:
+            assert k % 64 == 0
+        tm, tn = cdiv(m, 256), cdiv(n, 256)
+        if p["split_first"] == 0:
+            assert gx == tm * tn and p["workspace_bytes"] == 0
+        else:
+            assert name.endswith("_edge") and batch == 1
+            mode, whole = p["split_first"] >> 30, (p["split_first"] & 0x3FFFFFFF) - 1
+            ks = p["ksplit"]
+            assert mode in (1, 2) and 2 <= ks <= 16
+            nedge = tm if mode == 1 else tn
+            assert whole == (tm * (tn - 1) if mode == 1 else (tm - 1) * tn)
+            assert gx == whole + nedge * ks
+            # the edge that is split is narrow: its partial tiles are cheap to combine
+            assert (n - (tn - 1) * 256 if mode == 1 else m - (tm - 1) * 256) <= 32
+            # K ranges: ceil(steps / ks) steps each, none empty, each at least 4 steps long
+            nk = cdiv(k, 64)
+            per = cdiv(nk, ks)
+            assert per * (ks - 1) < nk and per >= 4
+            # one ticket counter per edge tile, one fp32 tile per (edge tile, range)
+            assert nedge <= 16384
+            assert p["workspace_bytes"] >= TICKET_BYTES + nedge * ks * 256 * 256 * 4
+            assert p["workspace_bytes"] < (1 << 31)
+    elif name == "maize_gemm_bf16_skinny_nn":
+        assert p["block"] == (512, 1, 1)
+        assert layout == mz.LAYOUT_NN and m <= 16 and n % 8 == 0
+        ks = p["ksplit"]
+        assert gx == cdiv(n, 256) and gy == ks and 1 <= ks <= 16
+        assert k % (32 * ks) == 0                              # whole 32-row blocks in every range
+        if ks > 1:
+            assert k // ks // 32 >= 8                          # the 8-slot ring is filled at least once
+            assert gx * batch <= 16384                         # one ticket counter per (batch member, slab)
+            assert p["workspace_bytes"] >= TICKET_BYTES + gx * batch * ks * 16 * 256 * 4
+            assert p["workspace_bytes"] < (1 << 31)
+        else:
+            assert p["workspace_bytes"] == 0
+    else:
+        raise AssertionError(f"no invariants written for kernel {name}")
+
+
+def test_north_star_configurations_get_the_kernels_they_were_designed_for():
+    picks = {
+        (4096, 4096, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn",
+        (4000, 4104, 4032, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_edge",
+        (8192, 8192, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt",
+        (16, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn",
+        (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
+        (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
+    }
+    for (m, n, k, layout, batch), want in picks.items():
+        assert mz.gemm_plan(desc(m, n, k, layout, batch), compute_units=CUS)["kernel"] == want
+
+
+def test_skinny_split_fills_the_chip_without_overshooting():
+    p = mz.gemm_plan(desc(16, 14336, 4096), compute_units=CUS)
+    assert p["grid"] == (56, 4, 1)                              # 224 workgroups on 256 compute units
+    p = mz.gemm_plan(desc(16, 14336, 4096), compute_units=64)
+    assert p["grid"] == (56, 1, 1)                              # already a workgroup per compute unit
+    p = mz.gemm_plan(desc(16, 256, 8192), compute_units=CUS)
+    assert p["grid"][0] == 1 and p["ksplit"] == 16             # capped at 16 ranges
+
+
+def test_plan_rejects_bad_arguments():
+    d = desc(64, 64, 64)
+    with pytest.raises(mz.MaizeError) as e:
+        mz.gemm_plan(d, kernel="no_such_kernel")
+    assert e.value.code == _ffi.MAIZE_ERR_KERNEL
+    with pytest.raises(mz.MaizeError) as e:
+        mz.gemm_plan(d, compute_units=0)
+    assert e.value.code == _ffi.MAIZE_ERR_ARG
+    assert _ffi.lib().maize_hip_gemm_plan(None, None, 256, None) == _ffi.MAIZE_ERR_NULL
+    bad = desc(64, 64, 64)
+    bad.c.nrows = 65
+    with pytest.raises(mz.MaizeError) as e:
+        mz.gemm_plan(bad)
+    assert e.value.code == _ffi.MAIZE_ERR_SHAPE

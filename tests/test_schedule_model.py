@@ -1,0 +1,255 @@
+"""CPU model of the two LDS pipelines (prime / wait-consume-refill / drain), checked for the
+properties the reference's CpAsyncPipeline promises (crates/maize_core/src/intrinsics/cuda/
+cp_async.rs:122-210): every K tile is copied exactly once and consumed exactly once, in order,
+never before its copy has completed for every wave, and no ring slot is refilled while a wave
+may still be reading it.
+
+The model replays each wave's instruction stream as the kernels issue it (the request slots,
+ring depth and counter waits are read from the kernel sources, not retyped here) and tracks
+barrier epochs: waves only synchronise at workgroup barriers, so an access in epoch e of one
+wave can race with any access in epoch e of another.  A direct-to-LDS request issued in epoch e
+is complete for everyone from epoch e+1 on only if the wave waited for it before the barrier.
+Mutated schedules (a late barrier, a short counter wait, a request slot past the barrier) must
+be rejected, which shows the checks have teeth."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+KDIR = os.path.join(ROOT, "maize_amd", "csrc", "kernels")
+
+
+class Hazard(AssertionError):
+    pass
+
+
+# ---------------------------------------------------------------------------------------
+# macro-tile kernel: two-stage ring, 16 requests per tile per wave spread over MFMA slots
+# ---------------------------------------------------------------------------------------
+
+def mt256_issue_slots():
+    src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
+    m = re.search(r"#define MAIZE_MT256_SCHED \{([0-9,\s]+)\}", src)
+    slots = [int(x) for x in m.group(1).split(",")]
+    assert len(slots) == 16
+    return slots
+
+
+def mt256_wave_program(nk, slots, nreads, barrier_quarter=3):
+    """Instruction stream of one wave for nk K tiles: a list of
+    ("dma", tile, piece, stage) | ("wait_all",) | ("barrier",) | ("read", tile, quarter, stage) | ("mfma", tile, quarter)."""
+    ops = []
+    for pc in range(16):
+        ops.append(("dma", 0, pc, 0))
+    ops += [("wait_all",), ("barrier",)]
+    ops += [("read", 0, 0, 0)] * nreads
+    early = [pc for pc in range(16) if slots[pc] < 16]
+    for pc in early:
+        ops.append(("dma", 1, pc, 1))
+    k_early, k_late = 2, 1
+    steps = nk + (nk & 1)                                   # the loop body holds two steps
+    for t in range(steps):
+        cur, nxt = t & 1, (t & 1) ^ 1
+        for kk in range(4):
+            if kk == barrier_quarter:
+                ops += [("wait_all",), ("barrier",)]
+            for s in range(16):
+                ops.append(("mfma", t, kk))
+                if s < nreads:
+                    ops.append(("read", t, kk + 1, cur) if kk < 3 else ("read", t + 1, 0, nxt))
+                slot = s if kk == 3 else 16 * (kk + 1) + s
+                for pc in range(16):
+                    if slots[pc] == slot:
+                        ops.append(("dma", k_early, pc, cur) if kk == 3 else ("dma", k_late, pc, nxt))
+        k_early += 1
+        k_late += 1
+    ops.append(("wait_all",))
+    return ops, steps
+
+
+def check_two_stage(ops, steps, nreads):
+    epoch = 0
+    dma_epoch = {}          # (tile, piece) -> epoch of issue
+    completed = set()       # (tile, piece) waited for by this wave
+    pending = []
+    visible_from = {}       # (tile, piece) -> first epoch in which every wave may read it
+    last_read_epoch = {}    # tile -> epoch of its last fragment read
+    stage_of = {}
+    reads_seen = {}
+    consumed = []
+    for op in ops:
+        if op[0] == "dma":
+            _, tile, pc, stage = op
+            if (tile, pc) in dma_epoch:
+                raise Hazard(f"piece {pc} of tile {tile} requested twice")
+            if stage != tile % 2:
+                raise Hazard(f"tile {tile} requested into stage {stage}")
+            # WAR: the stage still holds tile-2; every wave must be past its last read of it
+            old = tile - 2
+            if old >= 0 and last_read_epoch.get(old, -1) >= epoch:
+                raise Hazard(f"tile {tile} piece {pc} overwrites tile {old} in epoch {epoch}, still being read")
+            if old >= 0 and old < steps and reads_seen.get(old, 0) < 4 * nreads:
+                raise Hazard(f"tile {tile} overwrites tile {old} before all of its fragments were read")
+            dma_epoch[(tile, pc)] = epoch
+            stage_of[tile] = stage
+            pending.append((tile, pc))
+        elif op[0] == "wait_all":
+            completed.update(pending)
+            pending = []
+        elif op[0] == "barrier":
+            if pending:
+                raise Hazard("barrier with requests of this wave still in flight")
+            epoch += 1
+            for key in completed:
+                visible_from.setdefault(key, epoch)
+        elif op[0] == "read":
+            _, tile, quarter, stage = op
+            if stage != tile % 2:
+                raise Hazard(f"tile {tile} read from stage {stage}")
+            for pc in range(16):
+                if visible_from.get((tile, pc), 1 << 30) > epoch:
+                    raise Hazard(f"tile {tile} quarter {quarter} read in epoch {epoch} before piece {pc} is complete")
+            last_read_epoch[tile] = epoch
+            reads_seen[tile] = reads_seen.get(tile, 0) + 1
+        elif op[0] == "mfma":
+            _, tile, quarter = op
+            if reads_seen.get(tile, 0) < (quarter + 1) * nreads:
+                raise Hazard(f"tile {tile} quarter {quarter} multiplied before its fragments were read")
+            if not consumed or consumed[-1] != (tile, quarter):
+                consumed.append((tile, quarter))
+    if pending:
+        raise Hazard("requests still in flight at the end of the K loop")
+    want = [(t, q) for t in range(steps) for q in range(4)]
+    if consumed != want:
+        raise Hazard("K tiles not consumed exactly once, in order")
+    for t in range(steps + 1):
+        got = sorted(pc for (tile, pc) in dma_epoch if tile == t)
+        if t < steps and got != list(range(16)):
+            raise Hazard(f"tile {t}: pieces requested {got}")
+    return max(t for (t, _) in dma_epoch)
+
+
+@pytest.mark.parametrize("nk", [1, 2, 3, 7, 64])
+@pytest.mark.parametrize("nreads", [8, 12])
+def test_macro_tile_schedule_is_hazard_free(nk, nreads):
+    slots = mt256_issue_slots()
+    assert all(0 <= s < 64 for s in slots), "every request of tile t+2 must be issued before the barrier of step t+1"
+    ops, steps = mt256_wave_program(nk, slots, nreads)
+    last_tile = check_two_stage(ops, steps, nreads)
+    # tiles past the end are requested (through a zero-length descriptor) but never multiplied
+    assert steps <= last_tile <= steps + 1
+
+
+def test_macro_tile_checker_rejects_broken_schedules():
+    slots = mt256_issue_slots()
+    # barrier one quarter early: fragments of the current tile are still being read behind it
+    ops, steps = mt256_wave_program(8, slots, 8, barrier_quarter=2)
+    with pytest.raises(Hazard):
+        check_two_stage(ops, steps, 8)
+    # a request scheduled past the next barrier never gets issued
+    bad = list(slots)
+    bad[5] = 64
+    ops, steps = mt256_wave_program(8, bad, 8)
+    with pytest.raises(Hazard):
+        check_two_stage(ops, steps, 8)
+    # a missing wait before the barrier: data not guaranteed to have landed
+    ops, steps = mt256_wave_program(8, slots, 8)
+    k = [i for i, o in enumerate(ops) if o == ("wait_all",)][3]
+    with pytest.raises(Hazard):
+        check_two_stage(ops[:k] + ops[k + 1:], steps, 8)
+
+
+# ---------------------------------------------------------------------------------------
+# skinny kernel: 8-slot ring, 3 loads per block per wave, counter wait instead of wait-all
+# ---------------------------------------------------------------------------------------
+
+def skinny_constants():
+    src = open(os.path.join(KDIR, "gemm_skinny.hpp")).read()
+    ring = int(re.search(r"constexpr int RING = (\d+);", src).group(1))
+    waits = [int(x) for x in re.findall(r"s_waitcnt vmcnt\((\d+)\)\\n\\ts_barrier", src)]
+    assert len(waits) == 1
+    primed = len(re.findall(r"request\(\d+, s\d+, \d+\);", src))
+    return ring, waits[0], primed
+
+
+def skinny_wave_program(nb, ring, wait, primed, loads_per_request=3):
+    ops = []
+    for j in range(primed):
+        ops.append(("request", j, j % ring))
+    turns = -(-nb // ring) * ring
+    for b in range(turns):
+        ops += [("wait", wait), ("barrier",)]
+        ops.append(("request", b + primed, (b + primed) % ring))
+        ops.append(("consume", b, b % ring))
+    ops.append(("wait", 0))
+    return ops, turns, loads_per_request
+
+
+def check_ring(ops, turns, loads_per_request, ring):
+    epoch = 0
+    issued = []                 # blocks in request order (each stands for loads_per_request loads)
+    done = 0                    # number of requests known complete for this wave
+    visible_from = {}
+    consumed_epoch = {}
+    slot_holds = {}
+    consumed = []
+    for op in ops:
+        if op[0] == "request":
+            _, blk, slot = op
+            old = slot_holds.get(slot)
+            if old is not None:
+                if old not in consumed_epoch:
+                    raise Hazard(f"block {blk} overwrites block {old}, never consumed")
+                if consumed_epoch[old] >= epoch:
+                    raise Hazard(f"block {blk} overwrites block {old} in the epoch it is read in")
+            slot_holds[slot] = blk
+            issued.append(blk)
+        elif op[0] == "wait":
+            # the counter retires loads in order: at most op[1] of the newest may be outstanding
+            outstanding_requests = -(-op[1] // loads_per_request)
+            done = max(done, len(issued) - outstanding_requests)
+        elif op[0] == "barrier":
+            epoch += 1
+            for blk in issued[:done]:
+                visible_from.setdefault(blk, epoch)
+        elif op[0] == "consume":
+            _, blk, slot = op
+            if slot_holds.get(slot) != blk:
+                raise Hazard(f"block {blk} expected in slot {slot}, which holds {slot_holds.get(slot)}")
+            if visible_from.get(blk, 1 << 30) > epoch:
+                raise Hazard(f"block {blk} consumed in epoch {epoch} before every wave's share has landed")
+            consumed_epoch[blk] = epoch
+            consumed.append(blk)
+    if done != len(issued):
+        raise Hazard("loads still in flight at the end")
+    if consumed != list(range(turns)):
+        raise Hazard("blocks not consumed exactly once, in order")
+    if sorted(issued) != list(range(len(issued))):
+        raise Hazard("blocks not requested exactly once")
+
+
+@pytest.mark.parametrize("nb", [8, 16, 32, 128, 9])
+def test_skinny_ring_is_hazard_free(nb):
+    ring, wait, primed = skinny_constants()
+    assert primed == ring - 1
+    ops, turns, lpr = skinny_wave_program(nb, ring, wait, primed)
+    check_ring(ops, turns, lpr, ring)
+    # the wait leaves exactly the requests of the blocks behind the current one in flight
+    assert wait == lpr * (primed - 1)
+
+
+def test_skinny_checker_rejects_broken_rings():
+    ring, wait, primed = skinny_constants()
+    ops, turns, lpr = skinny_wave_program(32, ring, wait + 3, primed)       # waits for one request too few
+    with pytest.raises(Hazard):
+        check_ring(ops, turns, lpr, ring)
+    ops, turns, lpr = skinny_wave_program(32, ring - 1, wait, primed)        # ring one slot short: refill hits the block being read
+    with pytest.raises(Hazard):
+        check_ring(ops, turns, lpr, ring - 1)
+    ops, turns, lpr = skinny_wave_program(32, ring, wait, primed)
+    swapped = [o for o in ops]
+    i = next(k for k, o in enumerate(swapped) if o[0] == "barrier")
+    del swapped[i]                                                         # first barrier missing
+    with pytest.raises(Hazard):
+        check_ring(swapped, turns, lpr, ring)
