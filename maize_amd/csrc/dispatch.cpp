@@ -80,9 +80,21 @@ bool mt256_plan_impl(const maize_gemm_desc_t& d, uint32_t compute_units, bool al
     if (tiles > 0x1FFFFFFFull) return false;
     EdgeSplit e = mt256_edge(s, d.batch, compute_units);
     if (!allow_edge) e = EdgeSplit{0, (uint32_t)tiles, 0, 0};
-    ld->grid[0] = e.mode ? e.whole + e.nedge * e.ks : (uint32_t)tiles;
+    if (allow_edge) {
+        // The edge-splitting kernels compute one tile, or one K range of an edge tile, per workgroup.
+        ld->grid[0] = e.mode ? e.whole + e.nedge * e.ks : (uint32_t)tiles;
+        ld->grid[2] = d.batch;
+    } else {
+        // Persistent: one workgroup per compute unit walks the list of all tiles of all batch
+        // members (a multiple of 8 workgroups, so that the tiles one XCD works on at a time stay
+        // neighbours); with fewer tiles than compute units, one workgroup per tile.
+        const uint64_t all = tiles * d.batch;
+        if (all > 0x1FFFFFFFull) return false;
+        uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+        ld->grid[0] = (resident && all > resident) ? resident : (uint32_t)all;
+        ld->grid[2] = 1;
+    }
     ld->grid[1] = 1;
-    ld->grid[2] = d.batch;
     ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;  // static LDS
     ld->ksplit = e.ks;

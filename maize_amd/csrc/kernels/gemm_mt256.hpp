@@ -114,6 +114,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     __shared__ __attribute__((aligned(1024))) char lds_a1[TILE];
     __shared__ __attribute__((aligned(1024))) char lds_b0[TILE];
     __shared__ __attribute__((aligned(1024))) char lds_b1[TILE];
+    // Epilogue staging (8 KiB per wave), apart from the operand stages so that the first K tile
+    // of the workgroup's next C tile can land while this one is converted and stored.
+    __shared__ __attribute__((aligned(1024))) char lds_e[TILE];
     lds_ptr const A0 = (lds_ptr)lds_a0, A1 = (lds_ptr)lds_a1, B0 = (lds_ptr)lds_b0, B1 = (lds_ptr)lds_b1;
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
@@ -133,14 +136,6 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t ks = split ? p.ksplit : 1u;
     const uint32_t edge = split ? (blockIdx.x - whole) / ks : 0u;     // which edge tile
     const uint32_t z = split ? (blockIdx.x - whole) % ks : 0u;        // which K range
-    uint32_t tile_m, tile_n;
-    if (!split) {
-        tile_of(xcd_run(blockIdx.x, whole), tm - (mode == 2u), tn - (mode == 1u), &tile_m, &tile_n);
-    } else {
-        tile_m = mode == 1u ? edge : tm - 1u;
-        tile_n = mode == 1u ? tn - 1u : edge;
-    }
-    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     // K steps of this workgroup: [kt0, kt0 + nk) of the ceil(K / BK) steps.
     const uint32_t nk_all = (K + BK - 1) / BK;
     const uint32_t per_range = (nk_all + ks - 1u) / ks;
@@ -148,39 +143,71 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t nk = kt0 < nk_all ? (nk_all - kt0 < per_range ? nk_all - kt0 : per_range) : 0u;
     const uint32_t k_begin = kt0 * BK;
     const uint32_t k_end = (kt0 + nk) * BK < K ? (kt0 + nk) * BK : K;   // loads at or past k_end return zeros
-
-    const uint64_t bz = blockIdx.z;
-    const uint16_t* Ag = p.a + bz * p.stride_a;
-    const uint16_t* Bg = p.b + bz * p.stride_b;
-    uint16_t* Cg = p.c + bz * p.stride_c;
     const uint32_t a_bytes = M * K * 2u, b_bytes = N * K * 2u;
 
-    // ---- global -> LDS copy maps (direct-to-LDS buffer loads) -----------------------
-    // One wave-wide 128-bit load deposits 1 KiB contiguously in LDS (lane l at byte 16*l),
-    // so the swizzle is applied on the global side: lane l fetches the chunk whose swizzled
-    // home is position l.  Wave w issues pieces w*8 .. w*8+7 of each operand tile.
+    // The plain kernels are persistent: the grid is one workgroup per compute unit (or one per
+    // tile if there are fewer), workgroup g computes tiles g, g + grid, g + 2 grid, ... of the
+    // list of all tiles of all batch members.  The edge-splitting kernels compute one tile (or
+    // one K range of one) per workgroup.
+    const uint32_t tiles_per = tm * tn;
+    const uint32_t total = EDGE ? gridDim.x : tiles_per * p.batch;
+    uint32_t pid = blockIdx.x;
+    if (pid >= total) return;
+
+    // ---- per-tile state ---------------------------------------------------------------
+    // global -> LDS copy maps (direct-to-LDS buffer loads).  One wave-wide 128-bit load deposits
+    // 1 KiB contiguously in LDS (lane l at byte 16*l), so the swizzle is applied on the global
+    // side: lane l fetches the chunk whose swizzled home is position l.  Wave w issues pieces
+    // w*8 .. w*8+7 of each operand tile.
     //   K-contiguous tile (A, and B when NT): piece = 8 rows of 128 B; position l -> row l/8,
     //     stored chunk l%8 = logical chunk ^ ((row>>1)&7).
     //   K x N tile (B when NN): piece = 2 rows of 512 B; position l -> row l/32, stored chunk
     //     l%32 = logical chunk ^ ((row&3)<<2).
     // vo = byte offset of the lane's chunk at k = 0 (with the N-edge mask folded in); the K
     // advance is a scalar offset (plain kernels) or added per lane (K-tail kernels).
+    uint32_t m0, n0;
+    const uint16_t* Ag;
+    const uint16_t* Bg;
+    uint16_t* Cg;
     uint32_t a_vo[8], b_vo[8];
     uint32_t a_k[2];                      // k index of the lane's chunk inside a tile, even/odd piece (K masks)
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t row = (wave * 8u + i) * 8u + (lane >> 3);
-        const uint32_t c = (lane & 7u) ^ ((row >> 1) & 7u);
-        a_vo[i] = ((m0 + row) * K + c * 8u) * 2u;
-        if (i < 2) a_k[i] = c * 8u;
-        if (NT) {
-            b_vo[i] = ((n0 + row) * K + c * 8u) * 2u;
+    auto select_tile = [&](uint32_t id) {
+        uint32_t tile_m, tile_n;
+        uint64_t bz;
+        if (EDGE) {
+            bz = blockIdx.z;
+            if (!split) {
+                tile_of(xcd_run(id, whole), tm - (mode == 2u), tn - (mode == 1u), &tile_m, &tile_n);
+            } else {
+                tile_m = mode == 1u ? edge : tm - 1u;
+                tile_n = mode == 1u ? tn - 1u : edge;
+            }
         } else {
-            const uint32_t brow = (wave * 8u + i) * 2u + (lane >> 5);
-            const uint32_t bc = (lane & 31u) ^ ((brow & 3u) << 2);
-            b_vo[i] = ((brow * N + n0 + bc * 8u) * 2u) | ((n0 + bc * 8u) < N ? 0u : OOB);
+            const uint32_t t = xcd_run(id, total);
+            bz = t / tiles_per;
+            tile_of(t - (uint32_t)bz * tiles_per, tm, tn, &tile_m, &tile_n);
         }
-    }
+        m0 = tile_m * BM;
+        n0 = tile_n * BN;
+        Ag = p.a + bz * p.stride_a;
+        Bg = p.b + bz * p.stride_b;
+        Cg = p.c + bz * p.stride_c;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t row = (wave * 8u + i) * 8u + (lane >> 3);
+            const uint32_t c = (lane & 7u) ^ ((row >> 1) & 7u);
+            a_vo[i] = ((m0 + row) * K + c * 8u) * 2u;
+            if (i < 2) a_k[i] = c * 8u;
+            if (NT) {
+                b_vo[i] = ((n0 + row) * K + c * 8u) * 2u;
+            } else {
+                const uint32_t brow = (wave * 8u + i) * 2u + (lane >> 5);
+                const uint32_t bc = (lane & 31u) ^ ((brow & 3u) << 2);
+                b_vo[i] = ((brow * N + n0 + bc * 8u) * 2u) | ((n0 + bc * 8u) < N ? 0u : OOB);
+            }
+        }
+    };
+    select_tile(pid);
     const uint32_t b_kscale = NT ? 2u : N * 2u;    // bytes per unit of k in B
     // Issues piece pc (0..7 = A, 8..15 = B) of the tile that starts at k into stages (sa, sb).
     auto dma = [&](int pc, lds_ptr sa, lds_ptr sb, uint32_t k) {
@@ -252,23 +279,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     };
 
     floatx16 acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-    // ---- prime ---------------------------------------------------------------------
-#pragma unroll
-    for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, k_begin);  // tile 0, whole
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-#pragma unroll
-    for (int r = 0; r < NREADS; ++r) read_frag(0, 0, r, A0, B0);
-#pragma unroll
-    for (int pc = 0; pc < early_pieces(); ++pc) dma(pc, A1, B1, k_begin + BK);   // tile 1, early pieces
-    uint32_t k_early = k_begin + 2 * BK;   // tile whose early pieces are issued next (last quarter of a step)
-    uint32_t k_late = k_begin + BK;        // tile whose late pieces are issued next (first quarter of a step)
+    uint32_t k_early = 0;                  // tile whose early pieces are issued next (last quarter of a step)
+    uint32_t k_late = 0;                   // tile whose late pieces are issued next (first quarter of a step)
 
     // ---- steady state ----------------------------------------------------------------
     // One K step.  On entry: (ca, cb) hold tile t, fragment buffer 0 holds its quarter-0
@@ -310,35 +322,54 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         k_early += BK;
         k_late += BK;
     };
+    // ---- prime: the first K tile of the first C tile, whole ------------------------------
+#pragma unroll
+    for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, k_begin);
+
+    for (;;) {                                                  // one trip per C tile
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    // The wait also covers the C stores of the previous tile (loads and stores share the counter).
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+    for (int r = 0; r < NREADS; ++r) read_frag(0, 0, r, A0, B0);
+#pragma unroll
+    for (int pc = 0; pc < early_pieces(); ++pc) dma(pc, A1, B1, k_begin + BK);   // tile 1, early pieces
+    k_early = k_begin + 2 * BK;
+    k_late = k_begin + BK;
     // Two steps per trip so that each step sees its stages as compile-time constants.  An odd
     // step count runs one extra step on an all-zero tile (loads past K return zeros).
     for (uint32_t kt = 0; kt < nk; kt += 2) {
         step(A0, B0, A1, B1);
         step(A1, B1, A0, B0);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no direct-to-LDS write may land during the epilogue
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // every direct-to-LDS write of this tile has landed
 
     // ---- K ranges: publish the partial tile, take a ticket, last arriver sums in range order ----
+    constexpr int COHERENT = 17;                          // buffer cache policy sc0 | sc1: visible across the XCDs' L2s
+    constexpr uint32_t UNIT = BM * BN * 4u;               // one fp32 partial tile
+    constexpr uint32_t DROP = 0xFFFFFFF0u;                // out-of-range offset: store dropped, load returns zeros
+    // A partial tile is stored in register order, not row-major: chunk c = (i, j, q) of wave w is
+    // 64 lanes x 16 bytes = 1 KiB contiguous, so every store and load instruction moves whole
+    // cache lines.  Lane's chunk = row wm*128 + i*32 + l%32, columns wn*128 + j*32 + 8q + 4(l/32)
+    // + 0..3.  Chunks wholly outside the matrix are skipped (a wave-uniform test); lanes outside
+    // it inside a chunk use an out-of-range offset.
+    const uint32_t nedge = mode == 1u ? tm : tn;
+    const uint32_t slot = EDGE ? blockIdx.z * nedge + edge : 0u;
+    const __amdgpu_buffer_rsrc_t rws =
+        make_rsrc((const char*)p.workspace + 65536, (EDGE && split) ? gridDim.z * nedge * ks * UNIT : 0u);
+    const uint32_t wmu = wave_u >> 1, wnu = wave_u & 1u;
+    const uint32_t lane_off = wave_u * 65536u + lane * 16u;
+    const uint32_t rows_ok = M - m0, cols_ok = N - n0;    // valid extent of this tile (may exceed 256)
+    auto chunk_live = [&](int c) { return wmu * 128u + (c >> 4) * 32u < rows_ok && wnu * 128u + ((c >> 2) & 3) * 32u + (c & 3) * 8u < cols_ok; };
+    auto lane_live = [&](int c) { return wm * 128u + (c >> 4) * 32u + l32 < rows_ok && wn * 128u + ((c >> 2) & 3) * 32u + (c & 3) * 8u + lhi * 4u < cols_ok; };
     if (EDGE && split) {
-        constexpr int COHERENT = 17;                      // buffer cache policy sc0 | sc1: visible across the XCDs' L2s
-        constexpr uint32_t UNIT = BM * BN * 4u;           // one fp32 partial tile
-        constexpr uint32_t DROP = 0xFFFFFFF0u;            // out-of-range offset: store dropped, load returns zeros
-        __shared__ uint32_t ticket;
+        volatile uint32_t& ticket = *(volatile uint32_t*)lds_e;   // the staging region is idle until the epilogue
         uint32_t* counters = (uint32_t*)p.workspace;      // 16384 counters (zero between launches), then the tiles
-        const uint32_t nedge = mode == 1u ? tm : tn;
-        const uint32_t slot = (uint32_t)bz * nedge + edge;
-        const __amdgpu_buffer_rsrc_t rws = make_rsrc((const char*)p.workspace + 65536, gridDim.z * nedge * ks * UNIT);
-        // A partial tile is stored in register order, not row-major: chunk c = (i, j, q) of wave w is
-        // 64 lanes x 16 bytes = 1 KiB contiguous, so every store and load instruction moves whole
-        // cache lines.  Lane's chunk = row wm*128 + i*32 + l%32, columns wn*128 + j*32 + 8q + 4(l/32)
-        // + 0..3.  Chunks wholly outside the matrix are skipped (a wave-uniform test); lanes outside
-        // it inside a chunk use an out-of-range offset.
-        const uint32_t l32e = lane & 31u, lhie = lane >> 5;
-        const uint32_t wmu = wave_u >> 1, wnu = wave_u & 1u;
-        const uint32_t lane_off = wave_u * 65536u + lane * 16u;
-        const uint32_t rows_ok = M - m0, cols_ok = N - n0;    // valid extent of this tile (may exceed 256)
-        auto chunk_live = [&](int c) { return wmu * 128u + (c >> 4) * 32u < rows_ok && wnu * 128u + ((c >> 2) & 3) * 32u + (c & 3) * 8u < cols_ok; };
-        auto lane_live = [&](int c) { return wm * 128u + (c >> 4) * 32u + l32e < rows_ok && wn * 128u + ((c >> 2) & 3) * 32u + (c & 3) * 8u + lhie * 4u < cols_ok; };
 #pragma unroll
         for (int c = 0; c < 64; ++c) {
             if (!chunk_live(c)) continue;
@@ -352,62 +383,78 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         if (tid == 0) ticket = __hip_atomic_fetch_add(&counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (ticket != ks - 1u) return;                    // another workgroup will finish this tile
-        // Sum the ranges in order, chunk by chunk; the (up to 16) loads of one chunk are issued
-        // together, ranges past ksplit read zeros.
-#pragma unroll
-        for (int c = 0; c < 64; ++c) {
-            const int i = c >> 4, j = (c >> 2) & 3, q = c & 3;
-            floatx4 sum = {0.f, 0.f, 0.f, 0.f};
-            if (chunk_live(c)) {
-                const uint32_t base = lane_live(c) ? slot * ks * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
-                floatx4 t[16];
-#pragma unroll
-                for (int zz = 0; zz < 16; ++zz)
-                    t[zz] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
-                        rws, ((uint32_t)zz < ks && base != DROP) ? base + (uint32_t)zz * UNIT : DROP, 0, COHERENT));
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int zz = 0; zz < 16; ++zz) { sum[0] += t[zz][0]; sum[1] += t[zz][1]; sum[2] += t[zz][2]; sum[3] += t[zz][3]; }
-            }
-            acc[i][j][4 * q] = sum[0]; acc[i][j][4 * q + 1] = sum[1]; acc[i][j][4 * q + 2] = sum[2]; acc[i][j][4 * q + 3] = sum[3];
-        }
         if (tid == 0) counters[slot] = 0u;                // ready for the next launch
+    }
+    // The last arriver replaces each chunk of its accumulators by the sum of all ranges, in range
+    // order, as the epilogue reaches it; the loads of a chunk are issued eight ranges at a time,
+    // ranges past ksplit read zeros.
+    auto reduced_chunk = [&](int c) -> floatx4 {
+        floatx4 sum = {0.f, 0.f, 0.f, 0.f};
+        if (chunk_live(c)) {
+            const uint32_t base = lane_live(c) ? slot * ks * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
+            for (uint32_t z0 = 0; z0 < ks; z0 += 8u) {
+                floatx4 t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    t[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                        rws, (z0 + u < ks && base != DROP) ? base + (z0 + u) * UNIT : DROP, 0, COHERENT));
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { sum[0] += t[u][0]; sum[1] += t[u][1]; sum[2] += t[u][2]; sum[3] += t[u][3]; }
+            }
+        }
+        return sum;
+    };
+
+    // ---- hand-over: request the next C tile's first K tile before this one is stored -------
+    __syncthreads();                                           // all waves are done with the operand stages
+    const uint32_t em0 = m0, en0 = n0;
+    uint16_t* const Ce = Cg;
+    const uint32_t next = pid + gridDim.x;
+    const bool more = !EDGE && next < total;
+    if (more) {
+        select_tile(next);
+#pragma unroll
+        for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, k_begin);
     }
 
     // ---- epilogue: fp32 -> bf16 (RNE), stage through LDS, 128-bit row stores --------------
-    // Each wave stages its 128 x 128 sub-tile in a private 32 KiB array (row = 256 B).  The
-    // 16-byte chunk index is XOR-ed with row%16 and the 8-byte half with bit 4 of the row, so
-    // the 8-byte writes of 32 rows and the 16-byte reads of 4 rows are conflict free.
-    __syncthreads();                                           // all waves are done with the operand stages
-    lds_ptr cw = wave_u == 0 ? A0 : wave_u == 1 ? A1 : wave_u == 2 ? B0 : B1;
+    // Each wave stages its 128 x 128 sub-tile 32 rows at a time in a private 8 KiB region
+    // (row = 256 B).  The 16-byte chunk index is XOR-ed with row%16 and the 8-byte half with
+    // bit 4 of the row, so the 8-byte writes of 32 rows and the 16-byte reads of 4 rows are
+    // conflict free.  The region is wave-private and LDS operations of one wave complete in
+    // order, so no barrier is needed between the passes.
+    lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
+    const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per read
+    const uint32_t gcol = en0 + wn * 128u + cc * 8u;
+    const bool col_ok = gcol < N;                            // N % 8 == 0: a chunk is all in or all out
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 // lane holds C[row = i*32 + l32][col = j*32 + 8q + 4*lhi + 0..3]
-                u32x2 v = {cvt_pk_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]),
-                           cvt_pk_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
-                const uint32_t row = i * 32 + l32;
-                const uint32_t chunk = (uint32_t)(j * 4 + q) ^ (row & 15u);
-                const uint32_t hf = lhi ^ ((row >> 4) & 1u);
-                *(lds_v2)(cw + row * 256u + chunk * 16u + hf * 8u) = v;
+                floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                if (EDGE && split) f = reduced_chunk(i * 16 + j * 4 + q);
+                u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
+                const uint32_t chunk = (uint32_t)(j * 4 + q) ^ (l32 & 15u);
+                const uint32_t hf = lhi ^ ((l32 >> 4) & 1u);
+                *(lds_v2)(ew + l32 * 256u + chunk * 16u + hf * 8u) = v;
             }
-    // Wave-private region: LDS operations of one wave complete in order, no barrier needed.
-    const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per pass
-    const uint32_t gcol = n0 + wn * 128u + cc * 8u;
-    const bool col_ok = gcol < N;                            // N % 8 == 0: a chunk is all in or all out
 #pragma unroll
-    for (int r = 0; r < 32; ++r) {
-        const uint32_t row = r * 4 + cr;
-        u32x4 v = *(lds_v4)(cw + row * 256u + ((cc ^ (row & 15u)) * 16u));
-        if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
-        const uint32_t grow = m0 + wm * 128u + row;
-        // C is written once and not read again by this kernel: non-temporal stores keep it from
-        // displacing the operand panels in L2.
-        if (col_ok && grow < M) __builtin_nontemporal_store(v, (u32x4*)(Cg + (uint64_t)grow * N + gcol));
+        for (int r = 0; r < 8; ++r) {
+            const uint32_t row = r * 4 + cr;                 // 0..31 within the pass
+            u32x4 v = *(lds_v4)(ew + row * 256u + ((cc ^ (row & 15u)) * 16u));
+            if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
+            const uint32_t grow = em0 + wm * 128u + i * 32u + row;
+            // C is written once and not read again by this kernel: non-temporal stores keep it from
+            // displacing the operand panels in L2.
+            if (col_ok && grow < M) __builtin_nontemporal_store(v, (u32x4*)(Ce + (uint64_t)grow * N + gcol));
+        }
     }
+    if (!more) break;
+    pid = next;
+    }  // C tiles
 }
 
 }  // namespace mt256

@@ -54,12 +54,13 @@ def test_every_kernel_that_accepts_a_descriptor_plans_a_covering_grid(m, n, k, l
                 mz.gemm_plan(d, kernel=name, compute_units=CUS)
             continue
         for cus in (1, 8, 80, 256, 304):
-            check_plan(mz.gemm_plan(d, kernel=name, compute_units=cus), m, n, k, layout, 1)
+            check_plan(mz.gemm_plan(d, kernel=name, compute_units=cus), m, n, k, layout, 1, cus)
 
 
-def check_plan(p, m, n, k, layout, batch):
+def check_plan(p, m, n, k, layout, batch, cus=CUS):
     gx, gy, gz = p["grid"]
-    assert gx >= 1 and gy >= 1 and gz == batch
+    persistent = p["kernel"].startswith("maize_gemm_bf16_mt256") and not p["kernel"].endswith("_edge")
+    assert gx >= 1 and gy >= 1 and gz == (1 if persistent else batch)
     assert gy <= 65535 and gz <= 65535 and gx < (1 << 31)
     name = p["kernel"]
     if name == "maize_gemm_bf16_wave32":
@@ -73,7 +74,12 @@ def check_plan(p, m, n, k, layout, batch):
         if "ktail" not in name:
             assert k % 64 == 0
         tm, tn = cdiv(m, 256), cdiv(n, 256)
-        if p["split_first"] == 0:
+        if persistent:
+            # one workgroup per compute unit (a multiple of 8) walks all tiles of all batch members
+            resident = cus - cus % 8 if cus >= 8 else cus
+            assert gx == min(tm * tn * batch, resident) and p["split_first"] == 0 and p["workspace_bytes"] == 0
+            assert gx == tm * tn * batch or gx % 8 == 0 or cus < 8
+        elif p["split_first"] == 0:
             assert gx == tm * tn and p["workspace_bytes"] == 0
         else:
             assert name.endswith("_edge") and batch == 1
