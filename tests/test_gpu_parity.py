@@ -205,6 +205,34 @@ def test_builder_chain_launches_the_kernel(ctx, oracle):
         x.free()
 
 
+@pytest.mark.parametrize("grid_x", [1, 5, 24, 300])
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+def test_persistent_kernel_accepts_any_grid(ctx, oracle, grid_x, layout):
+    """The reference's panel loopers stride by the grid, so any grid is a legal launch
+    (crates/maize_tile/src/gmem/row_panel.rs:95-100, col_panel.rs:95-99).  The persistent macro-tile kernels
+    keep that property: whatever grid.x the caller launches -- one workgroup, a count that does not divide
+    the 3 x 4 x 2 = 24 tiles, exactly the tiles, more workgroups than tiles -- every tile is computed once."""
+    from maize_amd import _ffi
+    m, n, k, batch = 600, 1000, 192, 2
+    a = mz.gen.uniform_bf16(batch * m * k, 11)
+    b = mz.gen.uniform_bf16(batch * k * n, 12)
+    da, db = ctx.upload(a), ctx.upload(b)
+    dc = ctx.malloc(batch * m * n * 2)
+    dc.fill(0xFF)
+    name = "maize_gemm_bf16_mt256_nn" if layout == mz.LAYOUT_NN else "maize_gemm_bf16_mt256_nt"
+    kern = mz.new_hip_kernel(name).with_launch_bounds_2d((256, 1)).finalize().compile(mz.Gfx.Gfx950, ctx)
+    brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+    args = _ffi.GemmArgsT(da.ptr, m, k, db.ptr, brows, bcols, dc.ptr, m, n, m * k, k * n, m * n, batch, layout, None, 0, 0)
+    _say(f"persistent any-grid: {name} grid {grid_x}")
+    kern.launch((grid_x, 1, 1), args)
+    ctx.sync()
+    got = dc.download(np.uint16)
+    kern.release()
+    check_against_oracle(oracle, got, a, b, m, n, k, layout=layout, batch=batch, label=f"grid {grid_x}")
+    for x in (da, db, dc):
+        x.free()
+
+
 # ---- the five benchmark configurations at full size (sampled rows + invariants) ---------
 
 def _full_size(ctx, oracle, m, n, k, layout, dist, label, sigma_b=None):
