@@ -78,12 +78,30 @@ typedef struct {
     uint64_t stride_a, stride_b, stride_c;
 } maize_gemm_desc_t;
 
+/* The same product with the knobs the reference's descriptor has no room for: leading
+ * dimensions (the reference's rows are compact, crates/maize_tile/src/gmem/row_panel.rs:55,
+ * col_panel.rs:108), an fp32 C (the accumulator type of the reference's fragments,
+ * crates/maize_tile/src/mma/sm80.rs:136-160) and C = alpha * A.B + beta * C.
+ *   lda/ldb/ldc: elements between consecutive rows of A / B / C; 0 = that matrix's ncols.
+ *   out_type:    element type of C; batch stride stride_c counts elements of that type.
+ *   beta == 0:   C is not read (it may hold anything, NaNs included).
+ * All-zero extension fields with alpha = 1 describe exactly the plain descriptor. */
+typedef enum { MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1 } maize_out_type_t;
+typedef struct {
+    maize_gemm_desc_t gemm;
+    uint32_t lda, ldb, ldc;
+    uint32_t out_type; /* maize_out_type_t */
+    float alpha, beta;
+    uint32_t reserved[2]; /* must be 0 */
+} maize_gemm_ex_desc_t;
+
 /* Kernel parameter block of every GEMM kernel in the embedded code object.
  * It keeps the order and widths of the reference kernel's parameter list
  * (example_ptx/gen.ptx:12-19: A ptr, arows u32, acols u32, B ptr, brows u32,
  * bcols u32) and appends the C operand the reference never had, the batch
  * strides, the batch count, the layout and -- for the split-K kernel only --
- * a library-owned workspace and the number of K ranges (0 elsewhere). */
+ * a library-owned workspace and the number of K ranges (0 elsewhere) -- and, last, the
+ * leading dimensions and epilogue of the extended descriptor. */
 typedef struct {
     const void* a; uint32_t arows, acols;
     const void* b; uint32_t brows, bcols;
@@ -94,6 +112,10 @@ typedef struct {
     void* workspace;
     uint32_t ksplit;
     uint32_t reserved;
+    /* extended part; all zero = compact rows, bf16 C = A.B */
+    uint32_t lda, ldb, ldc; /* 0 = ncols */
+    uint32_t epi;           /* bit 0: C is fp32; bit 1: apply alpha and beta */
+    float alpha, beta;
 } maize_gemm_args_t;
 
 typedef struct {
@@ -164,6 +186,13 @@ typedef struct {
 } maize_gemm_plan_t;
 int32_t maize_hip_gemm_plan(const maize_gemm_desc_t* desc, const char* kernel, uint32_t compute_units,
                             maize_gemm_plan_t* out);
+/* The extended product: `kernel` == NULL lets the dispatcher choose.  Shapes that the fast
+ * kernels cannot take (rows not 16-byte aligned, alpha/beta or fp32 C on a large M) still
+ * compute, on the any-shape kernel. */
+int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const char* kernel, void* stream);
+int32_t maize_hip_gemm_ex_validate(const maize_gemm_ex_desc_t* desc);
+int32_t maize_hip_gemm_ex_plan(const maize_gemm_ex_desc_t* desc, const char* kernel, uint32_t compute_units,
+                               maize_gemm_plan_t* out);
 /* Validation only (no device access): the checks gemm_bf16 performs first. */
 int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* desc);
 /* Enumerates the GEMM kernels of the embedded code object. */

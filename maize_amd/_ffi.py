@@ -15,7 +15,8 @@ EXPORTS = (
     "maize_hip_last_error", "maize_hip_ctx_create", "maize_hip_ctx_destroy", "maize_hip_device_info",
     "maize_hip_module_load", "maize_hip_module_unload", "maize_hip_kernel_get", "maize_hip_kernel_release",
     "maize_hip_launch", "maize_hip_embedded_code_object", "maize_hip_gemm_bf16", "maize_hip_gemm_bf16_with",
-    "maize_hip_gemm_select", "maize_hip_gemm_plan", "maize_hip_gemm_validate", "maize_hip_kernel_count", "maize_hip_kernel_name",
+    "maize_hip_gemm_select", "maize_hip_gemm_plan", "maize_hip_gemm_validate",
+    "maize_hip_gemm_bf16_ex", "maize_hip_gemm_ex_validate", "maize_hip_gemm_ex_plan", "maize_hip_kernel_count", "maize_hip_kernel_name",
     "maize_hip_kernel_supports", "maize_hip_malloc", "maize_hip_free", "maize_hip_memcpy_h2d",
     "maize_hip_memcpy_d2h", "maize_hip_memset", "maize_hip_stream_create", "maize_hip_stream_destroy",
     "maize_hip_sync", "maize_hip_event_create", "maize_hip_event_record", "maize_hip_event_synchronize",
@@ -34,6 +35,8 @@ MAIZE_ERR_ARG = -7
 
 LAYOUT_NN = 0
 LAYOUT_NT = 1
+OUT_BF16 = 0
+OUT_F32 = 1
 
 
 class MatrixT(C.Structure):
@@ -53,7 +56,15 @@ class GemmArgsT(C.Structure):
                 ("c", C.c_void_p), ("crows", C.c_uint32), ("ccols", C.c_uint32),
                 ("stride_a", C.c_uint64), ("stride_b", C.c_uint64), ("stride_c", C.c_uint64),
                 ("batch", C.c_uint32), ("layout", C.c_uint32),
-                ("workspace", C.c_void_p), ("ksplit", C.c_uint32), ("reserved", C.c_uint32)]
+                ("workspace", C.c_void_p), ("ksplit", C.c_uint32), ("reserved", C.c_uint32),
+                ("lda", C.c_uint32), ("ldb", C.c_uint32), ("ldc", C.c_uint32), ("epi", C.c_uint32),
+                ("alpha", C.c_float), ("beta", C.c_float)]
+
+
+class GemmExDescT(C.Structure):
+    """maize_gemm_ex_desc_t: the descriptor plus leading dimensions, output type, alpha and beta."""
+    _fields_ = [("gemm", GemmDescT), ("lda", C.c_uint32), ("ldb", C.c_uint32), ("ldc", C.c_uint32),
+                ("out_type", C.c_uint32), ("alpha", C.c_float), ("beta", C.c_float), ("reserved", C.c_uint32 * 2)]
 
 
 class DeviceInfoT(C.Structure):
@@ -69,7 +80,8 @@ class GemmPlanT(C.Structure):
 
 
 assert C.sizeof(GemmPlanT) == 112
-assert C.sizeof(MatrixT) == 16 and C.sizeof(GemmArgsT) == 96 and C.sizeof(GemmDescT) == 80
+assert C.sizeof(MatrixT) == 16 and C.sizeof(GemmArgsT) == 120 and C.sizeof(GemmDescT) == 80
+assert C.sizeof(GemmExDescT) == 112
 
 _lib = None
 
@@ -102,6 +114,9 @@ def lib():
         "maize_hip_gemm_select": (i32, [vp, P(GemmDescT), C.c_char_p, sz]),
         "maize_hip_gemm_plan": (i32, [P(GemmDescT), C.c_char_p, u32, P(GemmPlanT)]),
         "maize_hip_gemm_validate": (i32, [P(GemmDescT)]),
+        "maize_hip_gemm_bf16_ex": (i32, [vp, P(GemmExDescT), C.c_char_p, vp]),
+        "maize_hip_gemm_ex_validate": (i32, [P(GemmExDescT)]),
+        "maize_hip_gemm_ex_plan": (i32, [P(GemmExDescT), C.c_char_p, u32, P(GemmPlanT)]),
         "maize_hip_kernel_count": (u32, []),
         "maize_hip_kernel_name": (C.c_char_p, [u32]),
         "maize_hip_kernel_supports": (i32, [C.c_char_p, P(GemmDescT)]),

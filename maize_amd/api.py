@@ -84,7 +84,9 @@ class Context:
     def gemm_bf16(self, desc, stream=None, kernel=None):
         """Launch C = A.B for ``desc`` (a GemmDescT); asynchronous on ``stream``."""
         L = _ffi.lib()
-        if kernel is None:
+        if isinstance(desc, _ffi.GemmExDescT):
+            check(L.maize_hip_gemm_bf16_ex(self._h, C.byref(desc), kernel.encode() if kernel else None, stream))
+        elif kernel is None:
             check(L.maize_hip_gemm_bf16(self._h, C.byref(desc), stream))
         else:
             check(L.maize_hip_gemm_bf16_with(self._h, C.byref(desc), kernel.encode(), stream))
@@ -188,15 +190,31 @@ def gemm_desc(a, b, c, layout=LAYOUT_NN, batch=1, stride_a=0, stride_b=0, stride
     return d
 
 
+def gemm_ex_desc(a, b, c, layout=LAYOUT_NN, batch=1, stride_a=0, stride_b=0, stride_c=0, lda=0, ldb=0, ldc=0,
+                 out_type=_ffi.OUT_BF16, alpha=1.0, beta=0.0):
+    """Build a maize_gemm_ex_desc_t: the descriptor plus leading dimensions (0 = ncols), the
+    element type of C and C = alpha * A.B + beta * C."""
+    x = _ffi.GemmExDescT()
+    x.gemm = gemm_desc(a, b, c, layout, batch, stride_a, stride_b, stride_c)
+    x.lda, x.ldb, x.ldc = lda, ldb, ldc
+    x.out_type = out_type
+    x.alpha, x.beta = alpha, beta
+    return x
+
+
 def validate(desc):
     """The host-side checks alone (no device needed); raises MaizeError."""
-    check(_ffi.lib().maize_hip_gemm_validate(C.byref(desc)))
+    if isinstance(desc, _ffi.GemmExDescT):
+        check(_ffi.lib().maize_hip_gemm_ex_validate(C.byref(desc)))
+    else:
+        check(_ffi.lib().maize_hip_gemm_validate(C.byref(desc)))
 
 
 def gemm_plan(desc, kernel=None, compute_units=256):
     """Kernel choice and launch geometry for ``desc`` (no device needed); a dict."""
     out = _ffi.GemmPlanT()
-    check(_ffi.lib().maize_hip_gemm_plan(C.byref(desc), kernel.encode() if kernel else None, compute_units, C.byref(out)))
+    fn = _ffi.lib().maize_hip_gemm_ex_plan if isinstance(desc, _ffi.GemmExDescT) else _ffi.lib().maize_hip_gemm_plan
+    check(fn(C.byref(desc), kernel.encode() if kernel else None, compute_units, C.byref(out)))
     return {"kernel": out.kernel.decode(), "grid": tuple(out.grid), "block": tuple(out.block), "lds_bytes": out.lds_bytes,
             "ksplit": out.ksplit, "split_first": out.split_first, "workspace_bytes": out.workspace_bytes}
 

@@ -8,13 +8,30 @@ namespace {
 
 inline uint32_t cdiv(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
+// Leading dimensions with their defaults, and the extent (in elements) of each operand view.
+struct Lds { uint32_t a, b, c; uint64_t ext_a, ext_b, ext_c; };
+inline Lds lds_of(const maize_gemm_ex_desc_t& d) {
+    Lds l;
+    l.a = d.lda ? d.lda : d.gemm.a.ncols;
+    l.b = d.ldb ? d.ldb : d.gemm.b.ncols;
+    l.c = d.ldc ? d.ldc : d.gemm.c.ncols;
+    l.ext_a = (uint64_t)(d.gemm.a.nrows - 1u) * l.a + d.gemm.a.ncols;
+    l.ext_b = (uint64_t)(d.gemm.b.nrows - 1u) * l.b + d.gemm.b.ncols;
+    l.ext_c = (uint64_t)(d.gemm.c.nrows - 1u) * l.c + d.gemm.c.ncols;
+    return l;
+}
+// The plain product: bf16 C = A.B (alpha == 1, beta == 0).
+inline bool plain_epilogue(const maize_gemm_ex_desc_t& d) {
+    return d.out_type == MAIZE_OUT_BF16 && d.alpha == 1.0f && d.beta == 0.0f;
+}
+
 // ---- maize_gemm_bf16_wave32: any shape ------------------------------------
-bool wave32_supports(const maize_gemm_desc_t&) { return true; }
-bool wave32_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
+bool wave32_supports(const maize_gemm_ex_desc_t&) { return true; }
+bool wave32_plan(const maize_gemm_ex_desc_t& d, uint32_t, LaunchDims* ld) {
     const Dims s = dims_of(d);
     ld->grid[0] = cdiv(s.n, 64);
     ld->grid[1] = cdiv(s.m, 64);
-    ld->grid[2] = d.batch;
+    ld->grid[2] = d.gemm.batch;
     ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
     ld->ksplit = 0; ld->workspace_bytes = 0; ld->split_first = 0;
@@ -25,25 +42,28 @@ bool wave32_plan(const maize_gemm_desc_t& d, uint32_t, LaunchDims* ld) {
 // 128-bit loads and stores: K % 8 == 0 (A rows, and B rows when NT), N % 8 == 0
 // (C rows, and B rows when NN), 16-byte aligned bases and batch strides.
 // 32-bit buffer offsets: every matrix of one batch member stays below 2 GiB.
-bool aligned16(const maize_gemm_desc_t& d) {
-    if (((uintptr_t)d.a.ptr | (uintptr_t)d.b.ptr | (uintptr_t)d.c.ptr) & 15u) return false;
-    if (d.batch > 1 && ((d.stride_a | d.stride_b | d.stride_c) & 7u)) return false;
+bool aligned16(const maize_gemm_ex_desc_t& d) {
+    if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr | (uintptr_t)d.gemm.c.ptr) & 15u) return false;
+    if (d.gemm.batch > 1 && ((d.gemm.stride_a | d.gemm.stride_b | d.gemm.stride_c) & 7u)) return false;
+    const Lds l = lds_of(d);
+    if ((l.a | l.b | l.c) & 7u) return false;              // rows start on 16-byte boundaries
     return true;
 }
-bool mt256_common(const maize_gemm_desc_t& d) {
+bool mt256_common(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
     if ((s.k & 7u) || (s.n & 7u) || !aligned16(d)) return false;
     const uint64_t lim = 1ull << 31;
-    if ((uint64_t)s.m * s.k * 2 >= lim || (uint64_t)s.n * s.k * 2 >= lim || (uint64_t)s.m * s.n * 2 >= lim) return false;
-    if (s.k >= (1u << 21) || s.n >= (1u << 21)) return false;
-    return true;
+    const Lds l = lds_of(d);
+    if (l.ext_a * 2 >= lim || l.ext_b * 2 >= lim || l.ext_c * 2 >= lim) return false;
+    if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21)) return false;
+    return plain_epilogue(d);                               // the staged epilogue stores bf16 of A.B only
 }
 // The plain kernels advance K with a scalar offset and never mask a lane in K: K % 64 == 0.
-bool k64(const maize_gemm_desc_t& d) { return (d.a.ncols & 63u) == 0; }
-bool mt256_nn_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d) && k64(d); }
-bool mt256_nt_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k64(d); }
-bool mt256_nn_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
-bool mt256_nt_ktail_supports(const maize_gemm_desc_t& d) { return d.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
+bool k64(const maize_gemm_ex_desc_t& d) { return (d.gemm.a.ncols & 63u) == 0; }
+bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NN && mt256_common(d) && k64(d); }
+bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k64(d); }
+bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
+bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
 // Edge splitting.  A ragged N leaves a last column of tiles that are almost empty but cost a
 // whole tile each (likewise a ragged M and the last row).  When that edge is at most 32 elements
 // wide and setting it aside saves a round of workgroups (one workgroup per compute unit per
@@ -74,21 +94,21 @@ EdgeSplit mt256_edge(const Dims& s, uint32_t batch, uint32_t cus) {
     e.whole = mode == 1 ? tm * (tn - 1u) : (tm - 1u) * tn;
     return e;
 }
-bool mt256_plan_impl(const maize_gemm_desc_t& d, uint32_t compute_units, bool allow_edge, LaunchDims* ld) {
+bool mt256_plan_impl(const maize_gemm_ex_desc_t& d, uint32_t compute_units, bool allow_edge, LaunchDims* ld) {
     const Dims s = dims_of(d);
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256);
     if (tiles > 0x1FFFFFFFull) return false;
-    EdgeSplit e = mt256_edge(s, d.batch, compute_units);
+    EdgeSplit e = mt256_edge(s, d.gemm.batch, compute_units);
     if (!allow_edge) e = EdgeSplit{0, (uint32_t)tiles, 0, 0};
     if (allow_edge) {
         // The edge-splitting kernels compute one tile, or one K range of an edge tile, per workgroup.
         ld->grid[0] = e.mode ? e.whole + e.nedge * e.ks : (uint32_t)tiles;
-        ld->grid[2] = d.batch;
+        ld->grid[2] = d.gemm.batch;
     } else {
         // Persistent: one workgroup per compute unit walks the list of all tiles of all batch
         // members (a multiple of 8 workgroups, so that the tiles one XCD works on at a time stay
         // neighbours); with fewer tiles than compute units, one workgroup per tile.
-        const uint64_t all = tiles * d.batch;
+        const uint64_t all = tiles * d.gemm.batch;
         if (all > 0x1FFFFFFFull) return false;
         uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
         ld->grid[0] = (resident && all > resident) ? resident : (uint32_t)all;
@@ -102,16 +122,17 @@ bool mt256_plan_impl(const maize_gemm_desc_t& d, uint32_t compute_units, bool al
     ld->workspace_bytes = e.mode ? kTicketBytes + (size_t)e.nedge * e.ks * 256u * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31) && e.nedge <= 16384u;
 }
-bool mt256_plan(const maize_gemm_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, false, ld); }
-bool mt256_edge_plan(const maize_gemm_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
+bool mt256_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, false, ld); }
+bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
 
 // ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
-bool skinny_nn_supports(const maize_gemm_desc_t& d) {
+bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
-    if (d.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
+    if (d.gemm.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
     const uint64_t lim = 1ull << 31;
-    if ((uint64_t)s.n * s.k * 2 >= lim || (uint64_t)s.m * s.k * 2 >= lim || s.n >= (1u << 21)) return false;
-    return (uint64_t)cdiv(s.n, 256) * d.batch <= 16384u;   // one ticket counter per (batch member, slab)
+    const Lds l = lds_of(d);
+    if (l.ext_a * 2 >= lim || l.ext_b * 2 >= lim || s.n >= (1u << 21) || l.b >= (1u << 21)) return false;
+    return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
 }
 // K ranges: the smallest power of two that gives the grid at least ~7/8 of a workgroup per
 // compute unit, as long as every range keeps a whole number of 32-row blocks and at least 8 of them.
@@ -122,17 +143,17 @@ uint32_t skinny_ksplit(const Dims& s, uint32_t batch, uint32_t compute_units) {
         ks *= 2;
     return ks;
 }
-bool skinny_plan(const maize_gemm_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
     const Dims s = dims_of(d);
-    const uint32_t ks = skinny_ksplit(s, d.batch, compute_units ? compute_units : 256u);
+    const uint32_t ks = skinny_ksplit(s, d.gemm.batch, compute_units ? compute_units : 256u);
     ld->grid[0] = cdiv(s.n, 256);
     ld->grid[1] = ks;
-    ld->grid[2] = d.batch;
+    ld->grid[2] = d.gemm.batch;
     ld->block[0] = 512; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
     ld->ksplit = ks;
     ld->split_first = 0;
-    ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.batch * ks * 16u * 256u * 4u : 0;
+    ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * 16u * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
 }
 
@@ -161,7 +182,7 @@ int kernel_index(const char* name) {
     return -1;
 }
 
-uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units) {
+uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     const Dims s = dims_of(d);
     // Few rows against a wide row-major B: bound by streaming B once.
     const int sk = kernel_index("maize_gemm_bf16_skinny_nn");
@@ -171,7 +192,7 @@ uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units) {
          {"maize_gemm_bf16_mt256_nn_ktail", "maize_gemm_bf16_mt256_nt_ktail"}},
         {{"maize_gemm_bf16_mt256_nn_edge", "maize_gemm_bf16_mt256_nt_edge"},
          {"maize_gemm_bf16_mt256_nn_ktail_edge", "maize_gemm_bf16_mt256_nt_ktail_edge"}}};
-    const bool edge = mt256_edge(s, d.batch, compute_units).mode != 0;
+    const bool edge = mt256_edge(s, d.gemm.batch, compute_units).mode != 0;
     const int ti = kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt]);
     // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below
     // half a tile in either direction the per-wave kernel wastes less.

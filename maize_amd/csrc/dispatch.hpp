@@ -26,27 +26,27 @@ constexpr size_t kTicketBytes = 16384 * 4;  // ticket counters at the start of a
 
 struct KernelInfo {
     const char* name;
-    bool (*supports)(const maize_gemm_desc_t&);
+    bool (*supports)(const maize_gemm_ex_desc_t&);
     // Fills the launch dimensions; false if the grid would exceed HIP limits.
-    bool (*plan)(const maize_gemm_desc_t&, uint32_t compute_units, LaunchDims*);
+    bool (*plan)(const maize_gemm_ex_desc_t&, uint32_t compute_units, LaunchDims*);
 };
 
 uint32_t kernel_count();
 const KernelInfo& kernel_at(uint32_t i);
 int kernel_index(const char* name);  // -1 if unknown
 // Index of the kernel the dispatcher picks for a validated descriptor.
-uint32_t select_kernel(const maize_gemm_desc_t& d, uint32_t compute_units);
+uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units);
 
 struct Dims {
     uint32_t m, n, k;
     bool nt;
 };
-inline Dims dims_of(const maize_gemm_desc_t& d) {
+inline Dims dims_of(const maize_gemm_ex_desc_t& d) {
     Dims r;
-    r.m = d.c.nrows;
-    r.n = d.c.ncols;
-    r.k = d.a.ncols;
-    r.nt = d.layout == MAIZE_LAYOUT_NT;
+    r.m = d.gemm.c.nrows;
+    r.n = d.gemm.c.ncols;
+    r.k = d.gemm.a.ncols;
+    r.nt = d.gemm.layout == MAIZE_LAYOUT_NT;
     return r;
 }
 

@@ -18,8 +18,19 @@ struct GemmArgs {
     void* workspace;  // split-K kernels: ticket counters + fp32 partial tiles (library owned)
     uint32_t ksplit;  // split-K kernels: number of K ranges (grid.y)
     uint32_t reserved;
+    // Extended part (all zero = the plain product: compact rows, bf16 C = A.B).
+    uint32_t lda, ldb, ldc;  // elements between consecutive rows; 0 = the matrix's column count
+    uint32_t epi;            // bit 0: C is fp32; bit 1: C = alpha * A.B + beta * C
+    float alpha, beta;
 };
-static_assert(sizeof(GemmArgs) == 96, "kernel parameter block layout");
+static_assert(sizeof(GemmArgs) == 120, "kernel parameter block layout");
+constexpr uint32_t EPI_F32 = 1u, EPI_SCALE = 2u;
+
+// Leading dimensions with their defaults: the reference's rows are compact (row stride ==
+// ncols, crates/maize_tile/src/gmem/row_panel.rs:55).
+__device__ __forceinline__ uint32_t lda_of(const GemmArgs& p) { return p.lda ? p.lda : p.acols; }
+__device__ __forceinline__ uint32_t ldb_of(const GemmArgs& p) { return p.ldb ? p.ldb : p.bcols; }
+__device__ __forceinline__ uint32_t ldc_of(const GemmArgs& p) { return p.ldc ? p.ldc : p.ccols; }
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
@@ -38,9 +49,69 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// Two fp32 -> packed bf16x2 with the hardware converter (v_cvt_pk_bf16_f32, RNE).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+    float2v f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
+// bf16 bits -> fp32 (exact).
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }
+
+// The general epilogue on one element: acc -> alpha * acc + beta * c_old (one fused multiply-add
+// on top of one multiply).
+__device__ __forceinline__ float epi_scale(float acc, float c_old, float alpha, float beta) {
+    return __builtin_fmaf(beta, c_old, alpha * acc);
+}
+
 // Two fp32 -> packed bf16x2 (lo in bits 0..15), RNE.
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+}
+
+// Writes NV (4 or 8) consecutive elements of one row of C, starting at element offset `at` (a
+// multiple of NV) of the batch member's C: the plain product as packed bf16, or the general
+// epilogue (alpha/beta, fp32 output).  `c` points at the batch member (bf16 or fp32 elements).
+template <int NV>
+__device__ __forceinline__ void store_c_run(const GemmArgs& p, void* c, uint64_t at, const float (&acc)[NV]) {
+    static_assert(NV == 4 || NV == 8, "a run is 4 or 8 elements");
+    float x[NV];
+#pragma unroll
+    for (int e = 0; e < NV; ++e) x[e] = acc[e];
+    const bool f32_out = p.epi & EPI_F32;
+    if ((p.epi & EPI_SCALE)) {
+        float old[NV];
+#pragma unroll
+        for (int e = 0; e < NV; ++e) old[e] = 0.0f;
+        if (p.beta != 0.0f) {                               // beta == 0: C is not read (it may hold anything)
+            if (f32_out) {
+#pragma unroll
+                for (int e = 0; e < NV; e += 4) {
+                    const floatx4 o = *(const floatx4*)((const float*)c + at + e);
+                    old[e] = o[0]; old[e + 1] = o[1]; old[e + 2] = o[2]; old[e + 3] = o[3];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < NV; e += 4) {
+                    const u32x2 o = *(const u32x2*)((const uint16_t*)c + at + e);
+                    old[e] = bf16_bits_to_f32(o[0] & 0xFFFFu); old[e + 1] = bf16_bits_to_f32(o[0] >> 16);
+                    old[e + 2] = bf16_bits_to_f32(o[1] & 0xFFFFu); old[e + 3] = bf16_bits_to_f32(o[1] >> 16);
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < NV; ++e) x[e] = epi_scale(x[e], old[e], p.alpha, p.beta);
+    }
+    if (f32_out) {
+#pragma unroll
+        for (int e = 0; e < NV; e += 4) *(floatx4*)((float*)c + at + e) = floatx4{x[e], x[e + 1], x[e + 2], x[e + 3]};
+    } else {
+#pragma unroll
+        for (int e = 0; e < NV; e += 4)
+            *(u32x2*)((uint16_t*)c + at + e) = u32x2{cvt_pk_bf16(x[e], x[e + 1]), cvt_pk_bf16(x[e + 2], x[e + 3])};
+    }
 }
 
 }  // namespace maize

@@ -76,12 +76,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float float2v __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
-    float2v f = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));  // v_cvt_pk_bf16_f32, RNE
-}
 
 // Maps the linear workgroup id to a tile so that (a) the workgroups that land
 // on one XCD (ids congruent mod 8) form a contiguous run of tiles and (b) a
@@ -120,6 +114,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     lds_ptr const A0 = (lds_ptr)lds_a0, A1 = (lds_ptr)lds_a1, B0 = (lds_ptr)lds_b0, B1 = (lds_ptr)lds_b1;
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
+    const uint32_t lda = lda_of(p), ldb = ldb_of(p), ldc = ldc_of(p);
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
     const uint32_t wave = tid >> 6;
@@ -143,7 +138,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t nk = kt0 < nk_all ? (nk_all - kt0 < per_range ? nk_all - kt0 : per_range) : 0u;
     const uint32_t k_begin = kt0 * BK;
     const uint32_t k_end = (kt0 + nk) * BK < K ? (kt0 + nk) * BK : K;   // loads at or past k_end return zeros
-    const uint32_t a_bytes = M * K * 2u, b_bytes = N * K * 2u;
+    // Extent of each operand view: the last row ends at (rows - 1) * ld + cols.
+    const uint32_t a_bytes = ((M - 1u) * lda + K) * 2u;
+    const uint32_t b_bytes = (NT ? (N - 1u) * ldb + K : (K - 1u) * ldb + N) * 2u;
 
     // The plain kernels are persistent: the grid is one workgroup per compute unit (or one per
     // tile if there are fewer), workgroup g computes tiles g, g + grid, g + 2 grid, ... of the
@@ -196,19 +193,19 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int i = 0; i < 8; ++i) {
             const uint32_t row = (wave * 8u + i) * 8u + (lane >> 3);
             const uint32_t c = (lane & 7u) ^ ((row >> 1) & 7u);
-            a_vo[i] = ((m0 + row) * K + c * 8u) * 2u;
+            a_vo[i] = ((m0 + row) * lda + c * 8u) * 2u;
             if (i < 2) a_k[i] = c * 8u;
             if (NT) {
-                b_vo[i] = ((n0 + row) * K + c * 8u) * 2u;
+                b_vo[i] = ((n0 + row) * ldb + c * 8u) * 2u;
             } else {
                 const uint32_t brow = (wave * 8u + i) * 2u + (lane >> 5);
                 const uint32_t bc = (lane & 31u) ^ ((brow & 3u) << 2);
-                b_vo[i] = ((brow * N + n0 + bc * 8u) * 2u) | ((n0 + bc * 8u) < N ? 0u : OOB);
+                b_vo[i] = ((brow * ldb + n0 + bc * 8u) * 2u) | ((n0 + bc * 8u) < N ? 0u : OOB);
             }
         }
     };
     select_tile(pid);
-    const uint32_t b_kscale = NT ? 2u : N * 2u;    // bytes per unit of k in B
+    const uint32_t b_kscale = NT ? 2u : ldb * 2u;  // bytes per unit of k in B
     // Issues piece pc (0..7 = A, 8..15 = B) of the tile that starts at k into stages (sa, sb).
     auto dma = [&](int pc, lds_ptr sa, lds_ptr sb, uint32_t k) {
         typedef __attribute__((address_space(3))) void* lvp;
@@ -449,7 +446,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             const uint32_t grow = em0 + wm * 128u + i * 32u + row;
             // C is written once and not read again by this kernel: non-temporal stores keep it from
             // displacing the operand panels in L2.
-            if (col_ok && grow < M) __builtin_nontemporal_store(v, (u32x4*)(Ce + (uint64_t)grow * N + gcol));
+            if (col_ok && grow < M) __builtin_nontemporal_store(v, (u32x4*)(Ce + (uint64_t)grow * ldc + gcol));
         }
     }
     if (!more) break;

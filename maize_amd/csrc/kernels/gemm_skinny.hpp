@@ -48,12 +48,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float float2v __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
-    float2v f = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));  // v_cvt_pk_bf16_f32, RNE
-}
 
 // Granule swizzle of a block: the 32-byte granule index (0..15) of row r is XOR-ed with
 // f(r) = r%4 + 4*bit3(r), so the 8 rows one transposing read touches land in 8 different
@@ -74,6 +68,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     __shared__ uint32_t ticket;
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
+    const uint32_t lda = lda_of(p), ldb = ldb_of(p), ldc = ldc_of(p);
     const uint32_t ks = p.ksplit ? p.ksplit : 1u;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
@@ -83,9 +78,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint64_t bz = blockIdx.z;
     const uint16_t* Ag = p.a + bz * p.stride_a;
     const uint16_t* Bg = p.b + bz * p.stride_b;
-    uint16_t* Cg = p.c + bz * p.stride_c;
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ag, M * K * 2u);
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bg, K * N * 2u);
+    uint16_t* Cg = p.c + bz * p.stride_c * ((p.epi & EPI_F32) ? 2u : 1u);   // strides count elements of C
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ag, ((M - 1u) * lda + K) * 2u);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bg, ((K - 1u) * ldb + N) * 2u);
     const __amdgpu_buffer_rsrc_t rnull = make_rsrc(Bg, 0u);
 
     lds_ptr const s0 = (lds_ptr)ring0, s1 = (lds_ptr)ring1, s2 = (lds_ptr)ring2, s3 = (lds_ptr)ring3;
@@ -100,10 +95,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const uint32_t row = (wave * 2u + i) * 2u + (lane >> 5);
         const uint32_t c = (lane & 31u) ^ (gsw(row) << 1);
         const uint32_t col = n0 + c * 8u;
-        b_vo[i] = ((row * N + col) * 2u) | (col < N ? 0u : OOB);       // N % 8 == 0: a chunk is all in or all out
+        b_vo[i] = ((row * ldb + col) * 2u) | (col < N ? 0u : OOB);       // N % 8 == 0: a chunk is all in or all out
     }
     // A operand of MFMA 16x16x32: lane l holds row l%16, k = 8*(l/16) + 0..7 of the block.
-    const uint32_t a_vo = ((lane & 15u) * K + (lane >> 4) * 8u) * 2u;  // rows >= M fall past the descriptor: zeros
+    const uint32_t a_vo = ((lane & 15u) * lda + (lane >> 4) * 8u) * 2u;  // rows >= M fall past the descriptor: zeros
 
     // ---- transposing-read map.  In each group of 16 lanes, lane q addresses 4 consecutive
     // columns (q%4) of row (q/4) of a 4 x 16 sub-block and receives column q, rows 0..3.  Lane
@@ -143,7 +138,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lvp)(slot + (wave * 2u + i) * 1024u), 16, b_vo[i],
-                                                     kb * N * 2u, 0, 0);
+                                                     kb * ldb * 2u, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
     auto consume = [&](lds_ptr slot, int ai) {
@@ -192,8 +187,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int c2 = 0; c2 < 2; ++c2) {
             const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
             if (m < M && col < N) {
-                u32x2 v = {cvt_pk_bf16(acc[c2][0], acc[c2][1]), cvt_pk_bf16(acc[c2][2], acc[c2][3])};
-                *(u32x2*)(Cg + (uint64_t)m * N + col) = v;
+                const float v[4] = {acc[c2][0], acc[c2][1], acc[c2][2], acc[c2][3]};
+                store_c_run<4>(p, Cg, (uint64_t)m * ldc + col, v);
             }
         }
         return;
@@ -246,9 +241,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         }
         const uint32_t col = n0 + cq;
         if (row < M && col < N) {                          // N % 8 == 0: 8 columns are all in or all out
-            u32x4 v = {cvt_pk_bf16(s_lo[0], s_lo[1]), cvt_pk_bf16(s_lo[2], s_lo[3]),
-                       cvt_pk_bf16(s_hi[0], s_hi[1]), cvt_pk_bf16(s_hi[2], s_hi[3])};
-            *(u32x4*)(Cg + (uint64_t)row * N + col) = v;
+            const float v[8] = {s_lo[0], s_lo[1], s_lo[2], s_lo[3], s_hi[0], s_hi[1], s_hi[2], s_hi[3]};
+            store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);
         }
     }
     if (tid == 0) counters[slab_id] = 0u;                 // ready for the next launch

@@ -26,6 +26,7 @@ __device__ __forceinline__ __bf16 bf16_from_bits(uint16_t h) {
 
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArgs p) {
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
+    const uint32_t lda = lda_of(p), ldb = ldb_of(p), ldc = ldc_of(p);
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;  // 0..3, arranged 2 x 2
     const uint32_t m0 = blockIdx.y * 64u + (wave >> 1) * 32u;
@@ -35,7 +36,9 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
     const uint64_t bz = blockIdx.z;
     const uint16_t* __restrict__ A = p.a + bz * p.stride_a;
     const uint16_t* __restrict__ B = p.b + bz * p.stride_b;
-    uint16_t* __restrict__ C = p.c + bz * p.stride_c;
+    const bool f32_out = p.epi & EPI_F32, scaled = p.epi & EPI_SCALE;
+    uint16_t* __restrict__ C = p.c + bz * p.stride_c * (f32_out ? 2u : 1u);   // strides count elements of C
+    float* __restrict__ Cf = (float*)C;
 
     const uint32_t r = lane & 31u;   // row of A / column of B owned by this lane
     const uint32_t kg = lane >> 5;   // which 8-wide k group
@@ -51,8 +54,8 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
             const uint32_t k = k0 + kg * 8u + e;
             uint16_t av = 0, bv = 0;
             if (k < K) {
-                if (am < M) av = A[(uint64_t)am * K + k];
-                if (bn < N) bv = nt ? B[(uint64_t)bn * K + k] : B[(uint64_t)k * N + bn];
+                if (am < M) av = A[(uint64_t)am * lda + k];
+                if (bn < N) bv = nt ? B[(uint64_t)bn * ldb + k] : B[(uint64_t)k * ldb + bn];
             }
             fa[e] = bf16_from_bits(av);
             fb[e] = bf16_from_bits(bv);
@@ -65,7 +68,12 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
 #pragma unroll
         for (uint32_t v = 0; v < 16u; ++v) {
             const uint32_t cn = n0 + 8u * (v >> 2) + 4u * kg + (v & 3u);
-            if (cn < N) C[(uint64_t)cm * N + cn] = f32_to_bf16_rne(acc[v]);
+            if (cn < N) {
+                const uint64_t at = (uint64_t)cm * ldc + cn;
+                float x = acc[v];
+                if (scaled) x = epi_scale(x, p.beta == 0.0f ? 0.0f : (f32_out ? Cf[at] : bf16_bits_to_f32(C[at])), p.alpha, p.beta);
+                if (f32_out) Cf[at] = x; else C[at] = f32_to_bf16_rne(x);
+            }
         }
     }
 }

@@ -20,7 +20,8 @@ extern "C" const unsigned char maize_embedded_hsaco[];
 extern "C" const unsigned char maize_embedded_hsaco_end[];
 
 static_assert(sizeof(maize_matrix_t) == 16 && alignof(maize_matrix_t) == 16, "GlobalMatrix twin");
-static_assert(sizeof(maize_gemm_args_t) == 96, "kernel parameter block");
+static_assert(sizeof(maize_gemm_args_t) == 120, "kernel parameter block");
+static_assert(sizeof(maize_gemm_ex_desc_t) == 112, "extended descriptor");
 static_assert(offsetof(maize_gemm_args_t, arows) == 8 && offsetof(maize_gemm_args_t, acols) == 12 &&
                   offsetof(maize_gemm_args_t, b) == 16 && offsetof(maize_gemm_args_t, brows) == 24 &&
                   offsetof(maize_gemm_args_t, bcols) == 28 && offsetof(maize_gemm_args_t, c) == 32,
@@ -229,8 +230,20 @@ int32_t maize_hip_launch(maize_kernel_t* k, const uint32_t grid[3], const uint32
 
 /* ---- the GEMM path --------------------------------------------------------- */
 
-int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* d) {
-    if (!d) return fail(MAIZE_ERR_NULL, "gemm: descriptor is NULL");
+// The plain descriptor as an extended one: compact rows, bf16 C = A.B.
+static maize_gemm_ex_desc_t widen(const maize_gemm_desc_t& d) {
+    maize_gemm_ex_desc_t x;
+    memset(&x, 0, sizeof x);
+    x.gemm = d;
+    x.out_type = MAIZE_OUT_BF16;
+    x.alpha = 1.0f;
+    x.beta = 0.0f;
+    return x;
+}
+
+int32_t maize_hip_gemm_ex_validate(const maize_gemm_ex_desc_t* x) {
+    if (!x) return fail(MAIZE_ERR_NULL, "gemm: descriptor is NULL");
+    const maize_gemm_desc_t* d = &x->gemm;
     if (d->layout != MAIZE_LAYOUT_NN && d->layout != MAIZE_LAYOUT_NT)
         return fail(MAIZE_ERR_LAYOUT, "gemm: unknown layout %u", d->layout);
     if (d->batch == 0) return fail(MAIZE_ERR_SHAPE, "gemm: batch is 0");
@@ -244,13 +257,29 @@ int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* d) {
     if (d->c.nrows != M || d->c.ncols != N)
         return fail(MAIZE_ERR_SHAPE, "gemm: C is %ux%u, expected %ux%u", d->c.nrows, d->c.ncols, M, N);
     if (!d->a.ptr || !d->b.ptr || !d->c.ptr) return fail(MAIZE_ERR_NULL, "gemm: NULL matrix pointer");
-    if (((uintptr_t)d->a.ptr | (uintptr_t)d->b.ptr | (uintptr_t)d->c.ptr) & 1u)
-        return fail(MAIZE_ERR_ALIGN, "gemm: matrix pointers must be 2-byte aligned");
+    if (x->out_type != MAIZE_OUT_BF16 && x->out_type != MAIZE_OUT_F32)
+        return fail(MAIZE_ERR_ARG, "gemm: unknown output type %u", x->out_type);
+    if (x->reserved[0] || x->reserved[1]) return fail(MAIZE_ERR_ARG, "gemm: reserved fields must be 0");
+    if (((uintptr_t)d->a.ptr | (uintptr_t)d->b.ptr) & 1u || (uintptr_t)d->c.ptr & (x->out_type == MAIZE_OUT_F32 ? 3u : 1u))
+        return fail(MAIZE_ERR_ALIGN, "gemm: matrix pointers must be aligned to their element size");
+    if ((x->lda && x->lda < d->a.ncols) || (x->ldb && x->ldb < d->b.ncols) || (x->ldc && x->ldc < d->c.ncols))
+        return fail(MAIZE_ERR_SHAPE, "gemm: a leading dimension is smaller than the row it strides (lda=%u ldb=%u ldc=%u)",
+                    x->lda, x->ldb, x->ldc);
+    if (!(x->alpha == x->alpha) || !(x->beta == x->beta)) return fail(MAIZE_ERR_ARG, "gemm: alpha or beta is NaN");
     if (d->batch > 1) {
-        if (d->stride_a < (uint64_t)M * K || d->stride_b < (uint64_t)K * N || d->stride_c < (uint64_t)M * N)
+        const uint64_t lda = x->lda ? x->lda : d->a.ncols, ldb = x->ldb ? x->ldb : d->b.ncols, ldc = x->ldc ? x->ldc : d->c.ncols;
+        const uint64_t ea = (uint64_t)(d->a.nrows - 1u) * lda + d->a.ncols, eb = (uint64_t)(d->b.nrows - 1u) * ldb + d->b.ncols,
+                       ec = (uint64_t)(d->c.nrows - 1u) * ldc + d->c.ncols;
+        if (d->stride_a < ea || d->stride_b < eb || d->stride_c < ec)
             return fail(MAIZE_ERR_SHAPE, "gemm: batch stride smaller than one matrix");
     }
     return MAIZE_OK;
+}
+
+int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* d) {
+    if (!d) return fail(MAIZE_ERR_NULL, "gemm: descriptor is NULL");
+    const maize_gemm_ex_desc_t x = widen(*d);
+    return maize_hip_gemm_ex_validate(&x);
 }
 
 uint32_t maize_hip_kernel_count(void) { return maize::kernel_count(); }
@@ -265,13 +294,13 @@ int32_t maize_hip_kernel_supports(const char* kernel, const maize_gemm_desc_t* d
     if (rc != MAIZE_OK) return rc;
     const int idx = maize::kernel_index(kernel);
     if (idx < 0) return fail(MAIZE_ERR_KERNEL, "kernel_supports: no kernel named %s", kernel);
-    return maize::kernel_at((uint32_t)idx).supports(*desc) ? 1 : 0;
+    return maize::kernel_at((uint32_t)idx).supports(widen(*desc)) ? 1 : 0;
 }
 
-int32_t maize_hip_gemm_plan(const maize_gemm_desc_t* desc, const char* kernel, uint32_t compute_units,
-                            maize_gemm_plan_t* out) {
+int32_t maize_hip_gemm_ex_plan(const maize_gemm_ex_desc_t* desc, const char* kernel, uint32_t compute_units,
+                               maize_gemm_plan_t* out) {
     if (!out) return fail(MAIZE_ERR_NULL, "gemm_plan: NULL argument");
-    int32_t rc = maize_hip_gemm_validate(desc);
+    int32_t rc = maize_hip_gemm_ex_validate(desc);
     if (rc != MAIZE_OK) return rc;
     if (compute_units == 0) return fail(MAIZE_ERR_ARG, "gemm_plan: compute_units must be positive");
     int idx;
@@ -296,11 +325,19 @@ int32_t maize_hip_gemm_plan(const maize_gemm_desc_t* desc, const char* kernel, u
     return MAIZE_OK;
 }
 
+int32_t maize_hip_gemm_plan(const maize_gemm_desc_t* desc, const char* kernel, uint32_t compute_units,
+                            maize_gemm_plan_t* out) {
+    if (!out) return fail(MAIZE_ERR_NULL, "gemm_plan: NULL argument");
+    if (!desc) return fail(MAIZE_ERR_NULL, "gemm: descriptor is NULL");
+    const maize_gemm_ex_desc_t x = widen(*desc);
+    return maize_hip_gemm_ex_plan(&x, kernel, compute_units, out);
+}
+
 int32_t maize_hip_gemm_select(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, char* name, size_t cap) {
     if (!ctx || !name || cap == 0) return fail(MAIZE_ERR_NULL, "gemm_select: NULL argument");
     int32_t rc = maize_hip_gemm_validate(desc);
     if (rc != MAIZE_OK) return rc;
-    const uint32_t idx = maize::select_kernel(*desc, (uint32_t)ctx->prop.multiProcessorCount);
+    const uint32_t idx = maize::select_kernel(widen(*desc), (uint32_t)ctx->prop.multiProcessorCount);
     snprintf(name, cap, "%s", maize::kernel_at(idx).name);
     return MAIZE_OK;
 }
@@ -326,8 +363,9 @@ static int32_t workspace_for(maize_ctx_t* ctx, void* stream, size_t bytes, void*
     return MAIZE_OK;
 }
 
-static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_desc_t* d, uint32_t idx, void* stream) {
+static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint32_t idx, void* stream) {
     const maize::KernelInfo& ki = maize::kernel_at(idx);
+    const maize_gemm_desc_t* d = &x->gemm;
     maize_gemm_args_t args;
     memset(&args, 0, sizeof args);
     args.a = d->a.ptr; args.arows = d->a.nrows; args.acols = d->a.ncols;
@@ -338,8 +376,11 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_desc_t* d, uint32_
     if (d->batch > 1) {
         args.stride_a = d->stride_a; args.stride_b = d->stride_b; args.stride_c = d->stride_c;
     }
+    args.lda = x->lda; args.ldb = x->ldb; args.ldc = x->ldc;
+    args.alpha = x->alpha; args.beta = x->beta;
+    args.epi = (x->out_type == MAIZE_OUT_F32 ? 1u : 0u) | ((x->alpha != 1.0f || x->beta != 0.0f) ? 2u : 0u);
     maize::LaunchDims ld;
-    if (!ki.plan(*d, (uint32_t)ctx->prop.multiProcessorCount, &ld))
+    if (!ki.plan(*x, (uint32_t)ctx->prop.multiProcessorCount, &ld))
         return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s cannot run M=%u N=%u K=%u batch=%u (grid limit)", ki.name,
                     d->c.nrows, d->c.ncols, d->a.ncols, d->batch);
     args.ksplit = ld.ksplit;
@@ -352,22 +393,30 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_desc_t* d, uint32_
                       ld.lds_bytes, stream, &args, sizeof args);
 }
 
+int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const char* kernel, void* stream) {
+    if (!ctx) return fail(MAIZE_ERR_NULL, "gemm: ctx is NULL");
+    int32_t rc = maize_hip_gemm_ex_validate(desc);
+    if (rc != MAIZE_OK) return rc;
+    if (!kernel) return gemm_launch(ctx, desc, maize::select_kernel(*desc, (uint32_t)ctx->prop.multiProcessorCount), stream);
+    const int idx = maize::kernel_index(kernel);
+    if (idx < 0) return fail(MAIZE_ERR_KERNEL, "gemm: no kernel named %s", kernel);
+    if (!maize::kernel_at((uint32_t)idx).supports(*desc))
+        return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s does not support this descriptor", kernel);
+    return gemm_launch(ctx, desc, (uint32_t)idx, stream);
+}
+
 int32_t maize_hip_gemm_bf16(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "gemm: ctx is NULL");
-    int32_t rc = maize_hip_gemm_validate(desc);
-    if (rc != MAIZE_OK) return rc;
-    return gemm_launch(ctx, desc, maize::select_kernel(*desc, (uint32_t)ctx->prop.multiProcessorCount), stream);
+    if (!desc) return fail(MAIZE_ERR_NULL, "gemm: descriptor is NULL");
+    const maize_gemm_ex_desc_t x = widen(*desc);
+    return maize_hip_gemm_bf16_ex(ctx, &x, nullptr, stream);
 }
 
 int32_t maize_hip_gemm_bf16_with(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, const char* kernel, void* stream) {
     if (!ctx || !kernel) return fail(MAIZE_ERR_NULL, "gemm_with: NULL argument");
-    int32_t rc = maize_hip_gemm_validate(desc);
-    if (rc != MAIZE_OK) return rc;
-    const int idx = maize::kernel_index(kernel);
-    if (idx < 0) return fail(MAIZE_ERR_KERNEL, "gemm_with: no kernel named %s", kernel);
-    if (!maize::kernel_at((uint32_t)idx).supports(*desc))
-        return fail(MAIZE_ERR_KERNEL, "gemm_with: kernel %s does not support this descriptor", kernel);
-    return gemm_launch(ctx, desc, (uint32_t)idx, stream);
+    if (!desc) return fail(MAIZE_ERR_NULL, "gemm: descriptor is NULL");
+    const maize_gemm_ex_desc_t x = widen(*desc);
+    return maize_hip_gemm_bf16_ex(ctx, &x, kernel, stream);
 }
 
 /* ---- thin pass-throughs ------------------------------------------------------ */

@@ -84,6 +84,49 @@ def ref_gemm_rows(a, b, m, n, k, rows, layout=NN, want_abs=True, nthreads=None):
     return c, f64, ab
 
 
+def bf16_bits_from_f64(x):
+    """Round an array of doubles to bf16 bit patterns with the oracle's own RNE (mzo_bf16_from_f64)."""
+    L = lib()
+    flat = np.asarray(x, dtype=np.float64).ravel()
+    return np.fromiter((L.mzo_bf16_from_f64(float(v)) for v in flat), dtype=np.uint16, count=flat.size).reshape(np.shape(x))
+
+
+def bf16_bits_to_f64(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
+def ref_gemm_ex(a, b, m, n, k, layout=NN, lda=None, ldb=None, alpha=1.0, beta=0.0, c_old=None, out_f32=False,
+                nthreads=None):
+    """The extended product for one batch member, on operand views with leading dimensions:
+        C = round( alpha * (A.B in fp64) + beta * C_old ),   round = RNE to bf16, or to fp32.
+    ``a`` and ``b`` are flat uint16 arrays holding the views (row r of A starts at r*lda); ``c_old`` is a
+    dense M x N array (bf16 bits or float32) or None when beta == 0.  alpha and beta are taken as fp32
+    values.  Returns (C dense M x N: uint16 bits or float32, exact fp64 value, error scale
+    |alpha| * sum|a||b| + |beta| * |C_old|).  The product itself is mzo_ref_gemm_bf16's fp64 sum; the
+    scaling is two more fp64 operations (relative error 2^-52, far below either output format)."""
+    brows, bcols = (k, n) if layout == NN else (n, k)
+    lda = k if lda is None else lda
+    ldb = bcols if ldb is None else ldb
+    a = np.asarray(a, dtype=np.uint16).ravel()
+    b = np.asarray(b, dtype=np.uint16).ravel()
+    av = np.lib.stride_tricks.as_strided(a, shape=(m, k), strides=(2 * lda, 2))
+    bv = np.lib.stride_tricks.as_strided(b, shape=(brows, bcols), strides=(2 * ldb, 2))
+    assert a.size >= (m - 1) * lda + k and b.size >= (brows - 1) * ldb + bcols
+    _, f64, ab = ref_gemm(np.ascontiguousarray(av), np.ascontiguousarray(bv), m, n, k, layout=layout, want_f64=True,
+                          want_abs=True, nthreads=nthreads)
+    alpha = float(np.float32(alpha))
+    beta = float(np.float32(beta))
+    val = alpha * f64[0]
+    scale = abs(alpha) * ab[0]
+    if beta != 0.0:
+        old = np.asarray(c_old).reshape(m, n)
+        old64 = bf16_bits_to_f64(old) if old.dtype == np.uint16 else old.astype(np.float64)
+        val = val + beta * old64
+        scale = scale + abs(beta) * np.abs(old64)
+    out = val.astype(np.float32) if out_f32 else bf16_bits_from_f64(val)
+    return out, val, scale
+
+
 # ---- comparator -----------------------------------------------------------------
 
 def _ordinal(bits):

@@ -1,0 +1,130 @@
+"""CPU-only checks of the extended descriptor (leading dimensions, fp32 C, alpha/beta): validation,
+dispatch, and the oracle-side restatement of the extended product against closed forms."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import maize_amd as mz
+from maize_amd import _ffi
+
+
+def ex(m=64, n=64, k=64, layout=mz.LAYOUT_NN, ptrs=(0x1000, 0x100000, 0x2000000), **kw):
+    a = mz.GlobalMatrix(ptrs[0], m, k)
+    b = mz.GlobalMatrix(ptrs[1], k, n) if layout == mz.LAYOUT_NN else mz.GlobalMatrix(ptrs[1], n, k)
+    c = mz.GlobalMatrix(ptrs[2], m, n)
+    return mz.gemm_ex_desc(a, b, c, layout=layout, **kw)
+
+
+def test_plain_descriptor_is_the_all_default_extended_one():
+    x = ex(4096, 4096, 4096)
+    d = x.gemm
+    assert mz.gemm_plan(x) == mz.gemm_plan(d)
+    x = ex(16, 14336, 4096)
+    assert mz.gemm_plan(x) == mz.gemm_plan(x.gemm)
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(lda=63), _ffi.MAIZE_ERR_SHAPE), (dict(ldb=8), _ffi.MAIZE_ERR_SHAPE), (dict(ldc=1), _ffi.MAIZE_ERR_SHAPE),
+    (dict(out_type=7), _ffi.MAIZE_ERR_ARG), (dict(alpha=float("nan")), _ffi.MAIZE_ERR_ARG),
+    (dict(beta=float("nan")), _ffi.MAIZE_ERR_ARG),
+    (dict(batch=2, lda=80, stride_a=64 * 64, stride_b=64 * 64, stride_c=64 * 64), _ffi.MAIZE_ERR_SHAPE),
+])
+def test_validate_rejects(kw, code):
+    with pytest.raises(mz.MaizeError) as e:
+        mz.validate(ex(**kw))
+    assert e.value.code == code
+
+
+def test_validate_rejects_reserved_and_misaligned_fp32_c():
+    x = ex()
+    x.reserved[1] = 1
+    with pytest.raises(mz.MaizeError) as e:
+        mz.validate(x)
+    assert e.value.code == _ffi.MAIZE_ERR_ARG
+    x = ex(ptrs=(0x1000, 0x100000, 0x2000002), out_type=mz.OUT_F32)
+    with pytest.raises(mz.MaizeError) as e:
+        mz.validate(x)
+    assert e.value.code == _ffi.MAIZE_ERR_ALIGN
+    mz.validate(ex(ptrs=(0x1000, 0x100000, 0x2000002)))        # fine for a bf16 C
+    assert _ffi.lib().maize_hip_gemm_ex_validate(None) == _ffi.MAIZE_ERR_NULL
+
+
+def test_accepts_leading_dimensions_and_batches_of_views():
+    mz.validate(ex(lda=64, ldb=64, ldc=64))
+    mz.validate(ex(lda=100, ldb=72, ldc=4096))
+    mz.validate(ex(batch=2, lda=80, stride_a=63 * 80 + 64, stride_b=64 * 64, stride_c=64 * 64))
+
+
+def test_dispatch_of_extended_descriptors():
+    big = dict(m=4096, n=4096, k=4096)
+    assert mz.gemm_plan(ex(**big, lda=4104, ldb=4224, ldc=8192))["kernel"] == "maize_gemm_bf16_mt256_nn"
+    assert mz.gemm_plan(ex(**big, layout=mz.LAYOUT_NT, ldb=4104))["kernel"] == "maize_gemm_bf16_mt256_nt"
+    # rows that do not start on 16-byte boundaries: only the any-shape kernel takes them
+    assert mz.gemm_plan(ex(**big, lda=4100))["kernel"] == "maize_gemm_bf16_wave32"
+    # the macro-tile epilogue stores bf16 of A.B only
+    for kw in (dict(alpha=0.5), dict(beta=1.0), dict(out_type=mz.OUT_F32)):
+        x = ex(**big, **kw)
+        assert mz.gemm_plan(x)["kernel"] == "maize_gemm_bf16_wave32"
+        assert not _supports("maize_gemm_bf16_mt256_nn", x)
+    # the skinny kernel carries the general epilogue
+    for kw in (dict(alpha=0.5, beta=2.0), dict(out_type=mz.OUT_F32), dict(ldb=14400, ldc=14344)):
+        assert mz.gemm_plan(ex(16, 14336, 4096, **kw))["kernel"] == "maize_gemm_bf16_skinny_nn"
+    assert mz.gemm_plan(ex(16, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_wave32"
+
+
+def _supports(name, x):
+    try:
+        mz.gemm_plan(x, kernel=name)
+        return True
+    except mz.MaizeError as e:
+        assert e.code == _ffi.MAIZE_ERR_KERNEL
+        return False
+
+
+# ---- the oracle's extended product against what the mathematics fixes -------------------
+
+def _bits(x):
+    return (np.asarray(x, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def test_oracle_ex_closed_forms(oracle):
+    rng = np.random.default_rng(5)
+    m, n, k = 9, 12, 16
+    a = _bits(rng.integers(-3, 4, (m, k)).astype(np.float32))             # |sum| <= 16 * 9 < 256: exact even in bf16
+    b = _bits(rng.integers(-3, 4, (k, n)).astype(np.float32))
+    exact = oracle.bf16_bits_to_f64(a).reshape(m, k) @ oracle.bf16_bits_to_f64(b).reshape(k, n)
+    c_old = _bits(rng.integers(-4, 5, (m, n)).astype(np.float32))
+    old = oracle.bf16_bits_to_f64(c_old)
+    # fp32 output of exact integer sums: exact
+    out, val, _ = oracle.ref_gemm_ex(a, b, m, n, k, out_f32=True)
+    assert out.dtype == np.float32 and np.array_equal(out.astype(np.float64), exact) and np.array_equal(val, exact)
+    # alpha = 0, beta = 1: C comes back unchanged; alpha = 1, beta = 0: C_old (here NaN) is never read
+    out, _, _ = oracle.ref_gemm_ex(a, b, m, n, k, alpha=0.0, beta=1.0, c_old=c_old)
+    assert np.array_equal(out, c_old)
+    out, _, _ = oracle.ref_gemm_ex(a, b, m, n, k, alpha=1.0, beta=0.0, c_old=np.full((m, n), 0x7FC0, np.uint16))
+    assert np.array_equal(oracle.bf16_bits_to_f64(out), exact)
+    # powers of two scale exactly; the general case is one rounding of the exact value
+    out, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, alpha=0.5, beta=-2.0, c_old=c_old, out_f32=True)
+    assert np.array_equal(val, 0.5 * exact - 2.0 * old) and np.array_equal(out.astype(np.float64), val)
+    assert np.array_equal(scale, 0.5 * (np.abs(oracle.bf16_bits_to_f64(a).reshape(m, k)) @ np.abs(oracle.bf16_bits_to_f64(b).reshape(k, n))) + 2.0 * np.abs(old))
+    out, val, _ = oracle.ref_gemm_ex(a, b, m, n, k, alpha=3.0, beta=0.25, c_old=c_old)
+    want = np.array([oracle.lib().mzo_bf16_from_f64(float(v)) for v in (3.0 * exact + 0.25 * old).ravel()], np.uint16).reshape(m, n)
+    assert np.array_equal(out, want)
+
+
+def test_oracle_ex_views_equal_compact_copies(oracle):
+    rng = np.random.default_rng(6)
+    m, n, k, lda, ldb = 7, 10, 24, 40, 16
+    for layout in (oracle.NN, oracle.NT):
+        brows, bcols = (k, n) if layout == oracle.NN else (n, k)
+        ldb_ = max(ldb, bcols + 3)
+        a = rng.integers(0, 0x4000, m * lda).astype(np.uint16)            # finite positive bf16 patterns, padding included
+        b = rng.integers(0, 0x4000, brows * ldb_).astype(np.uint16)
+        ac = a.reshape(m, lda)[:, :k].copy()
+        bc = b.reshape(brows, ldb_)[:, :bcols].copy()
+        got = oracle.ref_gemm_ex(a, b, m, n, k, layout=layout, lda=lda, ldb=ldb_)
+        want = oracle.ref_gemm_ex(ac, bc, m, n, k, layout=layout)
+        plain, f64, _ = oracle.ref_gemm(ac, bc, m, n, k, layout=layout, want_f64=True, want_abs=True)
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+        assert np.array_equal(got[0].ravel(), plain) and np.array_equal(got[1], f64[0])

@@ -1,0 +1,143 @@
+"""GPU parity of the extended product (leading dimensions, fp32 C, C = alpha * A.B + beta * C),
+through maize_hip_gemm_bf16_ex, against the oracle's restatement on the same inputs.
+
+Tolerances.  bf16 C: the bar of the plain product -- within 1 bf16 ULP of the oracle's bits, or,
+where the result nearly cancels, |got - exact| <= (K/16 + 2) * 2^-24 * scale + half a bf16 ULP of
+the value returned, with scale = |alpha| * sum|a||b| + |beta| * |C_old|.  fp32 C: |got - exact| <=
+(K/16 + 4) * 2^-24 * scale (the accumulation bound plus the roundings of alpha * acc, the fused
+beta * C + ..., and the fp32 result itself)."""
+import sys
+
+import numpy as np
+import pytest
+
+import maize_amd as mz
+
+pytestmark = pytest.mark.gpu
+
+
+
+def _say(msg):
+    print(f"[gemm_ex] {msg}", file=sys.stderr, flush=True)
+
+
+def run_ex(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, lda=None, ldb=None, ldc=None, alpha=1.0, beta=0.0, out_f32=False,
+           kernel=None, seed=1, c_nan=False, label=""):
+    """One launch on padded views whose padding (and C's) holds canaries; checks the result against the
+    oracle and that nothing outside the M x N view of C changed.  Returns the kernel the dispatcher took."""
+    brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+    lda = k if lda is None else lda
+    ldb = bcols if ldb is None else ldb
+    ldc = n if ldc is None else ldc
+    a = mz.gen.uniform_bf16(m * lda, 100 + seed)
+    b = mz.gen.uniform_bf16(brows * ldb, 200 + seed)
+    cdt = np.float32 if out_f32 else np.uint16
+    if out_f32:
+        c0 = (np.random.default_rng(seed).standard_normal(m * ldc) * 2).astype(np.float32)
+    else:
+        c0 = mz.gen.uniform_bf16(m * ldc, 300 + seed)
+    if c_nan:
+        c0 = np.full(m * ldc, np.nan, np.float32) if out_f32 else np.full(m * ldc, 0x7FC0, np.uint16)
+    da, db, dc = ctx.upload(a), ctx.upload(b), ctx.upload(c0)
+    try:
+        x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, brows, bcols), mz.Matrix(dc, m, n), layout=layout,
+                            lda=0 if lda == k else lda, ldb=0 if ldb == bcols else ldb, ldc=0 if ldc == n else ldc,
+                            out_type=mz.OUT_F32 if out_f32 else mz.OUT_BF16, alpha=alpha, beta=beta)
+        took = mz.gemm_plan(x, kernel=kernel, compute_units=ctx.info()["compute_units"])["kernel"]
+        _say(f"{label} M={m} N={n} K={k} ld=({lda},{ldb},{ldc}) alpha={alpha} beta={beta} f32={out_f32} -> {took}")
+        ctx.gemm_bf16(x, kernel=kernel)
+        ctx.sync()
+        got = dc.download(cdt)
+    finally:
+        da.free(); db.free(); dc.free()
+    gv = got.reshape(m, ldc)
+    ov = c0.reshape(m, ldc)
+    # the padding of C's rows is untouched (bit for bit)
+    assert np.array_equal(gv[:, n:].view(np.uint8), ov[:, n:].view(np.uint8)), f"{label}: wrote into C's row padding"
+    ref, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, layout=layout, lda=lda, ldb=ldb, alpha=alpha, beta=beta,
+                                         c_old=None if beta == 0.0 else ov[:, :n].copy(), out_f32=out_f32)
+    g = gv[:, :n]
+    if out_f32:
+        err = np.abs(g.astype(np.float64) - val)
+        tol = (k / 16.0 + 4.0) * 2.0 ** -24 * scale + 1e-45
+        bad = ~(err <= tol)
+        assert not bad.any(), f"{label}: {int(bad.sum())} of {bad.size} fp32 elements out of tolerance, worst {float((err / tol).max()):.2f}x"
+    else:
+        s = oracle.compare(g, ref, val, scale, k)
+        assert s["n_fail"] == 0, f"{label}: {s}"
+    return took
+
+
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape", [(33, 17, 65), (64, 64, 48), (100, 200, 72)])
+def test_any_shape_kernel_all_knobs(ctx, oracle, layout, shape):
+    m, n, k = shape
+    bcols = n if layout == mz.LAYOUT_NN else k
+    for kw in (dict(lda=k + 3, ldb=bcols + 5, ldc=n + 7), dict(alpha=0.5), dict(alpha=-1.25, beta=0.75),
+               dict(out_f32=True), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 1), dict(alpha=0.0, beta=1.0),
+               dict(alpha=2.0, beta=0.0, c_nan=True), dict(out_f32=True, beta=0.0, alpha=1.0, c_nan=True)):
+        run_ex(ctx, oracle, m, n, k, layout=layout, kernel="maize_gemm_bf16_wave32", label="wave32", **kw)
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape,lds", [((256, 256, 64), (72, 264, 320)), ((520, 776, 192), (200, 1000, 784)),
+                                       ((300, 520, 136), (144, 528, 1024))])
+def test_macro_tile_kernels_on_strided_views(ctx, oracle, layout, shape, lds):
+    m, n, k = shape
+    lda, ldb, ldc = lds
+    if layout == mz.LAYOUT_NT:
+        ldb = max(k + 8, 200)
+    took = run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, label="mt256 views")
+    assert took.startswith("maize_gemm_bf16_mt256"), took
+    # each variant that accepts the shape, by name
+    for name in mz.kernel_names():
+        if not name.startswith("maize_gemm_bf16_mt256") or ("_nt" in name) != (layout == mz.LAYOUT_NT):
+            continue
+        if "ktail" not in name and k % 64:
+            continue
+        run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, kernel=name, label=name)
+
+
+def test_macro_tile_view_of_a_larger_matrix_matches_the_compact_run(ctx, oracle):
+    """A 512 x 512 x 256 product taken out of the middle of larger buffers equals (bit for bit) the same product
+    on compact copies: leading dimensions change addresses, not arithmetic."""
+    m, n, k, lda, ldb, ldc = 512, 512, 256, 1024, 2048, 640
+    a = mz.gen.uniform_bf16(m * lda, 7)
+    b = mz.gen.uniform_bf16(k * ldb, 8)
+    ac = a.reshape(m, lda)[:, :k].copy()
+    bc = b.reshape(k, ldb)[:, :n].copy()
+    outs = []
+    for (aa, bb, la, lb, lc) in ((a, b, lda, ldb, ldc), (ac, bc, 0, 0, 0)):
+        da, db = ctx.upload(aa), ctx.upload(bb)
+        dc = ctx.malloc(m * (lc or n) * 2)
+        dc.fill(0)
+        x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n), mz.Matrix(dc, m, n), lda=la, ldb=lb, ldc=lc)
+        ctx.gemm_bf16(x)
+        ctx.sync()
+        outs.append(dc.download(np.uint16).reshape(m, lc or n)[:, :n].copy())
+        da.free(); db.free(); dc.free()
+    assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("m", [1, 7, 16])
+def test_skinny_kernel_all_knobs(ctx, oracle, m):
+    n, k = 1024, 2048
+    for kw in (dict(ldb=n + 8, ldc=n + 16, lda=k + 8), dict(alpha=0.5), dict(alpha=-1.25, beta=0.75),
+               dict(out_f32=True), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(alpha=0.0, beta=1.0),
+               dict(alpha=2.0, beta=0.0, c_nan=True)):
+        took = run_ex(ctx, oracle, m, n, k, label="skinny", **kw)
+        assert took == "maize_gemm_bf16_skinny_nn", took
+    # single K range (no workspace): a narrow N with a short K
+    took = run_ex(ctx, oracle, m, 4096, 256, alpha=1.5, beta=0.5, out_f32=True, ldc=4104, label="skinny ks=1")
+    assert took == "maize_gemm_bf16_skinny_nn", took
+
+
+def test_large_shape_with_general_epilogue_still_computes(ctx, oracle):
+    """alpha/beta or an fp32 C on a shape the macro-tile kernels would take: the dispatcher falls back to the
+    any-shape kernel rather than refusing."""
+    took = run_ex(ctx, oracle, 384, 512, 256, alpha=0.5, beta=1.0, label="fallback")
+    assert took == "maize_gemm_bf16_wave32"
+    took = run_ex(ctx, oracle, 384, 512, 256, out_f32=True, label="fallback f32")
+    assert took == "maize_gemm_bf16_wave32"

@@ -39,7 +39,11 @@ def test_struct_layouts_match_the_reference_abi():
     A = _ffi.GemmArgsT
     assert (A.a.offset, A.arows.offset, A.acols.offset, A.b.offset, A.brows.offset, A.bcols.offset) == (0, 8, 12, 16, 24, 28)
     assert (A.c.offset, A.crows.offset, A.ccols.offset) == (32, 40, 44)
-    assert C.sizeof(A) == 96 and C.sizeof(_ffi.GemmDescT) == 80
+    assert C.sizeof(A) == 120 and C.sizeof(_ffi.GemmDescT) == 80
+    # the extension sits behind the fields the plain kernels read; all-zero = compact rows, bf16 C = A.B
+    assert (A.lda.offset, A.ldb.offset, A.ldc.offset, A.epi.offset, A.alpha.offset, A.beta.offset) == (96, 100, 104, 108, 112, 116)
+    X = _ffi.GemmExDescT
+    assert C.sizeof(X) == 112 and (X.lda.offset, X.out_type.offset, X.alpha.offset, X.beta.offset) == (80, 92, 96, 100)
 
 
 def test_embedded_code_object_is_a_gfx950_elf_with_all_kernels():
