@@ -56,14 +56,20 @@ bool mt256_common(const maize_gemm_ex_desc_t& d) {
     const Lds l = lds_of(d);
     if (l.ext_a * 2 >= lim || l.ext_b * 2 >= lim || l.ext_c * 2 >= lim) return false;
     if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21)) return false;
-    return plain_epilogue(d);                               // the staged epilogue stores bf16 of A.B only
+    return true;
 }
 // The plain kernels advance K with a scalar offset and never mask a lane in K: K % 64 == 0.
 bool k64(const maize_gemm_ex_desc_t& d) { return (d.gemm.a.ncols & 63u) == 0; }
-bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NN && mt256_common(d) && k64(d); }
-bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NT && mt256_common(d) && k64(d); }
-bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NN && mt256_common(d); }
-bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NT && mt256_common(d); }
+// The plain and edge-splitting kernels store bf16 of A.B only; the _gen kernels carry the general epilogue.
+bool nn(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NN; }
+bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d); }
+bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d); }
+bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && plain_epilogue(d); }
+bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && plain_epilogue(d); }
+bool mt256_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d); }
+bool mt256_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d); }
+bool mt256_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d); }
+bool mt256_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d); }
 // Edge splitting.  A ragged N leaves a last column of tiles that are almost empty but cost a
 // whole tile each (likewise a ragged M and the last row).  When that edge is at most 32 elements
 // wide and setting it aside saves a round of workgroups (one workgroup per compute unit per
@@ -168,6 +174,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nn_ktail_edge", mt256_nn_ktail_supports, mt256_edge_plan},
     {"maize_gemm_bf16_mt256_nt_ktail_edge", mt256_nt_ktail_supports, mt256_edge_plan},
     {"maize_gemm_bf16_skinny_nn", skinny_nn_supports, skinny_plan},
+    {"maize_gemm_bf16_mt256_nn_gen", mt256_nn_gen_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nt_gen", mt256_nt_gen_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_ktail_gen", mt256_nn_ktail_gen_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nt_ktail_gen", mt256_nt_ktail_gen_supports, mt256_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -192,8 +202,12 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
          {"maize_gemm_bf16_mt256_nn_ktail", "maize_gemm_bf16_mt256_nt_ktail"}},
         {{"maize_gemm_bf16_mt256_nn_edge", "maize_gemm_bf16_mt256_nt_edge"},
          {"maize_gemm_bf16_mt256_nn_ktail_edge", "maize_gemm_bf16_mt256_nt_ktail_edge"}}};
+    static const char* const kGeneral[2][2] = {    // [K tail][NT]: alpha / beta / fp32 C
+        {"maize_gemm_bf16_mt256_nn_gen", "maize_gemm_bf16_mt256_nt_gen"},
+        {"maize_gemm_bf16_mt256_nn_ktail_gen", "maize_gemm_bf16_mt256_nt_ktail_gen"}};
     const bool edge = mt256_edge(s, d.gemm.batch, compute_units).mode != 0;
-    const int ti = kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt]);
+    const int ti = plain_epilogue(d) ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
+                                     : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
     // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below
     // half a tile in either direction the per-wave kernel wastes less.
     if (ti >= 0 && kKernels[ti].supports(d) && s.m >= 128 && s.n >= 128) return (uint32_t)ti;

@@ -1,4 +1,4 @@
-// maize_gemm_bf16_mt256_{nn,nt}[_ktail][_edge]: the pipelined macro-tile kernel.
+// maize_gemm_bf16_mt256_{nn,nt}[_ktail][_edge | _gen]: the pipelined macro-tile kernel.
 //
 // The reference schedule (sm80_gemm_smem_multibuffer, crates/maize_tile/src/
 // gemm/mod.rs:37-90: prime a ring of shared-memory TilePairs, then
@@ -36,6 +36,9 @@
 //     writes the part of its fp32 partial tile that lies inside the matrix to a library-owned
 //     workspace (device-coherent stores), takes a ticket with a device-scope atomic, and the last
 //     arriver re-reads all partials in range order (deterministic), then runs the normal epilogue.
+//
+// The _gen kernels are the plain (persistent) kernels with the general epilogue: C = alpha * A.B +
+// beta * C, C in bf16 or fp32.
 //
 // Requirements (checked by the dispatcher): K % 8 == 0, N % 8 == 0, 16-byte
 // aligned operands, each matrix (per batch member) below 2 GiB.  The plain
@@ -99,7 +102,7 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 
 #define MAIZE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <bool NT, bool KTAIL, bool EDGE>
+template <bool NT, bool KTAIL, bool EDGE, bool GEN>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     // Four separate arrays (operand x ring stage): the compiler can then tell that a
     // direct-to-LDS load into one stage does not alias fragment reads of the other, and does
@@ -188,7 +191,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         n0 = tile_n * BN;
         Ag = p.a + bz * p.stride_a;
         Bg = p.b + bz * p.stride_b;
-        Cg = p.c + bz * p.stride_c;
+        Cg = p.c + bz * p.stride_c * ((GEN && (p.epi & EPI_F32)) ? 2u : 1u);   // strides count elements of C
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t row = (wave * 8u + i) * 8u + (lane >> 3);
@@ -420,33 +423,68 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // bit 4 of the row, so the 8-byte writes of 32 rows and the 16-byte reads of 4 rows are
     // conflict free.  The region is wave-private and LDS operations of one wave complete in
     // order, so no barrier is needed between the passes.
-    lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
-    const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per read
-    const uint32_t gcol = en0 + wn * 128u + cc * 8u;
-    const bool col_ok = gcol < N;                            // N % 8 == 0: a chunk is all in or all out
+    if (GEN) {
+        // General epilogue (alpha, beta, fp32 C): the sub-tile is staged as fp32, 32 rows x 64 columns
+        // at a time (row = 256 B, 16-byte chunk index XOR-ed with row%16), read back as runs of 8
+        // consecutive columns of a row and finished by store_c_run.
+        lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
+        const uint32_t c8 = lane & 7u, r8 = lane >> 3;           // 8 lanes per 64-column row, 8 rows per read
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+            for (int jh = 0; jh < 2; ++jh) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                // lane holds C[row = i*32 + l32][col = j*32 + 8q + 4*lhi + 0..3]
-                floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                if (EDGE && split) f = reduced_chunk(i * 16 + j * 4 + q);
-                u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
-                const uint32_t chunk = (uint32_t)(j * 4 + q) ^ (l32 & 15u);
-                const uint32_t hf = lhi ^ ((l32 >> 4) & 1u);
-                *(lds_v2)(ew + l32 * 256u + chunk * 16u + hf * 8u) = v;
+                for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int j = jh * 2 + jj;
+                        // lane holds C[row = i*32 + l32][col = j*32 + 8q + 4*lhi + 0..3]
+                        const floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                        const uint32_t chunk = ((uint32_t)(jj * 8 + q * 2) + lhi) ^ (l32 & 15u);
+                        *(__attribute__((address_space(3))) floatx4*)(ew + l32 * 256u + chunk * 16u) = f;
+                    }
+                const uint32_t gcol = en0 + wn * 128u + jh * 64u + c8 * 8u;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t row = r * 8 + r8;                 // 0..31 within the pass
+                    const floatx4 lo = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8) ^ (row & 15u)) * 16u));
+                    const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8 + 1u) ^ (row & 15u)) * 16u));
+                    const uint32_t grow = em0 + wm * 128u + i * 32u + row;
+                    if (gcol < N && grow < M) {                   // N % 8 == 0: a run is all in or all out
+                        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        store_c_run<8>(p, Ce, (uint64_t)grow * ldc + gcol, v);
+                    }
+                }
             }
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            const uint32_t row = r * 4 + cr;                 // 0..31 within the pass
-            u32x4 v = *(lds_v4)(ew + row * 256u + ((cc ^ (row & 15u)) * 16u));
-            if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
-            const uint32_t grow = em0 + wm * 128u + i * 32u + row;
-            // C is written once and not read again by this kernel: non-temporal stores keep it from
-            // displacing the operand panels in L2.
-            if (col_ok && grow < M) __builtin_nontemporal_store(v, (u32x4*)(Ce + (uint64_t)grow * ldc + gcol));
+    } else {
+        lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
+        const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per read
+        const uint32_t gcol = en0 + wn * 128u + cc * 8u;
+        const bool col_ok = gcol < N;                            // N % 8 == 0: a chunk is all in or all out
+    #pragma unroll
+        for (int i = 0; i < 4; ++i) {
+    #pragma unroll
+            for (int j = 0; j < 4; ++j)
+    #pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    // lane holds C[row = i*32 + l32][col = j*32 + 8q + 4*lhi + 0..3]
+                    floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    if (EDGE && split) f = reduced_chunk(i * 16 + j * 4 + q);
+                    u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
+                    const uint32_t chunk = (uint32_t)(j * 4 + q) ^ (l32 & 15u);
+                    const uint32_t hf = lhi ^ ((l32 >> 4) & 1u);
+                    *(lds_v2)(ew + l32 * 256u + chunk * 16u + hf * 8u) = v;
+                }
+    #pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const uint32_t row = r * 4 + cr;                 // 0..31 within the pass
+                u32x4 v = *(lds_v4)(ew + row * 256u + ((cc ^ (row & 15u)) * 16u));
+                if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
+                const uint32_t grow = em0 + wm * 128u + i * 32u + row;
+                // C is written once and not read again by this kernel: non-temporal stores keep it from
+                // displacing the operand panels in L2.
+                if (col_ok && grow < M) __builtin_nontemporal_store(v, (u32x4*)(Ce + (uint64_t)grow * ldc + gcol));
+            }
         }
     }
     if (!more) break;
@@ -457,7 +495,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 }  // namespace mt256
 
 #define MAIZE_MT256_KERNEL(name, nt, ktail, edge) \
-    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, edge>(p); }
+    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, edge, false>(p); }
+#define MAIZE_MT256_KERNEL_GEN(name, nt, ktail) \
+    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, false, true>(p); }
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn, false, false, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt, true, false, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail, false, true, false)
@@ -466,6 +506,11 @@ MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_edge, false, false, true)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_edge, true, false, true)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail_edge, false, true, true)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_ktail_edge, true, true, true)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nn_gen, false, false)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nt_gen, true, false)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nn_ktail_gen, false, true)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nt_ktail_gen, true, true)
 #undef MAIZE_MT256_KERNEL
+#undef MAIZE_MT256_KERNEL_GEN
 
 }  // namespace maize

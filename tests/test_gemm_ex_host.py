@@ -62,11 +62,14 @@ def test_dispatch_of_extended_descriptors():
     assert mz.gemm_plan(ex(**big, layout=mz.LAYOUT_NT, ldb=4104))["kernel"] == "maize_gemm_bf16_mt256_nt"
     # rows that do not start on 16-byte boundaries: only the any-shape kernel takes them
     assert mz.gemm_plan(ex(**big, lda=4100))["kernel"] == "maize_gemm_bf16_wave32"
-    # the macro-tile epilogue stores bf16 of A.B only
+    # alpha / beta / fp32 C: the macro-tile kernels with the general epilogue; the plain ones refuse
     for kw in (dict(alpha=0.5), dict(beta=1.0), dict(out_type=mz.OUT_F32)):
         x = ex(**big, **kw)
-        assert mz.gemm_plan(x)["kernel"] == "maize_gemm_bf16_wave32"
-        assert not _supports("maize_gemm_bf16_mt256_nn", x)
+        assert mz.gemm_plan(x)["kernel"] == "maize_gemm_bf16_mt256_nn_gen"
+        assert mz.gemm_plan(ex(4096, 4096, 4040, layout=mz.LAYOUT_NT, **kw))["kernel"] == "maize_gemm_bf16_mt256_nt_ktail_gen"
+        assert not _supports("maize_gemm_bf16_mt256_nn", x) and not _supports("maize_gemm_bf16_mt256_nn_edge", x)
+        assert _supports("maize_gemm_bf16_mt256_nn_gen", x) and _supports("maize_gemm_bf16_mt256_nn_ktail_gen", x)
+    assert _supports("maize_gemm_bf16_mt256_nn_gen", ex(**big))          # and they take the plain product too
     # the skinny kernel carries the general epilogue
     for kw in (dict(alpha=0.5, beta=2.0), dict(out_type=mz.OUT_F32), dict(ldb=14400, ldc=14344)):
         assert mz.gemm_plan(ex(16, 14336, 4096, **kw))["kernel"] == "maize_gemm_bf16_skinny_nn"

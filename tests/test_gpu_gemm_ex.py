@@ -134,10 +134,44 @@ def test_skinny_kernel_all_knobs(ctx, oracle, m):
     assert took == "maize_gemm_bf16_skinny_nn", took
 
 
-def test_large_shape_with_general_epilogue_still_computes(ctx, oracle):
-    """alpha/beta or an fp32 C on a shape the macro-tile kernels would take: the dispatcher falls back to the
-    any-shape kernel rather than refusing."""
-    took = run_ex(ctx, oracle, 384, 512, 256, alpha=0.5, beta=1.0, label="fallback")
-    assert took == "maize_gemm_bf16_wave32"
-    took = run_ex(ctx, oracle, 384, 512, 256, out_f32=True, label="fallback f32")
-    assert took == "maize_gemm_bf16_wave32"
+KNOBS = (dict(alpha=0.5), dict(alpha=-1.25, beta=0.75), dict(out_f32=True), dict(out_f32=True, alpha=3.0, beta=-0.5),
+         dict(alpha=0.0, beta=1.0), dict(alpha=2.0, beta=0.0, c_nan=True), dict(out_f32=True, c_nan=True), dict())
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape,lds", [((256, 256, 128), None), ((520, 776, 192), (200, 1000, 784)), ((300, 520, 136), (144, 528, 1024))])
+def test_macro_tile_general_epilogue(ctx, oracle, layout, shape, lds):
+    """alpha / beta / fp32 C on shapes the macro-tile kernels take: the _gen variants, compact and strided,
+    with and without a K tail, ragged M and N."""
+    m, n, k = shape
+    lda, ldb, ldc = lds if lds else (None, None, None)
+    if lds and layout == mz.LAYOUT_NT:
+        ldb = max(k + 8, 200)
+    want = "maize_gemm_bf16_mt256_" + ("nt" if layout == mz.LAYOUT_NT else "nn") + ("_ktail" if k % 64 else "") + "_gen"
+    for kw in KNOBS[:-1]:
+        took = run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, label="mt256 gen", **kw)
+        assert took == want, took
+    # the plain product through the general epilogue
+    run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, kernel=want, label="mt256 gen plain")
+
+
+def test_general_epilogue_with_several_tiles_per_workgroup_and_batches(ctx, oracle):
+    """More tiles than workgroups would be resident (forced by a raw launch with a small grid is covered
+    elsewhere); here: a batched fp32 product with beta, through the dispatcher."""
+    m, n, k, batch = 256, 384, 128, 3
+    a = mz.gen.uniform_bf16(batch * m * k, 21)
+    b = mz.gen.uniform_bf16(batch * k * n, 22)
+    c0 = np.random.default_rng(3).standard_normal(batch * m * n).astype(np.float32)
+    da, db, dc = ctx.upload(a), ctx.upload(b), ctx.upload(c0)
+    x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n), mz.Matrix(dc, m, n), batch=batch, stride_a=m * k,
+                        stride_b=k * n, stride_c=m * n, out_type=mz.OUT_F32, alpha=0.75, beta=1.5)
+    assert mz.gemm_plan(x)["kernel"] == "maize_gemm_bf16_mt256_nn_gen"
+    ctx.gemm_bf16(x)
+    ctx.sync()
+    got = dc.download(np.float32).reshape(batch, m, n)
+    da.free(); db.free(); dc.free()
+    for i in range(batch):
+        _, val, scale = oracle.ref_gemm_ex(a[i * m * k:(i + 1) * m * k], b[i * k * n:(i + 1) * k * n], m, n, k, alpha=0.75,
+                                           beta=1.5, c_old=c0.reshape(batch, m, n)[i], out_f32=True)
+        err = np.abs(got[i].astype(np.float64) - val)
+        assert (err <= (k / 16.0 + 4.0) * 2.0 ** -24 * scale + 1e-45).all(), f"batch member {i}"
