@@ -95,6 +95,17 @@ inline maize_gemm_desc_t gemm_desc(const Matrix& a, const Matrix& b, const Matri
 }
 
 // C = A.B through the dispatcher: the reference's mainloop entry, carried through to a launch.
+// The extended descriptor: leading dimensions (0 = ncols), element type of C, C = alpha * A.B + beta * C.
+inline maize_gemm_ex_desc_t gemm_ex_desc(const maize_gemm_desc_t& d, uint32_t lda = 0, uint32_t ldb = 0, uint32_t ldc = 0,
+                                         maize_out_type_t out = MAIZE_OUT_BF16, float alpha = 1.0f, float beta = 0.0f) {
+    maize_gemm_ex_desc_t x{};
+    x.gemm = d;
+    x.lda = lda; x.ldb = ldb; x.ldc = ldc;
+    x.out_type = out;
+    x.alpha = alpha; x.beta = beta;
+    return x;
+}
+
 // Kernel choice and launch geometry for a descriptor; needs no device.
 inline maize_gemm_plan_t gemm_plan(const maize_gemm_desc_t& d, uint32_t compute_units = 256, const char* kernel = nullptr) {
     maize_gemm_plan_t p;
@@ -106,6 +117,10 @@ inline void gemm_smem_multibuffer(Ctx& ctx, const Matrix& a, const Matrix& b, co
                                   void* stream = nullptr) {
     const maize_gemm_desc_t d = gemm_desc(a, b, c, layout);
     check(maize_hip_gemm_bf16(ctx.handle(), &d, stream));
+}
+
+inline void gemm_smem_multibuffer(Ctx& ctx, const maize_gemm_ex_desc_t& x, void* stream = nullptr, const char* kernel = nullptr) {
+    check(maize_hip_gemm_bf16_ex(ctx.handle(), &x, kernel, stream));
 }
 
 // ---- builder chain: kernel name -> launch bounds -> finalize -> compile(target) -> launch ------
