@@ -86,13 +86,19 @@ typedef struct {
  *   out_type:    element type of C; batch stride stride_c counts elements of that type.
  *   beta == 0:   C is not read (it may hold anything, NaNs included).
  * All-zero extension fields with alpha = 1 describe exactly the plain descriptor. */
-typedef enum { MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1 } maize_out_type_t;
+/* MAIZE_OUT_SAME: C has the 16-bit type of A and B (bf16, or half for half operands). */
+typedef enum { MAIZE_OUT_SAME = 0, MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1 } maize_out_type_t;
+/* Element type of A and B.  The reference's MMA catalogue lists the half-precision twin of its bf16
+ * op (Sm80MmaF16F32_16x8x16 beside Sm80MmaBf16F32_16x8x16, crates/maize_tile/src/mma/sm80.rs);
+ * here it is v_mfma_f32_*_f16 on the same tiles. */
+typedef enum { MAIZE_IN_BF16 = 0, MAIZE_IN_F16 = 1 } maize_in_type_t;
 typedef struct {
     maize_gemm_desc_t gemm;
     uint32_t lda, ldb, ldc;
     uint32_t out_type; /* maize_out_type_t */
     float alpha, beta;
-    uint32_t reserved[2]; /* must be 0 */
+    uint32_t in_type;  /* maize_in_type_t */
+    uint32_t reserved; /* must be 0 */
 } maize_gemm_ex_desc_t;
 
 /* Kernel parameter block of every GEMM kernel in the embedded code object.
@@ -114,7 +120,7 @@ typedef struct {
     uint32_t reserved;
     /* extended part; all zero = compact rows, bf16 C = A.B */
     uint32_t lda, ldb, ldc; /* 0 = ncols */
-    uint32_t epi;           /* bit 0: C is fp32; bit 1: apply alpha and beta */
+    uint32_t epi;           /* bit 0: C is fp32; bit 1: apply alpha and beta; bit 2: A, B (and a 16-bit C) are half */
     float alpha, beta;
 } maize_gemm_args_t;
 

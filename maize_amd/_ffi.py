@@ -35,8 +35,11 @@ MAIZE_ERR_ARG = -7
 
 LAYOUT_NN = 0
 LAYOUT_NT = 1
+OUT_SAME = 0
 OUT_BF16 = 0
 OUT_F32 = 1
+IN_BF16 = 0
+IN_F16 = 1
 
 
 class MatrixT(C.Structure):
@@ -64,7 +67,8 @@ class GemmArgsT(C.Structure):
 class GemmExDescT(C.Structure):
     """maize_gemm_ex_desc_t: the descriptor plus leading dimensions, output type, alpha and beta."""
     _fields_ = [("gemm", GemmDescT), ("lda", C.c_uint32), ("ldb", C.c_uint32), ("ldc", C.c_uint32),
-                ("out_type", C.c_uint32), ("alpha", C.c_float), ("beta", C.c_float), ("reserved", C.c_uint32 * 2)]
+                ("out_type", C.c_uint32), ("alpha", C.c_float), ("beta", C.c_float), ("in_type", C.c_uint32),
+                ("reserved", C.c_uint32)]
 
 
 class DeviceInfoT(C.Structure):

@@ -22,8 +22,9 @@ inline Lds lds_of(const maize_gemm_ex_desc_t& d) {
 }
 // The plain product: bf16 C = A.B (alpha == 1, beta == 0).
 inline bool plain_epilogue(const maize_gemm_ex_desc_t& d) {
-    return d.out_type == MAIZE_OUT_BF16 && d.alpha == 1.0f && d.beta == 0.0f;
+    return d.out_type == MAIZE_OUT_SAME && d.alpha == 1.0f && d.beta == 0.0f;
 }
+inline bool half_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_F16; }
 
 // ---- maize_gemm_bf16_wave32: any shape ------------------------------------
 bool wave32_supports(const maize_gemm_ex_desc_t&) { return true; }
@@ -62,14 +63,19 @@ bool mt256_common(const maize_gemm_ex_desc_t& d) {
 bool k64(const maize_gemm_ex_desc_t& d) { return (d.gemm.a.ncols & 63u) == 0; }
 // The plain and edge-splitting kernels store bf16 of A.B only; the _gen kernels carry the general epilogue.
 bool nn(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NN; }
-bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d); }
-bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d); }
-bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && plain_epilogue(d); }
-bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && plain_epilogue(d); }
-bool mt256_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d); }
-bool mt256_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d); }
-bool mt256_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d); }
-bool mt256_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d); }
+bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && !half_in(d); }
+bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && !half_in(d); }
+bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && plain_epilogue(d) && !half_in(d); }
+bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && plain_epilogue(d) && !half_in(d); }
+bool mt256_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && !half_in(d); }
+bool mt256_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && !half_in(d); }
+bool mt256_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && !half_in(d); }
+bool mt256_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && !half_in(d); }
+// IEEE half operands: the general-epilogue kernels instantiated on v_mfma_f32_32x32x16_f16.
+bool f16_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && half_in(d); }
+bool f16_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && half_in(d); }
+bool f16_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && half_in(d); }
+bool f16_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && half_in(d); }
 // Edge splitting.  A ragged N leaves a last column of tiles that are almost empty but cost a
 // whole tile each (likewise a ragged M and the last row).  When that edge is at most 32 elements
 // wide and setting it aside saves a round of workgroups (one workgroup per compute unit per
@@ -178,6 +184,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_gen", mt256_nt_gen_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_ktail_gen", mt256_nn_ktail_gen_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_ktail_gen", mt256_nt_ktail_gen_supports, mt256_plan},
+    {"maize_gemm_f16_mt256_nn_gen", f16_nn_gen_supports, mt256_plan},
+    {"maize_gemm_f16_mt256_nt_gen", f16_nt_gen_supports, mt256_plan},
+    {"maize_gemm_f16_mt256_nn_ktail_gen", f16_nn_ktail_gen_supports, mt256_plan},
+    {"maize_gemm_f16_mt256_nt_ktail_gen", f16_nt_ktail_gen_supports, mt256_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -206,8 +216,12 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         {"maize_gemm_bf16_mt256_nn_gen", "maize_gemm_bf16_mt256_nt_gen"},
         {"maize_gemm_bf16_mt256_nn_ktail_gen", "maize_gemm_bf16_mt256_nt_ktail_gen"}};
     const bool edge = mt256_edge(s, d.gemm.batch, compute_units).mode != 0;
-    const int ti = plain_epilogue(d) ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
-                                     : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
+    static const char* const kHalf[2][2] = {       // [K tail][NT]: IEEE half operands
+        {"maize_gemm_f16_mt256_nn_gen", "maize_gemm_f16_mt256_nt_gen"},
+        {"maize_gemm_f16_mt256_nn_ktail_gen", "maize_gemm_f16_mt256_nt_ktail_gen"}};
+    const int ti = half_in(d)          ? kernel_index(kHalf[(s.k & 63u) != 0][s.nt])
+                   : plain_epilogue(d) ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
+                                       : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
     // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below
     // half a tile in either direction the per-wave kernel wastes less.
     if (ti >= 0 && kKernels[ti].supports(d) && s.m >= 128 && s.n >= 128) return (uint32_t)ti;

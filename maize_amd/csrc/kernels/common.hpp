@@ -20,11 +20,11 @@ struct GemmArgs {
     uint32_t reserved;
     // Extended part (all zero = the plain product: compact rows, bf16 C = A.B).
     uint32_t lda, ldb, ldc;  // elements between consecutive rows; 0 = the matrix's column count
-    uint32_t epi;            // bit 0: C is fp32; bit 1: C = alpha * A.B + beta * C
+    uint32_t epi;            // bit 0: C is fp32; bit 1: C = alpha * A.B + beta * C; bit 2: A, B (and a 16-bit C) are IEEE half
     float alpha, beta;
 };
 static_assert(sizeof(GemmArgs) == 120, "kernel parameter block layout");
-constexpr uint32_t EPI_F32 = 1u, EPI_SCALE = 2u;
+constexpr uint32_t EPI_F32 = 1u, EPI_SCALE = 2u, EPI_F16 = 4u;
 
 // Leading dimensions with their defaults: the reference's rows are compact (row stride ==
 // ncols, crates/maize_tile/src/gmem/row_panel.rs:55).
@@ -57,6 +57,15 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
 
+// IEEE half: two fp32 -> packed halves (RNE), half bits -> fp32 (exact).
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ uint32_t cvt_pk_f16(float lo, float hi) {
+    float2v f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, halfx2));
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h); }
+
 // bf16 bits -> fp32 (exact).
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }
 
@@ -72,15 +81,15 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 
 // Writes NV (4 or 8) consecutive elements of one row of C, starting at element offset `at` (a
-// multiple of NV) of the batch member's C: the plain product as packed bf16, or the general
-// epilogue (alpha/beta, fp32 output).  `c` points at the batch member (bf16 or fp32 elements).
+// multiple of NV) of the batch member's C: the plain product as packed bf16 (or half), or the
+// general epilogue (alpha/beta, fp32 output).  `c` points at the batch member (bf16 or fp32 elements).
 template <int NV>
 __device__ __forceinline__ void store_c_run(const GemmArgs& p, void* c, uint64_t at, const float (&acc)[NV]) {
     static_assert(NV == 4 || NV == 8, "a run is 4 or 8 elements");
     float x[NV];
 #pragma unroll
     for (int e = 0; e < NV; ++e) x[e] = acc[e];
-    const bool f32_out = p.epi & EPI_F32;
+    const bool f32_out = p.epi & EPI_F32, half_io = p.epi & EPI_F16;
     if ((p.epi & EPI_SCALE)) {
         float old[NV];
 #pragma unroll
@@ -96,8 +105,13 @@ __device__ __forceinline__ void store_c_run(const GemmArgs& p, void* c, uint64_t
 #pragma unroll
                 for (int e = 0; e < NV; e += 4) {
                     const u32x2 o = *(const u32x2*)((const uint16_t*)c + at + e);
-                    old[e] = bf16_bits_to_f32(o[0] & 0xFFFFu); old[e + 1] = bf16_bits_to_f32(o[0] >> 16);
-                    old[e + 2] = bf16_bits_to_f32(o[1] & 0xFFFFu); old[e + 3] = bf16_bits_to_f32(o[1] >> 16);
+                    if (half_io) {
+                        old[e] = f16_bits_to_f32(o[0] & 0xFFFFu); old[e + 1] = f16_bits_to_f32(o[0] >> 16);
+                        old[e + 2] = f16_bits_to_f32(o[1] & 0xFFFFu); old[e + 3] = f16_bits_to_f32(o[1] >> 16);
+                    } else {
+                        old[e] = bf16_bits_to_f32(o[0] & 0xFFFFu); old[e + 1] = bf16_bits_to_f32(o[0] >> 16);
+                        old[e + 2] = bf16_bits_to_f32(o[1] & 0xFFFFu); old[e + 3] = bf16_bits_to_f32(o[1] >> 16);
+                    }
                 }
             }
         }
@@ -110,7 +124,8 @@ __device__ __forceinline__ void store_c_run(const GemmArgs& p, void* c, uint64_t
     } else {
 #pragma unroll
         for (int e = 0; e < NV; e += 4)
-            *(u32x2*)((uint16_t*)c + at + e) = u32x2{cvt_pk_bf16(x[e], x[e + 1]), cvt_pk_bf16(x[e + 2], x[e + 3])};
+            *(u32x2*)((uint16_t*)c + at + e) = half_io ? u32x2{cvt_pk_f16(x[e], x[e + 1]), cvt_pk_f16(x[e + 2], x[e + 3])}
+                                                       : u32x2{cvt_pk_bf16(x[e], x[e + 1]), cvt_pk_bf16(x[e + 2], x[e + 3])};
     }
 }
 

@@ -38,7 +38,8 @@
 //     arriver re-reads all partials in range order (deterministic), then runs the normal epilogue.
 //
 // The _gen kernels are the plain (persistent) kernels with the general epilogue: C = alpha * A.B +
-// beta * C, C in bf16 or fp32.
+// beta * C, C in bf16 or fp32.  maize_gemm_f16_mt256_* are the same kernels on IEEE half operands
+// (v_mfma_f32_32x32x16_f16; a 16-bit C is then half too).
 //
 // Requirements (checked by the dispatcher): K % 8 == 0, N % 8 == 0, 16-byte
 // aligned operands, each matrix (per batch member) below 2 GiB.  The plain
@@ -102,7 +103,7 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 
 #define MAIZE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <bool NT, bool KTAIL, bool EDGE, bool GEN>
+template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     // Four separate arrays (operand x ring stage): the compiler can then tell that a
     // direct-to-LDS load into one stage does not alias fragment reads of the other, and does
@@ -299,8 +300,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
 #pragma unroll
             for (int s = 0; s < 16; ++s) {
-                acc[s >> 2][s & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_operand(buf, s & 3), fa[buf][s >> 2],
-                                                                            acc[s >> 2][s & 3], 0, 0, 0);
+                if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
+                    acc[s >> 2][s & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        __builtin_bit_cast(halfx8, b_operand(buf, s & 3)), __builtin_bit_cast(halfx8, fa[buf][s >> 2]),
+                        acc[s >> 2][s & 3], 0, 0, 0);
+                else
+                    acc[s >> 2][s & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_operand(buf, s & 3), fa[buf][s >> 2],
+                                                                                acc[s >> 2][s & 3], 0, 0, 0);
                 // Side work of this slot: fragment reads for the next quarter ...
                 if (s < NREADS) {
                     if (kk < 3) read_frag(buf ^ 1, kk + 1, s, ca, cb);
@@ -495,9 +501,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 }  // namespace mt256
 
 #define MAIZE_MT256_KERNEL(name, nt, ktail, edge) \
-    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, edge, false>(p); }
-#define MAIZE_MT256_KERNEL_GEN(name, nt, ktail) \
-    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, false, true>(p); }
+    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, edge, false, false>(p); }
+#define MAIZE_MT256_KERNEL_GEN(name, nt, ktail, f16) \
+    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, false, true, f16>(p); }
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn, false, false, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt, true, false, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail, false, true, false)
@@ -506,10 +512,14 @@ MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_edge, false, false, true)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_edge, true, false, true)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail_edge, false, true, true)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_ktail_edge, true, true, true)
-MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nn_gen, false, false)
-MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nt_gen, true, false)
-MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nn_ktail_gen, false, true)
-MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nt_ktail_gen, true, true)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nn_gen, false, false, false)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nt_gen, true, false, false)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nn_ktail_gen, false, true, false)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_bf16_mt256_nt_ktail_gen, true, true, false)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nn_gen, false, false, true)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nt_gen, true, false, true)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nn_ktail_gen, false, true, true)
+MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nt_ktail_gen, true, true, true)
 #undef MAIZE_MT256_KERNEL
 #undef MAIZE_MT256_KERNEL_GEN
 

@@ -70,6 +70,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
     const uint32_t lda = lda_of(p), ldb = ldb_of(p), ldc = ldc_of(p);
     const uint32_t ks = p.ksplit ? p.ksplit : 1u;
+    const bool half_io = p.epi & EPI_F16;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -148,7 +149,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(slot + rd[0][c2]));
             short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(slot + rd[1][c2]));
             short8v bb = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bb), af[ai], acc[c2], 0, 0, 0);
+            if (half_io)   // same bits, read as IEEE half (a wave-uniform choice)
+                acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, bb), __builtin_bit_cast(halfx8, af[ai]), acc[c2], 0, 0, 0);
+            else
+                acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bb), af[ai], acc[c2], 0, 0, 0);
         }
     };
     // One block: wait until this wave's share of block b has landed (the 18 loads of blocks

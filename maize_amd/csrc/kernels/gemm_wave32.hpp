@@ -36,7 +36,7 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
     const uint64_t bz = blockIdx.z;
     const uint16_t* __restrict__ A = p.a + bz * p.stride_a;
     const uint16_t* __restrict__ B = p.b + bz * p.stride_b;
-    const bool f32_out = p.epi & EPI_F32, scaled = p.epi & EPI_SCALE;
+    const bool f32_out = p.epi & EPI_F32, scaled = p.epi & EPI_SCALE, half_io = p.epi & EPI_F16;
     uint16_t* __restrict__ C = p.c + bz * p.stride_c * (f32_out ? 2u : 1u);   // strides count elements of C
     float* __restrict__ Cf = (float*)C;
 
@@ -60,7 +60,10 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
             fa[e] = bf16_from_bits(av);
             fb[e] = bf16_from_bits(bv);
         }
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb, fa, acc, 0, 0, 0);
+        if (half_io)   // same bits, read as IEEE half (a wave-uniform choice)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, fb), __builtin_bit_cast(halfx8, fa), acc, 0, 0, 0);
+        else
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb, fa, acc, 0, 0, 0);
     }
     // D[i][j] with i = column of C (n), j = row of C (m).
     const uint32_t cm = m0 + r;
@@ -71,8 +74,13 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
             if (cn < N) {
                 const uint64_t at = (uint64_t)cm * ldc + cn;
                 float x = acc[v];
-                if (scaled) x = epi_scale(x, p.beta == 0.0f ? 0.0f : (f32_out ? Cf[at] : bf16_bits_to_f32(C[at])), p.alpha, p.beta);
-                if (f32_out) Cf[at] = x; else C[at] = f32_to_bf16_rne(x);
+                if (scaled) {
+                    const float old = p.beta == 0.0f ? 0.0f : f32_out ? Cf[at] : half_io ? f16_bits_to_f32(C[at]) : bf16_bits_to_f32(C[at]);
+                    x = epi_scale(x, old, p.alpha, p.beta);
+                }
+                if (f32_out) Cf[at] = x;
+                else if (half_io) C[at] = __builtin_bit_cast(uint16_t, (_Float16)x);
+                else C[at] = f32_to_bf16_rne(x);
             }
         }
     }

@@ -57,13 +57,52 @@ uint32_t mzo_bf16_ulp_distance(uint16_t a, uint16_t b) {
     return (uint32_t)(d < 0 ? -d : d);
 }
 
+/* ---- IEEE half (binary16) ---------------------------------------------------- */
+
+float mzo_f16_to_f32(uint16_t h) {
+    const int sign = h >> 15, e = (h >> 10) & 0x1F, m = h & 0x3FF;
+    double v;
+    if (e == 0) v = ldexp((double)m, -24);                    /* zero and subnormals */
+    else if (e == 31) v = m ? NAN : INFINITY;
+    else v = ldexp(1.0 + (double)m / 1024.0, e - 15);
+    return (float)(sign ? -v : v);
+}
+
+/* One RNE rounding from double, by the same scaling argument as mzo_bf16_from_f64:
+ * half keeps 10 fraction bits, its smallest normal binade is 2^-14, and a rounded
+ * magnitude above 65504 (the largest finite half) is infinity. */
+uint16_t mzo_f16_from_f64(double x) {
+    const uint16_t sign = signbit(x) ? 0x8000u : 0u;
+    if (isnan(x)) return (uint16_t)(sign | 0x7E00u);
+    if (isinf(x)) return (uint16_t)(sign | 0x7C00u);
+    if (x == 0.0) return sign;
+    int e;
+    (void)frexp(x, &e);
+    int ex = e - 1;
+    if (ex < -14) ex = -14;
+    const int q = ex - 10;
+    const double r = fabs(nearbyint(ldexp(x, -q)));            /* integer number of quanta, < 2^12 */
+    if (r == 0.0) return sign;
+    const double v = ldexp(r, q);
+    if (v > 65504.0) return (uint16_t)(sign | 0x7C00u);
+    if (v < ldexp(1.0, -14)) return (uint16_t)(sign | (uint16_t)r);   /* subnormal: r quanta of 2^-24 */
+    int ev;
+    const double f = frexp(v, &ev);                            /* v = f * 2^ev, f in [0.5, 1) */
+    const int be = ev - 1 + 15;
+    const uint16_t mant = (uint16_t)((f * 2.0 - 1.0) * 1024.0);
+    return (uint16_t)(sign | (uint16_t)(be << 10) | mant);
+}
+
+static float elem_to_f32(uint16_t h, int elem) { return elem == MZO_ELEM_F16 ? mzo_f16_to_f32(h) : mzo_bf16_to_f32(h); }
+static uint16_t elem_from_f64(double x, int elem) { return elem == MZO_ELEM_F16 ? mzo_f16_from_f64(x) : mzo_bf16_from_f64(x); }
+
 /* ---- GEMM ---------------------------------------------------------------- */
 
 typedef struct {
-    const uint16_t* a;   /* M x K, this batch */
+    const float* af;     /* rows x K: the rows of A this call computes, widened to float (exact) */
     const float* bf;     /* K x N, logical B of this batch widened to float (exact) */
     uint32_t n, k;
-    const uint32_t* rows; /* NULL: identity */
+    int elem;
     uint32_t r0, r1;      /* range of output rows handled by this worker */
     uint16_t* c;          /* row r of the output is at c + r * ldc */
     uint64_t ldc;
@@ -77,31 +116,30 @@ static void* worker(void* p) {
     double* acc = (double*)malloc(sizeof(double) * n * 2);
     double* aab = acc + n;
     for (uint32_t r = j->r0; r < j->r1; ++r) {
-        const uint32_t row = j->rows ? j->rows[r] : r;
-        const uint16_t* arow = j->a + (size_t)row * k;
+        const float* arow = j->af + (size_t)r * k;
         for (uint32_t x = 0; x < n; ++x) acc[x] = 0.0;
         if (j->c_abs) {
             for (uint32_t x = 0; x < n; ++x) aab[x] = 0.0;
             for (uint32_t kk = 0; kk < k; ++kk) {
-                const double av = (double)mzo_bf16_to_f32(arow[kk]);
+                const double av = (double)arow[kk];
                 const double aa = fabs(av);
                 const float* brow = j->bf + (size_t)kk * n;
                 for (uint32_t x = 0; x < n; ++x) {
                     const double bv = (double)brow[x];
-                    acc[x] += av * bv;          /* bf16 x bf16 is exact in fp64 */
+                    acc[x] += av * bv;          /* a 16-bit float times a 16-bit float is exact in fp64 */
                     aab[x] += aa * fabs(bv);
                 }
             }
         } else {
             for (uint32_t kk = 0; kk < k; ++kk) {
-                const double av = (double)mzo_bf16_to_f32(arow[kk]);
+                const double av = (double)arow[kk];
                 const float* brow = j->bf + (size_t)kk * n;
                 for (uint32_t x = 0; x < n; ++x) acc[x] += av * (double)brow[x];
             }
         }
         if (j->c) {
             uint16_t* crow = j->c + (size_t)r * j->ldc;
-            for (uint32_t x = 0; x < n; ++x) crow[x] = mzo_bf16_from_f64(acc[x]);
+            for (uint32_t x = 0; x < n; ++x) crow[x] = elem_from_f64(acc[x], j->elem);
         }
         if (j->c_f64) memcpy(j->c_f64 + (size_t)r * n, acc, sizeof(double) * n);
         if (j->c_abs) memcpy(j->c_abs + (size_t)r * n, aab, sizeof(double) * n);
@@ -110,16 +148,27 @@ static void* worker(void* p) {
     return NULL;
 }
 
+/* Rows rows[0..nrows) (NULL: 0..nrows) of A (leading dimension k) as floats, compacted. */
+static float* widen_a(const uint16_t* a, const uint32_t* rows, uint32_t nrows, uint32_t k, int elem) {
+    float* af = (float*)malloc(sizeof(float) * (size_t)(nrows ? nrows : 1) * k);
+    if (!af) return NULL;
+    for (uint32_t r = 0; r < nrows; ++r) {
+        const uint16_t* src = a + (size_t)(rows ? rows[r] : r) * k;
+        for (uint32_t kk = 0; kk < k; ++kk) af[(size_t)r * k + kk] = elem_to_f32(src[kk], elem);
+    }
+    return af;
+}
+
 /* Logical B (K x N) of one batch as floats. */
-static float* widen_b(const uint16_t* b, uint32_t n, uint32_t k, int layout) {
+static float* widen_b(const uint16_t* b, uint32_t n, uint32_t k, int layout, int elem) {
     float* bf = (float*)malloc(sizeof(float) * (size_t)n * k);
     if (!bf) return NULL;
     if (layout == MZO_LAYOUT_NN) {
-        for (size_t i = 0; i < (size_t)n * k; ++i) bf[i] = mzo_bf16_to_f32(b[i]);
+        for (size_t i = 0; i < (size_t)n * k; ++i) bf[i] = elem_to_f32(b[i], elem);
     } else {
         for (uint32_t x = 0; x < n; ++x)
             for (uint32_t kk = 0; kk < k; ++kk)
-                bf[(size_t)kk * n + x] = mzo_bf16_to_f32(b[(size_t)x * k + kk]);
+                bf[(size_t)kk * n + x] = elem_to_f32(b[(size_t)x * k + kk], elem);
     }
     return bf;
 }
@@ -145,31 +194,73 @@ static void run_rows(job_t base, uint32_t nrows, uint32_t nthreads) {
     for (uint32_t t = 0; t < nthreads; ++t) pthread_join(th[t], NULL);
 }
 
-int mzo_ref_gemm_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c,
-                      uint32_t m, uint32_t n, uint32_t k, int layout,
-                      uint32_t batch, uint64_t stride_a, uint64_t stride_b,
-                      uint64_t stride_c, double* c_f64, double* c_abs,
-                      uint32_t nthreads) {
+int mzo_ref_gemm16(const uint16_t* a, const uint16_t* b, uint16_t* c,
+                   uint32_t m, uint32_t n, uint32_t k, int layout,
+                   uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                   uint64_t stride_c, double* c_f64, double* c_abs,
+                   uint32_t nthreads, int elem) {
     if (!a || !b || !c || batch == 0) return -1;
     if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
+    if (elem != MZO_ELEM_BF16 && elem != MZO_ELEM_F16) return -1;
     if (m == 0 || n == 0) return 0;
     for (uint32_t bi = 0; bi < batch; ++bi) {
-        float* bf = widen_b(b + bi * stride_b, n, k, layout);
-        if (!bf) return -1;
+        float* bf = widen_b(b + bi * stride_b, n, k, layout, elem);
+        float* af = widen_a(a + bi * stride_a, NULL, m, k, elem);
+        if (!bf || !af) { free(bf); free(af); return -1; }
         job_t j;
         memset(&j, 0, sizeof j);
-        j.a = a + bi * stride_a;
+        j.af = af;
         j.bf = bf;
         j.n = n;
         j.k = k;
-        j.rows = NULL;
+        j.elem = elem;
         j.c = c + bi * stride_c;
         j.ldc = n;
         j.c_f64 = c_f64 ? c_f64 + (size_t)bi * m * n : NULL;
         j.c_abs = c_abs ? c_abs + (size_t)bi * m * n : NULL;
         run_rows(j, m, nthreads);
         free(bf);
+        free(af);
     }
+    return 0;
+}
+
+int mzo_ref_gemm_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c,
+                      uint32_t m, uint32_t n, uint32_t k, int layout,
+                      uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                      uint64_t stride_c, double* c_f64, double* c_abs,
+                      uint32_t nthreads) {
+    return mzo_ref_gemm16(a, b, c, m, n, k, layout, batch, stride_a, stride_b, stride_c, c_f64, c_abs, nthreads,
+                          MZO_ELEM_BF16);
+}
+
+int mzo_ref_gemm16_rows(const uint16_t* a, const uint16_t* b, uint32_t m,
+                        uint32_t n, uint32_t k, int layout, const uint32_t* rows,
+                        uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
+                        uint32_t nthreads, int elem) {
+    if (!a || !b || !rows) return -1;
+    if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
+    if (elem != MZO_ELEM_BF16 && elem != MZO_ELEM_F16) return -1;
+    for (uint32_t r = 0; r < nsel; ++r)
+        if (rows[r] >= m) return -1;
+    if (n == 0 || nsel == 0) return 0;
+    float* bf = widen_b(b, n, k, layout, elem);
+    float* af = widen_a(a, rows, nsel, k, elem);
+    if (!bf || !af) { free(bf); free(af); return -1; }
+    job_t j;
+    memset(&j, 0, sizeof j);
+    j.af = af;
+    j.bf = bf;
+    j.n = n;
+    j.k = k;
+    j.elem = elem;
+    j.c = c;
+    j.ldc = n;
+    j.c_f64 = c_f64;
+    j.c_abs = c_abs;
+    run_rows(j, nsel, nthreads);
+    free(bf);
+    free(af);
     return 0;
 }
 
@@ -177,25 +268,5 @@ int mzo_ref_gemm_rows(const uint16_t* a, const uint16_t* b, uint32_t m,
                       uint32_t n, uint32_t k, int layout, const uint32_t* rows,
                       uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
                       uint32_t nthreads) {
-    if (!a || !b || !rows) return -1;
-    if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
-    for (uint32_t r = 0; r < nsel; ++r)
-        if (rows[r] >= m) return -1;
-    if (n == 0 || nsel == 0) return 0;
-    float* bf = widen_b(b, n, k, layout);
-    if (!bf) return -1;
-    job_t j;
-    memset(&j, 0, sizeof j);
-    j.a = a;
-    j.bf = bf;
-    j.n = n;
-    j.k = k;
-    j.rows = rows;
-    j.c = c;
-    j.ldc = n;
-    j.c_f64 = c_f64;
-    j.c_abs = c_abs;
-    run_rows(j, nsel, nthreads);
-    free(bf);
-    return 0;
+    return mzo_ref_gemm16_rows(a, b, m, n, k, layout, rows, nsel, c, c_f64, c_abs, nthreads, MZO_ELEM_BF16);
 }

@@ -42,6 +42,14 @@ uint16_t mzo_bf16_from_f64(double x);   /* one round-to-nearest-even, f64 -> bf1
 uint16_t mzo_bf16_from_f32(float x);    /* one round-to-nearest-even, f32 -> bf16 */
 float    mzo_bf16_to_f32(uint16_t h);   /* exact */
 
+/* IEEE half (binary16), the operand type of the half-precision twin of the MMA op
+ * (Sm80MmaF16F32_16x8x16, crates/maize_tile/src/mma/sm80.rs).  Pinned against numpy's float16. */
+uint16_t mzo_f16_from_f64(double x);    /* one round-to-nearest-even, f64 -> half */
+float    mzo_f16_to_f32(uint16_t h);    /* exact */
+
+/* Element type of A, B and the rounded C of the *16 entry points below. */
+enum { MZO_ELEM_BF16 = 0, MZO_ELEM_F16 = 1 };
+
 /* Ordinal map: bf16 encodings -> signed integers so that adjacent finite
  * values differ by 1 and +0/-0 both map to 0.  NaN encodings are not ordered. */
 int32_t  mzo_bf16_ord(uint16_t h);
@@ -75,6 +83,18 @@ int mzo_ref_gemm_rows(const uint16_t* a, const uint16_t* b, uint32_t m,
                       uint32_t n, uint32_t k, int layout, const uint32_t* rows,
                       uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
                       uint32_t nthreads);
+
+/* The same two functions for either 16-bit element type (MZO_ELEM_*): the arithmetic is
+ * identical -- exact products, fp64 sums in ascending k, one RNE to the element type. */
+int mzo_ref_gemm16(const uint16_t* a, const uint16_t* b, uint16_t* c,
+                   uint32_t m, uint32_t n, uint32_t k, int layout,
+                   uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                   uint64_t stride_c, double* c_f64, double* c_abs,
+                   uint32_t nthreads, int elem);
+int mzo_ref_gemm16_rows(const uint16_t* a, const uint16_t* b, uint32_t m,
+                        uint32_t n, uint32_t k, int layout, const uint32_t* rows,
+                        uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
+                        uint32_t nthreads, int elem);
 
 #ifdef __cplusplus
 }

@@ -13,6 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmaize_oracle.so")
 
 NN, NT = 0, 1
+BF16, F16 = 0, 1          # element types (MZO_ELEM_*)
 _lib = None
 
 
@@ -37,6 +38,14 @@ def lib():
         L.mzo_ref_gemm_bf16.argtypes = [vp, vp, vp, u32, u32, u32, C.c_int, u32, u64, u64, u64, vp, vp, u32]
         L.mzo_ref_gemm_rows.restype = C.c_int
         L.mzo_ref_gemm_rows.argtypes = [vp, vp, u32, u32, u32, C.c_int, vp, u32, vp, vp, vp, u32]
+        L.mzo_ref_gemm16.restype = C.c_int
+        L.mzo_ref_gemm16.argtypes = [vp, vp, vp, u32, u32, u32, C.c_int, u32, u64, u64, u64, vp, vp, u32, C.c_int]
+        L.mzo_ref_gemm16_rows.restype = C.c_int
+        L.mzo_ref_gemm16_rows.argtypes = [vp, vp, u32, u32, u32, C.c_int, vp, u32, vp, vp, vp, u32, C.c_int]
+        L.mzo_f16_from_f64.restype = C.c_uint16
+        L.mzo_f16_from_f64.argtypes = [C.c_double]
+        L.mzo_f16_to_f32.restype = C.c_float
+        L.mzo_f16_to_f32.argtypes = [C.c_uint16]
         _lib = L
     return _lib
 
@@ -50,7 +59,7 @@ def _p(a):
 
 
 def ref_gemm(a, b, m, n, k, layout=NN, batch=1, stride_a=None, stride_b=None, stride_c=None,
-             want_f64=False, want_abs=False, nthreads=None):
+             want_f64=False, want_abs=False, nthreads=None, elem=BF16):
     """C (uint16, batch*stride_c elements) and optionally the fp64 sums / |a||b| sums (batch x M x N)."""
     a = np.ascontiguousarray(a, dtype=np.uint16).ravel()
     b = np.ascontiguousarray(b, dtype=np.uint16).ravel()
@@ -61,14 +70,14 @@ def ref_gemm(a, b, m, n, k, layout=NN, batch=1, stride_a=None, stride_b=None, st
     c = np.zeros((batch - 1) * sc + m * n, dtype=np.uint16)
     f64 = np.empty((batch, m, n), dtype=np.float64) if want_f64 else None
     ab = np.empty((batch, m, n), dtype=np.float64) if want_abs else None
-    rc = lib().mzo_ref_gemm_bf16(_p(a), _p(b), _p(c), m, n, k, layout, batch, sa, sb, sc, _p(f64), _p(ab),
-                                 nthreads or default_threads())
+    rc = lib().mzo_ref_gemm16(_p(a), _p(b), _p(c), m, n, k, layout, batch, sa, sb, sc, _p(f64), _p(ab),
+                              nthreads or default_threads(), elem)
     if rc != 0:
-        raise ValueError("mzo_ref_gemm_bf16 rejected its arguments")
+        raise ValueError("mzo_ref_gemm16 rejected its arguments")
     return c, f64, ab
 
 
-def ref_gemm_rows(a, b, m, n, k, rows, layout=NN, want_abs=True, nthreads=None):
+def ref_gemm_rows(a, b, m, n, k, rows, layout=NN, want_abs=True, nthreads=None, elem=BF16):
     """Rows ``rows`` of C = A.B for one batch: (bits nsel x N, f64 nsel x N, abs nsel x N)."""
     a = np.ascontiguousarray(a, dtype=np.uint16).ravel()
     b = np.ascontiguousarray(b, dtype=np.uint16).ravel()
@@ -77,30 +86,39 @@ def ref_gemm_rows(a, b, m, n, k, rows, layout=NN, want_abs=True, nthreads=None):
     c = np.zeros((nsel, n), dtype=np.uint16)
     f64 = np.empty((nsel, n), dtype=np.float64)
     ab = np.empty((nsel, n), dtype=np.float64) if want_abs else None
-    rc = lib().mzo_ref_gemm_rows(_p(a), _p(b), m, n, k, layout, _p(rows), nsel, _p(c), _p(f64), _p(ab),
-                                 nthreads or default_threads())
+    rc = lib().mzo_ref_gemm16_rows(_p(a), _p(b), m, n, k, layout, _p(rows), nsel, _p(c), _p(f64), _p(ab),
+                                   nthreads or default_threads(), elem)
     if rc != 0:
         raise ValueError("mzo_ref_gemm_rows rejected its arguments")
     return c, f64, ab
 
 
-def bf16_bits_from_f64(x):
-    """Round an array of doubles to bf16 bit patterns with the oracle's own RNE (mzo_bf16_from_f64)."""
+def bf16_bits_from_f64(x, elem=BF16):
+    """Round an array of doubles to bf16 (or half) bit patterns with the oracle's own RNE."""
     L = lib()
+    fn = L.mzo_f16_from_f64 if elem == F16 else L.mzo_bf16_from_f64
     flat = np.asarray(x, dtype=np.float64).ravel()
-    return np.fromiter((L.mzo_bf16_from_f64(float(v)) for v in flat), dtype=np.uint16, count=flat.size).reshape(np.shape(x))
+    return np.fromiter((fn(float(v)) for v in flat), dtype=np.uint16, count=flat.size).reshape(np.shape(x))
 
 
-def bf16_bits_to_f64(bits):
-    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+def bf16_bits_to_f64(bits, elem=BF16):
+    bits = np.asarray(bits, dtype=np.uint16)
+    if elem == F16:
+        L = lib()
+        table = getattr(bf16_bits_to_f64, "_half", None)
+        if table is None:
+            table = np.array([L.mzo_f16_to_f32(h) for h in range(65536)], dtype=np.float64)
+            bf16_bits_to_f64._half = table
+        return table[bits]
+    return (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
 
 
 def ref_gemm_ex(a, b, m, n, k, layout=NN, lda=None, ldb=None, alpha=1.0, beta=0.0, c_old=None, out_f32=False,
-                nthreads=None):
+                nthreads=None, elem=BF16):
     """The extended product for one batch member, on operand views with leading dimensions:
         C = round( alpha * (A.B in fp64) + beta * C_old ),   round = RNE to bf16, or to fp32.
     ``a`` and ``b`` are flat uint16 arrays holding the views (row r of A starts at r*lda); ``c_old`` is a
-    dense M x N array (bf16 bits or float32) or None when beta == 0.  alpha and beta are taken as fp32
+    dense M x N array (16-bit patterns of type ``elem``, or float32) or None when beta == 0.  alpha and beta are taken as fp32
     values.  Returns (C dense M x N: uint16 bits or float32, exact fp64 value, error scale
     |alpha| * sum|a||b| + |beta| * |C_old|).  The product itself is mzo_ref_gemm_bf16's fp64 sum; the
     scaling is two more fp64 operations (relative error 2^-52, far below either output format)."""
@@ -113,17 +131,17 @@ def ref_gemm_ex(a, b, m, n, k, layout=NN, lda=None, ldb=None, alpha=1.0, beta=0.
     bv = np.lib.stride_tricks.as_strided(b, shape=(brows, bcols), strides=(2 * ldb, 2))
     assert a.size >= (m - 1) * lda + k and b.size >= (brows - 1) * ldb + bcols
     _, f64, ab = ref_gemm(np.ascontiguousarray(av), np.ascontiguousarray(bv), m, n, k, layout=layout, want_f64=True,
-                          want_abs=True, nthreads=nthreads)
+                          want_abs=True, nthreads=nthreads, elem=elem)
     alpha = float(np.float32(alpha))
     beta = float(np.float32(beta))
     val = alpha * f64[0]
     scale = abs(alpha) * ab[0]
     if beta != 0.0:
         old = np.asarray(c_old).reshape(m, n)
-        old64 = bf16_bits_to_f64(old) if old.dtype == np.uint16 else old.astype(np.float64)
+        old64 = bf16_bits_to_f64(old, elem) if old.dtype == np.uint16 else old.astype(np.float64)
         val = val + beta * old64
         scale = scale + abs(beta) * np.abs(old64)
-    out = val.astype(np.float32) if out_f32 else bf16_bits_from_f64(val)
+    out = val.astype(np.float32) if out_f32 else bf16_bits_from_f64(val, elem)
     return out, val, scale
 
 
@@ -147,7 +165,7 @@ def floor_coeff(k):
     return (k / 16.0 + 2.0) * 2.0 ** -24
 
 
-def compare(got_bits, ref_bits, ref_f64, ref_abs, k):
+def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16):
     """Compare device output with the oracle.
 
     An element passes if it is within 1 bf16 ULP (ordinal distance) of the
@@ -155,20 +173,24 @@ def compare(got_bits, ref_bits, ref_f64, ref_abs, k):
     the tiny result is finer than fp32 accumulation can resolve -- if its
     absolute error against the fp64 sum is at most floor_coeff(K) * sum|a||b|
     plus half a bf16 ULP of the returned value.  Both counts are reported.
+    With elem=F16 the same bar in IEEE half: 1 half ULP, half a half ULP (2^-11 relative).
     """
     got = np.asarray(got_bits, dtype=np.uint16).ravel()
     ref = np.asarray(ref_bits, dtype=np.uint16).ravel()
     f64 = np.asarray(ref_f64, dtype=np.float64).ravel()
     ab = np.asarray(ref_abs, dtype=np.float64).ravel()
     assert got.size == ref.size == f64.size == ab.size
-    ng, nr = _isnan(got), _isnan(ref)
-    ulp = np.abs(_ordinal(got) - _ordinal(ref))
+    if elem == F16:
+        ng, nr = (got & 0x7FFF) > 0x7C00, (ref & 0x7FFF) > 0x7C00
+    else:
+        ng, nr = _isnan(got), _isnan(ref)
+    ulp = np.abs(_ordinal(got) - _ordinal(ref))          # sign-magnitude ordinals: valid for bf16 and half alike
     ulp = np.where(ng & nr, 0, ulp)
     ulp = np.where(ng ^ nr, 2 ** 31, ulp)
-    gotf = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    gotf = bf16_bits_to_f64(got, elem)
     with np.errstate(invalid="ignore", over="ignore"):
         err = np.abs(gotf - f64)
-        half_ulp = np.abs(gotf) * 2.0 ** -8
+        half_ulp = np.abs(gotf) * (2.0 ** -11 if elem == F16 else 2.0 ** -8)
         floor = floor_coeff(k) * ab + half_ulp
         strict_bad = ulp > 1
         bad = strict_bad & ~(err <= floor)

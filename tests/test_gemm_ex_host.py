@@ -38,7 +38,7 @@ def test_validate_rejects(kw, code):
 
 def test_validate_rejects_reserved_and_misaligned_fp32_c():
     x = ex()
-    x.reserved[1] = 1
+    x.reserved = 1
     with pytest.raises(mz.MaizeError) as e:
         mz.validate(x)
     assert e.value.code == _ffi.MAIZE_ERR_ARG
@@ -131,3 +131,21 @@ def test_oracle_ex_views_equal_compact_copies(oracle):
         plain, f64, _ = oracle.ref_gemm(ac, bc, m, n, k, layout=layout, want_f64=True, want_abs=True)
         assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
         assert np.array_equal(got[0].ravel(), plain) and np.array_equal(got[1], f64[0])
+
+
+def test_dispatch_of_half_operands():
+    big = dict(m=4096, n=4096, k=4096)
+    assert mz.gemm_plan(ex(**big, in_type=mz.IN_F16))["kernel"] == "maize_gemm_f16_mt256_nn_gen"
+    assert mz.gemm_plan(ex(4096, 4096, 4040, layout=mz.LAYOUT_NT, in_type=mz.IN_F16, beta=1.0))["kernel"] == "maize_gemm_f16_mt256_nt_ktail_gen"
+    assert mz.gemm_plan(ex(16, 14336, 4096, in_type=mz.IN_F16))["kernel"] == "maize_gemm_bf16_skinny_nn"   # type is a launch flag there
+    assert mz.gemm_plan(ex(33, 17, 65, in_type=mz.IN_F16))["kernel"] == "maize_gemm_bf16_wave32"
+    x = ex(**big, in_type=mz.IN_F16)
+    for name in mz.kernel_names():
+        if "mt256" in name:
+            assert _supports(name, x) == (name.startswith("maize_gemm_f16_") and "_nn" in name), name
+    for name in mz.kernel_names():
+        if name.startswith("maize_gemm_f16_"):
+            assert not _supports(name, ex(**big))
+    with pytest.raises(mz.MaizeError) as e:
+        mz.validate(ex(in_type=5))
+    assert e.value.code == _ffi.MAIZE_ERR_ARG

@@ -22,27 +22,35 @@ def _say(msg):
 
 
 def run_ex(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, lda=None, ldb=None, ldc=None, alpha=1.0, beta=0.0, out_f32=False,
-           kernel=None, seed=1, c_nan=False, label=""):
+           kernel=None, seed=1, c_nan=False, label="", half=False):
     """One launch on padded views whose padding (and C's) holds canaries; checks the result against the
     oracle and that nothing outside the M x N view of C changed.  Returns the kernel the dispatcher took."""
     brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
     lda = k if lda is None else lda
     ldb = bcols if ldb is None else ldb
     ldc = n if ldc is None else ldc
-    a = mz.gen.uniform_bf16(m * lda, 100 + seed)
-    b = mz.gen.uniform_bf16(brows * ldb, 200 + seed)
+    if half:      # IEEE half operands: uniform [-1, 1) rounded to half
+        rng = np.random.default_rng(1000 + seed)
+        a = (rng.random(m * lda) * 2 - 1).astype(np.float16).view(np.uint16)
+        b = (rng.random(brows * ldb) * 2 - 1).astype(np.float16).view(np.uint16)
+    else:
+        a = mz.gen.uniform_bf16(m * lda, 100 + seed)
+        b = mz.gen.uniform_bf16(brows * ldb, 200 + seed)
     cdt = np.float32 if out_f32 else np.uint16
     if out_f32:
         c0 = (np.random.default_rng(seed).standard_normal(m * ldc) * 2).astype(np.float32)
+    elif half:
+        c0 = np.random.default_rng(seed).standard_normal(m * ldc).astype(np.float16).view(np.uint16)
     else:
         c0 = mz.gen.uniform_bf16(m * ldc, 300 + seed)
     if c_nan:
-        c0 = np.full(m * ldc, np.nan, np.float32) if out_f32 else np.full(m * ldc, 0x7FC0, np.uint16)
+        c0 = np.full(m * ldc, np.nan, np.float32) if out_f32 else np.full(m * ldc, 0x7E00 if half else 0x7FC0, np.uint16)
     da, db, dc = ctx.upload(a), ctx.upload(b), ctx.upload(c0)
     try:
         x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, brows, bcols), mz.Matrix(dc, m, n), layout=layout,
                             lda=0 if lda == k else lda, ldb=0 if ldb == bcols else ldb, ldc=0 if ldc == n else ldc,
-                            out_type=mz.OUT_F32 if out_f32 else mz.OUT_BF16, alpha=alpha, beta=beta)
+                            out_type=mz.OUT_F32 if out_f32 else mz.OUT_SAME, alpha=alpha, beta=beta,
+                            in_type=mz.IN_F16 if half else mz.IN_BF16)
         took = mz.gemm_plan(x, kernel=kernel, compute_units=ctx.info()["compute_units"])["kernel"]
         _say(f"{label} M={m} N={n} K={k} ld=({lda},{ldb},{ldc}) alpha={alpha} beta={beta} f32={out_f32} -> {took}")
         ctx.gemm_bf16(x, kernel=kernel)
@@ -55,7 +63,8 @@ def run_ex(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, lda=None, ldb=None, ldc=No
     # the padding of C's rows is untouched (bit for bit)
     assert np.array_equal(gv[:, n:].view(np.uint8), ov[:, n:].view(np.uint8)), f"{label}: wrote into C's row padding"
     ref, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, layout=layout, lda=lda, ldb=ldb, alpha=alpha, beta=beta,
-                                         c_old=None if beta == 0.0 else ov[:, :n].copy(), out_f32=out_f32)
+                                         c_old=None if beta == 0.0 else ov[:, :n].copy(), out_f32=out_f32,
+                                         elem=oracle.F16 if half else oracle.BF16)
     g = gv[:, :n]
     if out_f32:
         err = np.abs(g.astype(np.float64) - val)
@@ -63,7 +72,7 @@ def run_ex(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, lda=None, ldb=None, ldc=No
         bad = ~(err <= tol)
         assert not bad.any(), f"{label}: {int(bad.sum())} of {bad.size} fp32 elements out of tolerance, worst {float((err / tol).max()):.2f}x"
     else:
-        s = oracle.compare(g, ref, val, scale, k)
+        s = oracle.compare(g, ref, val, scale, k, elem=oracle.F16 if half else oracle.BF16)
         assert s["n_fail"] == 0, f"{label}: {s}"
     return took
 
@@ -175,3 +184,53 @@ def test_general_epilogue_with_several_tiles_per_workgroup_and_batches(ctx, orac
                                            beta=1.5, c_old=c0.reshape(batch, m, n)[i], out_f32=True)
         err = np.abs(got[i].astype(np.float64) - val)
         assert (err <= (k / 16.0 + 4.0) * 2.0 ** -24 * scale + 1e-45).all(), f"batch member {i}"
+
+
+# ---- IEEE half operands (the half-precision twin of the MMA op) ---------------------------------
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+def test_half_operands_any_shape_kernel(ctx, oracle, layout):
+    for (m, n, k) in ((33, 17, 65), (100, 200, 72)):
+        for kw in KNOBS:
+            run_ex(ctx, oracle, m, n, k, layout=layout, kernel="maize_gemm_bf16_wave32", half=True, label="wave32 half", **kw)
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape,lds", [((256, 256, 128), None), ((520, 776, 192), (200, 1000, 784)), ((300, 520, 136), (144, 528, 1024))])
+def test_half_operands_macro_tile(ctx, oracle, layout, shape, lds):
+    m, n, k = shape
+    lda, ldb, ldc = lds if lds else (None, None, None)
+    if lds and layout == mz.LAYOUT_NT:
+        ldb = max(k + 8, 200)
+    want = "maize_gemm_f16_mt256_" + ("nt" if layout == mz.LAYOUT_NT else "nn") + ("_ktail" if k % 64 else "") + "_gen"
+    for kw in KNOBS:
+        took = run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, half=True, label="mt256 half", **kw)
+        assert took == want, took
+
+
+@pytest.mark.parametrize("m", [3, 16])
+def test_half_operands_skinny(ctx, oracle, m):
+    for kw in KNOBS:
+        took = run_ex(ctx, oracle, m, 1024, 2048, half=True, label="skinny half", **kw)
+        assert took == "maize_gemm_bf16_skinny_nn", took
+
+
+def test_half_full_size_4096_cubed(ctx, oracle):
+    """The headline shape on half operands: sampled rows against the oracle."""
+    from tests.gpu_util import sample_rows
+    m = n = k = 4096
+    rng = np.random.default_rng(77)
+    a = (rng.random(m * k) * 2 - 1).astype(np.float16).view(np.uint16)
+    b = (rng.random(k * n) * 2 - 1).astype(np.float16).view(np.uint16)
+    da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(m * n * 2)
+    x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n), mz.Matrix(dc, m, n), in_type=mz.IN_F16)
+    assert mz.gemm_plan(x)["kernel"] == "maize_gemm_f16_mt256_nn_gen"
+    _say("half 4096^3 launching")
+    ctx.gemm_bf16(x)
+    ctx.sync()
+    got = dc.download(np.uint16).reshape(m, n)
+    da.free(); db.free(); dc.free()
+    rows = sample_rows(m, count=16)
+    ref, f64, ab = oracle.ref_gemm_rows(a, b, m, n, k, rows, elem=oracle.F16)
+    s = oracle.compare(got[rows], ref, f64, ab, k, elem=oracle.F16)
+    assert s["n_fail"] == 0, s

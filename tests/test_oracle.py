@@ -225,3 +225,63 @@ def test_comparator_flags_and_floors(oracle):
     # 0x3F83 is 3 ULP off a large value -> fail; 0x3003 is 3 ULP off a tiny value under the floor -> counted, not failed
     assert s["n_gt1ulp"] == 3 and s["n_fail"] == 2 and s["max_ulp"] == 2 ** 31
     assert oracle.floor_coeff(k) == (k / 16 + 2) * 2.0 ** -24
+
+
+# ---- IEEE half: the operand type of the half-precision twin of the MMA op -------------------
+
+def test_half_conversions_match_numpy_float16(oracle):
+    L = oracle.lib()
+    bits = np.arange(65536, dtype=np.uint16)
+    ours = np.array([L.mzo_f16_to_f32(int(h)) for h in bits], dtype=np.float32)
+    theirs = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(ours.view(np.uint32)[~np.isnan(theirs)], theirs.view(np.uint32)[~np.isnan(theirs)])
+    assert np.isnan(ours[np.isnan(theirs)]).all()
+    # every finite half round-trips; every midpoint between neighbours goes to the even one
+    fin = bits[np.isfinite(theirs)]
+    vals = theirs[np.isfinite(theirs)].astype(np.float64)
+    back = np.array([L.mzo_f16_from_f64(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(back[vals != 0], fin[vals != 0])
+    pos = np.arange(0, 0x7BFF, dtype=np.uint16)                    # positive finite, has a finite successor
+    lo = pos.view(np.float16).astype(np.float64)
+    hi = (pos + 1).astype(np.uint16).view(np.float16).astype(np.float64)
+    mid = np.array([L.mzo_f16_from_f64(float(v)) for v in (lo + hi) / 2], dtype=np.uint16)
+    assert np.array_equal(mid, np.where(pos & 1, pos + 1, pos))
+    # numpy's own correctly rounded double -> half on random doubles, the overflow threshold, subnormals
+    rng = np.random.default_rng(11)
+    x = np.concatenate([rng.standard_normal(20000) * 10.0 ** rng.integers(-8, 5, 20000),
+                        [65504.0, 65519.999, 65520.0, 1e6, -65520.0, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001, 5.9e-8, -0.0]])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    got = np.array([L.mzo_f16_from_f64(float(v)) for v in x], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    assert L.mzo_f16_from_f64(float("nan")) & 0x7FFF > 0x7C00
+
+
+def test_half_gemm_vs_numpy_float64_and_closed_forms(oracle):
+    rng = np.random.default_rng(12)
+    m, n, k = 19, 23, 77
+    a = rng.standard_normal((m, k)).astype(np.float16)
+    b = rng.standard_normal((k, n)).astype(np.float16)
+    for layout, bs in ((oracle.NN, b), (oracle.NT, np.ascontiguousarray(b.T))):
+        c, f64, ab = oracle.ref_gemm(a.view(np.uint16), bs.view(np.uint16), m, n, k, layout=layout, want_f64=True,
+                                     want_abs=True, elem=oracle.F16)
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        assert np.allclose(f64[0], want, rtol=0, atol=1e-12 * k)
+        assert np.array_equal(c.reshape(m, n), f64[0].astype(np.float16).view(np.uint16))
+        assert np.allclose(ab[0], np.abs(a.astype(np.float64)) @ np.abs(b.astype(np.float64)), rtol=1e-14)
+    # identity: C = B exactly; small integers: exact sums
+    eye = np.eye(16, dtype=np.float16)
+    bb = rng.standard_normal((16, 9)).astype(np.float16)
+    c, _, _ = oracle.ref_gemm(eye.view(np.uint16), bb.view(np.uint16), 16, 9, 16, elem=oracle.F16)
+    assert np.array_equal(c.reshape(16, 9), bb.view(np.uint16))
+    ai = rng.integers(-3, 4, (5, 32)).astype(np.float16)
+    bi = rng.integers(-3, 4, (32, 6)).astype(np.float16)
+    c, _, _ = oracle.ref_gemm(ai.view(np.uint16), bi.view(np.uint16), 5, 6, 32, elem=oracle.F16)
+    assert np.array_equal(c.reshape(5, 6).view(np.float16).astype(np.int64), ai.astype(np.int64) @ bi.astype(np.int64))
+    # the same bit patterns read as bf16 give a different product: the element type is honoured
+    c2, _, _ = oracle.ref_gemm(ai.view(np.uint16), bi.view(np.uint16), 5, 6, 32)
+    assert not np.array_equal(c, c2)
+    rows = np.array([4, 0, 2], np.uint32)
+    cr, fr, _ = oracle.ref_gemm_rows(a.view(np.uint16), b.view(np.uint16), m, n, k, rows, elem=oracle.F16)
+    full, _, _ = oracle.ref_gemm(a.view(np.uint16), b.view(np.uint16), m, n, k, elem=oracle.F16)
+    assert np.array_equal(cr, full.reshape(m, n)[rows])
