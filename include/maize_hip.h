@@ -187,7 +187,7 @@ typedef struct {
     uint32_t lds_bytes;     /* dynamic LDS (the kernels here use static LDS: 0) */
     uint32_t ksplit;        /* K ranges per split tile / slab; 0 or 1 = no split */
     uint32_t split_first;   /* tiled kernels: edge mode << 30 | 1 + tiles computed whole; 0 = all whole */
-    uint32_t reserved;
+    uint32_t reduce_grid;   /* split-K macro-tile kernels: grid.x of the reduce pass that follows; 0 = none */
     uint64_t workspace_bytes;
 } maize_gemm_plan_t;
 int32_t maize_hip_gemm_plan(const maize_gemm_desc_t* desc, const char* kernel, uint32_t compute_units,

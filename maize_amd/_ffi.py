@@ -80,7 +80,7 @@ class GemmPlanT(C.Structure):
     """maize_gemm_plan_t: kernel choice and launch geometry for one descriptor."""
     _fields_ = [("kernel", C.c_char * 64), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3),
                 ("lds_bytes", C.c_uint32), ("ksplit", C.c_uint32), ("split_first", C.c_uint32),
-                ("reserved", C.c_uint32), ("workspace_bytes", C.c_uint64)]
+                ("reduce_grid", C.c_uint32), ("workspace_bytes", C.c_uint64)]
 
 
 assert C.sizeof(GemmPlanT) == 112

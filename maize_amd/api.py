@@ -218,7 +218,8 @@ def gemm_plan(desc, kernel=None, compute_units=256):
     fn = _ffi.lib().maize_hip_gemm_ex_plan if isinstance(desc, _ffi.GemmExDescT) else _ffi.lib().maize_hip_gemm_plan
     check(fn(C.byref(desc), kernel.encode() if kernel else None, compute_units, C.byref(out)))
     return {"kernel": out.kernel.decode(), "grid": tuple(out.grid), "block": tuple(out.block), "lds_bytes": out.lds_bytes,
-            "ksplit": out.ksplit, "split_first": out.split_first, "workspace_bytes": out.workspace_bytes}
+            "ksplit": out.ksplit, "split_first": out.split_first, "reduce_grid": out.reduce_grid,
+            "workspace_bytes": out.workspace_bytes}
 
 
 def kernel_names():

@@ -7,6 +7,7 @@ namespace maize {
 namespace {
 
 inline uint32_t cdiv(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+inline uint64_t cdiv64(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
 
 // Leading dimensions with their defaults, and the extent (in elements) of each operand view.
 struct Lds { uint32_t a, b, c; uint64_t ext_a, ext_b, ext_c; };
@@ -35,7 +36,7 @@ bool wave32_plan(const maize_gemm_ex_desc_t& d, uint32_t, LaunchDims* ld) {
     ld->grid[2] = d.gemm.batch;
     ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
-    ld->ksplit = 0; ld->workspace_bytes = 0; ld->split_first = 0;
+    ld->ksplit = 0; ld->workspace_bytes = 0; ld->split_first = 0; ld->reduce_grid = 0;
     return ld->grid[1] <= 65535u && ld->grid[2] <= 65535u;
 }
 
@@ -130,12 +131,53 @@ bool mt256_plan_impl(const maize_gemm_ex_desc_t& d, uint32_t compute_units, bool
     ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;  // static LDS
     ld->ksplit = e.ks;
+    ld->reduce_grid = 0;
     ld->split_first = e.mode ? ((e.mode << 30) | (e.whole + 1u)) : 0u;
     ld->workspace_bytes = e.mode ? kTicketBytes + (size_t)e.nedge * e.ks * 256u * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31) && e.nedge <= 16384u;
 }
 bool mt256_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, false, ld); }
 bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
+
+// ---- maize_gemm_{bf16,f16}_mt256_{nn,nt}_splitk: few tiles, long K ---------------------------
+// K ranges per tile: as many as fill the chip once with (tile, range) work items, at least 4 K
+// steps each, at most 64, no empty range; the fp32 partial tiles (256 KiB each) stay under 1 GiB.
+uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus) {
+    const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * batch;
+    const uint32_t nk = cdiv(s.k, 64);
+    if (cus == 0 || tiles == 0 || tiles * 2 > cus || nk < 8u) return 1;
+    uint32_t ks = (uint32_t)(cus / tiles);
+    if (ks > nk / 4u) ks = nk / 4u;
+    if (ks > 64u) ks = 64u;
+    while (ks > 1u && tiles * ks * 262144ull > (1ull << 30)) --ks;
+    if (ks < 2u) return 1;
+    return cdiv(nk, cdiv(nk, ks));
+}
+bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && !half_in(d); }
+bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && !half_in(d); }
+bool splitk_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && half_in(d); }
+bool splitk_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && half_in(d); }
+bool splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * d.gemm.batch;
+    uint32_t ks = splitk_ranges(s, d.gemm.batch, compute_units);
+    // Named explicitly for a shape the dispatcher would not split: two ranges if K allows, else one.
+    if (ks < 2u) ks = cdiv(s.k, 64) >= 2u && tiles * 2ull * 262144ull <= (1ull << 30) ? 2u : 1u;
+    const uint64_t items = tiles * ks;
+    if (items > 0x1FFFFFFFull || items * 262144ull > (1ull << 32)) return false;
+    uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+    ld->grid[0] = (resident && items > resident) ? resident : (uint32_t)items;
+    ld->grid[1] = 1; ld->grid[2] = 1;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0;
+    ld->ksplit = ks;
+    ld->split_first = 0;
+    ld->workspace_bytes = kTicketBytes + (size_t)items * 262144u;
+    const uint64_t runs = (uint64_t)s.m * cdiv(s.n, 8) * d.gemm.batch;
+    if (cdiv64(runs, 256) > 0x7FFFFFFFull) return false;
+    ld->reduce_grid = (uint32_t)cdiv64(runs, 256);
+    return true;
+}
 
 // ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
 bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
@@ -165,6 +207,7 @@ bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDi
     ld->lds_bytes = 0;
     ld->ksplit = ks;
     ld->split_first = 0;
+    ld->reduce_grid = 0;
     ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * 16u * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
 }
@@ -188,6 +231,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_f16_mt256_nt_gen", f16_nt_gen_supports, mt256_plan},
     {"maize_gemm_f16_mt256_nn_ktail_gen", f16_nn_ktail_gen_supports, mt256_plan},
     {"maize_gemm_f16_mt256_nt_ktail_gen", f16_nt_ktail_gen_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_splitk", splitk_nn_supports, splitk_plan},
+    {"maize_gemm_bf16_mt256_nt_splitk", splitk_nt_supports, splitk_plan},
+    {"maize_gemm_f16_mt256_nn_splitk", splitk_f16_nn_supports, splitk_plan},
+    {"maize_gemm_f16_mt256_nt_splitk", splitk_f16_nt_supports, splitk_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -207,6 +254,11 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // Few rows against a wide row-major B: bound by streaming B once.
     const int sk = kernel_index("maize_gemm_bf16_skinny_nn");
     if (sk >= 0 && kKernels[sk].supports(d) && s.n >= 64) return (uint32_t)sk;
+    // Few tiles and a long K: cut every tile into K ranges so that the whole chip works.
+    static const char* const kSplitK[2][2] = {{"maize_gemm_bf16_mt256_nn_splitk", "maize_gemm_bf16_mt256_nt_splitk"},
+                                              {"maize_gemm_f16_mt256_nn_splitk", "maize_gemm_f16_mt256_nt_splitk"}};
+    const int si = kernel_index(kSplitK[half_in(d)][s.nt]);
+    if (si >= 0 && kKernels[si].supports(d) && splitk_ranges(s, d.gemm.batch, compute_units) >= 2u) return (uint32_t)si;
     static const char* const kTiled[2][2][2] = {   // [edge split][K tail][NT]
         {{"maize_gemm_bf16_mt256_nn", "maize_gemm_bf16_mt256_nt"},
          {"maize_gemm_bf16_mt256_nn_ktail", "maize_gemm_bf16_mt256_nt_ktail"}},
@@ -222,9 +274,10 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     const int ti = half_in(d)          ? kernel_index(kHalf[(s.k & 63u) != 0][s.nt])
                    : plain_epilogue(d) ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
                                        : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
-    // The macro-tile kernel pays for a 256 x 256 tile whatever the shape; below
-    // half a tile in either direction the per-wave kernel wastes less.
-    if (ti >= 0 && kKernels[ti].supports(d) && s.m >= 128 && s.n >= 128) return (uint32_t)ti;
+    // The macro-tile kernel pays for a 256 x 256 tile and ~8 us whatever the shape, but it moves
+    // its operands in 128-bit requests: measured, it beats the per-wave kernel 4-7x from
+    // 16 x 4096 x 4096 up and loses (8 vs 4-7 us) only on short K with few rows or columns.
+    if (ti >= 0 && kKernels[ti].supports(d) && (s.k >= 128 || (s.m >= 128 && s.n >= 128))) return (uint32_t)ti;
     return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
 }
 

@@ -13,6 +13,7 @@
 namespace maize {
 
 constexpr uint32_t kMaxKernels = 32;
+constexpr const char* kReduceKernel = "maize_gemm_splitk_reduce";
 
 struct LaunchDims {
     uint32_t grid[3];
@@ -21,6 +22,7 @@ struct LaunchDims {
     uint32_t ksplit;          // split-K kernels: number of K ranges (0 = kernel takes no workspace)
     uint32_t split_first;     // tiled kernels: edge mode << 30 | 1 + number of tiles computed whole (0 = every tile whole)
     size_t workspace_bytes;   // bytes of zero-initialised, library-owned workspace the launch needs
+    uint32_t reduce_grid;     // split-K macro-tile kernels: grid.x of the maize_gemm_splitk_reduce pass that follows (0 = none)
 };
 constexpr size_t kTicketBytes = 16384 * 4;  // ticket counters at the start of a workspace
 

@@ -3,4 +3,5 @@
 #include "gemm_wave32.hpp"
 #include "gemm_mt256.hpp"
 #include "gemm_skinny.hpp"
+#include "splitk_reduce.hpp"
 #include "probes.hpp"

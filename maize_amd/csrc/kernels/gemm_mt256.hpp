@@ -41,6 +41,10 @@
 // beta * C, C in bf16 or fp32.  maize_gemm_f16_mt256_* are the same kernels on IEEE half operands
 // (v_mfma_f32_32x32x16_f16; a 16-bit C is then half too).
 //
+// The _splitk kernels serve shapes with few tiles and a long K: every tile is cut into `ksplit` K
+// ranges, each (tile, range) is a work item that leaves an fp32 partial tile in the workspace, and
+// maize_gemm_splitk_reduce (splitk_reduce.hpp) adds the ranges in order and applies the epilogue.
+//
 // Requirements (checked by the dispatcher): K % 8 == 0, N % 8 == 0, 16-byte
 // aligned operands, each matrix (per batch member) below 2 GiB.  The plain
 // kernels need K % 64 == 0 (the K advance is then a scalar offset and no lane
@@ -103,7 +107,7 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 
 #define MAIZE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16>
+template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     // Four separate arrays (operand x ring stage): the compiler can then tell that a
     // direct-to-LDS load into one stage does not alias fragment reads of the other, and does
@@ -135,13 +139,19 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t ks = split ? p.ksplit : 1u;
     const uint32_t edge = split ? (blockIdx.x - whole) / ks : 0u;     // which edge tile
     const uint32_t z = split ? (blockIdx.x - whole) % ks : 0u;        // which K range
-    // K steps of this workgroup: [kt0, kt0 + nk) of the ceil(K / BK) steps.
+    // K steps of this workgroup: [kt0, kt0 + nk) of the ceil(K / BK) steps.  The split-K kernels
+    // (SPLITK) give every work item its own range instead (select_tile).
     const uint32_t nk_all = (K + BK - 1) / BK;
-    const uint32_t per_range = (nk_all + ks - 1u) / ks;
-    const uint32_t kt0 = z * per_range;
-    const uint32_t nk = kt0 < nk_all ? (nk_all - kt0 < per_range ? nk_all - kt0 : per_range) : 0u;
-    const uint32_t k_begin = kt0 * BK;
-    const uint32_t k_end = (kt0 + nk) * BK < K ? (kt0 + nk) * BK : K;   // loads at or past k_end return zeros
+    const uint32_t nranges = SPLITK ? (p.ksplit ? p.ksplit : 1u) : ks;
+    const uint32_t per_range = (nk_all + nranges - 1u) / nranges;
+    uint32_t nk, k_begin, k_end;                                      // k_end: loads at or past it return zeros
+    auto select_range = [&](uint32_t zr) {
+        const uint32_t kt0 = zr * per_range;
+        nk = kt0 < nk_all ? (nk_all - kt0 < per_range ? nk_all - kt0 : per_range) : 0u;
+        k_begin = kt0 * BK;
+        k_end = (kt0 + nk) * BK < K ? (kt0 + nk) * BK : K;
+    };
+    select_range(z);
     // Extent of each operand view: the last row ends at (rows - 1) * ld + cols.
     const uint32_t a_bytes = ((M - 1u) * lda + K) * 2u;
     const uint32_t b_bytes = (NT ? (N - 1u) * ldb + K : (K - 1u) * ldb + N) * 2u;
@@ -151,7 +161,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // list of all tiles of all batch members.  The edge-splitting kernels compute one tile (or
     // one K range of one) per workgroup.
     const uint32_t tiles_per = tm * tn;
-    const uint32_t total = EDGE ? gridDim.x : tiles_per * p.batch;
+    // Split-K kernels: the work items are (tile, K range) pairs, ranges of one tile adjacent.
+    const uint32_t total = EDGE ? gridDim.x : tiles_per * p.batch * (SPLITK ? nranges : 1u);
     uint32_t pid = blockIdx.x;
     if (pid >= total) return;
 
@@ -172,6 +183,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     uint16_t* Cg;
     uint32_t a_vo[8], b_vo[8];
     uint32_t a_k[2];                      // k index of the lane's chunk inside a tile, even/odd piece (K masks)
+    uint32_t part_slot = 0;               // split-K: index of this item's fp32 partial tile in the workspace
     auto select_tile = [&](uint32_t id) {
         uint32_t tile_m, tile_n;
         uint64_t bz;
@@ -183,6 +195,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 tile_m = mode == 1u ? edge : tm - 1u;
                 tile_n = mode == 1u ? tn - 1u : edge;
             }
+        } else if (SPLITK) {
+            const uint32_t item = xcd_run(id, total);
+            const uint32_t t = item / nranges;                         // tile of the flattened (batch, tile) list
+            select_range(item - t * nranges);
+            bz = t / tiles_per;
+            tile_of(t - (uint32_t)bz * tiles_per, tm, tn, &tile_m, &tile_n);
+            part_slot = (((uint32_t)bz * tiles_per + tile_m * tn + tile_n) * nranges) + (item - t * nranges);
         } else {
             const uint32_t t = xcd_run(id, total);
             bz = t / tiles_per;
@@ -413,7 +432,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
     // ---- hand-over: request the next C tile's first K tile before this one is stored -------
     __syncthreads();                                           // all waves are done with the operand stages
-    const uint32_t em0 = m0, en0 = n0;
+    const uint32_t em0 = m0, en0 = n0, eslot = part_slot;
     uint16_t* const Ce = Cg;
     const uint32_t next = pid + gridDim.x;
     const bool more = !EDGE && next < total;
@@ -457,8 +476,18 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8 + 1u) ^ (row & 15u)) * 16u));
                     const uint32_t grow = em0 + wm * 128u + i * 32u + row;
                     if (gcol < N && grow < M) {                   // N % 8 == 0: a run is all in or all out
-                        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        store_c_run<8>(p, Ce, (uint64_t)grow * ldc + gcol, v);
+                        if (SPLITK) {
+                            // fp32 partial tile of this (tile, K range), row-major 256 x 256, behind the 64 KiB
+                            // of ticket counters every workspace starts with (other kernels on the stream rely
+                            // on finding them zero); the reduce kernel adds the ranges in order and applies
+                            // the epilogue.
+                            float* part = (float*)((char*)p.workspace + 65536) + (uint64_t)eslot * (BM * BN) + (grow - em0) * BN + (gcol - en0);
+                            *(floatx4*)part = lo;
+                            *(floatx4*)(part + 4) = hi;
+                        } else {
+                            const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                            store_c_run<8>(p, Ce, (uint64_t)grow * ldc + gcol, v);
+                        }
                     }
                 }
             }
@@ -501,9 +530,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 }  // namespace mt256
 
 #define MAIZE_MT256_KERNEL(name, nt, ktail, edge) \
-    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, edge, false, false>(p); }
+    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, edge, false, false, false>(p); }
 #define MAIZE_MT256_KERNEL_GEN(name, nt, ktail, f16) \
-    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, false, true, f16>(p); }
+    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, false, true, f16, false>(p); }
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn, false, false, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt, true, false, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail, false, true, false)
@@ -520,7 +549,15 @@ MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nn_gen, false, false, true)
 MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nt_gen, true, false, true)
 MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nn_ktail_gen, false, true, true)
 MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nt_ktail_gen, true, true, true)
+// Split-K: (tile, K range) work items, fp32 partial tiles to the workspace; any K % 8 == 0.
+#define MAIZE_MT256_KERNEL_SPLITK(name, nt, f16) \
+    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, true, false, true, f16, true>(p); }
+MAIZE_MT256_KERNEL_SPLITK(maize_gemm_bf16_mt256_nn_splitk, false, false)
+MAIZE_MT256_KERNEL_SPLITK(maize_gemm_bf16_mt256_nt_splitk, true, false)
+MAIZE_MT256_KERNEL_SPLITK(maize_gemm_f16_mt256_nn_splitk, false, true)
+MAIZE_MT256_KERNEL_SPLITK(maize_gemm_f16_mt256_nt_splitk, true, true)
 #undef MAIZE_MT256_KERNEL
 #undef MAIZE_MT256_KERNEL_GEN
+#undef MAIZE_MT256_KERNEL_SPLITK
 
 }  // namespace maize

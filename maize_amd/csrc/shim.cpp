@@ -61,6 +61,7 @@ struct maize_ctx {
     hipDeviceProp_t prop;
     hipModule_t module;
     hipFunction_t fn[maize::kMaxKernels];
+    hipFunction_t reduce_fn;
     // Split-K scratch, one per stream so that launches on different streams never share it.
     std::unordered_map<void*, maize_workspace> workspaces;
 };
@@ -124,6 +125,13 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
             delete ctx;
             return rc;
         }
+    }
+    e = hipModuleGetFunction(&ctx->reduce_fn, ctx->module, maize::kReduceKernel);
+    if (e != hipSuccess) {
+        int32_t rc = hip_fail(e, maize::kReduceKernel);
+        (void)hipModuleUnload(ctx->module);
+        delete ctx;
+        return rc;
     }
     *out = ctx;
     return MAIZE_OK;
@@ -323,6 +331,7 @@ int32_t maize_hip_gemm_ex_plan(const maize_gemm_ex_desc_t* desc, const char* ker
     out->lds_bytes = ld.lds_bytes;
     out->ksplit = ld.ksplit;
     out->split_first = ld.split_first;
+    out->reduce_grid = ld.reduce_grid;
     out->workspace_bytes = ld.workspace_bytes;
     return MAIZE_OK;
 }
@@ -392,8 +401,13 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
         int32_t rc = workspace_for(ctx, stream, ld.workspace_bytes, &args.workspace);
         if (rc != MAIZE_OK) return rc;
     }
-    return launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->fn[idx], ld.grid, ld.block,
-                      ld.lds_bytes, stream, &args, sizeof args);
+    int32_t rc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->fn[idx], ld.grid, ld.block,
+                            ld.lds_bytes, stream, &args, sizeof args);
+    if (rc != MAIZE_OK || ld.reduce_grid == 0) return rc;
+    // Split-K macro-tile kernels: the partial tiles are combined by a second pass on the same stream.
+    const uint32_t rgrid[3] = {ld.reduce_grid, 1, 1}, rblock[3] = {256, 1, 1};
+    return launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->reduce_fn, rgrid, rblock, 0, stream, &args,
+                      sizeof args);
 }
 
 int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const char* kernel, void* stream) {

@@ -86,7 +86,7 @@ pub struct MaizeGemmPlan {
     pub lds_bytes: u32,
     pub ksplit: u32,
     pub split_first: u32,
-    pub reserved: u32,
+    pub reduce_grid: u32,
     pub workspace_bytes: u64,
 }
 

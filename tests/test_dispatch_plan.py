@@ -59,7 +59,8 @@ def test_every_kernel_that_accepts_a_descriptor_plans_a_covering_grid(m, n, k, l
 
 def check_plan(p, m, n, k, layout, batch, cus=CUS):
     gx, gy, gz = p["grid"]
-    persistent = p["kernel"].startswith("maize_gemm_bf16_mt256") and not p["kernel"].endswith("_edge")
+    splitk = p["kernel"].endswith("_splitk")
+    persistent = "_mt256_" in p["kernel"] and not p["kernel"].endswith("_edge")
     assert gx >= 1 and gy >= 1 and gz == (1 if persistent else batch)
     assert gy <= 65535 and gz <= 65535 and gx < (1 << 31)
     name = p["kernel"]
@@ -67,7 +68,19 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         assert p["block"] == (256, 1, 1)
         assert gx == cdiv(n, 64) and gy == cdiv(m, 64)
         assert p["workspace_bytes"] == 0 and p["ksplit"] == 0
-    elif name.startswith("maize_gemm_bf16_mt256"):
+    elif splitk:
+        # (tile, K range) work items, one fp32 partial tile each, then the reduce pass over runs of 8 columns
+        assert p["block"] == (256, 1, 1) and gy == 1 and k % 8 == 0 and n % 8 == 0
+        ks = p["ksplit"]
+        items = cdiv(m, 256) * cdiv(n, 256) * batch * ks
+        resident = cus - cus % 8 if cus >= 8 else cus
+        assert 1 <= ks <= 64 and gx == min(items, resident)
+        nk = cdiv(k, 64)
+        assert cdiv(nk, ks) * (ks - 1) < nk                    # no empty range
+        assert p["workspace_bytes"] == TICKET_BYTES + items * 256 * 256 * 4 and p["workspace_bytes"] <= (1 << 32) + TICKET_BYTES
+        assert p["reduce_grid"] == cdiv(m * cdiv(n, 8) * batch, 256)
+    elif "_mt256_" in name:
+        assert p["reduce_grid"] == 0
         assert p["block"] == (256, 1, 1) and gy == 1
         assert ("_nt" in name) == (layout == mz.LAYOUT_NT)
         assert k % 8 == 0 and n % 8 == 0
@@ -123,10 +136,23 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (8192, 8192, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt",
         (16, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
+        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",      # 64 tiles: 4 K ranges each
+        (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
+        (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",        # no skinny kernel for N x K weights
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
     }
     for (m, n, k, layout, batch), want in picks.items():
         assert mz.gemm_plan(desc(m, n, k, layout, batch), compute_units=CUS)["kernel"] == want
+
+
+def test_split_k_of_few_tiles_fills_the_chip_once():
+    p = mz.gemm_plan(desc(64, 4096, 4096), compute_units=CUS)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 16 and p["grid"] == (256, 1, 1)
+    p = mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)
+    assert p["ksplit"] == 4 and p["grid"] == (256, 1, 1)
+    # more than half a chip of tiles, or a short K: no split
+    assert mz.gemm_plan(desc(4096, 2304, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
+    assert mz.gemm_plan(desc(512, 512, 448), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
 
 
 def test_skinny_split_fills_the_chip_without_overshooting():

@@ -234,3 +234,38 @@ def test_half_full_size_4096_cubed(ctx, oracle):
     ref, f64, ab = oracle.ref_gemm_rows(a, b, m, n, k, rows, elem=oracle.F16)
     s = oracle.compare(got[rows], ref, f64, ab, k, elem=oracle.F16)
     assert s["n_fail"] == 0, s
+
+
+# ---- split-K macro-tile kernels: few tiles, long K ------------------------------------------------
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape", [(64, 4096, 4096), (16, 1024, 8192), (300, 520, 1032), (256, 256, 2048), (130, 264, 4104)])
+def test_split_k_kernels(ctx, oracle, layout, shape):
+    m, n, k = shape
+    want = "maize_gemm_bf16_mt256_" + ("nt" if layout == mz.LAYOUT_NT else "nn") + "_splitk"
+    took = run_ex(ctx, oracle, m, n, k, layout=layout, label="splitk")
+    if not (layout == mz.LAYOUT_NN and m <= 16 and k % 32 == 0):       # those go to the skinny kernel
+        assert took == want, took
+    for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(half=True),
+               dict(lda=k + 8, ldc=n + 16)):
+        run_ex(ctx, oracle, m, n, k, layout=layout, kernel=("maize_gemm_f16_mt256_" + want[22:]) if kw.get("half") else want,
+               label="splitk knobs", **kw)
+
+
+def test_split_k_batched_and_more_items_than_workgroups(ctx, oracle):
+    """Batch members are separate tiles of the item list; and with more (tile, range) items than resident
+    workgroups each workgroup walks several (the persistent loop with a K range per item)."""
+    from tests.gpu_util import run_gemm, check_against_oracle
+    for (m, n, k, batch) in ((128, 256, 2048, 5), (2560, 3840, 256, 1)):
+        a = mz.gen.uniform_bf16(batch * m * k, 31)
+        b = mz.gen.uniform_bf16(batch * k * n, 32)
+        _say(f"splitk batched/multi-item {m}x{n}x{k} batch {batch}")
+        got = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel="maize_gemm_bf16_mt256_nn_splitk")
+        if m * n * k * batch <= 1 << 31:
+            check_against_oracle(oracle, got, a, b, m, n, k, batch=batch, label="splitk batched")
+        else:
+            from tests.gpu_util import sample_rows, check_rows_against_oracle
+            check_rows_against_oracle(oracle, got, a, b, m, n, k, sample_rows(m, count=24), label="splitk multi-item")
+        # bit-identical to itself on a second run (fixed summation order)
+        again = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel="maize_gemm_bf16_mt256_nn_splitk")
+        assert np.array_equal(got, again)
