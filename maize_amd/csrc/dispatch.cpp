@@ -140,18 +140,32 @@ bool mt256_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { r
 bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
 
 // ---- maize_gemm_{bf16,f16}_mt256_{nn,nt}_splitk: few tiles, long K ---------------------------
-// K ranges per tile: as many as fill the chip once with (tile, range) work items, at least 4 K
-// steps each, at most 64, no empty range; the fp32 partial tiles (256 KiB each) stay under 1 GiB.
+// K ranges per tile.  Candidates: up to one (tile, range) work item per compute unit, at least 4 K
+// steps per range, at most 64 ranges, no empty range, partial tiles (256 KiB slots) under 1 GiB.
+// The choice minimises a cost model fitted to measurements on this part (microseconds):
+//   unsplit:  8 + 1.0 * steps                       (few workgroups: each runs at full clock)
+//   split:    8 + 1.2 * steps / ks + 6 + 2e-6 * M * N * batch * ks
+// i.e. a second launch and the fp32 partial tiles written and read back at ~4 TB/s; the split is
+// taken only if it wins by 20 %.  (2048^3, 64 tiles: 38 us unsplit, 40 us split 4 ways -- not
+// split; 64 x 4096 x 4096: 63 -> 25 us; 256 x 256 x 16384: 237 -> 38 us.)
 uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus) {
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * batch;
     const uint32_t nk = cdiv(s.k, 64);
     if (cus == 0 || tiles == 0 || tiles * 2 > cus || nk < 8u) return 1;
-    uint32_t ks = (uint32_t)(cus / tiles);
-    if (ks > nk / 4u) ks = nk / 4u;
-    if (ks > 64u) ks = 64u;
-    while (ks > 1u && tiles * ks * 262144ull > (1ull << 30)) --ks;
-    if (ks < 2u) return 1;
-    return cdiv(nk, cdiv(nk, ks));
+    uint32_t kmax = (uint32_t)(cus / tiles);
+    if (kmax > nk / 4u) kmax = nk / 4u;
+    if (kmax > 64u) kmax = 64u;
+    const double unsplit = 8.0 + 1.0 * nk;
+    const double elems = (double)s.m * s.n * batch;
+    double best = unsplit * 0.8;
+    uint32_t best_ks = 1;
+    for (uint32_t ks = 2; ks <= kmax; ++ks) {
+        if (cdiv(nk, cdiv(nk, ks)) != ks) continue;            // would leave an empty range
+        if (tiles * ks * 262144ull > (1ull << 30)) break;
+        const double t = 8.0 + 1.2 * cdiv(nk, ks) + 6.0 + 2e-6 * elems * ks;
+        if (t < best) { best = t; best_ks = ks; }
+    }
+    return best_ks;
 }
 bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && !half_in(d); }
 bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && !half_in(d); }

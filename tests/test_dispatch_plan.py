@@ -136,7 +136,8 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (8192, 8192, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt",
         (16, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
-        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",      # 64 tiles: 4 K ranges each
+        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn",             # 64 tiles: partial tiles would cost more than they save
+        (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",
         (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",        # no skinny kernel for N x K weights
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
@@ -147,9 +148,11 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
 
 def test_split_k_of_few_tiles_fills_the_chip_once():
     p = mz.gemm_plan(desc(64, 4096, 4096), compute_units=CUS)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 16 and p["grid"] == (256, 1, 1)
-    p = mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)
-    assert p["ksplit"] == 4 and p["grid"] == (256, 1, 1)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and 8 <= p["ksplit"] <= 16 and p["grid"] == (16 * p["ksplit"], 1, 1)
+    p = mz.gemm_plan(desc(256, 256, 16384), compute_units=CUS)
+    assert 32 <= p["ksplit"] <= 64 and p["grid"] == (p["ksplit"], 1, 1)
+    p = mz.gemm_plan(desc(1024, 1024, 8192), compute_units=CUS)
+    assert 2 <= p["ksplit"] <= 16 and p["grid"][0] == 16 * p["ksplit"]
     # more than half a chip of tiles, or a short K: no split
     assert mz.gemm_plan(desc(4096, 2304, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
     assert mz.gemm_plan(desc(512, 512, 448), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
