@@ -193,6 +193,82 @@ bool splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDi
     return true;
 }
 
+// ---- maize_gemm_{bf16,f16}_mt256_{nn,nt}_packed: any alignment, any N and K ---------------------
+// The split-K kernels on zero-padded, 16-byte-aligned copies of whichever operands need one
+// (pack.hpp), with the reduce pass writing C element by element where its rows are not aligned.
+inline uint32_t up8(uint32_t x) { return (x + 7u) & ~7u; }
+struct Packing { bool a, b; uint32_t n8, k8; uint64_t a_elems, b_elems; };   // per batch member
+Packing packing_of(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    Packing p;
+    p.n8 = up8(s.n); p.k8 = up8(s.k);
+    const bool strides_ok = d.gemm.batch == 1 || ((d.gemm.stride_a | d.gemm.stride_b) & 7u) == 0;
+    const bool k_odd = (s.k & 7u) != 0, n_odd = (s.n & 7u) != 0;
+    p.a = k_odd || (l.a & 7u) || ((uintptr_t)d.gemm.a.ptr & 15u) || !strides_ok;
+    p.b = k_odd || n_odd || (l.b & 7u) || ((uintptr_t)d.gemm.b.ptr & 15u) || !strides_ok;
+    p.a_elems = (uint64_t)s.m * p.k8;
+    p.b_elems = s.nt ? (uint64_t)p.n8 * p.k8 : (uint64_t)p.k8 * p.n8;
+    return p;
+}
+// The product as the macro-tile kernel sees it after packing: padded extents, compact copies.
+maize_gemm_ex_desc_t packed_view(const maize_gemm_ex_desc_t& d, const Packing& p) {
+    maize_gemm_ex_desc_t v = d;
+    const Dims s = dims_of(d);
+    v.gemm.a.ncols = p.k8;
+    if (s.nt) { v.gemm.b.nrows = p.n8; v.gemm.b.ncols = p.k8; } else { v.gemm.b.nrows = p.k8; v.gemm.b.ncols = p.n8; }
+    v.gemm.c.ncols = p.n8;
+    if (p.a) { v.gemm.a.ptr = (void*)16; v.lda = 0; v.gemm.stride_a = p.a_elems; }
+    if (p.b) { v.gemm.b.ptr = (void*)16; v.ldb = 0; v.gemm.stride_b = p.b_elems; }
+    v.gemm.c.ptr = (void*)16; v.ldc = 0; v.gemm.stride_c = (uint64_t)s.m * p.n8;   // C is not touched by the first pass
+    return v;
+}
+bool packed_ok(const maize_gemm_ex_desc_t& d) {
+    const Packing p = packing_of(d);
+    const maize_gemm_ex_desc_t v = packed_view(d, p);
+    if (!mt256_common(v)) return false;                      // extents of what stays unpacked, 2 GiB limits
+    const uint64_t copies = ((p.a ? p.a_elems : 0) + (p.b ? p.b_elems : 0)) * d.gemm.batch * 2;
+    return copies <= (1ull << 31);
+}
+bool packed_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && !half_in(d) && packed_ok(d); }
+bool packed_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && !half_in(d) && packed_ok(d); }
+bool packed_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && half_in(d) && packed_ok(d); }
+bool packed_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && half_in(d) && packed_ok(d); }
+bool packed_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    const Packing p = packing_of(d);
+    const maize_gemm_ex_desc_t v = packed_view(d, p);
+    const Dims sv = dims_of(v);
+    const uint64_t tiles = (uint64_t)cdiv(sv.m, 256) * cdiv(sv.n, 256) * d.gemm.batch;
+    const uint32_t ks = splitk_ranges(sv, d.gemm.batch, compute_units);      // may be 1: the reduce pass still runs
+    const uint64_t items = tiles * ks;
+    if (items > 0x1FFFFFFFull || items * 262144ull > (1ull << 32)) return false;
+    uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+    ld->grid[0] = (resident && items > resident) ? resident : (uint32_t)items;
+    ld->grid[1] = 1; ld->grid[2] = 1;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0;
+    ld->ksplit = ks;
+    ld->split_first = 0;
+    size_t bytes = kTicketBytes + (size_t)items * 262144u;
+    ld->n_padded = p.n8; ld->k_padded = p.k8;
+    if (p.a) {
+        ld->pack_a = PackPlan{true, s.m, s.k, l.a, s.m, p.k8, bytes};
+        bytes += (size_t)p.a_elems * d.gemm.batch * 2;
+    }
+    if (p.b) {
+        const uint32_t brows = d.gemm.b.nrows, bcols = d.gemm.b.ncols;
+        ld->pack_b = PackPlan{true, brows, bcols, l.b, s.nt ? p.n8 : p.k8, s.nt ? p.k8 : p.n8, bytes};
+        bytes += (size_t)p.b_elems * d.gemm.batch * 2;
+    }
+    ld->workspace_bytes = bytes;
+    const uint64_t runs = (uint64_t)s.m * cdiv(s.n, 8) * d.gemm.batch;
+    if (cdiv64(runs, 256) > 0x7FFFFFFFull) return false;
+    ld->reduce_grid = (uint32_t)cdiv64(runs, 256);
+    return true;
+}
+
 // ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
 bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
@@ -227,28 +303,32 @@ bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDi
 }
 
 const KernelInfo kKernels[] = {
-    {"maize_gemm_bf16_wave32", wave32_supports, wave32_plan},
-    {"maize_gemm_bf16_mt256_nn", mt256_nn_supports, mt256_plan},
-    {"maize_gemm_bf16_mt256_nt", mt256_nt_supports, mt256_plan},
-    {"maize_gemm_bf16_mt256_nn_ktail", mt256_nn_ktail_supports, mt256_plan},
-    {"maize_gemm_bf16_mt256_nt_ktail", mt256_nt_ktail_supports, mt256_plan},
-    {"maize_gemm_bf16_mt256_nn_edge", mt256_nn_supports, mt256_edge_plan},
-    {"maize_gemm_bf16_mt256_nt_edge", mt256_nt_supports, mt256_edge_plan},
-    {"maize_gemm_bf16_mt256_nn_ktail_edge", mt256_nn_ktail_supports, mt256_edge_plan},
-    {"maize_gemm_bf16_mt256_nt_ktail_edge", mt256_nt_ktail_supports, mt256_edge_plan},
-    {"maize_gemm_bf16_skinny_nn", skinny_nn_supports, skinny_plan},
-    {"maize_gemm_bf16_mt256_nn_gen", mt256_nn_gen_supports, mt256_plan},
-    {"maize_gemm_bf16_mt256_nt_gen", mt256_nt_gen_supports, mt256_plan},
-    {"maize_gemm_bf16_mt256_nn_ktail_gen", mt256_nn_ktail_gen_supports, mt256_plan},
-    {"maize_gemm_bf16_mt256_nt_ktail_gen", mt256_nt_ktail_gen_supports, mt256_plan},
-    {"maize_gemm_f16_mt256_nn_gen", f16_nn_gen_supports, mt256_plan},
-    {"maize_gemm_f16_mt256_nt_gen", f16_nt_gen_supports, mt256_plan},
-    {"maize_gemm_f16_mt256_nn_ktail_gen", f16_nn_ktail_gen_supports, mt256_plan},
-    {"maize_gemm_f16_mt256_nt_ktail_gen", f16_nt_ktail_gen_supports, mt256_plan},
-    {"maize_gemm_bf16_mt256_nn_splitk", splitk_nn_supports, splitk_plan},
-    {"maize_gemm_bf16_mt256_nt_splitk", splitk_nt_supports, splitk_plan},
-    {"maize_gemm_f16_mt256_nn_splitk", splitk_f16_nn_supports, splitk_plan},
-    {"maize_gemm_f16_mt256_nt_splitk", splitk_f16_nt_supports, splitk_plan},
+    {"maize_gemm_bf16_wave32", nullptr, wave32_supports, wave32_plan},
+    {"maize_gemm_bf16_mt256_nn", nullptr, mt256_nn_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nt", nullptr, mt256_nt_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_ktail", nullptr, mt256_nn_ktail_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nt_ktail", nullptr, mt256_nt_ktail_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_edge", nullptr, mt256_nn_supports, mt256_edge_plan},
+    {"maize_gemm_bf16_mt256_nt_edge", nullptr, mt256_nt_supports, mt256_edge_plan},
+    {"maize_gemm_bf16_mt256_nn_ktail_edge", nullptr, mt256_nn_ktail_supports, mt256_edge_plan},
+    {"maize_gemm_bf16_mt256_nt_ktail_edge", nullptr, mt256_nt_ktail_supports, mt256_edge_plan},
+    {"maize_gemm_bf16_skinny_nn", nullptr, skinny_nn_supports, skinny_plan},
+    {"maize_gemm_bf16_mt256_nn_gen", nullptr, mt256_nn_gen_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nt_gen", nullptr, mt256_nt_gen_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_ktail_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nt_ktail_gen", nullptr, mt256_nt_ktail_gen_supports, mt256_plan},
+    {"maize_gemm_f16_mt256_nn_gen", nullptr, f16_nn_gen_supports, mt256_plan},
+    {"maize_gemm_f16_mt256_nt_gen", nullptr, f16_nt_gen_supports, mt256_plan},
+    {"maize_gemm_f16_mt256_nn_ktail_gen", nullptr, f16_nn_ktail_gen_supports, mt256_plan},
+    {"maize_gemm_f16_mt256_nt_ktail_gen", nullptr, f16_nt_ktail_gen_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_splitk", nullptr, splitk_nn_supports, splitk_plan},
+    {"maize_gemm_bf16_mt256_nt_splitk", nullptr, splitk_nt_supports, splitk_plan},
+    {"maize_gemm_f16_mt256_nn_splitk", nullptr, splitk_f16_nn_supports, splitk_plan},
+    {"maize_gemm_f16_mt256_nt_splitk", nullptr, splitk_f16_nt_supports, splitk_plan},
+    {"maize_gemm_bf16_mt256_nn_packed", "maize_gemm_bf16_mt256_nn_splitk", packed_nn_supports, packed_plan},
+    {"maize_gemm_bf16_mt256_nt_packed", "maize_gemm_bf16_mt256_nt_splitk", packed_nt_supports, packed_plan},
+    {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nn_splitk", packed_f16_nn_supports, packed_plan},
+    {"maize_gemm_f16_mt256_nt_packed", "maize_gemm_f16_mt256_nt_splitk", packed_f16_nt_supports, packed_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -292,6 +372,14 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // its operands in 128-bit requests: measured, it beats the per-wave kernel 4-7x from
     // 16 x 4096 x 4096 up and loses (8 vs 4-7 us) only on short K with few rows or columns.
     if (ti >= 0 && kKernels[ti].supports(d) && (s.k >= 128 || (s.m >= 128 && s.n >= 128))) return (uint32_t)ti;
+    // Odd extents or unaligned operands: the per-wave kernel reaches ~30 TFLOP/s, the macro-tile
+    // kernel on repacked operands ~1000, at the price of a few extra launches and copies (~50 us).
+    static const char* const kPacked[2][2] = {{"maize_gemm_bf16_mt256_nn_packed", "maize_gemm_bf16_mt256_nt_packed"},
+                                              {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nt_packed"}};
+    const int pi = kernel_index(kPacked[half_in(d)][s.nt]);
+    if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 1e9 &&
+        kKernels[pi].supports(d))
+        return (uint32_t)pi;
     return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
 }
 

@@ -14,6 +14,15 @@ namespace maize {
 
 constexpr uint32_t kMaxKernels = 32;
 constexpr const char* kReduceKernel = "maize_gemm_splitk_reduce";
+constexpr const char* kPackKernel = "maize_pack_2d";
+
+// Repacking of one operand into the workspace before the launch (pack.hpp).
+struct PackPlan {
+    bool on;
+    uint32_t rows, cols, ld_src;        // the operand as the caller gave it
+    uint32_t rows_dst, cols_dst;        // the zero-padded compact copy
+    size_t offset;                      // byte offset of the copy in the workspace
+};
 
 struct LaunchDims {
     uint32_t grid[3];
@@ -23,11 +32,14 @@ struct LaunchDims {
     uint32_t split_first;     // tiled kernels: edge mode << 30 | 1 + number of tiles computed whole (0 = every tile whole)
     size_t workspace_bytes;   // bytes of zero-initialised, library-owned workspace the launch needs
     uint32_t reduce_grid;     // split-K macro-tile kernels: grid.x of the maize_gemm_splitk_reduce pass that follows (0 = none)
+    PackPlan pack_a, pack_b;  // packed kernels: operands repacked first; the product then runs on n_padded x k_padded
+    uint32_t n_padded, k_padded;
 };
 constexpr size_t kTicketBytes = 16384 * 4;  // ticket counters at the start of a workspace
 
 struct KernelInfo {
     const char* name;
+    const char* device_name;  // kernel of the code object that runs it (NULL: the same name)
     bool (*supports)(const maize_gemm_ex_desc_t&);
     // Fills the launch dimensions; false if the grid would exceed HIP limits.
     bool (*plan)(const maize_gemm_ex_desc_t&, uint32_t compute_units, LaunchDims*);

@@ -4,4 +4,5 @@
 #include "gemm_mt256.hpp"
 #include "gemm_skinny.hpp"
 #include "splitk_reduce.hpp"
+#include "pack.hpp"
 #include "probes.hpp"

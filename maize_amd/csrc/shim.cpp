@@ -62,6 +62,7 @@ struct maize_ctx {
     hipModule_t module;
     hipFunction_t fn[maize::kMaxKernels];
     hipFunction_t reduce_fn;
+    hipFunction_t pack_fn;
     // Split-K scratch, one per stream so that launches on different streams never share it.
     std::unordered_map<void*, maize_workspace> workspaces;
 };
@@ -118,7 +119,8 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
         return hip_fail(e, "hipModuleLoadData(embedded code object)");
     }
     for (uint32_t i = 0; i < maize::kernel_count(); ++i) {
-        e = hipModuleGetFunction(&ctx->fn[i], ctx->module, maize::kernel_at(i).name);
+        const maize::KernelInfo& ki = maize::kernel_at(i);
+        e = hipModuleGetFunction(&ctx->fn[i], ctx->module, ki.device_name ? ki.device_name : ki.name);
         if (e != hipSuccess) {
             int32_t rc = hip_fail(e, maize::kernel_at(i).name);
             (void)hipModuleUnload(ctx->module);
@@ -127,8 +129,9 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
         }
     }
     e = hipModuleGetFunction(&ctx->reduce_fn, ctx->module, maize::kReduceKernel);
+    if (e == hipSuccess) e = hipModuleGetFunction(&ctx->pack_fn, ctx->module, maize::kPackKernel);
     if (e != hipSuccess) {
-        int32_t rc = hip_fail(e, maize::kReduceKernel);
+        int32_t rc = hip_fail(e, "helper kernels of the embedded code object");
         (void)hipModuleUnload(ctx->module);
         delete ctx;
         return rc;
@@ -324,6 +327,7 @@ int32_t maize_hip_gemm_ex_plan(const maize_gemm_ex_desc_t* desc, const char* ker
     }
     const maize::KernelInfo& ki = maize::kernel_at((uint32_t)idx);
     maize::LaunchDims ld;
+    memset(&ld, 0, sizeof ld);
     if (!ki.plan(*desc, compute_units, &ld)) return fail(MAIZE_ERR_SHAPE, "gemm_plan: grid of '%s' exceeds the launch limits", ki.name);
     memset(out, 0, sizeof(*out));
     snprintf(out->kernel, sizeof(out->kernel), "%s", ki.name);
@@ -392,6 +396,7 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
     args.epi = (x->out_type == MAIZE_OUT_F32 ? 1u : 0u) | ((x->alpha != 1.0f || x->beta != 0.0f) ? 2u : 0u) |
                (x->in_type == MAIZE_IN_F16 ? 4u : 0u);
     maize::LaunchDims ld;
+    memset(&ld, 0, sizeof ld);
     if (!ki.plan(*x, (uint32_t)ctx->prop.multiProcessorCount, &ld))
         return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s cannot run M=%u N=%u K=%u batch=%u (grid limit)", ki.name,
                     d->c.nrows, d->c.ncols, d->a.ncols, d->batch);
@@ -401,8 +406,34 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
         int32_t rc = workspace_for(ctx, stream, ld.workspace_bytes, &args.workspace);
         if (rc != MAIZE_OK) return rc;
     }
+    // Packed kernels: operands that break the 16-byte rules are first copied, zero-padded, into the
+    // workspace; the first pass then runs on the padded extents and only the reduce pass sees the real C.
+    maize_gemm_args_t first = args;
+    for (int which = 0; which < 2; ++which) {
+        const maize::PackPlan& pp = which == 0 ? ld.pack_a : ld.pack_b;
+        if (!pp.on) continue;
+        struct { const void* src; void* dst; uint32_t rows, cols, ld_src, rows_dst, cols_dst, pad; uint64_t stride_src, stride_dst; } pa;
+        static_assert(sizeof(pa) == 56, "pack parameter block");
+        pa.src = which == 0 ? d->a.ptr : d->b.ptr;
+        pa.dst = (char*)args.workspace + pp.offset;
+        pa.rows = pp.rows; pa.cols = pp.cols; pa.ld_src = pp.ld_src; pa.rows_dst = pp.rows_dst; pa.cols_dst = pp.cols_dst; pa.pad = 0;
+        pa.stride_src = d->batch > 1 ? (which == 0 ? d->stride_a : d->stride_b) : 0;
+        pa.stride_dst = (uint64_t)pp.rows_dst * pp.cols_dst;
+        const uint64_t total = (uint64_t)pp.rows_dst * pp.cols_dst;
+        const uint32_t pgrid[3] = {(uint32_t)((total + 255) / 256), d->batch, 1}, pblock[3] = {256, 1, 1};
+        int32_t prc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->pack_fn, pgrid, pblock, 0, stream, &pa, sizeof pa);
+        if (prc != MAIZE_OK) return prc;
+        if (which == 0) { first.a = pa.dst; first.lda = 0; first.stride_a = pa.stride_dst; }
+        else { first.b = pa.dst; first.ldb = 0; first.stride_b = pa.stride_dst; first.brows = pp.rows_dst; first.bcols = pp.cols_dst; }
+    }
+    if (ld.n_padded) {
+        first.acols = ld.k_padded;
+        first.ccols = ld.n_padded;
+        if (d->layout == MAIZE_LAYOUT_NN) { first.brows = ld.k_padded; first.bcols = ld.n_padded; }
+        else { first.brows = ld.n_padded; first.bcols = ld.k_padded; }
+    }
     int32_t rc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->fn[idx], ld.grid, ld.block,
-                            ld.lds_bytes, stream, &args, sizeof args);
+                            ld.lds_bytes, stream, &first, sizeof first);
     if (rc != MAIZE_OK || ld.reduce_grid == 0) return rc;
     // Split-K macro-tile kernels: the partial tiles are combined by a second pass on the same stream.
     const uint32_t rgrid[3] = {ld.reduce_grid, 1, 1}, rblock[3] = {256, 1, 1};

@@ -60,6 +60,7 @@ def test_every_kernel_that_accepts_a_descriptor_plans_a_covering_grid(m, n, k, l
 def check_plan(p, m, n, k, layout, batch, cus=CUS):
     gx, gy, gz = p["grid"]
     splitk = p["kernel"].endswith("_splitk")
+    packed = p["kernel"].endswith("_packed")
     persistent = "_mt256_" in p["kernel"] and not p["kernel"].endswith("_edge")
     assert gx >= 1 and gy >= 1 and gz == (1 if persistent else batch)
     assert gy <= 65535 and gz <= 65535 and gx < (1 << 31)
@@ -68,6 +69,17 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         assert p["block"] == (256, 1, 1)
         assert gx == cdiv(n, 64) and gy == cdiv(m, 64)
         assert p["workspace_bytes"] == 0 and p["ksplit"] == 0
+    elif packed:
+        # the split-K kernels on zero-padded copies: work items over the padded extents, then the reduce pass
+        # over the real C; the workspace also holds the copies
+        n8, k8 = (n + 7) // 8 * 8, (k + 7) // 8 * 8
+        ks = p["ksplit"]
+        items = cdiv(m, 256) * cdiv(n8, 256) * batch * ks
+        resident = cus - cus % 8 if cus >= 8 else cus
+        assert p["block"] == (256, 1, 1) and gy == 1 and 1 <= ks <= 64 and gx == min(items, resident)
+        assert cdiv(cdiv(k8, 64), ks) * (ks - 1) < cdiv(k8, 64)
+        assert TICKET_BYTES + items * 256 * 256 * 4 <= p["workspace_bytes"] <= TICKET_BYTES + items * 256 * 256 * 4 + 2 * batch * (m * k8 + n8 * k8)
+        assert p["reduce_grid"] == cdiv(m * cdiv(n, 8) * batch, 256)
     elif splitk:
         # (tile, K range) work items, one fp32 partial tile each, then the reduce pass over runs of 8 columns
         assert p["block"] == (256, 1, 1) and gy == 1 and k % 8 == 0 and n % 8 == 0
@@ -141,6 +153,10 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",        # no skinny kernel for N x K weights
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
+        (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_packed",      # odd N: B repacked, C written element-wise
+        (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",
+        (4096, 4096, 4100, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",      # K % 8 != 0: both operands repacked
+        (511, 513, 1027, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",                 # too small to pay for the copies
     }
     for (m, n, k, layout, batch), want in picks.items():
         assert mz.gemm_plan(desc(m, n, k, layout, batch), compute_units=CUS)["kernel"] == want

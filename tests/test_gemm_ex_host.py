@@ -60,8 +60,9 @@ def test_dispatch_of_extended_descriptors():
     big = dict(m=4096, n=4096, k=4096)
     assert mz.gemm_plan(ex(**big, lda=4104, ldb=4224, ldc=8192))["kernel"] == "maize_gemm_bf16_mt256_nn"
     assert mz.gemm_plan(ex(**big, layout=mz.LAYOUT_NT, ldb=4104))["kernel"] == "maize_gemm_bf16_mt256_nt"
-    # rows that do not start on 16-byte boundaries: only the any-shape kernel takes them
-    assert mz.gemm_plan(ex(**big, lda=4100))["kernel"] == "maize_gemm_bf16_wave32"
+    # rows that do not start on 16-byte boundaries: that operand is repacked first
+    assert mz.gemm_plan(ex(**big, lda=4100))["kernel"] == "maize_gemm_bf16_mt256_nn_packed"
+    assert mz.gemm_plan(ex(64, 64, 64, lda=68))["kernel"] == "maize_gemm_bf16_wave32"          # unless the product is small
     # alpha / beta / fp32 C: the macro-tile kernels with the general epilogue; the plain ones refuse
     for kw in (dict(alpha=0.5), dict(beta=1.0), dict(out_type=mz.OUT_F32)):
         x = ex(**big, **kw)
@@ -73,7 +74,8 @@ def test_dispatch_of_extended_descriptors():
     # the skinny kernel carries the general epilogue
     for kw in (dict(alpha=0.5, beta=2.0), dict(out_type=mz.OUT_F32), dict(ldb=14400, ldc=14344)):
         assert mz.gemm_plan(ex(16, 14336, 4096, **kw))["kernel"] == "maize_gemm_bf16_skinny_nn"
-    assert mz.gemm_plan(ex(16, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_wave32"
+    assert mz.gemm_plan(ex(16, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_wave32"   # 0.94 GFLOP-equivalent: below the packing threshold
+    assert mz.gemm_plan(ex(16, 14336, 8192, ldb=14340))["kernel"] == "maize_gemm_bf16_mt256_nn_packed"
 
 
 def _supports(name, x):

@@ -272,3 +272,99 @@ def test_split_k_batched_and_more_items_than_workgroups(ctx, oracle):
         # bit-identical to itself on a second run (fixed summation order)
         again = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel="maize_gemm_bf16_mt256_nn_splitk")
         assert np.array_equal(got, again)
+
+
+# ---- packed path: odd extents, unaligned operands, any leading dimension ---------------------------
+
+def run_packed(ctx, oracle, m, n, k, layout, kernel, lda=None, ldb=None, ldc=None, a_off=0, b_off=0, c_off=0, alpha=1.0,
+               beta=0.0, out_f32=False, half=False, label=""):
+    """Like run_ex, with operands that start `*_off` elements into their buffers (2-byte-aligned views)."""
+    brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+    lda = k if lda is None else lda
+    ldb = bcols if ldb is None else ldb
+    ldc = n if ldc is None else ldc
+    rng = np.random.default_rng(m * 7 + n * 3 + k)
+    if half:
+        a = (rng.random(a_off + m * lda) * 2 - 1).astype(np.float16).view(np.uint16)
+        b = (rng.random(b_off + brows * ldb) * 2 - 1).astype(np.float16).view(np.uint16)
+    else:
+        a = mz.gen.uniform_bf16(a_off + m * lda, 5)
+        b = mz.gen.uniform_bf16(b_off + brows * ldb, 6)
+    if out_f32:
+        c0 = rng.standard_normal(c_off + m * ldc).astype(np.float32)
+    else:
+        c0 = rng.standard_normal(c_off + m * ldc).astype(np.float16).view(np.uint16) if half else mz.gen.uniform_bf16(c_off + m * ldc, 9)
+    esz = 4 if out_f32 else 2
+    da, db, dc = ctx.upload(a), ctx.upload(b), ctx.upload(c0)
+    try:
+        x = mz.gemm_ex_desc(mz.GlobalMatrix(da.ptr + 2 * a_off, m, k), mz.GlobalMatrix(db.ptr + 2 * b_off, brows, bcols),
+                            mz.GlobalMatrix(dc.ptr + esz * c_off, m, n), layout=layout, lda=0 if lda == k else lda,
+                            ldb=0 if ldb == bcols else ldb, ldc=0 if ldc == n else ldc,
+                            out_type=mz.OUT_F32 if out_f32 else mz.OUT_SAME, alpha=alpha, beta=beta,
+                            in_type=mz.IN_F16 if half else mz.IN_BF16)
+        took = mz.gemm_plan(x, kernel=kernel, compute_units=ctx.info()["compute_units"])["kernel"]
+        _say(f"{label} M={m} N={n} K={k} ld=({lda},{ldb},{ldc}) off=({a_off},{b_off},{c_off}) alpha={alpha} beta={beta} f32={out_f32} half={half} -> {took}")
+        ctx.gemm_bf16(x, kernel=kernel)
+        ctx.sync()
+        got = dc.download(np.float32 if out_f32 else np.uint16)
+    finally:
+        da.free(); db.free(); dc.free()
+    assert np.array_equal(got[:c_off].view(np.uint8), c0[:c_off].view(np.uint8)), f"{label}: wrote before C"
+    gv, ov = got[c_off:].reshape(m, ldc), c0[c_off:].reshape(m, ldc)
+    assert np.array_equal(gv[:, n:].view(np.uint8), ov[:, n:].view(np.uint8)), f"{label}: wrote into C's row padding"
+    elem = oracle.F16 if half else oracle.BF16
+    ref, val, scale = oracle.ref_gemm_ex(a[a_off:], b[b_off:], m, n, k, layout=layout, lda=lda, ldb=ldb, alpha=alpha, beta=beta,
+                                         c_old=None if beta == 0.0 else ov[:, :n].copy(), out_f32=out_f32, elem=elem)
+    g = gv[:, :n]
+    if out_f32:
+        err = np.abs(g.astype(np.float64) - val)
+        assert (err <= (k / 16.0 + 4.0) * 2.0 ** -24 * scale + 1e-45).all(), f"{label}: fp32 out of tolerance"
+    else:
+        s = oracle.compare(g, ref, val, scale, k, elem=elem)
+        assert s["n_fail"] == 0, f"{label}: {s}"
+    return took
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape", [(33, 17, 65), (300, 523, 1027), (257, 259, 72), (64, 1001, 2050), (520, 264, 129)])
+def test_packed_kernels_odd_extents(ctx, oracle, layout, shape):
+    m, n, k = shape
+    name = "maize_gemm_bf16_mt256_" + ("nt" if layout == mz.LAYOUT_NT else "nn") + "_packed"
+    bcols = n if layout == mz.LAYOUT_NN else k
+    run_packed(ctx, oracle, m, n, k, layout, name, label="packed")
+    run_packed(ctx, oracle, m, n, k, layout, name, lda=k + 3, ldb=bcols + 5, ldc=n + 7, label="packed odd ld")
+    run_packed(ctx, oracle, m, n, k, layout, name, a_off=1, b_off=3, c_off=5, label="packed 2-byte-aligned views")
+    run_packed(ctx, oracle, m, n, k, layout, name, alpha=-1.25, beta=0.75, ldc=n + 1, label="packed alpha beta")
+    run_packed(ctx, oracle, m, n, k, layout, name, out_f32=True, alpha=0.5, beta=2.0, c_off=1, label="packed f32")
+    run_packed(ctx, oracle, m, n, k, layout, name.replace("_bf16_", "_f16_"), half=True, a_off=1, ldc=n + 3, label="packed half")
+
+
+def test_packed_path_is_what_odd_large_shapes_get(ctx, oracle):
+    """The dispatcher's choice for large products that break the 16-byte rules, checked on sampled rows."""
+    from tests.gpu_util import sample_rows
+    for (m, n, k, layout) in ((1024, 4099, 1024, mz.LAYOUT_NN), (1000, 5003, 776, mz.LAYOUT_NT), (2048, 2048, 1028, mz.LAYOUT_NN)):
+        brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+        a = mz.gen.uniform_bf16(m * k, 41)
+        b = mz.gen.uniform_bf16(k * n, 42)
+        da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(m * n * 2)
+        d = mz.gemm_desc(mz.Matrix(da, m, k), mz.Matrix(db, brows, bcols), mz.Matrix(dc, m, n), layout=layout)
+        took = ctx.gemm_select(d)
+        assert took.endswith("_packed"), took
+        _say(f"packed dispatch {m}x{n}x{k} -> {took}")
+        ctx.gemm_bf16(d)
+        ctx.sync()
+        got = dc.download(np.uint16).reshape(m, n)
+        da.free(); db.free(); dc.free()
+        rows = sample_rows(m, count=24)
+        ref, f64, ab = oracle.ref_gemm_rows(a, b, m, n, k, rows, layout=layout)
+        s = oracle.compare(got[rows], ref, f64, ab, k)
+        assert s["n_fail"] == 0, s
+
+
+def test_packed_batched(ctx, oracle):
+    from tests.gpu_util import run_gemm, check_against_oracle
+    m, n, k, batch = 130, 267, 1033, 3
+    a = mz.gen.uniform_bf16(batch * m * k, 51)
+    b = mz.gen.uniform_bf16(batch * k * n, 52)
+    got = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel="maize_gemm_bf16_mt256_nn_packed")
+    check_against_oracle(oracle, got, a, b, m, n, k, batch=batch, label="packed batched")

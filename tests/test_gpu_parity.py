@@ -337,7 +337,7 @@ def test_dispatcher_choices(ctx):
     assert pick(2048, 2048, 2048, batch=32) == "maize_gemm_bf16_mt256_nn"
     assert pick(4096, 4096, 4072) == "maize_gemm_bf16_mt256_nn_ktail"
     assert pick(4096, 4096, 4064) == "maize_gemm_bf16_mt256_nn_ktail"
-    assert pick(4096, 4099, 4096) == "maize_gemm_bf16_wave32"
+    assert pick(4096, 4099, 4096) == "maize_gemm_bf16_mt256_nn_packed"     # odd N: B repacked, C written element-wise
     assert pick(33, 17, 65) == "maize_gemm_bf16_wave32"
 
 

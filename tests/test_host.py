@@ -55,7 +55,11 @@ def test_embedded_code_object_is_a_gfx950_elf_with_all_kernels():
     assert (e_flags & 0xFF) == 0x4F                                 # EF_AMDGPU_MACH_AMDGCN_GFX950
     names = mz.kernel_names()
     assert "maize_gemm_bf16_wave32" in names
-    for n in names + ["maize_probe_mfma_32x32x16", "maize_probe_ds_read_tr16", "maize_copy_u128"]:
+    # every registry entry runs a kernel of the code object: under its own name, or -- the packed entries --
+    # the split-K kernel of the same layout and type behind a repacking pass
+    device = [n.replace("_packed", "_splitk") for n in names]
+    for n in device + ["maize_gemm_splitk_reduce", "maize_pack_2d", "maize_probe_mfma_32x32x16", "maize_probe_ds_read_tr16",
+                       "maize_copy_u128"]:
         assert n.encode() in co, n
 
 
