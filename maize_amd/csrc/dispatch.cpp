@@ -373,11 +373,13 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // 16 x 4096 x 4096 up and loses (8 vs 4-7 us) only on short K with few rows or columns.
     if (ti >= 0 && kKernels[ti].supports(d) && (s.k >= 128 || (s.m >= 128 && s.n >= 128))) return (uint32_t)ti;
     // Odd extents or unaligned operands: the per-wave kernel reaches ~30 TFLOP/s, the macro-tile
-    // kernel on repacked operands ~1000, at the price of a few extra launches and copies (~50 us).
+    // kernel on repacked operands several hundred, at the price of extra launches (the packed path
+    // starts at ~21 us; measured break-even near M*N*K = 3e7) and of copying the operands once,
+    // which a product with very few rows or columns does not earn back.
     static const char* const kPacked[2][2] = {{"maize_gemm_bf16_mt256_nn_packed", "maize_gemm_bf16_mt256_nt_packed"},
                                               {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nt_packed"}};
     const int pi = kernel_index(kPacked[half_in(d)][s.nt]);
-    if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 1e9 &&
+    if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && s.m >= 24u && s.n >= 24u &&
         kKernels[pi].supports(d))
         return (uint32_t)pi;
     return (uint32_t)kernel_index("maize_gemm_bf16_wave32");

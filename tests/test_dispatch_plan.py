@@ -156,7 +156,9 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_packed",      # odd N: B repacked, C written element-wise
         (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",
         (4096, 4096, 4100, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",      # K % 8 != 0: both operands repacked
-        (511, 513, 1027, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",                 # too small to pay for the copies
+        (511, 513, 1027, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_packed",
+        (100, 203, 72, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",                  # too small to pay for the copies
+        (17, 50257, 768, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",                # 17 rows do not earn back a copy of B
     }
     for (m, n, k, layout, batch), want in picks.items():
         assert mz.gemm_plan(desc(m, n, k, layout, batch), compute_units=CUS)["kernel"] == want
