@@ -495,7 +495,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
         const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per read
         const uint32_t gcol = en0 + wn * 128u + cc * 8u;
-        const bool col_ok = gcol < N;                            // N % 8 == 0: a chunk is all in or all out
+        // Stores go through a buffer descriptor over this batch member's C: rows at or past M fall
+        // behind its end and are dropped by the range check, columns at or past N (N % 8 == 0: a
+        // chunk is all in or all out) get an out-of-range offset; no 64-bit address arithmetic and
+        // no divergent branch per row.  Non-temporal: C is written once and not read again by this
+        // kernel, it should not displace the operand panels in L2.
+        const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce, ((M - 1u) * ldc + N) * 2u);
+        const uint32_t c_vo = (((em0 + wm * 128u + cr) * ldc + gcol) * 2u) | (gcol < N ? 0u : OOB);
+        const uint32_t row_bytes = __builtin_amdgcn_readfirstlane(ldc * 2u);
     #pragma unroll
         for (int i = 0; i < 4; ++i) {
     #pragma unroll
@@ -515,10 +522,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 const uint32_t row = r * 4 + cr;                 // 0..31 within the pass
                 u32x4 v = *(lds_v4)(ew + row * 256u + ((cc ^ (row & 15u)) * 16u));
                 if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
-                const uint32_t grow = em0 + wm * 128u + i * 32u + row;
-                // C is written once and not read again by this kernel: non-temporal stores keep it from
-                // displacing the operand panels in L2.
-                if (col_ok && grow < M) __builtin_nontemporal_store(v, (u32x4*)(Ce + (uint64_t)grow * ldc + gcol));
+                __builtin_amdgcn_raw_buffer_store_b128(v, rc, c_vo, (uint32_t)(i * 32 + r * 4) * row_bytes, 2 /* nt */);
             }
         }
     }
