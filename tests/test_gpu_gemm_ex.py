@@ -368,3 +368,30 @@ def test_packed_batched(ctx, oracle):
     b = mz.gen.uniform_bf16(batch * k * n, 52)
     got = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel="maize_gemm_bf16_mt256_nn_packed")
     check_against_oracle(oracle, got, a, b, m, n, k, batch=batch, label="packed batched")
+
+
+def test_workspace_is_shared_safely_between_kernel_families(ctx, oracle):
+    """All workspace users of one stream share one buffer: ticket counters (which the skinny and edge kernels
+    must find zero) at its start, partial tiles and packed copies behind them.  Interleave them, growing the
+    workspace on the way, and check every result."""
+    from tests.gpu_util import run_gemm, check_against_oracle, sample_rows, check_rows_against_oracle
+    plan = [
+        ("maize_gemm_bf16_skinny_nn", (16, 1024, 2048)),
+        ("maize_gemm_bf16_mt256_nn_splitk", (64, 512, 4096)),
+        ("maize_gemm_bf16_skinny_nn", (7, 2048, 4096)),
+        ("maize_gemm_bf16_mt256_nn_packed", (130, 267, 1033)),
+        ("maize_gemm_bf16_mt256_nn_edge", (4096, 4104, 512)),      # grows the workspace: reallocation, zero-fill
+        ("maize_gemm_bf16_skinny_nn", (16, 1024, 2048)),
+        ("maize_gemm_bf16_mt256_nn_splitk", (256, 256, 2048)),
+        ("maize_gemm_bf16_mt256_nn_edge", (4096, 4104, 512)),
+        ("maize_gemm_bf16_skinny_nn", (3, 512, 1024)),
+    ]
+    for name, (m, n, k) in plan:
+        a = mz.gen.uniform_bf16(m * k, 61)
+        b = mz.gen.uniform_bf16(k * n, 62)
+        _say(f"workspace sharing: {name} {m}x{n}x{k}")
+        got = run_gemm(ctx, a, b, m, n, k, kernel=name)
+        if m * n * k <= 1 << 31:
+            check_against_oracle(oracle, got, a, b, m, n, k, label=name)
+        else:
+            check_rows_against_oracle(oracle, got, a, b, m, n, k, sample_rows(m, count=16), label=name)
