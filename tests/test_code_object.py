@@ -1,0 +1,104 @@
+"""What the embedded gfx950 code object contains, kernel by kernel.
+
+The reference checks its MMA catalogue by compiling a one-op kernel and asserting that the emitted PTX
+contains the op's mnemonic (run_test_sync_mma, crates/maize_tile/src/mma/mod.rs:101-114).  The analogue
+here disassembles the library's own code object (llvm-objdump of the ROCm toolchain that built it) and
+asserts, for every GEMM kernel, the matrix instruction of its operand type, the data-movement
+instructions the design rests on, and what must be absent: scratch memory (its mere use slowed a launch
+by 13 us), scalar stores, and hand-written packed-fp32 arithmetic."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+import maize_amd as mz
+
+OBJDUMP = shutil.which("llvm-objdump") or "/opt/rocm/llvm/bin/llvm-objdump"
+READELF = shutil.which("llvm-readelf") or "/opt/rocm/llvm/bin/llvm-readelf"
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HSACO = os.path.join(ROOT, "maize_amd", "lib", "maize_gemm_gfx950.hsaco")
+
+pytestmark = pytest.mark.skipif(not (os.path.exists(OBJDUMP) and os.path.exists(HSACO)),
+                                reason="needs the ROCm llvm-objdump and the built code object")
+
+
+@pytest.fixture(scope="module")
+def kernels():
+    """{kernel name: list of instruction mnemonics+operands}."""
+    text = subprocess.run([OBJDUMP, "-d", "--mcpu=gfx950", HSACO], check=True, capture_output=True, text=True).stdout
+    out, cur = {}, None
+    for line in text.splitlines():
+        m = re.match(r"^[0-9a-f]+ <([A-Za-z0-9_]+)>:", line)
+        if m:
+            cur = out.setdefault(m.group(1), [])
+            continue
+        if cur is not None and "\t" in line:
+            ins = line.split("//")[0].strip()
+            if ins:
+                cur.append(ins)
+    return out
+
+
+def count(instrs, prefix):
+    return sum(1 for i in instrs if i.startswith(prefix))
+
+
+def test_every_registry_entry_has_its_device_kernel(kernels):
+    for name in mz.kernel_names():
+        assert name.replace("_packed", "_splitk") in kernels, name
+    for helper in ("maize_gemm_splitk_reduce", "maize_pack_2d"):
+        assert helper in kernels
+
+
+def test_matrix_instruction_per_kernel(kernels):
+    for name, ins in kernels.items():
+        if "_mt256_" in name:
+            want = "v_mfma_f32_32x32x16_f16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_32x32x16_bf16"
+            other = "v_mfma_f32_32x32x16_bf16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_32x32x16_f16"
+            assert count(ins, want) >= 128 and count(ins, other) == 0, name       # two fully unrolled K steps of 64
+        elif name == "maize_gemm_bf16_skinny_nn":
+            assert count(ins, "v_mfma_f32_16x16x32_bf16") >= 16 and count(ins, "v_mfma_f32_16x16x32_f16") >= 16
+        elif name == "maize_gemm_bf16_wave32":
+            assert count(ins, "v_mfma_f32_32x32x16_bf16") >= 1 and count(ins, "v_mfma_f32_32x32x16_f16") >= 1
+
+
+def test_data_movement_the_design_rests_on(kernels):
+    for name, ins in kernels.items():
+        if "_mt256_" in name or name == "maize_gemm_bf16_skinny_nn":
+            lds_dma = [i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]
+            assert len(lds_dma) >= 16, f"{name}: operands must reach LDS by 128-bit direct-to-LDS loads"
+            assert count(ins, "ds_write_b128") == 0 or "_gen" in name or "_splitk" in name, name   # no register round trip for operands
+        if "_mt256_nn" in name or name == "maize_gemm_bf16_skinny_nn":
+            assert count(ins, "ds_read_b64_tr_b16") >= 8, f"{name}: a row-major K x N B is read with transposing reads"
+        if "_mt256_nt" in name:
+            assert count(ins, "ds_read_b64_tr_b16") == 0 and count(ins, "ds_read_b128") >= 16, name
+    plain = kernels["maize_gemm_bf16_mt256_nn"]
+    assert any(i.startswith("buffer_store_dwordx4") and i.rstrip().endswith("nt") for i in plain), "non-temporal C stores"
+    assert count(plain, "v_cvt_pk_bf16_f32") >= 128
+
+
+def test_nothing_that_must_not_be_there(kernels):
+    for name, ins in kernels.items():
+        assert count(ins, "scratch_") == 0, f"{name} spills to scratch"
+        assert not any(i.startswith("s_store") or i.startswith("s_buffer_store") or i.startswith("s_atomic") or i.startswith("s_dcache_wb")
+                       for i in ins), f"{name} writes through the scalar cache"
+        for banned in ("v_pk_add_f32", "v_pk_mul_f32", "v_pk_fma_f32"):
+            assert count(ins, banned) == 0, f"{name} contains {banned}"
+
+
+def test_main_loop_of_the_headline_kernel_is_lean(kernels):
+    """Between the first and the last MFMA of the plain NN kernel's unrolled K loop nothing but matrix
+    instructions, LDS reads, direct-to-LDS loads, waits, barriers and scalar bookkeeping may appear
+    (a handful of vector ALU ops recompute addresses in the persistent form)."""
+    ins = kernels["maize_gemm_bf16_mt256_nn"]
+    idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
+    # the K loop is the densest run of 128 consecutive MFMAs: find the window with the fewest other instructions
+    best = min(range(len(idx) - 127), key=lambda j: idx[j + 127] - idx[j])
+    body = ins[idx[best]:idx[best + 127] + 1]
+    allowed = ("v_mfma", "ds_read", "buffer_load_dwordx4", "s_", "v_add_u32", "v_or_b32", "v_mov_b32", "v_lshl")
+    extra = [i for i in body if not i.startswith(allowed)]
+    assert not extra, extra[:5]
+    assert count(body, "v_mfma") == 128 and len(body) <= 400          # 96 LDS reads, 32 loads, ~60 waits, scalar bookkeeping
+    assert count(body, "s_barrier") == 2
