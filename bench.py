@@ -121,10 +121,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--config", default="cfg1", choices=sorted(CONFIGS) + ["copy"],
+    ap.add_argument("--config", default=None, choices=sorted(CONFIGS) + ["copy"],
                     help="cfg1..cfg5: a benchmark configuration; copy: the 256 MiB copy used to scale HBM counters")
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--others", action=argparse.BooleanOptionalAction, default=None,
+                    help="also measure the other BASELINE configurations (shorter runs) and report them under "
+                         "\"other_configs\" (default: on when no --config is given)")
     ap.add_argument("--rotate", type=int, default=0,
                     help="number of distinct operand sets cycled through (0: enough to exceed the 256 MiB "
                          "last-level cache for the HBM-bound config, 1 otherwise)")
@@ -134,10 +137,37 @@ def main():
               "every box here has one GPU) -- run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.others is None:
+        args.others = args.config is None and args.kernel is None
+    args.config = args.config or "cfg1"
     if args.config == "copy":
         copy_calibration(args.steps, args.warmup)
         return
     import maize_amd as mz
+    ctx = mz.Context(0)
+    line = measure(mz, ctx, args.config, args.steps, args.warmup, args.kernel, args.rotate, not args.no_cpu)
+    if args.others:
+        # The other BASELINE configurations, shorter runs, same process: reported beside the headline.
+        others = {}
+        for name in sorted(CONFIGS):
+            if name == args.config:
+                continue
+            o = measure(mz, ctx, name, max(20, args.steps // 4), max(10, args.warmup // 2), None, 0, False)
+            others[name] = {"workload": o["config"]["workload"], "us_per_step": o["ms_per_step"] * 1e3, "value": o["value"],
+                            "unit": o["unit"], "kernel": o["roofline"]["kernel"], "roofline_bound": o["roofline"]["bound"],
+                            "roofline_frac": o["roofline"]["frac"], "steps": o["steps"]}
+        line["other_configs"] = others
+    print(json.dumps(line), flush=True)
+    ctx.close()
+
+
+def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
+    """One configuration: untimed clock ramp and warm-up, then exactly `steps` launches timed by the wall
+    clock (sync on both sides) and by HIP events on the launch stream.  Returns the JSON line as a dict."""
+    class A:  # the names the body below was written against
+        pass
+    args = A()
+    args.config, args.steps, args.warmup, args.kernel, args.rotate, args.no_cpu = config, steps, warmup, force_kernel, rotate, not with_cpu
     cfg = CONFIGS[args.config]
     m, n, k, batch, nt = cfg["m"], cfg["n"], cfg["k"], cfg["batch"], cfg["nt"]
     flops = 2.0 * batch * m * n * k
@@ -148,7 +178,6 @@ def main():
     if nt:  # same logical B, stored N x K
         b = np.concatenate([b[i * k * n:(i + 1) * k * n].reshape(k, n).T.ravel() for i in range(batch)])
 
-    ctx = mz.Context(0)
     info = ctx.info()
     nsets = args.rotate or (max(2, int(np.ceil(3 * 256 * 2 ** 20 / alg_bytes))) if cfg["bound"] == "hbm" else 1)
     sets = []
@@ -224,12 +253,13 @@ def main():
         "roofline": roof, "cpu_baseline": cpu, "parity_vs_oracle": parity,
         "device": {"name": info["name"], "compute_units": info["compute_units"], "clock_khz": info["clock_khz"]},
     }
-    print(json.dumps(line), flush=True)
     for da, db, dc, _ in sets:
         da.free(); db.free(); dc.free()
     ev0.destroy(); ev1.destroy()
     ctx.stream_destroy(stream)
-    ctx.close()
+    return line
+
+
 
 
 if __name__ == "__main__":
