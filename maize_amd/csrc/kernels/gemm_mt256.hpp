@@ -51,6 +51,7 @@
 // ever needs a K mask); the _ktail kernels take any K % 8 == 0.
 #pragma once
 #include "common.hpp"
+#include "maps.hpp"
 
 namespace maize {
 namespace mt256 {
@@ -214,15 +215,15 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         Cg = p.c + bz * p.stride_c * ((GEN && (p.epi & EPI_F32)) ? 2u : 1u);   // strides count elements of C
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint32_t row = (wave * 8u + i) * 8u + (lane >> 3);
-            const uint32_t c = (lane & 7u) ^ ((row >> 1) & 7u);
+            const uint32_t row = maps::kc_piece_row(wave * 8u + i, lane);
+            const uint32_t c = maps::kc_piece_chunk(wave * 8u + i, lane);
             a_vo[i] = ((m0 + row) * lda + c * 8u) * 2u;
             if (i < 2) a_k[i] = c * 8u;
             if (NT) {
                 b_vo[i] = ((n0 + row) * ldb + c * 8u) * 2u;
             } else {
-                const uint32_t brow = (wave * 8u + i) * 2u + (lane >> 5);
-                const uint32_t bc = (lane & 31u) ^ ((brow & 3u) << 2);
+                const uint32_t brow = maps::kn_piece_row(wave * 8u + i, lane);
+                const uint32_t bc = maps::kn_piece_chunk(wave * 8u + i, lane);
                 b_vo[i] = ((brow * ldb + n0 + bc * 8u) * 2u) | ((n0 + bc * 8u) < N ? 0u : OOB);
             }
         }
@@ -251,23 +252,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // ---- fragment read maps ---------------------------------------------------
     // MFMA 32x32x16: lane l holds row/col l%32 and k = 8*(l/32) + 0..7 of each 16-deep step.
     const uint32_t l32 = lane & 31u, lhi = lane >> 5;
-    // K-contiguous tile: 16-byte chunk (2*kk + lhi) of row r lives at chunk' = chunk ^ ((r>>1)&7).
-    const uint32_t sw = lhi ^ ((l32 >> 1) & 7u);
-    uint32_t a_rd[4], b_rd[4];                                 // per kk (K-contiguous) or per j (K x N) addresses
+    // Byte offsets of the lane's fragment reads inside a tile (maps.hpp): per kk for a K-contiguous
+    // tile (add 32 rows * 128 B per fragment), per j for the K x N tile (add kk * 16 and h * 4 rows).
+    uint32_t a_rd[4], b_rd[4];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) a_rd[kk] = (wm * 128u + l32) * KROW + ((sw ^ (2u * kk)) * 16u);
+    for (int kk = 0; kk < 4; ++kk) a_rd[kk] = maps::kc_frag_offset(wm * 128u, kk, lane);
     if (NT) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) b_rd[kk] = (wn * 128u + l32) * KROW + ((sw ^ (2u * kk)) * 16u);
+        for (int kk = 0; kk < 4; ++kk) b_rd[kk] = maps::kc_frag_offset(wn * 128u, kk, lane);
     } else {
-        // Transposing read: in each group of 16 lanes, lane q addresses 4 consecutive columns
-        // (q%4) of row (q/4); lane q receives column q of the 4 x 16 block, rows 0..3.
-        const uint32_t q = lane & 15u, half = (lane >> 4) & 1u;
-        const uint32_t s = q >> 2;                             // row & 3 of the addressed row
-        const uint32_t row = lhi * 8u + s;                     // + kk*16 (+4 for the second read)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            b_rd[j] = row * NROW + (wn * 4u + ((uint32_t)j ^ s)) * 64u + half * 32u + (q & 3u) * 8u;
+        for (int j = 0; j < 4; ++j) b_rd[j] = maps::kn_tr_offset(wn * 128u, j, 0, 0, lane);
     }
 
     bf16x8 fa[2][4];
@@ -513,14 +508,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
                     if (EDGE && split) f = reduced_chunk(i * 16 + j * 4 + q);
                     u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
-                    const uint32_t chunk = (uint32_t)(j * 4 + q) ^ (l32 & 15u);
-                    const uint32_t hf = lhi ^ ((l32 >> 4) & 1u);
-                    *(lds_v2)(ew + l32 * 256u + chunk * 16u + hf * 8u) = v;
+                    *(lds_v2)(ew + maps::epi_write_offset(j, q, lane)) = v;
                 }
     #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                const uint32_t row = r * 4 + cr;                 // 0..31 within the pass
-                u32x4 v = *(lds_v4)(ew + row * 256u + ((cc ^ (row & 15u)) * 16u));
+                u32x4 v = *(lds_v4)(ew + maps::epi_read_offset(r, lane));
                 if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
                 __builtin_amdgcn_raw_buffer_store_b128(v, rc, c_vo, (uint32_t)(i * 32 + r * 4) * row_bytes, 2 /* nt */);
             }

@@ -30,6 +30,7 @@
 // N % 8 == 0, 16-byte aligned operands, every matrix (per batch member) below 2 GiB.
 #pragma once
 #include "common.hpp"
+#include "maps.hpp"
 
 namespace maize {
 namespace skinny {
@@ -52,7 +53,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 // Granule swizzle of a block: the 32-byte granule index (0..15) of row r is XOR-ed with
 // f(r) = r%4 + 4*bit3(r), so the 8 rows one transposing read touches land in 8 different
 // granules of the 256-byte bank period.
-__device__ __forceinline__ uint32_t gsw(uint32_t r) { return (r & 3u) | (((r >> 3) & 1u) << 2); }
 
 __device__ __forceinline__ void body(const GemmArgs& p) {
     // One array per ring slot: distinct objects let the compiler see that a load into one slot
@@ -89,12 +89,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
     // ---- copy map: wave w issues pieces 2w and 2w+1 of a block; piece pc = rows 2pc, 2pc+1.
     // Lane l lands at byte 16 l of the piece = row 2pc + l/32, stored chunk l%32, and therefore
-    // fetches logical chunk (l%32) ^ (gsw(row) << 1).
+    // fetches logical chunk (l%32) ^ (swizzle(row) << 1) (maps::sk_piece_chunk).
     uint32_t b_vo[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const uint32_t row = (wave * 2u + i) * 2u + (lane >> 5);
-        const uint32_t c = (lane & 31u) ^ (gsw(row) << 1);
+        const uint32_t row = maps::sk_piece_row(wave * 2u + i, lane);
+        const uint32_t c = maps::sk_piece_chunk(wave * 2u + i, lane);
         const uint32_t col = n0 + c * 8u;
         b_vo[i] = ((row * ldb + col) * 2u) | (col < N ? 0u : OOB);       // N % 8 == 0: a chunk is all in or all out
     }
@@ -104,16 +104,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // ---- transposing-read map.  In each group of 16 lanes, lane q addresses 4 consecutive
     // columns (q%4) of row (q/4) of a 4 x 16 sub-block and receives column q, rows 0..3.  Lane
     // group g = l/16 needs k = 8g .. 8g+7 (two reads, h = 0,1) of column group cg (16 columns).
-    // Byte address = row*512 + ((cg ^ gsw(row)) * 32) + ((q%4)/2)*16 + (q%2)*8.
-    const uint32_t q = lane & 15u, g = lane >> 4;
+    // Byte address: maps::sk_tr_offset.
+    const uint32_t g = lane >> 4;
     uint32_t rd[2][2];                                   // [h][which of the wave's two column groups]
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const uint32_t row = g * 8u + h * 4u + (q >> 2);
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2)
-            rd[h][c2] = row * ROW + (((wave * 2u + c2) ^ gsw(row)) * 32u) + ((q & 3u) >> 1) * 16u + (q & 1u) * 8u;
-    }
+        for (int c2 = 0; c2 < 2; ++c2) rd[h][c2] = maps::sk_tr_offset(wave * 2u + c2, h, lane);
 
     const uint32_t krange = K / ks, k0 = z * krange;
     const uint32_t nb = krange / KB;                     // blocks of this workgroup
