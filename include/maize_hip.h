@@ -20,7 +20,14 @@
  *    crates/maize_core/src/codegen/mod.rs:15-33); distinct contexts are
  *    independent.
  *  - Launches are asynchronous on the stream passed in (NULL = the null
- *    stream).
+ *    stream).  Every entry point makes the context's device current while it
+ *    runs and puts the calling thread's previous device back before returning.
+ *  - Kernels that split K or repack operands use a workspace the library owns,
+ *    one per (context, stream), allocated (or grown) by the first launch that
+ *    needs it: that launch calls hipMalloc and, when growing, waits for the
+ *    stream.  maize_hip_gemm_plan reports the bytes.  The workspace is released
+ *    by maize_hip_stream_destroy for streams made by maize_hip_stream_create,
+ *    and by maize_hip_ctx_destroy for every other stream it was used with.
  *  - All matrices are row-major with leading dimension == ncols, as in the
  *    reference (crates/maize_tile/src/gmem/row_panel.rs:55,
  *    crates/maize_tile/src/gmem/col_panel.rs:108).  BF16 is a 2-byte,
@@ -44,7 +51,8 @@ enum {
     MAIZE_ERR_LAYOUT = -4,      /* unknown maize_layout_t value */
     MAIZE_ERR_KERNEL = -5,      /* unknown kernel name, or the kernel cannot run this descriptor */
     MAIZE_ERR_NO_DEVICE = -6,   /* no usable HIP device / device is not gfx950 */
-    MAIZE_ERR_ARG = -7          /* any other invalid argument */
+    MAIZE_ERR_ARG = -7,         /* any other invalid argument */
+    MAIZE_ERR_NOMEM = -8        /* host memory for a handle could not be allocated */
 };
 
 typedef struct maize_ctx maize_ctx_t;
@@ -216,7 +224,7 @@ int32_t maize_hip_memcpy_h2d(maize_ctx_t* ctx, void* dst, const void* src, size_
 int32_t maize_hip_memcpy_d2h(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes);
 int32_t maize_hip_memset(maize_ctx_t* ctx, void* dst, int value, size_t nbytes);
 int32_t maize_hip_stream_create(maize_ctx_t* ctx, void** out);
-int32_t maize_hip_stream_destroy(maize_ctx_t* ctx, void* stream);
+int32_t maize_hip_stream_destroy(maize_ctx_t* ctx, void* stream); /* waits for the stream if it owns a workspace */
 int32_t maize_hip_sync(maize_ctx_t* ctx, void* stream); /* NULL: whole device */
 int32_t maize_hip_event_create(maize_ctx_t* ctx, maize_event_t** out);
 int32_t maize_hip_event_record(maize_event_t* ev, void* stream);

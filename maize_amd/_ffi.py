@@ -32,6 +32,7 @@ MAIZE_ERR_LAYOUT = -4
 MAIZE_ERR_KERNEL = -5
 MAIZE_ERR_NO_DEVICE = -6
 MAIZE_ERR_ARG = -7
+MAIZE_ERR_NOMEM = -8
 
 LAYOUT_NN = 0
 LAYOUT_NT = 1

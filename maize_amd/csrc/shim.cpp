@@ -44,6 +44,24 @@ int32_t hip_fail(hipError_t e, const char* what) {
     return (int32_t)e;
 }
 
+// Makes the context's device current for the duration of one entry point and puts the caller's
+// back afterwards: the library never changes the calling thread's current device.
+struct DeviceGuard {
+    int prev = -1;
+    bool changed = false;
+    hipError_t enter(int device) {
+        hipError_t e = hipGetDevice(&prev);
+        if (e != hipSuccess) return e;
+        if (prev == device) return hipSuccess;
+        e = hipSetDevice(device);
+        changed = e == hipSuccess;
+        return e;
+    }
+    ~DeviceGuard() {
+        if (changed) (void)hipSetDevice(prev);
+    }
+};
+
 #define HIP_TRY(expr)                                  \
     do {                                               \
         hipError_t e_ = (expr);                        \
@@ -98,9 +116,10 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
         return fail(MAIZE_ERR_NO_DEVICE, "ctx_create: no HIP device (%s)", hipGetErrorString(e));
     if (device < 0 || device >= count)
         return fail(MAIZE_ERR_NO_DEVICE, "ctx_create: device %d out of range (%d devices)", device, count);
-    HIP_TRY(hipSetDevice(device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(device));
     maize_ctx* ctx = new (std::nothrow) maize_ctx();
-    if (!ctx) return fail(MAIZE_ERR_ARG, "ctx_create: out of host memory");
+    if (!ctx) return fail(MAIZE_ERR_NOMEM, "ctx_create: out of host memory");
     ctx->device = device;
     e = hipGetDeviceProperties(&ctx->prop, device);
     if (e != hipSuccess) {
@@ -142,7 +161,8 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
 
 int32_t maize_hip_ctx_destroy(maize_ctx_t* ctx) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "ctx_destroy: ctx is NULL");
-    (void)hipSetDevice(ctx->device);
+    DeviceGuard guard_;
+    (void)guard_.enter(ctx->device);
     for (auto& kv : ctx->workspaces)
         if (kv.second.ptr) (void)hipFree(kv.second.ptr);
     hipError_t e = hipModuleUnload(ctx->module);
@@ -170,9 +190,10 @@ int32_t maize_hip_module_load(maize_ctx_t* ctx, const void* hsaco, size_t nbytes
     *out = nullptr;
     if (nbytes < 64 || memcmp(hsaco, "\177ELF", 4) != 0)
         return fail(MAIZE_ERR_ARG, "module_load: not an ELF code object (%zu bytes)", nbytes);
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     maize_module* m = new (std::nothrow) maize_module();
-    if (!m) return fail(MAIZE_ERR_ARG, "module_load: out of host memory");
+    if (!m) return fail(MAIZE_ERR_NOMEM, "module_load: out of host memory");
     m->ctx = ctx;
     hipError_t e = hipModuleLoadData(&m->module, hsaco);
     if (e != hipSuccess) {
@@ -185,7 +206,8 @@ int32_t maize_hip_module_load(maize_ctx_t* ctx, const void* hsaco, size_t nbytes
 
 int32_t maize_hip_module_unload(maize_module_t* mod) {
     if (!mod) return fail(MAIZE_ERR_NULL, "module_unload: module is NULL");
-    (void)hipSetDevice(mod->ctx->device);
+    DeviceGuard guard_;
+    (void)guard_.enter(mod->ctx->device);
     hipError_t e = hipModuleUnload(mod->module);
     delete mod;
     if (e != hipSuccess) return hip_fail(e, "hipModuleUnload");
@@ -195,12 +217,13 @@ int32_t maize_hip_module_unload(maize_module_t* mod) {
 int32_t maize_hip_kernel_get(maize_module_t* mod, const char* name, maize_kernel_t** out) {
     if (!mod || !name || !out) return fail(MAIZE_ERR_NULL, "kernel_get: NULL argument");
     *out = nullptr;
-    HIP_TRY(hipSetDevice(mod->ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(mod->ctx->device));
     hipFunction_t fn;
     hipError_t e = hipModuleGetFunction(&fn, mod->module, name);
     if (e != hipSuccess) return hip_fail(e, name);
     maize_kernel* k = new (std::nothrow) maize_kernel();
-    if (!k) return fail(MAIZE_ERR_ARG, "kernel_get: out of host memory");
+    if (!k) return fail(MAIZE_ERR_NOMEM, "kernel_get: out of host memory");
     k->ctx = mod->ctx;
     k->fn = fn;
     *out = k;
@@ -222,7 +245,8 @@ static int32_t launch_raw(int device, uint32_t lds_limit, hipFunction_t fn, cons
     if (threads > 1024) return fail(MAIZE_ERR_ARG, "launch: %llu threads per block exceeds 1024", (unsigned long long)threads);
     if (grid[1] > 65535u || grid[2] > 65535u) return fail(MAIZE_ERR_ARG, "launch: grid.y/z exceeds 65535");
     if (lds_bytes > lds_limit) return fail(MAIZE_ERR_ARG, "launch: %u bytes of LDS exceeds the device's %u", lds_bytes, lds_limit);
-    HIP_TRY(hipSetDevice(device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(device));
     size_t sz = args_bytes;
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(args), HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz,
                      HIP_LAUNCH_PARAM_END};
@@ -362,7 +386,8 @@ int32_t maize_hip_gemm_select(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, c
 static int32_t workspace_for(maize_ctx_t* ctx, void* stream, size_t bytes, void** out) {
     maize_workspace& w = ctx->workspaces[stream];
     if (w.bytes < bytes) {
-        HIP_TRY(hipSetDevice(ctx->device));
+        DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
         if (w.ptr) {
             HIP_TRY(hipStreamSynchronize((hipStream_t)stream));  // earlier launches may still use the old one
             HIP_TRY(hipFree(w.ptr));
@@ -473,7 +498,8 @@ int32_t maize_hip_malloc(maize_ctx_t* ctx, size_t nbytes, void** out) {
     if (!ctx || !out) return fail(MAIZE_ERR_NULL, "malloc: NULL argument");
     *out = nullptr;
     if (nbytes == 0) return fail(MAIZE_ERR_ARG, "malloc: zero bytes");
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipMalloc(out, nbytes));
     return MAIZE_OK;
 }
@@ -481,35 +507,40 @@ int32_t maize_hip_malloc(maize_ctx_t* ctx, size_t nbytes, void** out) {
 int32_t maize_hip_free(maize_ctx_t* ctx, void* ptr) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "free: ctx is NULL");
     if (!ptr) return MAIZE_OK;
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipFree(ptr));
     return MAIZE_OK;
 }
 
 int32_t maize_hip_memcpy_h2d(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes) {
     if (!ctx || !dst || !src) return fail(MAIZE_ERR_NULL, "memcpy_h2d: NULL argument");
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipMemcpy(dst, src, nbytes, hipMemcpyHostToDevice));
     return MAIZE_OK;
 }
 
 int32_t maize_hip_memcpy_d2h(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes) {
     if (!ctx || !dst || !src) return fail(MAIZE_ERR_NULL, "memcpy_d2h: NULL argument");
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipMemcpy(dst, src, nbytes, hipMemcpyDeviceToHost));
     return MAIZE_OK;
 }
 
 int32_t maize_hip_memset(maize_ctx_t* ctx, void* dst, int value, size_t nbytes) {
     if (!ctx || !dst) return fail(MAIZE_ERR_NULL, "memset: NULL argument");
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipMemset(dst, value, nbytes));
     return MAIZE_OK;
 }
 
 int32_t maize_hip_stream_create(maize_ctx_t* ctx, void** out) {
     if (!ctx || !out) return fail(MAIZE_ERR_NULL, "stream_create: NULL argument");
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     hipStream_t s;
     HIP_TRY(hipStreamCreate(&s));  // default priority
     *out = (void*)s;
@@ -518,14 +549,24 @@ int32_t maize_hip_stream_create(maize_ctx_t* ctx, void** out) {
 
 int32_t maize_hip_stream_destroy(maize_ctx_t* ctx, void* stream) {
     if (!ctx || !stream) return fail(MAIZE_ERR_NULL, "stream_destroy: NULL argument");
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
+    // The stream's workspace goes with it (its launches first run to completion).
+    auto it = ctx->workspaces.find(stream);
+    if (it != ctx->workspaces.end()) {
+        HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+        void* ws = it->second.ptr;
+        ctx->workspaces.erase(it);
+        if (ws) HIP_TRY(hipFree(ws));
+    }
     HIP_TRY(hipStreamDestroy((hipStream_t)stream));
     return MAIZE_OK;
 }
 
 int32_t maize_hip_sync(maize_ctx_t* ctx, void* stream) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "sync: ctx is NULL");
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     if (stream)
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     else
@@ -536,9 +577,10 @@ int32_t maize_hip_sync(maize_ctx_t* ctx, void* stream) {
 int32_t maize_hip_event_create(maize_ctx_t* ctx, maize_event_t** out) {
     if (!ctx || !out) return fail(MAIZE_ERR_NULL, "event_create: NULL argument");
     *out = nullptr;
-    HIP_TRY(hipSetDevice(ctx->device));
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
     maize_event* ev = new (std::nothrow) maize_event();
-    if (!ev) return fail(MAIZE_ERR_ARG, "event_create: out of host memory");
+    if (!ev) return fail(MAIZE_ERR_NOMEM, "event_create: out of host memory");
     hipError_t e = hipEventCreate(&ev->ev);
     if (e != hipSuccess) {
         delete ev;

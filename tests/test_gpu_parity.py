@@ -303,9 +303,10 @@ def test_skinny_split_k_repeats_streams_and_batches(ctx, oracle):
     check_against_oracle(oracle, first, a, b, m, n, k, label="skinny split-K")
     for _ in range(3):
         assert np.array_equal(run_gemm(ctx, a, b, m, n, k), first)
-    s = ctx.stream()
-    assert np.array_equal(run_gemm(ctx, a, b, m, n, k, stream=s), first)
-    ctx.stream_destroy(s)
+    for _ in range(3):                            # a destroyed stream takes its workspace with it: a recycled handle starts clean
+        s = ctx.stream()
+        assert np.array_equal(run_gemm(ctx, a, b, m, n, k, stream=s), first)
+        ctx.stream_destroy(s)
     # a different shape in between (its workspace layout differs), then the first one again
     a2 = mz.gen.normal_bf16(7 * 2048, 3, 1.0)
     b2 = mz.gen.normal_bf16(2048 * 264, 4, 0.02)
