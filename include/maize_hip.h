@@ -94,12 +94,16 @@ typedef struct {
  *   out_type:    element type of C; batch stride stride_c counts elements of that type.
  *   beta == 0:   C is not read (it may hold anything, NaNs included).
  * All-zero extension fields with alpha = 1 describe exactly the plain descriptor. */
-/* MAIZE_OUT_SAME: C has the 16-bit type of A and B (bf16, or half for half operands). */
+/* MAIZE_OUT_SAME: C has the 16-bit type of A and B (bf16, or half for half operands; bf16 for 8-bit operands). */
 typedef enum { MAIZE_OUT_SAME = 0, MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1 } maize_out_type_t;
 /* Element type of A and B.  The reference's MMA catalogue lists the half-precision twin of its bf16
  * op (Sm80MmaF16F32_16x8x16 beside Sm80MmaBf16F32_16x8x16, crates/maize_tile/src/mma/sm80.rs);
- * here it is v_mfma_f32_*_f16 on the same tiles. */
-typedef enum { MAIZE_IN_BF16 = 0, MAIZE_IN_F16 = 1 } maize_in_type_t;
+ * here it is v_mfma_f32_*_f16 on the same tiles.  E4M3 and E5M2 are the OCP 8-bit floats of the
+ * catalogue's Sm89MmaF8F32_* entries (crates/maize_tile/src/mma/sm89.rs:13-45; u8-backed,
+ * crates/maize_core/src/ty/sized.rs:68-69): A and B hold one byte per element, dimensions, leading
+ * dimensions and batch strides still count elements, and the matrix instruction is
+ * v_mfma_f32_32x32x64_f8f6f4 when B is stored N x K (MAIZE_LAYOUT_NT) with 16-byte aligned rows. */
+typedef enum { MAIZE_IN_BF16 = 0, MAIZE_IN_F16 = 1, MAIZE_IN_E4M3 = 2, MAIZE_IN_E5M2 = 3 } maize_in_type_t;
 typedef struct {
     maize_gemm_desc_t gemm;
     uint32_t lda, ldb, ldc;

@@ -41,6 +41,8 @@ OUT_BF16 = 0
 OUT_F32 = 1
 IN_BF16 = 0
 IN_F16 = 1
+IN_E4M3 = 2
+IN_E5M2 = 3
 
 
 class MatrixT(C.Structure):

@@ -163,8 +163,8 @@ def GlobalMatrix(ptr, nrows, ncols):
 class Matrix:
     """A device matrix: row-major, leading dimension == ncols (reference gmem/matrix.rs:6-19)."""
 
-    def __init__(self, buf, nrows, ncols, offset_elems=0):
-        self.buf, self.nrows, self.ncols, self.offset_elems = buf, nrows, ncols, offset_elems
+    def __init__(self, buf, nrows, ncols, offset_elems=0, elem_bytes=2):
+        self.buf, self.nrows, self.ncols, self.offset_elems, self.elem_bytes = buf, nrows, ncols, offset_elems, elem_bytes
 
     @classmethod
     def new(cls, buf, nrows, ncols):
@@ -172,7 +172,7 @@ class Matrix:
 
     @property
     def ptr(self):
-        return self.buf.ptr + 2 * self.offset_elems
+        return self.buf.ptr + self.elem_bytes * self.offset_elems
 
     def realize(self):
         return GlobalMatrix(self.ptr, self.nrows, self.ncols)

@@ -26,6 +26,8 @@ inline bool plain_epilogue(const maize_gemm_ex_desc_t& d) {
     return d.out_type == MAIZE_OUT_SAME && d.alpha == 1.0f && d.beta == 0.0f;
 }
 inline bool half_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_F16; }
+inline bool bf16_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_BF16; }
+inline bool fp8_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 || d.in_type == MAIZE_IN_E5M2; }
 
 // ---- maize_gemm_bf16_wave32: any shape ------------------------------------
 bool wave32_supports(const maize_gemm_ex_desc_t&) { return true; }
@@ -64,19 +66,36 @@ bool mt256_common(const maize_gemm_ex_desc_t& d) {
 bool k64(const maize_gemm_ex_desc_t& d) { return (d.gemm.a.ncols & 63u) == 0; }
 // The plain and edge-splitting kernels store bf16 of A.B only; the _gen kernels carry the general epilogue.
 bool nn(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NN; }
-bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && !half_in(d); }
-bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && !half_in(d); }
-bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && plain_epilogue(d) && !half_in(d); }
-bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && plain_epilogue(d) && !half_in(d); }
-bool mt256_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && !half_in(d); }
-bool mt256_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && !half_in(d); }
-bool mt256_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && !half_in(d); }
-bool mt256_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && !half_in(d); }
+bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && bf16_in(d); }
+bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && bf16_in(d); }
+bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && plain_epilogue(d) && bf16_in(d); }
+bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && plain_epilogue(d) && bf16_in(d); }
+bool mt256_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && bf16_in(d); }
+bool mt256_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && bf16_in(d); }
+bool mt256_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && bf16_in(d); }
+bool mt256_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && bf16_in(d); }
 // IEEE half operands: the general-epilogue kernels instantiated on v_mfma_f32_32x32x16_f16.
 bool f16_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && half_in(d); }
 bool f16_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && half_in(d); }
 bool f16_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && half_in(d); }
 bool f16_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && half_in(d); }
+// 8-bit operands (one byte per element), both K-contiguous: rows of A and B start on 16-byte
+// boundaries and K % 16 == 0; C as for the general-epilogue kernels (N % 8 == 0, rows on 16-byte
+// boundaries).  32-bit buffer offsets: each operand of one batch member stays below 2 GiB.
+bool f8_nt_common(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    if (nn(d) || (s.k & 15u) || (s.n & 7u)) return false;
+    if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr | (uintptr_t)d.gemm.c.ptr) & 15u) return false;
+    if ((l.a | l.b) & 15u || (l.c & 7u)) return false;
+    if (d.gemm.batch > 1 && (((d.gemm.stride_a | d.gemm.stride_b) & 15u) || (d.gemm.stride_c & 7u))) return false;
+    const uint64_t lim = 1ull << 31;
+    if (l.ext_a >= lim || l.ext_b >= lim || l.ext_c * 2 >= lim) return false;
+    if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21)) return false;
+    return true;
+}
+bool e4m3_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 && f8_nt_common(d); }
+bool e5m2_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E5M2 && f8_nt_common(d); }
 // Edge splitting.  A ragged N leaves a last column of tiles that are almost empty but cost a
 // whole tile each (likewise a ragged M and the last row).  When that edge is at most 32 elements
 // wide and setting it aside saves a round of workgroups (one workgroup per compute unit per
@@ -167,8 +186,8 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus) {
     }
     return best_ks;
 }
-bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && !half_in(d); }
-bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && !half_in(d); }
+bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && bf16_in(d); }
+bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && bf16_in(d); }
 bool splitk_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && half_in(d); }
 bool splitk_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && half_in(d); }
 bool splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
@@ -230,8 +249,8 @@ bool packed_ok(const maize_gemm_ex_desc_t& d) {
     const uint64_t copies = ((p.a ? p.a_elems : 0) + (p.b ? p.b_elems : 0)) * d.gemm.batch * 2;
     return copies <= (1ull << 31);
 }
-bool packed_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && !half_in(d) && packed_ok(d); }
-bool packed_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && !half_in(d) && packed_ok(d); }
+bool packed_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && bf16_in(d) && packed_ok(d); }
+bool packed_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && bf16_in(d) && packed_ok(d); }
 bool packed_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && half_in(d) && packed_ok(d); }
 bool packed_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && half_in(d) && packed_ok(d); }
 bool packed_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
@@ -272,7 +291,7 @@ bool packed_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDi
 // ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
 bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
-    if (d.gemm.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
+    if (fp8_in(d) || d.gemm.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
     const uint64_t lim = 1ull << 31;
     const Lds l = lds_of(d);
     if (l.ext_a * 2 >= lim || l.ext_b * 2 >= lim || s.n >= (1u << 21) || l.b >= (1u << 21)) return false;
@@ -329,6 +348,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_packed", "maize_gemm_bf16_mt256_nt_splitk", packed_nt_supports, packed_plan},
     {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nn_splitk", packed_f16_nn_supports, packed_plan},
     {"maize_gemm_f16_mt256_nt_packed", "maize_gemm_f16_mt256_nt_splitk", packed_f16_nt_supports, packed_plan},
+    {"maize_gemm_e4m3_mt256_nt", nullptr, e4m3_nt_supports, mt256_plan},
+    {"maize_gemm_e5m2_mt256_nt", nullptr, e5m2_nt_supports, mt256_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -345,6 +366,13 @@ int kernel_index(const char* name) {
 
 uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     const Dims s = dims_of(d);
+    if (fp8_in(d)) {
+        // 8-bit operands: the macro-tile kernel when both operands are K-contiguous and aligned (same
+        // size rule as below), else the per-wave kernel, which widens them to half as it loads.
+        const int fi = kernel_index(d.in_type == MAIZE_IN_E4M3 ? "maize_gemm_e4m3_mt256_nt" : "maize_gemm_e5m2_mt256_nt");
+        if (fi >= 0 && kKernels[fi].supports(d) && (s.k >= 256 || (s.m >= 128 && s.n >= 128))) return (uint32_t)fi;
+        return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
+    }
     // Few rows against a wide row-major B: bound by streaming B once.
     const int sk = kernel_index("maize_gemm_bf16_skinny_nn");
     if (sk >= 0 && kKernels[sk].supports(d) && s.n >= 64) return (uint32_t)sk;

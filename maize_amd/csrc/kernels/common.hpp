@@ -20,11 +20,12 @@ struct GemmArgs {
     uint32_t reserved;
     // Extended part (all zero = the plain product: compact rows, bf16 C = A.B).
     uint32_t lda, ldb, ldc;  // elements between consecutive rows; 0 = the matrix's column count
-    uint32_t epi;            // bit 0: C is fp32; bit 1: C = alpha * A.B + beta * C; bit 2: A, B (and a 16-bit C) are IEEE half
+    uint32_t epi;            // bit 0: C is fp32; bit 1: C = alpha * A.B + beta * C; bit 2: A, B (and a 16-bit C) are IEEE half;
+                             // bit 3 / bit 4: A and B are 8-bit E4M3 / E5M2 (a 16-bit C is bf16)
     float alpha, beta;
 };
 static_assert(sizeof(GemmArgs) == 120, "kernel parameter block layout");
-constexpr uint32_t EPI_F32 = 1u, EPI_SCALE = 2u, EPI_F16 = 4u;
+constexpr uint32_t EPI_F32 = 1u, EPI_SCALE = 2u, EPI_F16 = 4u, EPI_E4M3 = 8u, EPI_E5M2 = 16u;
 
 // Leading dimensions with their defaults: the reference's rows are compact (row stride ==
 // ncols, crates/maize_tile/src/gmem/row_panel.rs:55).
@@ -65,6 +66,25 @@ __device__ __forceinline__ uint32_t cvt_pk_f16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, halfx2));
 }
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h); }
+
+// OCP 8-bit floats -> the high half of the equal fp32 (a bf16 bit pattern; exact: at most 3 fraction
+// bits, and both formats' subnormals are normal numbers in bf16's exponent range).
+//   E4M3: bias 7, no infinity, S.1111.111 = NaN, subnormals m * 2^-9.
+//   E5M2: bias 15, S.11111.00 = infinity, S.11111.xx = NaN, subnormals m * 2^-16.
+__device__ __forceinline__ uint16_t fp8_to_bf16_bits(uint32_t b, bool e5m2) {
+    const uint32_t sign = (b & 0x80u) << 8;
+    const uint32_t mbits = e5m2 ? 2u : 3u, bias = e5m2 ? 15u : 7u, emax = e5m2 ? 31u : 15u;
+    const uint32_t e = (b & 0x7Fu) >> mbits, m = b & ((1u << mbits) - 1u);
+    uint32_t mag;
+    if (e == 0u) {
+        mag = __builtin_bit_cast(uint32_t, (float)m * (e5m2 ? 0x1p-16f : 0x1p-9f)) >> 16;
+    } else if (e == emax && (e5m2 || m == 7u)) {
+        mag = (e5m2 && m == 0u) ? 0x7F80u : 0x7FC0u;
+    } else {
+        mag = ((e + 127u - bias) << 7) | (m << (7u - mbits));
+    }
+    return (uint16_t)(sign | mag);
+}
 
 // bf16 bits -> fp32 (exact).
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }

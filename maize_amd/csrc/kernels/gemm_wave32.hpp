@@ -7,6 +7,8 @@
 // when a shape or pointer does not meet the tiled kernels' 16-byte rules.
 // Mirrors the reference's per-warp fragment loop (sync_mma_from_smem,
 // crates/maize_tile/src/gemm/mod.rs:18-33) without the shared-memory ring.
+// 8-bit operands (E4M3, E5M2) are widened to bf16 as they are loaded -- exactly, bf16 holds every
+// value of both formats -- and multiplied by the bf16 MFMA; their 16-bit C is bf16.
 //
 // MFMA 32x32x16 operand maps (lane l, 0..63):
 //   A operand: row  = l % 32, k = 8*(l/32) + e, e = 0..7
@@ -37,6 +39,9 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
     const uint16_t* __restrict__ A = p.a + bz * p.stride_a;
     const uint16_t* __restrict__ B = p.b + bz * p.stride_b;
     const bool f32_out = p.epi & EPI_F32, scaled = p.epi & EPI_SCALE, half_io = p.epi & EPI_F16;
+    const bool e5m2 = p.epi & EPI_E5M2, f8 = p.epi & (EPI_E4M3 | EPI_E5M2);
+    const uint8_t* __restrict__ A8 = (const uint8_t*)p.a + bz * p.stride_a;
+    const uint8_t* __restrict__ B8 = (const uint8_t*)p.b + bz * p.stride_b;
     uint16_t* __restrict__ C = p.c + bz * p.stride_c * (f32_out ? 2u : 1u);   // strides count elements of C
     float* __restrict__ Cf = (float*)C;
 
@@ -54,8 +59,16 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
             const uint32_t k = k0 + kg * 8u + e;
             uint16_t av = 0, bv = 0;
             if (k < K) {
-                if (am < M) av = A[(uint64_t)am * lda + k];
-                if (bn < N) bv = nt ? B[(uint64_t)bn * ldb + k] : B[(uint64_t)k * ldb + bn];
+                if (f8) {
+                    uint32_t a8 = 0, b8 = 0;
+                    if (am < M) a8 = A8[(uint64_t)am * lda + k];
+                    if (bn < N) b8 = nt ? B8[(uint64_t)bn * ldb + k] : B8[(uint64_t)k * ldb + bn];
+                    av = fp8_to_bf16_bits(a8, e5m2);
+                    bv = fp8_to_bf16_bits(b8, e5m2);
+                } else {
+                    if (am < M) av = A[(uint64_t)am * lda + k];
+                    if (bn < N) bv = nt ? B[(uint64_t)bn * ldb + k] : B[(uint64_t)k * ldb + bn];
+                }
             }
             fa[e] = bf16_from_bits(av);
             fb[e] = bf16_from_bits(bv);

@@ -36,6 +36,12 @@ MAIZE_MAP uint32_t kc_frag_offset(uint32_t row_base, uint32_t kk, uint32_t lane)
     return kc_offset(row_base + (lane & 31u), 2u * kk + (lane >> 5));
 }
 
+// Fragment read of MFMA 32x32x64 on 8-bit elements (the same tile: 128 elements per row): lane l
+// holds row base + l%32 and the 32 bytes k = 64 kh + 32 (l/32) + 0..31, read as two chunks (c01 = 0, 1).
+MAIZE_MAP uint32_t kc_frag8_offset(uint32_t row_base, uint32_t kh, uint32_t c01, uint32_t lane) {
+    return kc_offset(row_base + (lane & 31u), 4u * kh + 2u * (lane >> 5) + c01);
+}
+
 // ---- K x N operand tile of the macro-tile kernel (row-major B): 64 rows of 512 B ---------------------
 // Piece p (2 rows): lane l lands at row 2p + l/32, position l%32.  64-byte granules are XOR-ed with row%4.
 MAIZE_MAP uint32_t kn_swizzle(uint32_t row) { return (row & 3u) << 2; }

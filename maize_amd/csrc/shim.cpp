@@ -294,10 +294,10 @@ int32_t maize_hip_gemm_ex_validate(const maize_gemm_ex_desc_t* x) {
     if (!d->a.ptr || !d->b.ptr || !d->c.ptr) return fail(MAIZE_ERR_NULL, "gemm: NULL matrix pointer");
     if (x->out_type != MAIZE_OUT_BF16 && x->out_type != MAIZE_OUT_F32)
         return fail(MAIZE_ERR_ARG, "gemm: unknown output type %u", x->out_type);
-    if (x->in_type != MAIZE_IN_BF16 && x->in_type != MAIZE_IN_F16)
-        return fail(MAIZE_ERR_ARG, "gemm: unknown operand type %u", x->in_type);
+    if (x->in_type > MAIZE_IN_E5M2) return fail(MAIZE_ERR_ARG, "gemm: unknown operand type %u", x->in_type);
+    const bool in8 = x->in_type == MAIZE_IN_E4M3 || x->in_type == MAIZE_IN_E5M2;
     if (x->reserved) return fail(MAIZE_ERR_ARG, "gemm: reserved field must be 0");
-    if (((uintptr_t)d->a.ptr | (uintptr_t)d->b.ptr) & 1u || (uintptr_t)d->c.ptr & (x->out_type == MAIZE_OUT_F32 ? 3u : 1u))
+    if (((uintptr_t)d->a.ptr | (uintptr_t)d->b.ptr) & (in8 ? 0u : 1u) || (uintptr_t)d->c.ptr & (x->out_type == MAIZE_OUT_F32 ? 3u : 1u))
         return fail(MAIZE_ERR_ALIGN, "gemm: matrix pointers must be aligned to their element size");
     if ((x->lda && x->lda < d->a.ncols) || (x->ldb && x->ldb < d->b.ncols) || (x->ldc && x->ldc < d->c.ncols))
         return fail(MAIZE_ERR_SHAPE, "gemm: a leading dimension is smaller than the row it strides (lda=%u ldb=%u ldc=%u)",
@@ -419,7 +419,7 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
     args.lda = x->lda; args.ldb = x->ldb; args.ldc = x->ldc;
     args.alpha = x->alpha; args.beta = x->beta;
     args.epi = (x->out_type == MAIZE_OUT_F32 ? 1u : 0u) | ((x->alpha != 1.0f || x->beta != 0.0f) ? 2u : 0u) |
-               (x->in_type == MAIZE_IN_F16 ? 4u : 0u);
+               (x->in_type == MAIZE_IN_F16 ? 4u : 0u) | (x->in_type == MAIZE_IN_E4M3 ? 8u : 0u) | (x->in_type == MAIZE_IN_E5M2 ? 16u : 0u);
     maize::LaunchDims ld;
     memset(&ld, 0, sizeof ld);
     if (!ki.plan(*x, (uint32_t)ctx->prop.multiProcessorCount, &ld))

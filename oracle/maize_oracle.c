@@ -93,6 +93,53 @@ uint16_t mzo_f16_from_f64(double x) {
     return (uint16_t)(sign | (uint16_t)(be << 10) | mant);
 }
 
+/* ---- OCP 8-bit floats: E4M3 (bias 7, no infinity, S.1111.111 = NaN, max 448) and E5M2 (bias 15,
+ * IEEE-like: S.11111.00 = infinity, other S.11111.xx = NaN, max 57344).  The operand types of the
+ * 8-bit entries of the reference's MMA catalogue (crates/maize_tile/src/mma/sm89.rs). -------------- */
+
+float mzo_fp8_to_f32(uint8_t b, int elem) {
+    const int sign = b >> 7;
+    double v;
+    if (elem == MZO_ELEM_E5M2) {
+        const int e = (b >> 2) & 0x1F, m = b & 3;
+        if (e == 0) v = ldexp((double)m, -16);
+        else if (e == 31) v = m ? NAN : INFINITY;
+        else v = ldexp(1.0 + (double)m / 4.0, e - 15);
+    } else {
+        const int e = (b >> 3) & 0xF, m = b & 7;
+        if (e == 0) v = ldexp((double)m, -9);
+        else if (e == 15 && m == 7) v = NAN;
+        else v = ldexp(1.0 + (double)m / 8.0, e - 7);
+    }
+    return (float)(sign ? -v : v);
+}
+
+/* One RNE rounding from double; magnitudes that round past the largest finite value saturate to
+ * it (the OCP "satfinite" conversion), infinities too for E4M3 (which has none); NaN stays NaN. */
+uint8_t mzo_fp8_from_f64(double x, int elem) {
+    const int mbits = elem == MZO_ELEM_E5M2 ? 2 : 3, bias = elem == MZO_ELEM_E5M2 ? 15 : 7;
+    const double maxv = elem == MZO_ELEM_E5M2 ? 57344.0 : 448.0;
+    const uint8_t sign = signbit(x) ? 0x80u : 0u;
+    if (isnan(x)) return (uint8_t)(sign | (elem == MZO_ELEM_E5M2 ? 0x7Eu : 0x7Fu));
+    if (isinf(x) && elem == MZO_ELEM_E5M2) return (uint8_t)(sign | 0x7Cu);
+    if (x == 0.0) return sign;
+    int e;
+    (void)frexp(x, &e);
+    int ex = e - 1;
+    if (ex < 1 - bias) ex = 1 - bias;                          /* subnormals share the quantum of the smallest normal binade */
+    const int q = ex - mbits;
+    const double r = isinf(x) ? INFINITY : fabs(nearbyint(ldexp(x, -q)));
+    if (r == 0.0) return sign;
+    double v = isinf(x) ? INFINITY : ldexp(r, q);
+    if (v > maxv) v = maxv;
+    if (v < ldexp(1.0, 1 - bias)) return (uint8_t)(sign | (uint8_t)ldexp(v, bias - 1 + mbits));   /* subnormal: whole quanta */
+    int ev;
+    const double f = frexp(v, &ev);
+    const int be = ev - 1 + bias;
+    const uint8_t mant = (uint8_t)((f * 2.0 - 1.0) * (double)(1 << mbits));
+    return (uint8_t)(sign | (uint8_t)(be << mbits) | mant);
+}
+
 static float elem_to_f32(uint16_t h, int elem) { return elem == MZO_ELEM_F16 ? mzo_f16_to_f32(h) : mzo_bf16_to_f32(h); }
 static uint16_t elem_from_f64(double x, int elem) { return elem == MZO_ELEM_F16 ? mzo_f16_from_f64(x) : mzo_bf16_from_f64(x); }
 
@@ -149,26 +196,31 @@ static void* worker(void* p) {
 }
 
 /* Rows rows[0..nrows) (NULL: 0..nrows) of A (leading dimension k) as floats, compacted. */
-static float* widen_a(const uint16_t* a, const uint32_t* rows, uint32_t nrows, uint32_t k, int elem) {
+static int is_fp8(int elem) { return elem == MZO_ELEM_E4M3 || elem == MZO_ELEM_E5M2; }
+/* Element i of an operand array of the given element type (1-byte or 2-byte elements). */
+static float load_elem(const void* p, size_t i, int elem) {
+    return is_fp8(elem) ? mzo_fp8_to_f32(((const uint8_t*)p)[i], elem) : elem_to_f32(((const uint16_t*)p)[i], elem);
+}
+static float* widen_a(const void* a, const uint32_t* rows, uint32_t nrows, uint32_t k, int elem) {
     float* af = (float*)malloc(sizeof(float) * (size_t)(nrows ? nrows : 1) * k);
     if (!af) return NULL;
     for (uint32_t r = 0; r < nrows; ++r) {
-        const uint16_t* src = a + (size_t)(rows ? rows[r] : r) * k;
-        for (uint32_t kk = 0; kk < k; ++kk) af[(size_t)r * k + kk] = elem_to_f32(src[kk], elem);
+        const size_t src = (size_t)(rows ? rows[r] : r) * k;
+        for (uint32_t kk = 0; kk < k; ++kk) af[(size_t)r * k + kk] = load_elem(a, src + kk, elem);
     }
     return af;
 }
 
 /* Logical B (K x N) of one batch as floats. */
-static float* widen_b(const uint16_t* b, uint32_t n, uint32_t k, int layout, int elem) {
+static float* widen_b(const void* b, uint32_t n, uint32_t k, int layout, int elem) {
     float* bf = (float*)malloc(sizeof(float) * (size_t)n * k);
     if (!bf) return NULL;
     if (layout == MZO_LAYOUT_NN) {
-        for (size_t i = 0; i < (size_t)n * k; ++i) bf[i] = elem_to_f32(b[i], elem);
+        for (size_t i = 0; i < (size_t)n * k; ++i) bf[i] = load_elem(b, i, elem);
     } else {
         for (uint32_t x = 0; x < n; ++x)
             for (uint32_t kk = 0; kk < k; ++kk)
-                bf[(size_t)kk * n + x] = elem_to_f32(b[(size_t)x * k + kk], elem);
+                bf[(size_t)kk * n + x] = load_elem(b, (size_t)x * k + kk, elem);
     }
     return bf;
 }
@@ -269,4 +321,67 @@ int mzo_ref_gemm_rows(const uint16_t* a, const uint16_t* b, uint32_t m,
                       uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
                       uint32_t nthreads) {
     return mzo_ref_gemm16_rows(a, b, m, n, k, layout, rows, nsel, c, c_f64, c_abs, nthreads, MZO_ELEM_BF16);
+}
+
+/* ---- 8-bit operands: the same arithmetic (exact products, fp64 sums in ascending k), C rounded once to bf16 ---- */
+
+int mzo_ref_gemm8(const uint8_t* a, const uint8_t* b, uint16_t* c,
+                  uint32_t m, uint32_t n, uint32_t k, int layout,
+                  uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                  uint64_t stride_c, double* c_f64, double* c_abs,
+                  uint32_t nthreads, int elem) {
+    if (!a || !b || !c || batch == 0) return -1;
+    if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
+    if (!is_fp8(elem)) return -1;
+    if (m == 0 || n == 0) return 0;
+    for (uint32_t bi = 0; bi < batch; ++bi) {
+        float* bf = widen_b(b + bi * stride_b, n, k, layout, elem);
+        float* af = widen_a(a + bi * stride_a, NULL, m, k, elem);
+        if (!bf || !af) { free(bf); free(af); return -1; }
+        job_t j;
+        memset(&j, 0, sizeof j);
+        j.af = af;
+        j.bf = bf;
+        j.n = n;
+        j.k = k;
+        j.elem = MZO_ELEM_BF16;
+        j.c = c + bi * stride_c;
+        j.ldc = n;
+        j.c_f64 = c_f64 ? c_f64 + (size_t)bi * m * n : NULL;
+        j.c_abs = c_abs ? c_abs + (size_t)bi * m * n : NULL;
+        run_rows(j, m, nthreads);
+        free(bf);
+        free(af);
+    }
+    return 0;
+}
+
+int mzo_ref_gemm8_rows(const uint8_t* a, const uint8_t* b, uint32_t m,
+                       uint32_t n, uint32_t k, int layout, const uint32_t* rows,
+                       uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
+                       uint32_t nthreads, int elem) {
+    if (!a || !b || !rows) return -1;
+    if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
+    if (!is_fp8(elem)) return -1;
+    for (uint32_t r = 0; r < nsel; ++r)
+        if (rows[r] >= m) return -1;
+    if (n == 0 || nsel == 0) return 0;
+    float* bf = widen_b(b, n, k, layout, elem);
+    float* af = widen_a(a, rows, nsel, k, elem);
+    if (!bf || !af) { free(bf); free(af); return -1; }
+    job_t j;
+    memset(&j, 0, sizeof j);
+    j.af = af;
+    j.bf = bf;
+    j.n = n;
+    j.k = k;
+    j.elem = MZO_ELEM_BF16;
+    j.c = c;
+    j.ldc = n;
+    j.c_f64 = c_f64;
+    j.c_abs = c_abs;
+    run_rows(j, nsel, nthreads);
+    free(bf);
+    free(af);
+    return 0;
 }

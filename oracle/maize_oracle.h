@@ -47,8 +47,15 @@ float    mzo_bf16_to_f32(uint16_t h);   /* exact */
 uint16_t mzo_f16_from_f64(double x);    /* one round-to-nearest-even, f64 -> half */
 float    mzo_f16_to_f32(uint16_t h);    /* exact */
 
-/* Element type of A, B and the rounded C of the *16 entry points below. */
-enum { MZO_ELEM_BF16 = 0, MZO_ELEM_F16 = 1 };
+/* Element type of A, B and the rounded C of the *16 entry points below (BF16, F16), and of A and B
+ * of the *8 entry points (E4M3, E5M2; their C is bf16). */
+enum { MZO_ELEM_BF16 = 0, MZO_ELEM_F16 = 1, MZO_ELEM_E4M3 = 2, MZO_ELEM_E5M2 = 3 };
+
+/* OCP 8-bit floats, the operand types of the 8-bit entries of the MMA catalogue
+ * (crates/maize_tile/src/mma/sm89.rs): E4M3 has no infinity and one NaN per sign (S.1111.111), E5M2 is
+ * IEEE-like.  Pinned by the formats' published extremes and by torch's float8 dtypes on the CPU. */
+float   mzo_fp8_to_f32(uint8_t bits, int elem);     /* exact */
+uint8_t mzo_fp8_from_f64(double x, int elem);       /* one RNE; past the largest finite value saturates to it */
 
 /* Ordinal map: bf16 encodings -> signed integers so that adjacent finite
  * values differ by 1 and +0/-0 both map to 0.  NaN encodings are not ordered. */
@@ -95,6 +102,18 @@ int mzo_ref_gemm16_rows(const uint16_t* a, const uint16_t* b, uint32_t m,
                         uint32_t n, uint32_t k, int layout, const uint32_t* rows,
                         uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
                         uint32_t nthreads, int elem);
+
+
+/* The same two functions for 8-bit operands (MZO_ELEM_E4M3 / MZO_ELEM_E5M2); C is bf16. */
+int mzo_ref_gemm8(const uint8_t* a, const uint8_t* b, uint16_t* c,
+                  uint32_t m, uint32_t n, uint32_t k, int layout,
+                  uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                  uint64_t stride_c, double* c_f64, double* c_abs,
+                  uint32_t nthreads, int elem);
+int mzo_ref_gemm8_rows(const uint8_t* a, const uint8_t* b, uint32_t m,
+                       uint32_t n, uint32_t k, int layout, const uint32_t* rows,
+                       uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
+                       uint32_t nthreads, int elem);
 
 #ifdef __cplusplus
 }

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmaize_oracle.so")
 
 NN, NT = 0, 1
-BF16, F16 = 0, 1          # element types (MZO_ELEM_*)
+BF16, F16, E4M3, E5M2 = 0, 1, 2, 3   # element types (MZO_ELEM_*); C of the 8-bit types is bf16
 _lib = None
 
 
@@ -46,6 +46,14 @@ def lib():
         L.mzo_f16_from_f64.argtypes = [C.c_double]
         L.mzo_f16_to_f32.restype = C.c_float
         L.mzo_f16_to_f32.argtypes = [C.c_uint16]
+        L.mzo_fp8_to_f32.restype = C.c_float
+        L.mzo_fp8_to_f32.argtypes = [C.c_uint8, C.c_int]
+        L.mzo_fp8_from_f64.restype = C.c_uint8
+        L.mzo_fp8_from_f64.argtypes = [C.c_double, C.c_int]
+        L.mzo_ref_gemm8.restype = C.c_int
+        L.mzo_ref_gemm8.argtypes = [vp, vp, vp, u32, u32, u32, C.c_int, u32, u64, u64, u64, vp, vp, u32, C.c_int]
+        L.mzo_ref_gemm8_rows.restype = C.c_int
+        L.mzo_ref_gemm8_rows.argtypes = [vp, vp, u32, u32, u32, C.c_int, vp, u32, vp, vp, vp, u32, C.c_int]
         _lib = L
     return _lib
 
@@ -58,11 +66,20 @@ def _p(a):
     return None if a is None else a.ctypes.data
 
 
+def is_fp8(elem):
+    return elem in (E4M3, E5M2)
+
+
+def operand_dtype(elem):
+    return np.uint8 if is_fp8(elem) else np.uint16
+
+
 def ref_gemm(a, b, m, n, k, layout=NN, batch=1, stride_a=None, stride_b=None, stride_c=None,
              want_f64=False, want_abs=False, nthreads=None, elem=BF16):
-    """C (uint16, batch*stride_c elements) and optionally the fp64 sums / |a||b| sums (batch x M x N)."""
-    a = np.ascontiguousarray(a, dtype=np.uint16).ravel()
-    b = np.ascontiguousarray(b, dtype=np.uint16).ravel()
+    """C (uint16, batch*stride_c elements) and optionally the fp64 sums / |a||b| sums (batch x M x N).
+    Operands are uint16 bit patterns (bf16, half) or uint8 ones (E4M3, E5M2: C is then bf16)."""
+    a = np.ascontiguousarray(a, dtype=operand_dtype(elem)).ravel()
+    b = np.ascontiguousarray(b, dtype=operand_dtype(elem)).ravel()
     sa = m * k if stride_a is None else stride_a
     sb = k * n if stride_b is None else stride_b
     sc = m * n if stride_c is None else stride_c
@@ -70,8 +87,8 @@ def ref_gemm(a, b, m, n, k, layout=NN, batch=1, stride_a=None, stride_b=None, st
     c = np.zeros((batch - 1) * sc + m * n, dtype=np.uint16)
     f64 = np.empty((batch, m, n), dtype=np.float64) if want_f64 else None
     ab = np.empty((batch, m, n), dtype=np.float64) if want_abs else None
-    rc = lib().mzo_ref_gemm16(_p(a), _p(b), _p(c), m, n, k, layout, batch, sa, sb, sc, _p(f64), _p(ab),
-                              nthreads or default_threads(), elem)
+    fn = lib().mzo_ref_gemm8 if is_fp8(elem) else lib().mzo_ref_gemm16
+    rc = fn(_p(a), _p(b), _p(c), m, n, k, layout, batch, sa, sb, sc, _p(f64), _p(ab), nthreads or default_threads(), elem)
     if rc != 0:
         raise ValueError("mzo_ref_gemm16 rejected its arguments")
     return c, f64, ab
@@ -79,15 +96,15 @@ def ref_gemm(a, b, m, n, k, layout=NN, batch=1, stride_a=None, stride_b=None, st
 
 def ref_gemm_rows(a, b, m, n, k, rows, layout=NN, want_abs=True, nthreads=None, elem=BF16):
     """Rows ``rows`` of C = A.B for one batch: (bits nsel x N, f64 nsel x N, abs nsel x N)."""
-    a = np.ascontiguousarray(a, dtype=np.uint16).ravel()
-    b = np.ascontiguousarray(b, dtype=np.uint16).ravel()
+    a = np.ascontiguousarray(a, dtype=operand_dtype(elem)).ravel()
+    b = np.ascontiguousarray(b, dtype=operand_dtype(elem)).ravel()
     rows = np.ascontiguousarray(rows, dtype=np.uint32)
     nsel = rows.size
     c = np.zeros((nsel, n), dtype=np.uint16)
     f64 = np.empty((nsel, n), dtype=np.float64)
     ab = np.empty((nsel, n), dtype=np.float64) if want_abs else None
-    rc = lib().mzo_ref_gemm16_rows(_p(a), _p(b), m, n, k, layout, _p(rows), nsel, _p(c), _p(f64), _p(ab),
-                                   nthreads or default_threads(), elem)
+    fn = lib().mzo_ref_gemm8_rows if is_fp8(elem) else lib().mzo_ref_gemm16_rows
+    rc = fn(_p(a), _p(b), m, n, k, layout, _p(rows), nsel, _p(c), _p(f64), _p(ab), nthreads or default_threads(), elem)
     if rc != 0:
         raise ValueError("mzo_ref_gemm_rows rejected its arguments")
     return c, f64, ab
@@ -113,6 +130,35 @@ def bf16_bits_to_f64(bits, elem=BF16):
     return (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
 
 
+def fp8_bits_from_f64(x, elem):
+    """Round an array of doubles to E4M3 / E5M2 bit patterns: one RNE, saturating past the largest finite
+    value -- mzo_fp8_from_f64's rule, vectorised as a nearest-value search over the format's (at most 127)
+    finite magnitudes with ties going to the even code (tests pin it against the C function)."""
+    x = np.asarray(x, dtype=np.float64)
+    codes = np.arange(128, dtype=np.uint8)
+    vals = fp8_bits_to_f64(codes, elem)
+    vals = vals[np.isfinite(vals)]                       # codes 0 .. len-1, ascending
+    mid = (vals[:-1] + vals[1:]) / 2.0
+    ax = np.abs(x)
+    idx = np.searchsorted(mid, ax, side="left")
+    tie = (idx < mid.size) & (ax == mid[np.minimum(idx, mid.size - 1)])
+    idx = idx + (tie & (idx % 2 == 1))
+    out = idx.astype(np.uint8)
+    if elem == E5M2:
+        out = np.where(np.isinf(x), 0x7C, out).astype(np.uint8)
+    out = np.where(np.isnan(x), 0x7E if elem == E5M2 else 0x7F, out).astype(np.uint8)
+    return (out | np.where(np.signbit(x), 0x80, 0).astype(np.uint8)).astype(np.uint8)
+
+
+def fp8_bits_to_f64(bits, elem):
+    key = "_t%d" % elem
+    table = getattr(fp8_bits_to_f64, key, None)
+    if table is None:
+        table = np.array([lib().mzo_fp8_to_f32(h, elem) for h in range(256)], dtype=np.float64)
+        setattr(fp8_bits_to_f64, key, table)
+    return table[np.asarray(bits, dtype=np.uint8)]
+
+
 def ref_gemm_ex(a, b, m, n, k, layout=NN, lda=None, ldb=None, alpha=1.0, beta=0.0, c_old=None, out_f32=False,
                 nthreads=None, elem=BF16):
     """The extended product for one batch member, on operand views with leading dimensions:
@@ -125,10 +171,13 @@ def ref_gemm_ex(a, b, m, n, k, layout=NN, lda=None, ldb=None, alpha=1.0, beta=0.
     brows, bcols = (k, n) if layout == NN else (n, k)
     lda = k if lda is None else lda
     ldb = bcols if ldb is None else ldb
-    a = np.asarray(a, dtype=np.uint16).ravel()
-    b = np.asarray(b, dtype=np.uint16).ravel()
-    av = np.lib.stride_tricks.as_strided(a, shape=(m, k), strides=(2 * lda, 2))
-    bv = np.lib.stride_tricks.as_strided(b, shape=(brows, bcols), strides=(2 * ldb, 2))
+    dt = operand_dtype(elem)
+    isz = np.dtype(dt).itemsize
+    celem = BF16 if is_fp8(elem) else elem                      # element type of a 16-bit C
+    a = np.asarray(a, dtype=dt).ravel()
+    b = np.asarray(b, dtype=dt).ravel()
+    av = np.lib.stride_tricks.as_strided(a, shape=(m, k), strides=(isz * lda, isz))
+    bv = np.lib.stride_tricks.as_strided(b, shape=(brows, bcols), strides=(isz * ldb, isz))
     assert a.size >= (m - 1) * lda + k and b.size >= (brows - 1) * ldb + bcols
     _, f64, ab = ref_gemm(np.ascontiguousarray(av), np.ascontiguousarray(bv), m, n, k, layout=layout, want_f64=True,
                           want_abs=True, nthreads=nthreads, elem=elem)
@@ -138,10 +187,10 @@ def ref_gemm_ex(a, b, m, n, k, layout=NN, lda=None, ldb=None, alpha=1.0, beta=0.
     scale = abs(alpha) * ab[0]
     if beta != 0.0:
         old = np.asarray(c_old).reshape(m, n)
-        old64 = bf16_bits_to_f64(old, elem) if old.dtype == np.uint16 else old.astype(np.float64)
+        old64 = bf16_bits_to_f64(old, celem) if old.dtype == np.uint16 else old.astype(np.float64)
         val = val + beta * old64
         scale = scale + abs(beta) * np.abs(old64)
-    out = val.astype(np.float32) if out_f32 else bf16_bits_from_f64(val, elem)
+    out = val.astype(np.float32) if out_f32 else bf16_bits_from_f64(val, celem)
     return out, val, scale
 
 
@@ -165,7 +214,16 @@ def floor_coeff(k):
     return (k / 16.0 + 2.0) * 2.0 ** -24
 
 
-def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16):
+def floor_coeff_f8(k):
+    """The same floor for the 8-bit matrix instruction (v_mfma_f32_32x32x64_f8f6f4).  Its dot-product unit
+    aligns the 64 products of one instruction to the largest of them and drops what lies more than 13 binades
+    below it (pinned by a probe test on the device), so the absolute error is no longer a few fp32 roundings:
+    on uniform or normal operands it was measured at up to 2^-16.3 * sum|a||b| (mean 2^-21.7); granted: 2^-15,
+    plus one fp32 rounding per 64-deep step."""
+    return 2.0 ** -15 + (k / 64.0 + 2.0) * 2.0 ** -24
+
+
+def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16, coeff=None):
     """Compare device output with the oracle.
 
     An element passes if it is within 1 bf16 ULP (ordinal distance) of the
@@ -174,6 +232,7 @@ def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16):
     absolute error against the fp64 sum is at most floor_coeff(K) * sum|a||b|
     plus half a bf16 ULP of the returned value.  Both counts are reported.
     With elem=F16 the same bar in IEEE half: 1 half ULP, half a half ULP (2^-11 relative).
+    ``coeff`` replaces floor_coeff(K) (the 8-bit matrix instruction: floor_coeff_f8).
     """
     got = np.asarray(got_bits, dtype=np.uint16).ravel()
     ref = np.asarray(ref_bits, dtype=np.uint16).ravel()
@@ -191,7 +250,7 @@ def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16):
     with np.errstate(invalid="ignore", over="ignore"):
         err = np.abs(gotf - f64)
         half_ulp = np.abs(gotf) * (2.0 ** -11 if elem == F16 else 2.0 ** -8)
-        floor = floor_coeff(k) * ab + half_ulp
+        floor = (floor_coeff(k) if coeff is None else coeff) * ab + half_ulp
         strict_bad = ulp > 1
         bad = strict_bad & ~(err <= floor)
         rel = np.where(ab > 0, err / np.where(ab > 0, ab, 1.0), 0.0)
@@ -202,7 +261,7 @@ def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16):
         "n_gt1ulp": int(strict_bad.sum()),
         "n_fail": int(bad.sum()),
         "max_err_over_abs": float(rel.max()) if rel.size else 0.0,
-        "floor_coeff": floor_coeff(k),
+        "floor_coeff": floor_coeff(k) if coeff is None else coeff,
         "worst_index": worst,
         "first_fail": int(np.argmax(bad)) if bad.any() else -1,
     }

@@ -70,6 +70,21 @@ int main() {
                 }
                 CHECK(passes_conflict_free(off, 16), "kc fragment read base %u kk %u has bank conflicts", base, kk);
             }
+        // the 8-bit kernel's reads of the same tile: (kh, c01, l/32) name each of the 8 chunks of a row once
+        for (uint32_t base = 0; base < 256; base += 32) {
+            std::set<uint32_t> seen8;
+            for (uint32_t kh = 0; kh < 2; ++kh)
+                for (uint32_t c01 = 0; c01 < 2; ++c01) {
+                    uint32_t off[64];
+                    for (uint32_t lane = 0; lane < 64; ++lane) {
+                        off[lane] = kc_frag8_offset(base, kh, c01, lane);
+                        CHECK(off[lane] == kc_offset(base + lane % 32, 4 * kh + 2 * (lane / 32) + c01), "kc 8-bit fragment lane map");
+                        seen8.insert(off[lane]);
+                    }
+                    CHECK(passes_conflict_free(off, 16), "kc 8-bit fragment read base %u kh %u c01 %u has bank conflicts", base, kh, c01);
+                }
+            CHECK(seen8.size() == 32 * 8, "kc 8-bit fragment reads do not cover 32 rows x 8 chunks");
+        }
         std::printf("ok  K-contiguous tile: fragment reads are bank-conflict free\n");
     }
     // ---- K x N tile

@@ -54,7 +54,13 @@ def test_every_registry_entry_has_its_device_kernel(kernels):
 
 def test_matrix_instruction_per_kernel(kernels):
     for name, ins in kernels.items():
-        if "_mt256_" in name:
+        if name.startswith(("maize_gemm_e4m3_", "maize_gemm_e5m2_")):
+            # 8-bit operands: the 64-deep instruction, format code in cbsz / blgp (E4M3 = 0: not printed)
+            f8 = [i for i in ins if i.startswith("v_mfma_f32_32x32x64_f8f6f4")]
+            assert len(f8) >= 64 and count(ins, "v_mfma_f32_32x32x16") == 0, name   # two unrolled K steps of 128
+            assert all(("cbsz:1" in i and "blgp:1" in i) == name.startswith("maize_gemm_e5m2_") for i in f8), name
+            assert not any("cbsz" in i or "blgp" in i for i in f8) or name.startswith("maize_gemm_e5m2_"), name
+        elif "_mt256_" in name:
             want = "v_mfma_f32_32x32x16_f16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_32x32x16_bf16"
             other = "v_mfma_f32_32x32x16_bf16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_32x32x16_f16"
             assert count(ins, want) >= 128 and count(ins, other) == 0, name       # two fully unrolled K steps of 64
@@ -69,7 +75,8 @@ def test_data_movement_the_design_rests_on(kernels):
         if "_mt256_" in name or name == "maize_gemm_bf16_skinny_nn":
             lds_dma = [i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]
             assert len(lds_dma) >= 16, f"{name}: operands must reach LDS by 128-bit direct-to-LDS loads"
-            assert count(ins, "ds_write_b128") == 0 or "_gen" in name or "_splitk" in name, name   # no register round trip for operands
+            fp32_staging = "_gen" in name or "_splitk" in name or name.startswith(("maize_gemm_e4m3_", "maize_gemm_e5m2_"))
+            assert count(ins, "ds_write_b128") == 0 or fp32_staging, name   # no register round trip for operands
         if "_mt256_nn" in name or name == "maize_gemm_bf16_skinny_nn":
             assert count(ins, "ds_read_b64_tr_b16") >= 8, f"{name}: a row-major K x N B is read with transposing reads"
         if "_mt256_nt" in name:

@@ -1,0 +1,200 @@
+"""GPU parity of the product on 8-bit floating-point operands (OCP E4M3 / E5M2, the operand types of
+the reference's Sm89MmaF8F32_* catalogue entries, crates/maize_tile/src/mma/sm89.rs:13-45), through
+maize_hip_gemm_bf16_ex, against the oracle's 8-bit restatement (mzo_ref_gemm8) on the same bytes.
+
+Tolerance.  The per-wave kernel widens the operands to bf16 (exactly) and keeps the bar of the bf16
+product: bf16 C within 1 bf16 ULP of the oracle's bits or, where the result nearly cancels, |got - exact|
+<= (K/16 + 2) * 2^-24 * scale + half a bf16 ULP; fp32 C within (K/16 + 4) * 2^-24 * scale.  The macro-tile
+kernels use v_mfma_f32_32x32x64_f8f6f4, whose dot-product unit drops products more than 13 binades below
+the largest of the 64 it adds (test_what_the_8bit_matrix_instruction_keeps pins that): their floor is
+(2^-15 + (K/64 + 2) * 2^-24) * scale (measured on these operands: at most 2^-16.3 * scale), the 1-ULP bar
+is unchanged.  Closed forms whose products stay within 13 binades of each other are bit-exact."""
+import sys
+
+import numpy as np
+import pytest
+
+import maize_amd as mz
+
+pytestmark = pytest.mark.gpu
+
+FMT = {"e4m3": (mz.IN_E4M3, 2), "e5m2": (mz.IN_E5M2, 3)}      # name -> (in_type, oracle element code)
+
+
+def _say(msg):
+    print(f"[gemm_f8] {msg}", file=sys.stderr, flush=True)
+
+
+def f8_uniform(oracle, count, seed, elem, scale=1.0):
+    """uniform[-scale, scale) rounded to the 8-bit format."""
+    x = (np.random.default_rng(seed).random(count) * 2.0 - 1.0) * scale
+    return oracle.fp8_bits_from_f64(x, elem)
+
+
+def launch(ctx, a, b, c0, m, n, k, layout, fmt, lda, ldb, ldc, alpha=1.0, beta=0.0, out_f32=False, kernel=None, batch=1,
+           strides=(0, 0, 0)):
+    brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+    da, db, dc = ctx.upload(a), ctx.upload(b), ctx.upload(c0)
+    try:
+        x = mz.gemm_ex_desc(mz.Matrix(da, m, k, elem_bytes=1), mz.Matrix(db, brows, bcols, elem_bytes=1), mz.Matrix(dc, m, n),
+                            layout=layout, lda=0 if lda == k else lda, ldb=0 if ldb == bcols else ldb, ldc=0 if ldc == n else ldc,
+                            out_type=mz.OUT_F32 if out_f32 else mz.OUT_SAME, alpha=alpha, beta=beta, in_type=FMT[fmt][0],
+                            batch=batch, stride_a=strides[0], stride_b=strides[1], stride_c=strides[2])
+        took = mz.gemm_plan(x, kernel=kernel, compute_units=ctx.info()["compute_units"])["kernel"]
+        ctx.gemm_bf16(x, kernel=kernel)
+        ctx.sync()
+        got = dc.download(np.float32 if out_f32 else np.uint16)
+    finally:
+        da.free(); db.free(); dc.free()
+    return got, took
+
+
+def run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NT, fmt="e4m3", lda=None, ldb=None, ldc=None, alpha=1.0, beta=0.0,
+           out_f32=False, kernel=None, seed=1, label=""):
+    elem = FMT[fmt][1]
+    brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+    lda = k if lda is None else lda
+    ldb = bcols if ldb is None else ldb
+    ldc = n if ldc is None else ldc
+    a = f8_uniform(oracle, m * lda, 100 + seed, elem)
+    b = f8_uniform(oracle, brows * ldb, 200 + seed, elem)
+    if out_f32:
+        c0 = (np.random.default_rng(seed).standard_normal(m * ldc) * 2).astype(np.float32)
+    else:
+        c0 = mz.gen.uniform_bf16(m * ldc, 300 + seed)
+    got, took = launch(ctx, a, b, c0, m, n, k, layout, fmt, lda, ldb, ldc, alpha, beta, out_f32, kernel)
+    _say(f"{label} {fmt} M={m} N={n} K={k} ld=({lda},{ldb},{ldc}) alpha={alpha} beta={beta} f32={out_f32} -> {took}")
+    gv, ov = got.reshape(m, ldc), c0.reshape(m, ldc)
+    assert np.array_equal(gv[:, n:].view(np.uint8), ov[:, n:].view(np.uint8)), f"{label}: wrote into C's row padding"
+    ref, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, layout=layout, lda=lda, ldb=ldb, alpha=alpha, beta=beta,
+                                         c_old=None if beta == 0.0 else ov[:, :n].copy(), out_f32=out_f32, elem=elem)
+    g = gv[:, :n]
+    f8_unit = "mt256" in took
+    if out_f32:
+        err = np.abs(g.astype(np.float64) - val)
+        tol = ((oracle.floor_coeff_f8(k) + 2.0 ** -23) if f8_unit else (k / 16.0 + 4.0) * 2.0 ** -24) * scale + 1e-45
+        bad = ~(err <= tol)
+        assert not bad.any(), f"{label}: {int(bad.sum())} of {bad.size} fp32 elements out of tolerance, worst {float((err / tol).max()):.2f}x"
+    else:
+        s = oracle.compare(g, ref, val, scale, k, coeff=oracle.floor_coeff_f8(k) if f8_unit else None)
+        assert s["n_fail"] == 0, f"{label}: {s}"
+        _say(f"   max_ulp {s['max_ulp']} n_gt1ulp {s['n_gt1ulp']} of {s['n']}")
+    return took
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+def test_any_shape_kernel_on_8bit_operands(ctx, oracle, fmt, layout):
+    for (m, n, k) in ((33, 17, 65), (64, 64, 48), (100, 200, 72)):
+        bcols = n if layout == mz.LAYOUT_NN else k
+        for kw in (dict(), dict(lda=k + 3, ldb=bcols + 5, ldc=n + 7), dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5)):
+            took = run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, kernel="maize_gemm_bf16_wave32", label="wave32", **kw)
+            assert took == "maize_gemm_bf16_wave32"
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+def test_every_encoding_reaches_the_matrix_unit_unchanged(ctx, oracle, fmt):
+    """A = every finite encoding on a diagonal-like routing: C = A . I^T returns each of the 256 values exactly
+    (as bf16, which holds every 8-bit float), through the per-wave kernel and through the macro-tile kernel."""
+    elem = FMT[fmt][1]
+    vals = oracle.fp8_bits_to_f64(np.arange(256, dtype=np.uint8), elem)
+    finite = np.arange(256, dtype=np.uint8)[np.isfinite(vals)]
+    m, k = 256, 256
+    a = np.zeros((m, k), dtype=np.uint8)
+    a[:, :] = np.resize(finite, m * k).reshape(m, k)
+    one = oracle.fp8_bits_from_f64(np.array([1.0]), elem)[0]
+    eye = np.zeros((k, k), dtype=np.uint8)
+    eye[np.arange(k), np.arange(k)] = one
+    want = oracle.bf16_bits_from_f64(oracle.fp8_bits_to_f64(a, elem))
+    for kernel in ("maize_gemm_bf16_wave32", f"maize_gemm_{fmt}_mt256_nt"):
+        got, took = launch(ctx, a.ravel(), eye.ravel(), np.zeros(m * k, np.uint16), m, k, k, mz.LAYOUT_NT, fmt, k, k, k, kernel=kernel)
+        assert took == kernel
+        # -0 * 1 + 0 = +0 in the accumulator: compare values, not the sign of zero
+        assert np.array_equal(oracle.bf16_bits_to_f64(got), oracle.bf16_bits_to_f64(want.ravel())), kernel
+
+
+def test_what_the_8bit_matrix_instruction_keeps(ctx, oracle):
+    """One product of 1 * 1 and one of 2^-s in the same 64-deep group (E5M2, fp32 C): the small product is added
+    exactly while it is at most 13 binades below the large one and dropped entirely from 14 on.  The tolerance
+    of the macro-tile kernels rests on this."""
+    fmt, elem = "e5m2", FMT["e5m2"][1]
+    m = n = 256
+    k = 64
+    enc = lambda x: oracle.fp8_bits_from_f64(np.array([x]), elem)[0]
+    a = np.zeros((m, k), np.uint8)
+    b = np.zeros((n, k), np.uint8)
+    a[:, 0] = enc(1.0)
+    b[:, 0] = enc(1.0)
+    for r in range(m):
+        a[r, 1] = enc(2.0 ** -(r % 16))
+    for c in range(n):
+        b[c, 1] = enc(2.0 ** -(c % 16))
+    got, _ = launch(ctx, a.ravel(), b.ravel(), np.zeros(m * n, np.float32), m, n, k, mz.LAYOUT_NT, fmt, k, k, n, out_f32=True,
+                    kernel="maize_gemm_e5m2_mt256_nt")
+    g = got.reshape(m, n)
+    for r in range(16):
+        for c in range(16):
+            s = r + c
+            want = np.float32(1.0 + 2.0 ** -s) if s <= 13 else np.float32(1.0)
+            if s <= 23:                       # beyond, 1 + 2^-s rounds to 1 in fp32 anyway
+                assert g[r, c] == want, (s, g[r, c])
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (256, 256, 256), (512, 768, 384), (300, 520, 144), (1000, 264, 1040), (128, 2048, 16)])
+def test_macro_tile_kernel(ctx, oracle, fmt, shape):
+    m, n, k = shape
+    name = f"maize_gemm_{fmt}_mt256_nt"
+    assert run_f8(ctx, oracle, m, n, k, fmt=fmt, kernel=name, label="mt256f8") == name
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+def test_macro_tile_kernel_all_knobs(ctx, oracle, fmt):
+    m, n, k = 520, 776, 400
+    name = f"maize_gemm_{fmt}_mt256_nt"
+    for kw in (dict(lda=416, ldb=432, ldc=784), dict(alpha=0.5), dict(alpha=-1.25, beta=0.75), dict(out_f32=True),
+               dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(alpha=0.0, beta=1.0)):
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 knobs", **kw) == name
+
+
+def test_dispatch_of_8bit_products(ctx):
+    def pick(m, n, k, layout, in_type, **kw):
+        brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+        x = mz.gemm_ex_desc(mz.GlobalMatrix(0x10000, m, k), mz.GlobalMatrix(0x10000, brows, bcols), mz.GlobalMatrix(0x10000, m, n),
+                            layout=layout, in_type=in_type, **kw)
+        return mz.gemm_plan(x, compute_units=256)["kernel"]
+    assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt"
+    assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nt"
+    assert pick(4096, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_bf16_wave32"      # row-major B: not K-contiguous
+    assert pick(4096, 4096, 4104, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_bf16_wave32"      # K % 16
+    assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3, lda=4104) == "maize_gemm_bf16_wave32"
+    assert pick(64, 64, 64, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_bf16_wave32"
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+def test_full_size_sampled_rows_and_batches(ctx, oracle, fmt):
+    """4096^3 on sampled rows (both sides of every tile boundary), and a batched launch equal to its singles."""
+    elem = FMT[fmt][1]
+    m = n = k = 4096
+    a = f8_uniform(oracle, m * k, 11, elem)
+    b = f8_uniform(oracle, n * k, 12, elem)
+    got, took = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n)
+    assert took == f"maize_gemm_{fmt}_mt256_nt"
+    rows = np.unique(np.concatenate([np.arange(0, m, 256), np.arange(255, m, 256), np.array([1, 127, 128, 2049, 4094])])).astype(np.uint32)
+    ref, val, ab = oracle.ref_gemm_rows(a, b, m, n, k, rows, layout=oracle.NT, elem=elem)
+    s = oracle.compare(got.reshape(m, n)[rows], ref, val, ab, k, coeff=oracle.floor_coeff_f8(k))
+    _say(f"{fmt} 4096^3 sampled rows: {s}")
+    assert s["n_fail"] == 0, s
+    # batched: 3 x (384 x 512 x 640), padded strides
+    bm, bn, bk, batch = 384, 512, 640, 3
+    sa, sb, sc = bm * bk + 64, bn * bk + 128, bm * bn + 16
+    ab_ = f8_uniform(oracle, batch * sa, 21, elem)
+    bb_ = f8_uniform(oracle, batch * sb, 22, elem)
+    dense, took = launch(ctx, ab_, bb_, np.zeros(batch * sc, np.uint16), bm, bn, bk, mz.LAYOUT_NT, fmt, bk, bk, bn, batch=batch,
+                         strides=(sa, sb, sc))
+    assert took == f"maize_gemm_{fmt}_mt256_nt"
+    for i in range(batch):
+        single, _ = launch(ctx, ab_[i * sa:i * sa + bm * bk], bb_[i * sb:i * sb + bn * bk], np.zeros(bm * bn, np.uint16), bm, bn, bk,
+                           mz.LAYOUT_NT, fmt, bk, bk, bn)
+        assert np.array_equal(single, dense[i * sc:i * sc + bm * bn]), i
+        assert not dense[i * sc + bm * bn:(i + 1) * sc].any(), "wrote between batch members"
