@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BF16 GEMM path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5] [--kernel NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5|f8] [--kernel NAME]
 
 A step is one launch of maize_hip_gemm_bf16 on synthetic, seeded inputs that are already
 resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s (wall clock around exactly K
@@ -21,6 +21,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each
 # scaled by what the same counter reads for a 256 MiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x
@@ -39,10 +40,15 @@ CONFIGS = {
                  label="bf16 GEMM 16x14336x4096 NN skinny, A~N(0,1), B~N(0,0.02)"),
     "cfg5": dict(m=2048, n=2048, k=2048, nt=0, batch=32, da=("uniform",), db=("uniform",), bound="mfma",
                  label="bf16 strided-batched GEMM 32 x 2048^3 NN, uniform[-1,1)"),
+    # Beside the five bf16 configurations: the same product on 8-bit operands (E4M3), both K-contiguous.
+    "f8": dict(m=4096, n=4096, k=4096, nt=1, batch=1, da=("uniform",), db=("uniform",), bound="mfma", in_type="e4m3",
+               label="E4M3 GEMM 4096x4096x4096 NT (bf16 C), uniform[-1,1) rounded to E4M3"),
 }
 
 
-def make(mz, dist, count, seed):
+def make(mz, dist, count, seed, in_type=None):
+    if in_type is not None:
+        return mz.gen.uniform_f8(count, seed, mz.IN_E4M3 if in_type == "e4m3" else mz.IN_E5M2)
     if dist[0] == "uniform":
         return mz.gen.uniform_bf16(count, seed)
     sigma = mz.gen.SIGMA_INV_SQRT_8192 if dist[1] == "inv_sqrt_k" else dist[1]
@@ -55,18 +61,20 @@ def cpu_baseline(cfg, a, b_storage, got, seconds_target=12.0):
     the reported baseline here; it is never on the measured GPU path."""
     from oracle import pyoracle
     m, n, k = cfg["m"], cfg["n"], cfg["k"]
+    elem = {None: pyoracle.BF16, "e4m3": pyoracle.E4M3, "e5m2": pyoracle.E5M2}[cfg.get("in_type")]
+    coeff = pyoracle.floor_coeff_f8(k) if cfg.get("in_type") else None
     threads = pyoracle.default_threads()
     probe_rows = min(m, 4)
     t0 = time.perf_counter()
     pyoracle.ref_gemm_rows(a[:m * k], b_storage[:k * n], m, n, k, np.arange(probe_rows, dtype=np.uint32),
-                           layout=cfg["nt"], want_abs=False, nthreads=1)
+                           layout=cfg["nt"], want_abs=False, nthreads=1, elem=elem)
     per_row = max((time.perf_counter() - t0) / probe_rows, 1e-6)
     rows = int(min(m, max(threads, seconds_target * threads / per_row)))
     rows = max(1, (rows // threads) * threads) if rows >= threads else rows
     sel = np.arange(rows, dtype=np.uint32)
     t0 = time.perf_counter()
     ref, f64, _ = pyoracle.ref_gemm_rows(a[:m * k], b_storage[:k * n], m, n, k, sel, layout=cfg["nt"], want_abs=False,
-                                         nthreads=threads)
+                                         nthreads=threads, elem=elem)
     dt = time.perf_counter() - t0
     flops = 2.0 * rows * n * k
     out = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
@@ -75,9 +83,9 @@ def cpu_baseline(cfg, a, b_storage, got, seconds_target=12.0):
     parity = None
     if got is not None:
         _, _, ab = pyoracle.ref_gemm_rows(a[:m * k], b_storage[:k * n], m, n, k, sel[:min(rows, 64)], layout=cfg["nt"],
-                                          nthreads=threads)
+                                          nthreads=threads, elem=elem)
         r = min(rows, 64)
-        parity = pyoracle.compare(got[:r * n], ref[:r], f64[:r], ab, k)
+        parity = pyoracle.compare(got[:r * n], ref[:r], f64[:r], ab, k, coeff=coeff)
         parity = {key: parity[key] for key in ("n", "max_ulp", "n_gt1ulp", "n_fail", "max_err_over_abs")}
     return out, parity
 
@@ -122,7 +130,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", default=None, choices=sorted(CONFIGS) + ["copy"],
-                    help="cfg1..cfg5: a benchmark configuration; copy: the 256 MiB copy used to scale HBM counters")
+                    help="cfg1..cfg5: a benchmark configuration; f8: 4096^3 on E4M3 operands; copy: the 256 MiB copy "
+                         "used to scale HBM counters")
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--others", action=argparse.BooleanOptionalAction, default=None,
@@ -170,11 +179,13 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
     args.config, args.steps, args.warmup, args.kernel, args.rotate, args.no_cpu = config, steps, warmup, force_kernel, rotate, not with_cpu
     cfg = CONFIGS[args.config]
     m, n, k, batch, nt = cfg["m"], cfg["n"], cfg["k"], cfg["batch"], cfg["nt"]
+    f8 = cfg.get("in_type")
+    esz = 1 if f8 else 2                                   # bytes per element of A and B
     flops = 2.0 * batch * m * n * k
-    alg_bytes = 2.0 * batch * (m * k + k * n + m * n)
+    alg_bytes = float(batch) * (esz * (m * k + k * n) + 2 * m * n)
 
-    a = make(mz, cfg["da"], batch * m * k, mz.gen.SEED_A)
-    b = make(mz, cfg["db"], batch * k * n, mz.gen.SEED_B)
+    a = make(mz, cfg["da"], batch * m * k, mz.gen.SEED_A, f8)
+    b = make(mz, cfg["db"], batch * k * n, mz.gen.SEED_B, f8)
     if nt:  # same logical B, stored N x K
         b = np.concatenate([b[i * k * n:(i + 1) * k * n].reshape(k, n).T.ravel() for i in range(batch)])
 
@@ -183,12 +194,16 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
     sets = []
     for _ in range(nsets):
         da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(2 * batch * m * n)
-        A = mz.Matrix(da, m, k)
-        B = mz.Matrix(db, n, k) if nt else mz.Matrix(db, k, n)
-        desc = mz.gemm_desc(A, B, mz.Matrix(dc, m, n), layout=nt, batch=batch, stride_a=m * k, stride_b=k * n,
-                            stride_c=m * n)
+        A = mz.Matrix(da, m, k, elem_bytes=esz)
+        B = mz.Matrix(db, n, k, elem_bytes=esz) if nt else mz.Matrix(db, k, n, elem_bytes=esz)
+        if f8:
+            desc = mz.gemm_ex_desc(A, B, mz.Matrix(dc, m, n), layout=nt, batch=batch, stride_a=m * k, stride_b=k * n,
+                                   stride_c=m * n, in_type=mz.IN_E4M3 if f8 == "e4m3" else mz.IN_E5M2)
+        else:
+            desc = mz.gemm_desc(A, B, mz.Matrix(dc, m, n), layout=nt, batch=batch, stride_a=m * k, stride_b=k * n,
+                                stride_c=m * n)
         sets.append((da, db, dc, desc))
-    kernel = args.kernel or ctx.gemm_select(sets[0][3])
+    kernel = args.kernel or mz.gemm_plan(sets[0][3], compute_units=info["compute_units"])["kernel"]
     stream = ctx.stream()
     ev0, ev1 = ctx.event(), ctx.event()
 
@@ -223,10 +238,11 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
     ms_per_step = wall * 1e3 / args.steps
     kern_ms = ev_ms / args.steps
     value = flops / (wall / args.steps) / 1e12
+    peak_flops = PEAK_FP8_TFLOPS if f8 else PEAK_BF16_TFLOPS
     if cfg["bound"] == "mfma":
         ach = flops / (kern_ms * 1e-3) / 1e12
-        roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None}
+        roof = {"bound": "mfma", "achieved": ach, "peak": peak_flops, "unit": "TFLOP/s",
+                "frac": ach / peak_flops, "traffic": None}
     else:
         ach = alg_bytes / (kern_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
@@ -242,14 +258,15 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
         cpu, parity = cpu_baseline(cfg, a, b, got)
 
     line = {
-        "metric": "bf16 GEMM TFLOP/s at 4096^3 on 1 MI355X" if args.config == "cfg1" else f"bf16 GEMM TFLOP/s, {args.config}",
+        "metric": "bf16 GEMM TFLOP/s at 4096^3 on 1 MI355X" if args.config == "cfg1"
+                  else "E4M3 GEMM TFLOP/s at 4096^3 on 1 MI355X" if f8 else f"bf16 GEMM TFLOP/s, {args.config}",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic (seeded counter-based generators, inputs resident in HBM)",
+        "dtype": "fp8 (e4m3)" if f8 else "bf16", "data": "synthetic (seeded counter-based generators, inputs resident in HBM)",
         "config": {"workload": cfg["label"], "M": m, "N": n, "K": k, "batch": batch, "layout": "NT" if nt else "NN",
                    "accumulate": "fp32", "output": "bf16", "operand_sets_cycled": nsets,
                    "clock_ramp_launches": ramp_launches},
-        "pct_of_mfma_bf16_peak": 100.0 * flops / (wall / args.steps) / 1e12 / PEAK_BF16_TFLOPS,
+        ("pct_of_mfma_fp8_peak" if f8 else "pct_of_mfma_bf16_peak"): 100.0 * flops / (wall / args.steps) / 1e12 / peak_flops,
         "roofline": roof, "cpu_baseline": cpu, "parity_vs_oracle": parity,
         "device": {"name": info["name"], "compute_units": info["compute_units"], "clock_khz": info["clock_khz"]},
     }

@@ -1,7 +1,7 @@
 """Seeded input generators (thin wrappers over the library's host-side fill functions)."""
 import numpy as np
 
-from . import _ffi
+from . import _ffi, bf16, f8
 
 SEED_A = 0x5EED0001
 SEED_B = 0x5EED0002
@@ -22,3 +22,8 @@ def normal_bf16(n, seed, sigma=1.0, first_index=0):
     out = np.empty(n, dtype=np.uint16)
     _ffi.lib().maize_fill_normal_bf16(out.ctypes.data, n, seed, float(sigma), first_index)
     return out
+
+
+def uniform_f8(n, seed, in_type, first_index=0):
+    """n E4M3 / E5M2 encodings: the uniform [-1, 1) bf16 stream of the same seed, rounded (RNE) to the 8-bit format."""
+    return f8.from_f64(bf16.to_f64(uniform_bf16(n, seed, first_index)), in_type)

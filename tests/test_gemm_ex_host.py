@@ -151,3 +151,30 @@ def test_dispatch_of_half_operands():
     with pytest.raises(mz.MaizeError) as e:
         mz.validate(ex(in_type=5))
     assert e.value.code == _ffi.MAIZE_ERR_ARG
+
+
+def test_dispatch_of_8bit_operands():
+    """E4M3 / E5M2: the macro-tile kernels need both operands K-contiguous (B stored N x K) with rows on 16-byte
+    boundaries and K % 16 == 0; everything else goes to the per-wave kernel.  One byte per element: odd operand
+    pointers are valid."""
+    big = dict(m=4096, n=4096, k=4096, layout=mz.LAYOUT_NT)
+    for it, name in ((mz.IN_E4M3, "maize_gemm_e4m3_mt256_nt"), (mz.IN_E5M2, "maize_gemm_e5m2_mt256_nt")):
+        x = ex(**big, in_type=it)
+        plan = mz.gemm_plan(x)
+        assert plan["kernel"] == name and tuple(plan["grid"]) == (256, 1, 1) and plan["workspace_bytes"] == 0
+        assert mz.gemm_plan(ex(**big, in_type=it, alpha=2.0, beta=1.0, out_type=mz.OUT_F32))["kernel"] == name
+        for other in mz.kernel_names():
+            assert _supports(other, x) == (other in (name, "maize_gemm_bf16_wave32")), other
+        assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"            # row-major B
+        assert mz.gemm_plan(ex(4096, 4096, 4104, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"   # K % 16
+        assert mz.gemm_plan(ex(**big, in_type=it, ldb=4104))["kernel"] == "maize_gemm_bf16_wave32"             # rows off 16 bytes
+        assert mz.gemm_plan(ex(**big, in_type=it, ptrs=(0x1001, 0x100000, 0x2000000)))["kernel"] == "maize_gemm_bf16_wave32"
+        assert mz.gemm_plan(ex(64, 64, 64, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"
+        assert mz.gemm_plan(ex(64, 64, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name
+        mz.validate(ex(**big, in_type=it, ptrs=(0x1001, 0x100003, 0x2000000)))
+    for name in mz.kernel_names():
+        if name.startswith(("maize_gemm_e4m3_", "maize_gemm_e5m2_")):
+            assert not _supports(name, ex(**big)) and not _supports(name, ex(**big, in_type=mz.IN_F16))
+    with pytest.raises(mz.MaizeError) as e:
+        mz.validate(ex(in_type=4))
+    assert e.value.code == _ffi.MAIZE_ERR_ARG

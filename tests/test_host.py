@@ -218,3 +218,26 @@ def test_host_bf16_conversion_matches_oracle(oracle):
     for h in (0, 0x8000, 0x3F80, 0x7F7F, 0x0001):
         assert L.maize_bf16_to_f32(h) == O.mzo_bf16_to_f32(h)
     assert (L.maize_bf16_from_f32(float("nan")) & 0x7FFF) > 0x7F80
+
+
+def test_f8_host_helpers_agree_with_the_oracle(oracle):
+    """maize_amd.f8 (the product's host-side encoder / decoder of E4M3 and E5M2, used by its generators) against
+    the oracle's C functions: every encoding decodes alike, random doubles, every midpoint and the saturation
+    rule encode alike."""
+    import maize_amd as mz
+    L = oracle.lib()
+    rng = np.random.default_rng(5)
+    for in_type, elem in ((mz.IN_E4M3, oracle.E4M3), (mz.IN_E5M2, oracle.E5M2)):
+        bits = np.arange(256, dtype=np.uint8)
+        ours = mz.f8.to_f64(bits, in_type)
+        theirs = np.array([L.mzo_fp8_to_f32(int(b), elem) for b in bits], dtype=np.float64)
+        assert np.array_equal(ours[~np.isnan(theirs)], theirs[~np.isnan(theirs)]) and np.isnan(ours[np.isnan(theirs)]).all()
+        fin = np.sort(np.abs(theirs[np.isfinite(theirs)]))
+        x = np.concatenate([rng.standard_normal(3000) * 10.0 ** rng.integers(-6, 6, 3000), (fin[:-1] + fin[1:]) / 2, -fin,
+                            [0.0, -0.0, np.inf, -np.inf, 1e30, -1e30]])
+        want = np.array([L.mzo_fp8_from_f64(float(v), elem) for v in x], dtype=np.uint8)
+        assert np.array_equal(mz.f8.from_f64(x, in_type), want)
+        g = mz.gen.uniform_f8(4096, 7, in_type)
+        assert g.dtype == np.uint8 and np.array_equal(g, mz.gen.uniform_f8(4096, 7, in_type))
+        v = mz.f8.to_f64(g, in_type)
+        assert np.isfinite(v).all() and np.abs(v).max() <= 1.0 and abs(v.mean()) < 0.05

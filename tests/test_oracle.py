@@ -285,3 +285,88 @@ def test_half_gemm_vs_numpy_float64_and_closed_forms(oracle):
     cr, fr, _ = oracle.ref_gemm_rows(a.view(np.uint16), b.view(np.uint16), m, n, k, rows, elem=oracle.F16)
     full, _, _ = oracle.ref_gemm(a.view(np.uint16), b.view(np.uint16), m, n, k, elem=oracle.F16)
     assert np.array_equal(cr, full.reshape(m, n)[rows])
+
+
+# ---- OCP 8-bit floats: the operand types of the 8-bit entries of the MMA catalogue --------------------
+
+def test_fp8_formats_published_extremes_round_trip_and_ties(oracle):
+    L = oracle.lib()
+    E4, E5 = oracle.E4M3, oracle.E5M2
+    f = lambda b, e: L.mzo_fp8_to_f32(b, e)
+    # the formats' published table: E4M3 max 448 = S.1111.110, min normal 2^-6, min subnormal 2^-9, one NaN, no infinity;
+    # E5M2 max 57344 = S.11110.11, min normal 2^-14, min subnormal 2^-16, infinities and NaNs as in IEEE
+    assert f(0x7E, E4) == 448.0 and f(0xFE, E4) == -448.0 and f(0x08, E4) == 2.0 ** -6 and f(0x01, E4) == 2.0 ** -9
+    assert f(0x38, E4) == 1.0 and f(0x3C, E4) == 1.5 and f(0x40, E4) == 2.0 and f(0x77, E4) == 240.0 and f(0x78, E4) == 256.0
+    assert math.isnan(f(0x7F, E4)) and math.isnan(f(0xFF, E4)) and f(0x00, E4) == 0.0 and math.copysign(1.0, f(0x80, E4)) == -1.0
+    assert f(0x7B, E5) == 57344.0 and f(0x04, E5) == 2.0 ** -14 and f(0x01, E5) == 2.0 ** -16 and f(0x3C, E5) == 1.0 and f(0x3E, E5) == 1.5
+    assert f(0x7C, E5) == math.inf and f(0xFC, E5) == -math.inf and all(math.isnan(f(b, E5)) for b in (0x7D, 0x7E, 0x7F, 0xFD))
+    for elem, top in ((E4, 0x7E), (E5, 0x7B)):
+        vals = [f(b, elem) for b in range(top + 1)]
+        assert all(vals[i] < vals[i + 1] for i in range(top)), "positive finite codes are ordered"
+        for b in range(256):
+            v = f(b, elem)
+            if math.isfinite(v) and v != 0.0:
+                assert L.mzo_fp8_from_f64(v, elem) == b                       # round trip
+        for b in range(top):                                                   # midpoints go to the even code
+            assert L.mzo_fp8_from_f64((vals[b] + vals[b + 1]) / 2, elem) == (b + 1 if b & 1 else b)
+            assert L.mzo_fp8_from_f64(math.nextafter((vals[b] + vals[b + 1]) / 2, math.inf), elem) == b + 1
+            assert L.mzo_fp8_from_f64(math.nextafter((vals[b] + vals[b + 1]) / 2, 0.0), elem) == b
+        big = vals[top]
+        assert L.mzo_fp8_from_f64(big * 1.5, elem) == top and L.mzo_fp8_from_f64(-1e30, elem) == (0x80 | top)   # saturates
+        assert L.mzo_fp8_from_f64(vals[1] / 2, elem) == 0 and L.mzo_fp8_from_f64(vals[1] * 0.51, elem) == 1      # tie at half the smallest -> 0 (even)
+    assert L.mzo_fp8_from_f64(math.inf, E5) == 0x7C and L.mzo_fp8_from_f64(-math.inf, E4) == 0xFE
+    assert L.mzo_fp8_from_f64(math.nan, E4) & 0x7F == 0x7F and L.mzo_fp8_from_f64(math.nan, E5) & 0x7F in (0x7D, 0x7E, 0x7F)
+    # the vectorised encoder of the Python wrapper is the same function
+    rng = np.random.default_rng(21)
+    for elem in (E4, E5):
+        x = np.concatenate([rng.standard_normal(4000) * 10.0 ** rng.integers(-6, 6, 4000), [0.0, -0.0, math.inf, -math.inf]])
+        assert np.array_equal(oracle.fp8_bits_from_f64(x, elem), np.array([L.mzo_fp8_from_f64(float(v), elem) for v in x], np.uint8))
+
+
+def test_fp8_formats_match_torch_float8(oracle):
+    torch = pytest.importorskip("torch")
+    if not hasattr(torch, "float8_e4m3fn"):
+        pytest.skip("this torch has no float8 dtypes")
+    for elem, tdt, mx in ((oracle.E4M3, torch.float8_e4m3fn, 448.0), (oracle.E5M2, torch.float8_e5m2, 57344.0)):
+        bits = np.arange(256, dtype=np.uint8)
+        ours = oracle.fp8_bits_to_f64(bits, elem)
+        theirs = torch.from_numpy(bits.copy()).view(tdt).to(torch.float64).numpy()
+        assert np.array_equal(ours[~np.isnan(theirs)], theirs[~np.isnan(theirs)]) and np.isnan(ours[np.isnan(theirs)]).all()
+        rng = np.random.default_rng(22)
+        x = np.concatenate([rng.uniform(-mx, mx, 5000), rng.standard_normal(5000), 2.0 ** rng.uniform(-20, 8, 5000)]).astype(np.float32)
+        x = x[np.abs(x) <= mx]                                                # inside the finite range the two agree (beyond: we saturate)
+        theirs = torch.from_numpy(x).to(tdt).view(torch.uint8).numpy()
+        assert np.array_equal(oracle.fp8_bits_from_f64(x.astype(np.float64), elem), theirs)
+
+
+def test_fp8_gemm_vs_numpy_float64_and_closed_forms(oracle):
+    rng = np.random.default_rng(23)
+    m, n, k = 19, 23, 77
+    for elem in (oracle.E4M3, oracle.E5M2):
+        a = oracle.fp8_bits_from_f64(rng.standard_normal((m, k)), elem)
+        b = oracle.fp8_bits_from_f64(rng.standard_normal((k, n)), elem)
+        av, bv = oracle.fp8_bits_to_f64(a, elem), oracle.fp8_bits_to_f64(b, elem)
+        for layout, bs in ((oracle.NN, b), (oracle.NT, np.ascontiguousarray(b.T))):
+            c, f64, ab = oracle.ref_gemm(a, bs, m, n, k, layout=layout, want_f64=True, want_abs=True, elem=elem)
+            assert np.allclose(f64[0], av @ bv, rtol=0, atol=1e-12 * k)
+            assert np.array_equal(c.reshape(m, n), oracle.bf16_bits_from_f64(f64[0]))       # C is bf16
+            assert np.allclose(ab[0], np.abs(av) @ np.abs(bv), rtol=1e-14)
+        # identity: C = B exactly (bf16 holds every 8-bit float); small integers: exact sums
+        one = oracle.fp8_bits_from_f64(np.array([1.0]), elem)[0]
+        eye = np.zeros((16, 16), np.uint8)
+        eye[np.arange(16), np.arange(16)] = one
+        bb = oracle.fp8_bits_from_f64(rng.standard_normal((16, 9)), elem)
+        c, _, _ = oracle.ref_gemm(eye, bb, 16, 9, 16, elem=elem)
+        assert np.array_equal(oracle.bf16_bits_to_f64(c).reshape(16, 9), oracle.fp8_bits_to_f64(bb, elem))
+        ai, bi = rng.integers(-3, 4, (5, 32)), rng.integers(-3, 4, (32, 6))
+        c, _, _ = oracle.ref_gemm(oracle.fp8_bits_from_f64(ai, elem), oracle.fp8_bits_from_f64(bi, elem), 5, 6, 32, elem=elem)
+        assert np.array_equal(oracle.bf16_bits_to_f64(c).reshape(5, 6).astype(np.int64), ai @ bi)
+        rows = np.array([4, 0, 2], np.uint32)
+        cr, _, _ = oracle.ref_gemm_rows(a, b, m, n, k, rows, elem=elem)
+        full, _, _ = oracle.ref_gemm(a, b, m, n, k, elem=elem)
+        assert np.array_equal(cr, full.reshape(m, n)[rows])
+    # the same bytes read in the other format give a different product: the element type is honoured
+    c4, _, _ = oracle.ref_gemm(a, b, m, n, k, elem=oracle.E4M3)
+    c5, _, _ = oracle.ref_gemm(a, b, m, n, k, elem=oracle.E5M2)
+    assert not np.array_equal(c4, c5)
+    assert oracle.floor_coeff_f8(4096) == 2.0 ** -15 + (4096 / 64 + 2) * 2.0 ** -24
