@@ -97,12 +97,14 @@ inline maize_gemm_desc_t gemm_desc(const Matrix& a, const Matrix& b, const Matri
 // C = A.B through the dispatcher: the reference's mainloop entry, carried through to a launch.
 // The extended descriptor: leading dimensions (0 = ncols), element type of C, C = alpha * A.B + beta * C.
 inline maize_gemm_ex_desc_t gemm_ex_desc(const maize_gemm_desc_t& d, uint32_t lda = 0, uint32_t ldb = 0, uint32_t ldc = 0,
-                                         maize_out_type_t out = MAIZE_OUT_BF16, float alpha = 1.0f, float beta = 0.0f) {
+                                         maize_out_type_t out = MAIZE_OUT_BF16, float alpha = 1.0f, float beta = 0.0f,
+                                         maize_in_type_t in = MAIZE_IN_BF16) {
     maize_gemm_ex_desc_t x{};
     x.gemm = d;
     x.lda = lda; x.ldb = ldb; x.ldc = ldc;
     x.out_type = out;
     x.alpha = alpha; x.beta = beta;
+    x.in_type = in;            // half, or the 8-bit E4M3 / E5M2 (one byte per element; the Matrix views then wrap byte pointers)
     return x;
 }
 

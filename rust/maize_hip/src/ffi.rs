@@ -10,6 +10,8 @@ pub const MAIZE_OUT_SAME: u32 = 0;
 pub const MAIZE_OUT_F32: u32 = 1;
 pub const MAIZE_IN_BF16: u32 = 0;
 pub const MAIZE_IN_F16: u32 = 1;
+pub const MAIZE_IN_E4M3: u32 = 2;
+pub const MAIZE_IN_E5M2: u32 = 3;
 
 /// == GlobalMatrix<T>::Realized of the reference (src/main.rs:20-27): pointer + two u32 extents, 16-byte aligned.
 #[repr(C, align(16))]
