@@ -94,8 +94,10 @@ bool f8_nt_common(const maize_gemm_ex_desc_t& d) {
     if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21)) return false;
     return true;
 }
-bool e4m3_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 && f8_nt_common(d); }
-bool e5m2_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E5M2 && f8_nt_common(d); }
+bool e4m3_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 && f8_nt_common(d) && plain_epilogue(d); }
+bool e5m2_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E5M2 && f8_nt_common(d) && plain_epilogue(d); }
+bool e4m3_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 && f8_nt_common(d); }
+bool e5m2_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E5M2 && f8_nt_common(d); }
 // Edge splitting.  A ragged N leaves a last column of tiles that are almost empty but cost a
 // whole tile each (likewise a ragged M and the last row).  When that edge is at most 32 elements
 // wide and setting it aside saves a round of workgroups (one workgroup per compute unit per
@@ -350,6 +352,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_f16_mt256_nt_packed", "maize_gemm_f16_mt256_nt_splitk", packed_f16_nt_supports, packed_plan},
     {"maize_gemm_e4m3_mt256_nt", nullptr, e4m3_nt_supports, mt256_plan},
     {"maize_gemm_e5m2_mt256_nt", nullptr, e5m2_nt_supports, mt256_plan},
+    {"maize_gemm_e4m3_mt256_nt_gen", nullptr, e4m3_nt_gen_supports, mt256_plan},
+    {"maize_gemm_e5m2_mt256_nt_gen", nullptr, e5m2_nt_gen_supports, mt256_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -369,7 +373,9 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     if (fp8_in(d)) {
         // 8-bit operands: the macro-tile kernel when both operands are K-contiguous and aligned (same
         // size rule as below), else the per-wave kernel, which widens them to half as it loads.
-        const int fi = kernel_index(d.in_type == MAIZE_IN_E4M3 ? "maize_gemm_e4m3_mt256_nt" : "maize_gemm_e5m2_mt256_nt");
+        static const char* const kF8[2][2] = {{"maize_gemm_e4m3_mt256_nt", "maize_gemm_e4m3_mt256_nt_gen"},
+                                              {"maize_gemm_e5m2_mt256_nt", "maize_gemm_e5m2_mt256_nt_gen"}};
+        const int fi = kernel_index(kF8[d.in_type == MAIZE_IN_E5M2][!plain_epilogue(d)]);
         if (fi >= 0 && kKernels[fi].supports(d) && (s.k >= 256 || (s.m >= 128 && s.n >= 128))) return (uint32_t)fi;
         return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
     }

@@ -13,8 +13,9 @@
 // matter.  The whole of tile t+2 is requested during the second half of step t (one 1 KiB piece
 // per MFMA slot) and has to have landed at the barrier in the middle of step t+1.
 //
-// Epilogue: the general one (alpha, beta, bf16 or fp32 C, leading dimensions), staged through LDS
-// as fp32.  K % 16 == 0 and N % 8 == 0; rows of A and B start on 16-byte boundaries.
+// Epilogue: the bf16 kernel's two.  Plain (bf16 C = A.B): converted to bf16, staged through LDS,
+// 128-bit non-temporal row stores.  General (`_gen`: alpha, beta, fp32 C): staged as fp32.
+// K % 16 == 0 and N % 8 == 0; rows of A and B start on 16-byte boundaries.
 #pragma once
 #include "common.hpp"
 #include "gemm_mt256.hpp"
@@ -24,6 +25,7 @@ namespace maize {
 namespace mt256f8 {
 
 using mt256::lds_ptr;
+using mt256::lds_v2;
 using mt256::lds_v4;
 using mt256::make_rsrc;
 using mt256::tile_of;
@@ -35,7 +37,8 @@ constexpr uint32_t OOB = 0x80000000u;
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 // FMT: operand format code of the matrix instruction (0 = E4M3, 1 = E5M2), for A and B alike.
-template <int FMT>
+// GEN: the general epilogue instead of the plain one.
+template <int FMT, bool GEN>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     __shared__ __attribute__((aligned(1024))) char lds_a0[TILE];
     __shared__ __attribute__((aligned(1024))) char lds_a1[TILE];
@@ -191,38 +194,66 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, 0u);
         }
 
-        // ---- epilogue: each wave stages its 128 x 128 sub-tile as fp32, 32 rows x 64 columns at a
-        // time (row = 256 B, 16-byte chunk index XOR-ed with row%16), reads it back as runs of 8
-        // consecutive columns of a row and finishes them with store_c_run.
         lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
-        const uint32_t c8 = lane & 7u, r8 = lane >> 3;
+        if (GEN) {
+            // ---- general epilogue: each wave stages its 128 x 128 sub-tile as fp32, 32 rows x 64 columns
+            // at a time (row = 256 B, 16-byte chunk index XOR-ed with row%16), reads it back as runs of 8
+            // consecutive columns of a row and finishes them with store_c_run.
+            const uint32_t c8 = lane & 7u, r8 = lane >> 3;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int jh = 0; jh < 2; ++jh) {
+                for (int jh = 0; jh < 2; ++jh) {
 #pragma unroll
-                for (int jj = 0; jj < 2; ++jj)
+                    for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int j = jh * 2 + jj;
-                        // lane holds C[row = i*32 + l32][col = j*32 + 8q + 4*lhi + 0..3]
-                        const floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                        const uint32_t chunk = ((uint32_t)(jj * 8 + q * 2) + lhi) ^ (l32 & 15u);
-                        *(__attribute__((address_space(3))) floatx4*)(ew + l32 * 256u + chunk * 16u) = f;
-                    }
-                const uint32_t gcol = en0 + wn * 128u + jh * 64u + c8 * 8u;
+                        for (int q = 0; q < 4; ++q) {
+                            const int j = jh * 2 + jj;
+                            // lane holds C[row = i*32 + l32][col = j*32 + 8q + 4*lhi + 0..3]
+                            const floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                            const uint32_t chunk = ((uint32_t)(jj * 8 + q * 2) + lhi) ^ (l32 & 15u);
+                            *(__attribute__((address_space(3))) floatx4*)(ew + l32 * 256u + chunk * 16u) = f;
+                        }
+                    const uint32_t gcol = en0 + wn * 128u + jh * 64u + c8 * 8u;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint32_t row = r * 8 + r8;
-                    const floatx4 lo = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8) ^ (row & 15u)) * 16u));
-                    const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8 + 1u) ^ (row & 15u)) * 16u));
-                    const uint32_t grow = em0 + wm * 128u + i * 32u + row;
-                    if (gcol < N && grow < M) {                   // N % 8 == 0: a run is all in or all out
-                        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        store_c_run<8>(p, Ce, (uint64_t)grow * ldc + gcol, v);
+                    for (int r = 0; r < 4; ++r) {
+                        const uint32_t row = r * 8 + r8;
+                        const floatx4 lo = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8) ^ (row & 15u)) * 16u));
+                        const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8 + 1u) ^ (row & 15u)) * 16u));
+                        const uint32_t grow = em0 + wm * 128u + i * 32u + row;
+                        if (gcol < N && grow < M) {                   // N % 8 == 0: a run is all in or all out
+                            const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                            store_c_run<8>(p, Ce, (uint64_t)grow * ldc + gcol, v);
+                        }
                     }
                 }
+        } else {
+            // ---- plain epilogue: fp32 -> bf16 (RNE), 32 rows x 128 columns per pass through the wave's
+            // staging region (maps.hpp), 128-bit row stores through a descriptor over this batch
+            // member's C: rows at or past M fall behind its end, columns at or past N get an
+            // out-of-range offset.  Non-temporal: C is not read again.
+            const uint32_t cc = lane & 15u, cr = lane >> 4;
+            const uint32_t gcol = en0 + wn * 128u + cc * 8u;
+            const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce, ((M - 1u) * ldc + N) * 2u);
+            const uint32_t c_vo = (((em0 + wm * 128u + cr) * ldc + gcol) * 2u) | (gcol < N ? 0u : OOB);
+            const uint32_t row_bytes = __builtin_amdgcn_readfirstlane(ldc * 2u);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const u32x2 v = {cvt_pk_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1]), cvt_pk_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
+                        *(lds_v2)(ew + maps::epi_write_offset(j, q, lane)) = v;
+                    }
+#pragma unroll
+                for (int r = 0; r < 8; ++r) {
+                    u32x4 v = *(lds_v4)(ew + maps::epi_read_offset(r, lane));
+                    if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
+                    __builtin_amdgcn_raw_buffer_store_b128(v, rc, c_vo, (uint32_t)(i * 32 + r * 4) * row_bytes, 2 /* nt */);
+                }
             }
+        }
         if (!more) break;
         pid = next;
     }
@@ -230,7 +261,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
 }  // namespace mt256f8
 
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt(GemmArgs p) { mt256f8::body<0>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt(GemmArgs p) { mt256f8::body<1>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt(GemmArgs p) { mt256f8::body<0, false>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt(GemmArgs p) { mt256f8::body<1, false>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt_gen(GemmArgs p) { mt256f8::body<0, true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt_gen(GemmArgs p) { mt256f8::body<1, true>(p); }
 
 }  // namespace maize

@@ -75,7 +75,7 @@ def test_data_movement_the_design_rests_on(kernels):
         if "_mt256_" in name or name == "maize_gemm_bf16_skinny_nn":
             lds_dma = [i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]
             assert len(lds_dma) >= 16, f"{name}: operands must reach LDS by 128-bit direct-to-LDS loads"
-            fp32_staging = "_gen" in name or "_splitk" in name or name.startswith(("maize_gemm_e4m3_", "maize_gemm_e5m2_"))
+            fp32_staging = "_gen" in name or "_splitk" in name
             assert count(ins, "ds_write_b128") == 0 or fp32_staging, name   # no register round trip for operands
         if "_mt256_nn" in name or name == "maize_gemm_bf16_skinny_nn":
             assert count(ins, "ds_read_b64_tr_b16") >= 8, f"{name}: a row-major K x N B is read with transposing reads"

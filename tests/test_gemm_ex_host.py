@@ -162,9 +162,11 @@ def test_dispatch_of_8bit_operands():
         x = ex(**big, in_type=it)
         plan = mz.gemm_plan(x)
         assert plan["kernel"] == name and tuple(plan["grid"]) == (256, 1, 1) and plan["workspace_bytes"] == 0
-        assert mz.gemm_plan(ex(**big, in_type=it, alpha=2.0, beta=1.0, out_type=mz.OUT_F32))["kernel"] == name
+        general = ex(**big, in_type=it, alpha=2.0, beta=1.0, out_type=mz.OUT_F32)
+        assert mz.gemm_plan(general)["kernel"] == name + "_gen"
         for other in mz.kernel_names():
-            assert _supports(other, x) == (other in (name, "maize_gemm_bf16_wave32")), other
+            assert _supports(other, x) == (other in (name, name + "_gen", "maize_gemm_bf16_wave32")), other
+            assert _supports(other, general) == (other in (name + "_gen", "maize_gemm_bf16_wave32")), other
         assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"            # row-major B
         assert mz.gemm_plan(ex(4096, 4096, 4104, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"   # K % 16
         assert mz.gemm_plan(ex(**big, in_type=it, ldb=4104))["kernel"] == "maize_gemm_bf16_wave32"             # rows off 16 bytes

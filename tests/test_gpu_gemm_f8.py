@@ -106,7 +106,7 @@ def test_every_encoding_reaches_the_matrix_unit_unchanged(ctx, oracle, fmt):
     eye = np.zeros((k, k), dtype=np.uint8)
     eye[np.arange(k), np.arange(k)] = one
     want = oracle.bf16_bits_from_f64(oracle.fp8_bits_to_f64(a, elem))
-    for kernel in ("maize_gemm_bf16_wave32", f"maize_gemm_{fmt}_mt256_nt"):
+    for kernel in ("maize_gemm_bf16_wave32", f"maize_gemm_{fmt}_mt256_nt", f"maize_gemm_{fmt}_mt256_nt_gen"):
         got, took = launch(ctx, a.ravel(), eye.ravel(), np.zeros(m * k, np.uint16), m, k, k, mz.LAYOUT_NT, fmt, k, k, k, kernel=kernel)
         assert took == kernel
         # -0 * 1 + 0 = +0 in the accumulator: compare values, not the sign of zero
@@ -130,7 +130,7 @@ def test_what_the_8bit_matrix_instruction_keeps(ctx, oracle):
     for c in range(n):
         b[c, 1] = enc(2.0 ** -(c % 16))
     got, _ = launch(ctx, a.ravel(), b.ravel(), np.zeros(m * n, np.float32), m, n, k, mz.LAYOUT_NT, fmt, k, k, n, out_f32=True,
-                    kernel="maize_gemm_e5m2_mt256_nt")
+                    kernel="maize_gemm_e5m2_mt256_nt_gen")
     g = got.reshape(m, n)
     for r in range(16):
         for c in range(16):
@@ -152,9 +152,11 @@ def test_macro_tile_kernel(ctx, oracle, fmt, shape):
 def test_macro_tile_kernel_all_knobs(ctx, oracle, fmt):
     m, n, k = 520, 776, 400
     name = f"maize_gemm_{fmt}_mt256_nt"
-    for kw in (dict(lda=416, ldb=432, ldc=784), dict(alpha=0.5), dict(alpha=-1.25, beta=0.75), dict(out_f32=True),
-               dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(alpha=0.0, beta=1.0)):
-        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 knobs", **kw) == name
+    assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 views", lda=416, ldb=432, ldc=784) == name
+    assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 gen by name", kernel=name + "_gen") == name + "_gen"
+    for kw in (dict(alpha=0.5), dict(alpha=-1.25, beta=0.75), dict(out_f32=True), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8),
+               dict(alpha=0.0, beta=1.0), dict(alpha=2.0, lda=416, ldb=432, ldc=784)):
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 knobs", **kw) == name + "_gen"
 
 
 def test_dispatch_of_8bit_products(ctx):
