@@ -98,6 +98,7 @@ bool e4m3_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE
 bool e5m2_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E5M2 && f8_nt_common(d) && plain_epilogue(d); }
 bool e4m3_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 && f8_nt_common(d); }
 bool e5m2_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E5M2 && f8_nt_common(d); }
+bool splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld);
 // Edge splitting.  A ragged N leaves a last column of tiles that are almost empty but cost a
 // whole tile each (likewise a ragged M and the last row).  When that edge is at most 32 elements
 // wide and setting it aside saves a round of workgroups (one workgroup per compute unit per
@@ -169,9 +170,9 @@ bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld
 // i.e. a second launch and the fp32 partial tiles written and read back at ~4 TB/s; the split is
 // taken only if it wins by 20 %.  (2048^3, 64 tiles: 38 us unsplit, 40 us split 4 ways -- not
 // split; 64 x 4096 x 4096: 63 -> 25 us; 256 x 256 x 16384: 237 -> 38 us.)
-uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus) {
+uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * batch;
-    const uint32_t nk = cdiv(s.k, 64);
+    const uint32_t nk = cdiv(s.k, kstep);                    // K steps of 128 bytes per row: 64 16-bit elements, 128 8-bit ones
     if (cus == 0 || tiles == 0 || tiles * 2 > cus || nk < 8u) return 1;
     uint32_t kmax = (uint32_t)(cus / tiles);
     if (kmax > nk / 4u) kmax = nk / 4u;
@@ -194,10 +195,11 @@ bool splitk_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt2
 bool splitk_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && half_in(d); }
 bool splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
     const Dims s = dims_of(d);
+    const uint32_t kstep = fp8_in(d) ? 128u : 64u;
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * d.gemm.batch;
-    uint32_t ks = splitk_ranges(s, d.gemm.batch, compute_units);
+    uint32_t ks = splitk_ranges(s, d.gemm.batch, compute_units, kstep);
     // Named explicitly for a shape the dispatcher would not split: two ranges if K allows, else one.
-    if (ks < 2u) ks = cdiv(s.k, 64) >= 2u && tiles * 2ull * 262144ull <= (1ull << 30) ? 2u : 1u;
+    if (ks < 2u) ks = cdiv(s.k, kstep) >= 2u && tiles * 2ull * 262144ull <= (1ull << 30) ? 2u : 1u;
     const uint64_t items = tiles * ks;
     if (items > 0x1FFFFFFFull || items * 262144ull > (1ull << 32)) return false;
     uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
@@ -354,6 +356,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_e5m2_mt256_nt", nullptr, e5m2_nt_supports, mt256_plan},
     {"maize_gemm_e4m3_mt256_nt_gen", nullptr, e4m3_nt_gen_supports, mt256_plan},
     {"maize_gemm_e5m2_mt256_nt_gen", nullptr, e5m2_nt_gen_supports, mt256_plan},
+    {"maize_gemm_e4m3_mt256_nt_splitk", nullptr, e4m3_nt_gen_supports, splitk_plan},
+    {"maize_gemm_e5m2_mt256_nt_splitk", nullptr, e5m2_nt_gen_supports, splitk_plan},
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -375,6 +379,8 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         // size rule as below), else the per-wave kernel, which widens them to half as it loads.
         static const char* const kF8[2][2] = {{"maize_gemm_e4m3_mt256_nt", "maize_gemm_e4m3_mt256_nt_gen"},
                                               {"maize_gemm_e5m2_mt256_nt", "maize_gemm_e5m2_mt256_nt_gen"}};
+        const int fs = kernel_index(d.in_type == MAIZE_IN_E4M3 ? "maize_gemm_e4m3_mt256_nt_splitk" : "maize_gemm_e5m2_mt256_nt_splitk");
+        if (fs >= 0 && kKernels[fs].supports(d) && splitk_ranges(s, d.gemm.batch, compute_units, 128) >= 2u) return (uint32_t)fs;
         const int fi = kernel_index(kF8[d.in_type == MAIZE_IN_E5M2][!plain_epilogue(d)]);
         if (fi >= 0 && kKernels[fi].supports(d) && (s.k >= 256 || (s.m >= 128 && s.n >= 128))) return (uint32_t)fi;
         return (uint32_t)kernel_index("maize_gemm_bf16_wave32");

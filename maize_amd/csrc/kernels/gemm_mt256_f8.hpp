@@ -37,8 +37,10 @@ constexpr uint32_t OOB = 0x80000000u;
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 // FMT: operand format code of the matrix instruction (0 = E4M3, 1 = E5M2), for A and B alike.
-// GEN: the general epilogue instead of the plain one.
-template <int FMT, bool GEN>
+// GEN: the general epilogue instead of the plain one.  SPLITK: the work items are (tile, K range)
+// pairs and each leaves an fp32 partial tile in the workspace for maize_gemm_splitk_reduce (as the
+// bf16 split-K kernels do, same layout).
+template <int FMT, bool GEN, bool SPLITK>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     __shared__ __attribute__((aligned(1024))) char lds_a0[TILE];
     __shared__ __attribute__((aligned(1024))) char lds_a1[TILE];
@@ -60,9 +62,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t a_bytes = (M - 1u) * lda + K;
     const uint32_t b_bytes = (N - 1u) * ldb + K;
     const uint32_t tiles_per = tm * tn;
-    const uint32_t total = tiles_per * p.batch;
+    const uint32_t nranges = SPLITK ? (p.ksplit ? p.ksplit : 1u) : 1u;
+    const uint32_t per_range = (nk + nranges - 1u) / nranges;
+    const uint32_t total = tiles_per * p.batch * nranges;
     uint32_t pid = blockIdx.x;
     if (pid >= total) return;
+    uint32_t nk_r = nk, k_begin = 0u, k_end = K;     // K steps of this work item, its first k, loads at or past k_end read zeros
+    uint32_t part_slot = 0u;                           // split-K: index of this item's partial tile
 
     // ---- per-tile state: copy maps of the direct-to-LDS loads (maps.hpp) -------------------
     uint32_t m0, n0;
@@ -73,9 +79,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     uint32_t a_k[2];                      // k of the lane's chunk inside a tile, even/odd piece
     auto select_tile = [&](uint32_t id) {
         uint32_t tile_m, tile_n;
-        const uint32_t t = xcd_run(id, total);
+        const uint32_t item = xcd_run(id, total);
+        const uint32_t t = item / nranges;                       // ranges of one tile are adjacent items
         const uint64_t bz = t / tiles_per;
         tile_of(t - (uint32_t)bz * tiles_per, tm, tn, &tile_m, &tile_n);
+        if (SPLITK) {
+            const uint32_t zr = item - t * nranges, kt0 = zr * per_range;
+            nk_r = kt0 < nk ? (nk - kt0 < per_range ? nk - kt0 : per_range) : 0u;
+            k_begin = kt0 * BK;
+            k_end = (kt0 + nk_r) * BK < K ? (kt0 + nk_r) * BK : K;
+            part_slot = ((uint32_t)bz * tiles_per + tile_m * tn + tile_n) * nranges + zr;
+        }
         m0 = tile_m * BM;
         n0 = tile_n * BN;
         Ag = (const uint8_t*)p.a + bz * p.stride_a;                      // strides count elements
@@ -97,7 +111,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const bool is_a = pc < 8;
         const int i = is_a ? pc : pc - 8;
         lds_ptr dst = (is_a ? sa : sb) + (wave_u * 8u + i) * 1024u;
-        const uint32_t bytes = k < K ? (is_a ? a_bytes : b_bytes) : 0u;   // tiles past K: all zeros
+        const uint32_t bytes = k < k_end ? (is_a ? a_bytes : b_bytes) : 0u;   // tiles past the end: all zeros
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(is_a ? (const void*)Ag : (const void*)Bg, bytes);
         uint32_t off = (is_a ? a_vo[i] : b_vo[i]) + k;
         off |= (a_k[i & 1] + k) < K ? 0u : OOB;                          // K % 16 == 0: a chunk is all in or all out
@@ -158,7 +172,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
     // ---- prime: the first K tile of the first C tile ------------------------------------------
 #pragma unroll
-    for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, 0u);
+    for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, k_begin);
 
     for (;;) {                                                  // one trip per C tile
 #pragma unroll
@@ -172,11 +186,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) read_frag(0, 0, r, A0, B0);
 #pragma unroll
-        for (int pc = 0; pc < 16; ++pc) dma(pc, A1, B1, (uint32_t)BK);
-        k_next = 2 * BK;
+        for (int pc = 0; pc < 16; ++pc) dma(pc, A1, B1, k_begin + BK);
+        k_next = k_begin + 2 * BK;
         // Two steps per trip (stages as compile-time constants); an odd step count runs one
         // extra step on an all-zero tile.
-        for (uint32_t kt = 0; kt < nk; kt += 2) {
+        for (uint32_t kt = 0; kt < nk_r; kt += 2) {
             step(A0, B0, A1, B1);
             step(A1, B1, A0, B0);
         }
@@ -184,22 +198,28 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
         // ---- hand-over: request the next C tile's first K tile before this one is stored ----
         __syncthreads();
-        const uint32_t em0 = m0, en0 = n0;
+        const uint32_t em0 = m0, en0 = n0, eslot = part_slot;
         char* const Ce = Cg;
         const uint32_t next = pid + gridDim.x;
         const bool more = next < total;
         if (more) {
             select_tile(next);
 #pragma unroll
-            for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, 0u);
+            for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, k_begin);
         }
 
         lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
-        if (GEN) {
+        if (GEN || SPLITK) {
             // ---- general epilogue: each wave stages its 128 x 128 sub-tile as fp32, 32 rows x 64 columns
             // at a time (row = 256 B, 16-byte chunk index XOR-ed with row%16), reads it back as runs of 8
             // consecutive columns of a row and finishes them with store_c_run.
             const uint32_t c8 = lane & 7u, r8 = lane >> 3;
+            // Split-K: the lane's place inside the partial tile.  Recomputed per tile on purpose (the empty
+            // asm makes it opaque): hoisted out of the tile loop, the 32 addresses derived from it would
+            // be kept live across the K loop and spilled.
+            uint32_t lane_part = (wm * 128u + r8) * BN + wn * 128u + c8 * 8u;
+            asm volatile("" : "+v"(lane_part));
+            float* const part_base = (float*)((char*)p.workspace + 65536) + (uint64_t)eslot * (BM * BN) + lane_part;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -222,8 +242,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                         const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8 + 1u) ^ (row & 15u)) * 16u));
                         const uint32_t grow = em0 + wm * 128u + i * 32u + row;
                         if (gcol < N && grow < M) {                   // N % 8 == 0: a run is all in or all out
-                            const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                            store_c_run<8>(p, Ce, (uint64_t)grow * ldc + gcol, v);
+                            if (SPLITK) {
+                                // fp32 partial tile of this (tile, K range), row-major 256 x 256, behind the 64 KiB of
+                                // ticket counters every workspace starts with
+                                float* part = part_base + (uint32_t)((i * 32 + r * 8) * BN + jh * 64);
+                                *(floatx4*)part = lo;
+                                *(floatx4*)(part + 4) = hi;
+                            } else {
+                                const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                                store_c_run<8>(p, Ce, (uint64_t)grow * ldc + gcol, v);
+                            }
                         }
                     }
                 }
@@ -261,9 +289,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
 }  // namespace mt256f8
 
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt(GemmArgs p) { mt256f8::body<0, false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt(GemmArgs p) { mt256f8::body<1, false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt_gen(GemmArgs p) { mt256f8::body<0, true>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt_gen(GemmArgs p) { mt256f8::body<1, true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt(GemmArgs p) { mt256f8::body<0, false, false>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt(GemmArgs p) { mt256f8::body<1, false, false>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt_gen(GemmArgs p) { mt256f8::body<0, true, false>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt_gen(GemmArgs p) { mt256f8::body<1, true, false>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt_splitk(GemmArgs p) { mt256f8::body<0, true, true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt_splitk(GemmArgs p) { mt256f8::body<1, true, true>(p); }
 
 }  // namespace maize

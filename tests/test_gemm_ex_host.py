@@ -165,14 +165,17 @@ def test_dispatch_of_8bit_operands():
         general = ex(**big, in_type=it, alpha=2.0, beta=1.0, out_type=mz.OUT_F32)
         assert mz.gemm_plan(general)["kernel"] == name + "_gen"
         for other in mz.kernel_names():
-            assert _supports(other, x) == (other in (name, name + "_gen", "maize_gemm_bf16_wave32")), other
-            assert _supports(other, general) == (other in (name + "_gen", "maize_gemm_bf16_wave32")), other
+            assert _supports(other, x) == (other in (name, name + "_gen", name + "_splitk", "maize_gemm_bf16_wave32")), other
+            assert _supports(other, general) == (other in (name + "_gen", name + "_splitk", "maize_gemm_bf16_wave32")), other
         assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"            # row-major B
         assert mz.gemm_plan(ex(4096, 4096, 4104, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"   # K % 16
         assert mz.gemm_plan(ex(**big, in_type=it, ldb=4104))["kernel"] == "maize_gemm_bf16_wave32"             # rows off 16 bytes
         assert mz.gemm_plan(ex(**big, in_type=it, ptrs=(0x1001, 0x100000, 0x2000000)))["kernel"] == "maize_gemm_bf16_wave32"
         assert mz.gemm_plan(ex(64, 64, 64, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"
-        assert mz.gemm_plan(ex(64, 64, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name
+        split = mz.gemm_plan(ex(64, 64, 4096, layout=mz.LAYOUT_NT, in_type=it))              # one tile, 32 K steps of 128
+        assert split["kernel"] == name + "_splitk" and split["ksplit"] >= 2 and split["reduce_grid"] > 0
+        assert split["workspace_bytes"] == 65536 + split["ksplit"] * 256 * 256 * 4
+        assert mz.gemm_plan(ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"
         mz.validate(ex(**big, in_type=it, ptrs=(0x1001, 0x100003, 0x2000000)))
     for name in mz.kernel_names():
         if name.startswith(("maize_gemm_e4m3_", "maize_gemm_e5m2_")):

@@ -200,3 +200,40 @@ def test_full_size_sampled_rows_and_batches(ctx, oracle, fmt):
                            mz.LAYOUT_NT, fmt, bk, bk, bn)
         assert np.array_equal(single, dense[i * sc:i * sc + bm * bn]), i
         assert not dense[i * sc + bm * bn:(i + 1) * sc].any(), "wrote between batch members"
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+def test_split_k_on_8bit_operands(ctx, oracle, fmt):
+    """Few tiles and a long K: (tile, K range) work items + the reduce pass, as for bf16.  The dispatcher takes it by
+    itself; every epilogue goes through the reduce pass; repeated launches give the same bits."""
+    name = f"maize_gemm_{fmt}_mt256_nt_splitk"
+    for (m, n, k) in ((16, 1096, 4096), (64, 512, 8192), (256, 256, 16384)):
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="f8 split-K") == name
+    assert run_f8(ctx, oracle, 40, 264, 2064, fmt=fmt, kernel=name, label="f8 split-K ragged K") == name
+    assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, alpha=-1.25, beta=0.75, label="f8 split-K scaled") == name
+    assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, out_f32=True, ldc=520, label="f8 split-K f32") == name
+    assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, kernel=name, label="f8 split-K by name") == name     # a shape it would not split
+    elem = FMT[fmt][1]
+    m, n, k = 16, 1096, 4096
+    a = f8_uniform(oracle, m * k, 31, elem)
+    b = f8_uniform(oracle, n * k, 32, elem)
+    first, took = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n)
+    assert took == name
+    for _ in range(3):
+        again, _ = launch(ctx, a, b, np.full(m * n, 0x7FC0, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n)
+        assert np.array_equal(again, first)
+    # the bf16 skinny kernel shares the stream's workspace (its ticket counters must still be zero)
+    m2, n2, k2 = 16, 1096, 4096
+    a2 = mz.gen.normal_bf16(m2 * k2, 3, 1.0)
+    b2 = mz.gen.normal_bf16(k2 * n2, 4, 0.02)
+    da, db, dc = ctx.upload(a2), ctx.upload(b2), ctx.malloc(m2 * n2 * 2)
+    try:
+        d = mz.gemm_desc(mz.Matrix(da, m2, k2), mz.Matrix(db, k2, n2), mz.Matrix(dc, m2, n2))
+        assert mz.gemm_plan(d, compute_units=ctx.info()["compute_units"])["kernel"] == "maize_gemm_bf16_skinny_nn"
+        ctx.gemm_bf16(d)
+        ctx.sync()
+        got = dc.download(np.uint16)
+    finally:
+        da.free(); db.free(); dc.free()
+    ref, val, ab = oracle.ref_gemm(a2, b2, m2, n2, k2, want_f64=True, want_abs=True)
+    assert oracle.compare(got, ref, val[0], ab[0], k2)["n_fail"] == 0
