@@ -102,8 +102,12 @@ typedef enum { MAIZE_OUT_SAME = 0, MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1 } maize
  * catalogue's Sm89MmaF8F32_* entries (crates/maize_tile/src/mma/sm89.rs:13-45; u8-backed,
  * crates/maize_core/src/ty/sized.rs:68-69): A and B hold one byte per element, dimensions, leading
  * dimensions and batch strides still count elements, and the matrix instruction is
- * v_mfma_f32_32x32x64_f8f6f4 when B is stored N x K (MAIZE_LAYOUT_NT) with 16-byte aligned rows. */
-typedef enum { MAIZE_IN_BF16 = 0, MAIZE_IN_F16 = 1, MAIZE_IN_E4M3 = 2, MAIZE_IN_E5M2 = 3 } maize_in_type_t;
+ * v_mfma_f32_32x32x64_f8f6f4 when B is stored N x K (MAIZE_LAYOUT_NT) with 16-byte aligned rows.
+ * MAIZE_IN_E4M3_E5M2 / MAIZE_IN_E5M2_E4M3: A of the first format, B of the second (the catalogue's mixed pairs,
+ * sm89.rs:34-45). */
+typedef enum {
+    MAIZE_IN_BF16 = 0, MAIZE_IN_F16 = 1, MAIZE_IN_E4M3 = 2, MAIZE_IN_E5M2 = 3, MAIZE_IN_E4M3_E5M2 = 4, MAIZE_IN_E5M2_E4M3 = 5
+} maize_in_type_t;
 typedef struct {
     maize_gemm_desc_t gemm;
     uint32_t lda, ldb, ldc;

@@ -43,6 +43,8 @@ IN_BF16 = 0
 IN_F16 = 1
 IN_E4M3 = 2
 IN_E5M2 = 3
+IN_E4M3_E5M2 = 4   # A is E4M3, B is E5M2
+IN_E5M2_E4M3 = 5
 
 
 class MatrixT(C.Structure):

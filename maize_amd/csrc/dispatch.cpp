@@ -1,6 +1,7 @@
 #include "dispatch.hpp"
 
 #include <cstdint>
+#include <cstdio>
 #include <cstring>
 
 namespace maize {
@@ -27,7 +28,7 @@ inline bool plain_epilogue(const maize_gemm_ex_desc_t& d) {
 }
 inline bool half_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_F16; }
 inline bool bf16_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_BF16; }
-inline bool fp8_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 || d.in_type == MAIZE_IN_E5M2; }
+inline bool fp8_in(const maize_gemm_ex_desc_t& d) { return d.in_type >= MAIZE_IN_E4M3 && d.in_type <= MAIZE_IN_E5M2_E4M3; }
 
 // ---- maize_gemm_bf16_wave32: any shape ------------------------------------
 bool wave32_supports(const maize_gemm_ex_desc_t&) { return true; }
@@ -94,10 +95,14 @@ bool f8_nt_common(const maize_gemm_ex_desc_t& d) {
     if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21)) return false;
     return true;
 }
-bool e4m3_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 && f8_nt_common(d) && plain_epilogue(d); }
-bool e5m2_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E5M2 && f8_nt_common(d) && plain_epilogue(d); }
-bool e4m3_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E4M3 && f8_nt_common(d); }
-bool e5m2_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_E5M2 && f8_nt_common(d); }
+#define MAIZE_F8_SUPPORTS(tag, type) \
+    bool tag##_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d) && plain_epilogue(d); } \
+    bool tag##_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d); }
+MAIZE_F8_SUPPORTS(e4m3, MAIZE_IN_E4M3)
+MAIZE_F8_SUPPORTS(e5m2, MAIZE_IN_E5M2)
+MAIZE_F8_SUPPORTS(e4m3e5m2, MAIZE_IN_E4M3_E5M2)
+MAIZE_F8_SUPPORTS(e5m2e4m3, MAIZE_IN_E5M2_E4M3)
+#undef MAIZE_F8_SUPPORTS
 bool splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld);
 // Edge splitting.  A ragged N leaves a last column of tiles that are almost empty but cost a
 // whole tile each (likewise a ragged M and the last row).  When that edge is at most 32 elements
@@ -352,12 +357,12 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_packed", "maize_gemm_bf16_mt256_nt_splitk", packed_nt_supports, packed_plan},
     {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nn_splitk", packed_f16_nn_supports, packed_plan},
     {"maize_gemm_f16_mt256_nt_packed", "maize_gemm_f16_mt256_nt_splitk", packed_f16_nt_supports, packed_plan},
-    {"maize_gemm_e4m3_mt256_nt", nullptr, e4m3_nt_supports, mt256_plan},
-    {"maize_gemm_e5m2_mt256_nt", nullptr, e5m2_nt_supports, mt256_plan},
-    {"maize_gemm_e4m3_mt256_nt_gen", nullptr, e4m3_nt_gen_supports, mt256_plan},
-    {"maize_gemm_e5m2_mt256_nt_gen", nullptr, e5m2_nt_gen_supports, mt256_plan},
-    {"maize_gemm_e4m3_mt256_nt_splitk", nullptr, e4m3_nt_gen_supports, splitk_plan},
-    {"maize_gemm_e5m2_mt256_nt_splitk", nullptr, e5m2_nt_gen_supports, splitk_plan},
+#define MAIZE_F8_ENTRIES(tag) \
+    {"maize_gemm_" #tag "_mt256_nt", nullptr, tag##_nt_supports, mt256_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_gen", nullptr, tag##_nt_gen_supports, mt256_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan},
+    MAIZE_F8_ENTRIES(e4m3) MAIZE_F8_ENTRIES(e5m2) MAIZE_F8_ENTRIES(e4m3e5m2) MAIZE_F8_ENTRIES(e5m2e4m3)
+#undef MAIZE_F8_ENTRIES
 };
 constexpr uint32_t kCount = sizeof(kKernels) / sizeof(kKernels[0]);
 static_assert(kCount <= kMaxKernels, "raise kMaxKernels");
@@ -376,12 +381,14 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     const Dims s = dims_of(d);
     if (fp8_in(d)) {
         // 8-bit operands: the macro-tile kernel when both operands are K-contiguous and aligned (same
-        // size rule as below), else the per-wave kernel, which widens them to half as it loads.
-        static const char* const kF8[2][2] = {{"maize_gemm_e4m3_mt256_nt", "maize_gemm_e4m3_mt256_nt_gen"},
-                                              {"maize_gemm_e5m2_mt256_nt", "maize_gemm_e5m2_mt256_nt_gen"}};
-        const int fs = kernel_index(d.in_type == MAIZE_IN_E4M3 ? "maize_gemm_e4m3_mt256_nt_splitk" : "maize_gemm_e5m2_mt256_nt_splitk");
+        // size rule as below), else the per-wave kernel, which widens them to bf16 as it loads.
+        static const char* const kTag[4] = {"e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"};
+        char name[64];
+        std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_splitk", kTag[d.in_type - MAIZE_IN_E4M3]);
+        const int fs = kernel_index(name);
         if (fs >= 0 && kKernels[fs].supports(d) && splitk_ranges(s, d.gemm.batch, compute_units, 128) >= 2u) return (uint32_t)fs;
-        const int fi = kernel_index(kF8[d.in_type == MAIZE_IN_E5M2][!plain_epilogue(d)]);
+        std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt%s", kTag[d.in_type - MAIZE_IN_E4M3], plain_epilogue(d) ? "" : "_gen");
+        const int fi = kernel_index(name);
         if (fi >= 0 && kKernels[fi].supports(d) && (s.k >= 256 || (s.m >= 128 && s.n >= 128))) return (uint32_t)fi;
         return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
     }

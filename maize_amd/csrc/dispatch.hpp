@@ -12,7 +12,7 @@
 
 namespace maize {
 
-constexpr uint32_t kMaxKernels = 32;
+constexpr uint32_t kMaxKernels = 48;
 constexpr const char* kReduceKernel = "maize_gemm_splitk_reduce";
 constexpr const char* kPackKernel = "maize_pack_2d";
 

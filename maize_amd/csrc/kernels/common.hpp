@@ -21,11 +21,11 @@ struct GemmArgs {
     // Extended part (all zero = the plain product: compact rows, bf16 C = A.B).
     uint32_t lda, ldb, ldc;  // elements between consecutive rows; 0 = the matrix's column count
     uint32_t epi;            // bit 0: C is fp32; bit 1: C = alpha * A.B + beta * C; bit 2: A, B (and a 16-bit C) are IEEE half;
-                             // bit 3 / bit 4: A and B are 8-bit E4M3 / E5M2 (a 16-bit C is bf16)
+                             // bit 3: A and B are 8-bit floats (a 16-bit C is bf16), E4M3 unless bit 4 (A) / bit 5 (B) says E5M2
     float alpha, beta;
 };
 static_assert(sizeof(GemmArgs) == 120, "kernel parameter block layout");
-constexpr uint32_t EPI_F32 = 1u, EPI_SCALE = 2u, EPI_F16 = 4u, EPI_E4M3 = 8u, EPI_E5M2 = 16u;
+constexpr uint32_t EPI_F32 = 1u, EPI_SCALE = 2u, EPI_F16 = 4u, EPI_F8 = 8u, EPI_A_E5M2 = 16u, EPI_B_E5M2 = 32u;
 
 // Leading dimensions with their defaults: the reference's rows are compact (row stride ==
 // ncols, crates/maize_tile/src/gmem/row_panel.rs:55).

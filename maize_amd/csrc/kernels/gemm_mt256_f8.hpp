@@ -1,4 +1,5 @@
-// maize_gemm_{e4m3,e5m2}_mt256_nt: the macro-tile pipeline on 8-bit floating-point operands.
+// maize_gemm_{e4m3,e5m2,e4m3e5m2,e5m2e4m3}_mt256_nt[_gen|_splitk]: the macro-tile pipeline on 8-bit
+// floating-point operands (A and B of the same or of different formats).
 //
 // The 8-bit entries of the reference's MMA catalogue (Sm89MmaF8F32_16x8x32 on E4M3 / E5M2,
 // crates/maize_tile/src/mma/sm89.rs:13-45; element types crates/maize_core/src/ty/sized.rs:68-69)
@@ -36,11 +37,11 @@ constexpr int TILE = 32768;
 constexpr uint32_t OOB = 0x80000000u;
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
-// FMT: operand format code of the matrix instruction (0 = E4M3, 1 = E5M2), for A and B alike.
+// FA, FB: operand format codes of the matrix instruction (0 = E4M3, 1 = E5M2) for A and for B.
 // GEN: the general epilogue instead of the plain one.  SPLITK: the work items are (tile, K range)
 // pairs and each leaves an fp32 partial tile in the workspace for maize_gemm_splitk_reduce (as the
 // bf16 split-K kernels do, same layout).
-template <int FMT, bool GEN, bool SPLITK>
+template <int FA, int FB, bool GEN, bool SPLITK>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     __shared__ __attribute__((aligned(1024))) char lds_a0[TILE];
     __shared__ __attribute__((aligned(1024))) char lds_a1[TILE];
@@ -158,7 +159,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #pragma unroll
             for (int s = 0; s < 16; ++s) {
                 acc[s >> 2][s & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    operand(fb[kh][s & 3]), operand(fa[kh][s >> 2]), acc[s >> 2][s & 3], FMT, FMT, 0, 0, 0, 0);
+                    operand(fb[kh][s & 3]), operand(fa[kh][s >> 2]), acc[s >> 2][s & 3], FB, FA, 0, 0, 0, 0);   // B is fed first
                 if (kh == 0) read_frag(1, 1, s, ca, cb);
                 else {
                     read_frag(0, 0, s, na, nb);
@@ -289,11 +290,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
 }  // namespace mt256f8
 
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt(GemmArgs p) { mt256f8::body<0, false, false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt(GemmArgs p) { mt256f8::body<1, false, false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt_gen(GemmArgs p) { mt256f8::body<0, true, false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt_gen(GemmArgs p) { mt256f8::body<1, true, false>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e4m3_mt256_nt_splitk(GemmArgs p) { mt256f8::body<0, true, true>(p); }
-extern "C" __global__ __launch_bounds__(256) void maize_gemm_e5m2_mt256_nt_splitk(GemmArgs p) { mt256f8::body<1, true, true>(p); }
+#define MAIZE_F8_KERNELS(tag, fa, fb) \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt(GemmArgs p) { mt256f8::body<fa, fb, false, false>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_gen(GemmArgs p) { mt256f8::body<fa, fb, true, false>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_splitk(GemmArgs p) { mt256f8::body<fa, fb, true, true>(p); }
+MAIZE_F8_KERNELS(e4m3, 0, 0)
+MAIZE_F8_KERNELS(e5m2, 1, 1)
+MAIZE_F8_KERNELS(e4m3e5m2, 0, 1)     // A is E4M3, B is E5M2
+MAIZE_F8_KERNELS(e5m2e4m3, 1, 0)
+#undef MAIZE_F8_KERNELS
 
 }  // namespace maize

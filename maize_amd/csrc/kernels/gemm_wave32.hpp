@@ -39,7 +39,7 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
     const uint16_t* __restrict__ A = p.a + bz * p.stride_a;
     const uint16_t* __restrict__ B = p.b + bz * p.stride_b;
     const bool f32_out = p.epi & EPI_F32, scaled = p.epi & EPI_SCALE, half_io = p.epi & EPI_F16;
-    const bool e5m2 = p.epi & EPI_E5M2, f8 = p.epi & (EPI_E4M3 | EPI_E5M2);
+    const bool f8 = p.epi & EPI_F8, a_e5m2 = p.epi & EPI_A_E5M2, b_e5m2 = p.epi & EPI_B_E5M2;
     const uint8_t* __restrict__ A8 = (const uint8_t*)p.a + bz * p.stride_a;
     const uint8_t* __restrict__ B8 = (const uint8_t*)p.b + bz * p.stride_b;
     uint16_t* __restrict__ C = p.c + bz * p.stride_c * (f32_out ? 2u : 1u);   // strides count elements of C
@@ -63,8 +63,8 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
                     uint32_t a8 = 0, b8 = 0;
                     if (am < M) a8 = A8[(uint64_t)am * lda + k];
                     if (bn < N) b8 = nt ? B8[(uint64_t)bn * ldb + k] : B8[(uint64_t)k * ldb + bn];
-                    av = fp8_to_bf16_bits(a8, e5m2);
-                    bv = fp8_to_bf16_bits(b8, e5m2);
+                    av = fp8_to_bf16_bits(a8, a_e5m2);
+                    bv = fp8_to_bf16_bits(b8, b_e5m2);
                 } else {
                     if (am < M) av = A[(uint64_t)am * lda + k];
                     if (bn < N) bv = nt ? B[(uint64_t)bn * ldb + k] : B[(uint64_t)k * ldb + bn];

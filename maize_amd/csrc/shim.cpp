@@ -294,8 +294,8 @@ int32_t maize_hip_gemm_ex_validate(const maize_gemm_ex_desc_t* x) {
     if (!d->a.ptr || !d->b.ptr || !d->c.ptr) return fail(MAIZE_ERR_NULL, "gemm: NULL matrix pointer");
     if (x->out_type != MAIZE_OUT_BF16 && x->out_type != MAIZE_OUT_F32)
         return fail(MAIZE_ERR_ARG, "gemm: unknown output type %u", x->out_type);
-    if (x->in_type > MAIZE_IN_E5M2) return fail(MAIZE_ERR_ARG, "gemm: unknown operand type %u", x->in_type);
-    const bool in8 = x->in_type == MAIZE_IN_E4M3 || x->in_type == MAIZE_IN_E5M2;
+    if (x->in_type > MAIZE_IN_E5M2_E4M3) return fail(MAIZE_ERR_ARG, "gemm: unknown operand type %u", x->in_type);
+    const bool in8 = x->in_type >= MAIZE_IN_E4M3;
     if (x->reserved) return fail(MAIZE_ERR_ARG, "gemm: reserved field must be 0");
     if (((uintptr_t)d->a.ptr | (uintptr_t)d->b.ptr) & (in8 ? 0u : 1u) || (uintptr_t)d->c.ptr & (x->out_type == MAIZE_OUT_F32 ? 3u : 1u))
         return fail(MAIZE_ERR_ALIGN, "gemm: matrix pointers must be aligned to their element size");
@@ -419,7 +419,9 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
     args.lda = x->lda; args.ldb = x->ldb; args.ldc = x->ldc;
     args.alpha = x->alpha; args.beta = x->beta;
     args.epi = (x->out_type == MAIZE_OUT_F32 ? 1u : 0u) | ((x->alpha != 1.0f || x->beta != 0.0f) ? 2u : 0u) |
-               (x->in_type == MAIZE_IN_F16 ? 4u : 0u) | (x->in_type == MAIZE_IN_E4M3 ? 8u : 0u) | (x->in_type == MAIZE_IN_E5M2 ? 16u : 0u);
+               (x->in_type == MAIZE_IN_F16 ? 4u : 0u) | (x->in_type >= MAIZE_IN_E4M3 ? 8u : 0u) |
+               ((x->in_type == MAIZE_IN_E5M2 || x->in_type == MAIZE_IN_E5M2_E4M3) ? 16u : 0u) |       // A is E5M2
+               ((x->in_type == MAIZE_IN_E5M2 || x->in_type == MAIZE_IN_E4M3_E5M2) ? 32u : 0u);        // B is E5M2
     maize::LaunchDims ld;
     memset(&ld, 0, sizeof ld);
     if (!ki.plan(*x, (uint32_t)ctx->prop.multiProcessorCount, &ld))

@@ -325,18 +325,18 @@ int mzo_ref_gemm_rows(const uint16_t* a, const uint16_t* b, uint32_t m,
 
 /* ---- 8-bit operands: the same arithmetic (exact products, fp64 sums in ascending k), C rounded once to bf16 ---- */
 
-int mzo_ref_gemm8(const uint8_t* a, const uint8_t* b, uint16_t* c,
-                  uint32_t m, uint32_t n, uint32_t k, int layout,
-                  uint32_t batch, uint64_t stride_a, uint64_t stride_b,
-                  uint64_t stride_c, double* c_f64, double* c_abs,
-                  uint32_t nthreads, int elem) {
+int mzo_ref_gemm8_ab(const uint8_t* a, const uint8_t* b, uint16_t* c,
+                     uint32_t m, uint32_t n, uint32_t k, int layout,
+                     uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                     uint64_t stride_c, double* c_f64, double* c_abs,
+                     uint32_t nthreads, int elem_a, int elem_b) {
     if (!a || !b || !c || batch == 0) return -1;
     if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
-    if (!is_fp8(elem)) return -1;
+    if (!is_fp8(elem_a) || !is_fp8(elem_b)) return -1;
     if (m == 0 || n == 0) return 0;
     for (uint32_t bi = 0; bi < batch; ++bi) {
-        float* bf = widen_b(b + bi * stride_b, n, k, layout, elem);
-        float* af = widen_a(a + bi * stride_a, NULL, m, k, elem);
+        float* bf = widen_b(b + bi * stride_b, n, k, layout, elem_b);
+        float* af = widen_a(a + bi * stride_a, NULL, m, k, elem_a);
         if (!bf || !af) { free(bf); free(af); return -1; }
         job_t j;
         memset(&j, 0, sizeof j);
@@ -356,18 +356,26 @@ int mzo_ref_gemm8(const uint8_t* a, const uint8_t* b, uint16_t* c,
     return 0;
 }
 
-int mzo_ref_gemm8_rows(const uint8_t* a, const uint8_t* b, uint32_t m,
-                       uint32_t n, uint32_t k, int layout, const uint32_t* rows,
-                       uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
-                       uint32_t nthreads, int elem) {
+int mzo_ref_gemm8(const uint8_t* a, const uint8_t* b, uint16_t* c,
+                  uint32_t m, uint32_t n, uint32_t k, int layout,
+                  uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                  uint64_t stride_c, double* c_f64, double* c_abs,
+                  uint32_t nthreads, int elem) {
+    return mzo_ref_gemm8_ab(a, b, c, m, n, k, layout, batch, stride_a, stride_b, stride_c, c_f64, c_abs, nthreads, elem, elem);
+}
+
+int mzo_ref_gemm8_rows_ab(const uint8_t* a, const uint8_t* b, uint32_t m,
+                          uint32_t n, uint32_t k, int layout, const uint32_t* rows,
+                          uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
+                          uint32_t nthreads, int elem_a, int elem_b) {
     if (!a || !b || !rows) return -1;
     if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
-    if (!is_fp8(elem)) return -1;
+    if (!is_fp8(elem_a) || !is_fp8(elem_b)) return -1;
     for (uint32_t r = 0; r < nsel; ++r)
         if (rows[r] >= m) return -1;
     if (n == 0 || nsel == 0) return 0;
-    float* bf = widen_b(b, n, k, layout, elem);
-    float* af = widen_a(a, rows, nsel, k, elem);
+    float* bf = widen_b(b, n, k, layout, elem_b);
+    float* af = widen_a(a, rows, nsel, k, elem_a);
     if (!bf || !af) { free(bf); free(af); return -1; }
     job_t j;
     memset(&j, 0, sizeof j);
@@ -384,4 +392,11 @@ int mzo_ref_gemm8_rows(const uint8_t* a, const uint8_t* b, uint32_t m,
     free(bf);
     free(af);
     return 0;
+}
+
+int mzo_ref_gemm8_rows(const uint8_t* a, const uint8_t* b, uint32_t m,
+                       uint32_t n, uint32_t k, int layout, const uint32_t* rows,
+                       uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
+                       uint32_t nthreads, int elem) {
+    return mzo_ref_gemm8_rows_ab(a, b, m, n, k, layout, rows, nsel, c, c_f64, c_abs, nthreads, elem, elem);
 }

@@ -114,6 +114,17 @@ int mzo_ref_gemm8_rows(const uint8_t* a, const uint8_t* b, uint32_t m,
                        uint32_t n, uint32_t k, int layout, const uint32_t* rows,
                        uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
                        uint32_t nthreads, int elem);
+/* A and B of different 8-bit types (the catalogue's (E4M3, E5M2) and (E5M2, E4M3) pairs,
+ * crates/maize_tile/src/mma/sm89.rs:28-45). */
+int mzo_ref_gemm8_ab(const uint8_t* a, const uint8_t* b, uint16_t* c,
+                     uint32_t m, uint32_t n, uint32_t k, int layout,
+                     uint32_t batch, uint64_t stride_a, uint64_t stride_b,
+                     uint64_t stride_c, double* c_f64, double* c_abs,
+                     uint32_t nthreads, int elem_a, int elem_b);
+int mzo_ref_gemm8_rows_ab(const uint8_t* a, const uint8_t* b, uint32_t m,
+                          uint32_t n, uint32_t k, int layout, const uint32_t* rows,
+                          uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
+                          uint32_t nthreads, int elem_a, int elem_b);
 
 #ifdef __cplusplus
 }

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libmaize_oracle.so")
 
 NN, NT = 0, 1
 BF16, F16, E4M3, E5M2 = 0, 1, 2, 3   # element types (MZO_ELEM_*); C of the 8-bit types is bf16
+E4M3_E5M2, E5M2_E4M3 = (2, 3), (3, 2)  # A and B of different 8-bit types: (type of A, type of B)
 _lib = None
 
 
@@ -54,6 +55,10 @@ def lib():
         L.mzo_ref_gemm8.argtypes = [vp, vp, vp, u32, u32, u32, C.c_int, u32, u64, u64, u64, vp, vp, u32, C.c_int]
         L.mzo_ref_gemm8_rows.restype = C.c_int
         L.mzo_ref_gemm8_rows.argtypes = [vp, vp, u32, u32, u32, C.c_int, vp, u32, vp, vp, vp, u32, C.c_int]
+        L.mzo_ref_gemm8_ab.restype = C.c_int
+        L.mzo_ref_gemm8_ab.argtypes = [vp, vp, vp, u32, u32, u32, C.c_int, u32, u64, u64, u64, vp, vp, u32, C.c_int, C.c_int]
+        L.mzo_ref_gemm8_rows_ab.restype = C.c_int
+        L.mzo_ref_gemm8_rows_ab.argtypes = [vp, vp, u32, u32, u32, C.c_int, vp, u32, vp, vp, vp, u32, C.c_int, C.c_int]
         _lib = L
     return _lib
 
@@ -67,7 +72,12 @@ def _p(a):
 
 
 def is_fp8(elem):
-    return elem in (E4M3, E5M2)
+    return elem in (E4M3, E5M2) or isinstance(elem, tuple)
+
+
+def _ab(elem):
+    """(type of A, type of B) of an 8-bit element code."""
+    return elem if isinstance(elem, tuple) else (elem, elem)
 
 
 def operand_dtype(elem):
@@ -87,8 +97,12 @@ def ref_gemm(a, b, m, n, k, layout=NN, batch=1, stride_a=None, stride_b=None, st
     c = np.zeros((batch - 1) * sc + m * n, dtype=np.uint16)
     f64 = np.empty((batch, m, n), dtype=np.float64) if want_f64 else None
     ab = np.empty((batch, m, n), dtype=np.float64) if want_abs else None
-    fn = lib().mzo_ref_gemm8 if is_fp8(elem) else lib().mzo_ref_gemm16
-    rc = fn(_p(a), _p(b), _p(c), m, n, k, layout, batch, sa, sb, sc, _p(f64), _p(ab), nthreads or default_threads(), elem)
+    if is_fp8(elem):
+        rc = lib().mzo_ref_gemm8_ab(_p(a), _p(b), _p(c), m, n, k, layout, batch, sa, sb, sc, _p(f64), _p(ab),
+                                    nthreads or default_threads(), *_ab(elem))
+    else:
+        rc = lib().mzo_ref_gemm16(_p(a), _p(b), _p(c), m, n, k, layout, batch, sa, sb, sc, _p(f64), _p(ab),
+                                  nthreads or default_threads(), elem)
     if rc != 0:
         raise ValueError("mzo_ref_gemm16 rejected its arguments")
     return c, f64, ab
@@ -103,8 +117,12 @@ def ref_gemm_rows(a, b, m, n, k, rows, layout=NN, want_abs=True, nthreads=None, 
     c = np.zeros((nsel, n), dtype=np.uint16)
     f64 = np.empty((nsel, n), dtype=np.float64)
     ab = np.empty((nsel, n), dtype=np.float64) if want_abs else None
-    fn = lib().mzo_ref_gemm8_rows if is_fp8(elem) else lib().mzo_ref_gemm16_rows
-    rc = fn(_p(a), _p(b), m, n, k, layout, _p(rows), nsel, _p(c), _p(f64), _p(ab), nthreads or default_threads(), elem)
+    if is_fp8(elem):
+        rc = lib().mzo_ref_gemm8_rows_ab(_p(a), _p(b), m, n, k, layout, _p(rows), nsel, _p(c), _p(f64), _p(ab),
+                                         nthreads or default_threads(), *_ab(elem))
+    else:
+        rc = lib().mzo_ref_gemm16_rows(_p(a), _p(b), m, n, k, layout, _p(rows), nsel, _p(c), _p(f64), _p(ab),
+                                       nthreads or default_threads(), elem)
     if rc != 0:
         raise ValueError("mzo_ref_gemm_rows rejected its arguments")
     return c, f64, ab

@@ -54,12 +54,14 @@ def test_every_registry_entry_has_its_device_kernel(kernels):
 
 def test_matrix_instruction_per_kernel(kernels):
     for name, ins in kernels.items():
-        if name.startswith(("maize_gemm_e4m3_", "maize_gemm_e5m2_")):
-            # 8-bit operands: the 64-deep instruction, format code in cbsz / blgp (E4M3 = 0: not printed)
+        if name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")):
+            # 8-bit operands: the 64-deep instruction.  B is fed as the first source, so cbsz carries B's format
+            # code and blgp A's (E4M3 = 0 is not printed, E5M2 = 1).
             f8 = [i for i in ins if i.startswith("v_mfma_f32_32x32x64_f8f6f4")]
             assert len(f8) >= 64 and count(ins, "v_mfma_f32_32x32x16") == 0, name   # two unrolled K steps of 128
-            assert all(("cbsz:1" in i and "blgp:1" in i) == name.startswith("maize_gemm_e5m2_") for i in f8), name
-            assert not any("cbsz" in i or "blgp" in i for i in f8) or name.startswith("maize_gemm_e5m2_"), name
+            tag = name[len("maize_gemm_"):].split("_")[0]
+            a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
+            assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
         elif "_mt256_" in name:
             want = "v_mfma_f32_32x32x16_f16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_32x32x16_bf16"
             other = "v_mfma_f32_32x32x16_bf16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_32x32x16_f16"

@@ -149,7 +149,7 @@ def test_dispatch_of_half_operands():
         if name.startswith("maize_gemm_f16_"):
             assert not _supports(name, ex(**big))
     with pytest.raises(mz.MaizeError) as e:
-        mz.validate(ex(in_type=5))
+        mz.validate(ex(in_type=9))
     assert e.value.code == _ffi.MAIZE_ERR_ARG
 
 
@@ -158,7 +158,8 @@ def test_dispatch_of_8bit_operands():
     boundaries and K % 16 == 0; everything else goes to the per-wave kernel.  One byte per element: odd operand
     pointers are valid."""
     big = dict(m=4096, n=4096, k=4096, layout=mz.LAYOUT_NT)
-    for it, name in ((mz.IN_E4M3, "maize_gemm_e4m3_mt256_nt"), (mz.IN_E5M2, "maize_gemm_e5m2_mt256_nt")):
+    for it, name in ((mz.IN_E4M3, "maize_gemm_e4m3_mt256_nt"), (mz.IN_E5M2, "maize_gemm_e5m2_mt256_nt"),
+                     (mz.IN_E4M3_E5M2, "maize_gemm_e4m3e5m2_mt256_nt"), (mz.IN_E5M2_E4M3, "maize_gemm_e5m2e4m3_mt256_nt")):
         x = ex(**big, in_type=it)
         plan = mz.gemm_plan(x)
         assert plan["kernel"] == name and tuple(plan["grid"]) == (256, 1, 1) and plan["workspace_bytes"] == 0
@@ -178,8 +179,8 @@ def test_dispatch_of_8bit_operands():
         assert mz.gemm_plan(ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"
         mz.validate(ex(**big, in_type=it, ptrs=(0x1001, 0x100003, 0x2000000)))
     for name in mz.kernel_names():
-        if name.startswith(("maize_gemm_e4m3_", "maize_gemm_e5m2_")):
+        if name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")):
             assert not _supports(name, ex(**big)) and not _supports(name, ex(**big, in_type=mz.IN_F16))
     with pytest.raises(mz.MaizeError) as e:
-        mz.validate(ex(in_type=4))
+        mz.validate(ex(in_type=6))
     assert e.value.code == _ffi.MAIZE_ERR_ARG

@@ -18,7 +18,8 @@ import maize_amd as mz
 
 pytestmark = pytest.mark.gpu
 
-FMT = {"e4m3": (mz.IN_E4M3, 2), "e5m2": (mz.IN_E5M2, 3)}      # name -> (in_type, oracle element code)
+# name -> (in_type, oracle element code: one code, or (type of A, type of B))
+FMT = {"e4m3": (mz.IN_E4M3, 2), "e5m2": (mz.IN_E5M2, 3), "e4m3e5m2": (mz.IN_E4M3_E5M2, (2, 3)), "e5m2e4m3": (mz.IN_E5M2_E4M3, (3, 2))}
 
 
 def _say(msg):
@@ -29,6 +30,10 @@ def f8_uniform(oracle, count, seed, elem, scale=1.0):
     """uniform[-scale, scale) rounded to the 8-bit format."""
     x = (np.random.default_rng(seed).random(count) * 2.0 - 1.0) * scale
     return oracle.fp8_bits_from_f64(x, elem)
+
+
+def ab_of(elem):
+    return elem if isinstance(elem, tuple) else (elem, elem)
 
 
 def launch(ctx, a, b, c0, m, n, k, layout, fmt, lda, ldb, ldc, alpha=1.0, beta=0.0, out_f32=False, kernel=None, batch=1,
@@ -56,8 +61,8 @@ def run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NT, fmt="e4m3", lda=None, ldb=
     lda = k if lda is None else lda
     ldb = bcols if ldb is None else ldb
     ldc = n if ldc is None else ldc
-    a = f8_uniform(oracle, m * lda, 100 + seed, elem)
-    b = f8_uniform(oracle, brows * ldb, 200 + seed, elem)
+    a = f8_uniform(oracle, m * lda, 100 + seed, ab_of(elem)[0])
+    b = f8_uniform(oracle, brows * ldb, 200 + seed, ab_of(elem)[1])
     if out_f32:
         c0 = (np.random.default_rng(seed).standard_normal(m * ldc) * 2).astype(np.float32)
     else:
@@ -237,3 +242,22 @@ def test_split_k_on_8bit_operands(ctx, oracle, fmt):
         da.free(); db.free(); dc.free()
     ref, val, ab = oracle.ref_gemm(a2, b2, m2, n2, k2, want_f64=True, want_abs=True)
     assert oracle.compare(got, ref, val[0], ab[0], k2)["n_fail"] == 0
+
+
+@pytest.mark.parametrize("fmt", ["e4m3e5m2", "e5m2e4m3"])
+def test_operands_of_different_8bit_formats(ctx, oracle, fmt):
+    """A of one format, B of the other (the catalogue's mixed pairs): per-wave kernel in both layouts, the three
+    macro-tile variants, and a check that the formats are not swapped (the same bytes the other way round differ)."""
+    for layout in (mz.LAYOUT_NN, mz.LAYOUT_NT):
+        assert run_f8(ctx, oracle, 100, 200, 72, layout=layout, fmt=fmt, kernel="maize_gemm_bf16_wave32", label="wave32 mixed") == "maize_gemm_bf16_wave32"
+    name = f"maize_gemm_{fmt}_mt256_nt"
+    assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, label="mixed plain") == name
+    assert run_f8(ctx, oracle, 300, 520, 144, fmt=fmt, alpha=-1.25, beta=0.75, label="mixed gen") == name + "_gen"
+    assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, label="mixed split-K") == name + "_splitk"
+    m = n = k = 256
+    a = f8_uniform(oracle, m * k, 41, 2)
+    b = f8_uniform(oracle, n * k, 42, 2)
+    got, _ = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n, kernel=name)
+    other = "e5m2e4m3" if fmt == "e4m3e5m2" else "e4m3e5m2"
+    swapped, _ = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, other, k, k, n, kernel=f"maize_gemm_{other}_mt256_nt")
+    assert not np.array_equal(got, swapped)
