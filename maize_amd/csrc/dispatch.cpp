@@ -330,6 +330,51 @@ bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDi
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
 }
 
+// ---- maize_gemm_*_skinny_nt: M <= 16 against B stored N x K, streamed once ---------------------
+// 16-bit (bf16 / half by launch flag) or 8-bit operands; rows of A and B on 16-byte boundaries,
+// K % 8 == 0 (16-bit) or K % 16 == 0 (8-bit), N % 8 == 0.
+bool skinny_nt_common(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    const uint32_t esz = fp8_in(d) ? 1u : 2u, per16 = 16u / esz;
+    if (nn(d) || s.m > 16u || (s.k % per16) || (s.n & 7u)) return false;
+    if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr | (uintptr_t)d.gemm.c.ptr) & 15u) return false;
+    if ((l.a % per16) || (l.b % per16) || (l.c & 7u)) return false;
+    if (d.gemm.batch > 1 && ((d.gemm.stride_a % per16) || (d.gemm.stride_b % per16) || (d.gemm.stride_c & 7u))) return false;
+    const uint64_t lim = 1ull << 31;
+    if (l.ext_a * esz >= lim || l.ext_b * esz >= lim || s.k >= (1u << 21) || l.b >= (1u << 21)) return false;
+    return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
+}
+bool skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && skinny_nt_common(d); }
+#define MAIZE_F8_SKINNY(tag, type) \
+    bool tag##_skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d); }
+MAIZE_F8_SKINNY(e4m3, MAIZE_IN_E4M3)
+MAIZE_F8_SKINNY(e5m2, MAIZE_IN_E5M2)
+MAIZE_F8_SKINNY(e4m3e5m2, MAIZE_IN_E4M3_E5M2)
+MAIZE_F8_SKINNY(e5m2e4m3, MAIZE_IN_E5M2_E4M3)
+#undef MAIZE_F8_SKINNY
+// K ranges: the smallest power of two that gives the grid ~7/8 of a workgroup per compute unit while
+// every range keeps at least 8 blocks of 128 bytes per row.
+bool skinny_nt_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const uint32_t cus = compute_units ? compute_units : 256u;
+    const uint32_t nblk = cdiv(s.k, fp8_in(d) ? 128u : 64u);
+    const uint64_t slabs = (uint64_t)cdiv(s.n, 256) * d.gemm.batch;
+    uint32_t ks = 1;
+    while (ks < 16u && slabs * ks * 8u < (uint64_t)cus * 7u && nblk / (2u * ks) >= 8u) ks *= 2;
+    ks = cdiv(nblk, cdiv(nblk, ks));                       // no empty range
+    ld->grid[0] = cdiv(s.n, 256);
+    ld->grid[1] = ks;
+    ld->grid[2] = d.gemm.batch;
+    ld->block[0] = 512; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0;
+    ld->ksplit = ks;
+    ld->split_first = 0;
+    ld->reduce_grid = 0;
+    ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * 16u * 256u * 4u : 0;
+    return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
+}
+
 const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_wave32", nullptr, wave32_supports, wave32_plan},
     {"maize_gemm_bf16_mt256_nn", nullptr, mt256_nn_supports, mt256_plan},
@@ -357,7 +402,9 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_packed", "maize_gemm_bf16_mt256_nt_splitk", packed_nt_supports, packed_plan},
     {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nn_splitk", packed_f16_nn_supports, packed_plan},
     {"maize_gemm_f16_mt256_nt_packed", "maize_gemm_f16_mt256_nt_splitk", packed_f16_nt_supports, packed_plan},
+    {"maize_gemm_bf16_skinny_nt", nullptr, skinny_nt_supports, skinny_nt_plan},
 #define MAIZE_F8_ENTRIES(tag) \
+    {"maize_gemm_" #tag "_skinny_nt", nullptr, tag##_skinny_nt_supports, skinny_nt_plan}, \
     {"maize_gemm_" #tag "_mt256_nt", nullptr, tag##_nt_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_gen", nullptr, tag##_nt_gen_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan},
@@ -384,6 +431,10 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         // size rule as below), else the per-wave kernel, which widens them to bf16 as it loads.
         static const char* const kTag[4] = {"e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"};
         char name[64];
+        // Few rows against N x K weights: bound by streaming B once.
+        std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nt", kTag[d.in_type - MAIZE_IN_E4M3]);
+        const int fk = kernel_index(name);
+        if (fk >= 0 && kKernels[fk].supports(d) && s.n >= 64 && s.k >= 1024) return (uint32_t)fk;
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_splitk", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fs = kernel_index(name);
         if (fs >= 0 && kKernels[fs].supports(d) && splitk_ranges(s, d.gemm.batch, compute_units, 128) >= 2u) return (uint32_t)fs;
@@ -395,6 +446,8 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // Few rows against a wide row-major B: bound by streaming B once.
     const int sk = kernel_index("maize_gemm_bf16_skinny_nn");
     if (sk >= 0 && kKernels[sk].supports(d) && s.n >= 64) return (uint32_t)sk;
+    const int st = kernel_index("maize_gemm_bf16_skinny_nt");
+    if (st >= 0 && kKernels[st].supports(d) && s.n >= 64 && s.k >= 512) return (uint32_t)st;
     // Few tiles and a long K: cut every tile into K ranges so that the whole chip works.
     static const char* const kSplitK[2][2] = {{"maize_gemm_bf16_mt256_nn_splitk", "maize_gemm_bf16_mt256_nt_splitk"},
                                               {"maize_gemm_f16_mt256_nn_splitk", "maize_gemm_f16_mt256_nt_splitk"}};

@@ -137,6 +137,20 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert p["workspace_bytes"] < (1 << 31)
         else:
             assert p["workspace_bytes"] == 0
+    elif name == "maize_gemm_bf16_skinny_nt":
+        assert p["block"] == (512, 1, 1)
+        assert layout == mz.LAYOUT_NT and m <= 16 and n % 8 == 0 and k % 8 == 0
+        ks = p["ksplit"]
+        nblk = cdiv(k, 64)                                     # blocks of 128 bytes per row
+        assert gx == cdiv(n, 256) and gy == ks and 1 <= ks <= 16
+        assert cdiv(nblk, ks) * (ks - 1) < nblk                # no empty range
+        if ks > 1:
+            assert nblk // ks >= 4                             # the 4-slot ring is filled at least once
+            assert gx * batch <= 16384
+            assert p["workspace_bytes"] >= TICKET_BYTES + gx * batch * ks * 16 * 256 * 4
+            assert p["workspace_bytes"] < (1 << 31)
+        else:
+            assert p["workspace_bytes"] == 0
     else:
         raise AssertionError(f"no invariants written for kernel {name}")
 
@@ -151,7 +165,9 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn",             # 64 tiles: partial tiles would cost more than they save
         (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",
         (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
-        (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",        # no skinny kernel for N x K weights
+        (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",              # N x K weights streamed once
+        (16, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",
+        (17, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",        # more than 16 rows
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
         (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_packed",      # odd N: B repacked, C written element-wise
         (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",

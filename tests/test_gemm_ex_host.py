@@ -176,7 +176,10 @@ def test_dispatch_of_8bit_operands():
         split = mz.gemm_plan(ex(64, 64, 4096, layout=mz.LAYOUT_NT, in_type=it))              # one tile, 32 K steps of 128
         assert split["kernel"] == name + "_splitk" and split["ksplit"] >= 2 and split["reduce_grid"] > 0
         assert split["workspace_bytes"] == 65536 + split["ksplit"] * 256 * 256 * 4
-        assert mz.gemm_plan(ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"
+        skinny = name.replace("_mt256_nt", "_skinny_nt")
+        assert mz.gemm_plan(ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny          # M <= 16: B streamed once
+        assert mz.gemm_plan(ex(17, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"
+        assert _supports(skinny, ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it)) and not _supports(skinny, x)
         mz.validate(ex(**big, in_type=it, ptrs=(0x1001, 0x100003, 0x2000000)))
     for name in mz.kernel_names():
         if name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")):
