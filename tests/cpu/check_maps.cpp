@@ -87,6 +87,28 @@ int main() {
         }
         std::printf("ok  K-contiguous tile: fragment reads are bank-conflict free\n");
     }
+    // ---- skinny NT kernel: a block is the same 256 x 128-byte tile; wave w issues pieces 4w .. 4w+3 and reads
+    // rows 32w .. 32w+31 (two groups of 16, lane l: row l%16, chunks given by l/16).  The loop has no barrier,
+    // which is only right if the rows a wave deposits are exactly the rows it reads.
+    {
+        for (uint32_t w = 0; w < 8; ++w) {
+            std::set<uint32_t> deposited, read;
+            for (uint32_t i = 0; i < 4; ++i)
+                for (uint32_t lane = 0; lane < 64; ++lane) deposited.insert(kc_piece_row(w * 4 + i, lane));
+            for (uint32_t c2 = 0; c2 < 2; ++c2)
+                for (uint32_t chunk = 0; chunk < 8; ++chunk) {
+                    uint32_t off[64];
+                    for (uint32_t lane = 0; lane < 64; ++lane) {
+                        const uint32_t row = (w * 2 + c2) * 16 + (lane & 15);
+                        read.insert(row);
+                        off[lane] = kc_offset(row, (chunk + (lane >> 4)) & 7);      // any chunk assignment per lane group
+                    }
+                    CHECK(passes_conflict_free(off, 16), "skinny NT operand read wave %u group %u chunk %u has bank conflicts", w, c2, chunk);
+                }
+            CHECK(deposited == read && read.size() == 32 && *read.begin() == 32 * w, "skinny NT wave %u reads rows it does not deposit", w);
+        }
+        std::printf("ok  skinny NT block: every wave reads exactly the rows it deposits, operand reads are bank-conflict free\n");
+    }
     // ---- K x N tile
     {
         std::set<uint32_t> seen;

@@ -68,7 +68,7 @@ def mt256_wave_program(nk, slots, nreads, barrier_quarter=3):
     return ops, steps
 
 
-def check_two_stage(ops, steps, nreads):
+def check_two_stage(ops, steps, nreads, parts=4):
     epoch = 0
     dma_epoch = {}          # (tile, piece) -> epoch of issue
     completed = set()       # (tile, piece) waited for by this wave
@@ -89,7 +89,7 @@ def check_two_stage(ops, steps, nreads):
             old = tile - 2
             if old >= 0 and last_read_epoch.get(old, -1) >= epoch:
                 raise Hazard(f"tile {tile} piece {pc} overwrites tile {old} in epoch {epoch}, still being read")
-            if old >= 0 and old < steps and reads_seen.get(old, 0) < 4 * nreads:
+            if old >= 0 and old < steps and reads_seen.get(old, 0) < parts * nreads:
                 raise Hazard(f"tile {tile} overwrites tile {old} before all of its fragments were read")
             dma_epoch[(tile, pc)] = epoch
             stage_of[tile] = stage
@@ -120,7 +120,7 @@ def check_two_stage(ops, steps, nreads):
                 consumed.append((tile, quarter))
     if pending:
         raise Hazard("requests still in flight at the end of the K loop")
-    want = [(t, q) for t in range(steps) for q in range(4)]
+    want = [(t, q) for t in range(steps) for q in range(parts)]
     if consumed != want:
         raise Hazard("K tiles not consumed exactly once, in order")
     for t in range(steps + 1):
@@ -158,6 +158,52 @@ def test_macro_tile_checker_rejects_broken_schedules():
     k = [i for i, o in enumerate(ops) if o == ("wait_all",)][3]
     with pytest.raises(Hazard):
         check_two_stage(ops[:k] + ops[k + 1:], steps, 8)
+
+
+# ---------------------------------------------------------------------------------------
+# 8-bit macro-tile kernel: the same two-stage ring, one K step = two halves of 16 MFMAs, the barrier
+# between them, all 16 requests of tile t+2 in the second half of step t
+# ---------------------------------------------------------------------------------------
+
+def f8_wave_program(nk, barrier_half=1, dma_half=1):
+    src = open(os.path.join(KDIR, "gemm_mt256_f8.hpp")).read()
+    step = src[src.index("auto step = "):src.index("// ---- prime")]
+    # the facts the model is built from, as the source states them
+    assert "if (kh == 1) {" in step and 's_waitcnt vmcnt(0) lgkmcnt(0)\\n\\ts_barrier' in step
+    assert "if (kh == 0) read_frag(1, 1, s, ca, cb);" in step
+    assert "read_frag(0, 0, s, na, nb);" in step and "dma(s, ca, cb, k_next);" in step
+    assert "for (int pc = 0; pc < 16; ++pc) dma(pc, A1, B1, k_begin + BK);" in src
+    ops = [("dma", 0, pc, 0) for pc in range(16)]
+    ops += [("wait_all",), ("barrier",)]
+    ops += [("read", 0, 0, 0)] * 16
+    ops += [("dma", 1, pc, 1) for pc in range(16)]
+    steps = nk + (nk & 1)
+    for t in range(steps):
+        cur, nxt = t & 1, (t & 1) ^ 1
+        for kh in range(2):
+            if kh == barrier_half:
+                ops += [("wait_all",), ("barrier",)]
+            for sl in range(16):
+                ops.append(("mfma", t, kh))
+                ops.append(("read", t, 1, cur) if kh == 0 else ("read", t + 1, 0, nxt))
+                if kh == dma_half:
+                    ops.append(("dma", t + 2, sl, cur))
+    ops.append(("wait_all",))
+    return ops, steps
+
+
+@pytest.mark.parametrize("nk", [1, 2, 3, 7, 32])
+def test_8bit_macro_tile_schedule_is_hazard_free(nk):
+    ops, steps = f8_wave_program(nk)
+    last_tile = check_two_stage(ops, steps, 16, parts=2)
+    assert last_tile == steps + 1
+
+
+def test_8bit_macro_tile_checker_rejects_broken_schedules():
+    with pytest.raises(Hazard):                 # requests in the first half: the stage still holds fragments to be read
+        check_two_stage(*f8_wave_program(8, dma_half=0), 16, parts=2)
+    with pytest.raises(Hazard):                 # barrier at the top of the step: tile t+1's reads race with its own landing
+        check_two_stage(*f8_wave_program(8, barrier_half=0), 16, parts=2)
 
 
 # ---------------------------------------------------------------------------------------
@@ -253,3 +299,72 @@ def test_skinny_checker_rejects_broken_rings():
     del swapped[i]                                                         # first barrier missing
     with pytest.raises(Hazard):
         check_ring(swapped, turns, lpr, ring)
+
+
+# ---------------------------------------------------------------------------------------
+# skinny NT kernel: 4-slot ring private to each wave (it fetches, reads and multiplies only its own 32
+# rows -- tests/cpu/check_maps.cpp proves that from the index maps), 6 loads per block, no barrier
+# ---------------------------------------------------------------------------------------
+
+def skinny_nt_constants():
+    src = open(os.path.join(KDIR, "gemm_skinny_nt.hpp")).read()
+    ring = int(re.search(r"constexpr int RING = (\d+);", src).group(1))
+    body = src[src.index("auto turn = "):]
+    waits = [int(x) for x in re.findall(r's_waitcnt vmcnt\((\d+)\)" ::: "memory"\);\n\s+__builtin_amdgcn_sched_barrier', body)]
+    assert len(waits) == 1 and "s_barrier" not in body[:body.index("request(0, s0, 0)")]
+    ahead = int(re.search(r"request\(b \+ (\d+), prev, pi\);", src).group(1))
+    primed = len(re.findall(r"request\(\d+, s\d+, \d+\);", src))
+    return ring, waits[0], primed, ahead
+
+
+def skinny_nt_wave_program(nb, ring, wait, primed, ahead):
+    ops = [("request", j, j % ring) for j in range(primed)]
+    turns = -(-nb // ring) * ring
+    for b in range(turns):
+        ops.append(("wait", wait))
+        ops.append(("request", b + ahead, (b + ahead) % ring))
+        ops.append(("consume", b, b % ring))
+    ops.append(("wait", 0))
+    return ops, turns
+
+
+def check_private_ring(ops, turns, loads_per_request):
+    issued, done, slot_holds, consumed = [], 0, {}, []
+    for op in ops:
+        if op[0] == "request":
+            _, blk, slot = op
+            old = slot_holds.get(slot)
+            if old is not None and old not in consumed:         # program order of one wave: its reads of `old` are behind it
+                raise Hazard(f"block {blk} overwrites block {old} before it is consumed")
+            slot_holds[slot] = blk
+            issued.append(blk)
+        elif op[0] == "wait":
+            done = max(done, len(issued) - -(-op[1] // loads_per_request))
+        elif op[0] == "consume":
+            _, blk, slot = op
+            if slot_holds.get(slot) != blk:
+                raise Hazard(f"block {blk} expected in slot {slot}, which holds {slot_holds.get(slot)}")
+            if blk not in issued[:done]:
+                raise Hazard(f"block {blk} consumed before its loads have landed")
+            consumed.append(blk)
+    if done != len(issued):
+        raise Hazard("loads still in flight at the end")
+    if consumed != list(range(turns)) or sorted(issued) != list(range(len(issued))):
+        raise Hazard("blocks not requested once and consumed once, in order")
+
+
+@pytest.mark.parametrize("nb", [4, 16, 32, 128, 9, 1])
+def test_skinny_nt_ring_is_hazard_free(nb):
+    ring, wait, primed, ahead = skinny_nt_constants()
+    assert primed == ring - 1 == ahead
+    ops, turns = skinny_nt_wave_program(nb, ring, wait, primed, ahead)
+    check_private_ring(ops, turns, 6)
+    assert wait == 6 * (primed - 1)                              # exactly the blocks behind the current one stay in flight
+
+
+def test_skinny_nt_checker_rejects_broken_rings():
+    ring, wait, primed, ahead = skinny_nt_constants()
+    with pytest.raises(Hazard):                                  # waits for one request too few
+        check_private_ring(*skinny_nt_wave_program(32, ring, wait + 6, primed, ahead), 6)
+    with pytest.raises(Hazard):                                  # refill aimed at the slot that is about to be read
+        check_private_ring(*skinny_nt_wave_program(32, ring - 1, wait, primed, ahead), 6)
