@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BF16 GEMM path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5|f8] [--kernel NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5|f8|f8s] [--kernel NAME]
 
 A step is one launch of maize_hip_gemm_bf16 on synthetic, seeded inputs that are already
 resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s (wall clock around exactly K
@@ -43,6 +43,9 @@ CONFIGS = {
     # Beside the five bf16 configurations: the same product on 8-bit operands (E4M3), both K-contiguous.
     "f8": dict(m=4096, n=4096, k=4096, nt=1, batch=1, da=("uniform",), db=("uniform",), bound="mfma", in_type="e4m3",
                label="E4M3 GEMM 4096x4096x4096 NT (bf16 C), uniform[-1,1) rounded to E4M3"),
+    # ... and the decode-style shape of cfg4 against 8-bit weights stored N x K.
+    "f8s": dict(m=16, n=14336, k=4096, nt=1, batch=1, da=("uniform",), db=("uniform",), bound="hbm", in_type="e4m3",
+                label="E4M3 GEMM 16x14336x4096 NT skinny (bf16 C), uniform[-1,1) rounded to E4M3"),
 }
 
 
@@ -130,7 +133,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", default=None, choices=sorted(CONFIGS) + ["copy"],
-                    help="cfg1..cfg5: a benchmark configuration; f8: 4096^3 on E4M3 operands; copy: the 256 MiB copy "
+                    help="cfg1..cfg5: a benchmark configuration; f8, f8s: 4096^3 and 16x14336x4096 on E4M3 operands; copy: the 256 MiB copy "
                          "used to scale HBM counters")
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -259,7 +262,7 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
 
     line = {
         "metric": "bf16 GEMM TFLOP/s at 4096^3 on 1 MI355X" if args.config == "cfg1"
-                  else "E4M3 GEMM TFLOP/s at 4096^3 on 1 MI355X" if f8 else f"bf16 GEMM TFLOP/s, {args.config}",
+                  else f"E4M3 GEMM TFLOP/s, {args.config}" if f8 else f"bf16 GEMM TFLOP/s, {args.config}",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8 (e4m3)" if f8 else "bf16", "data": "synthetic (seeded counter-based generators, inputs resident in HBM)",
