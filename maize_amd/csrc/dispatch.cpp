@@ -282,18 +282,135 @@ bool packed_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDi
     size_t bytes = kTicketBytes + (size_t)items * 262144u;
     ld->n_padded = p.n8; ld->k_padded = p.k8;
     if (p.a) {
-        ld->pack_a = PackPlan{true, s.m, s.k, l.a, s.m, p.k8, bytes};
+        ld->pack_a = PackPlan{true, s.m, s.k, l.a, s.m, p.k8, bytes, false, 2};
         bytes += (size_t)p.a_elems * d.gemm.batch * 2;
     }
     if (p.b) {
         const uint32_t brows = d.gemm.b.nrows, bcols = d.gemm.b.ncols;
-        ld->pack_b = PackPlan{true, brows, bcols, l.b, s.nt ? p.n8 : p.k8, s.nt ? p.k8 : p.n8, bytes};
+        ld->pack_b = PackPlan{true, brows, bcols, l.b, s.nt ? p.n8 : p.k8, s.nt ? p.k8 : p.n8, bytes, false, 2};
         bytes += (size_t)p.b_elems * d.gemm.batch * 2;
     }
     ld->workspace_bytes = bytes;
     const uint64_t runs = (uint64_t)s.m * cdiv(s.n, 8) * d.gemm.batch;
     if (cdiv64(runs, 256) > 0x7FFFFFFFull) return false;
     ld->reduce_grid = (uint32_t)cdiv64(runs, 256);
+    return true;
+}
+
+// ---- maize_gemm_{e4m3,...}_mt256_nt_packed: 8-bit operands in any layout, alignment, N and K --------
+// The 8-bit split-K kernels on compact N x K / M x K copies: a row-major (K x N) B is transposed as it is
+// copied (maize_pack_2d_u8), ragged or unaligned operands are zero-padded to K % 16 == 0; the reduce
+// pass writes C (element by element where its rows are not aligned).
+inline uint32_t up16(uint32_t x) { return (x + 15u) & ~15u; }
+struct Packing8 { bool a, b; uint32_t n8, k16; uint64_t a_elems, b_elems; };
+Packing8 packing8_of(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    Packing8 p;
+    p.n8 = up8(s.n); p.k16 = up16(s.k);
+    const bool strides_ok = d.gemm.batch == 1 || ((d.gemm.stride_a | d.gemm.stride_b) & 15u) == 0;
+    const bool k_odd = (s.k & 15u) != 0;
+    p.a = k_odd || (l.a & 15u) || ((uintptr_t)d.gemm.a.ptr & 15u) || !strides_ok;
+    p.b = !s.nt || k_odd || (s.n & 7u) || (l.b & 15u) || ((uintptr_t)d.gemm.b.ptr & 15u) || !strides_ok;   // N % 8: the padded rows must exist
+    p.a_elems = (uint64_t)s.m * p.k16;
+    p.b_elems = (uint64_t)p.n8 * p.k16;
+    return p;
+}
+maize_gemm_ex_desc_t packed_view8(const maize_gemm_ex_desc_t& d, const Packing8& p) {
+    maize_gemm_ex_desc_t v = d;
+    const Dims s = dims_of(d);
+    v.gemm.layout = MAIZE_LAYOUT_NT;
+    v.gemm.a.ncols = p.k16;
+    v.gemm.b.nrows = p.n8;
+    v.gemm.b.ncols = p.k16;
+    v.gemm.c.ncols = p.n8;
+    if (p.a) { v.gemm.a.ptr = (void*)16; v.lda = 0; v.gemm.stride_a = p.a_elems; }
+    if (p.b) { v.gemm.b.ptr = (void*)16; v.ldb = 0; v.gemm.stride_b = p.b_elems; }
+    v.gemm.c.ptr = (void*)16; v.ldc = 0; v.gemm.stride_c = (uint64_t)s.m * p.n8;   // C is not touched by the first pass
+    return v;
+}
+bool packed8_ok(const maize_gemm_ex_desc_t& d) {
+    if (!fp8_in(d)) return false;
+    const Packing8 p = packing8_of(d);
+    maize_gemm_ex_desc_t v = packed_view8(d, p);
+    v.gemm.c.nrows = dims_of(d).m;
+    if (!f8_nt_common(v)) return false;
+    const uint64_t copies = ((p.a ? p.a_elems : 0) + (p.b ? p.b_elems : 0)) * d.gemm.batch;
+    return copies <= (1ull << 31);
+}
+#define MAIZE_F8_PACKED(tag, type) \
+    bool tag##_packed_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && packed8_ok(d); }
+MAIZE_F8_PACKED(e4m3, MAIZE_IN_E4M3)
+MAIZE_F8_PACKED(e5m2, MAIZE_IN_E5M2)
+MAIZE_F8_PACKED(e4m3e5m2, MAIZE_IN_E4M3_E5M2)
+MAIZE_F8_PACKED(e5m2e4m3, MAIZE_IN_E5M2_E4M3)
+#undef MAIZE_F8_PACKED
+bool packed8_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    const Packing8 p = packing8_of(d);
+    const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(p.n8, 256) * d.gemm.batch;
+    Dims sv = s;
+    sv.n = p.n8; sv.k = p.k16; sv.nt = true;
+    const uint32_t ks = splitk_ranges(sv, d.gemm.batch, compute_units, 128);   // may be 1: the reduce pass still runs
+    const uint64_t items = tiles * ks;
+    if (items > 0x1FFFFFFFull || items * 262144ull > (1ull << 32)) return false;
+    uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+    ld->grid[0] = (resident && items > resident) ? resident : (uint32_t)items;
+    ld->grid[1] = 1; ld->grid[2] = 1;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0;
+    ld->ksplit = ks;
+    ld->split_first = 0;
+    size_t bytes = kTicketBytes + (size_t)items * 262144u;
+    ld->n_padded = p.n8; ld->k_padded = p.k16;
+    if (p.a) {
+        ld->pack_a = PackPlan{true, s.m, s.k, l.a, s.m, p.k16, bytes, false, 1};
+        bytes += (size_t)p.a_elems * d.gemm.batch;
+    }
+    if (p.b) {
+        // the copy is N x K: rows = N, cols = K of it are backed by the source, read transposed when B is K x N
+        ld->pack_b = PackPlan{true, s.n, s.k, l.b, p.n8, p.k16, bytes, !s.nt, 1};
+        bytes += (size_t)p.b_elems * d.gemm.batch;
+    }
+    ld->workspace_bytes = bytes;
+    const uint64_t runs = (uint64_t)s.m * cdiv(s.n, 8) * d.gemm.batch;
+    if (cdiv64(runs, 256) > 0x7FFFFFFFull) return false;
+    ld->reduce_grid = (uint32_t)cdiv64(runs, 256);
+    return true;
+}
+
+// ---- maize_gemm_{e4m3,...}_mt256_nt_trb[_gen]: 8-bit operands, row-major (K x N) B, everything else aligned ----
+// Only B needs a copy -- its transpose -- and the macro-tile kernel then writes C itself: no partial
+// tiles, no reduce pass.
+maize_gemm_ex_desc_t trb_view(const maize_gemm_ex_desc_t& d) {
+    maize_gemm_ex_desc_t v = d;
+    const Dims s = dims_of(d);
+    v.gemm.layout = MAIZE_LAYOUT_NT;
+    v.gemm.b.nrows = s.n; v.gemm.b.ncols = s.k;
+    v.gemm.b.ptr = (void*)16; v.ldb = 0; v.gemm.stride_b = (uint64_t)s.n * s.k;
+    return v;
+}
+bool trb_ok(const maize_gemm_ex_desc_t& d) {
+    if (!fp8_in(d) || !nn(d)) return false;
+    const Dims s = dims_of(d);
+    return f8_nt_common(trb_view(d)) && (uint64_t)s.n * s.k * d.gemm.batch <= (1ull << 31);
+}
+#define MAIZE_F8_TRB(tag, type) \
+    bool tag##_trb_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && trb_ok(d) && plain_epilogue(d); } \
+    bool tag##_trb_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && trb_ok(d); }
+MAIZE_F8_TRB(e4m3, MAIZE_IN_E4M3)
+MAIZE_F8_TRB(e5m2, MAIZE_IN_E5M2)
+MAIZE_F8_TRB(e4m3e5m2, MAIZE_IN_E4M3_E5M2)
+MAIZE_F8_TRB(e5m2e4m3, MAIZE_IN_E5M2_E4M3)
+#undef MAIZE_F8_TRB
+bool trb_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    if (!mt256_plan(trb_view(d), compute_units, ld)) return false;
+    ld->n_padded = s.n; ld->k_padded = s.k;                  // the launch runs on the copy's extents (unchanged here)
+    ld->pack_b = PackPlan{true, s.n, s.k, l.b, s.n, s.k, kTicketBytes, true, 1};
+    ld->workspace_bytes = kTicketBytes + (size_t)s.n * s.k * d.gemm.batch;
     return true;
 }
 
@@ -407,7 +524,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_" #tag "_skinny_nt", nullptr, tag##_skinny_nt_supports, skinny_nt_plan}, \
     {"maize_gemm_" #tag "_mt256_nt", nullptr, tag##_nt_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_gen", nullptr, tag##_nt_gen_supports, mt256_plan}, \
-    {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan},
+    {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_packed", "maize_gemm_" #tag "_mt256_nt_splitk", tag##_packed_supports, packed8_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_trb", "maize_gemm_" #tag "_mt256_nt", tag##_trb_supports, trb_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_trb_gen", "maize_gemm_" #tag "_mt256_nt_gen", tag##_trb_gen_supports, trb_plan},
     MAIZE_F8_ENTRIES(e4m3) MAIZE_F8_ENTRIES(e5m2) MAIZE_F8_ENTRIES(e4m3e5m2) MAIZE_F8_ENTRIES(e5m2e4m3)
 #undef MAIZE_F8_ENTRIES
 };
@@ -441,6 +561,21 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt%s", kTag[d.in_type - MAIZE_IN_E4M3], plain_epilogue(d) ? "" : "_gen");
         const int fi = kernel_index(name);
         if (fi >= 0 && kKernels[fi].supports(d) && (s.k >= 256 || (s.m >= 128 && s.n >= 128))) return (uint32_t)fi;
+        // A row-major B, odd extents or unaligned rows: transposed / padded copies and the split-K kernel, when the
+        // product is large enough to pay for the extra launches and the copies (same rule as for 16-bit operands).
+        // A row-major B with everything else aligned and enough tiles: only B is copied (transposed), no reduce pass.
+        std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_trb%s", kTag[d.in_type - MAIZE_IN_E4M3], plain_epilogue(d) ? "" : "_gen");
+        const int ft = kernel_index(name);
+        Dims st = s;
+        st.nt = true;
+        if (ft >= 0 && kKernels[ft].supports(d) && (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && s.m >= 24u &&
+            splitk_ranges(st, d.gemm.batch, compute_units, 128) < 2u)
+            return (uint32_t)ft;
+        std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_packed", kTag[d.in_type - MAIZE_IN_E4M3]);
+        const int fp = kernel_index(name);
+        if (fi >= 0 && !kKernels[fi].supports(d) && fp >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && s.m >= 24u && s.n >= 24u &&
+            kKernels[fp].supports(d))
+            return (uint32_t)fp;
         return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
     }
     // Few rows against a wide row-major B: bound by streaming B once.

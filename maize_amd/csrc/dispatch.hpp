@@ -12,9 +12,10 @@
 
 namespace maize {
 
-constexpr uint32_t kMaxKernels = 48;
+constexpr uint32_t kMaxKernels = 64;
 constexpr const char* kReduceKernel = "maize_gemm_splitk_reduce";
 constexpr const char* kPackKernel = "maize_pack_2d";
+constexpr const char* kPackKernelU8 = "maize_pack_2d_u8";
 
 // Repacking of one operand into the workspace before the launch (pack.hpp).
 struct PackPlan {
@@ -22,6 +23,8 @@ struct PackPlan {
     uint32_t rows, cols, ld_src;        // the operand as the caller gave it
     uint32_t rows_dst, cols_dst;        // the zero-padded compact copy
     size_t offset;                      // byte offset of the copy in the workspace
+    bool transpose;                     // 8-bit operands: the copy is the transpose of the source (rows, cols: the copy's orientation)
+    uint32_t elem_bytes;                // 2, or 1 for 8-bit operands (0 reads as 2)
 };
 
 struct LaunchDims {

@@ -1,4 +1,4 @@
-// maize_pack_2d: copies a matrix of 16-bit elements with any alignment and leading dimension into
+// maize_pack_2d, maize_pack_2d_u8: copy a matrix of 16-bit (8-bit) elements with any alignment and leading dimension into
 // a compact, 16-byte-aligned buffer whose extents are rounded up, zero-filling the padding.
 //
 // The macro-tile kernels move operands in 128-bit requests and so need 16-byte-aligned rows and
@@ -18,7 +18,7 @@ struct PackArgs {
     uint32_t rows, cols;          // extent of the source matrix
     uint32_t ld_src;              // elements between source rows
     uint32_t rows_dst, cols_dst;  // extent of the copy (>= source extent); its leading dimension is cols_dst
-    uint32_t pad;
+    uint32_t flags;               // maize_pack_2d_u8 only: bit 0 = the copy is the transpose of the source
     uint64_t stride_src, stride_dst;   // elements between batch members (grid.y)
 };
 static_assert(sizeof(PackArgs) == 56, "pack parameter block layout");
@@ -32,6 +32,37 @@ extern "C" __global__ __launch_bounds__(256) void maize_pack_2d(PackArgs p) {
     uint16_t v = 0;
     if (r < p.rows && c < p.cols) v = p.src[bz * p.stride_src + (uint64_t)r * p.ld_src + c];
     p.dst[bz * p.stride_dst + idx] = v;
+}
+
+// maize_pack_2d_u8: the same for 8-bit elements, optionally transposing: dst (rows_dst x cols_dst, compact)
+// receives element (r, c) of the source, or -- flags bit 0 -- element (c, r): the way a row-major
+// K x N operand of 8-bit floats becomes the N x K one the 8-bit macro-tile kernels take.  `rows`, `cols`
+// are the extent of the copy that is backed by the source (the rest is zero), in the copy's orientation.
+// One workgroup moves a 64 x 64 tile through LDS so that both the reads and the writes run along rows.
+extern "C" __global__ __launch_bounds__(256) void maize_pack_2d_u8(PackArgs p) {
+    __shared__ uint8_t tile[64][65];
+    const uint8_t* src = (const uint8_t*)p.src + (uint64_t)blockIdx.z * p.stride_src;
+    uint8_t* dst = (uint8_t*)p.dst + (uint64_t)blockIdx.z * p.stride_dst;
+    const bool tr = p.flags & 1u;
+    const uint32_t r0 = blockIdx.y * 64u, c0 = blockIdx.x * 64u;      // tile origin in the copy
+    const uint32_t tid = threadIdx.x, lo = tid & 63u, hi = tid >> 6;  // 64 consecutive lanes along a row
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t line = hi * 16u + i;                           // 0..63
+        // read along the source's rows: plain copy -> tile[line][lo] = (r0 + line, c0 + lo);
+        // transposing -> the source row is a column of the copy: tile[lo][line] = copy (r0 + lo, c0 + line)
+        const uint32_t r = tr ? r0 + lo : r0 + line, c = tr ? c0 + line : c0 + lo;
+        uint8_t v = 0;
+        if (r < p.rows && c < p.cols) v = tr ? src[(uint64_t)c * p.ld_src + r] : src[(uint64_t)r * p.ld_src + c];
+        if (tr) tile[lo][line] = v; else tile[line][lo] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t line = hi * 16u + i;
+        const uint32_t r = r0 + line, c = c0 + lo;
+        if (r < p.rows_dst && c < p.cols_dst) dst[(uint64_t)r * p.cols_dst + c] = tile[line][lo];
+    }
 }
 
 }  // namespace maize

@@ -80,7 +80,7 @@ struct maize_ctx {
     hipModule_t module;
     hipFunction_t fn[maize::kMaxKernels];
     hipFunction_t reduce_fn;
-    hipFunction_t pack_fn;
+    hipFunction_t pack_fn, pack_u8_fn;
     // Split-K scratch, one per stream so that launches on different streams never share it.
     std::unordered_map<void*, maize_workspace> workspaces;
 };
@@ -149,6 +149,7 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
     }
     e = hipModuleGetFunction(&ctx->reduce_fn, ctx->module, maize::kReduceKernel);
     if (e == hipSuccess) e = hipModuleGetFunction(&ctx->pack_fn, ctx->module, maize::kPackKernel);
+    if (e == hipSuccess) e = hipModuleGetFunction(&ctx->pack_u8_fn, ctx->module, maize::kPackKernelU8);
     if (e != hipSuccess) {
         int32_t rc = hip_fail(e, "helper kernels of the embedded code object");
         (void)hipModuleUnload(ctx->module);
@@ -443,12 +444,17 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
         static_assert(sizeof(pa) == 56, "pack parameter block");
         pa.src = which == 0 ? d->a.ptr : d->b.ptr;
         pa.dst = (char*)args.workspace + pp.offset;
-        pa.rows = pp.rows; pa.cols = pp.cols; pa.ld_src = pp.ld_src; pa.rows_dst = pp.rows_dst; pa.cols_dst = pp.cols_dst; pa.pad = 0;
+        pa.rows = pp.rows; pa.cols = pp.cols; pa.ld_src = pp.ld_src; pa.rows_dst = pp.rows_dst; pa.cols_dst = pp.cols_dst;
+        pa.pad = pp.transpose ? 1u : 0u;                     // flags of maize_pack_2d_u8
         pa.stride_src = d->batch > 1 ? (which == 0 ? d->stride_a : d->stride_b) : 0;
         pa.stride_dst = (uint64_t)pp.rows_dst * pp.cols_dst;
         const uint64_t total = (uint64_t)pp.rows_dst * pp.cols_dst;
-        const uint32_t pgrid[3] = {(uint32_t)((total + 255) / 256), d->batch, 1}, pblock[3] = {256, 1, 1};
-        int32_t prc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->pack_fn, pgrid, pblock, 0, stream, &pa, sizeof pa);
+        const bool u8 = pp.elem_bytes == 1;                  // 64 x 64 tiles through LDS, batch in grid.z; else one element per thread, batch in grid.y
+        const uint32_t pgrid[3] = {u8 ? (pp.cols_dst + 63u) / 64u : (uint32_t)((total + 255) / 256), u8 ? (pp.rows_dst + 63u) / 64u : d->batch,
+                                   u8 ? d->batch : 1u};
+        const uint32_t pblock[3] = {256, 1, 1};
+        int32_t prc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, u8 ? ctx->pack_u8_fn : ctx->pack_fn, pgrid, pblock, 0,
+                                 stream, &pa, sizeof pa);
         if (prc != MAIZE_OK) return prc;
         if (which == 0) { first.a = pa.dst; first.lda = 0; first.stride_a = pa.stride_dst; }
         else { first.b = pa.dst; first.ldb = 0; first.stride_b = pa.stride_dst; first.brows = pp.rows_dst; first.bcols = pp.cols_dst; }
@@ -456,8 +462,10 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
     if (ld.n_padded) {
         first.acols = ld.k_padded;
         first.ccols = ld.n_padded;
-        if (d->layout == MAIZE_LAYOUT_NN) { first.brows = ld.k_padded; first.bcols = ld.n_padded; }
+        const bool in8 = x->in_type >= MAIZE_IN_E4M3;        // 8-bit operands: the copy of a K x N B is N x K
+        if (d->layout == MAIZE_LAYOUT_NN && !in8) { first.brows = ld.k_padded; first.bcols = ld.n_padded; }
         else { first.brows = ld.n_padded; first.bcols = ld.k_padded; }
+        if (in8) first.layout = MAIZE_LAYOUT_NT;
     }
     int32_t rc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, ctx->fn[idx], ld.grid, ld.block,
                             ld.lds_bytes, stream, &first, sizeof first);

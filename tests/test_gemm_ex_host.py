@@ -166,12 +166,19 @@ def test_dispatch_of_8bit_operands():
         general = ex(**big, in_type=it, alpha=2.0, beta=1.0, out_type=mz.OUT_F32)
         assert mz.gemm_plan(general)["kernel"] == name + "_gen"
         for other in mz.kernel_names():
-            assert _supports(other, x) == (other in (name, name + "_gen", name + "_splitk", "maize_gemm_bf16_wave32")), other
-            assert _supports(other, general) == (other in (name + "_gen", name + "_splitk", "maize_gemm_bf16_wave32")), other
-        assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"            # row-major B
-        assert mz.gemm_plan(ex(4096, 4096, 4104, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"   # K % 16
-        assert mz.gemm_plan(ex(**big, in_type=it, ldb=4104))["kernel"] == "maize_gemm_bf16_wave32"             # rows off 16 bytes
-        assert mz.gemm_plan(ex(**big, in_type=it, ptrs=(0x1001, 0x100000, 0x2000000)))["kernel"] == "maize_gemm_bf16_wave32"
+            assert _supports(other, x) == (other in (name, name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32")), other
+            assert _supports(other, general) == (other in (name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32")), other
+        packed = name + "_packed"
+        nn_plan = mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))                                              # row-major B: transposed copy, nothing else
+        assert nn_plan["kernel"] == name + "_trb" and nn_plan["workspace_bytes"] == 65536 + 4096 * 4096 and nn_plan["reduce_grid"] == 0
+        assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it, beta=1.0))["kernel"] == name + "_trb_gen"
+        few = mz.gemm_plan(ex(64, 4096, 4096, in_type=it))                                                    # few tiles: split K on the copies
+        assert few["kernel"] == packed and few["ksplit"] >= 2 and few["workspace_bytes"] >= 65536 + 16 * few["ksplit"] * 262144 + 4096 * 4096
+        assert mz.gemm_plan(ex(4096, 4096, 4104, in_type=it))["kernel"] == packed                             # row-major B and K % 16
+        assert mz.gemm_plan(ex(4096, 4096, 4104, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == packed        # K % 16: padded copies
+        assert mz.gemm_plan(ex(**big, in_type=it, ldb=4104))["kernel"] == packed                              # rows off 16 bytes
+        assert mz.gemm_plan(ex(**big, in_type=it, ptrs=(0x1001, 0x100000, 0x2000000)))["kernel"] == packed
+        assert mz.gemm_plan(ex(100, 200, 72, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"               # too small to pay for the copies
         assert mz.gemm_plan(ex(64, 64, 64, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"
         split = mz.gemm_plan(ex(64, 64, 4096, layout=mz.LAYOUT_NT, in_type=it))              # one tile, 32 K steps of 128
         assert split["kernel"] == name + "_splitk" and split["ksplit"] >= 2 and split["reduce_grid"] > 0

@@ -172,10 +172,11 @@ def test_dispatch_of_8bit_products(ctx):
         return mz.gemm_plan(x, compute_units=256)["kernel"]
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt"
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nt"
-    assert pick(4096, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_bf16_wave32"      # row-major B: not K-contiguous
-    assert pick(4096, 4096, 4104, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_bf16_wave32"      # K % 16
-    assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3, lda=4104) == "maize_gemm_bf16_wave32"
+    assert pick(4096, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_trb"      # row-major B: transposed copy
+    assert pick(4096, 4096, 4104, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_packed"   # K % 16: padded copies
+    assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3, lda=4104) == "maize_gemm_e4m3_mt256_nt_packed"
     assert pick(64, 64, 64, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_bf16_wave32"
+    assert pick(100, 200, 72, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_bf16_wave32"               # too small to pay for the copies
 
 
 @pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
@@ -261,3 +262,37 @@ def test_operands_of_different_8bit_formats(ctx, oracle, fmt):
     other = "e5m2e4m3" if fmt == "e4m3e5m2" else "e4m3e5m2"
     swapped, _ = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, other, k, k, n, kernel=f"maize_gemm_{other}_mt256_nt")
     assert not np.array_equal(got, swapped)
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2e4m3"])
+def test_packed_path_for_8bit_operands(ctx, oracle, fmt):
+    """A row-major (K x N) B, odd K or N, unaligned rows: transposed / zero-padded copies in the workspace, the
+    split-K kernel on them, the reduce pass writing C.  Also with an odd pointer into the operands."""
+    name = f"maize_gemm_{fmt}_mt256_nt_packed"
+    NN, NT = mz.LAYOUT_NN, mz.LAYOUT_NT
+    assert run_f8(ctx, oracle, 512, 768, 384, layout=NN, fmt=fmt, kernel=name, label="packed NN") == name
+    assert run_f8(ctx, oracle, 300, 520, 1000, layout=NN, fmt=fmt, label="packed NN ragged") == name
+    # only B needs a copy (its transpose): the macro-tile kernel writes C itself
+    trb = f"maize_gemm_{fmt}_mt256_nt_trb"
+    assert run_f8(ctx, oracle, 1024, 2048, 512, layout=NN, fmt=fmt, label="trb") == trb
+    assert run_f8(ctx, oracle, 1000, 2056, 528, layout=NN, fmt=fmt, lda=544, ldb=2064, ldc=2072, label="trb views") == trb
+    assert run_f8(ctx, oracle, 1024, 2048, 512, layout=NN, fmt=fmt, alpha=-1.25, beta=0.75, label="trb gen") == trb + "_gen"
+    assert run_f8(ctx, oracle, 1024, 2048, 512, layout=NN, fmt=fmt, out_f32=True, label="trb f32") == trb + "_gen"
+    assert run_f8(ctx, oracle, 257, 263, 1031, layout=NN, fmt=fmt, label="packed NN odd N, K") == name
+    assert run_f8(ctx, oracle, 257, 263, 1031, layout=NT, fmt=fmt, label="packed NT odd N, K") == name
+    assert run_f8(ctx, oracle, 512, 768, 384, layout=NT, fmt=fmt, lda=391, ldb=397, ldc=771, label="packed NT odd ld") == name
+    assert run_f8(ctx, oracle, 512, 768, 392, layout=NN, fmt=fmt, alpha=-1.25, beta=0.75, label="packed NN scaled") == name
+    assert run_f8(ctx, oracle, 512, 768, 392, layout=NN, fmt=fmt, out_f32=True, ldc=776, label="packed NN f32") == name
+    assert run_f8(ctx, oracle, 64, 4096, 4096, layout=NN, fmt=fmt, label="packed NN few rows") == name
+    # batched, row-major B, padded strides: every member equals its single launch
+    elem = FMT[fmt][1]
+    m, n, k, batch = 256, 384, 512, 3
+    sa, sb, sc = m * k + 3, k * n + 5, m * n + 8
+    ab_ = f8_uniform(oracle, batch * sa, 61, ab_of(elem)[0])
+    bb_ = f8_uniform(oracle, batch * sb, 62, ab_of(elem)[1])
+    dense, took = launch(ctx, ab_, bb_, np.zeros(batch * sc, np.uint16), m, n, k, NN, fmt, k, n, n, batch=batch, strides=(sa, sb, sc))
+    assert took == name                                           # the odd strides make A unaligned too
+    for i in range(batch):
+        single, _ = launch(ctx, ab_[i * sa:i * sa + m * k], bb_[i * sb:i * sb + k * n], np.zeros(m * n, np.uint16), m, n, k, NN, fmt, k, n, n)
+        assert np.array_equal(single, dense[i * sc:i * sc + m * n]), i
+        assert not dense[i * sc + m * n:(i + 1) * sc].any(), "wrote between batch members"
