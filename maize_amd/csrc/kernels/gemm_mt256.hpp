@@ -6,19 +6,27 @@
 // intrinsics/cuda/cp_async.rs:92-210) re-designed for CDNA4:
 //
 //   * one workgroup of 4 wavefronts (2 x 2) owns a 256 x 256 tile of C; each
-//     wavefront owns a 128 x 128 sub-tile as 4 x 4 MFMA 32x32x16 accumulators
-//     (256 fp32 registers per lane, in AccVGPRs);
+//     wavefront owns a 128 x 128 sub-tile as 8 x 8 MFMA 16x16x32 accumulators
+//     (256 fp32 registers per lane, in AccVGPRs).  16x16x32 rather than 32x32x16:
+//     the same operand traffic from LDS, but 20 % less accumulator traffic per
+//     multiply-add, and under the board's power limit that is worth 8-10 % of
+//     run time on the large shapes;
 //   * K advances in steps of 64 through a two-stage LDS ring filled by 128-bit
 //     direct-to-LDS buffer loads (no register round trip; the hardware range
 //     check zero-fills the M/N/K edges, where the reference discards its
 //     ragged panels, src/main.rs:56-57);
+//   * a K step is four quarters of 32 MFMAs (K half x row half of the wave's
+//     sub-tile); the fragments of a quarter are read from LDS during the quarter
+//     before it, double-buffered in registers, by hand-placed ds_read
+//     instructions whose fragment and stage sit in the offset field (one address
+//     register per operand and K half) and hand-placed waits;
 //   * one barrier per K step, placed before the last quarter of the step's
 //     MFMAs: the fragments of that quarter are already in registers, so behind
 //     the barrier the first fragments of tile t+1 are read and the stage that
 //     held tile t is refilled with tile t+2 while the matrix pipe stays busy;
 //     the refill is spread over the last quarter of this step and the first
 //     quarter of the next one so the memory pipe sees a stream, not a burst;
-//   * LDS tiles are XOR-swizzled at 16-byte (K-contiguous tiles) or 64-byte
+//   * LDS tiles are XOR-swizzled at 16-byte (K-contiguous tiles) or 32-byte
 //     (row-major K x N tile) granularity so that the direct-to-LDS deposits,
 //     the 128-bit fragment reads and the transposing reads are all
 //     bank-conflict free without padding;
@@ -26,9 +34,11 @@
 //     row-major K x N B is read with ds_read_b64_tr_b16, which hands each lane
 //     the 4 K-consecutive values of its column;
 //   * MFMA is issued with B's fragment first, so each lane ends up holding 4
-//     consecutive columns of one row of C; the epilogue converts to bf16 (RNE)
-//     and stages the wave's sub-tile through LDS to store full 128-bit,
-//     row-contiguous segments with M/N edge masks.
+//     consecutive columns of one row of C; the MFMAs are inline assembly with
+//     the accumulator tied to itself, which keeps all 64 accumulator tuples in
+//     place across the loop; the epilogue converts to bf16 (RNE) and stages the
+//     wave's sub-tile through LDS to store full 128-bit, row-contiguous segments
+//     with M/N edge masks.
 //
 //   * a ragged N (or M) leaves a last column (row) of tiles that are almost empty but cost a full
 //     tile each, and can push the tile count just past a multiple of the CU count.  The _edge
@@ -39,7 +49,7 @@
 //
 // The _gen kernels are the plain (persistent) kernels with the general epilogue: C = alpha * A.B +
 // beta * C, C in bf16 or fp32.  maize_gemm_f16_mt256_* are the same kernels on IEEE half operands
-// (v_mfma_f32_32x32x16_f16; a 16-bit C is then half too).
+// (v_mfma_f32_16x16x32_f16; a 16-bit C is then half too).
 //
 // The _splitk kernels serve shapes with few tiles and a long K: every tile is cut into `ksplit` K
 // ranges, each (tile, range) is a work item that leaves an fp32 partial tile in the workspace, and
@@ -74,6 +84,8 @@ constexpr int kIssueSlot[16] = MAIZE_MT256_SCHED;
 #ifndef MAIZE_MT256_DMA_AUX
 #define MAIZE_MT256_DMA_AUX 0
 #endif
+constexpr bool sched_is_regular() { for (int i = 0; i < 16; ++i) if (kIssueSlot[i] != 2 * i + 1) return false; return true; }
+static_assert(sched_is_regular(), "the K loop issues piece pc at MFMA slot 2 * (2 pc + 1): keep the table in step with it");
 constexpr int early_pieces() { int n = 0; for (int i = 0; i < 16; ++i) n += kIssueSlot[i] < 16; return n; }
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
@@ -110,17 +122,16 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 
 template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK>
 __device__ __forceinline__ void body(const GemmArgs& p) {
-    // Four separate arrays (operand x ring stage): the compiler can then tell that a
-    // direct-to-LDS load into one stage does not alias fragment reads of the other, and does
-    // not make every read wait for the loads that were just issued.
-    __shared__ __attribute__((aligned(1024))) char lds_a0[TILE];
-    __shared__ __attribute__((aligned(1024))) char lds_a1[TILE];
-    __shared__ __attribute__((aligned(1024))) char lds_b0[TILE];
-    __shared__ __attribute__((aligned(1024))) char lds_b1[TILE];
+    // One array per operand, two ring stages each.  The fragment reads below are inline assembly (one
+    // base register per operand and K half, the stage and the fragment in the 16-bit offset field), so
+    // the compiler sees no read of these arrays and never makes one wait for the direct-to-LDS loads
+    // that are in flight; the waits are placed by hand.
+    __shared__ __attribute__((aligned(1024))) char lds_a[2 * TILE];
+    __shared__ __attribute__((aligned(1024))) char lds_b[2 * TILE];
     // Epilogue staging (8 KiB per wave), apart from the operand stages so that the first K tile
     // of the workgroup's next C tile can land while this one is converted and stored.
     __shared__ __attribute__((aligned(1024))) char lds_e[TILE];
-    lds_ptr const A0 = (lds_ptr)lds_a0, A1 = (lds_ptr)lds_a1, B0 = (lds_ptr)lds_b0, B1 = (lds_ptr)lds_b1;
+    lds_ptr const A0 = (lds_ptr)lds_a, A1 = A0 + TILE, B0 = (lds_ptr)lds_b, B1 = B0 + TILE;
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
     const uint32_t lda = lda_of(p), ldb = ldb_of(p), ldc = ldc_of(p);
@@ -175,7 +186,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     //   K-contiguous tile (A, and B when NT): piece = 8 rows of 128 B; position l -> row l/8,
     //     stored chunk l%8 = logical chunk ^ ((row>>1)&7).
     //   K x N tile (B when NN): piece = 2 rows of 512 B; position l -> row l/32, stored chunk
-    //     l%32 = logical chunk ^ ((row&3)<<2).
+    //     l%32 = logical chunk ^ (2 (row%4 + 4 bit3(row))) (maps::sk_*, the skinny kernel's block layout).
     // vo = byte offset of the lane's chunk at k = 0 (with the N-edge mask folded in); the K
     // advance is a scalar offset (plain kernels) or added per lane (K-tail kernels).
     uint32_t m0, n0;
@@ -222,8 +233,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             if (NT) {
                 b_vo[i] = ((n0 + row) * ldb + c * 8u) * 2u;
             } else {
-                const uint32_t brow = maps::kn_piece_row(wave * 8u + i, lane);
-                const uint32_t bc = maps::kn_piece_chunk(wave * 8u + i, lane);
+                const uint32_t brow = maps::sk_piece_row(wave * 8u + i, lane);
+                const uint32_t bc = maps::sk_piece_chunk(wave * 8u + i, lane);
                 b_vo[i] = ((brow * ldb + n0 + bc * 8u) * 2u) | ((n0 + bc * 8u) < N ? 0u : OOB);
             }
         }
@@ -250,41 +261,67 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     };
 
     // ---- fragment read maps ---------------------------------------------------
-    // MFMA 32x32x16: lane l holds row/col l%32 and k = 8*(l/32) + 0..7 of each 16-deep step.
-    const uint32_t l32 = lane & 31u, lhi = lane >> 5;
-    // Byte offsets of the lane's fragment reads inside a tile (maps.hpp): per kk for a K-contiguous
-    // tile (add 32 rows * 128 B per fragment), per j for the K x N tile (add kk * 16 and h * 4 rows).
-    uint32_t a_rd[4], b_rd[4];
+    // MFMA 16x16x32: lane l holds row/col l%16 and k = 8*(l/16) + 0..7 of each 32-deep step; a 64-deep
+    // K tile is two such steps (kh = 0, 1).  The wave's 128 x 128 sub-tile is 8 x 8 accumulators.
+    const uint32_t l16 = lane & 15u, lg = lane >> 4;
+    // Byte offsets of the lane's fragment reads inside a tile (maps.hpp): per kh for a K-contiguous tile
+    // (add 16 rows * 128 B per fragment), per j for the K x N tile (add kh * 32 and h * 4 rows).
+    // Base registers of the reads: LDS address of the operand's array + the lane's offset; everything
+    // else of an address (stage, fragment, K half of the K x N tile) is a compile-time offset.
+    uint32_t a_rd[2], b_rd[8];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) a_rd[kk] = maps::kc_frag_offset(wm * 128u, kk, lane);
+    for (int kh = 0; kh < 2; ++kh) a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * 128u, kh, lane);
     if (NT) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) b_rd[kk] = maps::kc_frag_offset(wn * 128u, kk, lane);
+        for (int kh = 0; kh < 2; ++kh) b_rd[kh] = (uint32_t)(uintptr_t)B0 + maps::kc_frag16_offset(wn * 128u, kh, lane);
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) b_rd[j] = maps::kn_tr_offset(wn * 128u, j, 0, 0, lane);
+        for (int j = 0; j < 8; ++j) b_rd[j] = (uint32_t)(uintptr_t)B0 + maps::sk_tr_offset(wn * 8u + j, 0, lane);
     }
 
+    // Fragment registers: A of one quarter (4 fragments), B of one half (8), each double-buffered.
+    // A quarter q = (kh = q / 2, rows 64 (q % 2) .. + 63 of the wave's 128): 32 MFMAs.
     bf16x8 fa[2][4];
-    bf16x8 fb[2][4];
-    short4v fbl[2][4], fbh[2][4];
-    constexpr int NREADS = NT ? 8 : 12;
-    // Read r of the fragments of quarter kk of the tile in (sa, sb) into buffer `buf`.
-    // Order: the operands of the first MFMA first.
-    auto read_frag = [&](int buf, int kk, int r, lds_ptr sa, lds_ptr sb) {
-        if (NT) {
-            if (r == 0) fa[buf][0] = *(lds_f8)(sa + a_rd[kk]);
-            else if (r <= 4) fb[buf][r - 1] = *(lds_f8)(sb + b_rd[kk] + (r - 1) * 32 * KROW);
-            else fa[buf][r - 4] = *(lds_f8)(sa + a_rd[kk] + (r - 4) * 32 * KROW);
-        } else {
-            typedef short4v __attribute__((address_space(3))) * v4p;
-            if (r == 0) fa[buf][0] = *(lds_f8)(sa + a_rd[kk]);
-            else if (r <= 8) {
-                const int j = (r - 1) >> 1, h = (r - 1) & 1;
-                short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(sb + b_rd[j] + kk * 16 * NROW + h * 4 * NROW));
-                if (h == 0) fbl[buf][j] = v; else fbh[buf][j] = v;
-            } else fa[buf][r - 8] = *(lds_f8)(sa + a_rd[kk] + (r - 8) * 32 * KROW);
+    bf16x8 fb[2][8];
+    short4v fbl[2][8], fbh[2][8];
+    constexpr int NB = NT ? 8 : 16;                     // reads that bring in the B fragments of one half
+    // Number of fragment reads quarter nq needs beyond what the quarter before it holds: a new half
+    // needs its B fragments and 4 A fragments, the second quarter of a half 4 A fragments.
+#define MAIZE_NREADS(nq) (((nq) & 1) ? 4 : 4 + NB)
+    // 128-bit read at base + 2048 * n (n = stage * 16 + fragment), 64-bit transposing read at
+    // base + 2048 * n (n = stage * 16 + kh * 8 + h).  The offsets are immediates: one case per value,
+    // folded away once the caller's loops are unrolled.
+#define MAIZE_RD_CASE(n) case n: asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(base), "n"((n) * 2048)); break;
+    auto lds_read128 = [&](bf16x8& dst, uint32_t base, int n) {
+        switch (n) {
+            MAIZE_RD_CASE(0) MAIZE_RD_CASE(1) MAIZE_RD_CASE(2) MAIZE_RD_CASE(3) MAIZE_RD_CASE(4) MAIZE_RD_CASE(5) MAIZE_RD_CASE(6) MAIZE_RD_CASE(7)
+            MAIZE_RD_CASE(16) MAIZE_RD_CASE(17) MAIZE_RD_CASE(18) MAIZE_RD_CASE(19) MAIZE_RD_CASE(20) MAIZE_RD_CASE(21) MAIZE_RD_CASE(22) MAIZE_RD_CASE(23)
+            default: __builtin_unreachable();
         }
+    };
+#undef MAIZE_RD_CASE
+#define MAIZE_RD_CASE(n) case n: asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(base), "n"((n) * 2048)); break;
+    auto lds_read_tr = [&](short4v& dst, uint32_t base, int n) {
+        switch (n) {
+            MAIZE_RD_CASE(0) MAIZE_RD_CASE(1) MAIZE_RD_CASE(8) MAIZE_RD_CASE(9) MAIZE_RD_CASE(16) MAIZE_RD_CASE(17) MAIZE_RD_CASE(24) MAIZE_RD_CASE(25)
+            default: __builtin_unreachable();
+        }
+    };
+#undef MAIZE_RD_CASE
+    // Read r of the fragments of quarter nq of the tile in stage st (0, 1); the operands of the quarter's
+    // first MFMA first.  A goes to buffer nq % 2, B to buffer (nq / 2) % 2.
+    auto read_for = [&](int nq, int r, int st) {
+        const int kh = nq >> 1, rh = nq & 1;
+        if (rh == 1) { lds_read128(fa[1][r], a_rd[kh], st * 16 + 4 + r); return; }
+        if (r == 0) lds_read128(fa[0][0], a_rd[kh], st * 16);
+        else if (r <= NB) {
+            if (NT) lds_read128(fb[kh][r - 1], b_rd[kh], st * 16 + r - 1);
+            else {
+                const int j = (r - 1) >> 1, h = (r - 1) & 1;      // rows 32 kh + 4 h + ...: 16 KiB and 2 KiB further on
+                if (h == 0) lds_read_tr(fbl[kh][j], b_rd[j], st * 16 + kh * 8);
+                else        lds_read_tr(fbh[kh][j], b_rd[j], st * 16 + kh * 8 + 1);
+            }
+        } else lds_read128(fa[0][r - NB], a_rd[kh], st * 16 + r - NB);
     };
     auto b_operand = [&](int buf, int j) -> bf16x8 {
         if (NT) return fb[buf][j];
@@ -293,18 +330,21 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         return __builtin_bit_cast(bf16x8, r);
     };
 
-    floatx16 acc[4][4];
+    floatx4 acc[8][8];
     uint32_t k_early = 0;                  // tile whose early pieces are issued next (last quarter of a step)
     uint32_t k_late = 0;                   // tile whose late pieces are issued next (first quarter of a step)
 
     // ---- steady state ----------------------------------------------------------------
-    // One K step.  On entry: (ca, cb) hold tile t, fragment buffer 0 holds its quarter-0
-    // fragments, the early pieces of tile t+1 are landing in (na, nb).
-    auto step = [&](lds_ptr ca, lds_ptr cb, lds_ptr na, lds_ptr nb) {
+    // One K step.  On entry: (ca, cb) hold tile t, the fragment buffers hold its quarter-0 fragments,
+    // the early pieces of tile t+1 are landing in (na, nb).
+    auto step = [&](int cur) {
+        lds_ptr const ca = A0 + cur * TILE, cb = B0 + cur * TILE, na = A0 + (cur ^ 1) * TILE, nb = B0 + (cur ^ 1) * TILE;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            const int buf = kk & 1;
-            if (kk == 3) {
+        for (int q = 0; q < 4; ++q) {
+            const int kh = q >> 1, rh = q & 1;
+            // The fragments of this quarter were requested during the one before: they have to be in.
+            if (q < 3) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (q == 3) {
                 // Every fragment this step still needs from (ca, cb) is in registers.  Wait until
                 // this wave's share of tile t+1 has landed, then meet the other waves: after the
                 // barrier (na, nb) is complete and (ca, cb) is free to be refilled with tile t+2.
@@ -313,29 +353,28 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 MAIZE_FENCE();
             }
 #pragma unroll
-            for (int s = 0; s < 16; ++s) {
+            for (int s = 0; s < 32; ++s) {
+                const int i = 4 * rh + (s >> 3), j = s & 7;
+                // The accumulator is tied to itself ("+a"): left to the register allocator, a few of the 64
+                // tuples were renamed across the loop and copied back through VGPRs at its end.  (Each
+                // accumulator comes up again 32 MFMAs later: no dependent back-to-back issue.)
                 if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
-                    acc[s >> 2][s & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                        __builtin_bit_cast(halfx8, b_operand(buf, s & 3)), __builtin_bit_cast(halfx8, fa[buf][s >> 2]),
-                        acc[s >> 2][s & 3], 0, 0, 0);
+                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(kh, j)), "v"(fa[rh][s >> 3]));
                 else
-                    acc[s >> 2][s & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_operand(buf, s & 3), fa[buf][s >> 2],
-                                                                                acc[s >> 2][s & 3], 0, 0, 0);
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(kh, j)), "v"(fa[rh][s >> 3]));
                 // Side work of this slot: fragment reads for the next quarter ...
-                if (s < NREADS) {
-                    if (kk < 3) read_frag(buf ^ 1, kk + 1, s, ca, cb);
-                    else        read_frag(buf ^ 1, 0, s, na, nb);
+                if (s < MAIZE_NREADS((q + 1) & 3)) {
+                    if (q < 3) read_for(q + 1, s, cur);
+                    else       read_for(0, s, cur ^ 1);
                 }
-                // ... and the direct-to-LDS requests scheduled for this slot: late pieces of tile
-                // t+1 (its stage was freed by the previous barrier) in the first three quarters,
-                // early pieces of tile t+2 behind this step's barrier.
-                const int slot = kk == 3 ? s : 16 * (kk + 1) + s;
-#pragma unroll
-                for (int pc = 0; pc < 16; ++pc)
-                    if (kIssueSlot[pc] == slot) {
-                        if (kk == 3) dma(pc, ca, cb, k_early);
-                        else         dma(pc, na, nb, k_late);
-                    }
+                // ... and the direct-to-LDS requests scheduled for this slot (kIssueSlot counts slots of
+                // two of these MFMAs): late pieces of tile t+1 (its stage was freed by the previous
+                // barrier) in the first three quarters, early pieces of tile t+2 behind this step's barrier.
+                const int slot = q == 3 ? s : 32 * (q + 1) + s;
+                if ((slot & 3) == 2 && slot < 64) {            // piece pc goes out at slot 4 pc + 2 = 2 kIssueSlot[pc]
+                    if (q == 3) dma(slot >> 2, ca, cb, k_early);
+                    else        dma(slot >> 2, na, nb, k_late);
+                }
                 MAIZE_FENCE();
             }
         }
@@ -348,15 +387,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
     for (;;) {                                                  // one trip per C tile
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     // The wait also covers the C stores of the previous tile (loads and stores share the counter).
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-    for (int r = 0; r < NREADS; ++r) read_frag(0, 0, r, A0, B0);
+    for (int r = 0; r < MAIZE_NREADS(0); ++r) read_for(0, r, 0);
 #pragma unroll
     for (int pc = 0; pc < early_pieces(); ++pc) dma(pc, A1, B1, k_begin + BK);   // tile 1, early pieces
     k_early = k_begin + 2 * BK;
@@ -364,18 +401,20 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // Two steps per trip so that each step sees its stages as compile-time constants.  An odd
     // step count runs one extra step on an all-zero tile (loads past K return zeros).
     for (uint32_t kt = 0; kt < nk; kt += 2) {
-        step(A0, B0, A1, B1);
-        step(A1, B1, A0, B0);
+        step(0);
+        step(1);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // every direct-to-LDS write of this tile has landed
+    // every direct-to-LDS write of this tile has landed; the last MFMAs have left the pipe before the
+    // epilogue reads their accumulators (the assembler-level MFMAs are invisible to the hazard recognizer)
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 7\n\ts_nop 7" ::: "memory");
 
     // ---- K ranges: publish the partial tile, take a ticket, last arriver sums in range order ----
     constexpr int COHERENT = 17;                          // buffer cache policy sc0 | sc1: visible across the XCDs' L2s
     constexpr uint32_t UNIT = BM * BN * 4u;               // one fp32 partial tile
     constexpr uint32_t DROP = 0xFFFFFFF0u;                // out-of-range offset: store dropped, load returns zeros
-    // A partial tile is stored in register order, not row-major: chunk c = (i, j, q) of wave w is
+    // A partial tile is stored in register order, not row-major: chunk c = (i, j) of wave w is
     // 64 lanes x 16 bytes = 1 KiB contiguous, so every store and load instruction moves whole
-    // cache lines.  Lane's chunk = row wm*128 + i*32 + l%32, columns wn*128 + j*32 + 8q + 4(l/32)
+    // cache lines.  Lane's chunk = row wm*128 + i*16 + l%16, columns wn*128 + j*16 + 4(l/16)
     // + 0..3.  Chunks wholly outside the matrix are skipped (a wave-uniform test); lanes outside
     // it inside a chunk use an out-of-range offset.
     const uint32_t nedge = mode == 1u ? tm : tn;
@@ -385,18 +424,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t wmu = wave_u >> 1, wnu = wave_u & 1u;
     const uint32_t lane_off = wave_u * 65536u + lane * 16u;
     const uint32_t rows_ok = M - m0, cols_ok = N - n0;    // valid extent of this tile (may exceed 256)
-    auto chunk_live = [&](int c) { return wmu * 128u + (c >> 4) * 32u < rows_ok && wnu * 128u + ((c >> 2) & 3) * 32u + (c & 3) * 8u < cols_ok; };
-    auto lane_live = [&](int c) { return wm * 128u + (c >> 4) * 32u + l32 < rows_ok && wn * 128u + ((c >> 2) & 3) * 32u + (c & 3) * 8u + lhi * 4u < cols_ok; };
+    auto chunk_live = [&](int c) { return wmu * 128u + (c >> 3) * 16u < rows_ok && wnu * 128u + (c & 7) * 16u < cols_ok; };
+    auto lane_live = [&](int c) { return wm * 128u + (c >> 3) * 16u + l16 < rows_ok && wn * 128u + (c & 7) * 16u + lg * 4u < cols_ok; };
     if (EDGE && split) {
         volatile uint32_t& ticket = *(volatile uint32_t*)lds_e;   // the staging region is idle until the epilogue
         uint32_t* counters = (uint32_t*)p.workspace;      // 16384 counters (zero between launches), then the tiles
 #pragma unroll
         for (int c = 0; c < 64; ++c) {
             if (!chunk_live(c)) continue;
-            const int i = c >> 4, j = (c >> 2) & 3, q = c & 3;
             const uint32_t off = lane_live(c) ? (slot * ks + z) * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
-            const floatx4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rws, off, 0, COHERENT);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[c >> 3][c & 7]), rws, off, 0, COHERENT);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of the tile has reached memory
         __syncthreads();
@@ -439,9 +476,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
     // ---- epilogue: fp32 -> bf16 (RNE), stage through LDS, 128-bit row stores --------------
     // Each wave stages its 128 x 128 sub-tile 32 rows at a time in a private 8 KiB region
-    // (row = 256 B).  The 16-byte chunk index is XOR-ed with row%16 and the 8-byte half with
-    // bit 4 of the row, so the 8-byte writes of 32 rows and the 16-byte reads of 4 rows are
-    // conflict free.  The region is wave-private and LDS operations of one wave complete in
+    // (row = 256 B).  The 16-byte chunk index is XOR-ed with row%16, so the 8-byte writes of 16
+    // rows and the 16-byte reads of 4 rows are conflict free (maps::epi16_*).  The region is wave-private and LDS operations of one wave complete in
     // order, so no barrier is needed between the passes.
     if (GEN) {
         // General epilogue (alpha, beta, fp32 C): the sub-tile is staged as fp32, 32 rows x 64 columns
@@ -449,26 +485,28 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // consecutive columns of a row and finished by store_c_run.
         lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
         const uint32_t c8 = lane & 7u, r8 = lane >> 3;           // 8 lanes per 64-column row, 8 rows per read
+        // Split-K: the lane's place inside the partial tile.  Recomputed per tile on purpose (the empty
+        // asm makes it opaque): hoisted out of the tile loop, the 32 addresses derived from it would
+        // be kept live across the K loop and spilled.
+        uint32_t lane_part = (wm * 128u + r8) * BN + wn * 128u + c8 * 8u;
+        asm volatile("" : "+v"(lane_part));
+        float* const part_base = (float*)((char*)p.workspace + 65536) + (uint64_t)eslot * (BM * BN) + lane_part;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i)                              // 32 rows per pass: accumulator rows 2i, 2i+1
 #pragma unroll
             for (int jh = 0; jh < 2; ++jh) {
 #pragma unroll
-                for (int jj = 0; jj < 2; ++jj)
+                for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int j = jh * 2 + jj;
-                        // lane holds C[row = i*32 + l32][col = j*32 + 8q + 4*lhi + 0..3]
-                        const floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                        const uint32_t chunk = ((uint32_t)(jj * 8 + q * 2) + lhi) ^ (l32 & 15u);
-                        *(__attribute__((address_space(3))) floatx4*)(ew + l32 * 256u + chunk * 16u) = f;
-                    }
+                    for (int jj = 0; jj < 4; ++jj)
+                        // lane holds C[row = (2i+ii)*16 + l16][col = (4jh+jj)*16 + 4*lg + 0..3]
+                        *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_write_offset(ii, jj, lane)) = acc[2 * i + ii][4 * jh + jj];
                 const uint32_t gcol = en0 + wn * 128u + jh * 64u + c8 * 8u;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const uint32_t row = r * 8 + r8;                 // 0..31 within the pass
-                    const floatx4 lo = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8) ^ (row & 15u)) * 16u));
-                    const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + row * 256u + (((2u * c8 + 1u) ^ (row & 15u)) * 16u));
+                    const uint32_t row = maps::epi32_read_row(r, lane);     // 0..31 within the pass
+                    const floatx4 lo = *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_read_offset(r, 0, lane));
+                    const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_read_offset(r, 1, lane));
                     const uint32_t grow = em0 + wm * 128u + i * 32u + row;
                     if (gcol < N && grow < M) {                   // N % 8 == 0: a run is all in or all out
                         if (SPLITK) {
@@ -476,7 +514,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                             // of ticket counters every workspace starts with (other kernels on the stream rely
                             // on finding them zero); the reduce kernel adds the ranges in order and applies
                             // the epilogue.
-                            float* part = (float*)((char*)p.workspace + 65536) + (uint64_t)eslot * (BM * BN) + (grow - em0) * BN + (gcol - en0);
+                            float* part = part_base + (uint32_t)((i * 32 + r * 8) * BN + jh * 64);
                             *(floatx4*)part = lo;
                             *(floatx4*)(part + 4) = hi;
                         } else {
@@ -501,19 +539,18 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     #pragma unroll
         for (int i = 0; i < 4; ++i) {
     #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int ii = 0; ii < 2; ++ii)                       // 32 rows per pass: accumulator rows 2i, 2i+1
     #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    // lane holds C[row = i*32 + l32][col = j*32 + 8q + 4*lhi + 0..3]
-                    floatx4 f = {acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                    if (EDGE && split) f = reduced_chunk(i * 16 + j * 4 + q);
+                for (int j = 0; j < 8; ++j) {
+                    // lane holds C[row = (2i+ii)*16 + l16][col = j*16 + 4*lg + 0..3]
+                    floatx4 f = acc[2 * i + ii][j];
+                    if (EDGE && split) f = reduced_chunk((2 * i + ii) * 8 + j);
                     u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
-                    *(lds_v2)(ew + maps::epi_write_offset(j, q, lane)) = v;
+                    *(lds_v2)(ew + maps::epi16_write_offset(ii, j, lane)) = v;
                 }
     #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                u32x4 v = *(lds_v4)(ew + maps::epi_read_offset(r, lane));
-                if ((r >> 2) & 1) v = u32x4{v.z, v.w, v.x, v.y};     // rows with bit 4 set hold their halves swapped
+                const u32x4 v = *(lds_v4)(ew + maps::epi16_read_offset(r, lane));
                 __builtin_amdgcn_raw_buffer_store_b128(v, rc, c_vo, (uint32_t)(i * 32 + r * 4) * row_bytes, 2 /* nt */);
             }
         }
@@ -523,6 +560,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }  // C tiles
 }
 
+#undef MAIZE_NREADS
 }  // namespace mt256
 
 #define MAIZE_MT256_KERNEL(name, nt, ktail, edge) \

@@ -31,39 +31,20 @@ MAIZE_MAP uint32_t kc_piece_row(uint32_t piece, uint32_t lane) { return piece * 
 MAIZE_MAP uint32_t kc_piece_chunk(uint32_t piece, uint32_t lane) { return (lane & 7u) ^ kc_swizzle(kc_piece_row(piece, lane)); }
 // Byte offset of logical chunk `chunk` (0..7) of row `row` in the tile.
 MAIZE_MAP uint32_t kc_offset(uint32_t row, uint32_t chunk) { return row * 128u + ((chunk ^ kc_swizzle(row)) * 16u); }
-// Fragment read of MFMA 32x32x16: lane l holds row base + l%32, k = 16 kk + 8 (l/32) + 0..7.
-MAIZE_MAP uint32_t kc_frag_offset(uint32_t row_base, uint32_t kk, uint32_t lane) {
-    return kc_offset(row_base + (lane & 31u), 2u * kk + (lane >> 5));
+// Fragment read of MFMA 16x16x32: lane l holds row base + l%16, k = 32 kh + 8 (l/16) + 0..7.  The swizzle has
+// period 16 rows, so fragment f of a wave (rows base + 16 f ..) sits 2048 f bytes further on: the kernel keeps
+// one address register per kh and puts the fragment (and the ring stage) into the instruction's offset field.
+MAIZE_MAP uint32_t kc_frag16_offset(uint32_t row_base, uint32_t kh, uint32_t lane) {
+    return kc_offset(row_base + (lane & 15u), 4u * kh + (lane >> 4));
 }
-
 // Fragment read of MFMA 32x32x64 on 8-bit elements (the same tile: 128 elements per row): lane l
 // holds row base + l%32 and the 32 bytes k = 64 kh + 32 (l/32) + 0..31, read as two chunks (c01 = 0, 1).
 MAIZE_MAP uint32_t kc_frag8_offset(uint32_t row_base, uint32_t kh, uint32_t c01, uint32_t lane) {
     return kc_offset(row_base + (lane & 31u), 4u * kh + 2u * (lane >> 5) + c01);
 }
 
-// ---- K x N operand tile of the macro-tile kernel (row-major B): 64 rows of 512 B ---------------------
-// Piece p (2 rows): lane l lands at row 2p + l/32, position l%32.  64-byte granules are XOR-ed with row%4.
-MAIZE_MAP uint32_t kn_swizzle(uint32_t row) { return (row & 3u) << 2; }
-MAIZE_MAP uint32_t kn_piece_row(uint32_t piece, uint32_t lane) { return piece * 2u + (lane >> 5); }
-MAIZE_MAP uint32_t kn_piece_chunk(uint32_t piece, uint32_t lane) { return (lane & 31u) ^ kn_swizzle(kn_piece_row(piece, lane)); }
-MAIZE_MAP uint32_t kn_offset(uint32_t row, uint32_t chunk) { return row * 512u + ((chunk ^ kn_swizzle(row)) * 16u); }
-// Transposing read (ds_read_b64_tr_b16): in each group of 16 lanes, lane q addresses 4 consecutive
-// columns (q%4) of row q/4 of a 4 x 16 block and receives column q, rows 0..3.  For MFMA 32x32x16 with
-// B first, lane l needs column col_base + 32 j + l%32 ... i.e. group (l/16)%2 covers columns 16..31 of
-// the 32-column fragment j, and l/32 selects k = 8 (l/32) + 4 h + 0..3 of the 16-deep step kk.
-// Address of lane l for fragment j, step kk, half h (rows 4h..4h+3 of the lane's 8):
-MAIZE_MAP uint32_t kn_tr_row(uint32_t kk, uint32_t h, uint32_t lane) { return kk * 16u + (lane >> 5) * 8u + h * 4u + ((lane & 15u) >> 2); }
-MAIZE_MAP uint32_t kn_tr_col(uint32_t col_base, uint32_t j, uint32_t lane) {
-    return col_base + j * 32u + ((lane >> 4) & 1u) * 16u + (lane & 3u) * 4u;   // first of the 4 columns addressed
-}
-MAIZE_MAP uint32_t kn_tr_offset(uint32_t col_base, uint32_t j, uint32_t kk, uint32_t h, uint32_t lane) {
-    const uint32_t col = kn_tr_col(col_base, j, lane);
-    return kn_offset(kn_tr_row(kk, h, lane), col >> 3) + (col & 7u) * 2u;
-}
-
-// ---- bf16 epilogue staging of the macro-tile kernel: 32 rows of 256 B per wave and pass ---------------
-// Write: lane l holds 4 consecutive columns (8 B) of row l%32: columns 32 j + 8 q + 4 (l/32) + 0..3.
+// ---- 16-bit epilogue staging of the macro-tile kernels: 32 rows of 256 B per wave and pass -----------
+// MFMA 32x32 accumulators (the 8-bit kernel).  Write: lane l holds 4 consecutive columns (8 B) of row l%32: columns 32 j + 8 q + 4 (l/32) + 0..3.
 MAIZE_MAP uint32_t epi_write_offset(uint32_t j, uint32_t q, uint32_t lane) {
     const uint32_t row = lane & 31u, lhi = lane >> 5;
     return row * 256u + (((j * 4u + q) ^ (row & 15u)) * 16u) + ((lhi ^ ((row >> 4) & 1u)) * 8u);
@@ -75,7 +56,30 @@ MAIZE_MAP uint32_t epi_read_offset(uint32_t r, uint32_t lane) {
     return row * 256u + (((lane & 15u) ^ (row & 15u)) * 16u);
 }
 
+// The same region for MFMA 16x16x32 accumulators (the 16-bit kernel): lane l holds 4 consecutive columns of row 16 ii + l%16
+// (ii = 0, 1: the pass's two accumulator rows): columns 16 j + 4 (l/16) + 0..3 of the 128.
+MAIZE_MAP uint32_t epi16_write_offset(uint32_t ii, uint32_t j, uint32_t lane) {
+    const uint32_t row = ii * 16u + (lane & 15u), g = lane >> 4;
+    return row * 256u + (((2u * j + (g >> 1)) ^ (row & 15u)) * 16u) + (g & 1u) * 8u;
+}
+MAIZE_MAP uint32_t epi16_read_offset(uint32_t r, uint32_t lane) { return epi_read_offset(r, lane); }   // no halves swapped
+// fp32 staging of the general epilogue: 32 rows x 64 columns (row = 256 B = 16 chunks of 4 columns); lane l
+// writes the 16 bytes of row 16 ii + l%16, columns 16 jj + 4 (l/16) + 0..3.
+MAIZE_MAP uint32_t epi32_write_offset(uint32_t ii, uint32_t jj, uint32_t lane) {
+    const uint32_t row = ii * 16u + (lane & 15u);
+    return row * 256u + (((4u * jj + (lane >> 4)) ^ (row & 15u)) * 16u);
+}
+// Read r (0..3): lane l reads columns 8 (l%8) + 4 half + 0..3 (half = 0, 1) of row 8 r + l/8.
+MAIZE_MAP uint32_t epi32_read_row(uint32_t r, uint32_t lane) { return r * 8u + (lane >> 3); }
+MAIZE_MAP uint32_t epi32_read_offset(uint32_t r, uint32_t half, uint32_t lane) {
+    const uint32_t row = epi32_read_row(r, lane);
+    return row * 256u + (((2u * (lane & 7u) + half) ^ (row & 15u)) * 16u);
+}
+
 // ---- block of the skinny kernel: 32 rows of 512 B (row-major K x 256 slab of B) -----------------------
+// Also the layout of the macro-tile kernel's K x N operand tile (row-major B), which holds 64 such rows in
+// 32 pieces: the swizzle only looks at bits 0, 1 and 3 of the row, so the read of K half kh, register half h
+// sits 16384 kh + 2048 h bytes behind the one of (0, 0) and the kernel keeps one address register per column group.
 // Piece p (2 rows): lane l lands at row 2p + l/32, position l%32.  32-byte granules (16 columns) are
 // XOR-ed with f(row) = row%4 + 4 bit3(row).
 MAIZE_MAP uint32_t sk_swizzle(uint32_t row) { return (row & 3u) | (((row >> 3) & 1u) << 2); }

@@ -60,16 +60,25 @@ int main() {
                 CHECK(chunks.size() == 8, "kc lane group does not cover its row");
             }
         std::printf("ok  K-contiguous tile: deposit map is a bijection onto the read map\n");
-        // fragment reads (128-bit): operands of MFMA 32x32x16, every fragment, every 16-deep step
-        for (uint32_t base = 0; base < 256; base += 32)
-            for (uint32_t kk = 0; kk < 4; ++kk) {
+        // fragment reads (128-bit): operands of MFMA 16x16x32, every fragment, both 32-deep halves of a K tile
+        for (uint32_t base = 0; base < 256; base += 16)
+            for (uint32_t kh = 0; kh < 2; ++kh) {
                 uint32_t off[64];
                 for (uint32_t lane = 0; lane < 64; ++lane) {
-                    off[lane] = kc_frag_offset(base, kk, lane);
-                    CHECK(off[lane] == kc_offset(base + lane % 32, 2 * kk + lane / 32), "kc fragment lane map");
+                    off[lane] = kc_frag16_offset(base, kh, lane);
+                    CHECK(off[lane] == kc_offset(base + lane % 16, 4 * kh + lane / 16), "kc fragment lane map");
+                    // the kernel addresses fragment f of a wave as (fragment 0) + 2048 f
+                    CHECK(off[lane] == kc_frag16_offset(base & 128u, kh, lane) + 2048 * ((base & 127u) / 16), "kc fragment %u is not 2048 B per fragment behind fragment 0", base / 16);
                 }
-                CHECK(passes_conflict_free(off, 16), "kc fragment read base %u kk %u has bank conflicts", base, kk);
+                CHECK(passes_conflict_free(off, 16), "kc fragment read base %u kh %u has bank conflicts", base, kh);
             }
+        // the two halves of a 64-deep tile name each of a row's 8 chunks once
+        for (uint32_t row = 0; row < 256; ++row) {
+            std::set<uint32_t> chunks;
+            for (uint32_t kh = 0; kh < 2; ++kh)
+                for (uint32_t g = 0; g < 4; ++g) chunks.insert(kc_frag16_offset(row & ~15u, kh, g * 16 + (row & 15u)));
+            CHECK(chunks.size() == 8 && *chunks.begin() == row * 128, "kc fragment reads do not cover row %u", row);
+        }
         // the 8-bit kernel's reads of the same tile: (kh, c01, l/32) name each of the 8 chunks of a row once
         for (uint32_t base = 0; base < 256; base += 32) {
             std::set<uint32_t> seen8;
@@ -109,39 +118,38 @@ int main() {
         }
         std::printf("ok  skinny NT block: every wave reads exactly the rows it deposits, operand reads are bank-conflict free\n");
     }
-    // ---- K x N tile
+    // ---- K x N tile of the macro-tile kernel: 64 rows of the skinny block's layout, 32 pieces
     {
         std::set<uint32_t> seen;
         for (uint32_t piece = 0; piece < 32; ++piece)
             for (uint32_t lane = 0; lane < 64; ++lane) {
-                const uint32_t row = kn_piece_row(piece, lane), chunk = kn_piece_chunk(piece, lane);
-                CHECK(row < 64 && chunk < 32, "kn piece out of range");
-                CHECK(kn_offset(row, chunk) == piece * 1024 + lane * 16, "kn deposit/read mismatch piece %u lane %u", piece, lane);
-                CHECK(seen.insert(row * 32 + chunk).second, "kn (row %u, chunk %u) deposited twice", row, chunk);
+                const uint32_t row = sk_piece_row(piece, lane), chunk = sk_piece_chunk(piece, lane);
+                CHECK(row < 64 && chunk < 32, "K x N piece out of range");
+                CHECK(sk_offset(row, chunk) == piece * 1024 + lane * 16, "K x N deposit/read mismatch piece %u lane %u", piece, lane);
+                CHECK(seen.insert(row * 32 + chunk).second, "K x N (row %u, chunk %u) deposited twice", row, chunk);
             }
-        CHECK(seen.size() == 64 * 32, "kn tile not covered");
+        CHECK(seen.size() == 64 * 32, "K x N tile not covered");
         std::printf("ok  K x N tile: deposit map is a bijection onto the read map\n");
-        for (uint32_t cb = 0; cb < 256; cb += 128)
-            for (uint32_t j = 0; j < 4; ++j)
-                for (uint32_t kk = 0; kk < 4; ++kk)
-                    for (uint32_t h = 0; h < 2; ++h) {
-                        uint32_t off[64];
-                        for (uint32_t lane = 0; lane < 64; ++lane) {
-                            off[lane] = kn_tr_offset(cb, j, kk, h, lane);
-                            // what the transposing read hands lane l: column q of the 4 x 16 block its 16-lane group addresses
-                            const uint32_t grp = lane & ~15u, q = lane & 15u;
-                            const uint32_t block_col0 = kn_tr_col(cb, j, grp);          // lane 0 of the group addresses the block's first 4 columns
-                            const uint32_t block_row0 = kn_tr_row(kk, h, grp);
-                            CHECK(kn_tr_row(kk, h, lane) == block_row0 + q / 4 && kn_tr_col(cb, j, lane) == block_col0 + 4 * (q % 4), "kn tr block shape");
-                            // lane receives column block_col0 + q, rows block_row0 .. +3: the MFMA wants column cb + 32 j + l%32, k = 16 kk + 8 (l/32) + 4 h + 0..3
-                            CHECK(block_col0 + q == cb + 32 * j + lane % 32, "kn tr: lane %u gets column %u", lane, block_col0 + q);
-                            CHECK(block_row0 == 16 * kk + 8 * (lane / 32) + 4 * h, "kn tr: lane %u gets k rows from %u", lane, block_row0);
-                        }
-                        CHECK(passes_conflict_free(off, 8), "kn transposing read cb %u j %u kk %u h %u has bank conflicts", cb, j, kk, h);
+        // the kernel's transposing reads: one address register per column group cg (= sk_tr_offset(cg, 0, lane)),
+        // K half kh and register half h as the immediate 16384 kh + 2048 h
+        for (uint32_t cg = 0; cg < 16; ++cg)
+            for (uint32_t kh = 0; kh < 2; ++kh)
+                for (uint32_t h = 0; h < 2; ++h) {
+                    uint32_t off[64];
+                    for (uint32_t lane = 0; lane < 64; ++lane) {
+                        off[lane] = sk_tr_offset(cg, 0, lane) + 16384 * kh + 2048 * h;
+                        const uint32_t q = lane & 15u, g = lane >> 4;
+                        // lane q of group g addresses columns 16 cg + 4 (q%4) .. +3 of row 32 kh + 8 g + 4 h + q/4 and receives
+                        // column 16 cg + q, k = 32 kh + 8 g + 4 h + 0..3: the B operand of MFMA 16x16x32 (column l%16,
+                        // k = 8 (l/16) + 0..7 of the 32-deep half, over h = 0, 1)
+                        const uint32_t row = 32 * kh + 8 * g + 4 * h + q / 4, col = 16 * cg + 4 * (q % 4);
+                        CHECK(off[lane] == sk_offset(row, col >> 3) + (col & 7) * 2, "K x N transposing read cg %u kh %u h %u lane %u", cg, kh, h, lane);
                     }
+                    CHECK(passes_conflict_free(off, 8), "K x N transposing read cg %u kh %u h %u has bank conflicts", cg, kh, h);
+                }
         std::printf("ok  K x N tile: transposing reads deliver the MFMA operand and are bank-conflict free\n");
     }
-    // ---- bf16 epilogue staging
+    // ---- 16-bit epilogue staging, MFMA 32x32 accumulators (the 8-bit kernel)
     {
         for (uint32_t row = 0; row < 32; ++row)
             for (uint32_t c = 0; c < 16; ++c)          // logical 16-byte chunk = 8 columns
@@ -164,7 +172,46 @@ int main() {
             for (uint32_t lane = 0; lane < 64; ++lane) off[lane] = epi_read_offset(r, lane);
             CHECK(passes_conflict_free(off, 16), "epilogue read %u has bank conflicts", r);
         }
-        std::printf("ok  epilogue staging: writes meet reads (halves swapped where bit 4 of the row is set), conflict free\n");
+        std::printf("ok  epilogue staging (32x32 accumulators): writes meet reads (halves swapped where bit 4 of the row is set), conflict free\n");
+    }
+    // ---- 16-bit epilogue staging, MFMA 16x16x32 accumulators
+    {
+        for (uint32_t row = 0; row < 32; ++row)
+            for (uint32_t c = 0; c < 16; ++c)          // logical 16-byte chunk = 8 columns
+                for (uint32_t hh = 0; hh < 2; ++hh) {  // its halves: columns 0..3 and 4..7
+                    // the writer of columns 8 c + 4 hh ..: accumulator column j = c / 2, lane group g = 2 (c % 2) + hh
+                    const uint32_t w = epi16_write_offset(row / 16, c / 2, (2 * (c % 2) + hh) * 16 + row % 16);
+                    const uint32_t r = row / 4, lane = (row % 4) * 16 + c;
+                    CHECK(epi_read_row(r, lane) == row, "epi read row");
+                    CHECK(w == epi16_read_offset(r, lane) + hh * 8, "epilogue (16x16): (row %u, chunk %u, half %u) written at %u, read at %u", row, c, hh, w, epi16_read_offset(r, lane));
+                }
+        for (uint32_t ii = 0; ii < 2; ++ii)
+            for (uint32_t j = 0; j < 8; ++j) {
+                uint32_t off[64];
+                for (uint32_t lane = 0; lane < 64; ++lane) off[lane] = epi16_write_offset(ii, j, lane);
+                CHECK(passes_conflict_free(off, 8), "epilogue (16x16) write ii %u j %u has bank conflicts", ii, j);
+            }
+        // fp32 staging of the general epilogue: 32 rows x 64 columns
+        for (uint32_t row = 0; row < 32; ++row)
+            for (uint32_t c = 0; c < 16; ++c) {        // logical 16-byte chunk = 4 columns
+                const uint32_t w = epi32_write_offset(row / 16, c / 4, (c % 4) * 16 + row % 16);
+                const uint32_t r = row / 8, lane = (row % 8) * 8 + c / 2;
+                CHECK(epi32_read_row(r, lane) == row, "fp32 staging read row");
+                CHECK(w == epi32_read_offset(r, c % 2, lane), "fp32 staging: (row %u, chunk %u) written at %u, read at %u", row, c, w, epi32_read_offset(r, c % 2, lane));
+            }
+        for (uint32_t ii = 0; ii < 2; ++ii)
+            for (uint32_t jj = 0; jj < 4; ++jj) {
+                uint32_t off[64];
+                for (uint32_t lane = 0; lane < 64; ++lane) off[lane] = epi32_write_offset(ii, jj, lane);
+                CHECK(passes_conflict_free(off, 16), "fp32 staging write ii %u jj %u has bank conflicts", ii, jj);
+            }
+        for (uint32_t r = 0; r < 4; ++r)
+            for (uint32_t half = 0; half < 2; ++half) {
+                uint32_t off[64];
+                for (uint32_t lane = 0; lane < 64; ++lane) off[lane] = epi32_read_offset(r, half, lane);
+                CHECK(passes_conflict_free(off, 16), "fp32 staging read %u half %u has bank conflicts", r, half);
+            }
+        std::printf("ok  epilogue staging (16x16 accumulators, 16-bit and fp32): writes meet reads, conflict free\n");
     }
     // ---- skinny block
     {

@@ -33,18 +33,34 @@ def mt256_issue_slots():
     m = re.search(r"#define MAIZE_MT256_SCHED \{([0-9,\s]+)\}", src)
     slots = [int(x) for x in m.group(1).split(",")]
     assert len(slots) == 16
+    # the table counts slots of two MFMAs; the loop tests (slot & 3) == 2 on single-MFMA slots and is tied to
+    # the table by a static_assert
+    assert "if ((slot & 3) == 2 && slot < 64)" in src and "static_assert(sched_is_regular()" in src
+    assert "kIssueSlot[i] != 2 * i + 1" in src
     return slots
+
+
+def mt256_reads_per_quarter(nt):
+    """Fragment reads that bring in quarter q = (K half q / 2, row half q % 2): a new K half needs its B
+    fragments (8 reads of 128 bits, or 16 transposing reads of 64) and 4 A fragments, its second quarter 4 more of A."""
+    src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
+    assert "#define MAIZE_NREADS(nq) (((nq) & 1) ? 4 : 4 + NB)" in src
+    assert "constexpr int NB = NT ? 8 : 16;" in src
+    nb = 8 if nt else 16
+    return [4 + nb, 4, 4 + nb, 4]
 
 
 def mt256_wave_program(nk, slots, nreads, barrier_quarter=3):
     """Instruction stream of one wave for nk K tiles: a list of
-    ("dma", tile, piece, stage) | ("wait_all",) | ("barrier",) | ("read", tile, quarter, stage) | ("mfma", tile, quarter)."""
+    ("dma", tile, piece, stage) | ("wait_all",) | ("barrier",) | ("read", tile, quarter, stage) | ("mfma", tile, quarter).
+    A K step is four quarters of 32 MFMA slots; `nreads[q]` fragment reads bring in quarter q, issued in the
+    first slots of the quarter before it."""
     ops = []
     for pc in range(16):
         ops.append(("dma", 0, pc, 0))
     ops += [("wait_all",), ("barrier",)]
-    ops += [("read", 0, 0, 0)] * nreads
-    early = [pc for pc in range(16) if slots[pc] < 16]
+    ops += [("read", 0, 0, 0)] * nreads[0]
+    early = [pc for pc in range(16) if 2 * slots[pc] < 32]
     for pc in early:
         ops.append(("dma", 1, pc, 1))
     k_early, k_late = 2, 1
@@ -54,13 +70,13 @@ def mt256_wave_program(nk, slots, nreads, barrier_quarter=3):
         for kk in range(4):
             if kk == barrier_quarter:
                 ops += [("wait_all",), ("barrier",)]
-            for s in range(16):
+            for s in range(32):
                 ops.append(("mfma", t, kk))
-                if s < nreads:
+                if s < nreads[(kk + 1) & 3]:
                     ops.append(("read", t, kk + 1, cur) if kk < 3 else ("read", t + 1, 0, nxt))
-                slot = s if kk == 3 else 16 * (kk + 1) + s
+                slot = s if kk == 3 else 32 * (kk + 1) + s
                 for pc in range(16):
-                    if slots[pc] == slot:
+                    if 2 * slots[pc] == slot and slot < 64:
                         ops.append(("dma", k_early, pc, cur) if kk == 3 else ("dma", k_late, pc, nxt))
         k_early += 1
         k_late += 1
@@ -69,6 +85,9 @@ def mt256_wave_program(nk, slots, nreads, barrier_quarter=3):
 
 
 def check_two_stage(ops, steps, nreads, parts=4):
+    """`nreads`: fragment reads per part of a K step, one number for all parts or a list with one per part."""
+    per_part = [nreads] * parts if isinstance(nreads, int) else list(nreads)
+    assert len(per_part) == parts
     epoch = 0
     dma_epoch = {}          # (tile, piece) -> epoch of issue
     completed = set()       # (tile, piece) waited for by this wave
@@ -89,7 +108,7 @@ def check_two_stage(ops, steps, nreads, parts=4):
             old = tile - 2
             if old >= 0 and last_read_epoch.get(old, -1) >= epoch:
                 raise Hazard(f"tile {tile} piece {pc} overwrites tile {old} in epoch {epoch}, still being read")
-            if old >= 0 and old < steps and reads_seen.get(old, 0) < parts * nreads:
+            if old >= 0 and old < steps and reads_seen.get(old, 0) < sum(per_part):
                 raise Hazard(f"tile {tile} overwrites tile {old} before all of its fragments were read")
             dma_epoch[(tile, pc)] = epoch
             stage_of[tile] = stage
@@ -114,7 +133,7 @@ def check_two_stage(ops, steps, nreads, parts=4):
             reads_seen[tile] = reads_seen.get(tile, 0) + 1
         elif op[0] == "mfma":
             _, tile, quarter = op
-            if reads_seen.get(tile, 0) < (quarter + 1) * nreads:
+            if reads_seen.get(tile, 0) < sum(per_part[:quarter + 1]):
                 raise Hazard(f"tile {tile} quarter {quarter} multiplied before its fragments were read")
             if not consumed or consumed[-1] != (tile, quarter):
                 consumed.append((tile, quarter))
@@ -131,10 +150,12 @@ def check_two_stage(ops, steps, nreads, parts=4):
 
 
 @pytest.mark.parametrize("nk", [1, 2, 3, 7, 64])
-@pytest.mark.parametrize("nreads", [8, 12])
-def test_macro_tile_schedule_is_hazard_free(nk, nreads):
+@pytest.mark.parametrize("nt", [False, True])
+def test_macro_tile_schedule_is_hazard_free(nk, nt):
     slots = mt256_issue_slots()
-    assert all(0 <= s < 64 for s in slots), "every request of tile t+2 must be issued before the barrier of step t+1"
+    nreads = mt256_reads_per_quarter(nt)
+    assert all(0 <= 2 * s < 64 for s in slots), "every request of tile t+2 must be issued before the barrier of step t+1"
+    assert max(nreads) <= 32, "the reads for a quarter are issued one per MFMA slot of the quarter before it"
     ops, steps = mt256_wave_program(nk, slots, nreads)
     last_tile = check_two_stage(ops, steps, nreads)
     # tiles past the end are requested (through a zero-length descriptor) but never multiplied
@@ -143,21 +164,27 @@ def test_macro_tile_schedule_is_hazard_free(nk, nreads):
 
 def test_macro_tile_checker_rejects_broken_schedules():
     slots = mt256_issue_slots()
+    nreads = mt256_reads_per_quarter(True)
     # barrier one quarter early: fragments of the current tile are still being read behind it
-    ops, steps = mt256_wave_program(8, slots, 8, barrier_quarter=2)
+    ops, steps = mt256_wave_program(8, slots, nreads, barrier_quarter=2)
     with pytest.raises(Hazard):
-        check_two_stage(ops, steps, 8)
+        check_two_stage(ops, steps, nreads)
     # a request scheduled past the next barrier never gets issued
     bad = list(slots)
     bad[5] = 64
-    ops, steps = mt256_wave_program(8, bad, 8)
+    ops, steps = mt256_wave_program(8, bad, nreads)
     with pytest.raises(Hazard):
-        check_two_stage(ops, steps, 8)
+        check_two_stage(ops, steps, nreads)
     # a missing wait before the barrier: data not guaranteed to have landed
-    ops, steps = mt256_wave_program(8, slots, 8)
+    ops, steps = mt256_wave_program(8, slots, nreads)
     k = [i for i, o in enumerate(ops) if o == ("wait_all",)][3]
     with pytest.raises(Hazard):
-        check_two_stage(ops[:k] + ops[k + 1:], steps, 8)
+        check_two_stage(ops[:k] + ops[k + 1:], steps, nreads)
+    # a fragment read dropped from a quarter: its MFMAs would run on stale registers
+    ops, steps = mt256_wave_program(8, slots, nreads)
+    k = [i for i, o in enumerate(ops) if o[0] == "read" and o[1] == 3][5]
+    with pytest.raises(Hazard):
+        check_two_stage(ops[:k] + ops[k + 1:], steps, nreads)
 
 
 # ---------------------------------------------------------------------------------------
