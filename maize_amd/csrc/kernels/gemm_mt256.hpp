@@ -15,11 +15,12 @@
 //     direct-to-LDS buffer loads (no register round trip; the hardware range
 //     check zero-fills the M/N/K edges, where the reference discards its
 //     ragged panels, src/main.rs:56-57);
-//   * a K step is four quarters of 32 MFMAs (K half x row half of the wave's
-//     sub-tile); the fragments of a quarter are read from LDS during the quarter
-//     before it, double-buffered in registers, by hand-placed ds_read
-//     instructions whose fragment and stage sit in the offset field (one address
-//     register per operand and K half) and hand-placed waits;
+//   * a K step is eight eighths of 16 MFMAs: per 32-deep K half the (A group,
+//     B group) pairs (0,0), (0,1), (1,1), (1,0), a group being 4 fragments.  Each
+//     eighth needs one new group, read from LDS during the eighth before it --
+//     uniform LDS traffic, two register buffers per operand -- by hand-placed
+//     ds_read instructions whose fragment and stage sit in the offset field (one
+//     address register per operand and K half) and hand-placed waits;
 //   * one barrier per K step, placed before the last quarter of the step's
 //     MFMAs: the fragments of that quarter are already in registers, so behind
 //     the barrier the first fragments of tile t+1 are read and the stage that
@@ -279,15 +280,22 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int j = 0; j < 8; ++j) b_rd[j] = (uint32_t)(uintptr_t)B0 + maps::sk_tr_offset(wn * 8u + j, 0, lane);
     }
 
-    // Fragment registers: A of one quarter (4 fragments), B of one half (8), each double-buffered.
-    // A quarter q = (kh = q / 2, rows 64 (q % 2) .. + 63 of the wave's 128): 32 MFMAs.
+    // Fragment registers.  A K half (32 deep) of the wave's sub-tile is walked in four eighths of 16 MFMAs
+    // each: (A group, B group) = (0,0), (0,1), (1,1), (1,0), a group being 4 fragments (64 rows or columns).
+    // Consecutive eighths share one group, so each needs exactly one new group: 4 fragments, read from LDS
+    // during the eighth before it.  LDS traffic is therefore uniform -- 4 KiB per wave and 16 MFMAs --
+    // and two buffers of 4 fragments per operand are enough:
+    //   A group ai lives in fa[ai]; B group bi of K half kh lives in buffer bi ^ kh (the group that is
+    //   held across the change of K half keeps its buffer, the other one is free for the new half).
     bf16x8 fa[2][4];
-    bf16x8 fb[2][8];
-    short4v fbl[2][8], fbh[2][8];
-    constexpr int NB = NT ? 8 : 16;                     // reads that bring in the B fragments of one half
-    // Number of fragment reads quarter nq needs beyond what the quarter before it holds: a new half
-    // needs its B fragments and 4 A fragments, the second quarter of a half 4 A fragments.
-#define MAIZE_NREADS(nq) (((nq) & 1) ? 4 : 4 + NB)
+    bf16x8 fb[2][4];
+    short4v fbl[2][4], fbh[2][4];
+    constexpr int NBR = NT ? 4 : 8;                     // reads that bring in one B group (transposing reads are 64-bit)
+    // Read r of a group is issued in MFMA slot r * RSTRIDE of the eighth.
+#ifndef MAIZE_MT256_RSTRIDE
+#define MAIZE_MT256_RSTRIDE 1
+#endif
+    static_assert(8 * MAIZE_MT256_RSTRIDE <= 16, "the reads of a group must fit into the 16 slots of an eighth");
     // 128-bit read at base + 2048 * n (n = stage * 16 + fragment), 64-bit transposing read at
     // base + 2048 * n (n = stage * 16 + kh * 8 + h).  The offsets are immediates: one case per value,
     // folded away once the caller's loops are unrolled.
@@ -308,25 +316,22 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         }
     };
 #undef MAIZE_RD_CASE
-    // Read r of the fragments of quarter nq of the tile in stage st (0, 1); the operands of the quarter's
-    // first MFMA first.  A goes to buffer nq % 2, B to buffer (nq / 2) % 2.
-    auto read_for = [&](int nq, int r, int st) {
-        const int kh = nq >> 1, rh = nq & 1;
-        if (rh == 1) { lds_read128(fa[1][r], a_rd[kh], st * 16 + 4 + r); return; }
-        if (r == 0) lds_read128(fa[0][0], a_rd[kh], st * 16);
-        else if (r <= NB) {
-            if (NT) lds_read128(fb[kh][r - 1], b_rd[kh], st * 16 + r - 1);
-            else {
-                const int j = (r - 1) >> 1, h = (r - 1) & 1;      // rows 32 kh + 4 h + ...: 16 KiB and 2 KiB further on
-                if (h == 0) lds_read_tr(fbl[kh][j], b_rd[j], st * 16 + kh * 8);
-                else        lds_read_tr(fbh[kh][j], b_rd[j], st * 16 + kh * 8 + 1);
-            }
-        } else lds_read128(fa[0][r - NB], a_rd[kh], st * 16 + r - NB);
+    // Read r (0..3) of A group ai, K half kh, of the tile in stage st.
+    auto read_a = [&](int ai, int kh, int st, int r) { lds_read128(fa[ai][r], a_rd[kh], st * 16 + 4 * ai + r); };
+    // Read r (0..NBR-1) of B group bi, K half kh, of the tile in stage st.
+    auto read_b = [&](int bi, int kh, int st, int r) {
+        const int buf = bi ^ kh;
+        if (NT) lds_read128(fb[buf][r], b_rd[kh], st * 16 + 4 * bi + r);
+        else {
+            const int c = r >> 1, h = r & 1;                  // rows 32 kh + 4 h + ...: 16 KiB and 2 KiB further on
+            if (h == 0) lds_read_tr(fbl[buf][c], b_rd[4 * bi + c], st * 16 + kh * 8);
+            else        lds_read_tr(fbh[buf][c], b_rd[4 * bi + c], st * 16 + kh * 8 + 1);
+        }
     };
-    auto b_operand = [&](int buf, int j) -> bf16x8 {
-        if (NT) return fb[buf][j];
-        short8v r = {fbl[buf][j][0], fbl[buf][j][1], fbl[buf][j][2], fbl[buf][j][3],
-                     fbh[buf][j][0], fbh[buf][j][1], fbh[buf][j][2], fbh[buf][j][3]};
+    auto b_operand = [&](int buf, int c) -> bf16x8 {
+        if (NT) return fb[buf][c];
+        short8v r = {fbl[buf][c][0], fbl[buf][c][1], fbl[buf][c][2], fbl[buf][c][3],
+                     fbh[buf][c][0], fbh[buf][c][1], fbh[buf][c][2], fbh[buf][c][3]};
         return __builtin_bit_cast(bf16x8, r);
     };
 
@@ -335,16 +340,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     uint32_t k_late = 0;                   // tile whose late pieces are issued next (first quarter of a step)
 
     // ---- steady state ----------------------------------------------------------------
-    // One K step.  On entry: (ca, cb) hold tile t, the fragment buffers hold its quarter-0 fragments,
+    // One K step = 8 eighths.  On entry: (ca, cb) hold tile t, fa[0] and B buffer 0 hold its first groups,
     // the early pieces of tile t+1 are landing in (na, nb).
     auto step = [&](int cur) {
         lds_ptr const ca = A0 + cur * TILE, cb = B0 + cur * TILE, na = A0 + (cur ^ 1) * TILE, nb = B0 + (cur ^ 1) * TILE;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int kh = q >> 1, rh = q & 1;
-            // The fragments of this quarter were requested during the one before: they have to be in.
-            if (q < 3) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (q == 3) {
+        for (int e = 0; e < 8; ++e) {
+            const int kh = e >> 2, h4 = e & 3;
+            const int ai = h4 >> 1, bi = (h4 == 1 || h4 == 2) ? 1 : 0;
+            // The group this eighth needs was requested during the one before: it has to be in.
+            if (e != 6) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (e == 6) {
                 // Every fragment this step still needs from (ca, cb) is in registers.  Wait until
                 // this wave's share of tile t+1 has landed, then meet the other waves: after the
                 // barrier (na, nb) is complete and (ca, cb) is free to be refilled with tile t+2.
@@ -353,26 +359,29 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 MAIZE_FENCE();
             }
 #pragma unroll
-            for (int s = 0; s < 32; ++s) {
-                const int i = 4 * rh + (s >> 3), j = s & 7;
+            for (int s = 0; s < 16; ++s) {
+                const int r4 = s >> 2, c4 = s & 3;
                 // The accumulator is tied to itself ("+a"): left to the register allocator, a few of the 64
                 // tuples were renamed across the loop and copied back through VGPRs at its end.  (Each
-                // accumulator comes up again 32 MFMAs later: no dependent back-to-back issue.)
+                // accumulator comes up again 128 MFMAs later: no dependent back-to-back issue.)
                 if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
-                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(kh, j)), "v"(fa[rh][s >> 3]));
+                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(bi ^ kh, c4)), "v"(fa[ai][r4]));
                 else
-                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(kh, j)), "v"(fa[rh][s >> 3]));
-                // Side work of this slot: fragment reads for the next quarter ...
-                if (s < MAIZE_NREADS((q + 1) & 3)) {
-                    if (q < 3) read_for(q + 1, s, cur);
-                    else       read_for(0, s, cur ^ 1);
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(bi ^ kh, c4)), "v"(fa[ai][r4]));
+                // Side work of this slot: the reads of the group the next eighth needs ...
+                if (s % MAIZE_MT256_RSTRIDE == 0) {
+                    const int r = s / MAIZE_MT256_RSTRIDE;
+                    if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);                       // (0,0) -> (0,1): B group 1
+                    if (h4 == 1 && r < 4) read_a(1, kh, cur, r);                         // (0,1) -> (1,1): A group 1
+                    if (h4 == 2 && r < 4) { if (kh == 0) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }     // next half: A group 0
+                    if (h4 == 3 && r < NBR) { if (kh == 0) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }   // next half: B group 0
                 }
                 // ... and the direct-to-LDS requests scheduled for this slot (kIssueSlot counts slots of
                 // two of these MFMAs): late pieces of tile t+1 (its stage was freed by the previous
-                // barrier) in the first three quarters, early pieces of tile t+2 behind this step's barrier.
-                const int slot = q == 3 ? s : 32 * (q + 1) + s;
+                // barrier) in the first quarter, early pieces of tile t+2 behind this step's barrier.
+                const int slot = e >= 6 ? 16 * (e - 6) + s : 32 + 16 * e + s;
                 if ((slot & 3) == 2 && slot < 64) {            // piece pc goes out at slot 4 pc + 2 = 2 kIssueSlot[pc]
-                    if (q == 3) dma(slot >> 2, ca, cb, k_early);
+                    if (e >= 6) dma(slot >> 2, ca, cb, k_early);
                     else        dma(slot >> 2, na, nb, k_late);
                 }
                 MAIZE_FENCE();
@@ -393,7 +402,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // The wait also covers the C stores of the previous tile (loads and stores share the counter).
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-    for (int r = 0; r < MAIZE_NREADS(0); ++r) read_for(0, r, 0);
+    for (int r = 0; r < 4; ++r) read_a(0, 0, 0, r);
+#pragma unroll
+    for (int r = 0; r < NBR; ++r) read_b(0, 0, 0, r);
 #pragma unroll
     for (int pc = 0; pc < early_pieces(); ++pc) dma(pc, A1, B1, k_begin + BK);   // tile 1, early pieces
     k_early = k_begin + 2 * BK;
@@ -560,7 +571,6 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }  // C tiles
 }
 
-#undef MAIZE_NREADS
 }  // namespace mt256
 
 #define MAIZE_MT256_KERNEL(name, nt, ktail, edge) \

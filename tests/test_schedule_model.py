@@ -40,26 +40,37 @@ def mt256_issue_slots():
     return slots
 
 
-def mt256_reads_per_quarter(nt):
-    """Fragment reads that bring in quarter q = (K half q / 2, row half q % 2): a new K half needs its B
-    fragments (8 reads of 128 bits, or 16 transposing reads of 64) and 4 A fragments, its second quarter 4 more of A."""
+def mt256_reads_per_eighth(nt):
+    """A K step is 8 eighths of 16 MFMAs; each needs one new group of 4 fragments beyond what the eighth
+    before it holds: 4 reads of 128 bits, or 8 transposing reads of 64 bits for a group of a row-major B.
+    Within a K half the groups come in the order B1, A1, then A0 and B0 of the next half (the source states it)."""
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
-    assert "#define MAIZE_NREADS(nq) (((nq) & 1) ? 4 : 4 + NB)" in src
-    assert "constexpr int NB = NT ? 8 : 16;" in src
-    nb = 8 if nt else 16
-    return [4 + nb, 4, 4 + nb, 4]
+    assert "constexpr int NBR = NT ? 4 : 8;" in src
+    for line in ("if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);",
+                 "if (h4 == 1 && r < 4) read_a(1, kh, cur, r);",
+                 "if (h4 == 2 && r < 4) { if (kh == 0) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
+                 "if (h4 == 3 && r < NBR) { if (kh == 0) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }"):
+        assert line in src, line
+    assert "if (e == 6) {" in src and "const int slot = e >= 6 ? 16 * (e - 6) + s : 32 + 16 * e + s;" in src
+    nbr = 4 if nt else 8
+    # reads that bring in eighth e (issued during e - 1): e = 0: A0 and B0 (the first of them, A0, a whole eighth earlier)
+    return [nbr, nbr, 4, 0, nbr, nbr, 4, 0], nbr
 
 
-def mt256_wave_program(nk, slots, nreads, barrier_quarter=3):
+def mt256_wave_program(nk, slots, nt, barrier_eighth=6):
     """Instruction stream of one wave for nk K tiles: a list of
-    ("dma", tile, piece, stage) | ("wait_all",) | ("barrier",) | ("read", tile, quarter, stage) | ("mfma", tile, quarter).
-    A K step is four quarters of 32 MFMA slots; `nreads[q]` fragment reads bring in quarter q, issued in the
-    first slots of the quarter before it."""
+    ("dma", tile, piece, stage) | ("wait_all",) | ("barrier",) | ("read", tile, eighth, stage) | ("mfma", tile, eighth).
+    Eighth e of a step issues, in its first slots, the reads of the group that eighth e + 1 needs -- except
+    that A group 0 of the next K half is read one eighth earlier (during e = 2 and e = 6), its buffer being free."""
+    _, nbr = mt256_reads_per_eighth(nt)
+    # (eighth whose MFMAs need it, number of reads, read from the next tile?) issued during eighth e
+    issued = {0: (1, nbr, False), 1: (2, 4, False), 2: (4, 4, False), 3: (4, nbr, False),
+              4: (5, nbr, False), 5: (6, 4, False), 6: (0, 4, True), 7: (0, nbr, True)}
     ops = []
     for pc in range(16):
         ops.append(("dma", 0, pc, 0))
     ops += [("wait_all",), ("barrier",)]
-    ops += [("read", 0, 0, 0)] * nreads[0]
+    ops += [("read", 0, 0, 0)] * (4 + nbr)
     early = [pc for pc in range(16) if 2 * slots[pc] < 32]
     for pc in early:
         ops.append(("dma", 1, pc, 1))
@@ -67,17 +78,18 @@ def mt256_wave_program(nk, slots, nreads, barrier_quarter=3):
     steps = nk + (nk & 1)                                   # the loop body holds two steps
     for t in range(steps):
         cur, nxt = t & 1, (t & 1) ^ 1
-        for kk in range(4):
-            if kk == barrier_quarter:
+        for e in range(8):
+            if e == barrier_eighth:
                 ops += [("wait_all",), ("barrier",)]
-            for s in range(32):
-                ops.append(("mfma", t, kk))
-                if s < nreads[(kk + 1) & 3]:
-                    ops.append(("read", t, kk + 1, cur) if kk < 3 else ("read", t + 1, 0, nxt))
-                slot = s if kk == 3 else 32 * (kk + 1) + s
+            need, n, next_tile = issued[e]
+            for s in range(16):
+                ops.append(("mfma", t, e))
+                if s < n:
+                    ops.append(("read", t + 1, need, nxt) if next_tile else ("read", t, need, cur))
+                slot = 16 * (e - 6) + s if e >= 6 else 32 + 16 * e + s
                 for pc in range(16):
                     if 2 * slots[pc] == slot and slot < 64:
-                        ops.append(("dma", k_early, pc, cur) if kk == 3 else ("dma", k_late, pc, nxt))
+                        ops.append(("dma", k_early, pc, cur) if e >= 6 else ("dma", k_late, pc, nxt))
         k_early += 1
         k_late += 1
     ops.append(("wait_all",))
@@ -85,9 +97,10 @@ def mt256_wave_program(nk, slots, nreads, barrier_quarter=3):
 
 
 def check_two_stage(ops, steps, nreads, parts=4):
-    """`nreads`: fragment reads per part of a K step, one number for all parts or a list with one per part."""
-    per_part = [nreads] * parts if isinstance(nreads, int) else list(nreads)
-    assert len(per_part) == parts
+    """`nreads`: fragment reads per part of a K step if a number; a list gives, per part, how many reads of the
+    tile must have been issued before the part's first MFMA (cumulative)."""
+    cumulative = [nreads * (q + 1) for q in range(parts)] if isinstance(nreads, int) else list(nreads)
+    assert len(cumulative) == parts
     epoch = 0
     dma_epoch = {}          # (tile, piece) -> epoch of issue
     completed = set()       # (tile, piece) waited for by this wave
@@ -108,7 +121,7 @@ def check_two_stage(ops, steps, nreads, parts=4):
             old = tile - 2
             if old >= 0 and last_read_epoch.get(old, -1) >= epoch:
                 raise Hazard(f"tile {tile} piece {pc} overwrites tile {old} in epoch {epoch}, still being read")
-            if old >= 0 and old < steps and reads_seen.get(old, 0) < sum(per_part):
+            if old >= 0 and old < steps and reads_seen.get(old, 0) < cumulative[-1]:
                 raise Hazard(f"tile {tile} overwrites tile {old} before all of its fragments were read")
             dma_epoch[(tile, pc)] = epoch
             stage_of[tile] = stage
@@ -133,7 +146,7 @@ def check_two_stage(ops, steps, nreads, parts=4):
             reads_seen[tile] = reads_seen.get(tile, 0) + 1
         elif op[0] == "mfma":
             _, tile, quarter = op
-            if reads_seen.get(tile, 0) < sum(per_part[:quarter + 1]):
+            if reads_seen.get(tile, 0) < cumulative[quarter]:
                 raise Hazard(f"tile {tile} quarter {quarter} multiplied before its fragments were read")
             if not consumed or consumed[-1] != (tile, quarter):
                 consumed.append((tile, quarter))
@@ -149,42 +162,53 @@ def check_two_stage(ops, steps, nreads, parts=4):
     return max(t for (t, _) in dma_epoch)
 
 
+def mt256_cumulative_reads(nt):
+    """Fragment reads of a tile that must have been issued before eighth e multiplies: per eighth the groups
+    (A, B) = (0,0), (0,1), (1,1), (1,0) of K half e / 4."""
+    _, nbr = mt256_reads_per_eighth(nt)
+    first = 4 + nbr                       # A0, B0 of K half 0
+    half = [first, first + nbr, first + nbr + 4, first + nbr + 4]
+    return half + [half[3] + 4 + nbr, half[3] + 4 + 2 * nbr, half[3] + 8 + 2 * nbr, half[3] + 8 + 2 * nbr]
+
+
 @pytest.mark.parametrize("nk", [1, 2, 3, 7, 64])
 @pytest.mark.parametrize("nt", [False, True])
 def test_macro_tile_schedule_is_hazard_free(nk, nt):
     slots = mt256_issue_slots()
-    nreads = mt256_reads_per_quarter(nt)
     assert all(0 <= 2 * s < 64 for s in slots), "every request of tile t+2 must be issued before the barrier of step t+1"
-    assert max(nreads) <= 32, "the reads for a quarter are issued one per MFMA slot of the quarter before it"
-    ops, steps = mt256_wave_program(nk, slots, nreads)
-    last_tile = check_two_stage(ops, steps, nreads)
+    ops, steps = mt256_wave_program(nk, slots, nt)
+    last_tile = check_two_stage(ops, steps, mt256_cumulative_reads(nt), parts=8)
     # tiles past the end are requested (through a zero-length descriptor) but never multiplied
     assert steps <= last_tile <= steps + 1
 
 
 def test_macro_tile_checker_rejects_broken_schedules():
     slots = mt256_issue_slots()
-    nreads = mt256_reads_per_quarter(True)
-    # barrier one quarter early: fragments of the current tile are still being read behind it
-    ops, steps = mt256_wave_program(8, slots, nreads, barrier_quarter=2)
+    need = mt256_cumulative_reads(True)
+    # barrier one eighth early: fragments of the current tile are still being read behind it
+    ops, steps = mt256_wave_program(8, slots, True, barrier_eighth=5)
     with pytest.raises(Hazard):
-        check_two_stage(ops, steps, nreads)
+        check_two_stage(ops, steps, need, parts=8)
+    # barrier one eighth late: the next tile is read before it is known to be complete
+    ops, steps = mt256_wave_program(8, slots, True, barrier_eighth=7)
+    with pytest.raises(Hazard):
+        check_two_stage(ops, steps, need, parts=8)
     # a request scheduled past the next barrier never gets issued
     bad = list(slots)
     bad[5] = 64
-    ops, steps = mt256_wave_program(8, bad, nreads)
+    ops, steps = mt256_wave_program(8, bad, True)
     with pytest.raises(Hazard):
-        check_two_stage(ops, steps, nreads)
+        check_two_stage(ops, steps, need, parts=8)
     # a missing wait before the barrier: data not guaranteed to have landed
-    ops, steps = mt256_wave_program(8, slots, nreads)
+    ops, steps = mt256_wave_program(8, slots, True)
     k = [i for i, o in enumerate(ops) if o == ("wait_all",)][3]
     with pytest.raises(Hazard):
-        check_two_stage(ops[:k] + ops[k + 1:], steps, nreads)
-    # a fragment read dropped from a quarter: its MFMAs would run on stale registers
-    ops, steps = mt256_wave_program(8, slots, nreads)
+        check_two_stage(ops[:k] + ops[k + 1:], steps, need, parts=8)
+    # a fragment read dropped from an eighth: its MFMAs would run on stale registers
+    ops, steps = mt256_wave_program(8, slots, True)
     k = [i for i, o in enumerate(ops) if o[0] == "read" and o[1] == 3][5]
     with pytest.raises(Hazard):
-        check_two_stage(ops[:k] + ops[k + 1:], steps, nreads)
+        check_two_stage(ops[:k] + ops[k + 1:], steps, need, parts=8)
 
 
 # ---------------------------------------------------------------------------------------
