@@ -133,9 +133,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // Read r (0..15) of the fragments of half kh of the tile in (sa, sb) into buffer buf; the
     // operands of the first MFMA first.
     auto read_frag = [&](int buf, int kh, int r, lds_ptr sa, lds_ptr sb) {
+        // in the order the MFMAs want them: A 0, B 0, A 1..3, B 1..3
         if (r < 2) fa[buf][0][r] = *(lds_v4)(sa + a_rd[kh][r]);
-        else if (r < 10) fb[buf][(r - 2) >> 1][r & 1] = *(lds_v4)(sb + b_rd[kh][r & 1] + ((r - 2) >> 1) * 32 * KROW);
-        else fa[buf][1 + ((r - 10) >> 1)][r & 1] = *(lds_v4)(sa + a_rd[kh][r & 1] + (1 + ((r - 10) >> 1)) * 32 * KROW);
+        else if (r < 4) fb[buf][0][r & 1] = *(lds_v4)(sb + b_rd[kh][r & 1]);
+        else if (r < 10) fa[buf][(r - 2) >> 1][r & 1] = *(lds_v4)(sa + a_rd[kh][r & 1] + ((r - 2) >> 1) * 32 * KROW);
+        else fb[buf][(r - 8) >> 1][r & 1] = *(lds_v4)(sb + b_rd[kh][r & 1] + ((r - 8) >> 1) * 32 * KROW);
     };
     auto operand = [&](const u32x4 (&f)[2]) -> i32x8 {
         return i32x8{(int)f[0][0], (int)f[0][1], (int)f[0][2], (int)f[0][3], (int)f[1][0], (int)f[1][1], (int)f[1][2], (int)f[1][3]};
@@ -158,8 +160,15 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
 #pragma unroll
             for (int s = 0; s < 16; ++s) {
-                acc[s >> 2][s & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    operand(fb[kh][s & 3]), operand(fa[kh][s >> 2]), acc[s >> 2][s & 3], FB, FA, 0, 0, 0, 0);   // B is fed first
+                // Boustrophedon order, B fragment held over four MFMAs: consecutive MFMAs differ in one
+                // operand only (measurably cheaper at the power limit than row-major order).
+#ifndef MAIZE_F8_ORDER
+#define MAIZE_F8_ORDER 1
+#endif
+                const int j = MAIZE_F8_ORDER ? s >> 2 : s & 3;
+                const int i = MAIZE_F8_ORDER ? ((j & 1) ? 3 - (s & 3) : (s & 3)) : s >> 2;
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    operand(fb[kh][j]), operand(fa[kh][i]), acc[i][j], FB, FA, 0, 0, 0, 0);   // B is fed first
                 if (kh == 0) read_frag(1, 1, s, ca, cb);
                 else {
                     read_frag(0, 0, s, na, nb);
