@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BF16 GEMM path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5|f8|f8s] [--kernel NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5|f8|f8s|f32|f64] [--kernel NAME]
 
 A step is one launch of maize_hip_gemm_bf16 on synthetic, seeded inputs that are already
 resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s (wall clock around exactly K
@@ -46,10 +46,18 @@ CONFIGS = {
     # ... and the decode-style shape of cfg4 against 8-bit weights stored N x K.
     "f8s": dict(m=16, n=14336, k=4096, nt=1, batch=1, da=("uniform",), db=("uniform",), bound="hbm", in_type="e4m3",
                 label="E4M3 GEMM 16x14336x4096 NT skinny (bf16 C), uniform[-1,1) rounded to E4M3"),
+    # The catalogue's fp32 and fp64 entries (v_mfma_f32_16x16x4_f32, v_mfma_f64_16x16x4_f64), C in the operands' type.
+    "f32": dict(m=4096, n=4096, k=4096, nt=0, batch=1, da=("uniform",), db=("uniform",), bound="mfma", in_type="f32",
+                label="fp32 GEMM 4096x4096x4096 NN (fp32 C), uniform[-1,1)"),
+    "f64": dict(m=4096, n=4096, k=4096, nt=0, batch=1, da=("uniform",), db=("uniform",), bound="mfma", in_type="f64",
+                label="fp64 GEMM 4096x4096x4096 NN (fp64 C), uniform[-1,1)"),
 }
+WIDE = {"f32": (np.float32, 157.3), "f64": (np.float64, 78.6)}     # element type, published dense MFMA peak in TFLOP/s
 
 
 def make(mz, dist, count, seed, in_type=None):
+    if in_type in WIDE:
+        return (np.random.default_rng(seed).random(count) * 2 - 1).astype(WIDE[in_type][0])
     if in_type is not None:
         return mz.gen.uniform_f8(count, seed, mz.IN_E4M3 if in_type == "e4m3" else mz.IN_E5M2)
     if dist[0] == "uniform":
@@ -64,6 +72,8 @@ def cpu_baseline(cfg, a, b_storage, got, seconds_target=12.0):
     the reported baseline here; it is never on the measured GPU path."""
     from oracle import pyoracle
     m, n, k = cfg["m"], cfg["n"], cfg["k"]
+    if cfg.get("in_type") in WIDE:
+        return cpu_baseline_wide(cfg, a, b_storage, got, seconds_target)
     elem = {None: pyoracle.BF16, "e4m3": pyoracle.E4M3, "e5m2": pyoracle.E5M2}[cfg.get("in_type")]
     coeff = pyoracle.floor_coeff_f8(k) if cfg.get("in_type") else None
     threads = pyoracle.default_threads()
@@ -90,6 +100,32 @@ def cpu_baseline(cfg, a, b_storage, got, seconds_target=12.0):
         r = min(rows, 64)
         parity = pyoracle.compare(got[:r * n], ref[:r], f64[:r], ab, k, coeff=coeff)
         parity = {key: parity[key] for key in ("n", "max_ulp", "n_gt1ulp", "n_fail", "max_err_over_abs")}
+    return out, parity
+
+
+def cpu_baseline_wide(cfg, a, b_storage, got, seconds_target):
+    """The same for fp32 / fp64 operands: the oracle's long-double sums on the first R rows."""
+    from oracle import pyoracle
+    m, n, k = cfg["m"], cfg["n"], cfg["k"]
+    threads = pyoracle.default_threads()
+    t0 = time.perf_counter()
+    pyoracle.ref_gemm_wide(a, b_storage, m, n, k, layout=cfg["nt"], rows=np.arange(2, dtype=np.uint32), nthreads=1)
+    per_row = max((time.perf_counter() - t0) / 2, 1e-6)
+    rows = int(min(m, max(threads, seconds_target * threads / per_row)))
+    rows = max(1, (rows // threads) * threads) if rows >= threads else rows
+    sel = np.arange(rows, dtype=np.uint32)
+    t0 = time.perf_counter()
+    hi, lo, ab = pyoracle.ref_gemm_wide(a, b_storage, m, n, k, layout=cfg["nt"], rows=sel, nthreads=threads)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * rows * n * k
+    out = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+           "sample": f"rows 0..{rows - 1} ({rows}x{n}x{k}, {flops / 1e9:.1f} GFLOP, {dt:.1f} s), long-double products and sums "
+                     f"(and sum|a||b| beside them), {threads} POSIX threads"}
+    parity = None
+    if got is not None:
+        worst = pyoracle.check_wide(got.reshape(m, n)[:rows], hi, lo, ab, k)
+        parity = {"n": int(rows * n), "worst_error_over_bound": worst, "n_fail": int(worst > 1.0),
+                  "bound": "(K/4 + 4) * u * sum|a||b|, u = 2^-24 (fp32) / 2^-53 (fp64)"}
     return out, parity
 
 
@@ -133,7 +169,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", default=None, choices=sorted(CONFIGS) + ["copy"],
-                    help="cfg1..cfg5: a benchmark configuration; f8, f8s: 4096^3 and 16x14336x4096 on E4M3 operands; copy: the 256 MiB copy "
+                    help="cfg1..cfg5: a benchmark configuration; f8, f8s: 4096^3 and 16x14336x4096 on E4M3 operands; f32, f64: 4096^3 on fp32 / fp64 operands; copy: the 256 MiB copy "
                          "used to scale HBM counters")
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -183,9 +219,11 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
     cfg = CONFIGS[args.config]
     m, n, k, batch, nt = cfg["m"], cfg["n"], cfg["k"], cfg["batch"], cfg["nt"]
     f8 = cfg.get("in_type")
-    esz = 1 if f8 else 2                                   # bytes per element of A and B
+    wide = f8 if f8 in WIDE else None                      # fp32 / fp64 operands: C has their type
+    esz = np.dtype(WIDE[wide][0]).itemsize if wide else 1 if f8 else 2     # bytes per element of A and B
+    csz = esz if wide else 2                               # ... and of C
     flops = 2.0 * batch * m * n * k
-    alg_bytes = float(batch) * (esz * (m * k + k * n) + 2 * m * n)
+    alg_bytes = float(batch) * (esz * (m * k + k * n) + csz * m * n)
 
     a = make(mz, cfg["da"], batch * m * k, mz.gen.SEED_A, f8)
     b = make(mz, cfg["db"], batch * k * n, mz.gen.SEED_B, f8)
@@ -196,12 +234,12 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
     nsets = args.rotate or (max(2, int(np.ceil(3 * 256 * 2 ** 20 / alg_bytes))) if cfg["bound"] == "hbm" else 1)
     sets = []
     for _ in range(nsets):
-        da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(2 * batch * m * n)
+        da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(csz * batch * m * n)
         A = mz.Matrix(da, m, k, elem_bytes=esz)
         B = mz.Matrix(db, n, k, elem_bytes=esz) if nt else mz.Matrix(db, k, n, elem_bytes=esz)
         if f8:
-            desc = mz.gemm_ex_desc(A, B, mz.Matrix(dc, m, n), layout=nt, batch=batch, stride_a=m * k, stride_b=k * n,
-                                   stride_c=m * n, in_type=mz.IN_E4M3 if f8 == "e4m3" else mz.IN_E5M2)
+            desc = mz.gemm_ex_desc(A, B, mz.Matrix(dc, m, n, elem_bytes=csz), layout=nt, batch=batch, stride_a=m * k, stride_b=k * n,
+                                   stride_c=m * n, in_type={"e4m3": mz.IN_E4M3, "e5m2": mz.IN_E5M2, "f32": mz.IN_F32, "f64": mz.IN_F64}[f8])
         else:
             desc = mz.gemm_desc(A, B, mz.Matrix(dc, m, n), layout=nt, batch=batch, stride_a=m * k, stride_b=k * n,
                                 stride_c=m * n)
@@ -237,11 +275,11 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
     wall = time.perf_counter() - t0
     ev_ms = ev0.elapsed_ms(ev1)
 
-    got = sets[(args.steps - 1) % nsets][2].download(np.uint16, count=m * n)
+    got = sets[(args.steps - 1) % nsets][2].download(WIDE[wide][0] if wide else np.uint16, count=m * n)
     ms_per_step = wall * 1e3 / args.steps
     kern_ms = ev_ms / args.steps
     value = flops / (wall / args.steps) / 1e12
-    peak_flops = PEAK_FP8_TFLOPS if f8 else PEAK_BF16_TFLOPS
+    peak_flops = WIDE[wide][1] if wide else PEAK_FP8_TFLOPS if f8 else PEAK_BF16_TFLOPS
     if cfg["bound"] == "mfma":
         ach = flops / (kern_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": ach, "peak": peak_flops, "unit": "TFLOP/s",
@@ -262,14 +300,15 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
 
     line = {
         "metric": "bf16 GEMM TFLOP/s at 4096^3 on 1 MI355X" if args.config == "cfg1"
+                  else f"{'fp32' if wide == 'f32' else 'fp64'} GEMM TFLOP/s, {args.config}" if wide
                   else f"E4M3 GEMM TFLOP/s, {args.config}" if f8 else f"bf16 GEMM TFLOP/s, {args.config}",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp8 (e4m3)" if f8 else "bf16", "data": "synthetic (seeded counter-based generators, inputs resident in HBM)",
+        "dtype": wide if wide else "fp8 (e4m3)" if f8 else "bf16", "data": "synthetic (seeded counter-based generators, inputs resident in HBM)",
         "config": {"workload": cfg["label"], "M": m, "N": n, "K": k, "batch": batch, "layout": "NT" if nt else "NN",
-                   "accumulate": "fp32", "output": "bf16", "operand_sets_cycled": nsets,
+                   "accumulate": wide or "fp32", "output": wide or "bf16", "operand_sets_cycled": nsets,
                    "clock_ramp_launches": ramp_launches},
-        ("pct_of_mfma_fp8_peak" if f8 else "pct_of_mfma_bf16_peak"): 100.0 * flops / (wall / args.steps) / 1e12 / peak_flops,
+        (f"pct_of_mfma_{wide}_peak" if wide else "pct_of_mfma_fp8_peak" if f8 else "pct_of_mfma_bf16_peak"): 100.0 * flops / (wall / args.steps) / 1e12 / peak_flops,
         "roofline": roof, "cpu_baseline": cpu, "parity_vs_oracle": parity,
         "device": {"name": info["name"], "compute_units": info["compute_units"], "clock_khz": info["clock_khz"]},
     }

@@ -104,9 +104,15 @@ typedef enum { MAIZE_OUT_SAME = 0, MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1 } maize
  * dimensions and batch strides still count elements, and the matrix instruction is
  * v_mfma_f32_32x32x64_f8f6f4 when B is stored N x K (MAIZE_LAYOUT_NT) with 16-byte aligned rows.
  * MAIZE_IN_E4M3_E5M2 / MAIZE_IN_E5M2_E4M3: A of the first format, B of the second (the catalogue's mixed pairs,
- * sm89.rs:34-45). */
+ * sm89.rs:34-45).
+ * MAIZE_IN_F32 / MAIZE_IN_F64: the catalogue's tf32 -> f32 and f64 -> f64 entries (Sm80MmaTf32F32_16x8x4 / _16x8x8,
+ * SM80MmaF64F64_8x8x4, sm80.rs:12-14) as v_mfma_f32_16x16x4_f32 (full fp32 operands; gfx950 has no tf32 matrix
+ * instruction) and v_mfma_f64_16x16x4_f64.  C has the operands' type (out_type MAIZE_OUT_SAME; MAIZE_OUT_F32 is
+ * accepted for fp32 operands and means the same), alpha and beta are applied in that type, any extents, leading
+ * dimensions and element-aligned pointers are taken. */
 typedef enum {
-    MAIZE_IN_BF16 = 0, MAIZE_IN_F16 = 1, MAIZE_IN_E4M3 = 2, MAIZE_IN_E5M2 = 3, MAIZE_IN_E4M3_E5M2 = 4, MAIZE_IN_E5M2_E4M3 = 5
+    MAIZE_IN_BF16 = 0, MAIZE_IN_F16 = 1, MAIZE_IN_E4M3 = 2, MAIZE_IN_E5M2 = 3, MAIZE_IN_E4M3_E5M2 = 4, MAIZE_IN_E5M2_E4M3 = 5,
+    MAIZE_IN_F32 = 6, MAIZE_IN_F64 = 7
 } maize_in_type_t;
 typedef struct {
     maize_gemm_desc_t gemm;

@@ -45,6 +45,8 @@ IN_E4M3 = 2
 IN_E5M2 = 3
 IN_E4M3_E5M2 = 4   # A is E4M3, B is E5M2
 IN_E5M2_E4M3 = 5
+IN_F32 = 6          # fp32 / fp64 operands; C has the operands' type
+IN_F64 = 7
 
 
 class MatrixT(C.Structure):

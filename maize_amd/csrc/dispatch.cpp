@@ -29,9 +29,10 @@ inline bool plain_epilogue(const maize_gemm_ex_desc_t& d) {
 inline bool half_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_F16; }
 inline bool bf16_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_BF16; }
 inline bool fp8_in(const maize_gemm_ex_desc_t& d) { return d.in_type >= MAIZE_IN_E4M3 && d.in_type <= MAIZE_IN_E5M2_E4M3; }
+inline bool wide_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_F32 || d.in_type == MAIZE_IN_F64; }
 
 // ---- maize_gemm_bf16_wave32: any shape ------------------------------------
-bool wave32_supports(const maize_gemm_ex_desc_t&) { return true; }
+bool wave32_supports(const maize_gemm_ex_desc_t& d) { return !wide_in(d); }   // 16-bit and 8-bit operands, any shape
 bool wave32_plan(const maize_gemm_ex_desc_t& d, uint32_t, LaunchDims* ld) {
     const Dims s = dims_of(d);
     ld->grid[0] = cdiv(s.n, 64);
@@ -417,7 +418,7 @@ bool trb_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims*
 // ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
 bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
-    if (fp8_in(d) || d.gemm.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
+    if (fp8_in(d) || wide_in(d) || d.gemm.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
     const uint64_t lim = 1ull << 31;
     const Lds l = lds_of(d);
     if (l.ext_a * 2 >= lim || l.ext_b * 2 >= lim || s.n >= (1u << 21) || l.b >= (1u << 21)) return false;
@@ -462,7 +463,7 @@ bool skinny_nt_common(const maize_gemm_ex_desc_t& d) {
     if (l.ext_a * esz >= lim || l.ext_b * esz >= lim || s.k >= (1u << 21) || l.b >= (1u << 21)) return false;
     return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
 }
-bool skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && skinny_nt_common(d); }
+bool skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d); }
 #define MAIZE_F8_SKINNY(tag, type) \
     bool tag##_skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d); }
 MAIZE_F8_SKINNY(e4m3, MAIZE_IN_E4M3)
@@ -492,8 +493,41 @@ bool skinny_nt_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Launc
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
 }
 
+// ---- maize_gemm_{f32,f64}_mt128_{nn,nt}: fp32 / fp64 operands, any shape ---------------------
+// 128 x 128 tiles, one workgroup each (x = tiles, XCD-aware order inside the kernel; z = batch).  Rows that
+// start on 16-byte boundaries and hold a whole number of 16-byte chunks are moved 128 bits at a time,
+// others element by element: bit 0 / 1 / 2 of split_first says so for A / B / C.
+template <uint32_t TYPE, bool NT>
+bool mt128_supports(const maize_gemm_ex_desc_t& d) {
+    return d.in_type == TYPE && (d.gemm.layout == MAIZE_LAYOUT_NT) == NT && (TYPE == MAIZE_IN_F32 || d.out_type == MAIZE_OUT_SAME);
+}
+bool mt128_plan(const maize_gemm_ex_desc_t& d, uint32_t, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    const uint32_t vec = d.in_type == MAIZE_IN_F64 ? 2u : 4u;                // elements per 16 bytes
+    const bool batched = d.gemm.batch > 1;
+    auto rows16 = [&](const void* ptr, uint32_t ldx, uint32_t cols, uint64_t stride) {
+        return ((uintptr_t)ptr & 15u) == 0 && ldx % vec == 0 && cols % vec == 0 && (!batched || stride % vec == 0);
+    };
+    const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128);
+    if (tiles > 0x7FFFFFFFull || d.gemm.batch > 65535u) return false;
+    ld->grid[0] = (uint32_t)tiles; ld->grid[1] = 1; ld->grid[2] = d.gemm.batch;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0;
+    ld->ksplit = 0; ld->workspace_bytes = 0; ld->reduce_grid = 0;
+    ld->split_first = (rows16(d.gemm.a.ptr, l.a, d.gemm.a.ncols, d.gemm.stride_a) ? 1u : 0u) |
+                      (rows16(d.gemm.b.ptr, l.b, d.gemm.b.ncols, d.gemm.stride_b) ? 2u : 0u) |
+                      // C: a lane stores 4 consecutive columns starting at a multiple of 4; only the row start matters
+                      ((((uintptr_t)d.gemm.c.ptr & 15u) == 0 && l.c % vec == 0 && (!batched || d.gemm.stride_c % vec == 0)) ? 4u : 0u);
+    return true;
+}
+
 const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_wave32", nullptr, wave32_supports, wave32_plan},
+    {"maize_gemm_f32_mt128_nn", nullptr, mt128_supports<MAIZE_IN_F32, false>, mt128_plan},
+    {"maize_gemm_f32_mt128_nt", nullptr, mt128_supports<MAIZE_IN_F32, true>, mt128_plan},
+    {"maize_gemm_f64_mt128_nn", nullptr, mt128_supports<MAIZE_IN_F64, false>, mt128_plan},
+    {"maize_gemm_f64_mt128_nt", nullptr, mt128_supports<MAIZE_IN_F64, true>, mt128_plan},
     {"maize_gemm_bf16_mt256_nn", nullptr, mt256_nn_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt", nullptr, mt256_nt_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_ktail", nullptr, mt256_nn_ktail_supports, mt256_plan},
@@ -546,6 +580,11 @@ int kernel_index(const char* name) {
 
 uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     const Dims s = dims_of(d);
+    if (wide_in(d)) {   // fp32 / fp64 operands: one kernel per type and layout, any shape
+        static const char* const kWide[2][2] = {{"maize_gemm_f32_mt128_nn", "maize_gemm_f32_mt128_nt"},
+                                                {"maize_gemm_f64_mt128_nn", "maize_gemm_f64_mt128_nt"}};
+        return (uint32_t)kernel_index(kWide[d.in_type == MAIZE_IN_F64][s.nt]);
+    }
     if (fp8_in(d)) {
         // 8-bit operands: the macro-tile kernel when both operands are K-contiguous and aligned (same
         // size rule as below), else the per-wave kernel, which widens them to bf16 as it loads.

@@ -295,10 +295,13 @@ int32_t maize_hip_gemm_ex_validate(const maize_gemm_ex_desc_t* x) {
     if (!d->a.ptr || !d->b.ptr || !d->c.ptr) return fail(MAIZE_ERR_NULL, "gemm: NULL matrix pointer");
     if (x->out_type != MAIZE_OUT_BF16 && x->out_type != MAIZE_OUT_F32)
         return fail(MAIZE_ERR_ARG, "gemm: unknown output type %u", x->out_type);
-    if (x->in_type > MAIZE_IN_E5M2_E4M3) return fail(MAIZE_ERR_ARG, "gemm: unknown operand type %u", x->in_type);
-    const bool in8 = x->in_type >= MAIZE_IN_E4M3;
+    if (x->in_type > MAIZE_IN_F64) return fail(MAIZE_ERR_ARG, "gemm: unknown operand type %u", x->in_type);
+    if (x->in_type == MAIZE_IN_F64 && x->out_type != MAIZE_OUT_SAME)
+        return fail(MAIZE_ERR_ARG, "gemm: fp64 operands have an fp64 C (out_type must be MAIZE_OUT_SAME)");
     if (x->reserved) return fail(MAIZE_ERR_ARG, "gemm: reserved field must be 0");
-    if (((uintptr_t)d->a.ptr | (uintptr_t)d->b.ptr) & (in8 ? 0u : 1u) || (uintptr_t)d->c.ptr & (x->out_type == MAIZE_OUT_F32 ? 3u : 1u))
+    const uint32_t in_bytes = x->in_type == MAIZE_IN_F64 ? 8u : x->in_type == MAIZE_IN_F32 ? 4u : x->in_type >= MAIZE_IN_E4M3 ? 1u : 2u;
+    const uint32_t out_bytes = x->in_type == MAIZE_IN_F64 ? 8u : (x->in_type == MAIZE_IN_F32 || x->out_type == MAIZE_OUT_F32) ? 4u : 2u;
+    if (((uintptr_t)d->a.ptr | (uintptr_t)d->b.ptr) & (in_bytes - 1u) || (uintptr_t)d->c.ptr & (out_bytes - 1u))
         return fail(MAIZE_ERR_ALIGN, "gemm: matrix pointers must be aligned to their element size");
     if ((x->lda && x->lda < d->a.ncols) || (x->ldb && x->ldb < d->b.ncols) || (x->ldc && x->ldc < d->c.ncols))
         return fail(MAIZE_ERR_SHAPE, "gemm: a leading dimension is smaller than the row it strides (lda=%u ldb=%u ldc=%u)",
@@ -420,7 +423,7 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
     args.lda = x->lda; args.ldb = x->ldb; args.ldc = x->ldc;
     args.alpha = x->alpha; args.beta = x->beta;
     args.epi = (x->out_type == MAIZE_OUT_F32 ? 1u : 0u) | ((x->alpha != 1.0f || x->beta != 0.0f) ? 2u : 0u) |
-               (x->in_type == MAIZE_IN_F16 ? 4u : 0u) | (x->in_type >= MAIZE_IN_E4M3 ? 8u : 0u) |
+               (x->in_type == MAIZE_IN_F16 ? 4u : 0u) | ((x->in_type >= MAIZE_IN_E4M3 && x->in_type <= MAIZE_IN_E5M2_E4M3) ? 8u : 0u) |
                ((x->in_type == MAIZE_IN_E5M2 || x->in_type == MAIZE_IN_E5M2_E4M3) ? 16u : 0u) |       // A is E5M2
                ((x->in_type == MAIZE_IN_E5M2 || x->in_type == MAIZE_IN_E4M3_E5M2) ? 32u : 0u);        // B is E5M2
     maize::LaunchDims ld;
@@ -462,7 +465,7 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
     if (ld.n_padded) {
         first.acols = ld.k_padded;
         first.ccols = ld.n_padded;
-        const bool in8 = x->in_type >= MAIZE_IN_E4M3;        // 8-bit operands: the copy of a K x N B is N x K
+        const bool in8 = x->in_type >= MAIZE_IN_E4M3 && x->in_type <= MAIZE_IN_E5M2_E4M3;   // 8-bit operands: the copy of a K x N B is N x K
         if (d->layout == MAIZE_LAYOUT_NN && !in8) { first.brows = ld.k_padded; first.bcols = ld.n_padded; }
         else { first.brows = ld.n_padded; first.bcols = ld.k_padded; }
         if (in8) first.layout = MAIZE_LAYOUT_NT;

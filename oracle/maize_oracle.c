@@ -400,3 +400,82 @@ int mzo_ref_gemm8_rows(const uint8_t* a, const uint8_t* b, uint32_t m,
                        uint32_t nthreads, int elem) {
     return mzo_ref_gemm8_rows_ab(a, b, m, n, k, layout, rows, nsel, c, c_f64, c_abs, nthreads, elem, elem);
 }
+
+/* ---- fp32 / fp64 operands: sums in long double, ascending k, returned as double-doubles ---- */
+
+typedef struct {
+    const void* a; const double* bd; const uint32_t* rows;
+    uint32_t n, k, r0, r1; uint64_t lda; int elem_bytes;
+    double *hi, *lo, *ab;
+} wide_job_t;
+
+static void* wide_worker(void* p) {
+    wide_job_t* j = (wide_job_t*)p;
+    long double* acc = (long double*)malloc(sizeof(long double) * j->n);
+    long double* aab = (long double*)malloc(sizeof(long double) * j->n);
+    if (!acc || !aab) { free(acc); free(aab); return NULL; }
+    for (uint32_t r = j->r0; r < j->r1; ++r) {
+        const uint64_t row = j->rows ? j->rows[r] : r;
+        for (uint32_t x = 0; x < j->n; ++x) { acc[x] = 0.0L; aab[x] = 0.0L; }
+        for (uint32_t kk = 0; kk < j->k; ++kk) {
+            const long double av = j->elem_bytes == 4 ? (long double)((const float*)j->a)[row * j->lda + kk]
+                                                      : (long double)((const double*)j->a)[row * j->lda + kk];
+            const long double aa = av < 0 ? -av : av;
+            const double* brow = j->bd + (size_t)kk * j->n;
+            for (uint32_t x = 0; x < j->n; ++x) {
+                const long double bv = (long double)brow[x];
+                acc[x] += av * bv;
+                aab[x] += aa * (bv < 0 ? -bv : bv);
+            }
+        }
+        for (uint32_t x = 0; x < j->n; ++x) {
+            const double h = (double)acc[x];
+            j->hi[(size_t)r * j->n + x] = h;
+            if (j->lo) j->lo[(size_t)r * j->n + x] = (double)(acc[x] - (long double)h);
+            if (j->ab) j->ab[(size_t)r * j->n + x] = (double)aab[x];
+        }
+    }
+    free(acc);
+    free(aab);
+    return NULL;
+}
+
+int mzo_ref_gemm_wide(const void* a, const void* b, uint32_t m, uint32_t n, uint32_t k, int layout,
+                      uint64_t lda, uint64_t ldb, int elem_bytes, const uint32_t* rows, uint32_t nsel,
+                      double* c_hi, double* c_lo, double* c_abs, uint32_t nthreads) {
+    if (!a || !b || !c_hi) return -1;
+    if (layout != MZO_LAYOUT_NN && layout != MZO_LAYOUT_NT) return -1;
+    if (elem_bytes != 4 && elem_bytes != 8) return -1;
+    if (sizeof(long double) < 10) return -1;                 /* needs the x87 extended format */
+    if (lda < k || ldb < (layout == MZO_LAYOUT_NN ? n : k)) return -1;
+    const uint32_t nrows = rows ? nsel : m;
+    if (rows) for (uint32_t r = 0; r < nsel; ++r) if (rows[r] >= m) return -1;
+    if (n == 0 || nrows == 0) return 0;
+    /* B as a compact K x N array of doubles (exact for both element types) */
+    double* bd = (double*)malloc(sizeof(double) * (size_t)n * (k ? k : 1));
+    if (!bd) return -1;
+    for (uint32_t kk = 0; kk < k; ++kk)
+        for (uint32_t x = 0; x < n; ++x) {
+            const uint64_t at = layout == MZO_LAYOUT_NN ? (uint64_t)kk * ldb + x : (uint64_t)x * ldb + kk;
+            bd[(size_t)kk * n + x] = elem_bytes == 4 ? (double)((const float*)b)[at] : ((const double*)b)[at];
+        }
+    wide_job_t base;
+    memset(&base, 0, sizeof base);
+    base.a = a; base.bd = bd; base.rows = rows; base.n = n; base.k = k; base.lda = lda; base.elem_bytes = elem_bytes;
+    base.hi = c_hi; base.lo = c_lo; base.ab = c_abs;
+    if (nthreads < 1) nthreads = 1;
+    if (nthreads > nrows) nthreads = nrows;
+    if (nthreads > 256) nthreads = 256;
+    pthread_t th[256];
+    wide_job_t jobs[256];
+    for (uint32_t t = 0; t < nthreads; ++t) {
+        jobs[t] = base;
+        jobs[t].r0 = (uint32_t)((uint64_t)nrows * t / nthreads);
+        jobs[t].r1 = (uint32_t)((uint64_t)nrows * (t + 1) / nthreads);
+        if (nthreads == 1) wide_worker(&jobs[0]);
+        else pthread_create(&th[t], NULL, wide_worker, &jobs[t]);
+    }
+    if (nthreads > 1) for (uint32_t t = 0; t < nthreads; ++t) pthread_join(th[t], NULL);
+    free(bd);
+    return 0;
+}

@@ -126,6 +126,19 @@ int mzo_ref_gemm8_rows_ab(const uint8_t* a, const uint8_t* b, uint32_t m,
                           uint32_t nsel, uint16_t* c, double* c_f64, double* c_abs,
                           uint32_t nthreads, int elem_a, int elem_b);
 
+/*
+ * fp32 / fp64 operands (elem_bytes 4 / 8), the catalogue's tf32 -> f32 and f64 -> f64 entries
+ * (crates/maize_tile/src/mma/sm80.rs:12-14): C = A.B with the products and sums carried in long double
+ * (64-bit significand on x86-64: fp32 products are exact, fp64 products and every addition round at 2^-64)
+ * in ascending k.  A is M x K with leading dimension lda, B is K x N (NN) or N x K (NT) with leading
+ * dimension ldb.  rows == NULL: all M rows; else the nsel listed rows.  Per element of the (rows x N) result:
+ * c_hi = the sum rounded to double, c_lo (optional) = the remainder rounded to double, c_abs (optional) =
+ * sum_k |a||b|.  Pinned by exact rational arithmetic, closed forms and numpy's longdouble (tests/test_oracle.py).
+ */
+int mzo_ref_gemm_wide(const void* a, const void* b, uint32_t m, uint32_t n, uint32_t k, int layout,
+                      uint64_t lda, uint64_t ldb, int elem_bytes, const uint32_t* rows, uint32_t nsel,
+                      double* c_hi, double* c_lo, double* c_abs, uint32_t nthreads);
+
 #ifdef __cplusplus
 }
 #endif

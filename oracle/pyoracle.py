@@ -59,6 +59,8 @@ def lib():
         L.mzo_ref_gemm8_ab.argtypes = [vp, vp, vp, u32, u32, u32, C.c_int, u32, u64, u64, u64, vp, vp, u32, C.c_int, C.c_int]
         L.mzo_ref_gemm8_rows_ab.restype = C.c_int
         L.mzo_ref_gemm8_rows_ab.argtypes = [vp, vp, u32, u32, u32, C.c_int, vp, u32, vp, vp, vp, u32, C.c_int, C.c_int]
+        L.mzo_ref_gemm_wide.restype = C.c_int
+        L.mzo_ref_gemm_wide.argtypes = [vp, vp, u32, u32, u32, C.c_int, u64, u64, C.c_int, vp, u32, vp, vp, vp, u32]
         _lib = L
     return _lib
 
@@ -283,3 +285,46 @@ def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16, coeff=None):
         "worst_index": worst,
         "first_fail": int(np.argmax(bad)) if bad.any() else -1,
     }
+
+
+# ---- fp32 / fp64 operands ---------------------------------------------------------------------------
+
+def ref_gemm_wide(a, b, m, n, k, layout=NN, lda=None, ldb=None, rows=None, nthreads=None):
+    """C = A.B for float32 / float64 arrays (flat, row-major views with leading dimensions lda, ldb), products
+    and sums in long double.  Returns (hi, lo, abs): hi + lo is the sum to ~2^-64, abs = sum |a||b|; each
+    (rows x n), float64.  `rows`: only these rows of A (and C)."""
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b)
+    assert a.dtype == b.dtype and a.dtype in (np.float32, np.float64)
+    lda = k if lda is None else lda
+    ldb = (n if layout == NN else k) if ldb is None else ldb
+    assert a.size >= (m - 1) * lda + k and b.size >= ((k if layout == NN else n) - 1) * ldb + (n if layout == NN else k)
+    sel = None if rows is None else np.ascontiguousarray(rows, dtype=np.uint32)
+    nr = m if sel is None else sel.size
+    hi, lo, ab = (np.zeros((nr, n), np.float64) for _ in range(3))
+    rc = lib().mzo_ref_gemm_wide(_p(a), _p(b), m, n, k, layout, lda, ldb, a.dtype.itemsize, None if sel is None else _p(sel), nr,
+                                 _p(hi), _p(lo), _p(ab), nthreads or default_threads())
+    if rc != 0:
+        raise ValueError("mzo_ref_gemm_wide rejected its arguments")
+    return hi, lo, ab
+
+
+def check_wide(got, hi, lo, ab, k, alpha=1.0, beta=0.0, c_old=None):
+    """Parity bar of the fp32 / fp64 product.  got: the device's C (float32 / float64, same shape as hi).
+    The exact value is alpha * (hi + lo) + beta * c_old; the device accumulates K / 4 four-deep matrix
+    instructions in its own type and applies alpha and beta with one multiply and one fused multiply-add, so
+    |got - exact| <= (K / 4 + 4) * u * (|alpha| * sum|a||b| + |beta| * |c_old|) with u = 2^-24 / 2^-53, plus
+    half an ulp of a subnormal result.  Returns the worst error / bound ratio (<= 1 passes)."""
+    ld = np.longdouble
+    u = 2.0 ** -24 if got.dtype == np.float32 else 2.0 ** -53
+    tiny = 2.0 ** -150 if got.dtype == np.float32 else 2.0 ** -1074
+    # alpha and beta reach the device as fp32
+    al, be = ld(np.float32(alpha)), ld(np.float32(beta))
+    exact = al * (hi.astype(ld) + lo.astype(ld))
+    scale = abs(al) * ab.astype(ld)
+    if c_old is not None and beta != 0.0:
+        exact = exact + be * c_old.astype(ld)
+        scale = scale + abs(be) * np.abs(c_old.astype(ld))
+    err = np.abs(got.astype(ld) - exact)
+    tol = (k / 4.0 + 4.0) * u * scale + tiny
+    return float((err / tol).max()) if err.size else 0.0

@@ -192,5 +192,50 @@ def test_dispatch_of_8bit_operands():
         if name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")):
             assert not _supports(name, ex(**big)) and not _supports(name, ex(**big, in_type=mz.IN_F16))
     with pytest.raises(mz.MaizeError) as e:
-        mz.validate(ex(in_type=6))
+        mz.validate(ex(in_type=8))
     assert e.value.code == _ffi.MAIZE_ERR_ARG
+
+
+def test_dispatch_of_fp32_and_fp64_operands():
+    """One kernel per type and layout takes every shape; rows that start on 16-byte boundaries and hold whole
+    16-byte chunks are flagged for 128-bit accesses (bit 0 / 1 / 2 = A / B / C), everything else goes element-wise."""
+    for it, tag, vec in ((mz.IN_F32, "f32", 4), (mz.IN_F64, "f64", 2)):
+        for layout, lay in ((mz.LAYOUT_NN, "nn"), (mz.LAYOUT_NT, "nt")):
+            name = f"maize_gemm_{tag}_mt128_{lay}"
+            for shape in ((4096, 4096, 4096), (1, 1, 1), (16, 14336, 4096), (33, 17, 65), (129, 131, 67)):
+                x = ex(*shape, layout=layout, in_type=it)
+                plan = mz.gemm_plan(x)
+                assert plan["kernel"] == name, (shape, plan)
+                m, n, k = shape
+                assert plan["grid"] == (-(-m // 128) * -(-n // 128), 1, 1) and plan["block"] == (256, 1, 1)
+                assert plan["workspace_bytes"] == 0 and plan["ksplit"] == 0
+                want = (1 if k % vec == 0 else 0) | (2 if (n if layout == mz.LAYOUT_NN else k) % vec == 0 else 0) | (4 if n % vec == 0 else 0)
+                assert plan["split_first"] == want, (shape, layout, plan)
+            # no other kernel claims these operands, and these kernels claim no others
+            x = ex(256, 256, 256, layout=layout, in_type=it)
+            assert [nm for nm in mz.kernel_names() if _supports(nm, x)] == [name]
+            for other in (mz.IN_BF16, mz.IN_F16, mz.IN_E4M3):
+                assert not _supports(name, ex(256, 256, 256, layout=layout, in_type=other))
+        # pointers that are only element aligned, a leading dimension that is not a multiple of 16 bytes, batch strides
+        es = 16 // vec
+        assert mz.gemm_plan(ex(256, 256, 256, in_type=it, ptrs=(0x1000 + es, 0x100000, 0x2000000)))["split_first"] == 6
+        assert mz.gemm_plan(ex(256, 256, 256, in_type=it, ptrs=(0x1000, 0x100000 + es, 0x2000000 + es)))["split_first"] == 1
+        assert mz.gemm_plan(ex(256, 256, 256, in_type=it, ldc=256 + vec + 1))["split_first"] == 3
+        assert mz.gemm_plan(ex(256, 256, 256, in_type=it, lda=256 + vec))["split_first"] == 7
+        s = 256 * 256
+        assert mz.gemm_plan(ex(256, 256, 256, in_type=it, batch=2, stride_a=s + 1, stride_b=s, stride_c=s))["split_first"] == 6
+        assert mz.gemm_plan(ex(256, 256, 256, in_type=it, batch=3, stride_a=s, stride_b=s, stride_c=s))["grid"] == (4, 1, 3)
+        # pointers must be aligned to the element
+        with pytest.raises(mz.MaizeError) as e:
+            mz.validate(ex(in_type=it, ptrs=(0x1000 + es // 2, 0x100000, 0x2000000)))
+        assert e.value.code == _ffi.MAIZE_ERR_ALIGN
+        with pytest.raises(mz.MaizeError) as e:
+            mz.validate(ex(in_type=it, ptrs=(0x1000, 0x100000, 0x2000000 + es // 2)))
+        assert e.value.code == _ffi.MAIZE_ERR_ALIGN
+    # C of fp64 operands is fp64; for fp32 operands both spellings of the output type mean fp32
+    with pytest.raises(mz.MaizeError) as e:
+        mz.validate(ex(in_type=mz.IN_F64, out_type=mz.OUT_F32))
+    assert e.value.code == _ffi.MAIZE_ERR_ARG
+    assert mz.gemm_plan(ex(in_type=mz.IN_F32, out_type=mz.OUT_F32))["kernel"] == "maize_gemm_f32_mt128_nn"
+    with pytest.raises(mz.MaizeError):
+        mz.validate(ex(in_type=8))

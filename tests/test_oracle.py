@@ -370,3 +370,87 @@ def test_fp8_gemm_vs_numpy_float64_and_closed_forms(oracle):
     c5, _, _ = oracle.ref_gemm(a, b, m, n, k, elem=oracle.E5M2)
     assert not np.array_equal(c4, c5)
     assert oracle.floor_coeff_f8(4096) == 2.0 ** -15 + (4096 / 64 + 2) * 2.0 ** -24
+
+
+# ---- fp32 / fp64 operands: the long-double reference --------------------------------------------------
+
+def test_wide_gemm_matches_exact_rational_arithmetic(oracle):
+    """hi + lo against sums of exact products in rational arithmetic: within 2^-62 of the scale, and hi is the
+    correctly rounded double wherever the exact sum is not within 2^-62 of a rounding boundary."""
+    rng = np.random.default_rng(41)
+    for dt in (np.float32, np.float64):
+        for layout in (oracle.NN, oracle.NT):
+            m, n, k = 3, 4, 9
+            a = (rng.random(m * k) * 2 - 1).astype(dt)
+            b = (rng.random(k * n) * 2 - 1).astype(dt)
+            B = b.reshape(k, n) if layout == oracle.NN else b.reshape(n, k).T
+            hi, lo, ab = oracle.ref_gemm_wide(a, b, m, n, k, layout=layout)
+            for i in range(m):
+                for j in range(n):
+                    exact = sum(Fraction(float(a[i * k + t])) * Fraction(float(B[t, j])) for t in range(k))
+                    scale = sum(abs(Fraction(float(a[i * k + t])) * Fraction(float(B[t, j]))) for t in range(k))
+                    got = Fraction(float(hi[i, j])) + Fraction(float(lo[i, j]))
+                    assert abs(got - exact) <= scale * Fraction(1, 2 ** 60)
+                    assert abs(Fraction(float(ab[i, j])) - scale) <= scale * Fraction(1, 2 ** 50)
+                    assert abs(Fraction(float(hi[i, j])) - exact) <= abs(exact) * Fraction(1, 2 ** 53) + scale * Fraction(1, 2 ** 60)
+
+
+def test_wide_gemm_closed_forms_views_rows_and_numpy(oracle):
+    rng = np.random.default_rng(42)
+    for dt in (np.float32, np.float64):
+        # integers: exact, lo == 0
+        A = rng.integers(-9, 10, (6, 11)).astype(dt)
+        B = rng.integers(-9, 10, (11, 5)).astype(dt)
+        hi, lo, ab = oracle.ref_gemm_wide(A.ravel(), B.ravel(), 6, 5, 11)
+        assert np.array_equal(hi, (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float64)) and not lo.any()
+        assert np.array_equal(ab, (np.abs(A).astype(np.int64) @ np.abs(B).astype(np.int64)).astype(np.float64))
+        # identity and a power-of-two scaling are exact
+        X = (rng.random((8, 8)) * 2 - 1).astype(dt)
+        hi, lo, _ = oracle.ref_gemm_wide(np.eye(8, dtype=dt).ravel() * dt(0.25), X.ravel(), 8, 8, 8)
+        assert np.array_equal(hi, X.astype(np.float64) * 0.25) and not lo.any()
+        # a transposed B (NT) is the same product; leading dimensions select views; rows select rows
+        m, n, k, lda, ldb = 7, 9, 13, 20, 17
+        a = (rng.random(m * lda) * 2 - 1).astype(dt)
+        b = (rng.random(k * ldb) * 2 - 1).astype(dt)
+        ac, bc = a.reshape(m, lda)[:, :k].copy(), b.reshape(k, ldb)[:, :n].copy()
+        want = oracle.ref_gemm_wide(ac.ravel(), bc.ravel(), m, n, k)
+        for got in (oracle.ref_gemm_wide(a, b, m, n, k, lda=lda, ldb=ldb),
+                    oracle.ref_gemm_wide(ac.ravel(), bc.T.copy().ravel(), m, n, k, layout=oracle.NT),
+                    oracle.ref_gemm_wide(ac.ravel(), bc.ravel(), m, n, k, nthreads=1)):
+            assert all(np.array_equal(g, w) for g, w in zip(got, want))
+        rows = np.array([5, 0, 5, 2], np.uint32)
+        sel = oracle.ref_gemm_wide(ac.ravel(), bc.ravel(), m, n, k, rows=rows)
+        assert all(np.array_equal(g, w[rows]) for g, w in zip(sel, want))
+        # numpy's long double matmul on the same values: equal to ~2^-62 of the scale
+        ld = np.longdouble
+        ref = ac.astype(ld) @ bc.astype(ld)
+        assert np.all(np.abs((want[0].astype(ld) + want[1].astype(ld)) - ref) <= want[2] * 2.0 ** -60)
+        # fp64 really is carried beyond double: (1 + 2^-30)^2 - 1 - 2^-29 = 2^-60 survives in hi + lo
+        if dt is np.float64:
+            x = 1.0 + 2.0 ** -30
+            hi, lo, _ = oracle.ref_gemm_wide(np.array([x, -1.0, -2.0 ** -29]), np.array([x, 1.0, 1.0]), 1, 1, 3)
+            assert hi[0, 0] + lo[0, 0] == 2.0 ** -60
+    with pytest.raises(ValueError):
+        oracle.ref_gemm_wide(np.zeros(4, np.float32), np.zeros(4, np.float32), 2, 2, 2, rows=np.array([2], np.uint32))
+
+
+def test_wide_comparator_has_teeth(oracle):
+    """The bar passes a result rounded once from the exact sum and one perturbed by a few ulps of the scale per
+    K / 4 terms, and rejects a dropped term, a transposed operand and a swapped alpha / beta."""
+    rng = np.random.default_rng(43)
+    for dt, u in ((np.float32, 2.0 ** -24), (np.float64, 2.0 ** -53)):
+        m, n, k = 24, 20, 64
+        a = (rng.random(m * k) * 2 - 1).astype(dt)
+        b = (rng.random(k * n) * 2 - 1).astype(dt)
+        c0 = rng.standard_normal((m, n)).astype(dt)
+        hi, lo, ab = oracle.ref_gemm_wide(a, b, m, n, k)
+        good = hi.astype(dt)
+        assert oracle.check_wide(good, hi, lo, ab, k) <= 1.0
+        assert oracle.check_wide((hi + 3 * u * ab).astype(dt), hi, lo, ab, k) <= 1.0
+        A, B = a.reshape(m, k).astype(np.float64), b.reshape(k, n).astype(np.float64)
+        dropped = (hi - np.outer(A[:, 17], B[17])).astype(dt)
+        assert oracle.check_wide(dropped, hi, lo, ab, k) > 100
+        assert oracle.check_wide((A[:, ::-1] @ B).astype(dt), hi, lo, ab, k) > 100
+        full = (0.5 * hi + 2.0 * c0.astype(np.float64)).astype(dt)
+        assert oracle.check_wide(full, hi, lo, ab, k, alpha=0.5, beta=2.0, c_old=c0) <= 1.0
+        assert oracle.check_wide(full, hi, lo, ab, k, alpha=2.0, beta=0.5, c_old=c0) > 100
