@@ -499,7 +499,11 @@ bool skinny_nt_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Launc
 // others element by element: bit 0 / 1 / 2 of split_first says so for A / B / C.
 template <uint32_t TYPE, bool NT>
 bool mt128_supports(const maize_gemm_ex_desc_t& d) {
-    return d.in_type == TYPE && (d.gemm.layout == MAIZE_LAYOUT_NT) == NT && (TYPE == MAIZE_IN_F32 || d.out_type == MAIZE_OUT_SAME);
+    if (d.in_type != TYPE || (d.gemm.layout == MAIZE_LAYOUT_NT) != NT || !(TYPE == MAIZE_IN_F32 || d.out_type == MAIZE_OUT_SAME)) return false;
+    // 32-bit byte offsets inside a tile's 128 rows: a row of A or B spans less than 16 MiB
+    const Lds l = lds_of(d);
+    const uint64_t es = TYPE == MAIZE_IN_F64 ? 8u : 4u;
+    return l.a * es < (1u << 24) && l.b * es < (1u << 24);
 }
 bool mt128_plan(const maize_gemm_ex_desc_t& d, uint32_t, LaunchDims* ld) {
     const Dims s = dims_of(d);

@@ -24,7 +24,10 @@
 //     row of C and stores them as one or two 128-bit words;
 //   * any M, N, K, leading dimension and element-aligned pointer: rows that are 16-byte aligned are
 //     loaded and stored 128 bits at a time, anything else element by element (a launch-uniform choice
-//     made on the host, bit 0 / 1 / 2 of `reserved` for A / B / C);
+//     made on the host, bit 0 / 1 / 2 of `reserved` for A / B / C; the loop exists in both versions).
+//     Operands are read by buffer loads whose range check supplies the zeros past M, N and K: no
+//     branch in the loop.  A tile's 128 rows must span less than 2 GiB (leading dimension times
+//     element size below 16 MiB);
 //   * C = alpha * A.B + beta * C in the operands' type (beta == 0: C is not read).
 #pragma once
 #include "common.hpp"
@@ -59,6 +62,9 @@ template <> struct Elem<double> {
 __device__ __forceinline__ float fma_t(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double fma_t(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
+struct aligned_yes { static constexpr bool value = true; };
+struct aligned_no { static constexpr bool value = false; };
+
 template <typename T, bool NT>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     typedef Elem<T> E;
@@ -86,30 +92,56 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
     // ---- global -> register -> LDS copy maps: 1024 chunks of 16 bytes per tile, 4 per thread --------
     // K-contiguous tile: chunk c = (row c / 8, 16-byte column c % 8); K x N tile: (k row c / CPR, column c % CPR).
+    // The loads are buffer loads without a branch: the descriptor starts at the tile's first row (re-based by
+    // the scalar unit for every K tile) and ends with the matrix view, so rows past the matrix are past the end
+    // and read as zero; columns past a row's end get an out-of-range offset instead.
     constexpr int CPR = 128 / VEC;                           // chunks per row of the K x N tile
-    u32x4 ra[4], rb[4];
-    auto load_chunk = [&](const T* base, uint64_t ld, uint32_t row, uint32_t rows, uint32_t col, uint32_t cols, bool vec) -> u32x4 {
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (row < rows && col < cols) {
-            const T* src = base + (uint64_t)row * ld + col;
-            if (vec) {
-                v = *(const u32x4*)src;                      // cols % VEC == 0: a chunk is all in or all out
-            } else {
-                T e[VEC];
+    constexpr uint32_t OOB = 0x80000000u;
+    const uint64_t a_end = ((uint64_t)(M - 1u) * lda + K) * ES;                           // bytes of each view
+    const uint64_t b_end = ((uint64_t)((NT ? N : K) - 1u) * ldb + (NT ? K : N)) * ES;
+    const char* const a_tile = (const char*)A + (uint64_t)m0 * lda * ES;                  // first row of this tile
+    const uint64_t a_left = a_end - (uint64_t)m0 * lda * ES;
+    const char* const b_tile = (const char*)B + (NT ? (uint64_t)n0 * ldb * ES : (uint64_t)n0 * ES);
+    const uint64_t b_left = b_end - (NT ? (uint64_t)n0 * ldb * ES : (uint64_t)n0 * ES);
+    uint32_t a_off[4], b_off[4], a_col[4], b_col[4];         // byte offset of the chunk inside the tile; its first column
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) e[i] = col + i < cols ? src[i] : (T)0;
-                v = __builtin_bit_cast(u32x4, e);
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t c = tid + 256u * i;
+        a_off[i] = ((c >> 3) * lda + (c & 7u) * VEC) * ES;
+        a_col[i] = (c & 7u) * VEC;                           // k inside the K tile
+        if (NT) { b_off[i] = ((c >> 3) * ldb + (c & 7u) * VEC) * ES; b_col[i] = (c & 7u) * VEC; }
+        else    { b_off[i] = ((c / CPR) * ldb + (c % CPR) * VEC) * ES; b_col[i] = n0 + (c % CPR) * VEC; }   // column of B
+    }
+    auto rsrc_at = [&](const char* base, uint64_t left) {
+        const uint64_t n = left < 0x7FFFFFFFull ? left : 0x7FFFFFFFull;
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, (uint32_t)n, 0x00020000);
+    };
+    u32x4 ra[4], rb[4];
+    // One chunk: 128 bits at once (ALIGNED: a chunk is all in or all out of its row), or element by element.
+    auto load_chunk = [&](__amdgpu_buffer_rsrc_t rs, uint32_t off, uint32_t col, uint32_t cols, bool aligned) -> u32x4 {
+        if (aligned) return __builtin_amdgcn_raw_buffer_load_b128(rs, off | (col < cols ? 0u : OOB), 0, 0);
+        u32x4 v;
+        if (ES == 8) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(rs, (off + 8u * e) | (col + e < cols ? 0u : OOB), 0, 0);
+                v[2 * e] = t[0]; v[2 * e + 1] = t[1];
             }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = __builtin_amdgcn_raw_buffer_load_b32(rs, (off + 4u * e) | (col + e < cols ? 0u : OOB), 0, 0);
         }
         return v;
     };
-    auto load_tile = [&](uint32_t k0) {
+    auto load_tile = [&](uint32_t k0, bool aligned) {
+        // the K tile's first column (A, B stored N x K) or first row (row-major B) becomes the descriptor's base
+        const uint64_t a_skip = (uint64_t)k0 * ES, b_skip = NT ? (uint64_t)k0 * ES : (uint64_t)k0 * ldb * ES;
+        const __amdgpu_buffer_rsrc_t rs_a = rsrc_at(a_tile + a_skip, a_left > a_skip ? a_left - a_skip : 0);
+        const __amdgpu_buffer_rsrc_t rs_b = rsrc_at(b_tile + b_skip, b_left > b_skip ? b_left - b_skip : 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t c = tid + 256u * i;
-            ra[i] = load_chunk(A, lda, m0 + (c >> 3), M, k0 + (c & 7u) * VEC, K, vec_a);
-            if (NT) rb[i] = load_chunk(B, ldb, n0 + (c >> 3), N, k0 + (c & 7u) * VEC, K, vec_b);
-            else    rb[i] = load_chunk(B, ldb, k0 + c / CPR, K, n0 + (c % CPR) * VEC, N, vec_b);
+            ra[i] = load_chunk(rs_a, a_off[i], k0 + a_col[i], K, aligned);
+            rb[i] = NT ? load_chunk(rs_b, b_off[i], k0 + b_col[i], K, aligned) : load_chunk(rs_b, b_off[i], b_col[i], N, aligned);
         }
     };
     auto store_tile = [&](int stage) {
@@ -139,30 +171,35 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int j = 0; j < 4; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
     const uint32_t nk = (K + BK - 1) / BK;
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-    for (uint32_t kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1u;
-        if (kt + 1 < nk) load_tile((kt + 1) * BK);          // lands while the MFMAs below run
-        lds_ptr sa = (lds_ptr)lds + cur * 2 * TILE, sb = sa + TILE;
-#pragma unroll
-        for (int kk = 0; kk < BK / 4; ++kk) {
-            T fa[4], fb[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = *(__attribute__((address_space(3))) T*)(sa + a_rd + i * 16 * KROW + kk * 4 * ES);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                fb[j] = NT ? *(__attribute__((address_space(3))) T*)(sb + b_rd + j * 16 * KROW + kk * 4 * ES)
-                           : *(__attribute__((address_space(3))) T*)(sb + b_rd + kk * 4 * E::NROW + j * 16 * ES);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = E::mfma(fb[j], fa[i], acc[i][j]);
-        }
-        if (kt + 1 < nk) store_tile(cur ^ 1);
+    auto main_loop = [&](auto aligned_tag) {
+        constexpr bool ALIGNED = decltype(aligned_tag)::value;
+        load_tile(0, ALIGNED);
+        store_tile(0);
         __syncthreads();
-    }
+        for (uint32_t kt = 0; kt < nk; ++kt) {
+            const int cur = kt & 1u;
+            if (kt + 1 < nk) load_tile((kt + 1) * BK, ALIGNED);  // lands while the MFMAs below run
+            lds_ptr sa = (lds_ptr)lds + cur * 2 * TILE, sb = sa + TILE;
+#pragma unroll
+            for (int kk = 0; kk < BK / 4; ++kk) {
+                T fa[4], fb[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) fa[i] = *(__attribute__((address_space(3))) T*)(sa + a_rd + i * 16 * KROW + kk * 4 * ES);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    fb[j] = NT ? *(__attribute__((address_space(3))) T*)(sb + b_rd + j * 16 * KROW + kk * 4 * ES)
+                               : *(__attribute__((address_space(3))) T*)(sb + b_rd + kk * 4 * E::NROW + j * 16 * ES);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[i][j] = E::mfma(fb[j], fa[i], acc[i][j]);
+            }
+            if (kt + 1 < nk) store_tile(cur ^ 1);
+            __syncthreads();
+        }
+    };
+    // rows of A and B on 16-byte boundaries (a launch-uniform fact): the 128-bit version of the loop
+    if (vec_a && vec_b) main_loop(aligned_yes{}); else main_loop(aligned_no{});
 
     // ---- epilogue: lane holds C[m0 + wm 64 + 16 i + l % 16][n0 + wn 64 + 16 j + 4 (l / 16) + 0..3] ----
     const bool scaled = p.epi & EPI_SCALE;
@@ -217,7 +254,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 }  // namespace mt128
 
 #define MAIZE_MT128_KERNEL(name, type, nt) \
-    extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt128::body<type, nt>(p); }
+    extern "C" __global__ __launch_bounds__(256, 2) void name(GemmArgs p) { mt128::body<type, nt>(p); }
 MAIZE_MT128_KERNEL(maize_gemm_f32_mt128_nn, float, false)
 MAIZE_MT128_KERNEL(maize_gemm_f32_mt128_nt, float, true)
 MAIZE_MT128_KERNEL(maize_gemm_f64_mt128_nn, double, false)

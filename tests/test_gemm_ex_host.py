@@ -232,6 +232,10 @@ def test_dispatch_of_fp32_and_fp64_operands():
         with pytest.raises(mz.MaizeError) as e:
             mz.validate(ex(in_type=it, ptrs=(0x1000, 0x100000, 0x2000000 + es // 2)))
         assert e.value.code == _ffi.MAIZE_ERR_ALIGN
+    # a row of A or B must span less than 16 MiB (32-bit offsets inside a tile's 128 rows)
+    assert _supports("maize_gemm_f64_mt128_nn", ex(256, 256, 256, in_type=mz.IN_F64, lda=(1 << 21) - 2))
+    assert not _supports("maize_gemm_f64_mt128_nn", ex(256, 256, 256, in_type=mz.IN_F64, lda=1 << 21))
+    assert not _supports("maize_gemm_f32_mt128_nt", ex(256, 256, 256, layout=mz.LAYOUT_NT, in_type=mz.IN_F32, ldb=1 << 22))
     # C of fp64 operands is fp64; for fp32 operands both spellings of the output type mean fp32
     with pytest.raises(mz.MaizeError) as e:
         mz.validate(ex(in_type=mz.IN_F64, out_type=mz.OUT_F32))
