@@ -104,7 +104,7 @@ inline maize_gemm_ex_desc_t gemm_ex_desc(const maize_gemm_desc_t& d, uint32_t ld
     x.lda = lda; x.ldb = ldb; x.ldc = ldc;
     x.out_type = out;
     x.alpha = alpha; x.beta = beta;
-    x.in_type = in;            // half, or the 8-bit E4M3 / E5M2 (one byte per element; the Matrix views then wrap byte pointers)
+    x.in_type = in;            // half, the 8-bit E4M3 / E5M2 (one byte per element), fp32 or fp64; the Matrix views then wrap pointers to elements of that size
     return x;
 }
 

@@ -14,6 +14,8 @@ pub const MAIZE_IN_E4M3: u32 = 2;
 pub const MAIZE_IN_E5M2: u32 = 3;
 pub const MAIZE_IN_E4M3_E5M2: u32 = 4;
 pub const MAIZE_IN_E5M2_E4M3: u32 = 5;
+pub const MAIZE_IN_F32: u32 = 6;
+pub const MAIZE_IN_F64: u32 = 7;
 
 /// == GlobalMatrix<T>::Realized of the reference (src/main.rs:20-27): pointer + two u32 extents, 16-byte aligned.
 #[repr(C, align(16))]

@@ -80,6 +80,13 @@ def test_matrix_instruction_per_kernel(kernels):
             want = "v_mfma_f32_16x16x32_f16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_16x16x32_bf16"
             other = "v_mfma_f32_16x16x32_bf16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_16x16x32_f16"
             assert count(ins, want) == 256 and count(ins, other) == 0 and count(ins, "v_mfma_f32_32x32") == 0, name   # two fully unrolled K steps of 64
+        elif "_mt128_" in name:
+            # the catalogue's tf32 and f64 entries: full fp32 / fp64 matrix instructions; one K tile of 128 bytes
+            # per row (8 or 4 steps of 16 MFMAs), in the 128-bit and in the element-wise version of the loop
+            want = "v_mfma_f64_16x16x4_f64" if "_f64_" in name else "v_mfma_f32_16x16x4_f32"
+            per_tile = 64 if "_f64_" in name else 128
+            assert count(ins, want) == 2 * per_tile and count(ins, "v_mfma") == 2 * per_tile, name
+            assert count(ins, "buffer_load_dwordx4") >= 16, name      # operands by buffer loads (range-checked edges), two tiles' worth
         elif name == "maize_gemm_bf16_skinny_nn":
             assert count(ins, "v_mfma_f32_16x16x32_bf16") >= 16 and count(ins, "v_mfma_f32_16x16x32_f16") >= 16
         elif name == "maize_gemm_bf16_wave32":
