@@ -74,20 +74,22 @@ constexpr int NROW = 512;               // bytes per LDS row of a K x N tile (25
 constexpr int TILE = 32768;             // bytes of one operand tile
 constexpr uint32_t OOB = 0x80000000u;   // OR-ed into an offset: >= num_records, reads as zero
 // When each of the 16 pieces of tile t+2 is requested, as an MFMA slot counted from the barrier of
-// step t: slots 0..15 are the last quarter of step t, 16..63 the first three quarters of step t+1.
-// A wave retires at most one 1 KiB direct-to-LDS load per ~64 cycles (two MFMA slots), so the
-// requests are spaced out; they all have to land before the barrier of step t+1 (slot 64).
-#ifndef MAIZE_MT256_SCHED
-#define MAIZE_MT256_SCHED {1, 3, 5, 7, 9, 11, 13, 15, 17, 19, 21, 23, 25, 27, 29, 31}
+// step t: slots 0..31 are the last quarter of step t (its last two eighths), 32..127 the first three
+// quarters of step t+1.  Piece pc goes out at slot DMA_STRIDE * pc + 2: a wave retires at most one 1 KiB
+// direct-to-LDS load per ~64 cycles (four MFMA slots), so the requests are spaced out; they all have to
+// land before the barrier of step t+1 (slot 128).
+#ifndef MAIZE_MT256_DMA_STRIDE
+#define MAIZE_MT256_DMA_STRIDE 4
 #endif
-constexpr int kIssueSlot[16] = MAIZE_MT256_SCHED;
+constexpr int DMA_STRIDE = MAIZE_MT256_DMA_STRIDE;
+constexpr int issue_slot(int pc) { return DMA_STRIDE * pc + 2; }
+static_assert(DMA_STRIDE >= 3 && issue_slot(15) < 96, "the last request needs at least a quarter of a step to land before the barrier");
+// Pieces requested behind the barrier of step t itself (the rest follow in step t+1).
+constexpr int early_pieces() { int n = 0; for (int i = 0; i < 16; ++i) n += issue_slot(i) < 32; return n; }
 // Cache policy bits of the direct-to-LDS loads (bit 0 sc0, bit 1 nt, bit 4 sc1).
 #ifndef MAIZE_MT256_DMA_AUX
 #define MAIZE_MT256_DMA_AUX 0
 #endif
-constexpr bool sched_is_regular() { for (int i = 0; i < 16; ++i) if (kIssueSlot[i] != 2 * i + 1) return false; return true; }
-static_assert(sched_is_regular(), "the K loop issues piece pc at MFMA slot 2 * (2 pc + 1): keep the table in step with it");
-constexpr int early_pieces() { int n = 0; for (int i = 0; i < 16; ++i) n += kIssueSlot[i] < 16; return n; }
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
 typedef __attribute__((address_space(3))) u32x4* lds_v4;
@@ -383,13 +385,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     if (h4 == 2 && r < 4) { if (kh == 0) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }     // next half: A group 0
                     if (h4 == 3 && r < NBR) { if (kh == 0) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }   // next half: B group 0
                 }
-                // ... and the direct-to-LDS requests scheduled for this slot (kIssueSlot counts slots of
-                // two of these MFMAs): late pieces of tile t+1 (its stage was freed by the previous
-                // barrier) in the first quarter, early pieces of tile t+2 behind this step's barrier.
+                // ... and the direct-to-LDS request scheduled for this slot (issue_slot): late pieces of
+                // tile t+1 (its stage was freed by the previous barrier) before this step's barrier, early
+                // pieces of tile t+2 behind it.
                 const int slot = e >= 6 ? 16 * (e - 6) + s : 32 + 16 * e + s;
-                if ((slot & 3) == 2 && slot < 64) {            // piece pc goes out at slot 4 pc + 2 = 2 kIssueSlot[pc]
-                    if (e >= 6) dma(slot >> 2, ca, cb, k_early);
-                    else        dma(slot >> 2, na, nb, k_late);
+                if (slot >= 2 && (slot - 2) % DMA_STRIDE == 0 && (slot - 2) / DMA_STRIDE < 16) {
+                    if (e >= 6) dma((slot - 2) / DMA_STRIDE, ca, cb, k_early);
+                    else        dma((slot - 2) / DMA_STRIDE, na, nb, k_late);
                 }
                 MAIZE_FENCE();
             }

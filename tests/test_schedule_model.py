@@ -29,15 +29,14 @@ class Hazard(AssertionError):
 # ---------------------------------------------------------------------------------------
 
 def mt256_issue_slots():
+    """MFMA slot (counted from the barrier of step t, 128 slots per step) at which each of the 16 pieces of tile
+    t + 2 is requested, as the kernel source defines it."""
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
-    m = re.search(r"#define MAIZE_MT256_SCHED \{([0-9,\s]+)\}", src)
-    slots = [int(x) for x in m.group(1).split(",")]
-    assert len(slots) == 16
-    # the table counts slots of two MFMAs; the loop tests (slot & 3) == 2 on single-MFMA slots and is tied to
-    # the table by a static_assert
-    assert "if ((slot & 3) == 2 && slot < 64)" in src and "static_assert(sched_is_regular()" in src
-    assert "kIssueSlot[i] != 2 * i + 1" in src
-    return slots
+    stride = int(re.search(r"#define MAIZE_MT256_DMA_STRIDE (\d+)", src).group(1))
+    assert "constexpr int issue_slot(int pc) { return DMA_STRIDE * pc + 2; }" in src
+    assert "if (slot >= 2 && (slot - 2) % DMA_STRIDE == 0 && (slot - 2) / DMA_STRIDE < 16) {" in src
+    assert "n += issue_slot(i) < 32;" in src                 # early pieces: those behind the barrier of step t itself
+    return [stride * pc + 2 for pc in range(16)]
 
 
 def mt256_reads_per_eighth(nt):
@@ -71,7 +70,7 @@ def mt256_wave_program(nk, slots, nt, barrier_eighth=6):
         ops.append(("dma", 0, pc, 0))
     ops += [("wait_all",), ("barrier",)]
     ops += [("read", 0, 0, 0)] * (4 + nbr)
-    early = [pc for pc in range(16) if 2 * slots[pc] < 32]
+    early = [pc for pc in range(16) if slots[pc] < 32]
     for pc in early:
         ops.append(("dma", 1, pc, 1))
     k_early, k_late = 2, 1
@@ -88,7 +87,7 @@ def mt256_wave_program(nk, slots, nt, barrier_eighth=6):
                     ops.append(("read", t + 1, need, nxt) if next_tile else ("read", t, need, cur))
                 slot = 16 * (e - 6) + s if e >= 6 else 32 + 16 * e + s
                 for pc in range(16):
-                    if 2 * slots[pc] == slot and slot < 64:
+                    if slots[pc] == slot:
                         ops.append(("dma", k_early, pc, cur) if e >= 6 else ("dma", k_late, pc, nxt))
         k_early += 1
         k_late += 1
@@ -175,7 +174,7 @@ def mt256_cumulative_reads(nt):
 @pytest.mark.parametrize("nt", [False, True])
 def test_macro_tile_schedule_is_hazard_free(nk, nt):
     slots = mt256_issue_slots()
-    assert all(0 <= 2 * s < 64 for s in slots), "every request of tile t+2 must be issued before the barrier of step t+1"
+    assert all(0 <= s < 96 for s in slots), "every request of tile t+2 must be issued a quarter of a step before the barrier of step t+1"
     ops, steps = mt256_wave_program(nk, slots, nt)
     last_tile = check_two_stage(ops, steps, mt256_cumulative_reads(nt), parts=8)
     # tiles past the end are requested (through a zero-length descriptor) but never multiplied
@@ -195,7 +194,7 @@ def test_macro_tile_checker_rejects_broken_schedules():
         check_two_stage(ops, steps, need, parts=8)
     # a request scheduled past the next barrier never gets issued
     bad = list(slots)
-    bad[5] = 64
+    bad[5] = 128
     ops, steps = mt256_wave_program(8, bad, True)
     with pytest.raises(Hazard):
         check_two_stage(ops, steps, need, parts=8)
