@@ -141,9 +141,12 @@ bool mt256_plan_impl(const maize_gemm_ex_desc_t& d, uint32_t compute_units, bool
     if (tiles > 0x1FFFFFFFull) return false;
     EdgeSplit e = mt256_edge(s, d.gemm.batch, compute_units);
     if (!allow_edge) e = EdgeSplit{0, (uint32_t)tiles, 0, 0};
+    const uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
     if (allow_edge) {
-        // The edge-splitting kernels compute one tile, or one K range of an edge tile, per workgroup.
-        ld->grid[0] = e.mode ? e.whole + e.nedge * e.ks : (uint32_t)tiles;
+        // The edge-splitting kernels walk, per batch member (grid.z), the list of whole tiles followed by the
+        // (edge tile, K range) items: persistent like the plain kernels, so the short edge items fill the tail.
+        const uint32_t items = e.mode ? e.whole + e.nedge * e.ks : (uint32_t)tiles;
+        ld->grid[0] = (resident && items > resident) ? resident : items;
         ld->grid[2] = d.gemm.batch;
     } else {
         // Persistent: one workgroup per compute unit walks the list of all tiles of all batch
@@ -151,7 +154,6 @@ bool mt256_plan_impl(const maize_gemm_ex_desc_t& d, uint32_t compute_units, bool
         // neighbours); with fewer tiles than compute units, one workgroup per tile.
         const uint64_t all = tiles * d.gemm.batch;
         if (all > 0x1FFFFFFFull) return false;
-        uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
         ld->grid[0] = (resident && all > resident) ? resident : (uint32_t)all;
         ld->grid[2] = 1;
     }

@@ -43,8 +43,9 @@
 //
 //   * a ragged N (or M) leaves a last column (row) of tiles that are almost empty but cost a full
 //     tile each, and can push the tile count just past a multiple of the CU count.  The _edge
-//     kernels let the dispatcher hand those tiles to `ksplit` workgroups each, one K range apiece.  Such a workgroup
-//     writes the part of its fp32 partial tile that lies inside the matrix to a library-owned
+//     kernels cut each of those tiles into `ksplit` K ranges: work items that follow the whole tiles in the
+//     persistent workgroups' list, so they fill the tail instead of forming a round of their own.  A workgroup
+//     with such an item writes the part of its fp32 partial tile that lies inside the matrix to a library-owned
 //     workspace (device-coherent stores), takes a ticket with a device-scope atomic, and the last
 //     arriver re-reads all partials in range order (deterministic), then runs the normal epilogue.
 //
@@ -150,34 +151,34 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // tiles, `ksplit` workgroups (K ranges) per tile.
     const uint32_t mode = EDGE ? p.reserved >> 30 : 0u;
     const uint32_t whole = (EDGE && p.reserved) ? (p.reserved & 0x3FFFFFFFu) - 1u : tm * tn;
-    const bool split = EDGE && blockIdx.x >= whole;
-    const uint32_t ks = split ? p.ksplit : 1u;
-    const uint32_t edge = split ? (blockIdx.x - whole) / ks : 0u;     // which edge tile
-    const uint32_t z = split ? (blockIdx.x - whole) % ks : 0u;        // which K range
-    // K steps of this workgroup: [kt0, kt0 + nk) of the ceil(K / BK) steps.  The split-K kernels
-    // (SPLITK) give every work item its own range instead (select_tile).
+    const uint32_t nedge = mode == 1u ? tm : tn;                      // edge tiles (0 K ranges each without edge splitting)
+    // Edge splitting: the work items of a batch member are the `whole` tiles, then (edge tile, K range) pairs.
+    // State of the item in hand (select_tile):
+    bool split = false;                                               // it is one K range of an edge tile
+    uint32_t ks = 1u, edge = 0u, z = 0u;                              // its number of ranges, which edge tile, which range
+    // K steps of a work item: [kt0, kt0 + nk) of the ceil(K / BK) steps -- all of them, or one of `nr` ranges.
     const uint32_t nk_all = (K + BK - 1) / BK;
-    const uint32_t nranges = SPLITK ? (p.ksplit ? p.ksplit : 1u) : ks;
-    const uint32_t per_range = (nk_all + nranges - 1u) / nranges;
+    const uint32_t nranges = SPLITK ? (p.ksplit ? p.ksplit : 1u) : 1u;
     uint32_t nk, k_begin, k_end;                                      // k_end: loads at or past it return zeros
-    auto select_range = [&](uint32_t zr) {
+    auto select_range = [&](uint32_t zr, uint32_t nr) {
+        const uint32_t per_range = (nk_all + nr - 1u) / nr;
         const uint32_t kt0 = zr * per_range;
         nk = kt0 < nk_all ? (nk_all - kt0 < per_range ? nk_all - kt0 : per_range) : 0u;
         k_begin = kt0 * BK;
         k_end = (kt0 + nk) * BK < K ? (kt0 + nk) * BK : K;
     };
-    select_range(z);
+    select_range(0u, 1u);
     // Extent of each operand view: the last row ends at (rows - 1) * ld + cols.
     const uint32_t a_bytes = ((M - 1u) * lda + K) * 2u;
     const uint32_t b_bytes = (NT ? (N - 1u) * ldb + K : (K - 1u) * ldb + N) * 2u;
 
-    // The plain kernels are persistent: the grid is one workgroup per compute unit (or one per
-    // tile if there are fewer), workgroup g computes tiles g, g + grid, g + 2 grid, ... of the
-    // list of all tiles of all batch members.  The edge-splitting kernels compute one tile (or
-    // one K range of one) per workgroup.
+    // The kernels are persistent: the grid is one workgroup per compute unit (or one per work item
+    // if there are fewer), workgroup g computes items g, g + grid, g + 2 grid, ... of the list of all
+    // tiles of all batch members; the edge-splitting kernels of the list of one batch member's whole
+    // tiles followed by its (edge tile, K range) items (grid.z = batch).
     const uint32_t tiles_per = tm * tn;
     // Split-K kernels: the work items are (tile, K range) pairs, ranges of one tile adjacent.
-    const uint32_t total = EDGE ? gridDim.x : tiles_per * p.batch * (SPLITK ? nranges : 1u);
+    const uint32_t total = EDGE ? whole + (mode ? nedge * p.ksplit : 0u) : tiles_per * p.batch * (SPLITK ? nranges : 1u);
     uint32_t pid = blockIdx.x;
     if (pid >= total) return;
 
@@ -204,6 +205,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         uint64_t bz;
         if (EDGE) {
             bz = blockIdx.z;
+            split = id >= whole;
+            ks = split ? p.ksplit : 1u;
+            edge = split ? (id - whole) / ks : 0u;
+            z = split ? (id - whole) % ks : 0u;
+            select_range(z, ks);
             if (!split) {
                 tile_of(xcd_run(id, whole), tm - (mode == 2u), tn - (mode == 1u), &tile_m, &tile_n);
             } else {
@@ -213,7 +219,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         } else if (SPLITK) {
             const uint32_t item = xcd_run(id, total);
             const uint32_t t = item / nranges;                         // tile of the flattened (batch, tile) list
-            select_range(item - t * nranges);
+            select_range(item - t * nranges, nranges);
             bz = t / tiles_per;
             tile_of(t - (uint32_t)bz * tiles_per, tm, tn, &tile_m, &tile_n);
             part_slot = (((uint32_t)bz * tiles_per + tile_m * tn + tile_n) * nranges) + (item - t * nranges);
@@ -437,7 +443,6 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // cache lines.  Lane's chunk = row wm*128 + i*16 + l%16, columns wn*128 + j*16 + 4(l/16)
     // + 0..3.  Chunks wholly outside the matrix are skipped (a wave-uniform test); lanes outside
     // it inside a chunk use an out-of-range offset.
-    const uint32_t nedge = mode == 1u ? tm : tn;
     const uint32_t slot = EDGE ? blockIdx.z * nedge + edge : 0u;
     const __amdgpu_buffer_rsrc_t rws =
         make_rsrc((const char*)p.workspace + 65536, (EDGE && split) ? gridDim.z * nedge * ks * UNIT : 0u);
@@ -446,6 +451,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t rows_ok = M - m0, cols_ok = N - n0;    // valid extent of this tile (may exceed 256)
     auto chunk_live = [&](int c) { return wmu * 128u + (c >> 3) * 16u < rows_ok && wnu * 128u + (c & 7) * 16u < cols_ok; };
     auto lane_live = [&](int c) { return wm * 128u + (c >> 3) * 16u + l16 < rows_ok && wn * 128u + (c & 7) * 16u + lg * 4u < cols_ok; };
+    bool finish = true;                                   // this workgroup stores the tile
     if (EDGE && split) {
         volatile uint32_t& ticket = *(volatile uint32_t*)lds_e;   // the staging region is idle until the epilogue
         uint32_t* counters = (uint32_t*)p.workspace;      // 16384 counters (zero between launches), then the tiles
@@ -459,22 +465,24 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         __syncthreads();
         if (tid == 0) ticket = __hip_atomic_fetch_add(&counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        if (ticket != ks - 1u) return;                    // another workgroup will finish this tile
-        if (tid == 0) counters[slot] = 0u;                // ready for the next launch
+        finish = ticket == ks - 1u;                       // else another workgroup will finish this tile
+        if (finish && tid == 0) counters[slot] = 0u;      // ready for the next launch
     }
+    const bool esplit = split;                            // the item in hand, past the hand-over below
+    const uint32_t eks = ks;
     // The last arriver replaces each chunk of its accumulators by the sum of all ranges, in range
     // order, as the epilogue reaches it; the loads of a chunk are issued eight ranges at a time,
     // ranges past ksplit read zeros.
     auto reduced_chunk = [&](int c) -> floatx4 {
         floatx4 sum = {0.f, 0.f, 0.f, 0.f};
         if (chunk_live(c)) {
-            const uint32_t base = lane_live(c) ? slot * ks * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
-            for (uint32_t z0 = 0; z0 < ks; z0 += 8u) {
+            const uint32_t base = lane_live(c) ? slot * eks * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
+            for (uint32_t z0 = 0; z0 < eks; z0 += 8u) {
                 floatx4 t[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u)
                     t[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
-                        rws, (z0 + u < ks && base != DROP) ? base + (z0 + u) * UNIT : DROP, 0, COHERENT));
+                        rws, (z0 + u < eks && base != DROP) ? base + (z0 + u) * UNIT : DROP, 0, COHERENT));
 #pragma unroll
                 for (int u = 0; u < 8; ++u) { sum[0] += t[u][0]; sum[1] += t[u][1]; sum[2] += t[u][2]; sum[3] += t[u][3]; }
             }
@@ -487,7 +495,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t em0 = m0, en0 = n0, eslot = part_slot;
     uint16_t* const Ce = Cg;
     const uint32_t next = pid + gridDim.x;
-    const bool more = !EDGE && next < total;
+    const bool more = next < total;
     if (more) {
         select_tile(next);
 #pragma unroll
@@ -544,7 +552,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     }
                 }
             }
-    } else {
+    } else if (finish) {                                         // (a K range that was not the last to arrive stores nothing)
         lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
         const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per read
         const uint32_t gcol = en0 + wn * 128u + cc * 8u;
@@ -564,7 +572,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 for (int j = 0; j < 8; ++j) {
                     // lane holds C[row = (2i+ii)*16 + l16][col = j*16 + 4*lg + 0..3]
                     floatx4 f = acc[2 * i + ii][j];
-                    if (EDGE && split) f = reduced_chunk((2 * i + ii) * 8 + j);
+                    if (EDGE && esplit) f = reduced_chunk((2 * i + ii) * 8 + j);
                     u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
                     *(lds_v2)(ew + maps::epi16_write_offset(ii, j, lane)) = v;
                 }

@@ -105,7 +105,9 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert gx == min(tm * tn * batch, resident) and p["split_first"] == 0 and p["workspace_bytes"] == 0
             assert gx == tm * tn * batch or gx % 8 == 0 or cus < 8
         elif p["split_first"] == 0:
-            assert gx == tm * tn and p["workspace_bytes"] == 0
+            # an edge kernel without an edge to split: persistent over the tiles of one batch member, batch in grid.z
+            resident = cus - cus % 8 if cus >= 8 else cus
+            assert gx == min(tm * tn, resident) and p["workspace_bytes"] == 0
         else:
             assert name.endswith("_edge") and batch == 1
             mode, whole = p["split_first"] >> 30, (p["split_first"] & 0x3FFFFFFF) - 1
@@ -113,7 +115,9 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert mode in (1, 2) and 2 <= ks <= 16
             nedge = tm if mode == 1 else tn
             assert whole == (tm * (tn - 1) if mode == 1 else (tm - 1) * tn)
-            assert gx == whole + nedge * ks
+            # persistent: the whole tiles, then the (edge tile, K range) items, shared out over one workgroup per compute unit
+            resident = cus - cus % 8 if cus >= 8 else cus
+            assert gx == min(whole + nedge * ks, resident)
             # the edge that is split is narrow: its partial tiles are cheap to combine
             assert (n - (tn - 1) * 256 if mode == 1 else m - (tm - 1) * 256) <= 32
             # K ranges: ceil(steps / ks) steps each, none empty, each at least 4 steps long
