@@ -117,7 +117,8 @@ EdgeSplit mt256_edge(const Dims& s, uint32_t batch, uint32_t cus) {
     EdgeSplit e = {0, tm * tn, 0, 0};
     if (batch != 1 || cus == 0) return e;
     const uint32_t nk = cdiv(s.k, 64);
-    uint32_t kmax = nk / 4u < 16u ? nk / 4u : 16u;
+    uint32_t kmax = nk >= 4u ? (nk - 1u) / 3u : 0u;        // the most ranges that still have 4 K steps each
+    if (kmax > 16u) kmax = 16u;
     if (kmax < 2u) return e;
     const uint32_t w_n = s.n - (tn - 1u) * 256u, h_m = s.m - (tm - 1u) * 256u;
     const uint32_t rounds = cdiv(tm * tn, cus);
@@ -126,10 +127,18 @@ EdgeSplit mt256_edge(const Dims& s, uint32_t batch, uint32_t cus) {
     else if (tm >= 2u && h_m <= 32u && cdiv((tm - 1u) * tn, cus) < rounds) mode = 2;
     if (!mode) return e;
     const uint32_t nedge = mode == 1 ? tm : tn;
-    uint32_t k = cus / nedge;                              // fill the chip once with edge workgroups
-    if (k > kmax) k = kmax;
-    if (k < 2u) return e;
-    k = cdiv(nk, cdiv(nk, k));                             // no empty range
+    uint32_t cap = cus / nedge;                            // at most one edge item per compute unit
+    if (cap > kmax) cap = kmax;
+    if (cap < 2u) return e;
+    // The kernels run K steps in pairs: among the range counts without an empty range, take the one whose ranges
+    // cost the fewest pairs (the larger count on a tie: more, shorter items fill the tail better).
+    uint32_t k = 0, best = ~0u;
+    for (uint32_t c = 2; c <= cap; ++c) {
+        const uint32_t per = cdiv(nk, c);
+        if (cdiv(nk, per) != c) continue;
+        const uint32_t pairs = (per + 1u) / 2u;
+        if (pairs <= best) { best = pairs; k = c; }
+    }
     if (k < 2u) return e;
     e.mode = mode; e.nedge = nedge; e.ks = k;
     e.whole = mode == 1 ? tm * (tn - 1u) : (tm - 1u) * tn;

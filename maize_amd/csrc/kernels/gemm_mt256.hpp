@@ -452,14 +452,32 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     auto chunk_live = [&](int c) { return wmu * 128u + (c >> 3) * 16u < rows_ok && wnu * 128u + (c & 7) * 16u < cols_ok; };
     auto lane_live = [&](int c) { return wm * 128u + (c >> 3) * 16u + l16 < rows_ok && wn * 128u + (c & 7) * 16u + lg * 4u < cols_ok; };
     bool finish = true;                                   // this workgroup stores the tile
+    // A narrow last tile column (mode 1: at most 32 columns) is published densely instead: 256 rows of cols_ok
+    // floats per (tile, range), so that the last arriver can sum it with one row per thread -- a few rounds of
+    // loads for the whole tile instead of a few per chunk (the chunk-wise sum of such a tile was half of the
+    // edge's cost).  The sums run over the ranges in the same order either way.
+    const bool dense = EDGE && mode == 1u;
+    const uint32_t dense_pitch = cols_ok * 4u;            // bytes per row of a dense partial tile
     if (EDGE && split) {
         volatile uint32_t& ticket = *(volatile uint32_t*)lds_e;   // the staging region is idle until the epilogue
         uint32_t* counters = (uint32_t*)p.workspace;      // 16384 counters (zero between launches), then the tiles
+        if (dense) {
+            if (wnu == 0u) {                              // the other two waves hold no column of the matrix
+#pragma unroll
+                for (int c = 0; c < 64; ++c) {
+                    if ((c & 7) >= 2 || (uint32_t)(c & 7) * 16u >= cols_ok) continue;
+                    const uint32_t row = wm * 128u + (c >> 3) * 16u + l16, col = (c & 7) * 16u + lg * 4u;
+                    const uint32_t off = col < cols_ok ? ((slot * ks + z) * 256u + row) * dense_pitch + col * 4u : DROP;
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[c >> 3][c & 7]), rws, off, 0, COHERENT);
+                }
+            }
+        } else {
 #pragma unroll
         for (int c = 0; c < 64; ++c) {
             if (!chunk_live(c)) continue;
             const uint32_t off = lane_live(c) ? (slot * ks + z) * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[c >> 3][c & 7]), rws, off, 0, COHERENT);
+        }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of the tile has reached memory
         __syncthreads();
@@ -552,6 +570,36 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     }
                 }
             }
+    } else if (EDGE && esplit && dense) {
+        // Last arriver of a narrow edge tile: thread t sums row t of the dense partial tiles over the ranges, in
+        // range order, 8 columns at a time with eight ranges' loads in flight, and stores the row.
+        if (finish) {
+            const uint32_t row = tid;
+            const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce, ((M - 1u) * ldc + N) * 2u);
+#pragma unroll
+            for (int c8 = 0; c8 < 4; ++c8) {                     // 8 columns at a time: two 16-byte loads per range, one 16-byte store
+                if ((uint32_t)c8 * 8u >= cols_ok) continue;      // uniform: cols_ok is a multiple of 8
+                floatx4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+                const uint32_t base = (slot * eks * 256u + row) * dense_pitch + (uint32_t)c8 * 32u;
+                for (uint32_t z0 = 0; z0 < eks; z0 += 8u) {
+                    floatx4 t[8], u[8];
+#pragma unroll
+                    for (int r = 0; r < 8; ++r) {
+                        const uint32_t off = z0 + r < eks ? base + (z0 + r) * 256u * dense_pitch : DROP;
+                        t[r] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off, 0, COHERENT));
+                        u[r] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off == DROP ? DROP : off + 16u, 0, COHERENT));
+                    }
+#pragma unroll
+                    for (int r = 0; r < 8; ++r) {
+                        lo[0] += t[r][0]; lo[1] += t[r][1]; lo[2] += t[r][2]; lo[3] += t[r][3];
+                        hi[0] += u[r][0]; hi[1] += u[r][1]; hi[2] += u[r][2]; hi[3] += u[r][3];
+                    }
+                }
+                const u32x4 v = {cvt_pk_bf16(lo[0], lo[1]), cvt_pk_bf16(lo[2], lo[3]), cvt_pk_bf16(hi[0], hi[1]), cvt_pk_bf16(hi[2], hi[3])};
+                const uint32_t off = row < rows_ok ? ((em0 + row) * ldc + en0 + (uint32_t)c8 * 8u) * 2u : OOB;
+                __builtin_amdgcn_raw_buffer_store_b128(v, rc, off, 0, 2 /* nt */);
+            }
+        }
     } else if (finish) {                                         // (a K range that was not the last to arrive stores nothing)
         lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
         const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per read

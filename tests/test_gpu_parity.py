@@ -346,8 +346,8 @@ def test_dispatcher_choices(ctx):
 
 @pytest.mark.parametrize("shape,layout", [((4096, 4104, 512), mz.LAYOUT_NN), ((4100, 4096, 1024), mz.LAYOUT_NN),
                                           ((4128, 4096, 576), mz.LAYOUT_NT), ((4090, 4120, 1000), mz.LAYOUT_NN),
-                                          ((520, 264, 2048), mz.LAYOUT_NN)],
-                         ids=["edge_col", "edge_row", "edge_row_nt", "edge_col_ktail", "forced_small"])
+                                          ((520, 264, 2048), mz.LAYOUT_NN), ((4000, 4112, 640), mz.LAYOUT_NT)],
+                         ids=["edge_col", "edge_row", "edge_row_nt", "edge_col_ktail", "forced_small", "edge_col_nt"])
 def test_edge_tiles_split_over_k(ctx, oracle, shape, layout):
     """A ragged last tile column (or row) that pushes the tile count past the CU count: the dispatcher
     gives each edge tile several K ranges, combined through the workspace in range order.  Checked in
