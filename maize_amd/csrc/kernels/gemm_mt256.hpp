@@ -438,46 +438,30 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr int COHERENT = 17;                          // buffer cache policy sc0 | sc1: visible across the XCDs' L2s
     constexpr uint32_t UNIT = BM * BN * 4u;               // one fp32 partial tile
     constexpr uint32_t DROP = 0xFFFFFFF0u;                // out-of-range offset: store dropped, load returns zeros
-    // A partial tile is stored in register order, not row-major: chunk c = (i, j) of wave w is
-    // 64 lanes x 16 bytes = 1 KiB contiguous, so every store and load instruction moves whole
-    // cache lines.  Lane's chunk = row wm*128 + i*16 + l%16, columns wn*128 + j*16 + 4(l/16)
-    // + 0..3.  Chunks wholly outside the matrix are skipped (a wave-uniform test); lanes outside
-    // it inside a chunk use an out-of-range offset.
     const uint32_t slot = EDGE ? blockIdx.z * nedge + edge : 0u;
     const __amdgpu_buffer_rsrc_t rws =
         make_rsrc((const char*)p.workspace + 65536, (EDGE && split) ? gridDim.z * nedge * ks * UNIT : 0u);
     const uint32_t wmu = wave_u >> 1, wnu = wave_u & 1u;
-    const uint32_t lane_off = wave_u * 65536u + lane * 16u;
     const uint32_t rows_ok = M - m0, cols_ok = N - n0;    // valid extent of this tile (may exceed 256)
     auto chunk_live = [&](int c) { return wmu * 128u + (c >> 3) * 16u < rows_ok && wnu * 128u + (c & 7) * 16u < cols_ok; };
     auto lane_live = [&](int c) { return wm * 128u + (c >> 3) * 16u + l16 < rows_ok && wn * 128u + (c & 7) * 16u + lg * 4u < cols_ok; };
     bool finish = true;                                   // this workgroup stores the tile
-    // A narrow last tile column (mode 1: at most 32 columns) is published densely instead: 256 rows of cols_ok
-    // floats per (tile, range), so that the last arriver can sum it with one row per thread -- a few rounds of
-    // loads for the whole tile instead of a few per chunk (the chunk-wise sum of such a tile was half of the
-    // edge's cost).  The sums run over the ranges in the same order either way.
-    const bool dense = EDGE && mode == 1u;
-    const uint32_t dense_pitch = cols_ok * 4u;            // bytes per row of a dense partial tile
+    // Split edge tiles are narrow (at most 32 columns in mode 1) or short (at most 32 rows in mode 2), and their
+    // partial tiles are published densely: row-major, 256 rows of cols_ok floats, or 32 rows of 256 floats, per
+    // (tile, range).  The last arriver then sums them with 8 columns of one row per thread -- a few rounds of loads
+    // for the whole tile (a chunk-by-chunk sum in register order took several rounds per chunk, one memory latency
+    // each, and was half of the edge's cost).  The sums run over the ranges in ascending order.
+    const uint32_t dense_rows = mode == 1u ? 256u : 32u;                  // rows per dense partial tile
+    const uint32_t dense_pitch = (mode == 1u ? cols_ok : 256u) * 4u;      // bytes per row
     if (EDGE && split) {
         volatile uint32_t& ticket = *(volatile uint32_t*)lds_e;   // the staging region is idle until the epilogue
         uint32_t* counters = (uint32_t*)p.workspace;      // 16384 counters (zero between launches), then the tiles
-        if (dense) {
-            if (wnu == 0u) {                              // the other two waves hold no column of the matrix
-#pragma unroll
-                for (int c = 0; c < 64; ++c) {
-                    if ((c & 7) >= 2 || (uint32_t)(c & 7) * 16u >= cols_ok) continue;
-                    const uint32_t row = wm * 128u + (c >> 3) * 16u + l16, col = (c & 7) * 16u + lg * 4u;
-                    const uint32_t off = col < cols_ok ? ((slot * ks + z) * 256u + row) * dense_pitch + col * 4u : DROP;
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[c >> 3][c & 7]), rws, off, 0, COHERENT);
-                }
-            }
-        } else {
 #pragma unroll
         for (int c = 0; c < 64; ++c) {
             if (!chunk_live(c)) continue;
-            const uint32_t off = lane_live(c) ? (slot * ks + z) * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
+            const uint32_t row = wm * 128u + (c >> 3) * 16u + l16, col = wn * 128u + (c & 7) * 16u + lg * 4u;
+            const uint32_t off = lane_live(c) ? ((slot * ks + z) * dense_rows + row) * dense_pitch + col * 4u : DROP;
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[c >> 3][c & 7]), rws, off, 0, COHERENT);
-        }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of the tile has reached memory
         __syncthreads();
@@ -488,26 +472,6 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }
     const bool esplit = split;                            // the item in hand, past the hand-over below
     const uint32_t eks = ks;
-    // The last arriver replaces each chunk of its accumulators by the sum of all ranges, in range
-    // order, as the epilogue reaches it; the loads of a chunk are issued eight ranges at a time,
-    // ranges past ksplit read zeros.
-    auto reduced_chunk = [&](int c) -> floatx4 {
-        floatx4 sum = {0.f, 0.f, 0.f, 0.f};
-        if (chunk_live(c)) {
-            const uint32_t base = lane_live(c) ? slot * eks * UNIT + lane_off + (uint32_t)c * 1024u : DROP;
-            for (uint32_t z0 = 0; z0 < eks; z0 += 8u) {
-                floatx4 t[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u)
-                    t[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
-                        rws, (z0 + u < eks && base != DROP) ? base + (z0 + u) * UNIT : DROP, 0, COHERENT));
-#pragma unroll
-                for (int u = 0; u < 8; ++u) { sum[0] += t[u][0]; sum[1] += t[u][1]; sum[2] += t[u][2]; sum[3] += t[u][3]; }
-            }
-        }
-        return sum;
-    };
-
     // ---- hand-over: request the next C tile's first K tile before this one is stored -------
     __syncthreads();                                           // all waves are done with the operand stages
     const uint32_t em0 = m0, en0 = n0, eslot = part_slot;
@@ -570,22 +534,24 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     }
                 }
             }
-    } else if (EDGE && esplit && dense) {
-        // Last arriver of a narrow edge tile: thread t sums row t of the dense partial tiles over the ranges, in
-        // range order, 8 columns at a time with eight ranges' loads in flight, and stores the row.
+    } else if (EDGE && esplit) {
+        // Last arriver of a split edge tile: a thread sums 8 columns of one row of the dense partial tiles over the
+        // ranges, in range order, eight ranges' loads in flight, and stores them; up to four such units per thread.
         if (finish) {
-            const uint32_t row = tid;
             const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce, ((M - 1u) * ldc + N) * 2u);
 #pragma unroll
-            for (int c8 = 0; c8 < 4; ++c8) {                     // 8 columns at a time: two 16-byte loads per range, one 16-byte store
-                if ((uint32_t)c8 * 8u >= cols_ok) continue;      // uniform: cols_ok is a multiple of 8
+            for (int q = 0; q < 4; ++q) {
+                // narrow tile: unit q of thread t = (row t, columns 8 q ..); short tile: (row t / 32 + 8 q, columns 8 (t % 32) ..)
+                if ((uint32_t)q * 8u >= (mode == 1u ? cols_ok : rows_ok)) continue;      // workgroup-uniform
+                const uint32_t row = mode == 1u ? tid : (tid >> 5) + 8u * q, c8 = mode == 1u ? (uint32_t)q : (tid & 31u);
+                const bool live = row < rows_ok && c8 * 8u < cols_ok;                   // N % 8 == 0: 8 columns are all in or all out
                 floatx4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
-                const uint32_t base = (slot * eks * 256u + row) * dense_pitch + (uint32_t)c8 * 32u;
+                const uint32_t base = (slot * eks * dense_rows + row) * dense_pitch + c8 * 32u;
                 for (uint32_t z0 = 0; z0 < eks; z0 += 8u) {
                     floatx4 t[8], u[8];
 #pragma unroll
                     for (int r = 0; r < 8; ++r) {
-                        const uint32_t off = z0 + r < eks ? base + (z0 + r) * 256u * dense_pitch : DROP;
+                        const uint32_t off = (live && z0 + r < eks) ? base + (z0 + r) * dense_rows * dense_pitch : DROP;
                         t[r] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off, 0, COHERENT));
                         u[r] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off == DROP ? DROP : off + 16u, 0, COHERENT));
                     }
@@ -596,7 +562,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     }
                 }
                 const u32x4 v = {cvt_pk_bf16(lo[0], lo[1]), cvt_pk_bf16(lo[2], lo[3]), cvt_pk_bf16(hi[0], hi[1]), cvt_pk_bf16(hi[2], hi[3])};
-                const uint32_t off = row < rows_ok ? ((em0 + row) * ldc + en0 + (uint32_t)c8 * 8u) * 2u : OOB;
+                const uint32_t off = live ? ((em0 + row) * ldc + en0 + c8 * 8u) * 2u : OOB;
                 __builtin_amdgcn_raw_buffer_store_b128(v, rc, off, 0, 2 /* nt */);
             }
         }
@@ -620,7 +586,6 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 for (int j = 0; j < 8; ++j) {
                     // lane holds C[row = (2i+ii)*16 + l16][col = j*16 + 4*lg + 0..3]
                     floatx4 f = acc[2 * i + ii][j];
-                    if (EDGE && esplit) f = reduced_chunk((2 * i + ii) * 8 + j);
                     u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
                     *(lds_v2)(ew + maps::epi16_write_offset(ii, j, lane)) = v;
                 }
