@@ -46,8 +46,8 @@
 //     kernels cut each of those tiles into `ksplit` K ranges: work items that follow the whole tiles in the
 //     persistent workgroups' list, so they fill the tail instead of forming a round of their own.  A workgroup
 //     with such an item writes the part of its fp32 partial tile that lies inside the matrix to a library-owned
-//     workspace (device-coherent stores), takes a ticket with a device-scope atomic, and the last
-//     arriver re-reads all partials in range order (deterministic), then runs the normal epilogue.
+//     workspace (device-coherent stores, row-major), takes a ticket with a device-scope atomic, and the last
+//     arriver adds up all partials in range order (deterministic), 8 columns of a row per thread, and stores C.
 //
 // The _gen kernels are the plain (persistent) kernels with the general epilogue: C = alpha * A.B +
 // beta * C, C in bf16 or fp32.  maize_gemm_f16_mt256_* are the same kernels on IEEE half operands
