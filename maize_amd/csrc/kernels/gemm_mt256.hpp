@@ -58,7 +58,8 @@
 // maize_gemm_splitk_reduce (splitk_reduce.hpp) adds the ranges in order and applies the epilogue.
 //
 // Requirements (checked by the dispatcher): K % 8 == 0, N % 8 == 0, 16-byte
-// aligned operands, each matrix (per batch member) below 2 GiB.  The plain
+// aligned operands, K, N and the leading dimensions below 2^21 elements, a K x N B
+// (per batch member) below 2 GiB; A, C and an N x K B may be of any size.  The plain
 // kernels need K % 64 == 0 (the K advance is then a scalar offset and no lane
 // ever needs a K mask); the _ktail kernels take any K % 8 == 0.
 #pragma once
@@ -168,9 +169,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         k_end = (kt0 + nk) * BK < K ? (kt0 + nk) * BK : K;
     };
     select_range(0u, 1u);
-    // Extent of each operand view: the last row ends at (rows - 1) * ld + cols.
-    const uint32_t a_bytes = ((M - 1u) * lda + K) * 2u;
-    const uint32_t b_bytes = (NT ? (N - 1u) * ldb + K : (K - 1u) * ldb + N) * 2u;
+    // Buffer descriptors start at the first row of the tile in hand and end with the operand's view (the last row
+    // ends at (rows - 1) * ld + cols), so the 32-bit offsets only have to span a tile's 256 rows and A, C and an
+    // N x K B may be of any size.  A length past 2 GiB is cut there: the out-of-range marker is bit 31 of an offset,
+    // and rows that far from the end of the view are all inside the matrix.  (A K x N B advances through K inside
+    // its descriptor and stays below 2 GiB; the dispatcher checks.)
+    auto span = [](uint64_t bytes) { return (uint32_t)(bytes < 0x7FFFFFFFull ? bytes : 0x7FFFFFFFull); };
+    uint32_t a_bytes, b_bytes;
 
     // The kernels are persistent: the grid is one workgroup per compute unit (or one per work item
     // if there are fewer), workgroup g computes items g, g + grid, g + 2 grid, ... of the list of all
@@ -230,17 +235,24 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         }
         m0 = tile_m * BM;
         n0 = tile_n * BN;
-        Ag = p.a + bz * p.stride_a;
-        Bg = p.b + bz * p.stride_b;
+        Ag = p.a + bz * p.stride_a + (uint64_t)m0 * lda;                       // the tile's first row of A
+        a_bytes = span(((uint64_t)(M - 1u - m0) * lda + K) * 2u);
+        if (NT) {
+            Bg = p.b + bz * p.stride_b + (uint64_t)n0 * ldb;                   // ... and of an N x K B
+            b_bytes = span(((uint64_t)(N - 1u - n0) * ldb + K) * 2u);
+        } else {
+            Bg = p.b + bz * p.stride_b;
+            b_bytes = span(((uint64_t)(K - 1u) * ldb + N) * 2u);
+        }
         Cg = p.c + bz * p.stride_c * ((GEN && (p.epi & EPI_F32)) ? 2u : 1u);   // strides count elements of C
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t row = maps::kc_piece_row(wave * 8u + i, lane);
             const uint32_t c = maps::kc_piece_chunk(wave * 8u + i, lane);
-            a_vo[i] = ((m0 + row) * lda + c * 8u) * 2u;
+            a_vo[i] = (row * lda + c * 8u) * 2u;
             if (i < 2) a_k[i] = c * 8u;
             if (NT) {
-                b_vo[i] = ((n0 + row) * ldb + c * 8u) * 2u;
+                b_vo[i] = (row * ldb + c * 8u) * 2u;
             } else {
                 const uint32_t brow = maps::sk_piece_row(wave * 8u + i, lane);
                 const uint32_t bc = maps::sk_piece_chunk(wave * 8u + i, lane);
@@ -538,7 +550,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // Last arriver of a split edge tile: a thread sums 8 columns of one row of the dense partial tiles over the
         // ranges, in range order, eight ranges' loads in flight, and stores them; up to four such units per thread.
         if (finish) {
-            const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce, ((M - 1u) * ldc + N) * 2u);
+            const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce + (uint64_t)em0 * ldc, span(((uint64_t)(M - 1u - em0) * ldc + N) * 2u));
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 // narrow tile: unit q of thread t = (row t, columns 8 q ..); short tile: (row t / 32 + 8 q, columns 8 (t % 32) ..)
@@ -562,7 +574,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     }
                 }
                 const u32x4 v = {cvt_pk_bf16(lo[0], lo[1]), cvt_pk_bf16(lo[2], lo[3]), cvt_pk_bf16(hi[0], hi[1]), cvt_pk_bf16(hi[2], hi[3])};
-                const uint32_t off = live ? ((em0 + row) * ldc + en0 + c8 * 8u) * 2u : OOB;
+                const uint32_t off = live ? (row * ldc + en0 + c8 * 8u) * 2u : OOB;
                 __builtin_amdgcn_raw_buffer_store_b128(v, rc, off, 0, 2 /* nt */);
             }
         }
@@ -575,8 +587,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // chunk is all in or all out) get an out-of-range offset; no 64-bit address arithmetic and
         // no divergent branch per row.  Non-temporal: C is written once and not read again by this
         // kernel, it should not displace the operand panels in L2.
-        const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce, ((M - 1u) * ldc + N) * 2u);
-        const uint32_t c_vo = (((em0 + wm * 128u + cr) * ldc + gcol) * 2u) | (gcol < N ? 0u : OOB);
+        const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce + (uint64_t)em0 * ldc, span(((uint64_t)(M - 1u - em0) * ldc + N) * 2u));
+        const uint32_t c_vo = (((wm * 128u + cr) * ldc + gcol) * 2u) | (gcol < N ? 0u : OOB);
         const uint32_t row_bytes = __builtin_amdgcn_readfirstlane(ldc * 2u);
     #pragma unroll
         for (int i = 0; i < 4; ++i) {

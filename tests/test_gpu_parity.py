@@ -361,3 +361,50 @@ def test_edge_tiles_split_over_k(ctx, oracle, shape, layout):
         got = run_gemm(ctx, a, bs, m, n, k, layout=layout, kernel=kern)
         check_against_oracle(oracle, got, a, bs, m, n, k, layout=layout, label=f"edge split {shape} {kern}")
         assert np.array_equal(run_gemm(ctx, a, bs, m, n, k, layout=layout, kernel=kern), got)
+
+
+# ---- matrices past 2 GiB ---------------------------------------------------------------------------------
+
+def _sampled_entries_check(oracle, got_rows, a_rows_bits, b_rows_bits, k, label):
+    """C entries = rows of A against rows of an N x K B, in float64 on the host (numpy), to the plain parity bar."""
+    A = mz.bf16.to_f64(a_rows_bits).reshape(-1, k)
+    B = mz.bf16.to_f64(b_rows_bits).reshape(-1, k)
+    val, scale = A @ B.T, np.abs(A) @ np.abs(B).T
+    s = oracle.compare(got_rows, oracle.bf16_bits_from_f64(val), val, scale, k)
+    assert s["n_fail"] == 0, f"{label}: {s}"
+
+
+@pytest.mark.parametrize("which", ["c", "a", "b_nt"])
+def test_operands_past_two_gib(ctx, oracle, which):
+    """The buffer descriptors of the macro-tile kernels are re-based on every tile's first row, so A, C and an N x K B
+    may exceed the 2 GiB a 32-bit offset with an out-of-range bit can span.  One case per operand, checked on sampled
+    rows that include the far end of the big matrix."""
+    if which == "c":        # C = 32808 x 36864 bf16 = 2.42 GB
+        m, n, k, layout = 32808, 36864, 128, mz.LAYOUT_NN
+    elif which == "a":      # A = 40000 x 28672 = 2.29 GB
+        m, n, k, layout = 40000, 256, 28672, mz.LAYOUT_NT
+    else:                   # B stored N x K = 40000 x 28672
+        m, n, k, layout = 256, 40000, 28672, mz.LAYOUT_NT
+    _say(f"past 2 GiB: {which} M={m} N={n} K={k}")
+    a = mz.gen.uniform_bf16(m * k, 71)
+    b = mz.gen.uniform_bf16(k * n, 72)              # NT cases: read as N x K
+    da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(m * n * 2)
+    try:
+        B = mz.Matrix(db, k, n) if layout == mz.LAYOUT_NN else mz.Matrix(db, n, k)
+        desc = mz.gemm_desc(mz.Matrix(da, m, k), B, mz.Matrix(dc, m, n), layout=layout)
+        took = ctx.gemm_select(desc)
+        assert "_mt256_" in took and "packed" not in took, took          # not the per-wave fallback
+        ctx.gemm_bf16(desc)
+        ctx.sync()
+        rows = sample_rows(m, count=24, seed=3)
+        if which == "b_nt":
+            cols = sample_rows(n, count=40, seed=4)
+            got = np.stack([dc.download(np.uint16, count=n, offset_bytes=int(r) * n * 2)[cols] for r in rows[:32]])
+            _sampled_entries_check(oracle, got, a.reshape(m, k)[rows[:32]], b.reshape(n, k)[cols], k, f"past 2 GiB {which} {took}")
+        else:
+            got = np.stack([dc.download(np.uint16, count=n, offset_bytes=int(r) * n * 2) for r in rows])
+            ref, f64, ab = oracle.ref_gemm_rows(a, b, m, n, k, rows, layout=layout)
+            s = oracle.compare(got, ref, f64, ab, k)
+            assert s["n_fail"] == 0, f"past 2 GiB {which} {took}: {s}"
+    finally:
+        da.free(); db.free(); dc.free()
