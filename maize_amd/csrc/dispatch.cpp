@@ -47,7 +47,7 @@ bool wave32_plan(const maize_gemm_ex_desc_t& d, uint32_t, LaunchDims* ld) {
 // ---- maize_gemm_bf16_mt256_{nn,nt}: 256 x 256 x 64 macro-tile pipeline -------
 // 128-bit loads and stores: K % 8 == 0 (A rows, and B rows when NT), N % 8 == 0
 // (C rows, and B rows when NN), 16-byte aligned bases and batch strides.
-// 32-bit buffer offsets span one tile's rows: K, N, leading dimensions below 2^21; a K x N B below 2 GiB.
+// 32-bit buffer offsets span one tile's rows: K, N and the leading dimensions below 2^21 elements.
 bool aligned16(const maize_gemm_ex_desc_t& d) {
     if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr | (uintptr_t)d.gemm.c.ptr) & 15u) return false;
     if (d.gemm.batch > 1 && ((d.gemm.stride_a | d.gemm.stride_b | d.gemm.stride_c) & 7u)) return false;
@@ -58,11 +58,10 @@ bool aligned16(const maize_gemm_ex_desc_t& d) {
 bool mt256_common(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
     if ((s.k & 7u) || (s.n & 7u) || !aligned16(d)) return false;
-    // 32-bit byte offsets span a tile's 256 rows (descriptors are re-based per tile): K, N and the leading
-    // dimensions stay below 2^21 elements.  A row-major K x N B is walked inside one descriptor: below 2 GiB.
+    // 32-bit byte offsets span a tile's 256 rows (descriptors are re-based per tile, for a K x N B per K tile):
+    // K, N and the leading dimensions stay below 2^21 elements; the matrices may be of any size.
     const Lds l = lds_of(d);
     if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21) || l.c >= (1u << 21)) return false;
-    if (d.gemm.layout == MAIZE_LAYOUT_NN && l.ext_b * 2 >= (1ull << 31)) return false;
     return true;
 }
 // The plain kernels advance K with a scalar offset and never mask a lane in K: K % 64 == 0.

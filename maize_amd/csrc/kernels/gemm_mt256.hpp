@@ -58,8 +58,8 @@
 // maize_gemm_splitk_reduce (splitk_reduce.hpp) adds the ranges in order and applies the epilogue.
 //
 // Requirements (checked by the dispatcher): K % 8 == 0, N % 8 == 0, 16-byte
-// aligned operands, K, N and the leading dimensions below 2^21 elements, a K x N B
-// (per batch member) below 2 GiB; A, C and an N x K B may be of any size.  The plain
+// aligned operands, K, N and the leading dimensions below 2^21 elements; the
+// matrices themselves may be of any size.  The plain
 // kernels need K % 64 == 0 (the K advance is then a scalar offset and no lane
 // ever needs a K mask); the _ktail kernels take any K % 8 == 0.
 #pragma once
@@ -172,8 +172,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // Buffer descriptors start at the first row of the tile in hand and end with the operand's view (the last row
     // ends at (rows - 1) * ld + cols), so the 32-bit offsets only have to span a tile's 256 rows and A, C and an
     // N x K B may be of any size.  A length past 2 GiB is cut there: the out-of-range marker is bit 31 of an offset,
-    // and rows that far from the end of the view are all inside the matrix.  (A K x N B advances through K inside
-    // its descriptor and stays below 2 GiB; the dispatcher checks.)
+    // and rows that far from the end of the view are all inside the matrix.  A K x N B is re-based on the K tile's
+    // first row instead (dma).
     auto span = [](uint64_t bytes) { return (uint32_t)(bytes < 0x7FFFFFFFull ? bytes : 0x7FFFFFFFull); };
     uint32_t a_bytes, b_bytes;
 
@@ -241,8 +241,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             Bg = p.b + bz * p.stride_b + (uint64_t)n0 * ldb;                   // ... and of an N x K B
             b_bytes = span(((uint64_t)(N - 1u - n0) * ldb + K) * 2u);
         } else {
-            Bg = p.b + bz * p.stride_b;
-            b_bytes = span(((uint64_t)(K - 1u) * ldb + N) * 2u);
+            Bg = p.b + bz * p.stride_b;                                        // (a K x N B is re-based per K tile, see dma)
+            b_bytes = 0u;
         }
         Cg = p.c + bz * p.stride_c * ((GEN && (p.epi & EPI_F32)) ? 2u : 1u);   // strides count elements of C
 #pragma unroll
@@ -261,7 +261,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         }
     };
     select_tile(pid);
-    const uint32_t b_kscale = NT ? 2u : ldb * 2u;  // bytes per unit of k in B
+    const uint64_t b_view = ((uint64_t)(K - 1u) * ldb + N) * 2u;               // bytes of a K x N B
     // Issues piece pc (0..7 = A, 8..15 = B) of the tile that starts at k into stages (sa, sb).
     auto dma = [&](int pc, lds_ptr sa, lds_ptr sb, uint32_t k) {
         typedef __attribute__((address_space(3))) void* lvp;
@@ -269,14 +269,22 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const int i = is_a ? pc : pc - 8;
         lds_ptr dst = (is_a ? sa : sb) + (wave_u * 8u + i) * 1024u;
         // Tiles that start at or past K read through a zero-length descriptor: all zeros.
+        if (!is_a && !NT) {
+            // K x N B: the descriptor starts at row k of B (scalar 64-bit arithmetic, once per K tile) and ends with
+            // the view; rows at or past K are past its end.
+            const uint64_t skip = (uint64_t)k * ldb * 2u;
+            const uint32_t bytes = k < k_end ? span(b_view - skip) : 0u;       // k < k_end <= K: skip < b_view
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc((const char*)Bg + skip, bytes);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, b_vo[i], 0, 0, MAIZE_MT256_DMA_AUX);
+            return;
+        }
         const uint32_t bytes = k < k_end ? (is_a ? a_bytes : b_bytes) : 0u;
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(is_a ? (const void*)Ag : (const void*)Bg, bytes);
         if (!KTAIL) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i],
-                                                     k * (is_a ? 2u : b_kscale), 0, MAIZE_MT256_DMA_AUX);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i], k * 2u, 0, MAIZE_MT256_DMA_AUX);
         } else {
-            uint32_t off = (is_a ? a_vo[i] : b_vo[i]) + k * (is_a ? 2u : b_kscale);
-            if (is_a || NT) off |= (a_k[i & 1] + k) < K ? 0u : OOB;
+            uint32_t off = (is_a ? a_vo[i] : b_vo[i]) + k * 2u;
+            off |= (a_k[i & 1] + k) < K ? 0u : OOB;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, off, 0, 0, MAIZE_MT256_DMA_AUX);
         }
     };

@@ -365,26 +365,29 @@ def test_edge_tiles_split_over_k(ctx, oracle, shape, layout):
 
 # ---- matrices past 2 GiB ---------------------------------------------------------------------------------
 
-def _sampled_entries_check(oracle, got_rows, a_rows_bits, b_rows_bits, k, label):
-    """C entries = rows of A against rows of an N x K B, in float64 on the host (numpy), to the plain parity bar."""
+def _sampled_entries_check(oracle, got_rows, a_rows_bits, bt_bits, k, label):
+    """C entries = rows of A against columns of B (given transposed: one row of K values per column), in float64 on the
+    host (numpy), to the plain parity bar."""
     A = mz.bf16.to_f64(a_rows_bits).reshape(-1, k)
-    B = mz.bf16.to_f64(b_rows_bits).reshape(-1, k)
+    B = mz.bf16.to_f64(bt_bits).reshape(-1, k)
     val, scale = A @ B.T, np.abs(A) @ np.abs(B).T
     s = oracle.compare(got_rows, oracle.bf16_bits_from_f64(val), val, scale, k)
     assert s["n_fail"] == 0, f"{label}: {s}"
 
 
-@pytest.mark.parametrize("which", ["c", "a", "b_nt"])
+@pytest.mark.parametrize("which", ["c", "a", "b_nt", "b_nn"])
 def test_operands_past_two_gib(ctx, oracle, which):
-    """The buffer descriptors of the macro-tile kernels are re-based on every tile's first row, so A, C and an N x K B
-    may exceed the 2 GiB a 32-bit offset with an out-of-range bit can span.  One case per operand, checked on sampled
-    rows that include the far end of the big matrix."""
+    """The buffer descriptors of the macro-tile kernels are re-based on every tile's first row (a K x N B: on every K
+    tile's), so every operand may exceed the 2 GiB a 32-bit offset with an out-of-range bit can span.  One case per
+    operand and layout of B, checked on sampled rows (columns) that include the far end of the big matrix."""
     if which == "c":        # C = 32808 x 36864 bf16 = 2.42 GB
         m, n, k, layout = 32808, 36864, 128, mz.LAYOUT_NN
     elif which == "a":      # A = 40000 x 28672 = 2.29 GB
         m, n, k, layout = 40000, 256, 28672, mz.LAYOUT_NT
-    else:                   # B stored N x K = 40000 x 28672
+    elif which == "b_nt":   # B stored N x K = 40000 x 28672
         m, n, k, layout = 256, 40000, 28672, mz.LAYOUT_NT
+    else:                   # B stored K x N = 40960 x 28672: re-based on every K tile
+        m, n, k, layout = 256, 28672, 40960, mz.LAYOUT_NN
     _say(f"past 2 GiB: {which} M={m} N={n} K={k}")
     a = mz.gen.uniform_bf16(m * k, 71)
     b = mz.gen.uniform_bf16(k * n, 72)              # NT cases: read as N x K
@@ -397,10 +400,11 @@ def test_operands_past_two_gib(ctx, oracle, which):
         ctx.gemm_bf16(desc)
         ctx.sync()
         rows = sample_rows(m, count=24, seed=3)
-        if which == "b_nt":
+        if which in ("b_nt", "b_nn"):
             cols = sample_rows(n, count=40, seed=4)
             got = np.stack([dc.download(np.uint16, count=n, offset_bytes=int(r) * n * 2)[cols] for r in rows[:32]])
-            _sampled_entries_check(oracle, got, a.reshape(m, k)[rows[:32]], b.reshape(n, k)[cols], k, f"past 2 GiB {which} {took}")
+            bt = b.reshape(n, k)[cols] if which == "b_nt" else np.ascontiguousarray(b.reshape(k, n)[:, cols].T)
+            _sampled_entries_check(oracle, got, a.reshape(m, k)[rows[:32]], bt, k, f"past 2 GiB {which} {took}")
         else:
             got = np.stack([dc.download(np.uint16, count=n, offset_bytes=int(r) * n * 2) for r in rows])
             ref, f64, ab = oracle.ref_gemm_rows(a, b, m, n, k, rows, layout=layout)
