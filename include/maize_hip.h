@@ -221,6 +221,12 @@ int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* des
 int32_t maize_hip_gemm_ex_validate(const maize_gemm_ex_desc_t* desc);
 int32_t maize_hip_gemm_ex_plan(const maize_gemm_ex_desc_t* desc, const char* kernel, uint32_t compute_units,
                                maize_gemm_plan_t* out);
+/* How the launcher (kernel == NULL) composes a product whose tile count is a little over a whole number of rounds of
+ * one workgroup per compute unit: *rows leading rows of A and C are computed first (by the kernel gemm_ex_plan names
+ * for that sub-product), the remaining rows behind them on the same stream as a product of their own (few tiles: the
+ * split-K kernels).  *rows == 0: one product.  The reference has no counterpart: its panel iterators assign whole
+ * panels to blocks and never balance a tail (crates/maize_tile/src/gmem/row_panel.rs:95-109). */
+int32_t maize_hip_gemm_ex_tail_rows(const maize_gemm_ex_desc_t* desc, uint32_t compute_units, uint32_t* rows);
 /* Validation only (no device access): the checks gemm_bf16 performs first. */
 int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* desc);
 /* Enumerates the GEMM kernels of the embedded code object. */

@@ -222,6 +222,16 @@ def gemm_plan(desc, kernel=None, compute_units=256):
             "workspace_bytes": out.workspace_bytes}
 
 
+def gemm_tail_rows(desc, compute_units=256):
+    """Leading rows of A and C the launcher computes as a product of their own when the tile count is a little over
+    a whole number of rounds (the rest follows as a second, split-K product); 0 = one product.  No device needed."""
+    x = desc if isinstance(desc, _ffi.GemmExDescT) else gemm_ex_desc(desc.a, desc.b, desc.c, layout=desc.layout, batch=desc.batch,
+                                                                      stride_a=desc.stride_a, stride_b=desc.stride_b, stride_c=desc.stride_c)
+    rows = C.c_uint32()
+    check(_ffi.lib().maize_hip_gemm_ex_tail_rows(C.byref(x), compute_units, C.byref(rows)))
+    return rows.value
+
+
 def kernel_names():
     L = _ffi.lib()
     return [L.maize_hip_kernel_name(i).decode() for i in range(L.maize_hip_kernel_count())]

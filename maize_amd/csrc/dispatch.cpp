@@ -674,4 +674,31 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
 }
 
+uint32_t tail_split_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
+    if (!(bf16_in(d) || half_in(d)) || d.gemm.batch != 1 || compute_units < 8u) return 0;
+    const Dims s = dims_of(d);
+    // only where the whole product would run on a persistent macro-tile kernel, one tile per work item
+    const char* name = kKernels[select_kernel(d, compute_units)].name;
+    if (!std::strstr(name, "_mt256_") || std::strstr(name, "_splitk") || std::strstr(name, "_packed") || std::strstr(name, "_edge")) return 0;
+    const uint32_t tm = cdiv(s.m, 256), tn = cdiv(s.n, 256);
+    const uint64_t tiles = (uint64_t)tm * tn;
+    const uint32_t resident = compute_units - compute_units % 8u;
+    if (tiles <= resident || tiles % resident == 0) return 0;
+    const uint64_t full_rounds = tiles / resident;
+    const uint32_t tm_top = (uint32_t)(full_rounds * resident / tn);     // tile rows that fit into the full rounds
+    if (tm_top == 0 || tm_top >= tm) return 0;
+    // The rows below: worth a launch of their own only if, split over K, they cost clearly less than the
+    // round they replace (the cost model of splitk_ranges, microseconds, plus ~3 for the extra launch).
+    Dims bottom = s;
+    bottom.m = s.m - tm_top * 256u;
+    const uint32_t nk = cdiv(s.k, 64);
+    const uint32_t ks = splitk_ranges(bottom, 1, compute_units);
+    if (ks < 2u) return 0;
+    const double t_round = 8.0 + 1.0 * nk;
+    const double t_bottom = 3.0 + 8.0 + 1.2 * cdiv(nk, ks) + 6.0 + 2e-6 * (double)bottom.m * s.n * ks;
+    if (t_bottom > 0.75 * t_round) return 0;
+    // the rows below start on a 16-byte boundary like the matrix itself (leading dimensions are multiples of 8)
+    return tm_top * 256u;
+}
+
 }  // namespace maize

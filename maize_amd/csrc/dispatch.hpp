@@ -54,6 +54,13 @@ int kernel_index(const char* name);  // -1 if unknown
 // Index of the kernel the dispatcher picks for a validated descriptor.
 uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units);
 
+// Tail splitting by rows.  When the tile count is a little over a whole number of rounds of the persistent
+// macro-tile kernels (one workgroup per compute unit), the last, nearly empty round costs as much as a full one.
+// Returns the number of leading rows of A and C (a multiple of 256, 0 = do not split) to compute with the kernel
+// the dispatcher picks for them; the rows below are then a product with few tiles, which the dispatcher runs on
+// the split-K kernels.  Host logic only; the launcher composes the two products on the caller's stream.
+uint32_t tail_split_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units);
+
 struct Dims {
     uint32_t m, n, k;
     bool nt;

@@ -325,6 +325,14 @@ int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* d) {
 
 uint32_t maize_hip_kernel_count(void) { return maize::kernel_count(); }
 
+int32_t maize_hip_gemm_ex_tail_rows(const maize_gemm_ex_desc_t* desc, uint32_t compute_units, uint32_t* rows) {
+    if (!rows) return fail(MAIZE_ERR_NULL, "gemm_tail_rows: NULL argument");
+    int32_t rc = maize_hip_gemm_ex_validate(desc);
+    if (rc != MAIZE_OK) return rc;
+    *rows = maize::tail_split_rows(*desc, compute_units);
+    return MAIZE_OK;
+}
+
 const char* maize_hip_kernel_name(uint32_t index) {
     return index < maize::kernel_count() ? maize::kernel_at(index).name : nullptr;
 }
@@ -483,7 +491,25 @@ int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* des
     if (!ctx) return fail(MAIZE_ERR_NULL, "gemm: ctx is NULL");
     int32_t rc = maize_hip_gemm_ex_validate(desc);
     if (rc != MAIZE_OK) return rc;
-    if (!kernel) return gemm_launch(ctx, desc, maize::select_kernel(*desc, (uint32_t)ctx->prop.multiProcessorCount), stream);
+    if (!kernel) {
+        const uint32_t cus = (uint32_t)ctx->prop.multiProcessorCount;
+        // A tile count a little over a whole number of rounds: the leading rows fill the rounds, the rest is a
+        // product with few tiles that runs split over K, behind it on the same stream.
+        const uint32_t top_rows = maize::tail_split_rows(*desc, cus);
+        if (top_rows) {
+            const uint64_t lda = desc->lda ? desc->lda : desc->gemm.a.ncols, ldc = desc->ldc ? desc->ldc : desc->gemm.c.ncols;
+            const uint64_t csz = desc->out_type == MAIZE_OUT_F32 ? 4u : 2u;
+            maize_gemm_ex_desc_t top = *desc, rest = *desc;
+            top.gemm.a.nrows = top.gemm.c.nrows = top_rows;
+            rest.gemm.a.nrows = rest.gemm.c.nrows = desc->gemm.a.nrows - top_rows;
+            rest.gemm.a.ptr = (char*)desc->gemm.a.ptr + (uint64_t)top_rows * lda * 2u;
+            rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)top_rows * ldc * csz;
+            rc = gemm_launch(ctx, &top, maize::select_kernel(top, cus), stream);
+            if (rc != MAIZE_OK) return rc;
+            return gemm_launch(ctx, &rest, maize::select_kernel(rest, cus), stream);
+        }
+        return gemm_launch(ctx, desc, maize::select_kernel(*desc, cus), stream);
+    }
     const int idx = maize::kernel_index(kernel);
     if (idx < 0) return fail(MAIZE_ERR_KERNEL, "gemm: no kernel named %s", kernel);
     if (!maize::kernel_at((uint32_t)idx).supports(*desc))

@@ -243,3 +243,28 @@ def test_dispatch_of_fp32_and_fp64_operands():
     assert mz.gemm_plan(ex(in_type=mz.IN_F32, out_type=mz.OUT_F32))["kernel"] == "maize_gemm_f32_mt128_nn"
     with pytest.raises(mz.MaizeError):
         mz.validate(ex(in_type=8))
+
+
+def test_tail_split_by_rows():
+    """A tile count a little over a whole number of rounds of one workgroup per compute unit: the leading tile rows
+    that fill the rounds are one product, the rest a second one that the dispatcher runs split over K."""
+    # 16 x 17 = 272 tiles on 256 compute units: 15 tile rows (255 tiles) on top, one tile row of 17 tiles below
+    x = ex(4096, 4352, 4096)
+    assert mz.gemm_tail_rows(x) == 15 * 256
+    top, rest = ex(15 * 256, 4352, 4096), ex(256, 4352, 4096)
+    assert mz.gemm_plan(top)["kernel"] == "maize_gemm_bf16_mt256_nn" and mz.gemm_plan(top)["grid"] == (255, 1, 1)
+    assert mz.gemm_plan(rest)["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and mz.gemm_plan(rest)["ksplit"] >= 2
+    assert mz.gemm_tail_rows(ex(4096, 4352, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_F16, beta=1.0)) == 15 * 256
+    # whole rounds, a single round, a round that is nearly full, or an edge the edge kernels take: one product
+    assert mz.gemm_tail_rows(ex(8192, 8192, 8192)) == 0          # 1024 tiles = 4 rounds
+    assert mz.gemm_tail_rows(ex(4096, 4096, 4096)) == 0          # 256 tiles
+    assert mz.gemm_tail_rows(ex(2048, 2048, 2048)) == 0          # 64 tiles
+    assert mz.gemm_tail_rows(ex(4000, 4104, 4032)) == 0          # narrow last tile column: edge splitting instead
+    assert mz.gemm_tail_rows(ex(4096, 6144, 4096)) == 0          # 384 tiles: the second round is half full, nothing to gain
+    # a short K: the round that would be saved is cheap, the extra launches are not
+    assert mz.gemm_tail_rows(ex(4096, 4352, 256)) == 0
+    # batches, 8-bit and wide operands are left alone; fewer compute units move the boundary
+    assert mz.gemm_tail_rows(ex(4096, 4352, 4096, batch=2, stride_a=4096 * 4096, stride_b=4096 * 4352, stride_c=4096 * 4352)) == 0
+    assert mz.gemm_tail_rows(ex(4096, 4352, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3)) == 0
+    assert mz.gemm_tail_rows(ex(4096, 4352, 4096, in_type=mz.IN_F32)) == 0
+    assert mz.gemm_tail_rows(x, compute_units=64) == 3840        # 272 = 4 x 64 + 16: 15 tile rows = 255 tiles fit 4 rounds of 64

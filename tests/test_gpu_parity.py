@@ -412,3 +412,25 @@ def test_operands_past_two_gib(ctx, oracle, which):
             assert s["n_fail"] == 0, f"past 2 GiB {which} {took}: {s}"
     finally:
         da.free(); db.free(); dc.free()
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+def test_tail_split_by_rows(ctx, oracle, layout):
+    """272 tiles on 256 compute units: the launcher computes the 15 leading tile rows as one product and the last tile row,
+    split over K, as a second one on the same stream.  Checked on sampled rows on both sides of the seam, and against
+    the single-kernel result, which the leading rows must equal bit for bit."""
+    m, n, k = 4096, 4352, 4096
+    x = mz.gemm_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x10000000, k, n) if layout == mz.LAYOUT_NN else mz.GlobalMatrix(0x10000000, n, k),
+                     mz.GlobalMatrix(0x20000000, m, n), layout=layout)
+    top = mz.gemm_tail_rows(x, compute_units=ctx.info()["compute_units"])
+    _say(f"tail split by rows: layout={layout} top rows {top}")
+    assert top == 15 * 256
+    a, b = inputs(m, n, k)
+    bs = b if layout == mz.LAYOUT_NN else b.reshape(k, n).T.copy().ravel()
+    got = run_gemm(ctx, a, bs, m, n, k, layout=layout)
+    rows = np.unique(np.concatenate([sample_rows(m, count=24, seed=5), [top - 1, top, top + 1, m - 1]])).astype(np.uint32)
+    check_rows_against_oracle(oracle, got, a, bs, m, n, k, rows, layout=layout, label="tail split by rows")
+    one = run_gemm(ctx, a, bs, m, n, k, layout=layout, kernel="maize_gemm_bf16_mt256_nn" if layout == mz.LAYOUT_NN else "maize_gemm_bf16_mt256_nt")
+    assert np.array_equal(got[:top * n], one[:top * n])             # the leading rows: the same kernel on the same tiles, bit for bit
+    below = np.arange(top, m, 8, dtype=np.uint32)                   # the rows below: another summation order, checked against the oracle
+    check_rows_against_oracle(oracle, got, a, bs, m, n, k, below, layout=layout, label="tail split by rows, rows below the seam")
