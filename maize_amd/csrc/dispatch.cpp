@@ -91,9 +91,8 @@ bool f8_nt_common(const maize_gemm_ex_desc_t& d) {
     if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr | (uintptr_t)d.gemm.c.ptr) & 15u) return false;
     if ((l.a | l.b) & 15u || (l.c & 7u)) return false;
     if (d.gemm.batch > 1 && (((d.gemm.stride_a | d.gemm.stride_b) & 15u) || (d.gemm.stride_c & 7u))) return false;
-    const uint64_t lim = 1ull << 31;                      // 32-bit offsets over a whole matrix (the kernel has no registers to spare for re-basing)
-    if (l.ext_a >= lim || l.ext_b >= lim || l.ext_c * 2 >= lim) return false;
-    if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21)) return false;
+    // 32-bit offsets span a tile's 256 rows (descriptors are re-based per tile): the matrices may be of any size
+    if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21) || l.c >= (1u << 21)) return false;
     return true;
 }
 #define MAIZE_F8_SUPPORTS(tag, type) \

@@ -125,8 +125,20 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 
 #define MAIZE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK>
+// F8: -1 = 16-bit operands; else 8-bit operands (one byte per element, both K-contiguous), bit 0: A is E5M2, bit 1:
+// B is E5M2 (else E4M3).  The 8-bit form is the same kernel on the same 128-byte LDS rows: a K tile is 128 elements
+// deep and one v_mfma_f32_16x16x128_f8f6f4 deep (not two 32-deep halves), a fragment is two 16-byte reads, and a K
+// step is four "eighths" of 16 MFMAs with the barrier before the third.
+template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1>
 __device__ __forceinline__ void body(const GemmArgs& p) {
+    constexpr bool IS8 = F8 >= 0;
+    static_assert(!IS8 || (NT && !F16 && !EDGE), "8-bit operands: both K-contiguous, no edge splitting");
+    constexpr uint32_t ES = IS8 ? 1u : 2u;              // bytes per element of A and B
+    constexpr uint32_t CH = 16u / ES;                   // elements per 16-byte chunk
+    constexpr int BKE = IS8 ? 128 : BK;                 // elements per K tile (128 bytes per row either way)
+    constexpr int NE = IS8 ? 4 : 8;                     // eighths (16 MFMAs each) per K step
+    constexpr int EB = IS8 ? 2 : 6;                     // the eighth the barrier stands in front of
+    constexpr int DS = IS8 ? 2 : DMA_STRIDE;            // MFMA slots between direct-to-LDS requests (an 8-bit MFMA is twice as long)
     // One array per operand, two ring stages each.  The fragment reads below are inline assembly (one
     // base register per operand and K half, the stage and the fragment in the 16-bit offset field), so
     // the compiler sees no read of these arrays and never makes one wait for the direct-to-LDS loads
@@ -158,15 +170,15 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     bool split = false;                                               // it is one K range of an edge tile
     uint32_t ks = 1u, edge = 0u, z = 0u;                              // its number of ranges, which edge tile, which range
     // K steps of a work item: [kt0, kt0 + nk) of the ceil(K / BK) steps -- all of them, or one of `nr` ranges.
-    const uint32_t nk_all = (K + BK - 1) / BK;
+    const uint32_t nk_all = (K + BKE - 1) / BKE;
     const uint32_t nranges = SPLITK ? (p.ksplit ? p.ksplit : 1u) : 1u;
     uint32_t nk, k_begin, k_end;                                      // k_end: loads at or past it return zeros
     auto select_range = [&](uint32_t zr, uint32_t nr) {
         const uint32_t per_range = (nk_all + nr - 1u) / nr;
         const uint32_t kt0 = zr * per_range;
         nk = kt0 < nk_all ? (nk_all - kt0 < per_range ? nk_all - kt0 : per_range) : 0u;
-        k_begin = kt0 * BK;
-        k_end = (kt0 + nk) * BK < K ? (kt0 + nk) * BK : K;
+        k_begin = kt0 * BKE;
+        k_end = (kt0 + nk) * BKE < K ? (kt0 + nk) * BKE : K;
     };
     select_range(0u, 1u);
     // Buffer descriptors start at the first row of the tile in hand and end with the operand's view (the last row
@@ -199,8 +211,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // vo = byte offset of the lane's chunk at k = 0 (with the N-edge mask folded in); the K
     // advance is a scalar offset (plain kernels) or added per lane (K-tail kernels).
     uint32_t m0, n0;
-    const uint16_t* Ag;
-    const uint16_t* Bg;
+    const char* Ag;                       // byte pointers: first row of the tile in hand
+    const char* Bg;
     uint16_t* Cg;
     uint32_t a_vo[8], b_vo[8];
     uint32_t a_k[2];                      // k index of the lane's chunk inside a tile, even/odd piece (K masks)
@@ -235,13 +247,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         }
         m0 = tile_m * BM;
         n0 = tile_n * BN;
-        Ag = p.a + bz * p.stride_a + (uint64_t)m0 * lda;                       // the tile's first row of A
-        a_bytes = span(((uint64_t)(M - 1u - m0) * lda + K) * 2u);
+        Ag = (const char*)p.a + (bz * p.stride_a + (uint64_t)m0 * lda) * ES;   // the tile's first row of A (strides count elements)
+        a_bytes = span(((uint64_t)(M - 1u - m0) * lda + K) * ES);
         if (NT) {
-            Bg = p.b + bz * p.stride_b + (uint64_t)n0 * ldb;                   // ... and of an N x K B
-            b_bytes = span(((uint64_t)(N - 1u - n0) * ldb + K) * 2u);
+            Bg = (const char*)p.b + (bz * p.stride_b + (uint64_t)n0 * ldb) * ES;   // ... and of an N x K B
+            b_bytes = span(((uint64_t)(N - 1u - n0) * ldb + K) * ES);
         } else {
-            Bg = p.b + bz * p.stride_b;                                        // (a K x N B is re-based per K tile, see dma)
+            Bg = (const char*)p.b + bz * p.stride_b * ES;                      // (a K x N B is re-based per K tile, see dma)
             b_bytes = 0u;
         }
         Cg = p.c + bz * p.stride_c * ((GEN && (p.epi & EPI_F32)) ? 2u : 1u);   // strides count elements of C
@@ -249,10 +261,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int i = 0; i < 8; ++i) {
             const uint32_t row = maps::kc_piece_row(wave * 8u + i, lane);
             const uint32_t c = maps::kc_piece_chunk(wave * 8u + i, lane);
-            a_vo[i] = (row * lda + c * 8u) * 2u;
-            if (i < 2) a_k[i] = c * 8u;
+            a_vo[i] = (row * lda + c * CH) * ES;
+            if (i < 2) a_k[i] = c * CH;
             if (NT) {
-                b_vo[i] = (row * ldb + c * 8u) * 2u;
+                b_vo[i] = (row * ldb + c * CH) * ES;
             } else {
                 const uint32_t brow = maps::sk_piece_row(wave * 8u + i, lane);
                 const uint32_t bc = maps::sk_piece_chunk(wave * 8u + i, lane);
@@ -274,16 +286,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             // the view; rows at or past K are past its end.
             const uint64_t skip = (uint64_t)k * ldb * 2u;
             const uint32_t bytes = k < k_end ? span(b_view - skip) : 0u;       // k < k_end <= K: skip < b_view
-            const __amdgpu_buffer_rsrc_t rs = make_rsrc((const char*)Bg + skip, bytes);
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(Bg + skip, bytes);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, b_vo[i], 0, 0, MAIZE_MT256_DMA_AUX);
             return;
         }
         const uint32_t bytes = k < k_end ? (is_a ? a_bytes : b_bytes) : 0u;
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(is_a ? (const void*)Ag : (const void*)Bg, bytes);
         if (!KTAIL) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i], k * 2u, 0, MAIZE_MT256_DMA_AUX);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i], k * ES, 0, MAIZE_MT256_DMA_AUX);
         } else {
-            uint32_t off = (is_a ? a_vo[i] : b_vo[i]) + k * 2u;
+            uint32_t off = (is_a ? a_vo[i] : b_vo[i]) + k * ES;
             off |= (a_k[i & 1] + k) < K ? 0u : OOB;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, off, 0, 0, MAIZE_MT256_DMA_AUX);
         }
@@ -298,12 +310,19 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // Base registers of the reads: LDS address of the operand's array + the lane's offset; everything
     // else of an address (stage, fragment, K half of the K x N tile) is a compile-time offset.
     uint32_t a_rd[2], b_rd[8];
+    if (IS8 || NT) {
+        // 8-bit operands, 16x16x128: lane l holds row l%16 and 32 bytes of K.  Which 32 is free as long as A and B agree
+        // (the instruction sums over all of K): the two chunks l/16 and 4 + l/16, i.e. exactly the two reads of the
+        // 16-bit kernel's K halves -- the access pattern that measures free of bank conflicts (chunks 2 (l/16) and
+        // 2 (l/16) + 1 cost every read a two-way conflict).
 #pragma unroll
-    for (int kh = 0; kh < 2; ++kh) a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * 128u, kh, lane);
-    if (NT) {
-#pragma unroll
-        for (int kh = 0; kh < 2; ++kh) b_rd[kh] = (uint32_t)(uintptr_t)B0 + maps::kc_frag16_offset(wn * 128u, kh, lane);
+        for (int kh = 0; kh < 2; ++kh) {
+            a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * 128u, kh, lane);
+            b_rd[kh] = (uint32_t)(uintptr_t)B0 + maps::kc_frag16_offset(wn * 128u, kh, lane);
+        }
     } else {
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh) a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * 128u, kh, lane);
 #pragma unroll
         for (int j = 0; j < 8; ++j) b_rd[j] = (uint32_t)(uintptr_t)B0 + maps::sk_tr_offset(wn * 8u + j, 0, lane);
     }
@@ -315,10 +334,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // and two buffers of 4 fragments per operand are enough:
     //   A group ai lives in fa[ai]; B group bi of K half kh lives in buffer bi ^ kh (the group that is
     //   held across the change of K half keeps its buffer, the other one is free for the new half).
+    // 8-bit operands: no K halves; the B buffer alternates with the ring stage instead (the group held across the
+    // change of K tile keeps its buffer), and a fragment is two 16-byte halves.
     bf16x8 fa[2][4];
     bf16x8 fb[2][4];
     short4v fbl[2][4], fbh[2][4];
-    constexpr int NBR = NT ? 4 : 8;                     // reads that bring in one B group (transposing reads are 64-bit)
+    u32x4 fa8[2][4][2], fb8[2][4][2];
+    constexpr int NAR = IS8 ? 8 : 4;                    // reads that bring in one A group
+    constexpr int NBR = (IS8 || !NT) ? 8 : 4;           // ... one B group (transposing reads are 64-bit, 8-bit fragments two reads)
     // Read r of a group is issued in MFMA slot r * RSTRIDE of the eighth.
 #ifndef MAIZE_MT256_RSTRIDE
 #define MAIZE_MT256_RSTRIDE 1
@@ -328,7 +351,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // base + 2048 * n (n = stage * 16 + kh * 8 + h).  The offsets are immediates: one case per value,
     // folded away once the caller's loops are unrolled.
 #define MAIZE_RD_CASE(n) case n: asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(base), "n"((n) * 2048)); break;
-    auto lds_read128 = [&](bf16x8& dst, uint32_t base, int n) {
+    auto lds_read128 = [&](auto& dst, uint32_t base, int n) {
         switch (n) {
             MAIZE_RD_CASE(0) MAIZE_RD_CASE(1) MAIZE_RD_CASE(2) MAIZE_RD_CASE(3) MAIZE_RD_CASE(4) MAIZE_RD_CASE(5) MAIZE_RD_CASE(6) MAIZE_RD_CASE(7)
             MAIZE_RD_CASE(16) MAIZE_RD_CASE(17) MAIZE_RD_CASE(18) MAIZE_RD_CASE(19) MAIZE_RD_CASE(20) MAIZE_RD_CASE(21) MAIZE_RD_CASE(22) MAIZE_RD_CASE(23)
@@ -344,12 +367,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         }
     };
 #undef MAIZE_RD_CASE
-    // Read r (0..3) of A group ai, K half kh, of the tile in stage st.
-    auto read_a = [&](int ai, int kh, int st, int r) { lds_read128(fa[ai][r], a_rd[kh], st * 16 + 4 * ai + r); };
+    // Read r (0..NAR-1) of A group ai, K half kh, of the tile in stage st.
+    auto read_a = [&](int ai, int kh, int st, int r) {
+        if (IS8) lds_read128(fa8[ai][r >> 1][r & 1], a_rd[r & 1], st * 16 + 4 * ai + (r >> 1));   // half r & 1 = the 16-bit kernel's kh
+        else     lds_read128(fa[ai][r], a_rd[kh], st * 16 + 4 * ai + r);
+    };
     // Read r (0..NBR-1) of B group bi, K half kh, of the tile in stage st.
     auto read_b = [&](int bi, int kh, int st, int r) {
-        const int buf = bi ^ kh;
-        if (NT) lds_read128(fb[buf][r], b_rd[kh], st * 16 + 4 * bi + r);
+        const int buf = bi ^ (IS8 ? st : kh);
+        if (IS8) lds_read128(fb8[buf][r >> 1][r & 1], b_rd[r & 1], st * 16 + 4 * bi + (r >> 1));
+        else if (NT) lds_read128(fb[buf][r], b_rd[kh], st * 16 + 4 * bi + r);
         else {
             const int c = r >> 1, h = r & 1;                  // rows 32 kh + 4 h + ...: 16 KiB and 2 KiB further on
             if (h == 0) lds_read_tr(fbl[buf][c], b_rd[4 * bi + c], st * 16 + kh * 8);
@@ -363,6 +390,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         return __builtin_bit_cast(bf16x8, r);
     };
 
+    typedef int i32x8 __attribute__((ext_vector_type(8)));
+    auto operand8 = [&](const u32x4 (&f)[2]) -> i32x8 {
+        return i32x8{(int)f[0][0], (int)f[0][1], (int)f[0][2], (int)f[0][3], (int)f[1][0], (int)f[1][1], (int)f[1][2], (int)f[1][3]};
+    };
+
     floatx4 acc[8][8];
     uint32_t k_early = 0;                  // tile whose early pieces are issued next (last quarter of a step)
     uint32_t k_late = 0;                   // tile whose late pieces are issued next (first quarter of a step)
@@ -373,12 +405,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     auto step = [&](int cur) {
         lds_ptr const ca = A0 + cur * TILE, cb = B0 + cur * TILE, na = A0 + (cur ^ 1) * TILE, nb = B0 + (cur ^ 1) * TILE;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int kh = e >> 2, h4 = e & 3;
+        for (int e = 0; e < NE; ++e) {
+            const int kh = IS8 ? 0 : e >> 2, h4 = e & 3;
             const int ai = h4 >> 1, bi = (h4 == 1 || h4 == 2) ? 1 : 0;
+            const bool last_half = IS8 || kh == 1;                // the groups after this half belong to the next K tile
             // The group this eighth needs was requested during the one before: it has to be in.
-            if (e != 6) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (e == 6) {
+            if (e != EB) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (e == EB) {
                 // Every fragment this step still needs from (ca, cb) is in registers.  Wait until
                 // this wave's share of tile t+1 has landed, then meet the other waves: after the
                 // barrier (na, nb) is complete and (ca, cb) is free to be refilled with tile t+2.
@@ -399,7 +432,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // The accumulator is tied to itself ("+a"): left to the register allocator, a few of the 64
                 // tuples were renamed across the loop and copied back through VGPRs at its end.  (Each
                 // accumulator comes up again 128 MFMAs later: no dependent back-to-back issue.)
-                if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
+                if (IS8)   // 8-bit operands: B is the first source, so cbsz carries B's format and blgp A's (0 = E4M3, 1 = E5M2)
+                    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(acc[4 * ai + r4][4 * bi + c4])
+                                 : "v"(operand8(fb8[bi ^ cur][c4])), "v"(operand8(fa8[ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
+                else if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
                     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(bi ^ kh, c4)), "v"(fa[ai][r4]));
                 else
                     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(bi ^ kh, c4)), "v"(fa[ai][r4]));
@@ -407,23 +443,23 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 if (s % MAIZE_MT256_RSTRIDE == 0) {
                     const int r = s / MAIZE_MT256_RSTRIDE;
                     if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);                       // (0,0) -> (0,1): B group 1
-                    if (h4 == 1 && r < 4) read_a(1, kh, cur, r);                         // (0,1) -> (1,1): A group 1
-                    if (h4 == 2 && r < 4) { if (kh == 0) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }     // next half: A group 0
-                    if (h4 == 3 && r < NBR) { if (kh == 0) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }   // next half: B group 0
+                    if (h4 == 1 && r < NAR) read_a(1, kh, cur, r);                       // (0,1) -> (1,1): A group 1
+                    if (h4 == 2 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }   // next half or tile: A group 0
+                    if (h4 == 3 && r < NBR) { if (!last_half) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }   // next half or tile: B group 0
                 }
                 // ... and the direct-to-LDS request scheduled for this slot (issue_slot): late pieces of
                 // tile t+1 (its stage was freed by the previous barrier) before this step's barrier, early
                 // pieces of tile t+2 behind it.
-                const int slot = e >= 6 ? 16 * (e - 6) + s : 32 + 16 * e + s;
-                if (slot >= 2 && (slot - 2) % DMA_STRIDE == 0 && (slot - 2) / DMA_STRIDE < 16) {
-                    if (e >= 6) dma((slot - 2) / DMA_STRIDE, ca, cb, k_early);
-                    else        dma((slot - 2) / DMA_STRIDE, na, nb, k_late);
+                const int slot = e >= EB ? 16 * (e - EB) + s : 32 + 16 * e + s;
+                if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {
+                    if (e >= EB) dma((slot - 2) / DS, ca, cb, k_early);
+                    else         dma((slot - 2) / DS, na, nb, k_late);
                 }
                 MAIZE_FENCE();
             }
         }
-        k_early += BK;
-        k_late += BK;
+        k_early += BKE;
+        k_late += BKE;
     };
     // ---- prime: the first K tile of the first C tile, whole ------------------------------
 #pragma unroll
@@ -437,13 +473,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // The wait also covers the C stores of the previous tile (loads and stores share the counter).
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-    for (int r = 0; r < 4; ++r) read_a(0, 0, 0, r);
+    for (int r = 0; r < NAR; ++r) read_a(0, 0, 0, r);
 #pragma unroll
     for (int r = 0; r < NBR; ++r) read_b(0, 0, 0, r);
 #pragma unroll
-    for (int pc = 0; pc < early_pieces(); ++pc) dma(pc, A1, B1, k_begin + BK);   // tile 1, early pieces
-    k_early = k_begin + 2 * BK;
-    k_late = k_begin + BK;
+    for (int pc = 0; pc < 16; ++pc)
+        if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);   // tile 1, early pieces
+    k_early = k_begin + 2 * BKE;
+    k_late = k_begin + BKE;
     // Two steps per trip so that each step sees its stages as compile-time constants.  An odd
     // step count runs one extra step on an all-zero tile (loads past K return zeros).
     for (uint32_t kt = 0; kt < nk; kt += 2) {

@@ -37,32 +37,25 @@ MAIZE_MAP uint32_t kc_offset(uint32_t row, uint32_t chunk) { return row * 128u +
 MAIZE_MAP uint32_t kc_frag16_offset(uint32_t row_base, uint32_t kh, uint32_t lane) {
     return kc_offset(row_base + (lane & 15u), 4u * kh + (lane >> 4));
 }
-// Fragment read of MFMA 32x32x64 on 8-bit elements (the same tile: 128 elements per row): lane l
-// holds row base + l%32 and the 32 bytes k = 64 kh + 32 (l/32) + 0..31, read as two chunks (c01 = 0, 1).
-MAIZE_MAP uint32_t kc_frag8_offset(uint32_t row_base, uint32_t kh, uint32_t c01, uint32_t lane) {
-    return kc_offset(row_base + (lane & 31u), 4u * kh + 2u * (lane >> 5) + c01);
-}
+// MFMA 16x16x128 on 8-bit elements (the same tile: 128 elements per row) uses the same two reads per fragment,
+// kh = 0 and 1: lane l then holds row base + l%16 and the 32 bytes of chunks l/16 and 4 + l/16.  Any assignment of K
+// to lanes is right as long as A and B share it; this one keeps the access pattern of the 16-bit reads.
 
 // ---- 16-bit epilogue staging of the macro-tile kernels: 32 rows of 256 B per wave and pass -----------
-// MFMA 32x32 accumulators (the 8-bit kernel).  Write: lane l holds 4 consecutive columns (8 B) of row l%32: columns 32 j + 8 q + 4 (l/32) + 0..3.
-MAIZE_MAP uint32_t epi_write_offset(uint32_t j, uint32_t q, uint32_t lane) {
-    const uint32_t row = lane & 31u, lhi = lane >> 5;
-    return row * 256u + (((j * 4u + q) ^ (row & 15u)) * 16u) + ((lhi ^ ((row >> 4) & 1u)) * 8u);
-}
-// Read r (0..7): lane l reads the 16-byte chunk l%16 of row 4 r + l/16; rows with bit 4 set hold their halves swapped.
+// Read r (0..7): lane l reads the 16-byte chunk l%16 of row 4 r + l/16.
 MAIZE_MAP uint32_t epi_read_row(uint32_t r, uint32_t lane) { return r * 4u + (lane >> 4); }
 MAIZE_MAP uint32_t epi_read_offset(uint32_t r, uint32_t lane) {
     const uint32_t row = epi_read_row(r, lane);
     return row * 256u + (((lane & 15u) ^ (row & 15u)) * 16u);
 }
 
-// The same region for MFMA 16x16x32 accumulators (the 16-bit kernel): lane l holds 4 consecutive columns of row 16 ii + l%16
+// Write, MFMA 16 x 16 accumulators (16-bit and 8-bit operands alike): lane l holds 4 consecutive columns of row 16 ii + l%16
 // (ii = 0, 1: the pass's two accumulator rows): columns 16 j + 4 (l/16) + 0..3 of the 128.
 MAIZE_MAP uint32_t epi16_write_offset(uint32_t ii, uint32_t j, uint32_t lane) {
     const uint32_t row = ii * 16u + (lane & 15u), g = lane >> 4;
     return row * 256u + (((2u * j + (g >> 1)) ^ (row & 15u)) * 16u) + (g & 1u) * 8u;
 }
-MAIZE_MAP uint32_t epi16_read_offset(uint32_t r, uint32_t lane) { return epi_read_offset(r, lane); }   // no halves swapped
+MAIZE_MAP uint32_t epi16_read_offset(uint32_t r, uint32_t lane) { return epi_read_offset(r, lane); }
 // fp32 staging of the general epilogue: 32 rows x 64 columns (row = 256 B = 16 chunks of 4 columns); lane l
 // writes the 16 bytes of row 16 ii + l%16, columns 16 jj + 4 (l/16) + 0..3.
 MAIZE_MAP uint32_t epi32_write_offset(uint32_t ii, uint32_t jj, uint32_t lane) {

@@ -67,19 +67,16 @@ def test_matrix_instruction_per_kernel(kernels):
             assert count(ins, "ds_read_b128") >= 16 and count(ins, "ds_read_b64_tr_b16") == 0, name
             assert len([i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]) >= 16, name
         elif name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")):
-            # 8-bit operands: the 64-deep instruction.  B is fed as the first source, so cbsz carries B's format
-            # code and blgp A's (E4M3 = 0 is not printed, E5M2 = 1).
-            f8 = [i for i in ins if i.startswith("v_mfma_f32_32x32x64_f8f6f4")]
-            assert len(f8) >= 64 and count(ins, "v_mfma_f32_32x32x16") == 0, name   # two unrolled K steps of 128
+            # 8-bit operands: the 128-deep 16 x 16 instruction (cheaper per multiply-add at the power limit than 32 x 32 x 64).
+            # B is fed as the first source, so cbsz carries B's format code and blgp A's (E4M3 = 0 is not printed, E5M2 = 1).
+            f8 = [i for i in ins if i.startswith("v_mfma_f32_16x16x128_f8f6f4")]
+            assert len(f8) == 128 and count(ins, "v_mfma") == 128, name       # two unrolled K steps of 128 elements, 64 MFMAs each
             tag = name[len("maize_gemm_"):].split("_")[0]
             a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
             assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
-        elif "_mt256_" in name:
-            # 16 x 16 x 32 on purpose: less accumulator traffic per multiply-add than 32 x 32 x 16, which the
-            # board's power limit turns into run time
-            want = "v_mfma_f32_16x16x32_f16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_16x16x32_bf16"
-            other = "v_mfma_f32_16x16x32_bf16" if name.startswith("maize_gemm_f16_") else "v_mfma_f32_16x16x32_f16"
-            assert count(ins, want) == 256 and count(ins, other) == 0 and count(ins, "v_mfma_f32_32x32") == 0, name   # two fully unrolled K steps of 64
+            body = ins[next(k for k, i in enumerate(ins) if i.startswith("v_mfma")):len(ins) - next(k for k, i in enumerate(reversed(ins)) if i.startswith("v_mfma"))]
+            assert count(body, "ds_read_b128") == 64 and count(body, "buffer_load_dwordx4") == 32 and count(body, "s_barrier") == 2, name
+            assert count(body, "v_accvgpr") == 0 and count(body, "v_mov_b32") == 0, name     # accumulators and fragments stay in place
         elif "_mt128_" in name:
             # the catalogue's tf32 and f64 entries: full fp32 / fp64 matrix instructions; one K tile of 128 bytes
             # per row (8 or 4 steps of 16 MFMAs), in the 128-bit and in the element-wise version of the loop

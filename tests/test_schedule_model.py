@@ -34,8 +34,8 @@ def mt256_issue_slots():
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
     stride = int(re.search(r"#define MAIZE_MT256_DMA_STRIDE (\d+)", src).group(1))
     assert "constexpr int issue_slot(int pc) { return DMA_STRIDE * pc + 2; }" in src
-    assert "if (slot >= 2 && (slot - 2) % DMA_STRIDE == 0 && (slot - 2) / DMA_STRIDE < 16) {" in src
-    assert "n += issue_slot(i) < 32;" in src                 # early pieces: those behind the barrier of step t itself
+    assert "constexpr int DS = IS8 ? 2 : DMA_STRIDE;" in src and "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {" in src
+    assert "if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);" in src      # early pieces: those behind the barrier of step t itself
     return [stride * pc + 2 for pc in range(16)]
 
 
@@ -44,13 +44,14 @@ def mt256_reads_per_eighth(nt):
     before it holds: 4 reads of 128 bits, or 8 transposing reads of 64 bits for a group of a row-major B.
     Within a K half the groups come in the order B1, A1, then A0 and B0 of the next half (the source states it)."""
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
-    assert "constexpr int NBR = NT ? 4 : 8;" in src
+    assert "constexpr int NBR = (IS8 || !NT) ? 8 : 4;" in src
     for line in ("if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);",
-                 "if (h4 == 1 && r < 4) read_a(1, kh, cur, r);",
-                 "if (h4 == 2 && r < 4) { if (kh == 0) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
-                 "if (h4 == 3 && r < NBR) { if (kh == 0) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }"):
+                 "if (h4 == 1 && r < NAR) read_a(1, kh, cur, r);",
+                 "if (h4 == 2 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
+                 "if (h4 == 3 && r < NBR) { if (!last_half) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }"):
         assert line in src, line
-    assert "if (e == 6) {" in src and "const int slot = e >= 6 ? 16 * (e - 6) + s : 32 + 16 * e + s;" in src
+    assert "constexpr int EB = IS8 ? 2 : 6;" in src and "if (e == EB) {" in src
+    assert "const int slot = e >= EB ? 16 * (e - EB) + s : 32 + 16 * e + s;" in src
     nbr = 4 if nt else 8
     # reads that bring in eighth e (issued during e - 1): e = 0: A0 and B0 (the first of them, A0, a whole eighth earlier)
     return [nbr, nbr, 4, 0, nbr, nbr, 4, 0], nbr
@@ -211,49 +212,70 @@ def test_macro_tile_checker_rejects_broken_schedules():
 
 
 # ---------------------------------------------------------------------------------------
-# 8-bit macro-tile kernel: the same two-stage ring, one K step = two halves of 16 MFMAs, the barrier
-# between them, all 16 requests of tile t+2 in the second half of step t
+# 8-bit macro-tile kernel: the same template with a K tile one matrix instruction deep: a K step is four groups of
+# 16 MFMAs, the barrier in front of the third, a group is 8 reads, one request per two MFMA slots
 # ---------------------------------------------------------------------------------------
 
-def f8_wave_program(nk, barrier_half=1, dma_half=1):
-    src = open(os.path.join(KDIR, "gemm_mt256_f8.hpp")).read()
-    step = src[src.index("auto step = "):src.index("// ---- prime")]
-    # the facts the model is built from, as the source states them
-    assert "if (kh == 1) {" in step and 's_waitcnt vmcnt(0) lgkmcnt(0)\\n\\ts_barrier' in step
-    assert "if (kh == 0) read_frag(1, 1, s, ca, cb);" in step
-    assert "read_frag(0, 0, s, na, nb);" in step and "dma(s, ca, cb, k_next);" in step
-    assert "for (int pc = 0; pc < 16; ++pc) dma(pc, A1, B1, k_begin + BK);" in src
+def f8_constants():
+    src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
+    for fact in ("constexpr int NE = IS8 ? 4 : 8;", "constexpr int EB = IS8 ? 2 : 6;", "constexpr int DS = IS8 ? 2 : DMA_STRIDE;",
+                 "constexpr int NAR = IS8 ? 8 : 4;", "const bool last_half = IS8 || kh == 1;",
+                 "const int slot = e >= EB ? 16 * (e - EB) + s : 32 + 16 * e + s;",
+                 "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {", "if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);"):
+        assert fact in src, fact
+    return dict(ne=4, eb=2, ds=2, reads=8)
+
+
+def f8_wave_program(nk, barrier_at=None, ds=None):
+    c = f8_constants()
+    eb = c["eb"] if barrier_at is None else barrier_at
+    ds = c["ds"] if ds is None else ds
+    slots = [ds * pc + 2 for pc in range(16)]
+    # reads issued during group e: (group whose MFMAs need them, from the next tile?)
+    issued = {0: (1, False), 1: (2, False), 2: (0, True), 3: (0, True)}
     ops = [("dma", 0, pc, 0) for pc in range(16)]
     ops += [("wait_all",), ("barrier",)]
-    ops += [("read", 0, 0, 0)] * 16
-    ops += [("dma", 1, pc, 1) for pc in range(16)]
+    ops += [("read", 0, 0, 0)] * (2 * c["reads"])
+    ops += [("dma", 1, pc, 1) for pc in range(16) if slots[pc] < 32]
+    k_early, k_late = 2, 1
     steps = nk + (nk & 1)
     for t in range(steps):
         cur, nxt = t & 1, (t & 1) ^ 1
-        for kh in range(2):
-            if kh == barrier_half:
+        for e in range(c["ne"]):
+            if e == eb:
                 ops += [("wait_all",), ("barrier",)]
+            need, next_tile = issued[e]
             for sl in range(16):
-                ops.append(("mfma", t, kh))
-                ops.append(("read", t, 1, cur) if kh == 0 else ("read", t + 1, 0, nxt))
-                if kh == dma_half:
-                    ops.append(("dma", t + 2, sl, cur))
+                ops.append(("mfma", t, e))
+                if sl < c["reads"]:
+                    ops.append(("read", t + 1, need, nxt) if next_tile else ("read", t, need, cur))
+                slot = 16 * (e - c["eb"]) + sl if e >= c["eb"] else 32 + 16 * e + sl
+                for pc in range(16):
+                    if slots[pc] == slot:
+                        ops.append(("dma", k_early, pc, cur) if e >= c["eb"] else ("dma", k_late, pc, nxt))
+        k_early += 1
+        k_late += 1
     ops.append(("wait_all",))
     return ops, steps
+
+
+F8_CUMULATIVE = [16, 24, 32, 32]      # reads of a tile that must have been issued before group e multiplies: A0 B0 | B1 | A1 | -
 
 
 @pytest.mark.parametrize("nk", [1, 2, 3, 7, 32])
 def test_8bit_macro_tile_schedule_is_hazard_free(nk):
     ops, steps = f8_wave_program(nk)
-    last_tile = check_two_stage(ops, steps, 16, parts=2)
-    assert last_tile == steps + 1
+    last_tile = check_two_stage(ops, steps, F8_CUMULATIVE, parts=4)
+    assert steps <= last_tile <= steps + 1
 
 
 def test_8bit_macro_tile_checker_rejects_broken_schedules():
-    with pytest.raises(Hazard):                 # requests in the first half: the stage still holds fragments to be read
-        check_two_stage(*f8_wave_program(8, dma_half=0), 16, parts=2)
-    with pytest.raises(Hazard):                 # barrier at the top of the step: tile t+1's reads race with its own landing
-        check_two_stage(*f8_wave_program(8, barrier_half=0), 16, parts=2)
+    with pytest.raises(Hazard):                 # barrier one group late: the next tile is read before it is known to be complete
+        check_two_stage(*f8_wave_program(8, barrier_at=3), F8_CUMULATIVE, parts=4)
+    with pytest.raises(Hazard):                 # barrier one group early: the stage is refilled while its last group is still being read
+        check_two_stage(*f8_wave_program(8, barrier_at=1), F8_CUMULATIVE, parts=4)
+    with pytest.raises(Hazard):                 # requests four slots apart: the last ones would come after the next barrier and never be issued
+        check_two_stage(*f8_wave_program(8, ds=5), F8_CUMULATIVE, parts=4)
 
 
 # ---------------------------------------------------------------------------------------
