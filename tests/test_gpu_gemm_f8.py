@@ -5,7 +5,7 @@ maize_hip_gemm_bf16_ex, against the oracle's 8-bit restatement (mzo_ref_gemm8) o
 Tolerance.  The per-wave kernel widens the operands to bf16 (exactly) and keeps the bar of the bf16
 product: bf16 C within 1 bf16 ULP of the oracle's bits or, where the result nearly cancels, |got - exact|
 <= (K/16 + 2) * 2^-24 * scale + half a bf16 ULP; fp32 C within (K/16 + 4) * 2^-24 * scale.  The macro-tile
-kernels use v_mfma_f32_32x32x64_f8f6f4, whose dot-product unit drops products more than 13 binades below
+kernels use v_mfma_f32_16x16x128_f8f6f4, whose dot-product unit drops products more than 13 binades below
 the largest of the 64 it adds (test_what_the_8bit_matrix_instruction_keeps pins that): their floor is
 (2^-15 + (K/64 + 2) * 2^-24) * scale (measured on these operands: at most 2^-16.3 * scale), the 1-ULP bar
 is unchanged.  Closed forms whose products stay within 13 binades of each other are bit-exact."""
