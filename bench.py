@@ -26,7 +26,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each
 # scaled by what the same counter reads for a 256 MiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x
 # 1.000): profiles/hbm_traffic_fetch_write_size.md.  Not measured for the other configurations.
-MEASURED_TRAFFIC_BYTES = {"cfg1": 235.1e6, "cfg4": 126.4e6, "f8": 134.5e6}   # f8: profiles/gemm_e4m3_mt256_nt_4096x4096x4096.md
+MEASURED_TRAFFIC_BYTES = {"cfg1": 235.2e6, "cfg2": 275.1e6, "cfg3": 1746.3e6, "cfg4": 126.4e6, "cfg5": 1074.3e6,
+                          "f8": 134.5e6, "f8s": 67.2e6, "f32": 828.9e6, "f64": 3162.3e6}
 
 # name -> (M, N, K, layout, batch, A distribution, B distribution, bound)
 CONFIGS = {
