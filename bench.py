@@ -175,7 +175,7 @@ def main():
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--others", action=argparse.BooleanOptionalAction, default=None,
-                    help="also measure the other BASELINE configurations (shorter runs) and report them under "
+                    help="also measure the other benchmark configurations (shorter runs) and report them under "
                          "\"other_configs\" (default: on when no --config is given)")
     ap.add_argument("--rotate", type=int, default=0,
                     help="number of distinct operand sets cycled through (0: enough to exceed the 256 MiB "
@@ -196,7 +196,7 @@ def main():
     ctx = mz.Context(0)
     line = measure(mz, ctx, args.config, args.steps, args.warmup, args.kernel, args.rotate, not args.no_cpu)
     if args.others:
-        # The other BASELINE configurations, shorter runs, same process: reported beside the headline.
+        # The other benchmark configurations, shorter runs, same process: reported beside the headline.
         others = {}
         for name in sorted(CONFIGS):
             if name == args.config:

@@ -192,7 +192,7 @@ int32_t maize_hip_module_load(maize_ctx_t* ctx, const void* hsaco, size_t nbytes
     if (nbytes < 64 || memcmp(hsaco, "\177ELF", 4) != 0)
         return fail(MAIZE_ERR_ARG, "module_load: not an ELF code object (%zu bytes)", nbytes);
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     maize_module* m = new (std::nothrow) maize_module();
     if (!m) return fail(MAIZE_ERR_NOMEM, "module_load: out of host memory");
     m->ctx = ctx;
@@ -399,7 +399,7 @@ static int32_t workspace_for(maize_ctx_t* ctx, void* stream, size_t bytes, void*
     maize_workspace& w = ctx->workspaces[stream];
     if (w.bytes < bytes) {
         DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
         if (w.ptr) {
             HIP_TRY(hipStreamSynchronize((hipStream_t)stream));  // earlier launches may still use the old one
             HIP_TRY(hipFree(w.ptr));
@@ -538,7 +538,7 @@ int32_t maize_hip_malloc(maize_ctx_t* ctx, size_t nbytes, void** out) {
     *out = nullptr;
     if (nbytes == 0) return fail(MAIZE_ERR_ARG, "malloc: zero bytes");
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipMalloc(out, nbytes));
     return MAIZE_OK;
 }
@@ -547,7 +547,7 @@ int32_t maize_hip_free(maize_ctx_t* ctx, void* ptr) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "free: ctx is NULL");
     if (!ptr) return MAIZE_OK;
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipFree(ptr));
     return MAIZE_OK;
 }
@@ -555,7 +555,7 @@ int32_t maize_hip_free(maize_ctx_t* ctx, void* ptr) {
 int32_t maize_hip_memcpy_h2d(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes) {
     if (!ctx || !dst || !src) return fail(MAIZE_ERR_NULL, "memcpy_h2d: NULL argument");
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipMemcpy(dst, src, nbytes, hipMemcpyHostToDevice));
     return MAIZE_OK;
 }
@@ -563,7 +563,7 @@ int32_t maize_hip_memcpy_h2d(maize_ctx_t* ctx, void* dst, const void* src, size_
 int32_t maize_hip_memcpy_d2h(maize_ctx_t* ctx, void* dst, const void* src, size_t nbytes) {
     if (!ctx || !dst || !src) return fail(MAIZE_ERR_NULL, "memcpy_d2h: NULL argument");
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipMemcpy(dst, src, nbytes, hipMemcpyDeviceToHost));
     return MAIZE_OK;
 }
@@ -571,7 +571,7 @@ int32_t maize_hip_memcpy_d2h(maize_ctx_t* ctx, void* dst, const void* src, size_
 int32_t maize_hip_memset(maize_ctx_t* ctx, void* dst, int value, size_t nbytes) {
     if (!ctx || !dst) return fail(MAIZE_ERR_NULL, "memset: NULL argument");
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     HIP_TRY(hipMemset(dst, value, nbytes));
     return MAIZE_OK;
 }
@@ -579,7 +579,7 @@ int32_t maize_hip_memset(maize_ctx_t* ctx, void* dst, int value, size_t nbytes) 
 int32_t maize_hip_stream_create(maize_ctx_t* ctx, void** out) {
     if (!ctx || !out) return fail(MAIZE_ERR_NULL, "stream_create: NULL argument");
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     hipStream_t s;
     HIP_TRY(hipStreamCreate(&s));  // default priority
     *out = (void*)s;
@@ -589,7 +589,7 @@ int32_t maize_hip_stream_create(maize_ctx_t* ctx, void** out) {
 int32_t maize_hip_stream_destroy(maize_ctx_t* ctx, void* stream) {
     if (!ctx || !stream) return fail(MAIZE_ERR_NULL, "stream_destroy: NULL argument");
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     // The stream's workspace goes with it (its launches first run to completion).
     auto it = ctx->workspaces.find(stream);
     if (it != ctx->workspaces.end()) {
@@ -605,7 +605,7 @@ int32_t maize_hip_stream_destroy(maize_ctx_t* ctx, void* stream) {
 int32_t maize_hip_sync(maize_ctx_t* ctx, void* stream) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "sync: ctx is NULL");
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     if (stream)
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     else
@@ -617,7 +617,7 @@ int32_t maize_hip_event_create(maize_ctx_t* ctx, maize_event_t** out) {
     if (!ctx || !out) return fail(MAIZE_ERR_NULL, "event_create: NULL argument");
     *out = nullptr;
     DeviceGuard guard_;
-    HIP_TRY(guard_.enter(ctx->device));
+        HIP_TRY(guard_.enter(ctx->device));
     maize_event* ev = new (std::nothrow) maize_event();
     if (!ev) return fail(MAIZE_ERR_NOMEM, "event_create: out of host memory");
     hipError_t e = hipEventCreate(&ev->ev);
