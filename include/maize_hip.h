@@ -94,8 +94,13 @@ typedef struct {
  *   out_type:    element type of C; batch stride stride_c counts elements of that type.
  *   beta == 0:   C is not read (it may hold anything, NaNs included).
  * All-zero extension fields with alpha = 1 describe exactly the plain descriptor. */
-/* MAIZE_OUT_SAME: C has the 16-bit type of A and B (bf16, or half for half operands; bf16 for 8-bit operands). */
-typedef enum { MAIZE_OUT_SAME = 0, MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1 } maize_out_type_t;
+/* MAIZE_OUT_SAME: C has the 16-bit type of A and B (bf16, or half for half operands; bf16 for 8-bit operands).
+ * MAIZE_OUT_F16: C is IEEE half -- the catalogue's entries with half results (Sm80MmaF16F16_16x8x16,
+ * crates/maize_tile/src/mma/sm80.rs:8; Sm89MmaF8F16_16x8x16 / _16x8x32, sm89.rs:18-19).  gfx950 has no matrix
+ * instruction that accumulates in half: the sum is kept in fp32 and rounded to half once, so the result is at
+ * least as close to the exact product as the reference op's.  Half operands (where it equals MAIZE_OUT_SAME)
+ * and 8-bit operands only. */
+typedef enum { MAIZE_OUT_SAME = 0, MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1, MAIZE_OUT_F16 = 2 } maize_out_type_t;
 /* Element type of A and B.  The reference's MMA catalogue lists the half-precision twin of its bf16
  * op (Sm80MmaF16F32_16x8x16 beside Sm80MmaBf16F32_16x8x16, crates/maize_tile/src/mma/sm80.rs);
  * here it is v_mfma_f32_*_f16 on the same tiles.  E4M3 and E5M2 are the OCP 8-bit floats of the

@@ -39,6 +39,7 @@ LAYOUT_NT = 1
 OUT_SAME = 0
 OUT_BF16 = 0
 OUT_F32 = 1
+OUT_F16 = 2     # C in IEEE half: half or 8-bit operands
 IN_BF16 = 0
 IN_F16 = 1
 IN_E4M3 = 2

@@ -193,8 +193,8 @@ def gemm_desc(a, b, c, layout=LAYOUT_NN, batch=1, stride_a=0, stride_b=0, stride
 def gemm_ex_desc(a, b, c, layout=LAYOUT_NN, batch=1, stride_a=0, stride_b=0, stride_c=0, lda=0, ldb=0, ldc=0,
                  out_type=_ffi.OUT_SAME, alpha=1.0, beta=0.0, in_type=_ffi.IN_BF16):
     """Build a maize_gemm_ex_desc_t: the descriptor plus leading dimensions (0 = ncols), the
-    element type of C (OUT_SAME: the operands' 16-bit type), C = alpha * A.B + beta * C, and the element
-    type of A and B (bf16 or IEEE half)."""
+    element type of C (OUT_SAME: the operands' 16-bit type, bf16 for 8-bit operands; OUT_F32; OUT_F16: IEEE half,
+    for half or 8-bit operands), C = alpha * A.B + beta * C, and the element type of A and B (IN_*)."""
     x = _ffi.GemmExDescT()
     x.gemm = gemm_desc(a, b, c, layout, batch, stride_a, stride_b, stride_c)
     x.lda, x.ldb, x.ldc = lda, ldb, ldc

@@ -24,7 +24,8 @@ inline Lds lds_of(const maize_gemm_ex_desc_t& d) {
 }
 // The plain product: bf16 C = A.B (alpha == 1, beta == 0).
 inline bool plain_epilogue(const maize_gemm_ex_desc_t& d) {
-    return d.out_type == MAIZE_OUT_SAME && d.alpha == 1.0f && d.beta == 0.0f;
+    // (a half C for half operands is MAIZE_OUT_SAME under its other name)
+    return (d.out_type == MAIZE_OUT_SAME || (d.out_type == MAIZE_OUT_F16 && d.in_type == MAIZE_IN_F16)) && d.alpha == 1.0f && d.beta == 0.0f;
 }
 inline bool half_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_F16; }
 inline bool bf16_in(const maize_gemm_ex_desc_t& d) { return d.in_type == MAIZE_IN_BF16; }

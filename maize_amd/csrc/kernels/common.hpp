@@ -26,6 +26,8 @@ struct GemmArgs {
 };
 static_assert(sizeof(GemmArgs) == 120, "kernel parameter block layout");
 constexpr uint32_t EPI_F32 = 1u, EPI_SCALE = 2u, EPI_F16 = 4u, EPI_F8 = 8u, EPI_A_E5M2 = 16u, EPI_B_E5M2 = 32u;
+constexpr uint32_t EPI_C_F16 = 64u;     // a 16-bit C is IEEE half whatever the operands are (with EPI_F16 it is anyway)
+__device__ __forceinline__ bool c_is_half(uint32_t epi) { return (epi & (EPI_F16 | EPI_C_F16)) != 0u; }
 
 // Leading dimensions with their defaults: the reference's rows are compact (row stride ==
 // ncols, crates/maize_tile/src/gmem/row_panel.rs:55).
@@ -109,7 +111,7 @@ __device__ __forceinline__ void store_c_run(const GemmArgs& p, void* c, uint64_t
     float x[NV];
 #pragma unroll
     for (int e = 0; e < NV; ++e) x[e] = acc[e];
-    const bool f32_out = p.epi & EPI_F32, half_io = p.epi & EPI_F16;
+    const bool f32_out = p.epi & EPI_F32, half_io = c_is_half(p.epi);
     if ((p.epi & EPI_SCALE)) {
         float old[NV];
 #pragma unroll

@@ -38,7 +38,7 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
     const uint64_t bz = blockIdx.z;
     const uint16_t* __restrict__ A = p.a + bz * p.stride_a;
     const uint16_t* __restrict__ B = p.b + bz * p.stride_b;
-    const bool f32_out = p.epi & EPI_F32, scaled = p.epi & EPI_SCALE, half_io = p.epi & EPI_F16;
+    const bool f32_out = p.epi & EPI_F32, scaled = p.epi & EPI_SCALE, half_io = p.epi & EPI_F16, c_half = c_is_half(p.epi);
     const bool f8 = p.epi & EPI_F8, a_e5m2 = p.epi & EPI_A_E5M2, b_e5m2 = p.epi & EPI_B_E5M2;
     const uint8_t* __restrict__ A8 = (const uint8_t*)p.a + bz * p.stride_a;
     const uint8_t* __restrict__ B8 = (const uint8_t*)p.b + bz * p.stride_b;
@@ -88,11 +88,11 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_wave32(GemmArg
                 const uint64_t at = (uint64_t)cm * ldc + cn;
                 float x = acc[v];
                 if (scaled) {
-                    const float old = p.beta == 0.0f ? 0.0f : f32_out ? Cf[at] : half_io ? f16_bits_to_f32(C[at]) : bf16_bits_to_f32(C[at]);
+                    const float old = p.beta == 0.0f ? 0.0f : f32_out ? Cf[at] : c_half ? f16_bits_to_f32(C[at]) : bf16_bits_to_f32(C[at]);
                     x = epi_scale(x, old, p.alpha, p.beta);
                 }
                 if (f32_out) Cf[at] = x;
-                else if (half_io) C[at] = __builtin_bit_cast(uint16_t, (_Float16)x);
+                else if (c_half) C[at] = __builtin_bit_cast(uint16_t, (_Float16)x);
                 else C[at] = f32_to_bf16_rne(x);
             }
         }

@@ -33,7 +33,7 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_splitk_reduce(GemmA
     const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     void* c = (char*)p.c + (uint64_t)bz * p.stride_c * ((p.epi & EPI_F32) ? 4u : 2u);
     const uint64_t at = (uint64_t)row * ldc + col;
-    const bool f32_out = p.epi & EPI_F32, half_io = p.epi & EPI_F16;
+    const bool f32_out = p.epi & EPI_F32, half_io = c_is_half(p.epi);
     // Vector path: the run is whole and 16-byte (bf16/half) or 32-byte (fp32) aligned.
     const uint64_t addr = (uint64_t)c + at * (f32_out ? 4u : 2u);
     if (col + 8u <= N && (addr & (f32_out ? 31u : 15u)) == 0) {

@@ -293,9 +293,11 @@ int32_t maize_hip_gemm_ex_validate(const maize_gemm_ex_desc_t* x) {
     if (d->c.nrows != M || d->c.ncols != N)
         return fail(MAIZE_ERR_SHAPE, "gemm: C is %ux%u, expected %ux%u", d->c.nrows, d->c.ncols, M, N);
     if (!d->a.ptr || !d->b.ptr || !d->c.ptr) return fail(MAIZE_ERR_NULL, "gemm: NULL matrix pointer");
-    if (x->out_type != MAIZE_OUT_BF16 && x->out_type != MAIZE_OUT_F32)
+    if (x->out_type != MAIZE_OUT_BF16 && x->out_type != MAIZE_OUT_F32 && x->out_type != MAIZE_OUT_F16)
         return fail(MAIZE_ERR_ARG, "gemm: unknown output type %u", x->out_type);
     if (x->in_type > MAIZE_IN_F64) return fail(MAIZE_ERR_ARG, "gemm: unknown operand type %u", x->in_type);
+    if (x->out_type == MAIZE_OUT_F16 && !(x->in_type == MAIZE_IN_F16 || (x->in_type >= MAIZE_IN_E4M3 && x->in_type <= MAIZE_IN_E5M2_E4M3)))
+        return fail(MAIZE_ERR_ARG, "gemm: a half C (MAIZE_OUT_F16) goes with half or 8-bit operands, not with operand type %u", x->in_type);
     if (x->in_type == MAIZE_IN_F64 && x->out_type != MAIZE_OUT_SAME)
         return fail(MAIZE_ERR_ARG, "gemm: fp64 operands have an fp64 C (out_type must be MAIZE_OUT_SAME)");
     if (x->reserved) return fail(MAIZE_ERR_ARG, "gemm: reserved field must be 0");
@@ -431,7 +433,7 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
     args.lda = x->lda; args.ldb = x->ldb; args.ldc = x->ldc;
     args.alpha = x->alpha; args.beta = x->beta;
     args.epi = (x->out_type == MAIZE_OUT_F32 ? 1u : 0u) | ((x->alpha != 1.0f || x->beta != 0.0f) ? 2u : 0u) |
-               (x->in_type == MAIZE_IN_F16 ? 4u : 0u) | ((x->in_type >= MAIZE_IN_E4M3 && x->in_type <= MAIZE_IN_E5M2_E4M3) ? 8u : 0u) |
+               (x->in_type == MAIZE_IN_F16 ? 4u : 0u) | (x->out_type == MAIZE_OUT_F16 ? 64u : 0u) | ((x->in_type >= MAIZE_IN_E4M3 && x->in_type <= MAIZE_IN_E5M2_E4M3) ? 8u : 0u) |
                ((x->in_type == MAIZE_IN_E5M2 || x->in_type == MAIZE_IN_E5M2_E4M3) ? 16u : 0u) |       // A is E5M2
                ((x->in_type == MAIZE_IN_E5M2 || x->in_type == MAIZE_IN_E4M3_E5M2) ? 32u : 0u);        // B is E5M2
     maize::LaunchDims ld;

@@ -180,7 +180,7 @@ def fp8_bits_to_f64(bits, elem):
 
 
 def ref_gemm_ex(a, b, m, n, k, layout=NN, lda=None, ldb=None, alpha=1.0, beta=0.0, c_old=None, out_f32=False,
-                nthreads=None, elem=BF16):
+                nthreads=None, elem=BF16, c_elem=None):
     """The extended product for one batch member, on operand views with leading dimensions:
         C = round( alpha * (A.B in fp64) + beta * C_old ),   round = RNE to bf16, or to fp32.
     ``a`` and ``b`` are flat uint16 arrays holding the views (row r of A starts at r*lda); ``c_old`` is a
@@ -193,7 +193,7 @@ def ref_gemm_ex(a, b, m, n, k, layout=NN, lda=None, ldb=None, alpha=1.0, beta=0.
     ldb = bcols if ldb is None else ldb
     dt = operand_dtype(elem)
     isz = np.dtype(dt).itemsize
-    celem = BF16 if is_fp8(elem) else elem                      # element type of a 16-bit C
+    celem = c_elem if c_elem is not None else BF16 if is_fp8(elem) else elem   # element type of a 16-bit C (c_elem=F16: a half C for 8-bit operands)
     a = np.asarray(a, dtype=dt).ravel()
     b = np.asarray(b, dtype=dt).ravel()
     av = np.lib.stride_tricks.as_strided(a, shape=(m, k), strides=(isz * lda, isz))

@@ -8,6 +8,7 @@ pub const MAIZE_LAYOUT_NN: u32 = 0;
 pub const MAIZE_LAYOUT_NT: u32 = 1;
 pub const MAIZE_OUT_SAME: u32 = 0;
 pub const MAIZE_OUT_F32: u32 = 1;
+pub const MAIZE_OUT_F16: u32 = 2;
 pub const MAIZE_IN_BF16: u32 = 0;
 pub const MAIZE_IN_F16: u32 = 1;
 pub const MAIZE_IN_E4M3: u32 = 2;

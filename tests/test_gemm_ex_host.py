@@ -268,3 +268,23 @@ def test_tail_split_by_rows():
     assert mz.gemm_tail_rows(ex(4096, 4352, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3)) == 0
     assert mz.gemm_tail_rows(ex(4096, 4352, 4096, in_type=mz.IN_F32)) == 0
     assert mz.gemm_tail_rows(x, compute_units=64) == 3840        # 272 = 4 x 64 + 16: 15 tile rows = 255 tiles fit 4 rounds of 64
+
+
+def test_half_c_goes_with_half_and_8bit_operands_only():
+    """MAIZE_OUT_F16: the catalogue's entries with half results (Sm80MmaF16F16_16x8x16, crates/maize_tile/src/mma/sm80.rs:8;
+    Sm89MmaF8F16_*, sm89.rs:18-19).  For half operands it is OUT_SAME under another name (same plan); for 8-bit ones
+    the kernels with the run-time epilogue take it; bf16, fp32 and fp64 operands are refused."""
+    big = dict(m=4096, n=4096, k=4096)
+    assert mz.gemm_plan(ex(**big, in_type=mz.IN_F16, out_type=mz.OUT_F16)) == mz.gemm_plan(ex(**big, in_type=mz.IN_F16))
+    plan = mz.gemm_plan(ex(**big, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3, out_type=mz.OUT_F16))
+    assert plan["kernel"] == "maize_gemm_e4m3_mt256_nt_gen"
+    assert not _supports("maize_gemm_e4m3_mt256_nt", ex(**big, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3, out_type=mz.OUT_F16))
+    assert mz.gemm_plan(ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_E5M2, out_type=mz.OUT_F16))["kernel"] == "maize_gemm_e5m2_skinny_nt"
+    for it in (mz.IN_BF16, mz.IN_F32, mz.IN_F64):
+        with pytest.raises(mz.MaizeError) as e:
+            mz.validate(ex(in_type=it, out_type=mz.OUT_F16))
+        assert e.value.code == _ffi.MAIZE_ERR_ARG
+    with pytest.raises(mz.MaizeError):
+        mz.validate(ex(out_type=3))
+    # a half C is 2 bytes per element: 2-byte aligned pointers pass
+    mz.validate(ex(ptrs=(0x1001, 0x100003, 0x2000002), in_type=mz.IN_E4M3, out_type=mz.OUT_F16))

@@ -208,6 +208,32 @@ def test_half_operands_macro_tile(ctx, oracle, layout, shape, lds):
         assert took == want, took
 
 
+def test_half_operands_out_f16_is_out_same(ctx, oracle):
+    """For half operands MAIZE_OUT_F16 names the C they have anyway (Sm80MmaF16F16_16x8x16's result type,
+    crates/maize_tile/src/mma/sm80.rs:8): same kernel, same bits."""
+    m, n, k = 300, 520, 136
+    rng = np.random.default_rng(77)
+    a = (rng.random(m * k) * 2 - 1).astype(np.float16).view(np.uint16)
+    b = (rng.random(k * n) * 2 - 1).astype(np.float16).view(np.uint16)
+    da, db = ctx.upload(a), ctx.upload(b)
+    out = {}
+    try:
+        for name, ot in (("same", mz.OUT_SAME), ("f16", mz.OUT_F16)):
+            dc = ctx.upload(np.zeros(m * n, np.uint16))
+            x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n), mz.Matrix(dc, m, n), out_type=ot, in_type=mz.IN_F16)
+            took = mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"]
+            ctx.gemm_bf16(x)
+            ctx.sync()
+            out[name] = (took, dc.download(np.uint16))
+            dc.free()
+    finally:
+        da.free(); db.free()
+    assert out["same"][0] == out["f16"][0]
+    assert np.array_equal(out["same"][1], out["f16"][1])
+    ref, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, elem=oracle.F16)
+    assert oracle.compare(out["f16"][1], ref, val, scale, k, elem=oracle.F16)["n_fail"] == 0
+
+
 @pytest.mark.parametrize("m", [3, 16])
 def test_half_operands_skinny(ctx, oracle, m):
     for kw in KNOBS:

@@ -37,13 +37,13 @@ def ab_of(elem):
 
 
 def launch(ctx, a, b, c0, m, n, k, layout, fmt, lda, ldb, ldc, alpha=1.0, beta=0.0, out_f32=False, kernel=None, batch=1,
-           strides=(0, 0, 0)):
+           strides=(0, 0, 0), out_f16=False):
     brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
     da, db, dc = ctx.upload(a), ctx.upload(b), ctx.upload(c0)
     try:
         x = mz.gemm_ex_desc(mz.Matrix(da, m, k, elem_bytes=1), mz.Matrix(db, brows, bcols, elem_bytes=1), mz.Matrix(dc, m, n),
                             layout=layout, lda=0 if lda == k else lda, ldb=0 if ldb == bcols else ldb, ldc=0 if ldc == n else ldc,
-                            out_type=mz.OUT_F32 if out_f32 else mz.OUT_SAME, alpha=alpha, beta=beta, in_type=FMT[fmt][0],
+                            out_type=mz.OUT_F32 if out_f32 else mz.OUT_F16 if out_f16 else mz.OUT_SAME, alpha=alpha, beta=beta, in_type=FMT[fmt][0],
                             batch=batch, stride_a=strides[0], stride_b=strides[1], stride_c=strides[2])
         took = mz.gemm_plan(x, kernel=kernel, compute_units=ctx.info()["compute_units"])["kernel"]
         ctx.gemm_bf16(x, kernel=kernel)
@@ -55,7 +55,7 @@ def launch(ctx, a, b, c0, m, n, k, layout, fmt, lda, ldb, ldc, alpha=1.0, beta=0
 
 
 def run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NT, fmt="e4m3", lda=None, ldb=None, ldc=None, alpha=1.0, beta=0.0,
-           out_f32=False, kernel=None, seed=1, label=""):
+           out_f32=False, kernel=None, seed=1, label="", out_f16=False):
     elem = FMT[fmt][1]
     brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
     lda = k if lda is None else lda
@@ -65,14 +65,17 @@ def run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NT, fmt="e4m3", lda=None, ldb=
     b = f8_uniform(oracle, brows * ldb, 200 + seed, ab_of(elem)[1])
     if out_f32:
         c0 = (np.random.default_rng(seed).standard_normal(m * ldc) * 2).astype(np.float32)
+    elif out_f16:
+        c0 = oracle.bf16_bits_from_f64(np.random.default_rng(seed).random(m * ldc) * 2.0 - 1.0, oracle.F16)
     else:
         c0 = mz.gen.uniform_bf16(m * ldc, 300 + seed)
-    got, took = launch(ctx, a, b, c0, m, n, k, layout, fmt, lda, ldb, ldc, alpha, beta, out_f32, kernel)
-    _say(f"{label} {fmt} M={m} N={n} K={k} ld=({lda},{ldb},{ldc}) alpha={alpha} beta={beta} f32={out_f32} -> {took}")
+    got, took = launch(ctx, a, b, c0, m, n, k, layout, fmt, lda, ldb, ldc, alpha, beta, out_f32, kernel, out_f16=out_f16)
+    _say(f"{label} {fmt} M={m} N={n} K={k} ld=({lda},{ldb},{ldc}) alpha={alpha} beta={beta} f32={out_f32} f16={out_f16} -> {took}")
     gv, ov = got.reshape(m, ldc), c0.reshape(m, ldc)
     assert np.array_equal(gv[:, n:].view(np.uint8), ov[:, n:].view(np.uint8)), f"{label}: wrote into C's row padding"
     ref, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, layout=layout, lda=lda, ldb=ldb, alpha=alpha, beta=beta,
-                                         c_old=None if beta == 0.0 else ov[:, :n].copy(), out_f32=out_f32, elem=elem)
+                                         c_old=None if beta == 0.0 else ov[:, :n].copy(), out_f32=out_f32, elem=elem,
+                                         c_elem=oracle.F16 if out_f16 else None)
     g = gv[:, :n]
     f8_unit = "mt256" in took
     if out_f32:
@@ -81,7 +84,8 @@ def run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NT, fmt="e4m3", lda=None, ldb=
         bad = ~(err <= tol)
         assert not bad.any(), f"{label}: {int(bad.sum())} of {bad.size} fp32 elements out of tolerance, worst {float((err / tol).max()):.2f}x"
     else:
-        s = oracle.compare(g, ref, val, scale, k, coeff=oracle.floor_coeff_f8(k) if f8_unit else None)
+        s = oracle.compare(g, ref, val, scale, k, elem=oracle.F16 if out_f16 else oracle.BF16,
+                           coeff=oracle.floor_coeff_f8(k) if f8_unit else None)
         assert s["n_fail"] == 0, f"{label}: {s}"
         _say(f"   max_ulp {s['max_ulp']} n_gt1ulp {s['n_gt1ulp']} of {s['n']}")
     return took
@@ -296,3 +300,41 @@ def test_packed_path_for_8bit_operands(ctx, oracle, fmt):
         single, _ = launch(ctx, ab_[i * sa:i * sa + m * k], bb_[i * sb:i * sb + k * n], np.zeros(m * n, np.uint16), m, n, k, NN, fmt, k, n, n)
         assert np.array_equal(single, dense[i * sc:i * sc + m * n]), i
         assert not dense[i * sc + m * n:(i + 1) * sc].any(), "wrote between batch members"
+
+
+# ---- a half C: the catalogue's 8-bit entries with half results (Sm89MmaF8F16_16x8x16 / _16x8x32,
+# crates/maize_tile/src/mma/sm89.rs:18-19), summed in fp32 and rounded to half once ------------------------------
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2"])
+@pytest.mark.parametrize("case", [
+    # (M, N, K, layout, leading dimensions or None, alpha, beta, kernel family expected in the name)
+    (512, 768, 384, mz.LAYOUT_NT, None, 1.0, 0.0, "mt256_nt_gen"),
+    (300, 520, 144, mz.LAYOUT_NT, (160, 176, 528), -0.75, 0.5, "mt256_nt_gen"),
+    (256, 512, 8192, mz.LAYOUT_NT, None, 1.0, 0.0, "splitk"),
+    (16, 2048, 1024, mz.LAYOUT_NT, None, 2.0, 1.0, "skinny_nt"),
+    (200, 264, 400, mz.LAYOUT_NN, None, 1.0, 0.0, ""),
+    (33, 17, 65, mz.LAYOUT_NN, None, 0.5, -1.0, "wave32"),
+])
+def test_half_c_for_8bit_operands(ctx, oracle, fmt, case):
+    m, n, k, layout, lds, alpha, beta, family = case
+    lda, ldb, ldc = lds if lds else (None, None, None)
+    took = run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, lda=lda, ldb=ldb, ldc=ldc, alpha=alpha, beta=beta,
+                  out_f16=True, label="half C")
+    assert family in took, f"expected a {family} kernel, the dispatcher took {took}"
+
+
+def test_half_c_is_rounded_to_half_not_through_bf16(ctx, oracle):
+    """All-ones operands, K = 4112: every element of C is 4112, which half holds exactly (13 bits, the low four
+    zero) and bf16 does not (it would come out as 4096 or 4128)."""
+    m, n, k = 256, 256, 4112
+    one = oracle.fp8_bits_from_f64(np.ones(1), 2)[0]
+    a = np.full(m * k, one, dtype=np.uint8)
+    b = np.full(n * k, one, dtype=np.uint8)
+    c0 = np.zeros(m * n, dtype=np.uint16)
+    got, took = launch(ctx, a, b, c0, m, n, k, mz.LAYOUT_NT, "e4m3", k, k, n, out_f16=True)
+    _say(f"all-ones K={k} half C -> {took}")
+    want = oracle.bf16_bits_from_f64(np.array([4112.0]), oracle.F16)[0]
+    assert float(np.array([want], dtype=np.uint16).view(np.float16)[0]) == 4112.0
+    assert np.all(got == want), f"{took}: {np.unique(got)[:8]} instead of {want:#06x}"
+    got_bf16, _ = launch(ctx, a, b, c0, m, n, k, mz.LAYOUT_NT, "e4m3", k, k, n)
+    assert not np.any(oracle.bf16_bits_to_f64(got_bf16) == 4112.0)          # the bf16 C of the same product cannot hold it
