@@ -182,11 +182,12 @@ bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld
 // K ranges per tile.  Candidates: up to one (tile, range) work item per compute unit, at least 4 K
 // steps per range, at most 64 ranges, no empty range, partial tiles (256 KiB slots) under 1 GiB.
 // The choice minimises a cost model fitted to measurements on this part (microseconds):
-//   unsplit:  8 + 1.0 * steps                       (few workgroups: each runs at full clock)
-//   split:    8 + 1.2 * steps / ks + 6 + 2e-6 * M * N * batch * ks
-// i.e. a second launch and the fp32 partial tiles written and read back at ~4 TB/s; the split is
-// taken only if it wins by 20 %.  (2048^3, 64 tiles: 38 us unsplit, 40 us split 4 ways -- not
-// split; 64 x 4096 x 4096: 63 -> 25 us; 256 x 256 x 16384: 237 -> 38 us.)
+//   unsplit:  8 + 1.0 * steps
+//   split:    8 + 1.0 * steps / ks + 6 + (1.2e-6 * M * N * batch + 0.15) * ks
+// i.e. a second launch, the fp32 partial tiles written and read back, and a little per range; the
+// split is taken only if it wins by 10 %.  (2048^3, 64 tiles: 38 us unsplit, 40 us split 4 ways -- not
+// split; 64 x 4096 x 4096: 63 -> 22 us; 256 x 256 x 16384: 237 -> 38 us; 256 x 14336 x 4096, 56 tiles:
+// 67 -> 46 us four ways; 768 x 8192 x 8192, 96 tiles: 128 -> 93 us two ways.)
 uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * batch;
     const uint32_t nk = cdiv(s.k, kstep);                    // K steps of 128 bytes per row: 64 16-bit elements, 128 8-bit ones
@@ -196,12 +197,12 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
     if (kmax > 64u) kmax = 64u;
     const double unsplit = 8.0 + 1.0 * nk;
     const double elems = (double)s.m * s.n * batch;
-    double best = unsplit * 0.8;
+    double best = unsplit * 0.9;
     uint32_t best_ks = 1;
     for (uint32_t ks = 2; ks <= kmax; ++ks) {
         if (cdiv(nk, cdiv(nk, ks)) != ks) continue;            // would leave an empty range
         if (tiles * ks * 262144ull > (1ull << 30)) break;
-        const double t = 8.0 + 1.2 * cdiv(nk, ks) + 6.0 + 2e-6 * elems * ks;
+        const double t = 8.0 + 1.0 * cdiv(nk, ks) + 6.0 + (1.2e-6 * elems + 0.15) * ks;
         if (t < best) { best = t; best_ks = ks; }
     }
     return best_ks;
@@ -695,7 +696,7 @@ uint32_t tail_split_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units) 
     const uint32_t ks = splitk_ranges(bottom, 1, compute_units);
     if (ks < 2u) return 0;
     const double t_round = 8.0 + 1.0 * nk;
-    const double t_bottom = 3.0 + 8.0 + 1.2 * cdiv(nk, ks) + 6.0 + 2e-6 * (double)bottom.m * s.n * ks;
+    const double t_bottom = 3.0 + 8.0 + 1.0 * cdiv(nk, ks) + 6.0 + (1.2e-6 * (double)bottom.m * s.n + 0.15) * ks;
     if (t_bottom > 0.75 * t_round) return 0;
     // the rows below start on a 16-byte boundary like the matrix itself (leading dimensions are multiples of 8)
     return tm_top * 256u;
