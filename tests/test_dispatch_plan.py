@@ -196,6 +196,20 @@ def test_split_k_of_few_tiles_fills_the_chip_once():
     assert mz.gemm_plan(desc(512, 512, 448), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
 
 
+def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
+    """56 to 128 tiles on 256 compute units leave most of the chip idle for a whole walk of K: two or four K ranges
+    per tile pay for the partial tiles (measured: 256 x 14336 x 4096 67 -> 46 us, 768 x 8192 x 8192 128 -> 93 us),
+    while 2048^3 (64 tiles, a short K) stays whole (37 us against 40)."""
+    p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 4 and p["grid"] == (224, 1, 1)
+    p = mz.gemm_plan(desc(768, 8192, 8192), compute_units=CUS)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 2 and p["grid"] == (192, 1, 1)
+    p = mz.gemm_plan(desc(640, 8192, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_splitk" and p["ksplit"] == 2
+    assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
+    assert mz.gemm_plan(desc(1024, 14336, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"   # 224 tiles: one round as it is
+
+
 def test_skinny_split_fills_the_chip_without_overshooting():
     p = mz.gemm_plan(desc(16, 14336, 4096), compute_units=CUS)
     assert p["grid"] == (56, 4, 1)                              # 224 workgroups on 256 compute units
