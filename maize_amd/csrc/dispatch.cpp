@@ -467,13 +467,20 @@ bool skinny_nt_common(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
     const Lds l = lds_of(d);
     const uint32_t esz = fp8_in(d) ? 1u : 2u, per16 = 16u / esz;
-    if (nn(d) || s.m > 16u || (s.k % per16) || (s.n & 7u)) return false;
-    if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr | (uintptr_t)d.gemm.c.ptr) & 15u) return false;
-    if ((l.a % per16) || (l.b % per16) || (l.c & 7u)) return false;
-    if (d.gemm.batch > 1 && ((d.gemm.stride_a % per16) || (d.gemm.stride_b % per16) || (d.gemm.stride_c & 7u))) return false;
+    if (nn(d) || s.m > 16u || (s.k % per16)) return false;
+    if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr) & 15u) return false;
+    if ((l.a % per16) || (l.b % per16)) return false;              // C: any N, leading dimension and pointer (skinny_nt_c_by_elements)
+    if (d.gemm.batch > 1 && ((d.gemm.stride_a % per16) || (d.gemm.stride_b % per16))) return false;
     const uint64_t lim = 1ull << 31;
     if (l.ext_a * esz >= lim || l.ext_b * esz >= lim || s.k >= (1u << 21) || l.b >= (1u << 21)) return false;
     return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
+}
+// C rows that cannot take 128-bit stores: the kernel then writes C element by element (bit 0 of split_first).
+bool skinny_nt_c_by_elements(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    const uint32_t per16 = d.out_type == MAIZE_OUT_F32 ? 4u : 8u;    // elements of C per 16 bytes
+    return (s.n & 7u) || (l.c % per16) || ((uintptr_t)d.gemm.c.ptr & 15u) || (d.gemm.batch > 1 && (d.gemm.stride_c % per16));
 }
 bool skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d); }
 #define MAIZE_F8_SKINNY(tag, type) \
@@ -499,7 +506,7 @@ bool skinny_nt_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Launc
     ld->block[0] = 512; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
     ld->ksplit = ks;
-    ld->split_first = 0;
+    ld->split_first = skinny_nt_c_by_elements(d) ? 1u : 0u;
     ld->reduce_grid = 0;
     ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * 16u * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets

@@ -151,4 +151,26 @@ __device__ __forceinline__ void store_c_run(const GemmArgs& p, void* c, uint64_t
     }
 }
 
+// The same for C rows that are not 16-byte material (any N, leading dimension and 2-byte aligned pointer):
+// the first `count` (<= NV) elements of the run, one by one.
+template <int NV>
+__device__ __forceinline__ void store_c_elems(const GemmArgs& p, void* c, uint64_t at, const float (&acc)[NV], uint32_t count) {
+    const bool f32_out = p.epi & EPI_F32, half_c = c_is_half(p.epi);
+#pragma unroll
+    for (int e = 0; e < NV; ++e) {
+        if ((uint32_t)e >= count) break;
+        float x = acc[e];
+        if (p.epi & EPI_SCALE) {
+            float old = 0.0f;
+            if (p.beta != 0.0f)
+                old = f32_out ? ((const float*)c)[at + e]
+                              : half_c ? f16_bits_to_f32(((const uint16_t*)c)[at + e]) : bf16_bits_to_f32(((const uint16_t*)c)[at + e]);
+            x = epi_scale(x, old, p.alpha, p.beta);
+        }
+        if (f32_out) ((float*)c)[at + e] = x;
+        else if (half_c) ((uint16_t*)c)[at + e] = __builtin_bit_cast(uint16_t, (_Float16)x);
+        else ((uint16_t*)c)[at + e] = f32_to_bf16_rne(x);
+    }
+}
+
 }  // namespace maize

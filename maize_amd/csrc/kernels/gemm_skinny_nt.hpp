@@ -25,8 +25,10 @@
 //   * ragged K: chunks at or past K are masked per lane (K % 8 == 0 for 16-bit, K % 16 == 0 for 8-bit
 //     operands); blocks past the end of a range read through a zero-length descriptor.
 //
-// Requirements (checked by the dispatcher): layout NT, M <= 16, N % 8 == 0, rows of A and B on 16-byte
-// boundaries, every matrix (per batch member) below 2 GiB.
+// Requirements (checked by the dispatcher): layout NT, M <= 16, rows of A and B on 16-byte boundaries, every
+// matrix (per batch member) below 2 GiB.  Any N, leading dimension of C and element-aligned C pointer (a
+// vocabulary of 50257 rows of B is as good as one of 50264): rows of B at or past N read as zeros, and C goes
+// out in 128-bit runs when its rows allow it, element by element otherwise.
 #pragma once
 #include "common.hpp"
 #include "gemm_skinny.hpp"
@@ -176,13 +178,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // ---- combine the K splits in split order, round once, store (as the NN kernel does) ----------
     // Lane holds C[m = l%16][n = n0 + 16(2w + c2) + 4g + 0..3].
     const uint32_t m = r16;
+    // Rows of C that are not 16-byte material (odd N or leading dimension, a pointer off the 16-byte grid: a
+    // launch-uniform flag from the dispatcher) are stored element by element; C is at most 16 rows.
+    const bool c_elems = p.reserved & 1u;
     if (ks == 1u) {
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {
             const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
             if (m < M && col < N) {
                 const float v[4] = {acc[c2][0], acc[c2][1], acc[c2][2], acc[c2][3]};
-                store_c_run<4>(p, Cg, (uint64_t)m * ldc + col, v);
+                if (c_elems) store_c_elems<4>(p, Cg, (uint64_t)m * ldc + col, v, N - col);
+                else store_c_run<4>(p, Cg, (uint64_t)m * ldc + col, v);
             }
         }
         return;
@@ -229,9 +235,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
         }
         const uint32_t col = n0 + cq;
-        if (row < M && col < N) {                          // N % 8 == 0: 8 columns are all in or all out
+        if (row < M && col < N) {                          // vector stores: N % 8 == 0, 8 columns are all in or all out
             const float v[8] = {s_lo[0], s_lo[1], s_lo[2], s_lo[3], s_hi[0], s_hi[1], s_hi[2], s_hi[3]};
-            store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);
+            if (c_elems) store_c_elems<8>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
+            else store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);
         }
     }
     if (tid == 0) counters[slab_id] = 0u;                 // ready for the next launch

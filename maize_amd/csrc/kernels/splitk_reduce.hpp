@@ -33,7 +33,7 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_splitk_reduce(GemmA
     const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     void* c = (char*)p.c + (uint64_t)bz * p.stride_c * ((p.epi & EPI_F32) ? 4u : 2u);
     const uint64_t at = (uint64_t)row * ldc + col;
-    const bool f32_out = p.epi & EPI_F32, half_io = c_is_half(p.epi);
+    const bool f32_out = p.epi & EPI_F32;
     // Vector path: the run is whole and 16-byte (bf16/half) or 32-byte (fp32) aligned.
     const uint64_t addr = (uint64_t)c + at * (f32_out ? 4u : 2u);
     if (col + 8u <= N && (addr & (f32_out ? 31u : 15u)) == 0) {
@@ -41,19 +41,7 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_splitk_reduce(GemmA
         return;
     }
     // Any N, leading dimension and alignment: element by element (the product ran on padded copies).
-    for (uint32_t e = 0; e < 8u && col + e < N; ++e) {
-        float x = v[e];
-        if (p.epi & EPI_SCALE) {
-            float old = 0.0f;
-            if (p.beta != 0.0f)
-                old = f32_out ? ((const float*)c)[at + e]
-                              : half_io ? f16_bits_to_f32(((const uint16_t*)c)[at + e]) : bf16_bits_to_f32(((const uint16_t*)c)[at + e]);
-            x = epi_scale(x, old, p.alpha, p.beta);
-        }
-        if (f32_out) ((float*)c)[at + e] = x;
-        else if (half_io) ((uint16_t*)c)[at + e] = __builtin_bit_cast(uint16_t, (_Float16)x);
-        else ((uint16_t*)c)[at + e] = f32_to_bf16_rne(x);
-    }
+    store_c_elems<8>(p, c, at, v, N - col);
 }
 
 }  // namespace maize

@@ -210,6 +210,16 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
     assert mz.gemm_plan(desc(1024, 14336, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"   # 224 tiles: one round as it is
 
 
+def test_skinny_nt_takes_any_n():
+    """N x K weights with an odd number of rows (50257) keep the streaming kernel; C then goes out element by element."""
+    p = mz.gemm_plan(desc(16, 50257, 768, layout=mz.LAYOUT_NT), compute_units=CUS)
+    assert p["kernel"] == "maize_gemm_bf16_skinny_nt" and p["split_first"] == 1 and p["grid"][0] == cdiv(50257, 256)
+    p = mz.gemm_plan(desc(16, 50264, 768, layout=mz.LAYOUT_NT), compute_units=CUS)
+    assert p["kernel"] == "maize_gemm_bf16_skinny_nt" and p["split_first"] == 0
+    # a K x N B with odd N has unaligned rows of B: not for the streaming kernels
+    assert "skinny" not in mz.gemm_plan(desc(16, 50257, 768), compute_units=CUS)["kernel"]
+
+
 def test_skinny_split_fills_the_chip_without_overshooting():
     p = mz.gemm_plan(desc(16, 14336, 4096), compute_units=CUS)
     assert p["grid"] == (56, 4, 1)                              # 224 workgroups on 256 compute units

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import maize_amd as mz
-from test_gpu_gemm_ex import run_ex
+from test_gpu_gemm_ex import run_ex, run_packed
 from test_gpu_gemm_f8 import FMT, f8_uniform, launch, run_f8
 
 pytestmark = pytest.mark.gpu
@@ -86,3 +86,24 @@ def test_repeats_batches_and_the_shared_workspace(ctx, oracle):
         assert not dense[i * sc + m * n:(i + 1) * sc].any(), "wrote between batch members"
     assert run_ex(ctx, oracle, 16, 1096, 4096, label="NN skinny after NT") == "maize_gemm_bf16_skinny_nn"
     assert run_ex(ctx, oracle, 16, 1096, 4096, layout=NT, label="NT skinny bf16") == "maize_gemm_bf16_skinny_nt"
+
+
+def test_any_n_and_any_c_rows(ctx, oracle):
+    """The weights' row count N and C's rows need not be 16-byte material (a vocabulary of 50257 rows of B): rows of
+    B at or past N read as zeros and C is stored element by element; nothing outside the M x N view of C changes."""
+    name = "maize_gemm_bf16_skinny_nt"
+    assert run_ex(ctx, oracle, 16, 50257, 768, layout=NT, label="odd N") == name
+    assert run_ex(ctx, oracle, 1, 1001, 4096, layout=NT, label="odd N, one row") == name
+    assert run_ex(ctx, oracle, 16, 1001, 4096, layout=NT, half=True, label="odd N, half") == name
+    assert run_ex(ctx, oracle, 7, 1000, 4096, layout=NT, ldc=1003, label="N % 8 == 0, odd ldc") == name
+    for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=1007),
+               dict(alpha=2.0, beta=0.0, c_nan=True, ldc=1005)):
+        assert run_ex(ctx, oracle, 16, 1001, 4096, layout=NT, label="odd N epilogue", **kw) == name
+    assert run_ex(ctx, oracle, 16, 263, 512, layout=NT, kernel=name, label="odd N, one K range") == name
+    # C starts 2 bytes past a 16-byte boundary (N and ldc fine): still this kernel, element stores
+    assert run_packed(ctx, oracle, 16, 1096, 4096, NT, None, c_off=1, label="C off the 16-byte grid") == name
+    assert run_packed(ctx, oracle, 16, 1001, 4096, NT, None, c_off=3, ldc=1002, out_f32=True, alpha=0.5, beta=2.0, label="fp32 C off the grid") == name
+    for fmt in ("e4m3", "e5m2e4m3"):
+        assert run_f8(ctx, oracle, 16, 32003, 1024, fmt=fmt, label="odd N f8") == f"maize_gemm_{fmt}_skinny_nt"
+        assert run_f8(ctx, oracle, 5, 1001, 4096, fmt=fmt, alpha=0.5, beta=1.0, ldc=1003, label="odd N f8 scaled") == f"maize_gemm_{fmt}_skinny_nt"
+        assert run_f8(ctx, oracle, 16, 1001, 2048, fmt=fmt, out_f16=True, label="odd N f8 half C") == f"maize_gemm_{fmt}_skinny_nt"
