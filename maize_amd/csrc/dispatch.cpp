@@ -437,13 +437,16 @@ bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
     return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
 }
 // K ranges: the smallest power of two that gives the grid at least 3/4 of a workgroup per
-// compute unit, as long as every range keeps a whole number of 32-row blocks and at least 8 of them.
+// compute unit, as long as every range keeps at least 16 blocks of 32 rows.
 uint32_t skinny_ksplit(const Dims& s, uint32_t batch, uint32_t compute_units) {
     const uint64_t slabs = (uint64_t)cdiv(s.n, 256) * batch;
+    const uint32_t nblk = s.k / 32u;
     uint32_t ks = 1;
-    while (ks < 16u && slabs * ks * 4u < (uint64_t)compute_units * 3u && s.k % (64u * ks) == 0 && s.k / (2u * ks) >= 256u)
+    while (ks < 16u && slabs * ks * 4u < (uint64_t)compute_units * 3u && s.k / (2u * ks) >= 256u)
         ks *= 2;
-    return ks;
+    // ... and if that power of two spills into a second round, the largest count that still fits the first
+    if (slabs * ks > compute_units && compute_units / slabs >= 1u) ks = (uint32_t)(compute_units / slabs);
+    return cdiv(nblk, cdiv(nblk, ks));                     // no empty range
 }
 bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
     const Dims s = dims_of(d);
@@ -500,6 +503,9 @@ bool skinny_nt_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Launc
     const uint64_t slabs = (uint64_t)cdiv(s.n, 256) * d.gemm.batch;
     uint32_t ks = 1;
     while (ks < 16u && slabs * ks * 4u < (uint64_t)cus * 3u && nblk / (2u * ks) >= 8u) ks *= 2;
+    // ... and if that power of two spills into a second round, the largest count that still fits the first
+    // (the kernel takes any number of ranges)
+    if (slabs * ks > cus && cus / slabs >= 1u) ks = (uint32_t)(cus / slabs);
     ks = cdiv(nblk, cdiv(nblk, ks));                       // no empty range
     ld->grid[0] = cdiv(s.n, 256);
     ld->grid[1] = ks;

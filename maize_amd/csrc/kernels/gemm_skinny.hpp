@@ -26,7 +26,7 @@
 //     the last one to arrive for a slab adds the partials in split order (deterministic),
 //     rounds once to bf16 (RNE), stores C and resets the ticket counter.
 //
-// Requirements (checked by the dispatcher): layout NN, M <= 16, K % (32 * ksplit) == 0,
+// Requirements (checked by the dispatcher): layout NN, M <= 16, K % 32 == 0 (any number of K ranges),
 // N % 8 == 0, 16-byte aligned operands, every matrix (per batch member) below 2 GiB.
 #pragma once
 #include "common.hpp"
@@ -112,8 +112,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) rd[h][c2] = maps::sk_tr_offset(wave * 2u + c2, h, lane);
 
-    const uint32_t krange = K / ks, k0 = z * krange;
-    const uint32_t nb = krange / KB;                     // blocks of this workgroup
+    // K blocks of this workgroup: [b_first, b_first + nb) of the K / 32 blocks, ceil(blocks / ks) per range (the
+    // dispatcher leaves no range empty); the ring below runs in turns of 8 and blocks past nb read as zeros.
+    const uint32_t nb_all = K / KB, per = (nb_all + ks - 1u) / ks, b_first = z * per;
+    const uint32_t k0 = b_first * KB;
+    const uint32_t nb = b_first < nb_all ? (nb_all - b_first < per ? nb_all - b_first : per) : 0u;
 
     floatx4 acc[2];
     acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};

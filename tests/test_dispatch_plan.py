@@ -133,9 +133,12 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         assert layout == mz.LAYOUT_NN and m <= 16 and n % 8 == 0
         ks = p["ksplit"]
         assert gx == cdiv(n, 256) and gy == ks and 1 <= ks <= 16
-        assert k % (32 * ks) == 0                              # whole 32-row blocks in every range
+        assert k % 32 == 0                                     # whole 32-row blocks
+        nblk = k // 32
+        assert cdiv(nblk, ks) * (ks - 1) < nblk                # no empty range
+        assert ks == 1 or gx * ks * batch <= cus                # K is split only within one round of workgroups
         if ks > 1:
-            assert k // ks // 32 >= 8                          # the 8-slot ring is filled at least once
+            assert nblk // ks >= 8                             # the 8-slot ring is filled at least once
             assert gx * batch <= 16384                         # one ticket counter per (batch member, slab)
             assert p["workspace_bytes"] >= TICKET_BYTES + gx * batch * ks * 16 * 256 * 4
             assert p["workspace_bytes"] < (1 << 31)

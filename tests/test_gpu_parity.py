@@ -292,6 +292,23 @@ def test_config5_batched(ctx, oracle):
 
 # ---- the split-K path of the skinny kernel -------------------------------------------------
 
+@pytest.mark.parametrize("shape,ks", [((16, 10240, 4096), 6), ((16, 17920, 4096), 3), ((16, 14336, 4128), 4), ((5, 9216, 8192), 7)])
+def test_skinny_k_ranges_of_unequal_length(ctx, oracle, shape, ks):
+    """The number of K ranges is whatever fills one round of workgroups (no power of two), so ranges differ in
+    length and the last one may end inside a turn of the ring: 128 blocks in 6 ranges are 22 x 5 + 18."""
+    m, n, k = shape
+    d = mz.gemm_desc(mz.GlobalMatrix(0x10000, m, k), mz.GlobalMatrix(0x4000000, k, n), mz.GlobalMatrix(0x20000000, m, n))
+    p = mz.gemm_plan(d, compute_units=ctx.info()["compute_units"])
+    assert p["kernel"] == "maize_gemm_bf16_skinny_nn"
+    if ctx.info()["compute_units"] == 256:
+        assert p["ksplit"] == ks
+    a, b = mz.gen.normal_bf16(m * k, mz.gen.SEED_A, 1.0), mz.gen.normal_bf16(k * n, mz.gen.SEED_B, 0.02)
+    got = run_gemm(ctx, a, b, m, n, k)
+    s = check_against_oracle(oracle, got, a, b, m, n, k, label=f"skinny {ks} ranges")
+    _say(f"skinny {m}x{n}x{k} in {p['ksplit']} ranges {s}")
+    assert np.array_equal(got, run_gemm(ctx, a, b, m, n, k))                      # the tickets are back at zero, same bits
+
+
 def test_skinny_split_k_repeats_streams_and_batches(ctx, oracle):
     """The M <= 16 kernel combines K ranges through a library-owned workspace whose ticket counters it
     must leave at zero: repeated launches, launches on another stream and batched launches all have to
