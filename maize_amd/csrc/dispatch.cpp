@@ -608,6 +608,15 @@ int kernel_index(const char* name) {
     return -1;
 }
 
+// Whether the kernel's own planner accepts the descriptor.  The packed paths keep one 256 KiB partial tile per work
+// item and address them with 32-bit offsets: a product with more than 16384 items plans to nothing and must fall
+// through to the any-shape kernel instead of being chosen and then refused at launch.
+static bool plan_fits(const KernelInfo& ki, const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
+    LaunchDims ld;
+    std::memset(&ld, 0, sizeof ld);
+    return ki.plan(d, compute_units, &ld);
+}
+
 uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     const Dims s = dims_of(d);
     if (wide_in(d)) {   // fp32 / fp64 operands: one kernel per type and layout, any shape
@@ -643,7 +652,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_packed", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fp = kernel_index(name);
         if (fi >= 0 && !kKernels[fi].supports(d) && fp >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && s.m >= 24u && s.n >= 24u &&
-            kKernels[fp].supports(d))
+            kKernels[fp].supports(d) && plan_fits(kKernels[fp], d, compute_units))
             return (uint32_t)fp;
         return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
     }
@@ -684,7 +693,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
                                               {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nt_packed"}};
     const int pi = kernel_index(kPacked[half_in(d)][s.nt]);
     if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && s.m >= 24u && s.n >= 24u &&
-        kKernels[pi].supports(d))
+        kKernels[pi].supports(d) && plan_fits(kKernels[pi], d, compute_units))
         return (uint32_t)pi;
     return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
 }

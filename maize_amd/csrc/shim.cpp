@@ -325,6 +325,18 @@ int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* d) {
     return maize_hip_gemm_ex_validate(&x);
 }
 
+// The dispatcher's choice for a validated descriptor, checked against the chosen kernel's own limits: the
+// fp32 / fp64 kernels are the only ones for their operand types, and rows of 16 MiB or more are beyond their
+// 32-bit tile offsets -- that is an error, never a launch.
+static int32_t select_checked(const maize_gemm_ex_desc_t& x, uint32_t cus, uint32_t* idx) {
+    *idx = maize::select_kernel(x, cus);
+    const maize::KernelInfo& ki = maize::kernel_at(*idx);
+    if (!ki.supports(x))
+        return fail(MAIZE_ERR_KERNEL, "gemm: no kernel takes this descriptor (%s, the only candidate for operand type %u, does not: "
+                    "M=%u N=%u K=%u lda=%u ldb=%u)", ki.name, x.in_type, x.gemm.c.nrows, x.gemm.c.ncols, x.gemm.a.ncols, x.lda, x.ldb);
+    return MAIZE_OK;
+}
+
 uint32_t maize_hip_kernel_count(void) { return maize::kernel_count(); }
 
 int32_t maize_hip_gemm_ex_tail_rows(const maize_gemm_ex_desc_t* desc, uint32_t compute_units, uint32_t* rows) {
@@ -361,7 +373,10 @@ int32_t maize_hip_gemm_ex_plan(const maize_gemm_ex_desc_t* desc, const char* ker
         if (!maize::kernel_at((uint32_t)idx).supports(*desc))
             return fail(MAIZE_ERR_KERNEL, "gemm_plan: kernel '%s' cannot run this descriptor", kernel);
     } else {
-        idx = (int)maize::select_kernel(*desc, compute_units);
+        uint32_t chosen;
+        rc = select_checked(*desc, compute_units, &chosen);
+        if (rc != MAIZE_OK) return rc;
+        idx = (int)chosen;
     }
     const maize::KernelInfo& ki = maize::kernel_at((uint32_t)idx);
     maize::LaunchDims ld;
@@ -390,7 +405,9 @@ int32_t maize_hip_gemm_select(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, c
     if (!ctx || !name || cap == 0) return fail(MAIZE_ERR_NULL, "gemm_select: NULL argument");
     int32_t rc = maize_hip_gemm_validate(desc);
     if (rc != MAIZE_OK) return rc;
-    const uint32_t idx = maize::select_kernel(widen(*desc), (uint32_t)ctx->prop.multiProcessorCount);
+    uint32_t idx;
+    rc = select_checked(widen(*desc), (uint32_t)ctx->prop.multiProcessorCount, &idx);
+    if (rc != MAIZE_OK) return rc;
     snprintf(name, cap, "%s", maize::kernel_at(idx).name);
     return MAIZE_OK;
 }
@@ -506,11 +523,15 @@ int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* des
             rest.gemm.a.nrows = rest.gemm.c.nrows = desc->gemm.a.nrows - top_rows;
             rest.gemm.a.ptr = (char*)desc->gemm.a.ptr + (uint64_t)top_rows * lda * 2u;
             rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)top_rows * ldc * csz;
-            rc = gemm_launch(ctx, &top, maize::select_kernel(top, cus), stream);
+            uint32_t itop, irest;
+            if ((rc = select_checked(top, cus, &itop)) != MAIZE_OK || (rc = select_checked(rest, cus, &irest)) != MAIZE_OK) return rc;
+            rc = gemm_launch(ctx, &top, itop, stream);
             if (rc != MAIZE_OK) return rc;
-            return gemm_launch(ctx, &rest, maize::select_kernel(rest, cus), stream);
+            return gemm_launch(ctx, &rest, irest, stream);
         }
-        return gemm_launch(ctx, desc, maize::select_kernel(*desc, cus), stream);
+        uint32_t chosen;
+        if ((rc = select_checked(*desc, cus, &chosen)) != MAIZE_OK) return rc;
+        return gemm_launch(ctx, desc, chosen, stream);
     }
     const int idx = maize::kernel_index(kernel);
     if (idx < 0) return fail(MAIZE_ERR_KERNEL, "gemm: no kernel named %s", kernel);

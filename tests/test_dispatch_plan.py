@@ -246,3 +246,68 @@ def test_plan_rejects_bad_arguments():
     with pytest.raises(mz.MaizeError) as e:
         mz.gemm_plan(bad)
     assert e.value.code == _ffi.MAIZE_ERR_SHAPE
+
+
+def ex_desc(m, n, k, layout=mz.LAYOUT_NN, batch=1, in_type=mz.IN_BF16, lda=0, ldb=0, ldc=0, esz=2, csz=2, base=0x10000):
+    a = mz.GlobalMatrix(base, m, k)
+    b = mz.GlobalMatrix(base + (1 << 40), k, n) if layout == mz.LAYOUT_NN else mz.GlobalMatrix(base + (1 << 40), n, k)
+    c = mz.GlobalMatrix(base + (2 << 40), m, n)
+    sa = (m - 1) * (lda or k) + k
+    sb = ((k - 1) * (ldb or n) + n) if layout == mz.LAYOUT_NN else ((n - 1) * (ldb or k) + k)
+    sc = (m - 1) * (ldc or n) + n
+    return mz.gemm_ex_desc(a, b, c, layout=layout, batch=batch, stride_a=sa, stride_b=sb, stride_c=sc, lda=lda, ldb=ldb, ldc=ldc,
+                           in_type=in_type)
+
+
+def test_the_dispatchers_choice_always_plans_when_named():
+    """plan(NULL) names a kernel; plan(that kernel) must then succeed too -- or plan(NULL) itself must be the error.
+    Fuzzed descriptors include rows of 16 MiB and more (beyond the fp32 / fp64 kernels' tile offsets) and products
+    whose packed form has more partial tiles than the workspace can address."""
+    import random
+    rng = random.Random(7)
+    cases = [
+        dict(m=100, n=15, k=5000000, layout=mz.LAYOUT_NT, in_type=mz.IN_F64),
+        dict(m=16, n=4194320, k=1024, layout=mz.LAYOUT_NN, in_type=mz.IN_F32),
+        dict(m=40000, n=40001, k=1024, layout=mz.LAYOUT_NN),
+        dict(m=4096, n=1048576, k=63, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3),
+        dict(m=14336, n=14336, k=24, layout=mz.LAYOUT_NN, batch=32, in_type=mz.IN_E4M3),
+        dict(m=14336, n=14337, k=24, layout=mz.LAYOUT_NN, batch=32),
+    ]
+    dims = [1, 7, 15, 16, 24, 63, 64, 100, 257, 1024, 4099, 40001, 1 << 20, (1 << 22) + 16, 5000000]
+    for _ in range(400):
+        m, n, k = rng.choice(dims), rng.choice(dims), rng.choice(dims)
+        if m * n > 1 << 34 or m * k > 1 << 34 or n * k > 1 << 34:
+            continue
+        cases.append(dict(m=m, n=n, k=k, layout=rng.choice([mz.LAYOUT_NN, mz.LAYOUT_NT]), batch=rng.choice([1, 1, 2, 32]),
+                          in_type=rng.choice([mz.IN_BF16, mz.IN_F16, mz.IN_E4M3, mz.IN_E5M2, mz.IN_F32, mz.IN_F64]),
+                          lda=rng.choice([0, 0, k + 8, k + (1 << 22)])))
+    refused = 0
+    for kw in cases:
+        d = ex_desc(**kw)
+        try:
+            p = mz.gemm_plan(d, compute_units=CUS)
+        except mz.MaizeError as e:
+            if e.code == _ffi.MAIZE_ERR_SHAPE:     # the any-shape kernel's grid: 64 rows per workgroup, at most 65535 of them
+                assert kw["m"] > 64 * 65535 and "wave32" in e.message, (kw, e)
+                continue
+            assert e.code == _ffi.MAIZE_ERR_KERNEL and kw.get("in_type") in (mz.IN_F32, mz.IN_F64), (kw, e)
+            refused += 1
+            continue
+        q = mz.gemm_plan(d, kernel=p["kernel"], compute_units=CUS)     # raises if the kernel refuses or cannot plan
+        assert q["grid"] == p["grid"] and q["workspace_bytes"] == p["workspace_bytes"], (kw, p, q)
+    assert refused >= 2                                          # the two wide cases at the top, at least
+
+
+def test_huge_packed_products_fall_through_to_the_any_shape_kernel():
+    for kw in (dict(m=40000, n=40001, k=1024), dict(m=4096, n=1048576, k=63, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3),
+               dict(m=14336, n=14336, k=24, batch=32, in_type=mz.IN_E4M3)):
+        p = mz.gemm_plan(ex_desc(**kw), compute_units=CUS)
+        assert p["kernel"] == "maize_gemm_bf16_wave32", (kw, p)
+
+
+def test_rows_beyond_the_wide_kernels_offsets_are_an_error_not_a_launch():
+    for kw in (dict(m=100, n=15, k=5000000, layout=mz.LAYOUT_NT, in_type=mz.IN_F64),
+               dict(m=16, n=4194320, k=1024, layout=mz.LAYOUT_NN, in_type=mz.IN_F32)):
+        with pytest.raises(mz.MaizeError) as e:
+            mz.gemm_plan(ex_desc(**kw), compute_units=CUS)
+        assert e.value.code == _ffi.MAIZE_ERR_KERNEL
