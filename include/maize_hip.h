@@ -196,6 +196,19 @@ int32_t maize_hip_embedded_code_object(const void** data, size_t* nbytes);
  * (crates/maize_tile/src/gemm/mod.rs:37-90), adds the C store and the
  * edge-tile handling the reference leaves out (src/main.rs:56-57,71). */
 int32_t maize_hip_gemm_bf16(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream);
+/* The same call for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same validation, same kernel
+ * choice, same launches and bit-identical results as maize_hip_gemm_bf16, but the ticket counters and fp32
+ * partial tiles of the kernels that split K come from a fixed array of MAIZE_NOALLOC_MAX_WORKSPACE_BYTES that
+ * each GPU holds from the first maize_hip_ctx_create on it until the process ends, instead of the per-stream
+ * workspace that maize_hip_gemm_bf16 allocates and grows: this call never calls hipMalloc or hipFree.
+ *  - A descriptor whose plan (maize_hip_gemm_plan: workspace_bytes) needs more than the array holds is refused with
+ *    MAIZE_ERR_ARG before anything is launched; use maize_hip_gemm_bf16 for it.
+ *  - All calls on one GPU share that GPU's array, whatever the context and stream: calls that may overlap in
+ *    time on one GPU race and must be ordered by the caller (one stream, or events between streams). */
+/* 64 KiB of ticket counters + 256 fp32 partial tiles of 256 x 256: one round of split-K work items on 256 compute units. */
+#define MAIZE_NOALLOC_MAX_WORKSPACE_BYTES ((64u << 20) + (64u << 10))
+int32_t maize_hip_gemm_bf16_noalloc(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream);
 /* Same, but with the kernel named by the caller (see maize_hip_kernel_name);
  * fails with MAIZE_ERR_KERNEL if that kernel cannot run the descriptor. */
 int32_t maize_hip_gemm_bf16_with(maize_ctx_t* ctx, const maize_gemm_desc_t* desc,

@@ -15,6 +15,7 @@ EXPORTS = (
     "maize_hip_last_error", "maize_hip_ctx_create", "maize_hip_ctx_destroy", "maize_hip_device_info",
     "maize_hip_module_load", "maize_hip_module_unload", "maize_hip_kernel_get", "maize_hip_kernel_release",
     "maize_hip_launch", "maize_hip_embedded_code_object", "maize_hip_gemm_bf16", "maize_hip_gemm_bf16_with",
+    "maize_hip_gemm_bf16_noalloc",
     "maize_hip_gemm_select", "maize_hip_gemm_plan", "maize_hip_gemm_validate",
     "maize_hip_gemm_bf16_ex", "maize_hip_gemm_ex_validate", "maize_hip_gemm_ex_plan", "maize_hip_gemm_ex_tail_rows", "maize_hip_kernel_count", "maize_hip_kernel_name",
     "maize_hip_kernel_supports", "maize_hip_malloc", "maize_hip_free", "maize_hip_memcpy_h2d",
@@ -33,6 +34,8 @@ MAIZE_ERR_KERNEL = -5
 MAIZE_ERR_NO_DEVICE = -6
 MAIZE_ERR_ARG = -7
 MAIZE_ERR_NOMEM = -8
+
+NOALLOC_MAX_WORKSPACE_BYTES = (64 << 20) + (64 << 10)    # MAIZE_NOALLOC_MAX_WORKSPACE_BYTES
 
 LAYOUT_NN = 0
 LAYOUT_NT = 1
@@ -123,6 +126,7 @@ def lib():
         "maize_hip_embedded_code_object": (i32, [P(vp), P(sz)]),
         "maize_hip_gemm_bf16": (i32, [vp, P(GemmDescT), vp]),
         "maize_hip_gemm_bf16_with": (i32, [vp, P(GemmDescT), C.c_char_p, vp]),
+        "maize_hip_gemm_bf16_noalloc": (i32, [vp, P(GemmDescT), vp]),
         "maize_hip_gemm_select": (i32, [vp, P(GemmDescT), C.c_char_p, sz]),
         "maize_hip_gemm_plan": (i32, [P(GemmDescT), C.c_char_p, u32, P(GemmPlanT)]),
         "maize_hip_gemm_validate": (i32, [P(GemmDescT)]),

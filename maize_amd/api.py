@@ -91,6 +91,11 @@ class Context:
         else:
             check(L.maize_hip_gemm_bf16_with(self._h, C.byref(desc), kernel.encode(), stream))
 
+    def gemm_bf16_noalloc(self, desc, stream=None):
+        """The same launch as ``gemm_bf16(desc)`` without any device allocation: split-K scratch comes from the
+        fixed per-GPU array (maize_hip_gemm_bf16_noalloc); raises MaizeError when the plan needs more than it holds."""
+        check(_ffi.lib().maize_hip_gemm_bf16_noalloc(self._h, C.byref(desc), stream))
+
     def gemm_select(self, desc):
         buf = C.create_string_buffer(128)
         check(_ffi.lib().maize_hip_gemm_select(self._h, C.byref(desc), buf, len(buf)))

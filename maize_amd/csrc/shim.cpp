@@ -15,6 +15,7 @@
 #include <unordered_map>
 
 #include "dispatch.hpp"
+#include "noalloc.hpp"
 
 extern "C" const unsigned char maize_embedded_hsaco[];
 extern "C" const unsigned char maize_embedded_hsaco_end[];
@@ -83,6 +84,9 @@ struct maize_ctx {
     hipFunction_t pack_fn, pack_u8_fn;
     // Split-K scratch, one per stream so that launches on different streams never share it.
     std::unordered_map<void*, maize_workspace> workspaces;
+    // This device's copy of the fixed scratch array behind maize_hip_gemm_bf16_noalloc (looked up at create time).
+    maize_workspace scratch;
+    hipError_t scratch_err;
 };
 struct maize_module {
     maize_ctx* ctx;
@@ -156,6 +160,9 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
         delete ctx;
         return rc;
     }
+    // The device is current here: look up the address of its copy of the no-allocation scratch array.  A failure
+    // only disables maize_hip_gemm_bf16_noalloc (which then reports it).
+    ctx->scratch_err = maize::noalloc_scratch(device, &ctx->scratch.ptr, &ctx->scratch.bytes);
     *out = ctx;
     return MAIZE_OK;
 }
@@ -434,7 +441,10 @@ static int32_t workspace_for(maize_ctx_t* ctx, void* stream, size_t bytes, void*
     return MAIZE_OK;
 }
 
-static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint32_t idx, void* stream) {
+// `fixed`: NULL = the stream's own workspace (allocated or grown here); else the caller's fixed scratch memory, which
+// is used as it is and never grown (a launch that needs more fails).
+static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint32_t idx, void* stream,
+                           const maize_workspace* fixed = nullptr) {
     const maize::KernelInfo& ki = maize::kernel_at(idx);
     const maize_gemm_desc_t* d = &x->gemm;
     maize_gemm_args_t args;
@@ -460,7 +470,13 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
                     d->c.nrows, d->c.ncols, d->a.ncols, d->batch);
     args.ksplit = ld.ksplit;
     args.reserved = ld.split_first;
-    if (ld.workspace_bytes) {
+    if (ld.workspace_bytes && fixed) {
+        if (ld.workspace_bytes > fixed->bytes)
+            return fail(MAIZE_ERR_ARG, "gemm_noalloc: kernel %s needs %zu bytes of scratch for M=%u N=%u K=%u batch=%u, the fixed "
+                        "scratch array holds %zu (use maize_hip_gemm_bf16, which allocates)", ki.name, (size_t)ld.workspace_bytes,
+                        d->c.nrows, d->c.ncols, d->a.ncols, d->batch, fixed->bytes);
+        args.workspace = fixed->ptr;
+    } else if (ld.workspace_bytes) {
         int32_t rc = workspace_for(ctx, stream, ld.workspace_bytes, &args.workspace);
         if (rc != MAIZE_OK) return rc;
     }
@@ -506,7 +522,8 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
                       sizeof args);
 }
 
-int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const char* kernel, void* stream) {
+static int32_t gemm_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const char* kernel, void* stream,
+                       const maize_workspace* fixed) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "gemm: ctx is NULL");
     int32_t rc = maize_hip_gemm_ex_validate(desc);
     if (rc != MAIZE_OK) return rc;
@@ -525,19 +542,33 @@ int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* des
             rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)top_rows * ldc * csz;
             uint32_t itop, irest;
             if ((rc = select_checked(top, cus, &itop)) != MAIZE_OK || (rc = select_checked(rest, cus, &irest)) != MAIZE_OK) return rc;
-            rc = gemm_launch(ctx, &top, itop, stream);
+            rc = gemm_launch(ctx, &top, itop, stream, fixed);
             if (rc != MAIZE_OK) return rc;
-            return gemm_launch(ctx, &rest, irest, stream);
+            return gemm_launch(ctx, &rest, irest, stream, fixed);
         }
         uint32_t chosen;
         if ((rc = select_checked(*desc, cus, &chosen)) != MAIZE_OK) return rc;
-        return gemm_launch(ctx, desc, chosen, stream);
+        return gemm_launch(ctx, desc, chosen, stream, fixed);
     }
     const int idx = maize::kernel_index(kernel);
     if (idx < 0) return fail(MAIZE_ERR_KERNEL, "gemm: no kernel named %s", kernel);
     if (!maize::kernel_at((uint32_t)idx).supports(*desc))
         return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s does not support this descriptor", kernel);
-    return gemm_launch(ctx, desc, (uint32_t)idx, stream);
+    return gemm_launch(ctx, desc, (uint32_t)idx, stream, fixed);
+}
+
+int32_t maize_hip_gemm_bf16_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const char* kernel, void* stream) {
+    return gemm_ex(ctx, desc, kernel, stream, nullptr);
+}
+
+int32_t maize_hip_gemm_bf16_noalloc(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream) {
+    if (!ctx) return fail(MAIZE_ERR_NULL, "gemm_noalloc: ctx is NULL");
+    if (!desc) return fail(MAIZE_ERR_NULL, "gemm_noalloc: descriptor is NULL");
+    if (!ctx->scratch.ptr)
+        return hip_fail(ctx->scratch_err != hipSuccess ? ctx->scratch_err : hipErrorInvalidSymbol,
+                        "gemm_noalloc: the device address of the fixed scratch array (hipGetSymbolAddress)");
+    const maize_gemm_ex_desc_t x = widen(*desc);
+    return gemm_ex(ctx, &x, nullptr, stream, &ctx->scratch);
 }
 
 int32_t maize_hip_gemm_bf16(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream) {

@@ -139,6 +139,8 @@ extern "C" {
                             args: *const c_void, args_bytes: usize) -> i32;
     pub fn maize_hip_embedded_code_object(data: *mut *const c_void, nbytes: *mut usize) -> i32;
     pub fn maize_hip_gemm_bf16(ctx: *mut MaizeCtx, desc: *const MaizeGemmDesc, stream: *mut c_void) -> i32;
+    /// For callers that cannot allocate: split-K scratch from the fixed per-GPU array (64 MiB + 64 KiB), never hipMalloc.
+    pub fn maize_hip_gemm_bf16_noalloc(ctx: *mut MaizeCtx, desc: *const MaizeGemmDesc, stream: *mut c_void) -> i32;
     pub fn maize_hip_gemm_bf16_with(ctx: *mut MaizeCtx, desc: *const MaizeGemmDesc, kernel: *const c_char, stream: *mut c_void) -> i32;
     pub fn maize_hip_gemm_bf16_ex(ctx: *mut MaizeCtx, desc: *const MaizeGemmExDesc, kernel: *const c_char, stream: *mut c_void) -> i32;
     pub fn maize_hip_gemm_validate(desc: *const MaizeGemmDesc) -> i32;
