@@ -100,7 +100,7 @@ def cpu_baseline(cfg, a, b_storage, got, seconds_target=12.0):
                                           nthreads=threads, elem=elem)
         r = min(rows, 64)
         parity = pyoracle.compare(got[:r * n], ref[:r], f64[:r], ab, k, coeff=coeff)
-        parity = {key: parity[key] for key in ("n", "max_ulp", "n_gt1ulp", "n_fail", "max_err_over_abs")}
+        parity = {key: parity[key] for key in ("n", "max_ulp", "n_gt1ulp", "n_fail", "max_floor_ratio", "max_err_over_abs")}
     return out, parity
 
 

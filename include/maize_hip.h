@@ -28,6 +28,10 @@
  *    stream.  maize_hip_gemm_plan reports the bytes.  The workspace is released
  *    by maize_hip_stream_destroy for streams made by maize_hip_stream_create,
  *    and by maize_hip_ctx_destroy for every other stream it was used with.
+ *  - Arithmetic: products of bf16 operands are exact, sums are kept in fp32 (one rounding per 16- or 32-deep matrix
+ *    instruction), C is rounded once to bf16 (nearest even).  IEEE special values follow through: NaN and +-Inf in A or
+ *    B give NaN / Inf exactly where an fp64 evaluation does (the zero fill of the M, N and K edges never meets a real
+ *    operand in a stored element), and subnormal operands and results are kept, not flushed.
  *  - All matrices are row-major with leading dimension == ncols, as in the
  *    reference (crates/maize_tile/src/gmem/row_panel.rs:55,
  *    crates/maize_tile/src/gmem/col_panel.rs:108).  BF16 is a 2-byte,

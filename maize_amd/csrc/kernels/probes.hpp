@@ -37,6 +37,24 @@ extern "C" __global__ __launch_bounds__(64) void maize_probe_mfma_16x16x32(
     for (int v = 0; v < 4; ++v) d[lane * 4 + v] = acc[v];
 }
 
+// The same instruction with the wave's MODE.FP_DENORM field (bits 4..7 of the MODE register: 2 bits for fp32,
+// 2 for fp64 / fp16) set to `denorm` first: shows whether the matrix core's handling of subnormal bf16 inputs and
+// subnormal fp32 results follows that field or is fixed.
+extern "C" __global__ __launch_bounds__(64) void maize_probe_mfma_16x16x32_denorm(
+    const uint16_t* a, const uint16_t* b, float* d, uint32_t denorm) {
+    const uint32_t lane = threadIdx.x;
+    bf16x8 fa, fb;
+    for (int e = 0; e < 8; ++e) {
+        fa[e] = __builtin_bit_cast(__bf16, a[lane * 8 + e]);
+        fb[e] = __builtin_bit_cast(__bf16, b[lane * 8 + e]);
+    }
+    floatx4 acc = {0, 0, 0, 0};
+    __builtin_amdgcn_s_setreg(1 | (4 << 6) | (3 << 11), denorm & 15u);   // hwreg(HW_REG_MODE, offset 4, width 4)
+    asm volatile("s_nop 4" ::: "memory");
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\ts_nop 7\n\ts_nop 7" : "+v"(acc) : "v"(fa), "v"(fb));
+    for (int v = 0; v < 4; ++v) d[lane * 4 + v] = acc[v];
+}
+
 // LDS transpose read (ds_read_b64_tr_b16).  LDS is filled with lds_init
 // (n_init u16 values); lane l reads at byte offset byte_off[l]; out receives
 // 4 u16 per lane.

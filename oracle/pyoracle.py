@@ -270,12 +270,18 @@ def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16, coeff=None):
     with np.errstate(invalid="ignore", over="ignore"):
         err = np.abs(gotf - f64)
         half_ulp = np.abs(gotf) * (2.0 ** -11 if elem == F16 else 2.0 ** -8)
-        floor = (floor_coeff(k) if coeff is None else coeff) * ab + half_ulp
+        # results in the subnormal range: the spacing no longer shrinks with the value (bf16: 2^-133, half: 2^-24),
+        # and each fp32 rounding of the accumulation is at least half of fp32's smallest step (2^-149)
+        half_ulp = np.maximum(half_ulp, 2.0 ** -25 if elem == F16 else 2.0 ** -134)
+        floor = (floor_coeff(k) if coeff is None else coeff) * ab + (k / 16.0 + 2.0) * 2.0 ** -150 + half_ulp
         strict_bad = ulp > 1
         bad = strict_bad & ~(err <= floor)
         rel = np.where(ab > 0, err / np.where(ab > 0, ab, 1.0), 0.0)
+        # how much of the floor the elements beyond 1 ULP use (1.0 = at the bar)
+        ratio = np.where(strict_bad & np.isfinite(err) & (floor > 0), err / np.where(floor > 0, floor, 1.0), 0.0)
     worst = int(np.argmax(ulp)) if ulp.size else -1
     return {
+        "max_floor_ratio": float(ratio.max()) if ratio.size else 0.0,
         "n": int(got.size),
         "max_ulp": int(ulp.max()) if ulp.size else 0,
         "n_gt1ulp": int(strict_bad.sum()),
