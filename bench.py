@@ -164,19 +164,177 @@ def copy_calibration(steps, warmup):
     ctx.close()
 
 
+class PowerSampler:
+    """Board power from sysfs (hwmon power1_input or power1_average, microwatts), sampled every 20 ms on a thread
+    while the GPU works.  No GPU runtime call is made here."""
+
+    def __init__(self):
+        import glob
+        cands = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")) or \
+            sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"))
+        self.path = cands[0] if cands else None
+        self.samples = []
+
+    def read(self):
+        try:
+            with open(self.path) as f:
+                return float(f.read().strip()) / 1e6
+        except Exception:
+            return None
+
+    def __enter__(self):
+        import threading
+        self._stop = False
+
+        def loop():
+            while not self._stop:
+                w = self.read()
+                if w is not None:
+                    self.samples.append((time.time(), w))
+                time.sleep(0.02)
+        self._t = threading.Thread(target=loop, daemon=True)
+        self._t.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        self._t.join()
+
+    def mean_between(self, t0, t1):
+        w = [x for t, x in self.samples if t0 <= t <= t1]
+        return sum(w) / len(w) if w else None
+
+
+def energy_vendor_child(seconds):
+    """Child process of --config energy --vendor: times torch.matmul (the vendor library) on the 4096^3 workload, NN
+    and NT, and prints one JSON line per row with wall-clock stamps for the parent's power samples."""
+    import torch
+    n = 4096
+    import maize_amd as mz
+    a = mz.gen.uniform_bf16(n * n, mz.gen.SEED_A)
+    b = mz.gen.uniform_bf16(n * n, mz.gen.SEED_B)
+    ta = torch.from_numpy(a.view(np.int16).reshape(n, n)).cuda().view(torch.bfloat16)
+    tb = torch.from_numpy(b.view(np.int16).reshape(n, n)).cuda().view(torch.bfloat16)
+    tbt = tb.t().contiguous()
+    tc = torch.empty(n, n, dtype=torch.bfloat16, device="cuda")
+    for label, fn in (("vendor library NN (torch.matmul(A, B))", lambda: torch.matmul(ta, tb, out=tc)),
+                      ("vendor library NT (torch.matmul(A, Bt.T))", lambda: torch.matmul(ta, tbt.t(), out=tc))):
+        t0, us = time.time(), 0.0
+        while time.time() - t0 < seconds:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(50):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / 50 * 1e3
+        print(json.dumps({"kernel": label, "us": us, "t0": t0, "t1": time.time()}), flush=True)
+        time.sleep(0.7)
+
+
+def energy_table(seconds, vendor):
+    """Power x time per launch for the 4096^3 workload: this library's NN and NT kernels, register-only loops of
+    the two bf16 matrix instructions doing the same multiply-adds (zeros and random operands), and -- with
+    --vendor -- the vendor library's kernels through torch.matmul.  Each row runs back to back for `seconds`;
+    power is averaged over the last 60 % of that time, when clocks and power have settled.  One JSON line."""
+    import ctypes as C
+    import maize_amd as mz
+
+    class LoopArgs(C.Structure):
+        _fields_ = [("out", C.c_void_p), ("iters", C.c_uint32), ("zero", C.c_uint32)]
+
+    n = 4096
+    rows = []
+    sampler = PowerSampler()
+    if sampler.path is None:
+        print("bench.py --config energy: no hwmon power file under /sys/class/drm", file=sys.stderr)
+    if vendor:
+        # The vendor library's kernels, for comparison only: torch.matmul in a child process (its HIP runtime and this
+        # library's do not share a process), run before this process touches the GPU; power is sampled here.
+        import subprocess
+        with sampler:
+            out = subprocess.run([sys.executable, os.path.abspath(__file__), "--config", "energy-vendor-child", "--seconds", str(seconds)],
+                                 capture_output=True, text=True, timeout=120)
+        if out.returncode != 0:
+            print("bench.py --config energy: the vendor rows failed:\n" + out.stderr[-2000:], file=sys.stderr)
+        for line in out.stdout.splitlines():
+            if line.startswith("{"):
+                r = json.loads(line)
+                watts = sampler.mean_between(r["t0"] + 0.4 * (r["t1"] - r["t0"]), r["t1"])
+                rows.append({"kernel": r["kernel"], "us_per_launch": r["us"], "watts": watts,
+                             "mj_per_launch": None if watts is None else watts * r["us"] / 1e3})
+                print(f"energy: {r['kernel']}: {r['us']:.1f} us, {watts} W", file=sys.stderr, flush=True)
+        sampler.samples = []
+    ctx = mz.Context(0)
+    info = ctx.info()
+    a = mz.gen.uniform_bf16(n * n, mz.gen.SEED_A)
+    b = mz.gen.uniform_bf16(n * n, mz.gen.SEED_B)
+    da, db, dbt, dc, dz = ctx.upload(a), ctx.upload(b), ctx.upload(np.ascontiguousarray(b.reshape(n, n).T)), ctx.malloc(2 * n * n), ctx.malloc(2 * n * n)
+    dz.fill(0)
+    out = ctx.malloc(4096)
+    time.sleep(1.0)
+    idle = sampler.read()
+
+    def run(label, launch, batch=50):
+        ev0, ev1 = ctx.event(), ctx.event()
+        with sampler:
+            t_begin = time.time()
+            launches, ev_ms = 0, 0.0
+            while time.time() - t_begin < seconds:
+                ev0.record(None)
+                for _ in range(batch):
+                    launch()
+                ev1.record(None)
+                ctx.sync()
+                ev_ms, launches = ev0.elapsed_ms(ev1), launches + batch       # the last batch: settled clocks
+            t_end = time.time()
+        us = ev_ms / batch * 1e3
+        watts = sampler.mean_between(t_begin + 0.4 * (t_end - t_begin), t_end)
+        rows.append({"kernel": label, "us_per_launch": us, "watts": watts, "mj_per_launch": None if watts is None else watts * us / 1e3,
+                     "launches": launches})
+        print(f"energy: {label}: {us:.1f} us, {watts} W", file=sys.stderr, flush=True)
+        ev0.destroy(); ev1.destroy()
+        time.sleep(0.7)                                           # let the board cool to the same starting point
+
+    def gemm(dA, dB, nt):
+        desc = mz.gemm_desc(mz.Matrix(dA, n, n), mz.Matrix(dB, n, n), mz.Matrix(dc, n, n), layout=nt)
+        return lambda: ctx.gemm_bf16(desc)
+
+    run("maize_gemm_bf16_mt256_nn, uniform[-1,1) operands", gemm(da, db, 0))
+    run("maize_gemm_bf16_mt256_nt, uniform[-1,1) operands", gemm(da, dbt, 1))
+    run("maize_gemm_bf16_mt256_nn, all-zero operands", gemm(dz, dz, 0))
+    for name in ("maize_probe_mfma_loop_16x16x32", "maize_probe_mfma_loop_32x32x16"):
+        k = mz.new_hip_kernel(name).with_launch_bounds_1d(256).finalize().compile(mz.Gfx.Gfx950, ctx)
+        for zero in (0, 1):
+            args = LoopArgs(out.ptr, 512, zero)                  # 256 workgroups x 4 waves x 512 rounds x 131072 MACs = 4096^3
+            run(f"{name} (registers only, same multiply-adds), {'zeros' if zero else 'random operands'}",
+                lambda: k.launch((256, 1, 1), args))
+        k.release()
+    flop = 2.0 * n ** 3
+    for r in rows:
+        r["frac_of_bf16_peak"] = flop / (r["us_per_launch"] * 1e-6) / 1e12 / PEAK_BF16_TFLOPS
+    print(json.dumps({"metric": "energy per 4096^3 launch", "unit": "mJ", "idle_watts": idle, "power_file": sampler.path,
+                      "seconds_per_row": seconds, "device": info, "rows": rows}), flush=True)
+    for x in (da, db, dbt, dc, dz, out):
+        x.free()
+    ctx.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--config", default=None, choices=sorted(CONFIGS) + ["copy"],
+    ap.add_argument("--config", default=None, choices=sorted(CONFIGS) + ["copy", "energy", "energy-vendor-child"],
                     help="cfg1..cfg5: a benchmark configuration; f8, f8s: 4096^3 and 16x14336x4096 on E4M3 operands; f32, f64: 4096^3 on fp32 / fp64 operands; copy: the 256 MiB copy "
-                         "used to scale HBM counters")
+                         "used to scale HBM counters; energy: board power x time per 4096^3 launch for this library's kernels and register-only MFMA loops")
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--others", action=argparse.BooleanOptionalAction, default=None,
                     help="also measure the other benchmark configurations (shorter runs) and report them under "
                          "\"other_configs\" (default: on when no --config is given)")
+    ap.add_argument("--seconds", type=float, default=2.5, help="--config energy: how long each row runs back to back")
+    ap.add_argument("--vendor", action="store_true", help="--config energy: add the vendor library's kernels (needs torch)")
     ap.add_argument("--rotate", type=int, default=0,
                     help="number of distinct operand sets cycled through (0: enough to exceed the 256 MiB "
                          "last-level cache for the HBM-bound config, 1 otherwise)")
@@ -191,6 +349,12 @@ def main():
     args.config = args.config or "cfg1"
     if args.config == "copy":
         copy_calibration(args.steps, args.warmup)
+        return
+    if args.config == "energy-vendor-child":
+        energy_vendor_child(args.seconds)
+        return
+    if args.config == "energy":
+        energy_table(args.seconds, args.vendor)
         return
     import maize_amd as mz
     ctx = mz.Context(0)

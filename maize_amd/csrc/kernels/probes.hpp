@@ -55,6 +55,59 @@ extern "C" __global__ __launch_bounds__(64) void maize_probe_mfma_16x16x32_denor
     for (int v = 0; v < 4; ++v) d[lane * 4 + v] = acc[v];
 }
 
+// Register-only loops of the two bf16 matrix instructions: no loads, no LDS, accumulators pinned in AccVGPRs by
+// the "+a" constraints, 16 (4) independent accumulators so that no MFMA waits for its predecessor.  One round is
+// 131072 multiply-adds per wave either way.  With `iters` = 512 and a grid of 256 workgroups of 4 waves a launch does
+// exactly the multiply-adds of a 4096^3 product: what the matrix pipe alone costs in time and energy, for operands of
+// zeros (zero = 1) or of pseudo-random values in [-1, 1) (zero = 0) -- the number every tiled kernel is measured against.
+struct MfmaLoopArgs { float* out; uint32_t iters; uint32_t zero; };
+__device__ __forceinline__ bf16x8 probe_operand(uint32_t salt, uint32_t zero) {
+    bf16x8 r;
+    for (int e = 0; e < 8; ++e) {
+        uint32_t h = threadIdx.x * 64 + salt * 8 + e + blockIdx.x * 77777;
+        h ^= h >> 16; h *= 0x7feb352dU; h ^= h >> 15; h *= 0x846ca68bU; h ^= h >> 16;
+        r[e] = zero ? (__bf16)0.0f : (__bf16)((float)(int)(h & 0xFFFF) / 32768.0f - 1.0f);
+    }
+    return r;
+}
+extern "C" __global__ __launch_bounds__(256) void maize_probe_mfma_loop_16x16x32(MfmaLoopArgs p) {
+    floatx4 c0 = {}, c1 = {}, c2 = {}, c3 = {}, c4 = {}, c5 = {}, c6 = {}, c7 = {}, c8 = {}, c9 = {}, c10 = {}, c11 = {}, c12 = {}, c13 = {}, c14 = {}, c15 = {};
+    bf16x8 a0 = probe_operand(0, p.zero), a1 = probe_operand(1, p.zero), a2 = probe_operand(2, p.zero), a3 = probe_operand(3, p.zero);
+    bf16x8 b0 = probe_operand(4, p.zero), b1 = probe_operand(5, p.zero), b2 = probe_operand(6, p.zero), b3 = probe_operand(7, p.zero);
+    for (uint32_t it = 0; it < p.iters; ++it) {
+        asm volatile(
+            "v_mfma_f32_16x16x32_bf16 %0, %16, %20, %0\n\tv_mfma_f32_16x16x32_bf16 %1, %16, %21, %1\n\t"
+            "v_mfma_f32_16x16x32_bf16 %2, %16, %22, %2\n\tv_mfma_f32_16x16x32_bf16 %3, %16, %23, %3\n\t"
+            "v_mfma_f32_16x16x32_bf16 %4, %17, %20, %4\n\tv_mfma_f32_16x16x32_bf16 %5, %17, %21, %5\n\t"
+            "v_mfma_f32_16x16x32_bf16 %6, %17, %22, %6\n\tv_mfma_f32_16x16x32_bf16 %7, %17, %23, %7\n\t"
+            "v_mfma_f32_16x16x32_bf16 %8, %18, %20, %8\n\tv_mfma_f32_16x16x32_bf16 %9, %18, %21, %9\n\t"
+            "v_mfma_f32_16x16x32_bf16 %10, %18, %22, %10\n\tv_mfma_f32_16x16x32_bf16 %11, %18, %23, %11\n\t"
+            "v_mfma_f32_16x16x32_bf16 %12, %19, %20, %12\n\tv_mfma_f32_16x16x32_bf16 %13, %19, %21, %13\n\t"
+            "v_mfma_f32_16x16x32_bf16 %14, %19, %22, %14\n\tv_mfma_f32_16x16x32_bf16 %15, %19, %23, %15"
+            : "+a"(c0), "+a"(c1), "+a"(c2), "+a"(c3), "+a"(c4), "+a"(c5), "+a"(c6), "+a"(c7), "+a"(c8), "+a"(c9), "+a"(c10), "+a"(c11),
+              "+a"(c12), "+a"(c13), "+a"(c14), "+a"(c15)
+            : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b0), "v"(b1), "v"(b2), "v"(b3));
+    }
+    floatx4 s = c0 + c1 + c2 + c3 + c4 + c5 + c6 + c7 + c8 + c9 + c10 + c11 + c12 + c13 + c14 + c15;
+    if (s[0] + s[1] + s[2] + s[3] == 12345.f) p.out[threadIdx.x] = s[0];
+}
+extern "C" __global__ __launch_bounds__(256) void maize_probe_mfma_loop_32x32x16(MfmaLoopArgs p) {
+    floatx16 c0 = {}, c1 = {}, c2 = {}, c3 = {};
+    bf16x8 a0 = probe_operand(0, p.zero), a1 = probe_operand(1, p.zero), a2 = probe_operand(2, p.zero), a3 = probe_operand(3, p.zero);
+    bf16x8 b0 = probe_operand(4, p.zero), b1 = probe_operand(5, p.zero), b2 = probe_operand(6, p.zero), b3 = probe_operand(7, p.zero);
+    for (uint32_t it = 0; it < p.iters; ++it) {
+        asm volatile(
+            "v_mfma_f32_32x32x16_bf16 %0, %4, %8, %0\n\tv_mfma_f32_32x32x16_bf16 %1, %4, %9, %1\n\t"
+            "v_mfma_f32_32x32x16_bf16 %2, %5, %8, %2\n\tv_mfma_f32_32x32x16_bf16 %3, %5, %9, %3\n\t"
+            "v_mfma_f32_32x32x16_bf16 %0, %6, %10, %0\n\tv_mfma_f32_32x32x16_bf16 %1, %6, %11, %1\n\t"
+            "v_mfma_f32_32x32x16_bf16 %2, %7, %10, %2\n\tv_mfma_f32_32x32x16_bf16 %3, %7, %11, %3"
+            : "+a"(c0), "+a"(c1), "+a"(c2), "+a"(c3)
+            : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b0), "v"(b1), "v"(b2), "v"(b3));
+    }
+    floatx16 s = c0 + c1 + c2 + c3;
+    if (s[0] + s[5] == 12345.f) p.out[threadIdx.x] = s[0];
+}
+
 // LDS transpose read (ds_read_b64_tr_b16).  LDS is filled with lds_init
 // (n_init u16 values); lane l reads at byte offset byte_off[l]; out receives
 // 4 u16 per lane.
