@@ -331,5 +331,10 @@ class LoadedKernel:
         self.mod.unload()
 
 
-def new_hip_kernel(name, code_object=None):
+def new_hip_kernel(name=None, code_object=None):
+    """With a name: a kernel of a code object, to be bound and launched by hand.  Without: the start of a trace in
+    the reference's tile vocabulary (maize_amd.tile), which finalize().compile() resolves to a GEMM launch."""
+    if name is None:
+        from .tile import TracedKernel
+        return TracedKernel()
     return HipKernel(name, code_object)
