@@ -19,6 +19,7 @@
 #include <cstring>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -124,6 +125,188 @@ inline void gemm_smem_multibuffer(Ctx& ctx, const Matrix& a, const Matrix& b, co
 inline void gemm_smem_multibuffer(Ctx& ctx, const maize_gemm_ex_desc_t& x, void* stream = nullptr, const char* kernel = nullptr) {
     check(maize_hip_gemm_bf16_ex(ctx.handle(), &x, kernel, stream));
 }
+
+// ---- the tile vocabulary ---------------------------------------------------------------------------
+// The reference's caller *traces* its kernel (src/main.rs:31-90): shared-memory ring, Matrix, row / column panels over
+// groups of blocks, sm80_gemm_smem_multibuffer per panel pair.  Here the kernels are hand-written, so the same calls
+// *describe* one: small host-side types with the reference's names, checked against what the kernels implement --
+// at compile time where the reference's trait bounds would refuse (tile types, K tile, ring depth), by exceptions
+// where it panics at trace time -- and resolved by finalize().compile() to the launch maize_hip_gemm_bf16_ex makes.
+//
+//   Tile<T>, TilePair<TA, TB>, tile types    crates/maize_tile/src/lib.rs:87-108,231-265, pair.rs:3-8
+//   RowPanel / ColPanel / PanelIterLooper    crates/maize_tile/src/gmem/row_panel.rs:10-161, col_panel.rs:10-158
+//   BlockX / BlockY / Wave (was Warp)        crates/maize_tile/src/group/by_block.rs:10-75, warp.rs:10-37
+//   SyncMMAOp catalogue                      crates/maize_tile/src/mma/mod.rs:19-99, sm80.rs, sm80_derived.rs:5-28, sm89.rs
+//   gemm_smem_multibuffer(mma, KTile, ...)   crates/maize_tile/src/gemm/mod.rs:37-90
+enum class Swizzle { None, KC16, KN32 };   // KC16: 128-byte rows along K, 16-byte chunk ^ ((row >> 1) & 7); KN32: row-major K x N, 32-byte granule ^ (row % 4 + 4 bit3(row))
+#define MAIZE_TILE_TY(name, rows, cols, bytes, swz) \
+    struct name { static constexpr uint32_t ROWS = rows, COLS = cols, ELEM_BYTES = bytes; static constexpr Swizzle SWIZZLE = swz; };
+MAIZE_TILE_TY(BF16_16x16, 16, 16, 2, Swizzle::None)      // the reference's tile (lib.rs:98-108); no kernel here takes it
+MAIZE_TILE_TY(BF16_256x64, 256, 64, 2, Swizzle::KC16)    // A stage; B stage when B is stored N x K
+MAIZE_TILE_TY(BF16_64x256, 64, 256, 2, Swizzle::KN32)    // B stage of a row-major K x N B
+MAIZE_TILE_TY(F16_256x64, 256, 64, 2, Swizzle::KC16)
+MAIZE_TILE_TY(F16_64x256, 64, 256, 2, Swizzle::KN32)
+MAIZE_TILE_TY(F8_256x128, 256, 128, 1, Swizzle::KC16)    // 8-bit operands: 128 elements of K per 128-byte row
+#undef MAIZE_TILE_TY
+template <class T> struct Tile { using Ty = T; static constexpr size_t SIZE = (size_t)T::ROWS * T::COLS * T::ELEM_BYTES; };
+template <class TA, class TB> struct TilePair { using A = TA; using B = TB; static constexpr size_t SIZE = TA::SIZE + TB::SIZE; };
+template <class Pair, size_t PIPE> struct SharedRing {   // [TilePair; PIPE] in LDS (src/main.rs:42-44)
+    using PairT = Pair;
+    static constexpr size_t DEPTH = PIPE, SIZE = Pair::SIZE * PIPE;
+    static_assert(SIZE <= 160 * 1024, "a compute unit has 160 KiB of LDS");
+    uint32_t align;
+};
+
+// The MMA catalogue: one matrix instruction as an operation on wave fragments, D = A.B + C.  FRAG_*: 32-bit registers
+// per lane; K_TILE: elements of K per ring stage of the kernels built on it.
+enum class Family { MT256, WAVE32, MT128 };
+#define MAIZE_MMA(name, m, n, k, in, fa, fb, fc, mnem, fam, ktile) \
+    struct name { static constexpr uint32_t M = m, N = n, K = k, FRAG_A = fa, FRAG_B = fb, FRAG_C = fc, K_TILE = ktile; \
+                  static constexpr maize_in_type_t IN_TYPE = in; static constexpr Family FAMILY = fam; \
+                  static constexpr const char* NAME = #name; static constexpr const char* MNEMONIC = mnem; };
+MAIZE_MMA(Gfx950MfmaBf16F32_16x16x32, 16, 16, 32, MAIZE_IN_BF16, 4, 4, 4, "v_mfma_f32_16x16x32_bf16", Family::MT256, 64)
+MAIZE_MMA(Gfx950MfmaBf16F32_32x32x16, 32, 32, 16, MAIZE_IN_BF16, 4, 4, 16, "v_mfma_f32_32x32x16_bf16", Family::WAVE32, 16)
+MAIZE_MMA(Gfx950MfmaF16F32_16x16x32, 16, 16, 32, MAIZE_IN_F16, 4, 4, 4, "v_mfma_f32_16x16x32_f16", Family::MT256, 64)
+MAIZE_MMA(Gfx950MfmaE4M3F32_16x16x128, 16, 16, 128, MAIZE_IN_E4M3, 8, 8, 4, "v_mfma_f32_16x16x128_f8f6f4", Family::MT256, 128)
+MAIZE_MMA(Gfx950MfmaE5M2F32_16x16x128, 16, 16, 128, MAIZE_IN_E5M2, 8, 8, 4, "v_mfma_f32_16x16x128_f8f6f4", Family::MT256, 128)
+MAIZE_MMA(Gfx950MfmaE4M3E5M2F32_16x16x128, 16, 16, 128, MAIZE_IN_E4M3_E5M2, 8, 8, 4, "v_mfma_f32_16x16x128_f8f6f4", Family::MT256, 128)
+MAIZE_MMA(Gfx950MfmaE5M2E4M3F32_16x16x128, 16, 16, 128, MAIZE_IN_E5M2_E4M3, 8, 8, 4, "v_mfma_f32_16x16x128_f8f6f4", Family::MT256, 128)
+MAIZE_MMA(Gfx950MfmaF32F32_16x16x4, 16, 16, 4, MAIZE_IN_F32, 1, 1, 4, "v_mfma_f32_16x16x4_f32", Family::MT128, 32)
+MAIZE_MMA(Gfx950MfmaF64F64_16x16x4, 16, 16, 4, MAIZE_IN_F64, 2, 2, 8, "v_mfma_f64_16x16x4_f64", Family::MT128, 16)
+#undef MAIZE_MMA
+
+class TracedKernel;
+// Groups (Group, group/mod.rs:19-29).  BlockX shares out row panels, BlockY column panels; both are realised by one
+// persistent 1-D grid whose workgroup g computes tiles g, g + grid, ... of an XCD-aware list (walk()).
+inline uint32_t xcd_run(uint32_t pid, uint32_t total) {
+    const uint32_t per = (total + 7u) / 8u, tall = (total % 8u) ? (total % 8u) : 8u, xcd = pid % 8u, local = pid / 8u;
+    return xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1u) + local;
+}
+inline std::pair<uint32_t, uint32_t> tile_of(uint32_t idx, uint32_t tm, uint32_t tn, uint32_t group_rows = 4) {
+    const uint32_t first = idx / (group_rows * tn) * group_rows, gsz = (tm - first) < group_rows ? (tm - first) : group_rows;
+    const uint32_t in = idx % (group_rows * tn);
+    return {first + in % gsz, in / gsz};
+}
+template <int AXIS> struct Block {
+    TracedKernel* kernel;
+    // Panel index of every tile workgroup `pid` of a grid of `grid` computes, and the number of panels (index_size()).
+    std::pair<std::vector<uint32_t>, uint32_t> index_size(uint32_t pid, uint32_t tm, uint32_t tn, uint32_t grid) const {
+        std::vector<uint32_t> walk;
+        for (uint32_t i = pid; i < tm * tn; i += grid) { const auto t = tile_of(xcd_run(i, tm * tn), tm, tn); walk.push_back(AXIS == 0 ? t.first : t.second); }
+        return {walk, AXIS == 0 ? tm : tn};
+    }
+};
+using BlockX = Block<0>;
+using BlockY = Block<1>;
+struct Wave {                              // the 64-lane wavefront: the group that issues one cooperative copy (was Warp, 32 lanes)
+    TracedKernel* kernel;
+    static constexpr uint32_t const_size() { return 64; }
+};
+
+// Panels: N rows (columns) x the whole other extent.  `extent` is the window: N for bulk panels, the remainder for the
+// ragged epilogue panel, which the reference's caller throws away (src/main.rs:56-57) and the kernels here compute.
+template <uint32_t N> struct RowPanel { Matrix matrix; uint32_t extent; bool ragged; static constexpr uint32_t WINDOW = N;
+    uint32_t row_size() const { return extent; } uint32_t col_size() const { return matrix.g.ncols; } };
+template <uint32_t N> struct ColPanel { Matrix matrix; uint32_t extent; bool ragged; static constexpr uint32_t WINDOW = N;
+    uint32_t row_size() const { return matrix.g.nrows; } uint32_t col_size() const { return extent; } };
+template <class Panel> struct PanelIterLooper {
+    Panel panel; uint32_t count;
+    template <class F> void for_every_value(F&& body) const { body(panel); }   // once, like the reference's looper at trace time
+};
+template <uint32_t N, class Group>
+std::pair<PanelIterLooper<RowPanel<N>>, RowPanel<N>> collective_aligned_row_panel_iter(const Matrix& m, Group) {
+    return {PanelIterLooper<RowPanel<N>>{RowPanel<N>{m, N, false}, m.g.nrows / N}, RowPanel<N>{m, m.g.nrows % N, true}};
+}
+template <uint32_t N, class Group>
+std::pair<PanelIterLooper<ColPanel<N>>, ColPanel<N>> collective_aligned_col_panel_iter(const Matrix& m, Group) {
+    return {PanelIterLooper<ColPanel<N>>{ColPanel<N>{m, N, false}, m.g.ncols / N}, ColPanel<N>{m, m.g.ncols % N, true}};
+}
+
+struct TracedOp { Matrix a, b, c; bool nt; maize_in_type_t in; Family family; bool stored; maize_out_type_t out; float alpha, beta; };
+class LoadedGemm {
+  public:
+    LoadedGemm(Ctx& ctx, const maize_gemm_ex_desc_t& x, const char* forced) : ctx_(ctx), x_(x), forced_(forced) {
+        int32_t cus = 256;
+        maize_device_info_t info;
+        if (maize_hip_device_info(ctx.handle(), &info) == MAIZE_OK) cus = (int32_t)info.compute_units;
+        check(maize_hip_gemm_ex_plan(&x_, forced_, (uint32_t)cus, &plan_));
+    }
+    std::string kernel_name() const { return plan_.kernel; }
+    const maize_gemm_plan_t& plan() const { return plan_; }
+    void launch(void* stream = nullptr) { check(maize_hip_gemm_bf16_ex(ctx_.handle(), &x_, forced_, stream)); }
+  private:
+    Ctx& ctx_; maize_gemm_ex_desc_t x_; const char* forced_; maize_gemm_plan_t plan_;
+};
+class PreLoadGemm {
+  public:
+    explicit PreLoadGemm(const TracedOp& op) : op_(op) {}
+    LoadedGemm compile(Gfx target, Ctx& ctx) const {
+        if (target != Gfx::Gfx950) throw std::invalid_argument("only Gfx::Gfx950 code is carried");
+        maize_gemm_desc_t d;
+        std::memset(&d, 0, sizeof d);
+        d.a = op_.a.g.realize(); d.b = op_.b.g.realize(); d.c = op_.c.g.realize();
+        d.layout = op_.nt ? MAIZE_LAYOUT_NT : MAIZE_LAYOUT_NN; d.batch = 1;
+        maize_gemm_ex_desc_t x{};
+        x.gemm = d; x.out_type = op_.out; x.alpha = op_.alpha; x.beta = op_.beta; x.in_type = op_.in;
+        return LoadedGemm(ctx, x, op_.family == Family::WAVE32 ? "maize_gemm_bf16_wave32" : nullptr);
+    }
+  private:
+    TracedOp op_;
+};
+class TracedKernel {                       // new_hip_kernel() without a name: the kernel being described
+  public:
+    TracedKernel& with_launch_bounds_2d(std::pair<uint32_t, uint32_t> xy) {
+        const uint64_t t = (uint64_t)xy.first * xy.second;
+        if (t != 256 && t != 512) throw std::invalid_argument("the GEMM kernels run 4 wavefronts (256 threads; the skinny kernels 8)");
+        bounds_ = true;
+        return *this;
+    }
+    template <class Pair, size_t PIPE> SharedRing<Pair, PIPE> alloc_aligned_shared(uint32_t align) { return SharedRing<Pair, PIPE>{align}; }
+    TracedKernel* cx() { return this; }
+    PreLoadGemm finalize() const {
+        if (!bounds_) throw std::invalid_argument("launch bounds not set");
+        if (ops_.size() != 1 || !ops_[0].stored) throw std::invalid_argument("the trace must hold exactly one stored GEMM");
+        return PreLoadGemm(ops_[0]);
+    }
+    std::vector<TracedOp> ops_;
+  private:
+    bool bounds_ = false;
+};
+class Accum {                              // the accumulator fragments of one panel pair; store() names the C they go to
+  public:
+    Accum(TracedKernel* k, const TracedOp& op) : k_(k), op_(op) {}
+    void store(const Matrix& c, maize_out_type_t out = MAIZE_OUT_SAME, float alpha = 1.0f, float beta = 0.0f) {
+        const uint32_t n = op_.nt ? op_.b.g.nrows : op_.b.g.ncols;
+        if (c.g.nrows != op_.a.g.nrows || c.g.ncols != n) throw std::invalid_argument("C does not have the shape the panels describe");
+        op_.c = c; op_.out = out; op_.alpha = alpha; op_.beta = beta; op_.stored = true;
+        k_->ops_.push_back(op_);
+    }
+  private:
+    TracedKernel* k_; TracedOp op_;
+};
+template <class Panel> struct is_row_panel : std::false_type {};
+template <uint32_t N> struct is_row_panel<RowPanel<N>> : std::true_type {};
+// sm80_gemm_smem_multibuffer(&mma, KTile::<K>, a_panel, b_panel, smem, cp_group, cp_size), gemm/mod.rs:37-90.  A B stored
+// N x K hands in row panels of B; a K x N B column panels.
+template <class MMA, uint32_t K_TILE, uint32_t NA, class BPanel, class Pair, size_t PIPE>
+Accum gemm_smem_multibuffer(const MMA&, KTile<K_TILE>, const RowPanel<NA>& a, const BPanel& b, const SharedRing<Pair, PIPE>&, Wave cp_group, uint8_t cp_size) {
+    constexpr bool NT = is_row_panel<BPanel>::value;
+    static_assert(MMA::FAMILY == Family::MT256, "a shared-memory ring goes with the macro-tile kernels' instructions");
+    static_assert(K_TILE == MMA::K_TILE, "KTile does not match the K a ring stage of this instruction's kernels holds");
+    static_assert(PIPE == 2, "the macro-tile kernels run a two-stage ring");
+    static_assert(NA == 256 && BPanel::WINDOW == 256, "the macro-tile kernels take panels of 256 rows (A) and 256 columns (B)");
+    using TA = typename Pair::A::Ty; using TB = typename Pair::B::Ty;
+    constexpr uint32_t ES = MMA::K_TILE == 128 ? 1 : 2;
+    static_assert(TA::ROWS == 256 && TA::COLS == MMA::K_TILE && TA::ELEM_BYTES == ES && TA::SWIZZLE == Swizzle::KC16, "A stage: 256 x K_TILE, K-contiguous");
+    static_assert(NT ? (TB::ROWS == 256 && TB::COLS == MMA::K_TILE && TB::SWIZZLE == Swizzle::KC16)
+                     : (TB::ROWS == MMA::K_TILE && TB::COLS == 256 && TB::SWIZZLE == Swizzle::KN32), "B stage does not match how B is stored");
+    static_assert(NT || ES == 2, "8-bit operands: both K-contiguous (B stored N x K)");
+    if (cp_size != 16) throw std::invalid_argument("direct-to-LDS copies are 16 bytes per lane");
+    const uint32_t ka = a.col_size(), kb = NT ? b.matrix.g.ncols : b.matrix.g.nrows;
+    if (ka != kb) throw std::invalid_argument("inner dimensions differ");
+    return Accum(cp_group.kernel, TracedOp{a.matrix, b.matrix, Matrix{}, NT, MMA::IN_TYPE, MMA::FAMILY, false, MAIZE_OUT_SAME, 1.0f, 0.0f});
+}
+inline TracedKernel new_hip_kernel() { return TracedKernel(); }
 
 // ---- builder chain: kernel name -> launch bounds -> finalize -> compile(target) -> launch ------
 class LoadedKernel {

@@ -4,8 +4,8 @@
 // 4096 x 4096 operands and prints the PTX; it cannot launch it and the kernel has no C operand.
 // This program keeps the same steps -- declare the kernel, fix its launch bounds, compile for a
 // target, describe A and B as GlobalMatrix -- and then launches on an MI355X, twice: through the
-// dispatcher (gemm_smem_multibuffer) and through the explicit builder chain, and checks that the
-// two agree bit for bit.  Output: one JSON line with the kernel chosen and checksums of C.
+// dispatcher (gemm_smem_multibuffer), through the explicit builder chain, and as a kernel described in the
+// reference's tile vocabulary (panels, groups, ring, MMA op), and checks that all agree bit for bit.  Output: one JSON line with the kernel chosen and checksums of C.
 //
 //   maize_gemm_example [M N K]        (default 4096 4096 4096, like src/main.rs:47-48)
 #include <cinttypes>
@@ -53,17 +53,39 @@ int main(int argc, char** argv) {
         k.launch(grid, args);
         ctx.sync();
 
-        const std::vector<BF16> c1 = ctx.download(dc, (size_t)M * N), c2 = ctx.download(dc2, (size_t)M * N);
-        uint64_t sum = 0, x = 0, diff = 0;
+        // 3. the kernel described in the reference's tile vocabulary, in the order of src/main.rs:32-73
+        BF16* dc3 = ctx.malloc<BF16>((size_t)M * N);
+        TracedKernel kernel = new_hip_kernel();
+        kernel.with_launch_bounds_2d({256, 1});
+        auto pipe_shared = kernel.alloc_aligned_shared<TilePair<Tile<BF16_256x64>, Tile<BF16_64x256>>, 2>(1024);
+        const BlockX a_panel_group{kernel.cx()};
+        const BlockY b_panel_group{kernel.cx()};
+        const Wave wave{kernel.cx()};
+        const auto a_iter = collective_aligned_row_panel_iter<256>(amat, a_panel_group);     // (bulk panels, ragged epilogue panel)
+        const auto b_iter = collective_aligned_col_panel_iter<256>(bmat, b_panel_group);
+        a_iter.first.for_every_value([&](const RowPanel<256>& a_panel) {
+            b_iter.first.for_every_value([&](const ColPanel<256>& b_panel) {
+                Accum ret = gemm_smem_multibuffer(Gfx950MfmaBf16F32_16x16x32{}, KTile<64>{}, a_panel, b_panel, pipe_shared, wave, 16);
+                ret.store(Matrix::make(dc3, M, N));                                          // where the reference traps on a zero sum
+            });
+        });
+        LoadedGemm described = kernel.finalize().compile(Gfx::Gfx950, ctx);
+        described.launch();
+        ctx.sync();
+
+        const std::vector<BF16> c1 = ctx.download(dc, (size_t)M * N), c2 = ctx.download(dc2, (size_t)M * N), c3 = ctx.download(dc3, (size_t)M * N);
+        uint64_t sum = 0, x = 0, diff = 0, diff3 = 0;
         for (size_t i = 0; i < c1.size(); ++i) {
             sum += c1[i].bits;
             x ^= (uint64_t)c1[i].bits << (i % 48);
             diff += c1[i].bits != c2[i].bits;
+            diff3 += c1[i].bits != c3[i].bits;
         }
-        printf("{\"M\": %u, \"N\": %u, \"K\": %u, \"kernel\": \"%s\", \"sum\": %" PRIu64 ", \"xor\": %" PRIu64
-               ", \"mismatch_vs_any_shape_kernel\": %" PRIu64 "}\n", M, N, K, chosen.c_str(), sum, x, diff);
-        ctx.free(da); ctx.free(db); ctx.free(dc); ctx.free(dc2);
-        return diff == 0 ? 0 : 3;
+        printf("{\"M\": %u, \"N\": %u, \"K\": %u, \"kernel\": \"%s\", \"described_kernel\": \"%s\", \"ragged_rows\": %u, \"ragged_cols\": %u, "
+               "\"sum\": %" PRIu64 ", \"xor\": %" PRIu64 ", \"mismatch_vs_any_shape_kernel\": %" PRIu64 ", \"mismatch_vs_described_kernel\": %" PRIu64 "}\n",
+               M, N, K, chosen.c_str(), described.kernel_name().c_str(), a_iter.second.extent, b_iter.second.extent, sum, x, diff, diff3);
+        ctx.free(da); ctx.free(db); ctx.free(dc); ctx.free(dc2); ctx.free(dc3);
+        return (diff == 0 && diff3 == 0) ? 0 : 3;
     } catch (const Error& e) {
         fprintf(stderr, "maize error: %s\n", e.what());
         return 2;

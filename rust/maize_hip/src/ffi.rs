@@ -4,6 +4,8 @@
 use core::ffi::{c_char, c_void};
 
 pub const MAIZE_OK: i32 = 0;
+pub const MAIZE_ERR_SHAPE: i32 = -2;
+pub const MAIZE_ERR_ARG: i32 = -7;
 pub const MAIZE_LAYOUT_NN: u32 = 0;
 pub const MAIZE_LAYOUT_NT: u32 = 1;
 pub const MAIZE_OUT_SAME: u32 = 0;

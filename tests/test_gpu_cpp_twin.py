@@ -25,6 +25,8 @@ def test_cpp_twin_matches_the_ctypes_path(ctx, oracle, shape):
     assert out.returncode == 0, out.stderr + out.stdout
     rec = json.loads(out.stdout.strip().splitlines()[-1])
     assert rec["mismatch_vs_any_shape_kernel"] == 0
+    assert rec["mismatch_vs_described_kernel"] == 0 and rec["described_kernel"] == rec["kernel"]     # the tile vocabulary resolves to the same launch
+    assert (rec["ragged_rows"], rec["ragged_cols"]) == (m % 256, n % 256)
     a, b = mz.gen.uniform_bf16(m * k, mz.gen.SEED_A), mz.gen.uniform_bf16(k * n, mz.gen.SEED_B)
     got = run_gemm(ctx, a, b, m, n, k)
     assert rec["sum"] == int(got.astype(np.uint64).sum())           # same bits as the ctypes path
