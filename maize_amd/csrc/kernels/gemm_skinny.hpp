@@ -18,8 +18,8 @@
 //     N contiguous: the block is deposited in LDS as it is in memory and read back with
 //     ds_read_b64_tr_b16 (4 K-consecutive values of the lane's column per read).  A 32-byte
 //     granule XOR keeps those reads bank-conflict free.  Wave w multiplies columns 32w .. 32w+31;
-//   * A (16 x K, L2 resident) is fetched straight into MFMA operand registers, one 16-byte load
-//     per lane per block, in the same in-order load stream as the block it multiplies;
+//   * A (16 x K, L2 resident) goes through LDS too: one 1 KiB direct-to-LDS load per block and
+//     workgroup, already in MFMA fragment order, in the same in-order load stream as the block;
 //   * v_mfma_f32_16x16x32_bf16 with B's fragment first: each lane ends up holding 4 consecutive
 //     columns of one row of C;
 //   * split K: every workgroup writes its fp32 partial tile to a workspace and takes a ticket;
@@ -66,6 +66,20 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     __shared__ __attribute__((aligned(1024))) char ring6[BLOCK_BYTES];
     __shared__ __attribute__((aligned(1024))) char ring7[BLOCK_BYTES];
     __shared__ uint32_t ticket;
+    // A blocks (16 rows x 32 k = 1 KiB), one per ring slot, fetched once per workgroup: lane l of a direct-to-LDS load
+    // asks for (row l % 16, k chunk l / 16) -- exactly the MFMA fragment of lane l -- and lands at 16 l, so every wave
+    // reads its A operand as one conflict-free 16-byte read at 16 l.  The block that goes into slot x is fetched by
+    // wave x: the duty rotates, every wave issues 17 loads per ring turn, and the number of loads a wave may leave in
+    // flight when it waits for a block is 12 or 13 depending on where its duty falls (turn()).  (Each wave fetching its own copy from L2 moved 8 KiB
+    // per 16 KiB block of B through the vector memory path and cost 0.5 us of 25.)
+    __shared__ __attribute__((aligned(1024))) char ablk0[1024];
+    __shared__ __attribute__((aligned(1024))) char ablk1[1024];
+    __shared__ __attribute__((aligned(1024))) char ablk2[1024];
+    __shared__ __attribute__((aligned(1024))) char ablk3[1024];
+    __shared__ __attribute__((aligned(1024))) char ablk4[1024];
+    __shared__ __attribute__((aligned(1024))) char ablk5[1024];
+    __shared__ __attribute__((aligned(1024))) char ablk6[1024];
+    __shared__ __attribute__((aligned(1024))) char ablk7[1024];
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
     const uint32_t lda = lda_of(p), ldb = ldb_of(p), ldc = ldc_of(p);
@@ -86,6 +100,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
     lds_ptr const s0 = (lds_ptr)ring0, s1 = (lds_ptr)ring1, s2 = (lds_ptr)ring2, s3 = (lds_ptr)ring3;
     lds_ptr const s4 = (lds_ptr)ring4, s5 = (lds_ptr)ring5, s6 = (lds_ptr)ring6, s7 = (lds_ptr)ring7;
+    lds_ptr const ablk[RING] = {(lds_ptr)ablk0, (lds_ptr)ablk1, (lds_ptr)ablk2, (lds_ptr)ablk3,
+                                (lds_ptr)ablk4, (lds_ptr)ablk5, (lds_ptr)ablk6, (lds_ptr)ablk7};
 
     // ---- copy map: wave w issues pieces 2w and 2w+1 of a block; piece pc = rows 2pc, 2pc+1.
     // Lane l lands at byte 16 l of the piece = row 2pc + l/32, stored chunk l%32, and therefore
@@ -121,20 +137,19 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     floatx4 acc[2];
     acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
     acc[1] = floatx4{0.f, 0.f, 0.f, 0.f};
-    bf16x8 af[RING];
 
-    // Requests block j (rows k0 + 32j ..) into `slot`, and its A fragment into af[ai]: 3 loads
-    // per wave in the in-order stream.  Blocks past the end read a zero-length descriptor.
+    // Requests block j (rows k0 + 32j ..) into `slot` -- two pieces per wave -- and, if this wave has the duty, its A
+    // block into ablk[ai] first.  Blocks past the end read a zero-length descriptor.
     auto request = [&](uint32_t j, lds_ptr slot, int ai) {
         typedef __attribute__((address_space(3))) void* lvp;
         const uint32_t kb = k0 + j * KB;
         const bool live = j < nb;
         const __amdgpu_buffer_rsrc_t rs_b = live ? rb : rnull;
         const __amdgpu_buffer_rsrc_t rs_a = live ? ra : rnull;
-        // The fences pin the issue order (A fragment, piece, piece): the counter waits below
+        // The fences pin the issue order (A block, piece, piece): the counter waits below
         // count loads in that order.
         __builtin_amdgcn_sched_barrier(0);
-        af[ai] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rs_a, a_vo, kb * 2u, 0));
+        if (wave == (uint32_t)ai) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lvp)ablk[ai], 16, a_vo, kb * 2u, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -143,23 +158,33 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         __builtin_amdgcn_sched_barrier(0);
     };
     auto consume = [&](lds_ptr slot, int ai) {
-        typedef short4v __attribute__((address_space(3))) * v4p;
+        // The reads are inline assembly so that the compiler sees no read of the ring: it would otherwise order every
+        // read behind the direct-to-LDS loads in flight with a counter wait of its own, computed without the duty loads.
+        bf16x8 af;
+        short4v lo[2], hi[2];
+        asm volatile("ds_read_b128 %0, %1" : "=v"(af) : "v"((uint32_t)(uintptr_t)ablk[ai] + lane * 16u));
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {
-            short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(slot + rd[0][c2]));
-            short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4p)(slot + rd[1][c2]));
-            short8v bb = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo[c2]) : "v"((uint32_t)(uintptr_t)slot + rd[0][c2]));
+            asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi[c2]) : "v"((uint32_t)(uintptr_t)slot + rd[1][c2]));
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2) {
+            short8v bb = {lo[c2][0], lo[c2][1], lo[c2][2], lo[c2][3], hi[c2][0], hi[c2][1], hi[c2][2], hi[c2][3]};
             if (half_io)   // same bits, read as IEEE half (a wave-uniform choice)
-                acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, bb), __builtin_bit_cast(halfx8, af[ai]), acc[c2], 0, 0, 0);
+                acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, bb), __builtin_bit_cast(halfx8, af), acc[c2], 0, 0, 0);
             else
-                acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bb), af[ai], acc[c2], 0, 0, 0);
+                acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bb), af, acc[c2], 0, 0, 0);
         }
     };
-    // One block: wait until this wave's share of block b has landed (the 18 loads of blocks
-    // b+1 .. b+6 may stay in flight), meet the other waves -- which also tells us everyone is
-    // done reading block b-1 -- refill that block's slot with block b+7, then multiply block b.
+    // One block: wait until this wave's share of block b has landed (the loads of blocks b+1 .. b+6 may stay in
+    // flight: 12 pieces, and one A block unless this wave's duty is block b itself -- older than b's pieces -- or
+    // block b+7, not requested yet), meet the other waves -- which also tells us everyone is done reading block
+    // b-1 -- refill that block's slot with block b+7, then multiply block b.
     auto turn = [&](uint32_t b, lds_ptr cur, int ai, lds_ptr prev, int pi) {
-        asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");
+        if (wave == (uint32_t)ai || wave == (uint32_t)pi) asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(13)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         request(b + 7, prev, pi);
         consume(cur, ai);

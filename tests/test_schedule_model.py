@@ -279,42 +279,51 @@ def test_8bit_macro_tile_checker_rejects_broken_schedules():
 
 
 # ---------------------------------------------------------------------------------------
-# skinny kernel: 8-slot ring, 3 loads per block per wave, counter wait instead of wait-all
+# skinny kernel: 8-slot ring, per wave 2 pieces per block plus the A block of the slot whose index is the wave's
+# (the duty rotates), counter wait instead of wait-all
 # ---------------------------------------------------------------------------------------
 
 def skinny_constants():
     src = open(os.path.join(KDIR, "gemm_skinny.hpp")).read()
     ring = int(re.search(r"constexpr int RING = (\d+);", src).group(1))
     waits = [int(x) for x in re.findall(r"s_waitcnt vmcnt\((\d+)\)\\n\\ts_barrier", src)]
-    assert len(waits) == 1
+    assert len(waits) == 2                  # with and without an A block among the loads that may stay in flight
+    # the duty rule and the rule that picks the wait, as written in the kernel
+    assert "if (wave == (uint32_t)ai) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a" in src
+    assert re.search(r"if \(wave == \(uint32_t\)ai \|\| wave == \(uint32_t\)pi\) asm volatile\(\"s_waitcnt vmcnt\(%d\)" % min(waits), src)
     primed = len(re.findall(r"request\(\d+, s\d+, \d+\);", src))
-    return ring, waits[0], primed
+    return ring, (min(waits), max(waits)), primed
 
 
-def skinny_wave_program(nb, ring, wait, primed, loads_per_request=3):
+def skinny_wave_program(nb, ring, waits, primed, wave=0):
+    """The program of one wave: ("request", block, slot, loads), ("wait", n), ("barrier",), ("consume", block, slot)."""
+    short, long_ = waits
+    loads = lambda slot: 3 if slot == wave else 2
     ops = []
     for j in range(primed):
-        ops.append(("request", j, j % ring))
+        ops.append(("request", j, j % ring, loads(j % ring)))
     turns = -(-nb // ring) * ring
     for b in range(turns):
-        ops += [("wait", wait), ("barrier",)]
-        ops.append(("request", b + primed, (b + primed) % ring))
-        ops.append(("consume", b, b % ring))
+        cur, refill = b % ring, (b + primed) % ring
+        ops += [("wait", short if wave in (cur, refill) else long_), ("barrier",)]
+        ops.append(("request", b + primed, refill, loads(refill)))
+        ops.append(("consume", b, cur))
     ops.append(("wait", 0))
-    return ops, turns, loads_per_request
+    return ops, turns, None
 
 
 def check_ring(ops, turns, loads_per_request, ring):
     epoch = 0
-    issued = []                 # blocks in request order (each stands for loads_per_request loads)
-    done = 0                    # number of requests known complete for this wave
+    issued = []                 # blocks in request order
+    loads = []                  # one entry per load, in issue order: the block it belongs to
+    done = 0                    # number of loads known complete for this wave (the counter retires them in order)
     visible_from = {}
     consumed_epoch = {}
     slot_holds = {}
     consumed = []
     for op in ops:
         if op[0] == "request":
-            _, blk, slot = op
+            _, blk, slot = op[:3]
             old = slot_holds.get(slot)
             if old is not None:
                 if old not in consumed_epoch:
@@ -323,14 +332,16 @@ def check_ring(ops, turns, loads_per_request, ring):
                     raise Hazard(f"block {blk} overwrites block {old} in the epoch it is read in")
             slot_holds[slot] = blk
             issued.append(blk)
+            loads += [blk] * (op[3] if len(op) > 3 else loads_per_request)
         elif op[0] == "wait":
             # the counter retires loads in order: at most op[1] of the newest may be outstanding
-            outstanding_requests = -(-op[1] // loads_per_request)
-            done = max(done, len(issued) - outstanding_requests)
+            done = max(done, len(loads) - op[1])
         elif op[0] == "barrier":
             epoch += 1
-            for blk in issued[:done]:
-                visible_from.setdefault(blk, epoch)
+            pending = set(loads[done:])
+            for blk in issued:
+                if blk not in pending:
+                    visible_from.setdefault(blk, epoch)
         elif op[0] == "consume":
             _, blk, slot = op
             if slot_holds.get(slot) != blk:
@@ -339,7 +350,7 @@ def check_ring(ops, turns, loads_per_request, ring):
                 raise Hazard(f"block {blk} consumed in epoch {epoch} before every wave's share has landed")
             consumed_epoch[blk] = epoch
             consumed.append(blk)
-    if done != len(issued):
+    if done != len(loads):
         raise Hazard("loads still in flight at the end")
     if consumed != list(range(turns)):
         raise Hazard("blocks not consumed exactly once, in order")
@@ -349,23 +360,37 @@ def check_ring(ops, turns, loads_per_request, ring):
 
 @pytest.mark.parametrize("nb", [8, 16, 32, 128, 9])
 def test_skinny_ring_is_hazard_free(nb):
-    ring, wait, primed = skinny_constants()
+    ring, waits, primed = skinny_constants()
     assert primed == ring - 1
-    ops, turns, lpr = skinny_wave_program(nb, ring, wait, primed)
-    check_ring(ops, turns, lpr, ring)
-    # the wait leaves exactly the requests of the blocks behind the current one in flight
-    assert wait == lpr * (primed - 1)
+    for wave in range(8):
+        ops, turns, lpr = skinny_wave_program(nb, ring, waits, primed, wave)
+        check_ring(ops, turns, lpr, ring)
+        # every wait is exact: it leaves just the loads issued after the current block's in flight
+        issued = []
+        for op in ops:
+            if op[0] == "request":
+                issued += [op[1]] * op[3]
+            elif op[0] == "consume":
+                # loads of later blocks, except this turn's refill (block op[1] + primed), which is issued after the wait
+                newer = sum(1 for blk in issued if op[1] < blk < op[1] + primed)
+                assert last_wait == newer, (wave, op, last_wait, newer)
+            elif op[0] == "wait":
+                last_wait = op[1]
 
 
 def test_skinny_checker_rejects_broken_rings():
-    ring, wait, primed = skinny_constants()
-    ops, turns, lpr = skinny_wave_program(32, ring, wait + 3, primed)       # waits for one request too few
-    with pytest.raises(Hazard):
-        check_ring(ops, turns, lpr, ring)
-    ops, turns, lpr = skinny_wave_program(32, ring - 1, wait, primed)        # ring one slot short: refill hits the block being read
+    ring, waits, primed = skinny_constants()
+    for wave in (0, 3, 7):
+        ops, turns, lpr = skinny_wave_program(32, ring, (waits[0] + 1, waits[1] + 1), primed, wave)   # waits for one load too few
+        with pytest.raises(Hazard):
+            check_ring(ops, turns, lpr, ring)
+        ops, turns, lpr = skinny_wave_program(32, ring, (waits[1], waits[1]), primed, wave)           # ignores where the duty falls
+        with pytest.raises(Hazard):
+            check_ring(ops, turns, lpr, ring)
+    ops, turns, lpr = skinny_wave_program(32, ring - 1, waits, primed)       # ring one slot short: refill hits the block being read
     with pytest.raises(Hazard):
         check_ring(ops, turns, lpr, ring - 1)
-    ops, turns, lpr = skinny_wave_program(32, ring, wait, primed)
+    ops, turns, lpr = skinny_wave_program(32, ring, waits, primed)
     swapped = [o for o in ops]
     i = next(k for k, o in enumerate(swapped) if o[0] == "barrier")
     del swapped[i]                                                         # first barrier missing
@@ -404,7 +429,7 @@ def check_private_ring(ops, turns, loads_per_request):
     issued, done, slot_holds, consumed = [], 0, {}, []
     for op in ops:
         if op[0] == "request":
-            _, blk, slot = op
+            _, blk, slot = op[:3]
             old = slot_holds.get(slot)
             if old is not None and old not in consumed:         # program order of one wave: its reads of `old` are behind it
                 raise Hazard(f"block {blk} overwrites block {old} before it is consumed")
