@@ -3,10 +3,12 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5|f8|f8s|f32|f64] [--kernel NAME]
 
-A step is one launch of maize_hip_gemm_bf16 on synthetic, seeded inputs that are already
-resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s (wall clock around exactly K
-steps), the roofline object of the kernel (HIP events on the launch stream) and the CPU
-oracle timed on a bounded slab of the same problem on this machine's host cores.
+A step is one launch of maize_hip_gemm_bf16 (maize_hip_gemm_bf16_ex for the 8-bit, fp32 and fp64
+configurations) on synthetic, seeded inputs that are already resident in HBM.  Prints ONE JSON line:
+whole-job TFLOP/s (wall clock around exactly K steps), the roofline object of the kernel (HIP events on
+the launch stream) and the CPU oracle timed on a bounded slab of the same problem on this machine's host
+cores.  The timed region follows a clock ramp (launches until the batch time settles) and W warm-up steps: it
+is a hot-clock figure of a few milliseconds; --config energy measures the sustained one.
 """
 import argparse
 import json
@@ -23,11 +25,16 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each
-# scaled by what the same counter reads for a 256 MiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x
-# 1.000): profiles/hbm_traffic_fetch_write_size.md.  Not measured for the other configurations.
-MEASURED_TRAFFIC_BYTES = {"cfg1": 235.2e6, "cfg2": 275.1e6, "cfg3": 1746.3e6, "cfg4": 126.4e6, "cfg5": 1074.3e6,
-                          "f8": 134.5e6, "f8s": 67.2e6, "f32": 828.9e6, "f64": 3162.3e6}
+# HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs per workload), each scaled by what
+# the same counter reads for a 256 MiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  These are figures of an earlier
+# profiling session, not of this run: each entry names the kernel it was measured on and is reported only when this
+# run's kernel is that one, together with its source file.
+TRAFFIC_SOURCE = "profiles/hbm_traffic_fetch_write_size.md"
+MEASURED_TRAFFIC = {"cfg1": ("maize_gemm_bf16_mt256_nn", 235.2e6), "cfg2": ("maize_gemm_bf16_mt256_nn_edge", 275.1e6),
+                    "cfg3": ("maize_gemm_bf16_mt256_nt", 1746.3e6), "cfg4": ("maize_gemm_bf16_skinny_nn", 126.4e6),
+                    "cfg5": ("maize_gemm_bf16_mt256_nn", 1074.3e6), "f8": ("maize_gemm_e4m3_mt256_nt", 134.5e6),
+                    "f8s": ("maize_gemm_e4m3_skinny_nt", 67.2e6), "f32": ("maize_gemm_f32_mt128_nn", 828.9e6),
+                    "f64": ("maize_gemm_f64_mt128_nn", 3162.3e6)}
 
 # name -> (M, N, K, layout, batch, A distribution, B distribution, bound)
 CONFIGS = {
@@ -368,7 +375,8 @@ def main():
             o = measure(mz, ctx, name, max(20, args.steps // 4), max(10, args.warmup // 2), None, 0, False)
             others[name] = {"workload": o["config"]["workload"], "us_per_step": o["ms_per_step"] * 1e3, "value": o["value"],
                             "unit": o["unit"], "kernel": o["roofline"]["kernel"], "roofline_bound": o["roofline"]["bound"],
-                            "roofline_frac": o["roofline"]["frac"], "steps": o["steps"]}
+                            "roofline_frac": o["roofline"]["frac"], "steps": o["steps"], "kernel_avg_us": o["roofline"]["kernel_avg_us"],
+                            "traffic": o["roofline"]["traffic"], "traffic_source": o["roofline"].get("traffic_source")}
         line["other_configs"] = others
     print(json.dumps(line), flush=True)
     ctx.close()
@@ -453,7 +461,10 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
         ach = alg_bytes / (kern_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
                 "traffic": None}
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.config) if args.kernel is None else None
+    profiled = MEASURED_TRAFFIC.get(args.config)
+    if profiled and profiled[0] == kernel:
+        roof["traffic"] = profiled[1]
+        roof["traffic_source"] = f"{TRAFFIC_SOURCE} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on {kernel}, an earlier session; not measured in this run)"
     roof["kernel"] = kernel
     roof["kernel_avg_us"] = kern_ms * 1e3
     roof["algorithmic_flop"] = flops

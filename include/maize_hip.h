@@ -32,10 +32,11 @@
  *    instruction), C is rounded once to bf16 (nearest even).  IEEE special values follow through: NaN and +-Inf in A or
  *    B give NaN / Inf exactly where an fp64 evaluation does (the zero fill of the M, N and K edges never meets a real
  *    operand in a stored element), and subnormal operands and results are kept, not flushed.
- *  - All matrices are row-major with leading dimension == ncols, as in the
+ *  - All matrices are row-major.  With the plain descriptor the leading dimension == ncols, as in the
  *    reference (crates/maize_tile/src/gmem/row_panel.rs:55,
- *    crates/maize_tile/src/gmem/col_panel.rs:108).  BF16 is a 2-byte,
- *    2-aligned, u16-backed type (crates/maize_core/src/ty/sized.rs:62-68).
+ *    crates/maize_tile/src/gmem/col_panel.rs:108); the extended descriptor carries lda / ldb / ldc.  BF16 is a
+ *    2-byte, 2-aligned, u16-backed type (crates/maize_core/src/ty/sized.rs:62-68); the extended descriptor also
+ *    takes half, 8-bit float, fp32 and fp64 operands.
  */
 #ifndef MAIZE_HIP_H
 #define MAIZE_HIP_H
@@ -51,7 +52,7 @@ enum {
     MAIZE_OK = 0,
     MAIZE_ERR_NULL = -1,        /* a required pointer argument is NULL */
     MAIZE_ERR_SHAPE = -2,       /* zero/mismatched dimensions or batch/stride inconsistency */
-    MAIZE_ERR_ALIGN = -3,       /* a device pointer is not 2-byte aligned */
+    MAIZE_ERR_ALIGN = -3,       /* a device pointer is not aligned to its element size (1, 2, 4 or 8 bytes) */
     MAIZE_ERR_LAYOUT = -4,      /* unknown maize_layout_t value */
     MAIZE_ERR_KERNEL = -5,      /* unknown kernel name, or the kernel cannot run this descriptor */
     MAIZE_ERR_NO_DEVICE = -6,   /* no usable HIP device / device is not gfx950 */

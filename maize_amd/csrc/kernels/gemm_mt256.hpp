@@ -80,18 +80,14 @@ constexpr uint32_t OOB = 0x80000000u;   // OR-ed into an offset: >= num_records,
 // quarters of step t+1.  Piece pc goes out at slot DMA_STRIDE * pc + 2: a wave retires at most one 1 KiB
 // direct-to-LDS load per ~64 cycles (four MFMA slots), so the requests are spaced out; they all have to
 // land before the barrier of step t+1 (slot 128).
-#ifndef MAIZE_MT256_DMA_STRIDE
-#define MAIZE_MT256_DMA_STRIDE 4
-#endif
-constexpr int DMA_STRIDE = MAIZE_MT256_DMA_STRIDE;
+constexpr int DMA_STRIDE = 4;
 constexpr int issue_slot(int pc) { return DMA_STRIDE * pc + 2; }
 static_assert(DMA_STRIDE >= 3 && issue_slot(15) < 96, "the last request needs at least a quarter of a step to land before the barrier");
 // Pieces requested behind the barrier of step t itself (the rest follow in step t+1).
 constexpr int early_pieces() { int n = 0; for (int i = 0; i < 16; ++i) n += issue_slot(i) < 32; return n; }
-// Cache policy bits of the direct-to-LDS loads (bit 0 sc0, bit 1 nt, bit 4 sc1).
-#ifndef MAIZE_MT256_DMA_AUX
-#define MAIZE_MT256_DMA_AUX 0
-#endif
+// Cache policy bits of the direct-to-LDS loads (bit 0 sc0, bit 1 nt, bit 4 sc1): none -- sc0 / sc1 measured no
+// difference, nt cost 15 %.
+constexpr int DMA_AUX = 0;
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
 typedef __attribute__((address_space(3))) u32x4* lds_v4;
@@ -287,17 +283,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             const uint64_t skip = (uint64_t)k * ldb * 2u;
             const uint32_t bytes = k < k_end ? span(b_view - skip) : 0u;       // k < k_end <= K: skip < b_view
             const __amdgpu_buffer_rsrc_t rs = make_rsrc(Bg + skip, bytes);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, b_vo[i], 0, 0, MAIZE_MT256_DMA_AUX);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, b_vo[i], 0, 0, DMA_AUX);
             return;
         }
         const uint32_t bytes = k < k_end ? (is_a ? a_bytes : b_bytes) : 0u;
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(is_a ? (const void*)Ag : (const void*)Bg, bytes);
         if (!KTAIL) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i], k * ES, 0, MAIZE_MT256_DMA_AUX);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, is_a ? a_vo[i] : b_vo[i], k * ES, 0, DMA_AUX);
         } else {
             uint32_t off = (is_a ? a_vo[i] : b_vo[i]) + k * ES;
             off |= (a_k[i & 1] + k) < K ? 0u : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, off, 0, 0, MAIZE_MT256_DMA_AUX);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, off, 0, 0, DMA_AUX);
         }
     };
 
@@ -343,10 +339,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr int NAR = IS8 ? 8 : 4;                    // reads that bring in one A group
     constexpr int NBR = (IS8 || !NT) ? 8 : 4;           // ... one B group (transposing reads are 64-bit, 8-bit fragments two reads)
     // Read r of a group is issued in MFMA slot r * RSTRIDE of the eighth.
-#ifndef MAIZE_MT256_RSTRIDE
-#define MAIZE_MT256_RSTRIDE 1
-#endif
-    static_assert(8 * MAIZE_MT256_RSTRIDE <= 16, "the reads of a group must fit into the 16 slots of an eighth");
+    constexpr int RSTRIDE = 1;
+    static_assert(8 * RSTRIDE <= 16, "the reads of a group must fit into the 16 slots of an eighth");
     // 128-bit read at base + 2048 * n (n = stage * 16 + fragment), 64-bit transposing read at
     // base + 2048 * n (n = stage * 16 + kh * 8 + h).  The offsets are immediates: one case per value,
     // folded away once the caller's loops are unrolled.
@@ -424,11 +418,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // Order of the 4 x 4 MFMAs of an eighth (bit 0: boustrophedon, bit 1: B fragment held over four
                 // MFMAs instead of A's).  Consecutive MFMAs then differ in one operand only, which measures
                 // ~1 % faster at the power limit than the row-major order (less switching on the operand paths).
-#ifndef MAIZE_MT256_ORDER
-#define MAIZE_MT256_ORDER 3
-#endif
-                const int hi4 = s >> 2, lo4 = (MAIZE_MT256_ORDER & 1) && (hi4 & 1) ? 3 - (s & 3) : (s & 3);
-                const int r4 = (MAIZE_MT256_ORDER & 2) ? lo4 : hi4, c4 = (MAIZE_MT256_ORDER & 2) ? hi4 : lo4;
+                constexpr int ORDER = 3;
+                const int hi4 = s >> 2, lo4 = (ORDER & 1) && (hi4 & 1) ? 3 - (s & 3) : (s & 3);
+                const int r4 = (ORDER & 2) ? lo4 : hi4, c4 = (ORDER & 2) ? hi4 : lo4;
                 // The accumulator is tied to itself ("+a"): left to the register allocator, a few of the 64
                 // tuples were renamed across the loop and copied back through VGPRs at its end.  (Each
                 // accumulator comes up again 128 MFMAs later: no dependent back-to-back issue.)
@@ -440,8 +432,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 else
                     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(bi ^ kh, c4)), "v"(fa[ai][r4]));
                 // Side work of this slot: the reads of the group the next eighth needs ...
-                if (s % MAIZE_MT256_RSTRIDE == 0) {
-                    const int r = s / MAIZE_MT256_RSTRIDE;
+                if (s % RSTRIDE == 0) {
+                    const int r = s / RSTRIDE;
                     if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);                       // (0,0) -> (0,1): B group 1
                     if (h4 == 1 && r < NAR) read_a(1, kh, cur, r);                       // (0,1) -> (1,1): A group 1
                     if (h4 == 2 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }   // next half or tile: A group 0
