@@ -32,7 +32,7 @@ def mt256_issue_slots():
     """MFMA slot (counted from the barrier of step t, 128 slots per step) at which each of the 16 pieces of tile
     t + 2 is requested, as the kernel source defines it."""
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
-    stride = int(re.search(r"#define MAIZE_MT256_DMA_STRIDE (\d+)", src).group(1))
+    stride = int(re.search(r"constexpr int DMA_STRIDE = (\d+);", src).group(1))
     assert "constexpr int issue_slot(int pc) { return DMA_STRIDE * pc + 2; }" in src
     assert "constexpr int DS = IS8 ? 2 : DMA_STRIDE;" in src and "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {" in src
     assert "if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);" in src      # early pieces: those behind the barrier of step t itself
