@@ -430,11 +430,25 @@ bool trb_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims*
 // ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
 bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
-    if (fp8_in(d) || wide_in(d) || d.gemm.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u) || (s.n & 7u) || !aligned16(d)) return false;
+    if (fp8_in(d) || wide_in(d) || d.gemm.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u)) return false;
+    // A: 16-byte rows (its blocks are fetched 16 bytes per lane in fragment order).  B and C: any N, leading dimension
+    // and 2-byte-aligned pointer -- the 128-bit requests for B may start on any even byte, C is stored element by
+    // element when its rows are not 16-byte material (skinny_c_by_elements).
+    {
+        const Lds la = lds_of(d);
+        if (((uintptr_t)d.gemm.a.ptr & 15u) || (la.a & 7u) || (d.gemm.batch > 1 && (d.gemm.stride_a & 7u))) return false;
+    }
     const uint64_t lim = 1ull << 31;
     const Lds l = lds_of(d);
     if (l.ext_a * 2 >= lim || l.ext_b * 2 >= lim || s.n >= (1u << 21) || l.b >= (1u << 21)) return false;
     return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
+}
+// C rows that cannot take 128-bit stores: the kernel then writes C element by element (bit 0 of split_first).
+bool skinny_c_by_elements(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    const uint32_t per16 = d.out_type == MAIZE_OUT_F32 ? 4u : 8u;    // elements of C per 16 bytes
+    return (s.n & 7u) || (l.c % per16) || ((uintptr_t)d.gemm.c.ptr & 15u) || (d.gemm.batch > 1 && (d.gemm.stride_c % per16));
 }
 // K ranges: the smallest power of two that gives the grid at least 3/4 of a workgroup per
 // compute unit, as long as every range keeps at least 16 blocks of 32 rows.
@@ -457,7 +471,7 @@ bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDi
     ld->block[0] = 512; ld->block[1] = 1; ld->block[2] = 1;
     ld->lds_bytes = 0;
     ld->ksplit = ks;
-    ld->split_first = 0;
+    ld->split_first = skinny_c_by_elements(d) ? 1u : 0u;
     ld->reduce_grid = 0;
     ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * 16u * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
@@ -478,13 +492,7 @@ bool skinny_nt_common(const maize_gemm_ex_desc_t& d) {
     if (l.ext_a * esz >= lim || l.ext_b * esz >= lim || s.k >= (1u << 21) || l.b >= (1u << 21)) return false;
     return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
 }
-// C rows that cannot take 128-bit stores: the kernel then writes C element by element (bit 0 of split_first).
-bool skinny_nt_c_by_elements(const maize_gemm_ex_desc_t& d) {
-    const Dims s = dims_of(d);
-    const Lds l = lds_of(d);
-    const uint32_t per16 = d.out_type == MAIZE_OUT_F32 ? 4u : 8u;    // elements of C per 16 bytes
-    return (s.n & 7u) || (l.c % per16) || ((uintptr_t)d.gemm.c.ptr & 15u) || (d.gemm.batch > 1 && (d.gemm.stride_c % per16));
-}
+bool skinny_nt_c_by_elements(const maize_gemm_ex_desc_t& d) { return skinny_c_by_elements(d); }
 bool skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d); }
 #define MAIZE_F8_SKINNY(tag, type) \
     bool tag##_skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d); }

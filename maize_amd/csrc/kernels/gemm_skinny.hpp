@@ -26,8 +26,10 @@
 //     the last one to arrive for a slab adds the partials in split order (deterministic),
 //     rounds once to bf16 (RNE), stores C and resets the ticket counter.
 //
-// Requirements (checked by the dispatcher): layout NN, M <= 16, K % 32 == 0 (any number of K ranges),
-// N % 8 == 0, 16-byte aligned operands, every matrix (per batch member) below 2 GiB.
+// Requirements (checked by the dispatcher): layout NN, M <= 16, K % 32 == 0 (any number of K ranges), rows of A on
+// 16-byte boundaries, every matrix (per batch member) below 2 GiB.  B and C may have any N, leading dimension and
+// 2-byte-aligned pointer: the 128-bit requests for B may start on any even byte (the hardware splits them), and C
+// is stored element by element when its rows are not 16-byte material.
 #pragma once
 #include "common.hpp"
 #include "maps.hpp"
@@ -134,6 +136,19 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t k0 = b_first * KB;
     const uint32_t nb = b_first < nb_all ? (nb_all - b_first < per ? nb_all - b_first : per) : 0u;
 
+    // N % 8 != 0: the last 16-byte chunk of a row of B is only partly inside the row.  For every row but the last
+    // that is harmless (what follows is the next row; those columns of C are never stored).  The chunk of row K - 1
+    // ends past the matrix; the range check works dword by dword, so its whole dwords arrive and only an odd last
+    // column -- half of a dword that straddles the end -- is answered with zero.  A zero there would meet A's real
+    // values (Inf x 0 = NaN), so the wave that multiplies that column puts the real element (one 2-byte load, in
+    // bounds) into the block once it has landed, before reading it: the workgroup of the last slab and last K range.
+    const bool patch = (N & 1u) && n0 + SN >= N && b_first + nb == nb_all && nb;
+    const uint32_t patch_col = patch ? N - 1u - n0 : 0u;
+    const bool patch_wave = patch && wave == patch_col / 32u;
+    const uint32_t patch_off = maps::sk_offset(KB - 1u, patch_col >> 3) + (patch_col & 7u) * 2u;   // row K - 1 is the block's last
+    uint32_t patch_val = 0u;
+    if (patch_wave) patch_val = Bg[(uint64_t)(K - 1u) * ldb + N - 1u];
+
     floatx4 acc[2];
     acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
     acc[1] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -187,6 +202,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         else asm volatile("s_waitcnt vmcnt(13)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         request(b + 7, prev, pi);
+        if (patch_wave && b + 1u == nb) {
+            asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)cur + patch_off), "v"(patch_val) : "memory");
+        }
         consume(cur, ai);
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -207,9 +225,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // nothing may land in LDS after this point
 
-    // ---- combine the K splits in split order, round once, store ---------------------------
     // Lane holds C[m = l%16][n = n0 + 16(2w + c2) + 4g + 0..3].
     const uint32_t m = lane & 15u;
+    // ---- combine the K splits in split order, round once, store ---------------------------
+    // Rows of C that are not 16-byte material (odd N or leading dimension, a pointer off the 16-byte grid: a
+    // launch-uniform flag from the dispatcher) are stored element by element; C is at most 16 rows.
+    const bool c_elems = p.reserved & 1u;
     if (ks == 1u) {
         // Single split: straight from registers, 8 bytes per lane.
 #pragma unroll
@@ -217,7 +238,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
             if (m < M && col < N) {
                 const float v[4] = {acc[c2][0], acc[c2][1], acc[c2][2], acc[c2][3]};
-                store_c_run<4>(p, Cg, (uint64_t)m * ldc + col, v);
+                if (c_elems) store_c_elems<4>(p, Cg, (uint64_t)m * ldc + col, v, N - col);
+                else store_c_run<4>(p, Cg, (uint64_t)m * ldc + col, v);
             }
         }
         return;
@@ -269,9 +291,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
         }
         const uint32_t col = n0 + cq;
-        if (row < M && col < N) {                          // N % 8 == 0: 8 columns are all in or all out
+        if (row < M && col < N) {
             const float v[8] = {s_lo[0], s_lo[1], s_lo[2], s_lo[3], s_hi[0], s_hi[1], s_hi[2], s_hi[3]};
-            store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);
+            if (c_elems) store_c_elems<8>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
+            else store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);      // N % 8 == 0: 8 columns are all in or all out
         }
     }
     if (tid == 0) counters[slab_id] = 0u;                 // ready for the next launch

@@ -219,8 +219,14 @@ def test_skinny_nt_takes_any_n():
     assert p["kernel"] == "maize_gemm_bf16_skinny_nt" and p["split_first"] == 1 and p["grid"][0] == cdiv(50257, 256)
     p = mz.gemm_plan(desc(16, 50264, 768, layout=mz.LAYOUT_NT), compute_units=CUS)
     assert p["kernel"] == "maize_gemm_bf16_skinny_nt" and p["split_first"] == 0
-    # a K x N B with odd N has unaligned rows of B: not for the streaming kernels
-    assert "skinny" not in mz.gemm_plan(desc(16, 50257, 768), compute_units=CUS)["kernel"]
+    # a K x N B with odd N has rows of B on 2-byte boundaries only: the NN streaming kernel takes them too
+    p = mz.gemm_plan(desc(16, 50257, 768), compute_units=CUS)
+    assert p["kernel"] == "maize_gemm_bf16_skinny_nn" and p["split_first"] == 1
+    assert mz.gemm_plan(desc(16, 50264, 768), compute_units=CUS)["split_first"] == 0
+    # ... but A's rows must be 16-byte material (its blocks are fetched in fragment order, 16 bytes per lane)
+    d = desc(16, 50257, 768)
+    d.a.ptr += 2
+    assert "skinny" not in mz.gemm_plan(d, compute_units=CUS)["kernel"]
 
 
 def test_skinny_split_fills_the_chip_without_overshooting():

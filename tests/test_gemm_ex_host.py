@@ -74,7 +74,8 @@ def test_dispatch_of_extended_descriptors():
     # the skinny kernel carries the general epilogue
     for kw in (dict(alpha=0.5, beta=2.0), dict(out_type=mz.OUT_F32), dict(ldb=14400, ldc=14344)):
         assert mz.gemm_plan(ex(16, 14336, 4096, **kw))["kernel"] == "maize_gemm_bf16_skinny_nn"
-    assert mz.gemm_plan(ex(16, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_wave32"   # 16 rows do not earn back a copy of B
+    assert mz.gemm_plan(ex(16, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_skinny_nn"   # rows of B on 8-byte boundaries: still streamed
+    assert mz.gemm_plan(ex(16, 14336, 4096, lda=4100))["kernel"] == "maize_gemm_bf16_wave32"      # rows of A off the 16-byte grid: 16 rows do not earn back a copy
     assert mz.gemm_plan(ex(32, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_mt256_nn_packed"
 
 

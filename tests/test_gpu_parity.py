@@ -449,3 +449,44 @@ def test_tail_split_by_rows(ctx, oracle, layout):
     assert np.array_equal(got[:top * n], one[:top * n])             # the leading rows: the same kernel on the same tiles, bit for bit
     below = np.arange(top, m, 8, dtype=np.uint32)                   # the rows below: another summation order, checked against the oracle
     check_rows_against_oracle(oracle, got, a, bs, m, n, k, below, layout=layout, label="tail split by rows, rows below the seam")
+
+
+@pytest.mark.parametrize("shape", [(16, 50257, 4096), (13, 515, 2080), (16, 257, 256), (1, 4099, 288), (16, 14337, 4096), (7, 1001, 1024),
+                                   (16, 1030, 512), (5, 2053, 2048), (16, 263, 64), (3, 12, 32), (16, 5, 4096), (16, 4102, 1024)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_skinny_nn_takes_any_n(ctx, oracle, shape):
+    """Few rows against a row-major K x N B with any N (an odd vocabulary size): rows of B start on 2-byte boundaries,
+    the 128-bit requests straddle them, the last odd column of the last row is patched into the LDS block, C goes out element by
+    element.  Every output is checked."""
+    m, n, k = shape
+    a, b = inputs(m, n, k, dist="normal")
+    d = mz.gemm_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x1000, k, n), mz.GlobalMatrix(0x1000, m, n))
+    assert mz.gemm_plan(d, compute_units=256)["kernel"] == ("maize_gemm_bf16_skinny_nn" if n >= 64 else "maize_gemm_bf16_wave32")
+    _say(f"skinny_nn any N: {shape}")
+    got = run_gemm(ctx, a, b, m, n, k, kernel="maize_gemm_bf16_skinny_nn")
+    check_against_oracle(oracle, got, a, b, m, n, k, label=f"skinny_nn {shape}")
+
+
+def test_skinny_nn_unaligned_b_and_c(ctx, oracle):
+    """B at a 2-byte offset with an odd leading dimension, C at an odd offset: same kernel, same bar, nothing written
+    outside C."""
+    m, n, k = 16, 1024, 2048
+    ldb = n + 3
+    a = mz.gen.normal_bf16(m * k, mz.gen.SEED_A, 1.0)
+    bfull = mz.gen.normal_bf16(k * ldb + 1, mz.gen.SEED_B, 0.02)
+    da, db, dc = ctx.upload(a), ctx.upload(bfull), ctx.upload(np.full(m * n + 7, 0xDEAD, dtype=np.uint16))
+    try:
+        x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n, offset_elems=1), mz.Matrix(dc, m, n, offset_elems=3), ldb=ldb)
+        plan = mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])
+        assert plan["kernel"] == "maize_gemm_bf16_skinny_nn" and plan["split_first"] == 1, plan
+        _say(f"skinny_nn unaligned B and C: {plan}")
+        ctx.gemm_bf16(x)
+        ctx.sync()
+        got = dc.download(np.uint16)
+    finally:
+        da.free(); db.free(); dc.free()
+    assert np.all(got[:3] == 0xDEAD) and np.all(got[3 + m * n:] == 0xDEAD), "kernel wrote outside C"
+    B = np.stack([bfull[1 + r * ldb: 1 + r * ldb + n] for r in range(k)]).ravel()
+    ref, f64, ab = oracle.ref_gemm(a, B, m, n, k, want_f64=True, want_abs=True)
+    s = oracle.compare(got[3:3 + m * n], ref, f64, ab, k)
+    assert s["n_fail"] == 0, s

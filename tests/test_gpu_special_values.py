@@ -32,6 +32,8 @@ FAMILIES = [
     ("maize_gemm_bf16_mt256_nn_edge", 4096, 4104, 512, NN),          # 272 tiles on 256 units: the last tile column is split over K
     ("maize_gemm_bf16_mt256_nt_ktail_edge", 4096, 4104, 520, NT),
     ("maize_gemm_bf16_skinny_nn", 13, 520, 2080, NN),
+    ("maize_gemm_bf16_skinny_nn", 13, 515, 2080, NN),               # odd N: the last element of B is patched into the landed block
+    ("maize_gemm_bf16_skinny_nn", 16, 262, 4096, NN),
     ("maize_gemm_bf16_skinny_nt", 16, 515, 1096, NT),
     ("maize_gemm_bf16_wave32", 33, 17, 65, NN),
     ("maize_gemm_bf16_wave32", 33, 17, 65, NT),
