@@ -65,6 +65,24 @@ bool mt256_common(const maize_gemm_ex_desc_t& d) {
     if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21) || l.c >= (1u << 21)) return false;
     return true;
 }
+// What the loads of the macro-tile kernels need, whatever the epilogue: K % 8 == 0 (a 16-byte chunk never straddles
+// the end of a row in K: the lanes cannot mask inside a chunk), extents and leading dimensions below 2^21.  N, the
+// leading dimensions and the pointers are otherwise free -- 128-bit requests may start on any even byte (the odd last
+// element of a row-major B with an odd N is patched into the landed K tile by the kernels).
+bool mt256_loads_ok(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    if (s.k & 7u) return false;
+    if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21) || l.c >= (1u << 21)) return false;
+    return true;
+}
+// Rows of C that take whole 128-bit stores (bf16 / half: 8 elements, fp32: 4 per 16 bytes; runs are 8 columns wide).
+bool c_rows16(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    if ((s.n & 7u) || (l.c & 7u) || ((uintptr_t)d.gemm.c.ptr & 15u)) return false;
+    return d.gemm.batch == 1 || (d.gemm.stride_c & 7u) == 0;
+}
 // The plain kernels advance K with a scalar offset and never mask a lane in K: K % 64 == 0.
 bool k64(const maize_gemm_ex_desc_t& d) { return (d.gemm.a.ncols & 63u) == 0; }
 // The plain and edge-splitting kernels store bf16 of A.B only; the _gen kernels carry the general epilogue.
@@ -73,15 +91,15 @@ bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_co
 bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && bf16_in(d); }
 bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && plain_epilogue(d) && bf16_in(d); }
 bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && plain_epilogue(d) && bf16_in(d); }
-bool mt256_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && bf16_in(d); }
-bool mt256_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && bf16_in(d); }
-bool mt256_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && bf16_in(d); }
-bool mt256_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && bf16_in(d); }
+bool mt256_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && c_rows16(d) && k64(d) && bf16_in(d); }
+bool mt256_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && c_rows16(d) && k64(d) && bf16_in(d); }
+bool mt256_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && c_rows16(d) && bf16_in(d); }
+bool mt256_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && c_rows16(d) && bf16_in(d); }
 // IEEE half operands: the general-epilogue kernels instantiated on v_mfma_f32_32x32x16_f16.
-bool f16_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && half_in(d); }
-bool f16_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && half_in(d); }
-bool f16_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && half_in(d); }
-bool f16_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && half_in(d); }
+bool f16_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && c_rows16(d) && k64(d) && half_in(d); }
+bool f16_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && c_rows16(d) && k64(d) && half_in(d); }
+bool f16_nn_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && c_rows16(d) && half_in(d); }
+bool f16_nt_ktail_gen_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && c_rows16(d) && half_in(d); }
 // 8-bit operands (one byte per element), both K-contiguous: rows of A and B start on 16-byte
 // boundaries and K % 16 == 0; C as for the general-epilogue kernels (N % 8 == 0, rows on 16-byte
 // boundaries).  32-bit buffer offsets: each operand of one batch member stays below 2 GiB.
@@ -207,17 +225,18 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
     }
     return best_ks;
 }
-bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && bf16_in(d); }
-bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && bf16_in(d); }
-bool splitk_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && half_in(d); }
-bool splitk_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && half_in(d); }
+bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && bf16_in(d); }
+bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && bf16_in(d); }
+bool splitk_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && half_in(d); }
+bool splitk_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && half_in(d); }
 bool splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
     const Dims s = dims_of(d);
     const uint32_t kstep = fp8_in(d) ? 128u : 64u;
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * d.gemm.batch;
     uint32_t ks = splitk_ranges(s, d.gemm.batch, compute_units, kstep);
-    // Named explicitly for a shape the dispatcher would not split: two ranges if K allows, else one.
-    if (ks < 2u) ks = cdiv(s.k, kstep) >= 2u && tiles * 2ull * 262144ull <= (1ull << 30) ? 2u : 1u;
+    // Named explicitly for a shape the dispatcher would not split: two ranges if K allows, else one.  (A product whose
+    // C is not 16-byte material comes here for the reduce pass's element-wise stores: one range is fine then.)
+    if (ks < 2u && (fp8_in(d) || c_rows16(d))) ks = cdiv(s.k, kstep) >= 2u && tiles * 2ull * 262144ull <= (1ull << 30) ? 2u : 1u;
     const uint64_t items = tiles * ks;
     if (items > 0x1FFFFFFFull || items * 262144ull > (1ull << 32)) return false;
     uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
@@ -686,9 +705,18 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     static const char* const kHalf[2][2] = {       // [K tail][NT]: IEEE half operands
         {"maize_gemm_f16_mt256_nn_gen", "maize_gemm_f16_mt256_nt_gen"},
         {"maize_gemm_f16_mt256_nn_ktail_gen", "maize_gemm_f16_mt256_nt_ktail_gen"}};
-    const int ti = half_in(d)          ? kernel_index(kHalf[(s.k & 63u) != 0][s.nt])
-                   : plain_epilogue(d) ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
-                                       : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
+    // The plain and edge-splitting kernels want 16-byte rows everywhere.  Unaligned A or B (odd leading dimensions,
+    // 2-byte-aligned pointers) take the general-epilogue kernels, which share the K loop; a C whose rows are not
+    // 16-byte material (odd N, odd ldc, unaligned pointer) takes the split-K kernels -- with a single K range if
+    // splitting does not pay -- for the element-wise stores of their reduce pass: one more launch and C once through
+    // fp32 in memory, against three or four launches and copies of both operands on the packed path.
+    const bool strict = mt256_common(d);
+    if (!strict && si >= 0 && kKernels[si].supports(d) && !c_rows16(d) && (s.k >= 128 || (s.m >= 128 && s.n >= 128)) &&
+        (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && plan_fits(kKernels[si], d, compute_units))
+        return (uint32_t)si;
+    const int ti = half_in(d)                    ? kernel_index(kHalf[(s.k & 63u) != 0][s.nt])
+                   : plain_epilogue(d) && strict ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
+                                                 : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
     // The macro-tile kernel pays for a 256 x 256 tile and ~8 us whatever the shape, but it moves
     // its operands in 128-bit requests: measured, it beats the per-wave kernel 4-7x from
     // 16 x 4096 x 4096 up and loses (8 vs 4-7 us) only on short K with few rows or columns.

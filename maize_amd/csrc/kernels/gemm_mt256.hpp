@@ -57,9 +57,11 @@
 // ranges, each (tile, range) is a work item that leaves an fp32 partial tile in the workspace, and
 // maize_gemm_splitk_reduce (splitk_reduce.hpp) adds the ranges in order and applies the epilogue.
 //
-// Requirements (checked by the dispatcher): K % 8 == 0, N % 8 == 0, 16-byte
-// aligned operands, K, N and the leading dimensions below 2^21 elements; the
-// matrices themselves may be of any size.  The plain
+// Requirements (checked by the dispatcher): K % 8 == 0; K, N and the leading dimensions below 2^21 elements; the
+// matrices themselves may be of any size.  A and B may have any leading dimension and any 2-byte-aligned pointer
+// (128-bit requests may start on any even byte: the hardware splits them).  The kernels that store C themselves -- whole
+// 128-bit runs -- need N % 8 == 0 and 16-byte rows of C, the plain and edge-splitting ones 16-byte rows of A and B too; any
+// other N or C goes through the _splitk kernels, whose reduce pass stores C element by element where it must.  The plain
 // kernels need K % 64 == 0 (the K advance is then a scalar offset and no lane
 // ever needs a K mask); the _ktail kernels take any K % 8 == 0.
 #pragma once
@@ -216,6 +218,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     uint32_t a_vo[8], b_vo[8];
     uint32_t a_k[2];                      // k index of the lane's chunk inside a tile, even/odd piece (K masks)
     uint32_t part_slot = 0;               // split-K: index of this item's fp32 partial tile in the workspace
+    // A row-major K x N B with an odd N: the range check of the loads works dword by dword, so the dword that holds the
+    // last element of B's last row straddles the end of the view and comes back as zero -- which would meet A's real
+    // values in a stored column (Inf x 0 = NaN).  The waves that multiply that column write the real element (one
+    // 2-byte load, in bounds) into the landed K tile before they read it; LDS operations of a wave execute in order.
+    constexpr bool PATCHES = !NT && !IS8 && GEN;        // (the kernels that store C themselves from bf16 staging take even N only)
+    bool patch_on = false;                // this work item holds column N - 1 (last tile column, N odd)
+    uint32_t patch_off = 0, patch_val = 0;
     auto select_tile = [&](uint32_t id) {
         uint32_t tile_m, tile_n;
         uint64_t bz;
@@ -256,6 +265,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             b_bytes = 0u;
         }
         Cg = p.c + bz * p.stride_c * ((GEN && (p.epi & EPI_F32)) ? 2u : 1u);   // strides count elements of C
+        if (PATCHES) {
+            const uint32_t pcol = N - 1u - n0;                                 // < 256 when this tile holds column N - 1
+            patch_on = (N & 1u) && n0 + BN >= N && (pcol >> 7) == wn;          // ... and this wave multiplies it
+            if (patch_on) {
+                patch_off = maps::sk_offset((K - 1u) & (BK - 1u), pcol >> 3) + (pcol & 7u) * 2u;
+                patch_val = ((const uint16_t*)Bg)[(uint64_t)(K - 1u) * ldb + N - 1u];
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t row = maps::kc_piece_row(wave * 8u + i, lane);
@@ -414,6 +431,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // barrier (na, nb) is complete and (ca, cb) is free to be refilled with tile t+2.
                 MAIZE_FENCE();
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                if (PATCHES && patch_on && K - 1u - k_late < (uint32_t)BKE)    // tile t+1 holds row K - 1 (k_late <= K - 1 here)
+                    asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)nb + patch_off), "v"(patch_val) : "memory");
                 MAIZE_FENCE();
             }
 #pragma unroll
@@ -467,6 +486,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     // The wait also covers the C stores of the previous tile (loads and stores share the counter).
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    if (PATCHES && patch_on && nk && K - 1u - k_begin < (uint32_t)BKE)        // the item's first K tile is also B's last
+        asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)B0 + patch_off), "v"(patch_val) : "memory");
 #pragma unroll
     for (int r = 0; r < NAR; ++r) read_a(0, 0, 0, r);
 #pragma unroll
@@ -570,7 +591,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     const floatx4 lo = *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_read_offset(r, 0, lane));
                     const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_read_offset(r, 1, lane));
                     const uint32_t grow = em0 + wm * 128u + i * 32u + row;
-                    if (gcol < N && grow < M) {                   // N % 8 == 0: a run is all in or all out
+                    if (gcol < N && grow < M) {                   // direct C: N % 8 == 0, a run is all in or all out
                         if (SPLITK) {
                             // fp32 partial tile of this (tile, K range), row-major 256 x 256, behind the 64 KiB
                             // of ticket counters every workspace starts with (other kernels on the stream rely

@@ -176,12 +176,12 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (16, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",
         (17, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",        # more than 16 rows
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
-        (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_packed",      # odd N: B repacked, C written element-wise
-        (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",
+        (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",      # odd N: operands read where they lie, C written element-wise by the reduce pass
+        (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
         (4096, 4096, 4100, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",      # K % 8 != 0: both operands repacked
-        (511, 513, 1027, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_packed",
+        (511, 513, 1027, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_packed",       # K % 8 != 0 again
         (100, 203, 72, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",                  # too small to pay for the copies
-        (17, 50257, 768, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",                # 17 rows do not earn back a copy of B
+        (17, 50257, 768, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",       # no copy of B is needed: odd rows are read where they lie
     }
     for (m, n, k, layout, batch), want in picks.items():
         assert mz.gemm_plan(desc(m, n, k, layout, batch), compute_units=CUS)["kernel"] == want

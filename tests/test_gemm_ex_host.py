@@ -60,8 +60,13 @@ def test_dispatch_of_extended_descriptors():
     big = dict(m=4096, n=4096, k=4096)
     assert mz.gemm_plan(ex(**big, lda=4104, ldb=4224, ldc=8192))["kernel"] == "maize_gemm_bf16_mt256_nn"
     assert mz.gemm_plan(ex(**big, layout=mz.LAYOUT_NT, ldb=4104))["kernel"] == "maize_gemm_bf16_mt256_nt"
-    # rows that do not start on 16-byte boundaries: that operand is repacked first
-    assert mz.gemm_plan(ex(**big, lda=4100))["kernel"] == "maize_gemm_bf16_mt256_nn_packed"
+    # rows of A or B that do not start on 16-byte boundaries are read where they lie (the general-epilogue kernels) ...
+    assert mz.gemm_plan(ex(**big, lda=4100))["kernel"] == "maize_gemm_bf16_mt256_nn_gen"
+    # ... rows of C that are not 16-byte material go through the split-K kernels' reduce pass, one K range if splitting does not pay ...
+    p1 = mz.gemm_plan(ex(**big, ldc=4100))
+    assert p1["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p1["ksplit"] == 1 and p1["reduce_grid"] > 0
+    # ... and only K % 8 != 0 still needs padded copies
+    assert mz.gemm_plan(ex(4096, 4096, 4100))["kernel"] == "maize_gemm_bf16_mt256_nn_packed"
     assert mz.gemm_plan(ex(64, 64, 64, lda=68))["kernel"] == "maize_gemm_bf16_wave32"          # unless the product is small
     # alpha / beta / fp32 C: the macro-tile kernels with the general epilogue; the plain ones refuse
     for kw in (dict(alpha=0.5), dict(beta=1.0), dict(out_type=mz.OUT_F32)):
@@ -75,8 +80,8 @@ def test_dispatch_of_extended_descriptors():
     for kw in (dict(alpha=0.5, beta=2.0), dict(out_type=mz.OUT_F32), dict(ldb=14400, ldc=14344)):
         assert mz.gemm_plan(ex(16, 14336, 4096, **kw))["kernel"] == "maize_gemm_bf16_skinny_nn"
     assert mz.gemm_plan(ex(16, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_skinny_nn"   # rows of B on 8-byte boundaries: still streamed
-    assert mz.gemm_plan(ex(16, 14336, 4096, lda=4100))["kernel"] == "maize_gemm_bf16_wave32"      # rows of A off the 16-byte grid: 16 rows do not earn back a copy
-    assert mz.gemm_plan(ex(32, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_mt256_nn_packed"
+    assert mz.gemm_plan(ex(16, 14336, 4096, lda=4100))["kernel"] == "maize_gemm_bf16_mt256_nn_splitk"   # rows of A off the 16-byte grid: the macro-tile kernels read them where they lie
+    assert mz.gemm_plan(ex(32, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_mt256_nn_splitk"
 
 
 def _supports(name, x):

@@ -366,17 +366,20 @@ def test_packed_kernels_odd_extents(ctx, oracle, layout, shape):
 
 
 def test_packed_path_is_what_odd_large_shapes_get(ctx, oracle):
-    """The dispatcher's choice for large products that break the 16-byte rules, checked on sampled rows."""
+    """The dispatcher's choice for large products that break the 16-byte rules, checked on sampled rows: padded copies
+    only where K % 8 != 0 (a 16-byte chunk would straddle a row's end in K); an odd N alone needs none."""
     from tests.gpu_util import sample_rows
-    for (m, n, k, layout) in ((1024, 4099, 1024, mz.LAYOUT_NN), (1000, 5003, 776, mz.LAYOUT_NT), (2048, 2048, 1028, mz.LAYOUT_NN)):
+    for (m, n, k, layout, want) in ((1024, 4099, 1028, mz.LAYOUT_NN, "_packed"), (1000, 5003, 777, mz.LAYOUT_NT, "_packed"),
+                                    (2048, 2048, 1028, mz.LAYOUT_NN, "_packed"), (1024, 4099, 1024, mz.LAYOUT_NN, "_splitk"),
+                                    (1000, 5003, 776, mz.LAYOUT_NT, "_splitk")):
         brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
         a = mz.gen.uniform_bf16(m * k, 41)
         b = mz.gen.uniform_bf16(k * n, 42)
         da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(m * n * 2)
         d = mz.gemm_desc(mz.Matrix(da, m, k), mz.Matrix(db, brows, bcols), mz.Matrix(dc, m, n), layout=layout)
         took = ctx.gemm_select(d)
-        assert took.endswith("_packed"), took
-        _say(f"packed dispatch {m}x{n}x{k} -> {took}")
+        assert took.endswith(want), took
+        _say(f"odd large shape {m}x{n}x{k} -> {took}")
         ctx.gemm_bf16(d)
         ctx.sync()
         got = dc.download(np.uint16).reshape(m, n)
@@ -421,3 +424,52 @@ def test_workspace_is_shared_safely_between_kernel_families(ctx, oracle):
             check_against_oracle(oracle, got, a, b, m, n, k, label=name)
         else:
             check_rows_against_oracle(oracle, got, a, b, m, n, k, sample_rows(m, count=16), label=name)
+
+
+# ---- operands and C that are not 16-byte material, read and written where they lie ------------------------------------
+
+@pytest.mark.parametrize("case", [
+    dict(m=300, n=515, k=264), dict(m=300, n=515, k=264, layout=mz.LAYOUT_NT), dict(m=1000, n=1001, k=1024),
+    dict(m=1000, n=1001, k=1000, layout=mz.LAYOUT_NT), dict(m=520, n=777, k=4104), dict(m=64, n=4099, k=4096),
+    dict(m=512, n=512, k=512, lda=515), dict(m=512, n=512, k=512, ldb=517), dict(m=512, n=512, k=512, layout=mz.LAYOUT_NT, ldb=519),
+    dict(m=512, n=512, k=512, ldc=515), dict(m=512, n=520, k=512, lda=513, ldb=523, ldc=521, alpha=0.5, beta=-1.25),
+    dict(m=384, n=2051, k=1024, out_f32=True), dict(m=384, n=2051, k=1024, half=True),
+], ids=lambda c: "-".join(f"{k}{v}" for k, v in c.items()))
+def test_macro_tile_kernels_read_unaligned_operands_where_they_lie(ctx, oracle, case):
+    """Odd N, odd leading dimensions: no padded copies.  A and B go through the same 128-bit direct-to-LDS requests
+    (which may start on any even byte), C goes through the general epilogue when its rows are 16-byte material and
+    through the split-K kernels' reduce pass (one K range if splitting does not pay) when they are not."""
+    took = run_ex(ctx, oracle, label="unaligned", **case)
+    assert "_mt256_" in took and not took.endswith("_packed"), took
+    c_unaligned = case["n"] % 8 != 0 or case.get("ldc", 8) % 8 != 0
+    assert took.endswith("_splitk") or not c_unaligned, took
+
+
+def test_odd_n_last_element_of_b_meets_infinity_in_a(ctx, oracle):
+    """The dword holding B[K-1, N-1] straddles the end of B when N is odd and is answered with zero; the kernels write
+    the real element into the landed K tile.  With -Inf in A[M-1, K-1] and +Inf there, C[M-1, N-1] must be -Inf, not
+    NaN (0 x Inf), for one K range and for several, for a first-and-only K tile and for a long K."""
+    for (m, n, k) in ((300, 515, 64), (300, 515, 264), (260, 1001, 4096), (64, 4099, 4096)):
+        a = mz.gen.uniform_bf16(m * k, 5).reshape(m, k).copy()
+        b = mz.gen.uniform_bf16(k * n, 6).reshape(k, n).copy()
+        a[m - 1, k - 1] = 0xFF80
+        b[k - 1, n - 1] = 0x7F80
+        da, db, dc = ctx.upload(a), ctx.upload(b), ctx.malloc(2 * m * n)
+        try:
+            d = mz.gemm_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n), mz.Matrix(dc, m, n))
+            kern = "maize_gemm_bf16_mt256_nn_splitk"                        # (the smallest case would go to the any-shape kernel)
+            plan = mz.gemm_plan(d, kernel=kern, compute_units=ctx.info()["compute_units"])
+            _say(f"odd N, Inf in the patched element: {m}x{n}x{k} -> {plan['kernel']} ks={plan['ksplit']}")
+            ctx.gemm_bf16(d, kernel=kern)
+            ctx.sync()
+            got = dc.download(np.uint16).reshape(m, n)
+        finally:
+            da.free(); db.free(); dc.free()
+        ref, f64, ab = oracle.ref_gemm(a.ravel(), b.ravel(), m, n, k, want_f64=True, want_abs=True)
+        ref = ref.reshape(m, n)
+        assert got[m - 1, n - 1] == 0xFF80 == ref[m - 1, n - 1], hex(int(got[m - 1, n - 1]))
+        nan_g, nan_r = (got & 0x7FFF) > 0x7F80, (ref & 0x7FFF) > 0x7F80
+        assert np.array_equal(nan_g, nan_r), f"NaN sets differ: {int(nan_g.sum())} vs {int(nan_r.sum())}"
+        fin = (ref & 0x7FFF) < 0x7F80
+        s = oracle.compare(got[fin], ref[fin], f64.reshape(m, n)[fin], ab.reshape(m, n)[fin], k)
+        assert s["n_fail"] == 0, s
