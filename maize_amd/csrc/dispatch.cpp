@@ -446,10 +446,10 @@ bool trb_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims*
     return true;
 }
 
-// ---- maize_gemm_bf16_skinny_nn: M <= 16 against a row-major K x N B, streamed once ----------
-bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
+// ---- maize_gemm_bf16_skinny_nn (M <= 16), _m32, _m64: few rows against a row-major K x N B, streamed once ----------
+static bool skinny_nn_rows(const maize_gemm_ex_desc_t& d, uint32_t max_rows) {
     const Dims s = dims_of(d);
-    if (fp8_in(d) || wide_in(d) || d.gemm.layout != MAIZE_LAYOUT_NN || s.m > 16u || (s.k & 31u)) return false;
+    if (fp8_in(d) || wide_in(d) || d.gemm.layout != MAIZE_LAYOUT_NN || s.m > max_rows || (s.k & 31u)) return false;
     // A: 16-byte rows (its blocks are fetched 16 bytes per lane in fragment order).  B and C: any N, leading dimension
     // and 2-byte-aligned pointer -- the 128-bit requests for B may start on any even byte, C is stored element by
     // element when its rows are not 16-byte material (skinny_c_by_elements).
@@ -462,6 +462,9 @@ bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) {
     if (l.ext_a * 2 >= lim || l.ext_b * 2 >= lim || s.n >= (1u << 21) || l.b >= (1u << 21)) return false;
     return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
 }
+bool skinny_nn_supports(const maize_gemm_ex_desc_t& d) { return skinny_nn_rows(d, 16u); }
+bool skinny_nn_m32_supports(const maize_gemm_ex_desc_t& d) { return skinny_nn_rows(d, 32u); }
+bool skinny_nn_m64_supports(const maize_gemm_ex_desc_t& d) { return skinny_nn_rows(d, 64u); }
 // C rows that cannot take 128-bit stores: the kernel then writes C element by element (bit 0 of split_first).
 bool skinny_c_by_elements(const maize_gemm_ex_desc_t& d) {
     const Dims s = dims_of(d);
@@ -470,18 +473,20 @@ bool skinny_c_by_elements(const maize_gemm_ex_desc_t& d) {
     return (s.n & 7u) || (l.c % per16) || ((uintptr_t)d.gemm.c.ptr & 15u) || (d.gemm.batch > 1 && (d.gemm.stride_c % per16));
 }
 // K ranges: the smallest power of two that gives the grid at least 3/4 of a workgroup per
-// compute unit, as long as every range keeps at least 16 blocks of 32 rows.
+// compute unit, as long as every range keeps at least 16 blocks of 32 rows -- two turns of the ring.  (With 8 blocks
+// per range the last workgroup of a slab adds twice the tiles for a K loop that is hardly shorter: 16 x 4096 x 4096
+// takes 15.3 us in 16 ranges and 11.9 in 8; at K = 8192, 16 ranges of 16 blocks are as good as 8 or better.)
 uint32_t skinny_ksplit(const Dims& s, uint32_t batch, uint32_t compute_units) {
     const uint64_t slabs = (uint64_t)cdiv(s.n, 256) * batch;
     const uint32_t nblk = s.k / 32u;
     uint32_t ks = 1;
-    while (ks < 16u && slabs * ks * 4u < (uint64_t)compute_units * 3u && s.k / (2u * ks) >= 256u)
+    while (ks < 16u && slabs * ks * 4u < (uint64_t)compute_units * 3u && s.k / (2u * ks) >= 512u)
         ks *= 2;
     // ... and if that power of two spills into a second round, the largest count that still fits the first
     if (slabs * ks > compute_units && compute_units / slabs >= 1u) ks = (uint32_t)(compute_units / slabs);
     return cdiv(nblk, cdiv(nblk, ks));                     // no empty range
 }
-bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+static bool skinny_plan_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld, uint32_t rows) {
     const Dims s = dims_of(d);
     const uint32_t ks = skinny_ksplit(s, d.gemm.batch, compute_units ? compute_units : 256u);
     ld->grid[0] = cdiv(s.n, 256);
@@ -492,9 +497,12 @@ bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDi
     ld->ksplit = ks;
     ld->split_first = skinny_c_by_elements(d) ? 1u : 0u;
     ld->reduce_grid = 0;
-    ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * 16u * 256u * 4u : 0;
+    ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * rows * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
 }
+bool skinny_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) { return skinny_plan_rows(d, compute_units, ld, 16u); }
+bool skinny_m32_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) { return skinny_plan_rows(d, compute_units, ld, 32u); }
+bool skinny_m64_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) { return skinny_plan_rows(d, compute_units, ld, 64u); }
 
 // ---- maize_gemm_*_skinny_nt: M <= 16 against B stored N x K, streamed once ---------------------
 // 16-bit (bf16 / half by launch flag) or 8-bit operands; rows of A and B on 16-byte boundaries,
@@ -594,6 +602,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nn_ktail_edge", nullptr, mt256_nn_ktail_supports, mt256_edge_plan},
     {"maize_gemm_bf16_mt256_nt_ktail_edge", nullptr, mt256_nt_ktail_supports, mt256_edge_plan},
     {"maize_gemm_bf16_skinny_nn", nullptr, skinny_nn_supports, skinny_plan},
+    {"maize_gemm_bf16_skinny_nn_m32", nullptr, skinny_nn_m32_supports, skinny_m32_plan},
+    {"maize_gemm_bf16_skinny_nn_m64", nullptr, skinny_nn_m64_supports, skinny_m64_plan},
     {"maize_gemm_bf16_mt256_nn_gen", nullptr, mt256_nn_gen_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_gen", nullptr, mt256_nt_gen_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_ktail_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_plan},
@@ -686,6 +696,15 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // Few rows against a wide row-major B: bound by streaming B once.
     const int sk = kernel_index("maize_gemm_bf16_skinny_nn");
     if (sk >= 0 && kKernels[sk].supports(d) && s.n >= 64) return (uint32_t)sk;
+    // 17 .. 64 rows: the same stream with 2 or 4 row groups, where it beats the macro-tile kernel cut over K
+    // (measured): a long K, and enough slabs that few K ranges cover the chip -- the last workgroup of a slab adds
+    // ranges x row groups x 16 KiB alone.  32 rows: 1024 columns up (32 x 1024 x 8192: 20.3 against 25.1 us,
+    // 32 x 14336 x 4096: 25.1 against 34.8); 64 rows: 8192 columns up (64 x 14336 x 4096: 30.8 against 37.3 us, but
+    // 64 x 4096 x 4096: 26.3 against 23.2).
+    if (s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 8192u)) {
+        const int sm = kernel_index(s.m <= 32u ? "maize_gemm_bf16_skinny_nn_m32" : "maize_gemm_bf16_skinny_nn_m64");
+        if (sm >= 0 && kKernels[sm].supports(d) && plan_fits(kKernels[sm], d, compute_units)) return (uint32_t)sm;
+    }
     const int st = kernel_index("maize_gemm_bf16_skinny_nt");
     if (st >= 0 && kKernels[st].supports(d) && s.n >= 64 && s.k >= 512) return (uint32_t)st;
     // Few tiles and a long K: cut every tile into K ranges so that the whole chip works.

@@ -1,5 +1,6 @@
-// maize_gemm_bf16_skinny_nn: the memory-bound kernel for M <= 16 (decode-style GEMM
-// against a row-major K x N weight matrix).
+// maize_gemm_bf16_skinny_nn (M <= 16), _m32 (M <= 32), _m64 (M <= 64): the memory-bound kernels for few rows
+// (decode-style GEMM against a row-major K x N weight matrix).  One body, instantiated for 1, 2 or 4 groups of
+// 16 rows of A; the description below is for one group, the others differ in the A blocks and accumulators only.
 //
 // Every byte of B is streamed from HBM exactly once and nothing else of size moves, so the
 // kernel is built around long contiguous requests and a deep queue of them:
@@ -26,7 +27,7 @@
 //     the last one to arrive for a slab adds the partials in split order (deterministic),
 //     rounds once to bf16 (RNE), stores C and resets the ticket counter.
 //
-// Requirements (checked by the dispatcher): layout NN, M <= 16, K % 32 == 0 (any number of K ranges), rows of A on
+// Requirements (checked by the dispatcher): layout NN, M <= 16 (32, 64), K % 32 == 0 (any number of K ranges), rows of A on
 // 16-byte boundaries, every matrix (per batch member) below 2 GiB.  B and C may have any N, leading dimension and
 // 2-byte-aligned pointer: the 128-bit requests for B may start on any even byte (the hardware splits them), and C
 // is stored element by element when its rows are not 16-byte material.
@@ -56,6 +57,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 // f(r) = r%4 + 4*bit3(r), so the 8 rows one transposing read touches land in 8 different
 // granules of the 256-byte bank period.
 
+template <int MR>     // groups of 16 rows of A and C: 1, 2 or 4
 __device__ __forceinline__ void body(const GemmArgs& p) {
     // One array per ring slot: distinct objects let the compiler see that a load into one slot
     // does not alias reads of another.
@@ -67,21 +69,22 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     __shared__ __attribute__((aligned(1024))) char ring5[BLOCK_BYTES];
     __shared__ __attribute__((aligned(1024))) char ring6[BLOCK_BYTES];
     __shared__ __attribute__((aligned(1024))) char ring7[BLOCK_BYTES];
-    __shared__ uint32_t ticket;
     // A blocks (16 rows x 32 k = 1 KiB), one per ring slot, fetched once per workgroup: lane l of a direct-to-LDS load
     // asks for (row l % 16, k chunk l / 16) -- exactly the MFMA fragment of lane l -- and lands at 16 l, so every wave
-    // reads its A operand as one conflict-free 16-byte read at 16 l.  The block that goes into slot x is fetched by
+    // reads its A operand as one conflict-free 16-byte read at 16 l.  (Four neighbouring lanes fetching one row's 64
+    // bytes instead -- a quarter of the requests -- changed nothing.)  The block that goes into slot x is fetched by
     // wave x: the duty rotates, every wave issues 17 loads per ring turn, and the number of loads a wave may leave in
     // flight when it waits for a block is 12 or 13 depending on where its duty falls (turn()).  (Each wave fetching its own copy from L2 moved 8 KiB
-    // per 16 KiB block of B through the vector memory path and cost 0.5 us of 25.)
-    __shared__ __attribute__((aligned(1024))) char ablk0[1024];
-    __shared__ __attribute__((aligned(1024))) char ablk1[1024];
-    __shared__ __attribute__((aligned(1024))) char ablk2[1024];
-    __shared__ __attribute__((aligned(1024))) char ablk3[1024];
-    __shared__ __attribute__((aligned(1024))) char ablk4[1024];
-    __shared__ __attribute__((aligned(1024))) char ablk5[1024];
-    __shared__ __attribute__((aligned(1024))) char ablk6[1024];
-    __shared__ __attribute__((aligned(1024))) char ablk7[1024];
+    // per 16 KiB block of B through the vector memory path and cost 0.5 us of 25.)  With MR row groups a slot holds MR
+    // such blocks, 1 KiB apart, and group r of slot x is fetched by wave (x + r) % 8.
+    __shared__ __attribute__((aligned(1024))) char ablk0[MR * 1024];
+    __shared__ __attribute__((aligned(1024))) char ablk1[MR * 1024];
+    __shared__ __attribute__((aligned(1024))) char ablk2[MR * 1024];
+    __shared__ __attribute__((aligned(1024))) char ablk3[MR * 1024];
+    __shared__ __attribute__((aligned(1024))) char ablk4[MR * 1024];
+    __shared__ __attribute__((aligned(1024))) char ablk5[MR * 1024];
+    __shared__ __attribute__((aligned(1024))) char ablk6[MR * 1024];
+    __shared__ __attribute__((aligned(1024))) char ablk7[MR * 1024];
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
     const uint32_t lda = lda_of(p), ldb = ldb_of(p), ldc = ldc_of(p);
@@ -118,6 +121,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }
     // A operand of MFMA 16x16x32: lane l holds row l%16, k = 8*(l/16) + 0..7 of the block.
     const uint32_t a_vo = ((lane & 15u) * lda + (lane >> 4) * 8u) * 2u;  // rows >= M fall past the descriptor: zeros
+    const uint32_t a_rd = lane * 16u;
 
     // ---- transposing-read map.  In each group of 16 lanes, lane q addresses 4 consecutive
     // columns (q%4) of row (q/4) of a 4 x 16 sub-block and receives column q, rows 0..3.  Lane
@@ -149,9 +153,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     uint32_t patch_val = 0u;
     if (patch_wave) patch_val = Bg[(uint64_t)(K - 1u) * ldb + N - 1u];
 
-    floatx4 acc[2];
-    acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
-    acc[1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    floatx4 acc[MR][2];
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+        acc[r][0] = floatx4{0.f, 0.f, 0.f, 0.f};
+        acc[r][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
 
     // Requests block j (rows k0 + 32j ..) into `slot` -- two pieces per wave -- and, if this wave has the duty, its A
     // block into ablk[ai] first.  Blocks past the end read a zero-length descriptor.
@@ -164,7 +171,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // The fences pin the issue order (A block, piece, piece): the counter waits below
         // count loads in that order.
         __builtin_amdgcn_sched_barrier(0);
-        if (wave == (uint32_t)ai) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lvp)ablk[ai], 16, a_vo, kb * 2u, 0, 0);
+#pragma unroll
+        for (int r = 0; r < MR; ++r)      // row group r of this block is the duty of wave (ai + r) % 8
+            if (wave == (uint32_t)((ai + r) & 7))
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lvp)(ablk[ai] + r * 1024), 16, a_vo + (uint32_t)r * 32u * lda, kb * 2u, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -175,9 +185,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     auto consume = [&](lds_ptr slot, int ai) {
         // The reads are inline assembly so that the compiler sees no read of the ring: it would otherwise order every
         // read behind the direct-to-LDS loads in flight with a counter wait of its own, computed without the duty loads.
-        bf16x8 af;
+        bf16x8 af[MR];
         short4v lo[2], hi[2];
-        asm volatile("ds_read_b128 %0, %1" : "=v"(af) : "v"((uint32_t)(uintptr_t)ablk[ai] + lane * 16u));
+#pragma unroll
+        for (int r = 0; r < MR; ++r)
+            asm volatile("ds_read_b128 %0, %1" : "=v"(af[r]) : "v"((uint32_t)(uintptr_t)ablk[ai] + (uint32_t)r * 1024u + a_rd));
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {
             asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo[c2]) : "v"((uint32_t)(uintptr_t)slot + rd[0][c2]));
@@ -187,10 +199,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {
             short8v bb = {lo[c2][0], lo[c2][1], lo[c2][2], lo[c2][3], hi[c2][0], hi[c2][1], hi[c2][2], hi[c2][3]};
-            if (half_io)   // same bits, read as IEEE half (a wave-uniform choice)
-                acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, bb), __builtin_bit_cast(halfx8, af), acc[c2], 0, 0, 0);
-            else
-                acc[c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bb), af, acc[c2], 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                if (half_io)   // same bits, read as IEEE half (a wave-uniform choice)
+                    acc[r][c2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, bb), __builtin_bit_cast(halfx8, af[r]), acc[r][c2], 0, 0, 0);
+                else
+                    acc[r][c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bb), af[r], acc[r][c2], 0, 0, 0);
+            }
         }
     };
     // One block: wait until this wave's share of block b has landed (the loads of blocks b+1 .. b+6 may stay in
@@ -198,8 +213,24 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // block b+7, not requested yet), meet the other waves -- which also tells us everyone is done reading block
     // b-1 -- refill that block's slot with block b+7, then multiply block b.
     auto turn = [&](uint32_t b, lds_ptr cur, int ai, lds_ptr prev, int pi) {
-        if (wave == (uint32_t)ai || wave == (uint32_t)pi) asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(13)\n\ts_barrier" ::: "memory");
+        if constexpr (MR == 1) {
+            if (wave == (uint32_t)ai || wave == (uint32_t)pi) asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(13)\n\ts_barrier" ::: "memory");
+        } else {
+            // Row group r of the block in slot x is this wave's duty when x = (wave - r) % 8; of the slots ai+1 .. ai+6
+            // (blocks b+1 .. b+6, requested after block b's pieces) that is one load for every r whose distance
+            // (wave - r - ai) % 8 lies in 1 .. 6.
+            uint32_t later = 0;
+#pragma unroll
+            for (int r = 0; r < MR; ++r) later += (((wave - (uint32_t)r - (uint32_t)ai) & 7u) - 1u) < 6u ? 1u : 0u;
+            switch (later) {
+                case 0: asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory"); break;
+                case 1: asm volatile("s_waitcnt vmcnt(13)\n\ts_barrier" ::: "memory"); break;
+                case 2: asm volatile("s_waitcnt vmcnt(14)\n\ts_barrier" ::: "memory"); break;
+                case 3: asm volatile("s_waitcnt vmcnt(15)\n\ts_barrier" ::: "memory"); break;
+                default: asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory"); break;
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);
         request(b + 7, prev, pi);
         if (patch_wave && b + 1u == nb) {
@@ -234,67 +265,92 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     if (ks == 1u) {
         // Single split: straight from registers, 8 bytes per lane.
 #pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2) {
-            const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
-            if (m < M && col < N) {
-                const float v[4] = {acc[c2][0], acc[c2][1], acc[c2][2], acc[c2][3]};
-                if (c_elems) store_c_elems<4>(p, Cg, (uint64_t)m * ldc + col, v, N - col);
-                else store_c_run<4>(p, Cg, (uint64_t)m * ldc + col, v);
+        for (int r = 0; r < MR; ++r)
+#pragma unroll
+            for (int c2 = 0; c2 < 2; ++c2) {
+                const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
+                const uint32_t row = 16u * r + m;
+                if (row < M && col < N) {
+                    const float v[4] = {acc[r][c2][0], acc[r][c2][1], acc[r][c2][2], acc[r][c2][3]};
+                    if (c_elems) store_c_elems<4>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
+                    else store_c_run<4>(p, Cg, (uint64_t)row * ldc + col, v);
+                }
             }
-        }
         return;
     }
-    // Workspace: 16384 ticket counters (zero between launches), then one fp32 tile of 16 x 256
+    // Workspace: 16384 ticket counters (zero between launches), then one fp32 tile of 16 MR x 256
     // per (batch member, slab, split).  The tiles are written and read with device-coherent
     // accesses (they cross the per-XCD L2s), so no cache-wide write-back or invalidate is needed:
     // each wave waits for its own stores, the barrier collects the waves, then one thread takes
     // the ticket with a device-scope atomic.
+    //
+    // The last workgroup to arrive adds all the tiles of its slab.  One workgroup draws about 50 GB/s of such data,
+    // so this costs ks x MR x 16 KiB at that rate with the rest of the chip idle (1.3 us for 16 rows and 4 ranges,
+    // 5 us for 64 rows).  Sharing the additions among the slab's workgroups (each waits, with a bound, until all
+    // have arrived and adds the part its arrival number names) was built and measured: the polling loads and the
+    // two more atomics per workgroup on the slab's counters cost 1.2 us at 16 rows x 4 ranges (22.8 against 21.6 us)
+    // and 2 us at 8 ranges of an 8192 x 8192 B; it won only from 16 ranges or 64 rows up (-1.7 us), so it stayed out.
     constexpr int COHERENT = 17;                          // buffer cache policy: sc0 | sc1
-    constexpr uint32_t TILE_BYTES = 16u * SN * 4u;
+    constexpr uint32_t TILE_BYTES = 16u * MR * SN * 4u;
+    typedef __attribute__((address_space(3))) volatile uint32_t* lds_word_ptr;
+    lds_word_ptr const ticket = (lds_word_ptr)ablk0;     // the A blocks are idle from here on (with four row groups
+                                                          // the ring and the A blocks fill the 160 KiB of LDS to the byte)
     uint32_t* counters = (uint32_t*)p.workspace;
     const uint32_t slab_id = (uint32_t)bz * gridDim.x + slab;
     const __amdgpu_buffer_rsrc_t rws =
         make_rsrc((const char*)p.workspace + 65536, gridDim.z * gridDim.x * ks * TILE_BYTES);
     const uint32_t tile0 = slab_id * ks * TILE_BYTES;     // byte offset of this slab's split-0 tile
 #pragma unroll
-    for (int c2 = 0; c2 < 2; ++c2)
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[c2]), rws,
-                                               tile0 + z * TILE_BYTES + (m * SN + (wave * 2u + c2) * 16u + g * 4u) * 4u,
-                                               0, COHERENT);
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[r][c2]), rws,
+                                                   tile0 + z * TILE_BYTES + ((16u * r + m) * SN + (wave * 2u + c2) * 16u + g * 4u) * 4u,
+                                                   0, COHERENT);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wave's partial tile has reached memory
     __syncthreads();
-    if (tid == 0) ticket = __hip_atomic_fetch_add(&counters[slab_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) *ticket = __hip_atomic_fetch_add(&counters[slab_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (ticket != ks - 1u) return;                        // not the last split of this slab to finish
+    if (*ticket != ks - 1u) return;                       // not the last split of this slab to finish
     {
-        const uint32_t row = tid >> 5, cq = (tid & 31u) * 8u;     // 512 threads x 8 columns = 16 x 256
-        const uint32_t off = tile0 + (row * SN + cq) * 4u;
-        // The partial tiles are requested four splits at a time, so a slab pays one memory round
-        // trip per group rather than one per split; the additions still run in split order.
+        // 512 threads x 8 columns = 16 x 256 per row group; thread t adds rows 16 r + t / 32.  The partial tiles are
+        // requested ZG splits at a time for all row groups at once (ZG x MR x 2 128-bit loads in flight per lane),
+        // so a slab pays one memory round trip per ZG splits; the additions still run in split order.
+        constexpr int ZG = MR == 4 ? 4 : 8;
         constexpr uint32_t DROP = 0xFFFFFFE0u;                    // past the descriptor: reads as zeros
-        floatx4 s_lo = floatx4{0.f, 0.f, 0.f, 0.f}, s_hi = floatx4{0.f, 0.f, 0.f, 0.f};
-        for (uint32_t z0 = 0; z0 < ks; z0 += 4u) {
-            floatx4 t_lo[4], t_hi[4];
+        const uint32_t cq = (tid & 31u) * 8u;
+        const uint32_t off = tile0 + ((tid >> 5) * SN + cq) * 4u;
+        floatx4 s_lo[MR], s_hi[MR];
+        for (uint32_t z0 = 0; z0 < ks; z0 += ZG) {
+            floatx4 t_lo[MR][ZG], t_hi[MR][ZG];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t o = z0 + u < ks ? off + (z0 + u) * TILE_BYTES : DROP;
-                t_lo[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o, 0, COHERENT));
-                t_hi[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o + 16u, 0, COHERENT));
-            }
+            for (int u = 0; u < ZG; ++u)
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (z0 + u == 0u) { s_lo = t_lo[0]; s_hi = t_hi[0]; }
-                else if (z0 + u < ks) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) { s_lo[e] += t_lo[u][e]; s_hi[e] += t_hi[u][e]; }
+                for (int r = 0; r < MR; ++r) {
+                    const uint32_t o = z0 + u < ks ? off + (z0 + u) * TILE_BYTES + (uint32_t)r * (16u * SN * 4u) : DROP;
+                    t_lo[r][u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o, 0, COHERENT));
+                    t_hi[r][u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o + 16u, 0, COHERENT));
                 }
-            }
+#pragma unroll
+            for (int u = 0; u < ZG; ++u)
+#pragma unroll
+                for (int r = 0; r < MR; ++r) {
+                    if (z0 + u == 0u) { s_lo[r] = t_lo[r][0]; s_hi[r] = t_hi[r][0]; }
+                    else if (z0 + u < ks) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { s_lo[r][e] += t_lo[r][u][e]; s_hi[r][e] += t_hi[r][u][e]; }
+                    }
+                }
         }
         const uint32_t col = n0 + cq;
-        if (row < M && col < N) {
-            const float v[8] = {s_lo[0], s_lo[1], s_lo[2], s_lo[3], s_hi[0], s_hi[1], s_hi[2], s_hi[3]};
-            if (c_elems) store_c_elems<8>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
-            else store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);      // N % 8 == 0: 8 columns are all in or all out
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+            const uint32_t row = 16u * r + (tid >> 5);
+            if (row < M && col < N) {
+                const float v[8] = {s_lo[r][0], s_lo[r][1], s_lo[r][2], s_lo[r][3], s_hi[r][0], s_hi[r][1], s_hi[r][2], s_hi[r][3]};
+                if (c_elems) store_c_elems<8>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
+                else store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);      // 8 columns are all in or all out
+            }
         }
     }
     if (tid == 0) counters[slab_id] = 0u;                 // ready for the next launch
@@ -302,6 +358,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
 }  // namespace skinny
 
-extern "C" __global__ __launch_bounds__(512) void maize_gemm_bf16_skinny_nn(GemmArgs p) { skinny::body(p); }
+extern "C" __global__ __launch_bounds__(512) void maize_gemm_bf16_skinny_nn(GemmArgs p) { skinny::body<1>(p); }
+extern "C" __global__ __launch_bounds__(512) void maize_gemm_bf16_skinny_nn_m32(GemmArgs p) { skinny::body<2>(p); }
+extern "C" __global__ __launch_bounds__(512) void maize_gemm_bf16_skinny_nn_m64(GemmArgs p) { skinny::body<4>(p); }
 
 }  // namespace maize

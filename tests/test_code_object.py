@@ -84,20 +84,22 @@ def test_matrix_instruction_per_kernel(kernels):
             per_tile = 64 if "_f64_" in name else 128
             assert count(ins, want) == 2 * per_tile and count(ins, "v_mfma") == 2 * per_tile, name
             assert count(ins, "buffer_load_dwordx4") >= 16, name      # operands by buffer loads (range-checked edges), two tiles' worth
-        elif name == "maize_gemm_bf16_skinny_nn":
-            assert count(ins, "v_mfma_f32_16x16x32_bf16") >= 16 and count(ins, "v_mfma_f32_16x16x32_f16") >= 16
+        elif name.startswith("maize_gemm_bf16_skinny_nn"):
+            groups = {"maize_gemm_bf16_skinny_nn": 1, "maize_gemm_bf16_skinny_nn_m32": 2, "maize_gemm_bf16_skinny_nn_m64": 4}[name]
+            # 8 turns of the ring x 2 column groups x row groups
+            assert count(ins, "v_mfma_f32_16x16x32_bf16") >= 16 * groups and count(ins, "v_mfma_f32_16x16x32_f16") >= 16 * groups
         elif name == "maize_gemm_bf16_wave32":
             assert count(ins, "v_mfma_f32_32x32x16_bf16") >= 1 and count(ins, "v_mfma_f32_32x32x16_f16") >= 1
 
 
 def test_data_movement_the_design_rests_on(kernels):
     for name, ins in kernels.items():
-        if "_mt256_" in name or name == "maize_gemm_bf16_skinny_nn":
+        if "_mt256_" in name or name.startswith("maize_gemm_bf16_skinny_nn"):
             lds_dma = [i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]
             assert len(lds_dma) >= 16, f"{name}: operands must reach LDS by 128-bit direct-to-LDS loads"
             fp32_staging = "_gen" in name or "_splitk" in name
             assert count(ins, "ds_write_b128") == 0 or fp32_staging, name   # no register round trip for operands
-        if "_mt256_nn" in name or name == "maize_gemm_bf16_skinny_nn":
+        if "_mt256_nn" in name or name.startswith("maize_gemm_bf16_skinny_nn"):
             assert count(ins, "ds_read_b64_tr_b16") >= 8, f"{name}: a row-major K x N B is read with transposing reads"
         if "_mt256_nt" in name:
             assert count(ins, "ds_read_b64_tr_b16") == 0 and count(ins, "ds_read_b128") >= 16, name

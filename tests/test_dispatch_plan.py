@@ -128,9 +128,10 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert nedge <= 16384
             assert p["workspace_bytes"] >= TICKET_BYTES + nedge * ks * 256 * 256 * 4
             assert p["workspace_bytes"] < (1 << 31)
-    elif name == "maize_gemm_bf16_skinny_nn":
+    elif name.startswith("maize_gemm_bf16_skinny_nn"):
+        rows = {"maize_gemm_bf16_skinny_nn": 16, "maize_gemm_bf16_skinny_nn_m32": 32, "maize_gemm_bf16_skinny_nn_m64": 64}[name]
         assert p["block"] == (512, 1, 1)
-        assert layout == mz.LAYOUT_NN and m <= 16 and n % 8 == 0
+        assert layout == mz.LAYOUT_NN and m <= rows and n % 8 == 0
         ks = p["ksplit"]
         assert gx == cdiv(n, 256) and gy == ks and 1 <= ks <= 16
         assert k % 32 == 0                                     # whole 32-row blocks
@@ -140,7 +141,7 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         if ks > 1:
             assert nblk // ks >= 8                             # the 8-slot ring is filled at least once
             assert gx * batch <= 16384                         # one ticket counter per (batch member, slab)
-            assert p["workspace_bytes"] >= TICKET_BYTES + gx * batch * ks * 16 * 256 * 4
+            assert p["workspace_bytes"] >= TICKET_BYTES + gx * batch * ks * rows * 256 * 4
             assert p["workspace_bytes"] < (1 << 31)
         else:
             assert p["workspace_bytes"] == 0

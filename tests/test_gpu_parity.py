@@ -469,6 +469,37 @@ def test_skinny_nn_takes_any_n(ctx, oracle, shape):
     check_against_oracle(oracle, got, a, b, m, n, k, label=f"skinny_nn {shape}")
 
 
+@pytest.mark.parametrize("shape", [(32, 14336, 4096), (17, 2048, 1024), (29, 4099, 2080), (32, 256, 64), (5, 515, 288), (24, 512, 16384),
+                                   (64, 14336, 4096), (33, 2048, 1024), (50, 4101, 2080), (64, 256, 32), (47, 50257, 768), (64, 1024, 8192)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_skinny_nn_with_two_and_four_row_groups(ctx, oracle, shape):
+    """17 .. 64 rows against a row-major K x N B: the streaming kernel with 2 or 4 groups of 16 rows (A blocks of 2 or
+    4 KiB per ring slot, fetched by rotating duty; partial tiles of 32 or 64 rows).  Every output is checked: whole
+    and ragged row groups, one and many K ranges, odd N."""
+    m, n, k = shape
+    kernel = "maize_gemm_bf16_skinny_nn_m32" if m <= 32 else "maize_gemm_bf16_skinny_nn_m64"
+    a, b = inputs(m, n, k, dist="normal")
+    d = mz.gemm_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x1000, k, n), mz.GlobalMatrix(0x1000, m, n))
+    plan = mz.gemm_plan(d, kernel=kernel, compute_units=ctx.info()["compute_units"])
+    _say(f"{kernel}: {shape} {plan['grid']} ks={plan['ksplit']}")
+    got = run_gemm(ctx, a, b, m, n, k, kernel=kernel)
+    check_against_oracle(oracle, got, a, b, m, n, k, label=f"{kernel} {shape}")
+    if m > 16 and k >= 1024 and n >= (1024 if m <= 32 else 8192):
+        assert mz.gemm_plan(d, compute_units=256)["kernel"] == kernel
+        assert np.array_equal(run_gemm(ctx, a, b, m, n, k), got)      # the dispatcher's launch is this one
+
+
+def test_skinny_nn_row_groups_agree_with_the_one_group_kernel(ctx):
+    """The same 16 rows through the kernels with 1, 2 and 4 row groups: identical K ranges and summation order, so
+    identical bits (the extra row groups read zeros past the end of A and are not stored)."""
+    m, n, k = 16, 3080, 4096
+    a, b = inputs(m, n, k, dist="normal")
+    one = run_gemm(ctx, a, b, m, n, k, kernel="maize_gemm_bf16_skinny_nn")
+    for kernel in ("maize_gemm_bf16_skinny_nn_m32", "maize_gemm_bf16_skinny_nn_m64"):
+        _say(f"{kernel} on 16 rows")
+        assert np.array_equal(run_gemm(ctx, a, b, m, n, k, kernel=kernel), one), kernel
+
+
 def test_skinny_nn_unaligned_b_and_c(ctx, oracle):
     """B at a 2-byte offset with an odd leading dimension, C at an odd offset: same kernel, same bar, nothing written
     outside C."""

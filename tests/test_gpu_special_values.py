@@ -34,10 +34,15 @@ FAMILIES = [
     ("maize_gemm_bf16_skinny_nn", 13, 520, 2080, NN),
     ("maize_gemm_bf16_skinny_nn", 13, 515, 2080, NN),               # odd N: the last element of B is patched into the landed block
     ("maize_gemm_bf16_skinny_nn", 16, 262, 4096, NN),
+    ("maize_gemm_bf16_skinny_nn_m32", 29, 515, 2080, NN),           # two row groups, one K range, odd N
+    ("maize_gemm_bf16_skinny_nn_m32", 32, 520, 4096, NN),
+    ("maize_gemm_bf16_skinny_nn_m64", 50, 519, 2080, NN),           # four row groups
+    ("maize_gemm_bf16_skinny_nn_m64", 64, 264, 8192, NN),
     ("maize_gemm_bf16_skinny_nt", 16, 515, 1096, NT),
     ("maize_gemm_bf16_wave32", 33, 17, 65, NN),
     ("maize_gemm_bf16_wave32", 33, 17, 65, NT),
     (None, 16, 14336, 4096, NN),
+    (None, 48, 8200, 1024, NN),
     (None, 1000, 1000, 1000, NN),
     (None, 24, 257, 4100, NT),
 ]

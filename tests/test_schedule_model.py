@@ -279,33 +279,44 @@ def test_8bit_macro_tile_checker_rejects_broken_schedules():
 
 
 # ---------------------------------------------------------------------------------------
-# skinny kernel: 8-slot ring, per wave 2 pieces per block plus the A block of the slot whose index is the wave's
-# (the duty rotates), counter wait instead of wait-all
+# skinny kernels (1, 2 or 4 groups of 16 rows): 8-slot ring, per wave 2 pieces per block plus the A blocks it has the
+# duty for (row group r of the block in slot x is fetched by wave (x + r) % 8), counter wait instead of wait-all
 # ---------------------------------------------------------------------------------------
 
 def skinny_constants():
     src = open(os.path.join(KDIR, "gemm_skinny.hpp")).read()
     ring = int(re.search(r"constexpr int RING = (\d+);", src).group(1))
     waits = [int(x) for x in re.findall(r"s_waitcnt vmcnt\((\d+)\)\\n\\ts_barrier", src)]
-    assert len(waits) == 2                  # with and without an A block among the loads that may stay in flight
+    # one row group: two waits, with and without an A block among the loads that may stay in flight; more row
+    # groups: 12 pieces plus 0 .. 4 A blocks, picked by a count
+    assert waits[:2] == [12, 13] and waits[2:] == [12, 13, 14, 15, 16]
     # the duty rule and the rule that picks the wait, as written in the kernel
-    assert "if (wave == (uint32_t)ai) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a" in src
-    assert re.search(r"if \(wave == \(uint32_t\)ai \|\| wave == \(uint32_t\)pi\) asm volatile\(\"s_waitcnt vmcnt\(%d\)" % min(waits), src)
+    assert "if (wave == (uint32_t)((ai + r) & 7))" in src
+    assert re.search(r"if \(wave == \(uint32_t\)ai \|\| wave == \(uint32_t\)pi\) asm volatile\(\"s_waitcnt vmcnt\(12\)", src)
+    assert "later += (((wave - (uint32_t)r - (uint32_t)ai) & 7u) - 1u) < 6u ? 1u : 0u;" in src
+    for n in range(5):
+        assert re.search(r"(case %d|default): asm volatile\(\"s_waitcnt vmcnt\(%d\)" % (n, 12 + n), src)
     primed = len(re.findall(r"request\(\d+, s\d+, \d+\);", src))
-    return ring, (min(waits), max(waits)), primed
+    return ring, (12, 13), primed
 
 
-def skinny_wave_program(nb, ring, waits, primed, wave=0):
+def skinny_wait(wave, cur, refill, waits, mr):
+    """The counter value a wave waits for before block `cur`'s barrier, as the kernel picks it."""
+    if mr == 1:
+        return waits[0] if wave in (cur, refill) else waits[1]
+    return 12 + sum(1 for r in range(mr) if 0 <= ((wave - r - cur) & 7) - 1 < 6)
+
+
+def skinny_wave_program(nb, ring, waits, primed, wave=0, mr=1):
     """The program of one wave: ("request", block, slot, loads), ("wait", n), ("barrier",), ("consume", block, slot)."""
-    short, long_ = waits
-    loads = lambda slot: 3 if slot == wave else 2
+    loads = lambda slot: 2 + sum(1 for r in range(mr) if (slot + r) % 8 == wave)
     ops = []
     for j in range(primed):
         ops.append(("request", j, j % ring, loads(j % ring)))
     turns = -(-nb // ring) * ring
     for b in range(turns):
         cur, refill = b % ring, (b + primed) % ring
-        ops += [("wait", short if wave in (cur, refill) else long_), ("barrier",)]
+        ops += [("wait", skinny_wait(wave, cur, refill, waits, mr)), ("barrier",)]
         ops.append(("request", b + primed, refill, loads(refill)))
         ops.append(("consume", b, cur))
     ops.append(("wait", 0))
@@ -358,12 +369,13 @@ def check_ring(ops, turns, loads_per_request, ring):
         raise Hazard("blocks not requested exactly once")
 
 
+@pytest.mark.parametrize("mr", [1, 2, 4])
 @pytest.mark.parametrize("nb", [8, 16, 32, 128, 9])
-def test_skinny_ring_is_hazard_free(nb):
+def test_skinny_ring_is_hazard_free(nb, mr):
     ring, waits, primed = skinny_constants()
     assert primed == ring - 1
     for wave in range(8):
-        ops, turns, lpr = skinny_wave_program(nb, ring, waits, primed, wave)
+        ops, turns, lpr = skinny_wave_program(nb, ring, waits, primed, wave, mr)
         check_ring(ops, turns, lpr, ring)
         # every wait is exact: it leaves just the loads issued after the current block's in flight
         issued = []
@@ -387,6 +399,11 @@ def test_skinny_checker_rejects_broken_rings():
         ops, turns, lpr = skinny_wave_program(32, ring, (waits[1], waits[1]), primed, wave)           # ignores where the duty falls
         with pytest.raises(Hazard):
             check_ring(ops, turns, lpr, ring)
+        for mr in (2, 4):               # more row groups: the wait of the one-group kernel leaves an A block unaccounted for
+            ops, turns, lpr = skinny_wave_program(32, ring, waits, primed, wave, mr)
+            lax = [("wait", o[1] + 1) if o[0] == "wait" and o[1] else o for o in ops]
+            with pytest.raises(Hazard):
+                check_ring(lax, turns, lpr, ring)
     ops, turns, lpr = skinny_wave_program(32, ring - 1, waits, primed)       # ring one slot short: refill hits the block being read
     with pytest.raises(Hazard):
         check_ring(ops, turns, lpr, ring - 1)
