@@ -31,7 +31,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 # run's kernel is that one, together with its source file.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_fetch_write_size.md"
 MEASURED_TRAFFIC = {"cfg1": ("maize_gemm_bf16_mt256_nn", 235.2e6), "cfg2": ("maize_gemm_bf16_mt256_nn_edge", 275.1e6),
-                    "cfg3": ("maize_gemm_bf16_mt256_nt", 1746.3e6), "cfg4": ("maize_gemm_bf16_skinny_nn", 126.4e6),
+                    "cfg3": ("maize_gemm_bf16_mt256_nt", 1746.3e6), "cfg4": ("maize_gemm_bf16_skinny_nn", 126.5e6),
+                    "m64": ("maize_gemm_bf16_skinny_nn_m64", 153.2e6),
                     "cfg5": ("maize_gemm_bf16_mt256_nn", 1074.3e6), "f8": ("maize_gemm_e4m3_mt256_nt", 134.5e6),
                     "f8s": ("maize_gemm_e4m3_skinny_nt", 67.2e6), "f32": ("maize_gemm_f32_mt128_nn", 828.9e6),
                     "f64": ("maize_gemm_f64_mt128_nn", 3162.3e6)}
@@ -46,6 +47,9 @@ CONFIGS = {
                  bound="mfma", label="bf16 GEMM 8192x8192x8192 NT, N(0,1)/sqrt(K)"),
     "cfg4": dict(m=16, n=14336, k=4096, nt=0, batch=1, da=("normal", 1.0), db=("normal", 0.02), bound="hbm",
                  label="bf16 GEMM 16x14336x4096 NN skinny, A~N(0,1), B~N(0,0.02)"),
+    # cfg4's weights against 64 rows: the four-row-group version of the streaming kernel.
+    "m64": dict(m=64, n=14336, k=4096, nt=0, batch=1, da=("normal", 1.0), db=("normal", 0.02), bound="hbm",
+                label="bf16 GEMM 64x14336x4096 NN few rows, A~N(0,1), B~N(0,0.02)"),
     "cfg5": dict(m=2048, n=2048, k=2048, nt=0, batch=32, da=("uniform",), db=("uniform",), bound="mfma",
                  label="bf16 strided-batched GEMM 32 x 2048^3 NN, uniform[-1,1)"),
     # Beside the five bf16 configurations: the same product on 8-bit operands (E4M3), both K-contiguous.
