@@ -507,11 +507,11 @@ bool skinny_m64_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Laun
 // ---- maize_gemm_*_skinny_nt: M <= 16 against B stored N x K, streamed once ---------------------
 // 16-bit (bf16 / half by launch flag) or 8-bit operands; rows of A and B on 16-byte boundaries,
 // K % 8 == 0 (16-bit) or K % 16 == 0 (8-bit), N % 8 == 0.
-bool skinny_nt_common(const maize_gemm_ex_desc_t& d) {
+bool skinny_nt_common(const maize_gemm_ex_desc_t& d, uint32_t max_rows = 16u) {
     const Dims s = dims_of(d);
     const Lds l = lds_of(d);
     const uint32_t esz = fp8_in(d) ? 1u : 2u, per16 = 16u / esz;
-    if (nn(d) || s.m > 16u || (s.k % per16)) return false;
+    if (nn(d) || s.m > max_rows || (s.k % per16)) return false;
     if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr) & 15u) return false;
     if ((l.a % per16) || (l.b % per16)) return false;              // C: any N, leading dimension and pointer (skinny_nt_c_by_elements)
     if (d.gemm.batch > 1 && ((d.gemm.stride_a % per16) || (d.gemm.stride_b % per16))) return false;
@@ -521,8 +521,12 @@ bool skinny_nt_common(const maize_gemm_ex_desc_t& d) {
 }
 bool skinny_nt_c_by_elements(const maize_gemm_ex_desc_t& d) { return skinny_c_by_elements(d); }
 bool skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d); }
+bool skinny_nt_m32_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d, 32u); }
+bool skinny_nt_m64_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d, 64u); }
 #define MAIZE_F8_SKINNY(tag, type) \
-    bool tag##_skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d); }
+    bool tag##_skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d); } \
+    bool tag##_skinny_nt_m32_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d, 32u); } \
+    bool tag##_skinny_nt_m64_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d, 64u); }
 MAIZE_F8_SKINNY(e4m3, MAIZE_IN_E4M3)
 MAIZE_F8_SKINNY(e5m2, MAIZE_IN_E5M2)
 MAIZE_F8_SKINNY(e4m3e5m2, MAIZE_IN_E4M3_E5M2)
@@ -531,7 +535,7 @@ MAIZE_F8_SKINNY(e5m2e4m3, MAIZE_IN_E5M2_E4M3)
 // K ranges: the smallest power of two that gives the grid 3/4 of a workgroup per compute unit (one round at
 // 0.75-1 workgroup per unit measures 10-25 % faster than the next power of two's 1.5-1.75 rounds) while
 // every range keeps at least 8 blocks of 128 bytes per row.
-bool skinny_nt_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+static bool skinny_nt_plan_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld, uint32_t rows) {
     const Dims s = dims_of(d);
     const uint32_t cus = compute_units ? compute_units : 256u;
     const uint32_t nblk = cdiv(s.k, fp8_in(d) ? 128u : 64u);
@@ -550,9 +554,12 @@ bool skinny_nt_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Launc
     ld->ksplit = ks;
     ld->split_first = skinny_nt_c_by_elements(d) ? 1u : 0u;
     ld->reduce_grid = 0;
-    ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * 16u * 256u * 4u : 0;
+    ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * rows * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
 }
+bool skinny_nt_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) { return skinny_nt_plan_rows(d, compute_units, ld, 16u); }
+bool skinny_nt_m32_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) { return skinny_nt_plan_rows(d, compute_units, ld, 32u); }
+bool skinny_nt_m64_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) { return skinny_nt_plan_rows(d, compute_units, ld, 64u); }
 
 // ---- maize_gemm_{f32,f64}_mt128_{nn,nt}: fp32 / fp64 operands, any shape ---------------------
 // 128 x 128 tiles, one workgroup each (x = tiles, XCD-aware order inside the kernel; z = batch).  Rows that
@@ -621,8 +628,12 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nn_splitk", packed_f16_nn_supports, packed_plan},
     {"maize_gemm_f16_mt256_nt_packed", "maize_gemm_f16_mt256_nt_splitk", packed_f16_nt_supports, packed_plan},
     {"maize_gemm_bf16_skinny_nt", nullptr, skinny_nt_supports, skinny_nt_plan},
+    {"maize_gemm_bf16_skinny_nt_m32", nullptr, skinny_nt_m32_supports, skinny_nt_m32_plan},
+    {"maize_gemm_bf16_skinny_nt_m64", nullptr, skinny_nt_m64_supports, skinny_nt_m64_plan},
 #define MAIZE_F8_ENTRIES(tag) \
     {"maize_gemm_" #tag "_skinny_nt", nullptr, tag##_skinny_nt_supports, skinny_nt_plan}, \
+    {"maize_gemm_" #tag "_skinny_nt_m32", nullptr, tag##_skinny_nt_m32_supports, skinny_nt_m32_plan}, \
+    {"maize_gemm_" #tag "_skinny_nt_m64", nullptr, tag##_skinny_nt_m64_supports, skinny_nt_m64_plan}, \
     {"maize_gemm_" #tag "_mt256_nt", nullptr, tag##_nt_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_gen", nullptr, tag##_nt_gen_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan}, \
@@ -670,6 +681,12 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nt", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fk = kernel_index(name);
         if (fk >= 0 && kKernels[fk].supports(d) && s.n >= 64 && s.k >= 1024) return (uint32_t)fk;
+        // 17 .. 64 rows: the same stream with 2 or 4 row groups (A through LDS), where B is what bounds the product.
+        if (s.m > 16u && s.m <= 64u && s.k >= 2048u && s.n >= (s.m <= 32u ? 1024u : 10240u)) {
+            std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nt_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.m <= 32u ? "m32" : "m64");
+            const int fm = kernel_index(name);
+            if (fm >= 0 && kKernels[fm].supports(d) && plan_fits(kKernels[fm], d, compute_units)) return (uint32_t)fm;
+        }
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_splitk", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fs = kernel_index(name);
         if (fs >= 0 && kKernels[fs].supports(d) && splitk_ranges(s, d.gemm.batch, compute_units, 128) >= 2u) return (uint32_t)fs;
@@ -699,14 +716,19 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // 17 .. 64 rows: the same stream with 2 or 4 row groups, where it beats the macro-tile kernel cut over K
     // (measured): a long K, and enough slabs that few K ranges cover the chip -- the last workgroup of a slab adds
     // ranges x row groups x 16 KiB alone.  32 rows: 1024 columns up (32 x 1024 x 8192: 20.3 against 25.1 us,
-    // 32 x 14336 x 4096: 25.1 against 34.8); 64 rows: 8192 columns up (64 x 14336 x 4096: 30.8 against 37.3 us, but
-    // 64 x 4096 x 4096: 26.3 against 23.2).
-    if (s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 8192u)) {
+    // 32 x 14336 x 4096: 25.1 against 34.8); 64 rows: 10240 columns up (64 x 14336 x 4096: 30.8 against 37.3 us, but
+    // 64 x 4096 x 4096: 26.3 against 23.2, and 64 x 8192 x 8192 N x K: 35.6 against 33.3).  The same thresholds serve
+    // the kernels for weights stored N x K below.
+    if (s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 10240u)) {
         const int sm = kernel_index(s.m <= 32u ? "maize_gemm_bf16_skinny_nn_m32" : "maize_gemm_bf16_skinny_nn_m64");
         if (sm >= 0 && kKernels[sm].supports(d) && plan_fits(kKernels[sm], d, compute_units)) return (uint32_t)sm;
     }
     const int st = kernel_index("maize_gemm_bf16_skinny_nt");
     if (st >= 0 && kKernels[st].supports(d) && s.n >= 64 && s.k >= 512) return (uint32_t)st;
+    if (s.nt && s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 10240u)) {
+        const int sm = kernel_index(s.m <= 32u ? "maize_gemm_bf16_skinny_nt_m32" : "maize_gemm_bf16_skinny_nt_m64");
+        if (sm >= 0 && kKernels[sm].supports(d) && plan_fits(kKernels[sm], d, compute_units)) return (uint32_t)sm;
+    }
     // Few tiles and a long K: cut every tile into K ranges so that the whole chip works.
     static const char* const kSplitK[2][2] = {{"maize_gemm_bf16_mt256_nn_splitk", "maize_gemm_bf16_mt256_nt_splitk"},
                                               {"maize_gemm_f16_mt256_nn_splitk", "maize_gemm_f16_mt256_nt_splitk"}};

@@ -53,6 +53,115 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 }
 
 
+// ---- the end of a few-row kernel (NN and NT alike): combine the K ranges in range order, round once, store -------
+// acc[r * 2 + c2]: lane l of wave w holds C[16 r + l % 16][n0 + 16 (2 w + c2) + 4 (l / 16) + 0..3] of its K range.
+// `word` is one 32-bit word of LDS that nothing else uses any more.
+template <int MR>
+__device__ __forceinline__ void finish(const GemmArgs& p, uint16_t* Cg, const floatx4* acc, lds_ptr word) {
+    const uint32_t M = p.crows, N = p.ccols, ldc = ldc_of(p);
+    const uint32_t ks = p.ksplit ? p.ksplit : 1u;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, g = lane >> 4;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t slab = blockIdx.x, z = blockIdx.y, n0 = slab * SN;
+    // Lane holds C[m = l%16][n = n0 + 16(2w + c2) + 4g + 0..3].
+    const uint32_t m = lane & 15u;
+    // ---- combine the K splits in split order, round once, store ---------------------------
+    // Rows of C that are not 16-byte material (odd N or leading dimension, a pointer off the 16-byte grid: a
+    // launch-uniform flag from the dispatcher) are stored element by element; C is at most 16 MR rows.
+    const bool c_elems = p.reserved & 1u;
+    if (ks == 1u) {
+        // Single split: straight from registers, 8 bytes per lane.
+#pragma unroll
+        for (int r = 0; r < MR; ++r)
+#pragma unroll
+            for (int c2 = 0; c2 < 2; ++c2) {
+                const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
+                const uint32_t row = 16u * r + m;
+                if (row < M && col < N) {
+                    const float v[4] = {acc[r * 2 + c2][0], acc[r * 2 + c2][1], acc[r * 2 + c2][2], acc[r * 2 + c2][3]};
+                    if (c_elems) store_c_elems<4>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
+                    else store_c_run<4>(p, Cg, (uint64_t)row * ldc + col, v);
+                }
+            }
+        return;
+    }
+    // Workspace: 16384 ticket counters (zero between launches), then one fp32 tile of 16 MR x 256
+    // per (batch member, slab, split).  The tiles are written and read with device-coherent
+    // accesses (they cross the per-XCD L2s), so no cache-wide write-back or invalidate is needed:
+    // each wave waits for its own stores, the barrier collects the waves, then one thread takes
+    // the ticket with a device-scope atomic.
+    //
+    // The last workgroup to arrive adds all the tiles of its slab.  One workgroup draws about 50 GB/s of such data,
+    // so this costs ks x MR x 16 KiB at that rate with the rest of the chip idle (1.3 us for 16 rows and 4 ranges,
+    // 5 us for 64 rows).  Sharing the additions among the slab's workgroups (each waits, with a bound, until all
+    // have arrived and adds the part its arrival number names) was built and measured: the polling loads and the
+    // two more atomics per workgroup on the slab's counters cost 1.2 us at 16 rows x 4 ranges (22.8 against 21.6 us)
+    // and 2 us at 8 ranges of an 8192 x 8192 B; it won only from 16 ranges or 64 rows up (-1.7 us), so it stayed out.
+    constexpr int COHERENT = 17;                          // buffer cache policy: sc0 | sc1
+    constexpr uint32_t TILE_BYTES = 16u * MR * SN * 4u;
+    typedef __attribute__((address_space(3))) volatile uint32_t* lds_word_ptr;
+    lds_word_ptr const ticket = (lds_word_ptr)word;
+    uint32_t* counters = (uint32_t*)p.workspace;
+    const uint32_t slab_id = blockIdx.z * gridDim.x + slab;
+    const __amdgpu_buffer_rsrc_t rws =
+        make_rsrc((const char*)p.workspace + 65536, gridDim.z * gridDim.x * ks * TILE_BYTES);
+    const uint32_t tile0 = slab_id * ks * TILE_BYTES;     // byte offset of this slab's split-0 tile
+#pragma unroll
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[r * 2 + c2]), rws,
+                                                   tile0 + z * TILE_BYTES + ((16u * r + m) * SN + (wave * 2u + c2) * 16u + g * 4u) * 4u,
+                                                   0, COHERENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wave's partial tile has reached memory
+    __syncthreads();
+    if (tid == 0) *ticket = __hip_atomic_fetch_add(&counters[slab_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*ticket != ks - 1u) return;                       // not the last split of this slab to finish
+    {
+        // 512 threads x 8 columns = 16 x 256 per row group; thread t adds rows 16 r + t / 32.  The partial tiles are
+        // requested ZG splits at a time for all row groups at once (ZG x MR x 2 128-bit loads in flight per lane),
+        // so a slab pays one memory round trip per ZG splits; the additions still run in split order.
+        constexpr int ZG = MR == 4 ? 4 : 8;
+        constexpr uint32_t DROP = 0xFFFFFFE0u;                    // past the descriptor: reads as zeros
+        const uint32_t cq = (tid & 31u) * 8u;
+        const uint32_t off = tile0 + ((tid >> 5) * SN + cq) * 4u;
+        floatx4 s_lo[MR], s_hi[MR];
+        for (uint32_t z0 = 0; z0 < ks; z0 += ZG) {
+            floatx4 t_lo[MR][ZG], t_hi[MR][ZG];
+#pragma unroll
+            for (int u = 0; u < ZG; ++u)
+#pragma unroll
+                for (int r = 0; r < MR; ++r) {
+                    const uint32_t o = z0 + u < ks ? off + (z0 + u) * TILE_BYTES + (uint32_t)r * (16u * SN * 4u) : DROP;
+                    t_lo[r][u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o, 0, COHERENT));
+                    t_hi[r][u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o + 16u, 0, COHERENT));
+                }
+#pragma unroll
+            for (int u = 0; u < ZG; ++u)
+#pragma unroll
+                for (int r = 0; r < MR; ++r) {
+                    if (z0 + u == 0u) { s_lo[r] = t_lo[r][0]; s_hi[r] = t_hi[r][0]; }
+                    else if (z0 + u < ks) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { s_lo[r][e] += t_lo[r][u][e]; s_hi[r][e] += t_hi[r][u][e]; }
+                    }
+                }
+        }
+        const uint32_t col = n0 + cq;
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+            const uint32_t row = 16u * r + (tid >> 5);
+            if (row < M && col < N) {
+                const float v[8] = {s_lo[r][0], s_lo[r][1], s_lo[r][2], s_lo[r][3], s_hi[r][0], s_hi[r][1], s_hi[r][2], s_hi[r][3]};
+                if (c_elems) store_c_elems<8>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
+                else store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);      // 8 columns are all in or all out
+            }
+        }
+    }
+    if (tid == 0) counters[slab_id] = 0u;                 // ready for the next launch
+}
+
 // Granule swizzle of a block: the 32-byte granule index (0..15) of row r is XOR-ed with
 // f(r) = r%4 + 4*bit3(r), so the 8 rows one transposing read touches land in 8 different
 // granules of the 256-byte bank period.
@@ -195,7 +304,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo[c2]) : "v"((uint32_t)(uintptr_t)slot + rd[0][c2]));
             asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi[c2]) : "v"((uint32_t)(uintptr_t)slot + rd[1][c2]));
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // The wait names every register the reads fill, so that nothing derived from them can move in front of it.
+        if constexpr (MR == 1)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0]), "+v"(lo[0]), "+v"(lo[1]), "+v"(hi[0]), "+v"(hi[1]) :: "memory");
+        else if constexpr (MR == 2)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0]), "+v"(af[1]), "+v"(lo[0]), "+v"(lo[1]), "+v"(hi[0]), "+v"(hi[1]) :: "memory");
+        else
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0]), "+v"(af[1]), "+v"(af[MR - 2]), "+v"(af[MR - 1]),
+                         "+v"(lo[0]), "+v"(lo[1]), "+v"(hi[0]), "+v"(hi[1]) :: "memory");
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {
             short8v bb = {lo[c2][0], lo[c2][1], lo[c2][2], lo[c2][3], hi[c2][0], hi[c2][1], hi[c2][2], hi[c2][3]};
@@ -256,104 +372,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // nothing may land in LDS after this point
 
-    // Lane holds C[m = l%16][n = n0 + 16(2w + c2) + 4g + 0..3].
-    const uint32_t m = lane & 15u;
-    // ---- combine the K splits in split order, round once, store ---------------------------
-    // Rows of C that are not 16-byte material (odd N or leading dimension, a pointer off the 16-byte grid: a
-    // launch-uniform flag from the dispatcher) are stored element by element; C is at most 16 rows.
-    const bool c_elems = p.reserved & 1u;
-    if (ks == 1u) {
-        // Single split: straight from registers, 8 bytes per lane.
-#pragma unroll
-        for (int r = 0; r < MR; ++r)
-#pragma unroll
-            for (int c2 = 0; c2 < 2; ++c2) {
-                const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
-                const uint32_t row = 16u * r + m;
-                if (row < M && col < N) {
-                    const float v[4] = {acc[r][c2][0], acc[r][c2][1], acc[r][c2][2], acc[r][c2][3]};
-                    if (c_elems) store_c_elems<4>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
-                    else store_c_run<4>(p, Cg, (uint64_t)row * ldc + col, v);
-                }
-            }
-        return;
-    }
-    // Workspace: 16384 ticket counters (zero between launches), then one fp32 tile of 16 MR x 256
-    // per (batch member, slab, split).  The tiles are written and read with device-coherent
-    // accesses (they cross the per-XCD L2s), so no cache-wide write-back or invalidate is needed:
-    // each wave waits for its own stores, the barrier collects the waves, then one thread takes
-    // the ticket with a device-scope atomic.
-    //
-    // The last workgroup to arrive adds all the tiles of its slab.  One workgroup draws about 50 GB/s of such data,
-    // so this costs ks x MR x 16 KiB at that rate with the rest of the chip idle (1.3 us for 16 rows and 4 ranges,
-    // 5 us for 64 rows).  Sharing the additions among the slab's workgroups (each waits, with a bound, until all
-    // have arrived and adds the part its arrival number names) was built and measured: the polling loads and the
-    // two more atomics per workgroup on the slab's counters cost 1.2 us at 16 rows x 4 ranges (22.8 against 21.6 us)
-    // and 2 us at 8 ranges of an 8192 x 8192 B; it won only from 16 ranges or 64 rows up (-1.7 us), so it stayed out.
-    constexpr int COHERENT = 17;                          // buffer cache policy: sc0 | sc1
-    constexpr uint32_t TILE_BYTES = 16u * MR * SN * 4u;
-    typedef __attribute__((address_space(3))) volatile uint32_t* lds_word_ptr;
-    lds_word_ptr const ticket = (lds_word_ptr)ablk0;     // the A blocks are idle from here on (with four row groups
-                                                          // the ring and the A blocks fill the 160 KiB of LDS to the byte)
-    uint32_t* counters = (uint32_t*)p.workspace;
-    const uint32_t slab_id = (uint32_t)bz * gridDim.x + slab;
-    const __amdgpu_buffer_rsrc_t rws =
-        make_rsrc((const char*)p.workspace + 65536, gridDim.z * gridDim.x * ks * TILE_BYTES);
-    const uint32_t tile0 = slab_id * ks * TILE_BYTES;     // byte offset of this slab's split-0 tile
-#pragma unroll
-    for (int r = 0; r < MR; ++r)
-#pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2)
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[r][c2]), rws,
-                                                   tile0 + z * TILE_BYTES + ((16u * r + m) * SN + (wave * 2u + c2) * 16u + g * 4u) * 4u,
-                                                   0, COHERENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wave's partial tile has reached memory
-    __syncthreads();
-    if (tid == 0) *ticket = __hip_atomic_fetch_add(&counters[slab_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (*ticket != ks - 1u) return;                       // not the last split of this slab to finish
-    {
-        // 512 threads x 8 columns = 16 x 256 per row group; thread t adds rows 16 r + t / 32.  The partial tiles are
-        // requested ZG splits at a time for all row groups at once (ZG x MR x 2 128-bit loads in flight per lane),
-        // so a slab pays one memory round trip per ZG splits; the additions still run in split order.
-        constexpr int ZG = MR == 4 ? 4 : 8;
-        constexpr uint32_t DROP = 0xFFFFFFE0u;                    // past the descriptor: reads as zeros
-        const uint32_t cq = (tid & 31u) * 8u;
-        const uint32_t off = tile0 + ((tid >> 5) * SN + cq) * 4u;
-        floatx4 s_lo[MR], s_hi[MR];
-        for (uint32_t z0 = 0; z0 < ks; z0 += ZG) {
-            floatx4 t_lo[MR][ZG], t_hi[MR][ZG];
-#pragma unroll
-            for (int u = 0; u < ZG; ++u)
-#pragma unroll
-                for (int r = 0; r < MR; ++r) {
-                    const uint32_t o = z0 + u < ks ? off + (z0 + u) * TILE_BYTES + (uint32_t)r * (16u * SN * 4u) : DROP;
-                    t_lo[r][u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o, 0, COHERENT));
-                    t_hi[r][u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o + 16u, 0, COHERENT));
-                }
-#pragma unroll
-            for (int u = 0; u < ZG; ++u)
-#pragma unroll
-                for (int r = 0; r < MR; ++r) {
-                    if (z0 + u == 0u) { s_lo[r] = t_lo[r][0]; s_hi[r] = t_hi[r][0]; }
-                    else if (z0 + u < ks) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) { s_lo[r][e] += t_lo[r][u][e]; s_hi[r][e] += t_hi[r][u][e]; }
-                    }
-                }
-        }
-        const uint32_t col = n0 + cq;
-#pragma unroll
-        for (int r = 0; r < MR; ++r) {
-            const uint32_t row = 16u * r + (tid >> 5);
-            if (row < M && col < N) {
-                const float v[8] = {s_lo[r][0], s_lo[r][1], s_lo[r][2], s_lo[r][3], s_hi[r][0], s_hi[r][1], s_hi[r][2], s_hi[r][3]};
-                if (c_elems) store_c_elems<8>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
-                else store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);      // 8 columns are all in or all out
-            }
-        }
-    }
-    if (tid == 0) counters[slab_id] = 0u;                 // ready for the next launch
+    // The A blocks are idle from here on: their first word serves the tail (with four row groups the ring and the A
+    // blocks fill the 160 KiB of LDS to the byte).
+    finish<MR>(p, Cg, &acc[0][0], (lds_ptr)ablk0);
 }
 
 }  // namespace skinny

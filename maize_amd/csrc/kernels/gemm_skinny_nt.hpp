@@ -25,7 +25,9 @@
 //   * ragged K: chunks at or past K are masked per lane (K % 8 == 0 for 16-bit, K % 16 == 0 for 8-bit
 //     operands); blocks past the end of a range read through a zero-length descriptor.
 //
-// Requirements (checked by the dispatcher): layout NT, M <= 16, rows of A and B on 16-byte boundaries, every
+// maize_gemm_*_skinny_nt_m32 / _m64 (body_rows below) carry 2 or 4 groups of 16 rows of A, staged through LDS.
+//
+// Requirements (checked by the dispatcher): layout NT, M <= 16 (32, 64), rows of A and B on 16-byte boundaries, every
 // matrix (per batch member) below 2 GiB.  Any N, leading dimension of C and element-aligned C pointer (a
 // vocabulary of 50257 rows of B is as good as one of 50264): rows of B at or past N read as zeros, and C goes
 // out in 128-bit runs when its rows allow it, element by element otherwise.
@@ -175,73 +177,183 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // nothing may land in LDS after this point
 
-    // ---- combine the K splits in split order, round once, store (as the NN kernel does) ----------
-    // Lane holds C[m = l%16][n = n0 + 16(2w + c2) + 4g + 0..3].
-    const uint32_t m = r16;
-    // Rows of C that are not 16-byte material (odd N or leading dimension, a pointer off the 16-byte grid: a
-    // launch-uniform flag from the dispatcher) are stored element by element; C is at most 16 rows.
-    const bool c_elems = p.reserved & 1u;
-    if (ks == 1u) {
+    // ---- combine the K ranges in range order, round once, store (shared with the NN kernel) ----------
+    // The ring is idle from here on: its first word serves the tail.
+    skinny::finish<1>(p, Cg, &acc[0], (lds_ptr)ring0);
+}
+
+// ---- 17 .. 64 rows of A: 2 or 4 groups of 16 rows --------------------------------------------------------------
+// Every wave needs all of A's block (MR x 16 rows x 128 bytes) next to its own 32 rows of B.  Loaded per wave from
+// L2 that is 8 x MR x 2 KiB per 32 KiB of B and the kernel is bound by it (measured: 64 x 14336 x 4096 52 us), so here
+// the A block goes through LDS once per workgroup, as in the NN kernel: a ring slot carries the block of B and MR A
+// groups of 2 KiB, each fetched by two direct-to-LDS loads (piece = 8 rows of 128 bytes, laid out like B's:
+// maps::kc_*); load i (0 .. 2 MR - 1) of the block in slot x is the duty of wave (x + i) % 8.  The price is one
+// workgroup barrier per block and waves that walk K in step.
+template <bool F8, int FA, int FB, int MR>
+__device__ __forceinline__ void body_rows(const GemmArgs& p) {
+    static_assert(MR == 2 || MR == 4, "row groups");
+    constexpr int ABYTES = MR * 2048;                  // A block of one ring slot
+    __shared__ __attribute__((aligned(1024))) char ring0[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring1[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring2[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring3[BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ablk0[ABYTES];
+    __shared__ __attribute__((aligned(1024))) char ablk1[ABYTES];
+    __shared__ __attribute__((aligned(1024))) char ablk2[ABYTES];
+    __shared__ __attribute__((aligned(1024))) char ablk3[ABYTES];
+    constexpr uint32_t ESZ = F8 ? 1u : 2u;             // bytes per element of A and B
+    constexpr uint32_t KB = ROWB / ESZ;                // elements of K per block
+
+    const uint32_t M = p.crows, N = p.ccols, K = p.acols;
+    const uint32_t lda = lda_of(p), ldb = ldb_of(p);
+    const uint32_t ks = p.ksplit ? p.ksplit : 1u;
+    const bool half_io = p.epi & EPI_F16;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t slab = blockIdx.x, z = blockIdx.y;
+    const uint32_t n0 = slab * SN;
+    const uint64_t bz = blockIdx.z;
+    const char* Ag = (const char*)p.a + bz * p.stride_a * ESZ;           // strides count elements
+    const char* Bg = (const char*)p.b + bz * p.stride_b * ESZ;
+    uint16_t* Cg = p.c + bz * p.stride_c * ((p.epi & EPI_F32) ? 2u : 1u);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ag, ((M - 1u) * lda + K) * ESZ);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bg, ((N - 1u) * ldb + K) * ESZ);
+    const __amdgpu_buffer_rsrc_t rnull = make_rsrc(Bg, 0u);
+
+    lds_ptr const s0 = (lds_ptr)ring0, s1 = (lds_ptr)ring1, s2 = (lds_ptr)ring2, s3 = (lds_ptr)ring3;
+    lds_ptr const ablk[RING] = {(lds_ptr)ablk0, (lds_ptr)ablk1, (lds_ptr)ablk2, (lds_ptr)ablk3};
+
+    // Copy maps.  B: wave w issues pieces 4w .. 4w+3 of a block (its own 32 rows).  A: piece i of the block holds rows
+    // 8 i .. 8 i + 7 of A; the lane's place inside a piece is the same for every piece (maps::kc_piece_* of piece 0
+    // and 1 give the two row parities of the swizzle).  Rows at or past N or M fall behind the views and read as zeros.
+    uint32_t b_vo[4], b_k[2], a_vo[2];
 #pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2) {
-            const uint32_t col = n0 + (wave * 2u + c2) * 16u + g * 4u;
-            if (m < M && col < N) {
-                const float v[4] = {acc[c2][0], acc[c2][1], acc[c2][2], acc[c2][3]};
-                if (c_elems) store_c_elems<4>(p, Cg, (uint64_t)m * ldc + col, v, N - col);
-                else store_c_run<4>(p, Cg, (uint64_t)m * ldc + col, v);
-            }
-        }
-        return;
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t row = maps::kc_piece_row(wave * 4u + i, lane);
+        const uint32_t c = maps::kc_piece_chunk(wave * 4u + i, lane);
+        b_vo[i] = (n0 + row) * ldb * ESZ + c * 16u;
+        if (i < 2) b_k[i] = c * (16u / ESZ);
     }
-    // Workspace: 16384 ticket counters (zero between launches), then one fp32 tile of 16 x 256 per
-    // (batch member, slab, split), written and read with device-coherent accesses; each wave waits
-    // for its own stores, the barrier collects the waves, one thread takes the ticket.
-    constexpr int COHERENT = 17;                          // buffer cache policy: sc0 | sc1
-    constexpr uint32_t TILE_BYTES = 16u * SN * 4u;
-    uint32_t* counters = (uint32_t*)p.workspace;
-    const uint32_t slab_id = (uint32_t)bz * gridDim.x + slab;
-    const __amdgpu_buffer_rsrc_t rws = make_rsrc((const char*)p.workspace + 65536, gridDim.z * gridDim.x * ks * TILE_BYTES);
-    const uint32_t tile0 = slab_id * ks * TILE_BYTES;
 #pragma unroll
-    for (int c2 = 0; c2 < 2; ++c2)
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[c2]), rws,
-                                               tile0 + z * TILE_BYTES + (m * SN + (wave * 2u + c2) * 16u + g * 4u) * 4u, 0, COHERENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    volatile uint32_t& ticket = *(volatile uint32_t*)ring0;      // the ring is idle from here on
-    if (tid == 0) ticket = __hip_atomic_fetch_add(&counters[slab_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (ticket != ks - 1u) return;                        // not the last split of this slab to finish
-    {
-        const uint32_t row = tid >> 5, cq = (tid & 31u) * 8u;     // 512 threads x 8 columns = 16 x 256
-        const uint32_t off = tile0 + (row * SN + cq) * 4u;
-        constexpr uint32_t DROP = 0xFFFFFFE0u;                    // past the descriptor: reads as zeros
-        floatx4 s_lo = floatx4{0.f, 0.f, 0.f, 0.f}, s_hi = floatx4{0.f, 0.f, 0.f, 0.f};
-        for (uint32_t z0 = 0; z0 < ks; z0 += 4u) {               // four splits per memory round trip, added in split order
-            floatx4 t_lo[4], t_hi[4];
+    for (int i = 0; i < 2; ++i)        // even and odd pieces: rows 0 .. 7 and 8 .. 15 of a 16-row group
+        a_vo[i] = maps::kc_piece_row((uint32_t)i, lane) * lda * ESZ + maps::kc_piece_chunk((uint32_t)i, lane) * 16u;
+    // Operand maps, as in the one-group kernel: lane l = row l % 16 of a 16-row group, chunks chunk[0], chunk[1].
+    const uint32_t g = lane >> 4, r16 = lane & 15u;
+    uint32_t chunk[2];
+    chunk[0] = F8 ? 2u * g : g;
+    chunk[1] = F8 ? 2u * g + 1u : 4u + g;
+    uint32_t rd[2][2], ard[2];                           // B: [which of the wave's two row groups][chunk]; A: [chunk]
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t o = z0 + u < ks ? off + (z0 + u) * TILE_BYTES : DROP;
-                t_lo[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o, 0, COHERENT));
-                t_hi[u] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o + 16u, 0, COHERENT));
-            }
+    for (int c = 0; c < 2; ++c) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (z0 + u == 0u) { s_lo = t_lo[0]; s_hi = t_hi[0]; }
-                else if (z0 + u < ks) {
+        for (int c2 = 0; c2 < 2; ++c2) rd[c2][c] = maps::kc_offset((wave * 2u + c2) * 16u + r16, chunk[c]);
+        ard[c] = maps::kc_offset(r16, chunk[c]);         // + 2048 per row group
+    }
+
+    const uint32_t nb_all = (K + KB - 1u) / KB, per = (nb_all + ks - 1u) / ks;
+    const uint32_t b0 = z * per;
+    const uint32_t nb = b0 < nb_all ? (nb_all - b0 < per ? nb_all - b0 : per) : 0u;
+
+    floatx4 acc[MR][2];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) { s_lo[e] += t_lo[u][e]; s_hi[e] += t_hi[u][e]; }
+    for (int r = 0; r < MR; ++r) {
+        acc[r][0] = floatx4{0.f, 0.f, 0.f, 0.f};
+        acc[r][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // Requests block j into `slot` (4 pieces per wave) and, before them, the A pieces this wave has the duty for.
+    auto request = [&](uint32_t j, lds_ptr slot, int ai) {
+        typedef __attribute__((address_space(3))) void* lvp;
+        const uint32_t kb = (b0 + j) * KB;
+        const bool live = j < nb;
+        const __amdgpu_buffer_rsrc_t rs_b = live ? rb : rnull;
+        const __amdgpu_buffer_rsrc_t rs_a = live ? ra : rnull;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 2 * MR; ++i)
+            if (wave == (uint32_t)((ai + i) & 7))
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lvp)(ablk[ai] + i * 1024), 16,
+                                                         (a_vo[i & 1] + (uint32_t)(i >> 1) * 16u * lda * ESZ + kb * ESZ) | ((b_k[i & 1] + kb) < K ? 0u : OOB), 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lvp)(slot + (wave * 4u + i) * 1024u), 16,
+                                                     (b_vo[i] + kb * ESZ) | ((b_k[i & 1] + kb) < K ? 0u : OOB), 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto consume = [&](lds_ptr slot, int ai) {
+        // Inline assembly, so that the compiler sees no read of the ring and places no counter wait of its own.
+        u32x4 af[MR][2], bf[2][2];
+#pragma unroll
+        for (int r = 0; r < MR; ++r)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+                asm volatile("ds_read_b128 %0, %1" : "=v"(af[r][c]) : "v"((uint32_t)(uintptr_t)ablk[ai] + (uint32_t)r * 2048u + ard[c]));
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+                asm volatile("ds_read_b128 %0, %1" : "=v"(bf[c2][c]) : "v"((uint32_t)(uintptr_t)slot + rd[c2][c]));
+        // The wait names every register the reads fill: without that the compiler is free to move what it derives from
+        // them (the copies that assemble an 8-bit operand) in front of the wait.
+        if constexpr (MR == 2)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0][0]), "+v"(af[0][1]), "+v"(af[1][0]), "+v"(af[1][1]),
+                         "+v"(bf[0][0]), "+v"(bf[0][1]), "+v"(bf[1][0]), "+v"(bf[1][1]) :: "memory");
+        else
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0][0]), "+v"(af[0][1]), "+v"(af[1][0]), "+v"(af[1][1]),
+                         "+v"(af[MR - 2][0]), "+v"(af[MR - 2][1]), "+v"(af[MR - 1][0]), "+v"(af[MR - 1][1]),
+                         "+v"(bf[0][0]), "+v"(bf[0][1]), "+v"(bf[1][0]), "+v"(bf[1][1]) :: "memory");
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2)
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                const u32x4 b_lo = bf[c2][0], b_hi = bf[c2][1];
+                if (F8) {
+                    const i32x8 bb = {(int)b_lo[0], (int)b_lo[1], (int)b_lo[2], (int)b_lo[3], (int)b_hi[0], (int)b_hi[1], (int)b_hi[2], (int)b_hi[3]};
+                    const i32x8 aa = {(int)af[r][0][0], (int)af[r][0][1], (int)af[r][0][2], (int)af[r][0][3],
+                                      (int)af[r][1][0], (int)af[r][1][1], (int)af[r][1][2], (int)af[r][1][3]};
+                    acc[r][c2] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bb, aa, acc[r][c2], FB, FA, 0, 0, 0, 0);   // B is fed first
+                } else if (half_io) {   // same bits, read as IEEE half (a wave-uniform choice)
+                    acc[r][c2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, b_lo), __builtin_bit_cast(halfx8, af[r][0]), acc[r][c2], 0, 0, 0);
+                    acc[r][c2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, b_hi), __builtin_bit_cast(halfx8, af[r][1]), acc[r][c2], 0, 0, 0);
+                } else {
+                    acc[r][c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, b_lo), __builtin_bit_cast(bf16x8, af[r][0]), acc[r][c2], 0, 0, 0);
+                    acc[r][c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, b_hi), __builtin_bit_cast(bf16x8, af[r][1]), acc[r][c2], 0, 0, 0);
                 }
             }
+    };
+    // One block: wait until this wave's share of block b has landed -- the loads of blocks b+1 and b+2 may stay in
+    // flight: 8 pieces of B plus this wave's A duties among them, piece i of the block in slot x being the duty of
+    // wave (x + i) % 8 -- meet the other waves (which also says everyone is done reading block b-1), refill that
+    // block's slot with block b+3, multiply block b.
+    auto turn = [&](uint32_t b, lds_ptr cur, int ai, lds_ptr prev, int pi) {
+        uint32_t later = 0;
+#pragma unroll
+        for (int x = 1; x <= 2; ++x)
+#pragma unroll
+            for (int i = 0; i < 2 * MR; ++i) later += wave == (uint32_t)((((ai + x) % RING) + i) & 7) ? 1u : 0u;   // blocks b+1, b+2 sit in slots (ai + 1), (ai + 2) mod RING
+        switch (later) {
+            case 0: asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(9)\n\ts_barrier" ::: "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(10)\n\ts_barrier" ::: "memory"); break;
         }
-        const uint32_t col = n0 + cq;
-        if (row < M && col < N) {                          // vector stores: N % 8 == 0, 8 columns are all in or all out
-            const float v[8] = {s_lo[0], s_lo[1], s_lo[2], s_lo[3], s_hi[0], s_hi[1], s_hi[2], s_hi[3]};
-            if (c_elems) store_c_elems<8>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
-            else store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        request(b + 3, prev, pi);
+        consume(cur, ai);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    request(0, s0, 0); request(1, s1, 1); request(2, s2, 2);
+    for (uint32_t b = 0; b < nb; b += RING) {
+        turn(b + 0, s0, 0, s3, 3);
+        turn(b + 1, s1, 1, s0, 0);
+        turn(b + 2, s2, 2, s1, 1);
+        turn(b + 3, s3, 3, s2, 2);
     }
-    if (tid == 0) counters[slab_id] = 0u;                 // ready for the next launch
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // nothing may land in LDS after this point
+    __syncthreads();                                      // ... and every wave is done reading the A blocks
+    skinny::finish<MR>(p, Cg, &acc[0][0], (lds_ptr)ablk0);
 }
 
 }  // namespace skinny_nt
@@ -251,5 +363,15 @@ extern "C" __global__ __launch_bounds__(512) void maize_gemm_e4m3_skinny_nt(Gemm
 extern "C" __global__ __launch_bounds__(512) void maize_gemm_e5m2_skinny_nt(GemmArgs p) { skinny_nt::body<true, 1, 1>(p); }
 extern "C" __global__ __launch_bounds__(512) void maize_gemm_e4m3e5m2_skinny_nt(GemmArgs p) { skinny_nt::body<true, 0, 1>(p); }
 extern "C" __global__ __launch_bounds__(512) void maize_gemm_e5m2e4m3_skinny_nt(GemmArgs p) { skinny_nt::body<true, 1, 0>(p); }
+// 17 .. 32 and 33 .. 64 rows of A.
+#define MAIZE_SKINNY_NT_ROWS(tag, f8, fa, fb) \
+    extern "C" __global__ __launch_bounds__(512) void maize_gemm_##tag##_skinny_nt_m32(GemmArgs p) { skinny_nt::body_rows<f8, fa, fb, 2>(p); } \
+    extern "C" __global__ __launch_bounds__(512) void maize_gemm_##tag##_skinny_nt_m64(GemmArgs p) { skinny_nt::body_rows<f8, fa, fb, 4>(p); }
+MAIZE_SKINNY_NT_ROWS(bf16, false, 0, 0)
+MAIZE_SKINNY_NT_ROWS(e4m3, true, 0, 0)
+MAIZE_SKINNY_NT_ROWS(e5m2, true, 1, 1)
+MAIZE_SKINNY_NT_ROWS(e4m3e5m2, true, 0, 1)
+MAIZE_SKINNY_NT_ROWS(e5m2e4m3, true, 1, 0)
+#undef MAIZE_SKINNY_NT_ROWS
 
 }  // namespace maize

@@ -54,7 +54,21 @@ def test_every_registry_entry_has_its_device_kernel(kernels):
 
 def test_matrix_instruction_per_kernel(kernels):
     for name, ins in kernels.items():
-        if name.endswith("_skinny_nt"):
+        if name.endswith(("_skinny_nt_m32", "_skinny_nt_m64")):
+            # 17 .. 64 rows against N x K weights: the same instructions, 2 or 4 row groups per fragment of B, A through LDS
+            groups = 2 if name.endswith("_m32") else 4
+            if name.startswith("maize_gemm_bf16"):
+                # 4 turns x 2 fragments of B x row groups x 2 K steps
+                assert count(ins, "v_mfma_f32_16x16x32_bf16") >= 16 * groups and count(ins, "v_mfma_f32_16x16x32_f16") >= 16 * groups, name
+            else:
+                f8 = [i for i in ins if i.startswith("v_mfma_f32_16x16x128_f8f6f4")]
+                tag = name[len("maize_gemm_"):].split("_")[0]
+                a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
+                assert len(f8) >= 8 * groups and all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
+            assert count(ins, "ds_read_b128") >= 16 + 8 * groups and count(ins, "ds_read_b64_tr_b16") == 0, name
+            assert len([i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]) >= 16 + 2 * groups, name
+            assert count(ins, "s_barrier") >= 4, name                     # one per block: the A blocks are shared
+        elif name.endswith("_skinny_nt"):
             # M <= 16 against N x K weights: 16-row instructions, 32 deep for 16-bit operands (bf16 and half in one
             # kernel), 128 deep for 8-bit ones (format codes as below)
             if name == "maize_gemm_bf16_skinny_nt":

@@ -145,9 +145,10 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert p["workspace_bytes"] < (1 << 31)
         else:
             assert p["workspace_bytes"] == 0
-    elif name == "maize_gemm_bf16_skinny_nt":
+    elif name.startswith("maize_gemm_bf16_skinny_nt"):
+        rows = {"maize_gemm_bf16_skinny_nt": 16, "maize_gemm_bf16_skinny_nt_m32": 32, "maize_gemm_bf16_skinny_nt_m64": 64}[name]
         assert p["block"] == (512, 1, 1)
-        assert layout == mz.LAYOUT_NT and m <= 16 and n % 8 == 0 and k % 8 == 0
+        assert layout == mz.LAYOUT_NT and m <= rows and n % 8 == 0 and k % 8 == 0
         ks = p["ksplit"]
         nblk = cdiv(k, 64)                                     # blocks of 128 bytes per row
         assert gx == cdiv(n, 256) and gy == ks and 1 <= ks <= 16
@@ -155,7 +156,7 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         if ks > 1:
             assert nblk // ks >= 4                             # the 4-slot ring is filled at least once
             assert gx * batch <= 16384
-            assert p["workspace_bytes"] >= TICKET_BYTES + gx * batch * ks * 16 * 256 * 4
+            assert p["workspace_bytes"] >= TICKET_BYTES + gx * batch * ks * rows * 256 * 4
             assert p["workspace_bytes"] < (1 << 31)
         else:
             assert p["workspace_bytes"] == 0
@@ -175,7 +176,12 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",              # N x K weights streamed once
         (16, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",
-        (17, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",        # more than 16 rows
+        (17, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m32",          # 17 .. 32 rows: two row groups
+        (64, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m64",         # 33 .. 64 rows and many slabs: four
+        (65, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",       # more than 64 rows
+        (32, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn_m32",
+        (64, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn_m64",
+        (64, 8192, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",        # 64 rows, 32 slabs: the tile kernel cut over K
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
         (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",      # odd N: operands read where they lie, C written element-wise by the reduce pass
         (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",

@@ -194,7 +194,10 @@ def test_dispatch_of_8bit_operands():
         assert split["workspace_bytes"] == 65536 + split["ksplit"] * 256 * 256 * 4
         skinny = name.replace("_mt256_nt", "_skinny_nt")
         assert mz.gemm_plan(ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny          # M <= 16: B streamed once
-        assert mz.gemm_plan(ex(17, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"
+        assert mz.gemm_plan(ex(17, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m32"    # 17 .. 64 rows: row groups
+        assert mz.gemm_plan(ex(64, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m64"
+        assert mz.gemm_plan(ex(64, 4096, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"     # few slabs
+        assert mz.gemm_plan(ex(65, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"
         assert _supports(skinny, ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it)) and not _supports(skinny, x)
         mz.validate(ex(**big, in_type=it, ptrs=(0x1001, 0x100003, 0x2000000)))
     for name in mz.kernel_names():

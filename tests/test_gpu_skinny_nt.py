@@ -107,3 +107,45 @@ def test_any_n_and_any_c_rows(ctx, oracle):
         assert run_f8(ctx, oracle, 16, 32003, 1024, fmt=fmt, label="odd N f8") == f"maize_gemm_{fmt}_skinny_nt"
         assert run_f8(ctx, oracle, 5, 1001, 4096, fmt=fmt, alpha=0.5, beta=1.0, ldc=1003, label="odd N f8 scaled") == f"maize_gemm_{fmt}_skinny_nt"
         assert run_f8(ctx, oracle, 16, 1001, 2048, fmt=fmt, out_f16=True, label="odd N f8 half C") == f"maize_gemm_{fmt}_skinny_nt"
+
+
+ROW_GROUP_SHAPES = [(32, 14336, 4096), (17, 2048, 1024), (29, 4099, 2080), (32, 256, 64), (5, 515, 264), (24, 512, 16384),
+                    (64, 14336, 4096), (33, 2048, 1024), (50, 4101, 2088), (64, 256, 8), (47, 50257, 768), (64, 1024, 8192)]
+
+
+def _rows_kernel(tag, m):
+    return f"maize_gemm_{tag}_skinny_nt_{'m32' if m <= 32 else 'm64'}"
+
+
+@pytest.mark.parametrize("shape", ROW_GROUP_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_row_groups_bf16_and_half(ctx, oracle, shape):
+    """17 .. 64 rows against weights stored N x K: the streaming kernel with 2 or 4 groups of 16 rows (A through
+    LDS, one barrier per block).  By name, so that ragged row groups, single ranges, odd N and K tails are all met."""
+    m, n, k = shape
+    name = _rows_kernel("bf16", m)
+    assert run_ex(ctx, oracle, m, n, k, layout=NT, kernel=name, label="skinny_nt rows") == name
+    assert run_ex(ctx, oracle, m, n, k, layout=NT, half=True, kernel=name, label="skinny_nt rows half") == name
+
+
+def test_row_groups_dispatch_views_and_epilogues(ctx, oracle):
+    assert run_ex(ctx, oracle, 32, 14336, 4096, layout=NT, label="auto m32") == "maize_gemm_bf16_skinny_nt_m32"
+    assert run_ex(ctx, oracle, 64, 14336, 4096, layout=NT, label="auto m64") == "maize_gemm_bf16_skinny_nt_m64"
+    assert run_ex(ctx, oracle, 64, 4096, 4096, layout=NT, label="few slabs") == "maize_gemm_bf16_mt256_nt_splitk"
+    for m in (24, 56):
+        name = _rows_kernel("bf16", m)
+        assert run_ex(ctx, oracle, m, 1096, 4104, layout=NT, kernel=name, label="K % 64 != 0") == name
+        assert run_ex(ctx, oracle, m, 1096, 4096, layout=NT, lda=4104, ldb=4160, ldc=1104, kernel=name, label="views") == name
+        for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=1104), dict(alpha=2.0, beta=0.0, c_nan=True)):
+            assert run_ex(ctx, oracle, m, 1096, 4096, layout=NT, kernel=name, label="epilogue", **kw) == name
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"])
+def test_row_groups_8bit_operands(ctx, oracle, fmt):
+    for (m, n, k) in ((32, 14336, 4096), (64, 14336, 4096), (21, 264, 2048), (45, 520, 8192), (64, 1096, 4112)):
+        name = _rows_kernel(fmt, m)
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, kernel=name, label="skinny_nt rows f8") == name
+    name = _rows_kernel(fmt, 40)
+    assert run_f8(ctx, oracle, 40, 1096, 4096, fmt=fmt, lda=4112, ldb=4224, ldc=1104, kernel=name, label="views") == name
+    assert run_f8(ctx, oracle, 40, 1001, 4096, fmt=fmt, alpha=-1.25, beta=0.75, kernel=name, label="scaled, odd N") == name
+    assert run_f8(ctx, oracle, 40, 1096, 4096, fmt=fmt, out_f32=True, alpha=3.0, beta=-0.5, kernel=name, label="f32") == name
+    assert run_f8(ctx, oracle, 32, 14336, 4096, fmt=fmt, label="auto") == _rows_kernel(fmt, 32)

@@ -39,6 +39,8 @@ FAMILIES = [
     ("maize_gemm_bf16_skinny_nn_m64", 50, 519, 2080, NN),           # four row groups
     ("maize_gemm_bf16_skinny_nn_m64", 64, 264, 8192, NN),
     ("maize_gemm_bf16_skinny_nt", 16, 515, 1096, NT),
+    ("maize_gemm_bf16_skinny_nt_m32", 29, 515, 1096, NT),           # A through LDS, ragged row group, K tail
+    ("maize_gemm_bf16_skinny_nt_m64", 50, 264, 4104, NT),
     ("maize_gemm_bf16_wave32", 33, 17, 65, NN),
     ("maize_gemm_bf16_wave32", 33, 17, 65, NT),
     (None, 16, 14336, 4096, NN),

@@ -423,6 +423,7 @@ def test_skinny_checker_rejects_broken_rings():
 def skinny_nt_constants():
     src = open(os.path.join(KDIR, "gemm_skinny_nt.hpp")).read()
     ring = int(re.search(r"constexpr int RING = (\d+);", src).group(1))
+    src = src[:src.index("void body_rows(")]               # the one-group kernel; the row-group kernel is modelled below
     body = src[src.index("auto turn = "):]
     waits = [int(x) for x in re.findall(r's_waitcnt vmcnt\((\d+)\)" ::: "memory"\);\n\s+__builtin_amdgcn_sched_barrier', body)]
     assert len(waits) == 1 and "s_barrier" not in body[:body.index("request(0, s0, 0)")]
@@ -482,3 +483,49 @@ def test_skinny_nt_checker_rejects_broken_rings():
         check_private_ring(*skinny_nt_wave_program(32, ring, wait + 6, primed, ahead), 6)
     with pytest.raises(Hazard):                                  # refill aimed at the slot that is about to be read
         check_private_ring(*skinny_nt_wave_program(32, ring - 1, wait, primed, ahead), 6)
+
+
+# ---------------------------------------------------------------------------------------
+# skinny NT kernels with 2 or 4 row groups: the ring is shared again (A blocks through LDS): 4 slots, per wave 4 pieces
+# of B per block plus the A pieces it has the duty for (piece i of the block in slot x: wave (x + i) % 8), one barrier
+# per block, counter wait
+# ---------------------------------------------------------------------------------------
+
+def skinny_nt_rows_constants():
+    src = open(os.path.join(KDIR, "gemm_skinny_nt.hpp")).read()
+    src = src[src.index("void body_rows("):]
+    waits = [int(x) for x in re.findall(r"s_waitcnt vmcnt\((\d+)\)\\n\\ts_barrier", src)]
+    assert waits == [8, 9, 10]
+    assert "if (wave == (uint32_t)((ai + i) & 7))" in src                                   # the duty rule
+    assert "later += wave == (uint32_t)((((ai + x) % RING) + i) & 7) ? 1u : 0u;" in src and "for (int x = 1; x <= 2; ++x)" in src
+    for n in range(3):
+        assert re.search(r"(case %d|default): asm volatile\(\"s_waitcnt vmcnt\(%d\)" % (n, 8 + n), src)
+    ahead = int(re.search(r"request\(b \+ (\d+), prev, pi\);", src).group(1))
+    primed = len(re.findall(r"request\(\d+, s\d+, \d+\);", src))
+    return 4, primed, ahead
+
+
+def skinny_nt_rows_program(nb, ring, primed, ahead, wave, mr, slack=0):
+    loads = lambda slot: 4 + sum(1 for i in range(2 * mr) if (slot + i) % 8 == wave)
+    ops = [("request", j, j % ring, loads(j % ring)) for j in range(primed)]
+    turns = -(-nb // ring) * ring
+    for b in range(turns):
+        cur = b % ring
+        later = sum(1 for x in (1, 2) for i in range(2 * mr) if ((cur + x) % ring + i) % 8 == wave)
+        ops += [("wait", 8 + later + slack), ("barrier",)]
+        ops.append(("request", b + ahead, (b + ahead) % ring, loads((b + ahead) % ring)))
+        ops.append(("consume", b, cur))
+    ops.append(("wait", 0))
+    return ops, turns
+
+
+@pytest.mark.parametrize("mr", [2, 4])
+@pytest.mark.parametrize("nb", [4, 16, 32, 9, 1])
+def test_skinny_nt_row_group_ring_is_hazard_free(nb, mr):
+    ring, primed, ahead = skinny_nt_rows_constants()
+    assert primed == ring - 1 == ahead
+    for wave in range(8):
+        ops, turns = skinny_nt_rows_program(nb, ring, primed, ahead, wave, mr)
+        check_ring(ops, turns, None, ring)
+        with pytest.raises(Hazard):                              # one load more left in flight: block b's last piece may be missing
+            check_ring(*skinny_nt_rows_program(32, ring, primed, ahead, wave, mr, slack=1), None, ring)
