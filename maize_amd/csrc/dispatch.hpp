@@ -16,6 +16,7 @@ constexpr uint32_t kMaxKernels = 96;
 constexpr const char* kReduceKernel = "maize_gemm_splitk_reduce";
 constexpr const char* kPackKernel = "maize_pack_2d";
 constexpr const char* kPackKernelU8 = "maize_pack_2d_u8";
+constexpr const char* kTransposeKernelU8 = "maize_transpose_u8";   // the 128-bit form of its transposing copy
 
 // Repacking of one operand into the workspace before the launch (pack.hpp).
 struct PackPlan {

@@ -81,7 +81,7 @@ struct maize_ctx {
     hipModule_t module;
     hipFunction_t fn[maize::kMaxKernels];
     hipFunction_t reduce_fn;
-    hipFunction_t pack_fn, pack_u8_fn;
+    hipFunction_t pack_fn, pack_u8_fn, transpose_u8_fn;
     // Split-K scratch, one per stream so that launches on different streams never share it.
     std::unordered_map<void*, maize_workspace> workspaces;
     // This device's copy of the fixed scratch array behind maize_hip_gemm_bf16_noalloc (looked up at create time).
@@ -154,6 +154,7 @@ int32_t maize_hip_ctx_create(int32_t device, maize_ctx_t** out) {
     e = hipModuleGetFunction(&ctx->reduce_fn, ctx->module, maize::kReduceKernel);
     if (e == hipSuccess) e = hipModuleGetFunction(&ctx->pack_fn, ctx->module, maize::kPackKernel);
     if (e == hipSuccess) e = hipModuleGetFunction(&ctx->pack_u8_fn, ctx->module, maize::kPackKernelU8);
+    if (e == hipSuccess) e = hipModuleGetFunction(&ctx->transpose_u8_fn, ctx->module, maize::kTransposeKernelU8);
     if (e != hipSuccess) {
         int32_t rc = hip_fail(e, "helper kernels of the embedded code object");
         (void)hipModuleUnload(ctx->module);
@@ -496,10 +497,14 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
         pa.stride_dst = (uint64_t)pp.rows_dst * pp.cols_dst;
         const uint64_t total = (uint64_t)pp.rows_dst * pp.cols_dst;
         const bool u8 = pp.elem_bytes == 1;                  // 64 x 64 tiles through LDS, batch in grid.z; else one element per thread, batch in grid.y
-        const uint32_t pgrid[3] = {u8 ? (pp.cols_dst + 63u) / 64u : (uint32_t)((total + 255) / 256), u8 ? (pp.rows_dst + 63u) / 64u : d->batch,
+        // A transposing copy whose source and destination both take 128-bit accesses: 128 x 128 tiles.
+        const bool fast = u8 && pp.transpose && (((uintptr_t)pa.src | (uintptr_t)pa.dst) & 15u) == 0 &&
+                          ((pp.rows | pp.cols | pp.ld_src | pp.rows_dst | pp.cols_dst) & 15u) == 0 && (pa.stride_src & 15u) == 0;
+        const uint32_t edge = fast ? 128u : 64u;
+        const uint32_t pgrid[3] = {u8 ? (pp.cols_dst + edge - 1u) / edge : (uint32_t)((total + 255) / 256), u8 ? (pp.rows_dst + edge - 1u) / edge : d->batch,
                                    u8 ? d->batch : 1u};
         const uint32_t pblock[3] = {256, 1, 1};
-        int32_t prc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, u8 ? ctx->pack_u8_fn : ctx->pack_fn, pgrid, pblock, 0,
+        int32_t prc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, fast ? ctx->transpose_u8_fn : u8 ? ctx->pack_u8_fn : ctx->pack_fn, pgrid, pblock, 0,
                                  stream, &pa, sizeof pa);
         if (prc != MAIZE_OK) return prc;
         if (which == 0) { first.a = pa.dst; first.lda = 0; first.stride_a = pa.stride_dst; }
