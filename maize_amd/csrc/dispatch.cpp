@@ -446,6 +446,54 @@ bool trb_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims*
     return true;
 }
 
+// ---- maize_gemm_{bf16,f16}_mt256_{nn,nt}_packed_gen: the same copies, C written by the first pass ----------------
+// When C itself takes 128-bit stores (N % 8 == 0, 16-byte rows) and splitting K does not pay, the general-epilogue
+// kernel runs on the copies and stores C directly: no fp32 partial tiles, no reduce pass, and the workspace holds the
+// copies only.  Here K is padded to a whole number of K tiles (64), not just to 8: the rows of the copies then start
+// on 128-byte boundaries and the kernel without K masks serves (4096 x 4096 x 4104 on rows 8208 bytes apart: 110 us,
+// x 4160: 96 us).
+Packing packing64_of(const maize_gemm_ex_desc_t& d) {
+    Packing p = packing_of(d);
+    const Dims s = dims_of(d);
+    p.k8 = (s.k + 63u) & ~63u;
+    p.a = p.b = true;                      // both operands carry K
+    p.a_elems = (uint64_t)s.m * p.k8;
+    p.b_elems = (uint64_t)p.n8 * p.k8;
+    return p;
+}
+bool packed_gen_ok(const maize_gemm_ex_desc_t& d) {
+    if (!c_rows16(d) || (dims_of(d).n & 7u)) return false;
+    const Packing p = packing64_of(d);
+    if (!mt256_common(packed_view(d, p))) return false;
+    return (p.a_elems + p.b_elems) * d.gemm.batch * 2 <= (1ull << 31);
+}
+bool packed_gen_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && bf16_in(d) && packed_gen_ok(d); }
+bool packed_gen_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && bf16_in(d) && packed_gen_ok(d); }
+bool packed_gen_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && half_in(d) && packed_gen_ok(d); }
+bool packed_gen_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && half_in(d) && packed_gen_ok(d); }
+bool packed_gen_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    const Packing p = packing64_of(d);
+    maize_gemm_ex_desc_t v = packed_view(d, p);
+    v.gemm.c = d.gemm.c; v.ldc = d.ldc; v.gemm.stride_c = d.gemm.stride_c;      // C is the caller's
+    if (!mt256_plan(v, compute_units, ld)) return false;
+    size_t bytes = kTicketBytes;
+    ld->n_padded = p.n8; ld->k_padded = p.k8;
+    if (p.a) {
+        ld->pack_a = PackPlan{true, s.m, s.k, l.a, s.m, p.k8, bytes, false, 2};
+        bytes += (size_t)p.a_elems * d.gemm.batch * 2;
+    }
+    if (p.b) {
+        const uint32_t brows = d.gemm.b.nrows, bcols = d.gemm.b.ncols;
+        ld->pack_b = PackPlan{true, brows, bcols, l.b, s.nt ? p.n8 : p.k8, s.nt ? p.k8 : p.n8, bytes, false, 2};
+        bytes += (size_t)p.b_elems * d.gemm.batch * 2;
+    }
+    ld->workspace_bytes = bytes;
+    ld->reduce_grid = 0;
+    return true;
+}
+
 // ---- maize_gemm_bf16_skinny_nn (M <= 16), _m32, _m64: few rows against a row-major K x N B, streamed once ----------
 static bool skinny_nn_rows(const maize_gemm_ex_desc_t& d, uint32_t max_rows) {
     const Dims s = dims_of(d);
@@ -627,6 +675,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_packed", "maize_gemm_bf16_mt256_nt_splitk", packed_nt_supports, packed_plan},
     {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nn_splitk", packed_f16_nn_supports, packed_plan},
     {"maize_gemm_f16_mt256_nt_packed", "maize_gemm_f16_mt256_nt_splitk", packed_f16_nt_supports, packed_plan},
+    {"maize_gemm_bf16_mt256_nn_packed_gen", "maize_gemm_bf16_mt256_nn_gen", packed_gen_nn_supports, packed_gen_plan},
+    {"maize_gemm_bf16_mt256_nt_packed_gen", "maize_gemm_bf16_mt256_nt_gen", packed_gen_nt_supports, packed_gen_plan},
+    {"maize_gemm_f16_mt256_nn_packed_gen", "maize_gemm_f16_mt256_nn_gen", packed_gen_f16_nn_supports, packed_gen_plan},
+    {"maize_gemm_f16_mt256_nt_packed_gen", "maize_gemm_f16_mt256_nt_gen", packed_gen_f16_nt_supports, packed_gen_plan},
     {"maize_gemm_bf16_skinny_nt", nullptr, skinny_nt_supports, skinny_nt_plan},
     {"maize_gemm_bf16_skinny_nt_m32", nullptr, skinny_nt_m32_supports, skinny_nt_m32_plan},
     {"maize_gemm_bf16_skinny_nt_m64", nullptr, skinny_nt_m64_supports, skinny_nt_m64_plan},
@@ -770,8 +822,17 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
                                               {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nt_packed"}};
     const int pi = kernel_index(kPacked[half_in(d)][s.nt]);
     if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && s.m >= 24u && s.n >= 24u &&
-        kKernels[pi].supports(d) && plan_fits(kKernels[pi], d, compute_units))
+        kKernels[pi].supports(d) && plan_fits(kKernels[pi], d, compute_units)) {
+        // C takes 128-bit stores and K need not be split: the first pass stores C itself.
+        static const char* const kPackedGen[2][2] = {{"maize_gemm_bf16_mt256_nn_packed_gen", "maize_gemm_bf16_mt256_nt_packed_gen"},
+                                                     {"maize_gemm_f16_mt256_nn_packed_gen", "maize_gemm_f16_mt256_nt_packed_gen"}};
+        const int pg = kernel_index(kPackedGen[half_in(d)][s.nt]);
+        Dims sv = s;
+        sv.k = (s.k + 63u) & ~63u; sv.n = up8(s.n);
+        if (pg >= 0 && kKernels[pg].supports(d) && splitk_ranges(sv, d.gemm.batch, compute_units) < 2u && plan_fits(kKernels[pg], d, compute_units))
+            return (uint32_t)pg;
         return (uint32_t)pi;
+    }
     return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
 }
 

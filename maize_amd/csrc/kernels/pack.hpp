@@ -23,15 +23,25 @@ struct PackArgs {
 };
 static_assert(sizeof(PackArgs) == 56, "pack parameter block layout");
 
+// A thread makes one 16-byte run of the copy (8 elements; cols_dst % 8 == 0 and the copy is 16-byte aligned) from
+// eight 2-byte loads of the source, which may start on any even byte: the stores are 128-bit and the loads of
+// neighbouring lanes share cache lines.  (One element per thread moved 4096 x 4100 in 42 us, 1.6 TB/s.)
 extern "C" __global__ __launch_bounds__(256) void maize_pack_2d(PackArgs p) {
-    const uint64_t total = (uint64_t)p.rows_dst * p.cols_dst;
-    const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;   // consecutive lanes, consecutive elements
+    const uint32_t runs_per_row = p.cols_dst >> 3;
+    const uint64_t total = (uint64_t)p.rows_dst * runs_per_row;
+    const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;   // consecutive lanes, consecutive runs
     if (idx >= total) return;
-    const uint32_t r = (uint32_t)(idx / p.cols_dst), c = (uint32_t)(idx % p.cols_dst);
+    const uint32_t r = (uint32_t)(idx / runs_per_row), c = (uint32_t)(idx % runs_per_row) * 8u;
     const uint64_t bz = blockIdx.y;
-    uint16_t v = 0;
-    if (r < p.rows && c < p.cols) v = p.src[bz * p.stride_src + (uint64_t)r * p.ld_src + c];
-    p.dst[bz * p.stride_dst + idx] = v;
+    const uint16_t* row = p.src + bz * p.stride_src + (uint64_t)r * p.ld_src;
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = (r < p.rows && c + 2 * i < p.cols) ? row[c + 2 * i] : 0u;
+        const uint32_t hi = (r < p.rows && c + 2 * i + 1 < p.cols) ? row[c + 2 * i + 1] : 0u;
+        w[i] = lo | (hi << 16);
+    }
+    *(u32x4*)(p.dst + bz * p.stride_dst + idx * 8u) = u32x4{w[0], w[1], w[2], w[3]};
 }
 
 // maize_pack_2d_u8: the same for 8-bit elements, optionally transposing: dst (rows_dst x cols_dst, compact)

@@ -496,12 +496,12 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
         pa.stride_src = d->batch > 1 ? (which == 0 ? d->stride_a : d->stride_b) : 0;
         pa.stride_dst = (uint64_t)pp.rows_dst * pp.cols_dst;
         const uint64_t total = (uint64_t)pp.rows_dst * pp.cols_dst;
-        const bool u8 = pp.elem_bytes == 1;                  // 64 x 64 tiles through LDS, batch in grid.z; else one element per thread, batch in grid.y
+        const bool u8 = pp.elem_bytes == 1;                  // 64 x 64 tiles through LDS, batch in grid.z; else one 8-element run per thread, batch in grid.y
         // A transposing copy whose source and destination both take 128-bit accesses: 128 x 128 tiles.
         const bool fast = u8 && pp.transpose && (((uintptr_t)pa.src | (uintptr_t)pa.dst) & 15u) == 0 &&
                           ((pp.rows | pp.cols | pp.ld_src | pp.rows_dst | pp.cols_dst) & 15u) == 0 && (pa.stride_src & 15u) == 0;
         const uint32_t edge = fast ? 128u : 64u;
-        const uint32_t pgrid[3] = {u8 ? (pp.cols_dst + edge - 1u) / edge : (uint32_t)((total + 255) / 256), u8 ? (pp.rows_dst + edge - 1u) / edge : d->batch,
+        const uint32_t pgrid[3] = {u8 ? (pp.cols_dst + edge - 1u) / edge : (uint32_t)((total / 8 + 255) / 256), u8 ? (pp.rows_dst + edge - 1u) / edge : d->batch,
                                    u8 ? d->batch : 1u};
         const uint32_t pblock[3] = {256, 1, 1};
         int32_t prc = launch_raw(ctx->device, (uint32_t)ctx->prop.sharedMemPerBlock, fast ? ctx->transpose_u8_fn : u8 ? ctx->pack_u8_fn : ctx->pack_fn, pgrid, pblock, 0,

@@ -47,8 +47,8 @@ def count(instrs, prefix):
 
 def test_every_registry_entry_has_its_device_kernel(kernels):
     for name in mz.kernel_names():
-        assert name.replace("_packed", "_splitk").replace("_trb", "") in kernels, name      # registry entries that reuse a device kernel
-    for helper in ("maize_gemm_splitk_reduce", "maize_pack_2d", "maize_pack_2d_u8"):
+        assert name.replace("_packed_gen", "_gen").replace("_packed", "_splitk").replace("_trb", "") in kernels, name      # registry entries that reuse a device kernel
+    for helper in ("maize_gemm_splitk_reduce", "maize_pack_2d", "maize_pack_2d_u8", "maize_transpose_u8"):
         assert helper in kernels
 
 

@@ -69,6 +69,14 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         assert p["block"] == (256, 1, 1)
         assert gx == cdiv(n, 64) and gy == cdiv(m, 64)
         assert p["workspace_bytes"] == 0 and p["ksplit"] == 0
+    elif name.endswith("_packed_gen"):
+        # the general-epilogue kernel on zero-padded copies, C stored by the first pass: persistent over the tiles, the
+        # workspace holds the copies only, no reduce pass.  C takes 128-bit stores.
+        n8, k8 = (n + 7) // 8 * 8, (k + 63) // 64 * 64           # K padded to whole K tiles
+        assert n8 == n and p["reduce_grid"] == 0 and p["ksplit"] == 0 and p["split_first"] == 0
+        resident = cus - cus % 8 if cus >= 8 else cus
+        assert p["block"] == (256, 1, 1) and gy == 1 and gx == min(cdiv(m, 256) * cdiv(n, 256) * batch, resident)
+        assert TICKET_BYTES <= p["workspace_bytes"] <= TICKET_BYTES + 2 * batch * (m * k8 + n8 * k8)
     elif packed:
         # the split-K kernels on zero-padded copies: work items over the padded extents, then the reduce pass
         # over the real C; the workspace also holds the copies
@@ -185,7 +193,8 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
         (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",      # odd N: operands read where they lie, C written element-wise by the reduce pass
         (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
-        (4096, 4096, 4100, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",      # K % 8 != 0: both operands repacked
+        (4096, 4096, 4100, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed_gen",  # K % 8 != 0: both operands repacked, C stored by the first pass
+        (64, 4096, 4100, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_packed",        # ... few tiles: split over K, reduce pass
         (511, 513, 1027, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_packed",       # K % 8 != 0 again
         (100, 203, 72, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",                  # too small to pay for the copies
         (17, 50257, 768, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",       # no copy of B is needed: odd rows are read where they lie

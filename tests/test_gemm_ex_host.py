@@ -66,7 +66,8 @@ def test_dispatch_of_extended_descriptors():
     p1 = mz.gemm_plan(ex(**big, ldc=4100))
     assert p1["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p1["ksplit"] == 1 and p1["reduce_grid"] > 0
     # ... and only K % 8 != 0 still needs padded copies
-    assert mz.gemm_plan(ex(4096, 4096, 4100))["kernel"] == "maize_gemm_bf16_mt256_nn_packed"
+    assert mz.gemm_plan(ex(4096, 4096, 4100))["kernel"] == "maize_gemm_bf16_mt256_nn_packed_gen"       # C takes 128-bit stores: no reduce pass
+    assert mz.gemm_plan(ex(4096, 4100, 4100))["kernel"] == "maize_gemm_bf16_mt256_nn_packed"           # N % 8 != 0: C through the reduce pass
     assert mz.gemm_plan(ex(64, 64, 64, lda=68))["kernel"] == "maize_gemm_bf16_wave32"          # unless the product is small
     # alpha / beta / fp32 C: the macro-tile kernels with the general epilogue; the plain ones refuse
     for kw in (dict(alpha=0.5), dict(beta=1.0), dict(out_type=mz.OUT_F32)):

@@ -365,12 +365,30 @@ def test_packed_kernels_odd_extents(ctx, oracle, layout, shape):
     run_packed(ctx, oracle, m, n, k, layout, name.replace("_bf16_", "_f16_"), half=True, a_off=1, ldc=n + 3, label="packed half")
 
 
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape", [(300, 520, 1027), (257, 264, 77), (1024, 2048, 1028), (520, 264, 129), (33, 24, 65)])
+def test_packed_kernels_that_store_c_themselves(ctx, oracle, layout, shape):
+    """K % 8 != 0 with a C that takes 128-bit stores: the general-epilogue kernel on the zero-padded copies, no fp32
+    partial tiles, no reduce pass -- every epilogue, views of A and B on odd leading dimensions and 2-byte offsets."""
+    m, n, k = shape
+    name = "maize_gemm_bf16_mt256_" + ("nt" if layout == mz.LAYOUT_NT else "nn") + "_packed_gen"
+    bcols = n if layout == mz.LAYOUT_NN else k
+    run_packed(ctx, oracle, m, n, k, layout, name, label="packed_gen")
+    run_packed(ctx, oracle, m, n, k, layout, name, lda=k + 3, ldb=bcols + 5, ldc=n + 8, label="packed_gen odd ld of A and B")
+    run_packed(ctx, oracle, m, n, k, layout, name, a_off=1, b_off=3, c_off=8, label="packed_gen 2-byte-aligned A and B")
+    run_packed(ctx, oracle, m, n, k, layout, name, alpha=-1.25, beta=0.75, ldc=n + 16, label="packed_gen alpha beta")
+    run_packed(ctx, oracle, m, n, k, layout, name, out_f32=True, alpha=0.5, beta=2.0, c_off=4, label="packed_gen f32")
+    run_packed(ctx, oracle, m, n, k, layout, name.replace("_bf16_", "_f16_"), half=True, a_off=1, ldc=n + 8, label="packed_gen half")
+    with pytest.raises(mz.MaizeError):          # a C off the 16-byte grid is the reduce pass's: refused by name
+        run_packed(ctx, oracle, m, n, k, layout, name, c_off=1, label="packed_gen unaligned C")
+
+
 def test_packed_path_is_what_odd_large_shapes_get(ctx, oracle):
     """The dispatcher's choice for large products that break the 16-byte rules, checked on sampled rows: padded copies
     only where K % 8 != 0 (a 16-byte chunk would straddle a row's end in K); an odd N alone needs none."""
     from tests.gpu_util import sample_rows
     for (m, n, k, layout, want) in ((1024, 4099, 1028, mz.LAYOUT_NN, "_packed"), (1000, 5003, 777, mz.LAYOUT_NT, "_packed"),
-                                    (2048, 2048, 1028, mz.LAYOUT_NN, "_packed"), (1024, 4099, 1024, mz.LAYOUT_NN, "_splitk"),
+                                    (2048, 2048, 1028, mz.LAYOUT_NN, "_packed_gen"), (1024, 4099, 1024, mz.LAYOUT_NN, "_splitk"),
                                     (1000, 5003, 776, mz.LAYOUT_NT, "_splitk")):
         brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
         a = mz.gen.uniform_bf16(m * k, 41)

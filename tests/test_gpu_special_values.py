@@ -29,6 +29,7 @@ FAMILIES = [
     ("maize_gemm_bf16_mt256_nt_splitk", 300, 264, 2056, NT),
     ("maize_gemm_bf16_mt256_nn_packed", 300, 515, 260, NN),
     ("maize_gemm_bf16_mt256_nt_packed", 100, 259, 133, NT),
+    ("maize_gemm_bf16_mt256_nn_packed_gen", 300, 520, 261, NN),      # zero-padded copies, C stored by the first pass
     ("maize_gemm_bf16_mt256_nn_edge", 4096, 4104, 512, NN),          # 272 tiles on 256 units: the last tile column is split over K
     ("maize_gemm_bf16_mt256_nt_ktail_edge", 4096, 4104, 520, NT),
     ("maize_gemm_bf16_skinny_nn", 13, 520, 2080, NN),
