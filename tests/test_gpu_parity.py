@@ -354,7 +354,7 @@ def test_dispatcher_choices(ctx):
     assert pick(4096, 4096, 4072) == "maize_gemm_bf16_mt256_nn_ktail"
     assert pick(4096, 4096, 4064) == "maize_gemm_bf16_mt256_nn_ktail"
     assert pick(4096, 4099, 4096) == "maize_gemm_bf16_mt256_nn_splitk"     # odd N: operands read where they lie, C written element-wise by the reduce pass
-    assert pick(4096, 4096, 4100) == "maize_gemm_bf16_mt256_nn_packed"     # K % 8 != 0: padded copies
+    assert pick(4096, 4096, 4100) == "maize_gemm_bf16_mt256_nn_packed_gen" # K % 8 != 0: padded copies, C stored by the first pass
     assert pick(33, 17, 65) == "maize_gemm_bf16_wave32"
 
 
