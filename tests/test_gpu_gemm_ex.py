@@ -241,6 +241,16 @@ def test_half_operands_skinny(ctx, oracle, m):
         assert took == "maize_gemm_bf16_skinny_nn", took
 
 
+@pytest.mark.parametrize("m", [24, 56])
+def test_row_group_skinny_knobs_and_half(ctx, oracle, m):
+    """The 17 .. 64-row streaming kernels for a row-major B under every epilogue and view knob, bf16 and half."""
+    name = "maize_gemm_bf16_skinny_nn_m32" if m <= 32 else "maize_gemm_bf16_skinny_nn_m64"
+    for kw in KNOBS:
+        assert run_ex(ctx, oracle, m, 1032, 2048, kernel=name, label="skinny rows", **kw) == name
+        assert run_ex(ctx, oracle, m, 1032, 2048, kernel=name, half=True, label="skinny rows half", **kw) == name
+    assert run_ex(ctx, oracle, 24, 2048, 2048, half=True, label="auto m32 half") == "maize_gemm_bf16_skinny_nn_m32"
+
+
 def test_half_full_size_4096_cubed(ctx, oracle):
     """The headline shape on half operands: sampled rows against the oracle."""
     from tests.gpu_util import sample_rows
