@@ -255,6 +255,12 @@ __device__ __forceinline__ void body_rows(const GemmArgs& p) {
     const uint32_t b0 = z * per;
     const uint32_t nb = b0 < nb_all ? (nb_all - b0 < per ? nb_all - b0 : per) : 0u;
 
+    // The waves of a workgroup walk K in step here, but the workgroups need not: slab s starts 7 s blocks into its
+    // range and wraps.  With a power-of-two row stride the rows of every slab would otherwise ask for the same few
+    // memory channels at the same time (64 x 128256 x 4096: 234 -> 189 us, 64 x 28672 x 8192: 109 -> 90; the one-group kernel gets the same effect from
+    // its waves being out of step).
+    const uint32_t wrot = nb ? (slab * 7u) % nb : 0u;
+
     floatx4 acc[MR][2];
 #pragma unroll
     for (int r = 0; r < MR; ++r) {
@@ -265,7 +271,8 @@ __device__ __forceinline__ void body_rows(const GemmArgs& p) {
     // Requests block j into `slot` (4 pieces per wave) and, before them, the A pieces this wave has the duty for.
     auto request = [&](uint32_t j, lds_ptr slot, int ai) {
         typedef __attribute__((address_space(3))) void* lvp;
-        const uint32_t kb = (b0 + j) * KB;
+        const uint32_t jr = j + wrot < nb ? j + wrot : j + wrot - nb;    // this workgroup's j-th block of the range
+        const uint32_t kb = (b0 + jr) * KB;
         const bool live = j < nb;
         const __amdgpu_buffer_rsrc_t rs_b = live ? rb : rnull;
         const __amdgpu_buffer_rsrc_t rs_a = live ? ra : rnull;
