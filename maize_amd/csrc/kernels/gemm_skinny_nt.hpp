@@ -108,7 +108,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // A wave fetches, reads and multiplies only its own 32 rows, so the waves need not walk K in step:
     // wave w starts an eighth of the range further on than wave w-1 (and wraps).  With a power-of-two
     // row stride, the 256 rows of a block at one k would otherwise sit on few memory channels at once.
-    const uint32_t wrot = (wave * nb) >> 3;
+    // ... and slab s starts 13 s blocks further on again: the eight offsets of the waves would otherwise be the same in
+    // every workgroup of the chip (16 x 28672 x 8192: 104 -> 85 us, 16 x 128256 x 4096: 190 -> 177; multipliers 3 .. 13
+    // within 2 % of each other).
+    const uint32_t wrot = nb ? (((wave * nb) >> 3) + slab * 13u) % nb : 0u;
 
     floatx4 acc[2];
     acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -255,11 +258,11 @@ __device__ __forceinline__ void body_rows(const GemmArgs& p) {
     const uint32_t b0 = z * per;
     const uint32_t nb = b0 < nb_all ? (nb_all - b0 < per ? nb_all - b0 : per) : 0u;
 
-    // The waves of a workgroup walk K in step here, but the workgroups need not: slab s starts 7 s blocks into its
+    // The waves of a workgroup walk K in step here, but the workgroups need not: slab s starts 3 s blocks into its
     // range and wraps.  With a power-of-two row stride the rows of every slab would otherwise ask for the same few
     // memory channels at the same time (64 x 128256 x 4096: 234 -> 189 us, 64 x 28672 x 8192: 109 -> 90; the one-group kernel gets the same effect from
     // its waves being out of step).
-    const uint32_t wrot = nb ? (slab * 7u) % nb : 0u;
+    const uint32_t wrot = nb ? (slab * 3u) % nb : 0u;
 
     floatx4 acc[MR][2];
 #pragma unroll
