@@ -2,6 +2,7 @@
 
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 namespace maize {
@@ -534,6 +535,28 @@ uint32_t skinny_ksplit(const Dims& s, uint32_t batch, uint32_t compute_units) {
     if (slabs * ks > compute_units && compute_units / slabs >= 1u) ks = (uint32_t)(compute_units / slabs);
     return cdiv(nblk, cdiv(nblk, ks));                     // no empty range
 }
+// The kernels for 17 .. 64 rows share the additions of a slab's K ranges among its workgroups (gemm_skinny.hpp, finish())
+// where the slab's partial tiles are 256 KiB or more -- below that the last workgroup to arrive is faster alone, and so
+// it is with 16 rows even at 16 ranges, where a part is 1 KiB (measured, same box, last arriver -> shared: 64 x 14336 x
+// 4096 NN 30.9 -> 28.3 us, NT 28.8 -> 27.1, E4M3 20.4 -> 18.3; 32 x 2048 x 8192 NT in 16 ranges 20.1 -> 14.2; but
+// 16 x 4096 x 14336 in 16 ranges NN 26.8 -> 31.1, NT 26.0 -> 28.5).  A workgroup
+// waits for the others at most this long (their skew: the grids keep a slab's workgroups resident together; the bound
+// matters only when something else holds compute units).  MAIZE_HIP_SPLIT_WAIT_US overrides it for diagnosis (0: nobody
+// waits, the last to arrive adds everything).
+static uint32_t split_wait_us() {
+    if (const char* e = std::getenv("MAIZE_HIP_SPLIT_WAIT_US")) {
+        const long v = std::strtol(e, nullptr, 10);
+        return v < 0 ? 0u : v > 60000 ? 60000u : (uint32_t)v;
+    }
+    return 30u;
+}
+static void share_additions(LaunchDims* ld, uint32_t rows, uint32_t ks, uint64_t slabs) {
+    ld->wait_us = 0;
+    if (rows >= 32u && ks >= 2u && ks <= 16u && (rows / 16u) * ks >= 16u && slabs <= 8192u) {
+        ld->split_first |= 2u;
+        ld->wait_us = split_wait_us();
+    }
+}
 static bool skinny_plan_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld, uint32_t rows) {
     const Dims s = dims_of(d);
     const uint32_t ks = skinny_ksplit(s, d.gemm.batch, compute_units ? compute_units : 256u);
@@ -544,6 +567,7 @@ static bool skinny_plan_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_uni
     ld->lds_bytes = 0;
     ld->ksplit = ks;
     ld->split_first = skinny_c_by_elements(d) ? 1u : 0u;
+    share_additions(ld, rows, ks, (uint64_t)ld->grid[0] * d.gemm.batch);
     ld->reduce_grid = 0;
     ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * rows * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets
@@ -601,6 +625,7 @@ static bool skinny_nt_plan_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_
     ld->lds_bytes = 0;
     ld->ksplit = ks;
     ld->split_first = skinny_nt_c_by_elements(d) ? 1u : 0u;
+    share_additions(ld, rows, ks, (uint64_t)ld->grid[0] * d.gemm.batch);
     ld->reduce_grid = 0;
     ld->workspace_bytes = ks > 1 ? kTicketBytes + (size_t)ld->grid[0] * d.gemm.batch * ks * rows * 256u * 4u : 0;
     return ld->workspace_bytes < (1ull << 31);            // the kernel addresses it with 32-bit offsets

@@ -35,6 +35,7 @@ struct LaunchDims {
     uint32_t ksplit;          // split-K kernels: number of K ranges (0 = kernel takes no workspace)
     uint32_t split_first;     // tiled kernels: edge mode << 30 | 1 + number of tiles computed whole (0 = every tile whole)
     size_t workspace_bytes;   // bytes of zero-initialised, library-owned workspace the launch needs
+    uint32_t wait_us;         // few-row kernels sharing the split-K additions: bound of a workgroup's wait for the slab's other K ranges, microseconds
     uint32_t reduce_grid;     // split-K macro-tile kernels: grid.x of the maize_gemm_splitk_reduce pass that follows (0 = none)
     PackPlan pack_a, pack_b;  // packed kernels: operands repacked first; the product then runs on n_padded x k_padded
     uint32_t n_padded, k_padded;

@@ -93,10 +93,10 @@ __device__ __forceinline__ void finish(const GemmArgs& p, uint16_t* Cg, const fl
     //
     // The last workgroup to arrive adds all the tiles of its slab.  One workgroup draws about 50 GB/s of such data,
     // so this costs ks x MR x 16 KiB at that rate with the rest of the chip idle (1.3 us for 16 rows and 4 ranges,
-    // 5 us for 64 rows).  Sharing the additions among the slab's workgroups (each waits, with a bound, until all
-    // have arrived and adds the part its arrival number names) was built and measured: the polling loads and the
-    // two more atomics per workgroup on the slab's counters cost 1.2 us at 16 rows x 4 ranges (22.8 against 21.6 us)
-    // and 2 us at 8 ranges of an 8192 x 8192 B; it won only from 16 ranges or 64 rows up (-1.7 us), so it stayed out.
+    // 5 us for 64 rows).  Sharing the additions among the slab's workgroups costs polling loads and two more atomics
+    // per workgroup: 1.2 us at 16 rows x 4 ranges (22.8 against 21.6 us), 2 us at 8 ranges of an 8192 x 8192 B; it
+    // wins from 256 KiB of tiles per slab up (16 ranges, or 64 rows x 4 ranges: -1.7 us).  The dispatcher asks for it
+    // there (bit 1 of GemmArgs::reserved); that path is share() below.
     constexpr int COHERENT = 17;                          // buffer cache policy: sc0 | sc1
     constexpr uint32_t TILE_BYTES = 16u * MR * SN * 4u;
     typedef __attribute__((address_space(3))) volatile uint32_t* lds_word_ptr;
@@ -115,6 +115,92 @@ __device__ __forceinline__ void finish(const GemmArgs& p, uint16_t* Cg, const fl
                                                    0, COHERENT);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wave's partial tile has reached memory
     __syncthreads();
+    if (p.reserved & 2u) {
+        // ---- the additions shared among the slab's workgroups --------------------------------------------------
+        //   * a workgroup counts itself in with one atomic add on the slab's word (low half: arrivals; high half: one
+        //     bit per arrival number that has given up); the value returned is its arrival number t;
+        //   * the last to arrive (t = ks - 1) never waits: the returned value also tells it which earlier arrivals gave
+        //     up, and it adds its own part of the tile and theirs;
+        //   * any other workgroup polls the word for a bounded time (reserved >> 8 microseconds; the dispatcher's
+        //     grids keep a slab's workgroups resident together, so the wait is their skew).  Once all have arrived it
+        //     adds part t.  If the time runs out it sets bit t with another atomic add on the same word and leaves --
+        //     unless that add returns a full arrival count: then the last arrival has already looked at the word
+        //     without the bit, and the workgroup adds part t after all.  One word, so the two cannot miss each other;
+        //   * once a workgroup knows its parts it no longer touches the word: it counts itself out on a second counter
+        //     while its loads are in flight, and the last one out zeroes both for the next launch.
+        // Additions run in range order whoever makes them: the bits do not depend on the race.  No workgroup waits
+        // without a bound and none depends on another being scheduled; with a bound of 0 the last to arrive adds
+        // everything, in one pass over the tile.  ks <= 16, slab_id < 8192 (the dispatcher checks).
+        uint32_t* const word_ctr = counters + slab_id;
+        if (tid == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(word_ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t t = old & 0xFFFFu;             // arrival number
+            uint32_t mine;
+            if (t == ks - 1u) mine = (1u << t) | (old >> 16);
+            else {
+                const uint64_t limit = (uint64_t)(p.reserved >> 8) * 100u;        // the wall clock ticks at 100 MHz
+                const uint64_t t0 = wall_clock64();
+                bool all_in = false;
+                while (!all_in && wall_clock64() - t0 < limit) {
+                    __builtin_amdgcn_s_sleep(1);
+                    all_in = (__hip_atomic_load(word_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xFFFFu) == ks;
+                }
+                if (!all_in)
+                    all_in = (__hip_atomic_fetch_add(word_ctr, 1u << (16u + t), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xFFFFu) == ks;
+                mine = all_in ? 1u << t : 0u;
+            }
+            *ticket = mine;
+        }
+        __syncthreads();
+        const uint32_t parts = *ticket;
+        // Count out.  Every lane runs the atomic, only thread 0's offset is inside the descriptor: branch-free, so that
+        // the returned value comes back while the loads below are in flight.
+        const __amdgpu_buffer_rsrc_t rctr = make_rsrc(p.workspace, 65536u);
+        const uint32_t left = (uint32_t)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, rctr, tid == 0 ? (8192u + slab_id) * 4u : 0xFFFFFFF0u, 0, 1);
+        if (parts) {
+            constexpr uint32_t UNITS = MR * 512u;             // runs of 8 columns (32 bytes of fp32) in a tile
+            constexpr uint32_t DROP = 0xFFFFFFE0u;            // past the descriptor: reads as zeros
+            const bool whole = parts == (1u << ks) - 1u;      // everything is ours: one pass over the tile
+            const uint32_t per = whole ? UNITS : (UNITS + ks - 1u) / ks;          // units per part
+            for (uint32_t rest = whole ? 1u : parts; rest; rest &= rest - 1u) {
+                const uint32_t part = (uint32_t)__builtin_ctz(rest);
+                const uint32_t u_end = (part + 1u) * per < UNITS ? (part + 1u) * per : UNITS;
+                for (uint32_t u = part * per + tid; u < u_end; u += 512u) {
+                    const uint32_t row = u >> 5, cq = (u & 31u) * 8u;
+                    const uint32_t off = tile0 + (row * SN + cq) * 4u;
+                    // all ranges of a unit are requested before the first addition, 8 at a time
+                    floatx4 s_lo = floatx4{0.f, 0.f, 0.f, 0.f}, s_hi = floatx4{0.f, 0.f, 0.f, 0.f};
+                    for (uint32_t z0 = 0; z0 < ks; z0 += 8u) {
+                        floatx4 t_lo[8], t_hi[8];
+#pragma unroll
+                        for (int v = 0; v < 8; ++v) {
+                            const uint32_t o = z0 + v < ks ? off + (z0 + v) * TILE_BYTES : DROP;
+                            t_lo[v] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o, 0, COHERENT));
+                            t_hi[v] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, o + 16u, 0, COHERENT));
+                        }
+#pragma unroll
+                        for (int v = 0; v < 8; ++v) {
+                            if (z0 + v == 0u) { s_lo = t_lo[0]; s_hi = t_hi[0]; }
+                            else if (z0 + v < ks) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) { s_lo[e] += t_lo[v][e]; s_hi[e] += t_hi[v][e]; }
+                            }
+                        }
+                    }
+                    const uint32_t col = n0 + cq;
+                    if (row < M && col < N) {
+                        const float v[8] = {s_lo[0], s_lo[1], s_lo[2], s_lo[3], s_hi[0], s_hi[1], s_hi[2], s_hi[3]};
+                        if (c_elems) store_c_elems<8>(p, Cg, (uint64_t)row * ldc + col, v, N - col);
+                        else store_c_run<8>(p, Cg, (uint64_t)row * ldc + col, v);
+                    }
+                }
+            }
+        }
+        if (tid == 0 && left == ks - 1u) {                // last one out: nobody touches the counters any more
+            counters[slab_id] = 0u; counters[8192u + slab_id] = 0u;
+        }
+        return;
+    }
     if (tid == 0) *ticket = __hip_atomic_fetch_add(&counters[slab_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*ticket != ks - 1u) return;                       // not the last split of this slab to finish

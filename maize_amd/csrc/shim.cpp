@@ -470,7 +470,7 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
         return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s cannot run M=%u N=%u K=%u batch=%u (grid limit)", ki.name,
                     d->c.nrows, d->c.ncols, d->a.ncols, d->batch);
     args.ksplit = ld.ksplit;
-    args.reserved = ld.split_first;
+    args.reserved = ld.split_first | (ld.wait_us << 8);    // few-row kernels: bit 0 = C by elements, bit 1 = shared additions, bits 8.. = their wait bound
     if (ld.workspace_bytes && fixed) {
         if (ld.workspace_bytes > fixed->bytes)
             return fail(MAIZE_ERR_ARG, "gemm_noalloc: kernel %s needs %zu bytes of scratch for M=%u N=%u K=%u batch=%u, the fixed "

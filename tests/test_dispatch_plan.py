@@ -138,6 +138,11 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert p["workspace_bytes"] < (1 << 31)
     elif name.startswith("maize_gemm_bf16_skinny_nn"):
         rows = {"maize_gemm_bf16_skinny_nn": 16, "maize_gemm_bf16_skinny_nn_m32": 32, "maize_gemm_bf16_skinny_nn_m64": 64}[name]
+        # bit 1 of the launch flag: the slab's workgroups share the additions -- row-group kernels with 256 KiB or more
+        # of partial tiles per slab (the kernel then uses two counters per slab and 16 bits of arrival numbers)
+        shares = bool(p["split_first"] & 2)
+        assert shares == (rows >= 32 and (rows // 16) * p["ksplit"] >= 16 and p["ksplit"] >= 2)
+        assert not shares or (p["ksplit"] <= 16 and gx * batch <= 8192)
         assert p["block"] == (512, 1, 1)
         assert layout == mz.LAYOUT_NN and m <= rows and n % 8 == 0
         ks = p["ksplit"]
@@ -155,6 +160,9 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert p["workspace_bytes"] == 0
     elif name.startswith("maize_gemm_bf16_skinny_nt"):
         rows = {"maize_gemm_bf16_skinny_nt": 16, "maize_gemm_bf16_skinny_nt_m32": 32, "maize_gemm_bf16_skinny_nt_m64": 64}[name]
+        shares = bool(p["split_first"] & 2)
+        assert shares == (rows >= 32 and (rows // 16) * p["ksplit"] >= 16 and p["ksplit"] >= 2)
+        assert not shares or (p["ksplit"] <= 16 and gx * batch <= 8192)
         assert p["block"] == (512, 1, 1)
         assert layout == mz.LAYOUT_NT and m <= rows and n % 8 == 0 and k % 8 == 0
         ks = p["ksplit"]

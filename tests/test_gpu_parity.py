@@ -500,6 +500,46 @@ def test_skinny_nn_row_groups_agree_with_the_one_group_kernel(ctx):
         assert np.array_equal(run_gemm(ctx, a, b, m, n, k, kernel=kernel), one), kernel
 
 
+@pytest.mark.parametrize("case", [(64, 14336, 4096, mz.LAYOUT_NN), (64, 14336, 4096, mz.LAYOUT_NT), (24, 512, 16384, mz.LAYOUT_NN),
+                                  (32, 2048, 8192, mz.LAYOUT_NT), (50, 4101, 2080, mz.LAYOUT_NN)],
+                         ids=lambda c: "x".join(map(str, c[:3])) + ("t" if c[3] else ""))
+def test_row_group_kernels_share_the_additions_whatever_the_wait(ctx, oracle, case):
+    """17 .. 64 rows, 256 KiB or more of partial tiles per slab: the workgroups of a slab share the additions.  Who
+    adds which part depends on a bounded wait; the bits must not.  The bound is forced from the host: the default,
+    1 us (some workgroups give up, some do not) and 0 (everybody gives up: the last to arrive adds everything)."""
+    import os
+    m, n, k, layout = case
+    tag = "nt" if layout == mz.LAYOUT_NT else "nn"
+    kernel = f"maize_gemm_bf16_skinny_{tag}_{'m32' if m <= 32 else 'm64'}"
+    a, b = inputs(m, n, k, dist="normal")
+    brows, bcols = (n, k) if layout == mz.LAYOUT_NT else (k, n)
+    d = mz.gemm_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x1000, brows, bcols), mz.GlobalMatrix(0x1000, m, n), layout=layout)
+    plan = mz.gemm_plan(d, kernel=kernel, compute_units=ctx.info()["compute_units"])
+    groups = 2 if m <= 32 else 4
+    assert (plan["split_first"] & 2) == (2 if groups * plan["ksplit"] >= 16 else 0), plan
+    assert plan["split_first"] & 2, "a case of this test is meant to share"
+    results = {}
+    old = os.environ.get("MAIZE_HIP_SPLIT_WAIT_US")
+    try:
+        for wait in (None, "1", "0"):
+            if wait is None:
+                os.environ.pop("MAIZE_HIP_SPLIT_WAIT_US", None)
+            else:
+                os.environ["MAIZE_HIP_SPLIT_WAIT_US"] = wait
+            _say(f"{kernel} {case[:3]} wait bound {wait or 'default'} us, {plan['ksplit']} ranges")
+            for rep in range(3):
+                results[(wait, rep)] = run_gemm(ctx, a, b, m, n, k, layout=layout, kernel=kernel)
+    finally:
+        if old is None:
+            os.environ.pop("MAIZE_HIP_SPLIT_WAIT_US", None)
+        else:
+            os.environ["MAIZE_HIP_SPLIT_WAIT_US"] = old
+    first = results[(None, 0)]
+    check_against_oracle(oracle, first, a, b, m, n, k, layout=layout, label=f"{kernel} shared additions")
+    for key, got in results.items():
+        assert np.array_equal(got, first), key
+
+
 def test_skinny_nn_unaligned_b_and_c(ctx, oracle):
     """B at a 2-byte offset with an odd leading dimension, C at an odd offset: same kernel, same bar, nothing written
     outside C."""
