@@ -112,7 +112,8 @@ typedef enum { MAIZE_OUT_SAME = 0, MAIZE_OUT_BF16 = 0, MAIZE_OUT_F32 = 1, MAIZE_
  * catalogue's Sm89MmaF8F32_* entries (crates/maize_tile/src/mma/sm89.rs:13-45; u8-backed,
  * crates/maize_core/src/ty/sized.rs:68-69): A and B hold one byte per element, dimensions, leading
  * dimensions and batch strides still count elements, and the matrix instruction is
- * v_mfma_f32_16x16x128_f8f6f4 when B is stored N x K (MAIZE_LAYOUT_NT) with 16-byte aligned rows.
+ * v_mfma_f32_16x16x128_f8f6f4 when the rows of A and B start on 16-byte boundaries and K % 16 == 0, with B stored
+ * N x K (MAIZE_LAYOUT_NT) or K x N with N % 16 == 0 (MAIZE_LAYOUT_NN).
  * MAIZE_IN_E4M3_E5M2 / MAIZE_IN_E5M2_E4M3: A of the first format, B of the second (the catalogue's mixed pairs,
  * sm89.rs:34-45).
  * MAIZE_IN_F32 / MAIZE_IN_F64: the catalogue's tf32 -> f32 and f64 -> f64 entries (Sm80MmaTf32F32_16x8x4 / _16x8x8,

@@ -115,9 +115,23 @@ bool f8_nt_common(const maize_gemm_ex_desc_t& d) {
     if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21) || l.c >= (1u << 21)) return false;
     return true;
 }
+// A row-major (K x N) 8-bit B read where it lies: its tile lands in 16-byte chunks of 16 columns, so N % 16 == 0 and rows
+// of B on 16-byte boundaries; A and C as above.
+bool f8_nn_common(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    if (!nn(d) || (s.k & 15u) || (s.n & 15u)) return false;
+    if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr | (uintptr_t)d.gemm.c.ptr) & 15u) return false;
+    if ((l.a | l.b) & 15u || (l.c & 7u)) return false;
+    if (d.gemm.batch > 1 && (((d.gemm.stride_a | d.gemm.stride_b) & 15u) || (d.gemm.stride_c & 7u))) return false;
+    if (s.k >= (1u << 21) || s.n >= (1u << 21) || l.a >= (1u << 21) || l.b >= (1u << 21) || l.c >= (1u << 21)) return false;
+    return true;
+}
 #define MAIZE_F8_SUPPORTS(tag, type) \
     bool tag##_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d) && plain_epilogue(d); } \
-    bool tag##_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d); }
+    bool tag##_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d); } \
+    bool tag##_nn_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nn_common(d) && plain_epilogue(d); } \
+    bool tag##_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nn_common(d); }
 MAIZE_F8_SUPPORTS(e4m3, MAIZE_IN_E4M3)
 MAIZE_F8_SUPPORTS(e5m2, MAIZE_IN_E5M2)
 MAIZE_F8_SUPPORTS(e4m3e5m2, MAIZE_IN_E4M3_E5M2)
@@ -714,6 +728,9 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_" #tag "_mt256_nt", nullptr, tag##_nt_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_gen", nullptr, tag##_nt_gen_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan}, \
+    {"maize_gemm_" #tag "_mt256_nn", nullptr, tag##_nn_supports, mt256_plan}, \
+    {"maize_gemm_" #tag "_mt256_nn_gen", nullptr, tag##_nn_gen_supports, mt256_plan}, \
+    {"maize_gemm_" #tag "_mt256_nn_splitk", nullptr, tag##_nn_gen_supports, splitk_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_packed", "maize_gemm_" #tag "_mt256_nt_splitk", tag##_packed_supports, packed8_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_trb", "maize_gemm_" #tag "_mt256_nt", tag##_trb_supports, trb_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_trb_gen", "maize_gemm_" #tag "_mt256_nt_gen", tag##_trb_gen_supports, trb_plan},
@@ -770,6 +787,13 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt%s", kTag[d.in_type - MAIZE_IN_E4M3], plain_epilogue(d) ? "" : "_gen");
         const int fi = kernel_index(name);
         if (fi >= 0 && kKernels[fi].supports(d) && (s.k >= 256 || (s.m >= 128 && s.n >= 128))) return (uint32_t)fi;
+        // A row-major B with 16-byte rows and N % 16 == 0: the same kernels with transposing LDS reads for B.
+        std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nn_splitk", kTag[d.in_type - MAIZE_IN_E4M3]);
+        const int ns = kernel_index(name);
+        if (ns >= 0 && kKernels[ns].supports(d) && splitk_ranges(s, d.gemm.batch, compute_units, 128) >= 2u) return (uint32_t)ns;
+        std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nn%s", kTag[d.in_type - MAIZE_IN_E4M3], plain_epilogue(d) ? "" : "_gen");
+        const int ni = kernel_index(name);
+        if (ni >= 0 && kKernels[ni].supports(d) && (s.k >= 256 || (s.m >= 128 && s.n >= 128))) return (uint32_t)ni;
         // A row-major B, odd extents or unaligned rows: transposed / padded copies and the split-K kernel, when the
         // product is large enough to pay for the extra launches and the copies (same rule as for 16-bit operands).
         // A row-major B with everything else aligned and enough tiles: only B is copied (transposed), no reduce pass.

@@ -126,14 +126,16 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 
 #define MAIZE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-// F8: -1 = 16-bit operands; else 8-bit operands (one byte per element, both K-contiguous), bit 0: A is E5M2, bit 1:
-// B is E5M2 (else E4M3).  The 8-bit form is the same kernel on the same 128-byte LDS rows: a K tile is 128 elements
-// deep and one v_mfma_f32_16x16x128_f8f6f4 deep (not two 32-deep halves), a fragment is two 16-byte reads, and a K
-// step is four "eighths" of 16 MFMAs with the barrier before the third.
+// F8: -1 = 16-bit operands; else 8-bit operands (one byte per element), bit 0: A is E5M2, bit 1: B is E5M2 (else
+// E4M3).  The 8-bit form is the same kernel on the same 128-byte LDS rows: a K tile is 128 elements deep and one
+// v_mfma_f32_16x16x128_f8f6f4 deep (not two 32-deep halves), a fragment is two 16-byte reads, and a K step is four
+// "eighths" of 16 MFMAs with the barrier before the third.  A row-major (K x N) 8-bit B lands as 128 rows of 256
+// bytes (maps::sk8_*) and a fragment is four transposing 8-byte reads (ds_read_b64_tr_b8), two per MFMA slot.
 template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
-    static_assert(!IS8 || (NT && !F16 && !EDGE), "8-bit operands: both K-contiguous, no edge splitting");
+    static_assert(!IS8 || (!F16 && !EDGE), "8-bit operands: no edge splitting");
+    constexpr bool TR8 = IS8 && !NT;                    // 8-bit row-major B: transposing reads
     constexpr uint32_t ES = IS8 ? 1u : 2u;              // bytes per element of A and B
     constexpr uint32_t CH = 16u / ES;                   // elements per 16-byte chunk
     constexpr int BKE = IS8 ? 128 : BK;                 // elements per K tile (128 bytes per row either way)
@@ -282,14 +284,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             if (NT) {
                 b_vo[i] = (row * ldb + c * CH) * ES;
             } else {
-                const uint32_t brow = maps::sk_piece_row(wave * 8u + i, lane);
-                const uint32_t bc = maps::sk_piece_chunk(wave * 8u + i, lane);
-                b_vo[i] = ((brow * ldb + n0 + bc * 8u) * 2u) | ((n0 + bc * 8u) < N ? 0u : OOB);
+                const uint32_t brow = TR8 ? maps::sk8_piece_row(wave * 8u + i, lane) : maps::sk_piece_row(wave * 8u + i, lane);
+                const uint32_t bc = TR8 ? maps::sk8_piece_chunk(wave * 8u + i, lane) : maps::sk_piece_chunk(wave * 8u + i, lane);
+                b_vo[i] = ((brow * ldb + n0 + bc * CH) * ES) | ((n0 + bc * CH) < N ? 0u : OOB);
             }
         }
     };
     select_tile(pid);
-    const uint64_t b_view = ((uint64_t)(K - 1u) * ldb + N) * 2u;               // bytes of a K x N B
+    const uint64_t b_view = ((uint64_t)(K - 1u) * ldb + N) * ES;               // bytes of a K x N B
     // Issues piece pc (0..7 = A, 8..15 = B) of the tile that starts at k into stages (sa, sb).
     auto dma = [&](int pc, lds_ptr sa, lds_ptr sb, uint32_t k) {
         typedef __attribute__((address_space(3))) void* lvp;
@@ -300,7 +302,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         if (!is_a && !NT) {
             // K x N B: the descriptor starts at row k of B (scalar 64-bit arithmetic, once per K tile) and ends with
             // the view; rows at or past K are past its end.
-            const uint64_t skip = (uint64_t)k * ldb * 2u;
+            const uint64_t skip = (uint64_t)k * ldb * ES;
             const uint32_t bytes = k < k_end ? span(b_view - skip) : 0u;       // k < k_end <= K: skip < b_view
             const __amdgpu_buffer_rsrc_t rs = make_rsrc(Bg + skip, bytes);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, b_vo[i], 0, 0, DMA_AUX);
@@ -326,7 +328,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // Base registers of the reads: LDS address of the operand's array + the lane's offset; everything
     // else of an address (stage, fragment, K half of the K x N tile) is a compile-time offset.
     uint32_t a_rd[2], b_rd[8];
-    if (IS8 || NT) {
+    if (NT) {
         // 8-bit operands, 16x16x128: lane l holds row l%16 and 32 bytes of K.  Which 32 is free as long as A and B agree
         // (the instruction sums over all of K): the two chunks l/16 and 4 + l/16, i.e. exactly the two reads of the
         // 16-bit kernel's K halves -- the access pattern that measures free of bank conflicts (chunks 2 (l/16) and
@@ -340,7 +342,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh) a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * 128u, kh, lane);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) b_rd[j] = (uint32_t)(uintptr_t)B0 + maps::sk_tr_offset(wn * 8u + j, 0, lane);
+        for (int j = 0; j < 8; ++j)
+            b_rd[j] = (uint32_t)(uintptr_t)B0 + (TR8 ? maps::sk8_tr_offset(wn * 8u + j, 0, 0, lane) : maps::sk_tr_offset(wn * 8u + j, 0, lane));
     }
 
     // Fragment registers.  A K half (32 deep) of the wave's sub-tile is walked in four eighths of 16 MFMAs
@@ -356,10 +359,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     bf16x8 fb[2][4];
     short4v fbl[2][4], fbh[2][4];
     u32x4 fa8[2][4][2], fb8[2][4][2];
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    u32x2 fb8t[2][4][4];                                // 8-bit row-major B: register pair 2 kk + h of a fragment
     constexpr int NAR = IS8 ? 8 : 4;                    // reads that bring in one A group
-    constexpr int NBR = (IS8 || !NT) ? 8 : 4;           // ... one B group (transposing reads are 64-bit, 8-bit fragments two reads)
-    // Read r of a group is issued in MFMA slot r * RSTRIDE of the eighth.
+    constexpr int NBR = TR8 ? 16 : (IS8 || !NT) ? 8 : 4; // ... one B group (transposing reads are 64-bit, 8-bit fragments two or four reads)
+    // Reads r = s * RPS .. of a group are issued in MFMA slot s of the eighth: all of them in its first half, so that
+    // the last has half an eighth to arrive.
     constexpr int RSTRIDE = 1;
+    constexpr int RPS = TR8 ? 2 : 1;
     static_assert(8 * RSTRIDE <= 16, "the reads of a group must fit into the 16 slots of an eighth");
     // 128-bit read at base + 2048 * n (n = stage * 16 + fragment), 64-bit transposing read at
     // base + 2048 * n (n = stage * 16 + kh * 8 + h).  The offsets are immediates: one case per value,
@@ -381,6 +388,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         }
     };
 #undef MAIZE_RD_CASE
+#define MAIZE_RD_CASE(n) case n: asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(base), "n"((n) * 2048)); break;
+    auto lds_read_tr8 = [&](u32x2& dst, uint32_t base, int n) {     // n = stage * 16 + kk * 8 + h
+        switch (n) {
+            MAIZE_RD_CASE(0) MAIZE_RD_CASE(1) MAIZE_RD_CASE(8) MAIZE_RD_CASE(9) MAIZE_RD_CASE(16) MAIZE_RD_CASE(17) MAIZE_RD_CASE(24) MAIZE_RD_CASE(25)
+            default: __builtin_unreachable();
+        }
+    };
+#undef MAIZE_RD_CASE
     // Read r (0..NAR-1) of A group ai, K half kh, of the tile in stage st.
     auto read_a = [&](int ai, int kh, int st, int r) {
         if (IS8) lds_read128(fa8[ai][r >> 1][r & 1], a_rd[r & 1], st * 16 + 4 * ai + (r >> 1));   // half r & 1 = the 16-bit kernel's kh
@@ -389,7 +404,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // Read r (0..NBR-1) of B group bi, K half kh, of the tile in stage st.
     auto read_b = [&](int bi, int kh, int st, int r) {
         const int buf = bi ^ (IS8 ? st : kh);
-        if (IS8) lds_read128(fb8[buf][r >> 1][r & 1], b_rd[r & 1], st * 16 + 4 * bi + (r >> 1));
+        if (TR8) lds_read_tr8(fb8t[buf][r >> 2][r & 3], b_rd[4 * bi + (r >> 2)], st * 16 + ((r >> 1) & 1) * 8 + (r & 1));
+        else if (IS8) lds_read128(fb8[buf][r >> 1][r & 1], b_rd[r & 1], st * 16 + 4 * bi + (r >> 1));
         else if (NT) lds_read128(fb[buf][r], b_rd[kh], st * 16 + 4 * bi + r);
         else {
             const int c = r >> 1, h = r & 1;                  // rows 32 kh + 4 h + ...: 16 KiB and 2 KiB further on
@@ -407,6 +423,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     typedef int i32x8 __attribute__((ext_vector_type(8)));
     auto operand8 = [&](const u32x4 (&f)[2]) -> i32x8 {
         return i32x8{(int)f[0][0], (int)f[0][1], (int)f[0][2], (int)f[0][3], (int)f[1][0], (int)f[1][1], (int)f[1][2], (int)f[1][3]};
+    };
+
+    auto b_operand8 = [&](int buf, int c) -> i32x8 {
+        if (!TR8) return operand8(fb8[buf][c]);
+        return i32x8{(int)fb8t[buf][c][0][0], (int)fb8t[buf][c][0][1], (int)fb8t[buf][c][1][0], (int)fb8t[buf][c][1][1],
+                     (int)fb8t[buf][c][2][0], (int)fb8t[buf][c][2][1], (int)fb8t[buf][c][3][0], (int)fb8t[buf][c][3][1]};
     };
 
     floatx4 acc[8][8];
@@ -448,7 +470,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // accumulator comes up again 128 MFMAs later: no dependent back-to-back issue.)
                 if (IS8)   // 8-bit operands: B is the first source, so cbsz carries B's format and blgp A's (0 = E4M3, 1 = E5M2)
                     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(acc[4 * ai + r4][4 * bi + c4])
-                                 : "v"(operand8(fb8[bi ^ cur][c4])), "v"(operand8(fa8[ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
+                                 : "v"(b_operand8(bi ^ cur, c4)), "v"(operand8(fa8[ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
                 else if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
                     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(bi ^ kh, c4)), "v"(fa[ai][r4]));
                 else
@@ -456,10 +478,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // Side work of this slot: the reads of the group the next eighth needs ...
                 if (s % RSTRIDE == 0) {
                     const int r = s / RSTRIDE;
-                    if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);                       // (0,0) -> (0,1): B group 1
+#pragma unroll
+                    for (int rb = r * RPS; rb < (r + 1) * RPS; ++rb) {
+                        if (h4 == 0 && rb < NBR) read_b(1, kh, cur, rb);                     // (0,0) -> (0,1): B group 1
+                        if (h4 == 3 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }   // next half or tile: B group 0
+                    }
                     if (h4 == 1 && r < NAR) read_a(1, kh, cur, r);                       // (0,1) -> (1,1): A group 1
                     if (h4 == 2 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }   // next half or tile: A group 0
-                    if (h4 == 3 && r < NBR) { if (!last_half) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }   // next half or tile: B group 0
                 }
                 // ... and the direct-to-LDS request scheduled for this slot (issue_slot): late pieces of
                 // tile t+1 (its stage was freed by the previous barrier) before this step's barrier, early

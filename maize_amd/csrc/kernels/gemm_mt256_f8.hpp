@@ -1,4 +1,4 @@
-// maize_gemm_{e4m3,e5m2,e4m3e5m2,e5m2e4m3}_mt256_nt[_gen|_splitk]: the macro-tile pipeline on 8-bit
+// maize_gemm_{e4m3,e5m2,e4m3e5m2,e5m2e4m3}_mt256_{nt,nn}[_gen|_splitk]: the macro-tile pipeline on 8-bit
 // floating-point operands (A and B of the same or of different formats).
 //
 // The 8-bit entries of the reference's MMA catalogue (Sm89MmaF8F32_16x8x32 on E4M3 / E5M2,
@@ -17,6 +17,10 @@
 // -> k assignment, so the order of k inside an instruction does not matter.  Tile t+2 is requested
 // behind the barrier of step t, one 1 KiB piece per two MFMAs.
 //
+// _nn: B stored K x N (row-major), read where it lies.  Its K tile lands as 128 rows of 256 bytes (maps::sk8_*) and a
+// lane assembles the same 32 bytes of K per MFMA from four transposing 8-byte LDS reads (ds_read_b64_tr_b8): no
+// transposed copy, no workspace; rows of B on 16-byte boundaries and N % 16 == 0.
+//
 // 16 x 16 x 128 and not 32 x 32 x 64 (the first version): register-only loops of the two on E4M3 data
 // from uniform[-1,1) measure 39.9 us against 42.9 us for the FLOP of 4096^3 at the board's power limit
 // (both 38 us on zeros).  K % 16 == 0 and N % 8 == 0; rows of A and B start on 16-byte boundaries; any K
@@ -30,7 +34,10 @@ namespace maize {
 #define MAIZE_F8_KERNELS(tag, fa, fb) \
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt(GemmArgs p) { mt256::body<true, true, false, false, false, false, (fa) | ((fb) << 1)>(p); } \
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, (fa) | ((fb) << 1)>(p); } \
-    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, (fa) | ((fb) << 1)>(p); }
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, (fa) | ((fb) << 1)>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn(GemmArgs p) { mt256::body<false, true, false, false, false, false, (fa) | ((fb) << 1)>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, (fa) | ((fb) << 1)>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, (fa) | ((fb) << 1)>(p); }
 MAIZE_F8_KERNELS(e4m3, 0, 0)
 MAIZE_F8_KERNELS(e5m2, 1, 1)
 MAIZE_F8_KERNELS(e4m3e5m2, 0, 1)     // A is E4M3, B is E5M2

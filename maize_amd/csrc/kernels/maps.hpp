@@ -87,5 +87,22 @@ MAIZE_MAP uint32_t sk_tr_offset(uint32_t cg, uint32_t h, uint32_t lane) {
     return sk_offset(sk_tr_row(h, lane), col >> 3) + (col & 7u) * 2u;
 }
 
+// ---- K x N operand tile of 8-bit elements (row-major B of the 8-bit macro-tile kernel): 128 rows of 256 B ----
+// Piece p (4 rows, 1 KiB): lane l lands at row 4p + l/16, position l%16.  16-byte chunks (16 columns) are XOR-ed
+// with f(row) = row%8 + 8 bit4(row): bits 3 and 6 of the row stay out of it, so the four reads of a fragment sit
+// 2048 (8 rows) and 16384 (64 rows) bytes apart and the kernel keeps one address register per column group.
+MAIZE_MAP uint32_t sk8_swizzle(uint32_t row) { return (row & 7u) | (((row >> 4) & 1u) << 3); }
+MAIZE_MAP uint32_t sk8_piece_row(uint32_t piece, uint32_t lane) { return piece * 4u + (lane >> 4); }
+MAIZE_MAP uint32_t sk8_piece_chunk(uint32_t piece, uint32_t lane) { return (lane & 15u) ^ sk8_swizzle(sk8_piece_row(piece, lane)); }
+MAIZE_MAP uint32_t sk8_offset(uint32_t row, uint32_t chunk) { return row * 256u + ((chunk ^ sk8_swizzle(row)) * 16u); }
+// Transposing read (ds_read_b64_tr_b8) for MFMA 16x16x128 (B first): within 16 lanes, lane q addresses the 8 bytes at
+// columns 8 (q%2) .. +7 of row q/2 of an 8 x 16 block and receives column q, rows 0..7.  Lane group g = l/16 holds
+// k = 16 g + 0..15 and 64 + 16 g + 0..15 (the K-contiguous operand's two chunks g and 4 + g): read (kk, h) fetches
+// rows 64 kk + 16 g + 8 h + 0..7 of column group cg (16 columns).
+MAIZE_MAP uint32_t sk8_tr_row(uint32_t kk, uint32_t h, uint32_t lane) { return 64u * kk + (lane >> 4) * 16u + h * 8u + ((lane & 15u) >> 1); }
+MAIZE_MAP uint32_t sk8_tr_offset(uint32_t cg, uint32_t kk, uint32_t h, uint32_t lane) {
+    return sk8_offset(sk8_tr_row(kk, h, lane), cg) + (lane & 1u) * 8u;
+}
+
 }  // namespace maps
 }  // namespace maize

@@ -124,6 +124,22 @@ extern "C" __global__ __launch_bounds__(64) void maize_probe_ds_read_tr16(
     for (int e = 0; e < 4; ++e) out[lane * 4 + e] = (uint16_t)v[e];
 }
 
+// The 8-bit form (ds_read_b64_tr_b8): LDS is filled with lds_init (n_init bytes), lane l reads at byte offset
+// byte_off[l], out receives 8 bytes per lane.
+extern "C" __global__ __launch_bounds__(64) void maize_probe_ds_read_tr8(
+    const uint8_t* lds_init, uint32_t n_init, const uint32_t* byte_off, uint8_t* out) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[8192];
+    const uint32_t lane = threadIdx.x;
+    for (uint32_t i = lane; i < 8192u; i += 64u) lds[i] = i < n_init ? lds_init[i] : (uint8_t)0xFFu;
+    __syncthreads();
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    typedef v2i __attribute__((address_space(3))) * lds_v2_ptr;
+    const uint32_t off = byte_off[lane] & 0x1FF8u;
+    lds_v2_ptr p = (lds_v2_ptr)((__attribute__((address_space(3))) char*)lds + off);
+    const v2i v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(p);
+    for (int e = 0; e < 8; ++e) out[lane * 8 + e] = (uint8_t)((uint32_t)v[e >> 2] >> (8 * (e & 3)));
+}
+
 // fp32 -> bf16 through the conversion the tiled kernels' epilogue uses.
 extern "C" __global__ void maize_probe_cvt_bf16(const float* in, uint16_t* out, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;

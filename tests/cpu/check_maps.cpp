@@ -136,6 +136,47 @@ int main() {
                 }
         std::printf("ok  K x N tile: transposing reads deliver the MFMA operand and are bank-conflict free\n");
     }
+    // ---- K x N tile of 8-bit elements: 128 rows of 256 B, 32 pieces of 4 rows
+    {
+        std::set<uint32_t> seen;
+        for (uint32_t piece = 0; piece < 32; ++piece)
+            for (uint32_t lane = 0; lane < 64; ++lane) {
+                const uint32_t row = sk8_piece_row(piece, lane), chunk = sk8_piece_chunk(piece, lane);
+                CHECK(row < 128 && chunk < 16, "8-bit K x N piece out of range");
+                CHECK(sk8_offset(row, chunk) == piece * 1024 + lane * 16, "8-bit K x N deposit/read mismatch piece %u lane %u", piece, lane);
+                CHECK(seen.insert(row * 16 + chunk).second, "8-bit K x N (row %u, chunk %u) deposited twice", row, chunk);
+            }
+        CHECK(seen.size() == 128 * 16, "8-bit K x N tile not covered");
+        // each group of 16 lanes fetches one whole 256-byte row segment
+        for (uint32_t piece = 0; piece < 32; ++piece)
+            for (uint32_t g = 0; g < 4; ++g) {
+                std::set<uint32_t> chunks;
+                for (uint32_t l = 0; l < 16; ++l) { chunks.insert(sk8_piece_chunk(piece, g * 16 + l)); CHECK(sk8_piece_row(piece, g * 16 + l) == piece * 4 + g, "8-bit K x N row of lane"); }
+                CHECK(chunks.size() == 16, "8-bit K x N lane group does not cover its row");
+            }
+        // the kernel's transposing reads: one address register per column group cg (= sk8_tr_offset(cg, 0, 0, lane)),
+        // the 64-row half kk and the 8-row half h as the immediate 16384 kk + 2048 h.  The hardware transposes an
+        // 8 x 16 block per 16 lanes: lane q supplies row q/2, columns 8 (q%2) .. +7 and receives column q, rows 0..7.
+        // The operand of MFMA 16x16x128 the K-contiguous A tile delivers: lane l holds k = 16 (l/16) + 0..15 and
+        // 64 + 16 (l/16) + 0..15, in that order; B must hold the same k in the same registers.
+        for (uint32_t cg = 0; cg < 16; ++cg)
+            for (uint32_t kk = 0; kk < 2; ++kk)
+                for (uint32_t h = 0; h < 2; ++h) {
+                    uint32_t off[64];
+                    for (uint32_t lane = 0; lane < 64; ++lane) {
+                        off[lane] = sk8_tr_offset(cg, 0, 0, lane) + 16384 * kk + 2048 * h;
+                        const uint32_t q = lane & 15u, g = lane >> 4;
+                        const uint32_t row = 64 * kk + 16 * g + 8 * h + q / 2, col = 16 * cg + 8 * (q % 2);
+                        CHECK(off[lane] == sk8_offset(row, col >> 4) + (col & 15), "8-bit transposing read cg %u kk %u h %u lane %u", cg, kk, h, lane);
+                        // what lane (g, q) ends up with in register pair 2 kk + h: column 16 cg + q, k = 64 kk + 16 g + 8 h + e
+                        // -- and A's chunk (kk ? 4 + g : g), bytes 8 h + e, is k = 64 kk + 16 g + 8 h + e as well
+                        const uint32_t a_chunk = kk ? 4 + g : g;
+                        CHECK(a_chunk * 16 + 8 * h == 64 * kk + 16 * g + 8 * h, "k assignment of A and B differ");
+                    }
+                    CHECK(passes_conflict_free(off, 8), "8-bit transposing read cg %u kk %u h %u has bank conflicts", cg, kk, h);
+                }
+        std::printf("ok  8-bit K x N tile: deposit map is a bijection, transposing reads deliver the MFMA operand and are bank-conflict free\n");
+    }
     // ---- 16-bit epilogue staging, MFMA 16 x 16 accumulators
     {
         for (uint32_t row = 0; row < 32; ++row)

@@ -89,7 +89,12 @@ def test_matrix_instruction_per_kernel(kernels):
             a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
             assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
             body = ins[next(k for k, i in enumerate(ins) if i.startswith("v_mfma")):len(ins) - next(k for k, i in enumerate(reversed(ins)) if i.startswith("v_mfma"))]
-            assert count(body, "ds_read_b128") == 64 and count(body, "buffer_load_dwordx4") == 32 and count(body, "s_barrier") == 2, name
+            if "_mt256_nn" in name:
+                # row-major B: A by 128-bit reads, B by four transposing 8-byte reads per fragment
+                assert count(body, "ds_read_b128") == 32 and count(body, "ds_read_b64_tr_b8") == 64, name
+            else:
+                assert count(body, "ds_read_b128") == 64 and count(body, "ds_read_b64_tr_b8") == 0, name
+            assert count(body, "buffer_load_dwordx4") == 32 and count(body, "s_barrier") == 2, name
             assert count(body, "v_accvgpr") == 0 and count(body, "v_mov_b32") == 0, name     # accumulators and fragments stay in place
         elif "_mt128_" in name:
             # the catalogue's tf32 and f64 entries: full fp32 / fp64 matrix instructions; one K tile of 128 bytes
@@ -114,7 +119,8 @@ def test_data_movement_the_design_rests_on(kernels):
             fp32_staging = "_gen" in name or "_splitk" in name
             assert count(ins, "ds_write_b128") == 0 or fp32_staging, name   # no register round trip for operands
         if "_mt256_nn" in name or name.startswith("maize_gemm_bf16_skinny_nn"):
-            assert count(ins, "ds_read_b64_tr_b16") >= 8, f"{name}: a row-major K x N B is read with transposing reads"
+            tr = "ds_read_b64_tr_b8" if name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")) else "ds_read_b64_tr_b16"
+            assert count(ins, tr) >= 8, f"{name}: a row-major K x N B is read with transposing reads"
         if "_mt256_nt" in name:
             assert count(ins, "ds_read_b64_tr_b16") == 0 and count(ins, "ds_read_b128") >= 16, name
     plain = kernels["maize_gemm_bf16_mt256_nn"]

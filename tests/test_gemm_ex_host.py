@@ -179,11 +179,19 @@ def test_dispatch_of_8bit_operands():
             assert _supports(other, x) == (other in (name, name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32")), other
             assert _supports(other, general) == (other in (name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32")), other
         packed = name + "_packed"
-        nn_plan = mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))                                              # row-major B: transposed copy, nothing else
-        assert nn_plan["kernel"] == name + "_trb" and nn_plan["workspace_bytes"] == 65536 + 4096 * 4096 and nn_plan["reduce_grid"] == 0
-        assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it, beta=1.0))["kernel"] == name + "_trb_gen"
-        few = mz.gemm_plan(ex(64, 4096, 4096, in_type=it))                                                    # few tiles: split K on the copies
-        assert few["kernel"] == packed and few["ksplit"] >= 2 and few["workspace_bytes"] >= 65536 + 16 * few["ksplit"] * 262144 + 4096 * 4096
+        direct = name.replace("_mt256_nt", "_mt256_nn")
+        nn_plan = mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))                                              # row-major B read where it lies
+        assert nn_plan["kernel"] == direct and nn_plan["workspace_bytes"] == 0 and nn_plan["reduce_grid"] == 0
+        assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it, beta=1.0))["kernel"] == direct + "_gen"
+        few = mz.gemm_plan(ex(64, 4096, 4096, in_type=it))                                                    # few tiles: split K
+        assert few["kernel"] == direct + "_splitk" and few["ksplit"] >= 2 and few["workspace_bytes"] == 65536 + 16 * few["ksplit"] * 262144
+        for other in mz.kernel_names():
+            assert _supports(other, ex(4096, 4096, 4096, in_type=it)) == (
+                other in (direct, direct + "_gen", direct + "_splitk", name + "_trb", name + "_trb_gen", packed, "maize_gemm_bf16_wave32")), other
+        tr_plan = mz.gemm_plan(ex(4096, 4104, 4096, in_type=it))                                              # N % 16 != 0: transposed copy of B, nothing else
+        assert tr_plan["kernel"] == name + "_trb" and tr_plan["workspace_bytes"] == 65536 + 4104 * 4096 and tr_plan["reduce_grid"] == 0
+        assert mz.gemm_plan(ex(4096, 4104, 4096, in_type=it, beta=1.0))["kernel"] == name + "_trb_gen"
+        assert mz.gemm_plan(ex(64, 4104, 4096, in_type=it))["kernel"] == packed                              # ... and few tiles: split K on the copies
         assert mz.gemm_plan(ex(4096, 4096, 4104, in_type=it))["kernel"] == packed                             # row-major B and K % 16
         assert mz.gemm_plan(ex(4096, 4096, 4104, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == packed        # K % 16: padded copies
         assert mz.gemm_plan(ex(**big, in_type=it, ldb=4104))["kernel"] == packed                              # rows off 16 bytes

@@ -122,6 +122,27 @@ def test_every_encoding_reaches_the_matrix_unit_unchanged(ctx, oracle, fmt):
         assert np.array_equal(oracle.bf16_bits_to_f64(got), oracle.bf16_bits_to_f64(want.ravel())), kernel
 
 
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+def test_row_major_b_routes_every_element(ctx, oracle, fmt):
+    """C = A . P with P a K x N selection matrix stored row-major (column j holds a single 1, at row pick[j]): C[:, j]
+    is A[:, pick[j]] exactly, for every encoding -- any slip in the transposing reads' lane or k assignment moves an element."""
+    elem = FMT[fmt][1]
+    vals = oracle.fp8_bits_to_f64(np.arange(256, dtype=np.uint8), elem)
+    finite = np.arange(256, dtype=np.uint8)[np.isfinite(vals)]
+    m, n, k = 256, 512, 400
+    a = np.resize(finite, m * k).reshape(m, k)
+    rng = np.random.default_rng(5)
+    pick = np.concatenate([rng.permutation(k), rng.permutation(k)[:n - k]])
+    one = oracle.fp8_bits_from_f64(np.array([1.0]), elem)[0]
+    p = np.zeros((k, n), dtype=np.uint8)
+    p[pick, np.arange(n)] = one
+    want = oracle.bf16_bits_from_f64(oracle.fp8_bits_to_f64(a[:, pick], elem))
+    for kernel in (f"maize_gemm_{fmt}_mt256_nn", f"maize_gemm_{fmt}_mt256_nn_gen", f"maize_gemm_{fmt}_mt256_nn_splitk"):
+        got, took = launch(ctx, a.ravel(), p.ravel(), np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NN, fmt, k, n, n, kernel=kernel)
+        assert took == kernel
+        assert np.array_equal(oracle.bf16_bits_to_f64(got), oracle.bf16_bits_to_f64(want.ravel())), kernel
+
+
 def test_what_the_8bit_matrix_instruction_keeps(ctx, oracle):
     """One product of 1 * 1 and one of 2^-s in the same 64-deep group (E5M2, fp32 C): the small product is added
     exactly while it is at most 13 binades below the large one and dropped entirely from 14 on.  The tolerance
@@ -168,6 +189,82 @@ def test_macro_tile_kernel_all_knobs(ctx, oracle, fmt):
         assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 knobs", **kw) == name + "_gen"
 
 
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"])
+def test_macro_tile_kernel_on_a_row_major_b(ctx, oracle, fmt):
+    """B stored K x N, one byte per element, read where it lies: its tiles land as 128 rows of 256 bytes and the
+    operand of the 128-deep instruction is assembled by transposing LDS reads.  Whole and ragged tiles, K tails
+    (rows of B past K read as zeros, whatever lies behind the view), views, every epilogue, split-K, and the
+    bits of the same product with B stored N x K (the same instruction sums the same 128-element groups)."""
+    name = f"maize_gemm_{fmt}_mt256_nn"
+    shapes = [(256, 256, 128), (256, 256, 256), (512, 768, 384), (300, 528, 144), (1000, 272, 1040), (128, 2048, 16), (520, 784, 400)]
+    for (m, n, k) in shapes if fmt in ("e4m3", "e5m2") else shapes[2:4]:
+        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn") == name
+    m, n, k = 520, 784, 400
+    assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn views", lda=416, ldb=800, ldc=792) == name
+    assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn gen by name", kernel=name + "_gen") == name + "_gen"
+    for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(alpha=2.0, lda=416, ldb=800, ldc=792)):
+        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn knobs", **kw) == name + "_gen"
+    for (m, n, k) in ((24, 528, 4096), (256, 256, 16384)):
+        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="f8 nn split-K") == name + "_splitk"
+    assert run_f8(ctx, oracle, 40, 272, 2064, layout=mz.LAYOUT_NN, fmt=fmt, kernel=name + "_splitk", label="f8 nn split-K ragged K") == name + "_splitk"
+    # the same product from the two layouts of B: same bits
+    elem = ab_of(FMT[fmt][1])
+    m, n, k = 384, 512, 1168
+    a = f8_uniform(oracle, m * k, 41, elem[0])
+    b_kn = f8_uniform(oracle, k * n, 42, elem[1])
+    b_nk = np.ascontiguousarray(b_kn.reshape(k, n).T).ravel()
+    c_nn, took = launch(ctx, a, b_kn, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NN, fmt, k, n, n)
+    assert took == name
+    c_nt, took = launch(ctx, a, b_nk, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n)
+    assert took == f"maize_gemm_{fmt}_mt256_nt"
+    assert np.array_equal(c_nn, c_nt)
+    # batched, padded strides; equal to its singles and nothing written between the members
+    bm, bn, bk, batch = 384, 512, 640, 3
+    sa, sb, sc = bm * bk + 64, bk * bn + 128, bm * bn + 16
+    ab_ = f8_uniform(oracle, batch * sa, 21, elem[0])
+    bb_ = f8_uniform(oracle, batch * sb, 22, elem[1])
+    dense, took = launch(ctx, ab_, bb_, np.zeros(batch * sc, np.uint16), bm, bn, bk, mz.LAYOUT_NN, fmt, bk, bn, bn, batch=batch, strides=(sa, sb, sc))
+    assert took == name
+    for i in range(batch):
+        single, _ = launch(ctx, ab_[i * sa:i * sa + bm * bk], bb_[i * sb:i * sb + bk * bn], np.zeros(bm * bn, np.uint16), bm, bn, bk,
+                           mz.LAYOUT_NN, fmt, bk, bn, bn)
+        assert np.array_equal(single, dense[i * sc:i * sc + bm * bn]), i
+        assert not dense[i * sc + bm * bn:(i + 1) * sc].any(), "wrote between batch members"
+
+
+def test_row_major_b_full_size_and_what_lies_behind_the_view(ctx, oracle):
+    """4096^3 E4M3 with B stored K x N on sampled rows; and a ragged K whose last K tile reaches past B's last row:
+    the bytes behind the view are NaN encodings and must not reach C."""
+    fmt, elem = "e4m3", 2
+    m = n = k = 4096
+    a = f8_uniform(oracle, m * k, 11, elem)
+    b = f8_uniform(oracle, k * n, 12, elem)
+    got, took = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NN, fmt, k, n, n)
+    assert took == "maize_gemm_e4m3_mt256_nn"
+    rows = np.unique(np.concatenate([np.arange(0, m, 256), np.arange(255, m, 256), np.array([1, 127, 128, 2049, 4094])])).astype(np.uint32)
+    ref, val, ab = oracle.ref_gemm_rows(a, b, m, n, k, rows, layout=oracle.NN, elem=elem)
+    s = oracle.compare(got.reshape(m, n)[rows], ref, val, ab, k, coeff=oracle.floor_coeff_f8(k))
+    _say(f"e4m3 4096^3 row-major B, sampled rows: {s}")
+    assert s["n_fail"] == 0, s
+    # B is the leading part of a larger allocation filled with NaN (0x7F): K = 400 leaves 112 rows of the last K tile behind the view
+    m, n, k = 300, 528, 400
+    a = f8_uniform(oracle, m * k, 51, elem)
+    b = f8_uniform(oracle, k * n, 52, elem)
+    pad = np.full(256 * n, 0x7F, np.uint8)
+    da, db, dc = ctx.upload(a), ctx.upload(np.concatenate([b, pad])), ctx.upload(np.zeros(m * n, np.uint16))
+    try:
+        x = mz.gemm_ex_desc(mz.Matrix(da, m, k, elem_bytes=1), mz.Matrix(db, k, n, elem_bytes=1), mz.Matrix(dc, m, n), layout=mz.LAYOUT_NN, in_type=mz.IN_E4M3)
+        assert mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"] == "maize_gemm_e4m3_mt256_nn"
+        ctx.gemm_bf16(x)
+        ctx.sync()
+        got = dc.download(np.uint16)
+    finally:
+        da.free(); db.free(); dc.free()
+    ref, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, layout=mz.LAYOUT_NN, lda=k, ldb=n, elem=elem)
+    s = oracle.compare(got.reshape(m, n), ref, val, scale, k, coeff=oracle.floor_coeff_f8(k))
+    assert s["n_fail"] == 0, s
+
+
 def test_dispatch_of_8bit_products(ctx):
     def pick(m, n, k, layout, in_type, **kw):
         brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
@@ -176,7 +273,8 @@ def test_dispatch_of_8bit_products(ctx):
         return mz.gemm_plan(x, compute_units=256)["kernel"]
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt"
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nt"
-    assert pick(4096, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_trb"      # row-major B: transposed copy
+    assert pick(4096, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn"          # row-major B: read where it lies
+    assert pick(4096, 4104, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_trb"      # ... N % 16: transposed copy
     assert pick(4096, 4096, 4104, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_packed"   # K % 16: padded copies
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3, lda=4104) == "maize_gemm_e4m3_mt256_nt_packed"
     assert pick(64, 64, 64, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_bf16_wave32"
@@ -276,18 +374,20 @@ def test_packed_path_for_8bit_operands(ctx, oracle, fmt):
     NN, NT = mz.LAYOUT_NN, mz.LAYOUT_NT
     assert run_f8(ctx, oracle, 512, 768, 384, layout=NN, fmt=fmt, kernel=name, label="packed NN") == name
     assert run_f8(ctx, oracle, 300, 520, 1000, layout=NN, fmt=fmt, label="packed NN ragged") == name
-    # only B needs a copy (its transpose): the macro-tile kernel writes C itself
+    # N % 16 != 0 (the kernels that read a row-major B where it lies take whole 16-byte chunks of its rows): only B
+    # needs a copy (its transpose), the macro-tile kernel writes C itself
     trb = f"maize_gemm_{fmt}_mt256_nt_trb"
-    assert run_f8(ctx, oracle, 1024, 2048, 512, layout=NN, fmt=fmt, label="trb") == trb
+    assert run_f8(ctx, oracle, 1024, 2056, 512, layout=NN, fmt=fmt, label="trb") == trb
+    assert run_f8(ctx, oracle, 1024, 2048, 512, layout=NN, fmt=fmt, kernel=trb, label="trb by name") == trb
     assert run_f8(ctx, oracle, 1000, 2056, 528, layout=NN, fmt=fmt, lda=544, ldb=2064, ldc=2072, label="trb views") == trb
-    assert run_f8(ctx, oracle, 1024, 2048, 512, layout=NN, fmt=fmt, alpha=-1.25, beta=0.75, label="trb gen") == trb + "_gen"
-    assert run_f8(ctx, oracle, 1024, 2048, 512, layout=NN, fmt=fmt, out_f32=True, label="trb f32") == trb + "_gen"
+    assert run_f8(ctx, oracle, 1024, 2056, 512, layout=NN, fmt=fmt, alpha=-1.25, beta=0.75, label="trb gen") == trb + "_gen"
+    assert run_f8(ctx, oracle, 1024, 2056, 512, layout=NN, fmt=fmt, out_f32=True, label="trb f32") == trb + "_gen"
     assert run_f8(ctx, oracle, 257, 263, 1031, layout=NN, fmt=fmt, label="packed NN odd N, K") == name
     assert run_f8(ctx, oracle, 257, 263, 1031, layout=NT, fmt=fmt, label="packed NT odd N, K") == name
     assert run_f8(ctx, oracle, 512, 768, 384, layout=NT, fmt=fmt, lda=391, ldb=397, ldc=771, label="packed NT odd ld") == name
     assert run_f8(ctx, oracle, 512, 768, 392, layout=NN, fmt=fmt, alpha=-1.25, beta=0.75, label="packed NN scaled") == name
     assert run_f8(ctx, oracle, 512, 768, 392, layout=NN, fmt=fmt, out_f32=True, ldc=776, label="packed NN f32") == name
-    assert run_f8(ctx, oracle, 64, 4096, 4096, layout=NN, fmt=fmt, label="packed NN few rows") == name
+    assert run_f8(ctx, oracle, 64, 4104, 4096, layout=NN, fmt=fmt, label="packed NN few rows") == name
     # batched, row-major B, padded strides: every member equals its single launch
     elem = FMT[fmt][1]
     m, n, k, batch = 256, 384, 512, 3

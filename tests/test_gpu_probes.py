@@ -106,6 +106,29 @@ def test_ds_read_tr16_b64_semantics(ctx):
         x.free()
 
 
+def test_ds_read_tr8_b64_semantics(ctx):
+    """The 8-bit form: within each group of 16 lanes, lane j supplies the address of 8 consecutive bytes of row j/2
+    (columns 8*(j%2)..+7 of an 8 x 16 block); lane i receives column i of that block, rows 0..7."""
+    _say("probe: ds_read_b64_tr_b8")
+    stride = 256                                            # bytes per LDS row in this probe
+    lanes = np.arange(64)
+    g, j = lanes // 16, lanes % 16
+    off = ((j // 2) * stride + 16 * g + 8 * (j % 2)).astype(np.uint32)
+    idx = np.arange(8192)
+    row, col = idx // stride, idx % stride
+    # a byte cannot number the 512 positions of the 8 x 64 window: one pattern tells (row, column within the block), the other the block
+    for init in ((row % 8 * 16 + col % 16).astype(np.uint8), (col // 16 + 16 * (row // 8)).astype(np.uint8)):
+        di, do, dout = ctx.upload(init), ctx.upload(off), ctx.malloc(64 * 8)
+        _launch(ctx, "maize_probe_ds_read_tr8", 64, (1, 1, 1), TrArgs(di.ptr, 8192, do.ptr, dout.ptr))
+        out = dout.download(np.uint8).reshape(64, 8)
+        want = init[np.arange(8)[None, :] * stride + 16 * g[:, None] + j[:, None]]
+        if not np.array_equal(out, want):
+            _say("ds_read_tr8 raw output (lane: 8 values):\n" + "\n".join(f"{l:2d}: {out[l].tolist()}" for l in range(64)))
+        assert np.array_equal(out, want)
+        for x in (di, do, dout):
+            x.free()
+
+
 class CvtArgs(C.Structure):
     _fields_ = [("inp", C.c_void_p), ("out", C.c_void_p), ("n", C.c_uint32)]
 

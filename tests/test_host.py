@@ -60,7 +60,7 @@ def test_embedded_code_object_is_a_gfx950_elf_with_all_kernels():
     # plain / general kernel behind a transposing copy of B
     # (the "_packed_gen" entries: the general-epilogue kernel on the copies)
     device = [n.replace("_packed_gen", "_gen").replace("_packed", "_splitk").replace("_trb", "") for n in names]
-    for n in device + ["maize_gemm_splitk_reduce", "maize_pack_2d", "maize_pack_2d_u8", "maize_transpose_u8", "maize_probe_mfma_32x32x16", "maize_probe_ds_read_tr16",
+    for n in device + ["maize_gemm_splitk_reduce", "maize_pack_2d", "maize_pack_2d_u8", "maize_transpose_u8", "maize_probe_mfma_32x32x16", "maize_probe_ds_read_tr16", "maize_probe_ds_read_tr8",
                        "maize_copy_u128"]:
         assert n.encode() in co, n
 

@@ -39,16 +39,21 @@ def mt256_issue_slots():
     return [stride * pc + 2 for pc in range(16)]
 
 
+# where the K step issues its fragment reads: slot s of an eighth issues reads s * RPS .. of the group the next eighth needs
+MT256_READ_LINES = ("for (int rb = r * RPS; rb < (r + 1) * RPS; ++rb) {",
+                    "if (h4 == 0 && rb < NBR) read_b(1, kh, cur, rb);",
+                    "if (h4 == 1 && r < NAR) read_a(1, kh, cur, r);",
+                    "if (h4 == 2 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
+                    "if (h4 == 3 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }")
+
+
 def mt256_reads_per_eighth(nt):
     """A K step is 8 eighths of 16 MFMAs; each needs one new group of 4 fragments beyond what the eighth
     before it holds: 4 reads of 128 bits, or 8 transposing reads of 64 bits for a group of a row-major B.
     Within a K half the groups come in the order B1, A1, then A0 and B0 of the next half (the source states it)."""
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
-    assert "constexpr int NBR = (IS8 || !NT) ? 8 : 4;" in src
-    for line in ("if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);",
-                 "if (h4 == 1 && r < NAR) read_a(1, kh, cur, r);",
-                 "if (h4 == 2 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
-                 "if (h4 == 3 && r < NBR) { if (!last_half) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }"):
+    assert "constexpr int NBR = TR8 ? 16 : (IS8 || !NT) ? 8 : 4;" in src and "constexpr int RPS = TR8 ? 2 : 1;" in src
+    for line in MT256_READ_LINES:
         assert line in src, line
     assert "constexpr int EB = IS8 ? 2 : 6;" in src and "if (e == EB) {" in src
     assert "const int slot = e >= EB ? 16 * (e - EB) + s : 32 + 16 * e + s;" in src
@@ -213,7 +218,8 @@ def test_macro_tile_checker_rejects_broken_schedules():
 
 # ---------------------------------------------------------------------------------------
 # 8-bit macro-tile kernel: the same template with a K tile one matrix instruction deep: a K step is four groups of
-# 16 MFMAs, the barrier in front of the third, a group is 8 reads, one request per two MFMA slots
+# 16 MFMAs, the barrier in front of the third, a group is 8 reads, one request per two MFMA slots.  With a row-major
+# B (transposing reads) a B group is 16 reads, two per MFMA slot.
 # ---------------------------------------------------------------------------------------
 
 def f8_constants():
@@ -221,13 +227,18 @@ def f8_constants():
     for fact in ("constexpr int NE = IS8 ? 4 : 8;", "constexpr int EB = IS8 ? 2 : 6;", "constexpr int DS = IS8 ? 2 : DMA_STRIDE;",
                  "constexpr int NAR = IS8 ? 8 : 4;", "const bool last_half = IS8 || kh == 1;",
                  "const int slot = e >= EB ? 16 * (e - EB) + s : 32 + 16 * e + s;",
-                 "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {", "if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);"):
+                 "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {", "if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);",
+                 "constexpr int NBR = TR8 ? 16 : (IS8 || !NT) ? 8 : 4;", "constexpr int RPS = TR8 ? 2 : 1;",
+                 "constexpr bool TR8 = IS8 && !NT;") + MT256_READ_LINES:
         assert fact in src, fact
     return dict(ne=4, eb=2, ds=2, reads=8)
 
 
-def f8_wave_program(nk, barrier_at=None, ds=None):
+def f8_wave_program(nk, barrier_at=None, ds=None, tr=False):
+    """tr: row-major B.  The groups read during group e of a step: B1, A1, then A0 and B0 of the next tile."""
     c = f8_constants()
+    b_reads = 16 if tr else c["reads"]
+    per_group = [b_reads, c["reads"], c["reads"], b_reads]
     eb = c["eb"] if barrier_at is None else barrier_at
     ds = c["ds"] if ds is None else ds
     slots = [ds * pc + 2 for pc in range(16)]
@@ -235,7 +246,7 @@ def f8_wave_program(nk, barrier_at=None, ds=None):
     issued = {0: (1, False), 1: (2, False), 2: (0, True), 3: (0, True)}
     ops = [("dma", 0, pc, 0) for pc in range(16)]
     ops += [("wait_all",), ("barrier",)]
-    ops += [("read", 0, 0, 0)] * (2 * c["reads"])
+    ops += [("read", 0, 0, 0)] * (c["reads"] + b_reads)
     ops += [("dma", 1, pc, 1) for pc in range(16) if slots[pc] < 32]
     k_early, k_late = 2, 1
     steps = nk + (nk & 1)
@@ -247,8 +258,9 @@ def f8_wave_program(nk, barrier_at=None, ds=None):
             need, next_tile = issued[e]
             for sl in range(16):
                 ops.append(("mfma", t, e))
-                if sl < c["reads"]:
-                    ops.append(("read", t + 1, need, nxt) if next_tile else ("read", t, need, cur))
+                if sl < 8:                                  # all of a group's reads in the first half of the group before
+                    for _ in range(per_group[e] // 8):
+                        ops.append(("read", t + 1, need, nxt) if next_tile else ("read", t, need, cur))
                 slot = 16 * (e - c["eb"]) + sl if e >= c["eb"] else 32 + 16 * e + sl
                 for pc in range(16):
                     if slots[pc] == slot:
@@ -260,12 +272,14 @@ def f8_wave_program(nk, barrier_at=None, ds=None):
 
 
 F8_CUMULATIVE = [16, 24, 32, 32]      # reads of a tile that must have been issued before group e multiplies: A0 B0 | B1 | A1 | -
+F8_CUMULATIVE_TR = [24, 40, 48, 48]   # ... with 16 reads per B group
 
 
+@pytest.mark.parametrize("tr", [False, True])
 @pytest.mark.parametrize("nk", [1, 2, 3, 7, 32])
-def test_8bit_macro_tile_schedule_is_hazard_free(nk):
-    ops, steps = f8_wave_program(nk)
-    last_tile = check_two_stage(ops, steps, F8_CUMULATIVE, parts=4)
+def test_8bit_macro_tile_schedule_is_hazard_free(nk, tr):
+    ops, steps = f8_wave_program(nk, tr=tr)
+    last_tile = check_two_stage(ops, steps, F8_CUMULATIVE_TR if tr else F8_CUMULATIVE, parts=4)
     assert steps <= last_tile <= steps + 1
 
 
@@ -276,6 +290,11 @@ def test_8bit_macro_tile_checker_rejects_broken_schedules():
         check_two_stage(*f8_wave_program(8, barrier_at=1), F8_CUMULATIVE, parts=4)
     with pytest.raises(Hazard):                 # requests four slots apart: the last ones would come after the next barrier and never be issued
         check_two_stage(*f8_wave_program(8, ds=5), F8_CUMULATIVE, parts=4)
+    for kw in (dict(barrier_at=3), dict(barrier_at=1)):
+        with pytest.raises(Hazard):             # the same with a row-major B
+            check_two_stage(*f8_wave_program(8, tr=True, **kw), F8_CUMULATIVE_TR, parts=4)
+    with pytest.raises(Hazard):                 # 8 reads per B group where a row-major B needs 16: MFMAs on stale registers
+        check_two_stage(*f8_wave_program(8), F8_CUMULATIVE_TR, parts=4)
 
 
 # ---------------------------------------------------------------------------------------
