@@ -143,6 +143,64 @@ def test_row_major_b_routes_every_element(ctx, oracle, fmt):
         assert np.array_equal(oracle.bf16_bits_to_f64(got), oracle.bf16_bits_to_f64(want.ravel())), kernel
 
 
+SPECIAL_FAMILIES = [
+    # (kernel suffix after maize_gemm_<fmt>_ or a full name, M, N, K, layout): every 8-bit family on a shape with ragged edges
+    ("mt256_nt", 300, 520, 400, mz.LAYOUT_NT),
+    ("mt256_nt_gen", 257, 264, 144, mz.LAYOUT_NT),
+    ("mt256_nt_splitk", 40, 264, 2064, mz.LAYOUT_NT),
+    ("mt256_nn", 300, 528, 400, mz.LAYOUT_NN),
+    ("mt256_nn_gen", 257, 272, 144, mz.LAYOUT_NN),
+    ("mt256_nn_splitk", 40, 272, 2064, mz.LAYOUT_NN),
+    ("mt256_nt_trb", 300, 520, 400, mz.LAYOUT_NN),
+    ("mt256_nt_packed", 257, 263, 1031, mz.LAYOUT_NN),
+    ("skinny_nt", 13, 515, 2064, mz.LAYOUT_NT),
+    ("skinny_nt_m32", 29, 520, 4112, mz.LAYOUT_NT),
+    ("skinny_nt_m64", 50, 264, 4112, mz.LAYOUT_NT),
+    ("maize_gemm_bf16_wave32", 33, 17, 65, mz.LAYOUT_NN),
+    ("maize_gemm_bf16_wave32", 33, 17, 65, mz.LAYOUT_NT),
+]
+
+
+@pytest.mark.parametrize("family", SPECIAL_FAMILIES, ids=lambda f: f"{f[0].replace('maize_gemm_', '')}-{f[1]}x{f[2]}x{f[3]}-{'nt' if f[4] else 'nn'}")
+@pytest.mark.parametrize("fmt", ["e5m2", "e4m3"])
+def test_8bit_nan_inf_and_negative_zero_next_to_the_zero_filled_regions(ctx, oracle, fmt, family):
+    """E5M2 has infinities and NaNs, E4M3 (the OCP "fn" form) NaNs only.  Planted in A and B in the interior, on the last
+    valid row / column / k (next to what the kernels fill with zeros) and beside rows and columns of -0: the device's NaN
+    set and its +Inf / -Inf sets must equal the oracle's element for element (a zero fill meeting a real Inf would show
+    as a NaN the oracle does not have), every other element meets the usual bar."""
+    suffix, m, n, k, layout = family
+    kernel = suffix if suffix.startswith("maize_") else f"maize_gemm_{fmt}_{suffix}"
+    elem = FMT[fmt][1]
+    a = f8_uniform(oracle, m * k, 71, elem).reshape(m, k).copy()
+    b = f8_uniform(oracle, k * n, 72, elem).reshape(k, n).copy()                 # logical K x N
+    nan = 0x7F
+    p_inf, n_inf = (0x7C, 0xFC) if fmt == "e5m2" else (nan, nan | 0x80)          # E4M3: more NaNs instead
+    a[1 % m, 3 % k] = p_inf                                   # interior
+    a[m - 1, k - 1] = n_inf                                   # last row, last k: next to the M and K fill
+    a[min(255, m - 2), min(127, k - 2)] = nan                 # last row of a tile, last k of a K tile
+    a[2 % m, :] = 0x80                                        # a row of -0
+    b[k - 1, n - 1] = p_inf                                   # last k, last column: next to the K and N fill
+    b[5 % k, min(256, n - 2)] = n_inf                         # first column of the second tile
+    b[0, 7 % n] = nan
+    b[:, 3 % n] = 0x80                                        # a column of -0 under A's +Inf: Inf x 0 = NaN where the oracle says so
+    bs = np.ascontiguousarray(b.T) if layout == mz.LAYOUT_NT else b
+    ldb = k if layout == mz.LAYOUT_NT else n
+    _say(f"8-bit special values: {fmt} {kernel} {m}x{n}x{k}")
+    got, took = launch(ctx, a.ravel(), bs.ravel(), np.zeros(m * n, np.uint16), m, n, k, layout, fmt, k, ldb, n, kernel=kernel)
+    assert took == kernel
+    ref, val, scale = oracle.ref_gemm_ex(a.ravel(), bs.ravel(), m, n, k, layout=layout, lda=k, ldb=ldb, elem=elem)
+    g, ref = np.asarray(got, dtype=np.uint16).ravel(), np.asarray(ref, dtype=np.uint16).ravel()
+    gn, rn = (g & 0x7FFF) > 0x7F80, (ref & 0x7FFF) > 0x7F80
+    assert np.array_equal(gn, rn), f"NaN sets differ at {np.flatnonzero(gn != rn)[:8]} ({int(gn.sum())} vs {int(rn.sum())})"
+    for inf in (0x7F80, 0xFF80):
+        assert np.array_equal(g == inf, ref == inf), f"Inf sets differ at {np.flatnonzero((g == inf) != (ref == inf))[:8]}"
+    fin = ~(rn | (ref == 0x7F80) | (ref == 0xFF80))
+    assert rn.sum() > 0 and fin.sum() > 0 and (fmt == "e4m3" or (~fin & ~rn).sum() > 0)          # the case really has all kinds
+    s = oracle.compare(g[fin], ref[fin], np.asarray(val).ravel()[fin], np.asarray(scale).ravel()[fin], k,
+                       coeff=oracle.floor_coeff_f8(k) if "wave32" not in kernel else None)
+    assert s["n_fail"] == 0, s
+
+
 def test_what_the_8bit_matrix_instruction_keeps(ctx, oracle):
     """One product of 1 * 1 and one of 2^-s in the same 64-deep group (E5M2, fp32 C): the small product is added
     exactly while it is at most 13 binades below the large one and dropped entirely from 14 on.  The tolerance
