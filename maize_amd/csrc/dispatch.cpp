@@ -609,7 +609,23 @@ bool skinny_nt_c_by_elements(const maize_gemm_ex_desc_t& d) { return skinny_c_by
 bool skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d); }
 bool skinny_nt_m32_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d, 32u); }
 bool skinny_nt_m64_supports(const maize_gemm_ex_desc_t& d) { return !fp8_in(d) && !wide_in(d) && skinny_nt_common(d, 64u); }
+// 8-bit operands against a row-major (K x N) B: rows of A and B on 16-byte boundaries, K % 16 == 0 (whole chunks of A's
+// rows) and N % 16 == 0 (whole chunks of B's); C as above.
+bool skinny_nn8_common(const maize_gemm_ex_desc_t& d, uint32_t max_rows) {
+    const Dims s = dims_of(d);
+    const Lds l = lds_of(d);
+    if (!fp8_in(d) || !nn(d) || s.m > max_rows || (s.k & 15u) || (s.n & 15u)) return false;
+    if (((uintptr_t)d.gemm.a.ptr | (uintptr_t)d.gemm.b.ptr) & 15u) return false;
+    if ((l.a & 15u) || (l.b & 15u)) return false;
+    if (d.gemm.batch > 1 && ((d.gemm.stride_a & 15u) || (d.gemm.stride_b & 15u))) return false;
+    const uint64_t lim = 1ull << 31;
+    if (l.ext_a >= lim || l.ext_b >= lim || s.k >= (1u << 21) || l.b >= (1u << 21)) return false;
+    return (uint64_t)cdiv(s.n, 256) * d.gemm.batch <= 16384u;   // one ticket counter per (batch member, slab)
+}
 #define MAIZE_F8_SKINNY(tag, type) \
+    bool tag##_skinny_nn_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nn8_common(d, 16u); } \
+    bool tag##_skinny_nn_m32_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nn8_common(d, 32u); } \
+    bool tag##_skinny_nn_m64_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nn8_common(d, 64u); } \
     bool tag##_skinny_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d); } \
     bool tag##_skinny_nt_m32_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d, 32u); } \
     bool tag##_skinny_nt_m64_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && skinny_nt_common(d, 64u); }
@@ -725,6 +741,9 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_" #tag "_skinny_nt", nullptr, tag##_skinny_nt_supports, skinny_nt_plan}, \
     {"maize_gemm_" #tag "_skinny_nt_m32", nullptr, tag##_skinny_nt_m32_supports, skinny_nt_m32_plan}, \
     {"maize_gemm_" #tag "_skinny_nt_m64", nullptr, tag##_skinny_nt_m64_supports, skinny_nt_m64_plan}, \
+    {"maize_gemm_" #tag "_skinny_nn", nullptr, tag##_skinny_nn_supports, skinny_nt_plan}, \
+    {"maize_gemm_" #tag "_skinny_nn_m32", nullptr, tag##_skinny_nn_m32_supports, skinny_nt_m32_plan}, \
+    {"maize_gemm_" #tag "_skinny_nn_m64", nullptr, tag##_skinny_nn_m64_supports, skinny_nt_m64_plan}, \
     {"maize_gemm_" #tag "_mt256_nt", nullptr, tag##_nt_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_gen", nullptr, tag##_nt_gen_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan}, \
@@ -780,6 +799,15 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
             std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nt_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.m <= 32u ? "m32" : "m64");
             const int fm = kernel_index(name);
             if (fm >= 0 && kKernels[fm].supports(d) && plan_fits(kKernels[fm], d, compute_units)) return (uint32_t)fm;
+        }
+        // The same against a row-major B (read where it lies through transposing LDS reads).
+        std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nn", kTag[d.in_type - MAIZE_IN_E4M3]);
+        const int gk = kernel_index(name);
+        if (gk >= 0 && kKernels[gk].supports(d) && s.n >= 64 && s.k >= 1024) return (uint32_t)gk;
+        if (s.m > 16u && s.m <= 64u && s.k >= 2048u && s.n >= (s.m <= 32u ? 1024u : 10240u)) {
+            std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nn_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.m <= 32u ? "m32" : "m64");
+            const int gm = kernel_index(name);
+            if (gm >= 0 && kKernels[gm].supports(d) && plan_fits(kKernels[gm], d, compute_units)) return (uint32_t)gm;
         }
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_splitk", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fs = kernel_index(name);

@@ -192,9 +192,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 // groups of 2 KiB, each fetched by two direct-to-LDS loads (piece = 8 rows of 128 bytes, laid out like B's:
 // maps::kc_*); load i (0 .. 2 MR - 1) of the block in slot x is the duty of wave (x + i) % 8.  The price is one
 // workgroup barrier per block and waves that walk K in step.
-template <bool F8, int FA, int FB, int MR>
+//
+// TRB: 8-bit operands with B stored K x N (row-major), read where it lies.  A block of B is then 128 rows (k) of 256
+// bytes (the slab's 256 columns), laid out like the 8-bit macro-tile kernel's row-major tile (maps::sk8_*: pieces of 4
+// rows, 16-byte chunks XOR-ed with row%8 + 8 bit4(row)); a wave assembles the operand of its two column groups from
+// four transposing reads each (ds_read_b64_tr_b8: k = 16 g + 8 h + 64 kk + 0..7 of column l%16), and A's lanes take the
+// matching chunks g and 4 + g of their rows.  One to four row groups, A through LDS in every case.
+template <bool F8, int FA, int FB, int MR, bool TRB = false>
 __device__ __forceinline__ void body_rows(const GemmArgs& p) {
-    static_assert(MR == 2 || MR == 4, "row groups");
+    static_assert(MR == 2 || MR == 4 || (TRB && MR == 1), "row groups");
+    static_assert(!TRB || F8, "the row-major B of this kernel is 8-bit");
     constexpr int ABYTES = MR * 2048;                  // A block of one ring slot
     __shared__ __attribute__((aligned(1024))) char ring0[BLOCK_BYTES];
     __shared__ __attribute__((aligned(1024))) char ring1[BLOCK_BYTES];
@@ -221,7 +228,7 @@ __device__ __forceinline__ void body_rows(const GemmArgs& p) {
     const char* Bg = (const char*)p.b + bz * p.stride_b * ESZ;
     uint16_t* Cg = p.c + bz * p.stride_c * ((p.epi & EPI_F32) ? 2u : 1u);
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ag, ((M - 1u) * lda + K) * ESZ);
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bg, ((N - 1u) * ldb + K) * ESZ);
+    const __amdgpu_buffer_rsrc_t rb = TRB ? make_rsrc(Bg, (K - 1u) * ldb + N) : make_rsrc(Bg, ((N - 1u) * ldb + K) * ESZ);
     const __amdgpu_buffer_rsrc_t rnull = make_rsrc(Bg, 0u);
 
     lds_ptr const s0 = (lds_ptr)ring0, s1 = (lds_ptr)ring1, s2 = (lds_ptr)ring2, s3 = (lds_ptr)ring3;
@@ -230,27 +237,39 @@ __device__ __forceinline__ void body_rows(const GemmArgs& p) {
     // Copy maps.  B: wave w issues pieces 4w .. 4w+3 of a block (its own 32 rows).  A: piece i of the block holds rows
     // 8 i .. 8 i + 7 of A; the lane's place inside a piece is the same for every piece (maps::kc_piece_* of piece 0
     // and 1 give the two row parities of the swizzle).  Rows at or past N or M fall behind the views and read as zeros.
-    uint32_t b_vo[4], b_k[2], a_vo[2];
+    // Row-major B: piece i of wave w holds rows (k) 16 w + 4 i .. + 3 of the block, 256 bytes each; columns at or past
+    // N (whole chunks: N % 16 == 0) get an out-of-range offset, rows at or past K too (b_k = the lane's row).
+    uint32_t b_vo[4], b_k[4], a_k[2], a_vo[2];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const uint32_t row = maps::kc_piece_row(wave * 4u + i, lane);
-        const uint32_t c = maps::kc_piece_chunk(wave * 4u + i, lane);
-        b_vo[i] = (n0 + row) * ldb * ESZ + c * 16u;
-        if (i < 2) b_k[i] = c * (16u / ESZ);
+        if (TRB) {
+            const uint32_t row = maps::sk8_piece_row(wave * 4u + i, lane);
+            const uint32_t c = maps::sk8_piece_chunk(wave * 4u + i, lane);
+            b_vo[i] = (row * ldb + n0 + c * 16u) | (n0 + c * 16u < N ? 0u : OOB);
+            b_k[i] = row;
+        } else {
+            const uint32_t row = maps::kc_piece_row(wave * 4u + i, lane);
+            const uint32_t c = maps::kc_piece_chunk(wave * 4u + i, lane);
+            b_vo[i] = (n0 + row) * ldb * ESZ + c * 16u;
+            b_k[i] = c * (16u / ESZ);                   // (the same for pieces of one parity)
+        }
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)        // even and odd pieces: rows 0 .. 7 and 8 .. 15 of a 16-row group
+    for (int i = 0; i < 2; ++i) {      // even and odd pieces: rows 0 .. 7 and 8 .. 15 of a 16-row group
         a_vo[i] = maps::kc_piece_row((uint32_t)i, lane) * lda * ESZ + maps::kc_piece_chunk((uint32_t)i, lane) * 16u;
+        a_k[i] = maps::kc_piece_chunk((uint32_t)i, lane) * (16u / ESZ);
+    }
     // Operand maps, as in the one-group kernel: lane l = row l % 16 of a 16-row group, chunks chunk[0], chunk[1].
     const uint32_t g = lane >> 4, r16 = lane & 15u;
     uint32_t chunk[2];
-    chunk[0] = F8 ? 2u * g : g;
-    chunk[1] = F8 ? 2u * g + 1u : 4u + g;
+    chunk[0] = (F8 && !TRB) ? 2u * g : g;
+    chunk[1] = (F8 && !TRB) ? 2u * g + 1u : 4u + g;
     uint32_t rd[2][2], ard[2];                           // B: [which of the wave's two row groups][chunk]; A: [chunk]
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
 #pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2) rd[c2][c] = maps::kc_offset((wave * 2u + c2) * 16u + r16, chunk[c]);
+        for (int c2 = 0; c2 < 2; ++c2)                   // (row-major B: one address per column group, the four reads by offset)
+            rd[c2][c] = TRB ? maps::sk8_tr_offset(wave * 2u + c2, 0, 0, lane) : maps::kc_offset((wave * 2u + c2) * 16u + r16, chunk[c]);
         ard[c] = maps::kc_offset(r16, chunk[c]);         // + 2048 per row group
     }
 
@@ -284,30 +303,51 @@ __device__ __forceinline__ void body_rows(const GemmArgs& p) {
         for (int i = 0; i < 2 * MR; ++i)
             if (wave == (uint32_t)((ai + i) & 7))
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lvp)(ablk[ai] + i * 1024), 16,
-                                                         (a_vo[i & 1] + (uint32_t)(i >> 1) * 16u * lda * ESZ + kb * ESZ) | ((b_k[i & 1] + kb) < K ? 0u : OOB), 0, 0, 0);
+                                                         (a_vo[i & 1] + (uint32_t)(i >> 1) * 16u * lda * ESZ + kb * ESZ) | ((a_k[i & 1] + kb) < K ? 0u : OOB), 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lvp)(slot + (wave * 4u + i) * 1024u), 16,
-                                                     (b_vo[i] + kb * ESZ) | ((b_k[i & 1] + kb) < K ? 0u : OOB), 0, 0, 0);
+                                                     (b_vo[i] + (TRB ? kb * ldb : kb * ESZ)) | ((b_k[i] + kb) < K ? 0u : OOB), 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
     auto consume = [&](lds_ptr slot, int ai) {
         // Inline assembly, so that the compiler sees no read of the ring and places no counter wait of its own.
         u32x4 af[MR][2], bf[2][2];
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        u32x2 bt[2][4];                                  // row-major B: [column group][2 kk + h]
 #pragma unroll
         for (int r = 0; r < MR; ++r)
 #pragma unroll
             for (int c = 0; c < 2; ++c)
                 asm volatile("ds_read_b128 %0, %1" : "=v"(af[r][c]) : "v"((uint32_t)(uintptr_t)ablk[ai] + (uint32_t)r * 2048u + ard[c]));
 #pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2)
+        for (int c2 = 0; c2 < 2; ++c2) {
+            if constexpr (TRB) {
+                const uint32_t at = (uint32_t)(uintptr_t)slot + rd[c2][0];
+                asm volatile("ds_read_b64_tr_b8 %0, %1" : "=v"(bt[c2][0]) : "v"(at));
+                asm volatile("ds_read_b64_tr_b8 %0, %1 offset:2048" : "=v"(bt[c2][1]) : "v"(at));
+                asm volatile("ds_read_b64_tr_b8 %0, %1 offset:16384" : "=v"(bt[c2][2]) : "v"(at));
+                asm volatile("ds_read_b64_tr_b8 %0, %1 offset:18432" : "=v"(bt[c2][3]) : "v"(at));
+            } else {
 #pragma unroll
-            for (int c = 0; c < 2; ++c)
-                asm volatile("ds_read_b128 %0, %1" : "=v"(bf[c2][c]) : "v"((uint32_t)(uintptr_t)slot + rd[c2][c]));
+                for (int c = 0; c < 2; ++c)
+                    asm volatile("ds_read_b128 %0, %1" : "=v"(bf[c2][c]) : "v"((uint32_t)(uintptr_t)slot + rd[c2][c]));
+            }
+        }
         // The wait names every register the reads fill: without that the compiler is free to move what it derives from
         // them (the copies that assemble an 8-bit operand) in front of the wait.
-        if constexpr (MR == 2)
+        if constexpr (TRB) {
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(bt[0][0]), "+v"(bt[0][1]), "+v"(bt[0][2]), "+v"(bt[0][3]),
+                         "+v"(bt[1][0]), "+v"(bt[1][1]), "+v"(bt[1][2]), "+v"(bt[1][3]) :: "memory");
+            if constexpr (MR == 1)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0][0]), "+v"(af[0][1]) :: "memory");
+            else if constexpr (MR == 2)                  // (an operand may be named once only)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0][0]), "+v"(af[0][1]), "+v"(af[1][0]), "+v"(af[1][1]) :: "memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0][0]), "+v"(af[0][1]), "+v"(af[1][0]), "+v"(af[1][1]),
+                             "+v"(af[MR - 2][0]), "+v"(af[MR - 2][1]), "+v"(af[MR - 1][0]), "+v"(af[MR - 1][1]) :: "memory");
+        } else if constexpr (MR == 2)
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0][0]), "+v"(af[0][1]), "+v"(af[1][0]), "+v"(af[1][1]),
                          "+v"(bf[0][0]), "+v"(bf[0][1]), "+v"(bf[1][0]), "+v"(bf[1][1]) :: "memory");
         else
@@ -318,9 +358,11 @@ __device__ __forceinline__ void body_rows(const GemmArgs& p) {
         for (int c2 = 0; c2 < 2; ++c2)
 #pragma unroll
             for (int r = 0; r < MR; ++r) {
-                const u32x4 b_lo = bf[c2][0], b_hi = bf[c2][1];
+                const u32x4 b_lo = TRB ? u32x4{0u, 0u, 0u, 0u} : bf[c2][0], b_hi = TRB ? u32x4{0u, 0u, 0u, 0u} : bf[c2][1];
                 if (F8) {
-                    const i32x8 bb = {(int)b_lo[0], (int)b_lo[1], (int)b_lo[2], (int)b_lo[3], (int)b_hi[0], (int)b_hi[1], (int)b_hi[2], (int)b_hi[3]};
+                    const i32x8 bb = TRB ? i32x8{(int)bt[c2][0][0], (int)bt[c2][0][1], (int)bt[c2][1][0], (int)bt[c2][1][1],
+                                                 (int)bt[c2][2][0], (int)bt[c2][2][1], (int)bt[c2][3][0], (int)bt[c2][3][1]}
+                                         : i32x8{(int)b_lo[0], (int)b_lo[1], (int)b_lo[2], (int)b_lo[3], (int)b_hi[0], (int)b_hi[1], (int)b_hi[2], (int)b_hi[3]};
                     const i32x8 aa = {(int)af[r][0][0], (int)af[r][0][1], (int)af[r][0][2], (int)af[r][0][3],
                                       (int)af[r][1][0], (int)af[r][1][1], (int)af[r][1][2], (int)af[r][1][3]};
                     acc[r][c2] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bb, aa, acc[r][c2], FB, FA, 0, 0, 0, 0);   // B is fed first
@@ -383,5 +425,15 @@ MAIZE_SKINNY_NT_ROWS(e5m2, true, 1, 1)
 MAIZE_SKINNY_NT_ROWS(e4m3e5m2, true, 0, 1)
 MAIZE_SKINNY_NT_ROWS(e5m2e4m3, true, 1, 0)
 #undef MAIZE_SKINNY_NT_ROWS
+// 8-bit operands against a row-major (K x N) B: 1, 2 or 4 row groups.
+#define MAIZE_SKINNY_NN8(tag, fa, fb) \
+    extern "C" __global__ __launch_bounds__(512) void maize_gemm_##tag##_skinny_nn(GemmArgs p) { skinny_nt::body_rows<true, fa, fb, 1, true>(p); } \
+    extern "C" __global__ __launch_bounds__(512) void maize_gemm_##tag##_skinny_nn_m32(GemmArgs p) { skinny_nt::body_rows<true, fa, fb, 2, true>(p); } \
+    extern "C" __global__ __launch_bounds__(512) void maize_gemm_##tag##_skinny_nn_m64(GemmArgs p) { skinny_nt::body_rows<true, fa, fb, 4, true>(p); }
+MAIZE_SKINNY_NN8(e4m3, 0, 0)
+MAIZE_SKINNY_NN8(e5m2, 1, 1)
+MAIZE_SKINNY_NN8(e4m3e5m2, 0, 1)
+MAIZE_SKINNY_NN8(e5m2e4m3, 1, 0)
+#undef MAIZE_SKINNY_NN8
 
 }  // namespace maize

@@ -68,6 +68,18 @@ def test_matrix_instruction_per_kernel(kernels):
             assert count(ins, "ds_read_b128") >= 16 + 8 * groups and count(ins, "ds_read_b64_tr_b16") == 0, name
             assert len([i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]) >= 16 + 2 * groups, name
             assert count(ins, "s_barrier") >= 4, name                     # one per block: the A blocks are shared
+        elif "_skinny_nn" in name and not name.startswith("maize_gemm_bf16"):
+            # 8-bit operands, few rows against a row-major (K x N) B: 1, 2 or 4 row groups, A through LDS by 128-bit reads,
+            # B's operand by four transposing 8-byte reads per column group; 4 turns x 2 column groups x row groups
+            groups = 2 if name.endswith("_m32") else 4 if name.endswith("_m64") else 1
+            f8 = [i for i in ins if i.startswith("v_mfma_f32_16x16x128_f8f6f4")]
+            tag = name[len("maize_gemm_"):].split("_")[0]
+            a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
+            assert len(f8) == 8 * groups and count(ins, "v_mfma") == 8 * groups, name
+            assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
+            assert count(ins, "ds_read_b64_tr_b8") == 32 and count(ins, "ds_read_b128") >= 8 * groups and count(ins, "ds_read_b64_tr_b16") == 0, name
+            assert len([i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]) >= 16 + 2 * groups, name
+            assert count(ins, "s_barrier") >= 4, name                     # one per block: the A blocks are shared
         elif name.endswith("_skinny_nt"):
             # M <= 16 against N x K weights: 16-row instructions, 32 deep for 16-bit operands (bf16 and half in one
             # kernel), 128 deep for 8-bit ones (format codes as below)

@@ -77,7 +77,7 @@ def run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NT, fmt="e4m3", lda=None, ldb=
                                          c_old=None if beta == 0.0 else ov[:, :n].copy(), out_f32=out_f32, elem=elem,
                                          c_elem=oracle.F16 if out_f16 else None)
     g = gv[:, :n]
-    f8_unit = "mt256" in took
+    f8_unit = "wave32" not in took               # every other kernel multiplies with the 8-bit matrix instruction
     if out_f32:
         err = np.abs(g.astype(np.float64) - val)
         tol = ((oracle.floor_coeff_f8(k) + 2.0 ** -23) if f8_unit else (k / 16.0 + 4.0) * 2.0 ** -24) * scale + 1e-45
@@ -153,6 +153,9 @@ SPECIAL_FAMILIES = [
     ("mt256_nn_splitk", 40, 272, 2064, mz.LAYOUT_NN),
     ("mt256_nt_trb", 300, 520, 400, mz.LAYOUT_NN),
     ("mt256_nt_packed", 257, 263, 1031, mz.LAYOUT_NN),
+    ("skinny_nn", 13, 528, 2064, mz.LAYOUT_NN),
+    ("skinny_nn_m32", 29, 528, 4112, mz.LAYOUT_NN),
+    ("skinny_nn_m64", 50, 272, 4112, mz.LAYOUT_NN),
     ("skinny_nt", 13, 515, 2064, mz.LAYOUT_NT),
     ("skinny_nt_m32", 29, 520, 4112, mz.LAYOUT_NT),
     ("skinny_nt_m64", 50, 264, 4112, mz.LAYOUT_NT),
@@ -286,6 +289,54 @@ def test_macro_tile_kernel_on_a_row_major_b(ctx, oracle, fmt):
     for i in range(batch):
         single, _ = launch(ctx, ab_[i * sa:i * sa + bm * bk], bb_[i * sb:i * sb + bk * bn], np.zeros(bm * bn, np.uint16), bm, bn, bk,
                            mz.LAYOUT_NN, fmt, bk, bn, bn)
+        assert np.array_equal(single, dense[i * sc:i * sc + bm * bn]), i
+        assert not dense[i * sc + bm * bn:(i + 1) * sc].any(), "wrote between batch members"
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"])
+def test_few_rows_against_a_row_major_b(ctx, oracle, fmt):
+    """M <= 64 against 8-bit weights stored K x N: the streaming kernels with 1, 2 or 4 row groups, B's blocks (128 rows
+    of 256 bytes) read through transposing LDS reads.  Whole and ragged slabs, K tails, one and several K ranges, views,
+    every epilogue, the dispatcher's own choice, and the bits of the same product with the weights stored N x K."""
+    name = f"maize_gemm_{fmt}_skinny_nn"
+    cases = [(16, 256, 128, ""), (16, 512, 1024, ""), (13, 528, 2064, ""), (1, 272, 4096, ""), (16, 14336, 4096, ""),
+             (32, 512, 1024, "_m32"), (29, 528, 4112, "_m32"), (17, 2048, 8192, "_m32"),
+             (64, 512, 1024, "_m64"), (50, 272, 4112, "_m64"), (33, 1040, 16384, "_m64"), (64, 14336, 4096, "_m64")]
+    for (m, n, k, suffix) in cases if fmt in ("e4m3", "e5m2") else cases[2::3]:
+        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, kernel=name + suffix, label="few rows nn") == name + suffix
+    for suffix, m in (("", 16), ("_m32", 24), ("_m64", 40)):
+        for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=1104), dict(lda=4128, ldb=1072, ldc=1047), dict(out_f16=True)):
+            assert run_f8(ctx, oracle, m, 1040, 4112, layout=mz.LAYOUT_NN, fmt=fmt, kernel=name + suffix, label="few rows nn knobs", **kw) == name + suffix
+    for (m, n, k, suffix) in ((16, 14336, 4096, ""), (8, 1024, 2048, ""), (32, 4096, 4096, "_m32"), (64, 10240, 2048, "_m64")):
+        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="few rows nn, dispatcher") == name + suffix
+    elem = ab_of(FMT[fmt][1])
+    for (m, n, k, suffix) in ((16, 1040, 4112, ""), (48, 784, 2048, "_m64")):
+        a = f8_uniform(oracle, m * k, 81, elem[0])
+        b_kn = f8_uniform(oracle, k * n, 82, elem[1])
+        b_nk = np.ascontiguousarray(b_kn.reshape(k, n).T).ravel()
+        c_nn, took = launch(ctx, a, b_kn, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NN, fmt, k, n, n, kernel=name + suffix)
+        assert took == name + suffix
+        first = c_nn.copy()
+        for _ in range(2):                                   # several K ranges: the same bits every time
+            again, _ = launch(ctx, a, b_kn, np.full(m * n, 0x7FC0, np.uint16), m, n, k, mz.LAYOUT_NN, fmt, k, n, n, kernel=name + suffix)
+            assert np.array_equal(again, first)
+        # the N x K kernels give a lane other k of a 128-deep group (chunks 2g, 2g+1 instead of g, 4+g): same sums up to the
+        # instruction's internal order, so compare both with the oracle rather than bit for bit
+        c_nt, _ = launch(ctx, a, b_nk, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n, kernel=name.replace("_nn", "_nt") + suffix)
+        ref, val, scale = oracle.ref_gemm_ex(a, b_kn, m, n, k, layout=mz.LAYOUT_NN, lda=k, ldb=n, elem=FMT[fmt][1])
+        for got in (c_nn, c_nt):
+            assert oracle.compare(got, ref, val, scale, k, coeff=oracle.floor_coeff_f8(k))["n_fail"] == 0
+    # batched, padded strides; equal to its singles and nothing written between the members
+    bm, bn, bk, batch = 24, 528, 2064, 3
+    sa, sb, sc = bm * bk + 64, bk * bn + 128, bm * bn + 16
+    ab_ = f8_uniform(oracle, batch * sa, 21, elem[0])
+    bb_ = f8_uniform(oracle, batch * sb, 22, elem[1])
+    dense, took = launch(ctx, ab_, bb_, np.zeros(batch * sc, np.uint16), bm, bn, bk, mz.LAYOUT_NN, fmt, bk, bn, bn, batch=batch, strides=(sa, sb, sc),
+                         kernel=name + "_m32")
+    assert took == name + "_m32"
+    for i in range(batch):
+        single, _ = launch(ctx, ab_[i * sa:i * sa + bm * bk], bb_[i * sb:i * sb + bk * bn], np.zeros(bm * bn, np.uint16), bm, bn, bk,
+                           mz.LAYOUT_NN, fmt, bk, bn, bn, kernel=name + "_m32")
         assert np.array_equal(single, dense[i * sc:i * sc + bm * bn]), i
         assert not dense[i * sc + bm * bn:(i + 1) * sc].any(), "wrote between batch members"
 
