@@ -778,6 +778,18 @@ static bool plan_fits(const KernelInfo& ki, const maize_gemm_ex_desc_t& d, uint3
     return ki.plan(d, compute_units, &ld);
 }
 
+// Whether a product that the aligned kernels refuse earns back the packed path's copies and extra launches (25-45 us in
+// all) against the per-wave kernel.  That kernel reaches ~30 TFLOP/s on products with many 32 x 32 tiles (break-even
+// measured near M*N*K = 3e7), but each wave walks all of K alone at ~65 ns per element, so with few tiles its time
+// is 0.065 us x K whatever M and N are: 16 x 4096 x 4100 283 us against 46 us packed, 16 x 512 x 4100 263 / 27,
+// 1 x 4096 x 4100 247 / 47, 16 x 16384 x 1028 74 / 43, 8-bit 16 x 4104 x 4096 1014 / 35 -- but 16 x 16384 x 516 37 / 35,
+// 16 x 65536 x 260 24 / 44 and 17 x 50257 x 768 70 / 90.
+static bool copies_pay(const Dims& s, uint32_t batch) {
+    if ((double)s.m * s.n * s.k * batch >= 3e7 && s.m >= 24u && s.n >= 24u) return true;
+    const double tiles = (double)cdiv(s.m, 32) * cdiv(s.n, 32) * batch;     // one wave each; ~1500 run at a time
+    return (double)s.k * (tiles > 1500.0 ? tiles / 1500.0 : 1.0) >= 1000.0;
+}
+
 uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     const Dims s = dims_of(d);
     if (wide_in(d)) {   // fp32 / fp64 operands: one kernel per type and layout, any shape
@@ -834,7 +846,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
             return (uint32_t)ft;
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_packed", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fp = kernel_index(name);
-        if (fi >= 0 && !kKernels[fi].supports(d) && fp >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && s.m >= 24u && s.n >= 24u &&
+        if (fi >= 0 && !kKernels[fi].supports(d) && fp >= 0 && copies_pay(s, d.gemm.batch) &&
             kKernels[fp].supports(d) && plan_fits(kKernels[fp], d, compute_units))
             return (uint32_t)fp;
         return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
@@ -892,13 +904,12 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // 16 x 4096 x 4096 up and loses (8 vs 4-7 us) only on short K with few rows or columns.
     if (ti >= 0 && kKernels[ti].supports(d) && (s.k >= 128 || (s.m >= 128 && s.n >= 128))) return (uint32_t)ti;
     // Odd extents or unaligned operands: the per-wave kernel reaches ~30 TFLOP/s, the macro-tile
-    // kernel on repacked operands several hundred, at the price of extra launches (the packed path
-    // starts at ~21 us; measured break-even near M*N*K = 3e7) and of copying the operands once,
-    // which a product with very few rows or columns does not earn back.
+    // kernel on repacked operands several hundred, at the price of extra launches and of copying
+    // the operands once (copies_pay).
     static const char* const kPacked[2][2] = {{"maize_gemm_bf16_mt256_nn_packed", "maize_gemm_bf16_mt256_nt_packed"},
                                               {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nt_packed"}};
     const int pi = kernel_index(kPacked[half_in(d)][s.nt]);
-    if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && s.m >= 24u && s.n >= 24u &&
+    if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && copies_pay(s, d.gemm.batch) &&
         kKernels[pi].supports(d) && plan_fits(kKernels[pi], d, compute_units)) {
         // C takes 128-bit stores and K need not be split: the first pass stores C itself.
         static const char* const kPackedGen[2][2] = {{"maize_gemm_bf16_mt256_nn_packed_gen", "maize_gemm_bf16_mt256_nt_packed_gen"},
