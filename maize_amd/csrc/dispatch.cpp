@@ -783,11 +783,13 @@ static bool plan_fits(const KernelInfo& ki, const maize_gemm_ex_desc_t& d, uint3
 // measured near M*N*K = 3e7), but each wave walks all of K alone at ~65 ns per element, so with few tiles its time
 // is 0.065 us x K whatever M and N are: 16 x 4096 x 4100 283 us against 46 us packed, 16 x 512 x 4100 263 / 27,
 // 1 x 4096 x 4100 247 / 47, 16 x 16384 x 1028 74 / 43, 8-bit 16 x 4104 x 4096 1014 / 35 -- but 16 x 16384 x 516 37 / 35,
-// 16 x 65536 x 260 24 / 44 and 17 x 50257 x 768 70 / 90.
-static bool copies_pay(const Dims& s, uint32_t batch) {
+// 16 x 65536 x 260 24 / 44 and 17 x 50257 x 768 70 / 90 (804 by this measure).
+// 8-bit operands cost that kernel twice the time per element of K (it widens them as it loads: 24 x 768 x 960 124 us,
+// 100 x 112 x 512 83 us, 13 x 520 x 769 116 us).
+static bool copies_pay(const Dims& s, uint32_t batch, bool bytes8) {
     if ((double)s.m * s.n * s.k * batch >= 3e7 && s.m >= 24u && s.n >= 24u) return true;
     const double tiles = (double)cdiv(s.m, 32) * cdiv(s.n, 32) * batch;     // one wave each; ~1500 run at a time
-    return (double)s.k * (tiles > 1500.0 ? tiles / 1500.0 : 1.0) >= 1000.0;
+    return (double)s.k * (tiles > 1500.0 ? tiles / 1500.0 : 1.0) >= (bytes8 ? 400.0 : 850.0);
 }
 
 uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
@@ -846,7 +848,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
             return (uint32_t)ft;
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_packed", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fp = kernel_index(name);
-        if (fi >= 0 && !kKernels[fi].supports(d) && fp >= 0 && copies_pay(s, d.gemm.batch) &&
+        if (fi >= 0 && !kKernels[fi].supports(d) && fp >= 0 && copies_pay(s, d.gemm.batch, true) &&
             kKernels[fp].supports(d) && plan_fits(kKernels[fp], d, compute_units))
             return (uint32_t)fp;
         return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
@@ -909,7 +911,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     static const char* const kPacked[2][2] = {{"maize_gemm_bf16_mt256_nn_packed", "maize_gemm_bf16_mt256_nt_packed"},
                                               {"maize_gemm_f16_mt256_nn_packed", "maize_gemm_f16_mt256_nt_packed"}};
     const int pi = kernel_index(kPacked[half_in(d)][s.nt]);
-    if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && copies_pay(s, d.gemm.batch) &&
+    if (ti >= 0 && !kKernels[ti].supports(d) && pi >= 0 && copies_pay(s, d.gemm.batch, false) &&
         kKernels[pi].supports(d) && plan_fits(kKernels[pi], d, compute_units)) {
         // C takes 128-bit stores and K need not be split: the first pass stores C itself.
         static const char* const kPackedGen[2][2] = {{"maize_gemm_bf16_mt256_nn_packed_gen", "maize_gemm_bf16_mt256_nt_packed_gen"},

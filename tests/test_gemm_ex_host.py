@@ -216,7 +216,7 @@ def test_dispatch_of_8bit_operands():
             assert p["workspace_bytes"] == 65536 + 56 * 4 * tile_rows * 256 * 4, p       # one fp32 partial tile per (slab, K range)
         assert mz.gemm_plan(ex(64, 4096, 4096, in_type=it))["kernel"] == direct + "_splitk"                       # few slabs
         assert mz.gemm_plan(ex(16, 14344, 4096, in_type=it))["kernel"] == packed                                  # N % 16 != 0: copies (the per-wave kernel would walk K = 4096 alone)
-        assert mz.gemm_plan(ex(16, 14344, 520, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"                 # ... a short K: not worth the copies
+        assert mz.gemm_plan(ex(16, 14344, 264, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"                 # ... a short K: not worth the copies
         assert not _supports(few_nn, ex(16, 14344, 4096, in_type=it)) and not _supports(few_nn, ex(17, 14336, 4096, in_type=it))
         assert not _supports(few_nn, ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it)) and _supports(few_nn + "_m64", ex(17, 14336, 4096, in_type=it))
         mz.validate(ex(**big, in_type=it, ptrs=(0x1001, 0x100003, 0x2000000)))
