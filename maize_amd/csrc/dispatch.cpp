@@ -209,6 +209,18 @@ bool mt256_plan_impl(const maize_gemm_ex_desc_t& d, uint32_t compute_units, bool
     return ld->workspace_bytes < (1ull << 31) && e.nedge <= 16384u;
 }
 bool mt256_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, false, ld); }
+// 128 x 256 tiles: persistent over all tiles of all batch members like the plain kernels.
+bool mt256_h128_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const uint64_t all = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch;
+    if (all > 0x7FFFFFFFull) return false;
+    const uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+    ld->grid[0] = (resident && all > resident) ? resident : (uint32_t)all;
+    ld->grid[1] = 1; ld->grid[2] = 1;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0; ld->ksplit = 1; ld->split_first = 0; ld->reduce_grid = 0; ld->workspace_bytes = 0;
+    return true;
+}
 bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
 
 // ---- maize_gemm_{bf16,f16}_mt256_{nn,nt}_splitk: few tiles, long K ---------------------------
@@ -221,9 +233,11 @@ bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld
 // split is taken only if it wins by 10 %.  (2048^3, 64 tiles: 38 us unsplit, 40 us split 4 ways -- not
 // split; 64 x 4096 x 4096: 63 -> 22 us; 256 x 256 x 16384: 237 -> 38 us; 256 x 14336 x 4096, 56 tiles:
 // 67 -> 46 us four ways; 768 x 8192 x 8192, 96 tiles: 128 -> 93 us two ways.)
-uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
+// cost: what the model expects of the choice, in K steps of the unsplit kernel (~1.1 us), rounds of tiles counted.
+uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64, double* cost = nullptr) {
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * batch;
     const uint32_t nk = cdiv(s.k, kstep);                    // K steps of 128 bytes per row: 64 16-bit elements, 128 8-bit ones
+    if (cost) *cost = (8.0 + 1.0 * nk) * (double)(cus ? cdiv64(tiles, cus) : 1u);
     if (cus == 0 || tiles == 0 || tiles * 2 > cus || nk < 8u) return 1;
     uint32_t kmax = (uint32_t)(cus / tiles);
     if (kmax > nk / 4u) kmax = nk / 4u;
@@ -238,7 +252,21 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
         const double t = 8.0 + 1.0 * cdiv(nk, ks) + 6.0 + (1.2e-6 * elems + 0.15) * ks;
         if (t < best) { best = t; best_ks = ks; }
     }
+    if (cost && best_ks > 1u) *cost = best;
     return best_ks;
+}
+// 128 x 256 tiles instead: when they fit one round of the compute units (the 256 x 256 tiles fill half of them or
+// less) and a round of them -- 8 + 0.67 per K step, measured -- beats what the model expects of the 256-row kernels,
+// split over K or not (512 x 14336 x 4096: 70.4 us in two K ranges, 56.0 us here; 784 x 4096 x 2048 N x K: 36.4 -> 28.5;
+// but 128 x 14336 x 4096: 41.9 us in four ranges against 54.7, and more than one round never pays: a round of
+// half tiles costs 0.63 of a round of whole ones, 4096^3 89 -> 112 us, 2048 x 11008 x 4096 152 -> 162).
+bool h128_pays(const Dims& s, uint32_t batch, uint32_t cus) {
+    const uint32_t resident = cus >= 8u ? cus - cus % 8u : cus;
+    const uint64_t half_tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * batch;
+    if (resident == 0 || half_tiles > resident || s.k < 128u) return false;
+    double other = 0.0;
+    (void)splitk_ranges(s, batch, cus, 64, &other);
+    return 8.0 + 0.67 * cdiv(s.k, 64) < 1.03 * other;     // (a tie goes to the tiles: the model flatters large splits, 768 x 8192 x 8192 109.6 us in two ranges, 94.4 here)
 }
 bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && bf16_in(d); }
 bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && bf16_in(d); }
@@ -705,6 +733,12 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_f64_mt128_nt", nullptr, mt128_supports<MAIZE_IN_F64, true>, mt128_plan},
     {"maize_gemm_bf16_mt256_nn", nullptr, mt256_nn_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt", nullptr, mt256_nt_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_h128", nullptr, mt256_nn_supports, mt256_h128_plan},
+    {"maize_gemm_bf16_mt256_nt_h128", nullptr, mt256_nt_supports, mt256_h128_plan},
+    {"maize_gemm_bf16_mt256_nn_h128_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_h128_plan},
+    {"maize_gemm_bf16_mt256_nt_h128_gen", nullptr, mt256_nt_ktail_gen_supports, mt256_h128_plan},
+    {"maize_gemm_f16_mt256_nn_h128_gen", nullptr, f16_nn_ktail_gen_supports, mt256_h128_plan},
+    {"maize_gemm_f16_mt256_nt_h128_gen", nullptr, f16_nt_ktail_gen_supports, mt256_h128_plan},
     {"maize_gemm_bf16_mt256_nn_ktail", nullptr, mt256_nn_ktail_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_ktail", nullptr, mt256_nt_ktail_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_edge", nullptr, mt256_nn_supports, mt256_edge_plan},
@@ -876,6 +910,15 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     static const char* const kSplitK[2][2] = {{"maize_gemm_bf16_mt256_nn_splitk", "maize_gemm_bf16_mt256_nt_splitk"},
                                               {"maize_gemm_f16_mt256_nn_splitk", "maize_gemm_f16_mt256_nt_splitk"}};
     const int si = kernel_index(kSplitK[half_in(d)][s.nt]);
+    // ... or, where that is faster, compute it in 128-row tiles (the kernels that store C themselves: 16-byte rows of C).
+    if (h128_pays(s, d.gemm.batch, compute_units)) {
+        static const char* const kH128[2] = {"maize_gemm_bf16_mt256_nn_h128", "maize_gemm_bf16_mt256_nt_h128"};
+        static const char* const kH128Gen[2][2] = {{"maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_bf16_mt256_nt_h128_gen"},
+                                                   {"maize_gemm_f16_mt256_nn_h128_gen", "maize_gemm_f16_mt256_nt_h128_gen"}};
+        const int hp = kernel_index(kH128[s.nt]), hg = kernel_index(kH128Gen[half_in(d)][s.nt]);
+        if (hp >= 0 && !half_in(d) && kKernels[hp].supports(d)) return (uint32_t)hp;
+        if (hg >= 0 && kKernels[hg].supports(d)) return (uint32_t)hg;
+    }
     if (si >= 0 && kKernels[si].supports(d) && splitk_ranges(s, d.gemm.batch, compute_units) >= 2u) return (uint32_t)si;
     static const char* const kTiled[2][2][2] = {   // [edge split][K tail][NT]
         {{"maize_gemm_bf16_mt256_nn", "maize_gemm_bf16_mt256_nt"},

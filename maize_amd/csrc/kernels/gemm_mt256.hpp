@@ -131,17 +131,29 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 // v_mfma_f32_16x16x128_f8f6f4 deep (not two 32-deep halves), a fragment is two 16-byte reads, and a K step is four
 // "eighths" of 16 MFMAs with the barrier before the third.  A row-major (K x N) 8-bit B lands as 128 rows of 256
 // bytes (maps::sk8_*) and a fragment is four transposing 8-byte reads (ds_read_b64_tr_b8), two per MFMA slot.
-template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1>
+// BMT = 128: tiles of 128 x 256 for products whose 256 x 256 tiles would fill the compute units badly (half a round, or a
+// little over a whole number of rounds).  A wave then owns 64 x 128 as 4 x 8 accumulators and has one A group: a K
+// step is four eighths -- per K half (A0, B0), (A0, B1) -- the second of each pair reads the next half's (or tile's)
+// A0 and B0, B group b lives in buffer b, A's two buffers alternate with the K half, and the barrier stands in front of
+// the last eighth; 12 pieces per wave and K tile, one every three MFMA slots.
+template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
+    constexpr bool H128 = BMT == 128;
+    static_assert(BMT == 256 || (H128 && !IS8 && !EDGE && !SPLITK), "128-row tiles: 16-bit operands, whole K, C stored by the kernel");
+    constexpr int MI = BMT / 32;                        // accumulator rows of a wave (16 rows each)
+    constexpr int PA = BMT / 32;                        // 1 KiB pieces of A per wave and K tile (8 rows each, 4 waves)
+    constexpr uint32_t WROWS = BMT / 2;                 // rows of the tile per wave row
     static_assert(!IS8 || (!F16 && !EDGE), "8-bit operands: no edge splitting");
     constexpr bool TR8 = IS8 && !NT;                    // 8-bit row-major B: transposing reads
     constexpr uint32_t ES = IS8 ? 1u : 2u;              // bytes per element of A and B
     constexpr uint32_t CH = 16u / ES;                   // elements per 16-byte chunk
     constexpr int BKE = IS8 ? 128 : BK;                 // elements per K tile (128 bytes per row either way)
-    constexpr int NE = IS8 ? 4 : 8;                     // eighths (16 MFMAs each) per K step
-    constexpr int EB = IS8 ? 2 : 6;                     // the eighth the barrier stands in front of
-    constexpr int DS = IS8 ? 2 : DMA_STRIDE;            // MFMA slots between direct-to-LDS requests (an 8-bit MFMA is twice as long)
+    constexpr int NE = (IS8 || H128) ? 4 : 8;           // eighths (16 MFMAs each) per K step
+    constexpr int EB = IS8 ? 2 : H128 ? 3 : 6;          // the eighth the barrier stands in front of
+    constexpr int DS = IS8 ? 2 : H128 ? 3 : DMA_STRIDE; // MFMA slots between direct-to-LDS requests (an 8-bit MFMA is twice as long)
+    constexpr int AFTER = 16 * (NE - EB);               // MFMA slots of a step behind its barrier
+    constexpr int NP = PA + 8;                          // pieces per wave and K tile
     // One array per operand, two ring stages each.  The fragment reads below are inline assembly (one
     // base register per operand and K half, the stage and the fragment in the 16-bit offset field), so
     // the compiler sees no read of these arrays and never makes one wait for the direct-to-LDS loads
@@ -160,7 +172,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t wave = tid >> 6;
     const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t wm = wave >> 1, wn = wave & 1u;
-    const uint32_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    const uint32_t tm = (M + BMT - 1) / BMT, tn = (N + BN - 1) / BN;
     // Workgroups 0 .. whole-1 compute one tile each over all of K.  With edge splitting
     // (p.reserved = mode << 30 | whole + 1; mode 1: last tile column, mode 2: last tile row) the
     // whole tiles are the grid without that edge, and the rest of the workgroups share the edge
@@ -255,7 +267,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             bz = t / tiles_per;
             tile_of(t - (uint32_t)bz * tiles_per, tm, tn, &tile_m, &tile_n);
         }
-        m0 = tile_m * BM;
+        m0 = tile_m * BMT;
         n0 = tile_n * BN;
         Ag = (const char*)p.a + (bz * p.stride_a + (uint64_t)m0 * lda) * ES;   // the tile's first row of A (strides count elements)
         a_bytes = span(((uint64_t)(M - 1u - m0) * lda + K) * ES);
@@ -279,8 +291,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int i = 0; i < 8; ++i) {
             const uint32_t row = maps::kc_piece_row(wave * 8u + i, lane);
             const uint32_t c = maps::kc_piece_chunk(wave * 8u + i, lane);
-            a_vo[i] = (row * lda + c * CH) * ES;
-            if (i < 2) a_k[i] = c * CH;
+            if (i < PA) {                                   // A: pieces wave * PA + i (the lane's chunk depends on the piece's parity only)
+                const uint32_t arow = maps::kc_piece_row(wave * PA + i, lane), ac = maps::kc_piece_chunk(wave * PA + i, lane);
+                a_vo[i] = (arow * lda + ac * CH) * ES;
+                if (i < 2) a_k[i] = ac * CH;
+            }
             if (NT) {
                 b_vo[i] = (row * ldb + c * CH) * ES;
             } else {
@@ -292,12 +307,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     };
     select_tile(pid);
     const uint64_t b_view = ((uint64_t)(K - 1u) * ldb + N) * ES;               // bytes of a K x N B
-    // Issues piece pc (0..7 = A, 8..15 = B) of the tile that starts at k into stages (sa, sb).
+    // Issues piece pc (0..PA-1 = A, PA..PA+7 = B) of the tile that starts at k into stages (sa, sb).
     auto dma = [&](int pc, lds_ptr sa, lds_ptr sb, uint32_t k) {
         typedef __attribute__((address_space(3))) void* lvp;
-        const bool is_a = pc < 8;
-        const int i = is_a ? pc : pc - 8;
-        lds_ptr dst = (is_a ? sa : sb) + (wave_u * 8u + i) * 1024u;
+        const bool is_a = pc < PA;
+        const int i = is_a ? pc : pc - PA;
+        lds_ptr dst = (is_a ? sa : sb) + (wave_u * (is_a ? (uint32_t)PA : 8u) + i) * 1024u;
         // Tiles that start at or past K read through a zero-length descriptor: all zeros.
         if (!is_a && !NT) {
             // K x N B: the descriptor starts at row k of B (scalar 64-bit arithmetic, once per K tile) and ends with
@@ -335,12 +350,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // 2 (l/16) + 1 cost every read a two-way conflict).
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh) {
-            a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * 128u, kh, lane);
+            a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * WROWS, kh, lane);
             b_rd[kh] = (uint32_t)(uintptr_t)B0 + maps::kc_frag16_offset(wn * 128u, kh, lane);
         }
     } else {
 #pragma unroll
-        for (int kh = 0; kh < 2; ++kh) a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * 128u, kh, lane);
+        for (int kh = 0; kh < 2; ++kh) a_rd[kh] = (uint32_t)(uintptr_t)A0 + maps::kc_frag16_offset(wm * WROWS, kh, lane);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             b_rd[j] = (uint32_t)(uintptr_t)B0 + (TR8 ? maps::sk8_tr_offset(wn * 8u + j, 0, 0, lane) : maps::sk_tr_offset(wn * 8u + j, 0, lane));
@@ -399,11 +414,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // Read r (0..NAR-1) of A group ai, K half kh, of the tile in stage st.
     auto read_a = [&](int ai, int kh, int st, int r) {
         if (IS8) lds_read128(fa8[ai][r >> 1][r & 1], a_rd[r & 1], st * 16 + 4 * ai + (r >> 1));   // half r & 1 = the 16-bit kernel's kh
+        else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * 16 + r);                             // one A group; the buffer alternates with the K half
         else     lds_read128(fa[ai][r], a_rd[kh], st * 16 + 4 * ai + r);
     };
     // Read r (0..NBR-1) of B group bi, K half kh, of the tile in stage st.
     auto read_b = [&](int bi, int kh, int st, int r) {
-        const int buf = bi ^ (IS8 ? st : kh);
+        const int buf = H128 ? bi : bi ^ (IS8 ? st : kh);
         if (TR8) lds_read_tr8(fb8t[buf][r >> 2][r & 3], b_rd[4 * bi + (r >> 2)], st * 16 + ((r >> 1) & 1) * 8 + (r & 1));
         else if (IS8) lds_read128(fb8[buf][r >> 1][r & 1], b_rd[r & 1], st * 16 + 4 * bi + (r >> 1));
         else if (NT) lds_read128(fb[buf][r], b_rd[kh], st * 16 + 4 * bi + r);
@@ -431,7 +447,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                      (int)fb8t[buf][c][2][0], (int)fb8t[buf][c][2][1], (int)fb8t[buf][c][3][0], (int)fb8t[buf][c][3][1]};
     };
 
-    floatx4 acc[8][8];
+    floatx4 acc[MI][8];
     uint32_t k_early = 0;                  // tile whose early pieces are issued next (last quarter of a step)
     uint32_t k_late = 0;                   // tile whose late pieces are issued next (first quarter of a step)
 
@@ -442,8 +458,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         lds_ptr const ca = A0 + cur * TILE, cb = B0 + cur * TILE, na = A0 + (cur ^ 1) * TILE, nb = B0 + (cur ^ 1) * TILE;
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
-            const int kh = IS8 ? 0 : e >> 2, h4 = e & 3;
-            const int ai = h4 >> 1, bi = (h4 == 1 || h4 == 2) ? 1 : 0;
+            const int kh = IS8 ? 0 : H128 ? e >> 1 : e >> 2, h4 = H128 ? e & 1 : e & 3;
+            const int ai = H128 ? 0 : h4 >> 1, bi = H128 ? h4 : (h4 == 1 || h4 == 2) ? 1 : 0;
             const bool last_half = IS8 || kh == 1;                // the groups after this half belong to the next K tile
             // The group this eighth needs was requested during the one before: it has to be in.
             if (e != EB) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -472,11 +488,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(acc[4 * ai + r4][4 * bi + c4])
                                  : "v"(b_operand8(bi ^ cur, c4)), "v"(operand8(fa8[ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
                 else if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
-                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(bi ^ kh, c4)), "v"(fa[ai][r4]));
+                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(H128 ? bi : bi ^ kh, c4)), "v"(fa[H128 ? kh : ai][r4]));
                 else
-                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(bi ^ kh, c4)), "v"(fa[ai][r4]));
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(H128 ? bi : bi ^ kh, c4)), "v"(fa[H128 ? kh : ai][r4]));
                 // Side work of this slot: the reads of the group the next eighth needs ...
-                if (s % RSTRIDE == 0) {
+                if (H128) {
+                    // (A0, B0): B group 1 of this half; (A0, B1): A group 0 and B group 0 of the next half or tile
+                    const int r = s;
+                    if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);
+                    if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }
+                    if (h4 == 1 && r < NBR) { if (!last_half) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }
+                } else if (s % RSTRIDE == 0) {
                     const int r = s / RSTRIDE;
 #pragma unroll
                     for (int rb = r * RPS; rb < (r + 1) * RPS; ++rb) {
@@ -489,8 +511,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // ... and the direct-to-LDS request scheduled for this slot (issue_slot): late pieces of
                 // tile t+1 (its stage was freed by the previous barrier) before this step's barrier, early
                 // pieces of tile t+2 behind it.
-                const int slot = e >= EB ? 16 * (e - EB) + s : 32 + 16 * e + s;
-                if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {
+                const int slot = e >= EB ? 16 * (e - EB) + s : AFTER + 16 * e + s;
+                if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < NP) {
                     if (e >= EB) dma((slot - 2) / DS, ca, cb, k_early);
                     else         dma((slot - 2) / DS, na, nb, k_late);
                 }
@@ -502,11 +524,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     };
     // ---- prime: the first K tile of the first C tile, whole ------------------------------
 #pragma unroll
-    for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, k_begin);
+    for (int pc = 0; pc < NP; ++pc) dma(pc, A0, B0, k_begin);
 
     for (;;) {                                                  // one trip per C tile
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     // The wait also covers the C stores of the previous tile (loads and stores share the counter).
@@ -518,8 +540,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #pragma unroll
     for (int r = 0; r < NBR; ++r) read_b(0, 0, 0, r);
 #pragma unroll
-    for (int pc = 0; pc < 16; ++pc)
-        if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);   // tile 1, early pieces
+    for (int pc = 0; pc < NP; ++pc)
+        if (DS * pc + 2 < AFTER) dma(pc, A1, B1, k_begin + BKE);   // tile 1, early pieces
     k_early = k_begin + 2 * BKE;
     k_late = k_begin + BKE;
     // Two steps per trip so that each step sees its stages as compile-time constants.  An odd
@@ -555,7 +577,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         volatile uint32_t& ticket = *(volatile uint32_t*)lds_e;   // the staging region is idle until the epilogue
         uint32_t* counters = (uint32_t*)p.workspace;      // 16384 counters (zero between launches), then the tiles
 #pragma unroll
-        for (int c = 0; c < 64; ++c) {
+        for (int c = 0; c < MI * 8; ++c) {
             if (!chunk_live(c)) continue;
             const uint32_t row = wm * 128u + (c >> 3) * 16u + l16, col = wn * 128u + (c & 7) * 16u + lg * 4u;
             const uint32_t off = lane_live(c) ? ((slot * ks + z) * dense_rows + row) * dense_pitch + col * 4u : DROP;
@@ -579,7 +601,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     if (more) {
         select_tile(next);
 #pragma unroll
-        for (int pc = 0; pc < 16; ++pc) dma(pc, A0, B0, k_begin);
+        for (int pc = 0; pc < NP; ++pc) dma(pc, A0, B0, k_begin);
     }
 
     // ---- epilogue: fp32 -> bf16 (RNE), stage through LDS, 128-bit row stores --------------
@@ -596,11 +618,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // Split-K: the lane's place inside the partial tile.  Recomputed per tile on purpose (the empty
         // asm makes it opaque): hoisted out of the tile loop, the 32 addresses derived from it would
         // be kept live across the K loop and spilled.
-        uint32_t lane_part = (wm * 128u + r8) * BN + wn * 128u + c8 * 8u;
+        uint32_t lane_part = (wm * WROWS + r8) * BN + wn * 128u + c8 * 8u;
         asm volatile("" : "+v"(lane_part));
         float* const part_base = (float*)((char*)p.workspace + 65536) + (uint64_t)eslot * (BM * BN) + lane_part;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)                              // 32 rows per pass: accumulator rows 2i, 2i+1
+        for (int i = 0; i < MI / 2; ++i)                         // 32 rows per pass: accumulator rows 2i, 2i+1
 #pragma unroll
             for (int jh = 0; jh < 2; ++jh) {
 #pragma unroll
@@ -615,7 +637,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     const uint32_t row = maps::epi32_read_row(r, lane);     // 0..31 within the pass
                     const floatx4 lo = *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_read_offset(r, 0, lane));
                     const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_read_offset(r, 1, lane));
-                    const uint32_t grow = em0 + wm * 128u + i * 32u + row;
+                    const uint32_t grow = em0 + wm * WROWS + i * 32u + row;
                     if (gcol < N && grow < M) {                   // direct C: N % 8 == 0, a run is all in or all out
                         if (SPLITK) {
                             // fp32 partial tile of this (tile, K range), row-major 256 x 256, behind the 64 KiB
@@ -674,10 +696,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // no divergent branch per row.  Non-temporal: C is written once and not read again by this
         // kernel, it should not displace the operand panels in L2.
         const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce + (uint64_t)em0 * ldc, span(((uint64_t)(M - 1u - em0) * ldc + N) * 2u));
-        const uint32_t c_vo = (((wm * 128u + cr) * ldc + gcol) * 2u) | (gcol < N ? 0u : OOB);
+        const uint32_t c_vo = (((wm * WROWS + cr) * ldc + gcol) * 2u) | (gcol < N ? 0u : OOB);
         const uint32_t row_bytes = __builtin_amdgcn_readfirstlane(ldc * 2u);
     #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < MI / 2; ++i) {
     #pragma unroll
             for (int ii = 0; ii < 2; ++ii)                       // 32 rows per pass: accumulator rows 2i, 2i+1
     #pragma unroll
@@ -721,6 +743,13 @@ MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nn_gen, false, false, true)
 MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nt_gen, true, false, true)
 MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nn_ktail_gen, false, true, true)
 MAIZE_MT256_KERNEL_GEN(maize_gemm_f16_mt256_nt_ktail_gen, true, true, true)
+// 128 x 256 tiles: the plain kernels (K % 64 == 0, bf16 C = A.B) and the general ones (any K % 8 == 0, alpha / beta, fp32 C, half operands).
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128(GemmArgs p) { mt256::body<false, false, false, false, false, false, -1, 128>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128(GemmArgs p) { mt256::body<true, false, false, false, false, false, -1, 128>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, -1, 128>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, -1, 128>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nn_h128_gen(GemmArgs p) { mt256::body<false, true, false, true, true, false, -1, 128>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nt_h128_gen(GemmArgs p) { mt256::body<true, true, false, true, true, false, -1, 128>(p); }
 // Split-K: (tile, K range) work items, fp32 partial tiles to the workspace; any K % 8 == 0.
 #define MAIZE_MT256_KERNEL_SPLITK(name, nt, f16) \
     extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, true, false, true, f16, true>(p); }

@@ -169,3 +169,26 @@ def test_main_loop_of_the_headline_kernel_is_lean(kernels):
         assert count(body, "buffer_load_dwordx4") == 32                # 16 pieces of 1 KiB per wave and K step
         assert count(body, "s_barrier") == 2
         assert count(body, "s_waitcnt") <= 16                          # one per eighth of a K step, placed by hand
+
+
+def test_main_loop_of_the_half_height_kernels_is_lean(kernels):
+    """The 128 x 256 tile kernels: two unrolled K steps of 64 MFMAs per wave, one A group (8 reads per step) and two
+    B groups (16 reads, or 32 transposing ones), 12 pieces per wave and step, one barrier per step."""
+    for name, reads in (("maize_gemm_bf16_mt256_nn_h128", {"ds_read_b128": 16, "ds_read_b64_tr_b16": 64}),
+                        ("maize_gemm_bf16_mt256_nt_h128", {"ds_read_b128": 48})):
+        ins = kernels[name]
+        idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
+        assert len(idx) == 128 and count(ins, "v_mfma_f32_16x16x32_bf16") == 128
+        body = ins[idx[0]:idx[-1] + 1]
+        # (the row-major B's descriptor is re-based per K tile and cut at 2 GiB: the compiler does that one 64-bit compare,
+        # for which there is no scalar instruction, on the vector unit -- one uniform compare per K step)
+        extra = [i for i in body if not i.startswith(("v_mfma", "ds_read", "buffer_load_dwordx4", "s_", "v_cmp_lt_u64"))]
+        assert not extra and count(body, "v_cmp_lt_u64") <= 2, extra[:5]
+        for mnemonic, n in reads.items():
+            assert count(body, mnemonic) == n, (name, mnemonic)
+        assert count(body, "buffer_load_dwordx4") == 24 and count(body, "s_barrier") == 2
+        assert count(body, "s_waitcnt") <= 8
+    for name in ("maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_f16_mt256_nt_h128_gen"):
+        want = "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16"
+        assert count(kernels[name], want) == 128 and count(kernels[name], "v_mfma") == 128, name
+

@@ -99,6 +99,14 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         assert cdiv(nk, ks) * (ks - 1) < nk                    # no empty range
         assert p["workspace_bytes"] == TICKET_BYTES + items * 256 * 256 * 4 and p["workspace_bytes"] <= (1 << 32) + TICKET_BYTES
         assert p["reduce_grid"] == cdiv(m * cdiv(n, 8) * batch, 256)
+    elif "_h128" in name:
+        # 128 x 256 tiles, persistent over all of them; the plain form wants whole K tiles, the general form any K % 8 == 0
+        assert p["reduce_grid"] == 0 and p["workspace_bytes"] == 0 and p["split_first"] == 0 and p["ksplit"] == 1
+        assert p["block"] == (256, 1, 1) and gy == 1
+        assert ("_nt" in name) == (layout == mz.LAYOUT_NT)
+        assert k % 8 == 0 and n % 8 == 0 and (name.endswith("_gen") or k % 64 == 0)
+        resident = cus - cus % 8 if cus >= 8 else cus
+        assert gx == min(cdiv(m, 128) * cdiv(n, 256) * batch, resident)
     elif "_mt256_" in name:
         assert p["reduce_grid"] == 0
         assert p["block"] == (256, 1, 1) and gy == 1
@@ -187,7 +195,8 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (8192, 8192, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt",
         (16, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
-        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn",             # 64 tiles: partial tiles would cost more than they save
+        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128",        # 64 tiles: partial tiles would cost more than they save, 128 tiles of 128 rows fill half the chip
+        (512, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128",        # 112 tiles: 224 of 128 rows are one round
         (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",
         (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",              # N x K weights streamed once
@@ -220,20 +229,23 @@ def test_split_k_of_few_tiles_fills_the_chip_once():
     assert 2 <= p["ksplit"] <= 16 and p["grid"][0] == 16 * p["ksplit"]
     # more than half a chip of tiles, or a short K: no split
     assert mz.gemm_plan(desc(4096, 2304, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
-    assert mz.gemm_plan(desc(512, 512, 448), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
+    assert mz.gemm_plan(desc(512, 512, 448), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"      # (in 128-row tiles: 13.3 -> 8.6 us)
 
 
 def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
     """56 to 128 tiles on 256 compute units leave most of the chip idle for a whole walk of K: two or four K ranges
-    per tile pay for the partial tiles (measured: 256 x 14336 x 4096 67 -> 46 us, 768 x 8192 x 8192 128 -> 93 us),
-    while 2048^3 (64 tiles, a short K) stays whole (37 us against 40)."""
+    per tile pay for the partial tiles (measured: 256 x 14336 x 4096 67 -> 46 us, 768 x 8192 x 8192 128 -> 110 us) --
+    or, where one round of them is cheaper than the split, tiles of 128 rows (768 x 8192 x 8192 94 us, 2048^3 37 -> 29)."""
     p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 4 and p["grid"] == (224, 1, 1)
+    p = mz.gemm_plan(desc(128, 14336, 4096), compute_units=CUS)                  # one row of tiles either way: split (41.9 against 54.7 us)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 4
     p = mz.gemm_plan(desc(768, 8192, 8192), compute_units=CUS)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 2 and p["grid"] == (192, 1, 1)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128" and p["ksplit"] == 1 and p["grid"] == (192, 1, 1)
     p = mz.gemm_plan(desc(640, 8192, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_splitk" and p["ksplit"] == 2
-    assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128" and p["grid"] == (160, 1, 1)
+    assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"
+    assert mz.gemm_plan(desc(4096, 2304, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"       # 288 tiles of 128 rows would need two rounds
     assert mz.gemm_plan(desc(1024, 14336, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"   # 224 tiles: one round as it is
 
 

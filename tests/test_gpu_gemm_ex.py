@@ -157,36 +157,71 @@ def test_macro_tile_general_epilogue(ctx, oracle, layout, shape, lds):
     if lds and layout == mz.LAYOUT_NT:
         ldb = max(k + 8, 200)
     want = "maize_gemm_bf16_mt256_" + ("nt" if layout == mz.LAYOUT_NT else "nn") + ("_ktail" if k % 64 else "") + "_gen"
+    # (named: on shapes this small the dispatcher itself takes the 128-row form of the same kernels, test_half_height_tiles)
     for kw in KNOBS[:-1]:
-        took = run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, label="mt256 gen", **kw)
+        took = run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, kernel=want, label="mt256 gen", **kw)
         assert took == want, took
     # the plain product through the general epilogue
     run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, kernel=want, label="mt256 gen plain")
 
 
 def test_general_epilogue_with_several_tiles_per_workgroup_and_batches(ctx, oracle):
-    """More tiles than workgroups would be resident (forced by a raw launch with a small grid is covered
-    elsewhere); here: a batched fp32 product with beta, through the dispatcher."""
+    """A batched fp32 product with beta, through the dispatcher (which takes 128-row tiles for it: 18 of them) and
+    through the 256-row general kernel by name."""
     m, n, k, batch = 256, 384, 128, 3
     a = mz.gen.uniform_bf16(batch * m * k, 21)
     b = mz.gen.uniform_bf16(batch * k * n, 22)
     c0 = np.random.default_rng(3).standard_normal(batch * m * n).astype(np.float32)
     da, db, dc = ctx.upload(a), ctx.upload(b), ctx.upload(c0)
-    x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n), mz.Matrix(dc, m, n), batch=batch, stride_a=m * k,
-                        stride_b=k * n, stride_c=m * n, out_type=mz.OUT_F32, alpha=0.75, beta=1.5)
-    assert mz.gemm_plan(x)["kernel"] == "maize_gemm_bf16_mt256_nn_gen"
-    ctx.gemm_bf16(x)
-    ctx.sync()
-    got = dc.download(np.float32).reshape(batch, m, n)
-    da.free(); db.free(); dc.free()
-    for i in range(batch):
-        _, val, scale = oracle.ref_gemm_ex(a[i * m * k:(i + 1) * m * k], b[i * k * n:(i + 1) * k * n], m, n, k, alpha=0.75,
-                                           beta=1.5, c_old=c0.reshape(batch, m, n)[i], out_f32=True)
-        err = np.abs(got[i].astype(np.float64) - val)
-        assert (err <= (k / 16.0 + 4.0) * 2.0 ** -24 * scale + 1e-45).all(), f"batch member {i}"
+    try:
+        x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n), mz.Matrix(dc, m, n), batch=batch, stride_a=m * k,
+                            stride_b=k * n, stride_c=m * n, out_type=mz.OUT_F32, alpha=0.75, beta=1.5)
+        assert mz.gemm_plan(x)["kernel"] == "maize_gemm_bf16_mt256_nn_h128_gen"
+        for kernel in (None, "maize_gemm_bf16_mt256_nn_gen"):
+            dc.write(c0)
+            ctx.gemm_bf16(x, kernel=kernel)
+            ctx.sync()
+            got = dc.download(np.float32).reshape(batch, m, n)
+            for i in range(batch):
+                _, val, scale = oracle.ref_gemm_ex(a[i * m * k:(i + 1) * m * k], b[i * k * n:(i + 1) * k * n], m, n, k, alpha=0.75,
+                                                   beta=1.5, c_old=c0.reshape(batch, m, n)[i], out_f32=True)
+                err = np.abs(got[i].astype(np.float64) - val)
+                assert (err <= (k / 16.0 + 4.0) * 2.0 ** -24 * scale + 1e-45).all(), f"{kernel}: batch member {i}"
+    finally:
+        da.free(); db.free(); dc.free()
 
 
 # ---- IEEE half operands (the half-precision twin of the MMA op) ---------------------------------
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+def test_half_height_tiles(ctx, oracle, layout):
+    """The 128 x 256 tile kernels: plain (whole K tiles, C = A.B) and general (K tails, views, alpha / beta, fp32 C, half
+    operands), by name and as the dispatcher's choice for products whose 256-row tiles fill half the chip or less;
+    same bits as the 256-row kernels (the same sums in the same order)."""
+    tag = "nt" if layout == mz.LAYOUT_NT else "nn"
+    plain, gen, gen16 = (f"maize_gemm_bf16_mt256_{tag}_h128", f"maize_gemm_bf16_mt256_{tag}_h128_gen", f"maize_gemm_f16_mt256_{tag}_h128_gen")
+    for (m, n, k) in ((128, 256, 64), (512, 1024, 448), (1000, 1032, 192), (100, 264, 1024), (640, 776, 2048)):
+        assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=plain, label="h128") == plain
+    m, n, k = 520, 776, 328                                       # K % 64 != 0: the general form
+    bcols = n if layout == mz.LAYOUT_NN else k
+    for kw in (dict(), dict(lda=k + 8, ldb=bcols + 16, ldc=n + 8), dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8),
+               dict(alpha=2.0, beta=0.0, c_nan=True), dict(lda=k + 3, ldb=bcols + 5)):
+        assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen, label="h128 gen", **kw) == gen
+        assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen16, half=True, label="h128 gen half", **kw) == gen16
+    # the dispatcher's choice
+    assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, label="h128 auto") == plain
+    assert run_ex(ctx, oracle, 520, 776, 328, layout=layout, label="h128 auto tail") == gen
+    assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, alpha=0.5, beta=1.0, label="h128 auto scaled") == gen
+    assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, half=True, label="h128 auto half") == gen16
+    # batched, several tiles per workgroup: 5 x 640 x 768 in 128-row tiles = 75 tiles on the grid the plan gives
+    from tests.gpu_util import run_gemm
+    bm, bn, bk, batch = 640, 768, 512, 5
+    a = mz.gen.uniform_bf16(batch * bm * bk, 7)
+    b = mz.gen.uniform_bf16(batch * bk * bn, 8)
+    got = run_gemm(ctx, a, b, bm, bn, bk, layout=layout, batch=batch, kernel=plain)
+    base = run_gemm(ctx, a, b, bm, bn, bk, layout=layout, batch=batch, kernel=plain[:-5])
+    assert np.array_equal(got, base)
+
 
 @pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
 def test_half_operands_any_shape_kernel(ctx, oracle, layout):
@@ -204,7 +239,7 @@ def test_half_operands_macro_tile(ctx, oracle, layout, shape, lds):
         ldb = max(k + 8, 200)
     want = "maize_gemm_f16_mt256_" + ("nt" if layout == mz.LAYOUT_NT else "nn") + ("_ktail" if k % 64 else "") + "_gen"
     for kw in KNOBS:
-        took = run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, half=True, label="mt256 half", **kw)
+        took = run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, half=True, kernel=want, label="mt256 half", **kw)
         assert took == want, took
 
 

@@ -28,14 +28,25 @@ class Hazard(AssertionError):
 # macro-tile kernel: two-stage ring, 16 requests per tile per wave spread over MFMA slots
 # ---------------------------------------------------------------------------------------
 
+# how the K step numbers its MFMA slots and places the requests (16 pieces per wave and K tile with 256-row tiles, 12
+# with 128-row tiles; AFTER = the slots of a step behind its barrier: 32, or 16 with 128-row tiles)
+MT256_SLOT_FACTS = ("constexpr int DS = IS8 ? 2 : H128 ? 3 : DMA_STRIDE;", "constexpr int AFTER = 16 * (NE - EB);",
+                    "constexpr int NP = PA + 8;", "constexpr int PA = BMT / 32;",
+                    "constexpr int NE = (IS8 || H128) ? 4 : 8;", "constexpr int EB = IS8 ? 2 : H128 ? 3 : 6;",
+                    "const int slot = e >= EB ? 16 * (e - EB) + s : AFTER + 16 * e + s;",
+                    "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < NP) {",
+                    "if (DS * pc + 2 < AFTER) dma(pc, A1, B1, k_begin + BKE);",       # early pieces: those behind the barrier of step t itself
+                    "if (e >= EB) dma((slot - 2) / DS, ca, cb, k_early);", "else         dma((slot - 2) / DS, na, nb, k_late);")
+
+
 def mt256_issue_slots():
     """MFMA slot (counted from the barrier of step t, 128 slots per step) at which each of the 16 pieces of tile
     t + 2 is requested, as the kernel source defines it."""
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
     stride = int(re.search(r"constexpr int DMA_STRIDE = (\d+);", src).group(1))
     assert "constexpr int issue_slot(int pc) { return DMA_STRIDE * pc + 2; }" in src
-    assert "constexpr int DS = IS8 ? 2 : DMA_STRIDE;" in src and "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {" in src
-    assert "if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);" in src      # early pieces: those behind the barrier of step t itself
+    for fact in MT256_SLOT_FACTS:
+        assert fact in src, fact
     return [stride * pc + 2 for pc in range(16)]
 
 
@@ -55,8 +66,7 @@ def mt256_reads_per_eighth(nt):
     assert "constexpr int NBR = TR8 ? 16 : (IS8 || !NT) ? 8 : 4;" in src and "constexpr int RPS = TR8 ? 2 : 1;" in src
     for line in MT256_READ_LINES:
         assert line in src, line
-    assert "constexpr int EB = IS8 ? 2 : 6;" in src and "if (e == EB) {" in src
-    assert "const int slot = e >= EB ? 16 * (e - EB) + s : 32 + 16 * e + s;" in src
+    assert "if (e == EB) {" in src
     nbr = 4 if nt else 8
     # reads that bring in eighth e (issued during e - 1): e = 0: A0 and B0 (the first of them, A0, a whole eighth earlier)
     return [nbr, nbr, 4, 0, nbr, nbr, 4, 0], nbr
@@ -101,7 +111,7 @@ def mt256_wave_program(nk, slots, nt, barrier_eighth=6):
     return ops, steps
 
 
-def check_two_stage(ops, steps, nreads, parts=4):
+def check_two_stage(ops, steps, nreads, parts=4, pieces=16):
     """`nreads`: fragment reads per part of a K step if a number; a list gives, per part, how many reads of the
     tile must have been issued before the part's first MFMA (cumulative)."""
     cumulative = [nreads * (q + 1) for q in range(parts)] if isinstance(nreads, int) else list(nreads)
@@ -144,7 +154,7 @@ def check_two_stage(ops, steps, nreads, parts=4):
             _, tile, quarter, stage = op
             if stage != tile % 2:
                 raise Hazard(f"tile {tile} read from stage {stage}")
-            for pc in range(16):
+            for pc in range(pieces):
                 if visible_from.get((tile, pc), 1 << 30) > epoch:
                     raise Hazard(f"tile {tile} quarter {quarter} read in epoch {epoch} before piece {pc} is complete")
             last_read_epoch[tile] = epoch
@@ -162,7 +172,7 @@ def check_two_stage(ops, steps, nreads, parts=4):
         raise Hazard("K tiles not consumed exactly once, in order")
     for t in range(steps + 1):
         got = sorted(pc for (tile, pc) in dma_epoch if tile == t)
-        if t < steps and got != list(range(16)):
+        if t < steps and got != list(range(pieces)):
             raise Hazard(f"tile {t}: pieces requested {got}")
     return max(t for (t, _) in dma_epoch)
 
@@ -217,6 +227,80 @@ def test_macro_tile_checker_rejects_broken_schedules():
 
 
 # ---------------------------------------------------------------------------------------
+# 128 x 256 tiles: one A group per wave.  A K step is four eighths -- per K half (A0, B0), (A0, B1) --, the second of
+# each pair reads the next half's (or tile's) A0 and B0, the barrier stands in front of the last eighth, 12 pieces per
+# wave and K tile, one every three MFMA slots
+# ---------------------------------------------------------------------------------------
+
+H128_READ_LINES = ("if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);",
+                   "if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
+                   "if (h4 == 1 && r < NBR) { if (!last_half) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }",
+                   "const int kh = IS8 ? 0 : H128 ? e >> 1 : e >> 2, h4 = H128 ? e & 1 : e & 3;",
+                   "const int buf = H128 ? bi : bi ^ (IS8 ? st : kh);",
+                   "else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * 16 + r);")
+
+
+def h128_wave_program(nk, nt, barrier_at=3, ds=3, drop_read=None):
+    src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
+    for fact in MT256_SLOT_FACTS + H128_READ_LINES:
+        assert fact in src, fact
+    nbr = 4 if nt else 8
+    slots = [ds * pc + 2 for pc in range(12)]
+    # reads issued during eighth e: (eighth that needs them, how many, from the next tile?)
+    issued = {0: (1, nbr, False), 1: (2, 4 + nbr, False), 2: (3, nbr, False), 3: (0, 4 + nbr, True)}
+    ops = [("dma", 0, pc, 0) for pc in range(12)]
+    ops += [("wait_all",), ("barrier",)]
+    ops += [("read", 0, 0, 0)] * (4 + nbr)
+    ops += [("dma", 1, pc, 1) for pc in range(12) if slots[pc] < 16]
+    k_early, k_late = 2, 1
+    steps = nk + (nk & 1)
+    nread = 0
+    for t in range(steps):
+        cur, nxt = t & 1, (t & 1) ^ 1
+        for e in range(4):
+            if e == barrier_at:
+                ops += [("wait_all",), ("barrier",)]
+            need, n, next_tile = issued[e]
+            for sl in range(16):
+                ops.append(("mfma", t, e))
+                for _ in range((1 if sl < 4 else 0) + (1 if sl < nbr else 0) if n > nbr else (1 if sl < n else 0)):
+                    nread += 1
+                    if nread != drop_read:
+                        ops.append(("read", t + 1, need, nxt) if next_tile else ("read", t, need, cur))
+                slot = sl if e == 3 else 16 + 16 * e + sl
+                for pc in range(12):
+                    if slots[pc] == slot:
+                        ops.append(("dma", k_early, pc, cur) if e == 3 else ("dma", k_late, pc, nxt))
+        k_early += 1
+        k_late += 1
+    ops.append(("wait_all",))
+    return ops, steps
+
+
+def h128_cumulative_reads(nt):
+    nbr = 4 if nt else 8
+    return [4 + nbr, 4 + 2 * nbr, 8 + 3 * nbr, 8 + 4 * nbr]
+
+
+@pytest.mark.parametrize("nk", [1, 2, 3, 7, 64])
+@pytest.mark.parametrize("nt", [False, True])
+def test_half_height_tile_schedule_is_hazard_free(nk, nt):
+    ops, steps = h128_wave_program(nk, nt)
+    last_tile = check_two_stage(ops, steps, h128_cumulative_reads(nt), parts=4, pieces=12)
+    assert steps <= last_tile <= steps + 1
+
+
+def test_half_height_tile_checker_rejects_broken_schedules():
+    need = h128_cumulative_reads(True)
+    with pytest.raises(Hazard):                 # barrier one eighth early: the tile is refilled while its last B group is still being read
+        check_two_stage(*h128_wave_program(8, True, barrier_at=2), need, parts=4, pieces=12)
+    with pytest.raises(Hazard):                 # requests five slots apart: the last ones would come after the next barrier
+        check_two_stage(*h128_wave_program(8, True, ds=6), need, parts=4, pieces=12)
+    with pytest.raises(Hazard):                 # a fragment read dropped: MFMAs on stale registers
+        check_two_stage(*h128_wave_program(8, True, drop_read=30), need, parts=4, pieces=12)
+
+
+# ---------------------------------------------------------------------------------------
 # 8-bit macro-tile kernel: the same template with a K tile one matrix instruction deep: a K step is four groups of
 # 16 MFMAs, the barrier in front of the third, a group is 8 reads, one request per two MFMA slots.  With a row-major
 # B (transposing reads) a B group is 16 reads, two per MFMA slot.
@@ -224,10 +308,7 @@ def test_macro_tile_checker_rejects_broken_schedules():
 
 def f8_constants():
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
-    for fact in ("constexpr int NE = IS8 ? 4 : 8;", "constexpr int EB = IS8 ? 2 : 6;", "constexpr int DS = IS8 ? 2 : DMA_STRIDE;",
-                 "constexpr int NAR = IS8 ? 8 : 4;", "const bool last_half = IS8 || kh == 1;",
-                 "const int slot = e >= EB ? 16 * (e - EB) + s : 32 + 16 * e + s;",
-                 "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < 16) {", "if (DS * pc + 2 < 32) dma(pc, A1, B1, k_begin + BKE);",
+    for fact in MT256_SLOT_FACTS + ("constexpr int NAR = IS8 ? 8 : 4;", "const bool last_half = IS8 || kh == 1;",
                  "constexpr int NBR = TR8 ? 16 : (IS8 || !NT) ? 8 : 4;", "constexpr int RPS = TR8 ? 2 : 1;",
                  "constexpr bool TR8 = IS8 && !NT;") + MT256_READ_LINES:
         assert fact in src, fact
