@@ -260,18 +260,58 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
 // split over K or not (512 x 14336 x 4096: 70.4 us in two K ranges, 56.0 us here; 784 x 4096 x 2048 N x K: 36.4 -> 28.5;
 // but 128 x 14336 x 4096: 41.9 us in four ranges against 54.7, and more than one round never pays: a round of
 // half tiles costs 0.63 of a round of whole ones, 4096^3 89 -> 112 us, 2048 x 11008 x 4096 152 -> 162).
-bool h128_pays(const Dims& s, uint32_t batch, uint32_t cus) {
+// With few of them and a long K the 128-row tiles are cut over K too (same cost terms as above with 0.67 per K step: a
+// single row of tiles, 65 .. 128 rows of A, does half the matrix work of 256-row tiles).
+// Returns 0: the 256-row kernels; 1: 128-row tiles, whole K; >= 2: 128-row tiles in that many K ranges.
+uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus) {
     const uint32_t resident = cus >= 8u ? cus - cus % 8u : cus;
     const uint64_t half_tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * batch;
-    if (resident == 0 || half_tiles > resident || s.k < 128u) return false;
+    if (resident == 0 || half_tiles > resident || s.k < 128u) return 0;
     double other = 0.0;
     (void)splitk_ranges(s, batch, cus, 64, &other);
-    return 8.0 + 0.67 * cdiv(s.k, 64) < 1.03 * other;     // (a tie goes to the tiles: the model flatters large splits, 768 x 8192 x 8192 109.6 us in two ranges, 94.4 here)
+    const uint32_t nk = cdiv(s.k, 64);
+    double best = 8.0 + 0.67 * nk;
+    uint32_t best_ks = 1;
+    const double elems = (double)s.m * s.n * batch;
+    uint32_t kmax = (uint32_t)(resident / half_tiles);
+    if (kmax > nk / 4u) kmax = nk / 4u;
+    if (kmax > 64u) kmax = 64u;
+    if (half_tiles * 2 <= resident && nk >= 8u)
+        for (uint32_t ks = 2; ks <= kmax; ++ks) {
+            if (cdiv(nk, cdiv(nk, ks)) != ks) continue;            // would leave an empty range
+            if (half_tiles * ks * 131072ull > (1ull << 30)) break;
+            const double t = 8.0 + 0.67 * cdiv(nk, ks) + 6.0 + (1.2e-6 * elems + 0.15) * ks;
+            if (t < 0.9 * best) { best = t; best_ks = ks; }
+        }
+    // (a tie goes to the tiles: the model flatters large splits, 768 x 8192 x 8192 109.6 us in two ranges, 94.4 here)
+    return best < 1.03 * other ? best_ks : 0u;
 }
 bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && bf16_in(d); }
 bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && bf16_in(d); }
 bool splitk_f16_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && half_in(d); }
 bool splitk_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && half_in(d); }
+// The same for 128-row tiles: partial tiles of 128 x 256, flagged to the reduce pass by bit 0 of the launch flag.
+bool h128_splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch;
+    uint32_t ks = h128_choice(s, d.gemm.batch, compute_units);
+    // Named explicitly for a shape the dispatcher would not split this way: two ranges if K allows, else one.
+    if (ks < 2u) ks = cdiv(s.k, 64) >= 2u && tiles * 2ull * 131072ull <= (1ull << 30) ? 2u : 1u;
+    const uint64_t items = tiles * ks;
+    if (items > 0x1FFFFFFFull || items * 131072ull > (1ull << 32)) return false;
+    uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+    ld->grid[0] = (resident && items > resident) ? resident : (uint32_t)items;
+    ld->grid[1] = 1; ld->grid[2] = 1;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0;
+    ld->ksplit = ks;
+    ld->split_first = 1;                                          // 128-row partial tiles
+    ld->workspace_bytes = kTicketBytes + (size_t)items * 131072u;
+    const uint64_t runs = (uint64_t)s.m * cdiv(s.n, 8) * d.gemm.batch;
+    if (cdiv64(runs, 256) > 0x7FFFFFFFull) return false;
+    ld->reduce_grid = (uint32_t)cdiv64(runs, 256);
+    return true;
+}
 bool splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
     const Dims s = dims_of(d);
     const uint32_t kstep = fp8_in(d) ? 128u : 64u;
@@ -739,6 +779,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_h128_gen", nullptr, mt256_nt_ktail_gen_supports, mt256_h128_plan},
     {"maize_gemm_f16_mt256_nn_h128_gen", nullptr, f16_nn_ktail_gen_supports, mt256_h128_plan},
     {"maize_gemm_f16_mt256_nt_h128_gen", nullptr, f16_nt_ktail_gen_supports, mt256_h128_plan},
+    {"maize_gemm_bf16_mt256_nn_h128_splitk", nullptr, splitk_nn_supports, h128_splitk_plan},
+    {"maize_gemm_bf16_mt256_nt_h128_splitk", nullptr, splitk_nt_supports, h128_splitk_plan},
+    {"maize_gemm_f16_mt256_nn_h128_splitk", nullptr, splitk_f16_nn_supports, h128_splitk_plan},
+    {"maize_gemm_f16_mt256_nt_h128_splitk", nullptr, splitk_f16_nt_supports, h128_splitk_plan},
     {"maize_gemm_bf16_mt256_nn_ktail", nullptr, mt256_nn_ktail_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_ktail", nullptr, mt256_nt_ktail_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_edge", nullptr, mt256_nn_supports, mt256_edge_plan},
@@ -911,7 +955,14 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
                                               {"maize_gemm_f16_mt256_nn_splitk", "maize_gemm_f16_mt256_nt_splitk"}};
     const int si = kernel_index(kSplitK[half_in(d)][s.nt]);
     // ... or, where that is faster, compute it in 128-row tiles (the kernels that store C themselves: 16-byte rows of C).
-    if (h128_pays(s, d.gemm.batch, compute_units)) {
+    const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units);
+    if (hk >= 2u) {
+        static const char* const kH128Split[2][2] = {{"maize_gemm_bf16_mt256_nn_h128_splitk", "maize_gemm_bf16_mt256_nt_h128_splitk"},
+                                                     {"maize_gemm_f16_mt256_nn_h128_splitk", "maize_gemm_f16_mt256_nt_h128_splitk"}};
+        const int hs = kernel_index(kH128Split[half_in(d)][s.nt]);
+        if (hs >= 0 && kKernels[hs].supports(d) && plan_fits(kKernels[hs], d, compute_units)) return (uint32_t)hs;
+    }
+    if (hk == 1u) {
         static const char* const kH128[2] = {"maize_gemm_bf16_mt256_nn_h128", "maize_gemm_bf16_mt256_nt_h128"};
         static const char* const kH128Gen[2][2] = {{"maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_bf16_mt256_nt_h128_gen"},
                                                    {"maize_gemm_f16_mt256_nn_h128_gen", "maize_gemm_f16_mt256_nt_h128_gen"}};

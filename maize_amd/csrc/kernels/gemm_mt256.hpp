@@ -140,7 +140,7 @@ template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
     constexpr bool H128 = BMT == 128;
-    static_assert(BMT == 256 || (H128 && !IS8 && !EDGE && !SPLITK), "128-row tiles: 16-bit operands, whole K, C stored by the kernel");
+    static_assert(BMT == 256 || (H128 && !IS8 && !EDGE), "128-row tiles: 16-bit operands, no edge splitting");
     constexpr int MI = BMT / 32;                        // accumulator rows of a wave (16 rows each)
     constexpr int PA = BMT / 32;                        // 1 KiB pieces of A per wave and K tile (8 rows each, 4 waves)
     constexpr uint32_t WROWS = BMT / 2;                 // rows of the tile per wave row
@@ -620,7 +620,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // be kept live across the K loop and spilled.
         uint32_t lane_part = (wm * WROWS + r8) * BN + wn * 128u + c8 * 8u;
         asm volatile("" : "+v"(lane_part));
-        float* const part_base = (float*)((char*)p.workspace + 65536) + (uint64_t)eslot * (BM * BN) + lane_part;
+        float* const part_base = (float*)((char*)p.workspace + 65536) + (uint64_t)eslot * (BMT * BN) + lane_part;
 #pragma unroll
         for (int i = 0; i < MI / 2; ++i)                         // 32 rows per pass: accumulator rows 2i, 2i+1
 #pragma unroll
@@ -750,6 +750,11 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128_
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, -1, 128>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nn_h128_gen(GemmArgs p) { mt256::body<false, true, false, true, true, false, -1, 128>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nt_h128_gen(GemmArgs p) { mt256::body<true, true, false, true, true, false, -1, 128>(p); }
+// ... and split over K: (128 x 256 tile, K range) work items, fp32 partial tiles of 128 rows for the reduce pass.
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, -1, 128>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, -1, 128>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nn_h128_splitk(GemmArgs p) { mt256::body<false, true, false, true, true, true, -1, 128>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nt_h128_splitk(GemmArgs p) { mt256::body<true, true, false, true, true, true, -1, 128>(p); }
 // Split-K: (tile, K range) work items, fp32 partial tiles to the workspace; any K % 8 == 0.
 #define MAIZE_MT256_KERNEL_SPLITK(name, nt, f16) \
     extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, true, false, true, f16, true>(p); }

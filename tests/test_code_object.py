@@ -188,7 +188,7 @@ def test_main_loop_of_the_half_height_kernels_is_lean(kernels):
             assert count(body, mnemonic) == n, (name, mnemonic)
         assert count(body, "buffer_load_dwordx4") == 24 and count(body, "s_barrier") == 2
         assert count(body, "s_waitcnt") <= 8
-    for name in ("maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_f16_mt256_nt_h128_gen"):
+    for name in ("maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_f16_mt256_nt_h128_gen", "maize_gemm_bf16_mt256_nt_h128_splitk", "maize_gemm_f16_mt256_nn_h128_splitk"):
         want = "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16"
         assert count(kernels[name], want) == 128 and count(kernels[name], "v_mfma") == 128, name
 

@@ -90,14 +90,17 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         assert p["reduce_grid"] == cdiv(m * cdiv(n, 8) * batch, 256)
     elif splitk:
         # (tile, K range) work items, one fp32 partial tile each, then the reduce pass over runs of 8 columns
+        # (tiles of 256 x 256, or of 128 x 256 -- flagged to the reduce pass by bit 0 of the launch flag)
         assert p["block"] == (256, 1, 1) and gy == 1 and k % 8 == 0 and n % 8 == 0
         ks = p["ksplit"]
-        items = cdiv(m, 256) * cdiv(n, 256) * batch * ks
+        tile_rows = 128 if "_h128" in name else 256
+        assert p["split_first"] == (1 if tile_rows == 128 else 0)
+        items = cdiv(m, tile_rows) * cdiv(n, 256) * batch * ks
         resident = cus - cus % 8 if cus >= 8 else cus
         assert 1 <= ks <= 64 and gx == min(items, resident)
         nk = cdiv(k, 64)
         assert cdiv(nk, ks) * (ks - 1) < nk                    # no empty range
-        assert p["workspace_bytes"] == TICKET_BYTES + items * 256 * 256 * 4 and p["workspace_bytes"] <= (1 << 32) + TICKET_BYTES
+        assert p["workspace_bytes"] == TICKET_BYTES + items * tile_rows * 256 * 4 and p["workspace_bytes"] <= (1 << 32) + TICKET_BYTES
         assert p["reduce_grid"] == cdiv(m * cdiv(n, 8) * batch, 256)
     elif "_h128" in name:
         # 128 x 256 tiles, persistent over all of them; the plain form wants whole K tiles, the general form any K % 8 == 0
@@ -197,16 +200,16 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128",        # 64 tiles: partial tiles would cost more than they save, 128 tiles of 128 rows fill half the chip
         (512, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128",        # 112 tiles: 224 of 128 rows are one round
-        (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",
-        (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
+        (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128_splitk",  # few tiles, a long K: 128-row tiles cut over K
+        (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128_splitk",
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",              # N x K weights streamed once
         (16, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",
         (17, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m32",          # 17 .. 32 rows: two row groups
         (64, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m64",         # 33 .. 64 rows and many slabs: four
-        (65, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",       # more than 64 rows
+        (65, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128_splitk",  # more than 64 rows
         (32, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn_m32",
         (64, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn_m64",
-        (64, 8192, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",        # 64 rows, 32 slabs: the tile kernel cut over K
+        (64, 8192, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128_splitk",   # 64 rows, 32 slabs: the tile kernel cut over K
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
         (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",      # odd N: operands read where they lie, C written element-wise by the reduce pass
         (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
@@ -222,11 +225,13 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
 
 def test_split_k_of_few_tiles_fills_the_chip_once():
     p = mz.gemm_plan(desc(64, 4096, 4096), compute_units=CUS)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and 8 <= p["ksplit"] <= 16 and p["grid"] == (16 * p["ksplit"], 1, 1)
-    p = mz.gemm_plan(desc(256, 256, 16384), compute_units=CUS)
-    assert 32 <= p["ksplit"] <= 64 and p["grid"] == (p["ksplit"], 1, 1)
-    p = mz.gemm_plan(desc(1024, 1024, 8192), compute_units=CUS)
-    assert 2 <= p["ksplit"] <= 16 and p["grid"][0] == 16 * p["ksplit"]
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and 8 <= p["ksplit"] <= 16 and p["grid"] == (16 * p["ksplit"], 1, 1)
+    p = mz.gemm_plan(desc(256, 256, 16384), compute_units=CUS)                    # two tiles of 128 rows
+    assert 16 <= p["ksplit"] <= 64 and p["grid"] == (2 * p["ksplit"], 1, 1)
+    p = mz.gemm_plan(desc(1024, 1024, 8192), compute_units=CUS)                   # 32 tiles of 128 rows
+    assert 2 <= p["ksplit"] <= 16 and p["grid"][0] == 32 * p["ksplit"]
+    p = mz.gemm_plan(desc(64, 4096, 4096), kernel="maize_gemm_bf16_mt256_nn_splitk", compute_units=CUS)          # the 256-row form by name
+    assert 8 <= p["ksplit"] <= 16 and p["grid"] == (16 * p["ksplit"], 1, 1)
     # more than half a chip of tiles, or a short K: no split
     assert mz.gemm_plan(desc(4096, 2304, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
     assert mz.gemm_plan(desc(512, 512, 448), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"      # (in 128-row tiles: 13.3 -> 8.6 us)
@@ -236,10 +241,10 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
     """56 to 128 tiles on 256 compute units leave most of the chip idle for a whole walk of K: two or four K ranges
     per tile pay for the partial tiles (measured: 256 x 14336 x 4096 67 -> 46 us, 768 x 8192 x 8192 128 -> 110 us) --
     or, where one round of them is cheaper than the split, tiles of 128 rows (768 x 8192 x 8192 94 us, 2048^3 37 -> 29)."""
-    p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 4 and p["grid"] == (224, 1, 1)
-    p = mz.gemm_plan(desc(128, 14336, 4096), compute_units=CUS)                  # one row of tiles either way: split (41.9 against 54.7 us)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 4
+    p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)                  # 112 tiles of 128 rows in two K ranges
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and p["ksplit"] == 2 and p["grid"] == (224, 1, 1)
+    p = mz.gemm_plan(desc(128, 14336, 4096), compute_units=CUS)                  # one row of tiles: cut over K (40 us against 54.7 whole)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and p["ksplit"] == 3 and p["grid"] == (168, 1, 1)
     p = mz.gemm_plan(desc(768, 8192, 8192), compute_units=CUS)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128" and p["ksplit"] == 1 and p["grid"] == (192, 1, 1)
     p = mz.gemm_plan(desc(640, 8192, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)

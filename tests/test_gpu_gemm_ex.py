@@ -314,16 +314,19 @@ def test_half_full_size_4096_cubed(ctx, oracle):
 def test_split_k_kernels(ctx, oracle, layout, shape):
     m, n, k = shape
     want = "maize_gemm_bf16_mt256_" + ("nt" if layout == mz.LAYOUT_NT else "nn") + "_splitk"
+    half_tiles = want.replace("_splitk", "_h128_splitk")                 # the same on tiles of 128 x 256
     run_ex(ctx, oracle, m, n, k, layout=layout, label="dispatcher")      # whatever the cost model picks
     run_ex(ctx, oracle, m, n, k, layout=layout, kernel=want, label="splitk")
+    run_ex(ctx, oracle, m, n, k, layout=layout, kernel=half_tiles, label="splitk, 128-row tiles")
     if (m, n, k) == (64, 4096, 4096):
         x = mz.gemm_ex_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x1000000, *((k, n) if layout == mz.LAYOUT_NN else (n, k))),
                             mz.GlobalMatrix(0x4000000, m, n), layout=layout)
-        assert mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"] == want
+        assert mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"] == half_tiles
     for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(half=True),
                dict(lda=k + 8, ldc=n + 16)):
-        run_ex(ctx, oracle, m, n, k, layout=layout, kernel=("maize_gemm_f16_mt256_" + want[22:]) if kw.get("half") else want,
-               label="splitk knobs", **kw)
+        for name in (want, half_tiles):
+            run_ex(ctx, oracle, m, n, k, layout=layout, kernel=("maize_gemm_f16_mt256_" + name[22:]) if kw.get("half") else name,
+                   label="splitk knobs", **kw)
 
 
 def test_split_k_batched_and_more_items_than_workgroups(ctx, oracle):
