@@ -263,14 +263,18 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
 // With few of them and a long K the 128-row tiles are cut over K too (same cost terms as above with 0.67 per K step: a
 // single row of tiles, 65 .. 128 rows of A, does half the matrix work of 256-row tiles).
 // Returns 0: the 256-row kernels; 1: 128-row tiles, whole K; >= 2: 128-row tiles in that many K ranges.
-uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus) {
+uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
     const uint32_t resident = cus >= 8u ? cus - cus % 8u : cus;
     const uint64_t half_tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * batch;
     if (resident == 0 || half_tiles > resident || s.k < 128u) return 0;
     double other = 0.0;
-    (void)splitk_ranges(s, batch, cus, 64, &other);
-    const uint32_t nk = cdiv(s.k, 64);
-    double best = 8.0 + 0.67 * nk;
+    (void)splitk_ranges(s, batch, cus, kstep, &other);
+    const uint32_t nk = cdiv(s.k, kstep);
+    // per K step: 0.67 of the 256-row kernel's; an 8-bit step (128 deep) takes 1.3 of a 16-bit one, which the fixed terms
+    // here (in 16-bit steps) have to be weighed against (E4M3 128 x 14336 x 4096: 31.1 us whole, 25.8 in two ranges)
+    const double step = kstep == 128u ? 0.87 : 0.67;
+    const double whole = 8.0 + step * nk;
+    double best = 0.9 * whole;                                     // splitting has to win 10 %
     uint32_t best_ks = 1;
     const double elems = (double)s.m * s.n * batch;
     uint32_t kmax = (uint32_t)(resident / half_tiles);
@@ -280,9 +284,10 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus) {
         for (uint32_t ks = 2; ks <= kmax; ++ks) {
             if (cdiv(nk, cdiv(nk, ks)) != ks) continue;            // would leave an empty range
             if (half_tiles * ks * 131072ull > (1ull << 30)) break;
-            const double t = 8.0 + 0.67 * cdiv(nk, ks) + 6.0 + (1.2e-6 * elems + 0.15) * ks;
-            if (t < 0.9 * best) { best = t; best_ks = ks; }
+            const double t = 8.0 + step * cdiv(nk, ks) + 6.0 + (1.2e-6 * elems + 0.15) * ks;
+            if (t < best) { best = t; best_ks = ks; }
         }
+    if (best_ks == 1u) best = whole;
     // (a tie goes to the tiles: the model flatters large splits, 768 x 8192 x 8192 109.6 us in two ranges, 94.4 here)
     return best < 1.03 * other ? best_ks : 0u;
 }
@@ -294,9 +299,10 @@ bool splitk_f16_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt
 bool h128_splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
     const Dims s = dims_of(d);
     const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch;
-    uint32_t ks = h128_choice(s, d.gemm.batch, compute_units);
+    const uint32_t kstep = fp8_in(d) ? 128u : 64u;
+    uint32_t ks = h128_choice(s, d.gemm.batch, compute_units, kstep);
     // Named explicitly for a shape the dispatcher would not split this way: two ranges if K allows, else one.
-    if (ks < 2u) ks = cdiv(s.k, 64) >= 2u && tiles * 2ull * 131072ull <= (1ull << 30) ? 2u : 1u;
+    if (ks < 2u) ks = cdiv(s.k, kstep) >= 2u && tiles * 2ull * 131072ull <= (1ull << 30) ? 2u : 1u;
     const uint64_t items = tiles * ks;
     if (items > 0x1FFFFFFFull || items * 131072ull > (1ull << 32)) return false;
     uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
@@ -828,6 +834,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_" #tag "_mt256_nn", nullptr, tag##_nn_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nn_gen", nullptr, tag##_nn_gen_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nn_splitk", nullptr, tag##_nn_gen_supports, splitk_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_h128_gen", nullptr, tag##_nt_gen_supports, mt256_h128_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_h128_splitk", nullptr, tag##_nt_gen_supports, h128_splitk_plan}, \
+    {"maize_gemm_" #tag "_mt256_nn_h128_gen", nullptr, tag##_nn_gen_supports, mt256_h128_plan}, \
+    {"maize_gemm_" #tag "_mt256_nn_h128_splitk", nullptr, tag##_nn_gen_supports, h128_splitk_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_packed", "maize_gemm_" #tag "_mt256_nt_splitk", tag##_packed_supports, packed8_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_trb", "maize_gemm_" #tag "_mt256_nt", tag##_trb_supports, trb_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_trb_gen", "maize_gemm_" #tag "_mt256_nt_gen", tag##_trb_gen_supports, trb_plan},
@@ -900,6 +910,15 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
             std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nn_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.m <= 32u ? "m32" : "m64");
             const int gm = kernel_index(name);
             if (gm >= 0 && kKernels[gm].supports(d) && plan_fits(kKernels[gm], d, compute_units)) return (uint32_t)gm;
+        }
+        // Tiles of 128 x 256, whole or cut over K, where they beat the 256-row kernels (half a round of tiles or less).
+        {
+            const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units, 128);
+            if (hk >= 1u) {
+                std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_%s_h128_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.nt ? "nt" : "nn", hk >= 2u ? "splitk" : "gen");
+                const int fh = kernel_index(name);
+                if (fh >= 0 && kKernels[fh].supports(d) && plan_fits(kKernels[fh], d, compute_units)) return (uint32_t)fh;
+            }
         }
         std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_nt_splitk", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fs = kernel_index(name);

@@ -135,12 +135,14 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 // little over a whole number of rounds).  A wave then owns 64 x 128 as 4 x 8 accumulators and has one A group: a K
 // step is four eighths -- per K half (A0, B0), (A0, B1) -- the second of each pair reads the next half's (or tile's)
 // A0 and B0, B group b lives in buffer b, A's two buffers alternate with the K half, and the barrier stands in front of
-// the last eighth; 12 pieces per wave and K tile, one every three MFMA slots.
+// the last eighth; 12 pieces per wave and K tile, one every three MFMA slots.  8-bit operands: a K tile is one matrix
+// instruction deep, so the step is just the pair (A0, B0), (A0, B1) with the barrier between the two, A's buffers
+// alternate with the K tile, and the 12 pieces go out one every two (twice as long) MFMA slots.
 template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
     constexpr bool H128 = BMT == 128;
-    static_assert(BMT == 256 || (H128 && !IS8 && !EDGE), "128-row tiles: 16-bit operands, no edge splitting");
+    static_assert(BMT == 256 || (H128 && !EDGE), "128-row tiles: no edge splitting");
     constexpr int MI = BMT / 32;                        // accumulator rows of a wave (16 rows each)
     constexpr int PA = BMT / 32;                        // 1 KiB pieces of A per wave and K tile (8 rows each, 4 waves)
     constexpr uint32_t WROWS = BMT / 2;                 // rows of the tile per wave row
@@ -149,9 +151,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr uint32_t ES = IS8 ? 1u : 2u;              // bytes per element of A and B
     constexpr uint32_t CH = 16u / ES;                   // elements per 16-byte chunk
     constexpr int BKE = IS8 ? 128 : BK;                 // elements per K tile (128 bytes per row either way)
-    constexpr int NE = (IS8 || H128) ? 4 : 8;           // eighths (16 MFMAs each) per K step
-    constexpr int EB = IS8 ? 2 : H128 ? 3 : 6;          // the eighth the barrier stands in front of
-    constexpr int DS = IS8 ? 2 : H128 ? 3 : DMA_STRIDE; // MFMA slots between direct-to-LDS requests (an 8-bit MFMA is twice as long)
+    constexpr int NE = (IS8 && H128) ? 2 : (IS8 || H128) ? 4 : 8;   // eighths (16 MFMAs each) per K step
+    constexpr int EB = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : 6;  // the eighth the barrier stands in front of
+    // MFMA slots between direct-to-LDS requests (an 8-bit MFMA is twice as long; with 128-row tiles its step has 32 slots
+    // only, and one request per slot leaves the last of the twelve 18 slots to land)
+    constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : DMA_STRIDE;
     constexpr int AFTER = 16 * (NE - EB);               // MFMA slots of a step behind its barrier
     constexpr int NP = PA + 8;                          // pieces per wave and K tile
     // One array per operand, two ring stages each.  The fragment reads below are inline assembly (one
@@ -413,7 +417,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #undef MAIZE_RD_CASE
     // Read r (0..NAR-1) of A group ai, K half kh, of the tile in stage st.
     auto read_a = [&](int ai, int kh, int st, int r) {
-        if (IS8) lds_read128(fa8[ai][r >> 1][r & 1], a_rd[r & 1], st * 16 + 4 * ai + (r >> 1));   // half r & 1 = the 16-bit kernel's kh
+        if (IS8 && H128) lds_read128(fa8[st & 1][r >> 1][r & 1], a_rd[r & 1], st * 16 + (r >> 1));   // one A group; the buffer alternates with the K tile
+        else if (IS8) lds_read128(fa8[ai][r >> 1][r & 1], a_rd[r & 1], st * 16 + 4 * ai + (r >> 1));   // half r & 1 = the 16-bit kernel's kh
         else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * 16 + r);                             // one A group; the buffer alternates with the K half
         else     lds_read128(fa[ai][r], a_rd[kh], st * 16 + 4 * ai + r);
     };
@@ -486,7 +491,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // accumulator comes up again 128 MFMAs later: no dependent back-to-back issue.)
                 if (IS8)   // 8-bit operands: B is the first source, so cbsz carries B's format and blgp A's (0 = E4M3, 1 = E5M2)
                     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(acc[4 * ai + r4][4 * bi + c4])
-                                 : "v"(b_operand8(bi ^ cur, c4)), "v"(operand8(fa8[ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
+                                 : "v"(b_operand8(H128 ? bi : bi ^ cur, c4)), "v"(operand8(fa8[H128 ? cur & 1 : ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
                 else if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
                     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(H128 ? bi : bi ^ kh, c4)), "v"(fa[H128 ? kh : ai][r4]));
                 else
@@ -495,9 +500,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 if (H128) {
                     // (A0, B0): B group 1 of this half; (A0, B1): A group 0 and B group 0 of the next half or tile
                     const int r = s;
-                    if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);
+#pragma unroll
+                    for (int rb = r * RPS; rb < (r + 1) * RPS; ++rb) {
+                        if (h4 == 0 && rb < NBR) read_b(1, kh, cur, rb);
+                        if (h4 == 1 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }
+                    }
                     if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }
-                    if (h4 == 1 && r < NBR) { if (!last_half) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }
                 } else if (s % RSTRIDE == 0) {
                     const int r = s / RSTRIDE;
 #pragma unroll

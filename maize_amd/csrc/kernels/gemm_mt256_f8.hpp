@@ -21,6 +21,9 @@
 // lane assembles the same 32 bytes of K per MFMA from four transposing 8-byte LDS reads (ds_read_b64_tr_b8): no
 // transposed copy, no workspace; rows of B on 16-byte boundaries and N % 16 == 0.
 //
+// _h128: tiles of 128 x 256 (general epilogue, and cut over K), for products whose 256-row tiles would fill half the
+// compute units or less: the K step is the pair (A0, B0), (A0, B1) with the barrier between the two.
+//
 // 16 x 16 x 128 and not 32 x 32 x 64 (the first version): register-only loops of the two on E4M3 data
 // from uniform[-1,1) measure 39.9 us against 42.9 us for the FLOP of 4096^3 at the board's power limit
 // (both 38 us on zeros).  K % 16 == 0 and N % 8 == 0; rows of A and B start on 16-byte boundaries; any K
@@ -37,7 +40,11 @@ namespace maize {
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, (fa) | ((fb) << 1)>(p); } \
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn(GemmArgs p) { mt256::body<false, true, false, false, false, false, (fa) | ((fb) << 1)>(p); } \
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, (fa) | ((fb) << 1)>(p); } \
-    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, (fa) | ((fb) << 1)>(p); }
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, (fa) | ((fb) << 1)>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_h128_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, (fa) | ((fb) << 1), 128>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_h128_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, (fa) | ((fb) << 1), 128>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, (fa) | ((fb) << 1), 128>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, (fa) | ((fb) << 1), 128>(p); }
 MAIZE_F8_KERNELS(e4m3, 0, 0)
 MAIZE_F8_KERNELS(e5m2, 1, 1)
 MAIZE_F8_KERNELS(e4m3e5m2, 0, 1)     // A is E4M3, B is E5M2

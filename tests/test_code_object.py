@@ -96,17 +96,19 @@ def test_matrix_instruction_per_kernel(kernels):
             # 8-bit operands: the 128-deep 16 x 16 instruction (cheaper per multiply-add at the power limit than 32 x 32 x 64).
             # B is fed as the first source, so cbsz carries B's format code and blgp A's (E4M3 = 0 is not printed, E5M2 = 1).
             f8 = [i for i in ins if i.startswith("v_mfma_f32_16x16x128_f8f6f4")]
-            assert len(f8) == 128 and count(ins, "v_mfma") == 128, name       # two unrolled K steps of 128 elements, 64 MFMAs each
+            h128 = "_h128" in name                                            # 128 x 256 tiles: half the MFMAs, one A group
+            per = 64 if h128 else 128
+            assert len(f8) == per and count(ins, "v_mfma") == per, name       # two unrolled K steps of 128 elements, 64 (32) MFMAs each
             tag = name[len("maize_gemm_"):].split("_")[0]
             a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
             assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
             body = ins[next(k for k, i in enumerate(ins) if i.startswith("v_mfma")):len(ins) - next(k for k, i in enumerate(reversed(ins)) if i.startswith("v_mfma"))]
             if "_mt256_nn" in name:
                 # row-major B: A by 128-bit reads, B by four transposing 8-byte reads per fragment
-                assert count(body, "ds_read_b128") == 32 and count(body, "ds_read_b64_tr_b8") == 64, name
+                assert count(body, "ds_read_b128") == (16 if h128 else 32) and count(body, "ds_read_b64_tr_b8") == 64, name
             else:
-                assert count(body, "ds_read_b128") == 64 and count(body, "ds_read_b64_tr_b8") == 0, name
-            assert count(body, "buffer_load_dwordx4") == 32 and count(body, "s_barrier") == 2, name
+                assert count(body, "ds_read_b128") == (48 if h128 else 64) and count(body, "ds_read_b64_tr_b8") == 0, name
+            assert count(body, "buffer_load_dwordx4") == (24 if h128 else 32) and count(body, "s_barrier") == 2, name
             assert count(body, "v_accvgpr") == 0 and count(body, "v_mov_b32") == 0, name     # accumulators and fragments stay in place
         elif "_mt128_" in name:
             # the catalogue's tf32 and f64 entries: full fp32 / fp64 matrix instructions; one K tile of 128 bytes

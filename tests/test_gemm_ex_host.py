@@ -175,19 +175,20 @@ def test_dispatch_of_8bit_operands():
         assert plan["kernel"] == name and tuple(plan["grid"]) == (256, 1, 1) and plan["workspace_bytes"] == 0
         general = ex(**big, in_type=it, alpha=2.0, beta=1.0, out_type=mz.OUT_F32)
         assert mz.gemm_plan(general)["kernel"] == name + "_gen"
+        half_tiles = (name + "_h128_gen", name + "_h128_splitk")                        # the same on tiles of 128 x 256
         for other in mz.kernel_names():
-            assert _supports(other, x) == (other in (name, name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32")), other
-            assert _supports(other, general) == (other in (name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32")), other
+            assert _supports(other, x) == (other in (name, name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32") + half_tiles), other
+            assert _supports(other, general) == (other in (name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32") + half_tiles), other
         packed = name + "_packed"
         direct = name.replace("_mt256_nt", "_mt256_nn")
         nn_plan = mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))                                              # row-major B read where it lies
         assert nn_plan["kernel"] == direct and nn_plan["workspace_bytes"] == 0 and nn_plan["reduce_grid"] == 0
         assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it, beta=1.0))["kernel"] == direct + "_gen"
         few = mz.gemm_plan(ex(64, 4096, 4096, in_type=it))                                                    # few tiles: split K
-        assert few["kernel"] == direct + "_splitk" and few["ksplit"] >= 2 and few["workspace_bytes"] == 65536 + 16 * few["ksplit"] * 262144
+        assert few["kernel"] == direct + "_h128_splitk" and few["ksplit"] >= 2 and few["workspace_bytes"] == 65536 + 16 * few["ksplit"] * 131072   # 16 tiles of 128 x 256
         for other in mz.kernel_names():
             assert _supports(other, ex(4096, 4096, 4096, in_type=it)) == (
-                other in (direct, direct + "_gen", direct + "_splitk", name + "_trb", name + "_trb_gen", packed, "maize_gemm_bf16_wave32")), other
+                other in (direct, direct + "_gen", direct + "_splitk", direct + "_h128_gen", direct + "_h128_splitk", name + "_trb", name + "_trb_gen", packed, "maize_gemm_bf16_wave32")), other
         tr_plan = mz.gemm_plan(ex(4096, 4104, 4096, in_type=it))                                              # N % 16 != 0: transposed copy of B, nothing else
         assert tr_plan["kernel"] == name + "_trb" and tr_plan["workspace_bytes"] == 65536 + 4104 * 4096 and tr_plan["reduce_grid"] == 0
         assert mz.gemm_plan(ex(4096, 4104, 4096, in_type=it, beta=1.0))["kernel"] == name + "_trb_gen"
@@ -199,14 +200,14 @@ def test_dispatch_of_8bit_operands():
         assert mz.gemm_plan(ex(100, 200, 72, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"               # too small to pay for the copies
         assert mz.gemm_plan(ex(64, 64, 64, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"
         split = mz.gemm_plan(ex(64, 64, 4096, layout=mz.LAYOUT_NT, in_type=it))              # one tile, 32 K steps of 128
-        assert split["kernel"] == name + "_splitk" and split["ksplit"] >= 2 and split["reduce_grid"] > 0
-        assert split["workspace_bytes"] == 65536 + split["ksplit"] * 256 * 256 * 4
+        assert split["kernel"] == name + "_h128_splitk" and split["ksplit"] >= 2 and split["reduce_grid"] > 0
+        assert split["workspace_bytes"] == 65536 + split["ksplit"] * 128 * 256 * 4
         skinny = name.replace("_mt256_nt", "_skinny_nt")
         assert mz.gemm_plan(ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny          # M <= 16: B streamed once
         assert mz.gemm_plan(ex(17, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m32"    # 17 .. 64 rows: row groups
         assert mz.gemm_plan(ex(64, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m64"
-        assert mz.gemm_plan(ex(64, 4096, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"     # few slabs
-        assert mz.gemm_plan(ex(65, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_splitk"
+        assert mz.gemm_plan(ex(64, 4096, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_h128_splitk"     # few slabs
+        assert mz.gemm_plan(ex(65, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_h128_splitk"
         assert _supports(skinny, ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it)) and not _supports(skinny, x)
         # the same rows against a row-major (K x N) B: the streaming kernels with transposing LDS reads (N % 16 == 0)
         few_nn = name.replace("_mt256_nt", "_skinny_nn")
@@ -214,7 +215,7 @@ def test_dispatch_of_8bit_operands():
             p = mz.gemm_plan(ex(rows, 14336, 4096, in_type=it))
             assert p["kernel"] == few_nn + suffix and tuple(p["grid"]) == (56, 4, 1) and tuple(p["block"]) == (512, 1, 1), p
             assert p["workspace_bytes"] == 65536 + 56 * 4 * tile_rows * 256 * 4, p       # one fp32 partial tile per (slab, K range)
-        assert mz.gemm_plan(ex(64, 4096, 4096, in_type=it))["kernel"] == direct + "_splitk"                       # few slabs
+        assert mz.gemm_plan(ex(64, 4096, 4096, in_type=it))["kernel"] == direct + "_h128_splitk"                  # few slabs
         assert mz.gemm_plan(ex(16, 14344, 4096, in_type=it))["kernel"] == packed                                  # N % 16 != 0: copies (the per-wave kernel would walk K = 4096 alone)
         assert mz.gemm_plan(ex(16, 14344, 264, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"                 # ... a short K: not worth the copies
         assert not _supports(few_nn, ex(16, 14344, 4096, in_type=it)) and not _supports(few_nn, ex(17, 14336, 4096, in_type=it))

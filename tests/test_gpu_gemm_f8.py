@@ -151,6 +151,8 @@ SPECIAL_FAMILIES = [
     ("mt256_nn", 300, 528, 400, mz.LAYOUT_NN),
     ("mt256_nn_gen", 257, 272, 144, mz.LAYOUT_NN),
     ("mt256_nn_splitk", 40, 272, 2064, mz.LAYOUT_NN),
+    ("mt256_nt_h128_gen", 300, 520, 400, mz.LAYOUT_NT),
+    ("mt256_nn_h128_splitk", 100, 272, 2064, mz.LAYOUT_NN),
     ("mt256_nt_trb", 300, 520, 400, mz.LAYOUT_NN),
     ("mt256_nt_packed", 257, 263, 1031, mz.LAYOUT_NN),
     ("skinny_nn", 13, 528, 2064, mz.LAYOUT_NN),
@@ -243,11 +245,12 @@ def test_macro_tile_kernel(ctx, oracle, fmt, shape):
 def test_macro_tile_kernel_all_knobs(ctx, oracle, fmt):
     m, n, k = 520, 776, 400
     name = f"maize_gemm_{fmt}_mt256_nt"
-    assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 views", lda=416, ldb=432, ldc=784) == name
+    # (named: on shapes this small the dispatcher takes the 128-row form of the same kernels, test_half_height_tiles_on_8bit_operands)
+    assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 views", lda=416, ldb=432, ldc=784, kernel=name) == name
     assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 gen by name", kernel=name + "_gen") == name + "_gen"
     for kw in (dict(alpha=0.5), dict(alpha=-1.25, beta=0.75), dict(out_f32=True), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8),
                dict(alpha=0.0, beta=1.0), dict(alpha=2.0, lda=416, ldb=432, ldc=784)):
-        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 knobs", **kw) == name + "_gen"
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="mt256f8 knobs", kernel=name + "_gen", **kw) == name + "_gen"
 
 
 @pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"])
@@ -259,14 +262,14 @@ def test_macro_tile_kernel_on_a_row_major_b(ctx, oracle, fmt):
     name = f"maize_gemm_{fmt}_mt256_nn"
     shapes = [(256, 256, 128), (256, 256, 256), (512, 768, 384), (300, 528, 144), (1000, 272, 1040), (128, 2048, 16), (520, 784, 400)]
     for (m, n, k) in shapes if fmt in ("e4m3", "e5m2") else shapes[2:4]:
-        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn") == name
+        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, kernel=name, label="mt256f8 nn") == name
     m, n, k = 520, 784, 400
-    assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn views", lda=416, ldb=800, ldc=792) == name
+    assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn views", lda=416, ldb=800, ldc=792, kernel=name) == name
     assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn gen by name", kernel=name + "_gen") == name + "_gen"
     for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(alpha=2.0, lda=416, ldb=800, ldc=792)):
-        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn knobs", **kw) == name + "_gen"
+        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="mt256f8 nn knobs", kernel=name + "_gen", **kw) == name + "_gen"
     for (m, n, k) in ((24, 528, 4096), (256, 256, 16384)):
-        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, label="f8 nn split-K") == name + "_splitk"
+        assert run_f8(ctx, oracle, m, n, k, layout=mz.LAYOUT_NN, fmt=fmt, kernel=name + "_splitk", label="f8 nn split-K") == name + "_splitk"
     assert run_f8(ctx, oracle, 40, 272, 2064, layout=mz.LAYOUT_NN, fmt=fmt, kernel=name + "_splitk", label="f8 nn split-K ragged K") == name + "_splitk"
     # the same product from the two layouts of B: same bits
     elem = ab_of(FMT[fmt][1])
@@ -274,9 +277,9 @@ def test_macro_tile_kernel_on_a_row_major_b(ctx, oracle, fmt):
     a = f8_uniform(oracle, m * k, 41, elem[0])
     b_kn = f8_uniform(oracle, k * n, 42, elem[1])
     b_nk = np.ascontiguousarray(b_kn.reshape(k, n).T).ravel()
-    c_nn, took = launch(ctx, a, b_kn, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NN, fmt, k, n, n)
+    c_nn, took = launch(ctx, a, b_kn, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NN, fmt, k, n, n, kernel=name)
     assert took == name
-    c_nt, took = launch(ctx, a, b_nk, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n)
+    c_nt, took = launch(ctx, a, b_nk, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n, kernel=f"maize_gemm_{fmt}_mt256_nt")
     assert took == f"maize_gemm_{fmt}_mt256_nt"
     assert np.array_equal(c_nn, c_nt)
     # batched, padded strides; equal to its singles and nothing written between the members
@@ -284,11 +287,12 @@ def test_macro_tile_kernel_on_a_row_major_b(ctx, oracle, fmt):
     sa, sb, sc = bm * bk + 64, bk * bn + 128, bm * bn + 16
     ab_ = f8_uniform(oracle, batch * sa, 21, elem[0])
     bb_ = f8_uniform(oracle, batch * sb, 22, elem[1])
-    dense, took = launch(ctx, ab_, bb_, np.zeros(batch * sc, np.uint16), bm, bn, bk, mz.LAYOUT_NN, fmt, bk, bn, bn, batch=batch, strides=(sa, sb, sc))
+    dense, took = launch(ctx, ab_, bb_, np.zeros(batch * sc, np.uint16), bm, bn, bk, mz.LAYOUT_NN, fmt, bk, bn, bn, batch=batch, strides=(sa, sb, sc),
+                         kernel=name)
     assert took == name
     for i in range(batch):
         single, _ = launch(ctx, ab_[i * sa:i * sa + bm * bk], bb_[i * sb:i * sb + bk * bn], np.zeros(bm * bn, np.uint16), bm, bn, bk,
-                           mz.LAYOUT_NN, fmt, bk, bn, bn)
+                           mz.LAYOUT_NN, fmt, bk, bn, bn, kernel=name)
         assert np.array_equal(single, dense[i * sc:i * sc + bm * bn]), i
         assert not dense[i * sc + bm * bn:(i + 1) * sc].any(), "wrote between batch members"
 
@@ -363,15 +367,41 @@ def test_row_major_b_full_size_and_what_lies_behind_the_view(ctx, oracle):
     da, db, dc = ctx.upload(a), ctx.upload(np.concatenate([b, pad])), ctx.upload(np.zeros(m * n, np.uint16))
     try:
         x = mz.gemm_ex_desc(mz.Matrix(da, m, k, elem_bytes=1), mz.Matrix(db, k, n, elem_bytes=1), mz.Matrix(dc, m, n), layout=mz.LAYOUT_NN, in_type=mz.IN_E4M3)
-        assert mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"] == "maize_gemm_e4m3_mt256_nn"
-        ctx.gemm_bf16(x)
-        ctx.sync()
-        got = dc.download(np.uint16)
+        assert mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"] == "maize_gemm_e4m3_mt256_nn_h128_gen"
+        ref, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, layout=mz.LAYOUT_NN, lda=k, ldb=n, elem=elem)
+        for kernel in (None, "maize_gemm_e4m3_mt256_nn", "maize_gemm_e4m3_mt256_nn_splitk", "maize_gemm_e4m3_mt256_nn_h128_splitk"):
+            dc.write(np.zeros(m * n, np.uint16))
+            ctx.gemm_bf16(x, kernel=kernel)
+            ctx.sync()
+            s = oracle.compare(dc.download(np.uint16).reshape(m, n), ref, val, scale, k, coeff=oracle.floor_coeff_f8(k))
+            assert s["n_fail"] == 0, (kernel, s)
     finally:
         da.free(); db.free(); dc.free()
-    ref, val, scale = oracle.ref_gemm_ex(a, b, m, n, k, layout=mz.LAYOUT_NN, lda=k, ldb=n, elem=elem)
-    s = oracle.compare(got.reshape(m, n), ref, val, scale, k, coeff=oracle.floor_coeff_f8(k))
-    assert s["n_fail"] == 0, s
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"])
+def test_half_height_tiles_on_8bit_operands(ctx, oracle, fmt):
+    """Tiles of 128 x 256 (general epilogue) and the same cut over K, both layouts of B, by name and as the dispatcher's
+    choice for products whose 256-row tiles fill half the chip or less; same bits as the 256-row kernels."""
+    elem = ab_of(FMT[fmt][1])
+    for layout, tag in ((mz.LAYOUT_NT, "nt"), (mz.LAYOUT_NN, "nn")):
+        gen, split = f"maize_gemm_{fmt}_mt256_{tag}_h128_gen", f"maize_gemm_{fmt}_mt256_{tag}_h128_splitk"
+        shapes = [(128, 256, 128), (256, 512, 384), (300, 528, 400), (1000, 1040, 1040), (100, 272, 2064), (512, 2048, 1024)]
+        for (m, n, k) in shapes if fmt in ("e4m3", "e5m2") else shapes[2:4]:
+            for kern in (gen, split):
+                assert run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, kernel=kern, label="h128 f8") == kern
+        bcols = 784 if layout == mz.LAYOUT_NN else 400
+        for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=792), dict(lda=416, ldb=bcols + 16, ldc=800), dict(out_f16=True)):
+            assert run_f8(ctx, oracle, 520, 784, 400, layout=layout, fmt=fmt, kernel=gen, label="h128 f8 knobs", **kw) == gen
+        assert run_f8(ctx, oracle, 512, 2048, 1024, layout=layout, fmt=fmt, label="h128 f8 auto") == gen
+        assert run_f8(ctx, oracle, 100, 2048, 8192, layout=layout, fmt=fmt, label="h128 f8 auto, cut over K") == split
+        m, n, k = 640, 784, 1168
+        a = f8_uniform(oracle, m * k, 91, elem[0])
+        b = f8_uniform(oracle, n * k, 92, elem[1])
+        ldb = k if layout == mz.LAYOUT_NT else n
+        half, _ = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, layout, fmt, k, ldb, n, kernel=gen)
+        whole, _ = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, layout, fmt, k, ldb, n, kernel=gen.replace("_h128", ""))
+        assert np.array_equal(half, whole)
 
 
 def test_dispatch_of_8bit_products(ctx):
@@ -410,32 +440,36 @@ def test_full_size_sampled_rows_and_batches(ctx, oracle, fmt):
     ab_ = f8_uniform(oracle, batch * sa, 21, elem)
     bb_ = f8_uniform(oracle, batch * sb, 22, elem)
     dense, took = launch(ctx, ab_, bb_, np.zeros(batch * sc, np.uint16), bm, bn, bk, mz.LAYOUT_NT, fmt, bk, bk, bn, batch=batch,
-                         strides=(sa, sb, sc))
+                         strides=(sa, sb, sc), kernel=f"maize_gemm_{fmt}_mt256_nt")
     assert took == f"maize_gemm_{fmt}_mt256_nt"
     for i in range(batch):
         single, _ = launch(ctx, ab_[i * sa:i * sa + bm * bk], bb_[i * sb:i * sb + bn * bk], np.zeros(bm * bn, np.uint16), bm, bn, bk,
-                           mz.LAYOUT_NT, fmt, bk, bk, bn)
+                           mz.LAYOUT_NT, fmt, bk, bk, bn, kernel=f"maize_gemm_{fmt}_mt256_nt")
         assert np.array_equal(single, dense[i * sc:i * sc + bm * bn]), i
         assert not dense[i * sc + bm * bn:(i + 1) * sc].any(), "wrote between batch members"
 
 
 @pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
 def test_split_k_on_8bit_operands(ctx, oracle, fmt):
-    """Few tiles and a long K: (tile, K range) work items + the reduce pass, as for bf16.  The dispatcher takes it by
-    itself; every epilogue goes through the reduce pass; repeated launches give the same bits."""
+    """Few tiles and a long K: (tile, K range) work items + the reduce pass, as for bf16, on tiles of 256 x 256 (by name)
+    and of 128 x 256 (what the dispatcher takes by itself for these shapes); every epilogue goes through the reduce pass;
+    repeated launches give the same bits."""
     name = f"maize_gemm_{fmt}_mt256_nt_splitk"
+    half_tiles = f"maize_gemm_{fmt}_mt256_nt_h128_splitk"
     for (m, n, k) in ((24, 520, 4096), (64, 512, 8192), (256, 256, 16384)):        # more than 16 rows and few columns: not the streaming kernels'
-        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="f8 split-K") == name
-    assert run_f8(ctx, oracle, 40, 264, 2064, fmt=fmt, kernel=name, label="f8 split-K ragged K") == name
-    assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, alpha=-1.25, beta=0.75, label="f8 split-K scaled") == name
-    assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, out_f32=True, ldc=520, label="f8 split-K f32") == name
-    assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, kernel=name, label="f8 split-K by name") == name     # a shape it would not split
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="f8 split-K") == half_tiles
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, kernel=name, label="f8 split-K, 256-row tiles") == name
+    for kern in (name, half_tiles):
+        assert run_f8(ctx, oracle, 40, 264, 2064, fmt=fmt, kernel=kern, label="f8 split-K ragged K") == kern
+        assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, alpha=-1.25, beta=0.75, kernel=kern, label="f8 split-K scaled") == kern
+        assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, out_f32=True, ldc=520, kernel=kern, label="f8 split-K f32") == kern
+        assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, kernel=kern, label="f8 split-K by name") == kern     # a shape it would not split
     elem = FMT[fmt][1]
     m, n, k = 24, 520, 4096
     a = f8_uniform(oracle, m * k, 31, elem)
     b = f8_uniform(oracle, n * k, 32, elem)
     first, took = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n)
-    assert took == name
+    assert took == half_tiles
     for _ in range(3):
         again, _ = launch(ctx, a, b, np.full(m * n, 0x7FC0, np.uint16), m, n, k, mz.LAYOUT_NT, fmt, k, k, n)
         assert np.array_equal(again, first)
@@ -463,9 +497,11 @@ def test_operands_of_different_8bit_formats(ctx, oracle, fmt):
     for layout in (mz.LAYOUT_NN, mz.LAYOUT_NT):
         assert run_f8(ctx, oracle, 100, 200, 72, layout=layout, fmt=fmt, kernel="maize_gemm_bf16_wave32", label="wave32 mixed") == "maize_gemm_bf16_wave32"
     name = f"maize_gemm_{fmt}_mt256_nt"
-    assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, label="mixed plain") == name
-    assert run_f8(ctx, oracle, 300, 520, 144, fmt=fmt, alpha=-1.25, beta=0.75, label="mixed gen") == name + "_gen"
-    assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, label="mixed split-K") == name + "_splitk"
+    assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, kernel=name, label="mixed plain") == name
+    assert run_f8(ctx, oracle, 300, 520, 144, fmt=fmt, alpha=-1.25, beta=0.75, kernel=name + "_gen", label="mixed gen") == name + "_gen"
+    assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, kernel=name + "_splitk", label="mixed split-K") == name + "_splitk"
+    assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, label="mixed, 128-row tiles") == name + "_h128_gen"      # what the dispatcher takes for these
+    assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, label="mixed split-K, 128-row tiles") == name + "_h128_splitk"
     m = n = k = 256
     a = f8_uniform(oracle, m * k, 41, 2)
     b = f8_uniform(oracle, n * k, 42, 2)
@@ -517,8 +553,9 @@ def test_packed_path_for_8bit_operands(ctx, oracle, fmt):
 @pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2"])
 @pytest.mark.parametrize("case", [
     # (M, N, K, layout, leading dimensions or None, alpha, beta, kernel family expected in the name)
-    (512, 768, 384, mz.LAYOUT_NT, None, 1.0, 0.0, "mt256_nt_gen"),
-    (300, 520, 144, mz.LAYOUT_NT, (160, 176, 528), -0.75, 0.5, "mt256_nt_gen"),
+    (512, 768, 384, mz.LAYOUT_NT, None, 1.0, 0.0, "mt256_nt_h128_gen"),
+    (300, 520, 144, mz.LAYOUT_NT, (160, 176, 528), -0.75, 0.5, "mt256_nt_h128_gen"),
+    (2048, 4352, 256, mz.LAYOUT_NT, None, 1.0, 0.0, "mt256_nt_gen"),
     (256, 512, 8192, mz.LAYOUT_NT, None, 1.0, 0.0, "splitk"),
     (16, 2048, 1024, mz.LAYOUT_NT, None, 2.0, 1.0, "skinny_nt"),
     (200, 264, 400, mz.LAYOUT_NN, None, 1.0, 0.0, ""),

@@ -30,9 +30,10 @@ class Hazard(AssertionError):
 
 # how the K step numbers its MFMA slots and places the requests (16 pieces per wave and K tile with 256-row tiles, 12
 # with 128-row tiles; AFTER = the slots of a step behind its barrier: 32, or 16 with 128-row tiles)
-MT256_SLOT_FACTS = ("constexpr int DS = IS8 ? 2 : H128 ? 3 : DMA_STRIDE;", "constexpr int AFTER = 16 * (NE - EB);",
+MT256_SLOT_FACTS = ("constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : DMA_STRIDE;", "constexpr int AFTER = 16 * (NE - EB);",
                     "constexpr int NP = PA + 8;", "constexpr int PA = BMT / 32;",
-                    "constexpr int NE = (IS8 || H128) ? 4 : 8;", "constexpr int EB = IS8 ? 2 : H128 ? 3 : 6;",
+                    "constexpr int NE = (IS8 && H128) ? 2 : (IS8 || H128) ? 4 : 8;",
+                    "constexpr int EB = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : 6;",
                     "const int slot = e >= EB ? 16 * (e - EB) + s : AFTER + 16 * e + s;",
                     "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < NP) {",
                     "if (DS * pc + 2 < AFTER) dma(pc, A1, B1, k_begin + BKE);",       # early pieces: those behind the barrier of step t itself
@@ -232,9 +233,9 @@ def test_macro_tile_checker_rejects_broken_schedules():
 # wave and K tile, one every three MFMA slots
 # ---------------------------------------------------------------------------------------
 
-H128_READ_LINES = ("if (h4 == 0 && r < NBR) read_b(1, kh, cur, r);",
+H128_READ_LINES = ("if (h4 == 0 && rb < NBR) read_b(1, kh, cur, rb);",
                    "if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
-                   "if (h4 == 1 && r < NBR) { if (!last_half) read_b(0, 1, cur, r); else read_b(0, 0, cur ^ 1, r); }",
+                   "if (h4 == 1 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }",
                    "const int kh = IS8 ? 0 : H128 ? e >> 1 : e >> 2, h4 = H128 ? e & 1 : e & 3;",
                    "const int buf = H128 ? bi : bi ^ (IS8 ? st : kh);",
                    "else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * 16 + r);")
@@ -298,6 +299,63 @@ def test_half_height_tile_checker_rejects_broken_schedules():
         check_two_stage(*h128_wave_program(8, True, ds=6), need, parts=4, pieces=12)
     with pytest.raises(Hazard):                 # a fragment read dropped: MFMAs on stale registers
         check_two_stage(*h128_wave_program(8, True, drop_read=30), need, parts=4, pieces=12)
+
+
+# ---------------------------------------------------------------------------------------
+# 128 x 256 tiles on 8-bit operands: a K tile is one matrix instruction deep, so a K step is the pair (A0, B0), (A0, B1)
+# with the barrier between the two; the second eighth reads the next tile's A0 (8 reads) and B0 (8, or 16 transposing
+# ones, two per slot); 12 pieces per wave and K tile, one per MFMA slot behind the barrier
+# ---------------------------------------------------------------------------------------
+
+def h128_f8_wave_program(nk, tr, barrier_at=1, ds=1):
+    src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
+    for fact in MT256_SLOT_FACTS + H128_READ_LINES + ("if (IS8 && H128) lds_read128(fa8[st & 1][r >> 1][r & 1], a_rd[r & 1], st * 16 + (r >> 1));",):
+        assert fact in src, fact
+    nbr, per_slot = (16, 2) if tr else (8, 1)
+    slots = [ds * pc + 2 for pc in range(12)]
+    ops = [("dma", 0, pc, 0) for pc in range(12)]
+    ops += [("wait_all",), ("barrier",)]
+    ops += [("read", 0, 0, 0)] * (8 + nbr)
+    ops += [("dma", 1, pc, 1) for pc in range(12) if slots[pc] < 16]
+    k_early, k_late = 2, 1
+    steps = nk + (nk & 1)
+    for t in range(steps):
+        cur, nxt = t & 1, (t & 1) ^ 1
+        for e in range(2):
+            if e == barrier_at:
+                ops += [("wait_all",), ("barrier",)]
+            for sl in range(16):
+                ops.append(("mfma", t, e))
+                if e == 0:                                   # B group 1 of this tile
+                    ops += [("read", t, 1, cur)] * (per_slot if sl * per_slot < nbr else 0)
+                else:                                        # A group 0 and B group 0 of the next tile
+                    ops += [("read", t + 1, 0, nxt)] * ((1 if sl < 8 else 0) + (per_slot if sl * per_slot < nbr else 0))
+                slot = sl if e == 1 else 16 + sl
+                for pc in range(12):
+                    if slots[pc] == slot:
+                        ops.append(("dma", k_early, pc, cur) if e == 1 else ("dma", k_late, pc, nxt))
+        k_early += 1
+        k_late += 1
+    ops.append(("wait_all",))
+    return ops, steps
+
+
+@pytest.mark.parametrize("tr", [False, True])
+@pytest.mark.parametrize("nk", [1, 2, 3, 7, 32])
+def test_8bit_half_height_tile_schedule_is_hazard_free(nk, tr):
+    nbr = 16 if tr else 8
+    ops, steps = h128_f8_wave_program(nk, tr)
+    last_tile = check_two_stage(ops, steps, [8 + nbr, 8 + 2 * nbr], parts=2, pieces=12)
+    assert steps <= last_tile <= steps + 1
+
+
+def test_8bit_half_height_tile_checker_rejects_broken_schedules():
+    with pytest.raises(Hazard):                 # no barrier between the two eighths: the next tile is read before it is known to be complete
+        check_two_stage(*h128_f8_wave_program(8, False, barrier_at=2), [16, 24], parts=2, pieces=12)
+    with pytest.raises(Hazard):                 # barrier in front of the first eighth: the stage is refilled while B group 1 is still being read
+        check_two_stage(*h128_f8_wave_program(8, False, barrier_at=0), [16, 24], parts=2, pieces=12)
+    with pytest.raises(Hazard):                 # requests three slots apart: the last ones would never be issued
+        check_two_stage(*h128_f8_wave_program(8, False, ds=3), [16, 24], parts=2, pieces=12)
 
 
 # ---------------------------------------------------------------------------------------
