@@ -374,6 +374,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     //   held across the change of K half keeps its buffer, the other one is free for the new half).
     // 8-bit operands: no K halves; the B buffer alternates with the ring stage instead (the group held across the
     // change of K tile keeps its buffer), and a fragment is two 16-byte halves.
+    // 128-row tiles: a wave holds one A group (64 rows), so a K half is two eighths, (0,0) and (0,1); B group bi lives in
+    // buffer bi, the A group in the buffer of its K half (8-bit: of its K tile), and each eighth reads one B group and,
+    // in the second, the next A group.
     bf16x8 fa[2][4];
     bf16x8 fb[2][4];
     short4v fbl[2][4], fbh[2][4];
