@@ -262,6 +262,16 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
 // half tiles costs 0.63 of a round of whole ones, 4096^3 89 -> 112 us, 2048 x 11008 x 4096 152 -> 162).
 // With few of them and a long K the 128-row tiles are cut over K too (same cost terms as above with 0.67 per K step: a
 // single row of tiles, 65 .. 128 rows of A, does half the matrix work of 256-row tiles).
+// Whole K in 128-row tiles: from 28 K steps of 16-bit operands on, the kernels with three ring stages (below that their
+// longer start and the step count rounded up to a multiple of three cost more than the two-stage loop's waits:
+// 512 x 8192 x 1024 14.5 us with two stages, 15.8 with three; 512 x 2048 x 1536 17.5 / 18.0) -- provided enough compute
+// units pull on the memory system for those waits to exist (32 tiles, 512 x 2048 x 1792: 19.7 us with two stages, 21.2
+// with three, 0.55 us per step either way; 112 to 224 tiles: 0.70 against 0.52 per step) or K is long enough for the
+// rounding not to matter.
+bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles) {
+    const uint32_t nk = cdiv(k, 64u);
+    return kstep == 64u && nk >= 28u && (nk >= 48u || half_tiles >= 48u);
+}
 // Returns 0: the 256-row kernels; 1: 128-row tiles, whole K; >= 2: 128-row tiles in that many K ranges.
 uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
     const uint32_t resident = cus >= 8u ? cus - cus % 8u : cus;
@@ -273,7 +283,9 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     // per K step: 0.67 of the 256-row kernel's; an 8-bit step (128 deep) takes 1.3 of a 16-bit one, which the fixed terms
     // here (in 16-bit steps) have to be weighed against (E4M3 128 x 14336 x 4096: 31.1 us whole, 25.8 in two ranges)
     const double step = kstep == 128u ? 0.87 : 0.67;
-    const double whole = 8.0 + step * nk;
+    // 16-bit operands and a long K: the three-stage kernels, 0.52 per step, steps in threes (2048^3 28.6 -> 24.9 us,
+    // 1024 x 4096 x 4096 51.1 -> 42.0, 640 x 8192 x 4096 N x K 60.4 -> 45.9)
+    const double whole = h128_three_stages(s.k, kstep, half_tiles) ? 8.0 + 0.52 * 3.0 * cdiv(nk, 3u) : 8.0 + step * nk;
     double best = 0.9 * whole;                                     // splitting has to win 10 %
     uint32_t best_ks = 1;
     const double elems = (double)s.m * s.n * batch;
@@ -785,6 +797,12 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_h128_gen", nullptr, mt256_nt_ktail_gen_supports, mt256_h128_plan},
     {"maize_gemm_f16_mt256_nn_h128_gen", nullptr, f16_nn_ktail_gen_supports, mt256_h128_plan},
     {"maize_gemm_f16_mt256_nt_h128_gen", nullptr, f16_nt_ktail_gen_supports, mt256_h128_plan},
+    {"maize_gemm_bf16_mt256_nn_h128r3", nullptr, mt256_nn_supports, mt256_h128_plan},
+    {"maize_gemm_bf16_mt256_nt_h128r3", nullptr, mt256_nt_supports, mt256_h128_plan},
+    {"maize_gemm_bf16_mt256_nn_h128r3_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_h128_plan},
+    {"maize_gemm_bf16_mt256_nt_h128r3_gen", nullptr, mt256_nt_ktail_gen_supports, mt256_h128_plan},
+    {"maize_gemm_f16_mt256_nn_h128r3_gen", nullptr, f16_nn_ktail_gen_supports, mt256_h128_plan},
+    {"maize_gemm_f16_mt256_nt_h128r3_gen", nullptr, f16_nt_ktail_gen_supports, mt256_h128_plan},
     {"maize_gemm_bf16_mt256_nn_h128_splitk", nullptr, splitk_nn_supports, h128_splitk_plan},
     {"maize_gemm_bf16_mt256_nt_h128_splitk", nullptr, splitk_nt_supports, h128_splitk_plan},
     {"maize_gemm_f16_mt256_nn_h128_splitk", nullptr, splitk_f16_nn_supports, h128_splitk_plan},
@@ -982,10 +1000,14 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         if (hs >= 0 && kKernels[hs].supports(d) && plan_fits(kKernels[hs], d, compute_units)) return (uint32_t)hs;
     }
     if (hk == 1u) {
-        static const char* const kH128[2] = {"maize_gemm_bf16_mt256_nn_h128", "maize_gemm_bf16_mt256_nt_h128"};
-        static const char* const kH128Gen[2][2] = {{"maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_bf16_mt256_nt_h128_gen"},
-                                                   {"maize_gemm_f16_mt256_nn_h128_gen", "maize_gemm_f16_mt256_nt_h128_gen"}};
-        const int hp = kernel_index(kH128[s.nt]), hg = kernel_index(kH128Gen[half_in(d)][s.nt]);
+        static const char* const kH128[2][2] = {{"maize_gemm_bf16_mt256_nn_h128", "maize_gemm_bf16_mt256_nt_h128"},
+                                                {"maize_gemm_bf16_mt256_nn_h128r3", "maize_gemm_bf16_mt256_nt_h128r3"}};
+        static const char* const kH128Gen[2][2][2] = {{{"maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_bf16_mt256_nt_h128_gen"},
+                                                       {"maize_gemm_f16_mt256_nn_h128_gen", "maize_gemm_f16_mt256_nt_h128_gen"}},
+                                                      {{"maize_gemm_bf16_mt256_nn_h128r3_gen", "maize_gemm_bf16_mt256_nt_h128r3_gen"},
+                                                       {"maize_gemm_f16_mt256_nn_h128r3_gen", "maize_gemm_f16_mt256_nt_h128r3_gen"}}};
+        const int r3 = h128_three_stages(s.k, 64u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch);
+        const int hp = kernel_index(kH128[r3][s.nt]), hg = kernel_index(kH128Gen[r3][half_in(d)][s.nt]);
         if (hp >= 0 && !half_in(d) && kKernels[hp].supports(d)) return (uint32_t)hp;
         if (hg >= 0 && kKernels[hg].supports(d)) return (uint32_t)hg;
     }

@@ -138,11 +138,22 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 // the last eighth; 12 pieces per wave and K tile, one every three MFMA slots.  8-bit operands: a K tile is one matrix
 // instruction deep, so the step is just the pair (A0, B0), (A0, B1) with the barrier between the two, A's buffers
 // alternate with the K tile, and the 12 pieces go out one every two (twice as long) MFMA slots.
-template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256>
+// NST = 3 (128-row tiles of 16-bit operands): three ring stages -- 3 x 16 KiB of A, 3 x 32 KiB of B, 16 KiB of epilogue
+// staging (passes of 16 rows) -- so that a K tile is requested two steps before it is read.  Behind the barrier of step t
+// go the early pieces of tile t+3, into the stage step t has just read; before the barrier of step t+1 its late pieces;
+// it is read from the last eighth of step t+2 on.  The wait in front of the barrier of step t is `vmcnt(12)`: tile t+1
+// has landed, the twelve requests of tile t+2 -- younger -- stay in flight.  Three steps per trip, the step count rounded
+// up to a multiple of three with all-zero tiles.  B's third stage lies 64 KiB behind the first, past the reads' 16-bit
+// offset field, and has base registers of its own.
+template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
     constexpr bool H128 = BMT == 128;
     static_assert(BMT == 256 || (H128 && !EDGE), "128-row tiles: no edge splitting");
+    constexpr bool R3 = NST == 3;                       // three ring stages (128-row tiles of 16-bit operands)
+    static_assert(NST == 2 || (R3 && H128 && F8 < 0), "three ring stages: 128-row tiles of 16-bit operands only");
+    constexpr int ASTR = R3 ? TILE / 2 : TILE;          // bytes from one stage of A to the next
+    constexpr int EPR = R3 ? 1 : 2;                     // accumulator rows per epilogue pass (the staging region is 4 or 8 KiB per wave)
     constexpr int MI = BMT / 32;                        // accumulator rows of a wave (16 rows each)
     constexpr int PA = BMT / 32;                        // 1 KiB pieces of A per wave and K tile (8 rows each, 4 waves)
     constexpr uint32_t WROWS = BMT / 2;                 // rows of the tile per wave row
@@ -158,16 +169,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : DMA_STRIDE;
     constexpr int AFTER = 16 * (NE - EB);               // MFMA slots of a step behind its barrier
     constexpr int NP = PA + 8;                          // pieces per wave and K tile
+    static_assert(!R3 || NP == 12, "the counted waits of the three-stage ring assume twelve pieces per K tile");
     // One array per operand, two ring stages each.  The fragment reads below are inline assembly (one
     // base register per operand and K half, the stage and the fragment in the 16-bit offset field), so
     // the compiler sees no read of these arrays and never makes one wait for the direct-to-LDS loads
     // that are in flight; the waits are placed by hand.
-    __shared__ __attribute__((aligned(1024))) char lds_a[2 * TILE];
-    __shared__ __attribute__((aligned(1024))) char lds_b[2 * TILE];
+    __shared__ __attribute__((aligned(1024))) char lds_a[NST * ASTR];
+    __shared__ __attribute__((aligned(1024))) char lds_b[NST * TILE];
     // Epilogue staging (8 KiB per wave), apart from the operand stages so that the first K tile
     // of the workgroup's next C tile can land while this one is converted and stored.
-    __shared__ __attribute__((aligned(1024))) char lds_e[TILE];
-    lds_ptr const A0 = (lds_ptr)lds_a, A1 = A0 + TILE, B0 = (lds_ptr)lds_b, B1 = B0 + TILE;
+    __shared__ __attribute__((aligned(1024))) char lds_e[R3 ? TILE / 2 : TILE];
+    lds_ptr const A0 = (lds_ptr)lds_a, A1 = A0 + ASTR, B0 = (lds_ptr)lds_b, B1 = B0 + TILE;
 
     const uint32_t M = p.crows, N = p.ccols, K = p.acols;
     const uint32_t lda = lda_of(p), ldb = ldb_of(p), ldc = ldc_of(p);
@@ -364,6 +376,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int j = 0; j < 8; ++j)
             b_rd[j] = (uint32_t)(uintptr_t)B0 + (TR8 ? maps::sk8_tr_offset(wn * 8u + j, 0, 0, lane) : maps::sk_tr_offset(wn * 8u + j, 0, lane));
     }
+    // B's third stage starts 64 KiB behind the first, out of reach of the reads' 16-bit offset field: second base registers.
+    uint32_t b_rd2[8];
+    if (R3) {
+#pragma unroll
+        for (int j = 0; j < (NT ? 2 : 8); ++j) b_rd2[j] = b_rd[j] + 2u * TILE;
+    }
 
     // Fragment registers.  A K half (32 deep) of the wave's sub-tile is walked in four eighths of 16 MFMAs
     // each: (A group, B group) = (0,0), (0,1), (1,1), (1,0), a group being 4 fragments (64 rows or columns).
@@ -397,6 +415,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     auto lds_read128 = [&](auto& dst, uint32_t base, int n) {
         switch (n) {
             MAIZE_RD_CASE(0) MAIZE_RD_CASE(1) MAIZE_RD_CASE(2) MAIZE_RD_CASE(3) MAIZE_RD_CASE(4) MAIZE_RD_CASE(5) MAIZE_RD_CASE(6) MAIZE_RD_CASE(7)
+            MAIZE_RD_CASE(8) MAIZE_RD_CASE(9) MAIZE_RD_CASE(10) MAIZE_RD_CASE(11)
             MAIZE_RD_CASE(16) MAIZE_RD_CASE(17) MAIZE_RD_CASE(18) MAIZE_RD_CASE(19) MAIZE_RD_CASE(20) MAIZE_RD_CASE(21) MAIZE_RD_CASE(22) MAIZE_RD_CASE(23)
             default: __builtin_unreachable();
         }
@@ -422,19 +441,21 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     auto read_a = [&](int ai, int kh, int st, int r) {
         if (IS8 && H128) lds_read128(fa8[st & 1][r >> 1][r & 1], a_rd[r & 1], st * 16 + (r >> 1));   // one A group; the buffer alternates with the K tile
         else if (IS8) lds_read128(fa8[ai][r >> 1][r & 1], a_rd[r & 1], st * 16 + 4 * ai + (r >> 1));   // half r & 1 = the 16-bit kernel's kh
-        else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * 16 + r);                             // one A group; the buffer alternates with the K half
+        else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * (ASTR / 2048) + r);                            // one A group; the buffer alternates with the K half
         else     lds_read128(fa[ai][r], a_rd[kh], st * 16 + 4 * ai + r);
     };
     // Read r (0..NBR-1) of B group bi, K half kh, of the tile in stage st.
     auto read_b = [&](int bi, int kh, int st, int r) {
         const int buf = H128 ? bi : bi ^ (IS8 ? st : kh);
+        const bool far = R3 && st == 2;                       // third stage: from the second base register
+        const int so = far ? 0 : st * 16;
         if (TR8) lds_read_tr8(fb8t[buf][r >> 2][r & 3], b_rd[4 * bi + (r >> 2)], st * 16 + ((r >> 1) & 1) * 8 + (r & 1));
         else if (IS8) lds_read128(fb8[buf][r >> 1][r & 1], b_rd[r & 1], st * 16 + 4 * bi + (r >> 1));
-        else if (NT) lds_read128(fb[buf][r], b_rd[kh], st * 16 + 4 * bi + r);
+        else if (NT) lds_read128(fb[buf][r], far ? b_rd2[kh] : b_rd[kh], so + 4 * bi + r);
         else {
             const int c = r >> 1, h = r & 1;                  // rows 32 kh + 4 h + ...: 16 KiB and 2 KiB further on
-            if (h == 0) lds_read_tr(fbl[buf][c], b_rd[4 * bi + c], st * 16 + kh * 8);
-            else        lds_read_tr(fbh[buf][c], b_rd[4 * bi + c], st * 16 + kh * 8 + 1);
+            if (h == 0) lds_read_tr(fbl[buf][c], far ? b_rd2[4 * bi + c] : b_rd[4 * bi + c], so + kh * 8);
+            else        lds_read_tr(fbh[buf][c], far ? b_rd2[4 * bi + c] : b_rd[4 * bi + c], so + kh * 8 + 1);
         }
     };
     auto b_operand = [&](int buf, int c) -> bf16x8 {
@@ -463,7 +484,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // One K step = 8 eighths.  On entry: (ca, cb) hold tile t, fa[0] and B buffer 0 hold its first groups,
     // the early pieces of tile t+1 are landing in (na, nb).
     auto step = [&](int cur) {
-        lds_ptr const ca = A0 + cur * TILE, cb = B0 + cur * TILE, na = A0 + (cur ^ 1) * TILE, nb = B0 + (cur ^ 1) * TILE;
+        // Two stages: tile t+1 is in the other stage, and so go its late pieces.  Three stages: tile t+1 is in the next
+        // stage, complete since the step before; the late pieces issued here are tile t+2's, into the stage after that
+        // one, and the early pieces behind the barrier are tile t+3's, into the stage this step has just read.
+        const int nxt = R3 ? (cur + 1) % 3 : cur ^ 1, lat = R3 ? (cur + 2) % 3 : cur ^ 1;
+        lds_ptr const ca = A0 + cur * ASTR, cb = B0 + cur * TILE, na = A0 + lat * ASTR, nb = B0 + lat * TILE, pb = B0 + nxt * TILE;
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
             const int kh = IS8 ? 0 : H128 ? e >> 1 : e >> 2, h4 = H128 ? e & 1 : e & 3;
@@ -476,9 +501,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // this wave's share of tile t+1 has landed, then meet the other waves: after the
                 // barrier (na, nb) is complete and (ca, cb) is free to be refilled with tile t+2.
                 MAIZE_FENCE();
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                if (PATCHES && patch_on && K - 1u - k_late < (uint32_t)BKE)    // tile t+1 holds row K - 1 (k_late <= K - 1 here)
-                    asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)nb + patch_off), "v"(patch_val) : "memory");
+                // (three stages: the twelve requests of tile t+2 are younger and may still be out)
+                if (R3) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                else    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                const uint32_t k_next = R3 ? k_late - (uint32_t)BKE : k_late;  // where tile t+1 starts
+                if (PATCHES && patch_on && K - 1u - k_next < (uint32_t)BKE)    // tile t+1 holds row K - 1 (k_next <= K - 1 here)
+                    asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)pb + patch_off), "v"(patch_val) : "memory");
                 MAIZE_FENCE();
             }
 #pragma unroll
@@ -506,9 +534,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #pragma unroll
                     for (int rb = r * RPS; rb < (r + 1) * RPS; ++rb) {
                         if (h4 == 0 && rb < NBR) read_b(1, kh, cur, rb);
-                        if (h4 == 1 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }
+                        if (h4 == 1 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, nxt, rb); }
                     }
-                    if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }
+                    if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, nxt, r); }
                 } else if (s % RSTRIDE == 0) {
                     const int r = s / RSTRIDE;
 #pragma unroll
@@ -536,6 +564,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // ---- prime: the first K tile of the first C tile, whole ------------------------------
 #pragma unroll
     for (int pc = 0; pc < NP; ++pc) dma(pc, A0, B0, k_begin);
+    if (R3) {                                                   // three stages: the second one too
+#pragma unroll
+        for (int pc = 0; pc < NP; ++pc) dma(pc, A1, B1, k_begin + BKE);
+    }
 
     for (;;) {                                                  // one trip per C tile
 #pragma unroll
@@ -552,14 +584,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     for (int r = 0; r < NBR; ++r) read_b(0, 0, 0, r);
 #pragma unroll
     for (int pc = 0; pc < NP; ++pc)
-        if (DS * pc + 2 < AFTER) dma(pc, A1, B1, k_begin + BKE);   // tile 1, early pieces
-    k_early = k_begin + 2 * BKE;
-    k_late = k_begin + BKE;
-    // Two steps per trip so that each step sees its stages as compile-time constants.  An odd
-    // step count runs one extra step on an all-zero tile (loads past K return zeros).
-    for (uint32_t kt = 0; kt < nk; kt += 2) {
+        if (DS * pc + 2 < AFTER) dma(pc, A0 + (NST - 1) * ASTR, B0 + (NST - 1) * TILE, k_begin + (NST - 1) * BKE);   // tile 1 (three stages: 2), early pieces
+    k_early = k_begin + NST * BKE;
+    k_late = k_begin + (NST - 1) * BKE;
+    // Two (three) steps per trip so that each step sees its stages as compile-time constants.  A step count that
+    // is not a multiple runs the extra steps on all-zero tiles (loads past K return zeros).  (Leaving the trip after
+    // the step that was the last costs more than it saves: with exits between the steps the register allocator no
+    // longer keeps the loop's operands in place.)
+    for (uint32_t kt = 0; kt < nk; kt += NST) {
         step(0);
         step(1);
+        if (R3) step(2);
     }
     // every direct-to-LDS write of this tile has landed; the last MFMAs have left the pipe before the
     // epilogue reads their accumulators (the assembler-level MFMAs are invisible to the hazard recognizer)
@@ -613,6 +648,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         select_tile(next);
 #pragma unroll
         for (int pc = 0; pc < NP; ++pc) dma(pc, A0, B0, k_begin);
+        if (R3) {
+#pragma unroll
+            for (int pc = 0; pc < NP; ++pc) dma(pc, A1, B1, k_begin + BKE);
+        }
     }
 
     // ---- epilogue: fp32 -> bf16 (RNE), stage through LDS, 128-bit row stores --------------
@@ -624,7 +663,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // General epilogue (alpha, beta, fp32 C): the sub-tile is staged as fp32, 32 rows x 64 columns
         // at a time (row = 256 B, 16-byte chunk index XOR-ed with row%16), read back as runs of 8
         // consecutive columns of a row and finished by store_c_run.
-        lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
+        lds_ptr ew = (lds_ptr)lds_e + wave_u * (R3 ? 4096u : 8192u);
         const uint32_t c8 = lane & 7u, r8 = lane >> 3;           // 8 lanes per 64-column row, 8 rows per read
         // Split-K: the lane's place inside the partial tile.  Recomputed per tile on purpose (the empty
         // asm makes it opaque): hoisted out of the tile loop, the 32 addresses derived from it would
@@ -633,29 +672,29 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         asm volatile("" : "+v"(lane_part));
         float* const part_base = (float*)((char*)p.workspace + 65536) + (uint64_t)eslot * (BMT * BN) + lane_part;
 #pragma unroll
-        for (int i = 0; i < MI / 2; ++i)                         // 32 rows per pass: accumulator rows 2i, 2i+1
+        for (int i = 0; i < MI / EPR; ++i)                       // 32 rows per pass: accumulator rows 2i, 2i+1 (three stages: 16 rows, row i)
 #pragma unroll
             for (int jh = 0; jh < 2; ++jh) {
 #pragma unroll
-                for (int ii = 0; ii < 2; ++ii)
+                for (int ii = 0; ii < EPR; ++ii)
 #pragma unroll
                     for (int jj = 0; jj < 4; ++jj)
                         // lane holds C[row = (2i+ii)*16 + l16][col = (4jh+jj)*16 + 4*lg + 0..3]
-                        *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_write_offset(ii, jj, lane)) = acc[2 * i + ii][4 * jh + jj];
+                        *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_write_offset(ii, jj, lane)) = acc[EPR * i + ii][4 * jh + jj];
                 const uint32_t gcol = en0 + wn * 128u + jh * 64u + c8 * 8u;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
+                for (int r = 0; r < 2 * EPR; ++r) {
                     const uint32_t row = maps::epi32_read_row(r, lane);     // 0..31 within the pass
                     const floatx4 lo = *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_read_offset(r, 0, lane));
                     const floatx4 hi = *(__attribute__((address_space(3))) floatx4*)(ew + maps::epi32_read_offset(r, 1, lane));
-                    const uint32_t grow = em0 + wm * WROWS + i * 32u + row;
+                    const uint32_t grow = em0 + wm * WROWS + i * (16u * EPR) + row;
                     if (gcol < N && grow < M) {                   // direct C: N % 8 == 0, a run is all in or all out
                         if (SPLITK) {
                             // fp32 partial tile of this (tile, K range), row-major 256 x 256, behind the 64 KiB
                             // of ticket counters every workspace starts with (other kernels on the stream rely
                             // on finding them zero); the reduce kernel adds the ranges in order and applies
                             // the epilogue.
-                            float* part = part_base + (uint32_t)((i * 32 + r * 8) * BN + jh * 64);
+                            float* part = part_base + (uint32_t)((i * 16 * EPR + r * 8) * BN + jh * 64);
                             *(floatx4*)part = lo;
                             *(floatx4*)(part + 4) = hi;
                         } else {
@@ -698,7 +737,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
         }
     } else if (finish) {                                         // (a K range that was not the last to arrive stores nothing)
-        lds_ptr ew = (lds_ptr)lds_e + wave_u * 8192u;
+        lds_ptr ew = (lds_ptr)lds_e + wave_u * (R3 ? 4096u : 8192u);
         const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per read
         const uint32_t gcol = en0 + wn * 128u + cc * 8u;
         // Stores go through a buffer descriptor over this batch member's C: rows at or past M fall
@@ -710,20 +749,20 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const uint32_t c_vo = (((wm * WROWS + cr) * ldc + gcol) * 2u) | (gcol < N ? 0u : OOB);
         const uint32_t row_bytes = __builtin_amdgcn_readfirstlane(ldc * 2u);
     #pragma unroll
-        for (int i = 0; i < MI / 2; ++i) {
+        for (int i = 0; i < MI / EPR; ++i) {
     #pragma unroll
-            for (int ii = 0; ii < 2; ++ii)                       // 32 rows per pass: accumulator rows 2i, 2i+1
+            for (int ii = 0; ii < EPR; ++ii)                     // 32 rows per pass: accumulator rows 2i, 2i+1 (three stages: 16 rows, row i)
     #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     // lane holds C[row = (2i+ii)*16 + l16][col = j*16 + 4*lg + 0..3]
-                    floatx4 f = acc[2 * i + ii][j];
+                    floatx4 f = acc[EPR * i + ii][j];
                     u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
                     *(lds_v2)(ew + maps::epi16_write_offset(ii, j, lane)) = v;
                 }
     #pragma unroll
-            for (int r = 0; r < 8; ++r) {
+            for (int r = 0; r < 4 * EPR; ++r) {
                 const u32x4 v = *(lds_v4)(ew + maps::epi16_read_offset(r, lane));
-                __builtin_amdgcn_raw_buffer_store_b128(v, rc, c_vo, (uint32_t)(i * 32 + r * 4) * row_bytes, 2 /* nt */);
+                __builtin_amdgcn_raw_buffer_store_b128(v, rc, c_vo, (uint32_t)(i * 16 * EPR + r * 4) * row_bytes, 2 /* nt */);
             }
         }
     }
@@ -761,6 +800,15 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128_
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, -1, 128>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nn_h128_gen(GemmArgs p) { mt256::body<false, true, false, true, true, false, -1, 128>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nt_h128_gen(GemmArgs p) { mt256::body<true, true, false, true, true, false, -1, 128>(p); }
+// ... with three ring stages (K tiles t+1 and t+2 on their way while t is multiplied): for a long K, where the two-stage
+// loop waits for its loads (2048^3 28.6 -> 24.9 us, 1024 x 4096 x 4096 51.1 -> 42.0; from 28 K steps on -- below, the two
+// K tiles in front and the step count rounded up to a multiple of three cost more than the waits).
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128r3(GemmArgs p) { mt256::body<false, false, false, false, false, false, -1, 128, 3>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128r3(GemmArgs p) { mt256::body<true, false, false, false, false, false, -1, 128, 3>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128r3_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, -1, 128, 3>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128r3_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, -1, 128, 3>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nn_h128r3_gen(GemmArgs p) { mt256::body<false, true, false, true, true, false, -1, 128, 3>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nt_h128r3_gen(GemmArgs p) { mt256::body<true, true, false, true, true, false, -1, 128, 3>(p); }
 // ... and split over K: (128 x 256 tile, K range) work items, fp32 partial tiles of 128 rows for the reduce pass.
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, -1, 128>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, -1, 128>(p); }

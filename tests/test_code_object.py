@@ -194,3 +194,24 @@ def test_main_loop_of_the_half_height_kernels_is_lean(kernels):
         want = "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16"
         assert count(kernels[name], want) == 128 and count(kernels[name], "v_mfma") == 128, name
 
+
+def test_main_loop_of_the_three_stage_kernels_is_lean(kernels):
+    """The 128 x 256 tile kernels with three ring stages: three unrolled K steps of 64 MFMAs, the same reads and requests
+    per step as the two-stage loop, one barrier per step, and a counted wait that leaves twelve requests in flight."""
+    for name, reads in (("maize_gemm_bf16_mt256_nn_h128r3", {"ds_read_b128": 24, "ds_read_b64_tr_b16": 96}),
+                        ("maize_gemm_bf16_mt256_nt_h128r3", {"ds_read_b128": 72})):
+        ins = kernels[name]
+        idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
+        assert len(idx) == 192 and count(ins, "v_mfma_f32_16x16x32_bf16") == 192
+        body = ins[idx[0]:idx[-1] + 1]
+        extra = [i for i in body if not i.startswith(("v_mfma", "ds_read", "buffer_load_dwordx4", "s_", "v_cmp_lt_u64"))]
+        assert not extra and count(body, "v_cmp_lt_u64") <= 3, extra[:5]
+        for mnemonic, n in reads.items():
+            assert count(body, mnemonic) == n, (name, mnemonic)
+        assert count(body, "buffer_load_dwordx4") == 36 and count(body, "s_barrier") == 3
+        assert count(body, "s_waitcnt") <= 12
+        assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(12)" in i) == 3, name
+    for name in ("maize_gemm_bf16_mt256_nn_h128r3_gen", "maize_gemm_f16_mt256_nt_h128r3_gen", "maize_gemm_f16_mt256_nn_h128r3_gen", "maize_gemm_bf16_mt256_nt_h128r3_gen"):
+        want = "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16"
+        assert count(kernels[name], want) == 192 and count(kernels[name], "v_mfma") == 192, name
+

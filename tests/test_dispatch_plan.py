@@ -198,8 +198,8 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (8192, 8192, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt",
         (16, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
-        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128",        # 64 tiles: partial tiles would cost more than they save, 128 tiles of 128 rows fill half the chip
-        (512, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128",        # 112 tiles: 224 of 128 rows are one round
+        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3",      # 64 tiles: partial tiles would cost more than they save, 128 tiles of 128 rows fill half the chip (32 K steps: three ring stages)
+        (512, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3",      # 112 tiles: 224 of 128 rows are one round
         (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128_splitk",  # few tiles, a long K: 128-row tiles cut over K
         (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128_splitk",
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",              # N x K weights streamed once
@@ -241,15 +241,19 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
     """56 to 128 tiles on 256 compute units leave most of the chip idle for a whole walk of K: two or four K ranges
     per tile pay for the partial tiles (measured: 256 x 14336 x 4096 67 -> 46 us, 768 x 8192 x 8192 128 -> 110 us) --
     or, where one round of them is cheaper than the split, tiles of 128 rows (768 x 8192 x 8192 94 us, 2048^3 37 -> 29)."""
-    p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)                  # 112 tiles of 128 rows in two K ranges
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and p["ksplit"] == 2 and p["grid"] == (224, 1, 1)
+    p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)                  # 112 tiles of 128 rows: whole K on three ring stages
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3" and p["ksplit"] == 1 and p["grid"] == (112, 1, 1)
     p = mz.gemm_plan(desc(128, 14336, 4096), compute_units=CUS)                  # one row of tiles: cut over K (38 us against 54.7 whole)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and p["ksplit"] == 4 and p["grid"] == (224, 1, 1)
     p = mz.gemm_plan(desc(768, 8192, 8192), compute_units=CUS)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128" and p["ksplit"] == 1 and p["grid"] == (192, 1, 1)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3" and p["ksplit"] == 1 and p["grid"] == (192, 1, 1)
     p = mz.gemm_plan(desc(640, 8192, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128" and p["grid"] == (160, 1, 1)
-    assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3" and p["grid"] == (160, 1, 1)
+    assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"
+    assert mz.gemm_plan(desc(512, 8192, 1024), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"         # 16 K steps: the two-stage loop (14.5 us against 15.8)
+    assert mz.gemm_plan(desc(1024, 4096, 1728), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"        # 27 steps
+    assert mz.gemm_plan(desc(1024, 4096, 1792), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"      # 28 steps, 128 tiles
+    assert mz.gemm_plan(desc(512, 2048, 1792), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"         # 32 tiles: too few to make the loads wait
     assert mz.gemm_plan(desc(4096, 2304, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"       # 288 tiles of 128 rows would need two rounds
     assert mz.gemm_plan(desc(1024, 14336, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"   # 224 tiles: one round as it is
 

@@ -208,6 +208,20 @@ def test_half_height_tiles(ctx, oracle, layout):
                dict(alpha=2.0, beta=0.0, c_nan=True), dict(lda=k + 3, ldb=bcols + 5)):
         assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen, label="h128 gen", **kw) == gen
         assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen16, half=True, label="h128 gen half", **kw) == gen16
+    # three ring stages (the dispatcher's choice from 28 K steps on): every step count mod 3, short and long K, several
+    # tiles per workgroup (1024 x 2304 x 256 on 256 compute units: 72 tiles -- one each -- but 9 x ... below goes round)
+    plain3, gen3, gen316 = (f"maize_gemm_bf16_mt256_{tag}_h128r3", f"maize_gemm_bf16_mt256_{tag}_h128r3_gen", f"maize_gemm_f16_mt256_{tag}_h128r3_gen")
+    for (m, n, k) in ((128, 256, 64), (128, 256, 128), (512, 1024, 192), (512, 1024, 448), (1000, 1032, 256), (100, 264, 1024), (640, 776, 2048), (384, 512, 4160)):
+        assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=plain3, label="h128r3") == plain3
+    m, n, k = 520, 776, 328
+    for kw in (dict(), dict(lda=k + 8, ldb=bcols + 16, ldc=n + 8), dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8),
+               dict(alpha=2.0, beta=0.0, c_nan=True), dict(lda=k + 3, ldb=bcols + 5)):
+        assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen3, label="h128r3 gen", **kw) == gen3
+        assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen316, half=True, label="h128r3 gen half", **kw) == gen316
+    assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, label="h128r3 auto") == plain3
+    assert run_ex(ctx, oracle, 1000, 2056, 1800, layout=layout, label="h128r3 auto tail") == gen3
+    assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, alpha=0.5, beta=1.0, label="h128r3 auto scaled") == gen3
+    assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, half=True, label="h128r3 auto half") == gen316
     # the dispatcher's choice
     assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, label="h128 auto") == plain
     assert run_ex(ctx, oracle, 520, 776, 328, layout=layout, label="h128 auto tail") == gen
@@ -221,6 +235,14 @@ def test_half_height_tiles(ctx, oracle, layout):
     got = run_gemm(ctx, a, b, bm, bn, bk, layout=layout, batch=batch, kernel=plain)
     base = run_gemm(ctx, a, b, bm, bn, bk, layout=layout, batch=batch, kernel=plain[:-5])
     assert np.array_equal(got, base)
+    assert np.array_equal(run_gemm(ctx, a, b, bm, bn, bk, layout=layout, batch=batch, kernel=plain3), base)
+    # ... and so many that every workgroup of the persistent grid walks several: 40 x 640 x 768 = 600 tiles of 128 rows
+    batch = 40
+    a = mz.gen.uniform_bf16(batch * bm * bk, 9)
+    b = mz.gen.uniform_bf16(batch * bk * bn, 10)
+    base = run_gemm(ctx, a, b, bm, bn, bk, layout=layout, batch=batch, kernel=plain[:-5])
+    assert np.array_equal(run_gemm(ctx, a, b, bm, bn, bk, layout=layout, batch=batch, kernel=plain3), base)
+    assert np.array_equal(run_gemm(ctx, a, b, bm, bn, bk, layout=layout, batch=batch, kernel=plain), base)
 
 
 @pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])

@@ -28,6 +28,9 @@ FAMILIES = [
     ("maize_gemm_bf16_mt256_nn_h128", 300, 520, 256, NN),           # 128 x 256 tiles
     ("maize_gemm_bf16_mt256_nt_h128_gen", 257, 264, 328, NT),
     ("maize_gemm_bf16_mt256_nn_h128_splitk", 100, 515, 2056, NN),   # ... cut over K, odd N through the reduce pass
+    ("maize_gemm_bf16_mt256_nn_h128r3", 300, 520, 256, NN),         # ... on three ring stages
+    ("maize_gemm_bf16_mt256_nt_h128r3_gen", 257, 264, 328, NT),
+    ("maize_gemm_bf16_mt256_nn_h128r3_gen", 130, 520, 456, NN),
     ("maize_gemm_bf16_mt256_nn_splitk", 64, 520, 2056, NN),
     ("maize_gemm_bf16_mt256_nt_splitk", 300, 264, 2056, NT),
     ("maize_gemm_bf16_mt256_nn_packed", 300, 515, 260, NN),

@@ -36,7 +36,9 @@ MT256_SLOT_FACTS = ("constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 :
                     "constexpr int EB = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : 6;",
                     "const int slot = e >= EB ? 16 * (e - EB) + s : AFTER + 16 * e + s;",
                     "if (slot >= 2 && (slot - 2) % DS == 0 && (slot - 2) / DS < NP) {",
-                    "if (DS * pc + 2 < AFTER) dma(pc, A1, B1, k_begin + BKE);",       # early pieces: those behind the barrier of step t itself
+                    # early pieces: those behind the barrier of step t itself (NST = 2 ring stages, or 3)
+                    "if (DS * pc + 2 < AFTER) dma(pc, A0 + (NST - 1) * ASTR, B0 + (NST - 1) * TILE, k_begin + (NST - 1) * BKE);",
+                    "k_early = k_begin + NST * BKE;", "k_late = k_begin + (NST - 1) * BKE;",
                     "if (e >= EB) dma((slot - 2) / DS, ca, cb, k_early);", "else         dma((slot - 2) / DS, na, nb, k_late);")
 
 
@@ -112,9 +114,10 @@ def mt256_wave_program(nk, slots, nt, barrier_eighth=6):
     return ops, steps
 
 
-def check_two_stage(ops, steps, nreads, parts=4, pieces=16):
+def check_two_stage(ops, steps, nreads, parts=4, pieces=16, nst=2):
     """`nreads`: fragment reads per part of a K step if a number; a list gives, per part, how many reads of the
-    tile must have been issued before the part's first MFMA (cumulative)."""
+    tile must have been issued before the part's first MFMA (cumulative).  `nst`: ring stages; with more than two a
+    barrier may stand with younger requests still in flight (("wait_keep", n) waits for all but the n youngest)."""
     cumulative = [nreads * (q + 1) for q in range(parts)] if isinstance(nreads, int) else list(nreads)
     assert len(cumulative) == parts
     epoch = 0
@@ -131,10 +134,10 @@ def check_two_stage(ops, steps, nreads, parts=4, pieces=16):
             _, tile, pc, stage = op
             if (tile, pc) in dma_epoch:
                 raise Hazard(f"piece {pc} of tile {tile} requested twice")
-            if stage != tile % 2:
+            if stage != tile % nst:
                 raise Hazard(f"tile {tile} requested into stage {stage}")
-            # WAR: the stage still holds tile-2; every wave must be past its last read of it
-            old = tile - 2
+            # WAR: the stage still holds tile-nst; every wave must be past its last read of it
+            old = tile - nst
             if old >= 0 and last_read_epoch.get(old, -1) >= epoch:
                 raise Hazard(f"tile {tile} piece {pc} overwrites tile {old} in epoch {epoch}, still being read")
             if old >= 0 and old < steps and reads_seen.get(old, 0) < cumulative[-1]:
@@ -145,15 +148,20 @@ def check_two_stage(ops, steps, nreads, parts=4, pieces=16):
         elif op[0] == "wait_all":
             completed.update(pending)
             pending = []
+        elif op[0] == "wait_keep":
+            keep = op[1]
+            done = pending[:len(pending) - keep] if keep else pending
+            completed.update(done)
+            pending = pending[len(done):]
         elif op[0] == "barrier":
-            if pending:
+            if pending and nst == 2:
                 raise Hazard("barrier with requests of this wave still in flight")
             epoch += 1
             for key in completed:
                 visible_from.setdefault(key, epoch)
         elif op[0] == "read":
             _, tile, quarter, stage = op
-            if stage != tile % 2:
+            if stage != tile % nst:
                 raise Hazard(f"tile {tile} read from stage {stage}")
             for pc in range(pieces):
                 if visible_from.get((tile, pc), 1 << 30) > epoch:
@@ -234,11 +242,13 @@ def test_macro_tile_checker_rejects_broken_schedules():
 # ---------------------------------------------------------------------------------------
 
 H128_READ_LINES = ("if (h4 == 0 && rb < NBR) read_b(1, kh, cur, rb);",
-                   "if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
-                   "if (h4 == 1 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }",
+                   "if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, nxt, r); }",
+                   "if (h4 == 1 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, nxt, rb); }",
+                   "const int nxt = R3 ? (cur + 1) % 3 : cur ^ 1, lat = R3 ? (cur + 2) % 3 : cur ^ 1;",
+                   "lds_ptr const ca = A0 + cur * ASTR, cb = B0 + cur * TILE, na = A0 + lat * ASTR, nb = B0 + lat * TILE, pb = B0 + nxt * TILE;",
                    "const int kh = IS8 ? 0 : H128 ? e >> 1 : e >> 2, h4 = H128 ? e & 1 : e & 3;",
                    "const int buf = H128 ? bi : bi ^ (IS8 ? st : kh);",
-                   "else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * 16 + r);")
+                   "else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * (ASTR / 2048) + r);")
 
 
 def h128_wave_program(nk, nt, barrier_at=3, ds=3, drop_read=None):
@@ -299,6 +309,75 @@ def test_half_height_tile_checker_rejects_broken_schedules():
         check_two_stage(*h128_wave_program(8, True, ds=6), need, parts=4, pieces=12)
     with pytest.raises(Hazard):                 # a fragment read dropped: MFMAs on stale registers
         check_two_stage(*h128_wave_program(8, True, drop_read=30), need, parts=4, pieces=12)
+
+
+# ---------------------------------------------------------------------------------------
+# 128 x 256 tiles with three ring stages: the same step, but tile t+1 sits complete in the next stage, the late pieces
+# issued before the barrier of step t are tile t+2's (into the stage after that one), the early pieces behind it tile
+# t+3's (into the stage step t has just read), and the wait in front of the barrier leaves the twelve requests of tile
+# t+2 in flight.  Two whole tiles are requested before the first step; three steps per trip
+# ---------------------------------------------------------------------------------------
+
+H128R3_LINES = ('if (R3) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");',
+                "for (uint32_t kt = 0; kt < nk; kt += NST) {", "if (R3) step(2);",
+                "for (int pc = 0; pc < NP; ++pc) dma(pc, A1, B1, k_begin + BKE);",
+                'static_assert(!R3 || NP == 12, "the counted waits of the three-stage ring assume twelve pieces per K tile");')
+
+
+def h128r3_wave_program(nk, nt, barrier_at=3, ds=3, keep=12, drop_read=None):
+    src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
+    for fact in MT256_SLOT_FACTS + H128_READ_LINES + H128R3_LINES:
+        assert fact in src, fact
+    nbr = 4 if nt else 8
+    slots = [ds * pc + 2 for pc in range(12)]
+    issued = {0: (1, nbr, False), 1: (2, 4 + nbr, False), 2: (3, nbr, False), 3: (0, 4 + nbr, True)}
+    ops = [("dma", 0, pc, 0) for pc in range(12)] + [("dma", 1, pc, 1) for pc in range(12)]
+    ops += [("wait_all",), ("barrier",)]
+    ops += [("read", 0, 0, 0)] * (4 + nbr)
+    ops += [("dma", 2, pc, 2) for pc in range(12) if slots[pc] < 16]
+    k_early, k_late = 3, 2
+    steps = 3 * ((nk + 2) // 3)
+    nread = 0
+    for t in range(steps):
+        cur, nxt, lat = t % 3, (t + 1) % 3, (t + 2) % 3
+        for e in range(4):
+            if e == barrier_at:
+                ops += [("wait_keep", keep), ("barrier",)]
+            need, n, next_tile = issued[e]
+            for sl in range(16):
+                ops.append(("mfma", t, e))
+                for _ in range((1 if sl < 4 else 0) + (1 if sl < nbr else 0) if n > nbr else (1 if sl < n else 0)):
+                    nread += 1
+                    if nread != drop_read:
+                        ops.append(("read", t + 1, need, nxt) if next_tile else ("read", t, need, cur))
+                slot = sl if e == 3 else 16 + 16 * e + sl
+                for pc in range(12):
+                    if slots[pc] == slot:
+                        ops.append(("dma", k_early, pc, cur) if e == 3 else ("dma", k_late, pc, lat))
+        k_early += 1
+        k_late += 1
+    ops.append(("wait_all",))
+    return ops, steps
+
+
+@pytest.mark.parametrize("nk", [1, 2, 3, 7, 28, 64])
+@pytest.mark.parametrize("nt", [False, True])
+def test_three_stage_schedule_is_hazard_free(nk, nt):
+    ops, steps = h128r3_wave_program(nk, nt)
+    last_tile = check_two_stage(ops, steps, h128_cumulative_reads(nt), parts=4, pieces=12, nst=3)
+    assert steps + 1 <= last_tile <= steps + 2          # tiles past the end are requested (zero-length descriptor), never multiplied
+
+
+def test_three_stage_checker_rejects_broken_schedules():
+    need = h128_cumulative_reads(True)
+    with pytest.raises(Hazard):                 # a wait that leaves one request more in flight: the next tile's last piece may not have landed
+        check_two_stage(*h128r3_wave_program(9, True, keep=13), need, parts=4, pieces=12, nst=3)
+    with pytest.raises(Hazard):                 # barrier one eighth early: the stage is refilled while its last B group is still being read
+        check_two_stage(*h128r3_wave_program(9, True, barrier_at=2), need, parts=4, pieces=12, nst=3)
+    with pytest.raises(Hazard):                 # requests six slots apart: the last ones are never issued
+        check_two_stage(*h128r3_wave_program(9, True, ds=6), need, parts=4, pieces=12, nst=3)
+    with pytest.raises(Hazard):                 # a fragment read dropped: MFMAs on stale registers
+        check_two_stage(*h128r3_wave_program(9, True, drop_read=30), need, parts=4, pieces=12, nst=3)
 
 
 # ---------------------------------------------------------------------------------------
