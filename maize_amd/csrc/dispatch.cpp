@@ -269,8 +269,10 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
 // with three, 0.55 us per step either way; 112 to 224 tiles: 0.70 against 0.52 per step) or K is long enough for the
 // rounding not to matter.
 bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles) {
-    const uint32_t nk = cdiv(k, 64u);
-    return kstep == 64u && nk >= 28u && (nk >= 48u || half_tiles >= 48u);
+    const uint32_t nk = cdiv(k, kstep);                         // (an 8-bit step, 128 deep, is as long as a 16-bit one)
+    // 8-bit operands: from 24 steps (E4M3 N x K, two -> three stages: 1024 x 4096 x 3072 26.2 -> 23.4 us, x 4096 31.2 -> 27.6,
+    // 768 x 8192 x 8192 58.8 -> 48.6; 2048^3, 16 steps: 17.6 -> 18.9)
+    return nk >= (kstep == 128u ? 24u : 28u) && (nk >= 48u || half_tiles >= 48u);
 }
 // Returns 0: the 256-row kernels; 1: 128-row tiles, whole K; >= 2: 128-row tiles in that many K ranges.
 uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
@@ -285,7 +287,7 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     const double step = kstep == 128u ? 0.87 : 0.67;
     // 16-bit operands and a long K: the three-stage kernels, 0.52 per step, steps in threes (2048^3 28.6 -> 24.9 us,
     // 1024 x 4096 x 4096 51.1 -> 42.0, 640 x 8192 x 4096 N x K 60.4 -> 45.9)
-    const double whole = h128_three_stages(s.k, kstep, half_tiles) ? 8.0 + 0.52 * 3.0 * cdiv(nk, 3u) : 8.0 + step * nk;
+    const double whole = h128_three_stages(s.k, kstep, half_tiles) ? 8.0 + (0.52 / 0.67) * step * 3.0 * cdiv(nk, 3u) : 8.0 + step * nk;
     double best = 0.9 * whole;                                     // splitting has to win 10 %
     uint32_t best_ks = 1;
     const double elems = (double)s.m * s.n * batch;
@@ -855,6 +857,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_" #tag "_mt256_nt_h128_gen", nullptr, tag##_nt_gen_supports, mt256_h128_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_h128_splitk", nullptr, tag##_nt_gen_supports, h128_splitk_plan}, \
     {"maize_gemm_" #tag "_mt256_nn_h128_gen", nullptr, tag##_nn_gen_supports, mt256_h128_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_h128r3_gen", nullptr, tag##_nt_gen_supports, mt256_h128_plan}, \
+    {"maize_gemm_" #tag "_mt256_nn_h128r3_gen", nullptr, tag##_nn_gen_supports, mt256_h128_plan}, \
     {"maize_gemm_" #tag "_mt256_nn_h128_splitk", nullptr, tag##_nn_gen_supports, h128_splitk_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_packed", "maize_gemm_" #tag "_mt256_nt_splitk", tag##_packed_supports, packed8_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_trb", "maize_gemm_" #tag "_mt256_nt", tag##_trb_supports, trb_plan}, \
@@ -933,7 +937,8 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         {
             const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units, 128);
             if (hk >= 1u) {
-                std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_%s_h128_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.nt ? "nt" : "nn", hk >= 2u ? "splitk" : "gen");
+                const bool r3 = hk == 1u && h128_three_stages(s.k, 128u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch);
+                std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_%s_h128%s_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.nt ? "nt" : "nn", r3 ? "r3" : "", hk >= 2u ? "splitk" : "gen");
                 const int fh = kernel_index(name);
                 if (fh >= 0 && kKernels[fh].supports(d) && plan_fits(kKernels[fh], d, compute_units)) return (uint32_t)fh;
             }

@@ -138,20 +138,22 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 // the last eighth; 12 pieces per wave and K tile, one every three MFMA slots.  8-bit operands: a K tile is one matrix
 // instruction deep, so the step is just the pair (A0, B0), (A0, B1) with the barrier between the two, A's buffers
 // alternate with the K tile, and the 12 pieces go out one every two (twice as long) MFMA slots.
-// NST = 3 (128-row tiles of 16-bit operands): three ring stages -- 3 x 16 KiB of A, 3 x 32 KiB of B, 16 KiB of epilogue
+// NST = 3 (128-row tiles): three ring stages -- 3 x 16 KiB of A, 3 x 32 KiB of B, 16 KiB of epilogue
 // staging (passes of 16 rows) -- so that a K tile is requested two steps before it is read.  Behind the barrier of step t
 // go the early pieces of tile t+3, into the stage step t has just read; before the barrier of step t+1 its late pieces;
 // it is read from the last eighth of step t+2 on.  The wait in front of the barrier of step t is `vmcnt(12)`: tile t+1
 // has landed, the twelve requests of tile t+2 -- younger -- stay in flight.  Three steps per trip, the step count rounded
 // up to a multiple of three with all-zero tiles.  B's third stage lies 64 KiB behind the first, past the reads' 16-bit
 // offset field, and has base registers of its own.
+// 8-bit operands on three stages: A's fragment buffer goes with the stage (three of them), all twelve pieces of tile
+// t+3 go out behind the barrier of step t, same wait.
 template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
     constexpr bool H128 = BMT == 128;
     static_assert(BMT == 256 || (H128 && !EDGE), "128-row tiles: no edge splitting");
-    constexpr bool R3 = NST == 3;                       // three ring stages (128-row tiles of 16-bit operands)
-    static_assert(NST == 2 || (R3 && H128 && F8 < 0), "three ring stages: 128-row tiles of 16-bit operands only");
+    constexpr bool R3 = NST == 3;                       // three ring stages (128-row tiles)
+    static_assert(NST == 2 || (R3 && H128), "three ring stages: 128-row tiles only");
     constexpr int ASTR = R3 ? TILE / 2 : TILE;          // bytes from one stage of A to the next
     constexpr int EPR = R3 ? 1 : 2;                     // accumulator rows per epilogue pass (the staging region is 4 or 8 KiB per wave)
     constexpr int MI = BMT / 32;                        // accumulator rows of a wave (16 rows each)
@@ -398,7 +400,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     bf16x8 fa[2][4];
     bf16x8 fb[2][4];
     short4v fbl[2][4], fbh[2][4];
-    u32x4 fa8[2][4][2], fb8[2][4][2];
+    u32x4 fa8[NST][4][2], fb8[2][4][2];                 // (8-bit 128-row tiles: A's buffer goes with the ring stage)
     typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
     u32x2 fb8t[2][4][4];                                // 8-bit row-major B: register pair 2 kk + h of a fragment
     constexpr int NAR = IS8 ? 8 : 4;                    // reads that bring in one A group
@@ -439,7 +441,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 #undef MAIZE_RD_CASE
     // Read r (0..NAR-1) of A group ai, K half kh, of the tile in stage st.
     auto read_a = [&](int ai, int kh, int st, int r) {
-        if (IS8 && H128) lds_read128(fa8[st & 1][r >> 1][r & 1], a_rd[r & 1], st * 16 + (r >> 1));   // one A group; the buffer alternates with the K tile
+        if (IS8 && H128) lds_read128(fa8[st][r >> 1][r & 1], a_rd[r & 1], st * (ASTR / 2048) + (r >> 1));   // one A group; the buffer goes with the stage, i.e. alternates with the K tile
         else if (IS8) lds_read128(fa8[ai][r >> 1][r & 1], a_rd[r & 1], st * 16 + 4 * ai + (r >> 1));   // half r & 1 = the 16-bit kernel's kh
         else if (H128) lds_read128(fa[kh][r], a_rd[kh], st * (ASTR / 2048) + r);                            // one A group; the buffer alternates with the K half
         else     lds_read128(fa[ai][r], a_rd[kh], st * 16 + 4 * ai + r);
@@ -449,8 +451,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const int buf = H128 ? bi : bi ^ (IS8 ? st : kh);
         const bool far = R3 && st == 2;                       // third stage: from the second base register
         const int so = far ? 0 : st * 16;
-        if (TR8) lds_read_tr8(fb8t[buf][r >> 2][r & 3], b_rd[4 * bi + (r >> 2)], st * 16 + ((r >> 1) & 1) * 8 + (r & 1));
-        else if (IS8) lds_read128(fb8[buf][r >> 1][r & 1], b_rd[r & 1], st * 16 + 4 * bi + (r >> 1));
+        if (TR8) lds_read_tr8(fb8t[buf][r >> 2][r & 3], far ? b_rd2[4 * bi + (r >> 2)] : b_rd[4 * bi + (r >> 2)], so + ((r >> 1) & 1) * 8 + (r & 1));
+        else if (IS8) lds_read128(fb8[buf][r >> 1][r & 1], far ? b_rd2[r & 1] : b_rd[r & 1], so + 4 * bi + (r >> 1));
         else if (NT) lds_read128(fb[buf][r], far ? b_rd2[kh] : b_rd[kh], so + 4 * bi + r);
         else {
             const int c = r >> 1, h = r & 1;                  // rows 32 kh + 4 h + ...: 16 KiB and 2 KiB further on
@@ -522,7 +524,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // accumulator comes up again 128 MFMAs later: no dependent back-to-back issue.)
                 if (IS8)   // 8-bit operands: B is the first source, so cbsz carries B's format and blgp A's (0 = E4M3, 1 = E5M2)
                     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(acc[4 * ai + r4][4 * bi + c4])
-                                 : "v"(b_operand8(H128 ? bi : bi ^ cur, c4)), "v"(operand8(fa8[H128 ? cur & 1 : ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
+                                 : "v"(b_operand8(H128 ? bi : bi ^ cur, c4)), "v"(operand8(fa8[H128 ? cur : ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
                 else if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
                     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[4 * ai + r4][4 * bi + c4]) : "v"(b_operand(H128 ? bi : bi ^ kh, c4)), "v"(fa[H128 ? kh : ai][r4]));
                 else

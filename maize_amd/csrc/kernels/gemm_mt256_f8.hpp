@@ -23,6 +23,7 @@
 //
 // _h128: tiles of 128 x 256 (general epilogue, and cut over K), for products whose 256-row tiles would fill half the
 // compute units or less: the K step is the pair (A0, B0), (A0, B1) with the barrier between the two.
+// _h128r3: the same on three ring stages (K tiles requested two steps ahead), for a long K.
 //
 // 16 x 16 x 128 and not 32 x 32 x 64 (the first version): register-only loops of the two on E4M3 data
 // from uniform[-1,1) measure 39.9 us against 42.9 us for the FLOP of 4096^3 at the board's power limit
@@ -44,7 +45,9 @@ namespace maize {
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_h128_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, (fa) | ((fb) << 1), 128>(p); } \
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_h128_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, (fa) | ((fb) << 1), 128>(p); } \
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, (fa) | ((fb) << 1), 128>(p); } \
-    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, (fa) | ((fb) << 1), 128>(p); }
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, (fa) | ((fb) << 1), 128>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_h128r3_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, (fa) | ((fb) << 1), 128, 3>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128r3_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, (fa) | ((fb) << 1), 128, 3>(p); }
 MAIZE_F8_KERNELS(e4m3, 0, 0)
 MAIZE_F8_KERNELS(e5m2, 1, 1)
 MAIZE_F8_KERNELS(e4m3e5m2, 0, 1)     // A is E4M3, B is E5M2

@@ -97,18 +97,20 @@ def test_matrix_instruction_per_kernel(kernels):
             # B is fed as the first source, so cbsz carries B's format code and blgp A's (E4M3 = 0 is not printed, E5M2 = 1).
             f8 = [i for i in ins if i.startswith("v_mfma_f32_16x16x128_f8f6f4")]
             h128 = "_h128" in name                                            # 128 x 256 tiles: half the MFMAs, one A group
-            per = 64 if h128 else 128
-            assert len(f8) == per and count(ins, "v_mfma") == per, name       # two unrolled K steps of 128 elements, 64 (32) MFMAs each
+            steps = 3 if "_h128r3" in name else 2                             # K steps per trip of the loop = ring stages
+            per = (32 if h128 else 64) * steps
+            assert len(f8) == per and count(ins, "v_mfma") == per, name       # unrolled K steps of 128 elements, 64 (32) MFMAs each
             tag = name[len("maize_gemm_"):].split("_")[0]
             a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
             assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
             body = ins[next(k for k, i in enumerate(ins) if i.startswith("v_mfma")):len(ins) - next(k for k, i in enumerate(reversed(ins)) if i.startswith("v_mfma"))]
             if "_mt256_nn" in name:
                 # row-major B: A by 128-bit reads, B by four transposing 8-byte reads per fragment
-                assert count(body, "ds_read_b128") == (16 if h128 else 32) and count(body, "ds_read_b64_tr_b8") == 64, name
+                assert count(body, "ds_read_b128") == (8 * steps if h128 else 32) and count(body, "ds_read_b64_tr_b8") == 32 * steps, name
             else:
-                assert count(body, "ds_read_b128") == (48 if h128 else 64) and count(body, "ds_read_b64_tr_b8") == 0, name
-            assert count(body, "buffer_load_dwordx4") == (24 if h128 else 32) and count(body, "s_barrier") == 2, name
+                assert count(body, "ds_read_b128") == (24 * steps if h128 else 64) and count(body, "ds_read_b64_tr_b8") == 0, name
+            assert count(body, "buffer_load_dwordx4") == (12 * steps if h128 else 32) and count(body, "s_barrier") == steps, name
+            assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(12)" in i) == (3 if steps == 3 else 0), name
             assert count(body, "v_accvgpr") == 0 and count(body, "v_mov_b32") == 0, name     # accumulators and fragments stay in place
         elif "_mt128_" in name:
             # the catalogue's tf32 and f64 entries: full fp32 / fp64 matrix instructions; one K tile of 128 bytes

@@ -386,13 +386,15 @@ def test_half_height_tiles_on_8bit_operands(ctx, oracle, fmt):
     elem = ab_of(FMT[fmt][1])
     for layout, tag in ((mz.LAYOUT_NT, "nt"), (mz.LAYOUT_NN, "nn")):
         gen, split = f"maize_gemm_{fmt}_mt256_{tag}_h128_gen", f"maize_gemm_{fmt}_mt256_{tag}_h128_splitk"
+        gen3 = f"maize_gemm_{fmt}_mt256_{tag}_h128r3_gen"                      # ... on three ring stages
         shapes = [(128, 256, 128), (256, 512, 384), (300, 528, 400), (1000, 1040, 1040), (100, 272, 2064), (512, 2048, 1024)]
         for (m, n, k) in shapes if fmt in ("e4m3", "e5m2") else shapes[2:4]:
-            for kern in (gen, split):
+            for kern in (gen, split, gen3):
                 assert run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, kernel=kern, label="h128 f8") == kern
         bcols = 784 if layout == mz.LAYOUT_NN else 400
         for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=792), dict(lda=416, ldb=bcols + 16, ldc=800), dict(out_f16=True)):
             assert run_f8(ctx, oracle, 520, 784, 400, layout=layout, fmt=fmt, kernel=gen, label="h128 f8 knobs", **kw) == gen
+            assert run_f8(ctx, oracle, 520, 784, 400, layout=layout, fmt=fmt, kernel=gen3, label="h128r3 f8 knobs", **kw) == gen3
         assert run_f8(ctx, oracle, 512, 2048, 1024, layout=layout, fmt=fmt, label="h128 f8 auto") == gen
         assert run_f8(ctx, oracle, 100, 2048, 8192, layout=layout, fmt=fmt, label="h128 f8 auto, cut over K") == split
         m, n, k = 640, 784, 1168
@@ -402,6 +404,8 @@ def test_half_height_tiles_on_8bit_operands(ctx, oracle, fmt):
         half, _ = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, layout, fmt, k, ldb, n, kernel=gen)
         whole, _ = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, layout, fmt, k, ldb, n, kernel=gen.replace("_h128", ""))
         assert np.array_equal(half, whole)
+        half3, _ = launch(ctx, a, b, np.zeros(m * n, np.uint16), m, n, k, layout, fmt, k, ldb, n, kernel=gen3)
+        assert np.array_equal(half3, whole)
 
 
 def test_dispatch_of_8bit_products(ctx):
@@ -414,6 +418,9 @@ def test_dispatch_of_8bit_products(ctx):
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nt"
     assert pick(4096, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn"          # row-major B: read where it lies
     assert pick(4096, 4104, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_trb"      # ... N % 16: transposed copy
+    assert pick(2048, 2048, 2048, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_h128_gen"      # half a round of 128-row tiles, 16 K steps
+    assert pick(1024, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_h128r3_gen"    # ... 32 K steps: three ring stages
+    assert pick(1024, 4096, 3072, mz.LAYOUT_NN, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nn_h128r3_gen"    # (from 24 steps on)
     assert pick(4096, 4096, 4104, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_packed"   # K % 16: padded copies
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3, lda=4104) == "maize_gemm_e4m3_mt256_nt_packed"
     assert pick(64, 64, 64, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_bf16_wave32"

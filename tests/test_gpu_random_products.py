@@ -65,3 +65,41 @@ def test_random_products_through_the_dispatcher(ctx, oracle, seed):
         reached[took.replace("maize_gemm_", "")] += 1
     _say(f"seed {seed}: kernels reached: {dict(reached)}")
     assert len(reached) >= 8           # the draw is wide enough to be worth its time
+
+
+def draw_midsize_case(rng):
+    """Half a round of 128-row tiles, give or take, and a K of 24 to 72 steps: the range where the dispatcher moves between
+    the 128-row kernels on two and three ring stages, their split-K form and the 256-row kernels."""
+    fmt = str(rng.choice(["bf16", "bf16", "f16", "e4m3", "e5m2"]))
+    layout = int(rng.choice([mz.LAYOUT_NN, mz.LAYOUT_NT]))
+    m = int(rng.choice([384, 512, 640, 768, 1000, 1024, 1536, 2048])) + int(rng.choice([0, 0, 0, 8, -8, 24]))
+    n = int(rng.choice([1024, 2048, 3072, 4096])) + int(rng.choice([0, 0, 0, 16, -16, 48]))
+    step = 64 if fmt in ("bf16", "f16") else 128
+    k = int(rng.integers(24, 73)) * step + int(rng.choice([0, 0, 0, 16, -16, 32]))
+    bcols = n if layout == mz.LAYOUT_NN else k
+    def ld(cols):
+        return None if rng.random() < 0.7 else cols + int(rng.choice([16, 64]))
+    kw = dict(lda=ld(k), ldb=ld(bcols), ldc=ld(n))
+    r = rng.random()
+    if r < 0.25:
+        kw.update(alpha=float(rng.choice([0.5, -1.25])), beta=float(rng.choice([0.0, 0.75])))
+    elif r < 0.4:
+        kw.update(out_f32=True, alpha=float(rng.choice([1.0, 3.0])), beta=float(rng.choice([0.0, -0.5])))
+    return fmt, layout, m, n, k, kw
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_random_midsize_products_with_a_long_k(ctx, oracle, seed):
+    rng = np.random.default_rng(seed)
+    reached = collections.Counter()
+    for i in range(12):
+        fmt, layout, m, n, k, kw = draw_midsize_case(rng)
+        label = f"midsize {seed}.{i}"
+        _say(f"{label}: {fmt} {'NT' if layout else 'NN'} {m}x{n}x{k} {kw}")
+        if fmt in ("bf16", "f16"):
+            took = run_ex(ctx, oracle, m, n, k, layout=layout, half=fmt == "f16", seed=seed * 100 + i, label=label, **kw)
+        else:
+            took = run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, seed=seed * 100 + i, label=label, **kw)
+        reached[took.replace("maize_gemm_", "")] += 1
+    _say(f"seed {seed}: kernels reached: {dict(reached)}")
+    assert any("h128r3" in name for name in reached)

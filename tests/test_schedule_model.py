@@ -386,23 +386,26 @@ def test_three_stage_checker_rejects_broken_schedules():
 # ones, two per slot); 12 pieces per wave and K tile, one per MFMA slot behind the barrier
 # ---------------------------------------------------------------------------------------
 
-def h128_f8_wave_program(nk, tr, barrier_at=1, ds=1):
+def h128_f8_wave_program(nk, tr, barrier_at=1, ds=1, nst=2, keep=12):
+    """nst = 3: the three-stage ring (two whole tiles requested in front, tile t+3 behind the barrier of step t, the wait
+    leaves the `keep` youngest requests in flight)."""
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
-    for fact in MT256_SLOT_FACTS + H128_READ_LINES + ("if (IS8 && H128) lds_read128(fa8[st & 1][r >> 1][r & 1], a_rd[r & 1], st * 16 + (r >> 1));",):
+    for fact in MT256_SLOT_FACTS + H128_READ_LINES + H128R3_LINES + ("if (IS8 && H128) lds_read128(fa8[st][r >> 1][r & 1], a_rd[r & 1], st * (ASTR / 2048) + (r >> 1));",
+                                                                     "u32x4 fa8[NST][4][2], fb8[2][4][2];", '"v"(operand8(fa8[H128 ? cur : ai][r4]))'):
         assert fact in src, fact
     nbr, per_slot = (16, 2) if tr else (8, 1)
     slots = [ds * pc + 2 for pc in range(12)]
-    ops = [("dma", 0, pc, 0) for pc in range(12)]
+    ops = [("dma", t, pc, t) for t in range(nst - 1) for pc in range(12)]
     ops += [("wait_all",), ("barrier",)]
     ops += [("read", 0, 0, 0)] * (8 + nbr)
-    ops += [("dma", 1, pc, 1) for pc in range(12) if slots[pc] < 16]
-    k_early, k_late = 2, 1
-    steps = nk + (nk & 1)
+    ops += [("dma", nst - 1, pc, nst - 1) for pc in range(12) if slots[pc] < 16]
+    k_early, k_late = nst, nst - 1
+    steps = nst * ((nk + nst - 1) // nst)
     for t in range(steps):
-        cur, nxt = t & 1, (t & 1) ^ 1
+        cur, nxt, lat = t % nst, (t + 1) % nst, (t + nst - 1) % nst
         for e in range(2):
             if e == barrier_at:
-                ops += [("wait_all",), ("barrier",)]
+                ops += [("wait_all",) if nst == 2 else ("wait_keep", keep), ("barrier",)]
             for sl in range(16):
                 ops.append(("mfma", t, e))
                 if e == 0:                                   # B group 1 of this tile
@@ -412,7 +415,7 @@ def h128_f8_wave_program(nk, tr, barrier_at=1, ds=1):
                 slot = sl if e == 1 else 16 + sl
                 for pc in range(12):
                     if slots[pc] == slot:
-                        ops.append(("dma", k_early, pc, cur) if e == 1 else ("dma", k_late, pc, nxt))
+                        ops.append(("dma", k_early, pc, cur) if e == 1 else ("dma", k_late, pc, lat))
         k_early += 1
         k_late += 1
     ops.append(("wait_all",))
@@ -426,6 +429,9 @@ def test_8bit_half_height_tile_schedule_is_hazard_free(nk, tr):
     ops, steps = h128_f8_wave_program(nk, tr)
     last_tile = check_two_stage(ops, steps, [8 + nbr, 8 + 2 * nbr], parts=2, pieces=12)
     assert steps <= last_tile <= steps + 1
+    ops, steps = h128_f8_wave_program(nk, tr, nst=3)
+    last_tile = check_two_stage(ops, steps, [8 + nbr, 8 + 2 * nbr], parts=2, pieces=12, nst=3)
+    assert steps + 1 <= last_tile <= steps + 2
 
 
 def test_8bit_half_height_tile_checker_rejects_broken_schedules():
@@ -435,6 +441,10 @@ def test_8bit_half_height_tile_checker_rejects_broken_schedules():
         check_two_stage(*h128_f8_wave_program(8, False, barrier_at=0), [16, 24], parts=2, pieces=12)
     with pytest.raises(Hazard):                 # requests three slots apart: the last ones would never be issued
         check_two_stage(*h128_f8_wave_program(8, False, ds=3), [16, 24], parts=2, pieces=12)
+    with pytest.raises(Hazard):                 # three stages, a wait that leaves thirteen requests in flight
+        check_two_stage(*h128_f8_wave_program(9, False, nst=3, keep=13), [16, 24], parts=2, pieces=12, nst=3)
+    with pytest.raises(Hazard):                 # three stages, barrier in front of the first eighth
+        check_two_stage(*h128_f8_wave_program(9, False, nst=3, barrier_at=0), [16, 24], parts=2, pieces=12, nst=3)
 
 
 # ---------------------------------------------------------------------------------------
