@@ -274,6 +274,11 @@ bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles) {
     // 768 x 8192 x 8192 58.8 -> 48.6; 2048^3, 16 steps: 17.6 -> 18.9)
     return nk >= (kstep == 128u ? 24u : 28u) && (nk >= 48u || half_tiles >= 48u);
 }
+// What a K step of a 128-row tile costs, in steps of the 256-row kernel at the power limit (~ microseconds): 0.67 on two
+// ring stages, 0.52 on three -- except for K ranges of a row-major B on three stages, i.e. long ranges, which measure
+// 0.82-0.91 whatever share of the chip is at work (1024 x 4096 x 14336 in two ranges 123.6 us, N x K 101.5;
+// 512 x 8192 x 8192 78.6 / 66.2; 384 x 6144 x 4096 44.4 / 35.0), so that whole tiles or the 256-row split win there.
+double h128_step(bool three, bool split, bool nt) { return !three ? 0.67 : (split && !nt) ? 0.85 : 0.52; }
 // Returns 0: the 256-row kernels; 1: 128-row tiles, whole K; >= 2: 128-row tiles in that many K ranges.
 uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
     const uint32_t resident = cus >= 8u ? cus - cus % 8u : cus;
@@ -284,10 +289,11 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     const uint32_t nk = cdiv(s.k, kstep);
     // per K step: 0.67 of the 256-row kernel's; an 8-bit step (128 deep) takes 1.3 of a 16-bit one, which the fixed terms
     // here (in 16-bit steps) have to be weighed against (E4M3 128 x 14336 x 4096: 31.1 us whole, 25.8 in two ranges)
-    const double step = kstep == 128u ? 0.87 : 0.67;
-    // 16-bit operands and a long K: the three-stage kernels, 0.52 per step, steps in threes (2048^3 28.6 -> 24.9 us,
-    // 1024 x 4096 x 4096 51.1 -> 42.0, 640 x 8192 x 4096 N x K 60.4 -> 45.9)
-    const double whole = h128_three_stages(s.k, kstep, half_tiles) ? 8.0 + (0.52 / 0.67) * step * 3.0 * cdiv(nk, 3u) : 8.0 + step * nk;
+    const double scale = kstep == 128u ? 0.87 / 0.67 : 1.0;
+    // a long K: the three-stage kernels, steps in threes (2048^3 28.6 -> 24.9 us, 1024 x 4096 x 4096 51.1 -> 42.0,
+    // 640 x 8192 x 4096 N x K 60.4 -> 45.9)
+    const bool three = h128_three_stages(s.k, kstep, half_tiles);
+    const double whole = 8.0 + scale * h128_step(three, false, s.nt) * (three ? 3u * cdiv(nk, 3u) : nk);
     double best = 0.9 * whole;                                     // splitting has to win 10 %
     uint32_t best_ks = 1;
     const double elems = (double)s.m * s.n * batch;
@@ -298,7 +304,11 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
         for (uint32_t ks = 2; ks <= kmax; ++ks) {
             if (cdiv(nk, cdiv(nk, ks)) != ks) continue;            // would leave an empty range
             if (half_tiles * ks * 131072ull > (1ull << 30)) break;
-            const double t = 8.0 + step * cdiv(nk, ks) + 6.0 + (1.2e-6 * elems + 0.15) * ks;
+            // (ranges long enough run on the three-stage kernels, in threes)
+            const uint32_t r = cdiv(nk, ks);
+            const bool three_r = h128_three_stages(r * kstep, kstep, half_tiles * ks);
+            const double loop = scale * h128_step(three_r, true, s.nt) * (three_r ? 3u * cdiv(r, 3u) : r);
+            const double t = 8.0 + loop + 6.0 + (1.2e-6 * elems + 0.15) * ks;
             if (t < best) { best = t; best_ks = ks; }
         }
     if (best_ks == 1u) best = whole;
@@ -809,6 +819,10 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_h128_splitk", nullptr, splitk_nt_supports, h128_splitk_plan},
     {"maize_gemm_f16_mt256_nn_h128_splitk", nullptr, splitk_f16_nn_supports, h128_splitk_plan},
     {"maize_gemm_f16_mt256_nt_h128_splitk", nullptr, splitk_f16_nt_supports, h128_splitk_plan},
+    {"maize_gemm_bf16_mt256_nn_h128r3_splitk", nullptr, splitk_nn_supports, h128_splitk_plan},
+    {"maize_gemm_bf16_mt256_nt_h128r3_splitk", nullptr, splitk_nt_supports, h128_splitk_plan},
+    {"maize_gemm_f16_mt256_nn_h128r3_splitk", nullptr, splitk_f16_nn_supports, h128_splitk_plan},
+    {"maize_gemm_f16_mt256_nt_h128r3_splitk", nullptr, splitk_f16_nt_supports, h128_splitk_plan},
     {"maize_gemm_bf16_mt256_nn_ktail", nullptr, mt256_nn_ktail_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_ktail", nullptr, mt256_nt_ktail_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_edge", nullptr, mt256_nn_supports, mt256_edge_plan},
@@ -859,6 +873,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_" #tag "_mt256_nn_h128_gen", nullptr, tag##_nn_gen_supports, mt256_h128_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_h128r3_gen", nullptr, tag##_nt_gen_supports, mt256_h128_plan}, \
     {"maize_gemm_" #tag "_mt256_nn_h128r3_gen", nullptr, tag##_nn_gen_supports, mt256_h128_plan}, \
+    {"maize_gemm_" #tag "_mt256_nt_h128r3_splitk", nullptr, tag##_nt_gen_supports, h128_splitk_plan}, \
+    {"maize_gemm_" #tag "_mt256_nn_h128r3_splitk", nullptr, tag##_nn_gen_supports, h128_splitk_plan}, \
     {"maize_gemm_" #tag "_mt256_nn_h128_splitk", nullptr, tag##_nn_gen_supports, h128_splitk_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_packed", "maize_gemm_" #tag "_mt256_nt_splitk", tag##_packed_supports, packed8_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_trb", "maize_gemm_" #tag "_mt256_nt", tag##_trb_supports, trb_plan}, \
@@ -937,7 +953,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         {
             const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units, 128);
             if (hk >= 1u) {
-                const bool r3 = hk == 1u && h128_three_stages(s.k, 128u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch);
+                const bool r3 = h128_three_stages(cdiv(cdiv(s.k, 128u), hk) * 128u, 128u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk);   // by the K steps of a range
                 std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_%s_h128%s_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.nt ? "nt" : "nn", r3 ? "r3" : "", hk >= 2u ? "splitk" : "gen");
                 const int fh = kernel_index(name);
                 if (fh >= 0 && kKernels[fh].supports(d) && plan_fits(kKernels[fh], d, compute_units)) return (uint32_t)fh;
@@ -999,9 +1015,12 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // ... or, where that is faster, compute it in 128-row tiles (the kernels that store C themselves: 16-byte rows of C).
     const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units);
     if (hk >= 2u) {
-        static const char* const kH128Split[2][2] = {{"maize_gemm_bf16_mt256_nn_h128_splitk", "maize_gemm_bf16_mt256_nt_h128_splitk"},
-                                                     {"maize_gemm_f16_mt256_nn_h128_splitk", "maize_gemm_f16_mt256_nt_h128_splitk"}};
-        const int hs = kernel_index(kH128Split[half_in(d)][s.nt]);
+        static const char* const kH128Split[2][2][2] = {{{"maize_gemm_bf16_mt256_nn_h128_splitk", "maize_gemm_bf16_mt256_nt_h128_splitk"},
+                                                         {"maize_gemm_f16_mt256_nn_h128_splitk", "maize_gemm_f16_mt256_nt_h128_splitk"}},
+                                                        {{"maize_gemm_bf16_mt256_nn_h128r3_splitk", "maize_gemm_bf16_mt256_nt_h128r3_splitk"},
+                                                         {"maize_gemm_f16_mt256_nn_h128r3_splitk", "maize_gemm_f16_mt256_nt_h128r3_splitk"}}};
+        const int r3 = h128_three_stages(cdiv(cdiv(s.k, 64u), hk) * 64u, 64u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk);
+        const int hs = kernel_index(kH128Split[r3][half_in(d)][s.nt]);
         if (hs >= 0 && kKernels[hs].supports(d) && plan_fits(kKernels[hs], d, compute_units)) return (uint32_t)hs;
     }
     if (hk == 1u) {

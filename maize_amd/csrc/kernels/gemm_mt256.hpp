@@ -816,6 +816,11 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128_
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, -1, 128>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nn_h128_splitk(GemmArgs p) { mt256::body<false, true, false, true, true, true, -1, 128>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nt_h128_splitk(GemmArgs p) { mt256::body<true, true, false, true, true, true, -1, 128>(p); }
+// ... on three ring stages, for K ranges of 28 steps or more
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_h128r3_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, -1, 128, 3>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_h128r3_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, -1, 128, 3>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nn_h128r3_splitk(GemmArgs p) { mt256::body<false, true, false, true, true, true, -1, 128, 3>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_mt256_nt_h128r3_splitk(GemmArgs p) { mt256::body<true, true, false, true, true, true, -1, 128, 3>(p); }
 // Split-K: (tile, K range) work items, fp32 partial tiles to the workspace; any K % 8 == 0.
 #define MAIZE_MT256_KERNEL_SPLITK(name, nt, f16) \
     extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, true, false, true, f16, true>(p); }

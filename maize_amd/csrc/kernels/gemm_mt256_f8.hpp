@@ -47,7 +47,9 @@ namespace maize {
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, (fa) | ((fb) << 1), 128>(p); } \
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, (fa) | ((fb) << 1), 128>(p); } \
     extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_h128r3_gen(GemmArgs p) { mt256::body<true, true, false, true, false, false, (fa) | ((fb) << 1), 128, 3>(p); } \
-    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128r3_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, (fa) | ((fb) << 1), 128, 3>(p); }
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128r3_gen(GemmArgs p) { mt256::body<false, true, false, true, false, false, (fa) | ((fb) << 1), 128, 3>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nt_h128r3_splitk(GemmArgs p) { mt256::body<true, true, false, true, false, true, (fa) | ((fb) << 1), 128, 3>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_mt256_nn_h128r3_splitk(GemmArgs p) { mt256::body<false, true, false, true, false, true, (fa) | ((fb) << 1), 128, 3>(p); }
 MAIZE_F8_KERNELS(e4m3, 0, 0)
 MAIZE_F8_KERNELS(e5m2, 1, 1)
 MAIZE_F8_KERNELS(e4m3e5m2, 0, 1)     // A is E4M3, B is E5M2

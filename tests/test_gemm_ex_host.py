@@ -175,7 +175,7 @@ def test_dispatch_of_8bit_operands():
         assert plan["kernel"] == name and tuple(plan["grid"]) == (256, 1, 1) and plan["workspace_bytes"] == 0
         general = ex(**big, in_type=it, alpha=2.0, beta=1.0, out_type=mz.OUT_F32)
         assert mz.gemm_plan(general)["kernel"] == name + "_gen"
-        half_tiles = (name + "_h128_gen", name + "_h128r3_gen", name + "_h128_splitk")   # the same on tiles of 128 x 256 (two or three ring stages)
+        half_tiles = (name + "_h128_gen", name + "_h128r3_gen", name + "_h128_splitk", name + "_h128r3_splitk")   # the same on tiles of 128 x 256 (two or three ring stages)
         for other in mz.kernel_names():
             assert _supports(other, x) == (other in (name, name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32") + half_tiles), other
             assert _supports(other, general) == (other in (name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32") + half_tiles), other
@@ -188,7 +188,7 @@ def test_dispatch_of_8bit_operands():
         assert few["kernel"] == direct + "_h128_splitk" and few["ksplit"] >= 2 and few["workspace_bytes"] == 65536 + 16 * few["ksplit"] * 131072   # 16 tiles of 128 x 256
         for other in mz.kernel_names():
             assert _supports(other, ex(4096, 4096, 4096, in_type=it)) == (
-                other in (direct, direct + "_gen", direct + "_splitk", direct + "_h128_gen", direct + "_h128r3_gen", direct + "_h128_splitk", name + "_trb", name + "_trb_gen", packed, "maize_gemm_bf16_wave32")), other
+                other in (direct, direct + "_gen", direct + "_splitk", direct + "_h128_gen", direct + "_h128r3_gen", direct + "_h128_splitk", direct + "_h128r3_splitk", name + "_trb", name + "_trb_gen", packed, "maize_gemm_bf16_wave32")), other
         tr_plan = mz.gemm_plan(ex(4096, 4104, 4096, in_type=it))                                              # N % 16 != 0: transposed copy of B, nothing else
         assert tr_plan["kernel"] == name + "_trb" and tr_plan["workspace_bytes"] == 65536 + 4104 * 4096 and tr_plan["reduce_grid"] == 0
         assert mz.gemm_plan(ex(4096, 4104, 4096, in_type=it, beta=1.0))["kernel"] == name + "_trb_gen"

@@ -340,13 +340,15 @@ def test_split_k_kernels(ctx, oracle, layout, shape):
     run_ex(ctx, oracle, m, n, k, layout=layout, label="dispatcher")      # whatever the cost model picks
     run_ex(ctx, oracle, m, n, k, layout=layout, kernel=want, label="splitk")
     run_ex(ctx, oracle, m, n, k, layout=layout, kernel=half_tiles, label="splitk, 128-row tiles")
+    three = want.replace("_splitk", "_h128r3_splitk")                    # ... on three ring stages
+    run_ex(ctx, oracle, m, n, k, layout=layout, kernel=three, label="splitk, 128-row tiles, three stages")
     if (m, n, k) == (64, 4096, 4096):
         x = mz.gemm_ex_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x1000000, *((k, n) if layout == mz.LAYOUT_NN else (n, k))),
                             mz.GlobalMatrix(0x4000000, m, n), layout=layout)
         assert mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"] == half_tiles
     for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(half=True),
                dict(lda=k + 8, ldc=n + 16)):
-        for name in (want, half_tiles):
+        for name in (want, half_tiles, three):
             run_ex(ctx, oracle, m, n, k, layout=layout, kernel=("maize_gemm_f16_mt256_" + name[22:]) if kw.get("half") else name,
                    label="splitk knobs", **kw)
 
@@ -368,6 +370,10 @@ def test_split_k_batched_and_more_items_than_workgroups(ctx, oracle):
         # bit-identical to itself on a second run (fixed summation order)
         again = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel="maize_gemm_bf16_mt256_nn_splitk")
         assert np.array_equal(got, again)
+        # 128-row tiles cut over K, two and three ring stages: the same ranges, the same sums
+        two = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel="maize_gemm_bf16_mt256_nn_h128_splitk")
+        three = run_gemm(ctx, a, b, m, n, k, batch=batch, kernel="maize_gemm_bf16_mt256_nn_h128r3_splitk")
+        assert np.array_equal(two, three)
 
 
 # ---- packed path: odd extents, unaligned operands, any leading dimension ---------------------------

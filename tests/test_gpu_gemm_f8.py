@@ -389,7 +389,7 @@ def test_half_height_tiles_on_8bit_operands(ctx, oracle, fmt):
         gen3 = f"maize_gemm_{fmt}_mt256_{tag}_h128r3_gen"                      # ... on three ring stages
         shapes = [(128, 256, 128), (256, 512, 384), (300, 528, 400), (1000, 1040, 1040), (100, 272, 2064), (512, 2048, 1024)]
         for (m, n, k) in shapes if fmt in ("e4m3", "e5m2") else shapes[2:4]:
-            for kern in (gen, split, gen3):
+            for kern in (gen, split, gen3, split.replace("_h128_", "_h128r3_")):
                 assert run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, kernel=kern, label="h128 f8") == kern
         bcols = 784 if layout == mz.LAYOUT_NN else 400
         for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=792), dict(lda=416, ldb=bcols + 16, ldc=800), dict(out_f16=True)):

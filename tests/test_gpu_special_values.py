@@ -29,6 +29,8 @@ FAMILIES = [
     ("maize_gemm_bf16_mt256_nt_h128_gen", 257, 264, 328, NT),
     ("maize_gemm_bf16_mt256_nn_h128_splitk", 100, 515, 2056, NN),   # ... cut over K, odd N through the reduce pass
     ("maize_gemm_bf16_mt256_nn_h128r3", 300, 520, 256, NN),         # ... on three ring stages
+    ("maize_gemm_bf16_mt256_nn_h128r3_splitk", 100, 515, 2056, NN), # (odd N: the last element of B is patched into the landed tile)
+    ("maize_gemm_bf16_mt256_nt_h128r3_splitk", 140, 264, 3080, NT),
     ("maize_gemm_bf16_mt256_nt_h128r3_gen", 257, 264, 328, NT),
     ("maize_gemm_bf16_mt256_nn_h128r3_gen", 130, 520, 456, NN),
     ("maize_gemm_bf16_mt256_nn_splitk", 64, 520, 2056, NN),
