@@ -168,7 +168,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr int EB = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : 6;  // the eighth the barrier stands in front of
     // MFMA slots between direct-to-LDS requests (an 8-bit MFMA is twice as long; with 128-row tiles its step has 32 slots
     // only, and one request per slot leaves the last of the twelve 18 slots to land)
-    constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : DMA_STRIDE;
+    // (three stages, 16-bit: the requests have a step more to land, and one every four slots holds up the MFMAs a little
+    // less than one every three: 0-5 % in a same-box A/B; one every one or two slots costs 3-20 % on either ring)
+    constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? (R3 ? 4 : 3) : DMA_STRIDE;
     constexpr int AFTER = 16 * (NE - EB);               // MFMA slots of a step behind its barrier
     constexpr int NP = PA + 8;                          // pieces per wave and K tile
     static_assert(!R3 || NP == 12, "the counted waits of the three-stage ring assume twelve pieces per K tile");

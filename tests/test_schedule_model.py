@@ -30,7 +30,7 @@ class Hazard(AssertionError):
 
 # how the K step numbers its MFMA slots and places the requests (16 pieces per wave and K tile with 256-row tiles, 12
 # with 128-row tiles; AFTER = the slots of a step behind its barrier: 32, or 16 with 128-row tiles)
-MT256_SLOT_FACTS = ("constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : DMA_STRIDE;", "constexpr int AFTER = 16 * (NE - EB);",
+MT256_SLOT_FACTS = ("constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? (R3 ? 4 : 3) : DMA_STRIDE;", "constexpr int AFTER = 16 * (NE - EB);",
                     "constexpr int NP = PA + 8;", "constexpr int PA = BMT / 32;",
                     "constexpr int NE = (IS8 && H128) ? 2 : (IS8 || H128) ? 4 : 8;",
                     "constexpr int EB = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : 6;",
@@ -324,7 +324,7 @@ H128R3_LINES = ('if (R3) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\\n\\ts_bar
                 'static_assert(!R3 || NP == 12, "the counted waits of the three-stage ring assume twelve pieces per K tile");')
 
 
-def h128r3_wave_program(nk, nt, barrier_at=3, ds=3, keep=12, drop_read=None):
+def h128r3_wave_program(nk, nt, barrier_at=3, ds=4, keep=12, drop_read=None):
     src = open(os.path.join(KDIR, "gemm_mt256.hpp")).read()
     for fact in MT256_SLOT_FACTS + H128_READ_LINES + H128R3_LINES:
         assert fact in src, fact
