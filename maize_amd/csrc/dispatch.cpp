@@ -270,9 +270,9 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
 // rounding not to matter.
 bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles) {
     const uint32_t nk = cdiv(k, kstep);                         // (an 8-bit step, 128 deep, is as long as a 16-bit one)
-    // 8-bit operands: from 24 steps (E4M3 N x K, two -> three stages: 1024 x 4096 x 3072 26.2 -> 23.4 us, x 4096 31.2 -> 27.6,
-    // 768 x 8192 x 8192 58.8 -> 48.6; 2048^3, 16 steps: 17.6 -> 18.9)
-    return nk >= (kstep == 128u ? 24u : 28u) && (nk >= 48u || half_tiles >= 48u);
+    // 8-bit operands: from 18 steps (E4M3 N x K, two -> three stages: 1024 x 4096 x 2560 21.3 -> 19.4 us, x 4096 31.1 -> 25.4,
+    // 768 x 8192 x 8192 58.8 -> 46.7; 2048^3, 16 steps: 17.5 either way)
+    return nk >= (kstep == 128u ? 18u : 28u) && (nk >= 48u || half_tiles >= 48u);
 }
 // What a K step of a 128-row tile costs, in steps of the 256-row kernel at the power limit (~ microseconds): 0.67 on two
 // ring stages, 0.52 on three -- except for K ranges of a row-major B on three stages, i.e. long ranges, which measure

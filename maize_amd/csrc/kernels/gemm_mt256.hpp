@@ -145,8 +145,8 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 // has landed, the twelve requests of tile t+2 -- younger -- stay in flight.  Three steps per trip, the step count rounded
 // up to a multiple of three with all-zero tiles.  B's third stage lies 64 KiB behind the first, past the reads' 16-bit
 // offset field, and has base registers of its own.
-// 8-bit operands on three stages: A's fragment buffer goes with the stage (three of them), all twelve pieces of tile
-// t+3 go out behind the barrier of step t, same wait.
+// 8-bit operands on three stages: A's fragment buffer goes with the stage (three of them), the twelve pieces of tile
+// t+3 go out one every two slots from the barrier of step t on (seven behind it, five in front of the next), same wait.
 template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
@@ -169,8 +169,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // MFMA slots between direct-to-LDS requests (an 8-bit MFMA is twice as long; with 128-row tiles its step has 32 slots
     // only, and one request per slot leaves the last of the twelve 18 slots to land)
     // (three stages, 16-bit: the requests have a step more to land, and one every four slots holds up the MFMAs a little
-    // less than one every three: 0-5 % in a same-box A/B; one every one or two slots costs 3-20 % on either ring)
-    constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? (R3 ? 4 : 3) : DMA_STRIDE;
+    // less than one every three: 0-5 % in a same-box A/B; one every one or two slots costs 3-20 % on either ring;
+    // 8-bit: one every two slots instead of every slot, 4-11 %)
+    constexpr int DS = (IS8 && H128) ? (R3 ? 2 : 1) : IS8 ? 2 : H128 ? (R3 ? 4 : 3) : DMA_STRIDE;
     constexpr int AFTER = 16 * (NE - EB);               // MFMA slots of a step behind its barrier
     constexpr int NP = PA + 8;                          // pieces per wave and K tile
     static_assert(!R3 || NP == 12, "the counted waits of the three-stage ring assume twelve pieces per K tile");

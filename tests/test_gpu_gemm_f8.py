@@ -420,7 +420,7 @@ def test_dispatch_of_8bit_products(ctx):
     assert pick(4096, 4104, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_trb"      # ... N % 16: transposed copy
     assert pick(2048, 2048, 2048, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_h128_gen"      # half a round of 128-row tiles, 16 K steps
     assert pick(1024, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_h128r3_gen"    # ... 32 K steps: three ring stages
-    assert pick(1024, 4096, 3072, mz.LAYOUT_NN, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nn_h128r3_gen"    # (from 24 steps on)
+    assert pick(1024, 4096, 2304, mz.LAYOUT_NN, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nn_h128r3_gen"    # (from 18 steps on)
     assert pick(4096, 4096, 4104, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_packed"   # K % 16: padded copies
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3, lda=4104) == "maize_gemm_e4m3_mt256_nt_packed"
     assert pick(64, 64, 64, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_bf16_wave32"

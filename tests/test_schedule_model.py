@@ -30,7 +30,7 @@ class Hazard(AssertionError):
 
 # how the K step numbers its MFMA slots and places the requests (16 pieces per wave and K tile with 256-row tiles, 12
 # with 128-row tiles; AFTER = the slots of a step behind its barrier: 32, or 16 with 128-row tiles)
-MT256_SLOT_FACTS = ("constexpr int DS = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? (R3 ? 4 : 3) : DMA_STRIDE;", "constexpr int AFTER = 16 * (NE - EB);",
+MT256_SLOT_FACTS = ("constexpr int DS = (IS8 && H128) ? (R3 ? 2 : 1) : IS8 ? 2 : H128 ? (R3 ? 4 : 3) : DMA_STRIDE;", "constexpr int AFTER = 16 * (NE - EB);",
                     "constexpr int NP = PA + 8;", "constexpr int PA = BMT / 32;",
                     "constexpr int NE = (IS8 && H128) ? 2 : (IS8 || H128) ? 4 : 8;",
                     "constexpr int EB = (IS8 && H128) ? 1 : IS8 ? 2 : H128 ? 3 : 6;",
@@ -429,7 +429,7 @@ def test_8bit_half_height_tile_schedule_is_hazard_free(nk, tr):
     ops, steps = h128_f8_wave_program(nk, tr)
     last_tile = check_two_stage(ops, steps, [8 + nbr, 8 + 2 * nbr], parts=2, pieces=12)
     assert steps <= last_tile <= steps + 1
-    ops, steps = h128_f8_wave_program(nk, tr, nst=3)
+    ops, steps = h128_f8_wave_program(nk, tr, nst=3, ds=2)
     last_tile = check_two_stage(ops, steps, [8 + nbr, 8 + 2 * nbr], parts=2, pieces=12, nst=3)
     assert steps + 1 <= last_tile <= steps + 2
 
@@ -442,9 +442,11 @@ def test_8bit_half_height_tile_checker_rejects_broken_schedules():
     with pytest.raises(Hazard):                 # requests three slots apart: the last ones would never be issued
         check_two_stage(*h128_f8_wave_program(8, False, ds=3), [16, 24], parts=2, pieces=12)
     with pytest.raises(Hazard):                 # three stages, a wait that leaves thirteen requests in flight
-        check_two_stage(*h128_f8_wave_program(9, False, nst=3, keep=13), [16, 24], parts=2, pieces=12, nst=3)
+        check_two_stage(*h128_f8_wave_program(9, False, nst=3, ds=2, keep=13), [16, 24], parts=2, pieces=12, nst=3)
     with pytest.raises(Hazard):                 # three stages, barrier in front of the first eighth
-        check_two_stage(*h128_f8_wave_program(9, False, nst=3, barrier_at=0), [16, 24], parts=2, pieces=12, nst=3)
+        check_two_stage(*h128_f8_wave_program(9, False, nst=3, ds=2, barrier_at=0), [16, 24], parts=2, pieces=12, nst=3)
+    with pytest.raises(Hazard):                 # three stages, requests three slots apart: the last two would never be issued
+        check_two_stage(*h128_f8_wave_program(9, False, nst=3, ds=3), [16, 24], parts=2, pieces=12, nst=3)
 
 
 # ---------------------------------------------------------------------------------------
