@@ -278,7 +278,8 @@ bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles) {
 // ring stages, 0.52 on three -- except for K ranges of a row-major B on three stages, i.e. long ranges, which measure
 // 0.82-0.91 whatever share of the chip is at work (1024 x 4096 x 14336 in two ranges 123.6 us, N x K 101.5;
 // 512 x 8192 x 8192 78.6 / 66.2; 384 x 6144 x 4096 44.4 / 35.0), so that whole tiles or the 256-row split win there.
-double h128_step(bool three, bool split, bool nt) { return !three ? 0.67 : (split && !nt) ? 0.85 : 0.52; }
+// (16-bit operands only: E4M3 K x N, 384 x 8192 x 8192 in two ranges 36.6 us against 42.2 whole and 44.0 in 256-row tiles.)
+double h128_step(bool three, bool split, bool nt, bool bits8) { return !three ? 0.67 : (split && !nt && !bits8) ? 0.85 : 0.52; }
 // Returns 0: the 256-row kernels; 1: 128-row tiles, whole K; >= 2: 128-row tiles in that many K ranges.
 uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
     const uint32_t resident = cus >= 8u ? cus - cus % 8u : cus;
@@ -293,7 +294,7 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     // a long K: the three-stage kernels, steps in threes (2048^3 28.6 -> 24.9 us, 1024 x 4096 x 4096 51.1 -> 42.0,
     // 640 x 8192 x 4096 N x K 60.4 -> 45.9)
     const bool three = h128_three_stages(s.k, kstep, half_tiles);
-    const double whole = 8.0 + scale * h128_step(three, false, s.nt) * (three ? 3u * cdiv(nk, 3u) : nk);
+    const double whole = 8.0 + scale * h128_step(three, false, s.nt, kstep == 128u) * (three ? 3u * cdiv(nk, 3u) : nk);
     double best = 0.9 * whole;                                     // splitting has to win 10 %
     uint32_t best_ks = 1;
     const double elems = (double)s.m * s.n * batch;
@@ -307,13 +308,16 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
             // (ranges long enough run on the three-stage kernels, in threes)
             const uint32_t r = cdiv(nk, ks);
             const bool three_r = h128_three_stages(r * kstep, kstep, half_tiles * ks);
-            const double loop = scale * h128_step(three_r, true, s.nt) * (three_r ? 3u * cdiv(r, 3u) : r);
+            const double loop = scale * h128_step(three_r, true, s.nt, kstep == 128u) * (three_r ? 3u * cdiv(r, 3u) : r);
             const double t = 8.0 + loop + 6.0 + (1.2e-6 * elems + 0.15) * ks;
             if (t < best) { best = t; best_ks = ks; }
         }
     if (best_ks == 1u) best = whole;
-    // (a tie goes to the tiles: the model flatters large splits, 768 x 8192 x 8192 109.6 us in two ranges, 94.4 here)
-    return best < 1.03 * other ? best_ks : 0u;
+    // (a tie goes to the tiles: the model flatters large splits, 768 x 8192 x 8192 109.6 us in two ranges, 94.4 here; more
+    // so with 8-bit operands, whose fixed terms it overrates: E4M3 N x K, 46 mid-size shapes with every candidate by name,
+    // the two it gave to the 256-row split were both faster in tiles -- 256 x 2048 x 2048 18.5 against 14.3-15.9 us,
+    // 768 x 4096 x 14336 55.4 against 50.1)
+    return best < (kstep == 128u ? 1.10 : 1.03) * other ? best_ks : 0u;
 }
 bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && bf16_in(d); }
 bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && bf16_in(d); }
