@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BF16 GEMM path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5|m64|sq2048|f8|f8n|f8s|f32|f64] [--kernel NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1..cfg5|m64|sq2048|mid|f8|f8n|f8s|f32|f64] [--kernel NAME]
 
 A step is one launch of maize_hip_gemm_bf16 (maize_hip_gemm_bf16_ex for the 8-bit, fp32 and fp64
 configurations) on synthetic, seeded inputs that are already resident in HBM.  Prints ONE JSON line:
@@ -33,7 +33,7 @@ TRAFFIC_SOURCE = "profiles/hbm_traffic_fetch_write_size.md"
 MEASURED_TRAFFIC = {"cfg1": ("maize_gemm_bf16_mt256_nn", 235.2e6), "cfg2": ("maize_gemm_bf16_mt256_nn_edge", 275.1e6),
                     "cfg3": ("maize_gemm_bf16_mt256_nt", 1746.3e6), "cfg4": ("maize_gemm_bf16_skinny_nn", 126.5e6),
                     "m64": ("maize_gemm_bf16_skinny_nn_m64", 153.1e6),
-                    "cfg5": ("maize_gemm_bf16_mt256_nn", 1074.3e6), "sq2048": ("maize_gemm_bf16_mt256_nn_h128r3", 58.9e6), "f8": ("maize_gemm_e4m3_mt256_nt", 134.5e6),
+                    "cfg5": ("maize_gemm_bf16_mt256_nn", 1074.3e6), "sq2048": ("maize_gemm_bf16_mt256_nn_h128r3", 58.9e6), "mid": ("maize_gemm_bf16_mt256_nt_h128r3", 109.2e6), "f8": ("maize_gemm_e4m3_mt256_nt", 134.5e6),
                     "f8n": ("maize_gemm_e4m3_mt256_nn", 134.5e6),
                     "f8s": ("maize_gemm_e4m3_skinny_nt", 67.2e6), "f32": ("maize_gemm_f32_mt128_nn", 828.9e6),
                     "f64": ("maize_gemm_f64_mt128_nn", 3162.3e6)}
@@ -56,6 +56,10 @@ CONFIGS = {
     # One product of cfg5's batch alone: 64 tiles of 256 x 256 on 256 compute units -- the dispatcher takes 128 x 256 tiles.
     "sq2048": dict(m=2048, n=2048, k=2048, nt=0, batch=1, da=("uniform",), db=("uniform",), bound="mfma",
                    label="bf16 GEMM 2048x2048x2048 NN, uniform[-1,1)"),
+    # A prefill-sized product against a 4096 x 4096 weight stored N x K: 128 tiles of 128 x 256, 64 K steps -- the
+    # three-stage form of the 128-row kernel.
+    "mid": dict(m=1024, n=4096, k=4096, nt=1, batch=1, da=("normal", 1.0), db=("normal", 0.02), bound="mfma",
+                label="bf16 GEMM 1024x4096x4096 NT, A~N(0,1), B~N(0,0.02)"),
     # Beside the five bf16 configurations: the same product on 8-bit operands (E4M3), both K-contiguous.
     "f8": dict(m=4096, n=4096, k=4096, nt=1, batch=1, da=("uniform",), db=("uniform",), bound="mfma", in_type="e4m3",
                label="E4M3 GEMM 4096x4096x4096 NT (bf16 C), uniform[-1,1) rounded to E4M3"),
@@ -344,7 +348,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", default=None, choices=sorted(CONFIGS) + ["copy", "energy", "energy-vendor-child"],
-                    help="cfg1..cfg5: a benchmark configuration; m64: 64x14336x4096; sq2048: 2048^3 (half a round of tiles); f8, f8n, f8s: 4096^3 (B stored N x K, K x N) and 16x14336x4096 on E4M3 operands; f32, f64: 4096^3 on fp32 / fp64 operands; copy: the 256 MiB copy "
+                    help="cfg1..cfg5: a benchmark configuration; m64: 64x14336x4096; sq2048: 2048^3 (half a round of tiles); mid: 1024x4096x4096 N x K; f8, f8n, f8s: 4096^3 (B stored N x K, K x N) and 16x14336x4096 on E4M3 operands; f32, f64: 4096^3 on fp32 / fp64 operands; copy: the 256 MiB copy "
                          "used to scale HBM counters; energy: board power x time per 4096^3 launch for this library's kernels and register-only MFMA loops")
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
