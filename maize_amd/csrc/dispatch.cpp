@@ -939,7 +939,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         const int fk = kernel_index(name);
         if (fk >= 0 && kKernels[fk].supports(d) && s.n >= 64 && s.k >= 1024) return (uint32_t)fk;
         // 17 .. 64 rows: the same stream with 2 or 4 row groups (A through LDS), where B is what bounds the product.
-        if (s.m > 16u && s.m <= 64u && s.k >= 2048u && s.n >= (s.m <= 32u ? 1024u : 10240u)) {
+        if (s.m > 16u && s.m <= 64u && s.k >= 2048u && s.n >= (s.m <= 32u ? 1024u : 8192u)) {   // (E4M3 64 x 8192 x 8192: K x N 19.9 us against 25.9 in 128-row tiles cut over K, N x K 21.5 / 22.9)
             std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nt_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.m <= 32u ? "m32" : "m64");
             const int fm = kernel_index(name);
             if (fm >= 0 && kKernels[fm].supports(d) && plan_fits(kKernels[fm], d, compute_units)) return (uint32_t)fm;
@@ -948,7 +948,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nn", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int gk = kernel_index(name);
         if (gk >= 0 && kKernels[gk].supports(d) && s.n >= 64 && s.k >= 1024) return (uint32_t)gk;
-        if (s.m > 16u && s.m <= 64u && s.k >= 2048u && s.n >= (s.m <= 32u ? 1024u : 10240u)) {
+        if (s.m > 16u && s.m <= 64u && s.k >= 2048u && s.n >= (s.m <= 32u ? 1024u : 8192u)) {   // (E4M3 64 x 8192 x 8192: K x N 19.9 us against 25.9 in 128-row tiles cut over K, N x K 21.5 / 22.9)
             std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nn_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.m <= 32u ? "m32" : "m64");
             const int gm = kernel_index(name);
             if (gm >= 0 && kKernels[gm].supports(d) && plan_fits(kKernels[gm], d, compute_units)) return (uint32_t)gm;
@@ -999,16 +999,17 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // 17 .. 64 rows: the same stream with 2 or 4 row groups, where it beats the macro-tile kernel cut over K
     // (measured): a long K, and enough slabs that few K ranges cover the chip -- the last workgroup of a slab adds
     // ranges x row groups x 16 KiB alone.  32 rows: 1024 columns up (32 x 1024 x 8192: 20.3 against 25.1 us,
-    // 32 x 14336 x 4096: 25.1 against 34.8); 64 rows: 10240 columns up (64 x 14336 x 4096: 30.8 against 37.3 us, but
+    // 32 x 14336 x 4096: 25.1 against 34.8); 64 rows: 12288 columns up (64 x 14336 x 4096: 28.4 against 30.6 us in
+    // 128-row tiles cut over K, N x K 27.2 against 28.8; but 64 x 11008 x 4096: 31.1 against 26.7, N x K 29.1 against 25.1;
     // 64 x 4096 x 4096: 26.3 against 23.2, and 64 x 8192 x 8192 N x K: 35.6 against 33.3).  The same thresholds serve
     // the kernels for weights stored N x K below.
-    if (s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 10240u)) {
+    if (s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 12288u)) {
         const int sm = kernel_index(s.m <= 32u ? "maize_gemm_bf16_skinny_nn_m32" : "maize_gemm_bf16_skinny_nn_m64");
         if (sm >= 0 && kKernels[sm].supports(d) && plan_fits(kKernels[sm], d, compute_units)) return (uint32_t)sm;
     }
     const int st = kernel_index("maize_gemm_bf16_skinny_nt");
     if (st >= 0 && kKernels[st].supports(d) && s.n >= 64 && s.k >= 512) return (uint32_t)st;
-    if (s.nt && s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 10240u)) {
+    if (s.nt && s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 12288u)) {
         const int sm = kernel_index(s.m <= 32u ? "maize_gemm_bf16_skinny_nt_m32" : "maize_gemm_bf16_skinny_nt_m64");
         if (sm >= 0 && kKernels[sm].supports(d) && plan_fits(kKernels[sm], d, compute_units)) return (uint32_t)sm;
     }
