@@ -122,7 +122,11 @@ def cpu_baseline(cfg, a, b_storage, got, seconds_target=12.0):
                                           nthreads=threads, elem=elem)
         r = min(rows, 64)
         parity = pyoracle.compare(got[:r * n], ref[:r], f64[:r], ab, k, coeff=coeff)
+        tight = pyoracle.tight_violations(parity) if coeff is None else None      # (16-bit operands: the bar below the floor)
         parity = {key: parity[key] for key in ("n", "max_ulp", "n_gt1ulp", "n_fail", "max_floor_ratio", "max_err_over_abs")}
+        if tight is not None:
+            parity.update({"gt1ulp_rate": parity["n_gt1ulp"] / max(1, parity["n"]), "gt1ulp_rate_bar": pyoracle.TIGHT_GT1ULP_RATE,
+                           "max_floor_ratio_bar": pyoracle.floor_ratio_bar(k), "sums_as_accurate_as_fp32": not tight})
     return out, parity
 
 
@@ -190,8 +194,9 @@ class PowerSampler:
     """Board power from sysfs (hwmon power1_input or power1_average, microwatts), sampled every 20 ms on a thread
     while the GPU works.  No GPU runtime call is made here."""
 
-    def __init__(self):
+    def __init__(self, period=0.02):
         import glob
+        self.period = period
         cands = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")) or \
             sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"))
         self.path = cands[0] if cands else None
@@ -213,7 +218,7 @@ class PowerSampler:
                 w = self.read()
                 if w is not None:
                     self.samples.append((time.time(), w))
-                time.sleep(0.02)
+                time.sleep(self.period)
         self._t = threading.Thread(target=loop, daemon=True)
         self._t.start()
         return self
@@ -225,6 +230,37 @@ class PowerSampler:
     def mean_between(self, t0, t1):
         w = [x for t, x in self.samples if t0 <= t <= t1]
         return sum(w) / len(w) if w else None
+
+    def count_between(self, t0, t1):
+        return sum(1 for t, _ in self.samples if t0 <= t <= t1)
+
+
+def box_ceiling(mz, ctx, stream, launches=50):
+    """What this box's matrix pipe does right now with no data movement at all: a register-only loop of
+    v_mfma_f32_16x16x32_bf16 on random operands, 256 workgroups x 4 waves x 512 rounds x 131072 multiply-adds = the
+    multiply-adds of 4096^3, timed by HIP events on `stream` straight after the timed region (same clocks, same
+    temperature).  A slow or hot box shows up here as a slow ceiling.  Returns microseconds per launch."""
+    import ctypes as C
+
+    class LoopArgs(C.Structure):
+        _fields_ = [("out", C.c_void_p), ("iters", C.c_uint32), ("zero", C.c_uint32)]
+
+    out = ctx.malloc(4096)
+    kern = mz.new_hip_kernel("maize_probe_mfma_loop_16x16x32").with_launch_bounds_1d(256).finalize().compile(mz.Gfx.Gfx950, ctx)
+    args = LoopArgs(out.ptr, 512, 0)
+    ev0, ev1 = ctx.event(), ctx.event()
+    for _ in range(10):
+        kern.launch((256, 1, 1), args, stream=stream)
+    ev0.record(stream)
+    for _ in range(launches):
+        kern.launch((256, 1, 1), args, stream=stream)
+    ev1.record(stream)
+    ctx.sync()
+    us = ev0.elapsed_ms(ev1) / launches * 1e3
+    ev0.destroy(); ev1.destroy()
+    kern.release()
+    out.free()
+    return us
 
 
 def energy_vendor_child(seconds):
@@ -380,7 +416,8 @@ def main():
         return
     import maize_amd as mz
     ctx = mz.Context(0)
-    line = measure(mz, ctx, args.config, args.steps, args.warmup, args.kernel, args.rotate, not args.no_cpu)
+    bf16_mfma = CONFIGS[args.config]['bound'] == 'mfma' and CONFIGS[args.config].get('in_type') is None
+    line = measure(mz, ctx, args.config, args.steps, args.warmup, args.kernel, args.rotate, not args.no_cpu, ceiling=bf16_mfma)
     if args.others:
         # The other benchmark configurations, shorter runs, same process: reported beside the headline.
         others = {}
@@ -397,7 +434,7 @@ def main():
     ctx.close()
 
 
-def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
+def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu, ceiling=False):
     """One configuration: untimed clock ramp and warm-up, then exactly `steps` launches timed by the wall
     clock (sync on both sides) and by HIP events on the launch stream.  Returns the JSON line as a dict."""
     class A:  # the names the body below was written against
@@ -454,6 +491,10 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
     for i in range(args.warmup):
         ctx.gemm_bf16(sets[i % nsets][3], stream=stream, kernel=args.kernel)
     ctx.sync()
+    sampler = PowerSampler(period=0.001) if ceiling else None     # (sysfs reads on a host thread; no GPU call)
+    if sampler is not None and sampler.path is not None:
+        sampler.__enter__()
+    wall_t0 = time.time()
     t0 = time.perf_counter()
     ev0.record(stream)
     for i in range(args.steps):
@@ -461,7 +502,12 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
     ev1.record(stream)
     ctx.sync()
     wall = time.perf_counter() - t0
+    wall_t1 = time.time()
     ev_ms = ev0.elapsed_ms(ev1)
+    # The box's own ceiling, straight behind the timed region: the same multiply-adds from registers only.
+    ceiling_us = box_ceiling(mz, ctx, stream) if ceiling else None
+    if sampler is not None and sampler.path is not None:
+        sampler.__exit__()
 
     got = sets[(args.steps - 1) % nsets][2].download(WIDE[wide][0] if wide else np.uint16, count=m * n)
     ms_per_step = wall * 1e3 / args.steps
@@ -482,6 +528,17 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu):
         roof["traffic_source"] = f"{TRAFFIC_SOURCE} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on {kernel}, an earlier session; not measured in this run)"
     roof["kernel"] = kernel
     roof["kernel_avg_us"] = kern_ms * 1e3
+    if ceiling_us is not None:
+        # the register-only loop does 4096^3 multiply-adds; scaled to this workload's
+        scaled = ceiling_us * flops / (2.0 * 4096 ** 3)
+        roof["box_ceiling_us"] = scaled
+        roof["box_ceiling_frac_of_peak"] = flops / (scaled * 1e-6) / 1e12 / peak_flops
+        roof["frac_of_box_ceiling"] = scaled / (kern_ms * 1e3)
+        roof["box_ceiling_source"] = ("maize_probe_mfma_loop_16x16x32: v_mfma_f32_16x16x32_bf16 from registers only, uniform random "
+                                      "operands, the workload's multiply-adds, 50 launches straight after the timed region")
+        watts = sampler.mean_between(wall_t0, wall_t1) if sampler.path else None
+        roof["board_watts_timed_region"] = watts
+        roof["board_watts_samples"] = sampler.count_between(wall_t0, wall_t1) if sampler.path else 0
     roof["algorithmic_flop"] = flops
     roof["algorithmic_bytes"] = alg_bytes
 

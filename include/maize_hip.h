@@ -215,6 +215,18 @@ int32_t maize_hip_gemm_bf16(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, voi
 /* 64 KiB of ticket counters + 256 fp32 partial tiles of 256 x 256: one round of split-K work items on 256 compute units. */
 #define MAIZE_NOALLOC_MAX_WORKSPACE_BYTES ((64u << 20) + (64u << 10))
 int32_t maize_hip_gemm_bf16_noalloc(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream);
+/* Recovery for that array (no counterpart in the reference either): zeroes its 64 KiB of ticket counters on `stream`
+ * (hipMemsetAsync; allocates nothing).  The kernels return every counter they use to zero, so this is only needed
+ * after calls that overlapped on one GPU against the rule above, or after a launch that was aborted: until then every
+ * later maize_hip_gemm_bf16_noalloc on that GPU may find counters that are not zero.  Call it with no
+ * maize_hip_gemm_bf16_noalloc in flight on the GPU, and outside graph capture. */
+int32_t maize_hip_noalloc_reset(maize_ctx_t* ctx, void* stream);
+/* The kernels for 17..64 rows that share the additions of their K ranges let a workgroup wait for the others of its
+ * slab for at most this many microseconds (default 30, or MAIZE_HIP_SPLIT_WAIT_US as read once when first needed; at
+ * most 1000; 0: nobody waits).  Process-wide; results do not depend on it (the sums are formed in range order by
+ * whoever forms them).  For diagnosis and tests; no counterpart in the reference. */
+void maize_hip_set_split_wait_us(uint32_t us);
+uint32_t maize_hip_get_split_wait_us(void);
 /* Same, but with the kernel named by the caller (see maize_hip_kernel_name);
  * fails with MAIZE_ERR_KERNEL if that kernel cannot run the descriptor. */
 int32_t maize_hip_gemm_bf16_with(maize_ctx_t* ctx, const maize_gemm_desc_t* desc,

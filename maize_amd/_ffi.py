@@ -15,7 +15,7 @@ EXPORTS = (
     "maize_hip_last_error", "maize_hip_ctx_create", "maize_hip_ctx_destroy", "maize_hip_device_info",
     "maize_hip_module_load", "maize_hip_module_unload", "maize_hip_kernel_get", "maize_hip_kernel_release",
     "maize_hip_launch", "maize_hip_embedded_code_object", "maize_hip_gemm_bf16", "maize_hip_gemm_bf16_with",
-    "maize_hip_gemm_bf16_noalloc",
+    "maize_hip_gemm_bf16_noalloc", "maize_hip_noalloc_reset", "maize_hip_set_split_wait_us", "maize_hip_get_split_wait_us",
     "maize_hip_gemm_select", "maize_hip_gemm_plan", "maize_hip_gemm_validate",
     "maize_hip_gemm_bf16_ex", "maize_hip_gemm_ex_validate", "maize_hip_gemm_ex_plan", "maize_hip_gemm_ex_tail_rows", "maize_hip_kernel_count", "maize_hip_kernel_name",
     "maize_hip_kernel_supports", "maize_hip_malloc", "maize_hip_free", "maize_hip_memcpy_h2d",
@@ -127,6 +127,9 @@ def lib():
         "maize_hip_gemm_bf16": (i32, [vp, P(GemmDescT), vp]),
         "maize_hip_gemm_bf16_with": (i32, [vp, P(GemmDescT), C.c_char_p, vp]),
         "maize_hip_gemm_bf16_noalloc": (i32, [vp, P(GemmDescT), vp]),
+        "maize_hip_noalloc_reset": (i32, [vp, vp]),
+        "maize_hip_set_split_wait_us": (None, [u32]),
+        "maize_hip_get_split_wait_us": (u32, []),
         "maize_hip_gemm_select": (i32, [vp, P(GemmDescT), C.c_char_p, sz]),
         "maize_hip_gemm_plan": (i32, [P(GemmDescT), C.c_char_p, u32, P(GemmPlanT)]),
         "maize_hip_gemm_validate": (i32, [P(GemmDescT)]),

@@ -96,6 +96,11 @@ class Context:
         fixed per-GPU array (maize_hip_gemm_bf16_noalloc); raises MaizeError when the plan needs more than it holds."""
         check(_ffi.lib().maize_hip_gemm_bf16_noalloc(self._h, C.byref(desc), stream))
 
+    def noalloc_reset(self, stream=None):
+        """Zeroes the ticket counters of this GPU's fixed scratch array (maize_hip_noalloc_reset): the recovery after
+        overlapping or aborted gemm_bf16_noalloc calls."""
+        check(_ffi.lib().maize_hip_noalloc_reset(self._h, stream))
+
     def gemm_select(self, desc):
         buf = C.create_string_buffer(128)
         check(_ffi.lib().maize_hip_gemm_select(self._h, C.byref(desc), buf, len(buf)))
@@ -235,6 +240,14 @@ def gemm_tail_rows(desc, compute_units=256):
     rows = C.c_uint32()
     check(_ffi.lib().maize_hip_gemm_ex_tail_rows(C.byref(x), compute_units, C.byref(rows)))
     return rows.value
+
+
+def set_split_wait_us(us):
+    """Process-wide bound (microseconds, at most 1000) of the wait inside the few-row kernels that share their
+    split-K additions (maize_hip_set_split_wait_us); returns the bound that was in force."""
+    old = _ffi.lib().maize_hip_get_split_wait_us()
+    _ffi.lib().maize_hip_set_split_wait_us(int(us))
+    return old
 
 
 def kernel_names():

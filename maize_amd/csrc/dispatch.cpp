@@ -1,9 +1,11 @@
 #include "dispatch.hpp"
 
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 namespace maize {
 namespace {
@@ -657,15 +659,10 @@ uint32_t skinny_ksplit(const Dims& s, uint32_t batch, uint32_t compute_units) {
 // 4096 NN 30.9 -> 28.3 us, NT 28.8 -> 27.1, E4M3 20.4 -> 18.3; 32 x 2048 x 8192 NT in 16 ranges 20.1 -> 14.2; but
 // 16 x 4096 x 14336 in 16 ranges NN 26.8 -> 31.1, NT 26.0 -> 28.5).  A workgroup
 // waits for the others at most this long (their skew: the grids keep a slab's workgroups resident together; the bound
-// matters only when something else holds compute units).  MAIZE_HIP_SPLIT_WAIT_US overrides it for diagnosis (0: nobody
-// waits, the last to arrive adds everything).
-static uint32_t split_wait_us() {
-    if (const char* e = std::getenv("MAIZE_HIP_SPLIT_WAIT_US")) {
-        const long v = std::strtol(e, nullptr, 10);
-        return v < 0 ? 0u : v > 60000 ? 60000u : (uint32_t)v;
-    }
-    return 30u;
-}
+// matters only when something else holds compute units).  The bound is a process-wide setting: 30 us unless
+// MAIZE_HIP_SPLIT_WAIT_US said otherwise when the library first planned such a launch (read once), or
+// set_split_wait_us() has been called since; never more than 1 ms of polling (0: nobody waits, the last to arrive
+// adds everything).  Results do not depend on it.
 static void share_additions(LaunchDims* ld, uint32_t rows, uint32_t ks, uint64_t slabs) {
     ld->wait_us = 0;
     if (rows >= 32u && ks >= 2u && ks <= 16u && (rows / 16u) * ks >= 16u && slabs <= 8192u) {
@@ -1115,6 +1112,25 @@ uint32_t tail_split_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units) 
     if (t_bottom > 0.75 * t_round) return 0;
     // the rows below start on a 16-byte boundary like the matrix itself (leading dimensions are multiples of 8)
     return tm_top * 256u;
+}
+
+// The wait bound of the few-row kernels that share their split-K additions (see share_additions).
+std::atomic<uint32_t> g_split_wait_us{0xFFFFFFFFu};        // not read from the environment yet
+static uint32_t clamp_wait(long v) { return v < 0 ? 0u : v > (long)kMaxSplitWaitUs ? kMaxSplitWaitUs : (uint32_t)v; }
+void set_split_wait_us(uint32_t us) { g_split_wait_us.store(clamp_wait((long)us), std::memory_order_relaxed); }
+uint32_t split_wait_us() {
+    uint32_t v = g_split_wait_us.load(std::memory_order_relaxed);
+    if (v == 0xFFFFFFFFu) {
+        static std::once_flag once;
+        std::call_once(once, [] {
+            uint32_t init = 30u;
+            if (const char* e = std::getenv("MAIZE_HIP_SPLIT_WAIT_US")) init = clamp_wait(std::strtol(e, nullptr, 10));
+            uint32_t expect = 0xFFFFFFFFu;
+            g_split_wait_us.compare_exchange_strong(expect, init, std::memory_order_relaxed);   // (a setter may have come first)
+        });
+        v = g_split_wait_us.load(std::memory_order_relaxed);
+    }
+    return v;
 }
 
 }  // namespace maize

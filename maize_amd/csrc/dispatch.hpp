@@ -41,6 +41,11 @@ struct LaunchDims {
     uint32_t n_padded, k_padded;
 };
 constexpr size_t kTicketBytes = 16384 * 4;  // ticket counters at the start of a workspace
+// Bound of the in-kernel wait of the few-row kernels that share their split-K additions (process-wide, see
+// share_additions in dispatch.cpp): at most kMaxSplitWaitUs.
+constexpr uint32_t kMaxSplitWaitUs = 1000;
+void set_split_wait_us(uint32_t us);
+uint32_t split_wait_us();
 
 struct KernelInfo {
     const char* name;

@@ -510,7 +510,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 if (R3) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
                 else    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
                 const uint32_t k_next = R3 ? k_late - (uint32_t)BKE : k_late;  // where tile t+1 starts
-                if (PATCHES && patch_on && K - 1u - k_next < (uint32_t)BKE)    // tile t+1 holds row K - 1 (k_next <= K - 1 here)
+                // tile t+1 holds row K - 1 and belongs to this item's K range (the steps that pad a range to a whole
+                // trip run on zero tiles at or past k_end: there A is zero, and a real Inf in B would make NaN of it)
+                if (PATCHES && patch_on && k_next < k_end && K - 1u - k_next < (uint32_t)BKE)
                     asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)pb + patch_off), "v"(patch_val) : "memory");
                 MAIZE_FENCE();
             }
@@ -581,7 +583,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     // The wait also covers the C stores of the previous tile (loads and stores share the counter).
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    if (PATCHES && patch_on && nk && K - 1u - k_begin < (uint32_t)BKE)        // the item's first K tile is also B's last
+    if (PATCHES && patch_on && k_begin < k_end && K - 1u - k_begin < (uint32_t)BKE)   // the item's first K tile is also B's last
         asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)B0 + patch_off), "v"(patch_val) : "memory");
 #pragma unroll
     for (int r = 0; r < NAR; ++r) read_a(0, 0, 0, r);

@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "noalloc.hpp"
 
 // In host code this name is only a stand-in for the device array (handing it to a kernel would
@@ -28,6 +30,7 @@ namespace {
 constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices];        // per device: address of its copy of `scratch` (NULL: not looked up yet)
 hipError_t g_scratch_err[kMaxDevices];   // ... or why the lookup failed
+std::mutex g_scratch_lock;               // contexts may be created from several threads
 }  // namespace
 
 namespace maize {
@@ -38,6 +41,7 @@ hipError_t noalloc_scratch(int device, void** ptr, size_t* bytes) {
     *ptr = nullptr;
     *bytes = 0;
     if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
     if (!g_scratch_ptr[device] && g_scratch_err[device] == hipSuccess) {
         void* p = nullptr;
         const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));

@@ -527,6 +527,21 @@ static int32_t gemm_launch(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint
                       sizeof args);
 }
 
+// Whether the plan of kernel `idx` for `x` fits the caller's fixed scratch memory; nothing is launched.
+static int32_t fits_fixed(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* x, uint32_t idx, const maize_workspace* fixed) {
+    const maize::KernelInfo& ki = maize::kernel_at(idx);
+    maize::LaunchDims ld;
+    memset(&ld, 0, sizeof ld);
+    if (!ki.plan(*x, (uint32_t)ctx->prop.multiProcessorCount, &ld))
+        return fail(MAIZE_ERR_KERNEL, "gemm: kernel %s cannot run M=%u N=%u K=%u batch=%u (grid limit)", ki.name,
+                    x->gemm.c.nrows, x->gemm.c.ncols, x->gemm.a.ncols, x->gemm.batch);
+    if (ld.workspace_bytes > fixed->bytes)
+        return fail(MAIZE_ERR_ARG, "gemm_noalloc: kernel %s needs %zu bytes of scratch for M=%u N=%u K=%u batch=%u, the fixed "
+                    "scratch array holds %zu (use maize_hip_gemm_bf16, which allocates)", ki.name, (size_t)ld.workspace_bytes,
+                    x->gemm.c.nrows, x->gemm.c.ncols, x->gemm.a.ncols, x->gemm.batch, fixed->bytes);
+    return MAIZE_OK;
+}
+
 static int32_t gemm_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const char* kernel, void* stream,
                        const maize_workspace* fixed) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "gemm: ctx is NULL");
@@ -547,6 +562,8 @@ static int32_t gemm_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const
             rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)top_rows * ldc * csz;
             uint32_t itop, irest;
             if ((rc = select_checked(top, cus, &itop)) != MAIZE_OK || (rc = select_checked(rest, cus, &irest)) != MAIZE_OK) return rc;
+            // Fixed scratch: both products must fit before the first one is launched (a refusal launches nothing).
+            if (fixed && ((rc = fits_fixed(ctx, &top, itop, fixed)) != MAIZE_OK || (rc = fits_fixed(ctx, &rest, irest, fixed)) != MAIZE_OK)) return rc;
             rc = gemm_launch(ctx, &top, itop, stream, fixed);
             if (rc != MAIZE_OK) return rc;
             return gemm_launch(ctx, &rest, irest, stream, fixed);
@@ -575,6 +592,20 @@ int32_t maize_hip_gemm_bf16_noalloc(maize_ctx_t* ctx, const maize_gemm_desc_t* d
     const maize_gemm_ex_desc_t x = widen(*desc);
     return gemm_ex(ctx, &x, nullptr, stream, &ctx->scratch);
 }
+
+int32_t maize_hip_noalloc_reset(maize_ctx_t* ctx, void* stream) {
+    if (!ctx) return fail(MAIZE_ERR_NULL, "noalloc_reset: ctx is NULL");
+    if (!ctx->scratch.ptr)
+        return hip_fail(ctx->scratch_err != hipSuccess ? ctx->scratch_err : hipErrorInvalidSymbol,
+                        "noalloc_reset: the device address of the fixed scratch array (hipGetSymbolAddress)");
+    DeviceGuard guard_;
+    HIP_TRY(guard_.enter(ctx->device));
+    HIP_TRY(hipMemsetAsync(ctx->scratch.ptr, 0, maize::kTicketBytes, (hipStream_t)stream));
+    return MAIZE_OK;
+}
+
+void maize_hip_set_split_wait_us(uint32_t us) { maize::set_split_wait_us(us); }
+uint32_t maize_hip_get_split_wait_us(void) { return maize::split_wait_us(); }
 
 int32_t maize_hip_gemm_bf16(maize_ctx_t* ctx, const maize_gemm_desc_t* desc, void* stream) {
     if (!ctx) return fail(MAIZE_ERR_NULL, "gemm: ctx is NULL");

@@ -283,6 +283,7 @@ def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16, coeff=None):
     return {
         "max_floor_ratio": float(ratio.max()) if ratio.size else 0.0,
         "n": int(got.size),
+        "k": int(k),
         "max_ulp": int(ulp.max()) if ulp.size else 0,
         "n_gt1ulp": int(strict_bad.sum()),
         "n_fail": int(bad.sum()),
@@ -291,6 +292,84 @@ def compare(got_bits, ref_bits, ref_f64, ref_abs, k, elem=BF16, coeff=None):
         "worst_index": worst,
         "first_fail": int(np.argmax(bad)) if bad.any() else -1,
     }
+
+
+
+# ---- the bar below the floor ---------------------------------------------------------------------
+# The floor of compare() is a deterministic worst case (every one of K / 16 fp32 roundings at its largest and all
+# in one direction); a kernel that really accumulates in fp32 uses a thousandth of it (measured: 4096^3 on
+# uniform operands, the worst element beyond 1 ULP sits at 0.001 of its floor, and 2.3e-5 of the elements are
+# beyond 1 ULP at all).  A kernel that lost ten bits in its sums -- partial results of K ranges rounded to a
+# 14-bit significand, say -- would still pass `n_fail == 0`: most elements move by less than one bf16 ULP and the
+# rest stay under the floor.  These two statistics tell the two apart and are asserted wherever the operands are
+# zero-mean random data:
+TIGHT_FLOOR_RATIO = 0.02      # the share of its floor the worst element beyond 1 ULP may use (long K)
+TIGHT_FLOOR_RATIO_K = 48.0    # ... or this over K, if larger
+TIGHT_GT1ULP_RATE = 1e-3      # the share of elements that may be beyond 1 ULP at all (at least 3 elements)
+
+
+def floor_ratio_bar(k):
+    """The floor grows like K * sum|a||b| ~ K^2, the error of fp32 accumulation on zero-mean data like sqrt(K) roundings
+    of partial sums ~ sqrt(K): the share of the floor in use falls like 1 / K.  Measured on the device over ~500 products
+    on uniform operands: the worst element sits at 2.5 / K ... 7.4 / K of its floor (0.035 at K = 72, 0.042 at K = 128,
+    0.023 at K = 328, 0.001 at K = 4096); a kernel whose partial sums keep 14 bits sits at 0.18 (K = 8192) ... 1.3 (K = 512)."""
+    return max(TIGHT_FLOOR_RATIO, TIGHT_FLOOR_RATIO_K / max(1.0, float(k)))
+
+
+def tight_violations(stats):
+    """What of the sensitive statistics of compare() is out of line with fp32 accumulation: a list of strings."""
+    out = []
+    bar = floor_ratio_bar(stats["k"])
+    if stats["max_floor_ratio"] > bar:
+        out.append(f"an element beyond 1 ULP uses {stats['max_floor_ratio']:.3f} of its floor (> {bar:.3f} at K = {stats['k']})")
+    if stats["n_gt1ulp"] > max(3.0, TIGHT_GT1ULP_RATE * stats["n"]):
+        out.append(f"{stats['n_gt1ulp']} of {stats['n']} elements are beyond 1 ULP (> {TIGHT_GT1ULP_RATE:g})")
+    return out
+
+
+def assert_parity(stats, label="", tight=True):
+    """The parity bar on the result of compare(): no element fails, and (tight) the statistics above."""
+    assert stats["n_fail"] == 0, f"{label}: {stats}"
+    if tight:
+        v = tight_violations(stats)
+        assert not v, f"{label}: sums are less accurate than fp32 accumulation: {'; '.join(v)}: {stats}"
+
+
+def sum_of_squares(a, b, m, n, k, layout=NN, lda=None, ldb=None, elem=BF16):
+    """sum_k a[i,k]^2 b[k,j]^2 (M x N, float64) for 16-bit operand views: the variance scale of a sum whose terms
+    are rounded independently."""
+    brows, bcols = (k, n) if layout == NN else (n, k)
+    lda = k if lda is None else lda
+    ldb = bcols if ldb is None else ldb
+    a = np.asarray(a, dtype=np.uint16).ravel()
+    b = np.asarray(b, dtype=np.uint16).ravel()
+    av = bf16_bits_to_f64(np.lib.stride_tricks.as_strided(a, shape=(m, k), strides=(2 * lda, 2)), elem)
+    bv = bf16_bits_to_f64(np.lib.stride_tricks.as_strided(b, shape=(brows, bcols), strides=(2 * ldb, 2)), elem)
+    return (av * av) @ ((bv * bv) if layout == NN else (bv * bv).T)
+
+
+def check_f32(got, exact, scale, k, sumsq=None, alpha=1.0, c_term=0.0):
+    """Parity bar of an fp32 C = alpha * A.B + beta * C_old.  Deterministic: |got - exact| <= (K/16 + 4) 2^-24 scale
+    (scale = |alpha| sum|a||b| + |beta||C_old|).  With `sumsq` (sum a^2 b^2; zero-mean operands) also the statistical
+    one: the K/32 roundings of the accumulation are independent, each at most half an fp32 ULP of a partial sum of
+    the order sqrt(sumsq), and the epilogue rounds alpha * sum and the fused multiply-add once each, so
+        |got - exact| <= 8 sqrt(K/32 + 1) 2^-24 |alpha| sqrt(sumsq) + 4 * 2^-24 (|exact| + c_term),  c_term = |beta C_old|.
+    Returns the worst error / bound ratios and the number of elements over each bound."""
+    got = np.asarray(got, dtype=np.float64)
+    exact = np.asarray(exact, dtype=np.float64)
+    scale = np.asarray(scale, dtype=np.float64)
+    with np.errstate(invalid="ignore", over="ignore"):
+        err = np.abs(got - exact)
+        det = (k / 16.0 + 4.0) * 2.0 ** -24 * scale + 1e-45
+        out = {"n": int(err.size), "worst_over_deterministic": float(np.nanmax(err / det)) if err.size else 0.0,
+               "n_fail": int((~(err <= det)).sum()), "worst_over_statistical": None, "n_fail_statistical": 0}
+        if sumsq is not None:
+            al = abs(float(np.float32(alpha)))
+            stat = 8.0 * np.sqrt(k / 32.0 + 1.0) * 2.0 ** -24 * al * np.sqrt(np.asarray(sumsq, dtype=np.float64)) \
+                + 4.0 * 2.0 ** -24 * (np.abs(exact) + np.asarray(c_term, dtype=np.float64)) + 1e-45
+            out["worst_over_statistical"] = float(np.nanmax(err / stat)) if err.size else 0.0
+            out["n_fail_statistical"] = int((~(err <= stat)).sum())
+    return out
 
 
 # ---- fp32 / fp64 operands ---------------------------------------------------------------------------

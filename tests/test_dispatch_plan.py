@@ -370,3 +370,38 @@ def test_rows_beyond_the_wide_kernels_offsets_are_an_error_not_a_launch():
         with pytest.raises(mz.MaizeError) as e:
             mz.gemm_plan(ex_desc(**kw), compute_units=CUS)
         assert e.value.code == _ffi.MAIZE_ERR_KERNEL
+
+
+def _padding_step_is_the_last_tile_of_b(k, ksplit, steps_per_trip):
+    """True when a K range that is not the last one is padded (to a whole trip of the unrolled loop) with a step
+    that falls on B's last K tile, which belongs to a later range."""
+    nk_all = cdiv(k, 64)
+    per = cdiv(nk_all, ksplit)
+    for z in range(ksplit):
+        kt0 = z * per
+        nk = max(0, min(per, nk_all - kt0))
+        padded = cdiv(nk, steps_per_trip) * steps_per_trip
+        if nk and kt0 + nk < nk_all and kt0 + padded > nk_all - 1:
+            return True
+    return False
+
+
+def test_the_special_value_families_hold_a_range_padded_with_bs_last_tile():
+    """Odd N, row-major B: the kernels write B's last element into the landed K tile that holds row K - 1.  A split
+    whose non-final range is padded with that very tile is the case where the write must not happen (A is zero
+    there, the element may be Inf).  The dispatcher produces such splits on its own; the GPU special-value test has
+    to keep one, whatever the cost model does later."""
+    from tests.test_gpu_special_values import FAMILIES
+    hit = []
+    for name, m, n, k, layout in FAMILIES:
+        if layout != mz.LAYOUT_NN or n % 2 == 0:
+            continue
+        p = mz.gemm_plan(desc(m, n, k), kernel=name, compute_units=CUS)
+        if not p["kernel"].endswith("_splitk") or p["ksplit"] < 2:
+            continue
+        if _padding_step_is_the_last_tile_of_b(k, p["ksplit"], 3 if "r3" in p["kernel"] else 2):
+            hit.append((p["kernel"], name is None))
+    assert any(kern.endswith("_h128_splitk") for kern, _ in hit), hit
+    assert any(kern.endswith("_h128r3_splitk") for kern, _ in hit), hit
+    assert any(kern == "maize_gemm_bf16_mt256_nn_splitk" for kern, _ in hit), hit
+    assert any(auto for _, auto in hit), hit

@@ -388,7 +388,7 @@ def _sampled_entries_check(oracle, got_rows, a_rows_bits, bt_bits, k, label):
     B = mz.bf16.to_f64(bt_bits).reshape(-1, k)
     val, scale = A @ B.T, np.abs(A) @ np.abs(B).T
     s = oracle.compare(got_rows, oracle.bf16_bits_from_f64(val), val, scale, k)
-    assert s["n_fail"] == 0, f"{label}: {s}"
+    oracle.assert_parity(s, label)
 
 
 @pytest.mark.parametrize("which", ["c", "a", "b_nt", "b_nn"])
@@ -425,7 +425,7 @@ def test_operands_past_two_gib(ctx, oracle, which):
             got = np.stack([dc.download(np.uint16, count=n, offset_bytes=int(r) * n * 2) for r in rows])
             ref, f64, ab = oracle.ref_gemm_rows(a, b, m, n, k, rows, layout=layout)
             s = oracle.compare(got, ref, f64, ab, k)
-            assert s["n_fail"] == 0, f"past 2 GiB {which} {took}: {s}"
+            oracle.assert_parity(s, f"past 2 GiB {which} {took}")
     finally:
         da.free(); db.free(); dc.free()
 
@@ -507,7 +507,6 @@ def test_row_group_kernels_share_the_additions_whatever_the_wait(ctx, oracle, ca
     """17 .. 64 rows, 256 KiB or more of partial tiles per slab: the workgroups of a slab share the additions.  Who
     adds which part depends on a bounded wait; the bits must not.  The bound is forced from the host: the default,
     1 us (some workgroups give up, some do not) and 0 (everybody gives up: the last to arrive adds everything)."""
-    import os
     m, n, k, layout = case
     tag = "nt" if layout == mz.LAYOUT_NT else "nn"
     kernel = f"maize_gemm_bf16_skinny_{tag}_{'m32' if m <= 32 else 'm64'}"
@@ -519,22 +518,16 @@ def test_row_group_kernels_share_the_additions_whatever_the_wait(ctx, oracle, ca
     assert (plan["split_first"] & 2) == (2 if groups * plan["ksplit"] >= 16 else 0), plan
     assert plan["split_first"] & 2, "a case of this test is meant to share"
     results = {}
-    old = os.environ.get("MAIZE_HIP_SPLIT_WAIT_US")
+    old = mz.set_split_wait_us(30)
     try:
-        for wait in (None, "1", "0"):
-            if wait is None:
-                os.environ.pop("MAIZE_HIP_SPLIT_WAIT_US", None)
-            else:
-                os.environ["MAIZE_HIP_SPLIT_WAIT_US"] = wait
-            _say(f"{kernel} {case[:3]} wait bound {wait or 'default'} us, {plan['ksplit']} ranges")
+        for wait in (30, 1, 0):
+            mz.set_split_wait_us(wait)
+            _say(f"{kernel} {case[:3]} wait bound {wait} us, {plan['ksplit']} ranges")
             for rep in range(3):
                 results[(wait, rep)] = run_gemm(ctx, a, b, m, n, k, layout=layout, kernel=kernel)
     finally:
-        if old is None:
-            os.environ.pop("MAIZE_HIP_SPLIT_WAIT_US", None)
-        else:
-            os.environ["MAIZE_HIP_SPLIT_WAIT_US"] = old
-    first = results[(None, 0)]
+        mz.set_split_wait_us(old)
+    first = results[(30, 0)]
     check_against_oracle(oracle, first, a, b, m, n, k, layout=layout, label=f"{kernel} shared additions")
     for key, got in results.items():
         assert np.array_equal(got, first), key
@@ -562,4 +555,4 @@ def test_skinny_nn_unaligned_b_and_c(ctx, oracle):
     B = np.stack([bfull[1 + r * ldb: 1 + r * ldb + n] for r in range(k)]).ravel()
     ref, f64, ab = oracle.ref_gemm(a, B, m, n, k, want_f64=True, want_abs=True)
     s = oracle.compare(got[3:3 + m * n], ref, f64, ab, k)
-    assert s["n_fail"] == 0, s
+    oracle.assert_parity(s, "unaligned")

@@ -227,6 +227,64 @@ def test_comparator_flags_and_floors(oracle):
     assert oracle.floor_coeff(k) == (k / 16 + 2) * 2.0 ** -24
 
 
+
+def _accumulate_like_the_matrix_core(a_bits, b_bits, m, n, k, round_partials=None, every=256):
+    """What an fp32-accumulating kernel returns, modelled on the CPU: 32 exact products per step added to an fp32
+    accumulator with one rounding.  `round_partials`: the running sum is handed on through that rounding every
+    `every` elements of K, as a kernel would that kept the partial results of its K ranges in a narrower type."""
+    af = f32_of(a_bits).reshape(m, k).astype(np.float64)
+    bf = f32_of(b_bits).reshape(k, n).astype(np.float64)
+    acc = np.zeros((m, n), np.float32)
+    total = np.zeros((m, n), np.float32)
+    for k0 in range(0, k, 32):
+        acc = (acc.astype(np.float64) + af[:, k0:k0 + 32] @ bf[k0:k0 + 32]).astype(np.float32)
+        if round_partials is not None and (k0 + 32) % every == 0:
+            total = round_partials((total.astype(np.float64) + acc.astype(np.float64)).astype(np.float32))
+            acc = np.zeros((m, n), np.float32)
+    return (total.astype(np.float64) + acc.astype(np.float64)).astype(np.float32)
+
+
+def _to_14_bits(x):
+    """fp32 -> a 14-bit significand (ten of the 24 bits lost), round to nearest even."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u + 0x1FF + ((u >> 10) & 1)) & np.uint32(0xFFFFFC00)).view(np.float32)
+
+
+def test_the_bar_below_the_floor_tells_fp32_sums_from_degraded_ones(oracle):
+    """`n_fail == 0` alone grants every element beyond 1 ULP a deterministic worst-case floor that real fp32
+    accumulation uses a thousandth of.  Three kernels modelled on the CPU at K = 4096, uniform operands:
+    fp32 accumulation passes everything; partial sums handed on in bf16 every 256 elements of K are caught by the
+    floor itself; partial sums with a 14-bit significand pass `n_fail == 0` and are caught only by the two
+    sensitive statistics (and, for an fp32 C, by the statistical bound beside the deterministic one)."""
+    import maize_amd as mz
+    m, n, k = 32, 1024, 4096
+    a = mz.gen.uniform_bf16(m * k, 31)
+    b = mz.gen.uniform_bf16(k * n, 32)
+    ref, f64, ab = oracle.ref_gemm(a, b, m, n, k, want_f64=True, want_abs=True)
+    sumsq = oracle.sum_of_squares(a, b, m, n, k)
+
+    good = _accumulate_like_the_matrix_core(a, b, m, n, k)
+    s = oracle.compare(mz.bf16.from_f32(good).ravel(), ref, f64, ab, k)
+    assert s["n_fail"] == 0 and oracle.tight_violations(s) == []
+    oracle.assert_parity(s, "fp32 accumulation")
+    c = oracle.check_f32(good.ravel(), f64.ravel(), ab.ravel(), k, sumsq=sumsq.ravel())
+    assert c["n_fail"] == 0 and c["n_fail_statistical"] == 0 and c["worst_over_statistical"] < 0.5
+
+    lossy = _accumulate_like_the_matrix_core(a, b, m, n, k, round_partials=_to_14_bits)
+    s = oracle.compare(mz.bf16.from_f32(lossy).ravel(), ref, f64, ab, k)
+    assert s["n_fail"] == 0                                   # the old bar: passes
+    v = oracle.tight_violations(s)
+    assert len(v) == 2, (v, s)                                # both statistics are out of line
+    with pytest.raises(AssertionError):
+        oracle.assert_parity(s, "14-bit partial sums")
+    oracle.assert_parity(s, "14-bit partial sums", tight=False)
+    c = oracle.check_f32(lossy.ravel(), f64.ravel(), ab.ravel(), k, sumsq=sumsq.ravel())
+    assert c["n_fail"] == 0 and c["n_fail_statistical"] > 0 and c["worst_over_statistical"] > 4.0
+
+    coarse = _accumulate_like_the_matrix_core(a, b, m, n, k, round_partials=lambda x: f32_of(mz.bf16.from_f32(x)).reshape(x.shape))
+    s = oracle.compare(mz.bf16.from_f32(coarse).ravel(), ref, f64, ab, k)
+    assert s["n_fail"] > 0                                    # bf16 partial sums: the floor itself catches them
+
 # ---- IEEE half: the operand type of the half-precision twin of the MMA op -------------------
 
 def test_half_conversions_match_numpy_float16(oracle):

@@ -62,7 +62,7 @@ def test_noalloc_matches_the_allocating_entry_point_twice_in_a_row(ctx, oracle):
         assert np.array_equal(ref, got), f"{m}x{n}x{k}: {int((ref != got).sum())} elements differ"
         full, f64, ab = oracle.ref_gemm(a, b, m, n, k, want_f64=True, want_abs=True)
         s = oracle.compare(got, full, f64, ab, k)
-        assert s["n_fail"] == 0, s
+        oracle.assert_parity(s, "noalloc")
 
 
 @pytest.mark.parametrize("shape", [(64, 4096, 4096, mz.LAYOUT_NN), (16, 4096, 4096, mz.LAYOUT_NT), (4000, 4104, 4032, mz.LAYOUT_NN),
@@ -89,3 +89,20 @@ def test_noalloc_refuses_what_does_not_fit(ctx):
         assert np.all(dc.download(np.uint16) == CANARY), "a refused call launched something"
     finally:
         da.free(); db.free(); dc.free()
+
+
+def test_noalloc_reset_restores_the_ticket_counters(ctx):
+    """maize_hip_noalloc_reset is the recovery after calls that overlapped on one GPU against the rule, or after an
+    aborted launch: it zeroes the array's ticket counters.  Here a product runs, the counters are
+    reset, and the next product -- a kernel that takes tickets -- is bit-identical
+    to the allocating entry point's."""
+    m, n, k = 16, 14336, 4096
+    ref, got, plan, _, _ = _both(ctx, m, n, k)
+    assert plan["ksplit"] > 1 and np.array_equal(ref, got)
+    _say("noalloc: reset")
+    ctx.noalloc_reset()
+    ctx.sync()
+    ref2, got2, _, _, _ = _both(ctx, m, n, k)
+    assert np.array_equal(ref2, ref) and np.array_equal(got2, ref)
+    with pytest.raises(mz.MaizeError):
+        mz._ffi.check(mz._ffi.lib().maize_hip_noalloc_reset(None, None))
