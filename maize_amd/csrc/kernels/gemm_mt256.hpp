@@ -488,7 +488,13 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // ---- steady state ----------------------------------------------------------------
     // One K step = 8 eighths.  On entry: (ca, cb) hold tile t, fa[0] and B buffer 0 hold its first groups,
     // the early pieces of tile t+1 are landing in (na, nb).
-    auto step = [&](int cur) {
+    // `narrow` (edge-splitting kernels, a K range of an edge tile): 1 = the tile's live part is at most 32 columns wide
+    // (the last tile column), 2 = at most 32 rows tall (the last tile row).  Such an item multiplies only what can be
+    // live -- B group 0, fragments 0 and 1, resp. A group 0, fragments 0 and 1: 16 of the 128 MFMAs of a K half -- and
+    // reads only those fragments; everything else of the step (the order of the eighths, the waits, the barrier, the
+    // requests) is the whole tile's, so the item is bound by its loads (32 KiB of A, resp. B, per step), not by the
+    // matrix pipe.  Waves whose half of the tile is dead multiply zeros (their operands past N, resp. M, are zero-filled).
+    auto step = [&](int cur, int narrow = 0) {
         // Two stages: tile t+1 is in the other stage, and so go its late pieces.  Three stages: tile t+1 is in the next
         // stage, complete since the step before; the late pieces issued here are tile t+2's, into the stage after that
         // one, and the early pieces behind the barrier are tile t+3's, into the stage this step has just read.
@@ -527,7 +533,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // The accumulator is tied to itself ("+a"): left to the register allocator, a few of the 64
                 // tuples were renamed across the loop and copied back through VGPRs at its end.  (Each
                 // accumulator comes up again 128 MFMAs later: no dependent back-to-back issue.)
-                if (IS8)   // 8-bit operands: B is the first source, so cbsz carries B's format and blgp A's (0 = E4M3, 1 = E5M2)
+                const bool dead = (narrow == 1 && (bi == 1 || c4 >= 2)) || (narrow == 2 && (ai == 1 || r4 >= 2));
+                if (dead) {}   // (an edge item: this product lies outside the matrix)
+                else if (IS8)   // 8-bit operands: B is the first source, so cbsz carries B's format and blgp A's (0 = E4M3, 1 = E5M2)
                     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(acc[4 * ai + r4][4 * bi + c4])
                                  : "v"(b_operand8(H128 ? bi : bi ^ cur, c4)), "v"(operand8(fa8[H128 ? cur : ai][r4])), "n"((F8 >> 1) & 1), "n"(F8 & 1));
                 else if (F16)   // IEEE half operands: same tiles, same fragment maps, the other MFMA
@@ -546,13 +554,15 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                     if (h4 == 1 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, nxt, r); }
                 } else if (s % RSTRIDE == 0) {
                     const int r = s / RSTRIDE;
+                    // (an edge item reads the live fragments only: the first two of B's group 0, resp. of A's)
+                    const int nbr = narrow == 1 ? NBR / 2 : NBR, nar = narrow == 2 ? NAR / 2 : NAR;
 #pragma unroll
                     for (int rb = r * RPS; rb < (r + 1) * RPS; ++rb) {
-                        if (h4 == 0 && rb < NBR) read_b(1, kh, cur, rb);                     // (0,0) -> (0,1): B group 1
-                        if (h4 == 3 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }   // next half or tile: B group 0
+                        if (h4 == 0 && rb < NBR && narrow != 1) read_b(1, kh, cur, rb);      // (0,0) -> (0,1): B group 1
+                        if (h4 == 3 && rb < nbr) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }   // next half or tile: B group 0
                     }
-                    if (h4 == 1 && r < NAR) read_a(1, kh, cur, r);                       // (0,1) -> (1,1): A group 1
-                    if (h4 == 2 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }   // next half or tile: A group 0
+                    if (h4 == 1 && r < NAR && narrow != 2) read_a(1, kh, cur, r);        // (0,1) -> (1,1): A group 1
+                    if (h4 == 2 && r < nar) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }   // next half or tile: A group 0
                 }
                 // ... and the direct-to-LDS request scheduled for this slot (issue_slot): late pieces of
                 // tile t+1 (its stage was freed by the previous barrier) before this step's barrier, early
@@ -598,10 +608,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // is not a multiple runs the extra steps on all-zero tiles (loads past K return zeros).  (Leaving the trip after
     // the step that was the last costs more than it saves: with exits between the steps the register allocator no
     // longer keeps the loop's operands in place.)
-    for (uint32_t kt = 0; kt < nk; kt += NST) {
-        step(0);
-        step(1);
-        if (R3) step(2);
+    if (EDGE && split && mode == 1u) {
+        for (uint32_t kt = 0; kt < nk; kt += 2) { step(0, 1); step(1, 1); }
+    } else if (EDGE && split) {
+        for (uint32_t kt = 0; kt < nk; kt += 2) { step(0, 2); step(1, 2); }
+    } else {
+        for (uint32_t kt = 0; kt < nk; kt += NST) {
+            step(0);
+            step(1);
+            if (R3) step(2);
+        }
     }
     // every direct-to-LDS write of this tile has landed; the last MFMAs have left the pipe before the
     // epilogue reads their accumulators (the assembler-level MFMAs are invisible to the hazard recognizer)
@@ -713,7 +729,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
     } else if (EDGE && esplit) {
         // Last arriver of a split edge tile: a thread sums 8 columns of one row of the dense partial tiles over the
-        // ranges, in range order, eight ranges' loads in flight, and stores them; up to four such units per thread.
+        // ranges, in range order, sixteen ranges' loads in flight, and stores them; up to four such units per thread.
         if (finish) {
             const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce + (uint64_t)em0 * ldc, span(((uint64_t)(M - 1u - em0) * ldc + N) * 2u));
 #pragma unroll
@@ -724,16 +740,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 const bool live = row < rows_ok && c8 * 8u < cols_ok;                   // N % 8 == 0: 8 columns are all in or all out
                 floatx4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
                 const uint32_t base = (slot * eks * dense_rows + row) * dense_pitch + c8 * 32u;
-                for (uint32_t z0 = 0; z0 < eks; z0 += 8u) {
-                    floatx4 t[8], u[8];
+                // (all sixteen ranges' loads in flight at once: one memory latency for the sum instead of two)
+                for (uint32_t z0 = 0; z0 < eks; z0 += 16u) {
+                    floatx4 t[16], u[16];
 #pragma unroll
-                    for (int r = 0; r < 8; ++r) {
+                    for (int r = 0; r < 16; ++r) {
                         const uint32_t off = (live && z0 + r < eks) ? base + (z0 + r) * dense_rows * dense_pitch : DROP;
                         t[r] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off, 0, COHERENT));
                         u[r] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rws, off == DROP ? DROP : off + 16u, 0, COHERENT));
                     }
 #pragma unroll
-                    for (int r = 0; r < 8; ++r) {
+                    for (int r = 0; r < 16; ++r) {
                         lo[0] += t[r][0]; lo[1] += t[r][1]; lo[2] += t[r][2]; lo[3] += t[r][3];
                         hi[0] += u[r][0]; hi[1] += u[r][1]; hi[2] += u[r][2]; hi[3] += u[r][3];
                     }

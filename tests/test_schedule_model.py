@@ -55,10 +55,12 @@ def mt256_issue_slots():
 
 # where the K step issues its fragment reads: slot s of an eighth issues reads s * RPS .. of the group the next eighth needs
 MT256_READ_LINES = ("for (int rb = r * RPS; rb < (r + 1) * RPS; ++rb) {",
-                    "if (h4 == 0 && rb < NBR) read_b(1, kh, cur, rb);",
-                    "if (h4 == 1 && r < NAR) read_a(1, kh, cur, r);",
-                    "if (h4 == 2 && r < NAR) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
-                    "if (h4 == 3 && rb < NBR) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }")
+                    # (whole tiles: narrow == 0, nbr == NBR, nar == NAR; the K ranges of an edge tile read a subset)
+                    "const int nbr = narrow == 1 ? NBR / 2 : NBR, nar = narrow == 2 ? NAR / 2 : NAR;",
+                    "if (h4 == 0 && rb < NBR && narrow != 1) read_b(1, kh, cur, rb);",
+                    "if (h4 == 1 && r < NAR && narrow != 2) read_a(1, kh, cur, r);",
+                    "if (h4 == 2 && r < nar) { if (!last_half) read_a(0, 1, cur, r); else read_a(0, 0, cur ^ 1, r); }",
+                    "if (h4 == 3 && rb < nbr) { if (!last_half) read_b(0, 1, cur, rb); else read_b(0, 0, cur ^ 1, rb); }")
 
 
 def mt256_reads_per_eighth(nt):
