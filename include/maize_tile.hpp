@@ -138,7 +138,7 @@ inline void gemm_smem_multibuffer(Ctx& ctx, const maize_gemm_ex_desc_t& x, void*
 //   BlockX / BlockY / Wave (was Warp)        crates/maize_tile/src/group/by_block.rs:10-75, warp.rs:10-37
 //   SyncMMAOp catalogue                      crates/maize_tile/src/mma/mod.rs:19-99, sm80.rs, sm80_derived.rs:5-28, sm89.rs
 //   gemm_smem_multibuffer(mma, KTile, ...)   crates/maize_tile/src/gemm/mod.rs:37-90
-enum class Swizzle { None, KC16, KN32 };   // KC16: 128-byte rows along K, 16-byte chunk ^ ((row >> 1) & 7); KN32: row-major K x N, 32-byte granule ^ (row % 4 + 4 bit3(row))
+enum class Swizzle { None, KC16, KN32, KN16 };   // KC16: 128-byte rows along K, 16-byte chunk ^ ((row >> 1) & 7); KN32: row-major K x N, 32-byte granule ^ (row % 4 + 4 bit3(row)); KN16: row-major K x N of 8-bit elements, 16-byte chunk ^ (row % 8 + 8 bit4(row))
 #define MAIZE_TILE_TY(name, rows, cols, bytes, swz) \
     struct name { static constexpr uint32_t ROWS = rows, COLS = cols, ELEM_BYTES = bytes; static constexpr Swizzle SWIZZLE = swz; };
 MAIZE_TILE_TY(BF16_16x16, 16, 16, 2, Swizzle::None)      // the reference's tile (lib.rs:98-108); no kernel here takes it
@@ -147,6 +147,10 @@ MAIZE_TILE_TY(BF16_64x256, 64, 256, 2, Swizzle::KN32)    // B stage of a row-maj
 MAIZE_TILE_TY(F16_256x64, 256, 64, 2, Swizzle::KC16)
 MAIZE_TILE_TY(F16_64x256, 64, 256, 2, Swizzle::KN32)
 MAIZE_TILE_TY(F8_256x128, 256, 128, 1, Swizzle::KC16)    // 8-bit operands: 128 elements of K per 128-byte row
+MAIZE_TILE_TY(F8_128x256, 128, 256, 1, Swizzle::KN16)    // B stage of a row-major K x N 8-bit B (read back by ds_read_b64_tr_b8)
+MAIZE_TILE_TY(BF16_128x64, 128, 64, 2, Swizzle::KC16)    // A stages of the 128 x 256 tile kernels (the B stages are the ones above)
+MAIZE_TILE_TY(F16_128x64, 128, 64, 2, Swizzle::KC16)
+MAIZE_TILE_TY(F8_128x128, 128, 128, 1, Swizzle::KC16)
 #undef MAIZE_TILE_TY
 template <class T> struct Tile { using Ty = T; static constexpr size_t SIZE = (size_t)T::ROWS * T::COLS * T::ELEM_BYTES; };
 template <class TA, class TB> struct TilePair { using A = TA; using B = TB; static constexpr size_t SIZE = TA::SIZE + TB::SIZE; };
@@ -222,20 +226,48 @@ std::pair<PanelIterLooper<ColPanel<N>>, ColPanel<N>> collective_aligned_col_pane
     return {PanelIterLooper<ColPanel<N>>{ColPanel<N>{m, N, false}, m.g.ncols / N}, ColPanel<N>{m, m.g.ncols % N, true}};
 }
 
-struct TracedOp { Matrix a, b, c; bool nt; maize_in_type_t in; Family family; bool stored; maize_out_type_t out; float alpha, beta; };
+// panel_rows, pipe: the panel height of A and the ring depth as described (0: the description has no ring)
+struct TracedOp { Matrix a, b, c; bool nt; maize_in_type_t in; Family family; bool stored; maize_out_type_t out; float alpha, beta; uint32_t panel_rows, pipe; };
+// The kernel that a description of the mainloop (panel height of A, ring depth) names for `x`; empty when the
+// dispatcher's own choice already is of that family.  A description is honoured wherever a kernel of its family accepts
+// the descriptor -- also where the dispatcher by itself would take another family -- and refused where none does.
+inline std::string described_kernel(const maize_gemm_ex_desc_t& x, bool nt, uint32_t panel_rows, uint32_t pipe, uint32_t cus) {
+    maize_gemm_plan_t plan;
+    check(maize_hip_gemm_ex_plan(&x, nullptr, cus, &plan));
+    const std::string chosen = plan.kernel;
+    static const char* const tags[] = {"bf16", "f16", "e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"};
+    if ((uint32_t)x.in_type > (uint32_t)MAIZE_IN_E5M2_E4M3) throw std::invalid_argument("no macro-tile kernel for this operand type");
+    const std::string base = std::string("maize_gemm_") + tags[(int)x.in_type] + "_mt256_" + (nt ? "nt" : "nn");
+    std::vector<std::string> names;
+    const bool is_h = chosen.find("_h128") != std::string::npos, is_r3 = chosen.find("_h128r3") != std::string::npos;
+    if (panel_rows == 256) {
+        if (!is_h) return "";                     // a 256-row kernel, a split of one, or a few-row kernel: the dispatcher's
+        names = {base, base + "_ktail", base + "_gen", base + "_ktail_gen"};
+    } else {
+        if (pipe == 3 ? is_r3 : (is_h && !is_r3)) return "";
+        const std::string tag = pipe == 3 ? "_h128r3" : "_h128";
+        names = {base + tag, base + tag + "_gen"};
+    }
+    for (const std::string& n : names)
+        if (maize_hip_gemm_ex_plan(&x, n.c_str(), cus, &plan) == MAIZE_OK) return n;
+    throw std::invalid_argument("no kernel with " + std::to_string(panel_rows) + "-row panels of A on " + std::to_string(pipe) + " ring stages runs this product");
+}
 class LoadedGemm {
   public:
-    LoadedGemm(Ctx& ctx, const maize_gemm_ex_desc_t& x, const char* forced) : ctx_(ctx), x_(x), forced_(forced) {
-        int32_t cus = 256;
+    LoadedGemm(Ctx& ctx, const maize_gemm_ex_desc_t& x, const TracedOp& op) : ctx_(ctx), x_(x) {
+        uint32_t cus = 256;
         maize_device_info_t info;
-        if (maize_hip_device_info(ctx.handle(), &info) == MAIZE_OK) cus = (int32_t)info.compute_units;
-        check(maize_hip_gemm_ex_plan(&x_, forced_, (uint32_t)cus, &plan_));
+        if (maize_hip_device_info(ctx.handle(), &info) == MAIZE_OK) cus = info.compute_units;
+        if (op.family == Family::WAVE32) forced_ = "maize_gemm_bf16_wave32";
+        else if (op.family == Family::MT256 && op.pipe) forced_ = described_kernel(x_, op.nt, op.panel_rows, op.pipe, cus);
+        check(maize_hip_gemm_ex_plan(&x_, forced(), cus, &plan_));
     }
     std::string kernel_name() const { return plan_.kernel; }
     const maize_gemm_plan_t& plan() const { return plan_; }
-    void launch(void* stream = nullptr) { check(maize_hip_gemm_bf16_ex(ctx_.handle(), &x_, forced_, stream)); }
+    void launch(void* stream = nullptr) { check(maize_hip_gemm_bf16_ex(ctx_.handle(), &x_, forced(), stream)); }
   private:
-    Ctx& ctx_; maize_gemm_ex_desc_t x_; const char* forced_; maize_gemm_plan_t plan_;
+    const char* forced() const { return forced_.empty() ? nullptr : forced_.c_str(); }
+    Ctx& ctx_; maize_gemm_ex_desc_t x_; std::string forced_; maize_gemm_plan_t plan_;
 };
 class PreLoadGemm {
   public:
@@ -248,7 +280,7 @@ class PreLoadGemm {
         d.layout = op_.nt ? MAIZE_LAYOUT_NT : MAIZE_LAYOUT_NN; d.batch = 1;
         maize_gemm_ex_desc_t x{};
         x.gemm = d; x.out_type = op_.out; x.alpha = op_.alpha; x.beta = op_.beta; x.in_type = op_.in;
-        return LoadedGemm(ctx, x, op_.family == Family::WAVE32 ? "maize_gemm_bf16_wave32" : nullptr);
+        return LoadedGemm(ctx, x, op_);
     }
   private:
     TracedOp op_;
@@ -293,18 +325,21 @@ Accum gemm_smem_multibuffer(const MMA&, KTile<K_TILE>, const RowPanel<NA>& a, co
     constexpr bool NT = is_row_panel<BPanel>::value;
     static_assert(MMA::FAMILY == Family::MT256, "a shared-memory ring goes with the macro-tile kernels' instructions");
     static_assert(K_TILE == MMA::K_TILE, "KTile does not match the K a ring stage of this instruction's kernels holds");
-    static_assert(PIPE == 2, "the macro-tile kernels run a two-stage ring");
-    static_assert(NA == 256 && BPanel::WINDOW == 256, "the macro-tile kernels take panels of 256 rows (A) and 256 columns (B)");
+    // Generic in the ring depth and the panel height like the reference's mainloop ([TilePair; PIPE], KTile<N>,
+    // gemm/mod.rs:37-45), within what kernels exist: 256- or 128-row panels of A on two stages, 128-row panels also on
+    // three (a 128 x 256 tile's stage is 48 KiB; three fit the 160 KiB of LDS).
+    static_assert(PIPE == 2 || PIPE == 3, "the macro-tile kernels run a ring of two or three stages");
+    static_assert((NA == 256 || NA == 128) && BPanel::WINDOW == 256, "the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B)");
+    static_assert(PIPE == 2 || NA == 128, "three ring stages fit the LDS with 128-row panels of A only");
     using TA = typename Pair::A::Ty; using TB = typename Pair::B::Ty;
     constexpr uint32_t ES = MMA::K_TILE == 128 ? 1 : 2;
-    static_assert(TA::ROWS == 256 && TA::COLS == MMA::K_TILE && TA::ELEM_BYTES == ES && TA::SWIZZLE == Swizzle::KC16, "A stage: 256 x K_TILE, K-contiguous");
-    static_assert(NT ? (TB::ROWS == 256 && TB::COLS == MMA::K_TILE && TB::SWIZZLE == Swizzle::KC16)
-                     : (TB::ROWS == MMA::K_TILE && TB::COLS == 256 && TB::SWIZZLE == Swizzle::KN32), "B stage does not match how B is stored");
-    static_assert(NT || ES == 2, "8-bit operands: both K-contiguous (B stored N x K)");
+    static_assert(TA::ROWS == NA && TA::COLS == MMA::K_TILE && TA::ELEM_BYTES == ES && TA::SWIZZLE == Swizzle::KC16, "A stage: panel rows x K_TILE, K-contiguous");
+    static_assert(NT ? (TB::ROWS == 256 && TB::COLS == MMA::K_TILE && TB::ELEM_BYTES == ES && TB::SWIZZLE == Swizzle::KC16)
+                     : (TB::ROWS == MMA::K_TILE && TB::COLS == 256 && TB::ELEM_BYTES == ES && TB::SWIZZLE == (ES == 2 ? Swizzle::KN32 : Swizzle::KN16)), "B stage does not match how B is stored");
     if (cp_size != 16) throw std::invalid_argument("direct-to-LDS copies are 16 bytes per lane");
     const uint32_t ka = a.col_size(), kb = NT ? b.matrix.g.ncols : b.matrix.g.nrows;
     if (ka != kb) throw std::invalid_argument("inner dimensions differ");
-    return Accum(cp_group.kernel, TracedOp{a.matrix, b.matrix, Matrix{}, NT, MMA::IN_TYPE, MMA::FAMILY, false, MAIZE_OUT_SAME, 1.0f, 0.0f});
+    return Accum(cp_group.kernel, TracedOp{a.matrix, b.matrix, Matrix{}, NT, MMA::IN_TYPE, MMA::FAMILY, false, MAIZE_OUT_SAME, 1.0f, 0.0f, NA, (uint32_t)PIPE});
 }
 inline TracedKernel new_hip_kernel() { return TracedKernel(); }
 

@@ -5,7 +5,9 @@
 // This program keeps the same steps -- declare the kernel, fix its launch bounds, compile for a
 // target, describe A and B as GlobalMatrix -- and then launches on an MI355X, twice: through the
 // dispatcher (gemm_smem_multibuffer), through the explicit builder chain, and as a kernel described in the
-// reference's tile vocabulary (panels, groups, ring, MMA op), and checks that all agree bit for bit.  Output: one JSON line with the kernel chosen and checksums of C.
+// reference's tile vocabulary (panels, groups, ring, MMA op) -- once as the reference's caller has it, with the panels and
+// the two-stage ring of the 256-row kernels, once with 128-row panels of A on a ring of three stages -- and checks that all
+// agree bit for bit.  Output: one JSON line with the kernels chosen and checksums of C.
 //
 //   maize_gemm_example [M N K]        (default 4096 4096 4096, like src/main.rs:47-48)
 #include <cinttypes>
@@ -73,19 +75,42 @@ int main(int argc, char** argv) {
         described.launch();
         ctx.sync();
 
-        const std::vector<BF16> c1 = ctx.download(dc, (size_t)M * N), c2 = ctx.download(dc2, (size_t)M * N), c3 = ctx.download(dc3, (size_t)M * N);
-        uint64_t sum = 0, x = 0, diff = 0, diff3 = 0;
+        // 4. the same mainloop with the ring depth and the panel height as parameters ([TilePair; PIPE], gemm/mod.rs:37-45):
+        //    128-row panels of A, three ring stages
+        BF16* dc4 = ctx.malloc<BF16>((size_t)M * N);
+        TracedKernel kernel3 = new_hip_kernel();
+        kernel3.with_launch_bounds_2d({256, 1});
+        auto ring3 = kernel3.alloc_aligned_shared<TilePair<Tile<BF16_128x64>, Tile<BF16_64x256>>, 3>(1024);
+        const BlockX a_group3{kernel3.cx()};
+        const BlockY b_group3{kernel3.cx()};
+        const Wave wave3{kernel3.cx()};
+        const auto a_iter3 = collective_aligned_row_panel_iter<128>(amat, a_group3);
+        const auto b_iter3 = collective_aligned_col_panel_iter<256>(bmat, b_group3);
+        a_iter3.first.for_every_value([&](const RowPanel<128>& a_panel) {
+            b_iter3.first.for_every_value([&](const ColPanel<256>& b_panel) {
+                gemm_smem_multibuffer(Gfx950MfmaBf16F32_16x16x32{}, KTile<64>{}, a_panel, b_panel, ring3, wave3, 16).store(Matrix::make(dc4, M, N));
+            });
+        });
+        LoadedGemm described3 = kernel3.finalize().compile(Gfx::Gfx950, ctx);
+        described3.launch();
+        ctx.sync();
+
+        const std::vector<BF16> c1 = ctx.download(dc, (size_t)M * N), c2 = ctx.download(dc2, (size_t)M * N), c3 = ctx.download(dc3, (size_t)M * N),
+                                c4 = ctx.download(dc4, (size_t)M * N);
+        uint64_t sum = 0, x = 0, diff = 0, diff3 = 0, diff4 = 0;
         for (size_t i = 0; i < c1.size(); ++i) {
             sum += c1[i].bits;
             x ^= (uint64_t)c1[i].bits << (i % 48);
             diff += c1[i].bits != c2[i].bits;
             diff3 += c1[i].bits != c3[i].bits;
+            diff4 += c1[i].bits != c4[i].bits;
         }
-        printf("{\"M\": %u, \"N\": %u, \"K\": %u, \"kernel\": \"%s\", \"described_kernel\": \"%s\", \"ragged_rows\": %u, \"ragged_cols\": %u, "
-               "\"sum\": %" PRIu64 ", \"xor\": %" PRIu64 ", \"mismatch_vs_any_shape_kernel\": %" PRIu64 ", \"mismatch_vs_described_kernel\": %" PRIu64 "}\n",
-               M, N, K, chosen.c_str(), described.kernel_name().c_str(), a_iter.second.extent, b_iter.second.extent, sum, x, diff, diff3);
-        ctx.free(da); ctx.free(db); ctx.free(dc); ctx.free(dc2); ctx.free(dc3);
-        return (diff == 0 && diff3 == 0) ? 0 : 3;
+        printf("{\"M\": %u, \"N\": %u, \"K\": %u, \"kernel\": \"%s\", \"described_kernel\": \"%s\", \"described_128_rows_3_stages\": \"%s\", \"ragged_rows\": %u, \"ragged_cols\": %u, "
+               "\"sum\": %" PRIu64 ", \"xor\": %" PRIu64 ", \"mismatch_vs_any_shape_kernel\": %" PRIu64 ", \"mismatch_vs_described_kernel\": %" PRIu64
+               ", \"mismatch_vs_described_128_rows_3_stages\": %" PRIu64 "}\n",
+               M, N, K, chosen.c_str(), described.kernel_name().c_str(), described3.kernel_name().c_str(), a_iter.second.extent, b_iter.second.extent, sum, x, diff, diff3, diff4);
+        ctx.free(da); ctx.free(db); ctx.free(dc); ctx.free(dc2); ctx.free(dc3); ctx.free(dc4);
+        return (diff == 0 && diff3 == 0 && diff4 == 0) ? 0 : 3;
     } catch (const Error& e) {
         fprintf(stderr, "maize error: %s\n", e.what());
         return 2;

@@ -27,7 +27,8 @@ from .api import Gfx, Matrix, gemm_ex_desc, gemm_plan
 class TileTy:
     """A tile type: ROWS x COLS elements of ELEM_BYTES bytes (ConstSizeTileTy, lib.rs:90-93) and how the kernels
     lay it out in LDS.  swizzle "kc16": rows of 128 bytes along K, 16-byte chunk index XOR-ed with (row >> 1) & 7;
-    "kn32": a row-major K x N tile, 32-byte granule index XOR-ed with row % 4 + 4 * bit3(row)."""
+    "kn32": a row-major K x N tile, 32-byte granule index XOR-ed with row % 4 + 4 * bit3(row); "kn16": a row-major
+    K x N tile of 8-bit elements, 16-byte chunk index XOR-ed with row % 8 + 8 * bit4(row)."""
     name: str
     rows: int
     cols: int
@@ -45,6 +46,11 @@ BF16_64x256 = TileTy("BF16_64x256", 64, 256, 2, "kn32")       # B stage of a row
 F16_256x64 = TileTy("F16_256x64", 256, 64, 2, "kc16")
 F16_64x256 = TileTy("F16_64x256", 64, 256, 2, "kn32")
 F8_256x128 = TileTy("F8_256x128", 256, 128, 1, "kc16")        # 8-bit operands: 128 elements of K per 128-byte row
+F8_128x256 = TileTy("F8_128x256", 128, 256, 1, "kn16")        # B stage of a row-major K x N 8-bit B (read back by ds_read_b64_tr_b8)
+# A stages of the 128 x 256 tile kernels (a wave then owns 64 x 128 of C; the B stages are the ones above)
+BF16_128x64 = TileTy("BF16_128x64", 128, 64, 2, "kc16")
+F16_128x64 = TileTy("F16_128x64", 128, 64, 2, "kc16")
+F8_128x128 = TileTy("F8_128x128", 128, 128, 1, "kc16")
 
 
 @dataclass(frozen=True)
@@ -279,24 +285,28 @@ def gemm_smem_multibuffer(mma, ktile, a_panel, b_panel, smem, cp_group, cp_size)
             raise ValueError(f"{mma.name}: a ring stage holds {mma.k_tile} elements of K, not {ktile.value}")
         if cp_size != 16:
             raise ValueError("direct-to-LDS copies are 16 bytes per lane")
-        if a_panel.rows != 256 or (b_panel.rows if nt else b_panel.cols) != 256:
-            raise ValueError("the macro-tile kernels take panels of 256 rows (A) and 256 columns (B)")
-        if smem is None or smem.depth != 2:
-            raise ValueError("the macro-tile kernels run a two-stage ring")
+        # The mainloop is generic in the panel height and the ring depth, like the reference's ([TilePair; PIPE],
+        # KTile<N>, gemm/mod.rs:37-45), within what kernels exist: 256- or 128-row panels of A on a two-stage ring,
+        # 128-row panels also on three stages (the stage of a 128 x 256 tile is 48 KiB: three fit the 160 KiB of LDS).
+        if a_panel.rows not in (256, 128) or (b_panel.rows if nt else b_panel.cols) != 256:
+            raise ValueError("the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B)")
+        if smem is None or smem.depth not in (2, 3):
+            raise ValueError("the macro-tile kernels run a ring of two or three stages")
+        if smem.depth == 3 and a_panel.rows != 128:
+            raise ValueError("three ring stages fit the LDS with 128-row panels of A only")
         es = 1 if mma.k_tile == 128 else 2
-        want_a = (256, mma.k_tile, es, "kc16")
-        want_b = want_a if nt else (mma.k_tile, 256, es, "kn32")
+        want_a = (a_panel.rows, mma.k_tile, es, "kc16")
+        want_b = (256, mma.k_tile, es, "kc16") if nt else (mma.k_tile, 256, es, "kn32" if es == 2 else "kn16")
         for which, tile, want in (("A", smem.pair.a, want_a), ("B", smem.pair.b, want_b)):
             t = tile.ty
             if (t.rows, t.cols, t.elem_bytes, t.swizzle) != want:
                 raise ValueError(f"{which} stage is {t.name}; {mma.name} with B stored {'N x K' if nt else 'K x N'} needs "
                                  f"{want[0]}x{want[1]} tiles of {want[2]}-byte elements, layout {want[3]}")
-        if es == 1 and not nt:
-            raise ValueError("8-bit operands: the matrix instruction wants both operands K-contiguous (B stored N x K)")
     elif mma.family == "wave32":
         if smem is not None:
             raise ValueError(f"{mma.name} is the any-shape kernel's instruction: operands go straight from global memory, no ring")
-    op = dict(mma=mma, a=a_panel, b=b_panel, nt=nt)
+    op = dict(mma=mma, a=a_panel, b=b_panel, nt=nt, panel_rows=a_panel.rows if mma.family == "mt256" else None,
+              pipe=smem.depth if smem is not None else None)
     return Accum(kernel, op)
 
 
@@ -335,6 +345,37 @@ class TracedKernel:
         return PreLoadGemm(self)
 
 
+_TYPE_TAG = {_ffi.IN_BF16: "bf16", _ffi.IN_F16: "f16", _ffi.IN_E4M3: "e4m3", _ffi.IN_E5M2: "e5m2",
+             _ffi.IN_E4M3_E5M2: "e4m3e5m2", _ffi.IN_E5M2_E4M3: "e5m2e4m3"}
+
+
+def described_kernel(desc, mma, nt, panel_rows, pipe, compute_units):
+    """The kernel that a description of the mainloop (panel height of A, ring depth) names for `desc`, or None when
+    the dispatcher's own choice already is of that family.  A description is honoured wherever a kernel of its family
+    accepts the descriptor -- also where the dispatcher by itself would rather take another family (128-row tiles for
+    a product of many rounds, say) -- and refused (ValueError) where none does."""
+    from .api import MaizeError
+    chosen = gemm_plan(desc, compute_units=compute_units)["kernel"]
+    base = f"maize_gemm_{_TYPE_TAG[mma.in_type]}_mt256_{'nt' if nt else 'nn'}"
+    if panel_rows == 256:
+        if "_h128" not in chosen:
+            return None                                # a 256-row kernel, a split of one, or a few-row kernel: the dispatcher's
+        names = [base, base + "_ktail", base + "_gen", base + "_ktail_gen"]
+    else:
+        tag = "_h128r3" if pipe == 3 else "_h128"
+        if tag in chosen and (pipe == 3 or "_h128r3" not in chosen):
+            return None
+        names = [base + tag, base + tag + "_gen"]
+    for name in names:
+        try:
+            gemm_plan(desc, kernel=name, compute_units=compute_units)
+            return name
+        except MaizeError:
+            continue
+    raise ValueError(f"no kernel with {panel_rows}-row panels of A on {pipe} ring stages runs this product "
+                     f"(tried {', '.join(names)})")
+
+
 class PreLoadGemm:
     def __init__(self, traced):
         self.traced = traced
@@ -347,6 +388,8 @@ class PreLoadGemm:
         desc = gemm_ex_desc(a, b, c, layout=_ffi.LAYOUT_NT if op["nt"] else _ffi.LAYOUT_NN, out_type=op["out_type"], alpha=op["alpha"],
                             beta=op["beta"], in_type=op["mma"].in_type)
         forced = "maize_gemm_bf16_wave32" if op["mma"].family == "wave32" else None
+        if op["mma"].family == "mt256":
+            forced = described_kernel(desc, op["mma"], op["nt"], op["panel_rows"], op["pipe"], ctx.info()["compute_units"])
         return LoadedGemm(ctx, desc, forced, op["mma"])
 
 

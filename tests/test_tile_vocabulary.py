@@ -26,14 +26,14 @@ def matrices(m, n, k, nt=False):
 
 
 def describe(a, b, c, mma=T.Gfx950MfmaBf16F32_16x16x32, nt=False, ktile=64, tiles=(T.BF16_256x64, T.BF16_64x256), depth=2, cp=16,
-             panel=256, ring=True):
+             panel=256, ring=True, a_panel=None):
     """The body of the reference's test_inner(), line for line (src/main.rs:32-73)."""
     kernel = mz.new_hip_kernel().with_launch_bounds_2d((256, 1), None, None)
     pipe_shared = kernel.alloc_aligned_shared(T.TilePair(T.Tile(tiles[0]), T.Tile(tiles[1])), depth, 1024) if ring else None
     a_panel_group = T.BlockX(kernel.cx())
     b_panel_group = T.BlockY(kernel.cx())
     wave = T.Wave(kernel.cx())
-    a_panels, _a_epilogue = T.collective_aligned_row_panel_iter(a, panel, a_panel_group)
+    a_panels, _a_epilogue = T.collective_aligned_row_panel_iter(a, a_panel or panel, a_panel_group)
     if nt:
         b_panels, _b_epilogue = T.collective_aligned_row_panel_iter(b, panel, b_panel_group)
     else:
@@ -91,14 +91,55 @@ def test_nt_f16_f8_and_the_any_shape_instruction():
     (dict(ktile=16), "ring stage holds 64"),                                    # the reference's KTile::<16>
     (dict(tiles=(T.BF16_16x16, T.BF16_16x16)), "A stage is BF16_16x16"),        # ... and its tile type
     (dict(depth=4), "bytes of LDS"),                                            # ... and its ring depth: four 64 KiB stages do not fit
-    (dict(depth=1), "two-stage ring"),
+    (dict(depth=1), "two or three stages"),
+    (dict(depth=3, a_panel=256, tiles=(T.BF16_128x64, T.BF16_64x256)), "128-row panels of A only"),    # (three 48 KiB stages fit, three 64 KiB ones do not)
+    (dict(a_panel=128), "A stage is BF16_256x64"),                              # 128-row panels need the 128-row A stage
+    (dict(a_panel=64, tiles=(T.BF16_128x64, T.BF16_64x256)), "256 or 128 rows"),
     (dict(cp=8), "16 bytes per lane"),
-    (dict(panel=16), "panels of 256 rows"),
+    (dict(panel=16), "256 or 128 rows"),
     (dict(tiles=(T.BF16_256x64, T.BF16_256x64)), "B stage is BF16_256x64"),     # K x N B needs the K x N stage
 ])
 def test_what_the_kernels_do_not_implement_is_refused_at_trace_time(kw, msg):
     with pytest.raises(ValueError, match=msg):
         describe(*matrices(4096, 4096, 4096), **kw)
+
+
+def test_the_description_chooses_the_panel_height_and_the_ring_depth():
+    """The mainloop is generic in the ring depth and the panel height, like the reference's ([TilePair; PIPE], KTile<N>,
+    crates/maize_tile/src/gemm/mod.rs:37-45): a description with 128-row panels of A gets the 128 x 256 tile kernels, on
+    two or three ring stages as it says, whatever the dispatcher would take by itself; one that no kernel runs is refused."""
+    cus = FakeCtx()
+    h128 = dict(a_panel=128, tiles=(T.BF16_128x64, T.BF16_64x256))
+    # 2048^3: the dispatcher itself takes 128-row tiles on three stages
+    a, b, c = matrices(2048, 2048, 2048)
+    assert mz.gemm_plan(mz.gemm_desc(a, b, c), compute_units=256)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"
+    got = {}
+    for tag, kw in (("r3", dict(depth=3, **h128)), ("r2", dict(depth=2, **h128)), ("256", dict())):
+        k, _ = describe(a, b, c, **kw)
+        got[tag] = k.finalize().compile(mz.Gfx.Gfx950, cus)
+    assert got["r3"].kernel_name == "maize_gemm_bf16_mt256_nn_h128r3" and got["r3"].forced is None     # the dispatcher's own launch
+    assert got["r3"].plan == mz.gemm_plan(mz.gemm_desc(a, b, c), compute_units=256)
+    assert got["r2"].kernel_name == got["r2"].forced == "maize_gemm_bf16_mt256_nn_h128"
+    assert got["256"].kernel_name == got["256"].forced == "maize_gemm_bf16_mt256_nn"
+    # 4096^3: two rounds of half tiles lose to one round of whole ones, the dispatcher takes 256 rows; described, it runs
+    a, b, c = matrices(4096, 4096, 4096)
+    k, _ = describe(a, b, c, depth=3, **h128)
+    assert k.finalize().compile(mz.Gfx.Gfx950, cus).kernel_name == "maize_gemm_bf16_mt256_nn_h128r3"
+    # N x K B, half operands, a K that is no multiple of 64 (the general-epilogue kernels), 8-bit operands both ways
+    a, b, c = matrices(1024, 4096, 4096, nt=True)
+    k, _ = describe(a, b, c, nt=True, depth=3, a_panel=128, tiles=(T.BF16_128x64, T.BF16_256x64))
+    assert k.finalize().compile(mz.Gfx.Gfx950, cus).kernel_name == "maize_gemm_bf16_mt256_nt_h128r3"
+    k, _ = describe(*matrices(1024, 2048, 2056), mma=T.Gfx950MfmaF16F32_16x16x32, depth=2, a_panel=128, tiles=(T.F16_128x64, T.F16_64x256))
+    assert k.finalize().compile(mz.Gfx.Gfx950, cus).kernel_name == "maize_gemm_f16_mt256_nn_h128_gen"
+    for nt, btile in ((True, T.F8_256x128), (False, T.F8_128x256)):
+        am, bm, cm = matrices(1024, 4096, 4096, nt=nt)
+        am.elem_bytes = bm.elem_bytes = 1
+        k, _ = describe(am, bm, cm, mma=T.Gfx950MfmaE4M3E5M2F32_16x16x128, nt=nt, ktile=128, depth=3, a_panel=128, tiles=(T.F8_128x128, btile))
+        assert k.finalize().compile(mz.Gfx.Gfx950, cus).kernel_name == f"maize_gemm_e4m3e5m2_mt256_{'nt' if nt else 'nn'}_h128r3_gen"
+    # K % 8 != 0: no macro-tile kernel reads such operands where they lie; the description is refused, not replaced
+    k, _ = describe(*matrices(512, 512, 516), depth=3, **h128)
+    with pytest.raises(ValueError, match="no kernel with 128-row panels of A on 3 ring stages"):
+        k.finalize().compile(mz.Gfx.Gfx950, cus)
 
 
 def test_trace_errors():
@@ -188,4 +229,37 @@ def test_gpu_described_kernel_is_bit_identical_to_gemm_bf16(ctx, shape):
         assert np.array_equal(c1, c2), f"{loaded.kernel_name}: {int((c1 != c2).sum())} elements differ"
     finally:
         for x in (da, db, dc1, dc2):
+            x.free()
+
+
+@pytest.mark.gpu
+def test_gpu_panel_height_and_ring_depth_as_described_give_the_dispatchers_bits(ctx):
+    """2048^3 described three ways -- 128-row panels on three stages (the dispatcher's own choice), on two stages, and
+    256-row panels -- runs three different kernels; every one returns the bits of maize_hip_gemm_bf16."""
+    m = n = k = 2048
+    a = mz.gen.uniform_bf16(m * k, mz.gen.SEED_A)
+    b = mz.gen.uniform_bf16(k * n, mz.gen.SEED_B)
+    da, db, dc0 = ctx.upload(a), ctx.upload(b), ctx.malloc(2 * m * n)
+    try:
+        A, B = mz.Matrix(da, m, k), mz.Matrix(db, k, n)
+        ctx.gemm_bf16(mz.gemm_desc(A, B, mz.Matrix(dc0, m, n)))
+        ctx.sync()
+        want = dc0.download(np.uint16)
+        names = []
+        for kw in (dict(depth=3, a_panel=128, tiles=(T.BF16_128x64, T.BF16_64x256)), dict(depth=2, a_panel=128, tiles=(T.BF16_128x64, T.BF16_64x256)), dict()):
+            dc = ctx.upload(np.zeros(m * n, np.uint16))
+            try:
+                kernel, _ = describe(A, B, mz.Matrix(dc, m, n), **kw)
+                loaded = kernel.finalize().compile(mz.Gfx.Gfx950, ctx)
+                print(f"vocabulary: 2048^3 described as {kw.get('a_panel', 256)}-row panels, {kw.get('depth', 2)} stages -> {loaded.kernel_name}", flush=True)
+                loaded.launch()
+                ctx.sync()
+                got = dc.download(np.uint16)
+            finally:
+                dc.free()
+            names.append(loaded.kernel_name)
+            assert np.array_equal(got, want), f"{loaded.kernel_name}: {int((got != want).sum())} elements differ"
+        assert names == ["maize_gemm_bf16_mt256_nn_h128r3", "maize_gemm_bf16_mt256_nn_h128", "maize_gemm_bf16_mt256_nn"], names
+    finally:
+        for x in (da, db, dc0):
             x.free()
