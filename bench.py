@@ -387,6 +387,9 @@ def main():
                     help="cfg1..cfg5: a benchmark configuration; m64: 64x14336x4096; sq2048: 2048^3 (half a round of tiles); mid: 1024x4096x4096 N x K; f8, f8n, f8s: 4096^3 (B stored N x K, K x N) and 16x14336x4096 on E4M3 operands; f32, f64: 4096^3 on fp32 / fp64 operands; copy: the 256 MiB copy "
                          "used to scale HBM counters; energy: board power x time per 4096^3 launch for this library's kernels and register-only MFMA loops")
     ap.add_argument("--kernel", default=None, help="force a kernel by name (default: the dispatcher's choice)")
+    ap.add_argument("--shape", default=None, help="M,N,K[,batch]: a bf16 product of that shape instead of a named configuration "
+                                                   "(uniform[-1,1) operands; --layout says how B is stored)")
+    ap.add_argument("--layout", default="nn", choices=["nn", "nt"], help="--shape: B stored K x N (nn) or N x K (nt)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--others", action=argparse.BooleanOptionalAction, default=None,
                     help="also measure the other benchmark configurations (shorter runs) and report them under "
@@ -404,6 +407,13 @@ def main():
 
     if args.others is None:
         args.others = args.config is None and args.kernel is None
+    if args.shape:
+        dims = [int(x) for x in args.shape.split(",")]
+        m_, n_, k_ = dims[:3]
+        batch_ = dims[3] if len(dims) > 3 else 1
+        CONFIGS["custom"] = dict(m=m_, n=n_, k=k_, nt=int(args.layout == "nt"), batch=batch_, da=("uniform",), db=("uniform",), bound="mfma",
+                                 label=f"bf16 GEMM {'%d x ' % batch_ if batch_ > 1 else ''}{m_}x{n_}x{k_} {args.layout.upper()}, uniform[-1,1)")
+        args.config, args.others = "custom", False
     args.config = args.config or "cfg1"
     if args.config == "copy":
         copy_calibration(args.steps, args.warmup)

@@ -339,8 +339,19 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             // K x N B: the descriptor starts at row k of B (scalar 64-bit arithmetic, once per K tile) and ends with
             // the view; rows at or past K are past its end.
             const uint64_t skip = (uint64_t)k * ldb * ES;
-            const uint32_t bytes = k < k_end ? span(b_view - skip) : 0u;       // k < k_end <= K: skip < b_view
-            const __amdgpu_buffer_rsrc_t rs = make_rsrc(Bg + skip, bytes);
+            uint32_t bytes = k < k_end ? span(b_view - skip) : 0u;             // k < k_end <= K: skip < b_view
+            const char* base = Bg + skip;
+            if (GEN) {
+                // In the general-epilogue kernels the compiler carries this (uniform) 64-bit induction in vector registers
+                // and then wraps every one of the eight requests of a K tile in a loop that makes the descriptor scalar
+                // again: sixteen such loops per pair of steps, 0.15-0.2 us per step.  Said here once per K tile instead.
+                // (the builtin returns a signed int: through uint32_t, or the low word's bit 31 would smear over the high word)
+                const uint64_t u = (uint64_t)(uintptr_t)base;
+                const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)u), hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+                base = (const char*)(uintptr_t)(((uint64_t)hi << 32) | (uint64_t)lo);
+                bytes = (uint32_t)__builtin_amdgcn_readfirstlane(bytes);
+            }
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(base, bytes);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, b_vo[i], 0, 0, DMA_AUX);
             return;
         }
@@ -517,9 +528,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 else    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
                 const uint32_t k_next = R3 ? k_late - (uint32_t)BKE : k_late;  // where tile t+1 starts
                 // tile t+1 holds row K - 1 and belongs to this item's K range (the steps that pad a range to a whole
-                // trip run on zero tiles at or past k_end: there A is zero, and a real Inf in B would make NaN of it)
-                if (PATCHES && patch_on && k_next < k_end && K - 1u - k_next < (uint32_t)BKE)
-                    asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)pb + patch_off), "v"(patch_val) : "memory");
+                // trip run on zero tiles at or past k_end: there A is zero, and a real Inf in B would make NaN of it).
+                // Without a branch (one inside the step splits the loop's single basic block): when there is nothing to
+                // patch the write goes to this wave's own epilogue staging, which is idle during the K loop.
+                if (PATCHES) {
+                    const bool on = patch_on && k_next < k_end && K - 1u - k_next < (uint32_t)BKE;
+                    const uint32_t at = on ? (uint32_t)(uintptr_t)pb + patch_off : (uint32_t)(uintptr_t)lds_e + wave * (R3 ? 4096u : 8192u);
+                    asm volatile("ds_write_b16 %0, %1" :: "v"(at), "v"(patch_val) : "memory");
+                }
                 MAIZE_FENCE();
             }
 #pragma unroll

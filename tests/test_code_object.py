@@ -217,3 +217,21 @@ def test_main_loop_of_the_three_stage_kernels_is_lean(kernels):
         want = "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16"
         assert count(kernels[name], want) == 192 and count(kernels[name], "v_mfma") == 192, name
 
+
+
+def test_no_k_loop_wraps_its_requests_in_scalarising_loops(kernels):
+    """A buffer descriptor that the compiler carries in vector registers makes it wrap every request in a loop that
+    reads the descriptor back lane by lane (v_readfirstlane / s_and_saveexec / s_cbranch_execnz): the general-epilogue
+    and split-K kernels on a row-major 16-bit B had sixteen of those per pair of K steps (and a branch around the odd-N
+    fix-up), 8-22 % of their run time.  Every macro-tile K loop is one basic block: no exec-mask juggling, no branch
+    between its first and its last matrix instruction other than the loop's own, a handful of readfirstlanes at most
+    (the descriptor of a K x N B, said once per K tile).  And no descriptor word is sign-extended on its way."""
+    for name, ins in kernels.items():
+        if "_mt256_" not in name or name.endswith("_edge"):       # (the edge kernels hold three loops, checked by their own test)
+            continue
+        idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
+        body = ins[idx[0]:idx[-1] + 1]
+        assert count(body, "s_and_saveexec") == 0 and count(body, "s_cbranch_exec") == 0, name
+        assert count(body, "v_readfirstlane") <= 12, (name, count(body, "v_readfirstlane"))
+        assert count(body, "s_cbranch") <= 1, name
+        assert count(ins, "s_bfe_i64") == 0, name

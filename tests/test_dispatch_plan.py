@@ -405,3 +405,29 @@ def test_the_special_value_families_hold_a_range_padded_with_bs_last_tile():
     assert any(kern.endswith("_h128r3_splitk") for kern, _ in hit), hit
     assert any(kern == "maize_gemm_bf16_mt256_nn_splitk" for kern, _ in hit), hit
     assert any(auto for _, auto in hit), hit
+
+
+def _steps_of_the_ranges(k, ksplit):
+    nk = cdiv(k, 64)
+    per = cdiv(nk, max(1, ksplit))
+    return [min(per, nk - z * per) for z in range(max(1, ksplit)) if nk - z * per > 0]
+
+
+def test_the_named_three_stage_cases_have_a_ragged_m_and_a_step_count_off_three():
+    """The GPU suite runs the three-stage 128-row kernels by name (tests/test_gpu_random_products.py: H128R3_CASES).  Here,
+    without a device: each kernel accepts its case, M is no multiple of 128, and some K range runs a number of steps
+    that is no multiple of three (the loop runs three steps per trip and pads with zero tiles); both layouts, the plain,
+    general and split-K forms are all there."""
+    from tests.test_gpu_random_products import H128R3_CASES
+    for name, layout, m, n, k, kw in H128R3_CASES:
+        brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+        x = mz.gemm_ex_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x1000, brows, bcols), mz.GlobalMatrix(0x1000, m, n), layout=layout,
+                            in_type=mz.IN_F16 if kw.get("half") else mz.IN_BF16, out_type=mz.OUT_F32 if kw.get("out_f32") else mz.OUT_SAME,
+                            alpha=kw.get("alpha", 1.0), beta=kw.get("beta", 0.0))
+        plan = mz.gemm_plan(x, kernel=name, compute_units=CUS)
+        assert plan["kernel"] == name and m % 128 != 0, name
+        assert any(s % 3 for s in _steps_of_the_ranges(k, plan["ksplit"] if name.endswith("_splitk") else 1)), (name, plan)
+    names = {c[0] for c in H128R3_CASES}
+    for lay in ("nn", "nt"):
+        for form in ("_h128r3", "_h128r3_gen", "_h128r3_splitk"):
+            assert f"maize_gemm_bf16_mt256_{lay}{form}" in names

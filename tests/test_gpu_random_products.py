@@ -103,3 +103,25 @@ def test_random_midsize_products_with_a_long_k(ctx, oracle, seed):
         reached[took.replace("maize_gemm_", "")] += 1
     _say(f"seed {seed}: kernels reached: {dict(reached)}")
     assert any("h128r3" in name for name in reached)
+
+
+# The three-stage 128-row kernels by name, not by the luck of a draw: every one of them on a ragged M (no multiple of
+# 128) and a K whose step count is no multiple of three (the loop runs three steps per trip and pads with zero tiles),
+# both layouts, K tails for the kernels that take them, half operands once.
+H128R3_CASES = [
+    ("maize_gemm_bf16_mt256_nn_h128r3", mz.LAYOUT_NN, 1000, 2048, 64 * 31, {}),
+    ("maize_gemm_bf16_mt256_nt_h128r3", mz.LAYOUT_NT, 904, 1024, 64 * 32, {}),
+    ("maize_gemm_bf16_mt256_nn_h128r3_gen", mz.LAYOUT_NN, 1000, 2056, 64 * 34 + 8, dict(alpha=-1.25, beta=0.75)),
+    ("maize_gemm_bf16_mt256_nt_h128r3_gen", mz.LAYOUT_NT, 648, 1032, 64 * 31 + 16, dict(out_f32=True, alpha=3.0, beta=-0.5)),
+    ("maize_gemm_f16_mt256_nn_h128r3_gen", mz.LAYOUT_NN, 520, 1024, 64 * 29, dict(half=True)),
+    ("maize_gemm_bf16_mt256_nn_h128r3_splitk", mz.LAYOUT_NN, 392, 1024, 64 * 61, {}),
+    ("maize_gemm_bf16_mt256_nt_h128r3_splitk", mz.LAYOUT_NT, 264, 2048, 64 * 59 + 8, {}),
+    ("maize_gemm_f16_mt256_nt_h128r3_splitk", mz.LAYOUT_NT, 200, 1536, 64 * 64, dict(half=True, out_f32=True)),
+]
+
+
+@pytest.mark.parametrize("case", H128R3_CASES, ids=lambda c: f"{c[0].replace('maize_gemm_', '')}-{c[2]}x{c[3]}x{c[4]}")
+def test_the_three_stage_kernels_by_name(ctx, oracle, case):
+    name, layout, m, n, k, kw = case
+    took = run_ex(ctx, oracle, m, n, k, layout=layout, kernel=name, seed=7, label=f"named {name}", **kw)
+    assert took == name
