@@ -236,10 +236,24 @@ bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld
 // split; 64 x 4096 x 4096: 63 -> 22 us; 256 x 256 x 16384: 237 -> 38 us; 256 x 14336 x 4096, 56 tiles:
 // 67 -> 46 us four ways; 768 x 8192 x 8192, 96 tiles: 128 -> 93 us two ways.)
 // cost: what the model expects of the choice, in K steps of the unsplit kernel (~1.1 us), rounds of tiles counted.
+// Bytes as well as steps.  Operands past the 256 MiB memory-side cache come from HBM on every launch; a workgroup draws
+// about 33 GB/s of such a stream and the chip at most 4.3 TB/s in the tile kernels' access pattern (128 x 28672 x 8192, a
+// 470 MB weight matrix: 112 whole 128-row tiles on 112 of the 256 compute units 124-130 us whatever their K steps cost,
+// two K ranges on 224 of them 115-119 us).  Lower bound, in microseconds, of `items` work items streaming the operands.
+double stream_us(const Dims& s, uint32_t batch, uint32_t kstep, uint64_t items) {
+    const double mbytes = (kstep == 128u ? 1.0 : 2.0) * ((double)s.m * s.k + (double)s.k * s.n) * batch / 1e6;
+    if (mbytes * 1e6 <= 256.0 * 1048576.0 || items == 0) return 0.0;
+    const double tbs = 0.033 * (double)items;
+    return mbytes / (tbs < 4.3 ? tbs : 4.3);
+}
 uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64, double* cost = nullptr) {
     const uint64_t tiles = (uint64_t)cdiv(s.m, 256) * cdiv(s.n, 256) * batch;
     const uint32_t nk = cdiv(s.k, kstep);                    // K steps of 128 bytes per row: 64 16-bit elements, 128 8-bit ones
-    if (cost) *cost = (8.0 + 1.0 * nk) * (double)(cus ? cdiv64(tiles, cus) : 1u);
+    if (cost) {
+        *cost = (8.0 + 1.0 * nk) * (double)(cus ? cdiv64(tiles, cus) : 1u);
+        const double st = stream_us(s, batch, kstep, cus && tiles > cus ? cus : tiles);
+        if (*cost < st) *cost = st;
+    }
     if (cus == 0 || tiles == 0 || tiles * 2 > cus || nk < 8u) return 1;
     uint32_t kmax = (uint32_t)(cus / tiles);
     if (kmax > nk / 4u) kmax = nk / 4u;
@@ -254,7 +268,11 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
         const double t = 8.0 + 1.0 * cdiv(nk, ks) + 6.0 + (1.2e-6 * elems + 0.15) * ks;
         if (t < best) { best = t; best_ks = ks; }
     }
-    if (cost && best_ks > 1u) *cost = best;
+    if (cost && best_ks > 1u) {
+        *cost = best;
+        const double st = stream_us(s, batch, kstep, tiles * best_ks) + 6.0;     // (the partial tiles travel in the stream's shadow)
+        if (*cost < st) *cost = st;
+    }
     return best_ks;
 }
 // 128 x 256 tiles instead: when they fit one round of the compute units (the 256 x 256 tiles fill half of them or
@@ -296,8 +314,10 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     // a long K: the three-stage kernels, steps in threes (2048^3 28.6 -> 24.9 us, 1024 x 4096 x 4096 51.1 -> 42.0,
     // 640 x 8192 x 4096 N x K 60.4 -> 45.9)
     const bool three = h128_three_stages(s.k, kstep, half_tiles);
-    const double whole = 8.0 + scale * h128_step(three, false, s.nt, kstep == 128u) * (three ? 3u * cdiv(nk, 3u) : nk);
-    double best = 0.9 * whole;                                     // splitting has to win 10 %
+    // (bytes as well as steps: stream_us)
+    double whole = 8.0 + scale * h128_step(three, false, s.nt, kstep == 128u) * (three ? 3u * cdiv(nk, 3u) : nk);
+    if (whole < stream_us(s, batch, kstep, half_tiles)) whole = stream_us(s, batch, kstep, half_tiles);
+    double best = 0.9 * whole, best_cost = whole;                  // splitting has to win 10 %
     uint32_t best_ks = 1;
     const double elems = (double)s.m * s.n * batch;
     uint32_t kmax = (uint32_t)(resident / half_tiles);
@@ -311,10 +331,16 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
             const uint32_t r = cdiv(nk, ks);
             const bool three_r = h128_three_stages(r * kstep, kstep, half_tiles * ks);
             const double loop = scale * h128_step(three_r, true, s.nt, kstep == 128u) * (three_r ? 3u * cdiv(r, 3u) : r);
-            const double t = 8.0 + loop + 6.0 + (1.2e-6 * elems + 0.15) * ks;
-            if (t < best) { best = t; best_ks = ks; }
+            double t = 8.0 + loop + 6.0 + (1.2e-6 * elems + 0.15) * ks;
+            // (bound by the stream: the partial tiles travel in its shadow, the second launch does not; and there a
+            // split that brings more compute units to the stream only has to win 5 %)
+            const double ts = stream_us(s, batch, kstep, half_tiles * ks) + 6.0;
+            const bool by_stream = ts > t;
+            if (by_stream) t = ts;
+            const double score = by_stream ? t * 0.9 / 0.95 : t;  // (what is compared with 0.9 x the whole tiles' cost)
+            if (score < best) { best = score; best_cost = t; best_ks = ks; }
         }
-    if (best_ks == 1u) best = whole;
+    best = best_cost;
     // (a tie goes to the tiles: the model flatters large splits, 768 x 8192 x 8192 109.6 us in two ranges, 94.4 here; more
     // so with 8-bit operands, whose fixed terms it overrates: E4M3 N x K, 46 mid-size shapes with every candidate by name,
     // the two it gave to the 256-row split were both faster in tiles -- 256 x 2048 x 2048 18.5 against 14.3-15.9 us,

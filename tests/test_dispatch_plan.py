@@ -431,3 +431,27 @@ def test_the_named_three_stage_cases_have_a_ragged_m_and_a_step_count_off_three(
     for lay in ("nn", "nt"):
         for form in ("_h128r3", "_h128r3_gen", "_h128r3_splitk"):
             assert f"maize_gemm_bf16_mt256_{lay}{form}" in names
+
+
+def test_operands_past_the_memory_side_cache_are_priced_by_their_bytes_too():
+    """The 128-row tile choice prices bytes as well as K steps: a 470 MB weight matrix (28672 x 8192) against 96 .. 128
+    rows is bound by its stream from HBM, which two K ranges on 224 compute units draw faster than 112 whole tiles on
+    112 of them (measured, K x N: 95.7 / 100.5 us against 123.6 / 129.9; N x K: 119.2 / 122.8 against 122.9 / 125.0);
+    with 192 rows the whole tiles already occupy 224 units and stay (122.9 us against 146.3 split).  Operands that fit
+    the cache keep the choice the K steps make."""
+    for m in (96, 128):
+        for layout in (mz.LAYOUT_NN, mz.LAYOUT_NT):
+            p = mz.gemm_plan(desc(m, 28672, 8192, layout), compute_units=CUS)
+            assert p["kernel"].endswith("_h128r3_splitk") and p["ksplit"] == 2 and p["grid"][0] == 224, p
+    for layout in (mz.LAYOUT_NN, mz.LAYOUT_NT):
+        p = mz.gemm_plan(desc(192, 28672, 8192, layout), compute_units=CUS)
+        assert p["kernel"].endswith("_h128r3") and p["ksplit"] <= 1, p
+    p = mz.gemm_plan(desc(96, 28672, 4096), compute_units=CUS)          # 235 MB: stays in whole tiles
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3", p
+
+
+def test_the_boundary_between_whole_128_row_tiles_and_their_split():
+    """640 x 8192 x 4096 with B stored N x K, 160 tiles of 128 x 256: whole tiles on three ring stages (45.9 us) beat
+    the split over K (56.7 us), which an earlier rule took here."""
+    p = mz.gemm_plan(desc(640, 8192, 4096, mz.LAYOUT_NT), compute_units=CUS)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3" and p["grid"][0] == 160, p
