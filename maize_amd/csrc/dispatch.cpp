@@ -830,6 +830,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_f64_mt128_nt", nullptr, mt128_supports<MAIZE_IN_F64, true>, mt128_plan},
     {"maize_gemm_bf16_mt256_nn", nullptr, mt256_nn_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt", nullptr, mt256_nt_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_asm", nullptr, mt256_nn_supports, mt256_plan},      // the K loop as one assembly statement
+    {"maize_gemm_bf16_mt256_nt_asm", nullptr, mt256_nt_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_h128", nullptr, mt256_nn_supports, mt256_h128_plan},
     {"maize_gemm_bf16_mt256_nt_h128", nullptr, mt256_nt_supports, mt256_h128_plan},
     {"maize_gemm_bf16_mt256_nn_h128_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_h128_plan},
@@ -1085,9 +1087,17 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     if (!strict && si >= 0 && kKernels[si].supports(d) && !c_rows16(d) && (s.k >= 128 || (s.m >= 128 && s.n >= 128)) &&
         (double)s.m * s.n * s.k * d.gemm.batch >= 3e7 && plan_fits(kKernels[si], d, compute_units))
         return (uint32_t)si;
-    const int ti = half_in(d)                    ? kernel_index(kHalf[(s.k & 63u) != 0][s.nt])
-                   : plain_epilogue(d) && strict ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
-                                                 : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
+    int ti = half_in(d)                    ? kernel_index(kHalf[(s.k & 63u) != 0][s.nt])
+             : plain_epilogue(d) && strict ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
+                                           : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
+    // An odd number of K steps: the plain kernel's statement loop runs two steps per trip and pads with a step on a
+    // zero tile; the same loop as one assembly statement leaves the trip after its first step (4096 x 4096 x K, K = 192:
+    // 14.1 -> 12.8 us, 576: 21.8 -> 20.2, 1088: 30.6 -> 29.4, 3008: 67.6 -> 66.5; at even counts it is level or up to 1 % behind).
+    if (!half_in(d) && plain_epilogue(d) && strict && !edge && (s.k & 63u) == 0 && ((s.k >> 6) & 1u)) {
+        static const char* const kOddSteps[2] = {"maize_gemm_bf16_mt256_nn_asm", "maize_gemm_bf16_mt256_nt_asm"};
+        const int oi = kernel_index(kOddSteps[s.nt]);
+        if (oi >= 0 && kKernels[oi].supports(d)) ti = oi;
+    }
     // The macro-tile kernel pays for a 256 x 256 tile and ~8 us whatever the shape, but it moves
     // its operands in 128-bit requests: measured, it beats the per-wave kernel 4-7x from
     // 16 x 4096 x 4096 up and loses (8 vs 4-7 us) only on short K with few rows or columns.

@@ -70,6 +70,7 @@
 
 namespace maize {
 namespace mt256 {
+#include "kloop_gen.inc"   // kloop_asm_nt / kloop_asm_nn: the plain 256-row K loop as one assembly statement (gen_kloop.py)
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int THREADS = 256;
@@ -147,9 +148,12 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 // offset field, and has base registers of its own.
 // 8-bit operands on three stages: A's fragment buffer goes with the stage (three of them), the twelve pieces of tile
 // t+3 go out one every two slots from the barrier of step t on (seven behind it, five in front of the next), same wait.
-template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2>
+// ASM: the K loop is the generated assembly statement (kloop_gen.inc) instead of the step() statements below: the same
+// schedule with registers assigned by hand, for the plain 256-row bf16 kernels.
+template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2, bool ASM = false>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
+    static_assert(!ASM || (!KTAIL && !EDGE && !GEN && !F16 && !SPLITK && F8 < 0 && BMT == 256 && NST == 2), "the assembly K loop: plain 256-row bf16 kernels");
     constexpr bool H128 = BMT == 128;
     static_assert(BMT == 256 || (H128 && !EDGE), "128-row tiles: no edge splitting");
     constexpr bool R3 = NST == 3;                       // three ring stages (128-row tiles)
@@ -308,20 +312,24 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 patch_val = ((const uint16_t*)Bg)[(uint64_t)(K - 1u) * ldb + N - 1u];
             }
         }
+        // (The hand-allocated K loop leaves the compiler sixty-odd registers: its offsets are derived again per tile from a
+        // lane number the compiler cannot see through, rather than from per-lane terms kept across the loop.)
+        uint32_t ln = lane;
+        if constexpr (ASM) asm volatile("" : "+v"(ln));
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint32_t row = maps::kc_piece_row(wave * 8u + i, lane);
-            const uint32_t c = maps::kc_piece_chunk(wave * 8u + i, lane);
+            const uint32_t row = maps::kc_piece_row(wave * 8u + i, ln);
+            const uint32_t c = maps::kc_piece_chunk(wave * 8u + i, ln);
             if (i < PA) {                                   // A: pieces wave * PA + i (the lane's chunk depends on the piece's parity only)
-                const uint32_t arow = maps::kc_piece_row(wave * PA + i, lane), ac = maps::kc_piece_chunk(wave * PA + i, lane);
+                const uint32_t arow = maps::kc_piece_row(wave * PA + i, ln), ac = maps::kc_piece_chunk(wave * PA + i, ln);
                 a_vo[i] = (arow * lda + ac * CH) * ES;
                 if (i < 2) a_k[i] = ac * CH;
             }
             if (NT) {
                 b_vo[i] = (row * ldb + c * CH) * ES;
             } else {
-                const uint32_t brow = TR8 ? maps::sk8_piece_row(wave * 8u + i, lane) : maps::sk_piece_row(wave * 8u + i, lane);
-                const uint32_t bc = TR8 ? maps::sk8_piece_chunk(wave * 8u + i, lane) : maps::sk_piece_chunk(wave * 8u + i, lane);
+                const uint32_t brow = TR8 ? maps::sk8_piece_row(wave * 8u + i, ln) : maps::sk_piece_row(wave * 8u + i, ln);
+                const uint32_t bc = TR8 ? maps::sk8_piece_chunk(wave * 8u + i, ln) : maps::sk_piece_chunk(wave * 8u + i, ln);
                 b_vo[i] = ((brow * ldb + n0 + bc * CH) * ES) | ((n0 + bc * CH) < N ? 0u : OOB);
             }
         }
@@ -493,6 +501,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     };
 
     floatx4 acc[MI][8];
+    // Assembly K loop, deferred C stores: a C tile that is not the workgroup's last is only rounded to bf16 (ct: pair
+    // (2 i + ii) * 8 + j of pass i, accumulator row ii, column block j) and stored while the first sixteen K steps of the
+    // next tile run (kloop_asm_*_drain) -- the stores of 128 KiB per compute unit, which the whole chip issues at the same
+    // moment, otherwise hold every wave at the store issue with the matrix pipe idle (4.6 us per tile at 32 x 2048^3).
+    // Taken when a tile has at least sixteen K steps.
+    constexpr uint32_t DRAIN_STEPS = KLOOP_DRAIN_STEPS;   // 0: C tiles are stored at once (the build that ships)
+    constexpr bool DEFER = ASM && DRAIN_STEPS > 0;
+    u32x4 ct[DEFER ? 32 : 1];
+    bool have_ct = false;
+    uint32_t ct_lo = 0, ct_hi = 0, ct_bytes = 0, ct_vo = 0;
     uint32_t k_early = 0;                  // tile whose early pieces are issued next (last quarter of a step)
     uint32_t k_late = 0;                   // tile whose late pieces are issued next (first quarter of a step)
 
@@ -611,10 +629,12 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     if (PATCHES && patch_on && k_begin < k_end && K - 1u - k_begin < (uint32_t)BKE)   // the item's first K tile is also B's last
         asm volatile("ds_write_b16 %0, %1" :: "v"((uint32_t)(uintptr_t)B0 + patch_off), "v"(patch_val) : "memory");
+    if (!ASM) {                                                 // (the assembly loop reads its first fragments itself)
 #pragma unroll
-    for (int r = 0; r < NAR; ++r) read_a(0, 0, 0, r);
+        for (int r = 0; r < NAR; ++r) read_a(0, 0, 0, r);
 #pragma unroll
-    for (int r = 0; r < NBR; ++r) read_b(0, 0, 0, r);
+        for (int r = 0; r < NBR; ++r) read_b(0, 0, 0, r);
+    }
 #pragma unroll
     for (int pc = 0; pc < NP; ++pc)
         if (DS * pc + 2 < AFTER) dma(pc, A0 + (NST - 1) * ASTR, B0 + (NST - 1) * TILE, k_begin + (NST - 1) * BKE);   // tile 1 (three stages: 2), early pieces
@@ -624,7 +644,38 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // is not a multiple runs the extra steps on all-zero tiles (loads past K return zeros).  (Leaving the trip after
     // the step that was the last costs more than it saves: with exits between the steps the register allocator no
     // longer keeps the loop's operands in place.)
-    if (EDGE && split && mode == 1u) {
+    if constexpr (ASM) {
+        // Descriptor words and LDS bases as scalars (uniform values; said so explicitly).
+        auto sc = [](uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane(x); };
+        const uint64_t au = (uint64_t)(uintptr_t)Ag;
+        const uint32_t lds_a = sc((uint32_t)(uintptr_t)A0 + wave_u * 8192u), lds_b = sc((uint32_t)(uintptr_t)B0 + wave_u * 8192u);
+        const uint32_t c_row_bytes = sc(ldc * 2u);                                    // one row of C, in bytes
+        // sixteen rows of a K-contiguous operand, resp. four rows of a row-major B: what separates pieces of one swizzle phase
+        const uint32_t a_step = sc(16u * lda * ES), b_step = sc((NT ? 16u : 4u) * ldb * ES);
+        bool drained = false;
+        if (NT) {
+            const uint64_t bu = (uint64_t)(uintptr_t)Bg;
+            if constexpr (DEFER) { if (have_ct) { drained = true;
+                kloop_asm_nt_drain(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu),
+                                   sc((uint32_t)(bu >> 32) & 0xFFFFu), sc(b_bytes), 0u, 0u, 0u, 0u, 0x00020000u, lds_a, lds_b, k_early, k_late, sc(k_end), sc(nk),
+                                   ct, ct_vo, sc(ct_lo), sc(ct_hi), sc(ct_bytes), c_row_bytes); } }
+            if (!drained)
+                kloop_asm_nt(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu),
+                             sc((uint32_t)(bu >> 32) & 0xFFFFu), sc(b_bytes), 0u, 0u, 0u, 0u, 0x00020000u, lds_a, lds_b, k_early, k_late, sc(k_end), sc(nk));
+        } else {
+            // a K x N B: the address of row k_late and the bytes from there to the end of the view, then one K tile's rows on
+            const uint64_t skip = (uint64_t)k_late * ldb * ES, bu = (uint64_t)(uintptr_t)Bg + skip, rem = b_view - skip, stp = (uint64_t)BKE * ldb * ES;
+            if constexpr (DEFER) { if (have_ct) { drained = true;
+                kloop_asm_nn_drain(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu), sc((uint32_t)(bu >> 32)),
+                                   0u, sc((uint32_t)rem), sc((uint32_t)(rem >> 32)), sc((uint32_t)stp), sc((uint32_t)(stp >> 32)), 0x00020000u, lds_a, lds_b, k_early, k_late,
+                                   sc(k_end), sc(nk), ct, ct_vo, sc(ct_lo), sc(ct_hi), sc(ct_bytes), c_row_bytes); } }
+            if (!drained)
+                kloop_asm_nn(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu), sc((uint32_t)(bu >> 32)),
+                             0u, sc((uint32_t)rem), sc((uint32_t)(rem >> 32)), sc((uint32_t)stp), sc((uint32_t)(stp >> 32)), 0x00020000u, lds_a, lds_b, k_early, k_late,
+                             sc(k_end), sc(nk));
+        }
+        have_ct = false;
+    } else if (EDGE && split && mode == 1u) {
         for (uint32_t kt = 0; kt < nk; kt += 2) { step(0, 1); step(1, 1); }
     } else if (EDGE && split) {
         for (uint32_t kt = 0; kt < nk; kt += 2) { step(0, 2); step(1, 2); }
@@ -778,7 +829,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         }
     } else if (finish) {                                         // (a K range that was not the last to arrive stores nothing)
         lds_ptr ew = (lds_ptr)lds_e + wave_u * (R3 ? 4096u : 8192u);
-        const uint32_t cc = lane & 15u, cr = lane >> 4;          // 16 lanes per 256-byte row, 4 rows per read
+        uint32_t le = lane;                                      // (hand-allocated K loop: per-lane terms derived here, not kept across it)
+        if constexpr (ASM) asm volatile("" : "+v"(le));
+        const uint32_t cc = le & 15u, cr = le >> 4;              // 16 lanes per 256-byte row, 4 rows per read
         const uint32_t gcol = en0 + wn * 128u + cc * 8u;
         // Stores go through a buffer descriptor over this batch member's C: rows at or past M fall
         // behind its end and are dropped by the range check, columns at or past N (N % 8 == 0: a
@@ -788,6 +841,32 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const __amdgpu_buffer_rsrc_t rc = make_rsrc(Ce + (uint64_t)em0 * ldc, span(((uint64_t)(M - 1u - em0) * ldc + N) * 2u));
         const uint32_t c_vo = (((wm * WROWS + cr) * ldc + gcol) * 2u) | (gcol < N ? 0u : OOB);
         const uint32_t row_bytes = __builtin_amdgcn_readfirstlane(ldc * 2u);
+        bool stored_later = false;
+        if constexpr (DEFER) {
+            if (more && nk_all >= DRAIN_STEPS) {
+                // Not the workgroup's last tile: round it to bf16, turn it through LDS into store order like below, and keep
+                // what the stores would have written; the next tile's K loop stores it from these registers.
+                const uint64_t cu = (uint64_t)(uintptr_t)(Ce + (uint64_t)em0 * ldc);
+                ct_lo = (uint32_t)cu; ct_hi = (uint32_t)(cu >> 32) & 0xFFFFu; ct_bytes = span(((uint64_t)(M - 1u - em0) * ldc + N) * 2u);
+                ct_vo = c_vo;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            asm volatile("" : "+a"(acc[2 * i + ii][j]));
+                            const floatx4 f = acc[2 * i + ii][j];
+                            *(lds_v2)(ew + maps::epi16_write_offset(ii, j, le)) = u32x2{cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
+                        }
+#pragma unroll
+                    for (int r = 0; r < 8; ++r) ct[i * 8 + r] = *(lds_v4)(ew + maps::epi16_read_offset(r, le));
+                }
+                have_ct = true;
+                stored_later = true;
+            }
+        }
+        if (!stored_later) {
     #pragma unroll
         for (int i = 0; i < MI / EPR; ++i) {
     #pragma unroll
@@ -795,15 +874,19 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     // lane holds C[row = (2i+ii)*16 + l16][col = j*16 + 4*lg + 0..3]
+                    // (behind the assembly K loop nothing else needs the accumulators in AccVGPRs, and the allocator would
+                    // move all 256 to vector registers at once, spilling: each is pinned there until its pass reads it)
+                    if constexpr (ASM) asm volatile("" : "+a"(acc[EPR * i + ii][j]));
                     floatx4 f = acc[EPR * i + ii][j];
                     u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
-                    *(lds_v2)(ew + maps::epi16_write_offset(ii, j, lane)) = v;
+                    *(lds_v2)(ew + maps::epi16_write_offset(ii, j, le)) = v;
                 }
     #pragma unroll
             for (int r = 0; r < 4 * EPR; ++r) {
-                const u32x4 v = *(lds_v4)(ew + maps::epi16_read_offset(r, lane));
+                const u32x4 v = *(lds_v4)(ew + maps::epi16_read_offset(r, le));
                 __builtin_amdgcn_raw_buffer_store_b128(v, rc, c_vo, (uint32_t)(i * 16 * EPR + r * 4) * row_bytes, 2 /* nt */);
             }
+        }
         }
     }
     if (!more) break;
@@ -819,6 +902,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     extern "C" __global__ __launch_bounds__(256) void name(GemmArgs p) { mt256::body<nt, ktail, false, true, f16, false>(p); }
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn, false, false, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt, true, false, false)
+// ... with the K loop as one assembly statement (gen_kloop.py)
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_asm(GemmArgs p) { mt256::body<false, false, false, false, false, false, -1, 256, 2, true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_asm(GemmArgs p) { mt256::body<true, false, false, false, false, false, -1, 256, 2, true>(p); }
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail, false, true, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_ktail, true, true, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_edge, false, false, true)

@@ -32,7 +32,8 @@ def kernels():
     for line in text.splitlines():
         m = re.match(r"^[0-9a-f]+ <([A-Za-z0-9_]+)>:", line)
         if m:
-            cur = out.setdefault(m.group(1), [])
+            if not m.group(1).startswith("L_"):       # (labels inside an assembly statement are not kernels)
+                cur = out.setdefault(m.group(1), [])
             continue
         if cur is not None and "\t" in line:
             ins = line.split("//")[0].strip()

@@ -455,3 +455,19 @@ def test_the_boundary_between_whole_128_row_tiles_and_their_split():
     the split over K (56.7 us), which an earlier rule took here."""
     p = mz.gemm_plan(desc(640, 8192, 4096, mz.LAYOUT_NT), compute_units=CUS)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3" and p["grid"][0] == 160, p
+
+
+def test_an_odd_number_of_k_steps_takes_the_loop_that_leaves_after_its_first_step():
+    """The plain 256-row kernel's statement loop pads an odd step count with a step on a zero tile; the assembly loop
+    does not.  Even counts, K tails, split edges and the general epilogue keep their kernels."""
+    for layout, tag in ((mz.LAYOUT_NN, "nn"), (mz.LAYOUT_NT, "nt")):
+        for k in (192, 576, 1088, 3008):
+            assert mz.gemm_plan(desc(4096, 4096, k, layout), compute_units=CUS)["kernel"] == f"maize_gemm_bf16_mt256_{tag}_asm", (tag, k)
+        for k in (256, 1024, 4096):
+            assert mz.gemm_plan(desc(4096, 4096, k, layout), compute_units=CUS)["kernel"] == f"maize_gemm_bf16_mt256_{tag}", (tag, k)
+        assert mz.gemm_plan(desc(4096, 4096, 576 + 8, layout), compute_units=CUS)["kernel"] == f"maize_gemm_bf16_mt256_{tag}_ktail"
+        assert mz.gemm_plan(desc(4000, 4104, 4032, layout), compute_units=CUS)["kernel"] == f"maize_gemm_bf16_mt256_{tag}_edge"
+        x = ex_desc(4096, 4096, 576, layout)
+        x.alpha = 0.5
+        p = mz.gemm_plan(x, compute_units=CUS)
+        assert p["kernel"] == f"maize_gemm_bf16_mt256_{tag}_gen", p
