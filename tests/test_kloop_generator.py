@@ -162,3 +162,13 @@ def test_replay_rejects_a_wrong_fragment():
     del lines[k]
     with pytest.raises(AssertionError):
         Replay(gen, True).run([l for l in lines if not l.startswith("L_")], stage_of_step=lambda t: t & 1)
+
+
+def test_the_default_make_target_builds_the_library_and_the_generated_loop_first():
+    """`make` with no target must build libmaize_hip.so (a rule placed in front of `all` silently becomes the default
+    target), and the code object depends on the generated include."""
+    import subprocess
+    csrc = os.path.dirname(os.path.dirname(GEN))
+    plan = subprocess.run(["make", "-n", "-B", "-C", csrc], check=True, capture_output=True, text=True).stdout
+    assert "gen_kloop.py" in plan and "gemm_kernels.hip" in plan and "libmaize_hip.so" in plan
+    assert plan.index("gen_kloop.py") < plan.index("gemm_kernels.hip") < plan.index("libmaize_hip.so")
