@@ -295,11 +295,12 @@ bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles) {
     return nk >= (kstep == 128u ? 18u : 28u) && (nk >= 48u || half_tiles >= 48u);
 }
 // What a K step of a 128-row tile costs, in steps of the 256-row kernel at the power limit (~ microseconds): 0.67 on two
-// ring stages, 0.52 on three -- except for K ranges of a row-major B on three stages, i.e. long ranges, which measure
-// 0.82-0.91 whatever share of the chip is at work (1024 x 4096 x 14336 in two ranges 123.6 us, N x K 101.5;
-// 512 x 8192 x 8192 78.6 / 66.2; 384 x 6144 x 4096 44.4 / 35.0), so that whole tiles or the 256-row split win there.
-// (16-bit operands only: E4M3 K x N, 384 x 8192 x 8192 in two ranges 36.6 us against 42.2 whole and 44.0 in 256-row tiles.)
-double h128_step(bool three, bool split, bool nt, bool bits8) { return !three ? 0.67 : (split && !nt && !bits8) ? 0.85 : 0.52; }
+// ring stages, 0.52 on three; K ranges of a row-major 16-bit B on three stages 0.55 (same plans, same box, K x N against
+// N x K: 512 x 4096 x 14336 in four ranges 65.0 / 61.3 us, 512 x 8192 x 8192 69.0 / 67.2, 384 x 6144 x 4096 36.6 / 34.2,
+// 384 x 4096 x 14336 51.7 / 50.2).  (These used to be priced at 0.85: the K x N loop then carried a scalarising loop around
+// every request, and once priced that way a kernel named for a shape got two ranges where N x K got four, which kept
+// the figure looking true.)
+double h128_step(bool three, bool split, bool nt, bool bits8) { return !three ? 0.67 : (split && !nt && !bits8) ? 0.55 : 0.52; }
 // Returns 0: the 256-row kernels; 1: 128-row tiles, whole K; >= 2: 128-row tiles in that many K ranges.
 uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
     const uint32_t resident = cus >= 8u ? cus - cus % 8u : cus;

@@ -346,18 +346,38 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         if (!is_a && !NT) {
             // K x N B: the descriptor starts at row k of B (scalar 64-bit arithmetic, once per K tile) and ends with
             // the view; rows at or past K are past its end.
-            const uint64_t skip = (uint64_t)k * ldb * ES;
-            uint32_t bytes = k < k_end ? span(b_view - skip) : 0u;             // k < k_end <= K: skip < b_view
-            const char* base = Bg + skip;
+            const char* base;
+            uint32_t bytes;
             if (GEN) {
-                // In the general-epilogue kernels the compiler carries this (uniform) 64-bit induction in vector registers
-                // and then wraps every one of the eight requests of a K tile in a loop that makes the descriptor scalar
-                // again: sixteen such loops per pair of steps, 0.15-0.2 us per step.  Said here once per K tile instead.
-                // (the builtin returns a signed int: through uint32_t, or the low word's bit 31 would smear over the high word)
-                const uint64_t u = (uint64_t)(uintptr_t)base;
-                const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)u), hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+                // In the kernels whose K range comes from the work item the compiler carries this (uniform) arithmetic on
+                // the vector unit -- the range and the batch index come out of divisions -- and then reads the descriptor
+                // back in front of the requests, which bunches them behind a chain of dependent vector instructions (and,
+                // in a first version, wrapped each request in a loop that made the descriptor scalar).  Scalar operands
+                // are asked for outright: once per K tile, eleven scalar instructions.
+                // (An "s" constraint alone does not do it: a value the compiler keeps in a vector register arrives as one.)
+                auto sc = [](uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane(x); };
+                const uint64_t bu = (uint64_t)(uintptr_t)Bg;
+                uint32_t lo, hi, t;
+                asm("s_mul_i32 %[lo], %[k], %[row]\n\t"            // bytes from B's first row to row k ...
+                    "s_mul_hi_u32 %[hi], %[k], %[row]\n\t"
+                    "s_sub_u32 %[n], %[vlo], %[lo]\n\t"            // ... and from there to the end of the view
+                    "s_subb_u32 %[t], %[vhi], %[hi]\n\t"
+                    "s_add_u32 %[lo], %[lo], %[blo]\n\t"
+                    "s_addc_u32 %[hi], %[hi], %[bhi]\n\t"
+                    "s_cmp_lg_u32 %[t], 0\n\t"
+                    "s_cselect_b32 %[n], 0x7fffffff, %[n]\n\t"
+                    "s_min_u32 %[n], %[n], 0x7fffffff\n\t"
+                    "s_cmp_lt_u32 %[k], %[kend]\n\t"               // at or past the end of the range: nothing
+                    "s_cselect_b32 %[n], %[n], 0"
+                    : [lo] "=&s"(lo), [hi] "=&s"(hi), [n] "=&s"(bytes), [t] "=&s"(t)
+                    : [k] "s"(sc(k)), [row] "s"(sc(ldb * ES)), [vlo] "s"(sc((uint32_t)b_view)), [vhi] "s"(sc((uint32_t)(b_view >> 32))),
+                      [blo] "s"(sc((uint32_t)bu)), [bhi] "s"(sc((uint32_t)(bu >> 32))), [kend] "s"(sc(k_end))
+                    : "scc");
                 base = (const char*)(uintptr_t)(((uint64_t)hi << 32) | (uint64_t)lo);
-                bytes = (uint32_t)__builtin_amdgcn_readfirstlane(bytes);
+            } else {
+                const uint64_t skip = (uint64_t)k * ldb * ES;
+                bytes = k < k_end ? span(b_view - skip) : 0u;                  // k < k_end <= K: skip < b_view
+                base = Bg + skip;
             }
             const __amdgpu_buffer_rsrc_t rs = make_rsrc(base, bytes);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)dst, 16, b_vo[i], 0, 0, DMA_AUX);

@@ -254,12 +254,19 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
     assert mz.gemm_plan(desc(1024, 4096, 1728), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"        # 27 steps
     assert mz.gemm_plan(desc(1024, 4096, 1792), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"      # 28 steps, 128 tiles
     assert mz.gemm_plan(desc(512, 2048, 1792), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"         # 32 tiles: too few to make the loads wait
-    # K ranges of 28 steps or more run on the three-stage kernels too -- with B stored N x K; K ranges of a row-major B
-    # measure 0.85 per step there, and the 256-row split or whole tiles win
+    # K ranges of 28 steps or more run on the three-stage kernels too, whichever way B is stored (a row-major B costs
+    # them 3-7 % more per step, not the 60 % it was once priced at)
     p = mz.gemm_plan(desc(512, 4096, 14336, layout=mz.LAYOUT_NT), compute_units=CUS)       # (61 us; two stages 67.5, 256-row split 65)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3_splitk" and p["ksplit"] == 4 and p["grid"] == (256, 1, 1)
-    p = mz.gemm_plan(desc(512, 4096, 14336), compute_units=CUS)                            # (69 us; 128-row tiles in four ranges 72)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_splitk" and p["ksplit"] == 8
+    p = mz.gemm_plan(desc(512, 4096, 14336), compute_units=CUS)                            # (65 us; two stages 67.7, 256-row split 69)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and p["ksplit"] == 4 and p["grid"] == (256, 1, 1)
+    p = mz.gemm_plan(desc(384, 4096, 14336), compute_units=CUS)                            # (51 us; 256-row split 61.6)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk"
+    # a named 128-row split kernel gets the same number of ranges for either layout of B
+    for m, n, k in ((512, 4096, 14336), (1024, 4096, 14336), (512, 8192, 8192)):
+        nn_plan = mz.gemm_plan(desc(m, n, k), kernel="maize_gemm_bf16_mt256_nn_h128r3_splitk", compute_units=CUS)
+        nt_plan = mz.gemm_plan(desc(m, n, k, layout=mz.LAYOUT_NT), kernel="maize_gemm_bf16_mt256_nt_h128r3_splitk", compute_units=CUS)
+        assert nn_plan["ksplit"] == nt_plan["ksplit"] and nn_plan["grid"] == nt_plan["grid"], (m, n, k, nn_plan, nt_plan)
     p = mz.gemm_plan(desc(384, 6144, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)        # (35 us; whole 39)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3_splitk" and p["ksplit"] == 2 and p["grid"] == (144, 1, 1)
     assert mz.gemm_plan(desc(4096, 2304, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"       # 288 tiles of 128 rows would need two rounds
