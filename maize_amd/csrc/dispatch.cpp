@@ -1,5 +1,6 @@
 #include "dispatch.hpp"
 
+#include <algorithm>
 #include <atomic>
 #include <cstdint>
 #include <cstdio>
@@ -358,8 +359,17 @@ bool h128_splitk_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Lau
     const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch;
     const uint32_t kstep = fp8_in(d) ? 128u : 64u;
     uint32_t ks = h128_choice(s, d.gemm.batch, compute_units, kstep);
-    // Named explicitly for a shape the dispatcher would not split this way: two ranges if K allows, else one.
-    if (ks < 2u) ks = cdiv(s.k, kstep) >= 2u && tiles * 2ull * 131072ull <= (1ull << 30) ? 2u : 1u;
+    // Named explicitly for a shape the dispatcher would not split this way: as many ranges as fill the compute units once,
+    // none shorter than eight steps; two if K allows no more, else one.  (Not a fixed two: what a named kernel measures
+    // is fed back into the cost model, and a kernel left on half the chip measures slow whatever its loop is like.)
+    if (ks < 2u) {
+        const uint32_t nk = cdiv(s.k, kstep);
+        const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+        uint32_t want = tiles ? (uint32_t)std::min<uint64_t>(units / tiles, nk / 8u) : 1u;
+        if (want < 2u) want = nk >= 2u ? 2u : 1u;
+        while (want > 1u && (cdiv(nk, cdiv(nk, want)) != want || tiles * want * 131072ull > (1ull << 30))) --want;
+        ks = want;
+    }
     const uint64_t items = tiles * ks;
     if (items > 0x1FFFFFFFull || items * 131072ull > (1ull << 32)) return false;
     uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
