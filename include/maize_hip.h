@@ -263,6 +263,12 @@ int32_t maize_hip_gemm_ex_plan(const maize_gemm_ex_desc_t* desc, const char* ker
  * split-K kernels).  *rows == 0: one product.  The reference has no counterpart: its panel iterators assign whole
  * panels to blocks and never balance a tail (crates/maize_tile/src/gmem/row_panel.rs:95-109). */
 int32_t maize_hip_gemm_ex_tail_rows(const maize_gemm_ex_desc_t* desc, uint32_t compute_units, uint32_t* rows);
+/* The same, by rows or by columns: (*rows, 0): as above; (0, *cols): the leading *cols columns of B and C first, the columns
+ * to their right behind them on the same stream, both as products that keep the whole matrices' leading dimensions (the
+ * part set aside runs in 128-row tiles where those fit one round -- bit-identical to the single-kernel result -- or split
+ * over K); (0, 0): one product.  2048 x 11008 x 4096: 344 tiles = 256 + 88, 155.7 -> 138.9 us.  maize_hip_gemm_ex_tail_rows
+ * reports 0 for a product cut by columns.  No counterpart in the reference (see above). */
+int32_t maize_hip_gemm_ex_tail_split(const maize_gemm_ex_desc_t* desc, uint32_t compute_units, uint32_t* rows, uint32_t* cols);
 /* Validation only (no device access): the checks gemm_bf16 performs first. */
 int32_t maize_hip_gemm_validate(const maize_gemm_desc_t* desc);
 /* Enumerates the GEMM kernels of the embedded code object. */

@@ -17,7 +17,7 @@ EXPORTS = (
     "maize_hip_launch", "maize_hip_embedded_code_object", "maize_hip_gemm_bf16", "maize_hip_gemm_bf16_with",
     "maize_hip_gemm_bf16_noalloc", "maize_hip_noalloc_reset", "maize_hip_set_split_wait_us", "maize_hip_get_split_wait_us",
     "maize_hip_gemm_select", "maize_hip_gemm_plan", "maize_hip_gemm_validate",
-    "maize_hip_gemm_bf16_ex", "maize_hip_gemm_ex_validate", "maize_hip_gemm_ex_plan", "maize_hip_gemm_ex_tail_rows", "maize_hip_kernel_count", "maize_hip_kernel_name",
+    "maize_hip_gemm_bf16_ex", "maize_hip_gemm_ex_validate", "maize_hip_gemm_ex_plan", "maize_hip_gemm_ex_tail_rows", "maize_hip_gemm_ex_tail_split", "maize_hip_kernel_count", "maize_hip_kernel_name",
     "maize_hip_kernel_supports", "maize_hip_malloc", "maize_hip_free", "maize_hip_memcpy_h2d",
     "maize_hip_memcpy_d2h", "maize_hip_memset", "maize_hip_stream_create", "maize_hip_stream_destroy",
     "maize_hip_sync", "maize_hip_event_create", "maize_hip_event_record", "maize_hip_event_synchronize",
@@ -137,6 +137,7 @@ def lib():
         "maize_hip_gemm_ex_validate": (i32, [P(GemmExDescT)]),
         "maize_hip_gemm_ex_plan": (i32, [P(GemmExDescT), C.c_char_p, u32, P(GemmPlanT)]),
         "maize_hip_gemm_ex_tail_rows": (i32, [P(GemmExDescT), u32, P(u32)]),
+        "maize_hip_gemm_ex_tail_split": (i32, [P(GemmExDescT), u32, P(u32), P(u32)]),
         "maize_hip_kernel_count": (u32, []),
         "maize_hip_kernel_name": (C.c_char_p, [u32]),
         "maize_hip_kernel_supports": (i32, [C.c_char_p, P(GemmDescT)]),

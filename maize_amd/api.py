@@ -242,6 +242,16 @@ def gemm_tail_rows(desc, compute_units=256):
     return rows.value
 
 
+def gemm_tail_split(desc, compute_units=256):
+    """(rows, cols): how the launcher cuts a product whose tile count is a little over a whole number of rounds -- the
+    leading rows first, or the leading columns first, the rest behind them as a product of its own; (0, 0) = one product."""
+    x = desc if isinstance(desc, _ffi.GemmExDescT) else gemm_ex_desc(desc.a, desc.b, desc.c, layout=desc.layout, batch=desc.batch,
+                                                                      stride_a=desc.stride_a, stride_b=desc.stride_b, stride_c=desc.stride_c)
+    rows, cols = C.c_uint32(), C.c_uint32()
+    check(_ffi.lib().maize_hip_gemm_ex_tail_split(C.byref(x), compute_units, C.byref(rows), C.byref(cols)))
+    return rows.value, cols.value
+
+
 def set_split_wait_us(us):
     """Process-wide bound (microseconds, at most 1000) of the wait inside the few-row kernels that share their
     split-K additions (maize_hip_set_split_wait_us); returns the bound that was in force."""

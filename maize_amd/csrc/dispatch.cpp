@@ -1134,32 +1134,70 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     return (uint32_t)kernel_index("maize_gemm_bf16_wave32");
 }
 
-uint32_t tail_split_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
-    if (!(bf16_in(d) || half_in(d)) || d.gemm.batch != 1 || compute_units < 8u) return 0;
+namespace {
+// What the part of a product that does not fill whole rounds costs as a launch of its own, in the units of the cost
+// models above (~ microseconds), or a negative value if it would run in whole 256-row tiles anyway (nothing gained).
+double tail_part_cost(const maize_gemm_ex_desc_t& part, uint32_t compute_units) {
+    const Dims s = dims_of(part);
+    const char* name = kKernels[select_kernel(part, compute_units)].name;
+    const uint32_t nk = cdiv(s.k, 64);
+    const bool h128 = std::strstr(name, "_h128") != nullptr, three = std::strstr(name, "_h128r3") != nullptr;
+    const double launch = 3.0 + 8.0;
+    if (std::strstr(name, "_splitk")) {
+        const uint32_t ks = h128 ? h128_choice(s, 1, compute_units) : splitk_ranges(s, 1, compute_units);
+        if (ks < 2u) return -1.0;
+        const uint32_t r = cdiv(nk, ks);
+        const double step = h128 ? h128_step(three, true, s.nt, false) * (three ? 3u * cdiv(r, 3u) : r) : 1.0 * r;
+        return launch + step + 6.0 + (1.2e-6 * (double)s.m * s.n + 0.15) * ks;
+    }
+    if (h128 && std::strstr(name, "_mt256_")) return launch + h128_step(three, false, s.nt, false) * (three ? 3u * cdiv(nk, 3u) : nk);
+    return -1.0;
+}
+}  // namespace
+
+TailSplit tail_split(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
+    TailSplit none = {0, 0};
+    if (!(bf16_in(d) || half_in(d)) || d.gemm.batch != 1 || compute_units < 8u) return none;
     const Dims s = dims_of(d);
     // only where the whole product would run on a persistent macro-tile kernel, one tile per work item
     const char* name = kKernels[select_kernel(d, compute_units)].name;
-    if (!std::strstr(name, "_mt256_") || std::strstr(name, "_splitk") || std::strstr(name, "_packed") || std::strstr(name, "_edge")) return 0;
+    if (!std::strstr(name, "_mt256_") || std::strstr(name, "_splitk") || std::strstr(name, "_packed") || std::strstr(name, "_edge") ||
+        std::strstr(name, "_h128"))
+        return none;
     const uint32_t tm = cdiv(s.m, 256), tn = cdiv(s.n, 256);
     const uint64_t tiles = (uint64_t)tm * tn;
     const uint32_t resident = compute_units - compute_units % 8u;
-    if (tiles <= resident || tiles % resident == 0) return 0;
-    const uint64_t full_rounds = tiles / resident;
-    const uint32_t tm_top = (uint32_t)(full_rounds * resident / tn);     // tile rows that fit into the full rounds
-    if (tm_top == 0 || tm_top >= tm) return 0;
-    // The rows below: worth a launch of their own only if, split over K, they cost clearly less than the
-    // round they replace (the cost model of splitk_ranges, microseconds, plus ~3 for the extra launch).
-    Dims bottom = s;
-    bottom.m = s.m - tm_top * 256u;
+    if (tiles <= resident || tiles % resident == 0) return none;
+    const uint64_t full = tiles / resident * resident;                   // tiles of the whole rounds
     const uint32_t nk = cdiv(s.k, 64);
-    const uint32_t ks = splitk_ranges(bottom, 1, compute_units);
-    if (ks < 2u) return 0;
     const double t_round = 8.0 + 1.0 * nk;
-    const double t_bottom = 3.0 + 8.0 + 1.0 * cdiv(nk, ks) + 6.0 + (1.2e-6 * (double)bottom.m * s.n + 0.15) * ks;
-    if (t_bottom > 0.75 * t_round) return 0;
-    // the rows below start on a 16-byte boundary like the matrix itself (leading dimensions are multiples of 8)
-    return tm_top * 256u;
+    // The part set aside is worth a launch of its own only if it costs clearly less than the round it replaces: as
+    // 128-row tiles that fit one round, or split over K.  By rows (the rows below the leading tile rows that fill the
+    // rounds) or by columns (the columns to the right of the leading tile columns), whichever part is cheaper.
+    const Lds l = lds_of(d);
+    double best = 0.75 * t_round;
+    TailSplit pick = none;
+    const uint32_t tm_top = (uint32_t)(full / tn), tn_left = (uint32_t)(full / tm);
+    if (tm_top > 0 && tm_top < tm) {
+        maize_gemm_ex_desc_t part = d;                                   // (pointers keep their alignment: whole tile rows)
+        part.gemm.a.nrows = part.gemm.c.nrows = s.m - tm_top * 256u;
+        part.lda = l.a; part.ldb = l.b; part.ldc = l.c;
+        const double c = tail_part_cost(part, compute_units);
+        if (c >= 0.0 && c < best) { best = c; pick = TailSplit{tm_top * 256u, 0}; }
+    }
+    if (tn_left > 0 && tn_left < tn) {
+        maize_gemm_ex_desc_t part = d;                                   // (512-byte steps along a row: alignment kept too)
+        const uint32_t n_part = s.n - tn_left * 256u;
+        if (s.nt) part.gemm.b.nrows = n_part; else part.gemm.b.ncols = n_part;
+        part.gemm.c.ncols = n_part;
+        part.lda = l.a; part.ldb = l.b; part.ldc = l.c;
+        const double c = tail_part_cost(part, compute_units);
+        if (c >= 0.0 && c < best) { best = c; pick = TailSplit{0, tn_left * 256u}; }
+    }
+    return pick;
 }
+
+uint32_t tail_split_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units) { return tail_split(d, compute_units).rows; }
 
 // The wait bound of the few-row kernels that share their split-K additions (see share_additions).
 std::atomic<uint32_t> g_split_wait_us{0xFFFFFFFFu};        // not read from the environment yet

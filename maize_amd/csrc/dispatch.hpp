@@ -67,6 +67,11 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units);
 // the dispatcher picks for them; the rows below are then a product with few tiles, which the dispatcher runs on
 // the split-K kernels.  Host logic only; the launcher composes the two products on the caller's stream.
 uint32_t tail_split_rows(const maize_gemm_ex_desc_t& d, uint32_t compute_units);
+// The same by rows or by columns: {rows, 0}: the leading `rows` rows first, the rows below behind them; {0, cols}: the
+// leading `cols` columns of B and C first, the columns to their right behind them (as a product with leading dimensions);
+// {0, 0}: one product.  The part set aside runs in 128-row tiles or split over K, whichever the dispatcher picks for it.
+struct TailSplit { uint32_t rows, cols; };
+TailSplit tail_split(const maize_gemm_ex_desc_t& d, uint32_t compute_units);
 
 struct Dims {
     uint32_t m, n, k;

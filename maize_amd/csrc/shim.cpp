@@ -355,6 +355,16 @@ int32_t maize_hip_gemm_ex_tail_rows(const maize_gemm_ex_desc_t* desc, uint32_t c
     return MAIZE_OK;
 }
 
+int32_t maize_hip_gemm_ex_tail_split(const maize_gemm_ex_desc_t* desc, uint32_t compute_units, uint32_t* rows, uint32_t* cols) {
+    if (!rows || !cols) return fail(MAIZE_ERR_NULL, "gemm_tail_split: NULL argument");
+    int32_t rc = maize_hip_gemm_ex_validate(desc);
+    if (rc != MAIZE_OK) return rc;
+    const maize::TailSplit cut = maize::tail_split(*desc, compute_units);
+    *rows = cut.rows;
+    *cols = cut.cols;
+    return MAIZE_OK;
+}
+
 const char* maize_hip_kernel_name(uint32_t index) {
     return index < maize::kernel_count() ? maize::kernel_at(index).name : nullptr;
 }
@@ -549,17 +559,31 @@ static int32_t gemm_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const
     if (rc != MAIZE_OK) return rc;
     if (!kernel) {
         const uint32_t cus = (uint32_t)ctx->prop.multiProcessorCount;
-        // A tile count a little over a whole number of rounds: the leading rows fill the rounds, the rest is a
-        // product with few tiles that runs split over K, behind it on the same stream.
-        const uint32_t top_rows = maize::tail_split_rows(*desc, cus);
-        if (top_rows) {
-            const uint64_t lda = desc->lda ? desc->lda : desc->gemm.a.ncols, ldc = desc->ldc ? desc->ldc : desc->gemm.c.ncols;
+        // A tile count a little over a whole number of rounds: the leading tile rows (or tile columns) fill the rounds,
+        // the rest is a product with few tiles that runs in 128-row tiles or split over K, behind it on the same stream.
+        const maize::TailSplit cut = maize::tail_split(*desc, cus);
+        if (cut.rows || cut.cols) {
+            const bool nt = desc->gemm.layout == MAIZE_LAYOUT_NT;
+            const uint64_t lda = desc->lda ? desc->lda : desc->gemm.a.ncols, ldb = desc->ldb ? desc->ldb : desc->gemm.b.ncols,
+                           ldc = desc->ldc ? desc->ldc : desc->gemm.c.ncols;
             const uint64_t csz = desc->out_type == MAIZE_OUT_F32 ? 4u : 2u;
             maize_gemm_ex_desc_t top = *desc, rest = *desc;
-            top.gemm.a.nrows = top.gemm.c.nrows = top_rows;
-            rest.gemm.a.nrows = rest.gemm.c.nrows = desc->gemm.a.nrows - top_rows;
-            rest.gemm.a.ptr = (char*)desc->gemm.a.ptr + (uint64_t)top_rows * lda * 2u;
-            rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)top_rows * ldc * csz;
+            if (cut.rows) {
+                top.gemm.a.nrows = top.gemm.c.nrows = cut.rows;
+                rest.gemm.a.nrows = rest.gemm.c.nrows = desc->gemm.a.nrows - cut.rows;
+                rest.gemm.a.ptr = (char*)desc->gemm.a.ptr + (uint64_t)cut.rows * lda * 2u;
+                rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)cut.rows * ldc * csz;
+            } else {
+                // by columns: both parts keep the leading dimensions of the whole matrices
+                const uint32_t n = desc->gemm.c.ncols;
+                top.lda = rest.lda = (uint32_t)lda; top.ldb = rest.ldb = (uint32_t)ldb; top.ldc = rest.ldc = (uint32_t)ldc;
+                top.gemm.c.ncols = cut.cols;
+                rest.gemm.c.ncols = n - cut.cols;
+                if (nt) { top.gemm.b.nrows = cut.cols; rest.gemm.b.nrows = n - cut.cols; }
+                else    { top.gemm.b.ncols = cut.cols; rest.gemm.b.ncols = n - cut.cols; }
+                rest.gemm.b.ptr = (char*)desc->gemm.b.ptr + (nt ? (uint64_t)cut.cols * ldb * 2u : (uint64_t)cut.cols * 2u);
+                rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)cut.cols * csz;
+            }
             uint32_t itop, irest;
             if ((rc = select_checked(top, cus, &itop)) != MAIZE_OK || (rc = select_checked(rest, cus, &irest)) != MAIZE_OK) return rc;
             // Fixed scratch: both products must fit before the first one is launched (a refusal launches nothing).

@@ -151,6 +151,7 @@ extern "C" {
     pub fn maize_hip_gemm_plan(desc: *const MaizeGemmDesc, kernel: *const c_char, compute_units: u32, out: *mut MaizeGemmPlan) -> i32;
     pub fn maize_hip_gemm_ex_plan(desc: *const MaizeGemmExDesc, kernel: *const c_char, compute_units: u32, out: *mut MaizeGemmPlan) -> i32;
     pub fn maize_hip_gemm_ex_tail_rows(desc: *const MaizeGemmExDesc, compute_units: u32, rows: *mut u32) -> i32;
+    pub fn maize_hip_gemm_ex_tail_split(desc: *const MaizeGemmExDesc, compute_units: u32, rows: *mut u32, cols: *mut u32) -> i32;
     pub fn maize_hip_kernel_count() -> u32;
     pub fn maize_hip_kernel_name(index: u32) -> *const c_char;
     pub fn maize_hip_kernel_supports(kernel: *const c_char, desc: *const MaizeGemmDesc) -> i32;

@@ -282,25 +282,34 @@ def test_tail_split_by_rows():
     """A tile count a little over a whole number of rounds of one workgroup per compute unit: the leading tile rows
     that fill the rounds are one product, the rest a second one that the dispatcher runs split over K."""
     # 16 x 17 = 272 tiles on 256 compute units: 15 tile rows (255 tiles) on top, one tile row of 17 tiles below
-    x = ex(4096, 4352, 4096)
-    assert mz.gemm_tail_rows(x) == 15 * 256
-    top, rest = ex(15 * 256, 4352, 4096), ex(256, 4352, 4096)
-    assert mz.gemm_plan(top)["kernel"] == "maize_gemm_bf16_mt256_nn" and mz.gemm_plan(top)["grid"] == (255, 1, 1)
+    x = ex(4352, 4096, 4096)
+    assert mz.gemm_tail_rows(x) == 16 * 256 and mz.gemm_tail_split(x) == (16 * 256, 0)
+    top, rest = ex(16 * 256, 4096, 4096), ex(256, 4096, 4096)
+    assert mz.gemm_plan(top)["kernel"] == "maize_gemm_bf16_mt256_nn" and mz.gemm_plan(top)["grid"] == (256, 1, 1)
     assert mz.gemm_plan(rest)["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and mz.gemm_plan(rest)["ksplit"] >= 2
-    assert mz.gemm_tail_rows(ex(4096, 4352, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_F16, beta=1.0)) == 15 * 256
+    assert mz.gemm_tail_rows(ex(4352, 4096, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_F16, beta=1.0)) == 16 * 256
+    # ... or by columns, where that leaves the cheaper part: 16 x 17 tiles = a full round of 16 tile columns and one more
+    assert mz.gemm_tail_split(ex(4096, 4352, 4096)) == (0, 16 * 256) and mz.gemm_tail_rows(ex(4096, 4352, 4096)) == 0
+    # 8 x 43 tiles: 32 tile columns are a round, the 11 to their right run in 128-row tiles (176 of them: one round)
+    assert mz.gemm_tail_split(ex(2048, 11008, 4096)) == (0, 8192)
+    right = ex(2048, 2816, 4096, ldb=11008, ldc=11008)
+    assert mz.gemm_plan(right)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3" and mz.gemm_plan(right)["grid"] == (176, 1, 1)
+    assert mz.gemm_tail_split(ex(2048, 11008, 4096, layout=mz.LAYOUT_NT)) == (0, 8192)
+    assert mz.gemm_tail_split(ex(4096, 6144, 4096)) == (0, 4096)           # 384 tiles: the 128 of the second round as 256 half tiles
+    assert mz.gemm_tail_split(ex(6144, 4096, 4096)) == (4096, 0)
+    assert mz.gemm_tail_split(ex(2048, 14336, 4096)) == (0, 0)             # 448 tiles: the 192 of the second round need a round either way
     # whole rounds, a single round, a round that is nearly full, or an edge the edge kernels take: one product
     assert mz.gemm_tail_rows(ex(8192, 8192, 8192)) == 0          # 1024 tiles = 4 rounds
     assert mz.gemm_tail_rows(ex(4096, 4096, 4096)) == 0          # 256 tiles
     assert mz.gemm_tail_rows(ex(2048, 2048, 2048)) == 0          # 64 tiles
     assert mz.gemm_tail_rows(ex(4000, 4104, 4032)) == 0          # narrow last tile column: edge splitting instead
-    assert mz.gemm_tail_rows(ex(4096, 6144, 4096)) == 0          # 384 tiles: the second round is half full, nothing to gain
     # a short K: the round that would be saved is cheap, the extra launches are not
-    assert mz.gemm_tail_rows(ex(4096, 4352, 256)) == 0
+    assert mz.gemm_tail_split(ex(4096, 4352, 256)) == (0, 0) and mz.gemm_tail_split(ex(2048, 11008, 1024)) == (0, 0)
     # batches, 8-bit and wide operands are left alone; fewer compute units move the boundary
-    assert mz.gemm_tail_rows(ex(4096, 4352, 4096, batch=2, stride_a=4096 * 4096, stride_b=4096 * 4352, stride_c=4096 * 4352)) == 0
-    assert mz.gemm_tail_rows(ex(4096, 4352, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3)) == 0
-    assert mz.gemm_tail_rows(ex(4096, 4352, 4096, in_type=mz.IN_F32)) == 0
-    assert mz.gemm_tail_rows(x, compute_units=64) == 3840        # 272 = 4 x 64 + 16: 15 tile rows = 255 tiles fit 4 rounds of 64
+    assert mz.gemm_tail_split(ex(4096, 4352, 4096, batch=2, stride_a=4096 * 4096, stride_b=4096 * 4352, stride_c=4096 * 4352)) == (0, 0)
+    assert mz.gemm_tail_split(ex(4096, 4352, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3)) == (0, 0)
+    assert mz.gemm_tail_split(ex(4096, 4352, 4096, in_type=mz.IN_F32)) == (0, 0)
+    assert mz.gemm_tail_rows(x, compute_units=64) == 4096        # 272 = 4 x 64 + 16: 16 tile rows = 256 tiles are 4 rounds of 64
 
 
 def test_half_c_goes_with_half_and_8bit_operands_only():

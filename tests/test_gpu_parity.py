@@ -431,16 +431,41 @@ def test_operands_past_two_gib(ctx, oracle, which):
 
 
 @pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
+@pytest.mark.parametrize("shape", [(2048, 11008, 4096), (2000, 11000, 4096), (4096, 4352, 4096)], ids=lambda s: "x".join(map(str, s)))
+def test_tail_split_by_columns(ctx, oracle, layout, shape):
+    """344 tiles on 256 compute units (8 x 43): the launcher computes the 32 leading tile columns as one product and the 11 to
+    their right as a second one on the same stream, in 128-row tiles -- the whole of C is then the single-kernel result
+    bit for bit (the 128-row kernels sum in the same order).  16 x 17 tiles: the one tile column set aside runs split
+    over K, another summation order, checked against the oracle.  Sampled rows, every column."""
+    m, n, k = shape
+    x = mz.gemm_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x10000000, k, n) if layout == mz.LAYOUT_NN else mz.GlobalMatrix(0x10000000, n, k),
+                     mz.GlobalMatrix(0x20000000, m, n), layout=layout)
+    rows_cut, left = mz.gemm_tail_split(x, compute_units=ctx.info()["compute_units"])
+    _say(f"tail split by columns: {shape} layout={layout} cut ({rows_cut}, {left})")
+    assert rows_cut == 0 and left == (8192 if n > 8192 else 4096)
+    a, b = inputs(m, n, k)
+    bs = b if layout == mz.LAYOUT_NN else b.reshape(k, n).T.copy().ravel()
+    got = run_gemm(ctx, a, bs, m, n, k, layout=layout)
+    rows = np.unique(np.concatenate([sample_rows(m, count=16, seed=6), [0, m - 1]])).astype(np.uint32)
+    check_rows_against_oracle(oracle, got, a, bs, m, n, k, rows, layout=layout, label=f"tail split by columns {shape}")
+    one = run_gemm(ctx, a, bs, m, n, k, layout=layout, kernel="maize_gemm_bf16_mt256_nn" if layout == mz.LAYOUT_NN else "maize_gemm_bf16_mt256_nt")
+    got2, one2 = got.reshape(m, n), one.reshape(m, n)
+    assert np.array_equal(got2[:, :left], one2[:, :left])           # the leading columns: the same kernel on the same tiles
+    if n > 8192:
+        assert np.array_equal(got2[:, left:], one2[:, left:])       # 128-row tiles: the same sums in the same order
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT])
 def test_tail_split_by_rows(ctx, oracle, layout):
-    """272 tiles on 256 compute units: the launcher computes the 15 leading tile rows as one product and the last tile row,
-    split over K, as a second one on the same stream.  Checked on sampled rows on both sides of the seam, and against
-    the single-kernel result, which the leading rows must equal bit for bit."""
-    m, n, k = 4096, 4352, 4096
+    """272 tiles on 256 compute units (17 x 16): the launcher computes the 16 leading tile rows as one product and the last
+    tile row, split over K, as a second one on the same stream.  Checked on sampled rows on both sides of the seam, and
+    against the single-kernel result, which the leading rows must equal bit for bit."""
+    m, n, k = 4352, 4096, 4096
     x = mz.gemm_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x10000000, k, n) if layout == mz.LAYOUT_NN else mz.GlobalMatrix(0x10000000, n, k),
                      mz.GlobalMatrix(0x20000000, m, n), layout=layout)
     top = mz.gemm_tail_rows(x, compute_units=ctx.info()["compute_units"])
     _say(f"tail split by rows: layout={layout} top rows {top}")
-    assert top == 15 * 256
+    assert top == 16 * 256
     a, b = inputs(m, n, k)
     bs = b if layout == mz.LAYOUT_NN else b.reshape(k, n).T.copy().ravel()
     got = run_gemm(ctx, a, bs, m, n, k, layout=layout)
