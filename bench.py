@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 # profiling session, not of this run: each entry names the kernel it was measured on and is reported only when this
 # run's kernel is that one, together with its source file.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_fetch_write_size.md"
-MEASURED_TRAFFIC = {"cfg1": ("maize_gemm_bf16_mt256_nn", 235.2e6), "cfg2": ("maize_gemm_bf16_mt256_nn_edge", 275.1e6),
+MEASURED_TRAFFIC = {"cfg1": ("maize_gemm_bf16_mt256_nn", 235.2e6), "cfg2": ("maize_gemm_bf16_mt256_nn_ragged", 239.4e6),
                     "cfg3": ("maize_gemm_bf16_mt256_nt", 1746.3e6), "cfg4": ("maize_gemm_bf16_skinny_nn", 126.5e6),
                     "m64": ("maize_gemm_bf16_skinny_nn_m64", 153.1e6),
                     "cfg5": ("maize_gemm_bf16_mt256_nn", 1074.3e6), "sq2048": ("maize_gemm_bf16_mt256_nn_h128r3", 58.9e6), "mid": ("maize_gemm_bf16_mt256_nt_h128r3", 109.2e6), "f8": ("maize_gemm_e4m3_mt256_nt", 134.5e6),

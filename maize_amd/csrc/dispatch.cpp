@@ -93,6 +93,18 @@ bool k64(const maize_gemm_ex_desc_t& d) { return (d.gemm.a.ncols & 63u) == 0; }
 bool nn(const maize_gemm_ex_desc_t& d) { return d.gemm.layout == MAIZE_LAYOUT_NN; }
 bool mt256_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && bf16_in(d); }
 bool mt256_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && k64(d) && plain_epilogue(d) && bf16_in(d); }
+// Ragged last columns that ride along in the K loop: N = 256 t + 8 or 16 with t >= 16 whole tile columns (the sixteen
+// 16-row blocks of a row panel go one each to the workgroups of its first sixteen tiles).  An N x K B is addressed from
+// its tile's first row with 32-bit offsets: the matrix stays under 2 GiB.
+bool ntail_shape(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const uint32_t w = s.n % 256u;
+    if (!(w == 8u || w == 16u) || s.n / 256u < 16u) return false;
+    if (s.nt && (uint64_t)s.n * lds_of(d).b * 2u >= 0x7FFFFFFFull) return false;
+    return true;
+}
+bool mt256_nn_ragged_supports(const maize_gemm_ex_desc_t& d) { return mt256_nn_supports(d) && ntail_shape(d); }
+bool mt256_nt_ragged_supports(const maize_gemm_ex_desc_t& d) { return mt256_nt_supports(d) && ntail_shape(d); }
 bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && plain_epilogue(d) && bf16_in(d); }
 bool mt256_nt_ktail_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_common(d) && plain_epilogue(d) && bf16_in(d); }
 bool mt256_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && c_rows16(d) && k64(d) && bf16_in(d); }
@@ -225,6 +237,18 @@ bool mt256_h128_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Laun
     return true;
 }
 bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
+// ... over the whole tile columns only (the ragged last columns have no tiles of their own)
+bool mt256_ntail_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const uint64_t all = (uint64_t)cdiv(s.m, 256) * (s.n / 256u) * d.gemm.batch;
+    if (all == 0 || all > 0x1FFFFFFFull) return false;
+    const uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+    ld->grid[0] = (resident && all > resident) ? resident : (uint32_t)all;
+    ld->grid[1] = 1; ld->grid[2] = 1;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0; ld->ksplit = 1; ld->split_first = 0; ld->reduce_grid = 0; ld->workspace_bytes = 0;
+    return true;
+}
 
 // ---- maize_gemm_{bf16,f16}_mt256_{nn,nt}_splitk: few tiles, long K ---------------------------
 // K ranges per tile.  Candidates: up to one (tile, range) work item per compute unit, at least 4 K
@@ -843,6 +867,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt", nullptr, mt256_nt_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_asm", nullptr, mt256_nn_supports, mt256_plan},      // the K loop as one assembly statement
     {"maize_gemm_bf16_mt256_nt_asm", nullptr, mt256_nt_supports, mt256_plan},
+    {"maize_gemm_bf16_mt256_nn_ragged", nullptr, mt256_nn_ragged_supports, mt256_ntail_plan},  // ... with ragged last columns riding along
+    {"maize_gemm_bf16_mt256_nt_ragged", nullptr, mt256_nt_ragged_supports, mt256_ntail_plan},
     {"maize_gemm_bf16_mt256_nn_h128", nullptr, mt256_nn_supports, mt256_h128_plan},
     {"maize_gemm_bf16_mt256_nt_h128", nullptr, mt256_nt_supports, mt256_h128_plan},
     {"maize_gemm_bf16_mt256_nn_h128_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_h128_plan},
@@ -1101,6 +1127,18 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     int ti = half_in(d)                    ? kernel_index(kHalf[(s.k & 63u) != 0][s.nt])
              : plain_epilogue(d) && strict ? kernel_index(kTiled[edge][(s.k & 63u) != 0][s.nt])
                                            : kernel_index(kGeneral[(s.k & 63u) != 0][s.nt]);
+    // Eight or sixteen ragged last columns behind sixteen or more whole tile columns, where a tile column of their own
+    // would cost a round of workgroups: they ride along in the whole tiles' K loop (two more matrix instructions per
+    // step) instead of being cut over K as edge items (4000 x 4104 x 4032: see the kernel).
+    if (!half_in(d) && plain_epilogue(d) && strict && (s.k & 63u) == 0) {
+        static const char* const kRagged[2] = {"maize_gemm_bf16_mt256_nn_ragged", "maize_gemm_bf16_mt256_nt_ragged"};
+        const int ri = kernel_index(kRagged[s.nt]);
+        const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+        if (ri >= 0 && units && kKernels[ri].supports(d)) {
+            const uint64_t tm = cdiv(s.m, 256), with = tm * cdiv(s.n, 256) * d.gemm.batch, without = tm * (s.n / 256u) * d.gemm.batch;
+            if ((with + units - 1) / units > (without + units - 1) / units) return (uint32_t)ri;
+        }
+    }
     // An odd number of K steps: the plain kernel's statement loop runs two steps per trip and pads with a step on a
     // zero tile; the same loop as one assembly statement leaves the trip after its first step (4096 x 4096 x K, K = 192:
     // 14.1 -> 12.8 us, 576: 21.8 -> 20.2, 1088: 30.6 -> 29.4, 3008: 67.6 -> 66.5; at even counts it is level or up to 1 % behind).
@@ -1162,7 +1200,7 @@ TailSplit tail_split(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // only where the whole product would run on a persistent macro-tile kernel, one tile per work item
     const char* name = kKernels[select_kernel(d, compute_units)].name;
     if (!std::strstr(name, "_mt256_") || std::strstr(name, "_splitk") || std::strstr(name, "_packed") || std::strstr(name, "_edge") ||
-        std::strstr(name, "_h128"))
+        std::strstr(name, "_h128") || std::strstr(name, "_ragged"))
         return none;
     const uint32_t tm = cdiv(s.m, 256), tn = cdiv(s.n, 256);
     const uint64_t tiles = (uint64_t)tm * tn;

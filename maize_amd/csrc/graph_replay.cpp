@@ -32,11 +32,11 @@ int main(int argc, char** argv) {
     maize_ctx_t* ctx = nullptr;
     MZ_OK(maize_hip_ctx_create(0, &ctx));
     // a few-row product in K ranges, the same against N x K weights, 64 rows in four row groups (the slab's workgroups
-    // share the additions), 128-row tiles cut over K with the reduce pass behind them, a ragged product whose edge tiles
+    // share the additions), 128-row tiles cut over K with the reduce pass behind them, a ragged product (24 columns past the last whole tile column) whose edge tiles
     // are split, and a plain one that needs no scratch
     std::vector<Product> ps = {{16, 14336, 4096, MAIZE_LAYOUT_NN, nullptr, nullptr, nullptr, {}, ""}, {16, 4096, 4096, MAIZE_LAYOUT_NT, nullptr, nullptr, nullptr, {}, ""},
                                {64, 14336, 4096, MAIZE_LAYOUT_NN, nullptr, nullptr, nullptr, {}, ""}, {100, 2048, 4096, MAIZE_LAYOUT_NN, nullptr, nullptr, nullptr, {}, ""},
-                               {4000, 4104, 512, MAIZE_LAYOUT_NN, nullptr, nullptr, nullptr, {}, ""}, {512, 512, 512, MAIZE_LAYOUT_NN, nullptr, nullptr, nullptr, {}, ""}};
+                               {4000, 4120, 512, MAIZE_LAYOUT_NN, nullptr, nullptr, nullptr, {}, ""}, {512, 512, 512, MAIZE_LAYOUT_NN, nullptr, nullptr, nullptr, {}, ""}};
     int with_scratch = 0;
     for (Product& p : ps) {
         MZ_OK(maize_hip_malloc(ctx, (size_t)p.m * p.k * 2, (void**)&p.a));

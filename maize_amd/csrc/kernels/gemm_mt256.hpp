@@ -150,10 +150,11 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 // t+3 go out one every two slots from the barrier of step t on (seven behind it, five in front of the next), same wait.
 // ASM: the K loop is the generated assembly statement (kloop_gen.inc) instead of the step() statements below: the same
 // schedule with registers assigned by hand, for the plain 256-row bf16 kernels.
-template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2, bool ASM = false>
+template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2, bool ASM = false, bool NTAIL = false>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
     static_assert(!ASM || (!KTAIL && !EDGE && !GEN && !F16 && !SPLITK && F8 < 0 && BMT == 256 && NST == 2), "the assembly K loop: plain 256-row bf16 kernels");
+    static_assert(!NTAIL || ASM, "the ragged last columns ride along in the assembly K loop only");
     constexpr bool H128 = BMT == 128;
     static_assert(BMT == 256 || (H128 && !EDGE), "128-row tiles: no edge splitting");
     constexpr bool R3 = NST == 3;                       // three ring stages (128-row tiles)
@@ -197,7 +198,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t wave = tid >> 6;
     const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t wm = wave >> 1, wn = wave & 1u;
-    const uint32_t tm = (M + BMT - 1) / BMT, tn = (N + BN - 1) / BN;
+    // NTAIL: N = 256 tn + 8 or 16; the columns past the last whole tile column have no tiles of their own (below)
+    const uint32_t tm = (M + BMT - 1) / BMT, tn = NTAIL ? N / BN : (N + BN - 1) / BN;
     // Workgroups 0 .. whole-1 compute one tile each over all of K.  With edge splitting
     // (p.reserved = mode << 30 | whole + 1; mode 1: last tile column, mode 2: last tile row) the
     // whole tiles are the grid without that edge, and the rest of the workgroups share the edge
@@ -264,6 +266,11 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool PATCHES = !NT && !IS8 && GEN;        // (the kernels that store C themselves from bf16 staging take even N only)
     bool patch_on = false;                // this work item holds column N - 1 (last tile column, N odd)
     uint32_t patch_off = 0, patch_val = 0;
+    // NTAIL: the 16-row block of its row panel that this tile's workgroup also multiplies against the ragged last columns
+    // (block tile_n % 16; only the first sixteen tile columns' results are stored), and the lane's byte offsets of the
+    // two 4-byte-per-lane requests per K tile with which its wave brings in a quarter of those columns' B tile.
+    uint32_t tail_x = 0u, t_vo[2] = {0u, 0u};
+    bool tail_live = false;
     auto select_tile = [&](uint32_t id) {
         uint32_t tile_m, tile_n;
         uint64_t bz;
@@ -304,6 +311,19 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             b_bytes = 0u;
         }
         Cg = p.c + bz * p.stride_c * ((GEN && (p.epi & EPI_F32)) ? 2u : 1u);   // strides count elements of C
+        if constexpr (NTAIL) {
+            tail_x = tile_n & 15u;
+            tail_live = tile_n < 16u;
+            uint32_t lt = lane;
+            asm volatile("" : "+v"(lt));                                       // (derived per tile, not kept across the K loop)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (NT)    // rows tn * 256 + r of the N x K B as 16 rows of a K-contiguous tile: 256 bytes = 2 rows per request
+                    t_vo[j] = (tn * BN - n0 + maps::rc_nk_row(wave * 2u + j, lt)) * ldb * ES + maps::rc_nk_byte(wave * 2u + j, lt);
+                else       // columns tn * 256 .. + 15 of rows k .. k + 63 of the K x N B, 32 bytes per row: 256 bytes = 8 rows per request
+                    t_vo[j] = (maps::rc_kn_row(wave * 2u + j, lt) * ldb + tn * BN) * ES + maps::rc_kn_byte(lt);
+            }
+        }
         if (PATCHES) {
             const uint32_t pcol = N - 1u - n0;                                 // < 256 when this tile holds column N - 1
             patch_on = (N & 1u) && n0 + BN >= N && (pcol >> 7) == wn;          // ... and this wave multiplies it
@@ -632,9 +652,27 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         k_early += BKE;
         k_late += BKE;
     };
+    // The ragged columns' B tile of the K tile at k into its stage 0 (the stages, 2 KiB each, lie at the start of the
+    // epilogue's staging region, which is idle from the top of a C tile's K loop to its end).
+    auto dma_tail = [&](uint32_t k) {
+        typedef __attribute__((address_space(3))) void* lvp;
+        const char* base = Bg;
+        uint32_t bytes = k < k_end ? b_bytes : 0u, soff = k * ES;
+        if (!NT) {
+            const uint64_t skip = (uint64_t)k * ldb * ES;
+            bytes = k < k_end ? span(b_view - skip) : 0u;
+            base = Bg + skip;
+            soff = 0u;
+        }
+        const __amdgpu_buffer_rsrc_t rs = make_rsrc(base, bytes);
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lvp)((lds_ptr)lds_e + (wave_u * 2u + j) * 256u), 4, t_vo[j], soff, 0, DMA_AUX);
+    };
     // ---- prime: the first K tile of the first C tile, whole ------------------------------
 #pragma unroll
     for (int pc = 0; pc < NP; ++pc) dma(pc, A0, B0, k_begin);
+    if constexpr (NTAIL) dma_tail(k_begin);
     if (R3) {                                                   // three stages: the second one too
 #pragma unroll
         for (int pc = 0; pc < NP; ++pc) dma(pc, A1, B1, k_begin + BKE);
@@ -645,6 +683,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[i][j] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    floatx4 acc_t = {0.0f, 0.0f, 0.0f, 0.0f};                  // (NTAIL) the 16 x 16 block against the ragged columns
     // The wait also covers the C stores of the previous tile (loads and stores share the counter).
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     if (PATCHES && patch_on && k_begin < k_end && K - 1u - k_begin < (uint32_t)BKE)   // the item's first K tile is also B's last
@@ -673,7 +712,28 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // sixteen rows of a K-contiguous operand, resp. four rows of a row-major B: what separates pieces of one swizzle phase
         const uint32_t a_step = sc(16u * lda * ES), b_step = sc((NT ? 16u : 4u) * ldb * ES);
         bool drained = false;
-        if (NT) {
+        if constexpr (NTAIL) {
+            const uint32_t lds_t = sc((uint32_t)(uintptr_t)lds_e + wave_u * 512u);
+            uint32_t lt = lane;
+            asm volatile("" : "+v"(lt));
+            const uint32_t a_rdt[2] = {a_rd[0] - wm * (WROWS * 128u) + tail_x * 2048u, a_rd[1] - wm * (WROWS * 128u) + tail_x * 2048u};
+            uint32_t t_rd[2];
+            if (NT) {
+                t_rd[0] = (uint32_t)(uintptr_t)lds_e + maps::kc_frag16_offset(0u, 0u, lt);
+                t_rd[1] = (uint32_t)(uintptr_t)lds_e + maps::kc_frag16_offset(0u, 1u, lt);
+                const uint64_t bu = (uint64_t)(uintptr_t)Bg;
+                kloop_asm_nt_ntail(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu),
+                                   sc((uint32_t)(bu >> 32) & 0xFFFFu), sc(b_bytes), 0u, 0u, 0u, 0u, 0x00020000u, lds_a, lds_b, k_early, k_late, sc(k_end), sc(nk),
+                                   acc_t, a_rdt, t_rd, t_vo, lds_t);
+            } else {
+                // the transposing read: lane q of group g addresses columns 4 (q % 4) .. + 3 of row 8 g + q / 4 (+ 4 h, + 32 kh)
+                t_rd[0] = t_rd[1] = (uint32_t)(uintptr_t)lds_e + maps::rc_kn_tr_offset(lt);
+                const uint64_t skip = (uint64_t)k_late * ldb * ES, bu = (uint64_t)(uintptr_t)Bg + skip, rem = b_view - skip, stp = (uint64_t)BKE * ldb * ES;
+                kloop_asm_nn_ntail(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu), sc((uint32_t)(bu >> 32)),
+                                   0u, sc((uint32_t)rem), sc((uint32_t)(rem >> 32)), sc((uint32_t)stp), sc((uint32_t)(stp >> 32)), 0x00020000u, lds_a, lds_b, k_early, k_late,
+                                   sc(k_end), sc(nk), acc_t, a_rdt, t_rd, t_vo, lds_t);
+            }
+        } else if (NT) {
             const uint64_t bu = (uint64_t)(uintptr_t)Bg;
             if constexpr (DEFER) { if (have_ct) { drained = true;
                 kloop_asm_nt_drain(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu),
@@ -750,7 +810,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t eks = ks;
     // ---- hand-over: request the next C tile's first K tile before this one is stored -------
     __syncthreads();                                           // all waves are done with the operand stages
-    const uint32_t em0 = m0, en0 = n0, eslot = part_slot;
+    const uint32_t em0 = m0, en0 = n0, eslot = part_slot, ex = tail_x;
+    const bool elive = tail_live;
     uint16_t* const Ce = Cg;
     const uint32_t next = pid + gridDim.x;
     const bool more = next < total;
@@ -908,6 +969,26 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
         }
         }
+        if constexpr (NTAIL) {
+            // The block against the ragged columns (the same in all four waves; wave 0 stores it): the lane holds columns
+            // 4 (l / 16) .. + 3 of row 16 x + l % 16 of the tile's row panel; columns at or past N get the out-of-range bit,
+            // rows at or past M fall behind the descriptor's end.
+            if (wave_u == 0u && elive) {
+                const uint32_t cq = (le >> 4) * 4u, col = tn * BN + cq, row = ex * 16u + (le & 15u);
+                const uint32_t off = ((row * ldc + col) * 2u) | (col < N ? 0u : OOB);
+                const floatx4 f = acc_t;
+                const u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
+                __builtin_amdgcn_raw_buffer_store_b64(v, rc, off, 0, 0);
+            }
+        }
+    }
+    if constexpr (NTAIL) {
+        // the next tile's first K tile of the ragged columns: its stage is part of the staging region, which every wave
+        // must have left
+        if (more) {
+            __syncthreads();
+            dma_tail(k_begin);
+        }
     }
     if (!more) break;
     pid = next;
@@ -925,6 +1006,9 @@ MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt, true, false, false)
 // ... with the K loop as one assembly statement (gen_kloop.py)
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_asm(GemmArgs p) { mt256::body<false, false, false, false, false, false, -1, 256, 2, true>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_asm(GemmArgs p) { mt256::body<true, false, false, false, false, false, -1, 256, 2, true>(p); }
+// ... for N = 256 t + 8 or 16 (t >= 16): whole tile columns only, the ragged last columns ride along in the K loop
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_ragged(GemmArgs p) { mt256::body<false, false, false, false, false, false, -1, 256, 2, true, true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_ragged(GemmArgs p) { mt256::body<true, false, false, false, false, false, -1, 256, 2, true, true>(p); }
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail, false, true, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_ktail, true, true, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_edge, false, false, true)

@@ -87,6 +87,22 @@ MAIZE_MAP uint32_t sk_tr_offset(uint32_t cg, uint32_t h, uint32_t lane) {
     return sk_offset(sk_tr_row(h, lane), col >> 3) + (col & 7u) * 2u;
 }
 
+// ---- The ragged last columns of a K x N / N x K B riding along in the macro-tile K loop: a 64 x 16 tile (2 KiB) ----
+// Brought in by 4-byte-per-lane requests of 256 bytes, two per wave (request q = 2 wave + j, 0..7), landing linearly.
+// K x N: 64 rows of 32 bytes (columns 0..15), no swizzle; request q covers rows 8 q .. + 7: lane l fetches row
+// 8 q + l / 8, bytes 4 (l % 8) .. + 3.  The transposing read: lane q16 = l % 16 of group g = l / 16 addresses columns
+// 4 (q16 % 4) .. + 3 of row 32 kh + 8 g + 4 h + q16 / 4 (K half kh, register half h as the immediate 1024 kh + 128 h).
+MAIZE_MAP uint32_t rc_kn_row(uint32_t request, uint32_t lane) { return request * 8u + (lane >> 3); }
+MAIZE_MAP uint32_t rc_kn_byte(uint32_t lane) { return (lane & 7u) * 4u; }
+MAIZE_MAP uint32_t rc_kn_tr_offset(uint32_t lane) { return ((lane >> 4) * 8u + ((lane & 15u) >> 2)) * 32u + (lane & 3u) * 8u; }
+// N x K: 16 rows of the K-contiguous layout above (128 bytes, chunk index XOR-ed with (row / 2) % 8): request q covers
+// rows 2 q, 2 q + 1: lane l lands at row 2 q + l / 32, position 4 (l % 32), i.e. fetches bytes 4 (l % 4) .. + 3 of the
+// logical chunk (l % 32) / 4 ^ swizzle(row).  Read like any K-contiguous fragment (kc_frag16_offset).
+MAIZE_MAP uint32_t rc_nk_row(uint32_t request, uint32_t lane) { return request * 2u + (lane >> 5); }
+MAIZE_MAP uint32_t rc_nk_byte(uint32_t request, uint32_t lane) {
+    return ((((lane & 31u) >> 2) ^ kc_swizzle(rc_nk_row(request, lane))) * 16u) + (lane & 3u) * 4u;
+}
+
 // ---- K x N operand tile of 8-bit elements (row-major B of the 8-bit macro-tile kernel): 128 rows of 256 B ----
 // Piece p (4 rows, 1 KiB): lane l lands at row 4p + l/16, position l%16.  16-byte chunks (16 columns) are XOR-ed
 // with f(row) = row%8 + 8 bit4(row): bits 3 and 6 of the row stay out of it, so the four reads of a fragment sit

@@ -247,6 +247,37 @@ int main() {
             }
         std::printf("ok  skinny block: deposit map is a bijection, transposing reads are bank-conflict free\n");
     }
+    // ---- the ragged last columns' 64 x 16 tile: eight requests of 256 bytes (4 bytes per lane) deposit it once, linearly
+    {
+        // K x N: row-major, 32 bytes per row; the transposing reads deliver the MFMA's B operand from it
+        std::set<uint32_t> seen;
+        for (uint32_t q = 0; q < 8; ++q)
+            for (uint32_t lane = 0; lane < 64; ++lane) {
+                const uint32_t row = rc_kn_row(q, lane), byte = rc_kn_byte(lane);
+                CHECK(row < 64 && byte < 32 && byte % 4 == 0, "ragged K x N request out of range");
+                CHECK(row * 32 + byte == q * 256 + lane * 4, "ragged K x N deposit is not linear: request %u lane %u", q, lane);
+                CHECK(seen.insert(row * 32 + byte).second, "ragged K x N byte deposited twice");
+            }
+        CHECK(seen.size() == 64 * 8, "ragged K x N tile not covered");
+        for (uint32_t kh = 0; kh < 2; ++kh)
+            for (uint32_t h = 0; h < 2; ++h)
+                for (uint32_t lane = 0; lane < 64; ++lane) {
+                    const uint32_t q16 = lane & 15u, g = lane >> 4;
+                    const uint32_t row = 32 * kh + 8 * g + 4 * h + q16 / 4, col = 4 * (q16 % 4);
+                    CHECK(rc_kn_tr_offset(lane) + 1024 * kh + 128 * h == row * 32 + col * 2, "ragged K x N transposing read kh %u h %u lane %u", kh, h, lane);
+                }
+        // N x K: sixteen rows of the K-contiguous layout; a fragment read of rows 0..15 finds what the requests deposit
+        std::set<uint32_t> seen2;
+        for (uint32_t q = 0; q < 8; ++q)
+            for (uint32_t lane = 0; lane < 64; ++lane) {
+                const uint32_t row = rc_nk_row(q, lane), byte = rc_nk_byte(q, lane);
+                CHECK(row < 16 && byte < 128, "ragged N x K request out of range");
+                CHECK(kc_offset(row, byte / 16) + byte % 16 == q * 256 + lane * 4, "ragged N x K deposit/read mismatch request %u lane %u", q, lane);
+                CHECK(seen2.insert(row * 128 + byte).second, "ragged N x K byte deposited twice");
+            }
+        CHECK(seen2.size() == 16 * 32, "ragged N x K tile not covered");
+        std::printf("ok  ragged columns' tile: requests deposit it once where the fragment reads expect it, both layouts\n");
+    }
     if (failures) { std::printf("%d violation(s)\n", failures); return 1; }
     std::printf("all LDS maps check out\n");
     return 0;

@@ -110,6 +110,14 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         assert k % 8 == 0 and n % 8 == 0 and (name.endswith("_gen") or k % 64 == 0)
         resident = cus - cus % 8 if cus >= 8 else cus
         assert gx == min(cdiv(m, 128) * cdiv(n, 256) * batch, resident)
+    elif name.endswith("_ragged"):
+        # whole tile columns only: the eight or sixteen ragged last columns ride along in the first sixteen tile columns' K loops
+        assert p["reduce_grid"] == 0 and p["workspace_bytes"] == 0 and p["split_first"] == 0 and p["ksplit"] == 1
+        assert p["block"] == (256, 1, 1) and gy == 1 and gz == 1
+        assert ("_nt" in name) == (layout == mz.LAYOUT_NT)
+        assert k % 64 == 0 and n % 256 in (8, 16) and n // 256 >= 16
+        resident = cus - cus % 8 if cus >= 8 else cus
+        assert gx == min(cdiv(m, 256) * (n // 256) * batch, resident)
     elif "_mt256_" in name:
         assert p["reduce_grid"] == 0
         assert p["block"] == (256, 1, 1) and gy == 1
@@ -194,7 +202,10 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
 def test_north_star_configurations_get_the_kernels_they_were_designed_for():
     picks = {
         (4096, 4096, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn",
-        (4000, 4104, 4032, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_edge",
+        (4000, 4104, 4032, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_ragged",     # eight ragged columns behind sixteen tile columns ride along in the whole tiles' K loops
+        (4000, 4120, 4032, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_edge",       # twenty-four: a narrow last tile column, cut over K
+        (4000, 4104, 4040, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_ktail_edge", # a K tail: the edge-splitting kernel takes any K % 8 == 0
+        (4096, 2056, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn",            # eight tile columns only, and no round to save
         (8192, 8192, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt",
         (16, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
@@ -473,7 +484,7 @@ def test_an_odd_number_of_k_steps_takes_the_loop_that_leaves_after_its_first_ste
         for k in (256, 1024, 4096):
             assert mz.gemm_plan(desc(4096, 4096, k, layout), compute_units=CUS)["kernel"] == f"maize_gemm_bf16_mt256_{tag}", (tag, k)
         assert mz.gemm_plan(desc(4096, 4096, 576 + 8, layout), compute_units=CUS)["kernel"] == f"maize_gemm_bf16_mt256_{tag}_ktail"
-        assert mz.gemm_plan(desc(4000, 4104, 4032, layout), compute_units=CUS)["kernel"] == f"maize_gemm_bf16_mt256_{tag}_edge"
+        assert mz.gemm_plan(desc(4000, 4120, 4032, layout), compute_units=CUS)["kernel"] == f"maize_gemm_bf16_mt256_{tag}_edge"
         x = ex_desc(4096, 4096, 576, layout)
         x.alpha = 0.5
         p = mz.gemm_plan(x, compute_units=CUS)

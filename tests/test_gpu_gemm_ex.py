@@ -116,6 +116,8 @@ def test_macro_tile_kernels_on_strided_views(ctx, oracle, layout, shape, lds):
             continue
         if "ktail" not in name and k % 64:
             continue
+        if name.endswith("_ragged") and not (n % 256 in (8, 16) and n // 256 >= 16):
+            continue                                       # (eight or sixteen columns past sixteen or more whole tile columns only)
         run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, kernel=name, label=name)
 
 

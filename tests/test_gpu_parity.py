@@ -347,7 +347,8 @@ def test_dispatcher_choices(ctx):
         return ctx.gemm_select(mz.gemm_desc(a, b, c, layout=layout, batch=batch, stride_a=m * k, stride_b=k * n,
                                             stride_c=m * n))
     assert pick(4096, 4096, 4096) == "maize_gemm_bf16_mt256_nn"
-    assert pick(4000, 4104, 4032) == "maize_gemm_bf16_mt256_nn_edge"     # 8-column last tile column, 272 tiles
+    assert pick(4000, 4104, 4032) == "maize_gemm_bf16_mt256_nn_ragged"   # 8 ragged columns ride along in the 256 whole tiles' K loops
+    assert pick(4000, 4120, 4032) == "maize_gemm_bf16_mt256_nn_edge"     # 24-column last tile column, 272 tiles: cut over K
     assert pick(8192, 8192, 8192, mz.LAYOUT_NT) == "maize_gemm_bf16_mt256_nt"
     assert pick(16, 14336, 4096) == "maize_gemm_bf16_skinny_nn"
     assert pick(2048, 2048, 2048, batch=32) == "maize_gemm_bf16_mt256_nn"

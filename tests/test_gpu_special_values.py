@@ -21,6 +21,11 @@ P_INF, N_INF, NAN, N_ZERO = 0x7F80, 0xFF80, 0x7FC0, 0x8000
 FAMILIES = [
     ("maize_gemm_bf16_mt256_nn", 512, 520, 256, NN),
     ("maize_gemm_bf16_mt256_nt", 300, 512, 192, NT),
+    # ... with the K loop as one assembly statement: an odd step count (the loop leaves after a trip's first step) and an even one
+    ("maize_gemm_bf16_mt256_nn_asm", 100, 136, 192, NN), ("maize_gemm_bf16_mt256_nt_asm", 260, 264, 320, NT),
+    ("maize_gemm_bf16_mt256_nn_asm", 300, 264, 128, NN),
+    # ... with eight / sixteen ragged last columns riding along (Inf / NaN next to the zero-filled columns past N and rows past M)
+    ("maize_gemm_bf16_mt256_nn_ragged", 300, 4104, 192, NN), ("maize_gemm_bf16_mt256_nt_ragged", 260, 4112, 128, NT),
     ("maize_gemm_bf16_mt256_nn_ktail", 300, 520, 264, NN),
     ("maize_gemm_bf16_mt256_nt_ktail", 257, 264, 328, NT),
     ("maize_gemm_bf16_mt256_nn_gen", 300, 520, 256, NN),

@@ -34,6 +34,7 @@ class Replay:
         self.gen, self.nt = gen, nt
         self.tag, self.unwaited = {}, set()
         self.mfma_of, self.requests, self.stores = {}, [], []
+        self.tail_mfma, self.tail_requests = {}, []
         self.since_barrier_reads = set()       # stages read since the last barrier
         self.outstanding = []                  # vector-memory operations in issue order ("load", stage) / ("store", quad)
 
@@ -41,7 +42,24 @@ class Replay:
         step = -1
         for ln in lines:
             op = ln.split()[0]
-            if op == "ds_read_b128":
+            if op == "ds_read_b128" and ("a_rdt" in ln or "t_rd" in ln):
+                # the block against the ragged columns: its A fragment from A's stage, its B fragment (N x K) from the stages of its own
+                dst, addr, off = re.match(r"ds_read_b128 (\S+), %\[(\w+)\] offset:(\d+)", ln).groups()
+                base, _ = quad(dst)
+                st = int(off) // (32768 if addr.startswith("a_rdt") else 2048)
+                assert int(off) % (32768 if addr.startswith("a_rdt") else 2048) == 0
+                for k in range(4):
+                    self.tag[base + k] = ("ta" if addr.startswith("a_rdt") else "tb", st, 0, int(addr[-1]), 0, k)
+                    self.unwaited.add(base + k)
+            elif op == "ds_read_b64_tr_b16" and "t_rd" in ln:
+                dst, off = re.match(r"ds_read_b64_tr_b16 (\S+), %\[t_rd0\] offset:(\d+)", ln).groups()
+                base, n = quad(dst)
+                st, kh, h = int(off) // 2048, (int(off) % 2048) // 1024, (int(off) % 1024) // 128
+                assert n == 2 and int(off) % 128 == 0 and h < 2
+                for k in range(2):
+                    self.tag[base + k] = ("tb", st, 0, kh, 0, 2 * h + k)
+                    self.unwaited.add(base + k)
+            elif op == "ds_read_b128":
                 dst, addr, off = re.match(r"ds_read_b128 (\S+), %\[(\w+)\] offset:(\d+)", ln).groups()
                 base, _ = quad(dst)
                 slot = int(off) // 2048
@@ -80,6 +98,21 @@ class Replay:
                 self.cur = stage_of_step(step)
                 self.behind_barrier = False
                 self.step = step
+            elif op == "v_mfma_f32_16x16x32_bf16" and "%[ct]" in ln:
+                b, a = re.match(r"\S+ %\[ct\], (\S+), (\S+), %\[ct\]", ln).groups()
+                regs = {quad(a)[0] + k for k in range(4)} | {quad(b)[0] + k for k in range(4)}
+                assert not regs & self.unwaited, f"{ln}: fragment read not waited for"
+                ta = [self.tag[quad(a)[0] + k] for k in range(4)]
+                tb = [self.tag[quad(b)[0] + k] for k in range(4)]
+                assert [t[5] for t in ta] == [0, 1, 2, 3] and [t[5] for t in tb] == [0, 1, 2, 3]
+                assert {t[0] for t in ta} == {"ta"} and {t[0] for t in tb} == {"tb"}
+                assert {t[1] for t in ta + tb} == {self.cur} and len({t[3] for t in ta + tb}) == 1
+                self.tail_mfma.setdefault(self.step, []).append(ta[0][3])
+            elif op == "buffer_load_dword":
+                which, off = self.last_m0
+                assert which == "t" and not self.behind_barrier and off // 2048 == self.cur ^ 1 and off % 2048 in (0, 256)
+                self.tail_requests.append((self.step, off % 2048))
+                self.outstanding.append(("load", off // 2048))
             elif op == "v_mfma_f32_16x16x32_bf16":
                 acc, b, a, acc2 = re.match(r"\S+ (%\[c\d\d\]), (\S+), (\S+), (%\[c\d\d\])", ln).groups()
                 assert acc == acc2
@@ -105,7 +138,7 @@ class Replay:
                 self.requests.append((self.step, which, st, piece))
                 self.outstanding.append(("load", st))
             elif op == "s_add_u32" and ln.split()[1] == "m0,":
-                base, off = re.match(r"s_add_u32 m0, %\[lds_(\w)\], (\d+)", ln).groups()
+                base, off = re.match(r"s_add_u32 m0, %\[lds_(\w)\], (\d+)", ln).groups()      # lds_a, lds_b, lds_t
                 self.last_m0 = (base, int(off))
             elif op == "buffer_store_dwordx4":
                 base, n = quad(ln.split()[1].rstrip(","))
@@ -172,3 +205,28 @@ def test_the_default_make_target_builds_the_library_and_the_generated_loop_first
     plan = subprocess.run(["make", "-n", "-B", "-C", csrc], check=True, capture_output=True, text=True).stdout
     assert "gen_kloop.py" in plan and "gemm_kernels.hip" in plan and "libmaize_hip.so" in plan
     assert plan.index("gen_kloop.py") < plan.index("gemm_kernels.hip") < plan.index("libmaize_hip.so")
+
+
+@pytest.mark.parametrize("nt", [False, True], ids=["nn", "nt"])
+def test_the_ragged_columns_block_rides_along(nt):
+    """The form of the loop that also multiplies one 16 x 16 block against the ragged last columns: per K step two more
+    matrix instructions (K half 0, then 1) on fragments of the step's own stage, read and waited for, and two 256-byte
+    requests per wave into the other stage of the block's B tile, in front of the barrier; the rest of the loop as before."""
+    gen = load_generator(0)
+    em = gen.Emitter(nt, False, True)
+    em.loop()
+    lines = [l for l in em.lines if not l.startswith("L_")]
+    rp = Replay(gen, nt)
+    rp.run(lines, stage_of_step=lambda t: t & 1)
+    assert rp.step == 1
+    for t in range(2):
+        assert rp.tail_mfma[t] == [0, 1]
+        assert sorted(o for s_, o in rp.tail_requests if s_ == t) == [0, 256]
+        for i in range(8):
+            for j in range(8):
+                assert rp.mfma_of[(t, i, j)] == [0, 1]
+    assert sum(l.startswith("v_mfma") for l in lines) == 2 * (128 + 2)
+    # the plain form has none of it
+    plain = gen.Emitter(nt)
+    plain.loop()
+    assert not any("%[ct]" in l or "lds_t" in l for l in plain.lines)

@@ -70,7 +70,7 @@ def test_ragged_panels_are_reported_and_still_computed():
     kernel, (a_epi, b_epi) = describe(a, b, c)
     assert (a_epi.rows, a_epi.ragged) == (4000 % 256, True) and b_epi.cols == 4104 % 256
     loaded = kernel.finalize().compile(mz.Gfx.Gfx950, FakeCtx())
-    assert loaded.kernel_name == "maize_gemm_bf16_mt256_nn_edge"     # the ragged last tile column is split over K
+    assert loaded.kernel_name == "maize_gemm_bf16_mt256_nn_ragged"   # the eight ragged columns ride along in the whole tiles' K loops
 
 
 def test_nt_f16_f8_and_the_any_shape_instruction():

@@ -65,7 +65,7 @@ def test_noalloc_matches_the_allocating_entry_point_twice_in_a_row(ctx, oracle):
         oracle.assert_parity(s, "noalloc")
 
 
-@pytest.mark.parametrize("shape", [(64, 4096, 4096, mz.LAYOUT_NN), (16, 4096, 4096, mz.LAYOUT_NT), (4000, 4104, 4032, mz.LAYOUT_NN),
+@pytest.mark.parametrize("shape", [(64, 4096, 4096, mz.LAYOUT_NN), (16, 4096, 4096, mz.LAYOUT_NT), (4000, 4120, 4032, mz.LAYOUT_NN),
                                    (512, 512, 512, mz.LAYOUT_NN)],
                          ids=["splitk_mt256", "skinny_nt", "edge_split", "no_scratch_needed"])
 def test_noalloc_every_scratch_user(ctx, shape):
