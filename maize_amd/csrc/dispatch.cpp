@@ -103,6 +103,18 @@ bool ntail_shape(const maize_gemm_ex_desc_t& d) {
     if (s.nt && (uint64_t)s.n * lds_of(d).b * 2u >= 0x7FFFFFFFull) return false;
     return true;
 }
+// ... and the mirror image: M = 256 t + 1 .. 16 with t >= 16 whole tile rows; the ragged rows of A and C are addressed
+// from a tile's first row with 32-bit offsets (A and C under 2 GiB).
+bool mtail_shape(const maize_gemm_ex_desc_t& d) {
+    const Dims s = dims_of(d);
+    const uint32_t h = s.m % 256u;
+    if (h == 0u || h > 16u || s.m / 256u < 16u) return false;
+    const Lds l = lds_of(d);
+    if ((uint64_t)s.m * l.a * 2u >= 0x7FFFFFFFull || (uint64_t)s.m * l.c * 2u >= 0x7FFFFFFFull) return false;
+    return true;
+}
+bool mt256_nn_ragged_m_supports(const maize_gemm_ex_desc_t& d) { return mt256_nn_supports(d) && mtail_shape(d); }
+bool mt256_nt_ragged_m_supports(const maize_gemm_ex_desc_t& d) { return mt256_nt_supports(d) && mtail_shape(d); }
 bool mt256_nn_ragged_supports(const maize_gemm_ex_desc_t& d) { return mt256_nn_supports(d) && ntail_shape(d); }
 bool mt256_nt_ragged_supports(const maize_gemm_ex_desc_t& d) { return mt256_nt_supports(d) && ntail_shape(d); }
 bool mt256_nn_ktail_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_common(d) && plain_epilogue(d) && bf16_in(d); }
@@ -237,10 +249,10 @@ bool mt256_h128_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Laun
     return true;
 }
 bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
-// ... over the whole tile columns only (the ragged last columns have no tiles of their own)
-bool mt256_ntail_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, LaunchDims* ld) {
+// ... over the whole tile columns (rows) only: the ragged last columns (rows) have no tiles of their own
+bool ragged_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, bool rows, LaunchDims* ld) {
     const Dims s = dims_of(d);
-    const uint64_t all = (uint64_t)cdiv(s.m, 256) * (s.n / 256u) * d.gemm.batch;
+    const uint64_t all = (rows ? (uint64_t)(s.m / 256u) * cdiv(s.n, 256) : (uint64_t)cdiv(s.m, 256) * (s.n / 256u)) * d.gemm.batch;
     if (all == 0 || all > 0x1FFFFFFFull) return false;
     const uint32_t resident = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
     ld->grid[0] = (resident && all > resident) ? resident : (uint32_t)all;
@@ -249,6 +261,8 @@ bool mt256_ntail_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Lau
     ld->lds_bytes = 0; ld->ksplit = 1; ld->split_first = 0; ld->reduce_grid = 0; ld->workspace_bytes = 0;
     return true;
 }
+bool mt256_ntail_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return ragged_plan(d, cus, false, ld); }
+bool mt256_mtail_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return ragged_plan(d, cus, true, ld); }
 
 // ---- maize_gemm_{bf16,f16}_mt256_{nn,nt}_splitk: few tiles, long K ---------------------------
 // K ranges per tile.  Candidates: up to one (tile, range) work item per compute unit, at least 4 K
@@ -869,6 +883,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_mt256_nt_asm", nullptr, mt256_nt_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_ragged", nullptr, mt256_nn_ragged_supports, mt256_ntail_plan},  // ... with ragged last columns riding along
     {"maize_gemm_bf16_mt256_nt_ragged", nullptr, mt256_nt_ragged_supports, mt256_ntail_plan},
+    {"maize_gemm_bf16_mt256_nn_ragged_m", nullptr, mt256_nn_ragged_m_supports, mt256_mtail_plan},  // ... with ragged last rows riding along
+    {"maize_gemm_bf16_mt256_nt_ragged_m", nullptr, mt256_nt_ragged_m_supports, mt256_mtail_plan},
     {"maize_gemm_bf16_mt256_nn_h128", nullptr, mt256_nn_supports, mt256_h128_plan},
     {"maize_gemm_bf16_mt256_nt_h128", nullptr, mt256_nt_supports, mt256_h128_plan},
     {"maize_gemm_bf16_mt256_nn_h128_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_h128_plan},
@@ -1137,6 +1153,13 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         if (ri >= 0 && units && kKernels[ri].supports(d)) {
             const uint64_t tm = cdiv(s.m, 256), with = tm * cdiv(s.n, 256) * d.gemm.batch, without = tm * (s.n / 256u) * d.gemm.batch;
             if ((with + units - 1) / units > (without + units - 1) / units) return (uint32_t)ri;
+        }
+        // ... or up to sixteen ragged last rows behind sixteen or more whole tile rows
+        static const char* const kRaggedM[2] = {"maize_gemm_bf16_mt256_nn_ragged_m", "maize_gemm_bf16_mt256_nt_ragged_m"};
+        const int mi = kernel_index(kRaggedM[s.nt]);
+        if (mi >= 0 && units && kKernels[mi].supports(d)) {
+            const uint64_t tnc = cdiv(s.n, 256), with = cdiv(s.m, 256) * tnc * d.gemm.batch, without = (s.m / 256u) * tnc * d.gemm.batch;
+            if ((with + units - 1) / units > (without + units - 1) / units) return (uint32_t)mi;
         }
     }
     // An odd number of K steps: the plain kernel's statement loop runs two steps per trip and pads with a step on a

@@ -150,11 +150,13 @@ __device__ __forceinline__ void tile_of(uint32_t id, uint32_t tm, uint32_t tn, u
 // t+3 go out one every two slots from the barrier of step t on (seven behind it, five in front of the next), same wait.
 // ASM: the K loop is the generated assembly statement (kloop_gen.inc) instead of the step() statements below: the same
 // schedule with registers assigned by hand, for the plain 256-row bf16 kernels.
-template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2, bool ASM = false, bool NTAIL = false>
+template <bool NT, bool KTAIL, bool EDGE, bool GEN, bool F16, bool SPLITK, int F8 = -1, int BMT = 256, int NST = 2, bool ASM = false, bool NTAIL = false, bool MTAIL = false>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
     static_assert(!ASM || (!KTAIL && !EDGE && !GEN && !F16 && !SPLITK && F8 < 0 && BMT == 256 && NST == 2), "the assembly K loop: plain 256-row bf16 kernels");
-    static_assert(!NTAIL || ASM, "the ragged last columns ride along in the assembly K loop only");
+    static_assert(!(NTAIL || MTAIL) || ASM, "ragged last columns or rows ride along in the assembly K loop only");
+    static_assert(!(NTAIL && MTAIL), "ragged columns or ragged rows, not both");
+    constexpr bool RTAIL = NTAIL || MTAIL;
     constexpr bool H128 = BMT == 128;
     static_assert(BMT == 256 || (H128 && !EDGE), "128-row tiles: no edge splitting");
     constexpr bool R3 = NST == 3;                       // three ring stages (128-row tiles)
@@ -199,7 +201,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t wm = wave >> 1, wn = wave & 1u;
     // NTAIL: N = 256 tn + 8 or 16; the columns past the last whole tile column have no tiles of their own (below)
-    const uint32_t tm = (M + BMT - 1) / BMT, tn = NTAIL ? N / BN : (N + BN - 1) / BN;
+    // (MTAIL, the mirror image: M = 256 tm + 1 .. 16; the rows past the last whole tile row have no tiles)
+    const uint32_t tm = MTAIL ? M / BMT : (M + BMT - 1) / BMT, tn = NTAIL ? N / BN : (N + BN - 1) / BN;
     // Workgroups 0 .. whole-1 compute one tile each over all of K.  With edge splitting
     // (p.reserved = mode << 30 | whole + 1; mode 1: last tile column, mode 2: last tile row) the
     // whole tiles are the grid without that edge, and the rest of the workgroups share the edge
@@ -311,6 +314,16 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             b_bytes = 0u;
         }
         Cg = p.c + bz * p.stride_c * ((GEN && (p.epi & EPI_F32)) ? 2u : 1u);   // strides count elements of C
+        if constexpr (MTAIL) {
+            // the ragged rows of A as 16 rows of a K-contiguous tile, addressed from this tile's first row
+            tail_x = tile_m & 15u;
+            tail_live = tile_m < 16u;
+            uint32_t lt = lane;
+            asm volatile("" : "+v"(lt));
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                t_vo[j] = (tm * BMT - m0 + maps::rc_nk_row(wave * 2u + j, lt)) * lda * ES + maps::rc_nk_byte(wave * 2u + j, lt);
+        }
         if constexpr (NTAIL) {
             tail_x = tile_n & 15u;
             tail_live = tile_n < 16u;
@@ -656,9 +669,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // epilogue's staging region, which is idle from the top of a C tile's K loop to its end).
     auto dma_tail = [&](uint32_t k) {
         typedef __attribute__((address_space(3))) void* lvp;
-        const char* base = Bg;
-        uint32_t bytes = k < k_end ? b_bytes : 0u, soff = k * ES;
-        if (!NT) {
+        const char* base = MTAIL ? Ag : Bg;
+        uint32_t bytes = k < k_end ? (MTAIL ? a_bytes : b_bytes) : 0u, soff = k * ES;
+        if (!NT && !MTAIL) {
             const uint64_t skip = (uint64_t)k * ldb * ES;
             bytes = k < k_end ? span(b_view - skip) : 0u;
             base = Bg + skip;
@@ -672,7 +685,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // ---- prime: the first K tile of the first C tile, whole ------------------------------
 #pragma unroll
     for (int pc = 0; pc < NP; ++pc) dma(pc, A0, B0, k_begin);
-    if constexpr (NTAIL) dma_tail(k_begin);
+    if constexpr (RTAIL) dma_tail(k_begin);
     if (R3) {                                                   // three stages: the second one too
 #pragma unroll
         for (int pc = 0; pc < NP; ++pc) dma(pc, A1, B1, k_begin + BKE);
@@ -712,7 +725,28 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // sixteen rows of a K-contiguous operand, resp. four rows of a row-major B: what separates pieces of one swizzle phase
         const uint32_t a_step = sc(16u * lda * ES), b_step = sc((NT ? 16u : 4u) * ldb * ES);
         bool drained = false;
-        if constexpr (NTAIL) {
+        if constexpr (MTAIL) {
+            const uint32_t lds_t = sc((uint32_t)(uintptr_t)lds_e + wave_u * 512u);
+            uint32_t lt = lane;
+            asm volatile("" : "+v"(lt));
+            const uint32_t t_rd[2] = {(uint32_t)(uintptr_t)lds_e + maps::kc_frag16_offset(0u, 0u, lt), (uint32_t)(uintptr_t)lds_e + maps::kc_frag16_offset(0u, 1u, lt)};
+            uint32_t b_rdt[2];
+            if (NT) {
+                // columns 16 x .. + 15 of the tile's column panel: fragment x of B's stage (this wave's own start at fragment 8 wn)
+                b_rdt[0] = b_rd[0] - wn * (128u * 128u) + tail_x * 2048u;
+                b_rdt[1] = b_rd[1] - wn * (128u * 128u) + tail_x * 2048u;
+                const uint64_t bu = (uint64_t)(uintptr_t)Bg;
+                kloop_asm_nt_mtail(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu),
+                                   sc((uint32_t)(bu >> 32) & 0xFFFFu), sc(b_bytes), 0u, 0u, 0u, 0u, 0x00020000u, lds_a, lds_b, k_early, k_late, sc(k_end), sc(nk),
+                                   acc_t, b_rdt, t_rd, t_vo, lds_t);
+            } else {
+                b_rdt[0] = b_rdt[1] = (uint32_t)(uintptr_t)B0 + maps::sk_tr_offset(tail_x, 0u, lt);
+                const uint64_t skip = (uint64_t)k_late * ldb * ES, bu = (uint64_t)(uintptr_t)Bg + skip, rem = b_view - skip, stp = (uint64_t)BKE * ldb * ES;
+                kloop_asm_nn_mtail(acc, a_rd, b_rd, a_vo, b_vo, a_step, b_step, sc((uint32_t)au), sc((uint32_t)(au >> 32) & 0xFFFFu), sc(a_bytes), sc((uint32_t)bu), sc((uint32_t)(bu >> 32)),
+                                   0u, sc((uint32_t)rem), sc((uint32_t)(rem >> 32)), sc((uint32_t)stp), sc((uint32_t)(stp >> 32)), 0x00020000u, lds_a, lds_b, k_early, k_late,
+                                   sc(k_end), sc(nk), acc_t, b_rdt, t_rd, t_vo, lds_t);
+            }
+        } else if constexpr (NTAIL) {
             const uint32_t lds_t = sc((uint32_t)(uintptr_t)lds_e + wave_u * 512u);
             uint32_t lt = lane;
             asm volatile("" : "+v"(lt));
@@ -969,6 +1003,17 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
         }
         }
+        if constexpr (MTAIL) {
+            // The ragged rows against this tile's columns 16 x .. + 15 (wave 0 stores): the lane holds columns 4 (l / 16) .. + 3 of
+            // ragged row l % 16; rows at or past M fall behind the descriptor's end, columns at or past N get the bit.
+            if (wave_u == 0u && elive) {
+                const uint32_t col = en0 + ex * 16u + (le >> 4) * 4u, row = tm * BMT - em0 + (le & 15u);
+                const uint32_t off = ((row * ldc + col) * 2u) | (col < N ? 0u : OOB);
+                const floatx4 f = acc_t;
+                const u32x2 v = {cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3])};
+                __builtin_amdgcn_raw_buffer_store_b64(v, rc, off, 0, 0);
+            }
+        }
         if constexpr (NTAIL) {
             // The block against the ragged columns (the same in all four waves; wave 0 stores it): the lane holds columns
             // 4 (l / 16) .. + 3 of row 16 x + l % 16 of the tile's row panel; columns at or past N get the out-of-range bit,
@@ -982,8 +1027,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
         }
     }
-    if constexpr (NTAIL) {
-        // the next tile's first K tile of the ragged columns: its stage is part of the staging region, which every wave
+    if constexpr (RTAIL) {
+        // the next tile's first K tile of the ragged columns (rows): its stage is part of the staging region, which every wave
         // must have left
         if (more) {
             __syncthreads();
@@ -1009,6 +1054,9 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_asm(G
 // ... for N = 256 t + 8 or 16 (t >= 16): whole tile columns only, the ragged last columns ride along in the K loop
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_ragged(GemmArgs p) { mt256::body<false, false, false, false, false, false, -1, 256, 2, true, true>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_ragged(GemmArgs p) { mt256::body<true, false, false, false, false, false, -1, 256, 2, true, true>(p); }
+// ... and the mirror image, M = 256 t + 1 .. 16 (t >= 16): whole tile rows only, the ragged last rows ride along
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nn_ragged_m(GemmArgs p) { mt256::body<false, false, false, false, false, false, -1, 256, 2, true, false, true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_mt256_nt_ragged_m(GemmArgs p) { mt256::body<true, false, false, false, false, false, -1, 256, 2, true, false, true>(p); }
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_ktail, false, true, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nt_ktail, true, true, false)
 MAIZE_MT256_KERNEL(maize_gemm_bf16_mt256_nn_edge, false, false, true)

@@ -42,7 +42,7 @@ CT0 = 64                   # v[64:191]: quad Q = 8 p + r in v[CT0 + 4 Q .. + 3]:
 S_DC = SW + 16             # s[96:99]  descriptor of the C tile being drained
 S_T2 = SW + 20             # s100      scratch of the requests
 VT0 = 63                   # v63       per-lane byte offset of a request (read when the request issues: the next may overwrite it)
-FT_A, FT_B = 184, 188     # v[184:187], v[188:191]: A and B fragment of the ragged-column block (the "ntail" form of the loop)
+FT_A, FT_B = 184, 188     # v[184:187], v[188:191]: A and B fragment of the ragged block (the "ntail" / "mtail" forms of the loop)
 DRAIN_POLICY = " nt"       # cache policy of the deferred stores (" nt": streaming, like the stores of the epilogue)
 # K steps a deferred tile is stored over (an even divisor of 32: 32 / DRAIN_STEPS stores of 16 bytes per lane and step), or
 # 0: no deferred stores, the build that ships.  Measured (4 x 4096^3, four tiles per workgroup): stores inside the K loop
@@ -70,10 +70,12 @@ def acc(i, j):
 
 
 class Emitter:
-    def __init__(self, nt, drain=False, ntail=False):
+    def __init__(self, nt, drain=False, ntail=False, mtail=False):
         self.nt = nt
         self.drain = drain
         self.ntail = ntail
+        self.mtail = mtail
+        assert not (ntail and mtail)
         self.lines = []
 
     # ---- the ragged last columns of B and C (N = 256 t + 8 or 16) -----------------------------------
@@ -83,13 +85,29 @@ class Emitter:
     # stores it).  Its B tile, 64 x 16 elements (2 KiB), has two stages of its own at %[lds_t]; each wave brings in a
     # quarter with two 4-byte-per-lane requests behind B's last piece, into the stage of tile t+1; its A fragment is
     # read from A's stage (address registers %[a_rdt0/1] point at the block's rows).
+    # The mirror image ("mtail"): up to sixteen ragged last rows of A and C (M = 256 t + 1 .. 16).  The workgroup of tile
+    # (tm, tn) multiplies them against columns 16 (tm % 16) .. + 15 of its column panel: the B fragment comes from B's
+    # stage (address registers %[b_rdt..]), the rows' A tile (16 x 64, K-contiguous, 2 KiB) has the two stages at
+    # %[lds_t] and is requested through A's descriptor -- whose length word still stands for tile t+1 in front of the
+    # barrier of step t -- at tile t+1's byte offset.
     def tail_request(self, j, stage):
         self.e(f"s_add_u32 m0, %[lds_t], {stage * 2048 + j * 256}")
         self.e("s_nop 0")
-        soff = f"s{S_OL}" if self.nt else "0"
-        self.e(f"buffer_load_dword %[t_vo{j}], s[{S_DB}:{S_DB + 3}], {soff} offen lds")
+        if self.mtail:
+            self.e(f"buffer_load_dword %[t_vo{j}], s[{S_DA}:{S_DA + 3}], s{S_OL} offen lds")
+        else:
+            soff = f"s{S_OL}" if self.nt else "0"
+            self.e(f"buffer_load_dword %[t_vo{j}], s[{S_DB}:{S_DB + 3}], {soff} offen lds")
 
     def tail_reads(self, kh, st):
+        if self.mtail:
+            self.e(f"ds_read_b128 v[{FT_A}:{FT_A + 3}], %[t_rd{kh}] offset:{st * 2048}")
+            if self.nt:
+                self.e(f"ds_read_b128 v[{FT_B}:{FT_B + 3}], %[b_rdt{kh}] offset:{st * 32768}")
+            else:
+                for h in range(2):
+                    self.e(f"ds_read_b64_tr_b16 v[{FT_B + 2 * h}:{FT_B + 2 * h + 1}], %[b_rdt0] offset:{st * 32768 + kh * 16384 + h * 2048}")
+            return
         self.e(f"ds_read_b128 v[{FT_A}:{FT_A + 3}], %[a_rdt{kh}] offset:{st * 32768}")
         if self.nt:
             self.e(f"ds_read_b128 v[{FT_B}:{FT_B + 3}], %[t_rd{kh}] offset:{st * 2048}")
@@ -243,7 +261,7 @@ class Emitter:
                     assert (pc < 8) == (e >= EB)
                     self.request(pc, cur if e >= EB else nxt)
                 self.drain_side_work(t, e, s)
-                if self.ntail:
+                if self.ntail or self.mtail:
                     if e == 2 and s in (2, 6):
                         self.tail_request((s - 2) // 4, nxt)
                     if e in (0, 4) and s == 10:
@@ -266,6 +284,11 @@ class Emitter:
             self.e(f"s_mov_b32 s{S_BASE + 1}, %[b_hi]")
             self.e(f"s_mov_b32 s{S_REM}, %[b_rem_lo]")
             self.e(f"s_mov_b32 s{S_REM + 1}, %[b_rem_hi]")
+        if self.mtail:
+            # (the ragged rows' first request, in front of step 0's barrier, goes through A's descriptor: its length word,
+            # otherwise first written behind that barrier, stands for the tile at k_late)
+            self.e("s_cmp_lt_u32 %[k_late], %[k_end]")
+            self.e(f"s_cselect_b32 s{S_DA + 2}, %[a_bytes], 0")
         self.e(f"s_lshl_b32 s{S_OE}, %[k_early], 1")
         self.e(f"s_lshl_b32 s{S_OL}, %[k_late], 1")
         self.e(f"s_mov_b32 s{S_KT}, 0")
@@ -297,10 +320,10 @@ class Emitter:
         self.e("L_kloop_end_%=:")
 
 
-def function(nt, drain=False, ntail=False):
-    em = Emitter(nt, drain, ntail)
+def function(nt, drain=False, ntail=False, mtail=False):
+    em = Emitter(nt, drain, ntail, mtail)
     em.loop()
-    name = ("kloop_asm_nt" if nt else "kloop_asm_nn") + ("_drain" if drain else "") + ("_ntail" if ntail else "")
+    name = ("kloop_asm_nt" if nt else "kloop_asm_nn") + ("_drain" if drain else "") + ("_ntail" if ntail else "") + ("_mtail" if mtail else "")
     nb_rd = 2 if nt else 8
     out = []
     out.append(f"// {'B stored N x K' if nt else 'B stored K x N (row-major)'}: {sum(l.startswith('v_mfma') for l in em.lines)} matrix instructions per trip")
@@ -310,8 +333,8 @@ def function(nt, drain=False, ntail=False):
               "uint32_t flags, uint32_t lds_a, uint32_t lds_b, uint32_t& k_early, uint32_t& k_late, uint32_t k_end, uint32_t nk"]
     if drain:
         params += ["const u32x4 (&ct)[32]", "uint32_t c_vo", "uint32_t c_lo, uint32_t c_hi, uint32_t c_bytes, uint32_t c_row_bytes"]
-    if ntail:
-        params += ["floatx4& acc_t", "const uint32_t (&a_rdt)[2]", "const uint32_t (&t_rd)[2]", "const uint32_t (&t_vo)[2]", "uint32_t lds_t"]
+    if ntail or mtail:    # (x_rdt: address registers of the fragment read from the whole tile's stage, A's or B's)
+        params += ["floatx4& acc_t", "const uint32_t (&x_rdt)[2]", "const uint32_t (&t_rd)[2]", "const uint32_t (&t_vo)[2]", "uint32_t lds_t"]
     out.append(f"__device__ __forceinline__ void {name}({', '.join(params)}) {{")
     out.append("    asm volatile(")
     for l in em.lines:
@@ -340,7 +363,11 @@ def function(nt, drain=False, ntail=False):
         clob += [f'"s{r}"' for r in range(S_DC, S_DC + 4)]
     if ntail:
         outs += ['[ct] "+v"(acc_t)']
-        ins += [f'[a_rdt{k}] "v"(a_rdt[{k}])' for k in range(2)] + [f'[t_rd{k}] "v"(t_rd[{k}])' for k in range(2 if nt else 1)]
+        ins += [f'[a_rdt{k}] "v"(x_rdt[{k}])' for k in range(2)] + [f'[t_rd{k}] "v"(t_rd[{k}])' for k in range(2 if nt else 1)]
+    if mtail:
+        outs += ['[ct] "+v"(acc_t)']
+        ins += [f'[b_rdt{k}] "v"(x_rdt[{k}])' for k in range(2 if nt else 1)] + [f'[t_rd{k}] "v"(t_rd[{k}])' for k in range(2)]
+    if ntail or mtail:
         ins += [f'[t_vo{k}] "v"(t_vo[{k}])' for k in range(2)] + ['[lds_t] "s"(lds_t)']
         clob += [f'"v{r}"' for r in range(FT_A, FT_B + 4)]
     out.append("        : " + ", ".join(outs))
@@ -360,7 +387,7 @@ def main():
     text = ["// GENERATED by gen_kloop.py -- do not edit.  The K loop of the 256 x 256 bf16 macro-tile kernel as one",
             "// inline-assembly statement with its own register assignment (see the generator for the register map).",
             "#pragma once", "", f"constexpr uint32_t KLOOP_DRAIN_STEPS = {DRAIN_STEPS};   // K steps a deferred C tile is stored over", "", function(True), "", function(False), ""]
-    text += [function(True, ntail=True), "", function(False, ntail=True), ""]
+    text += [function(True, ntail=True), "", function(False, ntail=True), "", function(True, mtail=True), "", function(False, mtail=True), ""]
     if DRAIN_STEPS:
         text += [function(True, True), "", function(False, True), ""]
     with open(sys.argv[1], "w") as f:

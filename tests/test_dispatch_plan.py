@@ -110,6 +110,14 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
         assert k % 8 == 0 and n % 8 == 0 and (name.endswith("_gen") or k % 64 == 0)
         resident = cus - cus % 8 if cus >= 8 else cus
         assert gx == min(cdiv(m, 128) * cdiv(n, 256) * batch, resident)
+    elif name.endswith("_ragged_m"):
+        # the mirror image: whole tile rows only, up to sixteen ragged last rows ride along in the first sixteen tile rows' K loops
+        assert p["reduce_grid"] == 0 and p["workspace_bytes"] == 0 and p["split_first"] == 0 and p["ksplit"] == 1
+        assert p["block"] == (256, 1, 1) and gy == 1 and gz == 1
+        assert ("_nt" in name) == (layout == mz.LAYOUT_NT)
+        assert k % 64 == 0 and 1 <= m % 256 <= 16 and m // 256 >= 16
+        resident = cus - cus % 8 if cus >= 8 else cus
+        assert gx == min((m // 256) * cdiv(n, 256) * batch, resident)
     elif name.endswith("_ragged"):
         # whole tile columns only: the eight or sixteen ragged last columns ride along in the first sixteen tile columns' K loops
         assert p["reduce_grid"] == 0 and p["workspace_bytes"] == 0 and p["split_first"] == 0 and p["ksplit"] == 1
@@ -206,6 +214,9 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (4000, 4120, 4032, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_edge",       # twenty-four: a narrow last tile column, cut over K
         (4000, 4104, 4040, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_ktail_edge", # a K tail: the edge-splitting kernel takes any K % 8 == 0
         (4096, 2056, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn",            # eight tile columns only, and no round to save
+        (4100, 4096, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_ragged_m",   # four ragged rows behind sixteen tile rows: the mirror image
+        (4104, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_ragged_m",
+        (4120, 4096, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_edge",       # twenty-four rows: a short last tile row, cut over K
         (8192, 8192, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt",
         (16, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",

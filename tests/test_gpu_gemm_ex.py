@@ -118,6 +118,8 @@ def test_macro_tile_kernels_on_strided_views(ctx, oracle, layout, shape, lds):
             continue
         if name.endswith("_ragged") and not (n % 256 in (8, 16) and n // 256 >= 16):
             continue                                       # (eight or sixteen columns past sixteen or more whole tile columns only)
+        if name.endswith("_ragged_m") and not (1 <= m % 256 <= 16 and m // 256 >= 16):
+            continue                                       # (up to sixteen rows past sixteen or more whole tile rows only)
         run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, kernel=name, label=name)
 
 

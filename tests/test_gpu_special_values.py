@@ -26,6 +26,8 @@ FAMILIES = [
     ("maize_gemm_bf16_mt256_nn_asm", 300, 264, 128, NN),
     # ... with eight / sixteen ragged last columns riding along (Inf / NaN next to the zero-filled columns past N and rows past M)
     ("maize_gemm_bf16_mt256_nn_ragged", 300, 4104, 192, NN), ("maize_gemm_bf16_mt256_nt_ragged", 260, 4112, 128, NT),
+    # ... and with one to sixteen ragged last rows riding along
+    ("maize_gemm_bf16_mt256_nn_ragged_m", 4099, 264, 192, NN), ("maize_gemm_bf16_mt256_nt_ragged_m", 4112, 304, 128, NT),
     ("maize_gemm_bf16_mt256_nn_ktail", 300, 520, 264, NN),
     ("maize_gemm_bf16_mt256_nt_ktail", 257, 264, 328, NT),
     ("maize_gemm_bf16_mt256_nn_gen", 300, 520, 256, NN),

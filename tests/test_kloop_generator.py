@@ -35,6 +35,7 @@ class Replay:
         self.tag, self.unwaited = {}, set()
         self.mfma_of, self.requests, self.stores = {}, [], []
         self.tail_mfma, self.tail_requests = {}, []
+        self.mtail_form = False
         self.since_barrier_reads = set()       # stages read since the last barrier
         self.outstanding = []                  # vector-memory operations in issue order ("load", stage) / ("store", quad)
 
@@ -42,20 +43,30 @@ class Replay:
         step = -1
         for ln in lines:
             op = ln.split()[0]
-            if op == "ds_read_b128" and ("a_rdt" in ln or "t_rd" in ln):
+            if op == "ds_read_b128" and ("a_rdt" in ln or "b_rdt" in ln or "t_rd" in ln):
                 # the block against the ragged columns: its A fragment from A's stage, its B fragment (N x K) from the stages of its own
                 dst, addr, off = re.match(r"ds_read_b128 (\S+), %\[(\w+)\] offset:(\d+)", ln).groups()
                 base, _ = quad(dst)
-                st = int(off) // (32768 if addr.startswith("a_rdt") else 2048)
-                assert int(off) % (32768 if addr.startswith("a_rdt") else 2048) == 0
+                stride = 2048 if addr.startswith("t_rd") else 32768         # the block's own tile, or a fragment of the whole tile's stage
+                st = int(off) // stride
+                assert int(off) % stride == 0
+                # which operand the registers feed is told by where they sit: the A fragment's or the B fragment's
+                side = "ta" if base == self.gen.FT_A else "tb"
+                assert base in (self.gen.FT_A, self.gen.FT_B)
+                assert addr.startswith("t_rd") == ((side == "tb") != self.mtail_form), f"{ln}: fragment from the wrong place"
                 for k in range(4):
-                    self.tag[base + k] = ("ta" if addr.startswith("a_rdt") else "tb", st, 0, int(addr[-1]), 0, k)
+                    self.tag[base + k] = (side, st, 0, int(addr[-1]), 0, k)
                     self.unwaited.add(base + k)
-            elif op == "ds_read_b64_tr_b16" and "t_rd" in ln:
-                dst, off = re.match(r"ds_read_b64_tr_b16 (\S+), %\[t_rd0\] offset:(\d+)", ln).groups()
+            elif op == "ds_read_b64_tr_b16" and ("t_rd" in ln or "b_rdt" in ln):
+                dst, addr, off = re.match(r"ds_read_b64_tr_b16 (\S+), %\[(t_rd0|b_rdt0)\] offset:(\d+)", ln).groups()
                 base, n = quad(dst)
-                st, kh, h = int(off) // 2048, (int(off) % 2048) // 1024, (int(off) % 1024) // 128
-                assert n == 2 and int(off) % 128 == 0 and h < 2
+                if addr == "t_rd0":      # the ragged columns' own K x N tile: 32 bytes per row
+                    st, kh, h = int(off) // 2048, (int(off) % 2048) // 1024, (int(off) % 1024) // 128
+                    assert int(off) % 128 == 0 and not self.mtail_form
+                else:                    # a column block of B's stage (ragged rows)
+                    st, kh, h = int(off) // 32768, (int(off) % 32768) // 16384, (int(off) % 16384) // 2048
+                    assert int(off) % 2048 == 0 and self.mtail_form
+                assert n == 2 and h < 2
                 for k in range(2):
                     self.tag[base + k] = ("tb", st, 0, kh, 0, 2 * h + k)
                     self.unwaited.add(base + k)
@@ -93,8 +104,8 @@ class Replay:
                 assert not self.unwaited, "barrier with fragment reads in flight"
                 self.since_barrier_reads = set()
                 self.behind_barrier = True
-            elif op.startswith("s_cmp") and "k_late" in ln:
-                step += 1                                   # bytes_of_b opens a K step
+            elif op == "s_cselect_b32" and ln.split()[1] == f"s{self.gen.S_DB + 2},":
+                step += 1                                   # B's length word for the tile at k_late opens a K step
                 self.cur = stage_of_step(step)
                 self.behind_barrier = False
                 self.step = step
@@ -109,6 +120,7 @@ class Replay:
                 assert {t[1] for t in ta + tb} == {self.cur} and len({t[3] for t in ta + tb}) == 1
                 self.tail_mfma.setdefault(self.step, []).append(ta[0][3])
             elif op == "buffer_load_dword":
+                assert (f"s[{self.gen.S_DA}:" in ln) == self.mtail_form      # through A's descriptor (ragged rows) or B's
                 which, off = self.last_m0
                 assert which == "t" and not self.behind_barrier and off // 2048 == self.cur ^ 1 and off % 2048 in (0, 256)
                 self.tail_requests.append((self.step, off % 2048))
@@ -208,15 +220,18 @@ def test_the_default_make_target_builds_the_library_and_the_generated_loop_first
 
 
 @pytest.mark.parametrize("nt", [False, True], ids=["nn", "nt"])
-def test_the_ragged_columns_block_rides_along(nt):
-    """The form of the loop that also multiplies one 16 x 16 block against the ragged last columns: per K step two more
-    matrix instructions (K half 0, then 1) on fragments of the step's own stage, read and waited for, and two 256-byte
-    requests per wave into the other stage of the block's B tile, in front of the barrier; the rest of the loop as before."""
+@pytest.mark.parametrize("rows", [False, True], ids=["columns", "rows"])
+def test_the_ragged_block_rides_along(nt, rows):
+    """The forms of the loop that also multiply one 16 x 16 block against the ragged last columns (rows): per K step two
+    more matrix instructions (K half 0, then 1) on fragments of the step's own stage -- one from the whole tile's stage,
+    one from the block's own tile -- read and waited for, and two 256-byte requests per wave into the other stage of that
+    tile, in front of the barrier, through B's (A's) descriptor; the rest of the loop as before."""
     gen = load_generator(0)
-    em = gen.Emitter(nt, False, True)
+    em = gen.Emitter(nt, False, not rows, rows)
     em.loop()
     lines = [l for l in em.lines if not l.startswith("L_")]
     rp = Replay(gen, nt)
+    rp.mtail_form = rows
     rp.run(lines, stage_of_step=lambda t: t & 1)
     assert rp.step == 1
     for t in range(2):
@@ -226,6 +241,10 @@ def test_the_ragged_columns_block_rides_along(nt):
             for j in range(8):
                 assert rp.mfma_of[(t, i, j)] == [0, 1]
     assert sum(l.startswith("v_mfma") for l in lines) == 2 * (128 + 2)
+    if rows:
+        # A's length word is set before the first request that goes through it
+        first_request = next(i for i, l in enumerate(lines) if l.startswith("buffer_load_dword "))
+        assert any(l.startswith(f"s_cselect_b32 s{gen.S_DA + 2}, %[a_bytes]") for l in lines[:first_request])
     # the plain form has none of it
     plain = gen.Emitter(nt)
     plain.loop()
