@@ -351,11 +351,11 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     // per K step: 0.67 of the 256-row kernel's; an 8-bit step (128 deep) takes 1.3 of a 16-bit one, which the fixed terms
     // here (in 16-bit steps) have to be weighed against (E4M3 128 x 14336 x 4096: 31.1 us whole, 25.8 in two ranges)
     const double scale = kstep == 128u ? 0.87 / 0.67 : 1.0;
-    // a long K: the three-stage kernels, steps in threes (2048^3 28.6 -> 24.9 us, 1024 x 4096 x 4096 51.1 -> 42.0,
+    // a long K: the three-stage kernels (2048^3 28.6 -> 24.9 us, 1024 x 4096 x 4096 51.1 -> 42.0,
     // 640 x 8192 x 4096 N x K 60.4 -> 45.9)
     const bool three = h128_three_stages(s.k, kstep, half_tiles);
     // (bytes as well as steps: stream_us)
-    double whole = 8.0 + scale * h128_step(three, false, s.nt, kstep == 128u) * (three ? 3u * cdiv(nk, 3u) : nk);
+    double whole = 8.0 + scale * h128_step(three, false, s.nt, kstep == 128u) * nk;
     if (whole < stream_us(s, batch, kstep, half_tiles)) whole = stream_us(s, batch, kstep, half_tiles);
     double best = 0.9 * whole, best_cost = whole;                  // splitting has to win 10 %
     uint32_t best_ks = 1;
@@ -367,10 +367,10 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
         for (uint32_t ks = 2; ks <= kmax; ++ks) {
             if (cdiv(nk, cdiv(nk, ks)) != ks) continue;            // would leave an empty range
             if (half_tiles * ks * 131072ull > (1ull << 30)) break;
-            // (ranges long enough run on the three-stage kernels, in threes)
+            // (ranges long enough run on the three-stage kernels)
             const uint32_t r = cdiv(nk, ks);
             const bool three_r = h128_three_stages(r * kstep, kstep, half_tiles * ks);
-            const double loop = scale * h128_step(three_r, true, s.nt, kstep == 128u) * (three_r ? 3u * cdiv(r, 3u) : r);
+            const double loop = scale * h128_step(three_r, true, s.nt, kstep == 128u) * r;
             double t = 8.0 + loop + 6.0 + (1.2e-6 * elems + 0.15) * ks;
             // (bound by the stream: the partial tiles travel in its shadow, the second launch does not; and there a
             // split that brings more compute units to the stream only has to win 5 %)
@@ -1208,10 +1208,10 @@ double tail_part_cost(const maize_gemm_ex_desc_t& part, uint32_t compute_units) 
         const uint32_t ks = h128 ? h128_choice(s, 1, compute_units) : splitk_ranges(s, 1, compute_units);
         if (ks < 2u) return -1.0;
         const uint32_t r = cdiv(nk, ks);
-        const double step = h128 ? h128_step(three, true, s.nt, false) * (three ? 3u * cdiv(r, 3u) : r) : 1.0 * r;
+        const double step = h128 ? h128_step(three, true, s.nt, false) * r : 1.0 * r;
         return launch + step + 6.0 + (1.2e-6 * (double)s.m * s.n + 0.15) * ks;
     }
-    if (h128 && std::strstr(name, "_mt256_")) return launch + h128_step(three, false, s.nt, false) * (three ? 3u * cdiv(nk, 3u) : nk);
+    if (h128 && std::strstr(name, "_mt256_")) return launch + h128_step(three, false, s.nt, false) * nk;
     return -1.0;
 }
 }  // namespace

@@ -793,6 +793,20 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (uint32_t kt = 0; kt < nk; kt += 2) { step(0, 1); step(1, 1); }
     } else if (EDGE && split) {
         for (uint32_t kt = 0; kt < nk; kt += 2) { step(0, 2); step(1, 2); }
+    } else if (H128) {
+        // 128-row tiles leave half the register file free: the one or two steps that a count which is no multiple of the
+        // trip leaves over get copies of their own behind the loop, instead of the trip being padded with steps on zero
+        // tiles (the 256-row kernels have no room for a second copy of the step; their plain form has the assembly loop).
+        uint32_t kt = 0;
+        for (; kt + NST <= nk; kt += NST) {
+            step(0);
+            step(1);
+            if (R3) step(2);
+        }
+        if (kt < nk) {
+            step(0);
+            if (R3 && kt + 1u < nk) step(1);
+        }
     } else {
         for (uint32_t kt = 0; kt < nk; kt += NST) {
             step(0);

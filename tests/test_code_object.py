@@ -98,20 +98,25 @@ def test_matrix_instruction_per_kernel(kernels):
             # B is fed as the first source, so cbsz carries B's format code and blgp A's (E4M3 = 0 is not printed, E5M2 = 1).
             f8 = [i for i in ins if i.startswith("v_mfma_f32_16x16x128_f8f6f4")]
             h128 = "_h128" in name                                            # 128 x 256 tiles: half the MFMAs, one A group
-            steps = 3 if "_h128r3" in name else 2                             # K steps per trip of the loop = ring stages
+            stages = 3 if "_h128r3" in name else 2                            # K steps per trip of the loop = ring stages
+            # 128-row tiles: the steps a count that is no multiple of the trip leaves over have copies of their own behind the loop
+            steps = stages + (stages - 1 if h128 else 0)
             per = (32 if h128 else 64) * steps
             assert len(f8) == per and count(ins, "v_mfma") == per, name       # unrolled K steps of 128 elements, 64 (32) MFMAs each
             tag = name[len("maize_gemm_"):].split("_")[0]
             a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
             assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
-            body = ins[next(k for k, i in enumerate(ins) if i.startswith("v_mfma")):len(ins) - next(k for k, i in enumerate(reversed(ins)) if i.startswith("v_mfma"))]
+            # the loop proper: from the first matrix instruction to the last one of a trip (what follows are the left-over
+            # steps' copies and the epilogue, in whatever order the compiler lays the blocks out)
+            at = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
+            body = ins[at[0]:at[(32 if h128 else 64) * stages - 1] + 1]
             if "_mt256_nn" in name:
                 # row-major B: A by 128-bit reads, B by four transposing 8-byte reads per fragment
-                assert count(body, "ds_read_b128") == (8 * steps if h128 else 32) and count(body, "ds_read_b64_tr_b8") == 32 * steps, name
+                assert count(body, "ds_read_b128") == (8 * stages if h128 else 32) and count(body, "ds_read_b64_tr_b8") == 32 * stages, name
             else:
-                assert count(body, "ds_read_b128") == (24 * steps if h128 else 64) and count(body, "ds_read_b64_tr_b8") == 0, name
-            assert count(body, "buffer_load_dwordx4") == (12 * steps if h128 else 32) and count(body, "s_barrier") == steps, name
-            assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(12)" in i) == (3 if steps == 3 else 0), name
+                assert count(body, "ds_read_b128") == (24 * stages if h128 else 64) and count(body, "ds_read_b64_tr_b8") == 0, name
+            assert count(body, "buffer_load_dwordx4") == (12 * stages if h128 else 32) and count(body, "s_barrier") == stages, name
+            assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(12)" in i) == (3 if stages == 3 else 0), name
             assert count(body, "v_accvgpr") == 0 and count(body, "v_mov_b32") == 0, name     # accumulators and fragments stay in place
         elif "_mt128_" in name:
             # the catalogue's tf32 and f64 entries: full fp32 / fp64 matrix instructions; one K tile of 128 bytes
@@ -178,13 +183,14 @@ def test_main_loop_of_the_headline_kernel_is_lean(kernels):
 
 def test_main_loop_of_the_half_height_kernels_is_lean(kernels):
     """The 128 x 256 tile kernels: two unrolled K steps of 64 MFMAs per wave, one A group (8 reads per step) and two
-    B groups (16 reads, or 32 transposing ones), 12 pieces per wave and step, one barrier per step."""
+    B groups (16 reads, or 32 transposing ones), 12 pieces per wave and step, one barrier per step; behind the loop one more
+    copy of the step for an odd step count."""
     for name, reads in (("maize_gemm_bf16_mt256_nn_h128", {"ds_read_b128": 16, "ds_read_b64_tr_b16": 64}),
                         ("maize_gemm_bf16_mt256_nt_h128", {"ds_read_b128": 48})):
         ins = kernels[name]
         idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
-        assert len(idx) == 128 and count(ins, "v_mfma_f32_16x16x32_bf16") == 128
-        body = ins[idx[0]:idx[-1] + 1]
+        assert len(idx) == 192 and count(ins, "v_mfma_f32_16x16x32_bf16") == 192
+        body = ins[idx[0]:idx[127] + 1]                                # the loop proper: the first two steps
         # (the row-major B's descriptor is re-based per K tile and cut at 2 GiB: the compiler does that one 64-bit compare,
         # for which there is no scalar instruction, on the vector unit -- one uniform compare per K step)
         extra = [i for i in body if not i.startswith(("v_mfma", "ds_read", "buffer_load_dwordx4", "s_", "v_cmp_lt_u64"))]
@@ -195,18 +201,19 @@ def test_main_loop_of_the_half_height_kernels_is_lean(kernels):
         assert count(body, "s_waitcnt") <= 8
     for name in ("maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_f16_mt256_nt_h128_gen", "maize_gemm_bf16_mt256_nt_h128_splitk", "maize_gemm_f16_mt256_nn_h128_splitk"):
         want = "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16"
-        assert count(kernels[name], want) == 128 and count(kernels[name], "v_mfma") == 128, name
+        assert count(kernels[name], want) == 192 and count(kernels[name], "v_mfma") == 192, name
 
 
 def test_main_loop_of_the_three_stage_kernels_is_lean(kernels):
     """The 128 x 256 tile kernels with three ring stages: three unrolled K steps of 64 MFMAs, the same reads and requests
-    per step as the two-stage loop, one barrier per step, and a counted wait that leaves twelve requests in flight."""
+    per step as the two-stage loop, one barrier per step, and a counted wait that leaves twelve requests in flight; behind
+    the loop two more copies of the step for a step count that is no multiple of three."""
     for name, reads in (("maize_gemm_bf16_mt256_nn_h128r3", {"ds_read_b128": 24, "ds_read_b64_tr_b16": 96}),
                         ("maize_gemm_bf16_mt256_nt_h128r3", {"ds_read_b128": 72})):
         ins = kernels[name]
         idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
-        assert len(idx) == 192 and count(ins, "v_mfma_f32_16x16x32_bf16") == 192
-        body = ins[idx[0]:idx[-1] + 1]
+        assert len(idx) == 320 and count(ins, "v_mfma_f32_16x16x32_bf16") == 320
+        body = ins[idx[0]:idx[191] + 1]                                # the loop proper: the first three steps
         extra = [i for i in body if not i.startswith(("v_mfma", "ds_read", "buffer_load_dwordx4", "s_", "v_cmp_lt_u64"))]
         assert not extra and count(body, "v_cmp_lt_u64") <= 3, extra[:5]
         for mnemonic, n in reads.items():
@@ -216,7 +223,7 @@ def test_main_loop_of_the_three_stage_kernels_is_lean(kernels):
         assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(12)" in i) == 3, name
     for name in ("maize_gemm_bf16_mt256_nn_h128r3_gen", "maize_gemm_f16_mt256_nt_h128r3_gen", "maize_gemm_f16_mt256_nn_h128r3_gen", "maize_gemm_bf16_mt256_nt_h128r3_gen"):
         want = "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16"
-        assert count(kernels[name], want) == 192 and count(kernels[name], "v_mfma") == 192, name
+        assert count(kernels[name], want) == 320 and count(kernels[name], "v_mfma") == 320, name
 
 
 
@@ -232,7 +239,15 @@ def test_no_k_loop_wraps_its_requests_in_scalarising_loops(kernels):
             continue
         idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
         body = ins[idx[0]:idx[-1] + 1]
-        assert count(body, "s_and_saveexec") == 0 and count(body, "s_cbranch_exec") == 0, name
-        assert count(body, "v_readfirstlane") <= 12, (name, count(body, "v_readfirstlane"))
-        assert count(body, "s_cbranch") <= 1, name
+        # (the 128-row kernels: behind the loop come one or two more copies of the step for the steps a trip leaves over, each
+        # under a uniform branch of its own, and the epilogue may be laid out among them)
+        h128 = "_h128" in name
+        trip = (32 if name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")) else 64) * (3 if "_h128r3" in name else 2)
+        loop = ins[idx[0]:idx[trip - 1] + 1] if h128 else body
+        assert count(loop, "s_and_saveexec") == 0 and count(loop, "s_cbranch_exec") == 0, name
+        assert count(loop, "v_readfirstlane") <= 12, (name, count(loop, "v_readfirstlane"))
+        assert count(loop, "s_cbranch") <= 1, name
+        if h128:
+            copies = 5 if "_h128r3" in name else 3
+            assert count(body, "v_readfirstlane") <= 4 * copies + 4 and count(body, "s_and_saveexec") <= 2, name
         assert count(ins, "s_bfe_i64") == 0, name
