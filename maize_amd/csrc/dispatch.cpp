@@ -321,17 +321,21 @@ uint32_t splitk_ranges(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kst
 // half tiles costs 0.63 of a round of whole ones, 4096^3 89 -> 112 us, 2048 x 11008 x 4096 152 -> 162).
 // With few of them and a long K the 128-row tiles are cut over K too (same cost terms as above with 0.67 per K step: a
 // single row of tiles, 65 .. 128 rows of A, does half the matrix work of 256-row tiles).
-// Whole K in 128-row tiles: from 28 K steps of 16-bit operands on, the kernels with three ring stages (below that their
-// longer start and the step count rounded up to a multiple of three cost more than the two-stage loop's waits:
-// 512 x 8192 x 1024 14.5 us with two stages, 15.8 with three; 512 x 2048 x 1536 17.5 / 18.0) -- provided enough compute
+// Whole K in 128-row tiles: from 16 K steps of 16-bit operands on, the kernels with three ring stages (below that their
+// longer start costs more than the two-stage loop's waits) -- provided enough compute
 // units pull on the memory system for those waits to exist (32 tiles, 512 x 2048 x 1792: 19.7 us with two stages, 21.2
 // with three, 0.55 us per step either way; 112 to 224 tiles: 0.70 against 0.52 per step) or K is long enough for the
 // rounding not to matter.
-bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles) {
+bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles, bool range = false) {
     const uint32_t nk = cdiv(k, kstep);                         // (an 8-bit step, 128 deep, is as long as a 16-bit one)
     // 8-bit operands: from 18 steps (E4M3 N x K, two -> three stages: 1024 x 4096 x 2560 21.3 -> 19.4 us, x 4096 31.1 -> 25.4,
     // 768 x 8192 x 8192 58.8 -> 46.7; 2048^3, 16 steps: 17.5 either way)
-    return nk >= (kstep == 128u ? 18u : 28u) && (nk >= 48u || half_tiles >= 48u);
+    // (16-bit: 28 steps while a step count that was no multiple of three was padded; without the padding three stages tie at
+    // 16 steps and win from 20 -- 1024 x 4096 x K, K = 1024 / 1280 / 1536 / 1792: 15.2 / 18.2 / 23.5 / 26.2 us on two stages,
+    // 14.9 / 17.2 / 19.7 / 21.7 on three; 32 tiles, 512 x 2048 x K: level throughout)
+    // (K ranges of a split: from 28 steps, as measured with the split kernels -- at 16 steps per range the two rings tie:
+    // 512 x 4096 x 4096 in four ranges 34.5 / 34.4 us)
+    return nk >= (kstep == 128u ? 18u : range ? 28u : 16u) && (nk >= 48u || half_tiles >= 48u);
 }
 // What a K step of a 128-row tile costs, in steps of the 256-row kernel at the power limit (~ microseconds): 0.67 on two
 // ring stages, 0.52 on three; K ranges of a row-major 16-bit B on three stages 0.55 (same plans, same box, K x N against
@@ -369,7 +373,7 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
             if (half_tiles * ks * 131072ull > (1ull << 30)) break;
             // (ranges long enough run on the three-stage kernels)
             const uint32_t r = cdiv(nk, ks);
-            const bool three_r = h128_three_stages(r * kstep, kstep, half_tiles * ks);
+            const bool three_r = h128_three_stages(r * kstep, kstep, half_tiles * ks, true);
             const double loop = scale * h128_step(three_r, true, s.nt, kstep == 128u) * r;
             double t = 8.0 + loop + 6.0 + (1.2e-6 * elems + 0.15) * ks;
             // (bound by the stream: the partial tiles travel in its shadow, the second launch does not; and there a
@@ -1102,7 +1106,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
                                                          {"maize_gemm_f16_mt256_nn_h128_splitk", "maize_gemm_f16_mt256_nt_h128_splitk"}},
                                                         {{"maize_gemm_bf16_mt256_nn_h128r3_splitk", "maize_gemm_bf16_mt256_nt_h128r3_splitk"},
                                                          {"maize_gemm_f16_mt256_nn_h128r3_splitk", "maize_gemm_f16_mt256_nt_h128r3_splitk"}}};
-        const int r3 = h128_three_stages(cdiv(cdiv(s.k, 64u), hk) * 64u, 64u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk);
+        const int r3 = h128_three_stages(cdiv(cdiv(s.k, 64u), hk) * 64u, 64u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk, true);
         const int hs = kernel_index(kH128Split[r3][half_in(d)][s.nt]);
         if (hs >= 0 && kKernels[hs].supports(d) && plan_fits(kKernels[hs], d, compute_units)) return (uint32_t)hs;
     }

@@ -272,9 +272,9 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
     p = mz.gemm_plan(desc(640, 8192, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3" and p["grid"] == (160, 1, 1)
     assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"
-    assert mz.gemm_plan(desc(512, 8192, 1024), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"         # 16 K steps: the two-stage loop (14.5 us against 15.8)
-    assert mz.gemm_plan(desc(1024, 4096, 1728), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"        # 27 steps
-    assert mz.gemm_plan(desc(1024, 4096, 1792), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"      # 28 steps, 128 tiles
+    assert mz.gemm_plan(desc(512, 8192, 960), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"          # 15 K steps: the two-stage loop
+    assert mz.gemm_plan(desc(512, 8192, 1024), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"       # 16 steps: three stages (15.2 -> 14.6 us now that no step is padded)
+    assert mz.gemm_plan(desc(1024, 4096, 1536), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"      # 24 steps, 128 tiles: 23.5 -> 19.7 us
     assert mz.gemm_plan(desc(512, 2048, 1792), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"         # 32 tiles: too few to make the loads wait
     # K ranges of 28 steps or more run on the three-stage kernels too, whichever way B is stored (a row-major B costs
     # them 3-7 % more per step, not the 60 % it was once priced at)
