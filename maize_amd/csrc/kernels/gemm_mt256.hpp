@@ -157,6 +157,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     static_assert(!(NTAIL || MTAIL) || ASM, "ragged last columns or rows ride along in the assembly K loop only");
     static_assert(!(NTAIL && MTAIL), "ragged columns or ragged rows, not both");
     constexpr bool RTAIL = NTAIL || MTAIL;
+    // 256-row kernels with the general epilogue (alpha / beta, fp32 C, K ranges): their allocation leaves room for a second
+    // copy of the K step, the plain kernels' does not (132-364 bytes of scratch when tried; their odd step counts go to
+    // the assembly loop instead)
+    constexpr bool PEEL256 = BMT == 256 && GEN && !EDGE && !ASM;
     constexpr bool H128 = BMT == 128;
     static_assert(BMT == 256 || (H128 && !EDGE), "128-row tiles: no edge splitting");
     constexpr bool R3 = NST == 3;                       // three ring stages (128-row tiles)
@@ -793,10 +797,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (uint32_t kt = 0; kt < nk; kt += 2) { step(0, 1); step(1, 1); }
     } else if (EDGE && split) {
         for (uint32_t kt = 0; kt < nk; kt += 2) { step(0, 2); step(1, 2); }
-    } else if (H128) {
+    } else if (H128 || PEEL256) {
         // 128-row tiles leave half the register file free: the one or two steps that a count which is no multiple of the
         // trip leaves over get copies of their own behind the loop, instead of the trip being padded with steps on zero
-        // tiles (the 256-row kernels have no room for a second copy of the step; their plain form has the assembly loop).
+        // tiles.  The same for the 256-row kernels that have the room (PEEL256).
         uint32_t kt = 0;
         for (; kt + NST <= nk; kt += NST) {
             step(0);

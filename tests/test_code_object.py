@@ -99,8 +99,10 @@ def test_matrix_instruction_per_kernel(kernels):
             f8 = [i for i in ins if i.startswith("v_mfma_f32_16x16x128_f8f6f4")]
             h128 = "_h128" in name                                            # 128 x 256 tiles: half the MFMAs, one A group
             stages = 3 if "_h128r3" in name else 2                            # K steps per trip of the loop = ring stages
-            # 128-row tiles: the steps a count that is no multiple of the trip leaves over have copies of their own behind the loop
-            steps = stages + (stages - 1 if h128 else 0)
+            # 128-row tiles, and 256-row tiles with the general epilogue (alpha / beta, fp32 C, K ranges): the steps a count that is
+            # no multiple of the trip leaves over have copies of their own behind the loop
+            peeled = h128 or name.endswith(("_gen", "_splitk"))
+            steps = stages + (stages - 1 if peeled else 0)
             per = (32 if h128 else 64) * steps
             assert len(f8) == per and count(ins, "v_mfma") == per, name       # unrolled K steps of 128 elements, 64 (32) MFMAs each
             tag = name[len("maize_gemm_"):].split("_")[0]
@@ -242,12 +244,13 @@ def test_no_k_loop_wraps_its_requests_in_scalarising_loops(kernels):
         # (the 128-row kernels: behind the loop come one or two more copies of the step for the steps a trip leaves over, each
         # under a uniform branch of its own, and the epilogue may be laid out among them)
         h128 = "_h128" in name
-        trip = (32 if name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")) else 64) * (3 if "_h128r3" in name else 2)
-        loop = ins[idx[0]:idx[trip - 1] + 1] if h128 else body
+        peeled = h128 or name.endswith(("_gen", "_splitk"))
+        trip = (32 if name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")) else 64) * (1 if h128 else 2) * (3 if "_h128r3" in name else 2)
+        loop = ins[idx[0]:idx[trip - 1] + 1] if peeled else body
         assert count(loop, "s_and_saveexec") == 0 and count(loop, "s_cbranch_exec") == 0, name
         assert count(loop, "v_readfirstlane") <= 12, (name, count(loop, "v_readfirstlane"))
         assert count(loop, "s_cbranch") <= 1, name
-        if h128:
+        if peeled:
             copies = 5 if "_h128r3" in name else 3
             assert count(body, "v_readfirstlane") <= 4 * copies + 4 and count(body, "s_and_saveexec") <= 2, name
         assert count(ins, "s_bfe_i64") == 0, name
