@@ -18,6 +18,13 @@ Everything else (address registers, per-piece offsets, descriptors' words, LDS b
 What this buys over the statement-by-statement loop: the trip can be left after its first step (an odd step
 count no longer runs a step on a zero tile), and side work can be given registers of its own.
 
+Forms written out (functions of kloop_gen.inc), each for B stored N x K (nt) and K x N (nn):
+  kloop_asm_{nt,nn}          the plain loop
+  kloop_asm_{nt,nn}_ntail    ... that also multiplies one 16 x 16 block against up to sixteen ragged last columns of B and C
+  kloop_asm_{nt,nn}_mtail    ... against up to sixteen ragged last rows of A and C (Emitter.tail_*)
+  kloop_asm_{nt,nn}_drain    (only with KLOOP_DRAIN_STEPS=n in the environment) ... that stores the previous C tile from
+                             registers during its first n steps (Emitter.drain_side_work): measured slower, not built by default
+
 Usage: gen_kloop.py OUT.inc
 """
 import os
