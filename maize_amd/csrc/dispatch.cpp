@@ -333,9 +333,10 @@ bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles, bool ran
     // (16-bit: 28 steps while a step count that was no multiple of three was padded; without the padding three stages tie at
     // 16 steps and win from 20 -- 1024 x 4096 x K, K = 1024 / 1280 / 1536 / 1792: 15.2 / 18.2 / 23.5 / 26.2 us on two stages,
     // 14.9 / 17.2 / 19.7 / 21.7 on three; 32 tiles, 512 x 2048 x K: level throughout)
-    // (K ranges of a split: from 28 steps, as measured with the split kernels -- at 16 steps per range the two rings tie:
-    // 512 x 4096 x 4096 in four ranges 34.5 / 34.4 us)
-    return nk >= (kstep == 128u ? 18u : range ? 28u : 16u) && (nk >= 48u || half_tiles >= 48u);
+    // (K ranges of a split, every candidate by name on 96 mid-size shapes: three stages win from 13 steps per range --
+    // 256 x 4096 x 4096 in five ranges 26.1 -> 24.7 us, 512 x 2048 x 8192 in eight ranges of 16 steps 37.4 -> 33.2,
+    // 384 x 4096 x 4096 in four 31.4 -> 29.2)
+    return nk >= (kstep == 128u ? 18u : range ? 12u : 16u) && (nk >= 48u || half_tiles >= 48u);
 }
 // What a K step of a 128-row tile costs, in steps of the 256-row kernel at the power limit (~ microseconds): 0.67 on two
 // ring stages, 0.52 on three; K ranges of a row-major 16-bit B on three stages 0.55 (same plans, same box, K x N against

@@ -222,16 +222,16 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3",      # 64 tiles: partial tiles would cost more than they save, 128 tiles of 128 rows fill half the chip (32 K steps: three ring stages)
         (512, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3",      # 112 tiles: 224 of 128 rows are one round
-        (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128_splitk",  # few tiles, a long K: 128-row tiles cut over K
+        (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3_splitk",  # few tiles, a long K: 128-row tiles cut over K (ranges of 16 steps: three stages)
         (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128_splitk",
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",              # N x K weights streamed once
         (16, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",
         (17, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m32",          # 17 .. 32 rows: two row groups
         (64, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m64",         # 33 .. 64 rows and many slabs: four
-        (65, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128_splitk",  # more than 64 rows
+        (65, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128r3_splitk",  # more than 64 rows
         (32, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn_m32",
         (64, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn_m64",
-        (64, 8192, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128_splitk",   # 64 rows, 32 slabs: the tile kernel cut over K
+        (64, 8192, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3_splitk", # 64 rows, 32 slabs: the tile kernel cut over K
         (33, 17, 65, mz.LAYOUT_NN, 1): "maize_gemm_bf16_wave32",
         (4096, 4099, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_splitk",      # odd N: operands read where they lie, C written element-wise by the reduce pass
         (1000, 50257, 768, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_splitk",
@@ -266,7 +266,7 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
     p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)                  # 112 tiles of 128 rows: whole K on three ring stages
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3" and p["ksplit"] == 1 and p["grid"] == (112, 1, 1)
     p = mz.gemm_plan(desc(128, 14336, 4096), compute_units=CUS)                  # one row of tiles: cut over K (38 us against 54.7 whole)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and p["ksplit"] == 4 and p["grid"] == (224, 1, 1)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and p["ksplit"] == 4 and p["grid"] == (224, 1, 1)   # (ranges of 16 steps: three stages)
     p = mz.gemm_plan(desc(768, 8192, 8192), compute_units=CUS)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3" and p["ksplit"] == 1 and p["grid"] == (192, 1, 1)
     p = mz.gemm_plan(desc(640, 8192, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)
@@ -289,8 +289,8 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
         nn_plan = mz.gemm_plan(desc(m, n, k), kernel="maize_gemm_bf16_mt256_nn_h128r3_splitk", compute_units=CUS)
         nt_plan = mz.gemm_plan(desc(m, n, k, layout=mz.LAYOUT_NT), kernel="maize_gemm_bf16_mt256_nt_h128r3_splitk", compute_units=CUS)
         assert nn_plan["ksplit"] == nt_plan["ksplit"] and nn_plan["grid"] == nt_plan["grid"], (m, n, k, nn_plan, nt_plan)
-    p = mz.gemm_plan(desc(384, 6144, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)        # (35 us; whole 39)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3_splitk" and p["ksplit"] == 2 and p["grid"] == (144, 1, 1)
+    p = mz.gemm_plan(desc(384, 6144, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)        # (three ranges 33 us; two 35; whole 39)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3_splitk" and p["ksplit"] == 3 and p["grid"] == (216, 1, 1)
     assert mz.gemm_plan(desc(4096, 2304, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"       # 288 tiles of 128 rows would need two rounds
     assert mz.gemm_plan(desc(1024, 14336, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"   # 224 tiles: one round as it is
 
@@ -445,8 +445,8 @@ def _steps_of_the_ranges(k, ksplit):
 def test_the_named_three_stage_cases_have_a_ragged_m_and_a_step_count_off_three():
     """The GPU suite runs the three-stage 128-row kernels by name (tests/test_gpu_random_products.py: H128R3_CASES).  Here,
     without a device: each kernel accepts its case, M is no multiple of 128, and some K range runs a number of steps
-    that is no multiple of three (the loop runs three steps per trip and pads with zero tiles); both layouts, the plain,
-    general and split-K forms are all there."""
+    that is no multiple of three (the loop runs three steps per trip; the steps left over run on copies of the step behind
+    it); both layouts, the plain, general and split-K forms are all there."""
     from tests.test_gpu_random_products import H128R3_CASES
     for name, layout, m, n, k, kw in H128R3_CASES:
         brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)

@@ -81,11 +81,11 @@ def test_dispatch_of_extended_descriptors():
     for kw in (dict(alpha=0.5, beta=2.0), dict(out_type=mz.OUT_F32), dict(ldb=14400, ldc=14344)):
         assert mz.gemm_plan(ex(16, 14336, 4096, **kw))["kernel"] == "maize_gemm_bf16_skinny_nn"
     assert mz.gemm_plan(ex(16, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_skinny_nn"   # rows of B on 8-byte boundaries: still streamed
-    assert mz.gemm_plan(ex(16, 14336, 4096, lda=4100))["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk"   # rows of A off the 16-byte grid: the macro-tile kernels read them where they lie
+    assert mz.gemm_plan(ex(16, 14336, 4096, lda=4100))["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk"   # rows of A off the 16-byte grid: the macro-tile kernels read them where they lie
     assert mz.gemm_plan(ex(32, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_skinny_nn_m32"     # 17 .. 64 rows: the same stream with more row groups
     assert mz.gemm_plan(ex(64, 14336, 4096))["kernel"] == "maize_gemm_bf16_skinny_nn_m64"
     assert mz.gemm_plan(ex(64, 4096, 4096))["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk"          # few slabs: the tile kernel (128-row tiles) cut over K is faster
-    assert mz.gemm_plan(ex(65, 14336, 4096))["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk"
+    assert mz.gemm_plan(ex(65, 14336, 4096))["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk"
 
 
 def _supports(name, x):
@@ -286,7 +286,7 @@ def test_tail_split_by_rows():
     assert mz.gemm_tail_rows(x) == 16 * 256 and mz.gemm_tail_split(x) == (16 * 256, 0)
     top, rest = ex(16 * 256, 4096, 4096), ex(256, 4096, 4096)
     assert mz.gemm_plan(top)["kernel"] == "maize_gemm_bf16_mt256_nn" and mz.gemm_plan(top)["grid"] == (256, 1, 1)
-    assert mz.gemm_plan(rest)["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and mz.gemm_plan(rest)["ksplit"] >= 2
+    assert mz.gemm_plan(rest)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and mz.gemm_plan(rest)["ksplit"] >= 2
     assert mz.gemm_tail_rows(ex(4352, 4096, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_F16, beta=1.0)) == 16 * 256
     # ... or by columns, where that leaves the cheaper part: 16 x 17 tiles = a full round of 16 tile columns and one more
     assert mz.gemm_tail_split(ex(4096, 4352, 4096)) == (0, 16 * 256) and mz.gemm_tail_rows(ex(4096, 4352, 4096)) == 0
