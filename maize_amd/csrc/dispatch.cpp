@@ -249,6 +249,17 @@ bool mt256_h128_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Laun
     return true;
 }
 bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
+// 128 x 128 tiles (maize_gemm_bf16_t128_*): one workgroup per tile of the flattened (batch, tile) list.
+bool t128_plan(const maize_gemm_ex_desc_t& d, uint32_t, LaunchDims* ld) {
+    const Dims s = dims_of(d);
+    const uint64_t all = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128) * d.gemm.batch;
+    if (all == 0 || all > 0x7FFFFFFFull) return false;
+    ld->grid[0] = (uint32_t)all;
+    ld->grid[1] = 1; ld->grid[2] = 1;
+    ld->block[0] = 256; ld->block[1] = 1; ld->block[2] = 1;
+    ld->lds_bytes = 0; ld->ksplit = 1; ld->split_first = 0; ld->reduce_grid = 0; ld->workspace_bytes = 0;
+    return true;
+}
 // ... over the whole tile columns (rows) only: the ragged last columns (rows) have no tiles of their own
 bool ragged_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, bool rows, LaunchDims* ld) {
     const Dims s = dims_of(d);
@@ -346,12 +357,14 @@ bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles, bool ran
 // the figure looking true.)
 double h128_step(bool three, bool split, bool nt, bool bits8) { return !three ? 0.67 : (split && !nt && !bits8) ? 0.55 : 0.52; }
 // Returns 0: the 256-row kernels; 1: 128-row tiles, whole K; >= 2: 128-row tiles in that many K ranges.
-uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64) {
+// `cost` (optional): what the model expects of the choice it returns.
+uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep = 64, double* cost = nullptr) {
     const uint32_t resident = cus >= 8u ? cus - cus % 8u : cus;
     const uint64_t half_tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * batch;
-    if (resident == 0 || half_tiles > resident || s.k < 128u) return 0;
     double other = 0.0;
     (void)splitk_ranges(s, batch, cus, kstep, &other);
+    if (cost) *cost = other;
+    if (resident == 0 || half_tiles > resident || s.k < 128u) return 0;
     const uint32_t nk = cdiv(s.k, kstep);
     // per K step: 0.67 of the 256-row kernel's; an 8-bit step (128 deep) takes 1.3 of a 16-bit one, which the fixed terms
     // here (in 16-bit steps) have to be weighed against (E4M3 128 x 14336 x 4096: 31.1 us whole, 25.8 in two ranges)
@@ -390,7 +403,17 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     // so with 8-bit operands, whose fixed terms it overrates: E4M3 N x K, 46 mid-size shapes with every candidate by name,
     // the two it gave to the 256-row split were both faster in tiles -- 256 x 2048 x 2048 18.5 against 14.3-15.9 us,
     // 768 x 4096 x 14336 55.4 against 50.1)
-    return best < (kstep == 128u ? 1.10 : 1.03) * other ? best_ks : 0u;
+    const bool tiles = best < (kstep == 128u ? 1.10 : 1.03) * other;
+    if (cost && tiles) *cost = best;
+    return tiles ? best_ks : 0u;
+}
+// 128 x 128 tiles (maize_gemm_bf16_t128_*), one round of them: what a K step costs in the same units.  N x K 0.34, K x N
+// (transposing reads) 0.42; 0.02 more from 129 tiles and 0.05 more from 193 (the compute units share the path from the
+// L2s), 0.04 more from 128 steps.  Every candidate by name on 54 products per layout, one box, N x K / K x N:
+// 512 x 4096 x 4096 30.6 / 35.6 us, 768 x 4096 x 4096 31.3 / 36.1, 1024 x 4096 x 4096 34.3 / 37.8, 512 x 8192 x 8192 63.5 / 70.7,
+// 1024 x 4096 x 14336 110.6 / 129.2 -- where the three-stage 128 x 256 tiles' 0.52 measures 0.51.
+double t128_step(bool nt, uint64_t tiles, uint32_t nk) {
+    return (nt ? 0.34 : 0.42) + (tiles > 192u ? 0.05 : tiles > 128u ? 0.02 : 0.0) + (nk >= 128u ? 0.04 : 0.0);
 }
 bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && bf16_in(d); }
 bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && bf16_in(d); }
@@ -919,6 +942,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_skinny_nn", nullptr, skinny_nn_supports, skinny_plan},
     {"maize_gemm_bf16_skinny_nn_m32", nullptr, skinny_nn_m32_supports, skinny_m32_plan},
     {"maize_gemm_bf16_skinny_nn_m64", nullptr, skinny_nn_m64_supports, skinny_m64_plan},
+    {"maize_gemm_bf16_t128_nn", nullptr, mt256_nn_gen_supports, t128_plan},
+    {"maize_gemm_bf16_t128_nt", nullptr, mt256_nt_gen_supports, t128_plan},
     {"maize_gemm_bf16_mt256_nn_gen", nullptr, mt256_nn_gen_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_gen", nullptr, mt256_nt_gen_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_ktail_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_plan},
@@ -1101,7 +1126,31 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
                                               {"maize_gemm_f16_mt256_nn_splitk", "maize_gemm_f16_mt256_nt_splitk"}};
     const int si = kernel_index(kSplitK[half_in(d)][s.nt]);
     // ... or, where that is faster, compute it in 128-row tiles (the kernels that store C themselves: 16-byte rows of C).
-    const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units);
+    double cost_hk = 0.0;
+    const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units, 64u, &cost_hk);
+    // ... or in 128 x 128 tiles, when one round of them beats both by the model (four times the 256 x 256 tiles: a
+    // product that fills half the compute units or less in 128 x 256 tiles has the whole chip work on it without a cut
+    // over K -- 1024 x 4096 x 4096 N x K: 40.7 us in 128 x 256 tiles on three stages, 34.3 here; 768 x 4096 x 4096 37.5 ->
+    // 31.3; 2048^3 23.1 -> 20.2; 256 x 14336 x 4096 39.8 -> 32.7; K x N 40.9 -> 37.8, 38.8 -> 36.1, 23.5 -> 22.0, 39.6 -> 36.6.
+    // Not with a long K and few tiles, where the cut over K wins: 1024 x 2048 x 8192 44.6 against 56.1, 256 x 4096 x 4096
+    // 23.4 against 29.6.)
+    {
+        static const char* const kT128[2] = {"maize_gemm_bf16_t128_nn", "maize_gemm_bf16_t128_nt"};
+        const int t8 = kernel_index(kT128[s.nt]);
+        const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+        const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128) * d.gemm.batch;
+        if (t8 >= 0 && !half_in(d) && s.k >= 128u && tiles <= units && kKernels[t8].supports(d)) {
+            double cost_t = 8.0 + t128_step(s.nt, tiles, cdiv(s.k, 64u)) * cdiv(s.k, 64u);
+            const double st = stream_us(s, d.gemm.batch, 64u, tiles);
+            const bool by_stream = cost_t < st;
+            if (by_stream) cost_t = st;
+            // (against a cut over K it has to win 8 % by the model, which prices the cuts of small C a little high:
+            // 384 x 4096 x 4096 N x K in four ranges 27.2 us measured, 30.4 by the model, 30.0 here; not where both are
+            // bound by the operands' stream from HBM and the cut only adds its second launch: 128 x 28672 x 8192 N x K
+            // 119.7 us in two ranges, 107.4 here, K x N 99.2 / 97.9)
+            if (cost_t < (hk >= 2u && !by_stream ? 0.92 : 0.97) * cost_hk) return (uint32_t)t8;
+        }
+    }
     if (hk >= 2u) {
         static const char* const kH128Split[2][2][2] = {{{"maize_gemm_bf16_mt256_nn_h128_splitk", "maize_gemm_bf16_mt256_nt_h128_splitk"},
                                                          {"maize_gemm_f16_mt256_nn_h128_splitk", "maize_gemm_f16_mt256_nt_h128_splitk"}},

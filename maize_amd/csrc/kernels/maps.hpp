@@ -87,6 +87,19 @@ MAIZE_MAP uint32_t sk_tr_offset(uint32_t cg, uint32_t h, uint32_t lane) {
     return sk_offset(sk_tr_row(h, lane), col >> 3) + (col & 7u) * 2u;
 }
 
+// ---- K x N operand tile of the 128 x 128 kernel (row-major B): 64 rows of 256 B (128 columns), 16 pieces ---------
+// Piece p (4 rows, 1 KiB): lane l lands at row 4p + l/16, position l%16.  The same 32-byte granules and the same
+// f(row) as above (eight granules per row, f = 0..7): the eight rows a 32-lane pass of a transposing read touches
+// (row%4 and bit 3 vary) spread over all 64 banks.  K half kh and register half h of a read sit 8192 kh + 1024 h bytes
+// behind (0, 0).
+MAIZE_MAP uint32_t sk128_piece_row(uint32_t piece, uint32_t lane) { return piece * 4u + (lane >> 4); }
+MAIZE_MAP uint32_t sk128_piece_chunk(uint32_t piece, uint32_t lane) { return (lane & 15u) ^ (sk_swizzle(sk128_piece_row(piece, lane)) << 1); }
+MAIZE_MAP uint32_t sk128_offset(uint32_t row, uint32_t chunk) { return row * 256u + ((chunk ^ (sk_swizzle(row) << 1)) * 16u); }
+MAIZE_MAP uint32_t sk128_tr_offset(uint32_t cg, uint32_t h, uint32_t lane) {
+    const uint32_t col = cg * 16u + (lane & 3u) * 4u;
+    return sk128_offset(sk_tr_row(h, lane), col >> 3) + (col & 7u) * 2u;
+}
+
 // ---- The ragged last columns of a K x N / N x K B riding along in the macro-tile K loop: a 64 x 16 tile (2 KiB) ----
 // Brought in by 4-byte-per-lane requests of 256 bytes, two per wave (request q = 2 wave + j, 0..7), landing linearly.
 // K x N: 64 rows of 32 bytes (columns 0..15), no swizzle; request q covers rows 8 q .. + 7: lane l fetches row

@@ -51,6 +51,8 @@ F8_128x256 = TileTy("F8_128x256", 128, 256, 1, "kn16")        # B stage of a row
 BF16_128x64 = TileTy("BF16_128x64", 128, 64, 2, "kc16")
 F16_128x64 = TileTy("F16_128x64", 128, 64, 2, "kc16")
 F8_128x128 = TileTy("F8_128x128", 128, 128, 1, "kc16")
+# B stage of the 128 x 128 tile kernels for a row-major K x N B (stored N x K, their B stage is BF16_128x64 like their A stage)
+BF16_64x128 = TileTy("BF16_64x128", 64, 128, 2, "kn32")
 
 
 @dataclass(frozen=True)
@@ -288,15 +290,24 @@ def gemm_smem_multibuffer(mma, ktile, a_panel, b_panel, smem, cp_group, cp_size)
         # The mainloop is generic in the panel height and the ring depth, like the reference's ([TilePair; PIPE],
         # KTile<N>, gemm/mod.rs:37-45), within what kernels exist: 256- or 128-row panels of A on a two-stage ring,
         # 128-row panels also on three stages (the stage of a 128 x 256 tile is 48 KiB: three fit the 160 KiB of LDS).
-        if a_panel.rows not in (256, 128) or (b_panel.rows if nt else b_panel.cols) != 256:
-            raise ValueError("the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B)")
-        if smem is None or smem.depth not in (2, 3):
+        b_cols = b_panel.rows if nt else b_panel.cols
+        # ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages,
+        # bf16 operands.
+        quarter = a_panel.rows == 128 and b_cols == 128
+        if a_panel.rows not in (256, 128) or b_cols not in (256, 128) or (b_cols == 128 and not quarter):
+            raise ValueError("the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B), or 128 rows and 128 columns")
+        if quarter:
+            if mma.in_type != _ffi.IN_BF16:
+                raise ValueError("the 128 x 128 tile kernels take bf16 operands")
+            if smem is None or smem.depth != 4:
+                raise ValueError("the 128 x 128 tile kernels run a ring of four stages")
+        elif smem is None or smem.depth not in (2, 3):
             raise ValueError("the macro-tile kernels run a ring of two or three stages")
         if smem.depth == 3 and a_panel.rows != 128:
             raise ValueError("three ring stages fit the LDS with 128-row panels of A only")
         es = 1 if mma.k_tile == 128 else 2
         want_a = (a_panel.rows, mma.k_tile, es, "kc16")
-        want_b = (256, mma.k_tile, es, "kc16") if nt else (mma.k_tile, 256, es, "kn32" if es == 2 else "kn16")
+        want_b = (b_cols, mma.k_tile, es, "kc16") if nt else (mma.k_tile, b_cols, es, "kn32" if es == 2 else "kn16")
         for which, tile, want in (("A", smem.pair.a, want_a), ("B", smem.pair.b, want_b)):
             t = tile.ty
             if (t.rows, t.cols, t.elem_bytes, t.swizzle) != want:
@@ -306,6 +317,7 @@ def gemm_smem_multibuffer(mma, ktile, a_panel, b_panel, smem, cp_group, cp_size)
         if smem is not None:
             raise ValueError(f"{mma.name} is the any-shape kernel's instruction: operands go straight from global memory, no ring")
     op = dict(mma=mma, a=a_panel, b=b_panel, nt=nt, panel_rows=a_panel.rows if mma.family == "mt256" else None,
+              panel_cols=(b_panel.rows if nt else b_panel.cols) if mma.family == "mt256" else None,
               pipe=smem.depth if smem is not None else None)
     return Accum(kernel, op)
 
@@ -349,7 +361,7 @@ _TYPE_TAG = {_ffi.IN_BF16: "bf16", _ffi.IN_F16: "f16", _ffi.IN_E4M3: "e4m3", _ff
              _ffi.IN_E4M3_E5M2: "e4m3e5m2", _ffi.IN_E5M2_E4M3: "e5m2e4m3"}
 
 
-def described_kernel(desc, mma, nt, panel_rows, pipe, compute_units):
+def described_kernel(desc, mma, nt, panel_rows, pipe, compute_units, panel_cols=256):
     """The kernel that a description of the mainloop (panel height of A, ring depth) names for `desc`, or None when
     the dispatcher's own choice already is of that family.  A description is honoured wherever a kernel of its family
     accepts the descriptor -- also where the dispatcher by itself would rather take another family (128-row tiles for
@@ -357,8 +369,12 @@ def described_kernel(desc, mma, nt, panel_rows, pipe, compute_units):
     from .api import MaizeError
     chosen = gemm_plan(desc, compute_units=compute_units)["kernel"]
     base = f"maize_gemm_{_TYPE_TAG[mma.in_type]}_mt256_{'nt' if nt else 'nn'}"
-    if panel_rows == 256:
-        if "_h128" not in chosen:
+    if panel_cols == 128:                              # 128 x 128 tiles
+        names = [f"maize_gemm_bf16_t128_{'nt' if nt else 'nn'}"]
+        if chosen == names[0]:
+            return None
+    elif panel_rows == 256:
+        if "_h128" not in chosen and "_t128_" not in chosen:
             return None                                # a 256-row kernel, a split of one, or a few-row kernel: the dispatcher's
         names = [base, base + "_ktail", base + "_gen", base + "_ktail_gen"]
     else:
@@ -372,7 +388,7 @@ def described_kernel(desc, mma, nt, panel_rows, pipe, compute_units):
             return name
         except MaizeError:
             continue
-    raise ValueError(f"no kernel with {panel_rows}-row panels of A on {pipe} ring stages runs this product "
+    raise ValueError(f"no kernel with {panel_rows}-row panels of A{' and 128-column panels of B' if panel_cols == 128 else ''} on {pipe} ring stages runs this product "
                      f"(tried {', '.join(names)})")
 
 
@@ -389,7 +405,7 @@ class PreLoadGemm:
                             beta=op["beta"], in_type=op["mma"].in_type)
         forced = "maize_gemm_bf16_wave32" if op["mma"].family == "wave32" else None
         if op["mma"].family == "mt256":
-            forced = described_kernel(desc, op["mma"], op["nt"], op["panel_rows"], op["pipe"], ctx.info()["compute_units"])
+            forced = described_kernel(desc, op["mma"], op["nt"], op["panel_rows"], op["pipe"], ctx.info()["compute_units"], op["panel_cols"])
         return LoadedGemm(ctx, desc, forced, op["mma"])
 
 

@@ -136,6 +136,31 @@ int main() {
                 }
         std::printf("ok  K x N tile: transposing reads deliver the MFMA operand and are bank-conflict free\n");
     }
+    // ---- K x N tile of the 128 x 128 kernel: 64 rows of 256 B, 16 pieces of 4 rows
+    {
+        std::set<uint32_t> seen;
+        for (uint32_t piece = 0; piece < 16; ++piece)
+            for (uint32_t lane = 0; lane < 64; ++lane) {
+                const uint32_t row = sk128_piece_row(piece, lane), chunk = sk128_piece_chunk(piece, lane);
+                CHECK(row < 64 && chunk < 16, "128-wide K x N piece out of range");
+                CHECK(sk128_offset(row, chunk) == piece * 1024 + lane * 16, "128-wide K x N deposit/read mismatch piece %u lane %u", piece, lane);
+                CHECK(seen.insert(row * 16 + chunk).second, "128-wide K x N (row %u, chunk %u) deposited twice", row, chunk);
+            }
+        CHECK(seen.size() == 64 * 16, "128-wide K x N tile not covered");
+        for (uint32_t cg = 0; cg < 8; ++cg)
+            for (uint32_t kh = 0; kh < 2; ++kh)
+                for (uint32_t h = 0; h < 2; ++h) {
+                    uint32_t off[64];
+                    for (uint32_t lane = 0; lane < 64; ++lane) {
+                        off[lane] = sk128_tr_offset(cg, 0, lane) + 8192 * kh + 1024 * h;
+                        const uint32_t q = lane & 15u, g = lane >> 4;
+                        const uint32_t row = 32 * kh + 8 * g + 4 * h + q / 4, col = 16 * cg + 4 * (q % 4);
+                        CHECK(off[lane] == sk128_offset(row, col >> 3) + (col & 7) * 2, "128-wide K x N transposing read cg %u kh %u h %u lane %u", cg, kh, h, lane);
+                    }
+                    CHECK(passes_conflict_free(off, 8), "128-wide K x N transposing read cg %u kh %u h %u has bank conflicts", cg, kh, h);
+                }
+        std::printf("ok  128-wide K x N tile: deposit map is a bijection onto the read map, transposing reads deliver the MFMA operand and are bank-conflict free\n");
+    }
     // ---- K x N tile of 8-bit elements: 128 rows of 256 B, 32 pieces of 4 rows
     {
         std::set<uint32_t> seen;

@@ -228,6 +228,26 @@ def test_main_loop_of_the_three_stage_kernels_is_lean(kernels):
         assert count(kernels[name], want) == 320 and count(kernels[name], "v_mfma") == 320, name
 
 
+def test_main_loop_of_the_128_by_128_tile_kernels_is_lean(kernels):
+    """The 128 x 128 tile kernels: one K step of 32 MFMAs per wave and trip, 16 128-bit fragment reads (K x N B: 8 and 16
+    transposing ones), eight requests, one barrier whose wait leaves sixteen requests in flight.  Between a fragment
+    read and the matrix instruction that takes it stands a wait and nothing else: no move of a fragment (the reads
+    are assembly statements whose results the compiler believes ready at once; a move would copy them early)."""
+    for name, reads in (("maize_gemm_bf16_t128_nn", {"ds_read_b128": 8, "ds_read_b64_tr_b16": 16}), ("maize_gemm_bf16_t128_nt", {"ds_read_b128": 16})):
+        ins = kernels[name]
+        idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
+        assert len(idx) == 32 and count(ins, "v_mfma_f32_16x16x32_bf16") == 32, name
+        body = ins[idx[0]:idx[-1] + 1]
+        for mnemonic, n in reads.items():
+            assert count(body, mnemonic) == n // 2, (name, mnemonic)          # (K half 0's reads of the next tile; K half 1's stand in front of the first MFMA)
+        assert count(body, "buffer_load_dwordx4") == 8 and count(body, "s_barrier") == 1
+        assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(16)" in i) == 1, name
+        moves = [i for i in body if i.startswith(("v_mov", "v_accvgpr", "v_perm", "v_pk_", "v_lshl", "v_bfi", "v_and", "v_alignbit"))]
+        assert not moves, (name, moves[:5])
+        vector = [i for i in body if i.startswith("v_") and not i.startswith(("v_mfma", "v_add_u32", "v_or_b32", "v_cmp_lt_u64"))]
+        assert not vector, (name, vector[:5])                                   # (the reads' addresses: ring stage added to the lane's base)
+
+
 
 def test_no_k_loop_wraps_its_requests_in_scalarising_loops(kernels):
     """A buffer descriptor that the compiler carries in vector registers makes it wrap every request in a loop that

@@ -61,7 +61,7 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
     gx, gy, gz = p["grid"]
     splitk = p["kernel"].endswith("_splitk")
     packed = p["kernel"].endswith("_packed")
-    persistent = "_mt256_" in p["kernel"] and not p["kernel"].endswith("_edge")
+    persistent = ("_mt256_" in p["kernel"] and not p["kernel"].endswith("_edge")) or "_t128_" in p["kernel"]   # (batch members in grid.x)
     assert gx >= 1 and gy >= 1 and gz == (1 if persistent else batch)
     assert gy <= 65535 and gz <= 65535 and gx < (1 << 31)
     name = p["kernel"]
@@ -203,6 +203,12 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert p["workspace_bytes"] < (1 << 31)
         else:
             assert p["workspace_bytes"] == 0
+    elif name.startswith("maize_gemm_bf16_t128_"):
+        # 128 x 128 tiles, one workgroup per tile of the flattened (batch, tile) list, whole K, no workspace
+        assert p["block"] == (256, 1, 1) and (gy, gz) == (1, 1)
+        assert gx == cdiv(m, 128) * cdiv(n, 128) * batch
+        assert k % 64 == 0 and n % 8 == 0
+        assert p["ksplit"] == 1 and p["workspace_bytes"] == 0 and p["reduce_grid"] == 0
     else:
         raise AssertionError(f"no invariants written for kernel {name}")
 
@@ -220,7 +226,9 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (8192, 8192, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt",
         (16, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn",
         (2048, 2048, 2048, mz.LAYOUT_NN, 32): "maize_gemm_bf16_mt256_nn",
-        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3",      # 64 tiles: partial tiles would cost more than they save, 128 tiles of 128 rows fill half the chip (32 K steps: three ring stages)
+        (2048, 2048, 2048, mz.LAYOUT_NN, 1): "maize_gemm_bf16_t128_nn",              # 64 tiles: partial tiles would cost more than they save, 128 tiles of 128 rows fill half the chip, 256 of 128 x 128 all of it (23.5 -> 22.0 us)
+        (768, 8192, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3",       # 384 tiles of 128 x 128 would be two rounds: 192 of 128 x 256 on three ring stages
+        (1024, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_t128_nt",              # 256 tiles of 128 x 128, one round (40.7 -> 34.3 us)
         (512, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3",      # 112 tiles: 224 of 128 rows are one round
         (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3_splitk",  # few tiles, a long K: 128-row tiles cut over K (ranges of 16 steps: three stages)
         (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128_splitk",
@@ -256,26 +264,33 @@ def test_split_k_of_few_tiles_fills_the_chip_once():
     assert 8 <= p["ksplit"] <= 16 and p["grid"] == (16 * p["ksplit"], 1, 1)
     # more than half a chip of tiles, or a short K: no split
     assert mz.gemm_plan(desc(4096, 2304, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"
-    assert mz.gemm_plan(desc(512, 512, 448), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"      # (in 128-row tiles: 13.3 -> 8.6 us)
+    assert mz.gemm_plan(desc(512, 512, 448), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nn"            # (in 128-row tiles: 13.3 -> 8.4 us; 128 x 128: 7.7)
 
 
 def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
     """56 to 128 tiles on 256 compute units leave most of the chip idle for a whole walk of K: two or four K ranges
     per tile pay for the partial tiles (measured: 256 x 14336 x 4096 67 -> 46 us, 768 x 8192 x 8192 128 -> 110 us) --
     or, where one round of them is cheaper than the split, tiles of 128 rows (768 x 8192 x 8192 94 us, 2048^3 37 -> 29)."""
-    p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)                  # 112 tiles of 128 rows: whole K on three ring stages
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3" and p["ksplit"] == 1 and p["grid"] == (112, 1, 1)
+    p = mz.gemm_plan(desc(256, 14336, 4096), compute_units=CUS)                  # 112 tiles of 128 rows: whole K -- in 224 tiles of 128 x 128 (39.6 -> 36.6 us)
+    assert p["kernel"] == "maize_gemm_bf16_t128_nn" and p["ksplit"] == 1 and p["grid"] == (224, 1, 1)
+    p = mz.gemm_plan(desc(256, 14336, 4096), kernel="maize_gemm_bf16_mt256_nn_h128r3", compute_units=CUS)
+    assert p["ksplit"] == 1 and p["grid"] == (112, 1, 1)
     p = mz.gemm_plan(desc(128, 14336, 4096), compute_units=CUS)                  # one row of tiles: cut over K (38 us against 54.7 whole)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and p["ksplit"] == 4 and p["grid"] == (224, 1, 1)   # (ranges of 16 steps: three stages)
     p = mz.gemm_plan(desc(768, 8192, 8192), compute_units=CUS)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3" and p["ksplit"] == 1 and p["grid"] == (192, 1, 1)
     p = mz.gemm_plan(desc(640, 8192, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3" and p["grid"] == (160, 1, 1)
-    assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"
-    assert mz.gemm_plan(desc(512, 8192, 960), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"          # 15 K steps: the two-stage loop
-    assert mz.gemm_plan(desc(512, 8192, 1024), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"       # 16 steps: three stages (15.2 -> 14.6 us now that no step is padded)
-    assert mz.gemm_plan(desc(1024, 4096, 1536), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"      # 24 steps, 128 tiles: 23.5 -> 19.7 us
-    assert mz.gemm_plan(desc(512, 2048, 1792), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"         # 32 tiles: too few to make the loads wait
+    assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nn"
+    assert mz.gemm_plan(desc(2048, 2048, 2048), compute_units=CUS)["grid"] == (256, 1, 1)
+    # (products of more than 256 tiles of 128 x 128, which would be two rounds of those)
+    assert mz.gemm_plan(desc(768, 8192, 960), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128"          # 15 K steps: the two-stage loop
+    assert mz.gemm_plan(desc(768, 8192, 1024), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"       # 16 steps: three stages (512 x 8192 x 1024: 15.2 -> 14.6 us now that no step is padded)
+    assert mz.gemm_plan(desc(1536, 4096, 1536), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"      # 24 steps (1024 x 4096 x 1536, 128 tiles: 23.5 -> 19.7 us)
+    # (up to 256 of them: one round of 128 x 128 tiles -- 512 x 8192 x 1024 14.0 -> 13.6 us, 512 x 2048 x 1792 19.8 -> 17.7)
+    assert mz.gemm_plan(desc(512, 8192, 1024), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nn"
+    assert mz.gemm_plan(desc(512, 2048, 1792), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nn"
+    assert mz.gemm_plan(desc(512, 2048, 1792), kernel="maize_gemm_bf16_mt256_nn_h128", compute_units=CUS)["grid"] == (32, 1, 1)
     # K ranges of 28 steps or more run on the three-stage kernels too, whichever way B is stored (a row-major B costs
     # them 3-7 % more per step, not the 60 % it was once priced at)
     p = mz.gemm_plan(desc(512, 4096, 14336, layout=mz.LAYOUT_NT), compute_units=CUS)       # (61 us; two stages 67.5, 256-row split 65)
@@ -289,8 +304,10 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
         nn_plan = mz.gemm_plan(desc(m, n, k), kernel="maize_gemm_bf16_mt256_nn_h128r3_splitk", compute_units=CUS)
         nt_plan = mz.gemm_plan(desc(m, n, k, layout=mz.LAYOUT_NT), kernel="maize_gemm_bf16_mt256_nt_h128r3_splitk", compute_units=CUS)
         assert nn_plan["ksplit"] == nt_plan["ksplit"] and nn_plan["grid"] == nt_plan["grid"], (m, n, k, nn_plan, nt_plan)
-    p = mz.gemm_plan(desc(384, 6144, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)        # (three ranges 33 us; two 35; whole 39)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3_splitk" and p["ksplit"] == 3 and p["grid"] == (216, 1, 1)
+    p = mz.gemm_plan(desc(384, 6144, 4096), compute_units=CUS)                             # (three ranges 33 us; two 35; whole 39)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and p["ksplit"] == 3 and p["grid"] == (216, 1, 1)
+    p = mz.gemm_plan(desc(384, 6144, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)        # (N x K: 144 tiles of 128 x 128 30.9 us, three ranges 31.5)
+    assert p["kernel"] == "maize_gemm_bf16_t128_nt" and p["grid"] == (144, 1, 1)
     assert mz.gemm_plan(desc(4096, 2304, 2048), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"       # 288 tiles of 128 rows would need two rounds
     assert mz.gemm_plan(desc(1024, 14336, 4096), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn"   # 224 tiles: one round as it is
 
@@ -470,13 +487,16 @@ def test_operands_past_the_memory_side_cache_are_priced_by_their_bytes_too():
     the cache keep the choice the K steps make."""
     for m in (96, 128):
         for layout in (mz.LAYOUT_NN, mz.LAYOUT_NT):
+            p = mz.gemm_plan(desc(m, 28672, 8192, layout), kernel=f"maize_gemm_bf16_mt256_{'nn' if layout == mz.LAYOUT_NN else 'nt'}_h128r3_splitk", compute_units=CUS)
+            assert p["ksplit"] == 2 and p["grid"][0] == 224, p
+            # ... and 224 tiles of 128 x 128 draw the same stream without the second launch (N x K 119.7 -> 107.4 us, K x N 99.2 -> 97.9)
             p = mz.gemm_plan(desc(m, 28672, 8192, layout), compute_units=CUS)
-            assert p["kernel"].endswith("_h128r3_splitk") and p["ksplit"] == 2 and p["grid"][0] == 224, p
+            assert "_t128_" in p["kernel"] and p["grid"][0] == 224, p
     for layout in (mz.LAYOUT_NN, mz.LAYOUT_NT):
         p = mz.gemm_plan(desc(192, 28672, 8192, layout), compute_units=CUS)
         assert p["kernel"].endswith("_h128r3") and p["ksplit"] <= 1, p
-    p = mz.gemm_plan(desc(96, 28672, 4096), compute_units=CUS)          # 235 MB: stays in whole tiles
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3", p
+    p = mz.gemm_plan(desc(96, 28672, 4096), compute_units=CUS)          # 235 MB: stays in whole tiles (of 128 x 128: one round of 224)
+    assert p["kernel"] == "maize_gemm_bf16_t128_nn" and p["ksplit"] == 1, p
 
 
 def test_the_boundary_between_whole_128_row_tiles_and_their_split():

@@ -1,0 +1,50 @@
+"""maize_gemm_bf16_t128_{nn,nt}: 128 x 128 tiles on a four-stage ring.  The same sums in the same order as the 256-row
+general-epilogue kernels (one MFMA 16x16x32 per 32 of K, K ascending): the whole of C is compared bit for bit with
+theirs, and sampled rows (every column) against the oracle.  Shapes: one to three K steps (the ring is primed with tiles
+past K), step counts of every residue mod 4, ragged M and N inside the last tiles, more tiles than compute units,
+batches with gaps between their members."""
+import sys
+
+import numpy as np
+import pytest
+
+import maize_amd as mz
+from tests.gpu_util import run_gemm, check_rows_against_oracle, sample_rows
+
+pytestmark = pytest.mark.gpu
+
+# (M, N, K, batch)
+SHAPES = [(128, 128, 64, 1), (130, 136, 128, 1), (256, 256, 192, 1), (1000, 1032, 1088, 1), (1024, 4096, 4096, 1), (2048, 2048, 2048, 1),
+          (300, 4104, 320, 1), (520, 264, 8192, 1), (4096, 2176, 448, 1), (100, 72, 64, 5), (500, 520, 256, 3), (1, 8, 64, 1), (2047, 2040, 576, 1)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT], ids=["nn", "nt"])
+def test_tiles_of_128_by_128_bit_for_bit(ctx, oracle, shape, layout):
+    m, n, k, batch = shape
+    tag = "nt" if layout == mz.LAYOUT_NT else "nn"
+    a = mz.gen.uniform_bf16(batch * m * k, 31)
+    b = mz.gen.uniform_bf16(batch * k * n, 32)
+    if layout == mz.LAYOUT_NT:
+        b = np.concatenate([b[i * k * n:(i + 1) * k * n].reshape(k, n).T.ravel() for i in range(batch)])
+    print(f"128 x 128 tiles: {shape} {tag}", flush=True)
+    sys.stdout.flush()
+    gap = 24 if batch > 1 else 0                      # members of C 24 elements apart (rows stay on 16-byte boundaries)
+    kw = dict(layout=layout, batch=batch, stride_c=m * n + gap)
+    want = run_gemm(ctx, a, b, m, n, k, kernel=f"maize_gemm_bf16_mt256_{tag}_gen", **kw)
+    print("  256-row kernel done", flush=True)
+    got = run_gemm(ctx, a, b, m, n, k, kernel=f"maize_gemm_bf16_t128_{tag}", **kw)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} elements differ"
+    if batch == 1:
+        check_rows_against_oracle(oracle, got, a, b, m, n, k, sample_rows(m, count=8, tile=128)[:12], layout=layout, label=f"t128 {shape} {tag}")
+
+
+def test_the_dispatcher_takes_them_for_one_round_of_tiles(ctx):
+    cus = ctx.info()["compute_units"]
+    if cus != 256:
+        pytest.skip("expectations are for 256 compute units")
+    for m, n, k, layout, want in ((1024, 4096, 4096, mz.LAYOUT_NT, "maize_gemm_bf16_t128_nt"), (2048, 2048, 2048, mz.LAYOUT_NN, "maize_gemm_bf16_t128_nn"),
+                                  (1536, 4096, 4096, mz.LAYOUT_NN, "maize_gemm_bf16_mt256_nn_h128r3")):
+        brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+        d = mz.gemm_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x1000, brows, bcols), mz.GlobalMatrix(0x1000, m, n), layout=layout)
+        assert mz.gemm_plan(d, compute_units=cus)["kernel"] == want

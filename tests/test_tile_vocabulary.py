@@ -110,8 +110,8 @@ def test_the_description_chooses_the_panel_height_and_the_ring_depth():
     two or three ring stages as it says, whatever the dispatcher would take by itself; one that no kernel runs is refused."""
     cus = FakeCtx()
     h128 = dict(a_panel=128, tiles=(T.BF16_128x64, T.BF16_64x256))
-    # 2048^3: the dispatcher itself takes 128-row tiles on three stages
-    a, b, c = matrices(2048, 2048, 2048)
+    # 768 x 8192 x 8192: the dispatcher itself takes 128-row tiles on three stages
+    a, b, c = matrices(768, 8192, 8192)
     assert mz.gemm_plan(mz.gemm_desc(a, b, c), compute_units=256)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3"
     got = {}
     for tag, kw in (("r3", dict(depth=3, **h128)), ("r2", dict(depth=2, **h128)), ("256", dict())):
@@ -136,6 +136,23 @@ def test_the_description_chooses_the_panel_height_and_the_ring_depth():
         am.elem_bytes = bm.elem_bytes = 1
         k, _ = describe(am, bm, cm, mma=T.Gfx950MfmaE4M3E5M2F32_16x16x128, nt=nt, ktile=128, depth=3, a_panel=128, tiles=(T.F8_128x128, btile))
         assert k.finalize().compile(mz.Gfx.Gfx950, cus).kernel_name == f"maize_gemm_e4m3e5m2_mt256_{'nt' if nt else 'nn'}_h128r3_gen"
+    # 128 x 128 tiles on a ring of four stages: the dispatcher's own choice for 2048^3, described for 4096^3; a description
+    # of 256-row panels for 2048^3 gets the 256-row kernel
+    q128 = dict(depth=4, a_panel=128, panel=128)
+    a, b, c = matrices(2048, 2048, 2048)
+    got = describe(a, b, c, tiles=(T.BF16_128x64, T.BF16_64x128), **q128)[0].finalize().compile(mz.Gfx.Gfx950, cus)
+    assert got.kernel_name == "maize_gemm_bf16_t128_nn" and got.forced is None and got.plan["grid"] == (256, 1, 1)
+    assert describe(a, b, c)[0].finalize().compile(mz.Gfx.Gfx950, cus).forced == "maize_gemm_bf16_mt256_nn"
+    assert describe(a, b, c, depth=3, **h128)[0].finalize().compile(mz.Gfx.Gfx950, cus).forced == "maize_gemm_bf16_mt256_nn_h128r3"
+    a, b, c = matrices(4096, 4096, 4096, nt=True)
+    got = describe(a, b, c, nt=True, tiles=(T.BF16_128x64, T.BF16_128x64), **q128)[0].finalize().compile(mz.Gfx.Gfx950, cus)
+    assert got.kernel_name == got.forced == "maize_gemm_bf16_t128_nt" and got.plan["grid"] == (1024, 1, 1)
+    with pytest.raises(ValueError, match="ring of four stages"):
+        describe(a, b, c, nt=True, tiles=(T.BF16_128x64, T.BF16_128x64), depth=3, a_panel=128, panel=128)
+    with pytest.raises(ValueError, match="B stage is BF16_128x64"):                     # K x N B needs the K x N stage
+        describe(*matrices(2048, 2048, 2048), tiles=(T.BF16_128x64, T.BF16_128x64), **q128)
+    with pytest.raises(ValueError, match="or 128 rows and 128 columns"):
+        describe(*matrices(2048, 2048, 2048), tiles=(T.BF16_256x64, T.BF16_64x128), depth=2, a_panel=256, panel=128)      # 256-row panels of A against 128 columns
     # K % 8 != 0: no macro-tile kernel reads such operands where they lie; the description is refused, not replaced
     k, _ = describe(*matrices(512, 512, 516), depth=3, **h128)
     with pytest.raises(ValueError, match="no kernel with 128-row panels of A on 3 ring stages"):
