@@ -109,10 +109,10 @@ def test_macro_tile_kernels_on_strided_views(ctx, oracle, layout, shape, lds):
     if layout == mz.LAYOUT_NT:
         ldb = max(k + 8, 200)
     took = run_ex(ctx, oracle, m, n, k, layout=layout, lda=lda, ldb=ldb, ldc=ldc, label="mt256 views")
-    assert took.startswith("maize_gemm_bf16_mt256"), took
+    assert took.startswith(("maize_gemm_bf16_mt256", "maize_gemm_bf16_t128")), took
     # each variant that accepts the shape, by name
     for name in mz.kernel_names():
-        if not name.startswith("maize_gemm_bf16_mt256") or ("_nt" in name) != (layout == mz.LAYOUT_NT):
+        if not name.startswith(("maize_gemm_bf16_mt256", "maize_gemm_bf16_t128")) or ("_nt" in name) != (layout == mz.LAYOUT_NT):
             continue
         if "ktail" not in name and k % 64:
             continue
@@ -190,8 +190,8 @@ def test_general_epilogue_with_several_tiles_per_workgroup_and_batches(ctx, orac
     try:
         x = mz.gemm_ex_desc(mz.Matrix(da, m, k), mz.Matrix(db, k, n), mz.Matrix(dc, m, n), batch=batch, stride_a=m * k,
                             stride_b=k * n, stride_c=m * n, out_type=mz.OUT_F32, alpha=0.75, beta=1.5)
-        assert mz.gemm_plan(x)["kernel"] == "maize_gemm_bf16_mt256_nn_h128_gen"
-        for kernel in (None, "maize_gemm_bf16_mt256_nn_gen"):
+        assert mz.gemm_plan(x)["kernel"] == "maize_gemm_bf16_t128_nn"
+        for kernel in (None, "maize_gemm_bf16_mt256_nn_h128_gen", "maize_gemm_bf16_mt256_nn_gen"):
             dc.write(c0)
             ctx.gemm_bf16(x, kernel=kernel)
             ctx.sync()
@@ -232,15 +232,21 @@ def test_half_height_tiles(ctx, oracle, layout):
                dict(alpha=2.0, beta=0.0, c_nan=True), dict(lda=k + 3, ldb=bcols + 5)):
         assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen3, label="h128r3 gen", **kw) == gen3
         assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen316, half=True, label="h128r3 gen half", **kw) == gen316
-    assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, label="h128r3 auto") == plain3
+    # (the dispatcher's own choice: products of more than 256 tiles of 128 x 128 -- up to 256 of those go to the 128 x 128
+    # tile kernels, bf16 operands and whole K tiles only)
+    t128 = f"maize_gemm_bf16_t128_{tag}"
+    assert run_ex(ctx, oracle, 1152, 4096, 1024, layout=layout, label="h128r3 auto") == plain3
     assert run_ex(ctx, oracle, 1000, 2056, 1800, layout=layout, label="h128r3 auto tail") == gen3
-    assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, alpha=0.5, beta=1.0, label="h128r3 auto scaled") == gen3
+    assert run_ex(ctx, oracle, 1152, 4096, 1024, layout=layout, alpha=0.5, beta=1.0, label="h128r3 auto scaled") == gen3
     assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, half=True, label="h128r3 auto half") == gen316
+    assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, label="t128 auto") == t128
+    assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, alpha=0.5, beta=1.0, label="t128 auto scaled") == t128
     # the dispatcher's choice
-    assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, label="h128 auto") == plain
+    assert run_ex(ctx, oracle, 1152, 4096, 512, layout=layout, label="h128 auto") == plain
     assert run_ex(ctx, oracle, 520, 776, 328, layout=layout, label="h128 auto tail") == gen
-    assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, alpha=0.5, beta=1.0, label="h128 auto scaled") == gen
+    assert run_ex(ctx, oracle, 1152, 4096, 512, layout=layout, alpha=0.5, beta=1.0, label="h128 auto scaled") == gen
     assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, half=True, label="h128 auto half") == gen16
+    assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, out_f32=True, alpha=-2.0, beta=0.25, label="t128 auto fp32") == t128
     # batched, several tiles per workgroup: 5 x 640 x 768 in 128-row tiles = 75 tiles on the grid the plan gives
     from tests.gpu_util import run_gemm
     bm, bn, bk, batch = 640, 768, 512, 5
@@ -547,7 +553,7 @@ def test_macro_tile_kernels_read_unaligned_operands_where_they_lie(ctx, oracle, 
     (which may start on any even byte), C goes through the general epilogue when its rows are 16-byte material and
     through the split-K kernels' reduce pass (one K range if splitting does not pay) when they are not."""
     took = run_ex(ctx, oracle, label="unaligned", **case)
-    assert "_mt256_" in took and not took.endswith("_packed"), took
+    assert ("_mt256_" in took or "_t128_" in took) and not took.endswith("_packed"), took
     c_unaligned = case["n"] % 8 != 0 or case.get("ldc", 8) % 8 != 0
     assert took.endswith("_splitk") or not c_unaligned, took
 
