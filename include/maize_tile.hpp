@@ -151,6 +151,7 @@ MAIZE_TILE_TY(F8_128x256, 128, 256, 1, Swizzle::KN16)    // B stage of a row-maj
 MAIZE_TILE_TY(BF16_128x64, 128, 64, 2, Swizzle::KC16)    // A stages of the 128 x 256 tile kernels (the B stages are the ones above)
 MAIZE_TILE_TY(F16_128x64, 128, 64, 2, Swizzle::KC16)
 MAIZE_TILE_TY(F8_128x128, 128, 128, 1, Swizzle::KC16)
+MAIZE_TILE_TY(BF16_64x128, 64, 128, 2, Swizzle::KN32)    // B stage of the 128 x 128 tile kernels for a row-major K x N B (stored N x K: BF16_128x64, like their A stage)
 #undef MAIZE_TILE_TY
 template <class T> struct Tile { using Ty = T; static constexpr size_t SIZE = (size_t)T::ROWS * T::COLS * T::ELEM_BYTES; };
 template <class TA, class TB> struct TilePair { using A = TA; using B = TB; static constexpr size_t SIZE = TA::SIZE + TB::SIZE; };
@@ -226,12 +227,12 @@ std::pair<PanelIterLooper<ColPanel<N>>, ColPanel<N>> collective_aligned_col_pane
     return {PanelIterLooper<ColPanel<N>>{ColPanel<N>{m, N, false}, m.g.ncols / N}, ColPanel<N>{m, m.g.ncols % N, true}};
 }
 
-// panel_rows, pipe: the panel height of A and the ring depth as described (0: the description has no ring)
-struct TracedOp { Matrix a, b, c; bool nt; maize_in_type_t in; Family family; bool stored; maize_out_type_t out; float alpha, beta; uint32_t panel_rows, pipe; };
+// panel_rows, pipe, panel_cols: the panel height of A, the ring depth and the panel width of B as described (pipe 0: the description has no ring)
+struct TracedOp { Matrix a, b, c; bool nt; maize_in_type_t in; Family family; bool stored; maize_out_type_t out; float alpha, beta; uint32_t panel_rows, pipe, panel_cols = 256; };
 // The kernel that a description of the mainloop (panel height of A, ring depth) names for `x`; empty when the
 // dispatcher's own choice already is of that family.  A description is honoured wherever a kernel of its family accepts
 // the descriptor -- also where the dispatcher by itself would take another family -- and refused where none does.
-inline std::string described_kernel(const maize_gemm_ex_desc_t& x, bool nt, uint32_t panel_rows, uint32_t pipe, uint32_t cus) {
+inline std::string described_kernel(const maize_gemm_ex_desc_t& x, bool nt, uint32_t panel_rows, uint32_t pipe, uint32_t cus, uint32_t panel_cols = 256) {
     maize_gemm_plan_t plan;
     check(maize_hip_gemm_ex_plan(&x, nullptr, cus, &plan));
     const std::string chosen = plan.kernel;
@@ -240,8 +241,12 @@ inline std::string described_kernel(const maize_gemm_ex_desc_t& x, bool nt, uint
     const std::string base = std::string("maize_gemm_") + tags[(int)x.in_type] + "_mt256_" + (nt ? "nt" : "nn");
     std::vector<std::string> names;
     const bool is_h = chosen.find("_h128") != std::string::npos, is_r3 = chosen.find("_h128r3") != std::string::npos;
-    if (panel_rows == 256) {
-        if (!is_h) return "";                     // a 256-row kernel, a split of one, or a few-row kernel: the dispatcher's
+    const bool is_q = chosen.find("_t128_") != std::string::npos;
+    if (panel_cols == 128) {                      // 128 x 128 tiles
+        names = {std::string("maize_gemm_bf16_t128_") + (nt ? "nt" : "nn")};
+        if (chosen == names[0]) return "";
+    } else if (panel_rows == 256) {
+        if (!is_h && !is_q) return "";            // a 256-row kernel, a split of one, or a few-row kernel: the dispatcher's
         names = {base, base + "_ktail", base + "_gen", base + "_ktail_gen"};
     } else {
         if (pipe == 3 ? is_r3 : (is_h && !is_r3)) return "";
@@ -259,7 +264,7 @@ class LoadedGemm {
         maize_device_info_t info;
         if (maize_hip_device_info(ctx.handle(), &info) == MAIZE_OK) cus = info.compute_units;
         if (op.family == Family::WAVE32) forced_ = "maize_gemm_bf16_wave32";
-        else if (op.family == Family::MT256 && op.pipe) forced_ = described_kernel(x_, op.nt, op.panel_rows, op.pipe, cus);
+        else if (op.family == Family::MT256 && op.pipe) forced_ = described_kernel(x_, op.nt, op.panel_rows, op.pipe, cus, op.panel_cols);
         check(maize_hip_gemm_ex_plan(&x_, forced(), cus, &plan_));
     }
     std::string kernel_name() const { return plan_.kernel; }
@@ -328,18 +333,22 @@ Accum gemm_smem_multibuffer(const MMA&, KTile<K_TILE>, const RowPanel<NA>& a, co
     // Generic in the ring depth and the panel height like the reference's mainloop ([TilePair; PIPE], KTile<N>,
     // gemm/mod.rs:37-45), within what kernels exist: 256- or 128-row panels of A on two stages, 128-row panels also on
     // three (a 128 x 256 tile's stage is 48 KiB; three fit the 160 KiB of LDS).
-    static_assert(PIPE == 2 || PIPE == 3, "the macro-tile kernels run a ring of two or three stages");
-    static_assert((NA == 256 || NA == 128) && BPanel::WINDOW == 256, "the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B)");
-    static_assert(PIPE == 2 || NA == 128, "three ring stages fit the LDS with 128-row panels of A only");
+    // ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages, bf16.
+    constexpr uint32_t NB = BPanel::WINDOW;
+    constexpr bool QUARTER = NA == 128 && NB == 128;
+    static_assert(QUARTER ? PIPE == 4 : (PIPE == 2 || PIPE == 3), "the macro-tile kernels run a ring of two or three stages, the 128 x 128 tile kernels one of four");
+    static_assert((NA == 256 || NA == 128) && (NB == 256 || QUARTER), "the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B), or 128 rows and 128 columns");
+    static_assert(!QUARTER || MMA::IN_TYPE == MAIZE_IN_BF16, "the 128 x 128 tile kernels take bf16 operands");
+    static_assert(PIPE != 3 || NA == 128, "three ring stages fit the LDS with 128-row panels of A only");
     using TA = typename Pair::A::Ty; using TB = typename Pair::B::Ty;
     constexpr uint32_t ES = MMA::K_TILE == 128 ? 1 : 2;
     static_assert(TA::ROWS == NA && TA::COLS == MMA::K_TILE && TA::ELEM_BYTES == ES && TA::SWIZZLE == Swizzle::KC16, "A stage: panel rows x K_TILE, K-contiguous");
-    static_assert(NT ? (TB::ROWS == 256 && TB::COLS == MMA::K_TILE && TB::ELEM_BYTES == ES && TB::SWIZZLE == Swizzle::KC16)
-                     : (TB::ROWS == MMA::K_TILE && TB::COLS == 256 && TB::ELEM_BYTES == ES && TB::SWIZZLE == (ES == 2 ? Swizzle::KN32 : Swizzle::KN16)), "B stage does not match how B is stored");
+    static_assert(NT ? (TB::ROWS == NB && TB::COLS == MMA::K_TILE && TB::ELEM_BYTES == ES && TB::SWIZZLE == Swizzle::KC16)
+                     : (TB::ROWS == MMA::K_TILE && TB::COLS == NB && TB::ELEM_BYTES == ES && TB::SWIZZLE == (ES == 2 ? Swizzle::KN32 : Swizzle::KN16)), "B stage does not match how B is stored");
     if (cp_size != 16) throw std::invalid_argument("direct-to-LDS copies are 16 bytes per lane");
     const uint32_t ka = a.col_size(), kb = NT ? b.matrix.g.ncols : b.matrix.g.nrows;
     if (ka != kb) throw std::invalid_argument("inner dimensions differ");
-    return Accum(cp_group.kernel, TracedOp{a.matrix, b.matrix, Matrix{}, NT, MMA::IN_TYPE, MMA::FAMILY, false, MAIZE_OUT_SAME, 1.0f, 0.0f, NA, (uint32_t)PIPE});
+    return Accum(cp_group.kernel, TracedOp{a.matrix, b.matrix, Matrix{}, NT, MMA::IN_TYPE, MMA::FAMILY, false, MAIZE_OUT_SAME, 1.0f, 0.0f, NA, (uint32_t)PIPE, NB});
 }
 inline TracedKernel new_hip_kernel() { return TracedKernel(); }
 

@@ -29,6 +29,7 @@ tile_ty!(F8_128x256, 128, 256, 1, Swizzle::Kn16);   // B stage of a row-major K 
 tile_ty!(BF16_128x64, 128, 64, 2, Swizzle::Kc16);   // A stages of the 128 x 256 tile kernels
 tile_ty!(F16_128x64, 128, 64, 2, Swizzle::Kc16);
 tile_ty!(F8_128x128, 128, 128, 1, Swizzle::Kc16);
+tile_ty!(BF16_64x128, 64, 128, 2, Swizzle::Kn32);   // B stage of the 128 x 128 tile kernels for a row-major K x N B
 pub struct Tile<T>(PhantomData<T>);
 pub struct TilePair<TA, TB> { pub a: PhantomData<TA>, pub b: PhantomData<TB> }
 /// `[TilePair<TA, TB>; PIPE]` in LDS (src/main.rs:42-44).
@@ -88,8 +89,8 @@ impl<const N: u32> BPanel for ColPanel<N> { const NT: bool = false; const WINDOW
 impl<const N: u32> BPanel for RowPanel<N> { const NT: bool = true; const WINDOW: u32 = N; fn matrix(&self) -> GlobalMatrix<BF16> { self.matrix } }
 
 /// The accumulator fragments of one panel pair, with what the description said of the mainloop.
-pub struct Accum { a: GlobalMatrix<BF16>, b: GlobalMatrix<BF16>, nt: bool, in_type: u32, panel_rows: u32, pipe: u32 }
-pub struct DescribedGemm { desc: ffi::MaizeGemmExDesc, nt: bool, panel_rows: u32, pipe: u32 }
+pub struct Accum { a: GlobalMatrix<BF16>, b: GlobalMatrix<BF16>, nt: bool, in_type: u32, panel_rows: u32, pipe: u32, panel_cols: u32 }
+pub struct DescribedGemm { desc: ffi::MaizeGemmExDesc, nt: bool, panel_rows: u32, pipe: u32, panel_cols: u32 }
 impl Accum {
     /// Names the C the accumulators are written to (the reference only sums them into a trap guard, src/main.rs:71).
     pub fn store(self, c: GlobalMatrix<BF16>) -> Result<DescribedGemm> {
@@ -99,7 +100,7 @@ impl Accum {
         }
         let gemm = crate::tile::gemm_desc(self.a, self.b, c, if self.nt { crate::tile::Layout::NT } else { crate::tile::Layout::NN });
         Ok(DescribedGemm { desc: ffi::MaizeGemmExDesc { gemm, lda: 0, ldb: 0, ldc: 0, out_type: 0, alpha: 1.0, beta: 0.0, in_type: self.in_type, reserved: 0 },
-                           nt: self.nt, panel_rows: self.panel_rows, pipe: self.pipe })
+                           nt: self.nt, panel_rows: self.panel_rows, pipe: self.pipe, panel_cols: self.panel_cols })
     }
 }
 fn plan_of(desc: &ffi::MaizeGemmExDesc, kernel: Option<&std::ffi::CStr>, cus: u32) -> Option<String> {
@@ -117,9 +118,14 @@ impl DescribedGemm {
             .ok_or(Error { code: ffi::MAIZE_ERR_ARG, message: "the dispatcher has no kernel for this product".into() })?;
         const TAGS: [&str; 6] = ["bf16", "f16", "e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"];
         let base = format!("maize_gemm_{}_mt256_{}", TAGS[self.desc.in_type as usize], if self.nt { "nt" } else { "nn" });
-        let (is_h, is_r3) = (chosen.contains("_h128"), chosen.contains("_h128r3"));
-        let names: Vec<String> = if self.panel_rows == 256 {
-            if !is_h { return Ok(None); }
+        let (is_h, is_r3, is_q) = (chosen.contains("_h128"), chosen.contains("_h128r3"), chosen.contains("_t128_"));
+        let names: Vec<String> = if self.panel_cols == 128 {
+            // 128 x 128 tiles
+            let name = format!("maize_gemm_bf16_t128_{}", if self.nt { "nt" } else { "nn" });
+            if chosen == name { return Ok(None); }
+            vec![name]
+        } else if self.panel_rows == 256 {
+            if !is_h && !is_q { return Ok(None); }
             vec![base.clone(), format!("{base}_ktail"), format!("{base}_gen"), format!("{base}_ktail_gen")]
         } else {
             if (self.pipe == 3 && is_r3) || (self.pipe == 2 && is_h && !is_r3) { return Ok(None); }
@@ -143,24 +149,29 @@ impl DescribedGemm {
 /// `sm80_gemm_smem_multibuffer(&mma, KTile::<K>, a_panel, b_panel, smem, cp_group, cp_size)` (gemm/mod.rs:37-90), generic
 /// in the ring depth and the panel height like the reference's mainloop (`[TilePair; PIPE]`, `KTile<N>`, gemm/mod.rs:37-45),
 /// within what kernels exist: 256- or 128-row panels of A on two ring stages, 128-row panels also on three; B in panels of
-/// 256 (column panels of a K x N B, row panels of a B stored N x K); 16-byte copies per lane of a Wave.
+/// 256 (column panels of a K x N B, row panels of a B stored N x K); 128-row panels of A against 128-wide panels of B on four
+/// stages (the 128 x 128 tile kernels, bf16); 16-byte copies per lane of a Wave.
 pub fn gemm_smem_multibuffer<MMA: SyncMMAOp, const K_TILE: u32, const NA: u32, B: BPanel, TA: ConstSizeTileTy, TB: ConstSizeTileTy, const PIPE: usize>(
         _mma: &MMA, _k: KTile<K_TILE>, a: RowPanel<NA>, b: B, _smem: &SharedRing<Tile<TA>, Tile<TB>, PIPE>, _cp_group: Wave, cp_size: u8) -> Result<Accum> {
     let refuse = |m: &str| Err(Error { code: ffi::MAIZE_ERR_ARG, message: m.into() });
     if MMA::FAMILY != Family::Mt256 { return refuse("a shared-memory ring goes with the macro-tile kernels' instructions"); }
     if K_TILE != MMA::K_TILE { return refuse("KTile does not match the K a ring stage of this instruction's kernels holds"); }
     if cp_size != 16 { return refuse("direct-to-LDS copies are 16 bytes per lane"); }
-    if !(PIPE == 2 || PIPE == 3) { return refuse("the macro-tile kernels run a ring of two or three stages"); }
-    if !(NA == 256 || NA == 128) || B::WINDOW != 256 { return refuse("the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B)"); }
+    // ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages, bf16
+    let quarter = NA == 128 && B::WINDOW == 128;
+    if quarter && PIPE != 4 { return refuse("the 128 x 128 tile kernels run a ring of four stages"); }
+    if quarter && MMA::IN_TYPE != ffi::MAIZE_IN_BF16 { return refuse("the 128 x 128 tile kernels take bf16 operands"); }
+    if !quarter && !(PIPE == 2 || PIPE == 3) { return refuse("the macro-tile kernels run a ring of two or three stages"); }
+    if !(NA == 256 || NA == 128) || !(B::WINDOW == 256 || quarter) { return refuse("the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B), or 128 rows and 128 columns"); }
     if PIPE == 3 && NA != 128 { return refuse("three ring stages fit the LDS with 128-row panels of A only"); }
     let es = if MMA::K_TILE == 128 { 1 } else { 2 };
     if !(TA::ROWS == NA && TA::COLS == MMA::K_TILE && TA::ELEM_BYTES == es && TA::SWIZZLE == Swizzle::Kc16) { return refuse("A stage: panel rows x K_TILE, K-contiguous"); }
-    let b_ok = if B::NT { TB::ROWS == 256 && TB::COLS == MMA::K_TILE && TB::ELEM_BYTES == es && TB::SWIZZLE == Swizzle::Kc16 }
-               else { TB::ROWS == MMA::K_TILE && TB::COLS == 256 && TB::ELEM_BYTES == es && TB::SWIZZLE == (if es == 2 { Swizzle::Kn32 } else { Swizzle::Kn16 }) };
+    let b_ok = if B::NT { TB::ROWS == B::WINDOW && TB::COLS == MMA::K_TILE && TB::ELEM_BYTES == es && TB::SWIZZLE == Swizzle::Kc16 }
+               else { TB::ROWS == MMA::K_TILE && TB::COLS == B::WINDOW && TB::ELEM_BYTES == es && TB::SWIZZLE == (if es == 2 { Swizzle::Kn32 } else { Swizzle::Kn16 }) };
     if !b_ok { return refuse("B stage does not match how B is stored"); }
     let bm = b.matrix();
     if a.matrix.ncols != (if B::NT { bm.ncols } else { bm.nrows }) {
         return Err(Error { code: ffi::MAIZE_ERR_SHAPE, message: "inner dimensions differ".into() });
     }
-    Ok(Accum { a: a.matrix, b: bm, nt: B::NT, in_type: MMA::IN_TYPE, panel_rows: NA, pipe: PIPE as u32 })
+    Ok(Accum { a: a.matrix, b: bm, nt: B::NT, in_type: MMA::IN_TYPE, panel_rows: NA, pipe: PIPE as u32, panel_cols: B::WINDOW })
 }

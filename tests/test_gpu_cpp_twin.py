@@ -30,6 +30,9 @@ def test_cpp_twin_matches_the_ctypes_path(ctx, oracle, shape):
     assert rec["mismatch_vs_described_kernel"] == 0 and "_h128" not in rec["described_kernel"]
     assert rec["described_kernel"] == rec["kernel"] or "_h128" in rec["kernel"]
     assert rec["mismatch_vs_described_128_rows_3_stages"] == 0 and "_h128r3" in rec["described_128_rows_3_stages"]
+    # ... one with 128-row panels against 128-column panels on four stages the 128 x 128 tile kernel (whole K tiles of 64 only)
+    assert rec["described_128_by_128_4_stages"] == ("maize_gemm_bf16_t128_nn" if k % 64 == 0 else "refused")
+    assert rec["mismatch_vs_described_128_by_128_4_stages"] == 0
     assert (rec["ragged_rows"], rec["ragged_cols"]) == (m % 256, n % 256)
     a, b = mz.gen.uniform_bf16(m * k, mz.gen.SEED_A), mz.gen.uniform_bf16(k * n, mz.gen.SEED_B)
     got = run_gemm(ctx, a, b, m, n, k)

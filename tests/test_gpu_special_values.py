@@ -28,6 +28,8 @@ FAMILIES = [
     ("maize_gemm_bf16_mt256_nn_ragged", 300, 4104, 192, NN), ("maize_gemm_bf16_mt256_nt_ragged", 260, 4112, 128, NT),
     # ... and with one to sixteen ragged last rows riding along
     ("maize_gemm_bf16_mt256_nn_ragged_m", 4099, 264, 192, NN), ("maize_gemm_bf16_mt256_nt_ragged_m", 4112, 304, 128, NT),
+    # 128 x 128 tiles on four ring stages: one and five K steps (the ring is primed with tiles past K), ragged M and N
+    ("maize_gemm_bf16_t128_nn", 300, 264, 64, NN), ("maize_gemm_bf16_t128_nt", 260, 136, 320, NT), ("maize_gemm_bf16_t128_nn", 130, 520, 320, NN),
     ("maize_gemm_bf16_mt256_nn_ktail", 300, 520, 264, NN),
     ("maize_gemm_bf16_mt256_nt_ktail", 257, 264, 328, NT),
     ("maize_gemm_bf16_mt256_nn_gen", 300, 520, 256, NN),
