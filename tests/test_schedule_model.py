@@ -383,6 +383,67 @@ def test_three_stage_checker_rejects_broken_schedules():
 
 
 # ---------------------------------------------------------------------------------------
+# 128 x 128 tiles (gemm_t128.hpp): four ring stages, eight pieces per wave and K tile.  A K step is two K halves of 16
+# MFMAs: K half 1's reads, K half 0's MFMAs with the pieces of tile t + 3 behind every second one, the wait that keeps
+# sixteen requests in flight, the barrier, K half 0's reads of tile t + 1, K half 1's MFMAs
+# ---------------------------------------------------------------------------------------
+T128_LINES = ("request(0u, 0u);", "request(BK, 1u);", "request(2u * BK, 2u);",
+              'asm volatile("s_waitcnt vmcnt(16)\\n\\ts_barrier" ::: "memory");\n    read_half(0, 0u);',
+              "const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;",
+              "read_half(1, so);",
+              "const TileReq r = tile_req((kt + 3u) * BK, (kt + 3u) & 3u);",
+              "if (j & 1) {\n                    piece(r, (4 * i + j) >> 1);",
+              'asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");\n        read_half(0, so_next);',
+              "for (int q = 0; q < 8; ++q) piece(r, q);")
+
+
+def t128_wave_program(nk, nt, keep=16, primed=3, ahead=3, reads_before_barrier=False, stages=4):
+    src = open(os.path.join(KDIR, "gemm_t128.hpp")).read()
+    for fact in T128_LINES:
+        assert fact in src, fact
+    assert int(re.search(r"constexpr int BT = 128, BK = 64, NS = (\d+);", src).group(1)) == 4
+    half = 8 if nt else 12                        # LDS reads of one K half: 4 of A + 4 of B, or 8 transposing ones
+    ops = [("dma", t, pc, t % stages) for t in range(primed) for pc in range(8)]
+    ops += [("wait_keep", keep), ("barrier",)]
+    ops += [("read", 0, 0, 0)] * half
+    for t in range(nk):
+        ops += [("read", t, 1, t % stages)] * half
+        for m in range(16):
+            ops.append(("mfma", t, 0))
+            if m & 1:
+                ops.append(("dma", t + ahead, m >> 1, (t + ahead) % stages))
+        if reads_before_barrier:
+            ops += [("read", t + 1, 0, (t + 1) % stages)] * half
+        ops += [("wait_keep", keep), ("barrier",)]
+        if not reads_before_barrier:
+            ops += [("read", t + 1, 0, (t + 1) % stages)] * half
+        ops += [("mfma", t, 1)] * 16
+    ops.append(("wait_all",))
+    return ops, nk
+
+
+@pytest.mark.parametrize("nk", [1, 2, 3, 4, 5, 7, 64])
+@pytest.mark.parametrize("nt", [False, True])
+def test_tiles_of_128_by_128_schedule_is_hazard_free(nk, nt):
+    ops, steps = t128_wave_program(nk, nt)
+    half = 8 if nt else 12
+    last_tile = check_two_stage(ops, steps, [half, 2 * half], parts=2, pieces=8, nst=4)
+    assert last_tile == steps + 2                       # tiles past the end are requested (zero-length descriptor) and read, never multiplied
+
+
+def test_tiles_of_128_by_128_checker_rejects_broken_schedules():
+    need = [8, 16]
+    with pytest.raises(Hazard):                 # a wait that leaves one request more in flight: the next tile's last piece may not have landed
+        check_two_stage(*t128_wave_program(9, True, keep=17), need, parts=2, pieces=8, nst=4)
+    with pytest.raises(Hazard):                 # the next tile read in front of the barrier: another wave's pieces may not have landed
+        check_two_stage(*t128_wave_program(9, True, reads_before_barrier=True), need, parts=2, pieces=8, nst=4)
+    with pytest.raises(Hazard):                 # a tile requested four steps ahead goes into the stage that is being read
+        check_two_stage(*t128_wave_program(9, True, ahead=4, primed=4, keep=24), need, parts=2, pieces=8, nst=4)
+    with pytest.raises(Hazard):                 # a ring primed with two tiles: the same wait no longer covers tile t + 1
+        check_two_stage(*t128_wave_program(9, True, primed=2, ahead=2), need, parts=2, pieces=8, nst=4)
+
+
+# ---------------------------------------------------------------------------------------
 # 128 x 256 tiles on 8-bit operands: a K tile is one matrix instruction deep, so a K step is the pair (A0, B0), (A0, B1)
 # with the barrier between the two; the second eighth reads the next tile's A0 (8 reads) and B0 (8, or 16 transposing
 # ones, two per slot); 12 pieces per wave and K tile, one per MFMA slot behind the barrier
