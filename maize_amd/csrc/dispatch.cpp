@@ -249,7 +249,7 @@ bool mt256_h128_plan(const maize_gemm_ex_desc_t& d, uint32_t compute_units, Laun
     return true;
 }
 bool mt256_edge_plan(const maize_gemm_ex_desc_t& d, uint32_t cus, LaunchDims* ld) { return mt256_plan_impl(d, cus, true, ld); }
-// 128 x 128 tiles (maize_gemm_bf16_t128_*): one workgroup per tile of the flattened (batch, tile) list.
+// 128 x 128 tiles (maize_gemm_{bf16,f16}_t128_*): one workgroup per tile of the flattened (batch, tile) list.
 bool t128_plan(const maize_gemm_ex_desc_t& d, uint32_t, LaunchDims* ld) {
     const Dims s = dims_of(d);
     const uint64_t all = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128) * d.gemm.batch;
@@ -944,6 +944,8 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_bf16_skinny_nn_m64", nullptr, skinny_nn_m64_supports, skinny_m64_plan},
     {"maize_gemm_bf16_t128_nn", nullptr, mt256_nn_gen_supports, t128_plan},
     {"maize_gemm_bf16_t128_nt", nullptr, mt256_nt_gen_supports, t128_plan},
+    {"maize_gemm_f16_t128_nn", nullptr, f16_nn_gen_supports, t128_plan},
+    {"maize_gemm_f16_t128_nt", nullptr, f16_nt_gen_supports, t128_plan},
     {"maize_gemm_bf16_mt256_nn_gen", nullptr, mt256_nn_gen_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nt_gen", nullptr, mt256_nt_gen_supports, mt256_plan},
     {"maize_gemm_bf16_mt256_nn_ktail_gen", nullptr, mt256_nn_ktail_gen_supports, mt256_plan},
@@ -1135,11 +1137,11 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // Not with a long K and few tiles, where the cut over K wins: 1024 x 2048 x 8192 44.6 against 56.1, 256 x 4096 x 4096
     // 23.4 against 29.6.)
     {
-        static const char* const kT128[2] = {"maize_gemm_bf16_t128_nn", "maize_gemm_bf16_t128_nt"};
-        const int t8 = kernel_index(kT128[s.nt]);
+        static const char* const kT128[2][2] = {{"maize_gemm_bf16_t128_nn", "maize_gemm_bf16_t128_nt"}, {"maize_gemm_f16_t128_nn", "maize_gemm_f16_t128_nt"}};
+        const int t8 = kernel_index(kT128[half_in(d)][s.nt]);
         const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
         const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128) * d.gemm.batch;
-        if (t8 >= 0 && !half_in(d) && s.k >= 128u && tiles <= units && kKernels[t8].supports(d)) {
+        if (t8 >= 0 && s.k >= 128u && tiles <= units && kKernels[t8].supports(d)) {
             double cost_t = 8.0 + t128_step(s.nt, tiles, cdiv(s.k, 64u)) * cdiv(s.k, 64u);
             const double st = stream_us(s, d.gemm.batch, 64u, tiles);
             const bool by_stream = cost_t < st;

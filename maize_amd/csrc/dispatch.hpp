@@ -12,7 +12,7 @@
 
 namespace maize {
 
-constexpr uint32_t kMaxKernels = 160;
+constexpr uint32_t kMaxKernels = 192;
 constexpr const char* kReduceKernel = "maize_gemm_splitk_reduce";
 constexpr const char* kPackKernel = "maize_pack_2d";
 constexpr const char* kPackKernelU8 = "maize_pack_2d_u8";

@@ -1,4 +1,4 @@
-// maize_gemm_bf16_t128_{nn,nt}: the pipelined tile kernel on 128 x 128 tiles of C.
+// maize_gemm_{bf16,f16}_t128_{nn,nt}: the pipelined tile kernel on 128 x 128 tiles of C.
 //
 // For products whose 128 x 256 tiles would occupy half of the compute units or less: four times as many tiles as
 // the 256 x 256 kernel has, one per workgroup, so the whole chip works on a product of 64 to 256 of them.  The
@@ -36,7 +36,8 @@ using mt256::OOB;
 constexpr int BT = 128, BK = 64, NS = 4;
 constexpr uint32_t STAGE = 16384;           // bytes of one operand tile
 
-template <bool NT>
+// F16: IEEE half operands (v_mfma_f32_16x16x32_f16; a 16-bit C is then half too): same tiles, same fragment maps.
+template <bool NT, bool F16 = false>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     __shared__ __attribute__((aligned(1024))) char lds_a[NS * STAGE];
     __shared__ __attribute__((aligned(1024))) char lds_b[NS * STAGE];
@@ -194,7 +195,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             for (int j = 0; j < 4; ++j) {
                 // B's fragment first: the lane ends up with 4 consecutive columns of one row of C
                 // (assembly with the accumulator tied to itself: the sixteen accumulators stay where they are)
-                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(0, j)), "v"(fa[0][i]));
+                if (F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(0, j)), "v"(fa[0][i]));
+                else     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(0, j)), "v"(fa[0][i]));
                 if (j & 1) {
                     piece(r, (4 * i + j) >> 1);
                     __builtin_amdgcn_sched_barrier(0);
@@ -206,7 +208,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(1, j)), "v"(fa[1][i]));
+                if (F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(1, j)), "v"(fa[1][i]));
+                else     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(1, j)), "v"(fa[1][i]));
         __builtin_amdgcn_sched_barrier(0);
     }
     // the trailing (empty) requests and the last reads (of a tile past K: never used) have landed before the registers
@@ -242,5 +245,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_t128_nn(GemmArgs p) { t128::body<false>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_t128_nt(GemmArgs p) { t128::body<true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_t128_nn(GemmArgs p) { t128::body<false, true>(p); }
+extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_t128_nt(GemmArgs p) { t128::body<true, true>(p); }
 
 }  // namespace maize

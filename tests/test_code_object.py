@@ -233,10 +233,11 @@ def test_main_loop_of_the_128_by_128_tile_kernels_is_lean(kernels):
     transposing ones), eight requests, one barrier whose wait leaves sixteen requests in flight.  Between a fragment
     read and the matrix instruction that takes it stands a wait and nothing else: no move of a fragment (the reads
     are assembly statements whose results the compiler believes ready at once; a move would copy them early)."""
-    for name, reads in (("maize_gemm_bf16_t128_nn", {"ds_read_b128": 8, "ds_read_b64_tr_b16": 16}), ("maize_gemm_bf16_t128_nt", {"ds_read_b128": 16})):
+    for name, reads in (("maize_gemm_bf16_t128_nn", {"ds_read_b128": 8, "ds_read_b64_tr_b16": 16}), ("maize_gemm_bf16_t128_nt", {"ds_read_b128": 16}),
+                        ("maize_gemm_f16_t128_nn", {"ds_read_b128": 8, "ds_read_b64_tr_b16": 16}), ("maize_gemm_f16_t128_nt", {"ds_read_b128": 16})):
         ins = kernels[name]
         idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
-        assert len(idx) == 32 and count(ins, "v_mfma_f32_16x16x32_bf16") == 32, name
+        assert len(idx) == 32 and count(ins, "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16") == 32, name
         body = ins[idx[0]:idx[-1] + 1]
         for mnemonic, n in reads.items():
             assert count(body, mnemonic) == n // 2, (name, mnemonic)          # (K half 0's reads of the next tile; K half 1's stand in front of the first MFMA)

@@ -203,7 +203,7 @@ def check_plan(p, m, n, k, layout, batch, cus=CUS):
             assert p["workspace_bytes"] < (1 << 31)
         else:
             assert p["workspace_bytes"] == 0
-    elif name.startswith("maize_gemm_bf16_t128_"):
+    elif name.startswith(("maize_gemm_bf16_t128_", "maize_gemm_f16_t128_")):
         # 128 x 128 tiles, one workgroup per tile of the flattened (batch, tile) list, whole K, no workspace
         assert p["block"] == (256, 1, 1) and (gy, gz) == (1, 1)
         assert gx == cdiv(m, 128) * cdiv(n, 128) * batch

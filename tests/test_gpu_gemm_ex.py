@@ -233,19 +233,19 @@ def test_half_height_tiles(ctx, oracle, layout):
         assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen3, label="h128r3 gen", **kw) == gen3
         assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=gen316, half=True, label="h128r3 gen half", **kw) == gen316
     # (the dispatcher's own choice: products of more than 256 tiles of 128 x 128 -- up to 256 of those go to the 128 x 128
-    # tile kernels, bf16 operands and whole K tiles only)
+    # tile kernels, 16-bit operands and whole K tiles only)
     t128 = f"maize_gemm_bf16_t128_{tag}"
     assert run_ex(ctx, oracle, 1152, 4096, 1024, layout=layout, label="h128r3 auto") == plain3
     assert run_ex(ctx, oracle, 1000, 2056, 1800, layout=layout, label="h128r3 auto tail") == gen3
     assert run_ex(ctx, oracle, 1152, 4096, 1024, layout=layout, alpha=0.5, beta=1.0, label="h128r3 auto scaled") == gen3
-    assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, half=True, label="h128r3 auto half") == gen316
+    assert run_ex(ctx, oracle, 1152, 4096, 1024, layout=layout, half=True, label="h128r3 auto half") == gen316
     assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, label="t128 auto") == t128
     assert run_ex(ctx, oracle, 1024, 2048, 2048, layout=layout, alpha=0.5, beta=1.0, label="t128 auto scaled") == t128
     # the dispatcher's choice
     assert run_ex(ctx, oracle, 1152, 4096, 512, layout=layout, label="h128 auto") == plain
     assert run_ex(ctx, oracle, 520, 776, 328, layout=layout, label="h128 auto tail") == gen
     assert run_ex(ctx, oracle, 1152, 4096, 512, layout=layout, alpha=0.5, beta=1.0, label="h128 auto scaled") == gen
-    assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, half=True, label="h128 auto half") == gen16
+    assert run_ex(ctx, oracle, 1152, 4096, 512, layout=layout, half=True, label="h128 auto half") == gen16
     assert run_ex(ctx, oracle, 512, 2048, 1024, layout=layout, out_f32=True, alpha=-2.0, beta=0.25, label="t128 auto fp32") == t128
     # batched, several tiles per workgroup: 5 x 640 x 768 in 128-row tiles = 75 tiles on the grid the plan gives
     from tests.gpu_util import run_gemm

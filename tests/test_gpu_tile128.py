@@ -39,6 +39,24 @@ def test_tiles_of_128_by_128_bit_for_bit(ctx, oracle, shape, layout):
         check_rows_against_oracle(oracle, got, a, b, m, n, k, sample_rows(m, count=8, tile=128)[:12], layout=layout, label=f"t128 {shape} {tag}")
 
 
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NN, mz.LAYOUT_NT], ids=["nn", "nt"])
+def test_half_operands_views_and_the_general_epilogue(ctx, oracle, layout):
+    """The same kernels on IEEE half operands (v_mfma_f32_16x16x32_f16), and both on views with leading dimensions,
+    alpha / beta and an fp32 C: the whole of C against the oracle, the padding of C's rows untouched."""
+    from tests.test_gpu_gemm_ex import run_ex
+    tag = "nt" if layout == mz.LAYOUT_NT else "nn"
+    for half in (False, True):
+        name = f"maize_gemm_{'f16' if half else 'bf16'}_t128_{tag}"
+        for (m, n, k) in ((256, 256, 64), (300, 264, 320), (520, 776, 192)):
+            bcols = n if layout == mz.LAYOUT_NN else k
+            for kw in (dict(), dict(lda=k + 8, ldb=bcols + 16, ldc=n + 8), dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8),
+                       dict(alpha=2.0, beta=0.0, c_nan=True), dict(lda=k + 3, ldb=bcols + 5)):
+                print(f"128 x 128 tiles: {name} {(m, n, k)} {kw}", flush=True)
+                assert run_ex(ctx, oracle, m, n, k, layout=layout, kernel=name, half=half, label=name, **kw) == name
+    # the dispatcher's own choice for half operands
+    assert run_ex(ctx, oracle, 1024, 2048, 1024, layout=layout, half=True, label="t128 auto half") == f"maize_gemm_f16_t128_{tag}"
+
+
 def test_the_dispatcher_takes_them_for_one_round_of_tiles(ctx):
     cus = ctx.info()["compute_units"]
     if cus != 256:
