@@ -1150,7 +1150,14 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
             // 384 x 4096 x 4096 N x K in four ranges 27.2 us measured, 30.4 by the model, 30.0 here; not where both are
             // bound by the operands' stream from HBM and the cut only adds its second launch: 128 x 28672 x 8192 N x K
             // 119.7 us in two ranges, 107.4 here, K x N 99.2 / 97.9)
-            if (cost_t < (hk >= 2u && !by_stream ? 0.92 : 0.97) * cost_hk) return (uint32_t)t8;
+            // (and the model prices long K ranges on nearly all compute units low: from 64 steps per range on more than 192
+            // work items the three-stage 128 x 256 tiles measure 0.66-0.74 per step, not 0.52 -- 512 x 8192 x 8192 N x K in two
+            // ranges 66.8-71.9 us, 57.6 by the model, 63.5 here; 2048 x 2048 x 8192 N x K 69.5, 62.5 here)
+            double rival = cost_hk;
+            const uint32_t per_range = hk >= 2u ? cdiv(cdiv(s.k, 64u), hk) : 0u;
+            const bool loaded = hk >= 2u && (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk > 192u && per_range >= 64u;
+            if (loaded && !by_stream) rival += 0.13 * per_range;
+            if (cost_t < (hk >= 2u && !by_stream && !loaded ? 0.92 : 0.97) * rival) return (uint32_t)t8;
         }
     }
     if (hk >= 2u) {
