@@ -377,6 +377,7 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     if (whole < stream_us(s, batch, kstep, half_tiles)) whole = stream_us(s, batch, kstep, half_tiles);
     double best = 0.9 * whole, best_cost = whole;                  // splitting has to win 10 %
     uint32_t best_ks = 1;
+    bool best_by_stream = false;
     const double elems = (double)s.m * s.n * batch;
     uint32_t kmax = (uint32_t)(resident / half_tiles);
     if (kmax > nk / 4u) kmax = nk / 4u;
@@ -396,14 +397,22 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
             const bool by_stream = ts > t;
             if (by_stream) t = ts;
             const double score = by_stream ? t * 0.9 / 0.95 : t;  // (what is compared with 0.9 x the whole tiles' cost)
-            if (score < best) { best = score; best_cost = t; best_ks = ks; }
+            if (score < best) { best = score; best_cost = t; best_ks = ks; best_by_stream = by_stream; }
         }
     best = best_cost;
+    // Long K ranges on most of the compute units: the three-stage tiles then measure 0.62-0.74 per step, not 0.52 (the
+    // operand panels no longer stay in the L2s).  Weighed as such against the 256-row kernels, whose shorter ranges do
+    // not: 768 x 4096 x 14336 in two ranges of 112 steps 97.5 us (N x K; 80.1 by the model), the 256-row kernel in five ranges
+    // 85.7; 1024 x 4096 x 14336 112.9 against 104.6 (K x N 112.0 / 103.2).  From 96 steps per range: at 86 the picture is mixed
+    // (768 x 4096 x 11008 79.0 against 73.4, but 1024 x 4096 x 11008 84.7 against more).
+    double weighed = best;
+    if (kstep == 64u && best_ks >= 2u && !best_by_stream && half_tiles * best_ks >= 192u && cdiv(nk, best_ks) >= 96u)
+        weighed += 0.10 * cdiv(nk, best_ks);
     // (a tie goes to the tiles: the model flatters large splits, 768 x 8192 x 8192 109.6 us in two ranges, 94.4 here; more
     // so with 8-bit operands, whose fixed terms it overrates: E4M3 N x K, 46 mid-size shapes with every candidate by name,
     // the two it gave to the 256-row split were both faster in tiles -- 256 x 2048 x 2048 18.5 against 14.3-15.9 us,
     // 768 x 4096 x 14336 55.4 against 50.1)
-    const bool tiles = best < (kstep == 128u ? 1.10 : 1.03) * other;
+    const bool tiles = weighed < (kstep == 128u ? 1.10 : 1.03) * other;
     if (cost && tiles) *cost = best;
     return tiles ? best_ks : 0u;
 }

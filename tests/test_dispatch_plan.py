@@ -311,8 +311,15 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
         assert mz.gemm_plan(desc(m, n, k, layout=mz.LAYOUT_NT), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nt"
         p = mz.gemm_plan(desc(m, n, k), compute_units=CUS)
         assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and p["ksplit"] == 2
-    p = mz.gemm_plan(desc(1024, 4096, 14336, layout=mz.LAYOUT_NT), compute_units=CUS)      # (107.0 us in two ranges, 110.6 in 128 x 128 tiles)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nt_h128r3_splitk" and p["ksplit"] == 2
+    # ... and against the 256-row kernels' shorter ranges, from 96 steps per range on (1024 x 4096 x 14336: two ranges of 112 steps
+    # 112.9 us, 128 x 128 tiles 110.6, the 256-row kernel in four ranges 104.6; 768 x 4096 x 14336 97.5 against 85.7 in five)
+    for layout, tag in ((mz.LAYOUT_NN, "nn"), (mz.LAYOUT_NT, "nt")):
+        p = mz.gemm_plan(desc(1024, 4096, 14336, layout=layout), compute_units=CUS)
+        assert p["kernel"] == f"maize_gemm_bf16_mt256_{tag}_splitk" and p["ksplit"] == 4
+        p = mz.gemm_plan(desc(768, 4096, 14336, layout=layout), compute_units=CUS)
+        assert p["kernel"] == f"maize_gemm_bf16_mt256_{tag}_splitk" and p["ksplit"] == 5
+        p = mz.gemm_plan(desc(1024, 4096, 11008, layout=layout), compute_units=CUS)        # (86 steps per range: stays; 84.7 us against more)
+        assert p["kernel"] == f"maize_gemm_bf16_mt256_{tag}_h128r3_splitk" and p["ksplit"] == 2
     p = mz.gemm_plan(desc(384, 6144, 4096), compute_units=CUS)                             # (three ranges 33 us; two 35; whole 39)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and p["ksplit"] == 3 and p["grid"] == (216, 1, 1)
     p = mz.gemm_plan(desc(384, 6144, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)        # (N x K: 144 tiles of 128 x 128 30.9 us, three ranges 31.5)
