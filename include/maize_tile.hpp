@@ -334,12 +334,12 @@ Accum gemm_smem_multibuffer(const MMA&, KTile<K_TILE>, const RowPanel<NA>& a, co
     // Generic in the ring depth and the panel height like the reference's mainloop ([TilePair; PIPE], KTile<N>,
     // gemm/mod.rs:37-45), within what kernels exist: 256- or 128-row panels of A on two stages, 128-row panels also on
     // three (a 128 x 256 tile's stage is 48 KiB; three fit the 160 KiB of LDS).
-    // ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages, 16-bit operands.
+    // ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages, 16-bit operands (8-bit ones with B stored N x K: stages F8_128x128).
     constexpr uint32_t NB = BPanel::WINDOW;
     constexpr bool QUARTER = NA == 128 && NB == 128;
     static_assert(QUARTER ? PIPE == 4 : (PIPE == 2 || PIPE == 3), "the macro-tile kernels run a ring of two or three stages, the 128 x 128 tile kernels one of four");
     static_assert((NA == 256 || NA == 128) && (NB == 256 || QUARTER), "the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B), or 128 rows and 128 columns");
-    static_assert(!QUARTER || MMA::IN_TYPE == MAIZE_IN_BF16 || MMA::IN_TYPE == MAIZE_IN_F16, "the 128 x 128 tile kernels take bf16 or half operands");
+    static_assert(!QUARTER || MMA::IN_TYPE == MAIZE_IN_BF16 || MMA::IN_TYPE == MAIZE_IN_F16 || NT, "the 128 x 128 tile kernels take 8-bit operands with B stored N x K only");
     static_assert(PIPE != 3 || NA == 128, "three ring stages fit the LDS with 128-row panels of A only");
     using TA = typename Pair::A::Ty; using TB = typename Pair::B::Ty;
     constexpr uint32_t ES = MMA::K_TILE == 128 ? 1 : 2;

@@ -157,6 +157,7 @@ bool f8_nn_common(const maize_gemm_ex_desc_t& d) {
 #define MAIZE_F8_SUPPORTS(tag, type) \
     bool tag##_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d) && plain_epilogue(d); } \
     bool tag##_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d); } \
+    bool tag##_t128_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d) && (dims_of(d).k & 127u) == 0; } \
     bool tag##_nn_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nn_common(d) && plain_epilogue(d); } \
     bool tag##_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nn_common(d); }
 MAIZE_F8_SUPPORTS(e4m3, MAIZE_IN_E4M3)
@@ -423,6 +424,13 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
 // 1024 x 4096 x 14336 110.6 / 129.2 -- where the three-stage 128 x 256 tiles' 0.52 measures 0.51.
 double t128_step(bool nt, uint64_t tiles, uint32_t nk) {
     return (nt ? 0.34 : 0.42) + (tiles > 192u ? 0.05 : tiles > 128u ? 0.02 : 0.0) + (nk >= 128u ? 0.04 : 0.0);
+}
+// ... on 8-bit operands (N x K; a step is 128 deep): the same bytes through the LDS per step, no conversion of halves in
+// the matrix pipe's way.  E4M3, uniform random operands, one box: 256 x 4096 x 4096 (64 tiles) 16.4 us, 512 x 4096 x 4096 17.0,
+// 768 x 4096 x 4096 17.9, 1024 x 4096 x 4096 19.1 (128 x 256 tiles on three stages: 22.3 / 23.3 / 23.9 / 25.1), 512 x 8192 x 8192
+// 32.1 (40.8 in two K ranges), 1024 x 4096 x 14336 52.9-55.5 (58.7).
+double t128_step8(uint64_t tiles, uint32_t nk) {
+    return 0.27 + (tiles > 192u ? 0.08 : tiles > 128u ? 0.04 : 0.0) + (nk >= 64u ? 0.05 : 0.0);
 }
 bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && bf16_in(d); }
 bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && bf16_in(d); }
@@ -987,6 +995,7 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_" #tag "_skinny_nn_m64", nullptr, tag##_skinny_nn_m64_supports, skinny_nt_m64_plan}, \
     {"maize_gemm_" #tag "_mt256_nt", nullptr, tag##_nt_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_gen", nullptr, tag##_nt_gen_supports, mt256_plan}, \
+    {"maize_gemm_" #tag "_t128_nt", nullptr, tag##_t128_nt_supports, t128_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan}, \
     {"maize_gemm_" #tag "_mt256_nn", nullptr, tag##_nn_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nn_gen", nullptr, tag##_nn_gen_supports, mt256_plan}, \
@@ -1057,6 +1066,17 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nt", kTag[d.in_type - MAIZE_IN_E4M3]);
         const int fk = kernel_index(name);
         if (fk >= 0 && kKernels[fk].supports(d) && s.n >= 64 && s.k >= 1024) return (uint32_t)fk;
+        // 17 .. 64 rows against many columns and a K of up to 4096: one round of 128 x 128 tiles streams B as fast and needs
+        // no second pass over partial tiles (E4M3 N x K, row-group kernel -> 128 x 128 tiles: 64 x 14336 x 4096 18.6 -> 16.5 us,
+        // 33 x 14336 x 4096 18.1 -> 15.4, 32 x 14336 x 4096 16.5 -> 15.2, 64 x 28672 x 4096 26.5 -> 21.0, 40 x 8192 x 2048 14.9 -> 9.5;
+        // not at K = 8192: 64 x 8192 x 8192 21.3 against 26.6, 64 x 14336 x 8192 level; nor with few columns: 17 x 4096 x 4096
+        // 12.6 against 15.0)
+        if (s.nt && s.m > 16u && s.m <= 64u && s.k >= 256u && s.k <= 4096u && s.n >= 8192u) {
+            std::snprintf(name, sizeof name, "maize_gemm_%s_t128_nt", kTag[d.in_type - MAIZE_IN_E4M3]);
+            const int t8 = kernel_index(name);
+            const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+            if (t8 >= 0 && kKernels[t8].supports(d) && (uint64_t)cdiv(s.n, 128) * d.gemm.batch <= units) return (uint32_t)t8;
+        }
         // 17 .. 64 rows: the same stream with 2 or 4 row groups (A through LDS), where B is what bounds the product.
         if (s.m > 16u && s.m <= 64u && s.k >= 2048u && s.n >= (s.m <= 32u ? 1024u : 8192u)) {   // (E4M3 64 x 8192 x 8192: K x N 19.9 us against 25.9 in 128-row tiles cut over K, N x K 21.5 / 22.9)
             std::snprintf(name, sizeof name, "maize_gemm_%s_skinny_nt_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.m <= 32u ? "m32" : "m64");
@@ -1072,9 +1092,21 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
             const int gm = kernel_index(name);
             if (gm >= 0 && kKernels[gm].supports(d) && plan_fits(kKernels[gm], d, compute_units)) return (uint32_t)gm;
         }
-        // Tiles of 128 x 256, whole or cut over K, where they beat the 256-row kernels (half a round of tiles or less).
+        // Tiles of 128 x 256, whole or cut over K, where they beat the 256-row kernels (half a round of tiles or less) -- or
+        // one round of 128 x 128 tiles (N x K, whole K tiles of 128) where the model has that beat both.
         {
-            const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units, 128);
+            double cost_hk = 0.0;
+            const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units, 128, &cost_hk);
+            std::snprintf(name, sizeof name, "maize_gemm_%s_t128_nt", kTag[d.in_type - MAIZE_IN_E4M3]);
+            const int t8 = kernel_index(name);
+            const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
+            const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128) * d.gemm.batch;
+            // (a long K on fewer than sixteen tiles is for the cut over K: one compute unit per tile walks it alone here)
+            if (t8 >= 0 && s.nt && s.k >= 256u && tiles <= units && (tiles >= 16u || s.k <= 1024u) && kKernels[t8].supports(d)) {
+                const uint32_t nk = cdiv(s.k, 128u);
+                const double cost_t = 8.0 + t128_step8(tiles, nk) * nk;
+                if (cost_t >= stream_us(s, d.gemm.batch, 128u, tiles) && cost_t < (hk >= 2u ? 0.92 : 0.97) * cost_hk) return (uint32_t)t8;
+            }
             if (hk >= 1u) {
                 const bool r3 = h128_three_stages(cdiv(cdiv(s.k, 128u), hk) * 128u, 128u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk);   // by the K steps of a range
                 std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_%s_h128%s_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.nt ? "nt" : "nn", r3 ? "r3" : "", hk >= 2u ? "splitk" : "gen");
@@ -1150,7 +1182,7 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         const int t8 = kernel_index(kT128[half_in(d)][s.nt]);
         const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
         const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128) * d.gemm.batch;
-        if (t8 >= 0 && s.k >= 128u && tiles <= units && kKernels[t8].supports(d)) {
+        if (t8 >= 0 && s.k >= 128u && tiles <= units && (tiles >= 16u || s.k <= 512u) && kKernels[t8].supports(d)) {
             double cost_t = 8.0 + t128_step(s.nt, tiles, cdiv(s.k, 64u)) * cdiv(s.k, 64u);
             const double st = stream_us(s, d.gemm.batch, 64u, tiles);
             const bool by_stream = cost_t < st;

@@ -1,4 +1,4 @@
-// maize_gemm_{bf16,f16}_t128_{nn,nt}: the pipelined tile kernel on 128 x 128 tiles of C.
+// maize_gemm_{bf16,f16}_t128_{nn,nt}, maize_gemm_{e4m3,e5m2,e4m3e5m2,e5m2e4m3}_t128_nt: the pipelined tile kernel on 128 x 128 tiles of C.
 //
 // For products whose 128 x 256 tiles would occupy half of the compute units or less: four times as many tiles as
 // the 256 x 256 kernel has, one per workgroup, so the whole chip works on a product of 64 to 256 of them.  The
@@ -19,9 +19,10 @@
 //   * the general epilogue of the 256-row kernels (alpha, beta, bf16 or fp32 C; common.hpp store_c_run) from fp32
 //     staging, 32 rows x 64 columns per pass and wave.
 //
-// Requirements (checked by the dispatcher): K % 64 == 0, N % 8 == 0, rows of C on 16-byte boundaries, K, N and the
+// Requirements (checked by the dispatcher): K % 64 == 0 (8-bit operands: K % 128 == 0 and 16-byte rows of A and B), N % 8 == 0, rows of C on 16-byte boundaries, K, N and the
 // leading dimensions below 2^21 elements.
 #pragma once
+#include <type_traits>
 #include "common.hpp"
 #include "gemm_mt256.hpp"
 #include "maps.hpp"
@@ -37,8 +38,18 @@ constexpr int BT = 128, BK = 64, NS = 4;
 constexpr uint32_t STAGE = 16384;           // bytes of one operand tile
 
 // F16: IEEE half operands (v_mfma_f32_16x16x32_f16; a 16-bit C is then half too): same tiles, same fragment maps.
-template <bool NT, bool F16 = false>
+// F8 >= 0: 8-bit operands stored N x K (one byte per element; bit 0: A is E5M2, bit 1: B is E5M2, else E4M3): the same 128-byte
+// rows hold 128 elements of K, a K tile is one v_mfma_f32_16x16x128_f8f6f4 deep, a fragment is the same two 16-byte reads.
+// A step then splits by accumulator rows, not K halves: rows 0-1 (A fragments 0, 1 and all of B: twelve reads), then
+// rows 2-3 (A fragments 2, 3: four reads).  B's fragments serve both, so the next tile's go into a second set of
+// registers: two steps per trip, the step count rounded up to an even number with a tile past K (zeros).
+template <bool NT, bool F16 = false, int F8 = -1>
 __device__ __forceinline__ void body(const GemmArgs& p) {
+    constexpr bool IS8 = F8 >= 0;
+    static_assert(!IS8 || (NT && !F16), "8-bit operands: both K-contiguous");
+    constexpr uint32_t ES = IS8 ? 1u : 2u;              // bytes per element of A and B
+    constexpr uint32_t CH = 16u / ES;                   // elements per 16-byte chunk
+    constexpr uint32_t BKE = IS8 ? 128u : (uint32_t)BK; // elements per K tile (128 bytes per row either way)
     __shared__ __attribute__((aligned(1024))) char lds_a[NS * STAGE];
     __shared__ __attribute__((aligned(1024))) char lds_b[NS * STAGE];
     __shared__ __attribute__((aligned(1024))) char lds_e[4 * 8192];
@@ -59,25 +70,25 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     uint32_t tile_m, tile_n;
     mt256::tile_of(t - bz * tiles_per, tm, tn, &tile_m, &tile_n);
     const uint32_t m0 = tile_m * BT, n0 = tile_n * BT;
-    const uint32_t nk = K / BK;
+    const uint32_t nk = K / BKE;
 
     auto span = [](uint64_t bytes) { return (uint32_t)(bytes < 0x7FFFFFFFull ? bytes : 0x7FFFFFFFull); };
     auto sc = [](uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane(x); };
     // Descriptors start at the tile's first row and end with the operand's view: rows at or past M (N) read as zeros.
-    const char* const Ag = (const char*)p.a + ((uint64_t)bz * p.stride_a + (uint64_t)m0 * lda) * 2u;
-    const uint32_t a_bytes = span(((uint64_t)(M - 1u - m0) * lda + K) * 2u);
-    const char* const Bg = NT ? (const char*)p.b + ((uint64_t)bz * p.stride_b + (uint64_t)n0 * ldb) * 2u
+    const char* const Ag = (const char*)p.a + ((uint64_t)bz * p.stride_a + (uint64_t)m0 * lda) * ES;
+    const uint32_t a_bytes = span(((uint64_t)(M - 1u - m0) * lda + K) * ES);
+    const char* const Bg = NT ? (const char*)p.b + ((uint64_t)bz * p.stride_b + (uint64_t)n0 * ldb) * ES
                               : (const char*)p.b + (uint64_t)bz * p.stride_b * 2u;
-    const uint32_t b_bytes = NT ? span(((uint64_t)(N - 1u - n0) * ldb + K) * 2u) : 0u;
+    const uint32_t b_bytes = NT ? span(((uint64_t)(N - 1u - n0) * ldb + K) * ES) : 0u;
     const uint64_t b_view = ((uint64_t)(K - 1u) * ldb + N) * 2u;              // bytes of a K x N B
     // The lane's byte offsets of its four requests per operand and K tile (pieces 4 wave .. 4 wave + 3), at k = 0.
     uint32_t a_vo[4], b_vo[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t pc = wave * 4u + i;
-        a_vo[i] = (maps::kc_piece_row(pc, lane) * lda + maps::kc_piece_chunk(pc, lane) * 8u) * 2u;
+        a_vo[i] = (maps::kc_piece_row(pc, lane) * lda + maps::kc_piece_chunk(pc, lane) * CH) * ES;
         if (NT) {
-            b_vo[i] = (maps::kc_piece_row(pc, lane) * ldb + maps::kc_piece_chunk(pc, lane) * 8u) * 2u;
+            b_vo[i] = (maps::kc_piece_row(pc, lane) * ldb + maps::kc_piece_chunk(pc, lane) * CH) * ES;
         } else {
             const uint32_t col = n0 + maps::sk128_piece_chunk(pc, lane) * 8u;
             b_vo[i] = ((maps::sk128_piece_row(pc, lane) * ldb + col) * 2u) | (col < N ? 0u : OOB);
@@ -92,7 +103,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         TileReq r;
         const bool live = k < K;
         r.ra = make_rsrc(Ag, live ? a_bytes : 0u);
-        r.a_so = sc(k * 2u);
+        r.a_so = sc(k * ES);
         if (NT) {
             r.rb = make_rsrc(Bg, live ? b_bytes : 0u);
             r.b_so = r.a_so;
@@ -131,7 +142,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     }
 
 #define MAIZE_RD_CASE(n) case n: asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(base), "n"((n) * 2048)); break;
-    auto rd128 = [&](bf16x8& dst, uint32_t base, int n) {
+    auto rd128 = [&](auto& dst, uint32_t base, int n) {
         switch (n) { MAIZE_RD_CASE(0) MAIZE_RD_CASE(1) MAIZE_RD_CASE(2) MAIZE_RD_CASE(3) }
     };
 #undef MAIZE_RD_CASE
@@ -174,9 +185,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
 
     // ---- prime the ring: tiles 0, 1, 2; K half 0 of tile 0 on its way to the registers ----------
     request(0u, 0u);
-    request(BK, 1u);
-    request(2u * BK, 2u);
+    request(BKE, 1u);
+    request(2u * BKE, 2u);
     asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+    if constexpr (!IS8) {
     read_half(0, 0u);
 
     // A step: K half 1's reads go out, K half 0's MFMAs run with the eight requests of tile t + 3 between them (into the
@@ -188,7 +200,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;
         read_half(1, so);
         if (NT) asm volatile("s_waitcnt lgkmcnt(8)"); else asm volatile("s_waitcnt lgkmcnt(12)");      // K half 0 has arrived
-        const TileReq r = tile_req((kt + 3u) * BK, (kt + 3u) & 3u);
+        const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -211,6 +223,65 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 if (F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(1, j)), "v"(fa[1][i]));
                 else     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(1, j)), "v"(fa[1][i]));
         __builtin_amdgcn_sched_barrier(0);
+    }
+    } else {
+        // ---- 8-bit operands ---------------------------------------------------------------------
+        typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+        typedef int i32x8 __attribute__((ext_vector_type(8)));
+        u32x4v a8[4][2];                 // A fragment f, 16-byte chunk kh (the lane's chunks l/16 and 4 + l/16 of its row)
+        u32x4v b8[2][4][2];              // B: register set, fragment, chunk
+        auto operand8 = [](const u32x4v (&f)[2]) -> i32x8 {
+            return i32x8{(int)f[0][0], (int)f[0][1], (int)f[0][2], (int)f[0][3], (int)f[1][0], (int)f[1][1], (int)f[1][2], (int)f[1][3]};
+        };
+        auto read_a = [&](int f0, uint32_t so) {
+#pragma unroll
+            for (int f = f0; f < f0 + 2; ++f)
+#pragma unroll
+                for (int kh = 0; kh < 2; ++kh) rd128(a8[f][kh], a_rd[kh] + so, f);
+        };
+        auto read_b = [&](auto set, uint32_t so) {
+            constexpr int S = decltype(set)::value;
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+#pragma unroll
+                for (int kh = 0; kh < 2; ++kh) rd128(b8[S][f][kh], b_rd[kh] + so, f);
+        };
+        // B first, so cbsz carries B's format and blgp A's (0 = E4M3, 1 = E5M2)
+        auto mfma8 = [&](floatx4& c, const u32x4v (&b)[2], const u32x4v (&a)[2]) {
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(c) : "v"(operand8(b)), "v"(operand8(a)), "n"((F8 >> 1) & 1), "n"(F8 & 1));
+        };
+        read_a(0, 0u);
+        read_b(std::integral_constant<int, 0>{}, 0u);
+        // A step: A fragments 2, 3 are read, rows 0-1 multiply (their twelve reads went out half a step ago) with the eight
+        // requests of tile t + 3 between the MFMAs; the wait and the barrier as above; the next tile's A fragments 0, 1 and B
+        // fragments (into the other register set) are read while rows 2-3 multiply.
+        auto step8 = [&](auto set, uint32_t kt) {
+            constexpr int S = decltype(set)::value;
+            const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;
+            read_a(2, so);
+            asm volatile("s_waitcnt lgkmcnt(4)");
+            const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    mfma8(acc[i][j], b8[S][j], a8[i]);
+                    piece(r, 4 * i + j);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            read_a(0, so_next);
+            read_b(std::integral_constant<int, 1 - S>{}, so_next);
+#pragma unroll
+            for (int i = 2; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) mfma8(acc[i][j], b8[S][j], a8[i]);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        for (uint32_t kt = 0; kt < nk; kt += 2u) {
+            step8(std::integral_constant<int, 0>{}, kt);
+            step8(std::integral_constant<int, 1>{}, kt + 1u);
+        }
     }
     // the trailing (empty) requests and the last reads (of a tile past K: never used) have landed before the registers
     // and the LDS are given up
@@ -247,5 +318,13 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_t128_nn(GemmAr
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_t128_nt(GemmArgs p) { t128::body<true>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_t128_nn(GemmArgs p) { t128::body<false, true>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_t128_nt(GemmArgs p) { t128::body<true, true>(p); }
+// 8-bit operands, B stored N x K (A's format, B's format: 0 = E4M3, 1 = E5M2)
+#define MAIZE_T128_F8(tag, fa, fb) \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_t128_nt(GemmArgs p) { t128::body<true, false, (fa) | ((fb) << 1)>(p); }
+MAIZE_T128_F8(e4m3, 0, 0)
+MAIZE_T128_F8(e5m2, 1, 1)
+MAIZE_T128_F8(e4m3e5m2, 0, 1)
+MAIZE_T128_F8(e5m2e4m3, 1, 0)
+#undef MAIZE_T128_F8
 
 }  // namespace maize

@@ -93,6 +93,19 @@ def test_matrix_instruction_per_kernel(kernels):
                 assert len(f8) >= 8 and all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
             assert count(ins, "ds_read_b128") >= 16 and count(ins, "ds_read_b64_tr_b16") == 0, name
             assert len([i for i in ins if i.startswith("buffer_load_dwordx4") and " lds" in i]) >= 16, name
+        elif name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")) and "_t128_" in name:
+            # 8-bit operands on 128 x 128 tiles: two K steps of 16 MFMAs per trip (B's fragments alternate between two register sets)
+            f8 = [i for i in ins if i.startswith("v_mfma_f32_16x16x128_f8f6f4")]
+            assert len(f8) == 32 and count(ins, "v_mfma") == 32, name
+            tag = name[len("maize_gemm_"):].split("_")[0]
+            a_e5m2, b_e5m2 = {"e4m3": (0, 0), "e5m2": (1, 1), "e4m3e5m2": (0, 1), "e5m2e4m3": (1, 0)}[tag]
+            assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
+            idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
+            body = ins[idx[0]:idx[-1] + 1]
+            assert count(body, "ds_read_b128") == 32 - 4 and count(body, "buffer_load_dwordx4") == 16 and count(body, "s_barrier") == 2, name   # (the trip's first four reads stand in front of its first MFMA)
+            assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(16)" in i) == 2, name
+            moves = [i for i in body if i.startswith(("v_mov", "v_accvgpr", "v_perm", "v_pk_", "v_lshl", "v_bfi", "v_alignbit"))]
+            assert not moves, (name, moves[:5])                               # (no move of a fragment between its read and its MFMA)
         elif name.startswith(("maize_gemm_e4m3", "maize_gemm_e5m2")):
             # 8-bit operands: the 128-deep 16 x 16 instruction (cheaper per multiply-add at the power limit than 32 x 32 x 64).
             # B is fed as the first source, so cbsz carries B's format code and blgp A's (E4M3 = 0 is not printed, E5M2 = 1).

@@ -175,7 +175,8 @@ def test_dispatch_of_8bit_operands():
         assert plan["kernel"] == name and tuple(plan["grid"]) == (256, 1, 1) and plan["workspace_bytes"] == 0
         general = ex(**big, in_type=it, alpha=2.0, beta=1.0, out_type=mz.OUT_F32)
         assert mz.gemm_plan(general)["kernel"] == name + "_gen"
-        half_tiles = (name + "_h128_gen", name + "_h128r3_gen", name + "_h128_splitk", name + "_h128r3_splitk")   # the same on tiles of 128 x 256 (two or three ring stages)
+        half_tiles = (name + "_h128_gen", name + "_h128r3_gen", name + "_h128_splitk", name + "_h128r3_splitk",   # the same on tiles of 128 x 256 (two or three ring stages)
+                      name.replace("_mt256_nt", "_t128_nt"))                                                   # ... and of 128 x 128 (K % 128 == 0)
         for other in mz.kernel_names():
             assert _supports(other, x) == (other in (name, name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32") + half_tiles), other
             assert _supports(other, general) == (other in (name + "_gen", name + "_splitk", name + "_packed", "maize_gemm_bf16_wave32") + half_tiles), other
@@ -204,10 +205,18 @@ def test_dispatch_of_8bit_operands():
         assert split["workspace_bytes"] == 65536 + split["ksplit"] * 128 * 256 * 4
         skinny = name.replace("_mt256_nt", "_skinny_nt")
         assert mz.gemm_plan(ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny          # M <= 16: B streamed once
-        assert mz.gemm_plan(ex(17, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m32"    # 17 .. 64 rows: row groups
-        assert mz.gemm_plan(ex(64, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m64"
-        assert mz.gemm_plan(ex(64, 4096, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_h128_splitk"     # few slabs
-        assert mz.gemm_plan(ex(65, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_h128_splitk"
+        assert mz.gemm_plan(ex(17, 14336, 8192, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m32"    # 17 .. 64 rows: row groups
+        assert mz.gemm_plan(ex(64, 14336, 8192, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m64"
+        assert mz.gemm_plan(ex(17, 4096, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == skinny + "_m32"
+        quarter = name.replace("_mt256_nt", "_t128_nt")                                                           # ... up to K = 4096 against 8192 columns or more: one round of 128 x 128 tiles
+        assert mz.gemm_plan(ex(17, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == quarter
+        assert mz.gemm_plan(ex(64, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == quarter
+        assert mz.gemm_plan(ex(1024, 4096, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == quarter          # and for one round of 64 to 256 of them
+        assert mz.gemm_plan(ex(1024, 4096, 4096, layout=mz.LAYOUT_NT, in_type=it, alpha=0.5, beta=1.0, out_type=mz.OUT_F32))["kernel"] == quarter
+        assert mz.gemm_plan(ex(64, 8192, 8192, layout=mz.LAYOUT_NT, in_type=it, ldc=8200))["kernel"] in (skinny + "_m64", name + "_h128_splitk", name + "_h128r3_splitk")
+        assert mz.gemm_plan(ex(100, 8192, 8192, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == name + "_h128_splitk"   # a long K on few tiles: 128 x 256 tiles cut over K (25.5 us; 128 x 128 tiles 27.3)
+        assert mz.gemm_plan(ex(64, 4096, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == quarter                 # few slabs (16.1 us; cut over K 15.1-15.6)
+        assert mz.gemm_plan(ex(65, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it))["kernel"] == quarter                # (16.4 us; cut over K 20.0)
         assert _supports(skinny, ex(16, 14336, 4096, layout=mz.LAYOUT_NT, in_type=it)) and not _supports(skinny, x)
         # the same rows against a row-major (K x N) B: the streaming kernels with transposing LDS reads (N % 16 == 0)
         few_nn = name.replace("_mt256_nt", "_skinny_nn")

@@ -395,7 +395,10 @@ def test_half_height_tiles_on_8bit_operands(ctx, oracle, fmt):
         for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=792), dict(lda=416, ldb=bcols + 16, ldc=800), dict(out_f16=True)):
             assert run_f8(ctx, oracle, 520, 784, 400, layout=layout, fmt=fmt, kernel=gen, label="h128 f8 knobs", **kw) == gen
             assert run_f8(ctx, oracle, 520, 784, 400, layout=layout, fmt=fmt, kernel=gen3, label="h128r3 f8 knobs", **kw) == gen3
-        assert run_f8(ctx, oracle, 512, 2048, 1024, layout=layout, fmt=fmt, label="h128 f8 auto") == gen
+        # (the dispatcher's own choice: N x K products of up to 256 tiles of 128 x 128 and whole K tiles of 128 go to the 128 x 128
+        # tile kernels, tests/test_gpu_tile128.py)
+        auto = (1152, 4096, 1024) if layout == mz.LAYOUT_NT else (512, 2048, 1024)
+        assert run_f8(ctx, oracle, *auto, layout=layout, fmt=fmt, label="h128 f8 auto") == gen
         assert run_f8(ctx, oracle, 100, 2048, 8192, layout=layout, fmt=fmt, label="h128 f8 auto, cut over K") == split
         m, n, k = 640, 784, 1168
         a = f8_uniform(oracle, m * k, 91, elem[0])
@@ -418,8 +421,11 @@ def test_dispatch_of_8bit_products(ctx):
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nt"
     assert pick(4096, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn"          # row-major B: read where it lies
     assert pick(4096, 4104, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_trb"      # ... N % 16: transposed copy
-    assert pick(2048, 2048, 2048, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_h128_gen"      # half a round of 128-row tiles, 16 K steps
-    assert pick(1024, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_h128r3_gen"    # ... 32 K steps: three ring stages
+    assert pick(2048, 2048, 2048, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn_h128_gen"      # half a round of 128-row tiles, 16 K steps
+    assert pick(1024, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn_h128r3_gen"    # ... 32 K steps: three ring stages
+    assert pick(2048, 2048, 2048, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_t128_nt"                # N x K: one round of 256 tiles of 128 x 128 (16.3 -> 12.0 us)
+    assert pick(1024, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_t128_nt"                # (25.1 -> 19.1 us)
+    assert pick(1536, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_h128r3_gen"    # 384 of them would be two rounds
     assert pick(1024, 4096, 2304, mz.LAYOUT_NN, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nn_h128r3_gen"    # (from 18 steps on)
     assert pick(4096, 4096, 4104, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_packed"   # K % 16: padded copies
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3, lda=4104) == "maize_gemm_e4m3_mt256_nt_packed"
@@ -464,7 +470,10 @@ def test_split_k_on_8bit_operands(ctx, oracle, fmt):
     name = f"maize_gemm_{fmt}_mt256_nt_splitk"
     half_tiles = f"maize_gemm_{fmt}_mt256_nt_h128_splitk"
     for (m, n, k) in ((24, 520, 4096), (64, 512, 8192), (256, 256, 16384)):        # more than 16 rows and few columns: not the streaming kernels'
-        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="f8 split-K") == half_tiles
+        # (a long K on fewer than four tiles of 128 x 128, or by the model: the cut over K; 24 x 520 x 4096 is five tiles and
+        # goes to them)
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, label="f8 split-K") in (half_tiles, f"maize_gemm_{fmt}_t128_nt")
+        assert run_f8(ctx, oracle, m, n, k, fmt=fmt, kernel=half_tiles, label="f8 split-K, 128-row tiles") == half_tiles
         assert run_f8(ctx, oracle, m, n, k, fmt=fmt, kernel=name, label="f8 split-K, 256-row tiles") == name
     for kern in (name, half_tiles):
         assert run_f8(ctx, oracle, 40, 264, 2064, fmt=fmt, kernel=kern, label="f8 split-K ragged K") == kern
@@ -507,7 +516,8 @@ def test_operands_of_different_8bit_formats(ctx, oracle, fmt):
     assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, kernel=name, label="mixed plain") == name
     assert run_f8(ctx, oracle, 300, 520, 144, fmt=fmt, alpha=-1.25, beta=0.75, kernel=name + "_gen", label="mixed gen") == name + "_gen"
     assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, kernel=name + "_splitk", label="mixed split-K") == name + "_splitk"
-    assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, label="mixed, 128-row tiles") == name + "_h128_gen"      # what the dispatcher takes for these
+    assert run_f8(ctx, oracle, 512, 768, 400, fmt=fmt, label="mixed, 128-row tiles") == name + "_h128_gen"      # what the dispatcher takes for these (K % 128 != 0)
+    assert run_f8(ctx, oracle, 512, 768, 384, fmt=fmt, label="mixed, 128 x 128 tiles") == name.replace("_mt256_nt", "_t128_nt")
     assert run_f8(ctx, oracle, 64, 512, 8192, fmt=fmt, label="mixed split-K, 128-row tiles") == name + "_h128_splitk"
     m = n = k = 256
     a = f8_uniform(oracle, m * k, 41, 2)
@@ -560,7 +570,8 @@ def test_packed_path_for_8bit_operands(ctx, oracle, fmt):
 @pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2"])
 @pytest.mark.parametrize("case", [
     # (M, N, K, layout, leading dimensions or None, alpha, beta, kernel family expected in the name)
-    (512, 768, 384, mz.LAYOUT_NT, None, 1.0, 0.0, "mt256_nt_h128_gen"),
+    (512, 768, 384, mz.LAYOUT_NT, None, 1.0, 0.0, "t128_nt"),
+    (512, 768, 400, mz.LAYOUT_NT, None, 1.0, 0.0, "mt256_nt_h128_gen"),
     (300, 520, 144, mz.LAYOUT_NT, (160, 176, 528), -0.75, 0.5, "mt256_nt_h128_gen"),
     (2048, 4352, 256, mz.LAYOUT_NT, None, 1.0, 0.0, "mt256_nt_gen"),
     (256, 512, 8192, mz.LAYOUT_NT, None, 1.0, 0.0, "splitk"),

@@ -148,4 +148,5 @@ def test_row_groups_8bit_operands(ctx, oracle, fmt):
     assert run_f8(ctx, oracle, 40, 1096, 4096, fmt=fmt, lda=4112, ldb=4224, ldc=1104, kernel=name, label="views") == name
     assert run_f8(ctx, oracle, 40, 1001, 4096, fmt=fmt, alpha=-1.25, beta=0.75, kernel=name, label="scaled, odd N") == name
     assert run_f8(ctx, oracle, 40, 1096, 4096, fmt=fmt, out_f32=True, alpha=3.0, beta=-0.5, kernel=name, label="f32") == name
-    assert run_f8(ctx, oracle, 32, 14336, 4096, fmt=fmt, label="auto") == _rows_kernel(fmt, 32)
+    assert run_f8(ctx, oracle, 32, 14336, 8192, fmt=fmt, label="auto") == _rows_kernel(fmt, 32)
+    assert run_f8(ctx, oracle, 32, 14336, 4096, fmt=fmt, label="auto, K up to 4096: 128 x 128 tiles") == f"maize_gemm_{fmt}_t128_nt"

@@ -387,14 +387,61 @@ def test_three_stage_checker_rejects_broken_schedules():
 # MFMAs: K half 1's reads, K half 0's MFMAs with the pieces of tile t + 3 behind every second one, the wait that keeps
 # sixteen requests in flight, the barrier, K half 0's reads of tile t + 1, K half 1's MFMAs
 # ---------------------------------------------------------------------------------------
-T128_LINES = ("request(0u, 0u);", "request(BK, 1u);", "request(2u * BK, 2u);",
-              'asm volatile("s_waitcnt vmcnt(16)\\n\\ts_barrier" ::: "memory");\n    read_half(0, 0u);',
+T128_LINES = ("request(0u, 0u);", "request(BKE, 1u);", "request(2u * BKE, 2u);",
+              'asm volatile("s_waitcnt vmcnt(16)\\n\\ts_barrier" ::: "memory");\n    if constexpr (!IS8) {\n    read_half(0, 0u);',
               "const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;",
               "read_half(1, so);",
-              "const TileReq r = tile_req((kt + 3u) * BK, (kt + 3u) & 3u);",
+              "const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);\n#pragma unroll\n        for (int i = 0; i < 4; ++i)",
               "if (j & 1) {\n                    piece(r, (4 * i + j) >> 1);",
               'asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");\n        read_half(0, so_next);',
               "for (int q = 0; q < 8; ++q) piece(r, q);")
+
+
+# ... on 8-bit operands: a step splits by accumulator rows -- rows 0-1 need A fragments 0, 1 and all of B (12 reads, issued
+# behind the barrier of the step before), rows 2-3 A fragments 2, 3 (4 reads, issued at the top of the step); one request
+# behind each of the first eight MFMAs; two steps per trip, the count rounded up to an even number with a tile past K
+T128_F8_LINES = ("read_a(0, 0u);\n        read_b(std::integral_constant<int, 0>{}, 0u);",
+                 "read_a(2, so);\n            asm volatile(\"s_waitcnt lgkmcnt(4)\");\n            const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);",
+                 "mfma8(acc[i][j], b8[S][j], a8[i]);\n                    piece(r, 4 * i + j);",
+                 'asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");\n            read_a(0, so_next);\n            read_b(std::integral_constant<int, 1 - S>{}, so_next);',
+                 "for (uint32_t kt = 0; kt < nk; kt += 2u) {\n            step8(std::integral_constant<int, 0>{}, kt);\n            step8(std::integral_constant<int, 1>{}, kt + 1u);")
+
+
+def t128_f8_wave_program(nk, keep=16, reads_before_barrier=False, late_rows=4):
+    src = open(os.path.join(KDIR, "gemm_t128.hpp")).read()
+    for fact in T128_LINES + T128_F8_LINES:
+        assert fact in src, fact
+    steps = nk + (nk & 1)
+    ops = [("dma", t, pc, t % 4) for t in range(3) for pc in range(8)]
+    ops += [("wait_keep", keep), ("barrier",)]
+    ops += [("read", 0, 0, 0)] * 12
+    for t in range(steps):
+        ops += [("read", t, 1, t % 4)] * late_rows
+        for m in range(8):
+            ops += [("mfma", t, 0), ("dma", t + 3, m, (t + 3) % 4)]
+        if reads_before_barrier:
+            ops += [("read", t + 1, 0, (t + 1) % 4)] * 12
+        ops += [("wait_keep", keep), ("barrier",)]
+        if not reads_before_barrier:
+            ops += [("read", t + 1, 0, (t + 1) % 4)] * 12
+        ops += [("mfma", t, 1)] * 8
+    ops.append(("wait_all",))
+    return ops, steps
+
+
+@pytest.mark.parametrize("nk", [1, 2, 3, 4, 5, 8, 33])
+def test_tiles_of_128_by_128_8bit_schedule_is_hazard_free(nk):
+    ops, steps = t128_f8_wave_program(nk)
+    assert check_two_stage(ops, steps, [12, 16], parts=2, pieces=8, nst=4) == steps + 2
+
+
+def test_tiles_of_128_by_128_8bit_checker_rejects_broken_schedules():
+    with pytest.raises(Hazard):                 # a wait that leaves one request more in flight
+        check_two_stage(*t128_f8_wave_program(9, keep=17), [12, 16], parts=2, pieces=8, nst=4)
+    with pytest.raises(Hazard):                 # the next tile read in front of the barrier
+        check_two_stage(*t128_f8_wave_program(9, reads_before_barrier=True), [12, 16], parts=2, pieces=8, nst=4)
+    with pytest.raises(Hazard):                 # A fragment 3's reads dropped: rows 2-3 multiply stale registers
+        check_two_stage(*t128_f8_wave_program(9, late_rows=2), [12, 16], parts=2, pieces=8, nst=4)
 
 
 def t128_wave_program(nk, nt, keep=16, primed=3, ahead=3, reads_before_barrier=False, stages=4):

@@ -147,6 +147,10 @@ def test_the_description_chooses_the_panel_height_and_the_ring_depth():
     a, b, c = matrices(4096, 4096, 4096, nt=True)
     got = describe(a, b, c, nt=True, tiles=(T.BF16_128x64, T.BF16_128x64), **q128)[0].finalize().compile(mz.Gfx.Gfx950, cus)
     assert got.kernel_name == got.forced == "maize_gemm_bf16_t128_nt" and got.plan["grid"] == (1024, 1, 1)
+    am, bm, cm = matrices(1024, 4096, 4096, nt=True)
+    am.elem_bytes = bm.elem_bytes = 1
+    k8, _ = describe(am, bm, cm, mma=T.Gfx950MfmaE4M3E5M2F32_16x16x128, nt=True, ktile=128, tiles=(T.F8_128x128, T.F8_128x128), **q128)
+    assert k8.finalize().compile(mz.Gfx.Gfx950, cus).kernel_name == "maize_gemm_e4m3e5m2_t128_nt"
     with pytest.raises(ValueError, match="ring of four stages"):
         describe(a, b, c, nt=True, tiles=(T.BF16_128x64, T.BF16_128x64), depth=3, a_panel=128, panel=128)
     with pytest.raises(ValueError, match="B stage is BF16_128x64"):                     # K x N B needs the K x N stage
