@@ -69,6 +69,9 @@ CONFIGS = {
     # ... and the decode-style shape of cfg4 against 8-bit weights stored N x K.
     "f8s": dict(m=16, n=14336, k=4096, nt=1, batch=1, da=("uniform",), db=("uniform",), bound="hbm", in_type="e4m3",
                 label="E4M3 GEMM 16x14336x4096 NT skinny (bf16 C), uniform[-1,1) rounded to E4M3"),
+    # ... and the 8-bit twin of "mid": a prefill of 1024 tokens against 8-bit 4096 x 4096 weights stored N x K.
+    "f8mid": dict(m=1024, n=4096, k=4096, nt=1, batch=1, da=("uniform",), db=("uniform",), bound="mfma", in_type="e4m3",
+                  label="E4M3 GEMM 1024x4096x4096 NT (bf16 C), uniform[-1,1) rounded to E4M3"),
     # The catalogue's fp32 and fp64 entries (v_mfma_f32_16x16x4_f32, v_mfma_f64_16x16x4_f64), C in the operands' type.
     "f32": dict(m=4096, n=4096, k=4096, nt=0, batch=1, da=("uniform",), db=("uniform",), bound="mfma", in_type="f32",
                 label="fp32 GEMM 4096x4096x4096 NN (fp32 C), uniform[-1,1)"),
@@ -390,6 +393,7 @@ def main():
     ap.add_argument("--shape", default=None, help="M,N,K[,batch]: a bf16 product of that shape instead of a named configuration "
                                                    "(uniform[-1,1) operands; --layout says how B is stored)")
     ap.add_argument("--layout", default="nn", choices=["nn", "nt"], help="--shape: B stored K x N (nn) or N x K (nt)")
+    ap.add_argument("--in-type", default="bf16", choices=["bf16", "e4m3", "e5m2"], help="--shape: element type of A and B")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--others", action=argparse.BooleanOptionalAction, default=None,
                     help="also measure the other benchmark configurations (shorter runs) and report them under "
@@ -412,7 +416,9 @@ def main():
         m_, n_, k_ = dims[:3]
         batch_ = dims[3] if len(dims) > 3 else 1
         CONFIGS["custom"] = dict(m=m_, n=n_, k=k_, nt=int(args.layout == "nt"), batch=batch_, da=("uniform",), db=("uniform",), bound="mfma",
-                                 label=f"bf16 GEMM {'%d x ' % batch_ if batch_ > 1 else ''}{m_}x{n_}x{k_} {args.layout.upper()}, uniform[-1,1)")
+                                 label=f"{args.in_type} GEMM {'%d x ' % batch_ if batch_ > 1 else ''}{m_}x{n_}x{k_} {args.layout.upper()}, uniform[-1,1)")
+        if args.in_type != "bf16":
+            CONFIGS["custom"]["in_type"] = args.in_type
         args.config, args.others = "custom", False
     args.config = args.config or "cfg1"
     if args.config == "copy":
