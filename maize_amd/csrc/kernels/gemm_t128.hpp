@@ -12,8 +12,8 @@
 //   * a step is two K halves of 16 MFMAs.  The eight requests of tile t + 3 go out between K half 0's MFMAs, into the
 //     stage step t - 1 read; the barrier stands between the halves -- behind it tile t + 1 has landed and nobody reads
 //     tile t any more -- and leaves the sixteen requests of tiles t + 2 and t + 3 in flight; each half's fragments are
-//     read while the other half's MFMAs run.  Requests past K go through an empty descriptor (zeros, no memory
-//     traffic), so every step issues and waits for the same number;
+//     read while the other half's MFMAs run, one read (K x N: two) behind each of its first MFMAs.  Requests past K go
+//     through an empty descriptor (zeros, no memory traffic), so every step issues and waits for the same number;
 //   * a step reads 16 KiB of fragments per wave for 32 MFMAs: the LDS port (64 KiB read + 32 KiB deposited per step
 //     and compute unit), not the matrix pipe, is what a step costs;
 //   * the general epilogue of the 256-row kernels (alpha, beta, bf16 or fp32 C; common.hpp store_c_run) from fp32
@@ -40,8 +40,9 @@ constexpr uint32_t STAGE = 16384;           // bytes of one operand tile
 // F16: IEEE half operands (v_mfma_f32_16x16x32_f16; a 16-bit C is then half too): same tiles, same fragment maps.
 // F8 >= 0: 8-bit operands stored N x K (one byte per element; bit 0: A is E5M2, bit 1: B is E5M2, else E4M3): the same 128-byte
 // rows hold 128 elements of K, a K tile is one v_mfma_f32_16x16x128_f8f6f4 deep, a fragment is the same two 16-byte reads.
-// A step then splits by accumulator rows, not K halves: rows 0-1 (A fragments 0, 1 and all of B: twelve reads), then
-// rows 2-3 (A fragments 2, 3: four reads).  B's fragments serve both, so the next tile's go into a second set of
+// A step then splits by accumulator rows, not K halves: rows 0-1 (A fragments 0, 1 and all of B: twelve reads, two behind
+// each of the first six MFMAs of the half step before), then rows 2-3 (A fragments 2, 3: four reads, behind the first four
+// MFMAs of rows 0-1).  B's fragments serve both, so the next tile's go into a second set of
 // registers: two steps per trip, the step count rounded up to an even number with a tile past K (zeros).
 template <bool NT, bool F16 = false, int F8 = -1>
 __device__ __forceinline__ void body(const GemmArgs& p) {
@@ -174,6 +175,14 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             }
         }
     };
+    // Read q of a K half: 0..3 A's fragments, then B's (N x K: 4..7; K x N: 4..11, the two register halves of a fragment in turn).
+    auto read_one = [&](int kh, uint32_t so, int q) {
+        if (q < 4) rd128(fa[kh][q], a_rd[kh] + so, q);
+        else if (NT) rd128(fb[kh][q - 4], b_rd[kh] + so, q - 4);
+        else if ((q - 4) & 1) rd_tr(fh[kh][(q - 4) >> 1], b_rd[(q - 4) >> 1] + so, kh * 8 + 1);
+        else rd_tr(fl[kh][(q - 4) >> 1], b_rd[(q - 4) >> 1] + so, kh * 8);
+    };
+    constexpr int HALF_READS = NT ? 8 : 12, PER_SLOT = NT ? 1 : 2;        // reads of a K half; how many go out behind one MFMA
     // Reads, waits and MFMAs are all assembly statements, which keep their order.  (The halves of a transposed fragment
     // are joined in the MFMA's operand: the register allocator gives them the two halves of one 128-bit tuple, no
     // move in between -- a move would read them before the wait.)
@@ -198,8 +207,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     // in flight.
     for (uint32_t kt = 0; kt < nk; ++kt) {
         const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;
-        read_half(1, so);
-        if (NT) asm volatile("s_waitcnt lgkmcnt(8)"); else asm volatile("s_waitcnt lgkmcnt(12)");      // K half 0 has arrived
+        asm volatile("s_waitcnt lgkmcnt(0)");                                                              // K half 0 has arrived
         const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -209,19 +217,27 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
                 // (assembly with the accumulator tied to itself: the sixteen accumulators stay where they are)
                 if (F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(0, j)), "v"(fa[0][i]));
                 else     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(0, j)), "v"(fa[0][i]));
+                // K half 1's reads, one (two) behind each of the first MFMAs: issued in a burst in front of the first MFMA they
+                // cost 5-10 % (1024 x 4096 x 4096 N x K 35.8 -> 33.1 us, K x N 36.9 -> 34.3; E4M3 19.8 -> 18.8)
+#pragma unroll
+                for (int q = (4 * i + j) * PER_SLOT; q < (4 * i + j + 1) * PER_SLOT; ++q)
+                    if (q < HALF_READS) read_one(1, so, q);
                 if (j & 1) {
                     piece(r, (4 * i + j) >> 1);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        read_half(0, so_next);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < 4; ++j) {
                 if (F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(1, j)), "v"(fa[1][i]));
                 else     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b_operand(1, j)), "v"(fa[1][i]));
+#pragma unroll
+                for (int q = (4 * i + j) * PER_SLOT; q < (4 * i + j + 1) * PER_SLOT; ++q)      // the next tile's K half 0
+                    if (q < HALF_READS) read_one(0, so_next, q);
+            }
         __builtin_amdgcn_sched_barrier(0);
     }
     } else {
@@ -258,24 +274,30 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         auto step8 = [&](auto set, uint32_t kt) {
             constexpr int S = decltype(set)::value;
             const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;
-            read_a(2, so);
-            asm volatile("s_waitcnt lgkmcnt(4)");
+            asm volatile("s_waitcnt lgkmcnt(0)");
             const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     mfma8(acc[i][j], b8[S][j], a8[i]);
+                    // (the reads go out one or two behind an MFMA, not in a burst in front of the first: their issue hides behind the matrix pipe)
+                    if (4 * i + j < 4) rd128(a8[2 + (4 * i + j) / 2][(4 * i + j) & 1], a_rd[(4 * i + j) & 1] + so, 2 + (4 * i + j) / 2);
                     piece(r, 4 * i + j);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            read_a(0, so_next);
-            read_b(std::integral_constant<int, 1 - S>{}, so_next);
 #pragma unroll
             for (int i = 2; i < 4; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) mfma8(acc[i][j], b8[S][j], a8[i]);
+                for (int j = 0; j < 4; ++j) {
+                    mfma8(acc[i][j], b8[S][j], a8[i]);
+#pragma unroll
+                    for (int q = 2 * (4 * (i - 2) + j); q < 2 * (4 * (i - 2) + j) + 2; ++q) {      // two of the next tile's twelve behind each of the first six
+                        if (q < 4) rd128(a8[q / 2][q & 1], a_rd[q & 1] + so_next, q / 2);
+                        else if (q < 12) rd128(b8[1 - S][(q - 4) / 2][q & 1], b_rd[q & 1] + so_next, (q - 4) / 2);
+                    }
+                }
             __builtin_amdgcn_sched_barrier(0);
         };
         for (uint32_t kt = 0; kt < nk; kt += 2u) {

@@ -102,7 +102,7 @@ def test_matrix_instruction_per_kernel(kernels):
             assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
             idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
             body = ins[idx[0]:idx[-1] + 1]
-            assert count(body, "ds_read_b128") == 32 - 4 and count(body, "buffer_load_dwordx4") == 16 and count(body, "s_barrier") == 2, name   # (the trip's first four reads stand in front of its first MFMA)
+            assert count(body, "ds_read_b128") == 32 and count(body, "buffer_load_dwordx4") == 16 and count(body, "s_barrier") == 2, name
             assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(16)" in i) == 2, name
             moves = [i for i in body if i.startswith(("v_mov", "v_accvgpr", "v_perm", "v_pk_", "v_lshl", "v_bfi", "v_alignbit"))]
             assert not moves, (name, moves[:5])                               # (no move of a fragment between its read and its MFMA)
@@ -253,7 +253,7 @@ def test_main_loop_of_the_128_by_128_tile_kernels_is_lean(kernels):
         assert len(idx) == 32 and count(ins, "v_mfma_f32_16x16x32_f16" if "_f16_" in name else "v_mfma_f32_16x16x32_bf16") == 32, name
         body = ins[idx[0]:idx[-1] + 1]
         for mnemonic, n in reads.items():
-            assert count(body, mnemonic) == n // 2, (name, mnemonic)          # (K half 0's reads of the next tile; K half 1's stand in front of the first MFMA)
+            assert count(body, mnemonic) == n, (name, mnemonic)               # (one, or two transposing ones, behind each of a half's first MFMAs)
         assert count(body, "buffer_load_dwordx4") == 8 and count(body, "s_barrier") == 1
         assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(16)" in i) == 1, name
         moves = [i for i in body if i.startswith(("v_mov", "v_accvgpr", "v_perm", "v_pk_", "v_lshl", "v_bfi", "v_and", "v_alignbit"))]

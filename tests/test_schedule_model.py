@@ -389,21 +389,25 @@ def test_three_stage_checker_rejects_broken_schedules():
 # ---------------------------------------------------------------------------------------
 T128_LINES = ("request(0u, 0u);", "request(BKE, 1u);", "request(2u * BKE, 2u);",
               'asm volatile("s_waitcnt vmcnt(16)\\n\\ts_barrier" ::: "memory");\n    if constexpr (!IS8) {\n    read_half(0, 0u);',
-              "const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;",
-              "read_half(1, so);",
+              "const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;\n        asm volatile(\"s_waitcnt lgkmcnt(0)\");",
               "const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);\n#pragma unroll\n        for (int i = 0; i < 4; ++i)",
+              "constexpr int HALF_READS = NT ? 8 : 12, PER_SLOT = NT ? 1 : 2;",
+              "for (int q = (4 * i + j) * PER_SLOT; q < (4 * i + j + 1) * PER_SLOT; ++q)\n                    if (q < HALF_READS) read_one(1, so, q);",
               "if (j & 1) {\n                    piece(r, (4 * i + j) >> 1);",
-              'asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");\n        read_half(0, so_next);',
+              'asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");\n#pragma unroll\n        for (int i = 0; i < 4; ++i)',
+              "if (q < HALF_READS) read_one(0, so_next, q);",
               "for (int q = 0; q < 8; ++q) piece(r, q);")
-
-
-# ... on 8-bit operands: a step splits by accumulator rows -- rows 0-1 need A fragments 0, 1 and all of B (12 reads, issued
-# behind the barrier of the step before), rows 2-3 A fragments 2, 3 (4 reads, issued at the top of the step); one request
-# behind each of the first eight MFMAs; two steps per trip, the count rounded up to an even number with a tile past K
+# ... on 8-bit operands: a step splits by accumulator rows -- rows 0-1 need A fragments 0, 1 and all of B (12 reads, two behind
+# each of the first six MFMAs of the half step before), rows 2-3 A fragments 2, 3 (4 reads, one behind each of the first four
+# MFMAs of rows 0-1); one request behind each of rows 0-1's eight MFMAs; two steps per trip, the count rounded up to an even
+# number with a tile past K
 T128_F8_LINES = ("read_a(0, 0u);\n        read_b(std::integral_constant<int, 0>{}, 0u);",
-                 "read_a(2, so);\n            asm volatile(\"s_waitcnt lgkmcnt(4)\");\n            const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);",
-                 "mfma8(acc[i][j], b8[S][j], a8[i]);\n                    piece(r, 4 * i + j);",
-                 'asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");\n            read_a(0, so_next);\n            read_b(std::integral_constant<int, 1 - S>{}, so_next);',
+                 "asm volatile(\"s_waitcnt lgkmcnt(0)\");\n            const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);",
+                 "mfma8(acc[i][j], b8[S][j], a8[i]);",
+                 "if (4 * i + j < 4) rd128(a8[2 + (4 * i + j) / 2][(4 * i + j) & 1], a_rd[(4 * i + j) & 1] + so, 2 + (4 * i + j) / 2);\n                    piece(r, 4 * i + j);",
+                 'asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");\n#pragma unroll\n            for (int i = 2; i < 4; ++i)',
+                 "for (int q = 2 * (4 * (i - 2) + j); q < 2 * (4 * (i - 2) + j) + 2; ++q) {",
+                 "else if (q < 12) rd128(b8[1 - S][(q - 4) / 2][q & 1], b_rd[q & 1] + so_next, (q - 4) / 2);",
                  "for (uint32_t kt = 0; kt < nk; kt += 2u) {\n            step8(std::integral_constant<int, 0>{}, kt);\n            step8(std::integral_constant<int, 1>{}, kt + 1u);")
 
 
@@ -416,15 +420,18 @@ def t128_f8_wave_program(nk, keep=16, reads_before_barrier=False, late_rows=4):
     ops += [("wait_keep", keep), ("barrier",)]
     ops += [("read", 0, 0, 0)] * 12
     for t in range(steps):
-        ops += [("read", t, 1, t % 4)] * late_rows
         for m in range(8):
-            ops += [("mfma", t, 0), ("dma", t + 3, m, (t + 3) % 4)]
+            ops.append(("mfma", t, 0))
+            if m < late_rows:
+                ops.append(("read", t, 1, t % 4))
+            ops.append(("dma", t + 3, m, (t + 3) % 4))
         if reads_before_barrier:
             ops += [("read", t + 1, 0, (t + 1) % 4)] * 12
         ops += [("wait_keep", keep), ("barrier",)]
-        if not reads_before_barrier:
-            ops += [("read", t + 1, 0, (t + 1) % 4)] * 12
-        ops += [("mfma", t, 1)] * 8
+        for m in range(8):
+            ops.append(("mfma", t, 1))
+            if not reads_before_barrier and m < 6:
+                ops += [("read", t + 1, 0, (t + 1) % 4)] * 2
     ops.append(("wait_all",))
     return ops, steps
 
@@ -450,21 +457,23 @@ def t128_wave_program(nk, nt, keep=16, primed=3, ahead=3, reads_before_barrier=F
         assert fact in src, fact
     assert int(re.search(r"constexpr int BT = 128, BK = 64, NS = (\d+);", src).group(1)) == 4
     half = 8 if nt else 12                        # LDS reads of one K half: 4 of A + 4 of B, or 8 transposing ones
+    per_slot = 1 if nt else 2                     # ... one (two) behind each of the other half's first MFMAs
     ops = [("dma", t, pc, t % stages) for t in range(primed) for pc in range(8)]
     ops += [("wait_keep", keep), ("barrier",)]
     ops += [("read", 0, 0, 0)] * half
     for t in range(nk):
-        ops += [("read", t, 1, t % stages)] * half
         for m in range(16):
             ops.append(("mfma", t, 0))
+            ops += [("read", t, 1, t % stages)] * (per_slot if m * per_slot < half else 0)
             if m & 1:
                 ops.append(("dma", t + ahead, m >> 1, (t + ahead) % stages))
         if reads_before_barrier:
             ops += [("read", t + 1, 0, (t + 1) % stages)] * half
         ops += [("wait_keep", keep), ("barrier",)]
-        if not reads_before_barrier:
-            ops += [("read", t + 1, 0, (t + 1) % stages)] * half
-        ops += [("mfma", t, 1)] * 16
+        for m in range(16):
+            ops.append(("mfma", t, 1))
+            if not reads_before_barrier:
+                ops += [("read", t + 1, 0, (t + 1) % stages)] * (per_slot if m * per_slot < half else 0)
     ops.append(("wait_all",))
     return ops, nk
 
