@@ -417,20 +417,21 @@ uint32_t h128_choice(const Dims& s, uint32_t batch, uint32_t cus, uint32_t kstep
     if (cost && tiles) *cost = best;
     return tiles ? best_ks : 0u;
 }
-// 128 x 128 tiles (maize_gemm_bf16_t128_*), one round of them: what a K step costs in the same units.  N x K 0.34, K x N
-// (transposing reads) 0.42; 0.02 more from 129 tiles and 0.05 more from 193 (the compute units share the path from the
+// 128 x 128 tiles (maize_gemm_bf16_t128_*), one round of them: what a K step costs in the same units.  N x K 0.31, K x N
+// (transposing reads) 0.36 (0.34 / 0.42, and the times below, while the fragment reads went out in bursts: 8 % more); 0.02 more from 129 tiles and 0.05 more from 193 (the compute units share the path from the
 // L2s), 0.04 more from 128 steps.  Every candidate by name on 54 products per layout, one box, N x K / K x N:
 // 512 x 4096 x 4096 30.6 / 35.6 us, 768 x 4096 x 4096 31.3 / 36.1, 1024 x 4096 x 4096 34.3 / 37.8, 512 x 8192 x 8192 63.5 / 70.7,
 // 1024 x 4096 x 14336 110.6 / 129.2 -- where the three-stage 128 x 256 tiles' 0.52 measures 0.51.
 double t128_step(bool nt, uint64_t tiles, uint32_t nk) {
-    return (nt ? 0.34 : 0.42) + (tiles > 192u ? 0.05 : tiles > 128u ? 0.02 : 0.0) + (nk >= 128u ? 0.04 : 0.0);
+    return (nt ? 0.31 : 0.36) + (tiles > 192u ? 0.05 : tiles > 128u ? 0.02 : 0.0) + (nk >= 128u ? 0.04 : 0.0);
 }
 // ... on 8-bit operands (N x K; a step is 128 deep): the same bytes through the LDS per step, no conversion of halves in
 // the matrix pipe's way.  E4M3, uniform random operands, one box: 256 x 4096 x 4096 (64 tiles) 16.4 us, 512 x 4096 x 4096 17.0,
 // 768 x 4096 x 4096 17.9, 1024 x 4096 x 4096 19.1 (128 x 256 tiles on three stages: 22.3 / 23.3 / 23.9 / 25.1), 512 x 8192 x 8192
 // 32.1 (40.8 in two K ranges), 1024 x 4096 x 14336 52.9-55.5 (58.7).
+// (0.25 since the reads go out between the MFMAs; the times above are from before: 5-9 % more.)
 double t128_step8(uint64_t tiles, uint32_t nk) {
-    return 0.27 + (tiles > 192u ? 0.08 : tiles > 128u ? 0.04 : 0.0) + (nk >= 64u ? 0.05 : 0.0);
+    return 0.25 + (tiles > 192u ? 0.08 : tiles > 128u ? 0.04 : 0.0) + (nk >= 64u ? 0.05 : 0.0);
 }
 bool splitk_nn_supports(const maize_gemm_ex_desc_t& d) { return nn(d) && mt256_loads_ok(d) && bf16_in(d); }
 bool splitk_nt_supports(const maize_gemm_ex_desc_t& d) { return !nn(d) && mt256_loads_ok(d) && bf16_in(d); }
@@ -1191,12 +1192,12 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
             // 384 x 4096 x 4096 N x K in four ranges 27.2 us measured, 30.4 by the model, 30.0 here; not where both are
             // bound by the operands' stream from HBM and the cut only adds its second launch: 128 x 28672 x 8192 N x K
             // 119.7 us in two ranges, 107.4 here, K x N 99.2 / 97.9)
-            // (and the model prices long K ranges on nearly all compute units low: from 64 steps per range on more than 192
+            // (and the model prices long K ranges on nearly all compute units low: from 64 steps per range on 192 or more
             // work items the three-stage 128 x 256 tiles measure 0.66-0.74 per step, not 0.52 -- 512 x 8192 x 8192 N x K in two
             // ranges 66.8-71.9 us, 57.6 by the model, 63.5 here; 2048 x 2048 x 8192 N x K 69.5, 62.5 here)
             double rival = cost_hk;
             const uint32_t per_range = hk >= 2u ? cdiv(cdiv(s.k, 64u), hk) : 0u;
-            const bool loaded = hk >= 2u && (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk > 192u && per_range >= 64u;
+            const bool loaded = hk >= 2u && (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk >= 192u && per_range >= 64u;
             if (loaded && !by_stream) rival += 0.13 * per_range;
             if (cost_t < (hk >= 2u && !by_stream && !loaded ? 0.92 : 0.97) * rival) return (uint32_t)t8;
         }
@@ -1316,6 +1317,7 @@ double tail_part_cost(const maize_gemm_ex_desc_t& part, uint32_t compute_units) 
         return launch + step + 6.0 + (1.2e-6 * (double)s.m * s.n + 0.15) * ks;
     }
     if (h128 && std::strstr(name, "_mt256_")) return launch + h128_step(three, false, s.nt, false) * nk;
+    if (std::strstr(name, "_t128_")) return launch + t128_step(s.nt, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128), nk) * nk;   // (the same sums in the same order too)
     return -1.0;
 }
 }  // namespace

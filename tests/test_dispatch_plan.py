@@ -304,13 +304,15 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
         nn_plan = mz.gemm_plan(desc(m, n, k), kernel="maize_gemm_bf16_mt256_nn_h128r3_splitk", compute_units=CUS)
         nt_plan = mz.gemm_plan(desc(m, n, k, layout=mz.LAYOUT_NT), kernel="maize_gemm_bf16_mt256_nt_h128r3_splitk", compute_units=CUS)
         assert nn_plan["ksplit"] == nt_plan["ksplit"] and nn_plan["grid"] == nt_plan["grid"], (m, n, k, nn_plan, nt_plan)
-    # two long K ranges on every compute unit cost more per step than the model's 0.52 (0.66-0.74 measured): N x K, one round of
-    # 128 x 128 tiles takes over (512 x 8192 x 8192 66.8-71.9 -> 63.5 us, 2048 x 2048 x 8192 69.5 -> 62.5); K x N, whose 128 x 128
-    # tiles cost more per step, keeps the cut (70.9 against 70.7, 69.0 against 72.2)
+    # two long K ranges on most compute units cost more per step than the model's 0.52 (0.66-0.74 measured): one round of
+    # 128 x 128 tiles takes over (N x K | K x N: 512 x 8192 x 8192 70.2 -> 58.5 us | 69.2 -> 63.0, 2048 x 2048 x 8192 69.5 -> 62.5 | 69.4 -> 65.0,
+    # 384 x 8192 x 8192 N x K 57.8 -> 52.5)
     for m, n, k in ((512, 8192, 8192), (2048, 2048, 8192)):
         assert mz.gemm_plan(desc(m, n, k, layout=mz.LAYOUT_NT), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nt"
-        p = mz.gemm_plan(desc(m, n, k), compute_units=CUS)
-        assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and p["ksplit"] == 2
+        assert mz.gemm_plan(desc(m, n, k), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nn"
+        p = mz.gemm_plan(desc(m, n, k), kernel="maize_gemm_bf16_mt256_nn_h128r3_splitk", compute_units=CUS)
+        assert p["ksplit"] == 2
+    assert mz.gemm_plan(desc(384, 8192, 8192, layout=mz.LAYOUT_NT), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nt"
     # ... and against the 256-row kernels' shorter ranges, from 96 steps per range on (1024 x 4096 x 14336: two ranges of 112 steps
     # 112.9 us, 128 x 128 tiles 110.6, the 256-row kernel in four ranges 104.6; 768 x 4096 x 14336 97.5 against 85.7 in five)
     for layout, tag in ((mz.LAYOUT_NN, "nn"), (mz.LAYOUT_NT, "nt")):
@@ -318,8 +320,11 @@ def test_a_quarter_to_half_a_tile_per_compute_unit_is_split_too():
         assert p["kernel"] == f"maize_gemm_bf16_mt256_{tag}_splitk" and p["ksplit"] == 4
         p = mz.gemm_plan(desc(768, 4096, 14336, layout=layout), compute_units=CUS)
         assert p["kernel"] == f"maize_gemm_bf16_mt256_{tag}_splitk" and p["ksplit"] == 5
-        p = mz.gemm_plan(desc(1024, 4096, 11008, layout=layout), compute_units=CUS)        # (86 steps per range: stays; 84.7 us against more)
-        assert p["kernel"] == f"maize_gemm_bf16_mt256_{tag}_h128r3_splitk" and p["ksplit"] == 2
+        p = mz.gemm_plan(desc(1024, 4096, 11008, layout=layout), kernel=f"maize_gemm_bf16_mt256_{tag}_h128r3_splitk", compute_units=CUS)
+        assert p["ksplit"] == 2                                                            # (86 steps per range: the 128-row cut stays ahead of the 256-row one, 84.7 us)
+    # (... where N x K has one round of 128 x 128 tiles at 77.8 us; K x N 85.2 against 86.2: the cut)
+    assert mz.gemm_plan(desc(1024, 4096, 11008, layout=mz.LAYOUT_NT), compute_units=CUS)["kernel"] == "maize_gemm_bf16_t128_nt"
+    assert mz.gemm_plan(desc(1024, 4096, 11008), compute_units=CUS)["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk"
     p = mz.gemm_plan(desc(384, 6144, 4096), compute_units=CUS)                             # (three ranges 33 us; two 35; whole 39)
     assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and p["ksplit"] == 3 and p["grid"] == (216, 1, 1)
     p = mz.gemm_plan(desc(384, 6144, 4096, layout=mz.LAYOUT_NT), compute_units=CUS)        # (N x K: 144 tiles of 128 x 128 30.9 us, three ranges 31.5)
