@@ -153,6 +153,7 @@ MAIZE_TILE_TY(F16_128x64, 128, 64, 2, Swizzle::KC16)
 MAIZE_TILE_TY(F8_128x128, 128, 128, 1, Swizzle::KC16)
 MAIZE_TILE_TY(BF16_64x128, 64, 128, 2, Swizzle::KN32)    // B stage of the 128 x 128 tile kernels for a row-major K x N B (stored N x K: BF16_128x64, like their A stage)
 MAIZE_TILE_TY(F16_64x128, 64, 128, 2, Swizzle::KN32)
+MAIZE_TILE_TY(F8_128x128_KN, 128, 128, 1, Swizzle::KN16) // ... for a row-major K x N 8-bit B (stored N x K: F8_128x128)
 #undef MAIZE_TILE_TY
 template <class T> struct Tile { using Ty = T; static constexpr size_t SIZE = (size_t)T::ROWS * T::COLS * T::ELEM_BYTES; };
 template <class TA, class TB> struct TilePair { using A = TA; using B = TB; static constexpr size_t SIZE = TA::SIZE + TB::SIZE; };
@@ -334,12 +335,11 @@ Accum gemm_smem_multibuffer(const MMA&, KTile<K_TILE>, const RowPanel<NA>& a, co
     // Generic in the ring depth and the panel height like the reference's mainloop ([TilePair; PIPE], KTile<N>,
     // gemm/mod.rs:37-45), within what kernels exist: 256- or 128-row panels of A on two stages, 128-row panels also on
     // three (a 128 x 256 tile's stage is 48 KiB; three fit the 160 KiB of LDS).
-    // ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages, 16-bit operands (8-bit ones with B stored N x K: stages F8_128x128).
+    // ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages, 16-bit or 8-bit operands.
     constexpr uint32_t NB = BPanel::WINDOW;
     constexpr bool QUARTER = NA == 128 && NB == 128;
     static_assert(QUARTER ? PIPE == 4 : (PIPE == 2 || PIPE == 3), "the macro-tile kernels run a ring of two or three stages, the 128 x 128 tile kernels one of four");
     static_assert((NA == 256 || NA == 128) && (NB == 256 || QUARTER), "the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B), or 128 rows and 128 columns");
-    static_assert(!QUARTER || MMA::IN_TYPE == MAIZE_IN_BF16 || MMA::IN_TYPE == MAIZE_IN_F16 || NT, "the 128 x 128 tile kernels take 8-bit operands with B stored N x K only");
     static_assert(PIPE != 3 || NA == 128, "three ring stages fit the LDS with 128-row panels of A only");
     using TA = typename Pair::A::Ty; using TB = typename Pair::B::Ty;
     constexpr uint32_t ES = MMA::K_TILE == 128 ? 1 : 2;

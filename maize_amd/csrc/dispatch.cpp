@@ -159,7 +159,8 @@ bool f8_nn_common(const maize_gemm_ex_desc_t& d) {
     bool tag##_nt_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d); } \
     bool tag##_t128_nt_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nt_common(d) && (dims_of(d).k & 127u) == 0; } \
     bool tag##_nn_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nn_common(d) && plain_epilogue(d); } \
-    bool tag##_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nn_common(d); }
+    bool tag##_nn_gen_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nn_common(d); } \
+    bool tag##_t128_nn_supports(const maize_gemm_ex_desc_t& d) { return d.in_type == type && f8_nn_common(d) && (dims_of(d).k & 127u) == 0; }
 MAIZE_F8_SUPPORTS(e4m3, MAIZE_IN_E4M3)
 MAIZE_F8_SUPPORTS(e5m2, MAIZE_IN_E5M2)
 MAIZE_F8_SUPPORTS(e4m3e5m2, MAIZE_IN_E4M3_E5M2)
@@ -997,6 +998,7 @@ const KernelInfo kKernels[] = {
     {"maize_gemm_" #tag "_mt256_nt", nullptr, tag##_nt_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_gen", nullptr, tag##_nt_gen_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_t128_nt", nullptr, tag##_t128_nt_supports, t128_plan}, \
+    {"maize_gemm_" #tag "_t128_nn", nullptr, tag##_t128_nn_supports, t128_plan}, \
     {"maize_gemm_" #tag "_mt256_nt_splitk", nullptr, tag##_nt_gen_supports, splitk_plan}, \
     {"maize_gemm_" #tag "_mt256_nn", nullptr, tag##_nn_supports, mt256_plan}, \
     {"maize_gemm_" #tag "_mt256_nn_gen", nullptr, tag##_nn_gen_supports, mt256_plan}, \
@@ -1098,14 +1100,14 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
         {
             double cost_hk = 0.0;
             const uint32_t hk = h128_choice(s, d.gemm.batch, compute_units, 128, &cost_hk);
-            std::snprintf(name, sizeof name, "maize_gemm_%s_t128_nt", kTag[d.in_type - MAIZE_IN_E4M3]);
+            std::snprintf(name, sizeof name, "maize_gemm_%s_t128_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.nt ? "nt" : "nn");
             const int t8 = kernel_index(name);
             const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
             const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128) * d.gemm.batch;
             // (a long K on fewer than sixteen tiles is for the cut over K: one compute unit per tile walks it alone here)
-            if (t8 >= 0 && s.nt && s.k >= 256u && tiles <= units && (tiles >= 16u || s.k <= 1024u) && kKernels[t8].supports(d)) {
+            if (t8 >= 0 && s.k >= 256u && tiles <= units && (tiles >= 16u || s.k <= 1024u) && kKernels[t8].supports(d)) {
                 const uint32_t nk = cdiv(s.k, 128u);
-                const double cost_t = 8.0 + t128_step8(tiles, nk) * nk;
+                const double cost_t = 8.0 + (t128_step8(tiles, nk) + (s.nt ? 0.0 : 0.04)) * nk;      // (K x N: twice the LDS instructions per fragment of B)
                 if (cost_t >= stream_us(s, d.gemm.batch, 128u, tiles) && cost_t < (hk >= 2u ? 0.92 : 0.97) * cost_hk) return (uint32_t)t8;
             }
             if (hk >= 1u) {

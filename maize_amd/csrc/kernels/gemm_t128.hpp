@@ -1,4 +1,4 @@
-// maize_gemm_{bf16,f16}_t128_{nn,nt}, maize_gemm_{e4m3,e5m2,e4m3e5m2,e5m2e4m3}_t128_nt: the pipelined tile kernel on 128 x 128 tiles of C.
+// maize_gemm_{bf16,f16}_t128_{nn,nt}, maize_gemm_{e4m3,e5m2,e4m3e5m2,e5m2e4m3}_t128_{nn,nt}: the pipelined tile kernel on 128 x 128 tiles of C.
 //
 // For products whose 128 x 256 tiles would occupy half of the compute units or less: four times as many tiles as
 // the 256 x 256 kernel has, one per workgroup, so the whole chip works on a product of 64 to 256 of them.  The
@@ -38,7 +38,7 @@ constexpr int BT = 128, BK = 64, NS = 4;
 constexpr uint32_t STAGE = 16384;           // bytes of one operand tile
 
 // F16: IEEE half operands (v_mfma_f32_16x16x32_f16; a 16-bit C is then half too): same tiles, same fragment maps.
-// F8 >= 0: 8-bit operands stored N x K (one byte per element; bit 0: A is E5M2, bit 1: B is E5M2, else E4M3): the same 128-byte
+// F8 >= 0: 8-bit operands (one byte per element; B stored N x K, or K x N with N % 16 == 0 and a fragment four transposing reads; bit 0: A is E5M2, bit 1: B is E5M2, else E4M3): the same 128-byte
 // rows hold 128 elements of K, a K tile is one v_mfma_f32_16x16x128_f8f6f4 deep, a fragment is the same two 16-byte reads.
 // A step then splits by accumulator rows, not K halves: rows 0-1 (A fragments 0, 1 and all of B: twelve reads, two behind
 // each of the first six MFMAs of the half step before), then rows 2-3 (A fragments 2, 3: four reads, behind the first four
@@ -47,7 +47,8 @@ constexpr uint32_t STAGE = 16384;           // bytes of one operand tile
 template <bool NT, bool F16 = false, int F8 = -1>
 __device__ __forceinline__ void body(const GemmArgs& p) {
     constexpr bool IS8 = F8 >= 0;
-    static_assert(!IS8 || (NT && !F16), "8-bit operands: both K-contiguous");
+    static_assert(!IS8 || !F16, "one operand type");
+    constexpr bool TR8 = IS8 && !NT;                    // 8-bit row-major B: 128 rows of 128 B (maps::sk8n_*), read through ds_read_b64_tr_b8
     constexpr uint32_t ES = IS8 ? 1u : 2u;              // bytes per element of A and B
     constexpr uint32_t CH = 16u / ES;                   // elements per 16-byte chunk
     constexpr uint32_t BKE = IS8 ? 128u : (uint32_t)BK; // elements per K tile (128 bytes per row either way)
@@ -79,9 +80,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
     const char* const Ag = (const char*)p.a + ((uint64_t)bz * p.stride_a + (uint64_t)m0 * lda) * ES;
     const uint32_t a_bytes = span(((uint64_t)(M - 1u - m0) * lda + K) * ES);
     const char* const Bg = NT ? (const char*)p.b + ((uint64_t)bz * p.stride_b + (uint64_t)n0 * ldb) * ES
-                              : (const char*)p.b + (uint64_t)bz * p.stride_b * 2u;
+                              : (const char*)p.b + (uint64_t)bz * p.stride_b * ES;
     const uint32_t b_bytes = NT ? span(((uint64_t)(N - 1u - n0) * ldb + K) * ES) : 0u;
-    const uint64_t b_view = ((uint64_t)(K - 1u) * ldb + N) * 2u;              // bytes of a K x N B
+    const uint64_t b_view = ((uint64_t)(K - 1u) * ldb + N) * ES;              // bytes of a K x N B
     // The lane's byte offsets of its four requests per operand and K tile (pieces 4 wave .. 4 wave + 3), at k = 0.
     uint32_t a_vo[4], b_vo[4];
 #pragma unroll
@@ -90,6 +91,9 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         a_vo[i] = (maps::kc_piece_row(pc, lane) * lda + maps::kc_piece_chunk(pc, lane) * CH) * ES;
         if (NT) {
             b_vo[i] = (maps::kc_piece_row(pc, lane) * ldb + maps::kc_piece_chunk(pc, lane) * CH) * ES;
+        } else if (TR8) {
+            const uint32_t col = n0 + maps::sk8n_piece_chunk(pc, lane) * 16u;
+            b_vo[i] = (maps::sk8n_piece_row(pc, lane) * ldb + col) | (col < N ? 0u : OOB);
         } else {
             const uint32_t col = n0 + maps::sk128_piece_chunk(pc, lane) * 8u;
             b_vo[i] = ((maps::sk128_piece_row(pc, lane) * ldb + col) * 2u) | (col < N ? 0u : OOB);
@@ -110,7 +114,7 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             r.b_so = r.a_so;
         } else {
             // K x N: the descriptor starts at row k of B and ends with the view (64-bit scalar arithmetic, once per tile)
-            const uint64_t skip = live ? (uint64_t)sc(k) * sc(ldb * 2u) : 0u;
+            const uint64_t skip = live ? (uint64_t)sc(k) * sc(ldb * ES) : 0u;
             const uint64_t base = (uint64_t)(uintptr_t)Bg + skip;
             r.rb = make_rsrc((const void*)(uintptr_t)(((uint64_t)sc((uint32_t)(base >> 32)) << 32) | sc((uint32_t)base)),
                              live ? sc(span(b_view - skip)) : 0u);
@@ -139,7 +143,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         for (int kh = 0; kh < 2; ++kh) b_rd[kh] = (uint32_t)(uintptr_t)(lds_ptr)lds_b + maps::kc_frag16_offset(wn * 64u, kh, lane);
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) b_rd[j] = (uint32_t)(uintptr_t)(lds_ptr)lds_b + maps::sk128_tr_offset(wn * 4u + j, 0, lane);
+        for (int j = 0; j < 4; ++j)
+            b_rd[j] = (uint32_t)(uintptr_t)(lds_ptr)lds_b + (TR8 ? maps::sk8n_tr_offset(wn * 4u + j, 0, 0, lane) : maps::sk128_tr_offset(wn * 4u + j, 0, lane));
     }
 
 #define MAIZE_RD_CASE(n) case n: asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(base), "n"((n) * 2048)); break;
@@ -244,33 +249,44 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
         // ---- 8-bit operands ---------------------------------------------------------------------
         typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
         typedef int i32x8 __attribute__((ext_vector_type(8)));
+        typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
         u32x4v a8[4][2];                 // A fragment f, 16-byte chunk kh (the lane's chunks l/16 and 4 + l/16 of its row)
-        u32x4v b8[2][4][2];              // B: register set, fragment, chunk
+        u32x4v b8[2][4][2];              // B stored N x K: register set, fragment, chunk
+        u32x2v b8t[2][4][4];             // B stored K x N: register set, fragment, register pair 2 kk + h (rows 64 kk + 16 g + 8 h + 0..7 transposed)
         auto operand8 = [](const u32x4v (&f)[2]) -> i32x8 {
             return i32x8{(int)f[0][0], (int)f[0][1], (int)f[0][2], (int)f[0][3], (int)f[1][0], (int)f[1][1], (int)f[1][2], (int)f[1][3]};
         };
-        auto read_a = [&](int f0, uint32_t so) {
-#pragma unroll
-            for (int f = f0; f < f0 + 2; ++f)
-#pragma unroll
-                for (int kh = 0; kh < 2; ++kh) rd128(a8[f][kh], a_rd[kh] + so, f);
+        auto operand8t = [](const u32x2v (&f)[4]) -> i32x8 {
+            return i32x8{(int)f[0][0], (int)f[0][1], (int)f[1][0], (int)f[1][1], (int)f[2][0], (int)f[2][1], (int)f[3][0], (int)f[3][1]};
         };
-        auto read_b = [&](auto set, uint32_t so) {
+#define MAIZE_RD_CASE(n) case n: asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(base), "n"(((n) >> 1) * 8192 + ((n) & 1) * 1024)); break;
+        auto rd_tr8 = [&](u32x2v& dst, uint32_t base, int n) {        // n = 2 kk + h
+            switch (n) { MAIZE_RD_CASE(0) MAIZE_RD_CASE(1) MAIZE_RD_CASE(2) MAIZE_RD_CASE(3) }
+        };
+#undef MAIZE_RD_CASE
+        // The reads rows 0-1 of tile t + 1 wait for, in the order they go out: A fragments 0, 1 (two chunks each), then B's
+        // (two chunks, or four transposed register pairs, each).
+        constexpr int NEXT_READS = TR8 ? 20 : 12, NEXT_PER_SLOT = TR8 ? 3 : 2;
+        auto read_next = [&](auto set, uint32_t so, int q) {
             constexpr int S = decltype(set)::value;
-#pragma unroll
-            for (int f = 0; f < 4; ++f)
-#pragma unroll
-                for (int kh = 0; kh < 2; ++kh) rd128(b8[S][f][kh], b_rd[kh] + so, f);
+            if (q < 4) rd128(a8[q / 2][q & 1], a_rd[q & 1] + so, q / 2);
+            else if (!TR8) rd128(b8[S][(q - 4) / 2][q & 1], b_rd[q & 1] + so, (q - 4) / 2);
+            else rd_tr8(b8t[S][(q - 4) / 4][(q - 4) & 3], b_rd[(q - 4) / 4] + so, (q - 4) & 3);
         };
         // B first, so cbsz carries B's format and blgp A's (0 = E4M3, 1 = E5M2)
-        auto mfma8 = [&](floatx4& c, const u32x4v (&b)[2], const u32x4v (&a)[2]) {
-            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(c) : "v"(operand8(b)), "v"(operand8(a)), "n"((F8 >> 1) & 1), "n"(F8 & 1));
+        auto mfma8 = [&](floatx4& c, auto set, int j, const u32x4v (&a)[2]) {
+            constexpr int S = decltype(set)::value;
+            i32x8 bv;
+            if constexpr (TR8) bv = operand8t(b8t[S][j]); else bv = operand8(b8[S][j]);
+            const i32x8 av = operand8(a);
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(c) : "v"(bv), "v"(av), "n"((F8 >> 1) & 1), "n"(F8 & 1));
         };
-        read_a(0, 0u);
-        read_b(std::integral_constant<int, 0>{}, 0u);
-        // A step: A fragments 2, 3 are read, rows 0-1 multiply (their twelve reads went out half a step ago) with the eight
-        // requests of tile t + 3 between the MFMAs; the wait and the barrier as above; the next tile's A fragments 0, 1 and B
-        // fragments (into the other register set) are read while rows 2-3 multiply.
+#pragma unroll
+        for (int q = 0; q < NEXT_READS; ++q) read_next(std::integral_constant<int, 0>{}, 0u, q);
+        // A step: rows 0-1 multiply (their reads went out half a step ago) with A fragments 2, 3 read behind the first four
+        // MFMAs and the eight requests of tile t + 3 one behind each; the wait and the barrier as above; rows 2-3 multiply
+        // with the next tile's A fragments 0, 1 and B fragments (into the other register set) read behind the MFMAs, two
+        // (K x N: three) each.
         auto step8 = [&](auto set, uint32_t kt) {
             constexpr int S = decltype(set)::value;
             const uint32_t so = (kt & 3u) * STAGE, so_next = ((kt + 1u) & 3u) * STAGE;
@@ -280,8 +296,8 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    mfma8(acc[i][j], b8[S][j], a8[i]);
-                    // (the reads go out one or two behind an MFMA, not in a burst in front of the first: their issue hides behind the matrix pipe)
+                    mfma8(acc[i][j], set, j, a8[i]);
+                    // (the reads go out behind the MFMAs, not in a burst in front of the first: their issue hides behind the matrix pipe)
                     if (4 * i + j < 4) rd128(a8[2 + (4 * i + j) / 2][(4 * i + j) & 1], a_rd[(4 * i + j) & 1] + so, 2 + (4 * i + j) / 2);
                     piece(r, 4 * i + j);
                     __builtin_amdgcn_sched_barrier(0);
@@ -291,12 +307,10 @@ __device__ __forceinline__ void body(const GemmArgs& p) {
             for (int i = 2; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    mfma8(acc[i][j], b8[S][j], a8[i]);
+                    mfma8(acc[i][j], set, j, a8[i]);
 #pragma unroll
-                    for (int q = 2 * (4 * (i - 2) + j); q < 2 * (4 * (i - 2) + j) + 2; ++q) {      // two of the next tile's twelve behind each of the first six
-                        if (q < 4) rd128(a8[q / 2][q & 1], a_rd[q & 1] + so_next, q / 2);
-                        else if (q < 12) rd128(b8[1 - S][(q - 4) / 2][q & 1], b_rd[q & 1] + so_next, (q - 4) / 2);
-                    }
+                    for (int q = NEXT_PER_SLOT * (4 * (i - 2) + j); q < NEXT_PER_SLOT * (4 * (i - 2) + j + 1); ++q)
+                        if (q < NEXT_READS) read_next(std::integral_constant<int, 1 - S>{}, so_next, q);
                 }
             __builtin_amdgcn_sched_barrier(0);
         };
@@ -340,9 +354,10 @@ extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_t128_nn(GemmAr
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_bf16_t128_nt(GemmArgs p) { t128::body<true>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_t128_nn(GemmArgs p) { t128::body<false, true>(p); }
 extern "C" __global__ __launch_bounds__(256) void maize_gemm_f16_t128_nt(GemmArgs p) { t128::body<true, true>(p); }
-// 8-bit operands, B stored N x K (A's format, B's format: 0 = E4M3, 1 = E5M2)
+// 8-bit operands, B stored N x K or K x N (A's format, B's format: 0 = E4M3, 1 = E5M2)
 #define MAIZE_T128_F8(tag, fa, fb) \
-    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_t128_nt(GemmArgs p) { t128::body<true, false, (fa) | ((fb) << 1)>(p); }
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_t128_nt(GemmArgs p) { t128::body<true, false, (fa) | ((fb) << 1)>(p); } \
+    extern "C" __global__ __launch_bounds__(256) void maize_gemm_##tag##_t128_nn(GemmArgs p) { t128::body<false, false, (fa) | ((fb) << 1)>(p); }
 MAIZE_T128_F8(e4m3, 0, 0)
 MAIZE_T128_F8(e5m2, 1, 1)
 MAIZE_T128_F8(e4m3e5m2, 0, 1)

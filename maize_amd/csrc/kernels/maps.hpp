@@ -133,5 +133,19 @@ MAIZE_MAP uint32_t sk8_tr_offset(uint32_t cg, uint32_t kk, uint32_t h, uint32_t 
     return sk8_offset(sk8_tr_row(kk, h, lane), cg) + (lane & 1u) * 8u;
 }
 
+// ---- K x N operand tile of 8-bit elements of the 128 x 128 kernel (row-major B): 128 rows of 128 B (128 columns), 16 pieces ----
+// Piece p (8 rows, 1 KiB): lane l lands at row 8p + l/8, position l%8.  A 32-lane pass of a transposing read touches 16 rows
+// (one 16-byte chunk each): rows of one parity share 32 banks, so the chunk index is XOR-ed with f(row) = (row / 2) % 4 +
+// 4 bit4(row), which tells the eight rows of a parity apart.  Bits 3 and 6 of the row stay out of it: the four reads of a
+// fragment sit 1024 (8 rows) and 8192 (64 rows) bytes apart behind one address register per column group.
+MAIZE_MAP uint32_t sk8n_swizzle(uint32_t row) { return ((row >> 1) & 3u) | (((row >> 4) & 1u) << 2); }
+MAIZE_MAP uint32_t sk8n_piece_row(uint32_t piece, uint32_t lane) { return piece * 8u + (lane >> 3); }
+MAIZE_MAP uint32_t sk8n_piece_chunk(uint32_t piece, uint32_t lane) { return (lane & 7u) ^ sk8n_swizzle(sk8n_piece_row(piece, lane)); }
+MAIZE_MAP uint32_t sk8n_offset(uint32_t row, uint32_t chunk) { return row * 128u + ((chunk ^ sk8n_swizzle(row)) * 16u); }
+// Transposing read (ds_read_b64_tr_b8) as for the wide tile: read (kk, h) of column group cg fetches rows 64 kk + 16 g + 8 h + 0..7.
+MAIZE_MAP uint32_t sk8n_tr_offset(uint32_t cg, uint32_t kk, uint32_t h, uint32_t lane) {
+    return sk8n_offset(sk8_tr_row(kk, h, lane), cg) + (lane & 1u) * 8u;
+}
+
 }  // namespace maps
 }  // namespace maize

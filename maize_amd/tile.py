@@ -54,6 +54,7 @@ F8_128x128 = TileTy("F8_128x128", 128, 128, 1, "kc16")
 # B stage of the 128 x 128 tile kernels for a row-major K x N B (stored N x K, their B stage is BF16_128x64 like their A stage)
 BF16_64x128 = TileTy("BF16_64x128", 64, 128, 2, "kn32")
 F16_64x128 = TileTy("F16_64x128", 64, 128, 2, "kn32")
+F8_128x128_KN = TileTy("F8_128x128_KN", 128, 128, 1, "kn16")      # ... for a row-major K x N 8-bit B (stored N x K: F8_128x128)
 
 
 @dataclass(frozen=True)
@@ -293,13 +294,11 @@ def gemm_smem_multibuffer(mma, ktile, a_panel, b_panel, smem, cp_group, cp_size)
         # 128-row panels also on three stages (the stage of a 128 x 256 tile is 48 KiB: three fit the 160 KiB of LDS).
         b_cols = b_panel.rows if nt else b_panel.cols
         # ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages,
-        # 16-bit operands, or 8-bit operands with B stored N x K (stages F8_128x128).
+        # 16-bit or 8-bit operands.
         quarter = a_panel.rows == 128 and b_cols == 128
         if a_panel.rows not in (256, 128) or b_cols not in (256, 128) or (b_cols == 128 and not quarter):
             raise ValueError("the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B), or 128 rows and 128 columns")
         if quarter:
-            if mma.in_type not in (_ffi.IN_BF16, _ffi.IN_F16) and not nt:
-                raise ValueError("the 128 x 128 tile kernels take 8-bit operands with B stored N x K only")
             if smem is None or smem.depth != 4:
                 raise ValueError("the 128 x 128 tile kernels run a ring of four stages")
         elif smem is None or smem.depth not in (2, 3):

@@ -31,6 +31,7 @@ tile_ty!(F16_128x64, 128, 64, 2, Swizzle::Kc16);
 tile_ty!(F8_128x128, 128, 128, 1, Swizzle::Kc16);
 tile_ty!(BF16_64x128, 64, 128, 2, Swizzle::Kn32);   // B stage of the 128 x 128 tile kernels for a row-major K x N B
 tile_ty!(F16_64x128, 64, 128, 2, Swizzle::Kn32);
+tile_ty!(F8_128x128_KN, 128, 128, 1, Swizzle::Kn16); // ... for a row-major K x N 8-bit B
 pub struct Tile<T>(PhantomData<T>);
 pub struct TilePair<TA, TB> { pub a: PhantomData<TA>, pub b: PhantomData<TB> }
 /// `[TilePair<TA, TB>; PIPE]` in LDS (src/main.rs:42-44).
@@ -151,7 +152,7 @@ impl DescribedGemm {
 /// in the ring depth and the panel height like the reference's mainloop (`[TilePair; PIPE]`, `KTile<N>`, gemm/mod.rs:37-45),
 /// within what kernels exist: 256- or 128-row panels of A on two ring stages, 128-row panels also on three; B in panels of
 /// 256 (column panels of a K x N B, row panels of a B stored N x K); 128-row panels of A against 128-wide panels of B on four
-/// stages (the 128 x 128 tile kernels: bf16, half, or 8-bit operands with B stored N x K); 16-byte copies per lane of a Wave.
+/// stages (the 128 x 128 tile kernels: bf16, half or 8-bit operands); 16-byte copies per lane of a Wave.
 pub fn gemm_smem_multibuffer<MMA: SyncMMAOp, const K_TILE: u32, const NA: u32, B: BPanel, TA: ConstSizeTileTy, TB: ConstSizeTileTy, const PIPE: usize>(
         _mma: &MMA, _k: KTile<K_TILE>, a: RowPanel<NA>, b: B, _smem: &SharedRing<Tile<TA>, Tile<TB>, PIPE>, _cp_group: Wave, cp_size: u8) -> Result<Accum> {
     let refuse = |m: &str| Err(Error { code: ffi::MAIZE_ERR_ARG, message: m.into() });
@@ -161,7 +162,6 @@ pub fn gemm_smem_multibuffer<MMA: SyncMMAOp, const K_TILE: u32, const NA: u32, B
     // ... and 128 x 128 tiles (128-row panels of A against 128-column panels of B) on a ring of four 32 KiB stages, 16-bit operands
     let quarter = NA == 128 && B::WINDOW == 128;
     if quarter && PIPE != 4 { return refuse("the 128 x 128 tile kernels run a ring of four stages"); }
-    if quarter && MMA::IN_TYPE != ffi::MAIZE_IN_BF16 && MMA::IN_TYPE != ffi::MAIZE_IN_F16 && !B::NT { return refuse("the 128 x 128 tile kernels take 8-bit operands with B stored N x K only"); }
     if !quarter && !(PIPE == 2 || PIPE == 3) { return refuse("the macro-tile kernels run a ring of two or three stages"); }
     if !(NA == 256 || NA == 128) || !(B::WINDOW == 256 || quarter) { return refuse("the macro-tile kernels take panels of 256 or 128 rows (A) and 256 columns (B), or 128 rows and 128 columns"); }
     if PIPE == 3 && NA != 128 { return refuse("three ring stages fit the LDS with 128-row panels of A only"); }

@@ -202,6 +202,31 @@ int main() {
                 }
         std::printf("ok  8-bit K x N tile: deposit map is a bijection, transposing reads deliver the MFMA operand and are bank-conflict free\n");
     }
+    // ---- 8-bit K x N tile of the 128 x 128 kernel: 128 rows of 128 B, 16 pieces of 8 rows
+    {
+        std::set<uint32_t> seen;
+        for (uint32_t piece = 0; piece < 16; ++piece)
+            for (uint32_t lane = 0; lane < 64; ++lane) {
+                const uint32_t row = sk8n_piece_row(piece, lane), chunk = sk8n_piece_chunk(piece, lane);
+                CHECK(row < 128 && chunk < 8, "128-wide 8-bit K x N piece out of range");
+                CHECK(sk8n_offset(row, chunk) == piece * 1024 + lane * 16, "128-wide 8-bit K x N deposit/read mismatch piece %u lane %u", piece, lane);
+                CHECK(seen.insert(row * 8 + chunk).second, "128-wide 8-bit K x N (row %u, chunk %u) deposited twice", row, chunk);
+            }
+        CHECK(seen.size() == 128 * 8, "128-wide 8-bit K x N tile not covered");
+        for (uint32_t cg = 0; cg < 8; ++cg)
+            for (uint32_t kk = 0; kk < 2; ++kk)
+                for (uint32_t h = 0; h < 2; ++h) {
+                    uint32_t off[64];
+                    for (uint32_t lane = 0; lane < 64; ++lane) {
+                        off[lane] = sk8n_tr_offset(cg, 0, 0, lane) + 8192 * kk + 1024 * h;
+                        const uint32_t q = lane & 15u, g = lane >> 4;
+                        const uint32_t row = 64 * kk + 16 * g + 8 * h + q / 2, col = 16 * cg + 8 * (q % 2);
+                        CHECK(off[lane] == sk8n_offset(row, col >> 4) + (col & 15), "128-wide 8-bit transposing read cg %u kk %u h %u lane %u", cg, kk, h, lane);
+                    }
+                    CHECK(passes_conflict_free(off, 8), "128-wide 8-bit transposing read cg %u kk %u h %u has bank conflicts", cg, kk, h);
+                }
+        std::printf("ok  128-wide 8-bit K x N tile: deposit map is a bijection, transposing reads deliver the MFMA operand and are bank-conflict free\n");
+    }
     // ---- 16-bit epilogue staging, MFMA 16 x 16 accumulators
     {
         for (uint32_t row = 0; row < 32; ++row)

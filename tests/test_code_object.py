@@ -102,7 +102,11 @@ def test_matrix_instruction_per_kernel(kernels):
             assert all(("cbsz:1" in i) == bool(b_e5m2) and ("blgp:1" in i) == bool(a_e5m2) for i in f8), name
             idx = [k for k, i in enumerate(ins) if i.startswith("v_mfma")]
             body = ins[idx[0]:idx[-1] + 1]
-            assert count(body, "ds_read_b128") == 32 and count(body, "buffer_load_dwordx4") == 16 and count(body, "s_barrier") == 2, name
+            if name.endswith("_nn"):      # B stored K x N: four transposing 64-bit reads per fragment of B
+                assert count(body, "ds_read_b128") == 16 and count(body, "ds_read_b64_tr_b8") == 32, name
+            else:
+                assert count(body, "ds_read_b128") == 32 and count(body, "ds_read_b64_tr_b8") == 0, name
+            assert count(body, "buffer_load_dwordx4") == 16 and count(body, "s_barrier") == 2, name
             assert sum(1 for i in body if i.startswith("s_waitcnt") and "vmcnt(16)" in i) == 2, name
             moves = [i for i in body if i.startswith(("v_mov", "v_accvgpr", "v_perm", "v_pk_", "v_lshl", "v_bfi", "v_alignbit"))]
             assert not moves, (name, moves[:5])                               # (no move of a fragment between its read and its MFMA)

@@ -185,11 +185,15 @@ def test_dispatch_of_8bit_operands():
         nn_plan = mz.gemm_plan(ex(4096, 4096, 4096, in_type=it))                                              # row-major B read where it lies
         assert nn_plan["kernel"] == direct and nn_plan["workspace_bytes"] == 0 and nn_plan["reduce_grid"] == 0
         assert mz.gemm_plan(ex(4096, 4096, 4096, in_type=it, beta=1.0))["kernel"] == direct + "_gen"
-        few = mz.gemm_plan(ex(64, 4096, 4096, in_type=it))                                                    # few tiles: split K
-        assert few["kernel"] == direct + "_h128_splitk" and few["ksplit"] >= 2 and few["workspace_bytes"] == 65536 + 16 * few["ksplit"] * 131072   # 16 tiles of 128 x 256
+        few = mz.gemm_plan(ex(64, 4096, 4096, in_type=it), kernel=direct + "_h128_splitk")                    # few tiles: split K
+        assert few["ksplit"] >= 2 and few["workspace_bytes"] == 65536 + 16 * few["ksplit"] * 131072           # 16 tiles of 128 x 256
+        quarter_nn = direct.replace("_mt256_nn", "_t128_nn")
+        assert mz.gemm_plan(ex(64, 4096, 4096, in_type=it))["kernel"] in (direct + "_h128_splitk", quarter_nn)
+        assert mz.gemm_plan(ex(64, 512, 8192, in_type=it))["kernel"] == direct + "_h128_splitk"               # a long K on four tiles of 128 x 128: the cut over K
+        assert mz.gemm_plan(ex(1024, 4096, 4096, in_type=it))["kernel"] == quarter_nn                         # one round of 256 tiles of 128 x 128 (E4M3 26.4 -> 19.2 us)
         for other in mz.kernel_names():
             assert _supports(other, ex(4096, 4096, 4096, in_type=it)) == (
-                other in (direct, direct + "_gen", direct + "_splitk", direct + "_h128_gen", direct + "_h128r3_gen", direct + "_h128_splitk", direct + "_h128r3_splitk", name + "_trb", name + "_trb_gen", packed, "maize_gemm_bf16_wave32")), other
+                other in (direct, direct + "_gen", direct + "_splitk", direct + "_h128_gen", direct + "_h128r3_gen", direct + "_h128_splitk", direct + "_h128r3_splitk", quarter_nn, name + "_trb", name + "_trb_gen", packed, "maize_gemm_bf16_wave32")), other
         tr_plan = mz.gemm_plan(ex(4096, 4104, 4096, in_type=it))                                              # N % 16 != 0: transposed copy of B, nothing else
         assert tr_plan["kernel"] == name + "_trb" and tr_plan["workspace_bytes"] == 65536 + 4104 * 4096 and tr_plan["reduce_grid"] == 0
         assert mz.gemm_plan(ex(4096, 4104, 4096, in_type=it, beta=1.0))["kernel"] == name + "_trb_gen"
@@ -225,7 +229,7 @@ def test_dispatch_of_8bit_operands():
             p = mz.gemm_plan(ex(rows, 14336, 4096, in_type=it))
             assert p["kernel"] == few_nn + suffix and tuple(p["grid"]) == (56, 4, 1) and tuple(p["block"]) == (512, 1, 1), p
             assert p["workspace_bytes"] == 65536 + 56 * 4 * tile_rows * 256 * 4, p       # one fp32 partial tile per (slab, K range)
-        assert mz.gemm_plan(ex(64, 4096, 4096, in_type=it))["kernel"] == direct + "_h128_splitk"                  # few slabs
+        assert mz.gemm_plan(ex(64, 4096, 4096, in_type=it))["kernel"] in (direct + "_h128_splitk", quarter_nn)   # few slabs (level)
         assert mz.gemm_plan(ex(16, 14344, 4096, in_type=it))["kernel"] == packed                                  # N % 16 != 0: copies (the per-wave kernel would walk K = 4096 alone)
         assert mz.gemm_plan(ex(16, 14344, 264, in_type=it))["kernel"] == "maize_gemm_bf16_wave32"                 # ... a short K: not worth the copies
         assert not _supports(few_nn, ex(16, 14344, 4096, in_type=it)) and not _supports(few_nn, ex(17, 14336, 4096, in_type=it))

@@ -395,10 +395,9 @@ def test_half_height_tiles_on_8bit_operands(ctx, oracle, fmt):
         for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=792), dict(lda=416, ldb=bcols + 16, ldc=800), dict(out_f16=True)):
             assert run_f8(ctx, oracle, 520, 784, 400, layout=layout, fmt=fmt, kernel=gen, label="h128 f8 knobs", **kw) == gen
             assert run_f8(ctx, oracle, 520, 784, 400, layout=layout, fmt=fmt, kernel=gen3, label="h128r3 f8 knobs", **kw) == gen3
-        # (the dispatcher's own choice: N x K products of up to 256 tiles of 128 x 128 and whole K tiles of 128 go to the 128 x 128
+        # (the dispatcher's own choice: products of up to 256 tiles of 128 x 128 and whole K tiles of 128 go to the 128 x 128
         # tile kernels, tests/test_gpu_tile128.py)
-        auto = (1152, 4096, 1024) if layout == mz.LAYOUT_NT else (512, 2048, 1024)
-        assert run_f8(ctx, oracle, *auto, layout=layout, fmt=fmt, label="h128 f8 auto") == gen
+        assert run_f8(ctx, oracle, 1152, 4096, 1024, layout=layout, fmt=fmt, label="h128 f8 auto") == gen
         assert run_f8(ctx, oracle, 100, 2048, 8192, layout=layout, fmt=fmt, label="h128 f8 auto, cut over K") == split
         m, n, k = 640, 784, 1168
         a = f8_uniform(oracle, m * k, 91, elem[0])
@@ -421,12 +420,13 @@ def test_dispatch_of_8bit_products(ctx):
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nt"
     assert pick(4096, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn"          # row-major B: read where it lies
     assert pick(4096, 4104, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_trb"      # ... N % 16: transposed copy
-    assert pick(2048, 2048, 2048, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn_h128_gen"      # half a round of 128-row tiles, 16 K steps
-    assert pick(1024, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn_h128r3_gen"    # ... 32 K steps: three ring stages
+    assert pick(1152, 4096, 2048, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn_h128_gen"      # half a round of 128-row tiles, 16 K steps
+    assert pick(1536, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nn_h128r3_gen"    # ... 32 K steps: three ring stages
+    assert pick(1024, 4096, 4096, mz.LAYOUT_NN, mz.IN_E4M3) == "maize_gemm_e4m3_t128_nn"                # K x N too (26.4 -> 19.2 us)
     assert pick(2048, 2048, 2048, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_t128_nt"                # N x K: one round of 256 tiles of 128 x 128 (16.3 -> 12.0 us)
     assert pick(1024, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_t128_nt"                # (25.1 -> 19.1 us)
     assert pick(1536, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_h128r3_gen"    # 384 of them would be two rounds
-    assert pick(1024, 4096, 2304, mz.LAYOUT_NN, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nn_h128r3_gen"    # (from 18 steps on)
+    assert pick(1536, 4096, 2304, mz.LAYOUT_NN, mz.IN_E5M2) == "maize_gemm_e5m2_mt256_nn_h128r3_gen"    # (from 18 steps on)
     assert pick(4096, 4096, 4104, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_e4m3_mt256_nt_packed"   # K % 16: padded copies
     assert pick(4096, 4096, 4096, mz.LAYOUT_NT, mz.IN_E4M3, lda=4104) == "maize_gemm_e4m3_mt256_nt_packed"
     assert pick(64, 64, 64, mz.LAYOUT_NT, mz.IN_E4M3) == "maize_gemm_bf16_wave32"

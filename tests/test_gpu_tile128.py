@@ -57,29 +57,34 @@ def test_half_operands_views_and_the_general_epilogue(ctx, oracle, layout):
     assert run_ex(ctx, oracle, 1024, 2048, 1024, layout=layout, half=True, label="t128 auto half") == f"maize_gemm_f16_t128_{tag}"
 
 
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NT, mz.LAYOUT_NN], ids=["nt", "nn"])
 @pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e4m3e5m2", "e5m2e4m3"])
-def test_8bit_operands(ctx, oracle, fmt):
-    """maize_gemm_{e4m3,...}_t128_nt: the same tiles on 8-bit operands stored N x K (a K step is one v_mfma_f32_16x16x128_f8f6f4
-    deep; B's fragments alternate between two register sets, two steps per trip, odd step counts padded with a tile past K).
+def test_8bit_operands(ctx, oracle, fmt, layout):
+    """maize_gemm_{e4m3,...}_t128_{nt,nn}: the same tiles on 8-bit operands (a K step is one v_mfma_f32_16x16x128_f8f6f4
+    deep; B's fragments alternate between two register sets, two steps per trip, odd step counts padded with a tile past K;
+    a row-major B lands as 128 rows of 128 B and is read through ds_read_b64_tr_b8).
     Against the oracle on views with leading dimensions, alpha / beta and an fp32 C; bit for bit against the 256-row
     general kernel; and as the dispatcher's choice."""
     from tests import test_gpu_gemm_f8 as T8
-    name = f"maize_gemm_{fmt}_t128_nt"
-    NT = mz.LAYOUT_NT
-    for (m, n, k) in ((128, 128, 128), (300, 264, 384), (520, 776, 640), (130, 136, 256)):          # 1, 3, 5 and 2 steps
-        for kw in (dict(), dict(lda=k + 16, ldb=k + 32, ldc=n + 8), dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5)):
+    nt = layout == mz.LAYOUT_NT
+    tag = "nt" if nt else "nn"
+    name = f"maize_gemm_{fmt}_t128_{tag}"
+    for (m, n, k) in ((128, 128, 128), (300, 272, 384), (520, 784, 640), (130, 144, 256)):          # 1, 3, 5 and 2 steps (N % 16 == 0 for a row-major B)
+        for kw in (dict(), dict(lda=k + 16, ldb=(k if nt else n) + 32, ldc=n + 8), dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5)):
             print(f"128 x 128 tiles: {name} {(m, n, k)} {kw}", flush=True)
-            assert T8.run_f8(ctx, oracle, m, n, k, layout=NT, fmt=fmt, kernel=name, label="t128 f8", **kw) == name
+            assert T8.run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, kernel=name, label="t128 f8", **kw) == name
     elem = T8.FMT[fmt][1]
-    for (m, n, k) in ((1024, 4096, 1152), (1000, 1032, 1152), (256, 256, 128), (2048, 2048, 1024)):
+    for (m, n, k) in ((1024, 4096, 1152), (1000, 1040, 1152), (256, 256, 128), (2048, 2048, 1024)):
         a = T8.f8_uniform(oracle, m * k, 5, T8.ab_of(elem)[0])
         b = T8.f8_uniform(oracle, n * k, 6, T8.ab_of(elem)[1])
         c0 = np.zeros(m * n, np.uint16)
-        want, _ = T8.launch(ctx, a, b, c0, m, n, k, NT, fmt, k, k, n, kernel=f"maize_gemm_{fmt}_mt256_nt_gen")
-        got, took = T8.launch(ctx, a, b, c0, m, n, k, NT, fmt, k, k, n, kernel=name)
+        ldb = k if nt else n
+        want, _ = T8.launch(ctx, a, b, c0, m, n, k, layout, fmt, k, ldb, n, kernel=f"maize_gemm_{fmt}_mt256_{tag}_gen")
+        got, took = T8.launch(ctx, a, b, c0, m, n, k, layout, fmt, k, ldb, n, kernel=name)
         assert took == name and np.array_equal(got, want), f"{(m, n, k)}: {int((got != want).sum())} of {got.size} elements differ"
-    assert T8.run_f8(ctx, oracle, 1024, 2048, 1024, layout=NT, fmt=fmt, label="t128 f8 auto") == name
-    assert T8.run_f8(ctx, oracle, 40, 8192, 512, layout=NT, fmt=fmt, label="t128 f8 auto, few rows") == name
+    assert T8.run_f8(ctx, oracle, 1024, 2048, 1024, layout=layout, fmt=fmt, label="t128 f8 auto") == name
+    if nt:
+        assert T8.run_f8(ctx, oracle, 40, 8192, 512, layout=layout, fmt=fmt, label="t128 f8 auto, few rows") == name
 
 
 def test_the_dispatcher_takes_them_for_one_round_of_tiles(ctx):

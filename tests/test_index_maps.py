@@ -25,7 +25,7 @@ def test_lds_maps_by_enumeration(tmp_path):
     r = subprocess.run([str(exe)], capture_output=True, text=True)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "all LDS maps check out" in r.stdout
-    assert r.stdout.count("ok  ") == 10
+    assert r.stdout.count("ok  ") == 11
 
 
 def test_kernels_use_the_shared_maps():

@@ -401,24 +401,26 @@ T128_LINES = ("request(0u, 0u);", "request(BKE, 1u);", "request(2u * BKE, 2u);",
 # each of the first six MFMAs of the half step before), rows 2-3 A fragments 2, 3 (4 reads, one behind each of the first four
 # MFMAs of rows 0-1); one request behind each of rows 0-1's eight MFMAs; two steps per trip, the count rounded up to an even
 # number with a tile past K
-T128_F8_LINES = ("read_a(0, 0u);\n        read_b(std::integral_constant<int, 0>{}, 0u);",
+T128_F8_LINES = ("constexpr int NEXT_READS = TR8 ? 20 : 12, NEXT_PER_SLOT = TR8 ? 3 : 2;",
+                 "for (int q = 0; q < NEXT_READS; ++q) read_next(std::integral_constant<int, 0>{}, 0u, q);",
                  "asm volatile(\"s_waitcnt lgkmcnt(0)\");\n            const TileReq r = tile_req((kt + 3u) * BKE, (kt + 3u) & 3u);",
-                 "mfma8(acc[i][j], b8[S][j], a8[i]);",
+                 "mfma8(acc[i][j], set, j, a8[i]);",
                  "if (4 * i + j < 4) rd128(a8[2 + (4 * i + j) / 2][(4 * i + j) & 1], a_rd[(4 * i + j) & 1] + so, 2 + (4 * i + j) / 2);\n                    piece(r, 4 * i + j);",
                  'asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");\n#pragma unroll\n            for (int i = 2; i < 4; ++i)',
-                 "for (int q = 2 * (4 * (i - 2) + j); q < 2 * (4 * (i - 2) + j) + 2; ++q) {",
-                 "else if (q < 12) rd128(b8[1 - S][(q - 4) / 2][q & 1], b_rd[q & 1] + so_next, (q - 4) / 2);",
+                 "for (int q = NEXT_PER_SLOT * (4 * (i - 2) + j); q < NEXT_PER_SLOT * (4 * (i - 2) + j + 1); ++q)\n                        if (q < NEXT_READS) read_next(std::integral_constant<int, 1 - S>{}, so_next, q);",
                  "for (uint32_t kt = 0; kt < nk; kt += 2u) {\n            step8(std::integral_constant<int, 0>{}, kt);\n            step8(std::integral_constant<int, 1>{}, kt + 1u);")
 
 
-def t128_f8_wave_program(nk, keep=16, reads_before_barrier=False, late_rows=4):
+def t128_f8_wave_program(nk, keep=16, reads_before_barrier=False, late_rows=4, tr=False):
+    """tr: B stored K x N -- a fragment of B is four transposing reads, the next tile's reads are 20, three behind an MFMA."""
     src = open(os.path.join(KDIR, "gemm_t128.hpp")).read()
     for fact in T128_LINES + T128_F8_LINES:
         assert fact in src, fact
+    nxt, per = (20, 3) if tr else (12, 2)
     steps = nk + (nk & 1)
     ops = [("dma", t, pc, t % 4) for t in range(3) for pc in range(8)]
     ops += [("wait_keep", keep), ("barrier",)]
-    ops += [("read", 0, 0, 0)] * 12
+    ops += [("read", 0, 0, 0)] * nxt
     for t in range(steps):
         for m in range(8):
             ops.append(("mfma", t, 0))
@@ -426,20 +428,22 @@ def t128_f8_wave_program(nk, keep=16, reads_before_barrier=False, late_rows=4):
                 ops.append(("read", t, 1, t % 4))
             ops.append(("dma", t + 3, m, (t + 3) % 4))
         if reads_before_barrier:
-            ops += [("read", t + 1, 0, (t + 1) % 4)] * 12
+            ops += [("read", t + 1, 0, (t + 1) % 4)] * nxt
         ops += [("wait_keep", keep), ("barrier",)]
         for m in range(8):
             ops.append(("mfma", t, 1))
-            if not reads_before_barrier and m < 6:
-                ops += [("read", t + 1, 0, (t + 1) % 4)] * 2
+            if not reads_before_barrier:
+                ops += [("read", t + 1, 0, (t + 1) % 4)] * max(0, min(per, nxt - per * m))
     ops.append(("wait_all",))
     return ops, steps
 
 
+@pytest.mark.parametrize("tr", [False, True])
 @pytest.mark.parametrize("nk", [1, 2, 3, 4, 5, 8, 33])
-def test_tiles_of_128_by_128_8bit_schedule_is_hazard_free(nk):
-    ops, steps = t128_f8_wave_program(nk)
-    assert check_two_stage(ops, steps, [12, 16], parts=2, pieces=8, nst=4) == steps + 2
+def test_tiles_of_128_by_128_8bit_schedule_is_hazard_free(nk, tr):
+    ops, steps = t128_f8_wave_program(nk, tr=tr)
+    first = 20 if tr else 12
+    assert check_two_stage(ops, steps, [first, first + 4], parts=2, pieces=8, nst=4) == steps + 2
 
 
 def test_tiles_of_128_by_128_8bit_checker_rejects_broken_schedules():

@@ -151,6 +151,10 @@ def test_the_description_chooses_the_panel_height_and_the_ring_depth():
     am.elem_bytes = bm.elem_bytes = 1
     k8, _ = describe(am, bm, cm, mma=T.Gfx950MfmaE4M3E5M2F32_16x16x128, nt=True, ktile=128, tiles=(T.F8_128x128, T.F8_128x128), **q128)
     assert k8.finalize().compile(mz.Gfx.Gfx950, cus).kernel_name == "maize_gemm_e4m3e5m2_t128_nt"
+    am, bm, cm = matrices(1024, 4096, 4096)
+    am.elem_bytes = bm.elem_bytes = 1
+    k8, _ = describe(am, bm, cm, mma=T.Gfx950MfmaE4M3E5M2F32_16x16x128, ktile=128, tiles=(T.F8_128x128, T.F8_128x128_KN), **q128)
+    assert k8.finalize().compile(mz.Gfx.Gfx950, cus).kernel_name == "maize_gemm_e4m3e5m2_t128_nn"
     with pytest.raises(ValueError, match="ring of four stages"):
         describe(a, b, c, nt=True, tiles=(T.BF16_128x64, T.BF16_128x64), depth=3, a_panel=128, panel=128)
     with pytest.raises(ValueError, match="B stage is BF16_128x64"):                     # K x N B needs the K x N stage
