@@ -35,6 +35,7 @@ MEASURED_TRAFFIC = {"cfg1": ("maize_gemm_bf16_mt256_nn", 235.2e6), "cfg2": ("mai
                     "m64": ("maize_gemm_bf16_skinny_nn_m64", 153.1e6),
                     "cfg5": ("maize_gemm_bf16_mt256_nn", 1074.3e6), "sq2048": ("maize_gemm_bf16_t128_nn", 58.9e6), "mid": ("maize_gemm_bf16_t128_nt", 109.2e6), "f8": ("maize_gemm_e4m3_mt256_nt", 134.5e6),
                     "f8n": ("maize_gemm_e4m3_mt256_nn", 134.5e6),
+                    "f8mid": ("maize_gemm_e4m3_t128_nt", 58.9e6),
                     "f8s": ("maize_gemm_e4m3_skinny_nt", 67.2e6), "f32": ("maize_gemm_f32_mt128_nn", 828.9e6),
                     "f64": ("maize_gemm_f64_mt128_nn", 3162.3e6)}
 
