@@ -239,19 +239,25 @@ class PowerSampler:
         return sum(1 for t, _ in self.samples if t0 <= t <= t1)
 
 
-def box_ceiling(mz, ctx, stream, launches=50):
+CEILING_PROBES = {None: ("maize_probe_mfma_loop_16x16x32", 512, "v_mfma_f32_16x16x32_bf16"),
+                  "e4m3": ("maize_probe_mfma_loop_16x16x128_e4m3", 128, "v_mfma_f32_16x16x128_f8f6f4 on E4M3")}
+
+
+def box_ceiling(mz, ctx, stream, launches=50, in_type=None):
     """What this box's matrix pipe does right now with no data movement at all: a register-only loop of
     v_mfma_f32_16x16x32_bf16 on random operands, 256 workgroups x 4 waves x 512 rounds x 131072 multiply-adds = the
-    multiply-adds of 4096^3, timed by HIP events on `stream` straight after the timed region (same clocks, same
-    temperature).  A slow or hot box shows up here as a slow ceiling.  Returns microseconds per launch."""
+    multiply-adds of 4096^3 (E4M3 operands: v_mfma_f32_16x16x128_f8f6f4, 128 rounds x 524288), timed by HIP events on
+    `stream` straight after the timed region (same clocks, same temperature).  A slow or hot box shows up here as a
+    slow ceiling.  Returns microseconds per launch."""
     import ctypes as C
 
     class LoopArgs(C.Structure):
         _fields_ = [("out", C.c_void_p), ("iters", C.c_uint32), ("zero", C.c_uint32)]
 
     out = ctx.malloc(4096)
-    kern = mz.new_hip_kernel("maize_probe_mfma_loop_16x16x32").with_launch_bounds_1d(256).finalize().compile(mz.Gfx.Gfx950, ctx)
-    args = LoopArgs(out.ptr, 512, 0)
+    probe, rounds, _ = CEILING_PROBES[in_type]
+    kern = mz.new_hip_kernel(probe).with_launch_bounds_1d(256).finalize().compile(mz.Gfx.Gfx950, ctx)
+    args = LoopArgs(out.ptr, rounds, 0)
     ev0, ev1 = ctx.event(), ctx.event()
     for _ in range(10):
         kern.launch((256, 1, 1), args, stream=stream)
@@ -433,8 +439,8 @@ def main():
         return
     import maize_amd as mz
     ctx = mz.Context(0)
-    bf16_mfma = CONFIGS[args.config]['bound'] == 'mfma' and CONFIGS[args.config].get('in_type') is None
-    line = measure(mz, ctx, args.config, args.steps, args.warmup, args.kernel, args.rotate, not args.no_cpu, ceiling=bf16_mfma)
+    probed = CONFIGS[args.config]['bound'] == 'mfma' and CONFIGS[args.config].get('in_type') in CEILING_PROBES
+    line = measure(mz, ctx, args.config, args.steps, args.warmup, args.kernel, args.rotate, not args.no_cpu, ceiling=probed)
     if args.others:
         # The other benchmark configurations, shorter runs, same process: reported beside the headline.
         others = {}
@@ -522,7 +528,7 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu, ceil
     wall_t1 = time.time()
     ev_ms = ev0.elapsed_ms(ev1)
     # The box's own ceiling, straight behind the timed region: the same multiply-adds from registers only.
-    ceiling_us = box_ceiling(mz, ctx, stream) if ceiling else None
+    ceiling_us = box_ceiling(mz, ctx, stream, in_type=cfg.get("in_type")) if ceiling else None
     if sampler is not None and sampler.path is not None:
         sampler.__exit__()
 
@@ -551,7 +557,8 @@ def measure(mz, ctx, config, steps, warmup, force_kernel, rotate, with_cpu, ceil
         roof["box_ceiling_us"] = scaled
         roof["box_ceiling_frac_of_peak"] = flops / (scaled * 1e-6) / 1e12 / peak_flops
         roof["frac_of_box_ceiling"] = scaled / (kern_ms * 1e3)
-        roof["box_ceiling_source"] = ("maize_probe_mfma_loop_16x16x32: v_mfma_f32_16x16x32_bf16 from registers only, uniform random "
+        probe, _, what = CEILING_PROBES[cfg.get("in_type")]
+        roof["box_ceiling_source"] = (f"{probe}: {what} from registers only, uniform random "
                                       "operands, the workload's multiply-adds, 50 launches straight after the timed region")
         watts = sampler.mean_between(wall_t0, wall_t1) if sampler.path else None
         roof["board_watts_timed_region"] = watts

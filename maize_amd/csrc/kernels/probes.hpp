@@ -108,6 +108,50 @@ extern "C" __global__ __launch_bounds__(256) void maize_probe_mfma_loop_32x32x16
     if (s[0] + s[5] == 12345.f) p.out[threadIdx.x] = s[0];
 }
 
+// The same for 8-bit operands: v_mfma_f32_16x16x128_f8f6f4 on E4M3 (cbsz = blgp = 0) from registers only, 16
+// independent accumulators.  One round is 524288 multiply-adds per wave: `iters` = 128 on 256 workgroups of 4 waves
+// does the multiply-adds of a 4096^3 product.  Operands: zeros, or uniform [-1, 1) rounded to E4M3 as the 8-bit
+// workloads' generators make them (built from bits here: sign, a geometric exponent, three random mantissa bits;
+// never the NaN pattern).
+typedef int probe_i32x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ probe_i32x8 probe_operand_e4m3(uint32_t salt, uint32_t zero) {
+    probe_i32x8 r;
+    for (int w = 0; w < 8; ++w) {
+        uint32_t word = 0;
+        for (int e = 0; e < 4; ++e) {
+            uint32_t h = threadIdx.x * 256 + salt * 32 + w * 4 + e + blockIdx.x * 77777;
+            h ^= h >> 16; h *= 0x7feb352dU; h ^= h >> 15; h *= 0x846ca68bU; h ^= h >> 16;
+            // |x| uniform in [0, 1): exponent field 6 with probability 1/2, 5 with 1/4, ... (bias 7)
+            const uint32_t lead = (uint32_t)__builtin_clz((h & 0xFFFFu) | 0x200u) - 16u;       // 0 .. 6
+            const uint32_t byte = ((h >> 31) << 7) | ((6u - lead) << 3) | ((h >> 16) & 7u);
+            word |= byte << (8 * e);
+        }
+        r[w] = zero ? 0 : (int)word;
+    }
+    return r;
+}
+extern "C" __global__ __launch_bounds__(256) void maize_probe_mfma_loop_16x16x128_e4m3(MfmaLoopArgs p) {
+    floatx4 c0 = {}, c1 = {}, c2 = {}, c3 = {}, c4 = {}, c5 = {}, c6 = {}, c7 = {}, c8 = {}, c9 = {}, c10 = {}, c11 = {}, c12 = {}, c13 = {}, c14 = {}, c15 = {};
+    probe_i32x8 a0 = probe_operand_e4m3(0, p.zero), a1 = probe_operand_e4m3(1, p.zero), a2 = probe_operand_e4m3(2, p.zero), a3 = probe_operand_e4m3(3, p.zero);
+    probe_i32x8 b0 = probe_operand_e4m3(4, p.zero), b1 = probe_operand_e4m3(5, p.zero), b2 = probe_operand_e4m3(6, p.zero), b3 = probe_operand_e4m3(7, p.zero);
+    for (uint32_t it = 0; it < p.iters; ++it) {
+        asm volatile(
+            "v_mfma_f32_16x16x128_f8f6f4 %0, %16, %20, %0\n\tv_mfma_f32_16x16x128_f8f6f4 %1, %16, %21, %1\n\t"
+            "v_mfma_f32_16x16x128_f8f6f4 %2, %16, %22, %2\n\tv_mfma_f32_16x16x128_f8f6f4 %3, %16, %23, %3\n\t"
+            "v_mfma_f32_16x16x128_f8f6f4 %4, %17, %20, %4\n\tv_mfma_f32_16x16x128_f8f6f4 %5, %17, %21, %5\n\t"
+            "v_mfma_f32_16x16x128_f8f6f4 %6, %17, %22, %6\n\tv_mfma_f32_16x16x128_f8f6f4 %7, %17, %23, %7\n\t"
+            "v_mfma_f32_16x16x128_f8f6f4 %8, %18, %20, %8\n\tv_mfma_f32_16x16x128_f8f6f4 %9, %18, %21, %9\n\t"
+            "v_mfma_f32_16x16x128_f8f6f4 %10, %18, %22, %10\n\tv_mfma_f32_16x16x128_f8f6f4 %11, %18, %23, %11\n\t"
+            "v_mfma_f32_16x16x128_f8f6f4 %12, %19, %20, %12\n\tv_mfma_f32_16x16x128_f8f6f4 %13, %19, %21, %13\n\t"
+            "v_mfma_f32_16x16x128_f8f6f4 %14, %19, %22, %14\n\tv_mfma_f32_16x16x128_f8f6f4 %15, %19, %23, %15"
+            : "+a"(c0), "+a"(c1), "+a"(c2), "+a"(c3), "+a"(c4), "+a"(c5), "+a"(c6), "+a"(c7), "+a"(c8), "+a"(c9), "+a"(c10), "+a"(c11),
+              "+a"(c12), "+a"(c13), "+a"(c14), "+a"(c15)
+            : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b0), "v"(b1), "v"(b2), "v"(b3));
+    }
+    floatx4 s = c0 + c1 + c2 + c3 + c4 + c5 + c6 + c7 + c8 + c9 + c10 + c11 + c12 + c13 + c14 + c15;
+    if (s[0] + s[1] + s[2] + s[3] == 12345.f) p.out[threadIdx.x] = s[0];
+}
+
 // LDS transpose read (ds_read_b64_tr_b16).  LDS is filled with lds_init
 // (n_init u16 values); lane l reads at byte offset byte_off[l]; out receives
 // 4 u16 per lane.
