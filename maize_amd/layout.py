@@ -306,17 +306,21 @@ def reference_row_panels(nrows, grid, panel=16):
     return tiled_divide(Layout(Shape(nrows), Stride(1)), Tile((grid,), (panel,))).canonicalize()
 
 
-def macro_tile_of_c(ldc):
-    """One 256 x 256 workgroup tile of C as the macro-tile kernel's epilogue sees it.  Rows: 2 waves (wm) x 8
-    accumulator rows (i) x 16 lanes (l % 16); columns: 2 waves (wn) x 8 accumulator columns (j) x 4 lane groups
-    (l / 16) x 4 consecutive elements (v).  Returns f(wm, i, l16, wn, j, lg, v) -> element offset inside the tile,
-    each mode divided step by step with tiled_divide."""
+def macro_tile_of_c(ldc, rows=256, cols=256):
+    """One workgroup tile of C as the tile kernels' epilogues see it: 256 x 256 (the macro-tile kernels), 128 x 256
+    (their half-height variants) or 128 x 128 (the four-stage kernels).  Rows: 2 waves (wm) x rows / 32 accumulator
+    rows (i) x 16 lanes (l % 16); columns: 2 waves (wn) x cols / 32 accumulator columns (j) x 4 lane groups (l / 16)
+    x 4 consecutive elements (v).  Returns f(wm, i, l16, wn, j, lg, v) -> element offset inside the tile, each mode
+    divided step by step with tiled_divide."""
+    if (rows, cols) not in ((256, 256), (128, 256), (128, 128)):
+        raise ValueError("tiles are 256 x 256, 128 x 256 or 128 x 128")
+
     def cut(extent, stride, parts):
         # `parts` tiles of extent / parts elements, side by side, each once: coordinate (part, (0, rest))
         return tiled_divide(Layout(Shape(extent), Stride(stride)), Tile((parts,), (extent // parts,))).canonicalize()
 
-    rows_by_wave, rows_by_acc = cut(256, ldc, 2), cut(128, ldc, 8)
-    cols_by_wave, cols_by_acc, cols_by_group = cut(256, 1, 2), cut(128, 1, 8), cut(16, 1, 4)
+    rows_by_wave, rows_by_acc = cut(rows, ldc, 2), cut(rows // 2, ldc, rows // 32)
+    cols_by_wave, cols_by_acc, cols_by_group = cut(cols, 1, 2), cut(cols // 2, 1, cols // 32), cut(16, 1, 4)
 
     def offset(wm, i, l16, wn, j, lg, v):
         return (rows_by_wave.offset((wm, (0, 0))) + rows_by_acc.offset((i, (0, l16))) +

@@ -124,3 +124,25 @@ def test_macro_tile_decomposition_is_the_epilogue_lane_map():
                             assert o == (wm * 128 + 16 * i + lane % 16) * ldc + wn * 128 + 16 * j + 4 * (lane // 16) + v
                             seen.add(o)
     assert len(seen) == 256 * 256                         # every element of the tile, once
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 256), (128, 128)])
+def test_the_smaller_tiles_decompose_the_same_way(rows, cols):
+    """The half-height and the 128 x 128 tile kernels keep the wave grid (2 x 2) and the lane map; only the number of
+    accumulators per wave changes: lane l of wave (wm, wn) holds, in accumulator (i, j),
+    C[row = wm rows/2 + 16 i + l % 16][col = wn cols/2 + 16 j + 4 (l / 16) + v]."""
+    ldc = 2056
+    off = L.macro_tile_of_c(ldc, rows, cols)
+    seen = set()
+    for wm in range(2):
+        for wn in range(2):
+            for i in range(rows // 32):
+                for j in range(cols // 32):
+                    for lane in range(64):
+                        for v in range(4):
+                            o = off(wm, i, lane % 16, wn, j, lane // 16, v)
+                            assert o == (wm * (rows // 2) + 16 * i + lane % 16) * ldc + wn * (cols // 2) + 16 * j + 4 * (lane // 16) + v
+                            seen.add(o)
+    assert len(seen) == rows * cols
+    with pytest.raises(ValueError):
+        L.macro_tile_of_c(ldc, 64, 64)
