@@ -152,6 +152,24 @@ def test_matrix_instruction_per_kernel(kernels):
             assert count(ins, "v_mfma_f32_32x32x16_bf16") >= 1 and count(ins, "v_mfma_f32_32x32x16_f16") >= 1
 
 
+def test_the_register_only_loops_are_nothing_but_matrix_instructions(kernels):
+    """The loops bench.py times as the box's ceiling: 16 independent matrix instructions per round and a branch, no
+    loads, no LDS, no moves between the register files."""
+    for name, mnemonic in (("maize_probe_mfma_loop_16x16x32", "v_mfma_f32_16x16x32_bf16"),
+                           ("maize_probe_mfma_loop_16x16x128_e4m3", "v_mfma_f32_16x16x128_f8f6f4")):
+        ins = kernels[name]
+        first = next(i for i, x in enumerate(ins) if x.startswith(mnemonic))
+        last = max(i for i, x in enumerate(ins) if x.startswith(mnemonic))
+        loop = ins[first:last + 1]
+        assert len(loop) == 16 and all(x.startswith(mnemonic) for x in loop), (name, loop)
+        assert "cbsz" not in " ".join(loop) and "blgp" not in " ".join(loop), name          # E4M3 on both sides
+        assert len({x.split()[1].rstrip(",") for x in loop}) == 16, name                    # 16 different accumulators
+        back = next(x for x in ins[last + 1:] if x.startswith("s_cbranch"))
+        assert back.startswith("s_cbranch_scc"), name
+        between = ins[last + 1:ins.index(back, last + 1)]
+        assert all(x.startswith(("s_add", "s_sub", "s_cmp")) for x in between), (name, between)
+
+
 def test_data_movement_the_design_rests_on(kernels):
     for name, ins in kernels.items():
         if "_mt256_" in name or name.startswith("maize_gemm_bf16_skinny_nn"):
