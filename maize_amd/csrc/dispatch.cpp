@@ -349,7 +349,10 @@ bool h128_three_stages(uint32_t k, uint32_t kstep, uint64_t half_tiles, bool ran
     // (K ranges of a split, every candidate by name on 96 mid-size shapes: three stages win from 13 steps per range --
     // 256 x 4096 x 4096 in five ranges 26.1 -> 24.7 us, 512 x 2048 x 8192 in eight ranges of 16 steps 37.4 -> 33.2,
     // 384 x 4096 x 4096 in four 31.4 -> 29.2)
-    return nk >= (kstep == 128u ? 18u : range ? 12u : 16u) && (nk >= 48u || half_tiles >= 48u);
+    // (K ranges of 8-bit operands: from 8 steps per range, the shortest measured -- E4M3, both layouts, 96 products with
+    // every candidate by name: three stages 1-8 % ahead at 8 steps a range (256 x 2048 x 8192 in eight 20.8 -> 19.0 us), 8 % at 11
+    // (512 x 2048 x 8192 in six 24.6 -> 22.7), 7-11 % at 16, 9-19 % from 19 on; never behind)
+    return nk >= (kstep == 128u ? (range ? 8u : 18u) : range ? 12u : 16u) && (nk >= 48u || half_tiles >= 48u);
 }
 // What a K step of a 128-row tile costs, in steps of the 256-row kernel at the power limit (~ microseconds): 0.67 on two
 // ring stages, 0.52 on three; K ranges of a row-major 16-bit B on three stages 0.55 (same plans, same box, K x N against
@@ -1108,10 +1111,15 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
             if (t8 >= 0 && s.k >= 256u && tiles <= units && (tiles >= 16u || s.k <= 1024u) && kKernels[t8].supports(d)) {
                 const uint32_t nk = cdiv(s.k, 128u);
                 const double cost_t = 8.0 + (t128_step8(tiles, nk) + (s.nt ? 0.0 : 0.04)) * nk;      // (K x N: twice the LDS instructions per fragment of B)
-                if (cost_t >= stream_us(s, d.gemm.batch, 128u, tiles) && cost_t < (hk >= 2u ? 0.92 : 0.97) * cost_hk) return (uint32_t)t8;
+                // (on a quarter of the compute units or fewer, 48 steps or more belong to the cut, whose fixed terms the model
+                // overrates by about 6 us for 8-bit operands -- E4M3 N x K, here / cut: 512 x 2048 x 8192, 64 tiles, 26.0 / 22.7 us,
+                // 384 x 2048 x 8192 25.9 / 20.8, 512 x 1024 x 8192 25.8 / 19.1, 100 x 8192 x 8192 25.4 / 23.2, 200 x 4096 x 6144 20.8 / 19.6;
+                // at 32 steps the tiles keep their lead: 128 x 4096 x 4096 14.6 / 16.9, 256 x 2048 x 4096 14.7 / 17.1, 256 x 4096 x 4096 14.9 / 20.1)
+                const double rival = hk >= 2u ? 0.92 * (cost_hk - (tiles * 4u <= units && nk >= 48u ? 6.0 : 0.0)) : 0.97 * cost_hk;
+                if (cost_t >= stream_us(s, d.gemm.batch, 128u, tiles) && cost_t < rival) return (uint32_t)t8;
             }
             if (hk >= 1u) {
-                const bool r3 = h128_three_stages(cdiv(cdiv(s.k, 128u), hk) * 128u, 128u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk);   // by the K steps of a range
+                const bool r3 = h128_three_stages(cdiv(cdiv(s.k, 128u), hk) * 128u, 128u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk, hk >= 2u);   // by the K steps of a range
                 std::snprintf(name, sizeof name, "maize_gemm_%s_mt256_%s_h128%s_%s", kTag[d.in_type - MAIZE_IN_E4M3], s.nt ? "nt" : "nn", r3 ? "r3" : "", hk >= 2u ? "splitk" : "gen");
                 const int fh = kernel_index(name);
                 if (fh >= 0 && kKernels[fh].supports(d) && plan_fits(kKernels[fh], d, compute_units)) return (uint32_t)fh;
