@@ -1316,25 +1316,33 @@ namespace {
 double tail_part_cost(const maize_gemm_ex_desc_t& part, uint32_t compute_units) {
     const Dims s = dims_of(part);
     const char* name = kKernels[select_kernel(part, compute_units)].name;
-    const uint32_t nk = cdiv(s.k, 64);
+    // (8-bit operands: a K step is 128 deep and takes 1.3 of a 16-bit one, as in h128_choice)
+    const bool bits8 = part.in_type >= MAIZE_IN_E4M3 && part.in_type <= MAIZE_IN_E5M2_E4M3;
+    const uint32_t kstep = bits8 ? 128u : 64u;
+    const double scale = bits8 ? 0.87 / 0.67 : 1.0;
+    const uint32_t nk = cdiv(s.k, kstep);
     const bool h128 = std::strstr(name, "_h128") != nullptr, three = std::strstr(name, "_h128r3") != nullptr;
     const double launch = 3.0 + 8.0;
     if (std::strstr(name, "_splitk")) {
-        const uint32_t ks = h128 ? h128_choice(s, 1, compute_units) : splitk_ranges(s, 1, compute_units);
+        const uint32_t ks = h128 ? h128_choice(s, 1, compute_units, kstep) : splitk_ranges(s, 1, compute_units, kstep);
         if (ks < 2u) return -1.0;
         const uint32_t r = cdiv(nk, ks);
-        const double step = h128 ? h128_step(three, true, s.nt, false) * r : 1.0 * r;
+        const double step = scale * (h128 ? h128_step(three, true, s.nt, bits8) * r : 1.0 * r);
         return launch + step + 6.0 + (1.2e-6 * (double)s.m * s.n + 0.15) * ks;
     }
-    if (h128 && std::strstr(name, "_mt256_")) return launch + h128_step(three, false, s.nt, false) * nk;
-    if (std::strstr(name, "_t128_")) return launch + t128_step(s.nt, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128), nk) * nk;   // (the same sums in the same order too)
+    if (h128 && std::strstr(name, "_mt256_")) return launch + scale * h128_step(three, false, s.nt, bits8) * nk;
+    if (std::strstr(name, "_t128_")) {                                                                                       // (the same sums in the same order too)
+        const uint64_t tiles = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 128);
+        return launch + (bits8 ? t128_step8(tiles, nk) + (s.nt ? 0.0 : 0.04) : t128_step(s.nt, tiles, nk)) * nk;
+    }
     return -1.0;
 }
 }  // namespace
 
 TailSplit tail_split(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     TailSplit none = {0, 0};
-    if (!(bf16_in(d) || half_in(d)) || d.gemm.batch != 1 || compute_units < 8u) return none;
+    const bool bits8 = d.in_type >= MAIZE_IN_E4M3 && d.in_type <= MAIZE_IN_E5M2_E4M3;
+    if (!(bf16_in(d) || half_in(d) || bits8) || d.gemm.batch != 1 || compute_units < 8u) return none;
     const Dims s = dims_of(d);
     // only where the whole product would run on a persistent macro-tile kernel, one tile per work item
     const char* name = kKernels[select_kernel(d, compute_units)].name;
@@ -1346,8 +1354,8 @@ TailSplit tail_split(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     const uint32_t resident = compute_units - compute_units % 8u;
     if (tiles <= resident || tiles % resident == 0) return none;
     const uint64_t full = tiles / resident * resident;                   // tiles of the whole rounds
-    const uint32_t nk = cdiv(s.k, 64);
-    const double t_round = 8.0 + 1.0 * nk;
+    const uint32_t nk = cdiv(s.k, bits8 ? 128u : 64u);
+    const double t_round = 8.0 + (bits8 ? 0.87 / 0.67 : 1.0) * nk;
     // The part set aside is worth a launch of its own only if it costs clearly less than the round it replaces: as
     // 128-row tiles that fit one round, or split over K.  By rows (the rows below the leading tile rows that fill the
     // rounds) or by columns (the columns to the right of the leading tile columns), whichever part is cheaper.

@@ -567,11 +567,12 @@ static int32_t gemm_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const
             const uint64_t lda = desc->lda ? desc->lda : desc->gemm.a.ncols, ldb = desc->ldb ? desc->ldb : desc->gemm.b.ncols,
                            ldc = desc->ldc ? desc->ldc : desc->gemm.c.ncols;
             const uint64_t csz = desc->out_type == MAIZE_OUT_F32 ? 4u : 2u;
+            const uint64_t esz = (desc->in_type >= MAIZE_IN_E4M3 && desc->in_type <= MAIZE_IN_E5M2_E4M3) ? 1u : 2u;   // bytes per element of A and B
             maize_gemm_ex_desc_t top = *desc, rest = *desc;
             if (cut.rows) {
                 top.gemm.a.nrows = top.gemm.c.nrows = cut.rows;
                 rest.gemm.a.nrows = rest.gemm.c.nrows = desc->gemm.a.nrows - cut.rows;
-                rest.gemm.a.ptr = (char*)desc->gemm.a.ptr + (uint64_t)cut.rows * lda * 2u;
+                rest.gemm.a.ptr = (char*)desc->gemm.a.ptr + (uint64_t)cut.rows * lda * esz;
                 rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)cut.rows * ldc * csz;
             } else {
                 // by columns: both parts keep the leading dimensions of the whole matrices
@@ -581,7 +582,7 @@ static int32_t gemm_ex(maize_ctx_t* ctx, const maize_gemm_ex_desc_t* desc, const
                 rest.gemm.c.ncols = n - cut.cols;
                 if (nt) { top.gemm.b.nrows = cut.cols; rest.gemm.b.nrows = n - cut.cols; }
                 else    { top.gemm.b.ncols = cut.cols; rest.gemm.b.ncols = n - cut.cols; }
-                rest.gemm.b.ptr = (char*)desc->gemm.b.ptr + (nt ? (uint64_t)cut.cols * ldb * 2u : (uint64_t)cut.cols * 2u);
+                rest.gemm.b.ptr = (char*)desc->gemm.b.ptr + (nt ? (uint64_t)cut.cols * ldb * esz : (uint64_t)cut.cols * esz);
                 rest.gemm.c.ptr = (char*)desc->gemm.c.ptr + (uint64_t)cut.cols * csz;
             }
             uint32_t itop, irest;

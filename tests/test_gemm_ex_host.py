@@ -319,9 +319,16 @@ def test_tail_split_by_rows():
     assert mz.gemm_tail_rows(ex(4000, 4104, 4032)) == 0          # narrow last tile column: edge splitting instead
     # a short K: the round that would be saved is cheap, the extra launches are not
     assert mz.gemm_tail_split(ex(4096, 4352, 256)) == (0, 0) and mz.gemm_tail_split(ex(2048, 11008, 1024)) == (0, 0)
-    # batches, 8-bit and wide operands are left alone; fewer compute units move the boundary
+    # 8-bit operands the same way, priced in their own K steps of 128 (E4M3 4352 x 4096 x 4096: 81.8 us in one kernel, 66.3 cut)
+    for it in (mz.IN_E4M3, mz.IN_E5M2, mz.IN_E4M3_E5M2, mz.IN_E5M2_E4M3):
+        for layout in (mz.LAYOUT_NT, mz.LAYOUT_NN):
+            assert mz.gemm_tail_split(ex(4352, 4096, 4096, layout=layout, in_type=it)) == (4096, 0)
+            assert mz.gemm_tail_split(ex(4096, 4352, 4096, layout=layout, in_type=it)) == (15 * 256, 0)     # 255 tiles on top, a tile row of 17 below
+            assert mz.gemm_tail_split(ex(2048, 11008, 4096, layout=layout, in_type=it)) == (0, 8192)
+            assert mz.gemm_tail_split(ex(4352, 4096, 512, layout=layout, in_type=it)) == (0, 0)               # a short K
+            assert mz.gemm_tail_split(ex(8192, 8192, 8192, layout=layout, in_type=it)) == (0, 0)              # whole rounds
+    # batches and wide operands are left alone; fewer compute units move the boundary
     assert mz.gemm_tail_split(ex(4096, 4352, 4096, batch=2, stride_a=4096 * 4096, stride_b=4096 * 4352, stride_c=4096 * 4352)) == (0, 0)
-    assert mz.gemm_tail_split(ex(4096, 4352, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3)) == (0, 0)
     assert mz.gemm_tail_split(ex(4096, 4352, 4096, in_type=mz.IN_F32)) == (0, 0)
     assert mz.gemm_tail_rows(x, compute_units=64) == 4096        # 272 = 4 x 64 + 16: 16 tile rows = 256 tiles are 4 rounds of 64
 

@@ -602,3 +602,36 @@ def test_half_c_is_rounded_to_half_not_through_bf16(ctx, oracle):
     assert np.all(got == want), f"{took}: {np.unique(got)[:8]} instead of {want:#06x}"
     got_bf16, _ = launch(ctx, a, b, c0, m, n, k, mz.LAYOUT_NT, "e4m3", k, k, n)
     assert not np.any(oracle.bf16_bits_to_f64(got_bf16) == 4112.0)          # the bf16 C of the same product cannot hold it
+
+
+@pytest.mark.parametrize("layout", [mz.LAYOUT_NT, mz.LAYOUT_NN], ids=["nt", "nn"])
+@pytest.mark.parametrize("fmt,shape", [("e4m3", (4352, 4096, 1024)), ("e4m3", (2048, 11008, 3072)), ("e5m2e4m3", (4100, 4352, 2048))],
+                         ids=lambda v: v if isinstance(v, str) else "x".join(map(str, v)))
+def test_tail_split_on_8bit_operands(ctx, oracle, fmt, shape, layout):
+    """A tile count a little over a round of compute units, 8-bit operands: the launcher runs the leading tile rows (or
+    columns) as one product and the rest as a second one behind it -- offsets into A and B counted in one-byte elements.
+    The whole of C against the oracle; the leading part bit for bit what the single kernel gives."""
+    m, n, k = shape
+    cus = ctx.info()["compute_units"]
+    brows, bcols = (k, n) if layout == mz.LAYOUT_NN else (n, k)
+    x = mz.gemm_ex_desc(mz.GlobalMatrix(0x10000, m, k), mz.GlobalMatrix(0x10000 + (1 << 40), brows, bcols), mz.GlobalMatrix(0x10000 + (2 << 40), m, n),
+                        layout=layout, in_type=FMT[fmt][0])
+    rows, cols = mz.gemm_tail_split(x, compute_units=cus)
+    _say(f"8-bit tail split {fmt} {shape} layout={layout}: cut ({rows}, {cols})")
+    if cus == 256:
+        assert (rows, cols) == {(4352, 4096, 1024): (4096, 0), (2048, 11008, 3072): (0, 8192), (4100, 4352, 2048): (3840, 0)}[shape]
+    single = run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, label="8-bit tail split (auto)")
+    elem = FMT[fmt][1]
+    a = f8_uniform(oracle, m * k, 101, ab_of(elem)[0])
+    b = f8_uniform(oracle, n * k, 201, ab_of(elem)[1])
+    c0 = np.zeros(m * n, np.uint16)
+    auto, _ = launch(ctx, a, b, c0, m, n, k, layout, fmt, k, bcols, n)
+    one, took = launch(ctx, a, b, c0, m, n, k, layout, fmt, k, bcols, n, kernel=single)
+    assert took == single
+    auto, one = auto.reshape(m, n), one.reshape(m, n)
+    if rows:
+        assert np.array_equal(auto[:rows], one[:rows])
+    elif cols:
+        assert np.array_equal(auto[:, :cols], one[:, :cols])
+    else:
+        assert np.array_equal(auto, one)
