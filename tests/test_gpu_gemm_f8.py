@@ -635,3 +635,12 @@ def test_tail_split_on_8bit_operands(ctx, oracle, fmt, shape, layout):
         assert np.array_equal(auto[:, :cols], one[:, :cols])
     else:
         assert np.array_equal(auto, one)
+    if shape == (4352, 4096, 1024):
+        # ... on views with leading dimensions, alpha / beta and an fp32 C: the seam's offsets follow lda / ldb / ldc
+        for kw in (dict(lda=k + 16, ldb=bcols + 32, ldc=n + 8, alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8)):
+            xv = mz.gemm_ex_desc(mz.GlobalMatrix(0x10000, m, k), mz.GlobalMatrix(0x10000 + (1 << 40), brows, bcols), mz.GlobalMatrix(0x10000 + (2 << 40), m, n),
+                                 layout=layout, in_type=FMT[fmt][0], lda=kw.get("lda", 0), ldb=kw.get("ldb", 0), ldc=kw.get("ldc", 0),
+                                 alpha=kw["alpha"], beta=kw["beta"], out_type=mz.OUT_F32 if kw.get("out_f32") else mz.OUT_SAME)
+            if cus == 256:
+                assert mz.gemm_tail_split(xv, compute_units=cus) == (4096, 0)
+            run_f8(ctx, oracle, m, n, k, layout=layout, fmt=fmt, label="8-bit tail split on views", **kw)
