@@ -1175,8 +1175,11 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     // fast as the four-row-group kernel and needs no second pass over partial tiles (row-group kernel -> 128 x 128 tiles, us:
     // 64 x 14336 x 4096 27.8 -> 25.9, 40 x 14336 x 4096 27.1 -> 25.2, 64 x 14336 x 2048 18.6 -> 15.8, 64 x 28672 x 4096 43.2 -> 36.8,
     // 64 x 32768 x 4096 52.7 -> 42.5, 56 x 28672 x 2048 26.4 -> 21.0, 64 x 16384 x 1024 16.6 -> 10.7; level at K = 8192, 47.4 / 46.9;
-    // 32 rows stay with the two-row-group kernel, 24.7 against 25.5; a row-major B with its own, 28.8 against 31.3)
-    if (s.nt && s.m > 32u && s.m <= 64u && s.k >= 256u && s.k <= 4096u && s.n >= 12288u) {
+    // 32 rows stay with the two-row-group kernel, 24.7 against 25.5; a row-major B with its own, 28.8 against 31.3).
+    // 65 .. 128 rows the same, where the model gives the cut over K partial tiles too cheap for their rows (128-row tiles in
+    // four ranges -> here: 80 x 16384 x 4096 32.0 -> 26.7, 72 x 14336 x 4096 28.7 -> 26.5, 128 x 14336 x 8192 53.1 -> 49.5; K x N is mixed,
+    // 128 x 14336 x 4096 33.6 / 31.3 but 72 x 14336 x 4096 29.0 / 30.6, and stays with the model)
+    if (s.nt && s.m > 32u && s.m <= 128u && s.k >= 256u && s.k <= (s.m > 64u ? 8192u : 4096u) && s.n >= 12288u) {
         const int t6 = kernel_index(half_in(d) ? "maize_gemm_f16_t128_nt" : "maize_gemm_bf16_t128_nt");
         const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
         if (t6 >= 0 && kKernels[t6].supports(d) && (uint64_t)cdiv(s.n, 128) * d.gemm.batch <= units) return (uint32_t)t6;
