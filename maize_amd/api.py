@@ -188,8 +188,27 @@ class Matrix:
         return GlobalMatrix(self.ptr, self.nrows, self.ncols)
 
 
-def gemm_desc(a, b, c, layout=LAYOUT_NN, batch=1, stride_a=0, stride_b=0, stride_c=0):
-    """Build a maize_gemm_desc_t from three Matrix (or MatrixT) operands."""
+def _check_extent(what, mat, ld, stride, batch, elem_bytes):
+    """A Matrix built on a DeviceBuffer knows how many bytes it may touch: refuse a descriptor that reaches past them
+    (the kernels trust the descriptor; an operand shorter than it says is a memory fault on the device)."""
+    nbytes = getattr(getattr(mat, "buf", None), "nbytes", None)
+    if nbytes is None or mat.nrows == 0 or mat.ncols == 0:
+        return
+    need = mat.offset_elems * mat.elem_bytes + ((batch - 1) * stride + (mat.nrows - 1) * (ld or mat.ncols) + mat.ncols) * elem_bytes
+    if need > nbytes:
+        raise ValueError(f"operand {what}: {mat.nrows} x {mat.ncols} (leading dimension {ld or mat.ncols}, batch {batch}, stride {stride}, "
+                         f"{elem_bytes}-byte elements) needs {need} bytes, its buffer holds {nbytes}")
+
+
+_IN_BYTES = {_ffi.IN_BF16: 2, _ffi.IN_F16: 2, _ffi.IN_E4M3: 1, _ffi.IN_E5M2: 1, _ffi.IN_E4M3_E5M2: 1, _ffi.IN_E5M2_E4M3: 1, _ffi.IN_F32: 4, _ffi.IN_F64: 8}
+
+
+def gemm_desc(a, b, c, layout=LAYOUT_NN, batch=1, stride_a=0, stride_b=0, stride_c=0, _sizes=(2, 2), _lds=(0, 0, 0)):
+    """Build a maize_gemm_desc_t from three Matrix (or MatrixT) operands.  Operands given as Matrix on a DeviceBuffer are
+    checked against the buffer's size (ValueError)."""
+    for what, mat, ld, stride, eb in (("A", a, _lds[0], stride_a, _sizes[0]), ("B", b, _lds[1], stride_b, _sizes[0]), ("C", c, _lds[2], stride_c, _sizes[1])):
+        if isinstance(mat, Matrix):
+            _check_extent(what, mat, ld, stride if batch > 1 else 0, batch, eb)
     d = _ffi.GemmDescT()
     d.a = a.realize() if isinstance(a, Matrix) else a
     d.b = b.realize() if isinstance(b, Matrix) else b
@@ -206,7 +225,9 @@ def gemm_ex_desc(a, b, c, layout=LAYOUT_NN, batch=1, stride_a=0, stride_b=0, str
     element type of C (OUT_SAME: the operands' 16-bit type, bf16 for 8-bit operands; OUT_F32; OUT_F16: IEEE half,
     for half or 8-bit operands), C = alpha * A.B + beta * C, and the element type of A and B (IN_*)."""
     x = _ffi.GemmExDescT()
-    x.gemm = gemm_desc(a, b, c, layout, batch, stride_a, stride_b, stride_c)
+    in_bytes = _IN_BYTES.get(in_type, 2)
+    c_bytes = 4 if out_type == _ffi.OUT_F32 else 2 if out_type == _ffi.OUT_F16 else max(in_bytes, 2)
+    x.gemm = gemm_desc(a, b, c, layout, batch, stride_a, stride_b, stride_c, _sizes=(in_bytes, c_bytes), _lds=(lda, ldb, ldc))
     x.lda, x.ldb, x.ldc = lda, ldb, ldc
     x.out_type = out_type
     x.in_type = in_type

@@ -351,3 +351,37 @@ def test_half_c_goes_with_half_and_8bit_operands_only():
         mz.validate(ex(out_type=3))
     # a half C is 2 bytes per element: 2-byte aligned pointers pass
     mz.validate(ex(ptrs=(0x1001, 0x100003, 0x2000002), in_type=mz.IN_E4M3, out_type=mz.OUT_F16))
+
+
+def test_a_descriptor_may_not_reach_past_its_buffers():
+    """A Matrix on a DeviceBuffer carries the buffer's size: a descriptor whose rows, leading dimension, batch stride or
+    element size reach past it is refused on the host (the kernels trust the descriptor)."""
+    from maize_amd.api import DeviceBuffer
+
+    def buf(nbytes):
+        return DeviceBuffer(None, 0x10000, nbytes)
+
+    m, n, k = 128, 256, 64
+    a, b, c = buf(m * k * 2), buf(k * n * 2), buf(m * n * 2)
+    mz.gemm_desc(mz.Matrix(a, m, k), mz.Matrix(b, k, n), mz.Matrix(c, m, n))                       # exact fit
+    with pytest.raises(ValueError, match="operand B"):
+        mz.gemm_desc(mz.Matrix(a, m, k), mz.Matrix(buf(k * n * 2 - 2), k, n), mz.Matrix(c, m, n))
+    with pytest.raises(ValueError, match="operand A"):
+        mz.gemm_desc(mz.Matrix(a, m, k, offset_elems=1), mz.Matrix(b, k, n), mz.Matrix(c, m, n))   # an offset into the buffer counts
+    with pytest.raises(ValueError, match="operand C"):
+        mz.gemm_desc(mz.Matrix(a, m, k), mz.Matrix(b, k, n), mz.Matrix(c, m, n), batch=2, stride_c=m * n)
+    mz.gemm_desc(mz.Matrix(a, m, k), mz.Matrix(b, k, n), mz.Matrix(buf(2 * m * n * 2), m, n), batch=2, stride_c=m * n)   # shared A and B (stride 0)
+    # leading dimensions, element sizes of the operand and result types
+    with pytest.raises(ValueError, match="operand A"):
+        mz.gemm_ex_desc(mz.Matrix(a, m, k), mz.Matrix(b, k, n), mz.Matrix(c, m, n), lda=k + 8)
+    mz.gemm_ex_desc(mz.Matrix(buf(((m - 1) * (k + 8) + k) * 2), m, k), mz.Matrix(b, k, n), mz.Matrix(c, m, n), lda=k + 8)
+    with pytest.raises(ValueError, match="operand C"):
+        mz.gemm_ex_desc(mz.Matrix(a, m, k), mz.Matrix(b, k, n), mz.Matrix(c, m, n), out_type=mz.OUT_F32)
+    mz.gemm_ex_desc(mz.Matrix(a, m, k), mz.Matrix(b, k, n), mz.Matrix(buf(m * n * 4), m, n), out_type=mz.OUT_F32)
+    mz.gemm_ex_desc(mz.Matrix(buf(m * k), m, k, elem_bytes=1), mz.Matrix(buf(n * k), n, k, elem_bytes=1), mz.Matrix(c, m, n), layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3)
+    with pytest.raises(ValueError, match="operand B"):
+        mz.gemm_ex_desc(mz.Matrix(buf(m * k), m, k, elem_bytes=1), mz.Matrix(buf(n * k), 2 * n, k, elem_bytes=1), mz.Matrix(c, m, n), layout=mz.LAYOUT_NT, in_type=mz.IN_E4M3)
+    with pytest.raises(ValueError, match="operand A"):
+        mz.gemm_ex_desc(mz.Matrix(a, m, k), mz.Matrix(buf(k * n * 4), k, n), mz.Matrix(buf(m * n * 4), m, n), in_type=mz.IN_F32)
+    # raw pointers (GlobalMatrix) carry no size and are taken as they are
+    mz.gemm_desc(mz.GlobalMatrix(0x1000, 1 << 20, 1 << 10), mz.GlobalMatrix(0x1000, 1 << 10, 1 << 10), mz.GlobalMatrix(0x1000, 1 << 20, 1 << 10))
