@@ -1171,18 +1171,19 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
     }
     const int st = kernel_index("maize_gemm_bf16_skinny_nt");
     if (st >= 0 && kKernels[st].supports(d) && s.n >= 64 && s.k >= 512) return (uint32_t)st;
-    // 33 .. 64 rows against 12288 or more rows of N x K weights and a K of up to 4096: one round of 128 x 128 tiles streams B as
-    // fast as the four-row-group kernel and needs no second pass over partial tiles (row-group kernel -> 128 x 128 tiles, us:
-    // 64 x 14336 x 4096 27.8 -> 25.9, 40 x 14336 x 4096 27.1 -> 25.2, 64 x 14336 x 2048 18.6 -> 15.8, 64 x 28672 x 4096 43.2 -> 36.8,
-    // 64 x 32768 x 4096 52.7 -> 42.5, 56 x 28672 x 2048 26.4 -> 21.0, 64 x 16384 x 1024 16.6 -> 10.7; level at K = 8192, 47.4 / 46.9;
-    // 32 rows stay with the two-row-group kernel, 24.7 against 25.5; a row-major B with its own, 28.8 against 31.3).
-    // 65 .. 128 rows the same, where the model gives the cut over K partial tiles too cheap for their rows (128-row tiles in
-    // four ranges -> here: 80 x 16384 x 4096 32.0 -> 26.7, 72 x 14336 x 4096 28.7 -> 26.5, 128 x 14336 x 8192 53.1 -> 49.5; K x N is mixed,
-    // 128 x 14336 x 4096 33.6 / 31.3 but 72 x 14336 x 4096 29.0 / 30.6, and stays with the model)
-    if (s.nt && s.m > 32u && s.m <= 128u && s.k >= 256u && s.k <= (s.m > 64u ? 8192u : 4096u) && s.n >= 12288u) {
+    // 33 .. 64 rows against 12288 or more rows of N x K weights: one round of 128 x 128 tiles needs no second pass over partial
+    // tiles, and beats the four-row-group kernel where it also keeps up when the weights come from HBM rather than from the
+    // memory-side cache -- a K of up to 2048, or 192 tiles and more (row-group kernel -> 128 x 128 tiles, us, weights resident |
+    // cycled past the cache: 64 x 14336 x 2048 18.6 -> 15.8 | 24.5 -> 22.3, 64 x 28672 x 4096 43.2 -> 36.8 | 52.9 -> 51.9,
+    // 64 x 32768 x 4096 52.7 -> 42.5, 56 x 28672 x 2048 26.4 -> 21.0, 64 x 16384 x 1024 16.6 -> 10.7; but 64 x 14336 x 4096, 112 tiles:
+    // 27.8 -> 25.9 | 35.1 -> 38.2, 40 x 14336 x 4096 27.1 -> 25.2 | 34.3 -> 35.8 -- 112 workgroups draw less from HBM than 256).
+    // (65 .. 128 rows were tried the same way: ahead with resident weights, 80 x 16384 x 4096 32.0 -> 26.7, and 9-20 % behind the
+    // 128-row tiles cut over K with cycled ones, 38.5 -> 42.2, 128 x 14336 x 8192 66.2 -> 79.6: left to the model.)
+    if (s.nt && s.m > 32u && s.m <= 64u && s.k >= 256u && s.k <= 4096u && s.n >= 12288u) {
         const int t6 = kernel_index(half_in(d) ? "maize_gemm_f16_t128_nt" : "maize_gemm_bf16_t128_nt");
         const uint32_t units = compute_units >= 8u ? compute_units - compute_units % 8u : compute_units;
-        if (t6 >= 0 && kKernels[t6].supports(d) && (uint64_t)cdiv(s.n, 128) * d.gemm.batch <= units) return (uint32_t)t6;
+        const uint64_t tiles = (uint64_t)cdiv(s.n, 128) * d.gemm.batch;
+        if (t6 >= 0 && kKernels[t6].supports(d) && tiles <= units && (s.k <= 2048u || tiles >= 192u)) return (uint32_t)t6;
     }
     if (s.nt && s.m > 16u && s.m <= 64u && s.k >= 1024u && s.n >= (s.m <= 32u ? 1024u : 12288u)) {
         const int sm = kernel_index(s.m <= 32u ? "maize_gemm_bf16_skinny_nt_m32" : "maize_gemm_bf16_skinny_nt_m64");

@@ -235,10 +235,10 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",              # N x K weights streamed once
         (16, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",
         (17, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m32",          # 17 .. 32 rows: two row groups
-        (64, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_t128_nt",               # 33 .. 64 rows, 12288 columns up, K up to 4096: one round of 128 x 128 tiles (27.8 -> 25.9 us)
-        (64, 14336, 8192, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m64",         # ... a longer K: four row groups
-        (65, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_t128_nt",               # more than 64 rows: the same round of 112 tiles (72 rows: 28.7 us cut over K, 26.5 here)
-        (65, 11008, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128r3_splitk",  # ... fewer than 12288 columns: 128-row tiles cut over K
+        (64, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m64",         # 33 .. 64 rows and many slabs: four
+        (64, 14336, 2048, mz.LAYOUT_NT, 1): "maize_gemm_bf16_t128_nt",               # ... a K of up to 2048, or 192 tiles and more: one round of 128 x 128 tiles (18.6 -> 15.8 us; weights from HBM 24.5 -> 22.3)
+        (64, 28672, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_t128_nt",
+        (65, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128r3_splitk",  # more than 64 rows
         (32, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn_m32",
         (64, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_skinny_nn_m64",
         (64, 8192, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3_splitk", # 64 rows, 32 slabs: the tile kernel cut over K

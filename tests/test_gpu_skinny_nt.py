@@ -129,8 +129,8 @@ def test_row_groups_bf16_and_half(ctx, oracle, shape):
 
 def test_row_groups_dispatch_views_and_epilogues(ctx, oracle):
     assert run_ex(ctx, oracle, 32, 14336, 4096, layout=NT, label="auto m32") == "maize_gemm_bf16_skinny_nt_m32"
-    assert run_ex(ctx, oracle, 64, 14336, 8192, layout=NT, label="auto m64") == "maize_gemm_bf16_skinny_nt_m64"
-    assert run_ex(ctx, oracle, 64, 14336, 4096, layout=NT, label="auto, 64 rows, K up to 4096") == "maize_gemm_bf16_t128_nt"
+    assert run_ex(ctx, oracle, 64, 14336, 4096, layout=NT, label="auto m64") == "maize_gemm_bf16_skinny_nt_m64"
+    assert run_ex(ctx, oracle, 64, 14336, 2048, layout=NT, label="auto, 64 rows, K up to 2048") == "maize_gemm_bf16_t128_nt"
     assert run_ex(ctx, oracle, 64, 4096, 4096, layout=NT, label="few slabs") == "maize_gemm_bf16_mt256_nt_h128_splitk"
     for m in (24, 56):
         name = _rows_kernel("bf16", m)
