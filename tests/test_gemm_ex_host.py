@@ -151,6 +151,10 @@ def test_dispatch_of_half_operands():
     assert mz.gemm_plan(ex(4096, 4096, 4040, layout=mz.LAYOUT_NT, in_type=mz.IN_F16, beta=1.0))["kernel"] == "maize_gemm_f16_mt256_nt_ktail_gen"
     assert mz.gemm_plan(ex(16, 14336, 4096, in_type=mz.IN_F16))["kernel"] == "maize_gemm_bf16_skinny_nn"   # type is a launch flag there
     assert mz.gemm_plan(ex(33, 17, 65, in_type=mz.IN_F16))["kernel"] == "maize_gemm_bf16_wave32"
+    # 33 .. 64 rows against many rows of N x K weights: half operands follow the same rule with their own tile kernel
+    assert mz.gemm_plan(ex(64, 14336, 2048, layout=mz.LAYOUT_NT, in_type=mz.IN_F16))["kernel"] == "maize_gemm_f16_t128_nt"
+    assert mz.gemm_plan(ex(64, 28672, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_F16))["kernel"] == "maize_gemm_f16_t128_nt"
+    assert mz.gemm_plan(ex(64, 14336, 4096, layout=mz.LAYOUT_NT, in_type=mz.IN_F16))["kernel"] == "maize_gemm_bf16_skinny_nt_m64"   # 112 tiles, K = 4096: the row-group kernel
     x = ex(**big, in_type=mz.IN_F16)
     for name in mz.kernel_names():
         if "mt256" in name:
