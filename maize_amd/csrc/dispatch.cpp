@@ -1231,7 +1231,13 @@ uint32_t select_kernel(const maize_gemm_ex_desc_t& d, uint32_t compute_units) {
                                                          {"maize_gemm_f16_mt256_nn_h128_splitk", "maize_gemm_f16_mt256_nt_h128_splitk"}},
                                                         {{"maize_gemm_bf16_mt256_nn_h128r3_splitk", "maize_gemm_bf16_mt256_nt_h128r3_splitk"},
                                                          {"maize_gemm_f16_mt256_nn_h128r3_splitk", "maize_gemm_f16_mt256_nt_h128r3_splitk"}}};
-        const int r3 = h128_three_stages(cdiv(cdiv(s.k, 64u), hk) * 64u, 64u, (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk, true);
+        // (which loop runs a range is decided from 8 steps a range on, though a range is priced as three-stage only from 12: at 8
+        // steps three stages were ahead on all eighteen cuts timed, two stages -> three, us: 64 x 4096 x 4096 N x K in eight ranges
+        // 18.0 -> 16.7, K x N 20.4 -> 19.4, 4 x 64 x 1024 x 4096 17.9 -> 16.4, 128 x 2048 x 4096 19.1 -> 18.4, 128 x 1024 x 8192 in sixteen
+        // 19.7 -> 19.2; at 5 steps a range level, 64 x 2048 x 4096 in thirteen 16.4 / 16.6)
+        const uint32_t range_steps = cdiv(cdiv(s.k, 64u), hk);
+        const uint64_t range_items = (uint64_t)cdiv(s.m, 128) * cdiv(s.n, 256) * d.gemm.batch * hk;
+        const int r3 = h128_three_stages(range_steps * 64u, 64u, range_items, true) || (range_steps >= 8u && range_items >= 48u);
         const int hs = kernel_index(kH128Split[r3][half_in(d)][s.nt]);
         if (hs >= 0 && kKernels[hs].supports(d) && plan_fits(kKernels[hs], d, compute_units)) return (uint32_t)hs;
     }

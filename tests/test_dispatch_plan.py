@@ -231,7 +231,8 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
         (1024, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_t128_nt",              # 256 tiles of 128 x 128, one round (40.7 -> 34.3 us)
         (512, 14336, 4096, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3",      # 112 tiles: 224 of 128 rows are one round
         (1024, 1024, 8192, mz.LAYOUT_NN, 1): "maize_gemm_bf16_mt256_nn_h128r3_splitk",  # few tiles, a long K: 128-row tiles cut over K (ranges of 16 steps: three stages)
-        (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128_splitk",
+        (64, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128r3_splitk",  # eight ranges of 8 steps: three ring stages (18.0 -> 16.7 us)
+        (64, 2048, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_mt256_nt_h128_splitk",    # thirteen ranges of 5: two
         (16, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",              # N x K weights streamed once
         (16, 14336, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt",
         (17, 4096, 4096, mz.LAYOUT_NT, 1): "maize_gemm_bf16_skinny_nt_m32",          # 17 .. 32 rows: two row groups
@@ -257,7 +258,7 @@ def test_north_star_configurations_get_the_kernels_they_were_designed_for():
 
 def test_split_k_of_few_tiles_fills_the_chip_once():
     p = mz.gemm_plan(desc(64, 4096, 4096), compute_units=CUS)
-    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk" and 8 <= p["ksplit"] <= 16 and p["grid"] == (16 * p["ksplit"], 1, 1)
+    assert p["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk" and 8 <= p["ksplit"] <= 16 and p["grid"] == (16 * p["ksplit"], 1, 1)
     p = mz.gemm_plan(desc(256, 256, 16384), compute_units=CUS)                    # two tiles of 128 rows
     assert 16 <= p["ksplit"] <= 64 and p["grid"] == (2 * p["ksplit"], 1, 1)
     p = mz.gemm_plan(desc(1024, 1024, 8192), compute_units=CUS)                   # 32 tiles of 128 rows

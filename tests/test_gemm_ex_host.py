@@ -84,7 +84,7 @@ def test_dispatch_of_extended_descriptors():
     assert mz.gemm_plan(ex(16, 14336, 4096, lda=4100))["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk"   # rows of A off the 16-byte grid: the macro-tile kernels read them where they lie
     assert mz.gemm_plan(ex(32, 14336, 4096, ldb=14340))["kernel"] == "maize_gemm_bf16_skinny_nn_m32"     # 17 .. 64 rows: the same stream with more row groups
     assert mz.gemm_plan(ex(64, 14336, 4096))["kernel"] == "maize_gemm_bf16_skinny_nn_m64"
-    assert mz.gemm_plan(ex(64, 4096, 4096))["kernel"] == "maize_gemm_bf16_mt256_nn_h128_splitk"          # few slabs: the tile kernel (128-row tiles) cut over K is faster
+    assert mz.gemm_plan(ex(64, 4096, 4096))["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk"        # few slabs: the tile kernel (128-row tiles) cut over K is faster
     assert mz.gemm_plan(ex(65, 14336, 4096))["kernel"] == "maize_gemm_bf16_mt256_nn_h128r3_splitk"
 
 

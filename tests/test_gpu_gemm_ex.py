@@ -365,7 +365,7 @@ def test_split_k_kernels(ctx, oracle, layout, shape):
     if (m, n, k) == (64, 4096, 4096):
         x = mz.gemm_ex_desc(mz.GlobalMatrix(0x1000, m, k), mz.GlobalMatrix(0x1000000, *((k, n) if layout == mz.LAYOUT_NN else (n, k))),
                             mz.GlobalMatrix(0x4000000, m, n), layout=layout)
-        assert mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"] == half_tiles
+        assert mz.gemm_plan(x, compute_units=ctx.info()["compute_units"])["kernel"] == three       # (ranges of 8 steps: three stages)
     for kw in (dict(alpha=-1.25, beta=0.75), dict(out_f32=True, alpha=3.0, beta=-0.5, ldc=n + 8), dict(half=True),
                dict(lda=k + 8, ldc=n + 16)):
         for name in (want, half_tiles, three):

@@ -131,7 +131,7 @@ def test_row_groups_dispatch_views_and_epilogues(ctx, oracle):
     assert run_ex(ctx, oracle, 32, 14336, 4096, layout=NT, label="auto m32") == "maize_gemm_bf16_skinny_nt_m32"
     assert run_ex(ctx, oracle, 64, 14336, 4096, layout=NT, label="auto m64") == "maize_gemm_bf16_skinny_nt_m64"
     assert run_ex(ctx, oracle, 64, 14336, 2048, layout=NT, label="auto, 64 rows, K up to 2048") == "maize_gemm_bf16_t128_nt"
-    assert run_ex(ctx, oracle, 64, 4096, 4096, layout=NT, label="few slabs") == "maize_gemm_bf16_mt256_nt_h128_splitk"
+    assert run_ex(ctx, oracle, 64, 4096, 4096, layout=NT, label="few slabs") == "maize_gemm_bf16_mt256_nt_h128r3_splitk"
     for m in (24, 56):
         name = _rows_kernel("bf16", m)
         assert run_ex(ctx, oracle, m, 1096, 4104, layout=NT, kernel=name, label="K % 64 != 0") == name
